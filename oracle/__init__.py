@@ -1,0 +1,37 @@
+"""CPU oracle for the KV-cache decode path.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the shipped package (``ohara_amd``) imports
+this directory.  The only callers are ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` - and there only as the checker / the reported
+host baseline, never as the thing measured or shipped.
+
+Every function restates, in plain PyTorch on the CPU (integer parts in numpy/torch
+integer arithmetic), the algorithm of the reference file:line it cites.  The
+restatement is functional (a flat ``dict`` of tensors keyed by the reference's
+state-dict names) rather than an ``nn.Module`` tree.
+
+Pinning status (what independently fixes each function; see tests/test_oracle_*.py):
+
+  rms_norm            closed form, unit-RMS invariant, fp64 brute force
+  rope_table          closed form cos/sin(t * theta^(-2i/D)) in fp64
+  apply_rope          complex multiply (torch.view_as_complex), norm preservation,
+                      identity at position 0
+  KVCacheRef          copy semantics + the reference's error substrings
+  attention           fp64 brute-force loops on tiny inputs; cached == uncached
+                      (the uncached path reduces to F.scaled_dot_product_attention
+                      with is_causal=True, a library routine)
+  swiglu / linear     F.silu / matmul library routines
+  llama_forward       composition: golden fixture tests/golden/llama_tiny_*.pt
+  moe_route/dispatch  per-token hand loop, k distinct experts, weights sum to 1,
+                      golden fixture tests/golden/moe_tiny.pt
+  sample_*            the reference tests' known answers; exhaustive small-V
+                      restatement in fp64; inverse-CDF identities
+  bitlinear_*         torch.int32 matmul (library routine), closed forms
+                      (W = c*T reproduces T, equal activations -> +-127)
+  generate loops      the reference tests' literal outputs ("1 2 3 5 5 5",
+                      call lengths [3,1,1], positions [0,3,4])
+
+bf16 GEMM accumulation order is "parity unpinned" by the reference (it holds no
+bf16 test); the oracle defines a Linear as an fp32-accumulated product of the
+dtype-rounded operands, rounded once to the model dtype.
+"""
