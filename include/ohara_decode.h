@@ -1,0 +1,113 @@
+/*
+ * ohara_decode.h - C ABI of libohara_decode.so, the MI355X (gfx950) kernels behind
+ * ohara's KV-cache decode path.
+ *
+ * The reference (joey00072/ohara) is pure Python/PyTorch and has no FFI of its own;
+ * each entry point below names the reference code it replaces (file:line in the
+ * reference tree).  Conventions shared by every function:
+ *
+ *   - plain C: raw device pointers, sizes, a hipStream_t passed as void*;
+ *   - returns OHARA_OK (0) or a negative OHARA_E* code; never throws, never exits,
+ *     never allocates or frees device memory, never synchronises the host;
+ *   - all work is enqueued on `stream` and is stream-ordered, so every call can be
+ *     recorded into a HIP graph;
+ *   - bf16 tensors are passed as uint16_t* (raw bfloat16 bits), row-major;
+ *   - `pos_dev` arguments: when non-NULL the kernel reads the cache position of the
+ *     token being fed from that device int32 instead of the host argument (the
+ *     visible length is then *pos_dev + 1), so a captured graph can be replayed
+ *     while the position advances on the device.
+ *
+ * Weight matrices of Linear layers are consumed in a packed tile order produced by
+ * ohara_pack_rows_bf16 (see below); everything else is in the reference's layout.
+ */
+#ifndef OHARA_DECODE_H
+#define OHARA_DECODE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OHARA_OK 0
+#define OHARA_EINVAL (-1)   /* an argument violates the documented constraints */
+#define OHARA_ELAUNCH (-2)  /* the HIP runtime rejected a launch */
+#define OHARA_ESIZE (-3)    /* a size exceeds what the entry point supports */
+
+/* Library version and a self-description string (build flags, arch). */
+int ohara_abi_version(void);
+
+/* ---- weight packing -------------------------------------------------------
+ * Packed layout "strip/kstep/lane": the (N, K) row-major bf16 matrix of a Linear
+ * (nn.Linear.weight, ohara/models/llama.py:60-63,252; ohara/modules/mlp.py:146-148)
+ * is cut into strips of 16 rows and k-steps of 32 columns; the tile (strip s,
+ * k-step j) is stored as 64 lanes x 8 bf16, lane = 16*g + m holding row
+ * perm[16*s + m], columns 32*j + 8*g .. +7.  N is padded to a multiple of 16 and
+ * K to a multiple of 32 with zeros.  `perm` (length padded N, int32, source row or
+ * -1 for a zero row) may be NULL for the identity.
+ * Returns the packed size in bytes through *bytes when `dst` is NULL. */
+int ohara_pack_rows_bf16(const uint16_t* w, int n, int k, int ldw, const int32_t* perm, int n_padded,
+                         uint16_t* dst, int64_t* bytes, void* stream);
+
+/* ---- embedding ------------------------------------------------------------
+ * out[t, :] = table[ids[t], :]            (nn.Embedding, llama.py:245,310) */
+int ohara_embed_bf16(const int64_t* ids, const uint16_t* table, uint16_t* out, int n_tokens, int d, int vocab,
+                     void* stream);
+
+/* ---- RMSNorm --------------------------------------------------------------
+ * out = bf16(x * rsqrt(mean(x^2) + eps)) * w      (ohara/modules/norm.py:16-21) */
+int ohara_rmsnorm_bf16(const uint16_t* x, const uint16_t* w, uint16_t* out, int rows, int d, float eps,
+                       void* stream);
+
+/* ---- skinny GEMM (decode projections), batch <= 64 ---------------------------
+ * y = [rmsnorm(x; norm_w, eps)] @ W^T  with one of four epilogues.  `wp` is W in
+ * the packed layout; n / k are the logical sizes of W.  norm_w may be NULL.
+ *
+ * OHARA_EPI_STORE      out[b, n] = bf16(y)                      (any Linear)
+ * OHARA_EPI_RESIDUAL   out[b, n] = bf16(resid[b, n] + bf16(y))  (llama.py:199-200)
+ * OHARA_EPI_SWIGLU     W packed with gate/up rows interleaved (ohara_swiglu_perm);
+ *                      out[b, f] = bf16(bf16(silu(bf16(gate))) * bf16(up))
+ *                                                               (mlp.py:152)
+ * The fused QKV + rotary + cache append is a separate entry point below. */
+#define OHARA_EPI_STORE 0
+#define OHARA_EPI_RESIDUAL 1
+#define OHARA_EPI_SWIGLU 2
+int ohara_gemm_skinny_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n, int k, const uint16_t* norm_w,
+                           float eps, int batch, int epilogue, const uint16_t* resid, int ldr, uint16_t* out,
+                           int ldo, void* stream);
+
+/* Row permutation that interleaves gate and up rows for OHARA_EPI_SWIGLU: packed
+ * row 16*s + 4*g + i is gate row 8*s + 2*g + i (i < 2) or up row 8*s + 2*g + i - 2.
+ * Source rows index the vertical concatenation [gate; up] of two (f, k) matrices.
+ * perm has 2 * f_padded entries, f_padded = f rounded up to a multiple of 8. */
+int ohara_swiglu_perm(int f, int32_t* perm_host);
+
+/* Fused q/k/v projection + rotary + KV-cache append for ONE new position per
+ * sequence (decode): replaces Attention.forward's three Linears, apply_rope and
+ * KVCache.forward (llama.py:84-98; ohara/embeddings_pos/rotary.py:55-93;
+ * ohara/modules/kv_cache.py:75-118).  `wp` packs the rows [W_q; W_k; W_v].
+ *   q_out  (batch, h*dh) bf16, rotated
+ *   kcache/vcache (batch_cap, t_max, h_kv, dh) bf16; row `pos` of sequence b is
+ *   written with the rotated key / the value.
+ * cos/sin: (>= pos+1, dh/2) bf16 tables (precompute_freqs_cis, rotary.py:24-38). */
+int ohara_qkv_rope_append_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int k, const uint16_t* norm_w,
+                               float eps, int batch, int h, int h_kv, int dh, const uint16_t* cos,
+                               const uint16_t* sin, int pos, const int32_t* pos_dev, uint16_t* q_out,
+                               uint16_t* kcache, uint16_t* vcache, int t_max, void* stream);
+
+/* ---- decode attention (one query position per sequence) ----------------------
+ * out[b, h, :] = softmax(q[b,h,:] . K[b, 0:len, h/(H/Hkv), :] / sqrt(dh)) V
+ * (llama.py:100-135 with S = 1: every cached position is visible).  Split along the
+ * context into `n_split` chunks; partial (max, sum, acc) triples go to `workspace`
+ * and the last chunk to finish merges them.  workspace bytes =
+ * ohara_attn_workspace_bytes(batch, h, h_kv, dh, n_split); it must be zero-filled
+ * once before first use (the kernels leave its counters at zero). */
+int64_t ohara_attn_workspace_bytes(int batch, int h, int h_kv, int dh, int n_split);
+int ohara_attn_decode_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch, int h,
+                           int h_kv, int dh, int t_max, int len, const int32_t* pos_dev, int n_split,
+                           void* workspace, uint16_t* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OHARA_DECODE_H */

@@ -1,0 +1,322 @@
+// Split-context GQA decode attention: one query position per sequence, every cached
+// position visible (ohara/models/llama.py:100-135 with S = 1; mask :109-113 is all
+// true; scale 1/sqrt(Dh) :116-125; GQA head mapping of repeat_interleave :101-103
+// done by indexing, the expanded K/V are never materialised).
+//
+// Grid (n_split, H_kv, batch).  A workgroup streams its chunk of the context for one
+// KV head once and serves all G = H/H_kv query heads from it.  Per 16-position tile
+// a wave holds one position per lane-column (16 columns x 4 quarter-rows of Dh), so
+// q.k needs two cross-lane adds; the running max/sum of the online softmax are
+// wavefront shuffle reductions.  Partial (max, sum, acc) triples of the chunks are
+// merged by whichever workgroup of the (sequence, KV head) finishes last, in chunk
+// order, so the result does not depend on scheduling.
+#include "common.h"
+
+namespace {
+
+struct AttnArgs {
+  const bf16_t* q;   // (B, H*D)
+  const bf16_t* k;   // (Bcap, Tmax, Hkv, D)
+  const bf16_t* v;
+  bf16_t* out;       // (B, H*D)
+  int B, H, Hkv, D, Tmax, len;
+  const int32_t* pos_dev;  // when set: len = *pos_dev + 1
+  int nsplit;
+  int* counters;     // (B*Hkv)
+  float* part_ml;    // (B, H, nsplit, 2)
+  float* part_acc;   // (B, H, nsplit, D)
+  float scale;
+};
+
+__device__ __forceinline__ float dot8(uint4 a, uint4 b, float s) {
+  s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.x), __builtin_bit_cast(bf16x2, b.x), s, false);
+  s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.y), __builtin_bit_cast(bf16x2, b.y), s, false);
+  s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.z), __builtin_bit_cast(bf16x2, b.z), s, false);
+  s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.w), __builtin_bit_cast(bf16x2, b.w), s, false);
+  return s;
+}
+
+// Merge the chunk partials of the G heads of (b, kvh) and write bf16 output.
+// Called by all 256 threads of the last workgroup to finish.
+template <int MAXD>
+__device__ void merge_partials(const AttnArgs& a, int b, int kvh, int G) {
+  const int D = a.D;
+  for (int idx = threadIdx.x; idx < G * D; idx += blockDim.x) {
+    const int hh = idx / D, d = idx - hh * D;
+    const int h = kvh * G + hh;
+    const float* ml = a.part_ml + ((size_t)(b * a.H + h) * a.nsplit) * 2;
+    const float* pa = a.part_acc + ((size_t)(b * a.H + h) * a.nsplit) * D + d;
+    float M = -INFINITY;
+    for (int s = 0; s < a.nsplit; ++s) M = fmaxf(M, ml[2 * s]);
+    float Lsum = 0.f, o = 0.f;
+    for (int s = 0; s < a.nsplit; ++s) {
+      const float ms = ml[2 * s];
+      if (ms == -INFINITY) continue;
+      const float w = __expf(ms - M);
+      Lsum += ml[2 * s + 1] * w;
+      o += pa[(size_t)s * D] * w;
+    }
+    a.out[(size_t)b * a.H * D + h * D + d] = f2bf(o / Lsum);
+  }
+}
+
+// Publishes this workgroup's partials and returns true in the workgroup that
+// observes all n_split chunks done (every thread gets the same answer).
+__device__ bool last_chunk_done(int* counter, int nsplit) {
+  __shared__ int is_last;
+  __threadfence();  // partials visible device-wide before the count
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    is_last = (old == nsplit - 1);
+    if (is_last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next call
+  }
+  __syncthreads();
+  const bool last = is_last != 0;
+  if (last) __threadfence();  // acquire the other chunks' partials
+  return last;
+}
+
+template <int D, int G>
+__global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
+  constexpr int NC = D / 32;        // 16-byte K loads per lane per tile
+  constexpr int DC = D / 8;         // lanes covering one V row with 16-byte loads
+  constexpr int PP = 64 / DC;       // V rows fetched per load instruction
+  constexpr int NV = 16 / PP;       // V load instructions per 16-position tile
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int L = a.pos_dev ? min(*a.pos_dev + 1, a.Tmax) : a.len;
+  const int chunk = (((L + a.nsplit - 1) / a.nsplit) + 63) & ~63;
+  const int t0 = split * chunk;
+  const int t1 = min(L, t0 + chunk);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int p = lane & 15, dq = lane >> 4;
+  const int pp = lane / DC, dc = lane % DC;
+
+  __shared__ float s_m[4][G], s_l[4][G];
+  __shared__ float s_acc[4][G][D];
+
+  // q for this lane's quarter-row: columns (4c + dq)*8 .. +7
+  uint4 qv[G][NC];
+#pragma unroll
+  for (int hh = 0; hh < G; ++hh)
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+      qv[hh][c] = ldg16(a.q + (size_t)b * a.H * D + (size_t)(kvh * G + hh) * D + (4 * c + dq) * 8);
+
+  float m_run[G], l_run[G], acc[G][8];
+#pragma unroll
+  for (int hh = 0; hh < G; ++hh) {
+    m_run[hh] = -INFINITY;
+    l_run[hh] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[hh][i] = 0.f;
+  }
+
+  const size_t row = (size_t)a.Hkv * D;
+  const bf16_t* kb = a.k + (size_t)b * a.Tmax * row + (size_t)kvh * D;
+  const bf16_t* vb = a.v + (size_t)b * a.Tmax * row + (size_t)kvh * D;
+
+  for (int tb = t0 + wave * 16; tb < t1; tb += 64) {
+    const int pos = tb + p;
+    const bool valid = pos < t1;
+    uint4 kv[NC], vv[NV];
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+      kv[c] = valid ? ldg16_nt(kb + (size_t)pos * row + (4 * c + dq) * 8) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+      const int vp = tb + c * PP + pp;
+      vv[c] = vp < t1 ? ldg16_nt(vb + (size_t)vp * row + dc * 8) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int hh = 0; hh < G; ++hh) {
+      float s = 0.f;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) s = dot8(kv[c], qv[hh][c], s);
+      s += __shfl_xor(s, 16, WAVE);
+      s += __shfl_xor(s, 32, WAVE);
+      s = valid ? s * a.scale : -INFINITY;
+      float tm = s;
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) tm = fmaxf(tm, __shfl_xor(tm, o, WAVE));
+      const float mn = fmaxf(m_run[hh], tm);  // finite: the tile holds at least one position
+      const float corr = __expf(m_run[hh] - mn);
+      const float pv = __expf(s - mn);
+      float ts = pv;
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) ts += __shfl_xor(ts, o, WAVE);
+      l_run[hh] = l_run[hh] * corr + ts;
+      m_run[hh] = mn;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[hh][i] *= corr;
+#pragma unroll
+      for (int c = 0; c < NV; ++c) {
+        const float pw = __shfl(pv, c * PP + pp, WAVE);
+        const uint32_t w4[4] = {vv[c].x, vv[c].y, vv[c].z, vv[c].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          acc[hh][2 * i] += pw * lo_bf(w4[i]);
+          acc[hh][2 * i + 1] += pw * hi_bf(w4[i]);
+        }
+      }
+    }
+  }
+
+  // fold the PP row-groups of the wave, then the four waves
+#pragma unroll
+  for (int hh = 0; hh < G; ++hh) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float v = acc[hh][i];
+#pragma unroll
+      for (int o = DC; o < 64; o <<= 1) v += __shfl_xor(v, o, WAVE);
+      acc[hh][i] = v;
+    }
+    if (lane < DC) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s_acc[wave][hh][dc * 8 + i] = acc[hh][i];
+    }
+    if (lane == 0) {
+      s_m[wave][hh] = m_run[hh];
+      s_l[wave][hh] = l_run[hh];
+    }
+  }
+  __syncthreads();
+  for (int idx = tid; idx < G * D; idx += 256) {
+    const int hh = idx / D, d = idx - hh * D;
+    const int h = kvh * G + hh;
+    float M = fmaxf(fmaxf(s_m[0][hh], s_m[1][hh]), fmaxf(s_m[2][hh], s_m[3][hh]));
+    float Ls = 0.f, o = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float mw = s_m[w][hh];
+      const float sc = (mw == -INFINITY) ? 0.f : __expf(mw - M);
+      Ls += s_l[w][hh] * sc;
+      o += s_acc[w][hh][d] * sc;
+    }
+    const size_t pi = (size_t)(b * a.H + h) * a.nsplit + split;
+    a.part_acc[pi * D + d] = o;
+    if (d == 0) {
+      a.part_ml[pi * 2] = M;
+      a.part_ml[pi * 2 + 1] = Ls;
+    }
+  }
+  if (last_chunk_done(a.counters + b * a.Hkv + kvh, a.nsplit)) merge_partials<D>(a, b, kvh, G);
+}
+
+// Any even head width up to 256, any group size: one thread per position for q.k,
+// one thread per column for p.V.  Slow path for shapes the tuned kernel skips.
+__global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
+  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int G = a.H / a.Hkv, D = a.D;
+  const int L = a.pos_dev ? min(*a.pos_dev + 1, a.Tmax) : a.len;
+  const int chunk = (((L + a.nsplit - 1) / a.nsplit) + 63) & ~63;
+  const int t0 = split * chunk;
+  const int t1 = min(L, t0 + chunk);
+  const int tid = threadIdx.x;
+  __shared__ float s_p[256];
+  __shared__ float s_red[4];
+  __shared__ float s_q[256];
+  const size_t row = (size_t)a.Hkv * D;
+  const bf16_t* kb = a.k + (size_t)b * a.Tmax * row + (size_t)kvh * D;
+  const bf16_t* vb = a.v + (size_t)b * a.Tmax * row + (size_t)kvh * D;
+  for (int hh = 0; hh < G; ++hh) {
+    const int h = kvh * G + hh;
+    __syncthreads();
+    if (tid < D) s_q[tid] = bf2f(a.q[(size_t)b * a.H * D + (size_t)h * D + tid]);
+    __syncthreads();
+    float m_run = -INFINITY, l_run = 0.f, acc = 0.f;
+    for (int tb = t0; tb < t1; tb += 256) {
+      const int pos = tb + tid;
+      float s = -INFINITY;
+      if (pos < t1) {
+        float d_ = 0.f;
+        for (int d = 0; d < D; ++d) d_ += s_q[d] * bf2f(kb[(size_t)pos * row + d]);
+        s = d_ * a.scale;
+      }
+      float tm = wave_max(s);
+      if ((tid & 63) == 0) s_red[tid >> 6] = tm;
+      __syncthreads();
+      tm = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+      __syncthreads();
+      const float mn = fmaxf(m_run, tm);
+      const float corr = __expf(m_run - mn);
+      const float pv = (pos < t1) ? __expf(s - mn) : 0.f;
+      s_p[tid] = pv;
+      float ts = wave_sum(pv);
+      if ((tid & 63) == 0) s_red[tid >> 6] = ts;
+      __syncthreads();
+      ts = ((s_red[0] + s_red[1]) + s_red[2]) + s_red[3];
+      l_run = l_run * corr + ts;
+      m_run = mn;
+      acc *= corr;
+      if (tid < D) {
+        const int n = min(256, t1 - tb);
+        for (int i = 0; i < n; ++i) acc += s_p[i] * bf2f(vb[(size_t)(tb + i) * row + tid]);
+      }
+      __syncthreads();
+    }
+    const size_t pi = (size_t)(b * a.H + h) * a.nsplit + split;
+    if (tid < D) a.part_acc[pi * D + tid] = acc;
+    if (tid == 0) {
+      a.part_ml[pi * 2] = m_run;
+      a.part_ml[pi * 2 + 1] = l_run;
+    }
+  }
+  if (last_chunk_done(a.counters + b * a.Hkv + kvh, a.nsplit)) merge_partials<256>(a, b, kvh, G);
+}
+
+template <int D>
+int launch_fast(const AttnArgs& a, int G, dim3 grid, hipStream_t st) {
+  switch (G) {
+    case 1: hipLaunchKernelGGL((attn_decode_kernel<D, 1>), grid, dim3(256), 0, st, a); break;
+    case 2: hipLaunchKernelGGL((attn_decode_kernel<D, 2>), grid, dim3(256), 0, st, a); break;
+    case 4: hipLaunchKernelGGL((attn_decode_kernel<D, 4>), grid, dim3(256), 0, st, a); break;
+    default: return 1;
+  }
+  return 0;
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+}  // namespace
+
+extern "C" {
+
+int64_t ohara_attn_workspace_bytes(int batch, int h, int h_kv, int dh, int n_split) {
+  if (batch < 1 || h < 1 || h_kv < 1 || dh < 1 || n_split < 1) return OHARA_EINVAL;
+  size_t c = align256((size_t)batch * h_kv * sizeof(int));
+  size_t ml = align256((size_t)batch * h * n_split * 2 * sizeof(float));
+  size_t acc = align256((size_t)batch * h * n_split * dh * sizeof(float));
+  return (int64_t)(c + ml + acc);
+}
+
+int ohara_attn_decode_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch, int h,
+                           int h_kv, int dh, int t_max, int len, const int32_t* pos_dev, int n_split,
+                           void* workspace, uint16_t* out, void* stream) {
+  if (!q || !kcache || !vcache || !workspace || !out) return OHARA_EINVAL;
+  if (batch < 1 || h < 1 || h_kv < 1 || h % h_kv || dh < 2 || (dh & 1) || dh > 256) return OHARA_EINVAL;
+  if (t_max < 1 || n_split < 1 || n_split > 1024) return OHARA_EINVAL;
+  if (!pos_dev && (len < 1 || len > t_max)) return OHARA_EINVAL;
+  AttnArgs a{};
+  a.q = q; a.k = kcache; a.v = vcache; a.out = out;
+  a.B = batch; a.H = h; a.Hkv = h_kv; a.D = dh; a.Tmax = t_max; a.len = len; a.pos_dev = pos_dev;
+  a.nsplit = n_split;
+  char* ws = reinterpret_cast<char*>(workspace);
+  a.counters = reinterpret_cast<int*>(ws);
+  ws += align256((size_t)batch * h_kv * sizeof(int));
+  a.part_ml = reinterpret_cast<float*>(ws);
+  ws += align256((size_t)batch * h * n_split * 2 * sizeof(float));
+  a.part_acc = reinterpret_cast<float*>(ws);
+  a.scale = 1.0f / sqrtf((float)dh);
+  dim3 grid(n_split, h_kv, batch);
+  hipStream_t st = (hipStream_t)stream;
+  const int G = h / h_kv;
+  int miss = 1;
+  if (dh == 128) miss = launch_fast<128>(a, G, grid, st);
+  else if (dh == 64) miss = launch_fast<64>(a, G, grid, st);
+  if (miss) hipLaunchKernelGGL(attn_decode_generic, grid, dim3(256), 0, st, a);
+  return ohara_launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,336 @@
+// Weight-streaming skinny GEMM for the decode projections (batch <= 64).
+//
+// y[b, n] = sum_k x[b, k] * W[n, k].  W is read exactly once, in a packed tile
+// order whose every wave-load is one contiguous 1 KiB (64 lanes x 16 B), straight
+// into the A operand of v_mfma_f32_16x16x32_bf16; the activations are the B
+// operand (16 batch columns per MFMA), so batch 1..16 costs the same weight
+// stream.  One workgroup (4 waves) owns one 16-row strip; the waves split K and
+// their fp32 partial tiles are summed in a fixed order through LDS, so results do
+// not depend on scheduling.
+//
+// Fusions (rounding points follow the reference's bf16 eager path):
+//   prologue  RMSNorm           ohara/modules/norm.py:16-21
+//   epilogue  residual add      ohara/models/llama.py:199-200
+//             SwiGLU            ohara/modules/mlp.py:152
+//             rotary + KV append ohara/embeddings_pos/rotary.py:55-93,
+//                               ohara/modules/kv_cache.py:104-105
+#include "common.h"
+
+namespace {
+
+enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_ROPE = 3 };
+
+struct SkinnyArgs {
+  const uint4* wp;
+  const bf16_t* x;
+  int ldx;
+  const bf16_t* norm_w;
+  float eps;
+  int B, N, K;  // logical sizes; packed sizes are the round-ups
+  bf16_t* out;
+  int ldo;
+  const bf16_t* resid;
+  int ldr;
+  // rotary + append
+  int H, Hkv, Dh, Tmax, pos;
+  const int32_t* pos_dev;
+  const bf16_t* cos;
+  const bf16_t* sin;
+  bf16_t* kcache;
+  bf16_t* vcache;
+};
+
+
+__device__ __forceinline__ float sumsq8(uint4 v) {
+  float s = 0.f;
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float a = lo_bf(w[i]), b = hi_bf(w[i]);
+    s += a * a + b * b;
+  }
+  return s;
+}
+
+// bf16(bf16(x * rinv) * w) on 8 packed values.
+__device__ __forceinline__ uint4 norm8(uint4 xv, uint4 wv, float rinv) {
+  const uint32_t xs[4] = {xv.x, xv.y, xv.z, xv.w};
+  const uint32_t ws[4] = {wv.x, wv.y, wv.z, wv.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float a = rbf(lo_bf(xs[i]) * rinv) * lo_bf(ws[i]);
+    float b = rbf(hi_bf(xs[i]) * rinv) * hi_bf(ws[i]);
+    o[i] = pack_bf(a, b);
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+template <int BT, bool NORM, int EPI>
+__global__ __launch_bounds__(256) void skinny_kernel(SkinnyArgs a) {
+  constexpr int CH = 6;  // k-steps whose weight loads are issued back to back
+  const int strip = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m = lane & 15, g = lane >> 4;
+  const int KS = (a.K + 31) >> 5;
+  const int per_wave = (KS + 3) >> 2;
+  const int j0 = wave * per_wave;
+  const int j1 = min(KS, j0 + per_wave);
+
+  __shared__ float red[3][BT][64][4];
+  __shared__ float ssq[4][BT * 16];
+
+  float rinv[BT];
+  if (NORM) {
+    float part[BT];
+#pragma unroll
+    for (int t = 0; t < BT; ++t) part[t] = 0.f;
+    for (int j = j0; j < j1; ++j) {
+      const int k0 = 32 * j + 8 * g;
+#pragma unroll
+      for (int t = 0; t < BT; ++t) {
+        const int b = m + 16 * t;
+        if (b < a.B && k0 < a.K) part[t] += sumsq8(ldg16(a.x + (size_t)b * a.ldx + k0));
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < BT; ++t) {
+      float p = part[t];
+      p += __shfl_xor(p, 16, WAVE);
+      p += __shfl_xor(p, 32, WAVE);
+      if (g == 0) ssq[wave][16 * t + m] = p;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < BT; ++t) {
+      const float tot = ((ssq[0][16 * t + m] + ssq[1][16 * t + m]) + ssq[2][16 * t + m]) + ssq[3][16 * t + m];
+      rinv[t] = 1.0f / sqrtf(tot / (float)a.K + a.eps);
+    }
+  }
+
+  f32x4 acc[BT];
+#pragma unroll
+  for (int t = 0; t < BT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  const uint4* wrow = a.wp + (size_t)strip * KS * 64 + lane;
+
+  auto step = [&](uint4 wv, int j) {
+    const int k0 = 32 * j + 8 * g;
+    uint4 nw = make_uint4(0, 0, 0, 0);
+    if (NORM && k0 < a.K) nw = ldg16(a.norm_w + k0);
+#pragma unroll
+    for (int t = 0; t < BT; ++t) {
+      const int b = m + 16 * t;
+      uint4 xv = make_uint4(0, 0, 0, 0);
+      if (b < a.B && k0 < a.K) {
+        xv = ldg16(a.x + (size_t)b * a.ldx + k0);
+        if (NORM) xv = norm8(xv, nw, rinv[t]);
+      }
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wv),
+                                                       __builtin_bit_cast(bf16x8, xv), acc[t], 0, 0, 0);
+    }
+  };
+
+  int j = j0;
+  for (; j + CH <= j1; j += CH) {
+    uint4 wv[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) wv[c] = ldg16_nt(wrow + (size_t)(j + c) * 64);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) step(wv[c], j + c);
+  }
+  for (; j < j1; ++j) step(ldg16_nt(wrow + (size_t)j * 64), j);
+
+  // Fixed-order cross-wave sum: ((w0 + w1) + w2) + w3.
+  if (wave > 0) {
+#pragma unroll
+    for (int t = 0; t < BT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave - 1][t][lane][i] = acc[t][i];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+#pragma unroll
+  for (int t = 0; t < BT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[t][i] = ((acc[t][i] + red[0][t][lane][i]) + red[1][t][lane][i]) + red[2][t][lane][i];
+
+  const int r0 = strip * 16 + 4 * g;  // first of this lane's four packed rows
+#pragma unroll
+  for (int t = 0; t < BT; ++t) {
+    const int b = m + 16 * t;
+    if (b >= a.B) continue;
+    const float y0 = rbf(acc[t][0]), y1 = rbf(acc[t][1]), y2 = rbf(acc[t][2]), y3 = rbf(acc[t][3]);
+    if (EPI == EPI_STORE || EPI == EPI_RESIDUAL) {
+      float v[4] = {y0, y1, y2, y3};
+      bf16_t* o = a.out + (size_t)b * a.ldo + r0;
+      if (EPI == EPI_RESIDUAL) {
+        const bf16_t* r = a.resid + (size_t)b * a.ldr + r0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (r0 + i < a.N) v[i] = bf2f(r[i]) + v[i];
+      }
+      if (r0 + 3 < a.N && ((a.ldo & 3) == 0)) {
+        uint2 pk = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
+        *reinterpret_cast<uint2*>(o) = pk;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (r0 + i < a.N) o[i] = f2bf(v[i]);
+      }
+    } else if (EPI == EPI_SWIGLU) {
+      // rows: gate f, gate f+1, up f, up f+1 with f = 8*strip + 2*g; N = hidden width F
+      const int f = strip * 8 + 2 * g;
+      const float s0 = rbf(silu_f(y0)), s1 = rbf(silu_f(y1));
+      bf16_t* o = a.out + (size_t)b * a.ldo + f;
+      if (f < a.N) o[0] = f2bf(s0 * y2);
+      if (f + 1 < a.N) o[1] = f2bf(s1 * y3);
+    } else {  // EPI_ROPE: rows [q (H*Dh); k (Hkv*Dh); v (Hkv*Dh)], one position per sequence
+      const int pos = a.pos_dev ? *a.pos_dev : a.pos;
+      const int nq = a.H * a.Dh, nk = a.Hkv * a.Dh;
+      if (r0 >= nq + 2 * nk || pos < 0 || pos >= a.Tmax) continue;
+      float v[4] = {y0, y1, y2, y3};
+      bf16_t* o;
+      if (r0 < nq + nk) {
+        const int d = (r0 < nq ? r0 : r0 - nq) % a.Dh;
+        const bf16_t* cs = a.cos + (size_t)pos * (a.Dh >> 1) + (d >> 1);
+        const bf16_t* sn = a.sin + (size_t)pos * (a.Dh >> 1) + (d >> 1);
+#pragma unroll
+        for (int pr = 0; pr < 2; ++pr) {
+          const float c = bf2f(cs[pr]), s = bf2f(sn[pr]);
+          const float e = v[2 * pr], od = v[2 * pr + 1];
+          // separate fp32 multiplies and add/sub, as the reference's eager ops round
+          v[2 * pr] = __fsub_rn(__fmul_rn(e, c), __fmul_rn(od, s));
+          v[2 * pr + 1] = __fadd_rn(__fmul_rn(e, s), __fmul_rn(od, c));
+        }
+        if (r0 < nq) {
+          o = a.out + (size_t)b * a.ldo + r0;
+        } else {
+          const int rk = r0 - nq;
+          o = a.kcache + (((size_t)b * a.Tmax + pos) * a.Hkv) * a.Dh + rk;
+        }
+      } else {
+        const int rv = r0 - nq - nk;
+        o = a.vcache + (((size_t)b * a.Tmax + pos) * a.Hkv) * a.Dh + rv;
+      }
+      *reinterpret_cast<uint2*>(o) = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
+    }
+  }
+}
+
+template <int BT, bool NORM>
+int launch_epi(const SkinnyArgs& a, int epi, int strips, hipStream_t st) {
+  dim3 grid(strips), block(256);
+  switch (epi) {
+    case EPI_STORE: hipLaunchKernelGGL((skinny_kernel<BT, NORM, EPI_STORE>), grid, block, 0, st, a); break;
+    case EPI_RESIDUAL: hipLaunchKernelGGL((skinny_kernel<BT, NORM, EPI_RESIDUAL>), grid, block, 0, st, a); break;
+    case EPI_SWIGLU: hipLaunchKernelGGL((skinny_kernel<BT, NORM, EPI_SWIGLU>), grid, block, 0, st, a); break;
+    case EPI_ROPE: hipLaunchKernelGGL((skinny_kernel<BT, NORM, EPI_ROPE>), grid, block, 0, st, a); break;
+    default: return OHARA_EINVAL;
+  }
+  return ohara_launch_status();
+}
+
+int launch_skinny(const SkinnyArgs& a, int epi, int packed_rows, hipStream_t st) {
+  const int strips = packed_rows / 16;
+  const bool norm = a.norm_w != nullptr;
+  const int bt = (a.B + 15) / 16;
+  if (bt == 1) return norm ? launch_epi<1, true>(a, epi, strips, st) : launch_epi<1, false>(a, epi, strips, st);
+  if (bt == 2) return norm ? launch_epi<2, true>(a, epi, strips, st) : launch_epi<2, false>(a, epi, strips, st);
+  if (bt <= 4) return norm ? launch_epi<4, true>(a, epi, strips, st) : launch_epi<4, false>(a, epi, strips, st);
+  return OHARA_ESIZE;
+}
+
+__global__ void pack_rows_kernel(const bf16_t* w, int n, int k, int ldw, const int32_t* perm, int n_padded,
+                                 int KS, uint4* dst) {
+  // one thread per (strip, kstep, lane)
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t total = (size_t)(n_padded / 16) * KS * 64;
+  if (idx >= total) return;
+  const int lane = idx & 63;
+  const size_t sj = idx >> 6;
+  const int j = (int)(sj % KS);
+  const int s = (int)(sj / KS);
+  const int m = lane & 15, g = lane >> 4;
+  const int prow = 16 * s + m;
+  const int src = perm ? perm[prow] : (prow < n ? prow : -1);
+  const int k0 = 32 * j + 8 * g;
+  uint16_t v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = (src >= 0 && src < n && k0 + i < k) ? w[(size_t)src * ldw + k0 + i] : 0;
+  dst[idx] = make_uint4(v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16));
+}
+
+}  // namespace
+
+extern "C" {
+
+int ohara_pack_rows_bf16(const uint16_t* w, int n, int k, int ldw, const int32_t* perm, int n_padded,
+                         uint16_t* dst, int64_t* bytes, void* stream) {
+  if (n < 1 || k < 1 || (n_padded < n && perm == nullptr)) return OHARA_EINVAL;
+  if (n_padded % 16) return OHARA_EINVAL;
+  const int KS = (k + 31) / 32;
+  const int64_t total = (int64_t)(n_padded / 16) * KS * 64;
+  if (bytes) *bytes = total * 16;
+  if (!dst) return OHARA_OK;
+  if (!w || ldw < k) return OHARA_EINVAL;
+  const int threads = 256;
+  const int64_t blocks = (total + threads - 1) / threads;
+  hipLaunchKernelGGL(pack_rows_kernel, dim3((unsigned)blocks), dim3(threads), 0, (hipStream_t)stream, w, n, k, ldw,
+                     perm, n_padded, KS, reinterpret_cast<uint4*>(dst));
+  return ohara_launch_status();
+}
+
+int ohara_swiglu_perm(int f, int32_t* perm_host) {
+  if (f < 1 || !perm_host) return OHARA_EINVAL;
+  const int fp = (f + 7) / 8 * 8;
+  for (int s = 0; s < fp / 8; ++s)
+    for (int g = 0; g < 4; ++g)
+      for (int i = 0; i < 4; ++i) {
+        const int fcol = 8 * s + 2 * g + (i & 1);
+        const int src = (i < 2) ? fcol : f + fcol;
+        perm_host[16 * s + 4 * g + i] = fcol < f ? src : -1;
+      }
+  return OHARA_OK;
+}
+
+int ohara_gemm_skinny_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n, int k, const uint16_t* norm_w,
+                           float eps, int batch, int epilogue, const uint16_t* resid, int ldr, uint16_t* out,
+                           int ldo, void* stream) {
+  if (!x || !wp || !out || n < 1 || k < 1 || batch < 1) return OHARA_EINVAL;
+  if (batch > 64) return OHARA_ESIZE;
+  if ((k & 7) || (ldx & 7) || ldx < k) return OHARA_EINVAL;  // 16-byte activation loads
+  if (epilogue == OHARA_EPI_RESIDUAL && (!resid || ldr < n)) return OHARA_EINVAL;
+  if (epilogue < OHARA_EPI_STORE || epilogue > OHARA_EPI_SWIGLU) return OHARA_EINVAL;
+  if (ldo < n) return OHARA_EINVAL;
+  SkinnyArgs a{};
+  a.wp = reinterpret_cast<const uint4*>(wp);
+  a.x = x; a.ldx = ldx; a.norm_w = norm_w; a.eps = eps;
+  a.B = batch; a.N = n; a.K = k;
+  a.out = out; a.ldo = ldo; a.resid = resid; a.ldr = ldr;
+  int packed_rows;
+  if (epilogue == OHARA_EPI_SWIGLU) packed_rows = 2 * ((n + 7) / 8 * 8);
+  else packed_rows = (n + 15) / 16 * 16;
+  return launch_skinny(a, epilogue, packed_rows, (hipStream_t)stream);
+}
+
+int ohara_qkv_rope_append_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int k, const uint16_t* norm_w,
+                               float eps, int batch, int h, int h_kv, int dh, const uint16_t* cos,
+                               const uint16_t* sin, int pos, const int32_t* pos_dev, uint16_t* q_out,
+                               uint16_t* kcache, uint16_t* vcache, int t_max, void* stream) {
+  if (!x || !wp || !cos || !sin || !q_out || !kcache || !vcache) return OHARA_EINVAL;
+  if (batch < 1 || h < 1 || h_kv < 1 || h % h_kv || dh < 4 || (dh & 3) || t_max < 1) return OHARA_EINVAL;
+  if (batch > 64) return OHARA_ESIZE;
+  if ((k & 7) || (ldx & 7) || ldx < k) return OHARA_EINVAL;
+  if (!pos_dev && (pos < 0 || pos >= t_max)) return OHARA_EINVAL;
+  SkinnyArgs a{};
+  a.wp = reinterpret_cast<const uint4*>(wp);
+  a.x = x; a.ldx = ldx; a.norm_w = norm_w; a.eps = eps;
+  a.B = batch; a.N = (h + 2 * h_kv) * dh; a.K = k;
+  a.out = q_out; a.ldo = h * dh;
+  a.H = h; a.Hkv = h_kv; a.Dh = dh; a.Tmax = t_max; a.pos = pos; a.pos_dev = pos_dev;
+  a.cos = cos; a.sin = sin; a.kcache = kcache; a.vcache = vcache;
+  return launch_skinny(a, EPI_ROPE, (a.N + 15) / 16 * 16, (hipStream_t)stream);
+}
+
+}  // extern "C"

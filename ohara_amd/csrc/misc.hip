@@ -1,0 +1,137 @@
+// Small memory-bound kernels of the decode step: embedding gather, standalone
+// RMSNorm, greedy token selection and the device-side step bookkeeping.
+#include "common.h"
+
+namespace {
+
+// out[t, :] = table[ids[t], :]   (nn.Embedding, ohara/models/llama.py:245,310)
+__global__ __launch_bounds__(256) void embed_kernel(const int64_t* ids, const bf16_t* table, bf16_t* out, int d,
+                                                    int vocab) {
+  const int t = blockIdx.x;
+  int64_t id = ids[t];
+  if (id < 0 || id >= vocab) id = 0;  // the host validates ids; never read out of bounds
+  const bf16_t* src = table + (size_t)id * d;
+  bf16_t* dst = out + (size_t)t * d;
+  if ((d & 7) == 0) {
+    for (int i = threadIdx.x; i < d / 8; i += blockDim.x)
+      reinterpret_cast<uint4*>(dst)[i] = reinterpret_cast<const uint4*>(src)[i];
+  } else {
+    for (int i = threadIdx.x; i < d; i += blockDim.x) dst[i] = src[i];
+  }
+}
+
+// ohara/modules/norm.py:16-21, one workgroup per row.
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const bf16_t* x, const bf16_t* w, bf16_t* out, int d,
+                                                      float eps) {
+  const size_t r = blockIdx.x;
+  const bf16_t* xr = x + r * d;
+  __shared__ float red[4];
+  float s = 0.f;
+  for (int i = threadIdx.x; i < d; i += 256) {
+    const float v = bf2f(xr[i]);
+    s += v * v;
+  }
+  s = wave_sum(s);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  const float tot = ((red[0] + red[1]) + red[2]) + red[3];
+  const float rinv = 1.0f / sqrtf(tot / (float)d + eps);
+  for (int i = threadIdx.x; i < d; i += 256) out[r * d + i] = f2bf(rbf(bf2f(xr[i]) * rinv) * bf2f(w[i]));
+}
+
+struct StepState {  // device-resident bookkeeping of a decode loop
+  int32_t pos;      // cache position of the token being fed
+  int32_t step;     // index of the token being produced
+  int32_t done;     // workgroups of the selection kernel that have finished
+  int32_t pad;
+};
+
+// Greedy selection: first index of the row maximum over the valid vocabulary
+// (argmax of the last position, ohara/chat_engine.py:61-63, ohara/inference.py:40-45;
+// padded ids masked as in chat_engine.py:398-399).  One workgroup per row.
+// Writes next_ids[b] (fed back to the embedding) and, when `history` is given,
+// history[step * B + b].  The last workgroup to finish advances pos and step.
+__global__ __launch_bounds__(1024) void argmax_kernel(const bf16_t* logits, int ldl, int vocab, int valid,
+                                                      int64_t* next_ids, int64_t* history, int hist_cap,
+                                                      StepState* st, int B) {
+  const int b = blockIdx.x;
+  const bf16_t* row = logits + (size_t)b * ldl;
+  const int n = min(valid, vocab);
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = threadIdx.x; i < n; i += 1024) {
+    const float v = bf2f(row[i]);
+    if (v > best || (v == best && i < bi)) {
+      best = v;
+      bi = i;
+    }
+  }
+  // NaN-free comparison network; ties resolve to the lowest index
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, WAVE);
+    const int oi = __shfl_xor(bi, o, WAVE);
+    if (ov > best || (ov == best && oi < bi)) {
+      best = ov;
+      bi = oi;
+    }
+  }
+  __shared__ float sv[16];
+  __shared__ int si[16];
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) {
+    sv[wave] = best;
+    si[wave] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 16; ++w)
+      if (sv[w] > best || (sv[w] == best && si[w] < bi)) {
+        best = sv[w];
+        bi = si[w];
+      }
+    if (bi == 0x7fffffff) bi = 0;  // all -inf / NaN row
+    next_ids[b] = bi;
+    if (st) {
+      const int step = st->step;
+      if (history && step < hist_cap) history[(size_t)step * B + b] = bi;
+      __threadfence();
+      const int old = __hip_atomic_fetch_add(&st->done, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      if (old == B - 1) {
+        st->done = 0;
+        st->pos += 1;
+        st->step = step + 1;
+      }
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int ohara_abi_version(void) { return 1; }
+
+int ohara_embed_bf16(const int64_t* ids, const uint16_t* table, uint16_t* out, int n_tokens, int d, int vocab,
+                     void* stream) {
+  if (!ids || !table || !out || n_tokens < 1 || d < 1 || vocab < 1) return OHARA_EINVAL;
+  hipLaunchKernelGGL(embed_kernel, dim3(n_tokens), dim3(256), 0, (hipStream_t)stream, ids, table, out, d, vocab);
+  return ohara_launch_status();
+}
+
+int ohara_rmsnorm_bf16(const uint16_t* x, const uint16_t* w, uint16_t* out, int rows, int d, float eps,
+                       void* stream) {
+  if (!x || !w || !out || rows < 1 || d < 1) return OHARA_EINVAL;
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, x, w, out, d, eps);
+  return ohara_launch_status();
+}
+
+int ohara_argmax_bf16(const uint16_t* logits, int ldl, int batch, int vocab, int valid_vocab, int64_t* next_ids,
+                      int64_t* history, int hist_cap, int32_t* step_state, void* stream) {
+  if (!logits || !next_ids || batch < 1 || vocab < 1 || valid_vocab < 1 || ldl < vocab) return OHARA_EINVAL;
+  hipLaunchKernelGGL(argmax_kernel, dim3(batch), dim3(1024), 0, (hipStream_t)stream, logits, ldl, vocab,
+                     valid_vocab, next_ids, history, hist_cap, reinterpret_cast<StepState*>(step_state), batch);
+  return ohara_launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,176 @@
+"""Tensor-level wrappers over the C ABI (one Python function per entry point).
+
+PyTorch is used for device memory and the current stream only; every function here
+hands raw pointers to libohara_decode.so.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._lib import check, lib
+
+BF16 = torch.bfloat16
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+def _need(t: torch.Tensor, dtype, name: str):
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a device tensor")
+    if t.dtype != dtype:
+        raise ValueError(f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+
+
+class PackedLinear:
+    """A Linear weight (N, K) in the kernels' strip/kstep/lane tile order."""
+
+    __slots__ = ("data", "n", "k", "kind")
+
+    def __init__(self, data, n, k, kind="rows"):
+        self.data, self.n, self.k, self.kind = data, n, k, kind
+
+
+def pack_rows(w: torch.Tensor, perm: torch.Tensor | None = None, n_padded: int | None = None) -> torch.Tensor:
+    """Pack a (N, K) bf16 matrix; ``perm`` (int32, device) maps packed row -> source row."""
+    _need(w, BF16, "w")
+    n, k = w.shape
+    if n_padded is None:
+        n_padded = (n + 15) // 16 * 16
+    nbytes = C.c_int64(0)
+    check(lib().ohara_pack_rows_bf16(0, n, k, k, 0, n_padded, 0, C.byref(nbytes), 0), "pack size")
+    dst = torch.empty(nbytes.value // 2, dtype=BF16, device=w.device)
+    check(lib().ohara_pack_rows_bf16(_ptr(w), n, k, k, _ptr(perm), n_padded, _ptr(dst), None, _stream()), "pack")
+    return dst
+
+
+def pack_linear(w: torch.Tensor) -> PackedLinear:
+    return PackedLinear(pack_rows(w), w.shape[0], w.shape[1])
+
+
+def swiglu_perm(f: int, device) -> torch.Tensor:
+    fp = (f + 7) // 8 * 8
+    buf = (C.c_int32 * (2 * fp))()
+    check(lib().ohara_swiglu_perm(f, buf), "swiglu_perm")
+    return torch.tensor(list(buf), dtype=torch.int32, device=device)
+
+
+def pack_gate_up(w_gate: torch.Tensor, w_up: torch.Tensor) -> PackedLinear:
+    """Interleave gate/up rows so the SwiGLU epilogue finds a gate/up pair in one lane."""
+    f, k = w_gate.shape
+    cat = torch.cat([w_gate, w_up], dim=0).contiguous()
+    perm = swiglu_perm(f, w_gate.device)
+    return PackedLinear(pack_rows(cat, perm, perm.numel()), f, k, kind="swiglu")
+
+
+def pack_qkv(wq, wk, wv) -> PackedLinear:
+    cat = torch.cat([wq, wk, wv], dim=0).contiguous()
+    return PackedLinear(pack_rows(cat), cat.shape[0], cat.shape[1], kind="qkv")
+
+
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    _need(table, BF16, "table")
+    ids = ids.reshape(-1).contiguous()
+    n, d = ids.numel(), table.shape[1]
+    if out is None:
+        out = torch.empty(n, d, dtype=BF16, device=table.device)
+    check(lib().ohara_embed_bf16(_ptr(ids), _ptr(table), _ptr(out), n, d, table.shape[0], _stream()), "embed")
+    return out
+
+
+def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float = 1e-5, out=None) -> torch.Tensor:
+    _need(x, BF16, "x")
+    d = x.shape[-1]
+    rows = x.numel() // d
+    if out is None:
+        out = torch.empty_like(x)
+    check(lib().ohara_rmsnorm_bf16(_ptr(x), _ptr(w), _ptr(out), rows, d, eps, _stream()), "rmsnorm")
+    return out
+
+
+def gemm_skinny(x, w: PackedLinear, norm_w=None, eps=1e-5, residual=None, out=None) -> torch.Tensor:
+    """y = [rmsnorm(x)] @ W^T (+ residual / SwiGLU epilogue by the packing kind). x: (B, K)."""
+    _need(x, BF16, "x")
+    b, k = x.shape
+    if k != w.k:
+        raise ValueError(f"x has {k} columns, weight expects {w.k}")
+    if out is None:
+        out = torch.empty(b, w.n, dtype=BF16, device=x.device)
+    if w.kind == "swiglu":
+        epi = _lib.EPI_SWIGLU
+    elif residual is not None:
+        epi = _lib.EPI_RESIDUAL
+    else:
+        epi = _lib.EPI_STORE
+    check(
+        lib().ohara_gemm_skinny_bf16(
+            _ptr(x), x.stride(0), _ptr(w.data), w.n, w.k, _ptr(norm_w), eps, b, epi,
+            _ptr(residual), 0 if residual is None else residual.stride(0), _ptr(out), out.stride(0), _stream(),
+        ),
+        "gemm_skinny",
+    )
+    return out
+
+
+def qkv_rope_append(x, wqkv: PackedLinear, norm_w, eps, h, h_kv, dh, cos, sin, pos, kcache, vcache,
+                    q_out=None, pos_dev=None):
+    _need(x, BF16, "x")
+    b = x.shape[0]
+    if q_out is None:
+        q_out = torch.empty(b, h * dh, dtype=BF16, device=x.device)
+    t_max = kcache.shape[1]
+    check(
+        lib().ohara_qkv_rope_append_bf16(
+            _ptr(x), x.stride(0), _ptr(wqkv.data), wqkv.k, _ptr(norm_w), eps, b, h, h_kv, dh, _ptr(cos), _ptr(sin),
+            int(pos), _ptr(pos_dev), _ptr(q_out), _ptr(kcache), _ptr(vcache), t_max, _stream(),
+        ),
+        "qkv_rope_append",
+    )
+    return q_out
+
+
+def attn_workspace(batch, h, h_kv, dh, n_split, device) -> torch.Tensor:
+    n = lib().ohara_attn_workspace_bytes(batch, h, h_kv, dh, n_split)
+    if n < 0:
+        raise ValueError("bad attention workspace shape")
+    return torch.zeros(n, dtype=torch.uint8, device=device)
+
+
+def attn_decode(q, kcache, vcache, h, h_kv, dh, length, n_split, workspace, out=None, pos_dev=None):
+    b = q.shape[0]
+    if out is None:
+        out = torch.empty(b, h * dh, dtype=BF16, device=q.device)
+    check(
+        lib().ohara_attn_decode_bf16(
+            _ptr(q), _ptr(kcache), _ptr(vcache), b, h, h_kv, dh, kcache.shape[1], int(length), _ptr(pos_dev),
+            n_split, _ptr(workspace), _ptr(out), _stream(),
+        ),
+        "attn_decode",
+    )
+    return out
+
+
+def argmax(logits: torch.Tensor, valid_vocab: int | None = None, next_ids=None, history=None, step_state=None):
+    _need(logits, BF16, "logits")
+    b, v = logits.shape
+    if next_ids is None:
+        next_ids = torch.empty(b, dtype=torch.int64, device=logits.device)
+    check(
+        lib().ohara_argmax_bf16(
+            _ptr(logits), logits.stride(0), b, v, v if valid_vocab is None else valid_vocab, _ptr(next_ids),
+            _ptr(history), 0 if history is None else history.shape[0], _ptr(step_state), _stream(),
+        ),
+        "argmax",
+    )
+    return next_ids

@@ -1,0 +1,187 @@
+"""Parity of each HIP entry point against the CPU oracle on identical seeded inputs.
+
+All calls go through the C ABI (ohara_amd.ops -> libohara_decode.so).  Tolerances:
+element-wise kernels must reproduce the oracle's bf16 values exactly except where an
+fp32 reduction order differs (then <= 1 bf16 ulp on a small fraction of elements);
+GEMM-like kernels are compared in units of the output scale.
+"""
+
+import math
+
+import pytest
+import torch
+
+from oracle import llama_ref as R
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+
+
+def _ulp_close(a, b, max_ulp=1, frac=0.02):
+    """bf16 tensors equal up to `max_ulp` units in the last place on at most `frac` of elements."""
+    a16 = a.cpu().view(torch.int16).to(torch.int32)
+    b16 = b.cpu().view(torch.int16).to(torch.int32)
+    diff = (a16 - b16).abs()
+    assert int(diff.max()) <= max_ulp, f"max ulp diff {int(diff.max())}"
+    assert float((diff > 0).float().mean()) <= frac, f"fraction differing {float((diff > 0).float().mean())}"
+
+
+def test_embed(cuda):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(0)
+    table = torch.randn(100, 48, generator=g).to(BF)
+    ids = torch.randint(0, 100, (3, 5), generator=g)
+    out = ops.embed(ids.to(cuda), table.to(cuda))
+    assert torch.equal(out.cpu(), table[ids.reshape(-1)])
+
+
+@pytest.mark.parametrize("d", [32, 768, 2048, 100])
+def test_rmsnorm(cuda, d):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(d)
+    x = (torch.randn(7, d, generator=g) * 3).to(BF)
+    w = (1 + 0.2 * torch.randn(d, generator=g)).to(BF)
+    ref = R.rms_norm(x, w)
+    out = ops.rmsnorm(x.to(cuda), w.to(cuda))
+    _ulp_close(out, ref)
+
+
+@pytest.mark.parametrize("B,N,K", [(1, 768, 768), (3, 64, 32), (8, 3072, 768), (16, 768, 3072), (17, 100, 96),
+                                   (32, 2304, 768), (64, 768, 3072), (5, 65, 40)])
+@pytest.mark.parametrize("norm", [False, True])
+def test_gemm_skinny_store(cuda, B, N, K, norm):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(B * 1000 + N + K)
+    x = torch.randn(B, K, generator=g).to(BF)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(BF)
+    nw = (1 + 0.2 * torch.randn(K, generator=g)).to(BF)
+    xin = R.rms_norm(x, nw) if norm else x
+    ref = R.linear(xin, w)
+    wp = ops.pack_linear(w.to(cuda))
+    out = ops.gemm_skinny(x.to(cuda), wp, norm_w=nw.to(cuda) if norm else None)
+    scale = ref.float().abs().max().item()
+    err = (out.cpu().float() - ref.float()).abs().max().item()
+    assert err <= 2 ** -7 * scale, (err, scale)  # one bf16 ulp at the output scale
+    # and nearly everything identical
+    assert (out.cpu() != ref).float().mean().item() < 0.05
+
+
+def test_gemm_skinny_residual(cuda):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(5)
+    B, N, K = 4, 768, 3072
+    x = torch.randn(B, K, generator=g).to(BF)
+    w = (torch.randn(N, K, generator=g) * 0.02).to(BF)
+    res = torch.randn(B, N, generator=g).to(BF)
+    ref = res + R.linear(x, w)
+    out = ops.gemm_skinny(x.to(cuda), ops.pack_linear(w.to(cuda)), residual=res.to(cuda))
+    _ulp_close(out, ref, max_ulp=2, frac=0.05)
+
+
+@pytest.mark.parametrize("B,F,K", [(1, 3072, 768), (8, 64, 32), (33, 520, 64), (2, 12, 32)])
+def test_gemm_skinny_swiglu(cuda, B, F, K):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(F)
+    x = torch.randn(B, K, generator=g).to(BF)
+    wg = (torch.randn(F, K, generator=g) * 0.1).to(BF)
+    wu = (torch.randn(F, K, generator=g) * 0.1).to(BF)
+    nw = (1 + 0.2 * torch.randn(K, generator=g)).to(BF)
+    h = R.rms_norm(x, nw)
+    ref = torch.nn.functional.silu(R.linear(h, wg)) * R.linear(h, wu)
+    wp = ops.pack_gate_up(wg.to(cuda), wu.to(cuda))
+    out = ops.gemm_skinny(x.to(cuda), wp, norm_w=nw.to(cuda))
+    scale = ref.float().abs().max().item()
+    err = (out.cpu().float() - ref.float()).abs().max().item()
+    assert err <= 2 ** -6 * scale, (err, scale)
+    assert (out.cpu() != ref).float().mean().item() < 0.08
+
+
+@pytest.mark.parametrize("B,H,Hkv,D,K", [(1, 6, 6, 128, 768), (3, 4, 2, 16, 64), (16, 32, 8, 128, 256), (2, 4, 4, 8, 32)])
+def test_qkv_rope_append(cuda, B, H, Hkv, D, K):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(H * D)
+    Tmax, pos = 32, 11
+    x = torch.randn(B, K, generator=g).to(BF)
+    wq = (torch.randn(H * D, K, generator=g) * 0.05).to(BF)
+    wk = (torch.randn(Hkv * D, K, generator=g) * 0.05).to(BF)
+    wv = (torch.randn(Hkv * D, K, generator=g) * 0.05).to(BF)
+    nw = (1 + 0.2 * torch.randn(K, generator=g)).to(BF)
+    cos, sin = R.rope_table(D, 2 * Tmax, 10000.0)
+    cos, sin = cos.to(BF), sin.to(BF)
+    h = R.rms_norm(x, nw)
+    q = R.linear(h, wq).view(B, 1, H, D)
+    k = R.linear(h, wk).view(B, 1, Hkv, D)
+    v = R.linear(h, wv).view(B, 1, Hkv, D)
+    qr, kr = R.apply_rope(q, k, cos[pos : pos + 1], sin[pos : pos + 1])
+    kc = torch.zeros(B + 1, Tmax, Hkv, D, dtype=BF, device=cuda)
+    vc = torch.zeros_like(kc)
+    wp = ops.pack_qkv(wq.to(cuda), wk.to(cuda), wv.to(cuda))
+    qo = ops.qkv_rope_append(x.to(cuda), wp, nw.to(cuda), 1e-5, H, Hkv, D, cos.to(cuda), sin.to(cuda), pos, kc, vc)
+    for got, ref in ((qo.view(B, H, D), qr[:, 0]), (kc[:B, pos], kr[:, 0]), (vc[:B, pos], v[:, 0])):
+        scale = ref.float().abs().max().item()
+        err = (got.cpu().float() - ref.float()).abs().max().item()
+        assert err <= 2 ** -6 * scale, (err, scale)
+        assert (got.cpu() != ref).float().mean().item() < 0.08
+    # nothing else in the cache was touched
+    kc[:B, pos] = 0
+    vc[:B, pos] = 0
+    assert not kc.any() and not vc.any()
+
+
+def _attn_ref64(q, k, v, L):
+    """fp64 brute force: q (B,H,D), k/v (B,T,Hkv,D) -> (B,H,D)."""
+    B, H, D = q.shape
+    Hkv = k.shape[2]
+    G = H // Hkv
+    qd, kd, vd = q.double(), k[:, :L].double(), v[:, :L].double()
+    out = torch.empty(B, H, D, dtype=torch.float64)
+    for h in range(H):
+        s = torch.einsum("bd,btd->bt", qd[:, h], kd[:, :, h // G]) / math.sqrt(D)
+        p = torch.softmax(s, dim=-1)
+        out[:, h] = torch.einsum("bt,btd->bd", p, vd[:, :, h // G])
+    return out
+
+
+@pytest.mark.parametrize("B,H,Hkv,D,L,ns", [(1, 6, 6, 128, 1153, 16), (2, 32, 8, 128, 700, 8), (3, 16, 16, 64, 64, 4),
+                                            (2, 4, 2, 16, 37, 3), (1, 4, 4, 8, 5, 1), (4, 8, 4, 128, 1, 4),
+                                            (2, 16, 2, 64, 300, 5)])
+def test_attn_decode(cuda, B, H, Hkv, D, L, ns):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(L)
+    Tmax = L + 9
+    q = torch.randn(B, H, D, generator=g).to(BF)
+    k = torch.randn(B, Tmax, Hkv, D, generator=g).to(BF)
+    v = torch.randn(B, Tmax, Hkv, D, generator=g).to(BF)
+    ref = _attn_ref64(q, k, v, L)
+    ws = ops.attn_workspace(B, H, Hkv, D, ns, cuda)
+    kd, vd, qd = k.to(cuda), v.to(cuda), q.to(cuda).view(B, H * D)
+    for _ in range(2):  # second call checks that the counters were left at zero
+        out = ops.attn_decode(qd, kd, vd, H, Hkv, D, L, ns, ws)
+        err = (out.cpu().double().view(B, H, D) - ref).abs().max().item()
+        assert err <= 2e-2 * max(1.0, ref.abs().max().item()), err
+    # device-side length
+    pos_dev = torch.tensor([L - 1], dtype=torch.int32, device=cuda)
+    out2 = ops.attn_decode(qd, kd, vd, H, Hkv, D, 0, ns, ws, pos_dev=pos_dev)
+    assert torch.equal(out2, out)
+
+
+def test_argmax(cuda):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn(5, 65536, generator=g).to(BF)
+    logits[1, 77] = logits[1, 9000] = 50.0  # tie -> lowest index
+    logits[2, 65000] = 60.0
+    ref = logits.float().argmax(-1)
+    assert ref[1] == 77
+    out = ops.argmax(logits.to(cuda))
+    assert torch.equal(out.cpu(), ref)
+    out = ops.argmax(logits.to(cuda), valid_vocab=60000)
+    assert torch.equal(out.cpu(), logits[:, :60000].float().argmax(-1))
