@@ -59,9 +59,11 @@ int ohara_embed_bf16(const int64_t* ids, const uint16_t* table, uint16_t* out, i
 int ohara_rmsnorm_bf16(const uint16_t* x, const uint16_t* w, uint16_t* out, int rows, int d, float eps,
                        void* stream);
 
-/* ---- skinny GEMM (decode projections), batch <= 64 ---------------------------
- * y = [rmsnorm(x; norm_w, eps)] @ W^T  with one of four epilogues.  `wp` is W in
+/* ---- skinny GEMM (decode projections) ------------------------------------------
+ * y = [rmsnorm(x; norm_w, eps)] @ W^T  with one of three epilogues.  `wp` is W in
  * the packed layout; n / k are the logical sizes of W.  norm_w may be NULL.
+ * `batch` rows of x; more than 64 rows are processed 64 at a time, each chunk
+ * streaming W once (the dense many-row case belongs to ohara_gemm_bf16).
  *
  * OHARA_EPI_STORE      out[b, n] = bf16(y)                      (any Linear)
  * OHARA_EPI_RESIDUAL   out[b, n] = bf16(resid[b, n] + bf16(y))  (llama.py:199-200)
@@ -82,30 +84,102 @@ int ohara_gemm_skinny_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n
  * perm has 2 * f_padded entries, f_padded = f rounded up to a multiple of 8. */
 int ohara_swiglu_perm(int f, int32_t* perm_host);
 
-/* Fused q/k/v projection + rotary + KV-cache append for ONE new position per
- * sequence (decode): replaces Attention.forward's three Linears, apply_rope and
- * KVCache.forward (llama.py:84-98; ohara/embeddings_pos/rotary.py:55-93;
- * ohara/modules/kv_cache.py:75-118).  `wp` packs the rows [W_q; W_k; W_v].
- *   q_out  (batch, h*dh) bf16, rotated
- *   kcache/vcache (batch_cap, t_max, h_kv, dh) bf16; row `pos` of sequence b is
- *   written with the rotated key / the value.
- * cos/sin: (>= pos+1, dh/2) bf16 tables (precompute_freqs_cis, rotary.py:24-38). */
+/* Fused q/k/v projection + rotary + KV-cache append: replaces Attention.forward's
+ * three Linears, apply_rope and KVCache.forward (llama.py:84-98;
+ * ohara/embeddings_pos/rotary.py:55-93; ohara/modules/kv_cache.py:75-118).
+ * x holds batch*seq_len rows, row b*seq_len + s being position pos + s of sequence b
+ * (seq_len = 1 at decode).  `wp` packs the rows [W_q; W_k; W_v].
+ *   q_out  (batch*seq_len, h*dh) bf16, rotated
+ *   kcache/vcache (batch_cap, t_max, h_kv, dh) bf16; rows pos..pos+seq_len-1 of
+ *   sequence b are written with the rotated keys / the values.
+ * cos/sin: (>= pos+seq_len, dh/2) bf16 tables (precompute_freqs_cis, rotary.py:24-38). */
 int ohara_qkv_rope_append_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int k, const uint16_t* norm_w,
-                               float eps, int batch, int h, int h_kv, int dh, const uint16_t* cos,
+                               float eps, int batch, int seq_len, int h, int h_kv, int dh, const uint16_t* cos,
                                const uint16_t* sin, int pos, const int32_t* pos_dev, uint16_t* q_out,
                                uint16_t* kcache, uint16_t* vcache, int t_max, void* stream);
 
-/* ---- decode attention (one query position per sequence) ----------------------
- * out[b, h, :] = softmax(q[b,h,:] . K[b, 0:len, h/(H/Hkv), :] / sqrt(dh)) V
- * (llama.py:100-135 with S = 1: every cached position is visible).  Split along the
- * context into `n_split` chunks; partial (max, sum, acc) triples go to `workspace`
- * and the last chunk to finish merges them.  workspace bytes =
- * ohara_attn_workspace_bytes(batch, h, h_kv, dh, n_split); it must be zero-filled
- * once before first use (the kernels leave its counters at zero). */
+/* ---- attention over the KV cache ------------------------------------------------
+ * Query s (0 <= s < seq_len) of sequence b sits at cache position pos + s and sees
+ * positions [0, pos + s] (the cache mask key_pos <= start_pos + q_idx, llama.py:109-113):
+ *   out[b, s, h, :] = softmax(q[b,s,h,:] . K[b, 0:pos+s+1, h/(H/Hkv), :] / sqrt(dh)) V
+ * (llama.py:100-135; GQA by head indexing instead of repeat_interleave :101-103).
+ * seq_len = 1 is the decode case.  The context is split into `n_split` chunks;
+ * partial (max, sum, acc) triples go to `workspace` and the last chunk to finish
+ * merges them in chunk order.  workspace bytes = ohara_attn_workspace_bytes(
+ * batch*seq_len, h, h_kv, dh, n_split); zero-fill it once before first use (the
+ * kernels leave its counters at zero).  n_split = 1 needs no workspace (NULL ok).
+ * q / out: (batch*seq_len, h*dh). */
 int64_t ohara_attn_workspace_bytes(int batch, int h, int h_kv, int dh, int n_split);
-int ohara_attn_decode_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch, int h,
-                           int h_kv, int dh, int t_max, int len, const int32_t* pos_dev, int n_split,
-                           void* workspace, uint16_t* out, void* stream);
+int ohara_attn_cached_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch,
+                           int seq_len, int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev,
+                           int n_split, void* workspace, uint16_t* out, void* stream);
+
+/* ---- greedy selection ---------------------------------------------------------
+ * next_ids[b] = first index of max(logits[b, 0:valid_vocab])  (argmax of the last
+ * position, ohara/chat_engine.py:61-63, ohara/inference.py:40-45; ids >= valid_vocab
+ * are the padded vocabulary masked at chat_engine.py:398-399).  When `step_state`
+ * (device, 4 x int32: pos, step, done, pad) is given, the token is also written to
+ * history[step * batch + b] (if step < hist_cap) and the last workgroup to finish
+ * advances pos and step by one - the device-side loop bookkeeping. */
+int ohara_argmax_bf16(const uint16_t* logits, int ldl, int batch, int vocab, int valid_vocab, int64_t* next_ids,
+                      int64_t* history, int hist_cap, int32_t* step_state, void* stream);
+
+/* ---- the whole forward pass through the KV cache ---------------------------------
+ * Llama.forward(x, kv_cache, position) (ohara/models/llama.py:279-323; Block.forward
+ * :191-201) for seq_len new tokens per sequence, as a fixed sequence of the kernels
+ * above enqueued on `stream`; optionally followed by greedy selection that feeds the
+ * next call, so a generate loop (ohara/chat_engine.py:395-405,
+ * ohara/inference.py:110-121) can run without touching the host.
+ * Host structs; every pointer inside is a device pointer owned by the caller. */
+typedef struct OharaLayer {
+  const uint16_t* wqkv;  /* packed rows [W_q; W_k; W_v], each (heads*dh, d)          */
+  const uint16_t* wo;    /* packed attn.proj (d, h*dh)                                */
+  const uint16_t* wgu;   /* packed ff.gate / ff.up, rows interleaved (swiglu perm)    */
+  const uint16_t* wdown; /* packed ff.down (d, f)                                     */
+  const uint16_t* norm1; /* (d) */
+  const uint16_t* norm2; /* (d) */
+} OharaLayer;
+
+typedef struct OharaModel {
+  int32_t n_layers, d_model, n_heads, n_kv_heads, head_dim, d_ff, vocab, t_max;
+  float eps;
+  int32_t reserved;
+  const uint16_t* token_emb;  /* (vocab, d) row-major, unpacked */
+  const uint16_t* final_norm; /* (d) */
+  const uint16_t* w_vocab;    /* packed vocab_proj (vocab, d) */
+  const uint16_t* cos;        /* (2*t_max, dh/2) bf16 */
+  const uint16_t* sin;
+  const OharaLayer* layers;   /* host array [n_layers] */
+} OharaModel;
+
+typedef struct OharaDecodeState {
+  int32_t batch;         /* sequences                                                     */
+  int32_t rows_cap;      /* rows (batch*seq_len) the activation buffers below can hold    */
+  int32_t n_split;       /* context chunks of decode attention (seq_len == 1)             */
+  int32_t valid_vocab;   /* ids >= this are never selected; 0 = whole vocabulary          */
+  int32_t hist_cap, reserved;
+  int64_t* ids;          /* (rows) tokens fed; ids[0:batch] overwritten by greedy select  */
+  uint16_t* x;           /* (rows, d) residual stream                                     */
+  uint16_t* q;           /* (rows, h*dh)                                                  */
+  uint16_t* attn;        /* (rows, h*dh)                                                  */
+  uint16_t* act;         /* (rows, f)                                                     */
+  uint16_t* logits;      /* (batch, vocab) or (rows, vocab), see logits_mode              */
+  void* attn_ws;         /* ohara_attn_workspace_bytes(batch, h, h_kv, dh, n_split)       */
+  int32_t* step_state;   /* 4 x int32 {pos, step, done, pad}, may be NULL                 */
+  int64_t* history;      /* (hist_cap, batch) generated ids, may be NULL                  */
+  uint16_t* const* kcache; /* host array [n_layers] of (batch_cap, t_max, h_kv, dh)       */
+  uint16_t* const* vcache;
+} OharaDecodeState;
+
+#define OHARA_LOGITS_NONE 0
+#define OHARA_LOGITS_LAST 1 /* logits (batch, vocab) of each sequence's last position     */
+#define OHARA_LOGITS_ALL 2  /* logits (batch*seq_len, vocab), what llama.py:321-322 returns */
+
+/* pos: cache position of the first fed token (ignored when use_pos_dev != 0, then
+ * step_state->pos is read on the device; that needs seq_len == 1).
+ * select_greedy != 0 (needs logits_mode LAST or seq_len == 1) appends the argmax. */
+int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* s, int seq_len, int pos, int use_pos_dev,
+                        int logits_mode, int select_greedy, void* stream);
 
 #ifdef __cplusplus
 }

@@ -21,42 +21,29 @@ _p, _i, _f, _i64 = C.c_void_p, C.c_int, C.c_float, C.c_int64
 
 
 class OharaLayer(C.Structure):
-    _fields_ = [
-        ("kind", _i),            # 0 dense SwiGLU, 1 grouped MoE
-        ("bitlinear", _i),       # 1: the seven projections are ternary BitLinears
-        ("wqkv", _p), ("wo", _p), ("wgu", _p), ("wdown", _p),
-        ("norm1", _p), ("norm2", _p),
-        ("kcache", _p), ("vcache", _p),
-        # BitLinear extras: per-projection RMSNorm weights and scales
-        ("bn_qkv", _p), ("bn_o", _p), ("bn_gu", _p), ("bn_down", _p),
-        ("gamma", _f * 7),       # q, k, v, o, gate, up, down
-        # MoE extras
-        ("router", _p), ("router_bias", _p),
-        ("e_gu", _p), ("e_down", _p),
-        ("s_gu", _p), ("s_down", _p),
-    ]
+    _fields_ = [("wqkv", _p), ("wo", _p), ("wgu", _p), ("wdown", _p), ("norm1", _p), ("norm2", _p)]
 
 
 class OharaModel(C.Structure):
     _fields_ = [
         ("n_layers", _i), ("d_model", _i), ("n_heads", _i), ("n_kv_heads", _i), ("head_dim", _i),
         ("d_ff", _i), ("vocab", _i), ("t_max", _i),
-        ("n_experts", _i), ("experts_per_tok", _i), ("n_shared", _i), ("moe_gate_sigmoid", _i),
-        ("moe_normalize", _i), ("moe_biased_topk", _i),
-        ("eps", _f),
+        ("eps", _f), ("reserved", _i),
         ("token_emb", _p), ("final_norm", _p), ("w_vocab", _p), ("cos", _p), ("sin", _p),
         ("layers", C.POINTER(OharaLayer)),
     ]
 
 
-class OharaDecodeBuffers(C.Structure):
+class OharaDecodeState(C.Structure):
     _fields_ = [
-        ("batch", _i), ("n_split", _i), ("valid_vocab", _i), ("hist_cap", _i),
+        ("batch", _i), ("rows_cap", _i), ("n_split", _i), ("valid_vocab", _i), ("hist_cap", _i), ("reserved", _i),
         ("ids", _p), ("x", _p), ("q", _p), ("attn", _p), ("act", _p), ("logits", _p),
         ("attn_ws", _p), ("step_state", _p), ("history", _p),
-        ("scratch", _p), ("scratch_bytes", _i64),
+        ("kcache", C.POINTER(_p)), ("vcache", C.POINTER(_p)),
     ]
 
+
+OHARA_LOGITS_NONE, OHARA_LOGITS_LAST, OHARA_LOGITS_ALL = 0, 1, 2
 
 _PROTOS = {
     "ohara_abi_version": (_i, []),
@@ -65,10 +52,11 @@ _PROTOS = {
     "ohara_embed_bf16": (_i, [_p, _p, _p, _i, _i, _i, _p]),
     "ohara_rmsnorm_bf16": (_i, [_p, _p, _p, _i, _i, _f, _p]),
     "ohara_gemm_skinny_bf16": (_i, [_p, _i, _p, _i, _i, _p, _f, _i, _i, _p, _i, _p, _i, _p]),
-    "ohara_qkv_rope_append_bf16": (_i, [_p, _i, _p, _i, _p, _f, _i, _i, _i, _i, _p, _p, _i, _p, _p, _p, _p, _i, _p]),
+    "ohara_qkv_rope_append_bf16": (_i, [_p, _i, _p, _i, _p, _f, _i, _i, _i, _i, _i, _p, _p, _i, _p, _p, _p, _p, _i, _p]),
     "ohara_attn_workspace_bytes": (_i64, [_i, _i, _i, _i, _i]),
-    "ohara_attn_decode_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
+    "ohara_attn_cached_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
     "ohara_argmax_bf16": (_i, [_p, _i, _i, _i, _i, _p, _p, _i, _p, _p]),
+    "ohara_llama_forward": (_i, [C.POINTER(OharaModel), C.POINTER(OharaDecodeState), _i, _i, _i, _i, _i, _p]),
 }
 
 _lib = None

@@ -3,7 +3,7 @@
 // true; scale 1/sqrt(Dh) :116-125; GQA head mapping of repeat_interleave :101-103
 // done by indexing, the expanded K/V are never materialised).
 //
-// Grid (n_split, H_kv, batch).  A workgroup streams its chunk of the context for one
+// Grid (query rows, H_kv, n_split).  A workgroup streams its chunk of the context for one
 // KV head once and serves all G = H/H_kv query heads from it.  Per 16-position tile
 // a wave holds one position per lane-column (16 columns x 4 quarter-rows of Dh), so
 // q.k needs two cross-lane adds; the running max/sum of the online softmax are
@@ -19,8 +19,8 @@ struct AttnArgs {
   const bf16_t* k;   // (Bcap, Tmax, Hkv, D)
   const bf16_t* v;
   bf16_t* out;       // (B, H*D)
-  int B, H, Hkv, D, Tmax, len;
-  const int32_t* pos_dev;  // when set: len = *pos_dev + 1
+  int B, S, H, Hkv, D, Tmax, start;  // query s of sequence b sees positions [0, start + s]
+  const int32_t* pos_dev;            // when set: start = *pos_dev
   int nsplit;
   int* counters;     // (B*Hkv)
   float* part_ml;    // (B, H, nsplit, 2)
@@ -39,7 +39,7 @@ __device__ __forceinline__ float dot8(uint4 a, uint4 b, float s) {
 // Merge the chunk partials of the G heads of (b, kvh) and write bf16 output.
 // Called by all 256 threads of the last workgroup to finish.
 template <int MAXD>
-__device__ void merge_partials(const AttnArgs& a, int b, int kvh, int G) {
+__device__ void merge_partials(const AttnArgs& a, int b /* query row */, int kvh, int G) {
   const int D = a.D;
   for (int idx = threadIdx.x; idx < G * D; idx += blockDim.x) {
     const int hh = idx / D, d = idx - hh * D;
@@ -83,8 +83,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   constexpr int DC = D / 8;         // lanes covering one V row with 16-byte loads
   constexpr int PP = 64 / DC;       // V rows fetched per load instruction
   constexpr int NV = 16 / PP;       // V load instructions per 16-position tile
-  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
-  const int L = a.pos_dev ? min(*a.pos_dev + 1, a.Tmax) : a.len;
+  const int split = blockIdx.z, kvh = blockIdx.y, b = blockIdx.x;  // b: query row = seq * S + s
+  const int seq = b / a.S;
+  const int L = min((a.pos_dev ? *a.pos_dev : a.start) + (b - seq * a.S) + 1, a.Tmax);
   const int chunk = (((L + a.nsplit - 1) / a.nsplit) + 63) & ~63;
   const int t0 = split * chunk;
   const int t1 = min(L, t0 + chunk);
@@ -113,8 +114,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   }
 
   const size_t row = (size_t)a.Hkv * D;
-  const bf16_t* kb = a.k + (size_t)b * a.Tmax * row + (size_t)kvh * D;
-  const bf16_t* vb = a.v + (size_t)b * a.Tmax * row + (size_t)kvh * D;
+  const bf16_t* kb = a.k + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
+  const bf16_t* vb = a.v + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
 
   for (int tb = t0 + wave * 16; tb < t1; tb += 64) {
     const int pos = tb + p;
@@ -194,6 +195,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
       Ls += s_l[w][hh] * sc;
       o += s_acc[w][hh][d] * sc;
     }
+    if (a.nsplit == 1) {  // whole context in this workgroup: no partials
+      a.out[(size_t)b * a.H * D + h * D + d] = f2bf(o / Ls);
+      continue;
+    }
     const size_t pi = (size_t)(b * a.H + h) * a.nsplit + split;
     a.part_acc[pi * D + d] = o;
     if (d == 0) {
@@ -201,15 +206,17 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
       a.part_ml[pi * 2 + 1] = Ls;
     }
   }
+  if (a.nsplit == 1) return;
   if (last_chunk_done(a.counters + b * a.Hkv + kvh, a.nsplit)) merge_partials<D>(a, b, kvh, G);
 }
 
 // Any even head width up to 256, any group size: one thread per position for q.k,
 // one thread per column for p.V.  Slow path for shapes the tuned kernel skips.
 __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
-  const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+  const int split = blockIdx.z, kvh = blockIdx.y, b = blockIdx.x;
+  const int seq = b / a.S;
   const int G = a.H / a.Hkv, D = a.D;
-  const int L = a.pos_dev ? min(*a.pos_dev + 1, a.Tmax) : a.len;
+  const int L = min((a.pos_dev ? *a.pos_dev : a.start) + (b - seq * a.S) + 1, a.Tmax);
   const int chunk = (((L + a.nsplit - 1) / a.nsplit) + 63) & ~63;
   const int t0 = split * chunk;
   const int t1 = min(L, t0 + chunk);
@@ -218,8 +225,8 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
   __shared__ float s_red[4];
   __shared__ float s_q[256];
   const size_t row = (size_t)a.Hkv * D;
-  const bf16_t* kb = a.k + (size_t)b * a.Tmax * row + (size_t)kvh * D;
-  const bf16_t* vb = a.v + (size_t)b * a.Tmax * row + (size_t)kvh * D;
+  const bf16_t* kb = a.k + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
+  const bf16_t* vb = a.v + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
   for (int hh = 0; hh < G; ++hh) {
     const int h = kvh * G + hh;
     __syncthreads();
@@ -256,6 +263,10 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
       }
       __syncthreads();
     }
+    if (a.nsplit == 1) {
+      if (tid < D) a.out[(size_t)b * a.H * D + h * D + tid] = f2bf(acc / l_run);
+      continue;
+    }
     const size_t pi = (size_t)(b * a.H + h) * a.nsplit + split;
     if (tid < D) a.part_acc[pi * D + tid] = acc;
     if (tid == 0) {
@@ -263,6 +274,7 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
       a.part_ml[pi * 2 + 1] = l_run;
     }
   }
+  if (a.nsplit == 1) return;
   if (last_chunk_done(a.counters + b * a.Hkv + kvh, a.nsplit)) merge_partials<256>(a, b, kvh, G);
 }
 
@@ -291,17 +303,21 @@ int64_t ohara_attn_workspace_bytes(int batch, int h, int h_kv, int dh, int n_spl
   return (int64_t)(c + ml + acc);
 }
 
-int ohara_attn_decode_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch, int h,
-                           int h_kv, int dh, int t_max, int len, const int32_t* pos_dev, int n_split,
-                           void* workspace, uint16_t* out, void* stream) {
-  if (!q || !kcache || !vcache || !workspace || !out) return OHARA_EINVAL;
-  if (batch < 1 || h < 1 || h_kv < 1 || h % h_kv || dh < 2 || (dh & 1) || dh > 256) return OHARA_EINVAL;
+int ohara_attn_cached_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch,
+                           int seq_len, int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev,
+                           int n_split, void* workspace, uint16_t* out, void* stream) {
+  if (!q || !kcache || !vcache || !out) return OHARA_EINVAL;
+  if (batch < 1 || seq_len < 1 || h < 1 || h_kv < 1 || h % h_kv || dh < 2 || (dh & 1) || dh > 256)
+    return OHARA_EINVAL;
   if (t_max < 1 || n_split < 1 || n_split > 1024) return OHARA_EINVAL;
-  if (!pos_dev && (len < 1 || len > t_max)) return OHARA_EINVAL;
+  if (n_split > 1 && !workspace) return OHARA_EINVAL;
+  if (!pos_dev && (pos < 0 || pos + seq_len > t_max)) return OHARA_EINVAL;
+  if ((int64_t)batch * seq_len > INT32_MAX / 2 || h_kv > 65535) return OHARA_ESIZE;
   AttnArgs a{};
   a.q = q; a.k = kcache; a.v = vcache; a.out = out;
-  a.B = batch; a.H = h; a.Hkv = h_kv; a.D = dh; a.Tmax = t_max; a.len = len; a.pos_dev = pos_dev;
+  a.B = batch; a.S = seq_len; a.H = h; a.Hkv = h_kv; a.D = dh; a.Tmax = t_max; a.start = pos; a.pos_dev = pos_dev;
   a.nsplit = n_split;
+  batch *= seq_len;  // one workspace slot per query row
   char* ws = reinterpret_cast<char*>(workspace);
   a.counters = reinterpret_cast<int*>(ws);
   ws += align256((size_t)batch * h_kv * sizeof(int));
@@ -309,7 +325,7 @@ int ohara_attn_decode_bf16(const uint16_t* q, const uint16_t* kcache, const uint
   ws += align256((size_t)batch * h * n_split * 2 * sizeof(float));
   a.part_acc = reinterpret_cast<float*>(ws);
   a.scale = 1.0f / sqrtf((float)dh);
-  dim3 grid(n_split, h_kv, batch);
+  dim3 grid(batch, h_kv, n_split);
   hipStream_t st = (hipStream_t)stream;
   const int G = h / h_kv;
   int miss = 1;

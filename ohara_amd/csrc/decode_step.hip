@@ -1,0 +1,61 @@
+// Llama.forward through the KV cache (ohara/models/llama.py:279-323) as a fixed chain
+// of five kernels per layer:
+//   norm1 + QKV projection + rotary + cache append     (Block :199, Attention :84-98)
+//   attention over the cache                           (:100-135)
+//   output projection + residual                       (:142, :199)
+//   norm2 + gate/up projection + SwiGLU                (:200, mlp.py:152)
+//   down projection + residual                         (:200)
+// then final norm + vocabulary projection (:321-322) and, optionally, greedy
+// selection feeding the next step.  No host synchronisation, no allocation: the
+// chain can be captured once into a HIP graph and replayed per token.
+#include "common.h"
+
+extern "C" int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* s, int seq_len, int pos,
+                                   int use_pos_dev, int logits_mode, int select_greedy, void* stream) {
+  if (!m || !s || !m->layers || !s->kcache || !s->vcache) return OHARA_EINVAL;
+  if (s->batch < 1 || seq_len < 1) return OHARA_EINVAL;
+  const int64_t rows64 = (int64_t)s->batch * seq_len;
+  if (rows64 > s->rows_cap) return OHARA_ESIZE;
+  if (use_pos_dev && (!s->step_state || seq_len != 1)) return OHARA_EINVAL;
+  if (!use_pos_dev && (pos < 0 || pos + seq_len > m->t_max)) return OHARA_EINVAL;
+  if (logits_mode < OHARA_LOGITS_NONE || logits_mode > OHARA_LOGITS_ALL) return OHARA_EINVAL;
+  if (select_greedy && !(logits_mode == OHARA_LOGITS_LAST || (logits_mode == OHARA_LOGITS_ALL && seq_len == 1)))
+    return OHARA_EINVAL;
+  const int B = s->batch, R = (int)rows64;
+  const int d = m->d_model, H = m->n_heads, Hkv = m->n_kv_heads, Dh = m->head_dim;
+  const int32_t* pos_dev = use_pos_dev ? s->step_state : nullptr;  // first field is pos
+  const int n_split = seq_len == 1 ? s->n_split : 1;
+  int rc = ohara_embed_bf16(s->ids, m->token_emb, s->x, R, d, m->vocab, stream);
+  if (rc) return rc;
+  for (int l = 0; l < m->n_layers; ++l) {
+    const OharaLayer& L = m->layers[l];
+    rc = ohara_qkv_rope_append_bf16(s->x, d, L.wqkv, d, L.norm1, m->eps, B, seq_len, H, Hkv, Dh, m->cos, m->sin, pos,
+                                    pos_dev, s->q, s->kcache[l], s->vcache[l], m->t_max, stream);
+    if (rc) return rc;
+    rc = ohara_attn_cached_bf16(s->q, s->kcache[l], s->vcache[l], B, seq_len, H, Hkv, Dh, m->t_max, pos, pos_dev,
+                                n_split, s->attn_ws, s->attn, stream);
+    if (rc) return rc;
+    rc = ohara_gemm_skinny_bf16(s->attn, H * Dh, L.wo, d, H * Dh, nullptr, m->eps, R, OHARA_EPI_RESIDUAL, s->x, d,
+                                s->x, d, stream);
+    if (rc) return rc;
+    rc = ohara_gemm_skinny_bf16(s->x, d, L.wgu, m->d_ff, d, L.norm2, m->eps, R, OHARA_EPI_SWIGLU, nullptr, 0, s->act,
+                                m->d_ff, stream);
+    if (rc) return rc;
+    rc = ohara_gemm_skinny_bf16(s->act, m->d_ff, L.wdown, d, m->d_ff, nullptr, m->eps, R, OHARA_EPI_RESIDUAL, s->x, d,
+                                s->x, d, stream);
+    if (rc) return rc;
+  }
+  if (logits_mode == OHARA_LOGITS_ALL) {
+    rc = ohara_gemm_skinny_bf16(s->x, d, m->w_vocab, m->vocab, d, m->final_norm, m->eps, R, OHARA_EPI_STORE, nullptr,
+                                0, s->logits, m->vocab, stream);
+  } else if (logits_mode == OHARA_LOGITS_LAST) {
+    // row b*seq_len + seq_len-1 of x for every sequence: a strided view, no gather
+    rc = ohara_gemm_skinny_bf16(s->x + (size_t)(seq_len - 1) * d, seq_len * d, m->w_vocab, m->vocab, d, m->final_norm,
+                                m->eps, B, OHARA_EPI_STORE, nullptr, 0, s->logits, m->vocab, stream);
+  }
+  if (rc) return rc;
+  if (select_greedy)
+    rc = ohara_argmax_bf16(s->logits, m->vocab, B, m->vocab, s->valid_vocab > 0 ? s->valid_vocab : m->vocab, s->ids,
+                           s->history, s->hist_cap, s->step_state, stream);
+  return rc;
+}

@@ -33,6 +33,7 @@ struct SkinnyArgs {
   int ldr;
   // rotary + append
   int H, Hkv, Dh, Tmax, pos;
+  int S, row0;  // rows are (sequence, position) pairs: row = seq * S + s, position = pos + s
   const int32_t* pos_dev;
   const bf16_t* cos;
   const bf16_t* sin;
@@ -186,7 +187,9 @@ __global__ __launch_bounds__(256) void skinny_kernel(SkinnyArgs a) {
       if (f < a.N) o[0] = f2bf(s0 * y2);
       if (f + 1 < a.N) o[1] = f2bf(s1 * y3);
     } else {  // EPI_ROPE: rows [q (H*Dh); k (Hkv*Dh); v (Hkv*Dh)], one position per sequence
-      const int pos = a.pos_dev ? *a.pos_dev : a.pos;
+      const int grow = a.row0 + b;
+      const int seq = grow / a.S;
+      const int pos = (a.pos_dev ? *a.pos_dev : a.pos) + (grow - seq * a.S);
       const int nq = a.H * a.Dh, nk = a.Hkv * a.Dh;
       if (r0 >= nq + 2 * nk || pos < 0 || pos >= a.Tmax) continue;
       float v[4] = {y0, y1, y2, y3};
@@ -204,14 +207,14 @@ __global__ __launch_bounds__(256) void skinny_kernel(SkinnyArgs a) {
           v[2 * pr + 1] = __fadd_rn(__fmul_rn(e, s), __fmul_rn(od, c));
         }
         if (r0 < nq) {
-          o = a.out + (size_t)b * a.ldo + r0;
+          o = a.out + (size_t)grow * a.ldo + r0;
         } else {
           const int rk = r0 - nq;
-          o = a.kcache + (((size_t)b * a.Tmax + pos) * a.Hkv) * a.Dh + rk;
+          o = a.kcache + (((size_t)seq * a.Tmax + pos) * a.Hkv) * a.Dh + rk;
         }
       } else {
         const int rv = r0 - nq - nk;
-        o = a.vcache + (((size_t)b * a.Tmax + pos) * a.Hkv) * a.Dh + rv;
+        o = a.vcache + (((size_t)seq * a.Tmax + pos) * a.Hkv) * a.Dh + rv;
       }
       *reinterpret_cast<uint2*>(o) = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
     }
@@ -231,14 +234,33 @@ int launch_epi(const SkinnyArgs& a, int epi, int strips, hipStream_t st) {
   return ohara_launch_status();
 }
 
-int launch_skinny(const SkinnyArgs& a, int epi, int packed_rows, hipStream_t st) {
-  const int strips = packed_rows / 16;
+int launch_chunk(const SkinnyArgs& a, int epi, int strips, hipStream_t st) {
   const bool norm = a.norm_w != nullptr;
   const int bt = (a.B + 15) / 16;
   if (bt == 1) return norm ? launch_epi<1, true>(a, epi, strips, st) : launch_epi<1, false>(a, epi, strips, st);
   if (bt == 2) return norm ? launch_epi<2, true>(a, epi, strips, st) : launch_epi<2, false>(a, epi, strips, st);
   if (bt <= 4) return norm ? launch_epi<4, true>(a, epi, strips, st) : launch_epi<4, false>(a, epi, strips, st);
   return OHARA_ESIZE;
+}
+
+// Rows beyond 64 are processed in chunks of 64 (each chunk streams the weights once).
+int launch_skinny(const SkinnyArgs& a0, int epi, int packed_rows, hipStream_t st) {
+  const int strips = packed_rows / 16;
+  const int rows = a0.B;
+  for (int r = 0; r < rows; r += 64) {
+    SkinnyArgs a = a0;
+    a.B = rows - r < 64 ? rows - r : 64;
+    a.x = a0.x + (size_t)r * a0.ldx;
+    if (epi == EPI_ROPE) {
+      a.row0 = r;
+    } else {
+      a.out = a0.out + (size_t)r * a0.ldo;
+      if (a0.resid) a.resid = a0.resid + (size_t)r * a0.ldr;
+    }
+    const int rc = launch_chunk(a, epi, strips, st);
+    if (rc) return rc;
+  }
+  return OHARA_OK;
 }
 
 __global__ void pack_rows_kernel(const bf16_t* w, int n, int k, int ldw, const int32_t* perm, int n_padded,
@@ -298,7 +320,6 @@ int ohara_gemm_skinny_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n
                            float eps, int batch, int epilogue, const uint16_t* resid, int ldr, uint16_t* out,
                            int ldo, void* stream) {
   if (!x || !wp || !out || n < 1 || k < 1 || batch < 1) return OHARA_EINVAL;
-  if (batch > 64) return OHARA_ESIZE;
   if ((k & 7) || (ldx & 7) || ldx < k) return OHARA_EINVAL;  // 16-byte activation loads
   if (epilogue == OHARA_EPI_RESIDUAL && (!resid || ldr < n)) return OHARA_EINVAL;
   if (epilogue < OHARA_EPI_STORE || epilogue > OHARA_EPI_SWIGLU) return OHARA_EINVAL;
@@ -315,18 +336,20 @@ int ohara_gemm_skinny_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n
 }
 
 int ohara_qkv_rope_append_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int k, const uint16_t* norm_w,
-                               float eps, int batch, int h, int h_kv, int dh, const uint16_t* cos,
+                               float eps, int batch, int seq_len, int h, int h_kv, int dh, const uint16_t* cos,
                                const uint16_t* sin, int pos, const int32_t* pos_dev, uint16_t* q_out,
                                uint16_t* kcache, uint16_t* vcache, int t_max, void* stream) {
   if (!x || !wp || !cos || !sin || !q_out || !kcache || !vcache) return OHARA_EINVAL;
-  if (batch < 1 || h < 1 || h_kv < 1 || h % h_kv || dh < 4 || (dh & 3) || t_max < 1) return OHARA_EINVAL;
-  if (batch > 64) return OHARA_ESIZE;
+  if (batch < 1 || seq_len < 1 || h < 1 || h_kv < 1 || h % h_kv || dh < 4 || (dh & 3) || t_max < 1)
+    return OHARA_EINVAL;
   if ((k & 7) || (ldx & 7) || ldx < k) return OHARA_EINVAL;
-  if (!pos_dev && (pos < 0 || pos >= t_max)) return OHARA_EINVAL;
+  if (!pos_dev && (pos < 0 || pos + seq_len > t_max)) return OHARA_EINVAL;
+  if ((int64_t)batch * seq_len > INT32_MAX) return OHARA_ESIZE;
   SkinnyArgs a{};
   a.wp = reinterpret_cast<const uint4*>(wp);
   a.x = x; a.ldx = ldx; a.norm_w = norm_w; a.eps = eps;
-  a.B = batch; a.N = (h + 2 * h_kv) * dh; a.K = k;
+  a.B = batch * seq_len; a.N = (h + 2 * h_kv) * dh; a.K = k;
+  a.S = seq_len; a.row0 = 0;
   a.out = q_out; a.ldo = h * dh;
   a.H = h; a.Hkv = h_kv; a.Dh = dh; a.Tmax = t_max; a.pos = pos; a.pos_dev = pos_dev;
   a.cos = cos; a.sin = sin; a.kcache = kcache; a.vcache = vcache;

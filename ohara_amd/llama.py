@@ -1,0 +1,375 @@
+"""Host-side mirror of ohara's Llama + KVCache for the KV-cache decode path.
+
+Same call surface as the reference (ohara/models/llama.py:16-45,204-348 and
+ohara/modules/kv_cache.py:35-118):
+
+    model = Llama(config, state_dict)              # reference state-dict keys
+    cache = model.build_kv_cache(batch_size)
+    logits = model(tokens, cache, position)        # (B, S, V)
+
+but every tensor operation runs in the HIP kernels of libohara_decode.so.  All
+argument validation happens on the host before any kernel is launched and raises the
+reference's ValueErrors (same messages).
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib, ops
+from ._lib import OharaDecodeState, OharaLayer, OharaModel, check, lib
+
+BF16 = torch.bfloat16
+
+
+@dataclass
+class Config:
+    """Field-for-field the reference's ``Config`` (ohara/models/llama.py:16-45)."""
+
+    vocab_size: int = 65
+    max_sequence_length: int = 64
+    hidden_size: int = 128
+    intermediate_size: int = 256
+    num_attention_heads: int = 4
+    num_key_value_heads: int = 0
+    num_hidden_layers: int = 4
+    dropout: float = 0.2
+    multiple_of: int = 4
+    bias: bool = False
+    weight_tying: bool = False
+    rope_theta: float = 100000
+    init_style: str = "standard"
+    moe_num_experts: int = 0
+    moe_experts_per_tok: int = 2
+    moe_layer_interval: int = 1
+    moe_gate_fn: str = "softmax"
+    moe_quantile_balancing: bool = True
+    moe_grouped: bool = False
+    moe_num_shared_experts: int = 0
+    moe_normalize_weights: bool = True
+
+
+def _validate_config(cfg: Config) -> None:
+    # ohara/models/llama.py:208-241
+    if cfg.vocab_size < 2:
+        raise ValueError("vocab_size must be at least 2")
+    if cfg.hidden_size < 1 or cfg.num_hidden_layers < 1:
+        raise ValueError("hidden_size and num_hidden_layers must be positive")
+    if cfg.intermediate_size < 1:
+        raise ValueError("intermediate_size must be positive")
+    if cfg.num_attention_heads < 1 or cfg.hidden_size % cfg.num_attention_heads != 0:
+        raise ValueError("hidden_size must be divisible by num_attention_heads")
+    if (cfg.hidden_size // cfg.num_attention_heads) % 2 != 0:
+        raise ValueError("attention head dimension must be even for rotary embeddings")
+    if cfg.max_sequence_length < 2:
+        raise ValueError("max_sequence_length must be at least 2")
+    kv = cfg.num_attention_heads if cfg.num_key_value_heads == 0 else cfg.num_key_value_heads
+    if kv < 1 or cfg.num_attention_heads % kv != 0:
+        raise ValueError("num_key_value_heads must divide num_attention_heads")
+    if cfg.bias:
+        raise ValueError("ohara_amd: Linear biases are not supported (the reference default is bias=False)")
+
+
+class KVCache:
+    """ohara/modules/kv_cache.py:35-118 (bf16 storage): (batch, T_max, H_kv, D) key and
+    value tensors written sequentially.  ``forward`` keeps the reference's semantics
+    and error messages for external callers; the model's own path appends inside the
+    fused projection kernel and only does the bookkeeping here (``_reserve``)."""
+
+    def __init__(self, shape, max_seq_length, idx=None, device=None, dtype=None, int8=False):
+        if int8:
+            raise NotImplementedError("ohara_amd: the int8 KV cache mode is not implemented")
+        self.idx = idx
+        self.int8 = False
+        self.max_seq_length = max_seq_length
+        self.length = 0
+        self.batch_size = None
+        self.dtype = dtype
+        self.key = torch.zeros(shape, device=device, dtype=dtype)
+        self.value = torch.zeros(shape, device=device, dtype=dtype)
+
+    def _reserve(self, bsz: int, seq_len: int, start_pos: int) -> int:
+        # ohara/modules/kv_cache.py:80-90, same order
+        if bsz > self.key.size(0):
+            raise ValueError("KV cache batch size is smaller than the input batch")
+        if self.batch_size is not None and bsz != self.batch_size:
+            raise ValueError("KV cache batch size cannot change during decoding")
+        if start_pos != self.length:
+            raise ValueError(
+                f"KV cache writes must be sequential: expected position {self.length}, got {start_pos}"
+            )
+        if start_pos < 0 or start_pos + seq_len > self.max_seq_length:
+            raise ValueError("KV cache position exceeds max_sequence_length")
+        return start_pos + seq_len
+
+    def _commit(self, bsz: int, end: int) -> None:
+        self.length = end
+        self.batch_size = bsz
+
+    def forward(self, keys, values, start_pos):
+        bsz, seq_len = keys.shape[0], keys.shape[1]
+        if values.shape != keys.shape:
+            raise ValueError("KV cache keys and values must have matching shapes")
+        end = self._reserve(bsz, seq_len, start_pos)
+        self.key[:bsz, start_pos:end] = keys
+        self.value[:bsz, start_pos:end] = values
+        self._commit(bsz, end)
+        return self.key[:bsz, :end], self.value[:bsz, :end]
+
+
+def rope_tables(head_dim: int, end: int, theta: float):
+    """precompute_freqs_cis (ohara/embeddings_pos/rotary.py:24-38): fp32 on the host,
+    exactly the reference's operation order, so the bf16-rounded tables match."""
+    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2)[: head_dim // 2].float() / head_dim))
+    ang = torch.outer(torch.arange(end), inv).float()
+    return torch.cos(ang), torch.sin(ang)
+
+
+class _Buffers:
+    """Activation buffers and the C state struct for up to `rows` rows."""
+
+    def __init__(self, model: "Llama", batch: int, rows: int, n_split: int):
+        c, dev = model.config, model.device
+        hd = c.num_attention_heads * model.head_dim
+        self.batch, self.rows, self.n_split = batch, rows, n_split
+        self.ids = torch.zeros(rows, dtype=torch.int64, device=dev)
+        self.x = torch.empty(rows, c.hidden_size, dtype=BF16, device=dev)
+        self.q = torch.empty(rows, hd, dtype=BF16, device=dev)
+        self.attn = torch.empty(rows, hd, dtype=BF16, device=dev)
+        self.act = torch.empty(rows, model.act_width, dtype=BF16, device=dev)
+        self.attn_ws = ops.attn_workspace(batch, c.num_attention_heads, model.kv_heads, model.head_dim, n_split, dev)
+        self.step_state = torch.zeros(4, dtype=torch.int32, device=dev)
+        self.logits = None
+        self.history = None
+
+
+class Llama:
+    """The reference's ``Llama`` call surface (ohara/models/llama.py:204-348) over HIP kernels.
+
+    ``state`` uses the reference's state-dict keys; tensors may live anywhere, they are
+    cast to bf16, moved to ``device`` and repacked once.
+    """
+
+    def __init__(self, config: Config, state: dict, device="cuda", dtype=BF16):
+        _validate_config(config)
+        if dtype != BF16:
+            raise ValueError("ohara_amd runs the decode path in bfloat16 only")
+        if config.moe_num_experts > 0:
+            raise NotImplementedError("MoE layers are served by ohara_amd.moe (not wired into Llama yet)")
+        lib()  # fail loudly now if the HIP library is missing
+        self.config = config
+        self.device = torch.device(device)
+        self.dtype = dtype
+        c = config
+        self.head_dim = c.hidden_size // c.num_attention_heads
+        self.kv_heads = c.num_attention_heads if c.num_key_value_heads == 0 else c.num_key_value_heads
+        self.act_width = c.intermediate_size
+        self.eps = 1e-5
+
+        def dev(t):
+            return t.detach().to(device=self.device, dtype=BF16).contiguous()
+
+        self.token_emb = dev(state["token_emb.weight"])
+        self.final_norm = dev(state["norm.weight"])
+        vocab_w = state["token_emb.weight"] if c.weight_tying else state["vocab_proj.weight"]
+        self.w_vocab = ops.pack_linear(dev(vocab_w))
+        if "freq_cos" in state:
+            cos, sin = state["freq_cos"], state["freq_sin"]
+        else:
+            cos, sin = rope_tables(self.head_dim, c.max_sequence_length * 2, c.rope_theta)
+        self.cos, self.sin = dev(cos), dev(sin)
+        self.layers = []
+        for i in range(c.num_hidden_layers):
+            p = f"layers.{i}."
+            self.layers.append(
+                dict(
+                    wqkv=ops.pack_qkv(dev(state[p + "attn.query.weight"]), dev(state[p + "attn.key.weight"]),
+                                      dev(state[p + "attn.value.weight"])),
+                    wo=ops.pack_linear(dev(state[p + "attn.proj.weight"])),
+                    wgu=ops.pack_gate_up(dev(state[p + "ff.gate.weight"]), dev(state[p + "ff.up.weight"])),
+                    wdown=ops.pack_linear(dev(state[p + "ff.down.weight"])),
+                    norm1=dev(state[p + "norm1.weight"]),
+                    norm2=dev(state[p + "norm2.weight"]),
+                )
+            )
+        torch.cuda.synchronize(self.device)
+        self._c_layers = (OharaLayer * c.num_hidden_layers)()
+        for i, L in enumerate(self.layers):
+            cl = self._c_layers[i]
+            cl.wqkv, cl.wo, cl.wgu, cl.wdown = (L[k].data.data_ptr() for k in ("wqkv", "wo", "wgu", "wdown"))
+            cl.norm1, cl.norm2 = L["norm1"].data_ptr(), L["norm2"].data_ptr()
+        m = OharaModel()
+        m.n_layers, m.d_model, m.n_heads, m.n_kv_heads = c.num_hidden_layers, c.hidden_size, c.num_attention_heads, self.kv_heads
+        m.head_dim, m.d_ff, m.vocab, m.t_max = self.head_dim, c.intermediate_size, c.vocab_size, c.max_sequence_length
+        m.eps = self.eps
+        m.token_emb, m.final_norm, m.w_vocab = self.token_emb.data_ptr(), self.final_norm.data_ptr(), self.w_vocab.data.data_ptr()
+        m.cos, m.sin = self.cos.data_ptr(), self.sin.data_ptr()
+        m.layers = C.cast(self._c_layers, C.POINTER(OharaLayer))
+        self._c_model = m
+        self._buffers: dict = {}
+
+    # -- reference surface -------------------------------------------------------
+
+    def eval(self):
+        return self
+
+    def to(self, *args, **kwargs):
+        return self
+
+    def parameters(self):
+        yield self.token_emb
+        yield self.final_norm
+        yield self.w_vocab.data
+        for L in self.layers:
+            for k in ("wqkv", "wo", "wgu", "wdown"):
+                yield L[k].data
+            yield L["norm1"]
+            yield L["norm2"]
+
+    def build_kv_cache(self, batch_size: int = 1) -> list[KVCache]:
+        """ohara/models/llama.py:325-348."""
+        if batch_size < 1:
+            raise ValueError("batch_size must be at least 1")
+        c = self.config
+        shape = (batch_size, c.max_sequence_length, self.kv_heads, self.head_dim)
+        return [KVCache(shape, c.max_sequence_length, i, device=self.device, dtype=BF16)
+                for i in range(c.num_hidden_layers)]
+
+    def default_n_split(self, batch: int) -> int:
+        """Context chunks per (sequence, KV head) so that decode attention launches about
+        two workgroups per CU; a chunk is never shorter than 64 positions."""
+        want = max(1, 512 // max(1, batch * self.kv_heads))
+        return max(1, min(want, self.config.max_sequence_length // 64, 64))
+
+    def _get_buffers(self, batch: int, rows: int) -> _Buffers:
+        key = (batch, rows)
+        buf = self._buffers.get(key)
+        if buf is None:
+            # keep at most one prefill-sized set alive
+            for k in [k for k in self._buffers if k[1] > k[0] and k != key]:
+                del self._buffers[k]
+            buf = _Buffers(self, batch, rows, self.default_n_split(batch))
+            self._buffers[key] = buf
+        return buf
+
+    def _state_struct(self, buf: _Buffers, kv_cache, logits, history=None, valid_vocab=0) -> OharaDecodeState:
+        n = self.config.num_hidden_layers
+        kc = (C.c_void_p * n)(*[c.key.data_ptr() for c in kv_cache])
+        vc = (C.c_void_p * n)(*[c.value.data_ptr() for c in kv_cache])
+        s = OharaDecodeState()
+        s.batch, s.rows_cap, s.n_split, s.valid_vocab = buf.batch, buf.rows, buf.n_split, valid_vocab
+        s.hist_cap = 0 if history is None else history.shape[0]
+        s.ids, s.x, s.q, s.attn, s.act = (t.data_ptr() for t in (buf.ids, buf.x, buf.q, buf.attn, buf.act))
+        s.logits = 0 if logits is None else logits.data_ptr()
+        s.attn_ws, s.step_state = buf.attn_ws.data_ptr(), buf.step_state.data_ptr()
+        s.history = 0 if history is None else history.data_ptr()
+        s.kcache, s.vcache = C.cast(kc, C.POINTER(C.c_void_p)), C.cast(vc, C.POINTER(C.c_void_p))
+        s._keep = (kc, vc)
+        return s
+
+    def forward(self, x: torch.Tensor, kv_cache: list | None = None, position_ids=None, *, last_only: bool = False):
+        """ohara/models/llama.py:279-323.  Returns logits (B, S, V) in bf16, or (B, 1, V)
+        with ``last_only=True`` (an extension: the generate loops read only the last row)."""
+        c = self.config
+        if x.ndim != 2:
+            raise ValueError("input token IDs must have shape (batch, sequence)")
+        if isinstance(position_ids, torch.Tensor):
+            if position_ids.numel() != 1:
+                raise ValueError("position_ids must be a scalar cache position")
+            position_ids = int(position_ids.item())
+        start_pos = 0
+        if kv_cache is not None:
+            if len(kv_cache) != c.num_hidden_layers:
+                raise ValueError("KV cache must contain one entry per model layer")
+            if position_ids is None or position_ids < 0:
+                raise ValueError("a non-negative position_ids is required with KV cache")
+            start_pos = position_ids
+        elif position_ids is not None:
+            raise ValueError("position_ids is only valid when using a KV cache")
+        B, S = x.shape
+        if S < 1:
+            raise ValueError("input sequence cannot be empty")
+        if start_pos + S > c.max_sequence_length:
+            raise ValueError("input exceeds max_sequence_length")
+        if kv_cache is None:
+            # Uncached causal forward == a fresh cache filled from position 0.
+            kv_cache = self.build_kv_cache(B)
+        ends = [cache._reserve(B, S, start_pos) for cache in kv_cache]
+
+        rows = B * S
+        buf = self._get_buffers(B, rows)
+        buf.ids.copy_(x.reshape(-1).to(device=self.device, dtype=torch.int64))
+        out_rows = B if last_only else rows
+        logits = torch.empty(out_rows, c.vocab_size, dtype=BF16, device=self.device)
+        st = self._state_struct(buf, kv_cache, logits)
+        mode = _lib.OHARA_LOGITS_LAST if last_only else _lib.OHARA_LOGITS_ALL
+        check(lib().ohara_llama_forward(C.byref(self._c_model), C.byref(st), S, start_pos, 0, mode, 0,
+                                        torch.cuda.current_stream().cuda_stream), "llama_forward")
+        for cache, end in zip(kv_cache, ends):
+            cache._commit(B, end)
+        return logits.view(B, 1 if last_only else S, c.vocab_size)
+
+    __call__ = forward
+
+    # -- device-resident greedy loop --------------------------------------------------
+
+    @torch.no_grad()
+    def generate_greedy(self, prompt_ids: torch.Tensor, steps: int, *, use_graph: bool = True,
+                        valid_vocab: int = 0, kv_cache: list | None = None) -> torch.Tensor:
+        """Prefill the prompt, then ``steps`` greedy tokens with no host round trip per
+        token (the loop of ohara/chat_engine.py:395-405 for a batch of equal-length
+        prompts).  Returns the generated ids (B, steps)."""
+        c = self.config
+        B, P = prompt_ids.shape
+        if P < 1:
+            raise ValueError("prompt must encode to at least one token")
+        if P + steps - 1 > c.max_sequence_length - 0 and steps > 0:
+            raise ValueError("input exceeds max_sequence_length")
+        cache = kv_cache if kv_cache is not None else self.build_kv_cache(B)
+        for cc in cache:
+            cc._reserve(B, P, 0)
+        history = torch.zeros(max(steps, 1), B, dtype=torch.int64, device=self.device)
+        stream = torch.cuda.current_stream().cuda_stream
+        # prefill + first token
+        pbuf = self._get_buffers(B, B * P)
+        pbuf.ids.copy_(prompt_ids.reshape(-1).to(device=self.device, dtype=torch.int64))
+        logits = torch.empty(B, c.vocab_size, dtype=BF16, device=self.device)
+        st = self._state_struct(pbuf, cache, logits, valid_vocab=valid_vocab)
+        st.step_state = 0
+        check(lib().ohara_llama_forward(C.byref(self._c_model), C.byref(st), P, 0, 0, _lib.OHARA_LOGITS_LAST, 1, stream),
+              "prefill")
+        for cc in cache:
+            cc._commit(B, P)
+        if steps < 1:
+            return history[:0].t()
+        dbuf = self._get_buffers(B, B)
+        history[0].copy_(pbuf.ids[:B])
+        dbuf.ids.copy_(pbuf.ids[:B])
+        dbuf.step_state.copy_(torch.tensor([P, 1, 0, 0], dtype=torch.int32))
+        dst = self._state_struct(dbuf, cache, logits, history=history, valid_vocab=valid_vocab)
+        self.last_logits = logits
+
+        def one_step():
+            check(lib().ohara_llama_forward(C.byref(self._c_model), C.byref(dst), 1, 0, 1, _lib.OHARA_LOGITS_LAST, 1,
+                                            torch.cuda.current_stream().cuda_stream), "decode step")
+
+        n = steps - 1
+        if n > 0:
+            if use_graph:
+                one_step()  # warm-up outside capture (also produces token 1)
+                n -= 1
+                if n > 0:
+                    g = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(g):
+                        one_step()
+                    for _ in range(n):
+                        g.replay()
+            else:
+                for _ in range(n):
+                    one_step()
+        for cc in cache:
+            cc._commit(B, P + steps - 1)
+        return history[:steps].t().contiguous()

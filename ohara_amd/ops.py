@@ -124,15 +124,17 @@ def gemm_skinny(x, w: PackedLinear, norm_w=None, eps=1e-5, residual=None, out=No
 
 
 def qkv_rope_append(x, wqkv: PackedLinear, norm_w, eps, h, h_kv, dh, cos, sin, pos, kcache, vcache,
-                    q_out=None, pos_dev=None):
+                    q_out=None, pos_dev=None, seq_len=1):
+    """x: (batch*seq_len, K) rows ordered (sequence, position)."""
     _need(x, BF16, "x")
-    b = x.shape[0]
+    rows = x.shape[0]
+    b = rows // seq_len
     if q_out is None:
-        q_out = torch.empty(b, h * dh, dtype=BF16, device=x.device)
+        q_out = torch.empty(rows, h * dh, dtype=BF16, device=x.device)
     t_max = kcache.shape[1]
     check(
         lib().ohara_qkv_rope_append_bf16(
-            _ptr(x), x.stride(0), _ptr(wqkv.data), wqkv.k, _ptr(norm_w), eps, b, h, h_kv, dh, _ptr(cos), _ptr(sin),
+            _ptr(x), x.stride(0), _ptr(wqkv.data), wqkv.k, _ptr(norm_w), eps, b, seq_len, h, h_kv, dh, _ptr(cos), _ptr(sin),
             int(pos), _ptr(pos_dev), _ptr(q_out), _ptr(kcache), _ptr(vcache), t_max, _stream(),
         ),
         "qkv_rope_append",
@@ -147,18 +149,24 @@ def attn_workspace(batch, h, h_kv, dh, n_split, device) -> torch.Tensor:
     return torch.zeros(n, dtype=torch.uint8, device=device)
 
 
-def attn_decode(q, kcache, vcache, h, h_kv, dh, length, n_split, workspace, out=None, pos_dev=None):
-    b = q.shape[0]
+def attn_cached(q, kcache, vcache, h, h_kv, dh, pos, n_split, workspace, out=None, pos_dev=None, seq_len=1):
+    """q: (batch*seq_len, h*dh); query s of a sequence sits at cache position pos + s."""
+    rows = q.shape[0]
     if out is None:
-        out = torch.empty(b, h * dh, dtype=BF16, device=q.device)
+        out = torch.empty(rows, h * dh, dtype=BF16, device=q.device)
     check(
-        lib().ohara_attn_decode_bf16(
-            _ptr(q), _ptr(kcache), _ptr(vcache), b, h, h_kv, dh, kcache.shape[1], int(length), _ptr(pos_dev),
-            n_split, _ptr(workspace), _ptr(out), _stream(),
+        lib().ohara_attn_cached_bf16(
+            _ptr(q), _ptr(kcache), _ptr(vcache), rows // seq_len, seq_len, h, h_kv, dh, kcache.shape[1], int(pos),
+            _ptr(pos_dev), n_split, _ptr(workspace), _ptr(out), _stream(),
         ),
-        "attn_decode",
+        "attn_cached",
     )
     return out
+
+
+def attn_decode(q, kcache, vcache, h, h_kv, dh, length, n_split, workspace, out=None, pos_dev=None):
+    """Decode case: one query per sequence seeing `length` cached positions."""
+    return attn_cached(q, kcache, vcache, h, h_kv, dh, length - 1, n_split, workspace, out, pos_dev, 1)
 
 
 def argmax(logits: torch.Tensor, valid_vocab: int | None = None, next_ids=None, history=None, step_state=None):
