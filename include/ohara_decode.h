@@ -157,7 +157,10 @@ typedef struct OharaDecodeState {
   int32_t rows_cap;      /* rows (batch*seq_len) the activation buffers below can hold    */
   int32_t n_split;       /* context chunks of decode attention (seq_len == 1)             */
   int32_t valid_vocab;   /* ids >= this are never selected; 0 = whole vocabulary          */
-  int32_t hist_cap, reserved;
+  int32_t hist_cap;
+  int32_t prof_kernel;   /* -1: off; else index of the launch (0 = embedding, 1 + 5*l + i = i-th
+                            kernel of layer l, 1 + 5*n_layers = vocabulary projection, then the
+                            selection) to bracket with prof_start / prof_stop                    */
   int64_t* ids;          /* (rows) tokens fed; ids[0:batch] overwritten by greedy select  */
   uint16_t* x;           /* (rows, d) residual stream                                     */
   uint16_t* q;           /* (rows, h*dh)                                                  */
@@ -169,6 +172,8 @@ typedef struct OharaDecodeState {
   int64_t* history;      /* (hist_cap, batch) generated ids, may be NULL                  */
   uint16_t* const* kcache; /* host array [n_layers] of (batch_cap, t_max, h_kv, dh)       */
   uint16_t* const* vcache;
+  void* prof_start;      /* hipEvent_t recorded on `stream` right before launch prof_kernel */
+  void* prof_stop;       /* hipEvent_t recorded right after it                             */
 } OharaDecodeState;
 
 #define OHARA_LOGITS_NONE 0
@@ -180,6 +185,41 @@ typedef struct OharaDecodeState {
  * select_greedy != 0 (needs logits_mode LAST or seq_len == 1) appends the argmax. */
 int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* s, int seq_len, int pos, int use_pos_dev,
                         int logits_mode, int select_greedy, void* stream);
+
+/* ---- one decode step as ONE persistent launch (batch <= 16) ------------------------
+ * Same result as ohara_llama_forward(seq_len = 1, use_pos_dev = 1, LOGITS_LAST) but the
+ * whole step (all layers, vocabulary projection, greedy selection) runs in a single
+ * kernel of `n_workgroups` resident workgroups (use the CU count) separated by
+ * grid-wide barriers; it has no counterpart in the reference, whose decode step is
+ * ~1000 eager launches (llama.py:279-323).  The cache position and step index are read
+ * from / advanced in s->step_state; s->attn and s->attn_ws are not used.
+ * `workspace`: ohara_persistent_workspace_bytes(m, batch, s->n_split, n_workgroups) of
+ * device memory.  Call once with init_workspace = 1 (copies the layer table and the
+ * cache pointers to the device, zeroes the barrier words; synchronises the stream; do
+ * it outside graph capture) whenever the model or the caches change; then each call
+ * with init_workspace = 0 enqueues one step.  spin_limit bounds every barrier wait
+ * (0 = default); if a wait expires the kernel still drains and the error word reads
+ * non-zero.  s->n_split must be 16.
+ * Requires head_dim 64 or 128, n_heads / n_kv_heads in {1, 2, 4}, d_model <= 1024,
+ * d_model and d_ff multiples of 8. */
+int64_t ohara_persistent_workspace_bytes(const OharaModel* m, int batch, int n_split, int n_workgroups);
+int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s, void* workspace, int n_workgroups,
+                                  int init_workspace, int select_greedy, unsigned int spin_limit, void* stream);
+/* Byte offsets inside the workspace: the barrier words; the sticky error word (uint32,
+ * non-zero after a barrier wait expired); 512 x uint64 shader-clock samples taken by
+ * workgroup 0 at every phase boundary when s->prof_kernel == -2 (measurement only). */
+int64_t ohara_persistent_barrier_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
+int64_t ohara_persistent_error_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
+int64_t ohara_persistent_profile_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
+
+/* ---- timing helpers (measurement only; no counterpart in the reference) -----------
+ * Thin wrappers over hipEventCreate / hipEventDestroy / hipEventElapsedTime so that a
+ * benchmark can time single launches on the stream they run on without another HIP
+ * binding.  elapsed needs both events completed (synchronise the stream first). */
+int ohara_event_create(void** event);
+int ohara_event_destroy(void* event);
+int ohara_event_record(void* event, void* stream);
+int ohara_event_elapsed_ms(void* start, void* stop, float* ms);
 
 #ifdef __cplusplus
 }

@@ -36,10 +36,11 @@ class OharaModel(C.Structure):
 
 class OharaDecodeState(C.Structure):
     _fields_ = [
-        ("batch", _i), ("rows_cap", _i), ("n_split", _i), ("valid_vocab", _i), ("hist_cap", _i), ("reserved", _i),
+        ("batch", _i), ("rows_cap", _i), ("n_split", _i), ("valid_vocab", _i), ("hist_cap", _i), ("prof_kernel", _i),
         ("ids", _p), ("x", _p), ("q", _p), ("attn", _p), ("act", _p), ("logits", _p),
         ("attn_ws", _p), ("step_state", _p), ("history", _p),
         ("kcache", C.POINTER(_p)), ("vcache", C.POINTER(_p)),
+        ("prof_start", _p), ("prof_stop", _p),
     ]
 
 
@@ -57,6 +58,16 @@ _PROTOS = {
     "ohara_attn_cached_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
     "ohara_argmax_bf16": (_i, [_p, _i, _i, _i, _i, _p, _p, _i, _p, _p]),
     "ohara_llama_forward": (_i, [C.POINTER(OharaModel), C.POINTER(OharaDecodeState), _i, _i, _i, _i, _i, _p]),
+    "ohara_persistent_workspace_bytes": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),
+    "ohara_persistent_barrier_offset": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),
+    "ohara_persistent_error_offset": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),
+    "ohara_persistent_profile_offset": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),
+    "ohara_llama_decode_persistent": (_i, [C.POINTER(OharaModel), C.POINTER(OharaDecodeState), _p, _i, _i, _i,
+                                           C.c_uint, _p]),
+    "ohara_event_create": (_i, [C.POINTER(_p)]),
+    "ohara_event_destroy": (_i, [_p]),
+    "ohara_event_record": (_i, [_p, _p]),
+    "ohara_event_elapsed_ms": (_i, [_p, _p, C.POINTER(_f)]),
 }
 
 _lib = None

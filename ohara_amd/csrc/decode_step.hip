@@ -25,37 +25,63 @@ extern "C" int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* 
   const int d = m->d_model, H = m->n_heads, Hkv = m->n_kv_heads, Dh = m->head_dim;
   const int32_t* pos_dev = use_pos_dev ? s->step_state : nullptr;  // first field is pos
   const int n_split = seq_len == 1 ? s->n_split : 1;
-  int rc = ohara_embed_bf16(s->ids, m->token_emb, s->x, R, d, m->vocab, stream);
-  if (rc) return rc;
+  hipStream_t hs = (hipStream_t)stream;
+  int launch = 0;
+  // Brackets launch number s->prof_kernel with the caller's events.
+#define OHARA_RUN(call)                                                                     \
+  do {                                                                                      \
+    const bool prof_ = (launch == s->prof_kernel) && s->prof_start && s->prof_stop;         \
+    if (prof_) (void)hipEventRecord((hipEvent_t)s->prof_start, hs);                         \
+    rc = (call);                                                                            \
+    if (prof_) (void)hipEventRecord((hipEvent_t)s->prof_stop, hs);                          \
+    ++launch;                                                                               \
+    if (rc) return rc;                                                                      \
+  } while (0)
+  int rc = 0;
+  OHARA_RUN(ohara_embed_bf16(s->ids, m->token_emb, s->x, R, d, m->vocab, stream));
   for (int l = 0; l < m->n_layers; ++l) {
     const OharaLayer& L = m->layers[l];
-    rc = ohara_qkv_rope_append_bf16(s->x, d, L.wqkv, d, L.norm1, m->eps, B, seq_len, H, Hkv, Dh, m->cos, m->sin, pos,
-                                    pos_dev, s->q, s->kcache[l], s->vcache[l], m->t_max, stream);
-    if (rc) return rc;
-    rc = ohara_attn_cached_bf16(s->q, s->kcache[l], s->vcache[l], B, seq_len, H, Hkv, Dh, m->t_max, pos, pos_dev,
-                                n_split, s->attn_ws, s->attn, stream);
-    if (rc) return rc;
-    rc = ohara_gemm_skinny_bf16(s->attn, H * Dh, L.wo, d, H * Dh, nullptr, m->eps, R, OHARA_EPI_RESIDUAL, s->x, d,
-                                s->x, d, stream);
-    if (rc) return rc;
-    rc = ohara_gemm_skinny_bf16(s->x, d, L.wgu, m->d_ff, d, L.norm2, m->eps, R, OHARA_EPI_SWIGLU, nullptr, 0, s->act,
-                                m->d_ff, stream);
-    if (rc) return rc;
-    rc = ohara_gemm_skinny_bf16(s->act, m->d_ff, L.wdown, d, m->d_ff, nullptr, m->eps, R, OHARA_EPI_RESIDUAL, s->x, d,
-                                s->x, d, stream);
-    if (rc) return rc;
+    OHARA_RUN(ohara_qkv_rope_append_bf16(s->x, d, L.wqkv, d, L.norm1, m->eps, B, seq_len, H, Hkv, Dh, m->cos, m->sin, pos,
+                                    pos_dev, s->q, s->kcache[l], s->vcache[l], m->t_max, stream));
+    OHARA_RUN(ohara_attn_cached_bf16(s->q, s->kcache[l], s->vcache[l], B, seq_len, H, Hkv, Dh, m->t_max, pos, pos_dev,
+                                n_split, s->attn_ws, s->attn, stream));
+    OHARA_RUN(ohara_gemm_skinny_bf16(s->attn, H * Dh, L.wo, d, H * Dh, nullptr, m->eps, R, OHARA_EPI_RESIDUAL, s->x, d,
+                                s->x, d, stream));
+    OHARA_RUN(ohara_gemm_skinny_bf16(s->x, d, L.wgu, m->d_ff, d, L.norm2, m->eps, R, OHARA_EPI_SWIGLU, nullptr, 0, s->act,
+                                m->d_ff, stream));
+    OHARA_RUN(ohara_gemm_skinny_bf16(s->act, m->d_ff, L.wdown, d, m->d_ff, nullptr, m->eps, R, OHARA_EPI_RESIDUAL, s->x, d,
+                                s->x, d, stream));
   }
   if (logits_mode == OHARA_LOGITS_ALL) {
-    rc = ohara_gemm_skinny_bf16(s->x, d, m->w_vocab, m->vocab, d, m->final_norm, m->eps, R, OHARA_EPI_STORE, nullptr,
-                                0, s->logits, m->vocab, stream);
+    OHARA_RUN(ohara_gemm_skinny_bf16(s->x, d, m->w_vocab, m->vocab, d, m->final_norm, m->eps, R, OHARA_EPI_STORE,
+                                     nullptr, 0, s->logits, m->vocab, stream));
   } else if (logits_mode == OHARA_LOGITS_LAST) {
     // row b*seq_len + seq_len-1 of x for every sequence: a strided view, no gather
-    rc = ohara_gemm_skinny_bf16(s->x + (size_t)(seq_len - 1) * d, seq_len * d, m->w_vocab, m->vocab, d, m->final_norm,
-                                m->eps, B, OHARA_EPI_STORE, nullptr, 0, s->logits, m->vocab, stream);
+    OHARA_RUN(ohara_gemm_skinny_bf16(s->x + (size_t)(seq_len - 1) * d, seq_len * d, m->w_vocab, m->vocab, d,
+                                     m->final_norm, m->eps, B, OHARA_EPI_STORE, nullptr, 0, s->logits, m->vocab,
+                                     stream));
   }
-  if (rc) return rc;
   if (select_greedy)
-    rc = ohara_argmax_bf16(s->logits, m->vocab, B, m->vocab, s->valid_vocab > 0 ? s->valid_vocab : m->vocab, s->ids,
-                           s->history, s->hist_cap, s->step_state, stream);
-  return rc;
+    OHARA_RUN(ohara_argmax_bf16(s->logits, m->vocab, B, m->vocab, s->valid_vocab > 0 ? s->valid_vocab : m->vocab,
+                                s->ids, s->history, s->hist_cap, s->step_state, stream));
+#undef OHARA_RUN
+  return OHARA_OK;
+}
+
+extern "C" int ohara_event_create(void** event) {
+  if (!event) return OHARA_EINVAL;
+  hipEvent_t e;
+  if (hipEventCreate(&e) != hipSuccess) return OHARA_ELAUNCH;
+  *event = e;
+  return OHARA_OK;
+}
+extern "C" int ohara_event_destroy(void* event) {
+  return hipEventDestroy((hipEvent_t)event) == hipSuccess ? OHARA_OK : OHARA_ELAUNCH;
+}
+extern "C" int ohara_event_record(void* event, void* stream) {
+  return hipEventRecord((hipEvent_t)event, (hipStream_t)stream) == hipSuccess ? OHARA_OK : OHARA_ELAUNCH;
+}
+extern "C" int ohara_event_elapsed_ms(void* start, void* stop, float* ms) {
+  if (!ms) return OHARA_EINVAL;
+  return hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop) == hipSuccess ? OHARA_OK : OHARA_ELAUNCH;
 }

@@ -262,6 +262,7 @@ class Llama:
         s = OharaDecodeState()
         s.batch, s.rows_cap, s.n_split, s.valid_vocab = buf.batch, buf.rows, buf.n_split, valid_vocab
         s.hist_cap = 0 if history is None else history.shape[0]
+        s.prof_kernel = -1
         s.ids, s.x, s.q, s.attn, s.act = (t.data_ptr() for t in (buf.ids, buf.x, buf.q, buf.attn, buf.act))
         s.logits = 0 if logits is None else logits.data_ptr()
         s.attn_ws, s.step_state = buf.attn_ws.data_ptr(), buf.step_state.data_ptr()
@@ -316,60 +317,187 @@ class Llama:
 
     # -- device-resident greedy loop --------------------------------------------------
 
+    def session(self, batch: int, max_new_tokens: int, valid_vocab: int = 0, kv_cache: list | None = None,
+                persistent: bool | None = None):
+        return DecodeSession(self, batch, max_new_tokens, valid_vocab, kv_cache, persistent)
+
+    def supports_persistent(self, batch: int) -> bool:
+        """Shapes the single-launch decode kernel covers."""
+        c = self.config
+        g = c.num_attention_heads // self.kv_heads
+        return (batch <= 16 and self.head_dim in (64, 128) and g in (1, 2, 4) and c.hidden_size <= 1024
+                and c.hidden_size % 8 == 0 and c.intermediate_size % 8 == 0)
+
     @torch.no_grad()
     def generate_greedy(self, prompt_ids: torch.Tensor, steps: int, *, use_graph: bool = True,
-                        valid_vocab: int = 0, kv_cache: list | None = None) -> torch.Tensor:
+                        valid_vocab: int = 0, kv_cache: list | None = None,
+                        persistent: bool | None = None) -> torch.Tensor:
         """Prefill the prompt, then ``steps`` greedy tokens with no host round trip per
         token (the loop of ohara/chat_engine.py:395-405 for a batch of equal-length
         prompts).  Returns the generated ids (B, steps)."""
-        c = self.config
         B, P = prompt_ids.shape
-        if P < 1:
-            raise ValueError("prompt must encode to at least one token")
-        if P + steps - 1 > c.max_sequence_length - 0 and steps > 0:
-            raise ValueError("input exceeds max_sequence_length")
-        cache = kv_cache if kv_cache is not None else self.build_kv_cache(B)
-        for cc in cache:
-            cc._reserve(B, P, 0)
-        history = torch.zeros(max(steps, 1), B, dtype=torch.int64, device=self.device)
-        stream = torch.cuda.current_stream().cuda_stream
-        # prefill + first token
-        pbuf = self._get_buffers(B, B * P)
-        pbuf.ids.copy_(prompt_ids.reshape(-1).to(device=self.device, dtype=torch.int64))
-        logits = torch.empty(B, c.vocab_size, dtype=BF16, device=self.device)
-        st = self._state_struct(pbuf, cache, logits, valid_vocab=valid_vocab)
-        st.step_state = 0
-        check(lib().ohara_llama_forward(C.byref(self._c_model), C.byref(st), P, 0, 0, _lib.OHARA_LOGITS_LAST, 1, stream),
-              "prefill")
-        for cc in cache:
-            cc._commit(B, P)
         if steps < 1:
-            return history[:0].t()
-        dbuf = self._get_buffers(B, B)
-        history[0].copy_(pbuf.ids[:B])
+            return torch.zeros(B, 0, dtype=torch.int64, device=self.device)
+        sess = self.session(B, steps, valid_vocab, kv_cache, persistent)
+        sess.prefill(prompt_ids)
+        sess.run(steps - 1, use_graph=use_graph)
+        return sess.tokens()
+
+
+class DecodeSession:
+    """One batch of equal-length sequences decoded greedily on the device: prefill once,
+    then one ``ohara_llama_forward`` (S = 1, device-side position, fused selection) per
+    token, replayed from a HIP graph.  The host reads tokens only when it asks for them."""
+
+    PERSISTENT_SPLITS = 16
+
+    def __init__(self, model: Llama, batch: int, max_new_tokens: int, valid_vocab: int = 0, kv_cache=None,
+                 persistent: bool | None = None):
+        self.model, self.batch = model, batch
+        if persistent is None:
+            persistent = model.supports_persistent(batch)
+        elif persistent and not model.supports_persistent(batch):
+            raise ValueError("the persistent decode kernel does not cover this shape")
+        self.persistent = persistent
+        self._pws = None
+        self.cache = kv_cache if kv_cache is not None else model.build_kv_cache(batch)
+        self.valid_vocab = valid_vocab
+        self.history = torch.zeros(max(max_new_tokens, 1), batch, dtype=torch.int64, device=model.device)
+        self.logits = torch.empty(batch, model.config.vocab_size, dtype=BF16, device=model.device)
+        self.produced = 0
+        self.pos = 0
+        self.graph = None
+        self._dst = None
+
+    def prefill(self, prompt_ids: torch.Tensor) -> None:
+        m, B = self.model, self.batch
+        if prompt_ids.ndim != 2 or prompt_ids.shape[0] != B:
+            raise ValueError("input token IDs must have shape (batch, sequence)")
+        P = prompt_ids.shape[1]
+        if P < 1:
+            raise ValueError("input sequence cannot be empty")
+        if P > m.config.max_sequence_length:
+            raise ValueError("input exceeds max_sequence_length")
+        for cc in self.cache:
+            cc._reserve(B, P, 0)
+        pbuf = m._get_buffers(B, B * P)
+        pbuf.ids.copy_(prompt_ids.reshape(-1).to(device=m.device, dtype=torch.int64))
+        st = m._state_struct(pbuf, self.cache, self.logits, valid_vocab=self.valid_vocab)
+        st.step_state = 0
+        check(lib().ohara_llama_forward(C.byref(m._c_model), C.byref(st), P, 0, 0, _lib.OHARA_LOGITS_LAST, 1,
+                                        torch.cuda.current_stream().cuda_stream), "prefill")
+        for cc in self.cache:
+            cc._commit(B, P)
+        self.pos = P
+        dbuf = m._get_buffers(B, B)
+        self.history[0].copy_(pbuf.ids[:B])
         dbuf.ids.copy_(pbuf.ids[:B])
         dbuf.step_state.copy_(torch.tensor([P, 1, 0, 0], dtype=torch.int32))
-        dst = self._state_struct(dbuf, cache, logits, history=history, valid_vocab=valid_vocab)
-        self.last_logits = logits
+        self.produced = 1
+        self._dbuf = dbuf
+        self._dst = m._state_struct(dbuf, self.cache, self.logits, history=self.history, valid_vocab=self.valid_vocab)
+        self.graph = None
+        if self.persistent:
+            self._dst.n_split = self.PERSISTENT_SPLITS
+            self._nwg = torch.cuda.get_device_properties(m.device).multi_processor_count
+            nbytes = lib().ohara_persistent_workspace_bytes(C.byref(m._c_model), B, self.PERSISTENT_SPLITS, self._nwg)
+            if nbytes < 0:
+                raise RuntimeError("persistent workspace query failed")
+            if self._pws is None or self._pws.numel() < nbytes:
+                self._pws = torch.zeros(nbytes, dtype=torch.uint8, device=m.device)
+            self._err_off = lib().ohara_persistent_error_offset(C.byref(m._c_model), B, self.PERSISTENT_SPLITS,
+                                                                self._nwg)
+            self._prof_off = lib().ohara_persistent_profile_offset(C.byref(m._c_model), B, self.PERSISTENT_SPLITS,
+                                                                   self._nwg)
+            torch.cuda.current_stream().synchronize()
+            check(lib().ohara_llama_decode_persistent(C.byref(m._c_model), C.byref(self._dst), self._pws.data_ptr(),
+                                                      self._nwg, 1, 1, 0, torch.cuda.current_stream().cuda_stream),
+                  "persistent init")
 
-        def one_step():
-            check(lib().ohara_llama_forward(C.byref(self._c_model), C.byref(dst), 1, 0, 1, _lib.OHARA_LOGITS_LAST, 1,
-                                            torch.cuda.current_stream().cuda_stream), "decode step")
+    def _launch_step(self) -> None:
+        m = self.model
+        stream = torch.cuda.current_stream().cuda_stream
+        if self.persistent:
+            check(lib().ohara_llama_decode_persistent(C.byref(m._c_model), C.byref(self._dst), self._pws.data_ptr(),
+                                                      self._nwg, 0, 1, 0, stream), "persistent decode step")
+        else:
+            check(lib().ohara_llama_forward(C.byref(m._c_model), C.byref(self._dst), 1, 0, 1, _lib.OHARA_LOGITS_LAST, 1,
+                                            stream), "decode step")
 
-        n = steps - 1
-        if n > 0:
-            if use_graph:
-                one_step()  # warm-up outside capture (also produces token 1)
-                n -= 1
-                if n > 0:
-                    g = torch.cuda.CUDAGraph()
-                    with torch.cuda.graph(g):
-                        one_step()
-                    for _ in range(n):
-                        g.replay()
-            else:
-                for _ in range(n):
-                    one_step()
-        for cc in cache:
-            cc._commit(B, P + steps - 1)
-        return history[:steps].t().contiguous()
+    def check_error(self) -> None:
+        """Raise if a barrier wait of the persistent kernel expired (synchronises)."""
+        if self.persistent and self._pws is not None:
+            word = self._pws[self._err_off : self._err_off + 4].view(torch.int32).cpu()
+            if int(word[0]) != 0:
+                raise RuntimeError("persistent decode kernel: a grid barrier wait expired")
+
+    def phase_clocks(self) -> torch.Tensor:
+        """Shader-clock samples of workgroup 0 at the phase boundaries of the last step run
+        with ``step(prof_kernel=-2)`` (measurement aid)."""
+        return self._pws[self._prof_off : self._prof_off + 4096].view(torch.int64).cpu()
+
+    def _room(self, n: int) -> None:
+        if self._dst is None:
+            raise RuntimeError("prefill first")
+        if self.pos + n > self.model.config.max_sequence_length:
+            raise ValueError("input exceeds max_sequence_length")
+        if self.produced + n > self.history.shape[0]:
+            raise ValueError("max_new_tokens exceeded")
+
+    def step(self, prof_kernel: int = -1, prof_start=None, prof_stop=None) -> None:
+        """One eager decode step (enqueue only)."""
+        self._room(1)
+        stream = torch.cuda.current_stream().cuda_stream
+        if self.persistent:
+            # a single launch: bracket it directly
+            if prof_start is not None:
+                check(lib().ohara_event_record(prof_start, stream), "event record")
+            self._dst.prof_kernel = -2 if prof_kernel == -2 else -1
+            self._launch_step()
+            self._dst.prof_kernel = -1
+            if prof_stop is not None:
+                check(lib().ohara_event_record(prof_stop, stream), "event record")
+        else:
+            self._dst.prof_kernel = prof_kernel
+            self._dst.prof_start, self._dst.prof_stop = prof_start, prof_stop
+            self._launch_step()
+            self._dst.prof_kernel = -1
+        self._advance(1)
+
+    def _advance(self, n: int) -> None:
+        self.pos += n
+        self.produced += n
+        for cc in self.cache:
+            cc._commit(self.batch, self.pos)
+
+    def capture(self) -> None:
+        """Record one decode step into a HIP graph (after one eager warm-up step)."""
+        if self.graph is not None:
+            return
+        self.step()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self._launch_step()
+        self.graph = g
+
+    def run(self, n: int, use_graph: bool = True) -> None:
+        """Enqueue n more decode steps."""
+        if n <= 0:
+            return
+        if not use_graph:
+            for _ in range(n):
+                self.step()
+            return
+        if self.graph is None:
+            self.capture()
+            n -= 1
+        self._room(n)
+        for _ in range(n):
+            self.graph.replay()
+        self._advance(n)
+
+    def tokens(self) -> torch.Tensor:
+        """(B, produced) generated ids (synchronises)."""
+        out = self.history[: self.produced].t().contiguous()
+        self.check_error()
+        return out

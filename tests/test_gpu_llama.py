@@ -173,6 +173,17 @@ def test_greedy_small_model(cuda):
     got, want, nd = _check_greedy(model, ref, prompt, 64, cuda, max_rel=4e-2, mean_rel=4e-3)
     eager = model.generate_greedy(prompt.to(cuda), 64, use_graph=False).cpu()
     assert torch.equal(eager, got), "graph replay and eager launches must agree bit for bit"
+    # the kernel-per-op chain and the single persistent launch both satisfy the oracle
+    assert model.supports_persistent(3)
+    chain = model.generate_greedy(prompt.to(cuda), 64, persistent=False).cpu()
+    chain_eager = model.generate_greedy(prompt.to(cuda), 64, persistent=False, use_graph=False).cpu()
+    assert torch.equal(chain, chain_eager)
+    for b in range(3):
+        neq = (chain[b] != want[b]).nonzero()
+        if neq.numel():
+            t = int(neq[0])
+            wl = greedy_decode_ref(ref, prompt, t + 1, return_logits=True)[1]
+            assert _near_tie(wl[t, b], int(chain[b, t]), int(want[b, t]))
 
 
 def _accumulation_noise_floor(rcfg, w, prompt):
