@@ -206,7 +206,7 @@ int64_t ohara_persistent_workspace_bytes(const OharaModel* m, int batch, int n_s
 int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s, void* workspace, int n_workgroups,
                                   int init_workspace, int select_greedy, unsigned int spin_limit, void* stream);
 /* Byte offsets inside the workspace: the barrier words; the sticky error word (uint32,
- * non-zero after a barrier wait expired); 512 x uint64 shader-clock samples taken by
+ * non-zero after a barrier wait expired); 1024 x uint64 shader-clock samples taken by
  * workgroup 0 at every phase boundary when s->prof_kernel == -2 (measurement only). */
 int64_t ohara_persistent_barrier_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
 int64_t ohara_persistent_error_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);

@@ -37,24 +37,41 @@ __device__ __forceinline__ float dot8(uint4 a, uint4 b, float s) {
 }
 
 // Merge the chunk partials of the G heads of (b, kvh) and write bf16 output.
-// Called by all 256 threads of the last workgroup to finish.
+// Called by all 256 threads of the last workgroup to finish.  The partial loads are
+// issued eight chunks at a time before any is consumed (a dependent chain of global
+// loads costs about a microsecond per link on this chip).
 template <int MAXD>
 __device__ void merge_partials(const AttnArgs& a, int b /* query row */, int kvh, int G) {
-  const int D = a.D;
+  const int D = a.D, ns = a.nsplit;
   for (int idx = threadIdx.x; idx < G * D; idx += blockDim.x) {
     const int hh = idx / D, d = idx - hh * D;
     const int h = kvh * G + hh;
-    const float* ml = a.part_ml + ((size_t)(b * a.H + h) * a.nsplit) * 2;
-    const float* pa = a.part_acc + ((size_t)(b * a.H + h) * a.nsplit) * D + d;
+    const float* ml = a.part_ml + ((size_t)(b * a.H + h) * ns) * 2;
+    const float* pa = a.part_acc + ((size_t)(b * a.H + h) * ns) * D + d;
     float M = -INFINITY;
-    for (int s = 0; s < a.nsplit; ++s) M = fmaxf(M, ml[2 * s]);
+    for (int s0 = 0; s0 < ns; s0 += 8) {
+      float mv[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) mv[i] = (s0 + i < ns) ? ml[2 * (s0 + i)] : -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) M = fmaxf(M, mv[i]);
+    }
     float Lsum = 0.f, o = 0.f;
-    for (int s = 0; s < a.nsplit; ++s) {
-      const float ms = ml[2 * s];
-      if (ms == -INFINITY) continue;
-      const float w = __expf(ms - M);
-      Lsum += ml[2 * s + 1] * w;
-      o += pa[(size_t)s * D] * w;
+    for (int s0 = 0; s0 < ns; s0 += 8) {
+      float mv[8], lv[8], av[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const bool in = s0 + i < ns;
+        mv[i] = in ? ml[2 * (s0 + i)] : -INFINITY;
+        lv[i] = in ? ml[2 * (s0 + i) + 1] : 0.f;
+        av[i] = in ? pa[(size_t)(s0 + i) * D] : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float w = (mv[i] == -INFINITY) ? 0.f : __expf(mv[i] - M);
+        Lsum += lv[i] * w;
+        o += av[i] * w;
+      }
     }
     a.out[(size_t)b * a.H * D + h * D + d] = f2bf(o / Lsum);
   }

@@ -4,8 +4,7 @@
 // Why: at batch 1 a layer streams only ~19 MB, so a chain of five kernels per layer
 // spends its time in launch and drain latency, not in HBM.  Here the whole chip stays
 // resident (one workgroup per CU) and walks the same five phases per layer, separated by
-// a grid-wide barrier (a device-scope counter), each phase spreading its work over all
-// workgroups:
+// a grid-wide barrier, each phase spreading its work over all workgroups:
 //   P1  [embedding] + norm1 + QKV projection + rotary + cache append
 //   P2  attention over the cache, split along the context, partial (max,sum,acc) triples
 //   P3  merge of the partials + output projection + residual
@@ -14,24 +13,43 @@
 // then final norm + vocabulary projection with a running arg-max per workgroup, and the
 // selection of the next token.  Rounding points are those of the unfused kernels.
 //
-// Every barrier wait is bounded: a workgroup that spins longer than the limit raises the
-// error flag and moves on, so the grid always drains.
+// Cross-workgroup data ("mailboxes").  The eight XCDs have private L2s, so a phase's
+// outputs must reach memory before the barrier and must not be served from a stale cache
+// line after it.  An L2 write-back / invalidate per barrier costs ~1.7 us each on this
+// chip - more than the barrier - so instead:
+//   * producers write with device-scope (sc1, write-through) stores and wait for their
+//     completion before arriving at the barrier;
+//   * every mailbox is written ONCE per launch and read only after the barrier that
+//     follows it (one buffer per layer and phase), so no cache anywhere can hold an older
+//     copy of it within the launch, and consumers use ordinary cached loads - an XCD
+//     fetches a line once and its 32 CUs share it;
+//   * every 128-byte line of a mailbox is written by exactly one workgroup (strip-blocked
+//     layout), so a partially written line is never completed from memory too early.
+// The one exception is the KV-cache row appended in this step (its lines are shared by
+// several writers): attention reads that single row with device-scope loads.
+//
+// Every barrier wait is bounded: a workgroup that spins longer than the limit raises a
+// sticky error word and moves on, all later waits return at once, and the grid drains.
 #include "common.h"
 
 namespace {
+
+#define OHARA_MEGA_NS 16  // context chunks per (sequence, kv head)
+#define OHARA_MAX_PF 24   // weight tiles (16 B per lane) a wave fetches ahead of a phase
 
 struct MegaArgs {
   OharaModel m;                 // by value; the layer table is read from layers_dev
   const OharaLayer* layers_dev;
   uint16_t* const* kcache_dev;  // device arrays [n_layers]
   uint16_t* const* vcache_dev;
-  int B, nsplit, valid_vocab, hist_cap, select;
+  int B, valid_vocab, hist_cap, select;
+  int blk_x, blk_a;             // bytes per strip block of the x/q and act mailboxes
   int64_t* ids;
-  bf16_t* x;       // (B, d) residual stream                    } "mailbox" buffers: written by
-  bf16_t* q;       // (B, H*Dh)                                 } one phase, read by a later one
-  bf16_t* act;     // (B, F)                                    } on other CUs/XCDs; accessed
-  float* part_ml;  // (B, H, nsplit, 2)                         } only through the coherent
-  float* part_acc; // (B, H, nsplit, Dh)                        } helpers below
+  char* xm;        // (2*NL + 1) x-mailboxes of xm_stride bytes: residual stream after each half layer
+  char* qm;        // NL q-mailboxes of qm_stride bytes
+  char* am;        // NL act-mailboxes of am_stride bytes
+  float* pm;       // NL partial mailboxes of pm_stride floats: [b*H + h][chunk][Dh + 32]
+  size_t xm_stride, qm_stride, am_stride, pm_stride;
   float* cand_val; // (nwg, B)
   int* cand_idx;   // (nwg, B)
   bf16_t* logits;  // (B, V)
@@ -42,33 +60,34 @@ struct MegaArgs {
   unsigned int spin_limit;
 };
 
-// ---------------------------------------------------------------------------------------
-// Cross-workgroup data goes through device-scope (sc1) loads and stores: each access is
-// coherent across the XCDs' L2s by itself, so the barrier needs no L2 write-back or
-// invalidate (those cost ~1.7 us each on this chip, more than the barrier).  A producer
-// waits for its stores to complete (workgroup release = s_waitcnt vmcnt(0)) before it
-// arrives at the barrier.
-// ---------------------------------------------------------------------------------------
+// Optional fine-grained timeline: thread 0 of workgroup 0 records the shader clock.
+struct Prof {
+  unsigned long long* p;
+  int n;
+  __device__ __forceinline__ void stamp() {
+    if (p) p[n] = __builtin_readcyclecounter();
+    ++n;
+  }
+};
+
+__device__ __forceinline__ void st_coh8(void* p, uint2 v) {
+  __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), ((unsigned long long)v.y << 32) | v.x,
+                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_coh4(void* p, uint32_t v) {
+  __hip_atomic_store(reinterpret_cast<uint32_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 __device__ __forceinline__ uint2 ld_coh8(const void* p) {
   const unsigned long long v =
       __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return make_uint2((uint32_t)v, (uint32_t)(v >> 32));
 }
-__device__ __forceinline__ void st_coh8(void* p, uint2 v) {
-  __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), ((unsigned long long)v.y << 32) | v.x,
-                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ uint32_t ld_coh4(const void* p) {
-  return __hip_atomic_load(reinterpret_cast<const uint32_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void st_coh4(void* p, uint32_t v) {
-  __hip_atomic_store(reinterpret_cast<uint32_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ float ld_cohf(const float* p) { return __uint_as_float(ld_coh4(p)); }
-__device__ __forceinline__ void st_cohf(float* p, float v) { st_coh4(p, __float_as_uint(v)); }
 __device__ __forceinline__ uint4 ld_coh16(const void* p) {
   const uint2 a = ld_coh8(p), b = ld_coh8(reinterpret_cast<const char*>(p) + 8);
   return make_uint4(a.x, a.y, b.x, b.y);
+}
+__device__ __forceinline__ uint32_t ld_coh4(const void* p) {
+  return __hip_atomic_load(reinterpret_cast<const uint32_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -77,8 +96,9 @@ __device__ __forceinline__ uint4 ld_coh16(const void* p) {
 // polls; a flat counter serialises 256 read-modify-writes on one address (~11 us here),
 // this takes ~1.6 us.  Words (uint32, stride 64 per counter): [g*64] group g, [ng*64] top,
 // [(ng+1)*64] release, [(ng+2)*64] sticky error, [(ng+3)*64] barriers completed by earlier
-// launches.  Every wait is bounded; an expired wait raises the error word, after which all
-// waits return at once and the grid drains.
+// launches.  arrive() and wait() are split so that a workgroup can issue the loads of its
+// next phase (weights, cache tiles: nothing that depends on this phase) in between and
+// have them in flight while it waits.
 // ---------------------------------------------------------------------------------------
 #define OHARA_BAR_GROUP 16
 struct GridSync {
@@ -91,6 +111,7 @@ struct GridSync {
   unsigned int gsize;  // workgroups in my group
   unsigned int ng;
   unsigned int limit;
+  unsigned int arrived;
   __device__ void init(unsigned int* bar, unsigned int nwg, unsigned int lim) {
     ng = (nwg + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP;
     const unsigned int g = blockIdx.x / OHARA_BAR_GROUP;
@@ -101,14 +122,23 @@ struct GridSync {
     err = bar + (ng + 2) * 64;
     done = bar + (ng + 3) * 64;
     limit = lim;
+    arrived = 0;
     k = *done + 1;  // written by the previous launch (or the host): plain load
   }
-  __device__ void sync() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // my coherent stores have completed
-    __syncthreads();
+  __device__ __forceinline__ void arrive(Prof& pf) {
+    pf.stamp();  // phase work issued
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // my stores (LDS and sc1 global) have completed
+    pf.stamp();  // stores complete
+    __builtin_amdgcn_s_barrier();
+    pf.stamp();  // workgroup barrier passed
+    if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(gc, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+    asm volatile("" ::: "memory");  // compiler only: keep the caller's prefetch loads after this point
+    pf.stamp();  // arrival issued
+  }
+  __device__ __forceinline__ void wait(Prof& pf) {
+    pf.stamp();  // prefetch issued
     if (threadIdx.x == 0) {
-      const unsigned int a = __hip_atomic_fetch_add(gc, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
-      if (a == k * gsize) {
+      if (arrived == k * gsize) {
         const unsigned int t = __hip_atomic_fetch_add(top, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
         if (t == k * ng) __hip_atomic_store(rel, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
@@ -123,7 +153,10 @@ struct GridSync {
         __builtin_amdgcn_s_sleep(1);
       }
     }
-    __syncthreads();
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): nothing of mine is still on its way to LDS
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");  // compiler only: mailbox loads of the next phase stay below the barrier
+    pf.stamp();  // barrier passed
     ++k;
   }
 };
@@ -136,113 +169,124 @@ __device__ __forceinline__ float dot8m(uint4 a, uint4 b, float s) {
   return s;
 }
 
+// Strip-blocked mailbox of a (B, N) bf16 matrix: the 16 columns [16s, 16s+16) of all rows
+// form block s of `blk` bytes (a multiple of 128), row b at byte b*32 inside it.
+__device__ __forceinline__ const char* xm_addr(const char* base, int blk, int b, int n) {
+  return base + (size_t)(n >> 4) * blk + b * 32 + (n & 15) * 2;
+}
+// act mailbox: 8 columns per block, row b at byte b*16.
+__device__ __forceinline__ const char* am_addr(const char* base, int blk, int b, int f) {
+  return base + (size_t)(f >> 3) * blk + b * 16 + (f & 7) * 2;
+}
+
 // ---------------------------------------------------------------------------------------
 // staging of the GEMM activations in LDS: xs[b][ldxs] bf16
 // ---------------------------------------------------------------------------------------
 
-// norm.py:16-21 on rows of the residual stream (mailbox `src`, (B, K)), or - for the first
-// layer - on rows gathered from the embedding table (llama.py:310), which workgroup 0 also
-// publishes as the residual stream.  One wave per row; all loads of a row are issued
-// before any is consumed.  K <= 8 * 64 * NLD elements.
-template <int NLD>
-__device__ void stage_norm(bf16_t* xs, int ldxs, const bf16_t* src, const int64_t* ids, const bf16_t* table,
-                           int vocab, bf16_t* x_out, const bf16_t* nw, float eps, int B, int K) {
+// norm.py:16-21 on rows of the residual stream (x-mailbox `src`), or - for the first layer
+// - on rows gathered from the embedding table (llama.py:310).  One wave per row; all loads
+// of a row are issued before any is consumed.  K <= 8 * 64 * NLD elements.
+template <int NLD, bool EMBED>
+__device__ void stage_norm(bf16_t* xs, int ldxs, const char* src, int blk, const int64_t* ids, const bf16_t* table,
+                           int vocab, const bf16_t* nw, float eps, int B, int K) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int b = wave; b < B; b += 4) {
-    uint2 v[NLD * 2], g[NLD * 2];
-    if (ids) {
+    uint4 v[NLD], g[NLD];
+    size_t row_off = 0;
+    if (EMBED) {
       int64_t id = ids[b];
       if (id < 0 || id >= vocab) id = 0;
-      const bf16_t* row = table + (size_t)id * K;
-#pragma unroll
-      for (int c = 0; c < NLD * 2; ++c) {
-        const int k = (c * 64 + lane) * 4;
-        v[c] = k < K ? *reinterpret_cast<const uint2*>(row + k) : make_uint2(0, 0);
-      }
-    } else {
-      const bf16_t* row = src + (size_t)b * K;
-#pragma unroll
-      for (int c = 0; c < NLD * 2; ++c) {
-        const int k = (c * 64 + lane) * 4;
-        v[c] = k < K ? ld_coh8(row + k) : make_uint2(0, 0);
-      }
+      row_off = (size_t)id * K;
     }
 #pragma unroll
-    for (int c = 0; c < NLD * 2; ++c) {
-      const int k = (c * 64 + lane) * 4;
-      g[c] = k < K ? *reinterpret_cast<const uint2*>(nw + k) : make_uint2(0, 0);
+    for (int c = 0; c < NLD; ++c) {
+      const int k = (c * 64 + lane) * 8;
+      v[c] = make_uint4(0, 0, 0, 0);
+      g[c] = make_uint4(0, 0, 0, 0);
+      if (k < K) {
+        if (EMBED) v[c] = ldg16(table + row_off + k);
+        else v[c] = ldg16(xm_addr(src, blk, b, k));
+        g[c] = ldg16(nw + k);
+      }
     }
     float ss = 0.f;
 #pragma unroll
-    for (int c = 0; c < NLD * 2; ++c) {
-      const float a0 = lo_bf(v[c].x), a1 = hi_bf(v[c].x), a2 = lo_bf(v[c].y), a3 = hi_bf(v[c].y);
-      ss += (a0 * a0 + a1 * a1) + (a2 * a2 + a3 * a3);
+    for (int c = 0; c < NLD; ++c) {
+      const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float a0 = lo_bf(w[i]), a1 = hi_bf(w[i]);
+        ss += a0 * a0 + a1 * a1;
+      }
     }
     ss = wave_sum(ss);
     const float rinv = 1.0f / sqrtf(ss / (float)K + eps);
 #pragma unroll
-    for (int c = 0; c < NLD * 2; ++c) {
-      const int k = (c * 64 + lane) * 4;
+    for (int c = 0; c < NLD; ++c) {
+      const int k = (c * 64 + lane) * 8;
       if (k < K) {
-        const uint2 o = make_uint2(
-            pack_bf(rbf(lo_bf(v[c].x) * rinv) * lo_bf(g[c].x), rbf(hi_bf(v[c].x) * rinv) * hi_bf(g[c].x)),
-            pack_bf(rbf(lo_bf(v[c].y) * rinv) * lo_bf(g[c].y), rbf(hi_bf(v[c].y) * rinv) * hi_bf(g[c].y)));
-        *reinterpret_cast<uint2*>(xs + (size_t)b * ldxs + k) = o;
-        if (ids && x_out && blockIdx.x == 0) st_coh8(x_out + (size_t)b * K + k, v[c]);
+        const uint32_t xv[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+        const uint32_t gv[4] = {g[c].x, g[c].y, g[c].z, g[c].w};
+        uint32_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          o[i] = pack_bf(rbf(lo_bf(xv[i]) * rinv) * lo_bf(gv[i]), rbf(hi_bf(xv[i]) * rinv) * hi_bf(gv[i]));
+        *reinterpret_cast<uint4*>(xs + (size_t)b * ldxs + k) = make_uint4(o[0], o[1], o[2], o[3]);
       }
     }
   }
 }
 
-// Plain copy of a mailbox matrix (B, K) into LDS.
-__device__ void stage_copy(bf16_t* xs, int ldxs, const bf16_t* src, int B, int K) {
-  const int n4 = K >> 2;
-  for (int i = threadIdx.x; i < B * n4; i += blockDim.x) {
-    const int b = i / n4, k = (i - b * n4) << 2;
-    *reinterpret_cast<uint2*>(xs + (size_t)b * ldxs + k) = ld_coh8(src + (size_t)b * K + k);
+// act mailbox (B, F) -> LDS
+__device__ void stage_act(bf16_t* xs, int ldxs, const char* src, int blk, int B, int F) {
+  const int n8 = F >> 3;
+  for (int i = threadIdx.x; i < B * n8; i += blockDim.x) {
+    const int b = i / n8, c = i - b * n8;
+    *reinterpret_cast<uint4*>(xs + (size_t)b * ldxs + c * 8) = ldg16(am_addr(src, blk, b, c * 8));
   }
 }
 
 // Merge of the attention partials of all chunks, in chunk order (llama.py:116-123 output,
-// rounded to bf16 as SDPA's result is) -> xs[b][h*Dh + d].  A thread owns two adjacent
+// rounded to bf16 as SDPA's result is) -> xs[b][h*Dh + d].  A thread owns four adjacent
 // columns; the (max, sum) pairs and the accumulators of all NS chunks are loaded before any
 // is used.
 template <int NS>
-__device__ void stage_attn_merge(bf16_t* xs, int ldxs, const MegaArgs& a) {
-  const int H = a.m.n_heads, Dh = a.m.head_dim;
-  const int HD = H * Dh;
-  for (int e = threadIdx.x * 2; e < a.B * HD; e += blockDim.x * 2) {
+__device__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh) {
+  const int HD = H * Dh, PS = Dh + 32;
+  for (int e = threadIdx.x * 4; e < B * HD; e += blockDim.x * 4) {
     const int b = e / HD, hd = e - b * HD;
     const int h = hd / Dh, d = hd - h * Dh;
-    const float* ml = a.part_ml + ((size_t)(b * H + h) * NS) * 2;
-    const float* pa = a.part_acc + ((size_t)(b * H + h) * NS) * Dh + d;
-    uint2 mlv[NS], av[NS];
+    const float* base = pm + (size_t)(b * H + h) * NS * PS;
+    uint2 mlv[NS];
+    uint4 av[NS];
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-      mlv[s] = ld_coh8(ml + 2 * s);
-      av[s] = ld_coh8(pa + (size_t)s * Dh);
+      mlv[s] = *reinterpret_cast<const uint2*>(base + (size_t)s * PS + Dh);
+      av[s] = ldg16(base + (size_t)s * PS + d);
     }
     float M = -INFINITY;
 #pragma unroll
     for (int s = 0; s < NS; ++s) M = fmaxf(M, __uint_as_float(mlv[s].x));
-    float Ls = 0.f, o0 = 0.f, o1 = 0.f;
+    float Ls = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
       const float ms = __uint_as_float(mlv[s].x);
       const float w = (ms == -INFINITY) ? 0.f : __expf(ms - M);
       Ls += __uint_as_float(mlv[s].y) * w;
-      o0 += __uint_as_float(av[s].x) * w;
-      o1 += __uint_as_float(av[s].y) * w;
+      o[0] += __uint_as_float(av[s].x) * w;
+      o[1] += __uint_as_float(av[s].y) * w;
+      o[2] += __uint_as_float(av[s].z) * w;
+      o[3] += __uint_as_float(av[s].w) * w;
     }
-    *reinterpret_cast<uint32_t*>(xs + (size_t)b * ldxs + hd) = pack_bf(o0 / Ls, o1 / Ls);
+    *reinterpret_cast<uint2*>(xs + (size_t)b * ldxs + hd) =
+        make_uint2(pack_bf(o[0] / Ls, o[1] / Ls), pack_bf(o[2] / Ls, o[3] / Ls));
   }
 }
 
 // ---------------------------------------------------------------------------------------
 // GEMM phase: strips of 16 packed rows, KP waves per strip, activations from LDS.  The
-// weights of a workgroup's first strip(s) are fetched into registers BEFORE the barrier
-// that precedes the phase (they do not depend on the activations), so the HBM stream runs
-// under the barrier latency.
+// weights of a workgroup's first strip(s) - and the residual it will add - are fetched
+// into registers between arrive() and wait() of the barrier that precedes the phase.
 // ---------------------------------------------------------------------------------------
 enum { E_RESID = 1, E_SWIGLU = 2, E_ROPE = 3, E_LOGITS = 4 };
 
@@ -250,23 +294,29 @@ struct GemmP {
   const uint4* wp;
   int N, K;        // logical rows (for E_SWIGLU: hidden width F) and columns
   int nstrips;
-  bf16_t* out;     // mailbox output (E_ROPE: q; E_RESID: residual stream, read-modify-write)
-  int ldo;
+  char* out;       // output mailbox (E_ROPE: q; E_RESID: x; E_SWIGLU: act) or logits
+  int blk;         // its block size
+  const char* resid;      // E_RESID: x mailbox to add
+  int resid_embed;        // E_RESID: add the embedding rows instead (first half layer)
+  const int64_t* ids;     // E_RESID with resid == nullptr
+  const bf16_t* table;
+  int vocab;
   int H, Hkv, Dh, Tmax, pos;
   const bf16_t* cos;
   const bf16_t* sin;
   bf16_t* kc;
   bf16_t* vc;
   int valid;       // E_LOGITS: ids >= valid never win
+  int ldo;         // E_LOGITS: row stride of the logits
 };
 
-#define OHARA_MAX_PF 24
 struct GemmPre {  // one register buffer, reused by every phase (only one prefetch is live at a time)
   uint4 w[OHARA_MAX_PF];
+  uint2 r;        // E_RESID: the four residual values of this lane (first strip)
 };
 
-template <int KP, int PF>
-__device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre) {
+template <int KP, int PF, int EPI>
+__device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int B) {
   constexpr int SPW = 4 / KP;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = wave / KP, kpart = wave % KP;
@@ -278,11 +328,25 @@ __device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre) {
 #pragma unroll
   for (int c = 0; c < PF; ++c)
     pre.w[c] = (strip < p.nstrips && j0 + c < j1) ? ldg16_nt(wrow + (size_t)(j0 + c) * 64) : make_uint4(0, 0, 0, 0);
+  if (EPI == E_RESID) {
+    const int m = lane & 15, g = lane >> 4;
+    const int r0 = strip * 16 + 4 * g;
+    pre.r = make_uint2(0, 0);
+    if (strip < p.nstrips && kpart == 0 && m < B && r0 < p.N) {
+      if (!p.resid_embed) {
+        pre.r = *reinterpret_cast<const uint2*>(xm_addr(p.resid, p.blk, m, r0));
+      } else {
+        int64_t id = p.ids[m];
+        if (id < 0 || id >= p.vocab) id = 0;
+        pre.r = *reinterpret_cast<const uint2*>(p.table + (size_t)id * p.N + r0);
+      }
+    }
+  }
 }
 
 template <int KP, int PF, int EPI>
-__device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, const bf16_t* xs, int ldxs, int B, float* red,
-                           float& best_v, int& best_i) {
+__device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, const bf16_t* xs, int ldxs, int B,
+                                           float* red, float& best_v, int& best_i, Prof& pf) {
   constexpr int SPW = 4 / KP;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 15, g = lane >> 4;
@@ -323,6 +387,7 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
         }
       }
     }
+    if (it == 0) pf.stamp();  // MFMAs issued
     if (KP > 1) {
       if (kpart > 0) {
 #pragma unroll
@@ -336,19 +401,29 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
           for (int i = 0; i < 4; ++i) acc[i] += red[(((wave + w) * 64) + lane) * 4 + i];
       }
     }
+    if (it == 0) pf.stamp();  // cross-wave sum done
     if (live && kpart == 0 && mine) {
       const int b = m;
       const int r0 = strip * 16 + 4 * g;
       const float y0 = rbf(acc[0]), y1 = rbf(acc[1]), y2 = rbf(acc[2]), y3 = rbf(acc[3]);
       if (EPI == E_RESID) {  // N % 4 == 0 is required by the entry point
         if (r0 < p.N) {
-          bf16_t* o = p.out + (size_t)b * p.ldo + r0;
-          const uint2 r = ld_coh8(o);
-          st_coh8(o, make_uint2(pack_bf(lo_bf(r.x) + y0, hi_bf(r.x) + y1), pack_bf(lo_bf(r.y) + y2, hi_bf(r.y) + y3)));
+          uint2 r = pre.r;
+          if (it > 0) {
+            if (!p.resid_embed) {
+              r = *reinterpret_cast<const uint2*>(xm_addr(p.resid, p.blk, b, r0));
+            } else {
+              int64_t id = p.ids[b];
+              if (id < 0 || id >= p.vocab) id = 0;
+              r = *reinterpret_cast<const uint2*>(p.table + (size_t)id * p.N + r0);
+            }
+          }
+          st_coh8(const_cast<char*>(xm_addr(p.out, p.blk, b, r0)),
+                  make_uint2(pack_bf(lo_bf(r.x) + y0, hi_bf(r.x) + y1), pack_bf(lo_bf(r.y) + y2, hi_bf(r.y) + y3)));
         }
       } else if (EPI == E_LOGITS) {
         const float v[4] = {y0, y1, y2, y3};
-        bf16_t* o = p.out + (size_t)b * p.ldo + r0;
+        bf16_t* o = reinterpret_cast<bf16_t*>(p.out) + (size_t)b * p.ldo + r0;
         if (r0 + 3 < p.N && ((p.ldo & 3) == 0)) {
           *reinterpret_cast<uint2*>(o) = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
         } else {
@@ -368,13 +443,13 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
         const int f = strip * 8 + 2 * g;
         if (f < p.N) {
           const float s0 = rbf(silu_f(y0)), s1 = rbf(silu_f(y1));
-          st_coh4(p.out + (size_t)b * p.ldo + f, pack_bf(s0 * y2, s1 * y3));
+          st_coh4(const_cast<char*>(am_addr(p.out, p.blk, b, f)), pack_bf(s0 * y2, s1 * y3));
         }
       } else {  // E_ROPE
         const int nq = p.H * p.Dh, nk = p.Hkv * p.Dh;
         if (r0 < nq + 2 * nk && p.pos >= 0 && p.pos < p.Tmax) {
           float v[4] = {y0, y1, y2, y3};
-          bf16_t* o;
+          char* o;
           if (r0 < nq + nk) {
             const int d = (r0 < nq ? r0 : r0 - nq) % p.Dh;
             const uint32_t cs = *reinterpret_cast<const uint32_t*>(p.cos + (size_t)p.pos * (p.Dh >> 1) + (d >> 1));
@@ -386,10 +461,10 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
               v[2 * pr] = __fsub_rn(__fmul_rn(e, c2[pr]), __fmul_rn(od, s2[pr]));
               v[2 * pr + 1] = __fadd_rn(__fmul_rn(e, s2[pr]), __fmul_rn(od, c2[pr]));
             }
-            o = (r0 < nq) ? p.out + (size_t)b * p.ldo + r0
-                          : p.kc + (((size_t)b * p.Tmax + p.pos) * p.Hkv) * p.Dh + (r0 - nq);
+            o = (r0 < nq) ? const_cast<char*>(xm_addr(p.out, p.blk, b, r0))
+                          : reinterpret_cast<char*>(p.kc + (((size_t)b * p.Tmax + p.pos) * p.Hkv) * p.Dh + (r0 - nq));
           } else {
-            o = p.vc + (((size_t)b * p.Tmax + p.pos) * p.Hkv) * p.Dh + (r0 - nq - nk);
+            o = reinterpret_cast<char*>(p.vc + (((size_t)b * p.Tmax + p.pos) * p.Hkv) * p.Dh + (r0 - nq - nk));
           }
           st_coh8(o, make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3])));
         }
@@ -400,27 +475,88 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
 }
 
 // ---------------------------------------------------------------------------------------
-// attention phase: items (sequence, kv head, chunk); writes partial triples
+// attention phase: items (sequence, kv head, chunk); writes partial triples.  The K/V
+// tiles of a wave's first 16 positions are fetched before the barrier.
 // ---------------------------------------------------------------------------------------
-template <int D, int G>
-__device__ void attn_phase(const MegaArgs& a, const bf16_t* kc, const bf16_t* vc, int L, float* lds) {
+template <int D>
+struct AttnPre {
+  uint4 k[D / 32];
+  uint4 v[D / 32];  // NV = 16 / (64 / (D / 8)) = D / 32
+};
+
+// One 16-position tile: positions >= t1 load nothing; position `coh_pos` (the row appended in
+// this step, or -1) is read with device-scope loads.
+template <int D>
+__device__ __forceinline__ void attn_tile_load(const bf16_t* kb, const bf16_t* vb, size_t row, int tb, int t1,
+                                               int coh_pos, uint4* kv, uint4* vv) {
   constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
-  const int H = a.m.n_heads, Hkv = a.m.n_kv_heads, Tmax = a.m.t_max, ns = a.nsplit;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lane = threadIdx.x & 63;
   const int p = lane & 15, dq = lane >> 4;
+  const int pp = lane / DC, dc = lane % DC;
+  const int pos = tb + p;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const bf16_t* src = kb + (size_t)pos * row + (4 * c + dq) * 8;
+    kv[c] = pos < t1 ? (pos == coh_pos ? ld_coh16(src) : ldg16_nt(src)) : make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int c = 0; c < NV; ++c) {
+    const int vp = tb + c * PP + pp;
+    const bf16_t* src = vb + (size_t)vp * row + dc * 8;
+    vv[c] = vp < t1 ? (vp == coh_pos ? ld_coh16(src) : ldg16_nt(src)) : make_uint4(0, 0, 0, 0);
+  }
+}
+
+__device__ __forceinline__ void attn_item_range(int item, int ns, int Hkv, int L, int& b, int& kvh, int& split, int& t0,
+                                                int& t1) {
+  const int chunk = (((L + ns - 1) / ns) + 15) & ~15;
+  split = item % ns;
+  kvh = (item / ns) % Hkv;
+  b = item / (ns * Hkv);
+  t0 = split * chunk;
+  t1 = min(L, t0 + chunk);
+}
+
+// The first tile of each wave's first item, if it lies wholly below the row being appended.
+template <int D>
+__device__ __forceinline__ bool attn_first_tile_prefetchable(int t0, int t1, int L) {
+  const int tb = t0 + (threadIdx.x >> 6) * 16;
+  return tb + 16 <= min(t1, L - 1);
+}
+
+template <int D>
+__device__ __forceinline__ void attn_prefetch(const MegaArgs& a, const bf16_t* kc, const bf16_t* vc, int L,
+                                              AttnPre<D>& pre) {
+  const int Hkv = a.m.n_kv_heads, wave = threadIdx.x >> 6;
+  const size_t row = (size_t)Hkv * D;
+  int b, kvh, split, t0, t1;
+  attn_item_range(blockIdx.x, OHARA_MEGA_NS, Hkv, L, b, kvh, split, t0, t1);
+  const bool has = (int)blockIdx.x < a.B * Hkv * OHARA_MEGA_NS && attn_first_tile_prefetchable<D>(t0, t1, L);
+  const bf16_t* kb = kc + (size_t)b * a.m.t_max * row + (size_t)kvh * D;
+  const bf16_t* vb = vc + (size_t)b * a.m.t_max * row + (size_t)kvh * D;
+  attn_tile_load<D>(kb, vb, row, t0 + wave * 16, has ? t1 : 0, -1, pre.k, pre.v);
+}
+
+template <int D, int G>
+__device__ void attn_phase(const MegaArgs& a, const AttnPre<D>& pre, const char* qm, float* pm, const bf16_t* kc,
+                           const bf16_t* vc, int L, float* lds) {
+  constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
+  const int H = a.m.n_heads, Hkv = a.m.n_kv_heads, Tmax = a.m.t_max, ns = OHARA_MEGA_NS;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int p = lane & 15;
+  const int dq = lane >> 4;
   const int pp = lane / DC, dc = lane % DC;
   const float scale = 1.0f / sqrtf((float)D);
   float* s_m = lds;                 // [4][G]
   float* s_l = lds + 4 * G;         // [4][G]
   float* s_acc = lds + 8 * G;       // [4][G][D]
-  const int chunk = (((L + ns - 1) / ns) + 15) & ~15;
   const int nitems = a.B * Hkv * ns;
   const size_t row = (size_t)Hkv * D;
+  const int PS = D + 32;
+  bool first = true;
   for (int item = blockIdx.x; item < nitems; item += gridDim.x) {
-    const int split = item % ns;
-    const int kvh = (item / ns) % Hkv;
-    const int b = item / (ns * Hkv);
-    const int t0 = split * chunk, t1 = min(L, t0 + chunk);
+    int b, kvh, split, t0, t1;
+    attn_item_range(item, ns, Hkv, L, b, kvh, split, t0, t1);
     const bf16_t* kb = kc + (size_t)b * Tmax * row + (size_t)kvh * D;
     const bf16_t* vb = vc + (size_t)b * Tmax * row + (size_t)kvh * D;
     float m_run[G], l_run[G], acc[G][8];
@@ -437,18 +573,18 @@ __device__ void attn_phase(const MegaArgs& a, const bf16_t* kc, const bf16_t* vc
       for (int hh = 0; hh < G; ++hh)
 #pragma unroll
         for (int c = 0; c < NC; ++c)
-          qv[hh][c] = ld_coh16(a.q + (size_t)b * H * D + (size_t)(kvh * G + hh) * D + (4 * c + dq) * 8);
+          qv[hh][c] = ldg16(xm_addr(qm, a.blk_x, b, (kvh * G + hh) * D + (4 * c + dq) * 8));
+      const bool use_pre = first && attn_first_tile_prefetchable<D>(t0, t1, L);
       for (int tb = t0 + wave * 16; tb < t1; tb += 64) {
-        const int pos = tb + p;
-        const bool valid = pos < t1;
+        const bool valid = tb + p < t1;
         uint4 kv[NC], vv[NV];
+        if (use_pre && tb == t0 + wave * 16) {
 #pragma unroll
-        for (int c = 0; c < NC; ++c)
-          kv[c] = valid ? ldg16_nt(kb + (size_t)pos * row + (4 * c + dq) * 8) : make_uint4(0, 0, 0, 0);
+          for (int c = 0; c < NC; ++c) kv[c] = pre.k[c];
 #pragma unroll
-        for (int c = 0; c < NV; ++c) {
-          const int vp = tb + c * PP + pp;
-          vv[c] = vp < t1 ? ldg16_nt(vb + (size_t)vp * row + dc * 8) : make_uint4(0, 0, 0, 0);
+          for (int c = 0; c < NV; ++c) vv[c] = pre.v[c];
+        } else {
+          attn_tile_load<D>(kb, vb, row, tb, t1, L - 1, kv, vv);
         }
 #pragma unroll
         for (int hh = 0; hh < G; ++hh) {
@@ -484,6 +620,7 @@ __device__ void attn_phase(const MegaArgs& a, const bf16_t* kc, const bf16_t* vc
         }
       }
     }
+    first = false;
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) {
 #pragma unroll
@@ -516,9 +653,9 @@ __device__ void attn_phase(const MegaArgs& a, const bf16_t* kc, const bf16_t* vc
         o0 += s_acc[(w * G + hh) * D + d] * sc;
         o1 += s_acc[(w * G + hh) * D + d + 1] * sc;
       }
-      const size_t pi = (size_t)(b * H + h) * ns + split;
-      st_coh8(a.part_acc + pi * D + d, make_uint2(__float_as_uint(o0), __float_as_uint(o1)));
-      if (d == 0) st_coh8(a.part_ml + pi * 2, make_uint2(__float_as_uint(M), __float_as_uint(Ls)));
+      float* dst = pm + ((size_t)(b * H + h) * ns + split) * PS;
+      st_coh8(dst + d, make_uint2(__float_as_uint(o0), __float_as_uint(o1)));
+      if (d == 0) st_coh8(dst + D, make_uint2(__float_as_uint(M), __float_as_uint(Ls)));
     }
     __syncthreads();
   }
@@ -527,8 +664,6 @@ __device__ void attn_phase(const MegaArgs& a, const bf16_t* kc, const bf16_t* vc
 // ---------------------------------------------------------------------------------------
 // the kernel
 // ---------------------------------------------------------------------------------------
-#define OHARA_MEGA_NS 16  // context chunks per (sequence, kv head)
-
 template <int D, int G>
 __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -547,88 +682,96 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   const int L = min(pos + 1, m.t_max);
   float best_v = -INFINITY;
   int best_i = 0x7fffffff;
-  int nprof = 0;
-  auto stamp = [&]() {
-    if (a.prof && blockIdx.x == 0 && threadIdx.x == 0) a.prof[nprof] = __builtin_readcyclecounter();
-    ++nprof;
-  };
+  Prof pf{(blockIdx.x == 0 && threadIdx.x == 0) ? a.prof : nullptr, 0};
 
   GemmP qkv{}, prj{}, gu{}, dn{}, lm{};
   qkv.H = H; qkv.Hkv = Hkv; qkv.Dh = D; qkv.Tmax = m.t_max; qkv.pos = pos; qkv.cos = m.cos; qkv.sin = m.sin;
-  qkv.N = (H + 2 * Hkv) * D; qkv.K = d; qkv.nstrips = (qkv.N + 15) / 16; qkv.out = a.q; qkv.ldo = H * D;
-  prj.N = d; prj.K = H * D; prj.nstrips = (d + 15) / 16; prj.out = a.x; prj.ldo = d;
-  gu.N = F; gu.K = d; gu.nstrips = 2 * ((F + 7) / 8 * 8) / 16; gu.out = a.act; gu.ldo = F;
-  dn.N = d; dn.K = F; dn.nstrips = (d + 15) / 16; dn.out = a.x; dn.ldo = d;
-  lm.N = V; lm.K = d; lm.nstrips = (V + 15) / 16; lm.out = a.logits; lm.ldo = V;
+  qkv.N = (H + 2 * Hkv) * D; qkv.K = d; qkv.nstrips = (qkv.N + 15) / 16; qkv.blk = a.blk_x;
+  prj.N = d; prj.K = H * D; prj.nstrips = (d + 15) / 16; prj.blk = a.blk_x;
+  prj.ids = a.ids; prj.table = m.token_emb; prj.vocab = V;
+  gu.N = F; gu.K = d; gu.nstrips = 2 * ((F + 7) / 8 * 8) / 16; gu.blk = a.blk_a;
+  dn.N = d; dn.K = F; dn.nstrips = (d + 15) / 16; dn.blk = a.blk_x;
+  dn.ids = a.ids; dn.table = m.token_emb; dn.vocab = V;
+  lm.N = V; lm.K = d; lm.nstrips = (V + 15) / 16; lm.out = reinterpret_cast<char*>(a.logits); lm.ldo = V;
   lm.valid = a.valid_vocab > 0 ? min(a.valid_vocab, V) : V;
   lm.wp = reinterpret_cast<const uint4*>(m.w_vocab);
 
   GemmPre pre;
-
-  {
-    const OharaLayer& L0 = a.layers_dev[0];
-    qkv.wp = reinterpret_cast<const uint4*>(L0.wqkv);
-    gemm_prefetch<4, 6>(qkv, pre);
-  }
-  stamp();
+  AttnPre<D> apre;
+  qkv.wp = reinterpret_cast<const uint4*>(a.layers_dev[0].wqkv);
+  gemm_prefetch<4, 6, E_ROPE>(qkv, pre, B);
+  pf.stamp();
   for (int l = 0; l < m.n_layers; ++l) {
     const OharaLayer& Lw = a.layers_dev[l];
     bf16_t* kc = a.kcache_dev[l];
     bf16_t* vc = a.vcache_dev[l];
+    const char* x_in = a.xm + (size_t)(2 * l) * a.xm_stride;       // residual stream entering the layer
+    char* x_mid = a.xm + (size_t)(2 * l + 1) * a.xm_stride;        // after attention
+    char* x_out = a.xm + (size_t)(2 * l + 2) * a.xm_stride;        // after the feed-forward
+    char* q_l = a.qm + (size_t)l * a.qm_stride;
+    char* a_l = a.am + (size_t)l * a.am_stride;
+    float* p_l = a.pm + (size_t)l * a.pm_stride;
     // P1: [embedding] + norm1 + QKV + rotary + append
-    qkv.kc = kc; qkv.vc = vc;
+    qkv.kc = kc; qkv.vc = vc; qkv.out = q_l;
     if ((int)blockIdx.x < qkv.nstrips) {
-      if (l == 0) stage_norm<2>(xs, ldxs, nullptr, a.ids, m.token_emb, V, a.x, Lw.norm1, m.eps, B, d);
-      else stage_norm<2>(xs, ldxs, a.x, nullptr, nullptr, 0, nullptr, Lw.norm1, m.eps, B, d);
+      if (l == 0) stage_norm<2, true>(xs, ldxs, a.xm, 0, a.ids, m.token_emb, V, Lw.norm1, m.eps, B, d);
+      else stage_norm<2, false>(xs, ldxs, x_in, a.blk_x, a.ids, m.token_emb, V, Lw.norm1, m.eps, B, d);
     }
     __syncthreads();
-    stamp();
-    gemm_phase<4, 6, E_ROPE>(qkv, pre, xs, ldxs, B, red, best_v, best_i);
-    stamp();
-    prj.wp = reinterpret_cast<const uint4*>(Lw.wo);
-    gemm_prefetch<4, 6>(prj, pre);
-    gs.sync();
-    stamp();
+    pf.stamp();
+    gemm_phase<4, 6, E_ROPE>(qkv, pre, xs, ldxs, B, red, best_v, best_i, pf);
+    pf.stamp();
+    gs.arrive(pf);
+    attn_prefetch<D>(a, kc, vc, L, apre);
+    gs.wait(pf);
+    pf.stamp();
     // P2: attention partials
-    attn_phase<D, G>(a, kc, vc, L, att);
-    gs.sync();
-    stamp();
+    attn_phase<D, G>(a, apre, q_l, p_l, kc, vc, L, att);
+    gs.arrive(pf);
+    prj.wp = reinterpret_cast<const uint4*>(Lw.wo); prj.out = x_mid; prj.resid = x_in; prj.resid_embed = l == 0;
+    gemm_prefetch<4, 6, E_RESID>(prj, pre, B);
+    gs.wait(pf);
+    pf.stamp();
     // P3: merge + output projection + residual
-    if ((int)blockIdx.x < prj.nstrips) stage_attn_merge<OHARA_MEGA_NS>(xs, ldxs, a);
+    if ((int)blockIdx.x < prj.nstrips) stage_attn_merge<OHARA_MEGA_NS>(xs, ldxs, p_l, B, H, D);
     __syncthreads();
-    stamp();
-    gemm_phase<4, 6, E_RESID>(prj, pre, xs, ldxs, B, red, best_v, best_i);
-    stamp();
-    gu.wp = reinterpret_cast<const uint4*>(Lw.wgu);
-    gemm_prefetch<2, 12>(gu, pre);
-    gs.sync();
-    stamp();
+    pf.stamp();
+    gemm_phase<4, 6, E_RESID>(prj, pre, xs, ldxs, B, red, best_v, best_i, pf);
+    pf.stamp();
+    gs.arrive(pf);
+    gu.wp = reinterpret_cast<const uint4*>(Lw.wgu); gu.out = a_l;
+    gemm_prefetch<2, 12, E_SWIGLU>(gu, pre, B);
+    gs.wait(pf);
+    pf.stamp();
     // P4: norm2 + gate/up + SwiGLU
-    if ((int)blockIdx.x * 2 < gu.nstrips) stage_norm<2>(xs, ldxs, a.x, nullptr, nullptr, 0, nullptr, Lw.norm2, m.eps, B, d);
+    if ((int)blockIdx.x * 2 < gu.nstrips) stage_norm<2, false>(xs, ldxs, x_mid, a.blk_x, a.ids, m.token_emb, V, Lw.norm2, m.eps, B, d);
     __syncthreads();
-    gemm_phase<2, 12, E_SWIGLU>(gu, pre, xs, ldxs, B, red, best_v, best_i);
-    dn.wp = reinterpret_cast<const uint4*>(Lw.wdown);
-    gemm_prefetch<4, 24>(dn, pre);
-    gs.sync();
-    stamp();
+    gemm_phase<2, 12, E_SWIGLU>(gu, pre, xs, ldxs, B, red, best_v, best_i, pf);
+    gs.arrive(pf);
+    dn.wp = reinterpret_cast<const uint4*>(Lw.wdown); dn.out = x_out; dn.resid = x_mid;
+    gemm_prefetch<4, 24, E_RESID>(dn, pre, B);
+    gs.wait(pf);
+    pf.stamp();
     // P5: down projection + residual
-    if ((int)blockIdx.x < dn.nstrips) stage_copy(xs, ldxs, a.act, B, F);
+    if ((int)blockIdx.x < dn.nstrips) stage_act(xs, ldxs, a_l, a.blk_a, B, F);
     __syncthreads();
-    gemm_phase<4, 24, E_RESID>(dn, pre, xs, ldxs, B, red, best_v, best_i);
+    gemm_phase<4, 24, E_RESID>(dn, pre, xs, ldxs, B, red, best_v, best_i, pf);
+    gs.arrive(pf);
     if (l + 1 < m.n_layers) {
       qkv.wp = reinterpret_cast<const uint4*>(a.layers_dev[l + 1].wqkv);
-      gemm_prefetch<4, 6>(qkv, pre);
+      gemm_prefetch<4, 6, E_ROPE>(qkv, pre, B);
     } else {
-      gemm_prefetch<1, 24>(lm, pre);
+      gemm_prefetch<1, 24, E_LOGITS>(lm, pre, B);
     }
-    gs.sync();
-    stamp();
+    gs.wait(pf);
+    pf.stamp();
   }
   // final norm + vocabulary projection, running arg-max per lane
-  stage_norm<2>(xs, ldxs, a.x, nullptr, nullptr, 0, nullptr, m.final_norm, m.eps, B, d);
+  stage_norm<2, false>(xs, ldxs, a.xm + (size_t)(2 * m.n_layers) * a.xm_stride, a.blk_x, a.ids, m.token_emb, V,
+                       m.final_norm, m.eps, B, d);
   __syncthreads();
-  gemm_phase<1, 24, E_LOGITS>(lm, pre, xs, ldxs, B, red, best_v, best_i);
-  stamp();
+  gemm_phase<1, 24, E_LOGITS>(lm, pre, xs, ldxs, B, red, best_v, best_i, pf);
+  pf.stamp();
   if (a.select) {
     // lanes with the same batch column (lane & 15) fold their candidates; then the waves
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -660,17 +803,18 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
           bi = oi;
         }
       }
-      st_cohf(a.cand_val + (size_t)blockIdx.x * B + threadIdx.x, bv);
+      st_coh4(a.cand_val + (size_t)blockIdx.x * B + threadIdx.x, __float_as_uint(bv));
       st_coh4(a.cand_idx + (size_t)blockIdx.x * B + threadIdx.x, (uint32_t)bi);
     }
-    gs.sync();
+    gs.arrive(pf);
+    gs.wait(pf);
     if (blockIdx.x == 0) {
       // one wave per sequence (round robin): reduce the per-workgroup candidates
       for (int b = wave; b < B; b += 4) {
         float bv = -INFINITY;
         int bi = 0x7fffffff;
         for (int w = lane; w < (int)gridDim.x; w += 64) {
-          const float ov = ld_cohf(a.cand_val + (size_t)w * B + b);
+          const float ov = __uint_as_float(ld_coh4(a.cand_val + (size_t)w * B + b));
           const int oi = (int)ld_coh4(a.cand_idx + (size_t)w * B + b);
           if (ov > bv || (ov == bv && oi < bi)) {
             bv = ov;
@@ -694,7 +838,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
       }
     }
   }
-  stamp();
+  pf.stamp();
   // bookkeeping by workgroup 0: everyone is past the last barrier, nobody reads these again
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     *gs.done = gs.k - 1;
@@ -705,32 +849,67 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   }
 }
 
+// ---- workspace layout ------------------------------------------------------------------
+#define OHARA_BAR_WORDS(nwg) ((((nwg) + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP + 4) * 64)
+#define OHARA_PROF_SLOTS 1024
+
+size_t mega_al(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct MegaLayout {
+  size_t layers, kptr, vptr, xm, qm, am, pm, candv, candi, prof, bar, total;
+  size_t xm_stride, qm_stride, am_stride, pm_stride;
+  int blk_x, blk_a;
+};
+
+MegaLayout mega_layout(const OharaModel* m, int B, int nwg) {
+  MegaLayout L{};
+  const int NL = m->n_layers, D = m->head_dim;
+  L.blk_x = (B * 32 + 127) / 128 * 128;
+  L.blk_a = (B * 16 + 127) / 128 * 128;
+  const int nq_rows = (m->n_heads + 2 * m->n_kv_heads) * D;
+  L.xm_stride = mega_al((size_t)((m->d_model + 15) / 16) * L.blk_x);
+  L.qm_stride = mega_al((size_t)((nq_rows + 15) / 16) * L.blk_x);
+  L.am_stride = mega_al((size_t)((m->d_ff + 7) / 8) * L.blk_a);
+  L.pm_stride = mega_al((size_t)B * m->n_heads * OHARA_MEGA_NS * (D + 32) * sizeof(float)) / sizeof(float);
+  size_t o = 0;
+  L.layers = o; o += mega_al(sizeof(OharaLayer) * NL);
+  L.kptr = o; o += mega_al(sizeof(void*) * NL);
+  L.vptr = o; o += mega_al(sizeof(void*) * NL);
+  L.xm = o; o += L.xm_stride * (2 * NL + 1);
+  L.qm = o; o += L.qm_stride * NL;
+  L.am = o; o += L.am_stride * NL;
+  L.pm = o; o += L.pm_stride * sizeof(float) * NL;
+  L.candv = o; o += mega_al((size_t)nwg * B * sizeof(float));
+  L.candi = o; o += mega_al((size_t)nwg * B * sizeof(int));
+  L.prof = o; o += mega_al(OHARA_PROF_SLOTS * sizeof(unsigned long long));
+  L.bar = o; o += mega_al(OHARA_BAR_WORDS(nwg) * sizeof(unsigned int));
+  L.total = o;
+  return L;
+}
+
 }  // namespace
 
 extern "C" {
 
-#define OHARA_BAR_WORDS(nwg) ((((nwg) + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP + 4) * 64)
-#define OHARA_PROF_SLOTS 512
-
-static size_t mega_al(size_t v) { return (v + 255) & ~(size_t)255; }
-
-// Bytes of the device scratch block ohara_llama_decode_persistent needs.
 int64_t ohara_persistent_workspace_bytes(const OharaModel* m, int batch, int n_split, int n_workgroups) {
-  if (!m || batch < 1 || n_split < 1 || n_workgroups < 1) return OHARA_EINVAL;
-  size_t tot = 0;
-  tot += mega_al(sizeof(OharaLayer) * m->n_layers);
-  tot += 2 * mega_al(sizeof(void*) * m->n_layers);
-  tot += mega_al((size_t)batch * m->n_heads * n_split * 2 * sizeof(float));
-  tot += mega_al((size_t)batch * m->n_heads * n_split * m->head_dim * sizeof(float));
-  tot += 2 * mega_al((size_t)n_workgroups * batch * sizeof(float));
-  tot += mega_al(OHARA_PROF_SLOTS * sizeof(unsigned long long));
-  tot += mega_al(OHARA_BAR_WORDS(n_workgroups) * sizeof(unsigned int));
-  return (int64_t)tot;
+  if (!m || batch < 1 || n_split != OHARA_MEGA_NS || n_workgroups < 1) return OHARA_EINVAL;
+  return (int64_t)mega_layout(m, batch, n_workgroups).total;
 }
 
 int64_t ohara_persistent_barrier_offset(const OharaModel* m, int batch, int n_split, int n_workgroups) {
-  const int64_t tot = ohara_persistent_workspace_bytes(m, batch, n_split, n_workgroups);
-  return tot < 0 ? tot : tot - (int64_t)mega_al(OHARA_BAR_WORDS(n_workgroups) * sizeof(unsigned int));
+  if (!m || batch < 1 || n_split != OHARA_MEGA_NS || n_workgroups < 1) return OHARA_EINVAL;
+  return (int64_t)mega_layout(m, batch, n_workgroups).bar;
+}
+
+int64_t ohara_persistent_error_offset(const OharaModel* m, int batch, int n_split, int n_workgroups) {
+  const int64_t b = ohara_persistent_barrier_offset(m, batch, n_split, n_workgroups);
+  const int ng = (n_workgroups + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP;
+  return b < 0 ? b : b + (int64_t)(ng + 2) * 64 * 4;
+}
+
+int64_t ohara_persistent_profile_offset(const OharaModel* m, int batch, int n_split, int n_workgroups) {
+  if (!m || batch < 1 || n_split != OHARA_MEGA_NS || n_workgroups < 1) return OHARA_EINVAL;
+  return (int64_t)mega_layout(m, batch, n_workgroups).prof;
 }
 
 int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s, void* workspace, int n_workgroups,
@@ -744,50 +923,42 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   if ((m->d_model & 7) || (m->d_ff & 7) || m->d_model > 1024) return OHARA_ESIZE;
   hipStream_t st = (hipStream_t)stream;
   char* ws = reinterpret_cast<char*>(workspace);
+  const MegaLayout L = mega_layout(m, s->batch, n_workgroups);
   MegaArgs a{};
   a.m = *m;
-  a.layers_dev = reinterpret_cast<const OharaLayer*>(ws);
-  ws += mega_al(sizeof(OharaLayer) * m->n_layers);
-  a.kcache_dev = reinterpret_cast<uint16_t* const*>(ws);
-  ws += mega_al(sizeof(void*) * m->n_layers);
-  a.vcache_dev = reinterpret_cast<uint16_t* const*>(ws);
-  ws += mega_al(sizeof(void*) * m->n_layers);
-  a.part_ml = reinterpret_cast<float*>(ws);
-  ws += mega_al((size_t)s->batch * m->n_heads * s->n_split * 2 * sizeof(float));
-  a.part_acc = reinterpret_cast<float*>(ws);
-  ws += mega_al((size_t)s->batch * m->n_heads * s->n_split * D * sizeof(float));
-  a.cand_val = reinterpret_cast<float*>(ws);
-  ws += mega_al((size_t)n_workgroups * s->batch * sizeof(float));
-  a.cand_idx = reinterpret_cast<int*>(ws);
-  ws += mega_al((size_t)n_workgroups * s->batch * sizeof(float));
-  unsigned long long* prof = reinterpret_cast<unsigned long long*>(ws);
-  ws += mega_al(OHARA_PROF_SLOTS * sizeof(unsigned long long));
-  a.bar = reinterpret_cast<unsigned int*>(ws);
+  a.layers_dev = reinterpret_cast<const OharaLayer*>(ws + L.layers);
+  a.kcache_dev = reinterpret_cast<uint16_t* const*>(ws + L.kptr);
+  a.vcache_dev = reinterpret_cast<uint16_t* const*>(ws + L.vptr);
+  a.xm = ws + L.xm; a.qm = ws + L.qm; a.am = ws + L.am; a.pm = reinterpret_cast<float*>(ws + L.pm);
+  a.xm_stride = L.xm_stride; a.qm_stride = L.qm_stride; a.am_stride = L.am_stride; a.pm_stride = L.pm_stride;
+  a.blk_x = L.blk_x; a.blk_a = L.blk_a;
+  a.cand_val = reinterpret_cast<float*>(ws + L.candv);
+  a.cand_idx = reinterpret_cast<int*>(ws + L.candi);
+  a.bar = reinterpret_cast<unsigned int*>(ws + L.bar);
   if (init_workspace) {
     // small synchronous copies: done once per (model, cache) binding, outside any capture
-    const size_t barb = mega_al(OHARA_BAR_WORDS(n_workgroups) * sizeof(unsigned int));
     if (hipMemcpyAsync((void*)a.layers_dev, m->layers, sizeof(OharaLayer) * m->n_layers, hipMemcpyHostToDevice, st) !=
             hipSuccess ||
         hipMemcpyAsync((void*)a.kcache_dev, s->kcache, sizeof(void*) * m->n_layers, hipMemcpyHostToDevice, st) !=
             hipSuccess ||
         hipMemcpyAsync((void*)a.vcache_dev, s->vcache, sizeof(void*) * m->n_layers, hipMemcpyHostToDevice, st) !=
             hipSuccess ||
-        hipMemsetAsync((void*)a.bar, 0, barb, st) != hipSuccess || hipStreamSynchronize(st) != hipSuccess)
+        hipMemsetAsync((void*)a.bar, 0, L.total - L.bar, st) != hipSuccess || hipStreamSynchronize(st) != hipSuccess)
       return OHARA_ELAUNCH;
     return OHARA_OK;
   }
-  a.B = s->batch; a.nsplit = s->n_split; a.valid_vocab = s->valid_vocab; a.hist_cap = s->hist_cap;
+  a.B = s->batch; a.valid_vocab = s->valid_vocab; a.hist_cap = s->hist_cap;
   a.select = select_greedy;
-  a.ids = s->ids; a.x = s->x; a.q = s->q; a.act = s->act; a.logits = s->logits;
+  a.ids = s->ids; a.logits = s->logits;
   a.step_state = s->step_state; a.history = s->history;
-  a.prof = s->prof_kernel == -2 ? prof : nullptr;  // -2: record per-phase clocks of workgroup 0
+  a.prof = s->prof_kernel == -2 ? reinterpret_cast<unsigned long long*>(ws + L.prof) : nullptr;
+  if (40 * m->n_layers + 16 > OHARA_PROF_SLOTS) a.prof = nullptr;
   a.spin_limit = spin_limit ? spin_limit : (1u << 19);
   const int kmax = m->d_model > m->d_ff ? m->d_model : m->d_ff;
   const int kmax2 = kmax > m->n_heads * D ? kmax : m->n_heads * D;
   const size_t xs_bytes = ((size_t)s->batch * (kmax2 + 8) * 2 + 255) & ~(size_t)255;
   const size_t smem = xs_bytes + 4096 + (size_t)(8 + 4 * D) * G * sizeof(float);
   if (smem > 160 * 1024) return OHARA_ESIZE;
-  if (9 * m->n_layers + 4 > OHARA_PROF_SLOTS) a.prof = nullptr;
   dim3 grid(n_workgroups), block(256);
 #define OHARA_MEGA(DD, GG)                                                                                  \
   do {                                                                                                      \
@@ -804,19 +975,6 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   else OHARA_MEGA(64, 4);
 #undef OHARA_MEGA
   return ohara_launch_status();
-}
-
-// Byte offset of the sticky barrier-error word (uint32) inside the workspace.
-int64_t ohara_persistent_error_offset(const OharaModel* m, int batch, int n_split, int n_workgroups) {
-  const int64_t b = ohara_persistent_barrier_offset(m, batch, n_split, n_workgroups);
-  const int ng = (n_workgroups + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP;
-  return b < 0 ? b : b + (int64_t)(ng + 2) * 64 * 4;
-}
-
-// Byte offset of the per-phase clock samples (uint64 x 256) inside the workspace.
-int64_t ohara_persistent_profile_offset(const OharaModel* m, int batch, int n_split, int n_workgroups) {
-  const int64_t b = ohara_persistent_barrier_offset(m, batch, n_split, n_workgroups);
-  return b < 0 ? b : b - (int64_t)mega_al(OHARA_PROF_SLOTS * sizeof(unsigned long long));
 }
 
 }  // extern "C"

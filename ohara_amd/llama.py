@@ -242,7 +242,7 @@ class Llama:
         """Context chunks per (sequence, KV head) so that decode attention launches about
         two workgroups per CU; a chunk is never shorter than 64 positions."""
         want = max(1, 512 // max(1, batch * self.kv_heads))
-        return max(1, min(want, self.config.max_sequence_length // 64, 64))
+        return max(1, min(want, self.config.max_sequence_length // 64, 32))
 
     def _get_buffers(self, batch: int, rows: int) -> _Buffers:
         key = (batch, rows)
@@ -434,7 +434,7 @@ class DecodeSession:
     def phase_clocks(self) -> torch.Tensor:
         """Shader-clock samples of workgroup 0 at the phase boundaries of the last step run
         with ``step(prof_kernel=-2)`` (measurement aid)."""
-        return self._pws[self._prof_off : self._prof_off + 4096].view(torch.int64).cpu()
+        return self._pws[self._prof_off : self._prof_off + 8192].view(torch.int64).cpu()
 
     def _room(self, n: int) -> None:
         if self._dst is None:
