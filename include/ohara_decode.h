@@ -124,6 +124,23 @@ int ohara_attn_cached_bf16(const uint16_t* q, const uint16_t* kcache, const uint
 int ohara_argmax_bf16(const uint16_t* logits, int ldl, int batch, int vocab, int valid_vocab, int64_t* next_ids,
                       int64_t* history, int hist_cap, int32_t* step_state, void* stream);
 
+/* ---- temperature / top-k / top-p sampling ------------------------------------------
+ * sample_next_token (ohara/chat_engine.py:51-82) and the nucleus branch of
+ * Inference.sampler (ohara/inference.py:46-64) for temperature > 0, fused into one
+ * launch, one workgroup per row:
+ *   x = logits / temperature, ids >= valid_vocab masked (:398-399); top_k > 0 keeps
+ *   x >= the k-th largest (ties survive, :66-69); p = softmax(x); 0 < top_p < 1 keeps the
+ *   smallest descending-sorted prefix whose preceding mass does not exceed top_p
+ *   (:72-81), renormalised; otherwise all of p in vocabulary order (:82).
+ * torch.multinomial is replaced by inverse-CDF sampling with the caller's uniform draw
+ * u[b] in [0,1); equal probabilities are ordered lowest id first.  Deterministic.
+ * logits: (batch, vocab) bf16 (logits_are_fp32 = 0) or fp32.  vocab <= 131072.
+ * history / step_state as in ohara_argmax_bf16.  temperature == 0 is ohara_argmax_bf16. */
+int ohara_sample_topk_topp(const void* logits, int logits_are_fp32, int ldl, int batch, int vocab,
+                           int valid_vocab, float temperature, int top_k, float top_p, const float* u,
+                           int64_t* out_ids, int64_t* history, int hist_cap, int32_t* step_state,
+                           void* stream);
+
 /* ---- the whole forward pass through the KV cache ---------------------------------
  * Llama.forward(x, kv_cache, position) (ohara/models/llama.py:279-323; Block.forward
  * :191-201) for seq_len new tokens per sequence, as a fixed sequence of the kernels

@@ -57,6 +57,7 @@ _PROTOS = {
     "ohara_attn_workspace_bytes": (_i64, [_i, _i, _i, _i, _i]),
     "ohara_attn_cached_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
     "ohara_argmax_bf16": (_i, [_p, _i, _i, _i, _i, _p, _p, _i, _p, _p]),
+    "ohara_sample_topk_topp": (_i, [_p, _i, _i, _i, _i, _i, _f, _i, _f, _p, _p, _p, _i, _p, _p]),
     "ohara_llama_forward": (_i, [C.POINTER(OharaModel), C.POINTER(OharaDecodeState), _i, _i, _i, _i, _i, _p]),
     "ohara_persistent_workspace_bytes": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),
     "ohara_persistent_barrier_offset": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),

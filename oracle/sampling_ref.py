@@ -73,6 +73,31 @@ def sample_next_token_ref(logits, temperature=0.8, top_p=0.95, top_k=0, u=None, 
     return (out, margin) if return_margin else out
 
 
+def candidate_cdf_ref(logits, temperature, top_p, top_k, valid_vocab=None):
+    """Ids in the order the draw walks them and their cumulative distribution (fp64, ends
+    at 1): the sorted, filtered, renormalised prefix when nucleus filtering is active
+    (chat_engine.py:72-81), the vocabulary-ordered probabilities otherwise (:82).
+    logits: (B, S, V).  Returns (ids (B, n), cdf (B, n)); dropped entries have cdf 1."""
+    x = logits[:, -1].float()
+    if valid_vocab is not None and valid_vocab < x.size(-1):
+        x = x.clone()
+        x[:, valid_vocab:] = float("-inf")
+    x = x / temperature
+    if top_k > 0:
+        k = min(top_k, x.size(-1))
+        thr = torch.sort(x, dim=-1, descending=True).values[:, k - 1 : k]
+        x = x.masked_fill(x < thr, float("-inf"))
+    probs = torch.softmax(x, dim=-1)
+    if 0.0 < top_p < 1.0:
+        sp, si = torch.sort(probs, dim=-1, descending=True, stable=True)
+        cum = torch.cumsum(sp, dim=-1)
+        sp = sp.masked_fill(cum - sp > top_p, 0.0)
+    else:
+        sp, si = probs, torch.arange(probs.size(-1)).expand_as(probs)
+    cdf = torch.cumsum(sp.double(), dim=-1)
+    return si, cdf / cdf[:, -1:]
+
+
 def kept_set_ref(logits_row: torch.Tensor, temperature, top_p, top_k):
     """The candidate ids and renormalised probabilities the reference would hand
     to multinomial for one row, in fp64, by direct loops (small V only).  A second,

@@ -1,0 +1,129 @@
+"""Fused sampler (C ABI: ohara_sample_topk_topp / ohara_argmax_bf16) against the CPU oracle
+and the known answers of the reference's own tests (tests/test_inference.py:45-48,
+tests/test_chat.py:355-390).
+
+Stochastic parity: both sides consume the same uniform draw u by inverse CDF over the same
+distribution.  The kernel sums the sorted probabilities sequentially in fp32 (as
+torch.cumsum does), the oracle's reference CDF is fp64, so the check is: u lies inside the
+CDF interval of the token the kernel returned, widened by 5e-5 (fp32 summation error over
+up to 65536 terms, which also moves the nucleus boundary by a few tail tokens), and the token is identical to the oracle's wherever u is further than
+that from an interval boundary.
+"""
+
+import pytest
+import torch
+
+from oracle.sampling_ref import candidate_cdf_ref, inference_sampler_ref, kept_set_ref, sample_next_token_ref
+
+pytestmark = pytest.mark.gpu
+
+
+def test_reference_known_answers(cuda):
+    from ohara_amd.sampling import SamplingConfig, inference_sampler, sample_next_token
+
+    t = sample_next_token(torch.tensor([[[0.1, 5.0, 0.2, 0.3]]]).to(cuda), SamplingConfig(temperature=0.0))
+    assert int(t.item()) == 1 and t.shape == (1, 1) and t.dtype == torch.int64
+    t = inference_sampler(torch.tensor([[[0.1, 0.2, 0.9]]]).to(cuda), temperature=0.0)
+    assert int(t.item()) == 2
+    # default Inference sampler (temperature 1, top_p 0) is greedy
+    assert int(inference_sampler(torch.tensor([[[0.1, 0.2, 0.9]]]).to(cuda)).item()) == 2
+    # top-k = 2 never leaks outside {0, 1}
+    logits = torch.tensor([[[10.0, 9.0, -50.0, -60.0]]]).to(cuda)
+    cfg = SamplingConfig(temperature=1.0, top_p=1.0, top_k=2)
+    seen = {int(sample_next_token(logits, cfg).item()) for _ in range(200)}
+    assert seen <= {0, 1} and len(seen) == 2
+    # a tiny top_p still keeps the most likely token
+    logits = torch.tensor([[[20.0, 0.0, 0.0, 0.0]]]).to(cuda)
+    cfg = SamplingConfig(temperature=1.0, top_p=0.01)
+    assert {int(sample_next_token(logits, cfg).item()) for _ in range(50)} == {0}
+    # seeded sampling is reproducible
+    logits = torch.randn(1, 1, 32).to(cuda)
+    cfg = SamplingConfig(temperature=1.0, top_p=0.9)
+    a = sample_next_token(logits, cfg, torch.Generator(device=cuda).manual_seed(7))
+    b = sample_next_token(logits, cfg, torch.Generator(device=cuda).manual_seed(7))
+    assert int(a.item()) == int(b.item())
+    # CPU logits and a CPU generator are accepted too (the result comes back on the CPU)
+    c = sample_next_token(logits.cpu(), cfg, torch.Generator().manual_seed(7))
+    assert c.device.type == "cpu"
+    for kw in ({"temperature": -1.0}, {"top_p": 1.5}, {"top_k": -1}, {"max_new_tokens": 0}):
+        with pytest.raises(ValueError):
+            SamplingConfig(**kw)
+
+
+CASES = [
+    # V, B, temperature, top_k, top_p, logit std, dtype
+    (32, 8, 1.0, 0, 0.9, 1.0, torch.float32),
+    (1000, 16, 0.8, 50, 0.9, 2.0, torch.bfloat16),
+    (1000, 16, 1.3, 0, 1.0, 2.0, torch.float32),
+    (1000, 16, 0.7, 7, 0.0, 2.0, torch.bfloat16),
+    (65536, 8, 0.8, 50, 0.9, 0.55, torch.bfloat16),    # the headline sampling setting
+    (65536, 4, 1.0, 0, 0.95, 3.0, torch.bfloat16),     # peaked, nucleus only
+    (65536, 3, 1.0, 0, 0.9, 0.5, torch.bfloat16),      # flat: tens of thousands kept (multi-round path)
+    (65536, 3, 1.0, 5000, 0.5, 0.5, torch.float32),
+    (32000, 4, 0.8, 0, 0.0, 1.0, torch.bfloat16),      # vocabulary-order draw
+    (50, 5, 1.0, 100, 0.3, 1.0, torch.float32),        # top_k larger than the vocabulary
+]
+
+
+@pytest.mark.parametrize("V,B,T,k,p,std,dtype", CASES)
+def test_sampler_matches_oracle(cuda, V, B, T, k, p, std, dtype):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(V + B + k)
+    logits = (torch.randn(B, V, generator=g) * std).to(dtype)
+    tol = 5e-5
+    for trial in range(4):
+        u = torch.rand(B, generator=g)
+        if trial == 0:
+            u[0] = 0.0
+            u[-1] = 0.999999
+        want, margin = sample_next_token_ref(logits.unsqueeze(1), T, p, k, u=u, return_margin=True)
+        ids, cdf = candidate_cdf_ref(logits.unsqueeze(1), T, p, k)
+        got = ops.sample_topk_topp(logits.to(cuda), T, k, p, u.to(cuda)).cpu()
+        for b in range(B):
+            j = int((ids[b] == int(got[b])).nonzero()[0])
+            lo = float(cdf[b, j - 1]) if j > 0 else 0.0
+            hi = float(cdf[b, j])
+            assert hi > lo, (b, "sampled a token outside the kept set")
+            assert lo - tol <= float(u[b]) <= hi + tol, (b, int(got[b]), lo, hi, float(u[b]))
+            if float(margin[b]) > tol:
+                assert int(got[b]) == int(want[b, 0]), (b, int(got[b]), int(want[b, 0]), float(margin[b]))
+
+
+def test_sampler_valid_vocab_and_ties(cuda):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(9)
+    V, B = 4096, 6
+    logits = torch.randn(B, V, generator=g).to(torch.bfloat16)  # bf16: many exactly equal values
+    logits[:, 3000:] += 8.0                                     # the padded region would dominate
+    u = torch.rand(B, generator=g)
+    want = sample_next_token_ref(logits.unsqueeze(1), 0.9, 0.92, 40, u=u, valid_vocab=3000)
+    got = ops.sample_topk_topp(logits.to(cuda), 0.9, 40, 0.92, u.to(cuda), valid_vocab=3000).cpu()
+    assert torch.equal(got, want[:, 0]) and int(got.max()) < 3000
+    # the kept set of the direct fp64 restatement contains every sampled id
+    for b in range(B):
+        kept, _ = kept_set_ref(logits[b, :3000], 0.9, 0.92, 40)
+        assert int(got[b]) in kept
+    # exact ties: four equal maxima, top_k = 1 keeps all four; u picks among them in id order
+    row = torch.full((1, 64), -3.0)
+    row[0, [5, 17, 33, 60]] = 2.0
+    for uu, expect in ((0.0, 5), (0.26, 17), (0.51, 33), (0.99, 60)):
+        got = ops.sample_topk_topp(row.to(cuda), 1.0, 1, 1.0, torch.tensor([uu], device=cuda))
+        assert int(got.item()) == expect
+        got = ops.sample_topk_topp(row.to(cuda), 1.0, 1, 0.999, torch.tensor([uu], device=cuda))
+        assert int(got.item()) == expect
+
+
+def test_inference_sampler_matches_oracle(cuda):
+    from ohara_amd.sampling import inference_sampler
+
+    g = torch.Generator().manual_seed(4)
+    logits = torch.randn(5, 3, 777, generator=g) * 2
+    u = torch.rand(5, generator=g)
+    want = inference_sampler_ref(logits, temperature=0.7, top_p=0.8, u=u)
+    got = inference_sampler(logits.to(cuda), temperature=0.7, top_p=0.8, u=u).cpu()
+    assert torch.equal(got, want)
+    want = inference_sampler_ref(logits, temperature=0.7, top_p=0.0, u=u)
+    got = inference_sampler(logits.to(cuda), temperature=0.7, top_p=0.0, u=u).cpu()
+    assert torch.equal(got, want)
