@@ -213,6 +213,8 @@ class Llama:
 
     # -- reference surface -------------------------------------------------------
 
+    supports_last_only = True  # forward(..., last_only=True) computes the last row of logits only
+
     def eval(self):
         return self
 
