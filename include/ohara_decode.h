@@ -141,6 +141,37 @@ int ohara_sample_topk_topp(const void* logits, int logits_are_fp32, int ldl, int
                            int64_t* out_ids, int64_t* history, int hist_cap, int32_t* step_state,
                            void* stream);
 
+/* ---- BitNet-b1.58 BitLinear (ternary weights x int8 activations, int32 accumulate) ------
+ * Integer form of BitLinear.forward (experiments/bitnet/bitnet.py:29-59):
+ *   x_hat = RMSNorm(x; norm_w, eps) in bf16 (:49,53); s = 127 / max(max|x_hat|, 1e-5) and
+ *   q = clamp(rint(x_hat * s), -128, 127) per row (:30-33); acc[n] = sum_k q[k] * T[n,k] in
+ *   int32; y = bf16((float(acc) / s) * gamma) [+ resid]  (:58-59, bias dropped).
+ * T in {-1,0,1} and gamma = max(mean|W|, 1e-5) come from weight_quant (:37-43), done once at
+ * load time.  ohara_bitlinear_pack_ternary turns T (n, k) int8 row-major into the packed
+ * 2-bit stream the kernels read (16 weights per dword; size through *bytes when dst is NULL).
+ * ohara_act_quant_int8 and ohara_gemv_ternary_i8 are the two halves; ohara_bitlinear_bf16
+ * fuses them (k <= 6144).  acc_out, when given, receives the raw int32 accumulators - the
+ * quantity that must match a CPU int32 matmul bit for bit.  ldq must be a multiple of 16. */
+int ohara_bitlinear_pack_ternary(const int8_t* t, int n, int k, int ldt, uint32_t* dst, int64_t* bytes, void* stream);
+int ohara_act_quant_int8(const uint16_t* x, int ldx, const uint16_t* norm_w, float eps, int rows, int k, int8_t* q,
+                         int ldq, float* s, int32_t* sumq, void* stream);
+int ohara_gemv_ternary_i8(const int8_t* q, int ldq, const float* s, const int32_t* sumq, const uint32_t* wp, int n,
+                          int k, float gamma, int rows, const uint16_t* resid, int ldr, uint16_t* out, int ldo,
+                          int32_t* acc_out, int ldacc, void* stream);
+int ohara_bitlinear_bf16(const uint16_t* x, int ldx, const uint16_t* norm_w, float eps, const uint32_t* wp, int n, int k,
+                         float gamma, int rows, const uint16_t* resid, int ldr, uint16_t* out, int ldo, int32_t* acc_out,
+                         int ldacc, void* stream);
+
+/* out = bf16(bf16(silu(gate)) * up), elementwise over n values (ohara/modules/mlp.py:152). */
+int ohara_silu_mul_bf16(const uint16_t* gate, const uint16_t* up, uint16_t* out, int64_t n, void* stream);
+
+/* Rotary on q (in place) and on k, and append of the rotated k and of v to the cache, for
+ * projections that were computed unfused (ohara/embeddings_pos/rotary.py:55-93,
+ * ohara/modules/kv_cache.py:104-105).  q: (batch*seq_len, h*dh), k/v: (batch*seq_len, h_kv*dh). */
+int ohara_rope_append_bf16(uint16_t* q, const uint16_t* k, const uint16_t* v, int batch, int seq_len, int h, int h_kv,
+                           int dh, const uint16_t* cos, const uint16_t* sin, int pos, const int32_t* pos_dev,
+                           uint16_t* kcache, uint16_t* vcache, int t_max, void* stream);
+
 /* ---- the whole forward pass through the KV cache ---------------------------------
  * Llama.forward(x, kv_cache, position) (ohara/models/llama.py:279-323; Block.forward
  * :191-201) for seq_len new tokens per sequence, as a fixed sequence of the kernels

@@ -58,6 +58,12 @@ _PROTOS = {
     "ohara_attn_cached_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
     "ohara_argmax_bf16": (_i, [_p, _i, _i, _i, _i, _p, _p, _i, _p, _p]),
     "ohara_sample_topk_topp": (_i, [_p, _i, _i, _i, _i, _i, _f, _i, _f, _p, _p, _p, _i, _p, _p]),
+    "ohara_bitlinear_pack_ternary": (_i, [_p, _i, _i, _i, _p, C.POINTER(_i64), _p]),
+    "ohara_act_quant_int8": (_i, [_p, _i, _p, _f, _i, _i, _p, _i, _p, _p, _p]),
+    "ohara_gemv_ternary_i8": (_i, [_p, _i, _p, _p, _p, _i, _i, _f, _i, _p, _i, _p, _i, _p, _i, _p]),
+    "ohara_bitlinear_bf16": (_i, [_p, _i, _p, _f, _p, _i, _i, _f, _i, _p, _i, _p, _i, _p, _i, _p]),
+    "ohara_silu_mul_bf16": (_i, [_p, _p, _p, _i64, _p]),
+    "ohara_rope_append_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _i, _p, _p, _p, _i, _p]),
     "ohara_llama_forward": (_i, [C.POINTER(OharaModel), C.POINTER(OharaDecodeState), _i, _i, _i, _i, _i, _p]),
     "ohara_persistent_workspace_bytes": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),
     "ohara_persistent_barrier_offset": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),

@@ -205,3 +205,81 @@ def sample_topk_topp(logits: torch.Tensor, temperature: float, top_k: int, top_p
         "sample_topk_topp",
     )
     return out
+
+
+# ---- BitLinear ---------------------------------------------------------------------------------
+
+
+class PackedTernary:
+    """Ternary weight (N, K) in the kernels' 2-bit layout with its per-tensor scale."""
+
+    __slots__ = ("data", "n", "k", "gamma")
+
+    def __init__(self, data, n, k, gamma):
+        self.data, self.n, self.k, self.gamma = data, n, k, float(gamma)
+
+
+def pack_ternary(t: torch.Tensor, gamma: float) -> PackedTernary:
+    _need(t, torch.int8, "t")
+    n, k = t.shape
+    nbytes = C.c_int64(0)
+    check(lib().ohara_bitlinear_pack_ternary(0, n, k, k, 0, C.byref(nbytes), 0), "pack_ternary size")
+    dst = torch.empty(nbytes.value // 4, dtype=torch.int32, device=t.device)
+    check(lib().ohara_bitlinear_pack_ternary(_ptr(t), n, k, k, _ptr(dst), None, _stream()), "pack_ternary")
+    return PackedTernary(dst, n, k, gamma)
+
+
+def act_quant(x: torch.Tensor, norm_w: torch.Tensor, eps: float = 1e-5):
+    """(rows, K) bf16 -> q int8 (rows, K padded to 16), s fp32 (rows,), sum q int32 (rows,)."""
+    _need(x, BF16, "x")
+    rows, k = x.shape
+    ldq = (k + 15) // 16 * 16
+    q = torch.zeros(rows, ldq, dtype=torch.int8, device=x.device)
+    s = torch.empty(rows, dtype=torch.float32, device=x.device)
+    sq = torch.empty(rows, dtype=torch.int32, device=x.device)
+    check(lib().ohara_act_quant_int8(_ptr(x), x.stride(0), _ptr(norm_w), eps, rows, k, _ptr(q), ldq, _ptr(s), _ptr(sq),
+                                     _stream()), "act_quant")
+    return q, s, sq
+
+
+def gemv_ternary(q, s, sumq, w: PackedTernary, residual=None, out=None, want_acc=False):
+    rows = q.shape[0]
+    if out is None:
+        out = torch.empty(rows, w.n, dtype=BF16, device=q.device)
+    acc = torch.empty(rows, w.n, dtype=torch.int32, device=q.device) if want_acc else None
+    check(lib().ohara_gemv_ternary_i8(_ptr(q), q.stride(0), _ptr(s), _ptr(sumq), _ptr(w.data), w.n, w.k, w.gamma, rows,
+                                      _ptr(residual), 0 if residual is None else residual.stride(0), _ptr(out),
+                                      out.stride(0), _ptr(acc), w.n, _stream()), "gemv_ternary")
+    return (out, acc) if want_acc else out
+
+
+def bitlinear(x, norm_w, w: PackedTernary, eps=1e-5, residual=None, out=None, want_acc=False):
+    """Fused BitLinear.forward on rows of x (rows, K) bf16."""
+    _need(x, BF16, "x")
+    rows, k = x.shape
+    if k != w.k:
+        raise ValueError(f"x has {k} columns, weight expects {w.k}")
+    if out is None:
+        out = torch.empty(rows, w.n, dtype=BF16, device=x.device)
+    acc = torch.empty(rows, w.n, dtype=torch.int32, device=x.device) if want_acc else None
+    check(lib().ohara_bitlinear_bf16(_ptr(x), x.stride(0), _ptr(norm_w), eps, _ptr(w.data), w.n, w.k, w.gamma, rows,
+                                     _ptr(residual), 0 if residual is None else residual.stride(0), _ptr(out),
+                                     out.stride(0), _ptr(acc), w.n, _stream()), "bitlinear")
+    return (out, acc) if want_acc else out
+
+
+def silu_mul(gate, up, out=None):
+    _need(gate, BF16, "gate")
+    _need(up, BF16, "up")
+    if out is None:
+        out = torch.empty_like(gate)
+    check(lib().ohara_silu_mul_bf16(_ptr(gate), _ptr(up), _ptr(out), gate.numel(), _stream()), "silu_mul")
+    return out
+
+
+def rope_append(q, k, v, batch, seq_len, h, h_kv, dh, cos, sin, pos, kcache, vcache, pos_dev=None):
+    """In-place rotary on q (rows, h*dh); rotated k and v appended to the cache."""
+    check(lib().ohara_rope_append_bf16(_ptr(q), _ptr(k), _ptr(v), batch, seq_len, h, h_kv, dh, _ptr(cos), _ptr(sin),
+                                       int(pos), _ptr(pos_dev), _ptr(kcache), _ptr(vcache), kcache.shape[1], _stream()),
+          "rope_append")
+    return q

@@ -1,0 +1,129 @@
+"""BitLinear integer kernels (C ABI: ohara_bitlinear_pack_ternary / ohara_act_quant_int8 /
+ohara_gemv_ternary_i8 / ohara_bitlinear_bf16) against the CPU oracle.
+
+Contract: the int32 accumulators are BIT-EXACT against a CPU int32 matmul of the same int8
+activations and ternary weights.  The float parts (RMSNorm before quantisation, the final
+scale) follow the bf16 tolerance of the other kernels.
+"""
+
+import pytest
+import torch
+
+from oracle import bitlinear_ref as BL
+from oracle import llama_ref as R
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+
+
+@pytest.mark.parametrize("rows,N,K", [(1, 2048, 2048), (8, 5632, 2048), (3, 2048, 5632), (17, 48, 96), (70, 100, 520),
+                                      (2, 16, 32)])
+def test_ternary_gemv_accumulators_bit_exact(cuda, rows, N, K):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(rows + N + K)
+    t = torch.randint(-1, 2, (N, K), generator=g, dtype=torch.int8)
+    q = torch.randint(-128, 128, (rows, K), generator=g, dtype=torch.int8)
+    s = (torch.rand(rows, generator=g) * 50 + 1).float()
+    gamma = 0.0213
+    want_acc = BL.int_accumulate(q, t)
+    ldq = (K + 15) // 16 * 16
+    qd = torch.zeros(rows, ldq, dtype=torch.int8)
+    qd[:, :K] = q
+    sumq = q.to(torch.int32).sum(-1).to(torch.int32)
+    w = ops.pack_ternary(t.to(cuda), gamma)
+    res = torch.randn(rows, N, generator=g).to(BF)
+    out, acc = ops.gemv_ternary(qd.to(cuda), s.to(cuda), sumq.to(cuda), w, residual=res.to(cuda), want_acc=True)
+    assert torch.equal(acc.cpu(), want_acc), "int32 accumulators must be bit-exact"
+    want = res + ((want_acc.float() / s[:, None]) * gamma).to(BF)
+    assert torch.equal(out.cpu(), want)
+
+
+def test_act_quant_matches_oracle(cuda):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(0)
+    for rows, K in ((5, 2048), (3, 5632), (4, 100)):
+        x = (torch.randn(rows, K, generator=g) * 2).to(BF)
+        nw = (1 + 0.2 * torch.randn(K, generator=g)).to(BF)
+        q_ref, s_ref = BL.activation_quant(R.rms_norm(x, nw))
+        q, s, sq = ops.act_quant(x.to(cuda), nw.to(cuda))
+        q = q.cpu()[:, :K]
+        # the norm's fp32 reduction order can flip a bf16 rounding of x_hat, i.e. move a q by one
+        diff = (q.int() - q_ref.int()).abs()
+        assert int(diff.max()) <= 1 and float((diff > 0).float().mean()) < 5e-3
+        torch.testing.assert_close(s.cpu(), s_ref[:, 0], rtol=1e-2, atol=0)
+        assert torch.equal(sq.cpu(), q.int().sum(-1).to(torch.int32))
+    # closed forms: equal magnitudes quantise to +-127; half-way cases round to even
+    x = torch.tensor([[0.5, -0.5, 0.5, -0.5] * 8]).to(BF)
+    q, s, _ = ops.act_quant(x.to(cuda), torch.ones(32, dtype=BF, device=cuda))
+    assert q.cpu()[0, :4].tolist() == [127, -127, 127, -127]
+
+
+@pytest.mark.parametrize("rows,N,K", [(1, 2048, 2048), (8, 2048, 5632), (33, 64, 128)])
+def test_fused_bitlinear(cuda, rows, N, K):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(N + K)
+    x = torch.randn(rows, K, generator=g).to(BF)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(BF)
+    wfloat = torch.randn(N, K, generator=g) * 0.03
+    t, gamma = BL.weight_ternarize(wfloat)
+    w = ops.pack_ternary(t.to(cuda), float(gamma))
+    out, acc = ops.bitlinear(x.to(cuda), nw.to(cuda), w, want_acc=True)
+    # accumulators: exact against the kernel's own quantised activations
+    q, s, sq = ops.act_quant(x.to(cuda), nw.to(cuda))
+    assert torch.equal(acc.cpu(), BL.int_accumulate(q.cpu()[:, :K], t))
+    # end to end against the oracle (which quantises on its own): bf16-level agreement
+    want = BL.bitlinear_forward(x, nw, t, gamma)
+    scale = want.float().abs().max().item()
+    d = (out.cpu().float() - want.float()).abs()
+    assert d.max().item() <= 3e-2 * scale and d.mean().item() <= 3e-3 * scale
+    # and against the reference's float fake-quant formulation (bitnet.py:29-59)
+    fq = BL.fake_quant_forward(x.float(), nw.float(), wfloat)
+    assert (out.cpu().float() - fq).abs().mean().item() <= 1e-2 * scale
+
+
+def test_ternarize_matches_oracle(cuda):
+    from ohara_amd.bitnet import ternarize
+
+    w = torch.randn(64, 96, generator=torch.Generator().manual_seed(1)) * 0.04
+    t, gamma = ternarize(w)
+    t2, g2 = BL.weight_ternarize(w)
+    assert torch.equal(t, t2) and abs(gamma - float(g2)) < 1e-9
+
+
+def test_bitnet_llama_parity(cuda):
+    """A small ternary Llama (d 256, 3 layers, 2 heads x 128, GQA off): prefill + cached steps
+    against the oracle; greedy tokens up to a near-tie."""
+    from ohara_amd.bitnet import BitLlama
+    from ohara_amd.llama import Config
+
+    kw = dict(vocab_size=320, hidden_size=256, intermediate_size=512, num_attention_heads=2,
+              num_key_value_heads=0, num_hidden_layers=3, max_sequence_length=64, rope_theta=10000.0)
+    rcfg = R.RefConfig(**kw)
+    w = BL.init_ternary_weights(rcfg, seed=2, dtype=BF, gamma=0.05)
+    ref = R.RefLlama(rcfg, w)
+    model = BitLlama(Config(**kw), w, device=cuda)
+    ids = torch.randint(0, 320, (2, 9), generator=torch.Generator().manual_seed(0))
+    rc, cache = ref.build_kv_cache(2), model.build_kv_cache(2)
+    want = ref(ids, rc, 0)
+    got = model(ids.to(cuda), cache, 0)
+    scale = want.float().abs().max().item()
+
+    def close(a, b):
+        d = (a.float().cpu() - b.float()).abs()
+        # int8 activation quantisation turns a one-ulp bf16 flip into a full quantisation step,
+        # so the ternary model's noise floor is several times the bf16 model's
+        assert d.max().item() <= 8e-2 * scale and d.mean().item() <= 1e-2 * scale, (d.max().item(), d.mean().item(), scale)
+
+    close(got, want)
+    nxt = want[:, -1].float().argmax(-1, keepdim=True)
+    for step in range(3):
+        want = ref(nxt, rc, 9 + step)
+        got = model(nxt.to(cuda), cache, 9 + step)
+        close(got, want)
+        nxt = want[:, -1].float().argmax(-1, keepdim=True)
+    assert cache[0].length == 12
+    toks = model.generate_greedy(ids.to(cuda), 6).cpu()
+    assert toks.shape == (2, 6)
