@@ -172,6 +172,37 @@ int ohara_rope_append_bf16(uint16_t* q, const uint16_t* k, const uint16_t* v, in
                            int dh, const uint16_t* cos, const uint16_t* sin, int pos, const int32_t* pos_dev,
                            uint16_t* kcache, uint16_t* vcache, int t_max, void* stream);
 
+/* ---- grouped mixture-of-experts feed-forward (eval mode) -------------------------------------
+ * GroupedMoE.forward (ohara/modules/moe_grouped.py:209-228) in five launches:
+ *  ohara_moe_route_topk     _route (:122-147) from the bf16 router logits (n_tokens, n_experts):
+ *                           experts = top-k of logits [+ router_bias when biased_topk] with ties
+ *                           to the lowest id; weights = softmax (or sigmoid, optionally normalised)
+ *                           of the k selected unbiased logits, cast to bf16.  k <= 16, E <= 1024.
+ *  ohara_moe_sort_pairs     the stable sort by expert of :161-168: offsets (E+1), pair_of[sorted
+ *                           position] = token*k + slot, pos_of = its inverse.  n_pairs <= 65536.
+ *  ohara_moe_experts_gate_up  act[sorted position] = bf16(silu(bf16(x W_gate[e]))) * bf16(x W_up[e])
+ *  ohara_moe_experts_down     y[sorted position]   = bf16(bf16(act W_down[e]) * weight)   (:175-181)
+ *                           expert weights: per expert, rows packed by ohara_pack_rows_bf16
+ *                           (gate/up rows interleaved with ohara_swiglu_perm), experts
+ *                           expert_stride_bytes apart.
+ *  ohara_moe_combine        out[token] = resid + (sum over its experts in ascending expert id,
+ *                           each add rounded to bf16 (:184) + shared[token]); shared / resid may
+ *                           be NULL. */
+int ohara_moe_route_topk(const uint16_t* router_logits, int ldl, const uint16_t* router_bias, int n_tokens, int n_experts,
+                         int k, int biased_topk, int gate_sigmoid, int normalize, int32_t* expert_idx,
+                         uint16_t* expert_w, void* stream);
+int ohara_moe_sort_pairs(const int32_t* expert_idx, int n_pairs, int n_experts, int32_t* offsets, int32_t* pair_of,
+                         int32_t* pos_of, void* stream);
+int ohara_moe_experts_gate_up(const uint16_t* x, int ldx, const uint16_t* wp_gate_up, int64_t expert_stride_bytes,
+                              int n_experts, int hidden, int d, int k, const int32_t* offsets, const int32_t* pair_of,
+                              uint16_t* act, int ld_act, void* stream);
+int ohara_moe_experts_down(const uint16_t* act, int ld_act, const uint16_t* wp_down, int64_t expert_stride_bytes,
+                           int n_experts, int d, int hidden, int k, const int32_t* offsets, const int32_t* pair_of,
+                           const uint16_t* expert_w, uint16_t* y, int ldy, void* stream);
+int ohara_moe_combine(const uint16_t* y, int ldy, const int32_t* expert_idx, const int32_t* pos_of, int n_tokens, int k,
+                      const uint16_t* shared, int ld_shared, const uint16_t* resid, int ldr, uint16_t* out, int ldo, int d,
+                      void* stream);
+
 /* ---- the whole forward pass through the KV cache ---------------------------------
  * Llama.forward(x, kv_cache, position) (ohara/models/llama.py:279-323; Block.forward
  * :191-201) for seq_len new tokens per sequence, as a fixed sequence of the kernels

@@ -64,6 +64,11 @@ _PROTOS = {
     "ohara_bitlinear_bf16": (_i, [_p, _i, _p, _f, _p, _i, _i, _f, _i, _p, _i, _p, _i, _p, _i, _p]),
     "ohara_silu_mul_bf16": (_i, [_p, _p, _p, _i64, _p]),
     "ohara_rope_append_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _i, _p, _p, _p, _i, _p]),
+    "ohara_moe_route_topk": (_i, [_p, _i, _p, _i, _i, _i, _i, _i, _i, _p, _p, _p]),
+    "ohara_moe_sort_pairs": (_i, [_p, _i, _i, _p, _p, _p, _p]),
+    "ohara_moe_experts_gate_up": (_i, [_p, _i, _p, _i64, _i, _i, _i, _i, _p, _p, _p, _i, _p]),
+    "ohara_moe_experts_down": (_i, [_p, _i, _p, _i64, _i, _i, _i, _i, _p, _p, _p, _p, _i, _p]),
+    "ohara_moe_combine": (_i, [_p, _i, _p, _p, _i, _i, _p, _i, _p, _i, _p, _i, _i, _p]),
     "ohara_llama_forward": (_i, [C.POINTER(OharaModel), C.POINTER(OharaDecodeState), _i, _i, _i, _i, _i, _p]),
     "ohara_persistent_workspace_bytes": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),
     "ohara_persistent_barrier_offset": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),

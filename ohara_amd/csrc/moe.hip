@@ -1,0 +1,322 @@
+// Grouped mixture-of-experts feed-forward for decode (eval mode of GroupedMoE,
+// ohara/modules/moe_grouped.py:122-228; same routing as the loop variant ohara/modules/moe.py:65-127).
+//
+//   route    logits = float(bf16 router Linear) (:126); experts = first k of top-(k+1) of
+//            logits + router_bias (:129-133) or plain top-k (:135), ties to the lowest id;
+//            weights = softmax over the k selected UNBIASED logits (:140-142) or sigmoid,
+//            optionally normalised (:144-146); cast to bf16 (:217)
+//   sort     (token, slot) pairs grouped by expert, token order kept inside an expert (the
+//            stable argsort + bincount + cumsum of :165-168), as a counting sort in LDS
+//   experts  per expert e and its pairs: hidden = bf16(silu(bf16(x W_gate[e]))) * bf16(x W_up[e]),
+//            y = bf16(bf16(hidden W_down[e]) * weight) (:175-181) - the expert weights are
+//            streamed once per 16-token column tile through the same packed MFMA tiles as the
+//            dense projections (at ~8 tokens per expert this is a weight stream, not a GEMM)
+//   combine  out[token] = sum over its experts in ascending expert id, each add rounded to bf16
+//            (index_add_ in the activation dtype, :184), + shared expert (:206-207,219-220),
+//            + residual (ohara/models/llama.py:200)
+#include "common.h"
+
+namespace {
+
+// ---- routing ---------------------------------------------------------------------------------
+// one wave per token; E <= 1024 experts, k <= 16
+__global__ __launch_bounds__(256) void moe_route_kernel(const bf16_t* logits, int ldl, const bf16_t* bias, int N, int E,
+                                                        int k, int biased, int sigmoid, int normalize, int32_t* idx,
+                                                        bf16_t* w) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = blockIdx.x * 4 + wave;
+  if (n >= N) return;
+  constexpr int MAXPL = 16;  // experts per lane
+  float sel[MAXPL], raw[MAXPL];
+#pragma unroll
+  for (int i = 0; i < MAXPL; ++i) {
+    const int e = i * 64 + lane;
+    if (e < E) {
+      raw[i] = bf2f(logits[(size_t)n * ldl + e]);
+      sel[i] = biased ? raw[i] + bf2f(bias[e]) : raw[i];
+    } else {
+      raw[i] = 0.f;
+      sel[i] = -INFINITY;
+    }
+  }
+  float chosen_raw[16];
+  int chosen_id[16];
+  for (int j = 0; j < k; ++j) {
+    // lane-local best (lowest id on ties), then across the wave
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < MAXPL; ++i) {
+      const int e = i * 64 + lane;
+      if (e < E && (sel[i] > bv || (sel[i] == bv && e < bi))) {
+        bv = sel[i];
+        bi = e;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, WAVE);
+      const int oi = __shfl_xor(bi, o, WAVE);
+      if (ov > bv || (ov == bv && oi < bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    // fetch the unbiased logit of the winner and retire it
+    float r = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXPL; ++i)
+      if (i * 64 + lane == bi) {
+        r = raw[i];
+        sel[i] = -INFINITY;
+      }
+    r = __shfl(r, bi & 63, WAVE);
+    chosen_raw[j] = r;
+    chosen_id[j] = bi;
+  }
+  if (lane == 0) {
+    float wts[16];
+    if (!sigmoid) {
+      float m = -INFINITY;
+      for (int j = 0; j < k; ++j) m = fmaxf(m, chosen_raw[j]);
+      float z = 0.f;
+      for (int j = 0; j < k; ++j) {
+        wts[j] = expf(chosen_raw[j] - m);
+        z += wts[j];
+      }
+      for (int j = 0; j < k; ++j) wts[j] /= z;
+    } else {
+      float z = 0.f;
+      for (int j = 0; j < k; ++j) {
+        wts[j] = 1.0f / (1.0f + expf(-chosen_raw[j]));
+        z += wts[j];
+      }
+      if (normalize) {
+        z = fmaxf(z, 1e-9f);
+        for (int j = 0; j < k; ++j) wts[j] /= z;
+      }
+    }
+    for (int j = 0; j < k; ++j) {
+      idx[(size_t)n * k + j] = chosen_id[j];
+      w[(size_t)n * k + j] = f2bf(wts[j]);
+    }
+  }
+}
+
+// ---- counting sort of the (token, slot) pairs by expert -----------------------------------------
+// offs[e] .. offs[e+1]: pairs of expert e, in token order; pair_of[sorted position] = n*k + j;
+// pos_of[n*k + j] = sorted position.  One workgroup; N*k <= 65536, E <= 1024.
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int32_t* idx, int NK, int E, int32_t* offs, int32_t* pair_of,
+                                                        int32_t* pos_of) {
+  __shared__ int cnt[1025];
+  const int tid = threadIdx.x;
+  for (int e = tid; e <= E; e += 1024) cnt[e] = 0;
+  __syncthreads();
+  for (int p = tid; p < NK; p += 1024) atomicAdd(&cnt[idx[p]], 1);
+  __syncthreads();
+  if (tid == 0) {
+    int run = 0;
+    for (int e = 0; e < E; ++e) {
+      const int c = cnt[e];
+      cnt[e] = run;
+      offs[e] = run;
+      run += c;
+    }
+    cnt[E] = run;
+    offs[E] = run;
+  }
+  __syncthreads();
+  // stable placement: expert by expert, pairs in increasing p (thread e walks all pairs; NK is small)
+  for (int e = tid; e < E; e += 1024) {
+    int o = cnt[e];
+    const int end = cnt[e + 1];
+    for (int p = 0; p < NK && o < end; ++p)
+      if (idx[p] == e) {
+        pair_of[o] = p;
+        pos_of[p] = o;
+        ++o;
+      }
+  }
+}
+
+// ---- expert projections --------------------------------------------------------------------------
+enum { X_SWIGLU = 0, X_DOWN = 1 };
+
+struct ExpertArgs {
+  const uint4* wp;        // [E][strips][KS][64] packed rows of every expert
+  size_t expert_stride;   // uint4 per expert
+  const bf16_t* x;        // X_SWIGLU: (N, K) activations, gathered by token; X_DOWN: (NK, K) by sorted position
+  int ldx;
+  const int32_t* offs;    // (E+1)
+  const int32_t* pair_of; // (NK)
+  const bf16_t* w;        // (NK) routing weights, pair order (X_DOWN)
+  int k;                  // experts per token
+  int N_out, K;           // output width (X_SWIGLU: hidden F; X_DOWN: d) and contraction length
+  bf16_t* out;            // (NK, N_out) by sorted position
+  int ldo;
+};
+
+template <int EPI>
+__global__ __launch_bounds__(256) void moe_expert_kernel(ExpertArgs a) {
+  const int strip = blockIdx.x, e = blockIdx.y;
+  const int p0 = a.offs[e], p1 = a.offs[e + 1];
+  if (p0 >= p1) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m = lane & 15, g = lane >> 4;
+  const int KS = (a.K + 31) >> 5;
+  const int per = (KS + 3) >> 2;
+  const int j0 = wave * per, j1 = min(KS, j0 + per);
+  __shared__ float red[3][64][4];
+  const uint4* wrow = a.wp + (size_t)e * a.expert_stride + (size_t)strip * KS * 64 + lane;
+  for (int pt = p0; pt < p1; pt += 16) {  // 16-token column tiles of this expert
+    const int pos = pt + m;
+    const bool has = pos < p1;
+    const bf16_t* xrow = a.x;
+    if (has) {
+      const int src = (EPI == X_SWIGLU) ? a.pair_of[pos] / a.k : pos;
+      xrow = a.x + (size_t)src * a.ldx;
+    }
+    f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+    constexpr int CH = 8;
+    for (int jb = j0; jb < j1; jb += CH) {
+      uint4 wv[CH], xv[CH];
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const int j = jb + c;
+        wv[c] = j < j1 ? ldg16_nt(wrow + (size_t)j * 64) : make_uint4(0, 0, 0, 0);
+        const int k0 = 32 * j + 8 * g;
+        xv[c] = make_uint4(0, 0, 0, 0);
+        if (has && j < j1 && k0 < a.K) xv[c] = ldg16(xrow + k0);
+      }
+#pragma unroll
+      for (int c = 0; c < CH; ++c)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wv[c]), __builtin_bit_cast(bf16x8, xv[c]),
+                                                      acc, 0, 0, 0);
+    }
+    if (wave > 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave - 1][lane][i] = acc[i];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = ((acc[i] + red[0][lane][i]) + red[1][lane][i]) + red[2][lane][i];
+      if (has) {
+        const float y0 = rbf(acc[0]), y1 = rbf(acc[1]), y2 = rbf(acc[2]), y3 = rbf(acc[3]);
+        if (EPI == X_SWIGLU) {
+          const int f = strip * 8 + 2 * g;
+          bf16_t* o = a.out + (size_t)pos * a.ldo + f;
+          if (f < a.N_out) o[0] = f2bf(rbf(silu_f(y0)) * y2);
+          if (f + 1 < a.N_out) o[1] = f2bf(rbf(silu_f(y1)) * y3);
+        } else {
+          const float wt = bf2f(a.w[a.pair_of[pos]]);
+          const int r0 = strip * 16 + 4 * g;
+          const float v[4] = {y0 * wt, y1 * wt, y2 * wt, y3 * wt};
+          bf16_t* o = a.out + (size_t)pos * a.ldo + r0;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (r0 + i < a.N_out) o[i] = f2bf(v[i]);
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// ---- combine ---------------------------------------------------------------------------------------
+// out[n] = resid[n] + ( (sum over the token's experts, ascending id, bf16 adds) + shared[n] )
+__global__ __launch_bounds__(256) void moe_combine_kernel(const bf16_t* y, int ldy, const int32_t* idx, const int32_t* pos_of,
+                                                          int k, const bf16_t* shared, int lds_, const bf16_t* resid, int ldr,
+                                                          bf16_t* out, int ldo, int d) {
+  const int n = blockIdx.x;
+  __shared__ int order[16];
+  if (threadIdx.x == 0) {
+    // slots of this token sorted by expert id (k <= 16)
+    int ids[16], sl[16];
+    for (int j = 0; j < k; ++j) {
+      ids[j] = idx[(size_t)n * k + j];
+      sl[j] = j;
+    }
+    for (int a_ = 1; a_ < k; ++a_) {
+      const int vi = ids[a_], vs = sl[a_];
+      int b = a_ - 1;
+      while (b >= 0 && ids[b] > vi) {
+        ids[b + 1] = ids[b];
+        sl[b + 1] = sl[b];
+        --b;
+      }
+      ids[b + 1] = vi;
+      sl[b + 1] = vs;
+    }
+    for (int j = 0; j < k; ++j) order[j] = pos_of[(size_t)n * k + sl[j]];
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < d; c += 256) {
+    float acc = 0.f;
+    for (int j = 0; j < k; ++j) acc = rbf(acc + bf2f(y[(size_t)order[j] * ldy + c]));
+    if (shared) acc = rbf(acc + bf2f(shared[(size_t)n * lds_ + c]));
+    if (resid) acc = rbf(bf2f(resid[(size_t)n * ldr + c]) + acc);
+    out[(size_t)n * ldo + c] = f2bf(acc);
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int ohara_moe_route_topk(const uint16_t* router_logits, int ldl, const uint16_t* router_bias, int n_tokens, int n_experts,
+                         int k, int biased_topk, int gate_sigmoid, int normalize, int32_t* expert_idx,
+                         uint16_t* expert_w, void* stream) {
+  if (!router_logits || !expert_idx || !expert_w || n_tokens < 1 || n_experts < 1 || k < 1) return OHARA_EINVAL;
+  if (k > 16 || n_experts > 1024 || k > n_experts || ldl < n_experts) return OHARA_ESIZE;
+  if (biased_topk && !router_bias) return OHARA_EINVAL;
+  hipLaunchKernelGGL(moe_route_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, (hipStream_t)stream, router_logits, ldl,
+                     router_bias, n_tokens, n_experts, k, biased_topk, gate_sigmoid, normalize, expert_idx, expert_w);
+  return ohara_launch_status();
+}
+
+int ohara_moe_sort_pairs(const int32_t* expert_idx, int n_pairs, int n_experts, int32_t* offsets, int32_t* pair_of,
+                         int32_t* pos_of, void* stream) {
+  if (!expert_idx || !offsets || !pair_of || !pos_of || n_pairs < 1 || n_experts < 1) return OHARA_EINVAL;
+  if (n_pairs > 65536 || n_experts > 1024) return OHARA_ESIZE;
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, expert_idx, n_pairs, n_experts, offsets,
+                     pair_of, pos_of);
+  return ohara_launch_status();
+}
+
+int ohara_moe_experts_gate_up(const uint16_t* x, int ldx, const uint16_t* wp_gate_up, int64_t expert_stride_bytes,
+                              int n_experts, int hidden, int d, int k, const int32_t* offsets, const int32_t* pair_of,
+                              uint16_t* act, int ld_act, void* stream) {
+  if (!x || !wp_gate_up || !offsets || !pair_of || !act || hidden < 1 || d < 1 || (d & 7) || (ldx & 7)) return OHARA_EINVAL;
+  ExpertArgs a{};
+  a.wp = reinterpret_cast<const uint4*>(wp_gate_up); a.expert_stride = (size_t)expert_stride_bytes / 16;
+  a.x = x; a.ldx = ldx; a.offs = offsets; a.pair_of = pair_of; a.k = k; a.N_out = hidden; a.K = d;
+  a.out = act; a.ldo = ld_act;
+  const int strips = 2 * ((hidden + 7) / 8 * 8) / 16;
+  hipLaunchKernelGGL((moe_expert_kernel<X_SWIGLU>), dim3(strips, n_experts), dim3(256), 0, (hipStream_t)stream, a);
+  return ohara_launch_status();
+}
+
+int ohara_moe_experts_down(const uint16_t* act, int ld_act, const uint16_t* wp_down, int64_t expert_stride_bytes,
+                           int n_experts, int d, int hidden, int k, const int32_t* offsets, const int32_t* pair_of,
+                           const uint16_t* expert_w, uint16_t* y, int ldy, void* stream) {
+  if (!act || !wp_down || !offsets || !pair_of || !expert_w || !y || hidden < 1 || d < 1 || (hidden & 7) || (ld_act & 7))
+    return OHARA_EINVAL;
+  ExpertArgs a{};
+  a.wp = reinterpret_cast<const uint4*>(wp_down); a.expert_stride = (size_t)expert_stride_bytes / 16;
+  a.x = act; a.ldx = ld_act; a.offs = offsets; a.pair_of = pair_of; a.w = expert_w; a.k = k; a.N_out = d; a.K = hidden;
+  a.out = y; a.ldo = ldy;
+  hipLaunchKernelGGL((moe_expert_kernel<X_DOWN>), dim3((d + 15) / 16, n_experts), dim3(256), 0, (hipStream_t)stream, a);
+  return ohara_launch_status();
+}
+
+int ohara_moe_combine(const uint16_t* y, int ldy, const int32_t* expert_idx, const int32_t* pos_of, int n_tokens, int k,
+                      const uint16_t* shared, int ld_shared, const uint16_t* resid, int ldr, uint16_t* out, int ldo, int d,
+                      void* stream) {
+  if (!y || !expert_idx || !pos_of || !out || n_tokens < 1 || k < 1 || k > 16 || d < 1) return OHARA_EINVAL;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(256), 0, (hipStream_t)stream, y, ldy, expert_idx, pos_of, k,
+                     shared, ld_shared, resid, ldr, out, ldo, d);
+  return ohara_launch_status();
+}
+
+}  // extern "C"

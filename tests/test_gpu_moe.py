@@ -1,0 +1,95 @@
+"""Grouped MoE kernels (C ABI: ohara_moe_*) against the CPU oracle and the reference fixture."""
+
+import dataclasses
+import os
+
+import pytest
+import torch
+
+from oracle import llama_ref as R
+from oracle import moe_ref as M
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+
+
+def _make(N, d, E, hidden, k, shared, seed, std=0.05):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: (torch.randn(*s, generator=g) * std).to(BF)
+    w = dict(w_gate=r(E, d, hidden), w_up=r(E, d, hidden), w_down=r(E, hidden, d),
+             router=(torch.randn(E, d, generator=g) * d ** -0.5).to(BF),
+             bias=(torch.randn(E, generator=g) * 0.3).to(BF))
+    sh = (r(hidden * shared, d), r(hidden * shared, d), r(d, hidden * shared)) if shared else None
+    x = torch.randn(N, d, generator=g).to(BF)
+    return w, sh, x
+
+
+@pytest.mark.parametrize("N,d,E,hidden,k,shared,gate", [(64, 1024, 64, 512, 8, 1, "softmax"), (9, 64, 6, 24, 2, 0, "softmax"),
+                                                       (40, 128, 16, 32, 4, 2, "sigmoid"), (5, 32, 8, 16, 2, 1, "softmax")])
+def test_grouped_moe_matches_oracle(cuda, N, d, E, hidden, k, shared, gate):
+    from ohara_amd.moe import GroupedMoE
+
+    w, sh, x = _make(N, d, E, hidden, k, shared, seed=N + E)
+    moe = GroupedMoE(w["w_gate"], w["w_up"], w["w_down"], w["router"], w["bias"], k, sh, gate_fn=gate, device=cuda)
+    idx_ref, wt_ref, logits = M.moe_route(x, w["router"], w["bias"], k, gate_fn=gate)
+    idx, wt = moe.route(x.to(cuda))
+    # selection: identical except where the router's own bf16 rounding noise swaps near-equal logits
+    same = (idx.cpu().long() == idx_ref).all(-1)
+    assert same.float().mean().item() >= 0.9
+    for n in (~same).nonzero().flatten().tolist():
+        biased = logits[n] + w["bias"].float()
+        a, b = set(idx.cpu()[n].tolist()), set(idx_ref[n].tolist())
+        gap = max(abs(float(biased[i]) - float(biased[j])) for i in a ^ b for j in a ^ b)
+        assert gap <= 2 ** -6 * max(1.0, float(biased.abs().max())), (n, gap)
+    ok = same.nonzero().flatten()
+    torch.testing.assert_close(wt.cpu().float()[ok], wt_ref.to(BF).float()[ok], atol=2e-3, rtol=2e-2)
+    # weights of every token sum to 1 (tests/test_moe_grouped.py:89-110)
+    assert (wt.float().sum(-1).cpu() - 1).abs().max().item() < 2e-2
+    want = M.moe_forward(x.view(1, N, d), w["router"], w["bias"], w["w_gate"], w["w_up"], w["w_down"], k, gate_fn=gate,
+                         shared=sh)[0]
+    got = moe.forward(x.view(1, N, d).to(cuda))[0].cpu()
+    scale = want.float().abs().max().item()
+    dd = (got.float() - want.float())[ok].abs()
+    assert dd.max().item() <= 3e-2 * scale and dd.mean().item() <= 3e-3 * scale, (dd.max().item(), dd.mean().item(), scale)
+
+
+def test_moe_sort_is_stable(cuda):
+    from ohara_amd._lib import check, lib
+
+    idx = torch.randint(0, 7, (50, 3), generator=torch.Generator().manual_seed(0), dtype=torch.int32)
+    offs = torch.empty(8, dtype=torch.int32, device=cuda)
+    pair_of = torch.empty(150, dtype=torch.int32, device=cuda)
+    pos_of = torch.empty(150, dtype=torch.int32, device=cuda)
+    check(lib().ohara_moe_sort_pairs(idx.to(cuda).data_ptr(), 150, 7, offs.data_ptr(), pair_of.data_ptr(),
+                                     pos_of.data_ptr(), 0), "sort")
+    torch.cuda.synchronize()
+    flat = idx.reshape(-1).long()
+    order = torch.argsort(flat, stable=True)  # ohara/modules/moe_grouped.py:165
+    assert torch.equal(pair_of.cpu().long(), order)
+    assert torch.equal(offs.cpu().long()[1:], torch.bincount(flat, minlength=7).cumsum(0))
+    assert torch.equal(pos_of.cpu().long()[order], torch.arange(150))
+
+
+def test_moe_llama_matches_reference_fixture(cuda):
+    """The tiny grouped-MoE Llama whose logits were written from the reference."""
+    from ohara_amd.llama import Config
+    from ohara_amd.moe import MoeLlama
+
+    g = torch.load(os.path.join(os.path.dirname(__file__), "golden", "llama_tiny_moe.pt"), weights_only=True)
+    fields = {f.name for f in dataclasses.fields(R.RefConfig)}
+    kw = {k: v for k, v in g["config"].items() if k in fields}
+    state = {k: (v.to(BF) if v.is_floating_point() else v) for k, v in g["state"].items()}
+    ref = R.RefLlama(R.RefConfig(**kw), state)
+    model = MoeLlama(Config(**kw), state, device=cuda)
+    ids = g["ids"]
+    want = ref(ids)
+    got = model(ids.to(cuda)).cpu()
+    scale = want.float().abs().max().item()
+    d = (got.float() - want.float()).abs()
+    assert d.max().item() <= 4e-2 * scale and d.mean().item() <= 5e-3 * scale, (d.max().item(), d.mean().item())
+    d = (got.float() - g["logits_full"]).abs()
+    assert d.mean().item() <= 1.5e-2 * scale
+    cache = model.build_kv_cache(2)
+    a = model(ids[:, :5].to(cuda), cache, 0)
+    b = model(ids[:, 5:6].to(cuda), cache, 5)
+    assert (torch.cat([a, b], 1).cpu().float() - got[:, :6].float()).abs().max().item() <= 4e-2 * scale
