@@ -27,6 +27,13 @@ import torch
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch of the persistent decode kernel at batch 1, prompt 1024, from two
+# rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same
+# counter reads for a 1 GiB copy (--pmc-calibration): 379.7 MB read + 1.5 MB written.  Counters
+# cannot be read from inside this process, so the figure is carried here; the runs and the
+# arithmetic are in profiles/decode_mega_kernel_d12_batch1_pmc.txt.
+PMC_TRAFFIC_BYTES = {("persistent", 1, 1024): 381.3e6}
+
 D12 = dict(vocab_size=65536, hidden_size=768, intermediate_size=3072, num_attention_heads=6,
            num_key_value_heads=0, num_hidden_layers=12, max_sequence_length=4096, dropout=0.0)
 
@@ -152,6 +159,9 @@ def main():
     ap.add_argument("--prompt", type=int, default=1024)
     ap.add_argument("--batches", type=str, default="1,8,32,64")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run three 1 GiB device-to-device copies (a kernel of known traffic to scale "
+                         "FETCH_SIZE / WRITE_SIZE counters against)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE MI355X (no sharding, no collectives); --gpus must be 1",
@@ -164,6 +174,13 @@ def main():
     from ohara_amd.llama import Llama
 
     dev = torch.device("cuda:0")
+    if args.pmc_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     cfg, st = d12_state(dev)
     model = Llama(cfg, st, device=dev)
     del st
@@ -199,7 +216,8 @@ def main():
                 kb = lm_head_bytes(cfg, 1)
                 kname = "skinny_kernel<1,true,STORE> (final norm + vocabulary projection 65536x768)"
             roof = {"kernel": kname, "bound": "hbm", "achieved": round(kb / t_k / 1e9, 1), "peak": HBM_PEAK_GBS,
-                    "unit": "GB/s", "frac": round(kb / t_k / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                    "unit": "GB/s", "frac": round(kb / t_k / 1e9 / HBM_PEAK_GBS, 4),
+                    "traffic": PMC_TRAFFIC_BYTES.get(("persistent" if sess2.persistent else "chain", 1, args.prompt)),
                     "bytes_per_launch": int(kb), "avg_launch_us": round(t_k * 1e6, 2)}
         del sess
         torch.cuda.empty_cache()

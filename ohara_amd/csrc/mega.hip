@@ -525,23 +525,24 @@ __device__ __forceinline__ bool attn_first_tile_prefetchable(int t0, int t1, int
 }
 
 template <int D>
-__device__ __forceinline__ void attn_prefetch(const MegaArgs& a, const bf16_t* kc, const bf16_t* vc, int L,
+__device__ __forceinline__ void attn_prefetch(int B, int Hkv, int Tmax, const bf16_t* kc, const bf16_t* vc, int L,
                                               AttnPre<D>& pre) {
-  const int Hkv = a.m.n_kv_heads, wave = threadIdx.x >> 6;
+  const int wave = threadIdx.x >> 6;
   const size_t row = (size_t)Hkv * D;
   int b, kvh, split, t0, t1;
   attn_item_range(blockIdx.x, OHARA_MEGA_NS, Hkv, L, b, kvh, split, t0, t1);
-  const bool has = (int)blockIdx.x < a.B * Hkv * OHARA_MEGA_NS && attn_first_tile_prefetchable<D>(t0, t1, L);
-  const bf16_t* kb = kc + (size_t)b * a.m.t_max * row + (size_t)kvh * D;
-  const bf16_t* vb = vc + (size_t)b * a.m.t_max * row + (size_t)kvh * D;
+  const bool has = (int)blockIdx.x < B * Hkv * OHARA_MEGA_NS && attn_first_tile_prefetchable<D>(t0, t1, L);
+  const bf16_t* kb = kc + (size_t)b * Tmax * row + (size_t)kvh * D;
+  const bf16_t* vb = vc + (size_t)b * Tmax * row + (size_t)kvh * D;
   attn_tile_load<D>(kb, vb, row, t0 + wave * 16, has ? t1 : 0, -1, pre.k, pre.v);
 }
 
 template <int D, int G>
-__device__ void attn_phase(const MegaArgs& a, const AttnPre<D>& pre, const char* qm, float* pm, const bf16_t* kc,
-                           const bf16_t* vc, int L, float* lds) {
+__device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int blk_x, const AttnPre<D>& pre,
+                                           const char* qm, float* pm, const bf16_t* kc, const bf16_t* vc, int L,
+                                           float* lds) {
   constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
-  const int H = a.m.n_heads, Hkv = a.m.n_kv_heads, Tmax = a.m.t_max, ns = OHARA_MEGA_NS;
+  constexpr int ns = OHARA_MEGA_NS;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int p = lane & 15;
   const int dq = lane >> 4;
@@ -550,7 +551,7 @@ __device__ void attn_phase(const MegaArgs& a, const AttnPre<D>& pre, const char*
   float* s_m = lds;                 // [4][G]
   float* s_l = lds + 4 * G;         // [4][G]
   float* s_acc = lds + 8 * G;       // [4][G][D]
-  const int nitems = a.B * Hkv * ns;
+  const int nitems = B * Hkv * ns;
   const size_t row = (size_t)Hkv * D;
   const int PS = D + 32;
   bool first = true;
@@ -573,7 +574,7 @@ __device__ void attn_phase(const MegaArgs& a, const AttnPre<D>& pre, const char*
       for (int hh = 0; hh < G; ++hh)
 #pragma unroll
         for (int c = 0; c < NC; ++c)
-          qv[hh][c] = ldg16(xm_addr(qm, a.blk_x, b, (kvh * G + hh) * D + (4 * c + dq) * 8));
+          qv[hh][c] = ldg16(xm_addr(qm, blk_x, b, (kvh * G + hh) * D + (4 * c + dq) * 8));
       const bool use_pre = first && attn_first_tile_prefetchable<D>(t0, t1, L);
       for (int tb = t0 + wave * 16; tb < t1; tb += 64) {
         const bool valid = tb + p < t1;
@@ -722,11 +723,11 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     gemm_phase<4, 6, E_ROPE>(qkv, pre, xs, ldxs, B, red, best_v, best_i, pf);
     pf.stamp();
     gs.arrive(pf);
-    attn_prefetch<D>(a, kc, vc, L, apre);
+    attn_prefetch<D>(B, Hkv, m.t_max, kc, vc, L, apre);
     gs.wait(pf);
     pf.stamp();
     // P2: attention partials
-    attn_phase<D, G>(a, apre, q_l, p_l, kc, vc, L, att);
+    attn_phase<D, G>(B, H, Hkv, m.t_max, a.blk_x, apre, q_l, p_l, kc, vc, L, att);
     gs.arrive(pf);
     prj.wp = reinterpret_cast<const uint4*>(Lw.wo); prj.out = x_mid; prj.resid = x_in; prj.resid_embed = l == 0;
     gemm_prefetch<4, 6, E_RESID>(prj, pre, B);
