@@ -62,8 +62,9 @@ int ohara_rmsnorm_bf16(const uint16_t* x, const uint16_t* w, uint16_t* out, int 
 /* ---- skinny GEMM (decode projections) ------------------------------------------
  * y = [rmsnorm(x; norm_w, eps)] @ W^T  with one of three epilogues.  `wp` is W in
  * the packed layout; n / k are the logical sizes of W.  norm_w may be NULL.
- * `batch` rows of x; more than 64 rows are processed 64 at a time, each chunk
- * streaming W once (the dense many-row case belongs to ohara_gemm_bf16).
+ * `batch` rows of x.  More than 64 rows without a fused norm go to the tiled MFMA
+ * kernel of ohara_gemm_bf16; with a fused norm they are processed 64 at a time, each
+ * chunk streaming W once.
  *
  * OHARA_EPI_STORE      out[b, n] = bf16(y)                      (any Linear)
  * OHARA_EPI_RESIDUAL   out[b, n] = bf16(resid[b, n] + bf16(y))  (llama.py:199-200)
@@ -83,6 +84,14 @@ int ohara_gemm_skinny_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n
  * Source rows index the vertical concatenation [gate; up] of two (f, k) matrices.
  * perm has 2 * f_padded entries, f_padded = f rounded up to a multiple of 8. */
 int ohara_swiglu_perm(int f, int32_t* perm_host);
+
+/* ---- tiled MFMA GEMM (batched prefill projections) ---------------------------
+ * out = epi(x @ W^T) for any number of rows: 128 x 128 output tiles, K in steps of 64,
+ * activations staged through LDS, packed weights streamed straight into the MFMA A operand.
+ * Same packed `wp`, same epilogues and the same rounding points as ohara_gemm_skinny_bf16
+ * (llama.py:84-86,142,322, mlp.py:152 with more than one position per call).  No fused norm. */
+int ohara_gemm_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n, int k, int rows, int epilogue,
+                    const uint16_t* resid, int ldr, uint16_t* out, int ldo, void* stream);
 
 /* Fused q/k/v projection + rotary + KV-cache append: replaces Attention.forward's
  * three Linears, apply_rope and KVCache.forward (llama.py:84-98;
@@ -245,6 +254,9 @@ typedef struct OharaDecodeState {
   uint16_t* q;           /* (rows, h*dh)                                                  */
   uint16_t* attn;        /* (rows, h*dh)                                                  */
   uint16_t* act;         /* (rows, f)                                                     */
+  uint16_t* xn;          /* (rows, d) normalised rows for calls with > 64 rows; may be NULL when
+                            rows_cap <= 64 (NULL with more rows: the skinny kernel runs 64 rows at
+                            a time instead of the tiled MFMA kernel)                           */
   uint16_t* logits;      /* (batch, vocab) or (rows, vocab), see logits_mode              */
   void* attn_ws;         /* ohara_attn_workspace_bytes(batch, h, h_kv, dh, n_split)       */
   int32_t* step_state;   /* 4 x int32 {pos, step, done, pad}, may be NULL                 */

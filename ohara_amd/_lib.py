@@ -37,7 +37,7 @@ class OharaModel(C.Structure):
 class OharaDecodeState(C.Structure):
     _fields_ = [
         ("batch", _i), ("rows_cap", _i), ("n_split", _i), ("valid_vocab", _i), ("hist_cap", _i), ("prof_kernel", _i),
-        ("ids", _p), ("x", _p), ("q", _p), ("attn", _p), ("act", _p), ("logits", _p),
+        ("ids", _p), ("x", _p), ("q", _p), ("attn", _p), ("act", _p), ("xn", _p), ("logits", _p),
         ("attn_ws", _p), ("step_state", _p), ("history", _p),
         ("kcache", C.POINTER(_p)), ("vcache", C.POINTER(_p)),
         ("prof_start", _p), ("prof_stop", _p),
@@ -53,6 +53,7 @@ _PROTOS = {
     "ohara_embed_bf16": (_i, [_p, _p, _p, _i, _i, _i, _p]),
     "ohara_rmsnorm_bf16": (_i, [_p, _p, _p, _i, _i, _f, _p]),
     "ohara_gemm_skinny_bf16": (_i, [_p, _i, _p, _i, _i, _p, _f, _i, _i, _p, _i, _p, _i, _p]),
+    "ohara_gemm_bf16": (_i, [_p, _i, _p, _i, _i, _i, _i, _p, _i, _p, _i, _p]),
     "ohara_qkv_rope_append_bf16": (_i, [_p, _i, _p, _i, _p, _f, _i, _i, _i, _i, _i, _p, _p, _i, _p, _p, _p, _p, _i, _p]),
     "ohara_attn_workspace_bytes": (_i64, [_i, _i, _i, _i, _i]),
     "ohara_attn_cached_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),

@@ -38,23 +38,37 @@ extern "C" int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* 
     if (rc) return rc;                                                                      \
   } while (0)
   int rc = 0;
+  const bool tiled = R > 64 && s->xn != nullptr;
   OHARA_RUN(ohara_embed_bf16(s->ids, m->token_emb, s->x, R, d, m->vocab, stream));
   for (int l = 0; l < m->n_layers; ++l) {
     const OharaLayer& L = m->layers[l];
-    OHARA_RUN(ohara_qkv_rope_append_bf16(s->x, d, L.wqkv, d, L.norm1, m->eps, B, seq_len, H, Hkv, Dh, m->cos, m->sin, pos,
-                                    pos_dev, s->q, s->kcache[l], s->vcache[l], m->t_max, stream));
+    if (tiled) {  // many rows: normalise once, then the tiled MFMA kernel (launches are not numbered)
+      rc = ohara_rmsnorm_bf16(s->x, L.norm1, s->xn, R, d, m->eps, stream);
+      if (rc) return rc;
+    }
+    OHARA_RUN(ohara_qkv_rope_append_bf16(tiled ? s->xn : s->x, d, L.wqkv, d, tiled ? nullptr : L.norm1, m->eps, B,
+                                         seq_len, H, Hkv, Dh, m->cos, m->sin, pos, pos_dev, s->q, s->kcache[l],
+                                         s->vcache[l], m->t_max, stream));
     OHARA_RUN(ohara_attn_cached_bf16(s->q, s->kcache[l], s->vcache[l], B, seq_len, H, Hkv, Dh, m->t_max, pos, pos_dev,
                                 n_split, s->attn_ws, s->attn, stream));
     OHARA_RUN(ohara_gemm_skinny_bf16(s->attn, H * Dh, L.wo, d, H * Dh, nullptr, m->eps, R, OHARA_EPI_RESIDUAL, s->x, d,
                                 s->x, d, stream));
-    OHARA_RUN(ohara_gemm_skinny_bf16(s->x, d, L.wgu, m->d_ff, d, L.norm2, m->eps, R, OHARA_EPI_SWIGLU, nullptr, 0, s->act,
-                                m->d_ff, stream));
+    if (tiled) {
+      rc = ohara_rmsnorm_bf16(s->x, L.norm2, s->xn, R, d, m->eps, stream);
+      if (rc) return rc;
+    }
+    OHARA_RUN(ohara_gemm_skinny_bf16(tiled ? s->xn : s->x, d, L.wgu, m->d_ff, d, tiled ? nullptr : L.norm2, m->eps, R,
+                                     OHARA_EPI_SWIGLU, nullptr, 0, s->act, m->d_ff, stream));
     OHARA_RUN(ohara_gemm_skinny_bf16(s->act, m->d_ff, L.wdown, d, m->d_ff, nullptr, m->eps, R, OHARA_EPI_RESIDUAL, s->x, d,
                                 s->x, d, stream));
   }
   if (logits_mode == OHARA_LOGITS_ALL) {
-    OHARA_RUN(ohara_gemm_skinny_bf16(s->x, d, m->w_vocab, m->vocab, d, m->final_norm, m->eps, R, OHARA_EPI_STORE,
-                                     nullptr, 0, s->logits, m->vocab, stream));
+    if (tiled) {
+      rc = ohara_rmsnorm_bf16(s->x, m->final_norm, s->xn, R, d, m->eps, stream);
+      if (rc) return rc;
+    }
+    OHARA_RUN(ohara_gemm_skinny_bf16(tiled ? s->xn : s->x, d, m->w_vocab, m->vocab, d, tiled ? nullptr : m->final_norm,
+                                     m->eps, R, OHARA_EPI_STORE, nullptr, 0, s->logits, m->vocab, stream));
   } else if (logits_mode == OHARA_LOGITS_LAST) {
     // row b*seq_len + seq_len-1 of x for every sequence: a strided view, no gather
     OHARA_RUN(ohara_gemm_skinny_bf16(s->x + (size_t)(seq_len - 1) * d, seq_len * d, m->w_vocab, m->vocab, d,

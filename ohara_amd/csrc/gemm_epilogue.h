@@ -1,0 +1,107 @@
+// Shared by the skinny (decode) and tiled (prefill) GEMM kernels: argument block and the
+// fused epilogues.  Rounding points follow the reference's bf16 eager path:
+//   residual add       ohara/models/llama.py:199-200
+//   SwiGLU             ohara/modules/mlp.py:152
+//   rotary + KV append ohara/embeddings_pos/rotary.py:55-93, ohara/modules/kv_cache.py:104-105
+#pragma once
+#include "common.h"
+
+enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_ROPE = 3 };
+
+struct GemmArgs {
+  const uint4* wp;
+  const bf16_t* x;
+  int ldx;
+  const bf16_t* norm_w;
+  float eps;
+  int B, N, K;  // rows, logical output width (EPI_SWIGLU: hidden width F) and depth
+  bf16_t* out;
+  int ldo;
+  const bf16_t* resid;
+  int ldr;
+  // rotary + append
+  int H, Hkv, Dh, Tmax, pos;
+  int S, row0;  // rows are (sequence, position) pairs: row = seq * S + s, position = pos + s
+  const int32_t* pos_dev;
+  const bf16_t* cos;
+  const bf16_t* sin;
+  bf16_t* kcache;
+  bf16_t* vcache;
+};
+
+// gemm_tile.hip: the tiled kernel for calls with many rows (a.B rows, no fused norm).
+int ohara_launch_gemm_tile(const GemmArgs& a, int epi, int packed_rows, hipStream_t st);
+
+namespace {
+
+// One MFMA output fragment: the four consecutive packed rows 16*strip + 4*g .. +3 of activation
+// row b (relative to a.out / a.resid; global row a.row0 + b for the rotary epilogue).
+template <int EPI>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, int b, int strip, int g, f32x4 acc) {
+  const int r0 = strip * 16 + 4 * g;
+  const float y0 = rbf(acc[0]), y1 = rbf(acc[1]), y2 = rbf(acc[2]), y3 = rbf(acc[3]);
+  if (EPI == EPI_STORE || EPI == EPI_RESIDUAL) {
+    float v[4] = {y0, y1, y2, y3};
+    bf16_t* o = a.out + (size_t)b * a.ldo + r0;
+    if (EPI == EPI_RESIDUAL) {
+      const bf16_t* r = a.resid + (size_t)b * a.ldr + r0;
+      if (r0 + 3 < a.N && ((a.ldr & 3) == 0)) {
+        const uint2 rv = *reinterpret_cast<const uint2*>(r);
+        v[0] = lo_bf(rv.x) + v[0]; v[1] = hi_bf(rv.x) + v[1]; v[2] = lo_bf(rv.y) + v[2]; v[3] = hi_bf(rv.y) + v[3];
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (r0 + i < a.N) v[i] = bf2f(r[i]) + v[i];
+      }
+    }
+    if (r0 + 3 < a.N && ((a.ldo & 3) == 0)) {
+      *reinterpret_cast<uint2*>(o) = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (r0 + i < a.N) o[i] = f2bf(v[i]);
+    }
+  } else if (EPI == EPI_SWIGLU) {
+    // rows: gate f, gate f+1, up f, up f+1 with f = 8*strip + 2*g; N = hidden width F
+    const int f = strip * 8 + 2 * g;
+    const float s0 = rbf(silu_f(y0)), s1 = rbf(silu_f(y1));
+    bf16_t* o = a.out + (size_t)b * a.ldo + f;
+    if (f + 1 < a.N && ((a.ldo & 1) == 0)) {
+      *reinterpret_cast<uint32_t*>(o) = pack_bf(s0 * y2, s1 * y3);
+    } else {
+      if (f < a.N) o[0] = f2bf(s0 * y2);
+      if (f + 1 < a.N) o[1] = f2bf(s1 * y3);
+    }
+  } else {  // EPI_ROPE: rows [q (H*Dh); k (Hkv*Dh); v (Hkv*Dh)], one position per sequence
+    const int grow = a.row0 + b;
+    const int seq = grow / a.S;
+    const int pos = (a.pos_dev ? *a.pos_dev : a.pos) + (grow - seq * a.S);
+    const int nq = a.H * a.Dh, nk = a.Hkv * a.Dh;
+    if (r0 >= nq + 2 * nk || pos < 0 || pos >= a.Tmax) return;
+    float v[4] = {y0, y1, y2, y3};
+    bf16_t* o;
+    if (r0 < nq + nk) {
+      const int d = (r0 < nq ? r0 : r0 - nq) % a.Dh;
+      const bf16_t* cs = a.cos + (size_t)pos * (a.Dh >> 1) + (d >> 1);
+      const bf16_t* sn = a.sin + (size_t)pos * (a.Dh >> 1) + (d >> 1);
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) {
+        const float c = bf2f(cs[pr]), s = bf2f(sn[pr]);
+        const float e = v[2 * pr], od = v[2 * pr + 1];
+        // separate fp32 multiplies and add/sub, as the reference's eager ops round
+        v[2 * pr] = __fsub_rn(__fmul_rn(e, c), __fmul_rn(od, s));
+        v[2 * pr + 1] = __fadd_rn(__fmul_rn(e, s), __fmul_rn(od, c));
+      }
+      if (r0 < nq) {
+        o = a.out + (size_t)grow * a.ldo + r0;
+      } else {
+        o = a.kcache + (((size_t)seq * a.Tmax + pos) * a.Hkv) * a.Dh + (r0 - nq);
+      }
+    } else {
+      o = a.vcache + (((size_t)seq * a.Tmax + pos) * a.Hkv) * a.Dh + (r0 - nq - nk);
+    }
+    *reinterpret_cast<uint2*>(o) = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
+  }
+}
+
+}  // namespace

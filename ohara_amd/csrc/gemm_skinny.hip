@@ -14,33 +14,9 @@
 //             SwiGLU            ohara/modules/mlp.py:152
 //             rotary + KV append ohara/embeddings_pos/rotary.py:55-93,
 //                               ohara/modules/kv_cache.py:104-105
-#include "common.h"
+#include "gemm_epilogue.h"
 
 namespace {
-
-enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_ROPE = 3 };
-
-struct SkinnyArgs {
-  const uint4* wp;
-  const bf16_t* x;
-  int ldx;
-  const bf16_t* norm_w;
-  float eps;
-  int B, N, K;  // logical sizes; packed sizes are the round-ups
-  bf16_t* out;
-  int ldo;
-  const bf16_t* resid;
-  int ldr;
-  // rotary + append
-  int H, Hkv, Dh, Tmax, pos;
-  int S, row0;  // rows are (sequence, position) pairs: row = seq * S + s, position = pos + s
-  const int32_t* pos_dev;
-  const bf16_t* cos;
-  const bf16_t* sin;
-  bf16_t* kcache;
-  bf16_t* vcache;
-};
-
 
 __device__ __forceinline__ float sumsq8(uint4 v) {
   float s = 0.f;
@@ -68,7 +44,7 @@ __device__ __forceinline__ uint4 norm8(uint4 xv, uint4 wv, float rinv) {
 }
 
 template <int BT, bool NORM, int EPI>
-__global__ __launch_bounds__(256) void skinny_kernel(SkinnyArgs a) {
+__global__ __launch_bounds__(256) void skinny_kernel(GemmArgs a) {
   constexpr int CH = 6;  // k-steps whose weight loads are issued back to back
   const int strip = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -156,73 +132,15 @@ __global__ __launch_bounds__(256) void skinny_kernel(SkinnyArgs a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) acc[t][i] = ((acc[t][i] + red[0][t][lane][i]) + red[1][t][lane][i]) + red[2][t][lane][i];
 
-  const int r0 = strip * 16 + 4 * g;  // first of this lane's four packed rows
 #pragma unroll
   for (int t = 0; t < BT; ++t) {
     const int b = m + 16 * t;
-    if (b >= a.B) continue;
-    const float y0 = rbf(acc[t][0]), y1 = rbf(acc[t][1]), y2 = rbf(acc[t][2]), y3 = rbf(acc[t][3]);
-    if (EPI == EPI_STORE || EPI == EPI_RESIDUAL) {
-      float v[4] = {y0, y1, y2, y3};
-      bf16_t* o = a.out + (size_t)b * a.ldo + r0;
-      if (EPI == EPI_RESIDUAL) {
-        const bf16_t* r = a.resid + (size_t)b * a.ldr + r0;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (r0 + i < a.N) v[i] = bf2f(r[i]) + v[i];
-      }
-      if (r0 + 3 < a.N && ((a.ldo & 3) == 0)) {
-        uint2 pk = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
-        *reinterpret_cast<uint2*>(o) = pk;
-      } else {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (r0 + i < a.N) o[i] = f2bf(v[i]);
-      }
-    } else if (EPI == EPI_SWIGLU) {
-      // rows: gate f, gate f+1, up f, up f+1 with f = 8*strip + 2*g; N = hidden width F
-      const int f = strip * 8 + 2 * g;
-      const float s0 = rbf(silu_f(y0)), s1 = rbf(silu_f(y1));
-      bf16_t* o = a.out + (size_t)b * a.ldo + f;
-      if (f < a.N) o[0] = f2bf(s0 * y2);
-      if (f + 1 < a.N) o[1] = f2bf(s1 * y3);
-    } else {  // EPI_ROPE: rows [q (H*Dh); k (Hkv*Dh); v (Hkv*Dh)], one position per sequence
-      const int grow = a.row0 + b;
-      const int seq = grow / a.S;
-      const int pos = (a.pos_dev ? *a.pos_dev : a.pos) + (grow - seq * a.S);
-      const int nq = a.H * a.Dh, nk = a.Hkv * a.Dh;
-      if (r0 >= nq + 2 * nk || pos < 0 || pos >= a.Tmax) continue;
-      float v[4] = {y0, y1, y2, y3};
-      bf16_t* o;
-      if (r0 < nq + nk) {
-        const int d = (r0 < nq ? r0 : r0 - nq) % a.Dh;
-        const bf16_t* cs = a.cos + (size_t)pos * (a.Dh >> 1) + (d >> 1);
-        const bf16_t* sn = a.sin + (size_t)pos * (a.Dh >> 1) + (d >> 1);
-#pragma unroll
-        for (int pr = 0; pr < 2; ++pr) {
-          const float c = bf2f(cs[pr]), s = bf2f(sn[pr]);
-          const float e = v[2 * pr], od = v[2 * pr + 1];
-          // separate fp32 multiplies and add/sub, as the reference's eager ops round
-          v[2 * pr] = __fsub_rn(__fmul_rn(e, c), __fmul_rn(od, s));
-          v[2 * pr + 1] = __fadd_rn(__fmul_rn(e, s), __fmul_rn(od, c));
-        }
-        if (r0 < nq) {
-          o = a.out + (size_t)grow * a.ldo + r0;
-        } else {
-          const int rk = r0 - nq;
-          o = a.kcache + (((size_t)seq * a.Tmax + pos) * a.Hkv) * a.Dh + rk;
-        }
-      } else {
-        const int rv = r0 - nq - nk;
-        o = a.vcache + (((size_t)seq * a.Tmax + pos) * a.Hkv) * a.Dh + rv;
-      }
-      *reinterpret_cast<uint2*>(o) = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
-    }
+    if (b < a.B) gemm_epilogue<EPI>(a, b, strip, g, acc[t]);
   }
 }
 
 template <int BT, bool NORM>
-int launch_epi(const SkinnyArgs& a, int epi, int strips, hipStream_t st) {
+int launch_epi(const GemmArgs& a, int epi, int strips, hipStream_t st) {
   dim3 grid(strips), block(256);
   switch (epi) {
     case EPI_STORE: hipLaunchKernelGGL((skinny_kernel<BT, NORM, EPI_STORE>), grid, block, 0, st, a); break;
@@ -234,7 +152,7 @@ int launch_epi(const SkinnyArgs& a, int epi, int strips, hipStream_t st) {
   return ohara_launch_status();
 }
 
-int launch_chunk(const SkinnyArgs& a, int epi, int strips, hipStream_t st) {
+int launch_chunk(const GemmArgs& a, int epi, int strips, hipStream_t st) {
   const bool norm = a.norm_w != nullptr;
   const int bt = (a.B + 15) / 16;
   if (bt == 1) return norm ? launch_epi<1, true>(a, epi, strips, st) : launch_epi<1, false>(a, epi, strips, st);
@@ -244,11 +162,11 @@ int launch_chunk(const SkinnyArgs& a, int epi, int strips, hipStream_t st) {
 }
 
 // Rows beyond 64 are processed in chunks of 64 (each chunk streams the weights once).
-int launch_skinny(const SkinnyArgs& a0, int epi, int packed_rows, hipStream_t st) {
+int launch_skinny(const GemmArgs& a0, int epi, int packed_rows, hipStream_t st) {
   const int strips = packed_rows / 16;
   const int rows = a0.B;
   for (int r = 0; r < rows; r += 64) {
-    SkinnyArgs a = a0;
+    GemmArgs a = a0;
     a.B = rows - r < 64 ? rows - r : 64;
     a.x = a0.x + (size_t)r * a0.ldx;
     if (epi == EPI_ROPE) {
@@ -324,7 +242,7 @@ int ohara_gemm_skinny_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n
   if (epilogue == OHARA_EPI_RESIDUAL && (!resid || ldr < n)) return OHARA_EINVAL;
   if (epilogue < OHARA_EPI_STORE || epilogue > OHARA_EPI_SWIGLU) return OHARA_EINVAL;
   if (ldo < n) return OHARA_EINVAL;
-  SkinnyArgs a{};
+  GemmArgs a{};
   a.wp = reinterpret_cast<const uint4*>(wp);
   a.x = x; a.ldx = ldx; a.norm_w = norm_w; a.eps = eps;
   a.B = batch; a.N = n; a.K = k;
@@ -332,6 +250,7 @@ int ohara_gemm_skinny_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n
   int packed_rows;
   if (epilogue == OHARA_EPI_SWIGLU) packed_rows = 2 * ((n + 7) / 8 * 8);
   else packed_rows = (n + 15) / 16 * 16;
+  if (batch > 64 && !norm_w) return ohara_launch_gemm_tile(a, epilogue, packed_rows, (hipStream_t)stream);
   return launch_skinny(a, epilogue, packed_rows, (hipStream_t)stream);
 }
 
@@ -345,7 +264,7 @@ int ohara_qkv_rope_append_bf16(const uint16_t* x, int ldx, const uint16_t* wp, i
   if ((k & 7) || (ldx & 7) || ldx < k) return OHARA_EINVAL;
   if (!pos_dev && (pos < 0 || pos + seq_len > t_max)) return OHARA_EINVAL;
   if ((int64_t)batch * seq_len > INT32_MAX) return OHARA_ESIZE;
-  SkinnyArgs a{};
+  GemmArgs a{};
   a.wp = reinterpret_cast<const uint4*>(wp);
   a.x = x; a.ldx = ldx; a.norm_w = norm_w; a.eps = eps;
   a.B = batch * seq_len; a.N = (h + 2 * h_kv) * dh; a.K = k;
@@ -353,6 +272,7 @@ int ohara_qkv_rope_append_bf16(const uint16_t* x, int ldx, const uint16_t* wp, i
   a.out = q_out; a.ldo = h * dh;
   a.H = h; a.Hkv = h_kv; a.Dh = dh; a.Tmax = t_max; a.pos = pos; a.pos_dev = pos_dev;
   a.cos = cos; a.sin = sin; a.kcache = kcache; a.vcache = vcache;
+  if (a.B > 64 && !norm_w) return ohara_launch_gemm_tile(a, EPI_ROPE, (a.N + 15) / 16 * 16, (hipStream_t)stream);
   return launch_skinny(a, EPI_ROPE, (a.N + 15) / 16 * 16, (hipStream_t)stream);
 }
 

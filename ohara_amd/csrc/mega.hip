@@ -161,6 +161,15 @@ struct GridSync {
   }
 };
 
+// A pointer from the workgroup's LDS copy of the layer table, made wave-uniform.
+template <typename T>
+__device__ __forceinline__ T* lds_ptr(const unsigned long long* tab, int i) {
+  const unsigned long long v = tab[i];
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return reinterpret_cast<T*>(((unsigned long long)hi << 32) | lo);
+}
+
 __device__ __forceinline__ float dot8m(uint4 a, uint4 b, float s) {
   s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.x), __builtin_bit_cast(bf16x2, b.x), s, false);
   s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.y), __builtin_bit_cast(bf16x2, b.y), s, false);
@@ -675,6 +684,17 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   bf16_t* xs = reinterpret_cast<bf16_t*>(smem);
   float* red = reinterpret_cast<float*>(smem + (((size_t)B * ldxs * 2 + 255) & ~(size_t)255));  // 4 KiB
   float* att = red + 1024;                                                                      // (8 + 4*D)*G floats
+  // per-layer pointers (6 weights/norms + K and V cache), copied once to LDS so that no phase
+  // starts with a chain of dependent global loads
+  unsigned long long* ptab = reinterpret_cast<unsigned long long*>(att + (8 + 4 * D) * G);
+  for (int i = threadIdx.x; i < m.n_layers * 8; i += blockDim.x) {
+    const int l = i >> 3, j = i & 7;
+    unsigned long long v;
+    if (j < 6) v = reinterpret_cast<const unsigned long long*>(a.layers_dev + l)[j];
+    else v = reinterpret_cast<const unsigned long long*>(j == 6 ? a.kcache_dev : a.vcache_dev)[l];
+    ptab[i] = v;
+  }
+  __syncthreads();
 
   GridSync gs;
   gs.init(a.bar, gridDim.x, a.spin_limit);
@@ -699,13 +719,13 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
 
   GemmPre pre;
   AttnPre<D> apre;
-  qkv.wp = reinterpret_cast<const uint4*>(a.layers_dev[0].wqkv);
+  qkv.wp = lds_ptr<const uint4>(ptab, 0);
   gemm_prefetch<4, 6, E_ROPE>(qkv, pre, B);
   pf.stamp();
   for (int l = 0; l < m.n_layers; ++l) {
-    const OharaLayer& Lw = a.layers_dev[l];
-    bf16_t* kc = a.kcache_dev[l];
-    bf16_t* vc = a.vcache_dev[l];
+    const unsigned long long* pl = ptab + l * 8;
+    bf16_t* kc = lds_ptr<bf16_t>(pl, 6);
+    bf16_t* vc = lds_ptr<bf16_t>(pl, 7);
     const char* x_in = a.xm + (size_t)(2 * l) * a.xm_stride;       // residual stream entering the layer
     char* x_mid = a.xm + (size_t)(2 * l + 1) * a.xm_stride;        // after attention
     char* x_out = a.xm + (size_t)(2 * l + 2) * a.xm_stride;        // after the feed-forward
@@ -715,8 +735,8 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     // P1: [embedding] + norm1 + QKV + rotary + append
     qkv.kc = kc; qkv.vc = vc; qkv.out = q_l;
     if ((int)blockIdx.x < qkv.nstrips) {
-      if (l == 0) stage_norm<2, true>(xs, ldxs, a.xm, 0, a.ids, m.token_emb, V, Lw.norm1, m.eps, B, d);
-      else stage_norm<2, false>(xs, ldxs, x_in, a.blk_x, a.ids, m.token_emb, V, Lw.norm1, m.eps, B, d);
+      if (l == 0) stage_norm<2, true>(xs, ldxs, a.xm, 0, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d);
+      else stage_norm<2, false>(xs, ldxs, x_in, a.blk_x, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d);
     }
     __syncthreads();
     pf.stamp();
@@ -729,7 +749,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     // P2: attention partials
     attn_phase<D, G>(B, H, Hkv, m.t_max, a.blk_x, apre, q_l, p_l, kc, vc, L, att);
     gs.arrive(pf);
-    prj.wp = reinterpret_cast<const uint4*>(Lw.wo); prj.out = x_mid; prj.resid = x_in; prj.resid_embed = l == 0;
+    prj.wp = lds_ptr<const uint4>(pl, 1); prj.out = x_mid; prj.resid = x_in; prj.resid_embed = l == 0;
     gemm_prefetch<4, 6, E_RESID>(prj, pre, B);
     gs.wait(pf);
     pf.stamp();
@@ -740,16 +760,16 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     gemm_phase<4, 6, E_RESID>(prj, pre, xs, ldxs, B, red, best_v, best_i, pf);
     pf.stamp();
     gs.arrive(pf);
-    gu.wp = reinterpret_cast<const uint4*>(Lw.wgu); gu.out = a_l;
+    gu.wp = lds_ptr<const uint4>(pl, 2); gu.out = a_l;
     gemm_prefetch<2, 12, E_SWIGLU>(gu, pre, B);
     gs.wait(pf);
     pf.stamp();
     // P4: norm2 + gate/up + SwiGLU
-    if ((int)blockIdx.x * 2 < gu.nstrips) stage_norm<2, false>(xs, ldxs, x_mid, a.blk_x, a.ids, m.token_emb, V, Lw.norm2, m.eps, B, d);
+    if ((int)blockIdx.x * 2 < gu.nstrips) stage_norm<2, false>(xs, ldxs, x_mid, a.blk_x, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 5), m.eps, B, d);
     __syncthreads();
     gemm_phase<2, 12, E_SWIGLU>(gu, pre, xs, ldxs, B, red, best_v, best_i, pf);
     gs.arrive(pf);
-    dn.wp = reinterpret_cast<const uint4*>(Lw.wdown); dn.out = x_out; dn.resid = x_mid;
+    dn.wp = lds_ptr<const uint4>(pl, 3); dn.out = x_out; dn.resid = x_mid;
     gemm_prefetch<4, 24, E_RESID>(dn, pre, B);
     gs.wait(pf);
     pf.stamp();
@@ -759,7 +779,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     gemm_phase<4, 24, E_RESID>(dn, pre, xs, ldxs, B, red, best_v, best_i, pf);
     gs.arrive(pf);
     if (l + 1 < m.n_layers) {
-      qkv.wp = reinterpret_cast<const uint4*>(a.layers_dev[l + 1].wqkv);
+      qkv.wp = lds_ptr<const uint4>(pl, 8);
       gemm_prefetch<4, 6, E_ROPE>(qkv, pre, B);
     } else {
       gemm_prefetch<1, 24, E_LOGITS>(lm, pre, B);
@@ -953,12 +973,12 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   a.ids = s->ids; a.logits = s->logits;
   a.step_state = s->step_state; a.history = s->history;
   a.prof = s->prof_kernel == -2 ? reinterpret_cast<unsigned long long*>(ws + L.prof) : nullptr;
-  if (40 * m->n_layers + 16 > OHARA_PROF_SLOTS) a.prof = nullptr;
+  if (48 * m->n_layers + 16 > OHARA_PROF_SLOTS) a.prof = nullptr;
   a.spin_limit = spin_limit ? spin_limit : (1u << 19);
   const int kmax = m->d_model > m->d_ff ? m->d_model : m->d_ff;
   const int kmax2 = kmax > m->n_heads * D ? kmax : m->n_heads * D;
   const size_t xs_bytes = ((size_t)s->batch * (kmax2 + 8) * 2 + 255) & ~(size_t)255;
-  const size_t smem = xs_bytes + 4096 + (size_t)(8 + 4 * D) * G * sizeof(float);
+  const size_t smem = xs_bytes + 4096 + (size_t)(8 + 4 * D) * G * sizeof(float) + (size_t)m->n_layers * 64;
   if (smem > 160 * 1024) return OHARA_ESIZE;
   dim3 grid(n_workgroups), block(256);
 #define OHARA_MEGA(DD, GG)                                                                                  \

@@ -140,6 +140,7 @@ class _Buffers:
         self.q = torch.empty(rows, hd, dtype=BF16, device=dev)
         self.attn = torch.empty(rows, hd, dtype=BF16, device=dev)
         self.act = torch.empty(rows, model.act_width, dtype=BF16, device=dev)
+        self.xn = torch.empty(rows, c.hidden_size, dtype=BF16, device=dev) if rows > 64 else None
         self.attn_ws = ops.attn_workspace(batch, c.num_attention_heads, model.kv_heads, model.head_dim, n_split, dev)
         self.step_state = torch.zeros(4, dtype=torch.int32, device=dev)
         self.logits = None
@@ -266,6 +267,7 @@ class Llama:
         s.hist_cap = 0 if history is None else history.shape[0]
         s.prof_kernel = -1
         s.ids, s.x, s.q, s.attn, s.act = (t.data_ptr() for t in (buf.ids, buf.x, buf.q, buf.attn, buf.act))
+        s.xn = 0 if buf.xn is None else buf.xn.data_ptr()
         s.logits = 0 if logits is None else logits.data_ptr()
         s.attn_ws, s.step_state = buf.attn_ws.data_ptr(), buf.step_state.data_ptr()
         s.history = 0 if history is None else history.data_ptr()

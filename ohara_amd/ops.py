@@ -123,6 +123,27 @@ def gemm_skinny(x, w: PackedLinear, norm_w=None, eps=1e-5, residual=None, out=No
     return out
 
 
+def gemm(x, w: PackedLinear, residual=None, out=None) -> torch.Tensor:
+    """y = x @ W^T (+ residual / SwiGLU epilogue by the packing kind) on the tiled MFMA kernel,
+    for any number of rows.  x: (rows, K), rows may be strided (a column slice of a wider buffer)."""
+    if not x.is_cuda or x.dtype != BF16 or x.ndim != 2 or x.stride(1) != 1:
+        raise ValueError("x must be a 2-D bfloat16 device tensor with unit column stride")
+    rows, k = x.shape
+    if k != w.k:
+        raise ValueError(f"x has {k} columns, weight expects {w.k}")
+    if out is None:
+        out = torch.empty(rows, w.n, dtype=BF16, device=x.device)
+    epi = _lib.EPI_SWIGLU if w.kind == "swiglu" else (_lib.EPI_RESIDUAL if residual is not None else _lib.EPI_STORE)
+    check(
+        lib().ohara_gemm_bf16(
+            _ptr(x), x.stride(0), _ptr(w.data), w.n, w.k, rows, epi,
+            _ptr(residual), 0 if residual is None else residual.stride(0), _ptr(out), out.stride(0), _stream(),
+        ),
+        "gemm",
+    )
+    return out
+
+
 def qkv_rope_append(x, wqkv: PackedLinear, norm_w, eps, h, h_kv, dh, cos, sin, pos, kcache, vcache,
                     q_out=None, pos_dev=None, seq_len=1):
     """x: (batch*seq_len, K) rows ordered (sequence, position)."""

@@ -185,3 +185,93 @@ def test_argmax(cuda):
     assert torch.equal(out.cpu(), ref)
     out = ops.argmax(logits.to(cuda), valid_vocab=60000)
     assert torch.equal(out.cpu(), logits[:, :60000].float().argmax(-1))
+
+
+# ---- tiled MFMA GEMM (many rows) -------------------------------------------------------------
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (1, 16, 32), (65, 768, 768), (300, 2304, 768), (257, 100, 96),
+                                   (1024, 768, 3072), (130, 65, 40), (2048, 640, 136)])
+def test_gemm_tiled_store(cuda, M, N, K):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(M * 7 + N + K)
+    x = torch.randn(M, K, generator=g).to(BF)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(BF)
+    ref = R.linear(x, w)
+    out = ops.gemm(x.to(cuda), ops.pack_linear(w.to(cuda)))
+    scale = ref.float().abs().max().item()
+    err = (out.cpu().float() - ref.float()).abs().max().item()
+    assert err <= 2 ** -7 * scale, (err, scale)
+    assert (out.cpu() != ref).float().mean().item() < 0.05
+
+
+def test_gemm_tiled_strided_rows_and_residual_in_place(cuda):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(77)
+    M, N, K = 200, 768, 3072
+    xw = torch.randn(M, K + 64, generator=g).to(BF)  # a view with a row stride larger than K
+    w = (torch.randn(N, K, generator=g) * 0.02).to(BF)
+    res = torch.randn(M, N, generator=g).to(BF)
+    ref = res + R.linear(xw[:, :K], w)
+    buf = res.to(cuda).clone()
+    out = ops.gemm(xw.to(cuda)[:, :K], ops.pack_linear(w.to(cuda)), residual=buf, out=buf)
+    assert out.data_ptr() == buf.data_ptr()
+    _ulp_close(out, ref, max_ulp=2, frac=0.05)
+
+
+@pytest.mark.parametrize("M,F,K", [(256, 3072, 768), (100, 520, 64), (70, 12, 32)])
+def test_gemm_tiled_swiglu(cuda, M, F, K):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(F + M)
+    x = torch.randn(M, K, generator=g).to(BF)
+    wg = (torch.randn(F, K, generator=g) * 0.1).to(BF)
+    wu = (torch.randn(F, K, generator=g) * 0.1).to(BF)
+    ref = torch.nn.functional.silu(R.linear(x, wg)) * R.linear(x, wu)
+    out = ops.gemm(x.to(cuda), ops.pack_gate_up(wg.to(cuda), wu.to(cuda)))
+    scale = ref.float().abs().max().item()
+    err = (out.cpu().float() - ref.float()).abs().max().item()
+    assert err <= 2 ** -6 * scale, (err, scale)
+    assert (out.cpu() != ref).float().mean().item() < 0.08
+
+
+def test_gemm_tiled_matches_skinny_bitwise_on_shared_rows(cuda):
+    """Both kernels accumulate a 32-column k-step per MFMA in the same lane order; with K = 32
+    there is a single MFMA per output, so the two must agree bit for bit."""
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(64, 32, generator=g).to(BF).to(cuda)
+    w = torch.randn(256, 32, generator=g).to(BF).to(cuda)
+    wp = ops.pack_linear(w)
+    assert torch.equal(ops.gemm(x, wp), ops.gemm_skinny(x, wp))
+
+
+@pytest.mark.parametrize("B,S,H,Hkv,D,K", [(2, 100, 6, 6, 128, 768), (3, 40, 4, 2, 16, 64)])
+def test_qkv_rope_append_many_rows(cuda, B, S, H, Hkv, D, K):
+    """More than 64 rows without a fused norm: the tiled kernel with the rotary/append epilogue."""
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(S)
+    Tmax, pos = 128, 5
+    x = torch.randn(B * S, K, generator=g).to(BF)
+    wq = (torch.randn(H * D, K, generator=g) * 0.05).to(BF)
+    wk = (torch.randn(Hkv * D, K, generator=g) * 0.05).to(BF)
+    wv = (torch.randn(Hkv * D, K, generator=g) * 0.05).to(BF)
+    cos, sin = R.rope_table(D, 2 * Tmax, 10000.0)
+    cos, sin = cos.to(BF), sin.to(BF)
+    q = R.linear(x, wq).view(B, S, H, D)
+    k = R.linear(x, wk).view(B, S, Hkv, D)
+    v = R.linear(x, wv).view(B, S, Hkv, D)
+    qr, kr = R.apply_rope(q, k, cos[pos : pos + S], sin[pos : pos + S])
+    kc = torch.zeros(B, Tmax, Hkv, D, dtype=BF, device=cuda)
+    vc = torch.zeros_like(kc)
+    wp = ops.pack_qkv(wq.to(cuda), wk.to(cuda), wv.to(cuda))
+    qo = ops.qkv_rope_append(x.to(cuda), wp, None, 1e-5, H, Hkv, D, cos.to(cuda), sin.to(cuda), pos, kc, vc, seq_len=S)
+    for got, ref in ((qo.view(B, S, H, D), qr), (kc[:, pos : pos + S], kr), (vc[:, pos : pos + S], v)):
+        scale = ref.float().abs().max().item()
+        err = (got.cpu().float() - ref.float()).abs().max().item()
+        assert err <= 2 ** -6 * scale, (err, scale)
+        assert (got.cpu() != ref).float().mean().item() < 0.08
+    assert kc[:, :pos].abs().sum().item() == 0 and kc[:, pos + S :].abs().sum().item() == 0
