@@ -36,6 +36,9 @@ __device__ __forceinline__ float dot8(uint4 a, uint4 b, float s) {
   return s;
 }
 
+__device__ __forceinline__ float ldf_coh(const float* p) { return __uint_as_float(ld_coh4(p)); }
+__device__ __forceinline__ void stf_coh(float* p, float v) { st_coh4(p, __float_as_uint(v)); }
+
 // Merge the chunk partials of the G heads of (b, kvh) and write bf16 output.
 // Called by all 256 threads of the last workgroup to finish.  The partial loads are
 // issued eight chunks at a time before any is consumed (a dependent chain of global
@@ -52,7 +55,7 @@ __device__ void merge_partials(const AttnArgs& a, int b /* query row */, int kvh
     for (int s0 = 0; s0 < ns; s0 += 8) {
       float mv[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) mv[i] = (s0 + i < ns) ? ml[2 * (s0 + i)] : -INFINITY;
+      for (int i = 0; i < 8; ++i) mv[i] = (s0 + i < ns) ? ldf_coh(ml + 2 * (s0 + i)) : -INFINITY;
 #pragma unroll
       for (int i = 0; i < 8; ++i) M = fmaxf(M, mv[i]);
     }
@@ -62,9 +65,9 @@ __device__ void merge_partials(const AttnArgs& a, int b /* query row */, int kvh
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const bool in = s0 + i < ns;
-        mv[i] = in ? ml[2 * (s0 + i)] : -INFINITY;
-        lv[i] = in ? ml[2 * (s0 + i) + 1] : 0.f;
-        av[i] = in ? pa[(size_t)(s0 + i) * D] : 0.f;
+        mv[i] = in ? ldf_coh(ml + 2 * (s0 + i)) : -INFINITY;
+        lv[i] = in ? ldf_coh(ml + 2 * (s0 + i) + 1) : 0.f;
+        av[i] = in ? ldf_coh(pa + (size_t)(s0 + i) * D) : 0.f;
       }
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -77,21 +80,22 @@ __device__ void merge_partials(const AttnArgs& a, int b /* query row */, int kvh
   }
 }
 
-// Publishes this workgroup's partials and returns true in the workgroup that
-// observes all n_split chunks done (every thread gets the same answer).
+// Counts this workgroup's chunk as done and returns true in the workgroup that observes all
+// n_split chunks done (every thread gets the same answer).  The partials were written with
+// write-through stores; the workgroup-scope fence waits for their completion, the counter is a
+// relaxed device-scope atomic and the merge reads with cache-bypassing loads: no L2
+// write-back or invalidate.
 __device__ bool last_chunk_done(int* counter, int nsplit) {
   __shared__ int is_last;
-  __threadfence();  // partials visible device-wide before the count
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __syncthreads();
   if (threadIdx.x == 0) {
-    const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     is_last = (old == nsplit - 1);
     if (is_last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next call
   }
   __syncthreads();
-  const bool last = is_last != 0;
-  if (last) __threadfence();  // acquire the other chunks' partials
-  return last;
+  return is_last != 0;
 }
 
 template <int D, int G>
@@ -134,18 +138,26 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   const bf16_t* kb = a.k + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
   const bf16_t* vb = a.v + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
 
-  for (int tb = t0 + wave * 16; tb < t1; tb += 64) {
+  // 16-position tiles, wave w takes tiles w, w+4, ...; the loads of the next tile are in
+  // flight while the current one is consumed
+  auto load_tile = [&](int tb, uint4* kv, uint4* vv) {
     const int pos = tb + p;
-    const bool valid = pos < t1;
-    uint4 kv[NC], vv[NV];
 #pragma unroll
     for (int c = 0; c < NC; ++c)
-      kv[c] = valid ? ldg16_nt(kb + (size_t)pos * row + (4 * c + dq) * 8) : make_uint4(0, 0, 0, 0);
+      kv[c] = pos < t1 ? ldg16_nt(kb + (size_t)pos * row + (4 * c + dq) * 8) : make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int c = 0; c < NV; ++c) {
       const int vp = tb + c * PP + pp;
       vv[c] = vp < t1 ? ldg16_nt(vb + (size_t)vp * row + dc * 8) : make_uint4(0, 0, 0, 0);
     }
+  };
+  uint4 kv[NC], vv[NV], kn[NC], vn[NV];
+  int tb = t0 + wave * 16;
+  if (tb < t1) load_tile(tb, kv, vv);
+  for (; tb < t1; tb += 64) {
+    const bool valid = tb + p < t1;
+    const bool more = tb + 64 < t1;
+    if (more) load_tile(tb + 64, kn, vn);
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) {
       float s = 0.f;
@@ -177,6 +189,12 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
           acc[hh][2 * i + 1] += pw * hi_bf(w4[i]);
         }
       }
+    }
+    if (more) {
+#pragma unroll
+      for (int c = 0; c < NC; ++c) kv[c] = kn[c];
+#pragma unroll
+      for (int c = 0; c < NV; ++c) vv[c] = vn[c];
     }
   }
 
@@ -217,10 +235,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
       continue;
     }
     const size_t pi = (size_t)(b * a.H + h) * a.nsplit + split;
-    a.part_acc[pi * D + d] = o;
+    stf_coh(a.part_acc + pi * D + d, o);
     if (d == 0) {
-      a.part_ml[pi * 2] = M;
-      a.part_ml[pi * 2 + 1] = Ls;
+      stf_coh(a.part_ml + pi * 2, M);
+      stf_coh(a.part_ml + pi * 2 + 1, Ls);
     }
   }
   if (a.nsplit == 1) return;
@@ -285,10 +303,10 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
       continue;
     }
     const size_t pi = (size_t)(b * a.H + h) * a.nsplit + split;
-    if (tid < D) a.part_acc[pi * D + tid] = acc;
+    if (tid < D) stf_coh(a.part_acc + pi * D + tid, acc);
     if (tid == 0) {
-      a.part_ml[pi * 2] = m_run;
-      a.part_ml[pi * 2 + 1] = l_run;
+      stf_coh(a.part_ml + pi * 2, m_run);
+      stf_coh(a.part_ml + pi * 2 + 1, l_run);
     }
   }
   if (a.nsplit == 1) return;

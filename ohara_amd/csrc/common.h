@@ -49,6 +49,32 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Device-coherent accesses without fences.  The eight XCDs' L2 caches are not coherent with
+// each other; relaxed agent-scope atomics compile to write-through stores / cache-bypassing
+// loads (sc1), so data handed from one workgroup to another is published by such stores, a
+// wait for their completion (a workgroup-scope release fence) and a relaxed atomic counter,
+// and is read with such loads.  An agent-scope fence instead writes back / invalidates a whole
+// L2, which serialises across workgroups (~0.2 us each on this chip).
+__device__ __forceinline__ void st_coh8(void* p, uint2 v) {
+  __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), ((unsigned long long)v.y << 32) | v.x,
+                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_coh4(void* p, uint32_t v) {
+  __hip_atomic_store(reinterpret_cast<uint32_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint2 ld_coh8(const void* p) {
+  const unsigned long long v =
+      __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return make_uint2((uint32_t)v, (uint32_t)(v >> 32));
+}
+__device__ __forceinline__ uint4 ld_coh16(const void* p) {
+  const uint2 a = ld_coh8(p), b = ld_coh8(reinterpret_cast<const char*>(p) + 8);
+  return make_uint4(a.x, a.y, b.x, b.y);
+}
+__device__ __forceinline__ uint32_t ld_coh4(const void* p) {
+  return __hip_atomic_load(reinterpret_cast<const uint32_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
 
 // Host-side launch check: every entry point returns OHARA_ELAUNCH when the

@@ -70,26 +70,6 @@ struct Prof {
   }
 };
 
-__device__ __forceinline__ void st_coh8(void* p, uint2 v) {
-  __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), ((unsigned long long)v.y << 32) | v.x,
-                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void st_coh4(void* p, uint32_t v) {
-  __hip_atomic_store(reinterpret_cast<uint32_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ uint2 ld_coh8(const void* p) {
-  const unsigned long long v =
-      __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  return make_uint2((uint32_t)v, (uint32_t)(v >> 32));
-}
-__device__ __forceinline__ uint4 ld_coh16(const void* p) {
-  const uint2 a = ld_coh8(p), b = ld_coh8(reinterpret_cast<const char*>(p) + 8);
-  return make_uint4(a.x, a.y, b.x, b.y);
-}
-__device__ __forceinline__ uint32_t ld_coh4(const void* p) {
-  return __hip_atomic_load(reinterpret_cast<const uint32_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 // ---------------------------------------------------------------------------------------
 // Grid barrier.  Two levels of monotonic counters (groups of 16 workgroups, each counter on
 // its own 256-byte line, then one counter over the groups) and a release word everyone

@@ -59,12 +59,36 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const bf16_t* logits, int 
   const int n = min(valid, vocab);
   float best = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < n; i += 1024) {
-    const float v = bf2f(row[i]);
+  auto take = [&](float v, int i) {
     if (v > best || (v == best && i < bi)) {
       best = v;
       bi = i;
     }
+  };
+  if (((ldl & 7) == 0) && ((reinterpret_cast<uintptr_t>(logits) & 15) == 0)) {
+    // 16-byte loads, four in flight per thread
+    const int n8 = n >> 3;
+    for (int c0 = threadIdx.x; c0 < n8; c0 += 4 * 1024) {
+      uint4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int c = c0 + u * 1024;
+        v[u] = c < n8 ? ldg16(row + (size_t)c * 8) : make_uint4(0xff80ff80u, 0xff80ff80u, 0xff80ff80u, 0xff80ff80u);  // -inf
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i0 = (c0 + u * 1024) * 8;
+        const uint32_t w[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          take(lo_bf(w[j]), i0 + 2 * j);
+          take(hi_bf(w[j]), i0 + 2 * j + 1);
+        }
+      }
+    }
+    for (int i = (n8 << 3) + threadIdx.x; i < n; i += 1024) take(bf2f(row[i]), i);
+  } else {
+    for (int i = threadIdx.x; i < n; i += 1024) take(bf2f(row[i]), i);
   }
   // NaN-free comparison network; ties resolve to the lowest index
 #pragma unroll
@@ -95,8 +119,8 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const bf16_t* logits, int 
     if (st) {
       const int step = st->step;
       if (history && step < hist_cap) history[(size_t)step * B + b] = bi;
-      __threadfence();
-      const int old = __hip_atomic_fetch_add(&st->done, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      // only the counter is shared between workgroups: no fence, the ids are read by later kernels
+      const int old = __hip_atomic_fetch_add(&st->done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (old == B - 1) {
         st->done = 0;
         st->pos += 1;

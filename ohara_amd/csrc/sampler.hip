@@ -383,8 +383,8 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
     if (a.step_state) {
       const int step = a.step_state[1];
       if (a.history && step < a.hist_cap) a.history[(size_t)step * a.B + b] = token;
-      __threadfence();
-      const int old = __hip_atomic_fetch_add(&a.step_state[2], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      // only the counter is shared between workgroups: no fence, the ids are read by later kernels
+      const int old = __hip_atomic_fetch_add(&a.step_state[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (old == a.B - 1) {
         a.step_state[2] = 0;
         a.step_state[0] += 1;
