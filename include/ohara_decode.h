@@ -123,6 +123,13 @@ int ohara_attn_cached_bf16(const uint16_t* q, const uint16_t* kcache, const uint
                            int seq_len, int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev,
                            int n_split, void* workspace, uint16_t* out, void* stream);
 
+/* Same contract for many query positions per sequence (prefill), as a causal flash-style kernel
+ * on MFMA: 128 queries per workgroup, keys/values walked in 64-position tiles through LDS,
+ * online softmax in fp32, probabilities rounded to bf16 for the second product.  dh 64 or 128.
+ * Needs no workspace.  (llama.py:100-135 with S > 1.) */
+int ohara_attn_prefill_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch,
+                            int seq_len, int h, int h_kv, int dh, int t_max, int pos, uint16_t* out, void* stream);
+
 /* ---- greedy selection ---------------------------------------------------------
  * next_ids[b] = first index of max(logits[b, 0:valid_vocab])  (argmax of the last
  * position, ohara/chat_engine.py:61-63, ohara/inference.py:40-45; ids >= valid_vocab

@@ -49,8 +49,12 @@ extern "C" int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* 
     OHARA_RUN(ohara_qkv_rope_append_bf16(tiled ? s->xn : s->x, d, L.wqkv, d, tiled ? nullptr : L.norm1, m->eps, B,
                                          seq_len, H, Hkv, Dh, m->cos, m->sin, pos, pos_dev, s->q, s->kcache[l],
                                          s->vcache[l], m->t_max, stream));
-    OHARA_RUN(ohara_attn_cached_bf16(s->q, s->kcache[l], s->vcache[l], B, seq_len, H, Hkv, Dh, m->t_max, pos, pos_dev,
-                                n_split, s->attn_ws, s->attn, stream));
+    if (seq_len >= 16 && (Dh == 64 || Dh == 128))
+      OHARA_RUN(ohara_attn_prefill_bf16(s->q, s->kcache[l], s->vcache[l], B, seq_len, H, Hkv, Dh, m->t_max, pos, s->attn,
+                                        stream));
+    else
+      OHARA_RUN(ohara_attn_cached_bf16(s->q, s->kcache[l], s->vcache[l], B, seq_len, H, Hkv, Dh, m->t_max, pos, pos_dev,
+                                       n_split, s->attn_ws, s->attn, stream));
     OHARA_RUN(ohara_gemm_skinny_bf16(s->attn, H * Dh, L.wo, d, H * Dh, nullptr, m->eps, R, OHARA_EPI_RESIDUAL, s->x, d,
                                 s->x, d, stream));
     if (tiled) {

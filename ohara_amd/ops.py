@@ -185,6 +185,23 @@ def attn_cached(q, kcache, vcache, h, h_kv, dh, pos, n_split, workspace, out=Non
     return out
 
 
+def attn_prefill(q, kcache, vcache, h, h_kv, dh, pos, seq_len, out=None):
+    """q: (batch*seq_len, h*dh); causal attention of seq_len queries per sequence over cache
+    positions [0, pos + s] on the MFMA prefill kernel."""
+    _need(q, BF16, "q")
+    rows = q.shape[0]
+    if out is None:
+        out = torch.empty(rows, h * dh, dtype=BF16, device=q.device)
+    check(
+        lib().ohara_attn_prefill_bf16(
+            _ptr(q), _ptr(kcache), _ptr(vcache), rows // seq_len, seq_len, h, h_kv, dh, kcache.shape[1], int(pos),
+            _ptr(out), _stream(),
+        ),
+        "attn_prefill",
+    )
+    return out
+
+
 def attn_decode(q, kcache, vcache, h, h_kv, dh, length, n_split, workspace, out=None, pos_dev=None):
     """Decode case: one query per sequence seeing `length` cached positions."""
     return attn_cached(q, kcache, vcache, h, h_kv, dh, length - 1, n_split, workspace, out, pos_dev, 1)

@@ -275,3 +275,30 @@ def test_qkv_rope_append_many_rows(cuda, B, S, H, Hkv, D, K):
         assert err <= 2 ** -6 * scale, (err, scale)
         assert (got.cpu() != ref).float().mean().item() < 0.08
     assert kc[:, :pos].abs().sum().item() == 0 and kc[:, pos + S :].abs().sum().item() == 0
+
+
+# ---- causal prefill attention on MFMA ----------------------------------------------------------
+
+@pytest.mark.parametrize("B,S,H,Hkv,D,pos", [(2, 128, 6, 6, 128, 0), (1, 300, 4, 2, 128, 0), (3, 77, 8, 8, 64, 0),
+                                             (2, 130, 8, 2, 64, 45), (1, 16, 2, 1, 128, 200), (1, 1024, 2, 2, 128, 0)])
+def test_attn_prefill(cuda, B, S, H, Hkv, D, pos):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(S + pos)
+    Tmax = pos + S + 5
+    q = torch.randn(B, S, H, D, generator=g).to(BF)
+    k = torch.randn(B, Tmax, Hkv, D, generator=g).to(BF)
+    v = torch.randn(B, Tmax, Hkv, D, generator=g).to(BF)
+    # positions past the fed tokens hold junk the kernel must not read into the result
+    k[:, pos + S :] = 1e4
+    v[:, pos + S :] = -1e4
+    ref = R.attention_core(q, k[:, : pos + S], v[:, : pos + S], pos).float()  # fp32 softmax, one rounding
+    out = ops.attn_prefill(q.to(cuda).view(B * S, H * D), k.to(cuda), v.to(cuda), H, Hkv, D, pos, S)
+    got = out.cpu().float().view(B, S, H * D)
+    scale = ref.abs().max().item()
+    assert (got - ref).abs().max().item() <= 2e-2 * max(1.0, scale)
+    assert (got - ref).abs().mean().item() <= 2e-3 * max(1.0, scale)
+    # the one-query-per-row decode kernel computes the same function
+    ws = ops.attn_workspace(B * S, H, Hkv, D, 1, cuda)
+    dec = ops.attn_cached(q.to(cuda).view(B * S, H * D), k.to(cuda), v.to(cuda), H, Hkv, D, pos, 1, ws, seq_len=S)
+    assert (dec.cpu().float().view(B, S, H * D) - got).abs().max().item() <= 2e-2 * max(1.0, scale)
