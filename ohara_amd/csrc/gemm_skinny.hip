@@ -45,7 +45,7 @@ __device__ __forceinline__ uint4 norm8(uint4 xv, uint4 wv, float rinv) {
 
 template <int BT, bool NORM, int EPI>
 __global__ __launch_bounds__(256) void skinny_kernel(GemmArgs a) {
-  constexpr int CH = 6;  // k-steps whose weight loads are issued back to back
+  constexpr int CH = BT <= 2 ? 6 : 4;  // k-steps whose loads are issued back to back
   const int strip = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 15, g = lane >> 4;
@@ -91,32 +91,37 @@ __global__ __launch_bounds__(256) void skinny_kernel(GemmArgs a) {
 
   const uint4* wrow = a.wp + (size_t)strip * KS * 64 + lane;
 
-  auto step = [&](uint4 wv, int j) {
-    const int k0 = 32 * j + 8 * g;
-    uint4 nw = make_uint4(0, 0, 0, 0);
-    if (NORM && k0 < a.K) nw = ldg16(a.norm_w + k0);
+  // A group of CH k-steps: all loads of the group (weights, norm weights, the activations of
+  // every 16-row block) are issued before the first product, so their latencies overlap.
+  auto group = [&](int j, int n) {  // k-steps j .. j+n-1, n <= CH
+    uint4 wv[CH], nw[CH], xv[CH][BT];
 #pragma unroll
-    for (int t = 0; t < BT; ++t) {
-      const int b = m + 16 * t;
-      uint4 xv = make_uint4(0, 0, 0, 0);
-      if (b < a.B && k0 < a.K) {
-        xv = ldg16(a.x + (size_t)b * a.ldx + k0);
-        if (NORM) xv = norm8(xv, nw, rinv[t]);
+    for (int c = 0; c < CH; ++c) {
+      const int k0 = 32 * (j + c) + 8 * g;
+      const bool in = c < n;
+      wv[c] = in ? ldg16_nt(wrow + (size_t)(j + c) * 64) : make_uint4(0, 0, 0, 0);
+      nw[c] = (NORM && in && k0 < a.K) ? ldg16(a.norm_w + k0) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < BT; ++t) {
+        const int b = m + 16 * t;
+        xv[c][t] = (in && b < a.B && k0 < a.K) ? ldg16(a.x + (size_t)b * a.ldx + k0) : make_uint4(0, 0, 0, 0);
       }
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wv),
-                                                       __builtin_bit_cast(bf16x8, xv), acc[t], 0, 0, 0);
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+#pragma unroll
+      for (int t = 0; t < BT; ++t) {
+        uint4 xn = xv[c][t];
+        if (NORM) xn = norm8(xn, nw[c], rinv[t]);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wv[c]),
+                                                         __builtin_bit_cast(bf16x8, xn), acc[t], 0, 0, 0);
+      }
     }
   };
 
   int j = j0;
-  for (; j + CH <= j1; j += CH) {
-    uint4 wv[CH];
-#pragma unroll
-    for (int c = 0; c < CH; ++c) wv[c] = ldg16_nt(wrow + (size_t)(j + c) * 64);
-#pragma unroll
-    for (int c = 0; c < CH; ++c) step(wv[c], j + c);
-  }
-  for (; j < j1; ++j) step(ldg16_nt(wrow + (size_t)j * 64), j);
+  for (; j + CH <= j1; j += CH) group(j, CH);
+  if (j < j1) group(j, j1 - j);
 
   // Fixed-order cross-wave sum: ((w0 + w1) + w2) + w3.
   if (wave > 0) {
