@@ -116,7 +116,8 @@ int ohara_qkv_rope_append_bf16(const uint16_t* x, int ldx, const uint16_t* wp, i
  * partial (max, sum, acc) triples go to `workspace` and the last chunk to finish
  * merges them in chunk order.  workspace bytes = ohara_attn_workspace_bytes(
  * batch*seq_len, h, h_kv, dh, n_split); zero-fill it once before first use (the
- * kernels leave its counters at zero).  n_split = 1 needs no workspace (NULL ok).
+ * kernels leave its counters at zero).  n_split = 1 needs no workspace (NULL ok);
+ * n_split > 1 needs (h / h_kv) * n_split <= 2048.
  * q / out: (batch*seq_len, h*dh). */
 int64_t ohara_attn_workspace_bytes(int batch, int h, int h_kv, int dh, int n_split);
 int ohara_attn_cached_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch,

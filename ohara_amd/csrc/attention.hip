@@ -39,44 +39,57 @@ __device__ __forceinline__ float dot8(uint4 a, uint4 b, float s) {
 __device__ __forceinline__ float ldf_coh(const float* p) { return __uint_as_float(ld_coh4(p)); }
 __device__ __forceinline__ void stf_coh(float* p, float v) { st_coh4(p, __float_as_uint(v)); }
 
-// Merge the chunk partials of the G heads of (b, kvh) and write bf16 output.
-// Called by all 256 threads of the last workgroup to finish.  The partial loads are
-// issued eight chunks at a time before any is consumed (a dependent chain of global
-// loads costs about a microsecond per link on this chip).
+// Merge the chunk partials of the G heads of (b, kvh) and write bf16 output.  Called by all
+// 256 threads of the last workgroup to finish.  A chain of dependent device-coherent loads
+// costs about a microsecond per link on this chip, so the (max, sum) pairs of all chunks are
+// fetched in one round into LDS, the chunk weights exp(m_s - M) are formed there, and the
+// accumulator columns are then summed in chunk order with their loads issued eight at a time.
+// Needs G * n_split <= OHARA_MERGE_CAP.
+#define OHARA_MERGE_CAP 2048
 template <int MAXD>
 __device__ void merge_partials(const AttnArgs& a, int b /* query row */, int kvh, int G) {
+  __shared__ float s_w[OHARA_MERGE_CAP];   // max, then weight, of (head, chunk)
+  __shared__ float s_ls[OHARA_MERGE_CAP];  // sum of (head, chunk)
+  __shared__ float s_tot[64];              // per head: normaliser
   const int D = a.D, ns = a.nsplit;
-  for (int idx = threadIdx.x; idx < G * D; idx += blockDim.x) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const float* ml0 = a.part_ml + ((size_t)(b * a.H + kvh * G) * ns) * 2;  // heads of a group are adjacent
+  for (int i = tid; i < G * ns; i += blockDim.x) {
+    const uint2 v = ld_coh8(ml0 + 2 * (size_t)i);
+    s_w[i] = __uint_as_float(v.x);
+    s_ls[i] = __uint_as_float(v.y);
+  }
+  __syncthreads();
+  for (int hh = wave; hh < G; hh += 4) {
+    float M = -INFINITY;
+    for (int s0 = lane; s0 < ns; s0 += 64) M = fmaxf(M, s_w[hh * ns + s0]);
+    M = wave_max(M);
+    float L = 0.f;
+    for (int s0 = lane; s0 < ns; s0 += 64) {
+      const float ms = s_w[hh * ns + s0];
+      const float w = (ms == -INFINITY) ? 0.f : __expf(ms - M);
+      s_w[hh * ns + s0] = w;
+      L += s_ls[hh * ns + s0] * w;
+    }
+    L = wave_sum(L);
+    if (lane == 0) s_tot[hh] = L;
+  }
+  __syncthreads();
+  for (int idx = tid; idx < G * D; idx += blockDim.x) {
     const int hh = idx / D, d = idx - hh * D;
     const int h = kvh * G + hh;
-    const float* ml = a.part_ml + ((size_t)(b * a.H + h) * ns) * 2;
     const float* pa = a.part_acc + ((size_t)(b * a.H + h) * ns) * D + d;
-    float M = -INFINITY;
+    const float* w = s_w + hh * ns;
+    float o = 0.f;
     for (int s0 = 0; s0 < ns; s0 += 8) {
-      float mv[8];
+      float av[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) mv[i] = (s0 + i < ns) ? ldf_coh(ml + 2 * (s0 + i)) : -INFINITY;
+      for (int i = 0; i < 8; ++i) av[i] = (s0 + i < ns) ? ldf_coh(pa + (size_t)(s0 + i) * D) : 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) M = fmaxf(M, mv[i]);
+      for (int i = 0; i < 8; ++i)
+        if (s0 + i < ns) o += av[i] * w[s0 + i];
     }
-    float Lsum = 0.f, o = 0.f;
-    for (int s0 = 0; s0 < ns; s0 += 8) {
-      float mv[8], lv[8], av[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const bool in = s0 + i < ns;
-        mv[i] = in ? ldf_coh(ml + 2 * (s0 + i)) : -INFINITY;
-        lv[i] = in ? ldf_coh(ml + 2 * (s0 + i) + 1) : 0.f;
-        av[i] = in ? ldf_coh(pa + (size_t)(s0 + i) * D) : 0.f;
-      }
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float w = (mv[i] == -INFINITY) ? 0.f : __expf(mv[i] - M);
-        Lsum += lv[i] * w;
-        o += av[i] * w;
-      }
-    }
-    a.out[(size_t)b * a.H * D + h * D + d] = f2bf(o / Lsum);
+    a.out[(size_t)b * a.H * D + h * D + d] = f2bf(o / s_tot[hh]);
   }
 }
 
@@ -345,6 +358,7 @@ int ohara_attn_cached_bf16(const uint16_t* q, const uint16_t* kcache, const uint
   if (batch < 1 || seq_len < 1 || h < 1 || h_kv < 1 || h % h_kv || dh < 2 || (dh & 1) || dh > 256)
     return OHARA_EINVAL;
   if (t_max < 1 || n_split < 1 || n_split > 1024) return OHARA_EINVAL;
+  if (n_split > 1 && ((h / h_kv) * n_split > OHARA_MERGE_CAP || h / h_kv > 64)) return OHARA_ESIZE;
   if (n_split > 1 && !workspace) return OHARA_EINVAL;
   if (!pos_dev && (pos < 0 || pos + seq_len > t_max)) return OHARA_EINVAL;
   if ((int64_t)batch * seq_len > INT32_MAX / 2 || h_kv > 65535) return OHARA_ESIZE;

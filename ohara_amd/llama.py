@@ -243,9 +243,9 @@ class Llama:
 
     def default_n_split(self, batch: int) -> int:
         """Context chunks per (sequence, KV head) so that decode attention launches about
-        two workgroups per CU; a chunk is never shorter than 64 positions."""
-        want = max(1, 512 // max(1, batch * self.kv_heads))
-        return max(1, min(want, self.config.max_sequence_length // 64, 32))
+        four workgroups per CU; a chunk is never shorter than 128 positions."""
+        want = max(1, 1024 // max(1, batch * self.kv_heads))
+        return max(1, min(want, self.config.max_sequence_length // 128, 64))
 
     def _get_buffers(self, batch: int, rows: int) -> _Buffers:
         key = (batch, rows)
