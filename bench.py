@@ -151,6 +151,213 @@ def cpu_baseline(budget_s=20.0):
     }
 
 
+# ---------------------------------------------------------------------------------------------
+# Per-kernel figures of the other configurations (attention microbench, prefill on MFMA, BitNet
+# ternary decode, MoE decode).  Each is timed as a HIP graph replay, so host launch cost is out.
+# ---------------------------------------------------------------------------------------------
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def graph_time(fn, iters=10):
+    """Seconds per call of fn(), captured once into a HIP graph and replayed `iters` times."""
+    fn()
+    fn()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters * 1e-3
+
+
+def bench_attention_microbench(dev):
+    """GQA decode attention, 32 query / 8 KV heads x 128, one query per sequence over L cached
+    positions.  Algorithmic bytes: K + V (4*Hkv*D*B*L) + Q and O (4*H*D*B)."""
+    from ohara_amd import ops
+
+    H, Hkv, D = 32, 8, 128
+    out = []
+    for B, L in ((1, 4096), (1, 32768), (16, 4096), (16, 32768), (64, 4096), (64, 32768)):
+        ns = max(1, min(1024 // (B * Hkv), L // 128, 64))
+        g = torch.Generator(device=dev).manual_seed(1)
+        q = torch.randn(B, H * D, device=dev, generator=g).to(torch.bfloat16)
+        k = torch.randn(B, L, Hkv, D, device=dev, generator=g).to(torch.bfloat16)
+        v = torch.randn(B, L, Hkv, D, device=dev, generator=g).to(torch.bfloat16)
+        ws = ops.attn_workspace(B, H, Hkv, D, ns, dev)
+        o = torch.empty(B, H * D, device=dev, dtype=torch.bfloat16)
+        t = graph_time(lambda: ops.attn_decode(q, k, v, H, Hkv, D, L, ns, ws, o))
+        by = 4.0 * Hkv * D * B * L + 4.0 * H * D * B
+        out.append({"batch": B, "context": L, "n_split": ns, "us": round(t * 1e6, 1), "GBs": round(by / t / 1e9, 1),
+                    "frac_of_hbm_peak": round(by / t / 1e9 / HBM_PEAK_GBS, 4)})
+        del q, k, v, ws, o
+        torch.cuda.empty_cache()
+    return out
+
+
+def bench_prefill(model, cfg, dev):
+    """Batched prefill of the d12 model (1024 tokens per sequence) and its MFMA kernels alone."""
+    from ohara_amd import ops
+
+    res = {}
+    B, S = 8, 1024
+    prompt = torch.randint(0, cfg.vocab_size, (B, S), device=dev)
+    for _ in range(2):
+        cache = model.build_kv_cache(B)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        model(prompt, cache, 0, last_only=True)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+    d, f = cfg.hidden_size, cfg.intermediate_size
+    flops = 2.0 * B * S * cfg.num_hidden_layers * (4 * d * d + 3 * d * f) + 4.0 * B * d * S * (S + 1) / 2 * cfg.num_hidden_layers
+    res["d12_prefill"] = {"batch": B, "prompt": S, "ms": round(dt * 1e3, 3), "tokens_per_s": round(B * S / dt, 1),
+                          "TFLOPs": round(flops / dt / 1e12, 1)}
+    del cache
+    M = B * S
+    x = torch.randn(M, f, device=dev).to(torch.bfloat16)
+    kern = []
+    for name, n, k, kind in (("qkv 2304x768", 3 * d, d, "store"), ("wo 768x768", d, d, "store"),
+                             ("gate/up 2x3072x768 + SwiGLU", f, d, "swiglu"), ("down 768x3072", d, f, "store")):
+        if kind == "swiglu":
+            wp = ops.pack_gate_up((torch.randn(n, k, device=dev) * 0.02).to(torch.bfloat16),
+                                  (torch.randn(n, k, device=dev) * 0.02).to(torch.bfloat16))
+            fl = 2.0 * M * 2 * n * k
+        else:
+            wp = ops.pack_linear((torch.randn(n, k, device=dev) * 0.02).to(torch.bfloat16))
+            fl = 2.0 * M * n * k
+        o = torch.empty(M, n, device=dev, dtype=torch.bfloat16)
+        xin = x[:, :k]
+        t = graph_time(lambda: ops.gemm(xin, wp, out=o))
+        kern.append({"kernel": "gemm_tile_kernel " + name, "rows": M, "us": round(t * 1e6, 1),
+                     "TFLOPs": round(fl / t / 1e12, 1), "mfma_util": round(fl / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
+    H, D = cfg.num_attention_heads, d // cfg.num_attention_heads
+    q = torch.randn(M, d, device=dev).to(torch.bfloat16)
+    kk = torch.randn(B, S, H, D, device=dev).to(torch.bfloat16)
+    vv = torch.randn(B, S, H, D, device=dev).to(torch.bfloat16)
+    o = torch.empty_like(q)
+    t = graph_time(lambda: ops.attn_prefill(q, kk, vv, H, H, D, 0, S, o))
+    fl = 4.0 * B * H * D * S * (S + 1) / 2
+    kern.append({"kernel": "attn_prefill_kernel<128> causal", "rows": M, "us": round(t * 1e6, 1),
+                 "TFLOPs": round(fl / t / 1e12, 1), "mfma_util": round(fl / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
+    res["mfma_kernels"] = kern
+    return res
+
+
+def _fill_cache(cache, length, batch):
+    for c in cache:
+        c.key.normal_()
+        c.value.normal_()
+        c.length, c.batch_size = length, batch
+
+
+def bench_bitnet(dev):
+    """BitNet-b1.58 ternary Llama (d 2048, 24 layers, 16 x 128 heads, FFN 5632, vocab 32000):
+    one decode step at context 2048, batch 1 and 8."""
+    from ohara_amd.bitnet import BIT_TARGETS, BitLlama
+    from ohara_amd.llama import Config
+
+    cfg = Config(vocab_size=32000, hidden_size=2048, intermediate_size=5632, num_attention_heads=16,
+                 num_key_value_heads=0, num_hidden_layers=24, max_sequence_length=2048, dropout=0.0)
+    g = torch.Generator(device=dev).manual_seed(2)
+    d, f, v = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    shapes = {"attn.key": (d, d), "attn.query": (d, d), "attn.value": (d, d), "attn.proj": (d, d),
+              "ff.gate": (f, d), "ff.up": (f, d), "ff.down": (d, f)}
+    st = {"token_emb.weight": (torch.randn(v, d, device=dev, generator=g) * 0.02).to(torch.bfloat16),
+          "vocab_proj.weight": (torch.randn(v, d, device=dev, generator=g) * 0.02).to(torch.bfloat16),
+          "norm.weight": torch.ones(d, device=dev)}
+    for i in range(cfg.num_hidden_layers):
+        p = f"layers.{i}."
+        for nm in BIT_TARGETS:
+            n, k = shapes[nm]
+            st[p + nm + ".ternary"] = torch.randint(-1, 2, (n, k), device=dev, generator=g, dtype=torch.int8)
+            st[p + nm + ".gamma"] = 0.02
+            st[p + nm + ".rms_norm.weight"] = torch.ones(k, device=dev)
+        st[p + "norm1.weight"] = torch.ones(d, device=dev)
+        st[p + "norm2.weight"] = torch.ones(d, device=dev)
+    model = BitLlama(cfg, st, device=dev)
+    del st
+    out = []
+    L = cfg.max_sequence_length
+    for B in (1, 8):
+        cache = model.build_kv_cache(B)
+        ids = torch.randint(0, v, (B, 1), device=dev)
+
+        def step():
+            _fill_len(cache, L - 1, B)
+            return model(ids, cache, L - 1, last_only=True)
+
+        _fill_cache(cache, L - 1, B)
+        t = graph_time(step)
+        by = model.packed_weight_bytes() + 2.0 * v * d + 2.0 * 2 * d * cfg.num_hidden_layers * B * L
+        out.append({"batch": B, "context": L, "ms_per_step": round(t * 1e3, 4), "tokens_per_s": round(B / t, 1),
+                    "step_bytes": int(by), "GBs": round(by / t / 1e9, 1),
+                    "frac_of_hbm_peak": round(by / t / 1e9 / HBM_PEAK_GBS, 4)})
+        del cache
+        torch.cuda.empty_cache()
+    return out
+
+
+def _fill_len(cache, length, batch):
+    for c in cache:
+        c.length, c.batch_size = length, batch
+
+
+def bench_moe(dev):
+    """MoE decode (16 layers, d 1024, 16 x 64 heads, 64 routed SwiGLU experts of hidden 512, top-8,
+    one shared expert): one step of 64 sequences at context 2048."""
+    from ohara_amd.llama import Config
+    from ohara_amd.moe import MoeLlama
+
+    cfg = Config(vocab_size=32000, hidden_size=1024, intermediate_size=512, num_attention_heads=16,
+                 num_key_value_heads=0, num_hidden_layers=16, max_sequence_length=2048, dropout=0.0,
+                 moe_num_experts=64, moe_experts_per_tok=8, moe_grouped=True, moe_num_shared_experts=1)
+    g = torch.Generator(device=dev).manual_seed(3)
+    d, f, v, E = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.moe_num_experts
+
+    def n(*shape):
+        return (torch.randn(*shape, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+
+    st = {"token_emb.weight": n(v, d), "vocab_proj.weight": n(v, d), "norm.weight": torch.ones(d, device=dev)}
+    for i in range(cfg.num_hidden_layers):
+        p = f"layers.{i}."
+        for nm in ("key", "query", "value", "proj"):
+            st[p + f"attn.{nm}.weight"] = n(d, d)
+        st[p + "ff.w_gate"], st[p + "ff.w_up"], st[p + "ff.w_down"] = n(E, d, f), n(E, d, f), n(E, f, d)
+        st[p + "ff.router.weight"] = (torch.randn(E, d, device=dev, generator=g) / d ** 0.5).to(torch.bfloat16)
+        st[p + "ff.router_bias"] = torch.zeros(E, device=dev)
+        st[p + "ff.shared_gate.weight"], st[p + "ff.shared_up.weight"] = n(f, d), n(f, d)
+        st[p + "ff.shared_down.weight"] = n(d, f)
+        st[p + "norm1.weight"] = torch.ones(d, device=dev)
+        st[p + "norm2.weight"] = torch.ones(d, device=dev)
+    model = MoeLlama(cfg, st, device=dev)
+    del st
+    B, L = 64, cfg.max_sequence_length
+    cache = model.build_kv_cache(B)
+    _fill_cache(cache, L - 1, B)
+    ids = torch.randint(0, v, (B, 1), device=dev)
+
+    def step():
+        _fill_len(cache, L - 1, B)
+        return model(ids, cache, L - 1, last_only=True)
+
+    t = graph_time(step, iters=5)
+    nl = cfg.num_hidden_layers
+    expert_b = nl * 3.0 * E * d * f * 2
+    by = expert_b + nl * (3.0 * d * f + 4.0 * d * d + E * d) * 2 + 2.0 * v * d + 2.0 * 2 * d * nl * B * L
+    flops = nl * 2.0 * 3 * (B * cfg.moe_experts_per_tok) * d * f
+    return {"batch": B, "context": L, "ms_per_step": round(t * 1e3, 4), "tokens_per_s": round(B / t, 1),
+            "step_bytes": int(by), "GBs": round(by / t / 1e9, 1), "frac_of_hbm_peak": round(by / t / 1e9 / HBM_PEAK_GBS, 4),
+            "expert_ffn_TFLOPs_if_all_time": round(flops / t / 1e12, 2),
+            "bound": "hbm (about 8 rows per expert: ~8 flop/byte)"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -159,6 +366,9 @@ def main():
     ap.add_argument("--prompt", type=int, default=1024)
     ap.add_argument("--batches", type=str, default="1,8,32,64")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extended", action="store_true",
+                    help="skip the per-kernel figures of the other configurations (attention microbench, "
+                         "prefill on MFMA, BitNet and MoE decode)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run three 1 GiB device-to-device copies (a kernel of known traffic to scale "
                          "FETCH_SIZE / WRITE_SIZE counters against)")
@@ -234,6 +444,13 @@ def main():
         "also": {f"batch{b}": r for b, r in results.items()},
         "roofline": roof,
     }
+    if not args.no_extended:
+        out["kernels"] = {"prefill_d12": bench_prefill(model, cfg, dev)}
+        del model
+        torch.cuda.empty_cache()
+        out["kernels"]["decode_attention_gqa_32q_8kv_128"] = bench_attention_microbench(dev)
+        out["kernels"]["bitnet_decode"] = bench_bitnet(dev)
+        out["kernels"]["moe_decode"] = bench_moe(dev)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

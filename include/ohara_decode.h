@@ -168,16 +168,19 @@ int ohara_sample_topk_topp(const void* logits, int logits_are_fp32, int ldl, int
  * 2-bit stream the kernels read (16 weights per dword; size through *bytes when dst is NULL).
  * ohara_act_quant_int8 and ohara_gemv_ternary_i8 are the two halves; ohara_bitlinear_bf16
  * fuses them (k <= 6144).  acc_out, when given, receives the raw int32 accumulators - the
- * quantity that must match a CPU int32 matmul bit for bit.  ldq must be a multiple of 16. */
+ * quantity that must match a CPU int32 matmul bit for bit.  ldq must be a multiple of 16,
+ * k and ldx multiples of 8.  pre_norm_w (may be NULL) is the weight of the block-level RMSNorm
+ * that precedes the projection (llama.py:199-200), applied in the same pass: x := bf16(
+ * RMSNorm(x; pre_norm_w, eps)) before the BitLinear's own norm. */
 int ohara_bitlinear_pack_ternary(const int8_t* t, int n, int k, int ldt, uint32_t* dst, int64_t* bytes, void* stream);
 int ohara_act_quant_int8(const uint16_t* x, int ldx, const uint16_t* norm_w, float eps, int rows, int k, int8_t* q,
                          int ldq, float* s, int32_t* sumq, void* stream);
 int ohara_gemv_ternary_i8(const int8_t* q, int ldq, const float* s, const int32_t* sumq, const uint32_t* wp, int n,
                           int k, float gamma, int rows, const uint16_t* resid, int ldr, uint16_t* out, int ldo,
                           int32_t* acc_out, int ldacc, void* stream);
-int ohara_bitlinear_bf16(const uint16_t* x, int ldx, const uint16_t* norm_w, float eps, const uint32_t* wp, int n, int k,
-                         float gamma, int rows, const uint16_t* resid, int ldr, uint16_t* out, int ldo, int32_t* acc_out,
-                         int ldacc, void* stream);
+int ohara_bitlinear_bf16(const uint16_t* x, int ldx, const uint16_t* pre_norm_w, const uint16_t* norm_w, float eps,
+                         const uint32_t* wp, int n, int k, float gamma, int rows, const uint16_t* resid, int ldr,
+                         uint16_t* out, int ldo, int32_t* acc_out, int ldacc, void* stream);
 
 /* out = bf16(bf16(silu(gate)) * up), elementwise over n values (ohara/modules/mlp.py:152). */
 int ohara_silu_mul_bf16(const uint16_t* gate, const uint16_t* up, uint16_t* out, int64_t n, void* stream);

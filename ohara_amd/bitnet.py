@@ -111,23 +111,22 @@ class BitLlama:
         ends = [cc._reserve(B, S, start) for cc in kv_cache]
         H, Hkv, D = c.num_attention_heads, self.kv_heads, self.head_dim
         rows = B * S
-        n_split = 1 if S > 1 else max(1, min(512 // max(1, B * Hkv), c.max_sequence_length // 64, 32))
+        n_split = 1 if S > 1 else max(1, min(1024 // max(1, B * Hkv), c.max_sequence_length // 128, 64))
         key = (B, n_split)
         ws = self._ws.get(key)
         if ws is None:
             ws = self._ws[key] = ops.attn_workspace(B, H, Hkv, D, n_split, self.device)
         h = ops.embed(x.to(self.device), self.token_emb)
         for L, cache in zip(self.layers, kv_cache):
-            n1 = ops.rmsnorm(h, L["norm1"], self.eps)
-            q = ops.bitlinear(n1, L["attn.query"][1], L["attn.query"][0], self.eps)
-            k = ops.bitlinear(n1, L["attn.key"][1], L["attn.key"][0], self.eps)
-            v = ops.bitlinear(n1, L["attn.value"][1], L["attn.value"][0], self.eps)
+            # the block norm (norm1 / norm2) is applied inside each projection's quantisation pass
+            q = ops.bitlinear(h, L["attn.query"][1], L["attn.query"][0], self.eps, pre_norm_w=L["norm1"])
+            k = ops.bitlinear(h, L["attn.key"][1], L["attn.key"][0], self.eps, pre_norm_w=L["norm1"])
+            v = ops.bitlinear(h, L["attn.value"][1], L["attn.value"][0], self.eps, pre_norm_w=L["norm1"])
             ops.rope_append(q, k, v, B, S, H, Hkv, D, self.cos, self.sin, start, cache.key, cache.value)
-            att = ops.attn_cached(q, cache.key, cache.value, H, Hkv, D, start, n_split, ws, seq_len=S)
+            att = ops.attn_auto(q, cache.key, cache.value, H, Hkv, D, start, n_split, ws, S)
             h = ops.bitlinear(att, L["attn.proj"][1], L["attn.proj"][0], self.eps, residual=h)
-            n2 = ops.rmsnorm(h, L["norm2"], self.eps)
-            g = ops.bitlinear(n2, L["ff.gate"][1], L["ff.gate"][0], self.eps)
-            u = ops.bitlinear(n2, L["ff.up"][1], L["ff.up"][0], self.eps)
+            g = ops.bitlinear(h, L["ff.gate"][1], L["ff.gate"][0], self.eps, pre_norm_w=L["norm2"])
+            u = ops.bitlinear(h, L["ff.up"][1], L["ff.up"][0], self.eps, pre_norm_w=L["norm2"])
             h = ops.bitlinear(ops.silu_mul(g, u), L["ff.down"][1], L["ff.down"][0], self.eps, residual=h)
         if last_only:
             h = h.view(B, S, -1)[:, -1].contiguous()

@@ -26,41 +26,81 @@ struct QuantOut {
   int sumq;     // sum of the quantised row
 };
 
-// One wave normalises and quantises one row held in registers.  xq: int8 destination (LDS or
-// global), row stride handled by the caller.  Returns (s, sum q) in every lane.
+// One wave normalises and quantises one row held in registers (16-byte loads: lane l owns the
+// 8-value pieces l, l + 64, ...).  pre_w (optional) is the weight of a block-level RMSNorm applied
+// first (ohara/models/llama.py:199-200 norm1 / norm2), nw the BitLinear's own norm weight.
+// xq: int8 destination (LDS or global).  Returns (s, sum q) in every lane.  K % 8 == 0.
 template <int EPL>
-__device__ __forceinline__ QuantOut wave_quant_row(const bf16_t* x, const bf16_t* nw, int K, float eps, int8_t* xq) {
+__device__ __forceinline__ QuantOut wave_quant_row(const bf16_t* x, const bf16_t* pre_w, const bf16_t* nw, int K,
+                                                   float eps, int8_t* xq) {
+  constexpr int NP = EPL / 8;  // pieces per lane
   const int lane = threadIdx.x & 63;
-  float v[EPL];
+  const int pieces = K >> 3;
+  float v[NP][8];
   float ss = 0.f;
 #pragma unroll
-  for (int i = 0; i < EPL; ++i) {
-    const int k = i * 64 + lane;
-    v[i] = k < K ? bf2f(x[k]) : 0.f;
-    ss += v[i] * v[i];
+  for (int i = 0; i < NP; ++i) {
+    const int p = i * 64 + lane;
+    const uint4 u = p < pieces ? ldg16(x + (size_t)p * 8) : make_uint4(0, 0, 0, 0);
+    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[i][2 * j] = lo_bf(w[j]);
+      v[i][2 * j + 1] = hi_bf(w[j]);
+      ss += v[i][2 * j] * v[i][2 * j] + v[i][2 * j + 1] * v[i][2 * j + 1];
+    }
+  }
+  if (pre_w) {
+    ss = wave_sum(ss);
+    const float rinv0 = 1.0f / sqrtf(ss / (float)K + eps);
+    ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = i * 64 + lane;
+      if (p < pieces) {
+        const uint4 u = ldg16(pre_w + (size_t)p * 8);
+        const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          v[i][2 * j] = rbf(rbf(v[i][2 * j] * rinv0) * lo_bf(w[j]));
+          v[i][2 * j + 1] = rbf(rbf(v[i][2 * j + 1] * rinv0) * hi_bf(w[j]));
+          ss += v[i][2 * j] * v[i][2 * j] + v[i][2 * j + 1] * v[i][2 * j + 1];
+        }
+      }
+    }
   }
   ss = wave_sum(ss);
   const float rinv = 1.0f / sqrtf(ss / (float)K + eps);
   float mx = 0.f;
 #pragma unroll
-  for (int i = 0; i < EPL; ++i) {
-    const int k = i * 64 + lane;
-    if (k < K) {
-      v[i] = rbf(rbf(v[i] * rinv) * bf2f(nw[k]));  // RMSNorm output in the model dtype
-      mx = fmaxf(mx, fabsf(v[i]));
+  for (int i = 0; i < NP; ++i) {
+    const int p = i * 64 + lane;
+    if (p < pieces) {
+      const uint4 u = ldg16(nw + (size_t)p * 8);
+      const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[i][2 * j] = rbf(rbf(v[i][2 * j] * rinv) * lo_bf(w[j]));  // RMSNorm output in the model dtype
+        v[i][2 * j + 1] = rbf(rbf(v[i][2 * j + 1] * rinv) * hi_bf(w[j]));
+        mx = fmaxf(mx, fmaxf(fabsf(v[i][2 * j]), fabsf(v[i][2 * j + 1])));
+      }
     }
   }
   mx = wave_max(mx);
   const float s = 127.0f / fmaxf(mx, 1e-5f);
   int sq = 0;
 #pragma unroll
-  for (int i = 0; i < EPL; ++i) {
-    const int k = i * 64 + lane;
-    if (k < K) {
-      const float r = fminf(fmaxf(rintf(v[i] * s), -128.f), 127.f);
-      const int qi = (int)r;
-      xq[k] = (int8_t)qi;
-      sq += qi;
+  for (int i = 0; i < NP; ++i) {
+    const int p = i * 64 + lane;
+    if (p < pieces) {
+      uint32_t pk[2] = {0u, 0u};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int qi = (int)fminf(fmaxf(rintf(v[i][j] * s), -128.f), 127.f);
+        sq += qi;
+        pk[j >> 2] |= ((uint32_t)qi & 0xffu) << (8 * (j & 3));
+      }
+      *reinterpret_cast<uint2*>(xq + (size_t)p * 8) = make_uint2(pk[0], pk[1]);
     }
   }
 #pragma unroll
@@ -73,7 +113,7 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const bf16_t* x, int ldx
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = blockIdx.x * 4 + wave;
   if (r >= rows) return;
-  const QuantOut o = wave_quant_row<BL_EPL>(x + (size_t)r * ldx, nw, K, eps, q + (size_t)r * ldq);
+  const QuantOut o = wave_quant_row<BL_EPL>(x + (size_t)r * ldx, nullptr, nw, K, eps, q + (size_t)r * ldq);
   if (lane == 0) {
     s_out[r] = o.s;
     sumq_out[r] = o.sumq;
@@ -86,6 +126,7 @@ struct BitArgs {
   const bf16_t* x;       // FUSED: (B, K) bf16 activations
   int ldx;
   const bf16_t* nw;      // FUSED: BitLinear's RMSNorm weight
+  const bf16_t* pre_w;   // FUSED, optional: weight of a block-level RMSNorm applied before it
   float eps;
   const int8_t* q;       // !FUSED: (B, ldq) int8
   int ldq;
@@ -114,12 +155,21 @@ __global__ __launch_bounds__(256) void bitlinear_kernel(BitArgs a) {
   int* s_sum = reinterpret_cast<int*>(s_s + BT * 16);
   int* red = s_sum + BT * 16;           // [3][BT][64][4]
 
+  // the first weights of this wave are requested before the activations are prepared
+  const int per = (KC + 3) >> 2;
+  const int c0 = wave * per, c1 = min(KC, c0 + per);
+  const uint4* wrow = a.wp + (size_t)strip * KC * 64 + lane;
+  constexpr int CH = 6;
+  uint4 wpre[CH];
+#pragma unroll
+  for (int c = 0; c < CH; ++c) wpre[c] = (c0 + c < c1) ? ldg16_nt(wrow + (size_t)(c0 + c) * 64) : make_uint4(0, 0, 0, 0);
+
   // ---- activations -> int8 rows in LDS ---------------------------------------------------
   for (int i = tid; i < BT * 16 * (ldq / 16); i += 256) reinterpret_cast<uint4*>(xq)[i] = make_uint4(0, 0, 0, 0);
   __syncthreads();
   if (FUSED) {
     for (int b = wave; b < a.B; b += 4) {
-      const QuantOut o = wave_quant_row<BL_EPL>(a.x + (size_t)b * a.ldx, a.nw, a.K, a.eps, xq + (size_t)b * ldq);
+      const QuantOut o = wave_quant_row<BL_EPL>(a.x + (size_t)b * a.ldx, a.pre_w, a.nw, a.K, a.eps, xq + (size_t)b * ldq);
       if (lane == 0) {
         s_s[b] = o.s;
         s_sum[b] = o.sumq;
@@ -139,17 +189,18 @@ __global__ __launch_bounds__(256) void bitlinear_kernel(BitArgs a) {
   __syncthreads();
 
   // ---- weight stream -----------------------------------------------------------------------
-  const int per = (KC + 3) >> 2;
-  const int c0 = wave * per, c1 = min(KC, c0 + per);
   i32x4 acc[BT];
 #pragma unroll
   for (int t = 0; t < BT; ++t) acc[t] = (i32x4){0, 0, 0, 0};
-  const uint4* wrow = a.wp + (size_t)strip * KC * 64 + lane;
-  constexpr int CH = 6;
   for (int cb = c0; cb < c1; cb += CH) {
     uint4 wv[CH];
+    if (cb == c0) {
 #pragma unroll
-    for (int c = 0; c < CH; ++c) wv[c] = (cb + c < c1) ? ldg16_nt(wrow + (size_t)(cb + c) * 64) : make_uint4(0, 0, 0, 0);
+      for (int c = 0; c < CH; ++c) wv[c] = wpre[c];
+    } else {
+#pragma unroll
+      for (int c = 0; c < CH; ++c) wv[c] = (cb + c < c1) ? ldg16_nt(wrow + (size_t)(cb + c) * 64) : make_uint4(0, 0, 0, 0);
+    }
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
       if (cb + c >= c1) continue;
@@ -328,6 +379,7 @@ int ohara_bitlinear_pack_ternary(const int8_t* t, int n, int k, int ldt, uint32_
 int ohara_act_quant_int8(const uint16_t* x, int ldx, const uint16_t* norm_w, float eps, int rows, int k, int8_t* q,
                          int ldq, float* s, int32_t* sumq, void* stream) {
   if (!x || !norm_w || !q || !s || !sumq || rows < 1 || k < 1 || ldx < k || ldq < k) return OHARA_EINVAL;
+  if ((k & 7) || (ldx & 7) || (ldq & 7)) return OHARA_EINVAL;  // 16-byte loads, 8-byte stores
   if (k > BL_EPL * 64) return OHARA_ESIZE;
   hipLaunchKernelGGL(act_quant_kernel, dim3((rows + 3) / 4), dim3(256), 0, (hipStream_t)stream, x, ldx, norm_w, rows, k,
                      eps, q, ldq, s, sumq);
@@ -347,15 +399,16 @@ int ohara_gemv_ternary_i8(const int8_t* q, int ldq, const float* s, const int32_
   return launch_bit<false>(a, (hipStream_t)stream);
 }
 
-int ohara_bitlinear_bf16(const uint16_t* x, int ldx, const uint16_t* norm_w, float eps, const uint32_t* wp, int n, int k,
-                         float gamma, int rows, const uint16_t* resid, int ldr, uint16_t* out, int ldo, int32_t* acc_out,
-                         int ldacc, void* stream) {
+int ohara_bitlinear_bf16(const uint16_t* x, int ldx, const uint16_t* pre_norm_w, const uint16_t* norm_w, float eps,
+                         const uint32_t* wp, int n, int k, float gamma, int rows, const uint16_t* resid, int ldr,
+                         uint16_t* out, int ldo, int32_t* acc_out, int ldacc, void* stream) {
   if (!x || !norm_w || !wp || !out || n < 1 || k < 1 || rows < 1) return OHARA_EINVAL;
   if (ldx < k || ldo < n || (resid && ldr < n) || (acc_out && ldacc < n)) return OHARA_EINVAL;
+  if ((k & 7) || (ldx & 7)) return OHARA_EINVAL;  // 16-byte activation loads
   if (k > BL_EPL * 64) return OHARA_ESIZE;
   BitArgs a{};
   a.wp = reinterpret_cast<const uint4*>(wp); a.gamma = gamma;
-  a.x = x; a.ldx = ldx; a.nw = norm_w; a.eps = eps;
+  a.x = x; a.ldx = ldx; a.nw = norm_w; a.pre_w = pre_norm_w; a.eps = eps;
   a.B = rows; a.N = n; a.K = k; a.out = out; a.ldo = ldo; a.resid = resid; a.ldr = ldr;
   a.acc_out = acc_out; a.ldacc = ldacc;
   return launch_bit<true>(a, (hipStream_t)stream);

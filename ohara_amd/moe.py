@@ -193,7 +193,7 @@ class MoeLlama:
             kv_cache = self.build_kv_cache(B)
         ends = [cc._reserve(B, S, start) for cc in kv_cache]
         H, Hkv, D = c.num_attention_heads, self.kv_heads, self.head_dim
-        n_split = 1 if S > 1 else max(1, min(512 // max(1, B * Hkv), c.max_sequence_length // 64, 32))
+        n_split = 1 if S > 1 else max(1, min(1024 // max(1, B * Hkv), c.max_sequence_length // 128, 64))
         ws = self._ws.get((B, n_split))
         if ws is None:
             ws = self._ws[(B, n_split)] = ops.attn_workspace(B, H, Hkv, D, n_split, self.device)
@@ -201,7 +201,7 @@ class MoeLlama:
         for L, cache in zip(self.layers, kv_cache):
             q = ops.qkv_rope_append(h, L["wqkv"], L["norm1"], self.eps, H, Hkv, D, self.cos, self.sin, start,
                                     cache.key, cache.value, seq_len=S)
-            att = ops.attn_cached(q, cache.key, cache.value, H, Hkv, D, start, n_split, ws, seq_len=S)
+            att = ops.attn_auto(q, cache.key, cache.value, H, Hkv, D, start, n_split, ws, S)
             h = ops.gemm_skinny(att, L["wo"], residual=h)
             if "moe" in L:
                 h = L["moe"].forward_rows(ops.rmsnorm(h, L["norm2"], self.eps), residual=h)

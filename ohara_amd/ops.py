@@ -202,6 +202,13 @@ def attn_prefill(q, kcache, vcache, h, h_kv, dh, pos, seq_len, out=None):
     return out
 
 
+def attn_auto(q, kcache, vcache, h, h_kv, dh, pos, n_split, workspace, seq_len, out=None):
+    """The MFMA prefill kernel for calls with many positions per sequence, else the decode kernel."""
+    if seq_len >= 16 and dh in (64, 128):
+        return attn_prefill(q, kcache, vcache, h, h_kv, dh, pos, seq_len, out)
+    return attn_cached(q, kcache, vcache, h, h_kv, dh, pos, n_split if seq_len == 1 else 1, workspace, out, None, seq_len)
+
+
 def attn_decode(q, kcache, vcache, h, h_kv, dh, length, n_split, workspace, out=None, pos_dev=None):
     """Decode case: one query per sequence seeing `length` cached positions."""
     return attn_cached(q, kcache, vcache, h, h_kv, dh, length - 1, n_split, workspace, out, pos_dev, 1)
@@ -291,8 +298,9 @@ def gemv_ternary(q, s, sumq, w: PackedTernary, residual=None, out=None, want_acc
     return (out, acc) if want_acc else out
 
 
-def bitlinear(x, norm_w, w: PackedTernary, eps=1e-5, residual=None, out=None, want_acc=False):
-    """Fused BitLinear.forward on rows of x (rows, K) bf16."""
+def bitlinear(x, norm_w, w: PackedTernary, eps=1e-5, residual=None, out=None, want_acc=False, pre_norm_w=None):
+    """Fused BitLinear.forward on rows of x (rows, K) bf16; ``pre_norm_w`` applies a block-level
+    RMSNorm to x first, in the same pass."""
     _need(x, BF16, "x")
     rows, k = x.shape
     if k != w.k:
@@ -300,7 +308,7 @@ def bitlinear(x, norm_w, w: PackedTernary, eps=1e-5, residual=None, out=None, wa
     if out is None:
         out = torch.empty(rows, w.n, dtype=BF16, device=x.device)
     acc = torch.empty(rows, w.n, dtype=torch.int32, device=x.device) if want_acc else None
-    check(lib().ohara_bitlinear_bf16(_ptr(x), x.stride(0), _ptr(norm_w), eps, _ptr(w.data), w.n, w.k, w.gamma, rows,
+    check(lib().ohara_bitlinear_bf16(_ptr(x), x.stride(0), _ptr(pre_norm_w), _ptr(norm_w), eps, _ptr(w.data), w.n, w.k, w.gamma, rows,
                                      _ptr(residual), 0 if residual is None else residual.stride(0), _ptr(out),
                                      out.stride(0), _ptr(acc), w.n, _stream()), "bitlinear")
     return (out, acc) if want_acc else out

@@ -43,7 +43,7 @@ def test_act_quant_matches_oracle(cuda):
     from ohara_amd import ops
 
     g = torch.Generator().manual_seed(0)
-    for rows, K in ((5, 2048), (3, 5632), (4, 100)):
+    for rows, K in ((5, 2048), (3, 5632), (4, 104)):
         x = (torch.randn(rows, K, generator=g) * 2).to(BF)
         nw = (1 + 0.2 * torch.randn(K, generator=g)).to(BF)
         q_ref, s_ref = BL.activation_quant(R.rms_norm(x, nw))
@@ -82,6 +82,30 @@ def test_fused_bitlinear(cuda, rows, N, K):
     # and against the reference's float fake-quant formulation (bitnet.py:29-59)
     fq = BL.fake_quant_forward(x.float(), nw.float(), wfloat)
     assert (out.cpu().float() - fq).abs().mean().item() <= 1e-2 * scale
+
+
+def test_fused_bitlinear_with_block_norm(cuda):
+    """pre_norm_w folds the block-level RMSNorm (llama.py:199-200) into the quantisation pass: same
+    result as normalising first with the stand-alone kernel."""
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(9)
+    rows, N, K = 5, 2048, 2048
+    x = (torch.randn(rows, K, generator=g) * 3).to(BF).to(cuda)
+    pre = (1 + 0.2 * torch.randn(K, generator=g)).to(BF).to(cuda)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(BF).to(cuda)
+    t = torch.randint(-1, 2, (N, K), generator=g, dtype=torch.int8)
+    w = ops.pack_ternary(t.to(cuda), 0.04)
+    fused, acc_f = ops.bitlinear(x, nw, w, want_acc=True, pre_norm_w=pre)
+    two, acc_t = ops.bitlinear(ops.rmsnorm(x, pre), nw, w, want_acc=True)
+    # the two norms' fp32 reduction orders can flip single bf16 roundings: nearly all accumulators
+    # identical, the rest off by a few units
+    d = (acc_f - acc_t).abs()
+    assert float((d > 0).float().mean()) < 0.2 and int(d.max()) <= 4 * 127
+    want = BL.bitlinear_forward(R.rms_norm(x.cpu(), pre.cpu()), nw.cpu(), t, 0.04)
+    scale = want.float().abs().max().item()
+    e = (fused.cpu().float() - want.float()).abs()
+    assert e.max().item() <= 3e-2 * scale and e.mean().item() <= 3e-3 * scale
 
 
 def test_ternarize_matches_oracle(cuda):
