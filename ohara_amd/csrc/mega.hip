@@ -43,6 +43,7 @@ struct MegaArgs {
   uint16_t* const* kcache_dev;  // device arrays [n_layers]
   uint16_t* const* vcache_dev;
   int B, valid_vocab, hist_cap, select;
+  int ns;                       // context chunks per (sequence, kv head) in this launch, <= OHARA_MEGA_NS
   int blk_x, blk_a;             // bytes per strip block of the x/q and act mailboxes
   int64_t* ids;
   char* xm;        // (2*NL + 1) x-mailboxes of xm_stride bytes: residual stream after each half layer
@@ -236,40 +237,109 @@ __device__ void stage_act(bf16_t* xs, int ldxs, const char* src, int blk, int B,
 }
 
 // Merge of the attention partials of all chunks, in chunk order (llama.py:116-123 output,
-// rounded to bf16 as SDPA's result is) -> xs[b][h*Dh + d].  A thread owns four adjacent
-// columns; the (max, sum) pairs and the accumulators of all NS chunks are loaded before any
-// is used.
-template <int NS>
-__device__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh) {
+// rounded to bf16 as SDPA's result is) -> xs[b][h*Dh + d].  The (max, sum) pairs of every
+// (sequence, head, chunk) are fetched in one round into LDS and turned into chunk weights
+// exp(m_s - M) / L there; a thread then owns four adjacent columns and issues the accumulator
+// loads of all chunks before using any.  `mw`: B*H*ns floats, `ml`: B*H*ns floats of LDS.
+__device__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh, int ns, float* mw,
+                                 float* ml) {
+  constexpr int NSM = OHARA_MEGA_NS;
   const int HD = H * Dh, PS = Dh + 32;
+  const int nbh = B * H;
+  // the accumulator loads of a thread's first columns go out first: they do not depend on the
+  // chunk weights, which are formed (two LDS rounds) while they are in flight
+  uint4 av[NSM];
+  {
+    const int e = threadIdx.x * 4;
+    const int b = e / HD, hd = e - b * HD;
+    const float* base = pm + (size_t)(b * H + hd / Dh) * NSM * PS + (hd % Dh);
+#pragma unroll
+    for (int sp = 0; sp < NSM; ++sp)
+      av[sp] = (e < B * HD && sp < ns) ? ldg16(base + (size_t)sp * PS) : make_uint4(0, 0, 0, 0);
+  }
+  // 16 lanes per (sequence, head): lane sp holds chunk sp's (max, sum); max and weighted sum by
+  // shuffles inside the 16-lane group
+  for (int i0 = 0; i0 < nbh * NSM; i0 += blockDim.x) {
+    const int i = i0 + threadIdx.x;
+    const int bh = i / NSM, sp = i % NSM;
+    const bool in = bh < nbh && sp < ns;
+    float ms = -INFINITY, ls = 0.f;
+    if (in) {
+      const uint2 v = *reinterpret_cast<const uint2*>(pm + ((size_t)bh * NSM + sp) * PS + Dh);
+      ms = __uint_as_float(v.x);
+      ls = __uint_as_float(v.y);
+    }
+    float M = ms;
+#pragma unroll
+    for (int o = NSM / 2; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, WAVE));
+    const float w = (ms == -INFINITY) ? 0.f : __expf(ms - M);
+    float Ls = ls * w;
+#pragma unroll
+    for (int o = NSM / 2; o > 0; o >>= 1) Ls += __shfl_xor(Ls, o, WAVE);
+    if (in) mw[bh * ns + sp] = w;
+    if (bh < nbh && sp == 0) ml[bh] = Ls;
+  }
+  __syncthreads();
   for (int e = threadIdx.x * 4; e < B * HD; e += blockDim.x * 4) {
     const int b = e / HD, hd = e - b * HD;
     const int h = hd / Dh, d = hd - h * Dh;
-    const float* base = pm + (size_t)(b * H + h) * NS * PS;
-    uint2 mlv[NS];
-    uint4 av[NS];
+    const int bh = b * H + h;
+    if (e != (int)threadIdx.x * 4) {
+      const float* base = pm + (size_t)bh * NSM * PS + d;
 #pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      mlv[s] = *reinterpret_cast<const uint2*>(base + (size_t)s * PS + Dh);
-      av[s] = ldg16(base + (size_t)s * PS + d);
+      for (int sp = 0; sp < NSM; ++sp) av[sp] = sp < ns ? ldg16(base + (size_t)sp * PS) : make_uint4(0, 0, 0, 0);
     }
-    float M = -INFINITY;
+    float o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int s = 0; s < NS; ++s) M = fmaxf(M, __uint_as_float(mlv[s].x));
-    float Ls = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      const float ms = __uint_as_float(mlv[s].x);
-      const float w = (ms == -INFINITY) ? 0.f : __expf(ms - M);
-      Ls += __uint_as_float(mlv[s].y) * w;
-      o[0] += __uint_as_float(av[s].x) * w;
-      o[1] += __uint_as_float(av[s].y) * w;
-      o[2] += __uint_as_float(av[s].z) * w;
-      o[3] += __uint_as_float(av[s].w) * w;
+    for (int sp = 0; sp < NSM; ++sp) {
+      if (sp < ns) {
+        const float w = mw[bh * ns + sp];
+        o[0] += __uint_as_float(av[sp].x) * w;
+        o[1] += __uint_as_float(av[sp].y) * w;
+        o[2] += __uint_as_float(av[sp].z) * w;
+        o[3] += __uint_as_float(av[sp].w) * w;
+      }
     }
+    const float Ls = ml[bh];
     *reinterpret_cast<uint2*>(xs + (size_t)b * ldxs + hd) =
         make_uint2(pack_bf(o[0] / Ls, o[1] / Ls), pack_bf(o[2] / Ls, o[3] / Ls));
   }
+}
+
+// One pass for the small case (all OHARA_MEGA_NS chunks in use, one group of four columns per
+// thread): every thread fetches the (max, sum) pairs itself, so there is a single round of loads
+// and no workgroup barrier.
+__device__ void stage_attn_merge_small(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh) {
+  constexpr int NS = OHARA_MEGA_NS;
+  const int HD = H * Dh, PS = Dh + 32;
+  const int e = threadIdx.x * 4;
+  if (e >= B * HD) return;
+  const int b = e / HD, hd = e - b * HD;
+  const int h = hd / Dh, d = hd - h * Dh;
+  const float* base = pm + (size_t)(b * H + h) * NS * PS;
+  uint2 mlv[NS];
+  uint4 av[NS];
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    mlv[s] = *reinterpret_cast<const uint2*>(base + (size_t)s * PS + Dh);
+    av[s] = ldg16(base + (size_t)s * PS + d);
+  }
+  float M = -INFINITY;
+#pragma unroll
+  for (int s = 0; s < NS; ++s) M = fmaxf(M, __uint_as_float(mlv[s].x));
+  float Ls = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    const float ms = __uint_as_float(mlv[s].x);
+    const float w = (ms == -INFINITY) ? 0.f : __expf(ms - M);
+    Ls += __uint_as_float(mlv[s].y) * w;
+    o[0] += __uint_as_float(av[s].x) * w;
+    o[1] += __uint_as_float(av[s].y) * w;
+    o[2] += __uint_as_float(av[s].z) * w;
+    o[3] += __uint_as_float(av[s].w) * w;
+  }
+  *reinterpret_cast<uint2*>(xs + (size_t)b * ldxs + hd) =
+      make_uint2(pack_bf(o[0] / Ls, o[1] / Ls), pack_bf(o[2] / Ls, o[3] / Ls));
 }
 
 // ---------------------------------------------------------------------------------------
@@ -514,24 +584,23 @@ __device__ __forceinline__ bool attn_first_tile_prefetchable(int t0, int t1, int
 }
 
 template <int D>
-__device__ __forceinline__ void attn_prefetch(int B, int Hkv, int Tmax, const bf16_t* kc, const bf16_t* vc, int L,
-                                              AttnPre<D>& pre) {
+__device__ __forceinline__ void attn_prefetch(int B, int Hkv, int Tmax, int ns, const bf16_t* kc, const bf16_t* vc,
+                                              int L, AttnPre<D>& pre) {
   const int wave = threadIdx.x >> 6;
   const size_t row = (size_t)Hkv * D;
   int b, kvh, split, t0, t1;
-  attn_item_range(blockIdx.x, OHARA_MEGA_NS, Hkv, L, b, kvh, split, t0, t1);
-  const bool has = (int)blockIdx.x < B * Hkv * OHARA_MEGA_NS && attn_first_tile_prefetchable<D>(t0, t1, L);
+  attn_item_range(blockIdx.x, ns, Hkv, L, b, kvh, split, t0, t1);
+  const bool has = (int)blockIdx.x < B * Hkv * ns && attn_first_tile_prefetchable<D>(t0, t1, L);
   const bf16_t* kb = kc + (size_t)b * Tmax * row + (size_t)kvh * D;
   const bf16_t* vb = vc + (size_t)b * Tmax * row + (size_t)kvh * D;
   attn_tile_load<D>(kb, vb, row, t0 + wave * 16, has ? t1 : 0, -1, pre.k, pre.v);
 }
 
 template <int D, int G>
-__device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int blk_x, const AttnPre<D>& pre,
+__device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int blk_x, int ns, const AttnPre<D>& pre,
                                            const char* qm, float* pm, const bf16_t* kc, const bf16_t* vc, int L,
                                            float* lds) {
   constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
-  constexpr int ns = OHARA_MEGA_NS;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int p = lane & 15;
   const int dq = lane >> 4;
@@ -564,18 +633,22 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
 #pragma unroll
         for (int c = 0; c < NC; ++c)
           qv[hh][c] = ldg16(xm_addr(qm, blk_x, b, (kvh * G + hh) * D + (4 * c + dq) * 8));
+      // the tile after the current one is in flight while the current one is consumed
       const bool use_pre = first && attn_first_tile_prefetchable<D>(t0, t1, L);
-      for (int tb = t0 + wave * 16; tb < t1; tb += 64) {
+      uint4 kv[NC], vv[NV], kn[NC], vn[NV];
+      int tb = t0 + wave * 16;
+      if (use_pre) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) kv[c] = pre.k[c];
+#pragma unroll
+        for (int c = 0; c < NV; ++c) vv[c] = pre.v[c];
+      } else {
+        attn_tile_load<D>(kb, vb, row, tb, t1, L - 1, kv, vv);
+      }
+      for (; tb < t1; tb += 64) {
         const bool valid = tb + p < t1;
-        uint4 kv[NC], vv[NV];
-        if (use_pre && tb == t0 + wave * 16) {
-#pragma unroll
-          for (int c = 0; c < NC; ++c) kv[c] = pre.k[c];
-#pragma unroll
-          for (int c = 0; c < NV; ++c) vv[c] = pre.v[c];
-        } else {
-          attn_tile_load<D>(kb, vb, row, tb, t1, L - 1, kv, vv);
-        }
+        const bool more = tb + 64 < t1;
+        if (more) attn_tile_load<D>(kb, vb, row, tb + 64, t1, L - 1, kn, vn);
 #pragma unroll
         for (int hh = 0; hh < G; ++hh) {
           float s = 0.f;
@@ -607,6 +680,12 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
               acc[hh][2 * i + 1] += pw * hi_bf(w4[i]);
             }
           }
+        }
+        if (more) {
+#pragma unroll
+          for (int c = 0; c < NC; ++c) kv[c] = kn[c];
+#pragma unroll
+          for (int c = 0; c < NV; ++c) vv[c] = vn[c];
         }
       }
     }
@@ -643,7 +722,7 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
         o0 += s_acc[(w * G + hh) * D + d] * sc;
         o1 += s_acc[(w * G + hh) * D + d + 1] * sc;
       }
-      float* dst = pm + ((size_t)(b * H + h) * ns + split) * PS;
+      float* dst = pm + ((size_t)(b * H + h) * OHARA_MEGA_NS + split) * PS;
       st_coh8(dst + d, make_uint2(__float_as_uint(o0), __float_as_uint(o1)));
       if (d == 0) st_coh8(dst + D, make_uint2(__float_as_uint(M), __float_as_uint(Ls)));
     }
@@ -666,7 +745,9 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   float* att = red + 1024;                                                                      // (8 + 4*D)*G floats
   // per-layer pointers (6 weights/norms + K and V cache), copied once to LDS so that no phase
   // starts with a chain of dependent global loads
-  unsigned long long* ptab = reinterpret_cast<unsigned long long*>(att + (8 + 4 * D) * G);
+  float* mrg_w = att + (8 + 4 * D) * G;       // B*H*ns chunk weights
+  float* mrg_l = mrg_w + ((B * H * a.ns + 1) & ~1);  // B*H*ns chunk sums
+  unsigned long long* ptab = reinterpret_cast<unsigned long long*>(mrg_l + ((B * H * a.ns + 1) & ~1));
   for (int i = threadIdx.x; i < m.n_layers * 8; i += blockDim.x) {
     const int l = i >> 3, j = i & 7;
     unsigned long long v;
@@ -723,18 +804,21 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     gemm_phase<4, 6, E_ROPE>(qkv, pre, xs, ldxs, B, red, best_v, best_i, pf);
     pf.stamp();
     gs.arrive(pf);
-    attn_prefetch<D>(B, Hkv, m.t_max, kc, vc, L, apre);
+    attn_prefetch<D>(B, Hkv, m.t_max, a.ns, kc, vc, L, apre);
     gs.wait(pf);
     pf.stamp();
     // P2: attention partials
-    attn_phase<D, G>(B, H, Hkv, m.t_max, a.blk_x, apre, q_l, p_l, kc, vc, L, att);
+    attn_phase<D, G>(B, H, Hkv, m.t_max, a.blk_x, a.ns, apre, q_l, p_l, kc, vc, L, att);
     gs.arrive(pf);
     prj.wp = lds_ptr<const uint4>(pl, 1); prj.out = x_mid; prj.resid = x_in; prj.resid_embed = l == 0;
     gemm_prefetch<4, 6, E_RESID>(prj, pre, B);
     gs.wait(pf);
     pf.stamp();
     // P3: merge + output projection + residual
-    if ((int)blockIdx.x < prj.nstrips) stage_attn_merge<OHARA_MEGA_NS>(xs, ldxs, p_l, B, H, D);
+    if ((int)blockIdx.x < prj.nstrips) {
+      if (a.ns == OHARA_MEGA_NS && B * H * D <= 4 * (int)blockDim.x) stage_attn_merge_small(xs, ldxs, p_l, B, H, D);
+      else stage_attn_merge(xs, ldxs, p_l, B, H, D, a.ns, mrg_w, mrg_l);
+    }
     __syncthreads();
     pf.stamp();
     gemm_phase<4, 6, E_RESID>(prj, pre, xs, ldxs, B, red, best_v, best_i, pf);
@@ -958,7 +1042,12 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   const int kmax = m->d_model > m->d_ff ? m->d_model : m->d_ff;
   const int kmax2 = kmax > m->n_heads * D ? kmax : m->n_heads * D;
   const size_t xs_bytes = ((size_t)s->batch * (kmax2 + 8) * 2 + 255) & ~(size_t)255;
-  const size_t smem = xs_bytes + 4096 + (size_t)(8 + 4 * D) * G * sizeof(float) + (size_t)m->n_layers * 64;
+  // one attention item per workgroup where the batch allows it
+  int ns = n_workgroups / (s->batch * m->n_kv_heads);
+  ns = ns < 1 ? 1 : (ns > OHARA_MEGA_NS ? OHARA_MEGA_NS : ns);
+  a.ns = ns;
+  const size_t mrg = (size_t)2 * ((s->batch * m->n_heads * ns + 1) & ~1) * sizeof(float);
+  const size_t smem = xs_bytes + 4096 + (size_t)(8 + 4 * D) * G * sizeof(float) + mrg + (size_t)m->n_layers * 64;
   if (smem > 160 * 1024) return OHARA_ESIZE;
   dim3 grid(n_workgroups), block(256);
 #define OHARA_MEGA(DD, GG)                                                                                  \

@@ -108,7 +108,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const bf16_t* logits, in
 // pos_of[n*k + j] = sorted position.  One workgroup; N*k <= 65536, E <= 1024.
 __global__ __launch_bounds__(1024) void moe_sort_kernel(const int32_t* idx, int NK, int E, int32_t* offs, int32_t* pair_of,
                                                         int32_t* pos_of) {
-  __shared__ int cnt[1025];
+  __shared__ int cnt[1025];   // histogram, then the next free sorted position of every expert
+  __shared__ __align__(16) int sidx[1024];  // expert ids of the current block of 1024 pairs
   const int tid = threadIdx.x;
   for (int e = tid; e <= E; e += 1024) cnt[e] = 0;
   __syncthreads();
@@ -122,20 +123,33 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int32_t* idx, int 
       offs[e] = run;
       run += c;
     }
-    cnt[E] = run;
     offs[E] = run;
   }
   __syncthreads();
-  // stable placement: expert by expert, pairs in increasing p (thread e walks all pairs; NK is small)
-  for (int e = tid; e < E; e += 1024) {
-    int o = cnt[e];
-    const int end = cnt[e + 1];
-    for (int p = 0; p < NK && o < end; ++p)
-      if (idx[p] == e) {
-        pair_of[o] = p;
-        pos_of[p] = o;
-        ++o;
-      }
+  // stable placement, 1024 pairs at a time: a pair's position is its expert's next free slot
+  // plus the number of earlier pairs of the block with the same expert (LDS broadcast reads)
+  for (int p0 = 0; p0 < NK; p0 += 1024) {
+    const int p = p0 + tid;
+    const int e = p < NK ? idx[p] : -1;
+    sidx[tid] = e;
+    __syncthreads();
+    const int n4 = (min(1024, NK - p0) + 3) >> 2;  // entries past the end hold -1 and never match
+    int rank = 0;
+    const int4* s4 = reinterpret_cast<const int4*>(sidx);
+#pragma unroll 4
+    for (int t4 = 0; t4 < n4; ++t4) {
+      const int4 v = s4[t4];
+      const int t = 4 * t4;
+      rank += (t < tid && v.x == e) + (t + 1 < tid && v.y == e) + (t + 2 < tid && v.z == e) + (t + 3 < tid && v.w == e);
+    }
+    if (e >= 0) {
+      const int o = cnt[e] + rank;
+      pair_of[o] = p;
+      pos_of[p] = o;
+    }
+    __syncthreads();
+    if (e >= 0) atomicAdd(&cnt[e], 1);
+    __syncthreads();
   }
 }
 
