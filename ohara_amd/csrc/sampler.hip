@@ -14,16 +14,16 @@
 // function of (logits, parameters, u).
 //
 // A thread owns EPT consecutive vocabulary entries in registers; the 1024 threads cover up
-// to 1024*EPT ids.  The sorted prefix is built 2048 candidates at a time (radix select on
+// to 1024*EPT ids.  The sorted prefix is built 1024 candidates at a time (radix select on
 // the probability bits, ordered compaction, bitonic sort in LDS) and scanned sequentially
-// in fp32, the order torch.cumsum uses; a peaked distribution or any top-k <= 2048 needs a
+// in fp32, the order torch.cumsum uses; a peaked distribution or any top-k <= 1024 needs a
 // single round.
 #include "common.h"
 
 namespace {
 
 constexpr int NT = 1024;
-constexpr int CAP = 2048;  // candidates sorted per round
+constexpr int CAP = 1024;  // candidates sorted per round
 
 struct SampleArgs {
   const void* logits;
@@ -93,18 +93,27 @@ __device__ __forceinline__ int block_sum_i(int v, Smem& s) {
 }
 
 // Exclusive prefix sum of one int per thread, in thread order.  Returns the total.
+// Wave-level shuffle scan, then the 16 wave totals.
 __device__ __forceinline__ int block_excl_scan_i(int v, int& excl, Smem& s) {
-  __syncthreads();
-  s.iscan[threadIdx.x] = v;
-  __syncthreads();
-  for (int o = 1; o < NT; o <<= 1) {
-    const int t = threadIdx.x >= o ? s.iscan[threadIdx.x - o] : 0;
-    __syncthreads();
-    s.iscan[threadIdx.x] += t;
-    __syncthreads();
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  int incl = v;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int t = __shfl_up(incl, o, WAVE);
+    if (lane >= o) incl += t;
   }
-  excl = s.iscan[threadIdx.x] - v;
-  return s.iscan[NT - 1];
+  __syncthreads();
+  if (lane == 63) s.wredi[w] = incl;
+  __syncthreads();
+  int before = 0, total = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int t = s.wredi[i];
+    if (i < w) before += t;
+    total += t;
+  }
+  excl = before + incl - v;
+  return total;
 }
 
 // The `want`-th largest key (1-based) among the keys for which live(i) holds; returns the
@@ -125,14 +134,29 @@ __device__ uint32_t radix_select(int want, int& n_greater, Smem& s, LiveFn live,
       }
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-      int acc = above, d = 255;
-      for (; d > 0; --d) {
-        if (acc + s.hist[d] >= want) break;
-        acc += s.hist[d];
+    // the digit whose bin holds the want-th largest: suffix sums of the 256 bins by four waves
+    {
+      const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+      int h = 0, incl = 0;
+      if (threadIdx.x < 256) {
+        h = s.hist[threadIdx.x];
+        incl = h;  // inclusive sum over bins >= mine within the wave
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+          const int t = __shfl_down(incl, o, WAVE);
+          if (lane + o < 64) incl += t;
+        }
+        if (lane == 0) s.wredi[w] = incl;
       }
-      s.misc[0] = d;
-      s.misc[1] = acc;
+      __syncthreads();
+      if (threadIdx.x < 256) {
+        for (int i = w + 1; i < 4; ++i) incl += s.wredi[i];
+        const int gt = above + incl - h;  // elements in bins above mine (and in earlier digits' higher bins)
+        if (gt < want && (threadIdx.x == 0 || want <= gt + h)) {
+          s.misc[0] = threadIdx.x;
+          s.misc[1] = gt;
+        }
+      }
     }
     __syncthreads();
     const int d = s.misc[0];
@@ -142,6 +166,26 @@ __device__ uint32_t radix_select(int want, int& n_greater, Smem& s, LiveFn live,
   }
   n_greater = above;
   return prefix;
+}
+
+// The same selection for want <= 1024, without a histogram pass over every element (tens of
+// thousands of LDS atomics on the handful of bins that share the leading key bits): the want-th
+// largest of the 1024 per-thread maxima is a lower bound of the answer (at least `want` elements
+// are >= it), so only the elements at or above that bound - usually a few times `want` - take part
+// in the exact radix select.
+template <int EPT, typename LiveFn, typename KeyFn>
+__device__ uint32_t select_small(int want, int& n_greater, Smem& s, LiveFn live, KeyFn key) {
+  uint32_t tmax = 0;  // keys of live elements are > 0
+#pragma unroll
+  for (int i = 0; i < EPT; ++i)
+    if (live(i)) tmax = max(tmax, key(i));
+  const int have = block_sum_i(tmax > 0 ? 1 : 0, s);
+  uint32_t bound = 0;
+  if (have >= want) {
+    int dummy;
+    bound = radix_select<1>(want, dummy, s, [&](int) { return tmax > 0; }, [&](int) { return tmax; });
+  }
+  return radix_select<EPT>(want, n_greater, s, [&](int i) { return live(i) && key(i) >= bound; }, key);
 }
 
 template <typename T>
@@ -172,8 +216,9 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
   if (a.top_k > 0) {
     const int k = min(a.top_k, V);
     int ngt;
-    const uint32_t tk = radix_select<EPT>(
-        k, ngt, s, [&](int i) { return base + i < V; }, [&](int i) { return fkey(x[i]); });
+    auto in_vocab = [&](int i) { return base + i < V; };
+    auto xkey = [&](int i) { return fkey(x[i]); };  // > 0 for every float but -NaN
+    const uint32_t tk = k <= 1024 ? select_small<EPT>(k, ngt, s, in_vocab, xkey) : radix_select<EPT>(k, ngt, s, in_vocab, xkey);
 #pragma unroll
     for (int i = 0; i < EPT; ++i)
       if (fkey(x[i]) < tk) x[i] = -INFINITY;
@@ -270,7 +315,7 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
         auto key = [&](int i) { return __float_as_uint(x[i]); };  // p > 0: bits are monotone
         int ngt = 0;
         uint32_t tk = 0;
-        if (take < remaining) tk = radix_select<EPT>(take, ngt, s, live, key);
+        if (take < remaining) tk = select_small<EPT>(take, ngt, s, live, key);
         // ordered compaction: all keys > tk, then ties at tk in id order until `take`
         int c_gt = 0, c_eq = 0;
 #pragma unroll
@@ -301,15 +346,17 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
             }
           }
         __syncthreads();
-        for (int i = take + tid; i < CAP; i += NT) {
+        int n2 = 64;  // sort length: the power of two that holds this round's candidates
+        while (n2 < take) n2 <<= 1;
+        for (int i = take + tid; i < n2; i += NT) {
           s.skey[i] = 0;  // padding sorts last
           s.sid[i] = 0x7fffffff;
         }
         __syncthreads();
         // bitonic sort, descending by key, ascending by id among equal keys
-        for (int k2 = 2; k2 <= CAP; k2 <<= 1) {
+        for (int k2 = 2; k2 <= n2; k2 <<= 1) {
           for (int j = k2 >> 1; j > 0; j >>= 1) {
-            for (int t = tid; t < CAP; t += NT) {
+            for (int t = tid; t < n2; t += NT) {
               const int ixj = t ^ j;
               if (ixj > t) {
                 const uint32_t ka = s.skey[t], kb = s.skey[ixj];
@@ -342,6 +389,24 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
             }
             S = kept;
             s.fmisc[1] = S;
+            if (cum == 0.f && (stop || remaining == take)) {
+              // the whole kept set sits in this sorted block: draw from it now, no second pass
+              const float target = u * S;
+              float r2 = 0.f;
+              int last = -1;
+              for (int j = 0; j < take; ++j) {
+                const float p = __uint_as_float(s.skey[j]);
+                if (r2 > a.top_p) break;
+                r2 += p;
+                last = s.sid[j];
+                if (r2 > target) {
+                  tok = s.sid[j];
+                  break;
+                }
+              }
+              if (tok < 0) tok = max(last, 0);  // rounding pushed the target past the end: last kept id
+              stop = 1;
+            }
           } else {
             const float target = u * S;
             int last = -1;
@@ -371,7 +436,7 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
         cum = s.fmisc[0];
         S = s.fmisc[1];
         done = s.misc[2] != 0;
-        if (pass == 1 && s.misc[3] >= 0) token = s.misc[3];
+        if (s.misc[3] >= 0) token = s.misc[3];
         remaining -= take;
         __syncthreads();
       }
