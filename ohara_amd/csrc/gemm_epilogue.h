@@ -22,6 +22,7 @@ struct GemmArgs {
   // rotary + append
   int H, Hkv, Dh, Tmax, pos;
   int S, row0;  // rows are (sequence, position) pairs: row = seq * S + s, position = pos + s
+  int ny, nstrips;  // skinny kernel: 16-row chunks per strip (workgroups of a strip share an XCD) and strips
   const int32_t* pos_dev;
   const bf16_t* cos;
   const bf16_t* sin;

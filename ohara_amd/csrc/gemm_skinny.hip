@@ -46,7 +46,12 @@ __device__ __forceinline__ uint4 norm8(uint4 xv, uint4 wv, float rinv) {
 template <int BT, bool NORM, int EPI>
 __global__ __launch_bounds__(256) void skinny_kernel(GemmArgs a) {
   constexpr int CH = BT <= 2 ? 6 : 4;  // k-steps whose loads are issued back to back
-  const int strip = blockIdx.x;
+  // workgroup id -> (strip, chunk of 16*BT rows).  Ids go round-robin over the 8 XCDs; the chunks of
+  // one strip get ids 8 apart, so they run on the same XCD and share its L2 copy of the weights.
+  const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  const int strip = (local / a.ny) * 8 + xcd;
+  const int rbase = (local % a.ny) * 16 * BT;
+  if (strip >= a.nstrips) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 15, g = lane >> 4;
   const int KS = (a.K + 31) >> 5;
@@ -66,7 +71,7 @@ __global__ __launch_bounds__(256) void skinny_kernel(GemmArgs a) {
       const int k0 = 32 * j + 8 * g;
 #pragma unroll
       for (int t = 0; t < BT; ++t) {
-        const int b = m + 16 * t;
+        const int b = rbase + m + 16 * t;
         if (b < a.B && k0 < a.K) part[t] += sumsq8(ldg16(a.x + (size_t)b * a.ldx + k0));
       }
     }
@@ -103,7 +108,7 @@ __global__ __launch_bounds__(256) void skinny_kernel(GemmArgs a) {
       nw[c] = (NORM && in && k0 < a.K) ? ldg16(a.norm_w + k0) : make_uint4(0, 0, 0, 0);
 #pragma unroll
       for (int t = 0; t < BT; ++t) {
-        const int b = m + 16 * t;
+        const int b = rbase + m + 16 * t;
         xv[c][t] = (in && b < a.B && k0 < a.K) ? ldg16(a.x + (size_t)b * a.ldx + k0) : make_uint4(0, 0, 0, 0);
       }
     }
@@ -139,14 +144,14 @@ __global__ __launch_bounds__(256) void skinny_kernel(GemmArgs a) {
 
 #pragma unroll
   for (int t = 0; t < BT; ++t) {
-    const int b = m + 16 * t;
+    const int b = rbase + m + 16 * t;
     if (b < a.B) gemm_epilogue<EPI>(a, b, strip, g, acc[t]);
   }
 }
 
 template <int BT, bool NORM>
 int launch_epi(const GemmArgs& a, int epi, int strips, hipStream_t st) {
-  dim3 grid(strips), block(256);
+  dim3 grid((unsigned)((strips + 7) / 8 * 8 * a.ny)), block(256);
   switch (epi) {
     case EPI_STORE: hipLaunchKernelGGL((skinny_kernel<BT, NORM, EPI_STORE>), grid, block, 0, st, a); break;
     case EPI_RESIDUAL: hipLaunchKernelGGL((skinny_kernel<BT, NORM, EPI_RESIDUAL>), grid, block, 0, st, a); break;
@@ -157,13 +162,15 @@ int launch_epi(const GemmArgs& a, int epi, int strips, hipStream_t st) {
   return ohara_launch_status();
 }
 
-int launch_chunk(const GemmArgs& a, int epi, int strips, hipStream_t st) {
-  const bool norm = a.norm_w != nullptr;
-  const int bt = (a.B + 15) / 16;
-  if (bt == 1) return norm ? launch_epi<1, true>(a, epi, strips, st) : launch_epi<1, false>(a, epi, strips, st);
-  if (bt == 2) return norm ? launch_epi<2, true>(a, epi, strips, st) : launch_epi<2, false>(a, epi, strips, st);
-  if (bt <= 4) return norm ? launch_epi<4, true>(a, epi, strips, st) : launch_epi<4, false>(a, epi, strips, st);
-  return OHARA_ESIZE;
+// Up to 64 rows: every workgroup multiplies one strip by 16 rows; more rows are more workgroups
+// per strip (the strip is then read once from HBM and again from L2), which keeps the per-wave
+// register footprint and the norm work of a workgroup at the 16-row level.
+int launch_chunk(const GemmArgs& a0, int epi, int strips, hipStream_t st) {
+  GemmArgs a = a0;
+  a.ny = (a.B + 15) / 16;
+  a.nstrips = strips;
+  if (a.ny > 4) return OHARA_ESIZE;
+  return a.norm_w ? launch_epi<1, true>(a, epi, strips, st) : launch_epi<1, false>(a, epi, strips, st);
 }
 
 // Rows beyond 64 are processed in chunks of 64 (each chunk streams the weights once).
