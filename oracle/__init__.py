@@ -10,7 +10,7 @@ integer arithmetic), the algorithm of the reference file:line it cites.  The
 restatement is functional (a flat ``dict`` of tensors keyed by the reference's
 state-dict names) rather than an ``nn.Module`` tree.
 
-Pinning status (what independently fixes each function; see tests/test_oracle_*.py):
+Pinning status (what independently fixes each function; see tests/test_oracle.py):
 
   rms_norm            closed form, unit-RMS invariant, fp64 brute force
   rope_table          closed form cos/sin(t * theta^(-2i/D)) in fp64
@@ -23,7 +23,7 @@ Pinning status (what independently fixes each function; see tests/test_oracle_*.
   swiglu / linear     F.silu / matmul library routines
   llama_forward       composition: golden fixture tests/golden/llama_tiny_*.pt
   moe_route/dispatch  per-token hand loop, k distinct experts, weights sum to 1,
-                      golden fixture tests/golden/moe_tiny.pt
+                      golden fixture tests/golden/llama_tiny_moe.pt
   sample_*            the reference tests' known answers; exhaustive small-V
                       restatement in fp64; inverse-CDF identities
   bitlinear_*         torch.int32 matmul (library routine), closed forms
