@@ -76,10 +76,13 @@ def lm_head_bytes(cfg, batch):
     return 2 * (v * d + d) + batch * 2 * (d + v)
 
 
-def time_decode(model, batch, prompt_len, warmup, steps, seed=0, persistent=None):
+def time_decode(model, batch, prompt_len, warmup, steps, seed=0, persistent=None, sampling=None):
     g = torch.Generator().manual_seed(seed)
     prompt = torch.randint(0, model.config.vocab_size, (batch, prompt_len), generator=g).to(model.device)
-    sess = model.session(batch, warmup + steps + 8, persistent=persistent)
+    u = None
+    if sampling is not None:  # one fixed, seeded tensor of uniform draws for the whole run
+        u = torch.rand(warmup + steps + 8, batch, generator=g).to(model.device)
+    sess = model.session(batch, warmup + steps + 8, persistent=persistent, sampling=sampling, u=u)
     sess.prefill(prompt)
     sess.capture()
     sess.run(max(0, warmup - 1))
@@ -432,6 +435,17 @@ def main():
         del sess
         torch.cuda.empty_cache()
 
+    # the same decode at batch 1 with temperature 0.8 / top-k 50 / top-p 0.9 sampling from a
+    # pre-drawn uniform tensor (forward + fused sampler per step, replayed from one graph)
+    from ohara_amd.sampling import SamplingConfig
+
+    dt, _, sess = time_decode(model, 1, args.prompt, args.warmup, args.steps,
+                              sampling=SamplingConfig(temperature=0.8, top_k=50, top_p=0.9))
+    results["1_sampled"] = {"tokens_per_s": round(args.steps / dt, 1), "ms_per_step": round(dt / args.steps * 1e3, 4),
+                            "sampling": "temperature 0.8, top-k 50, top-p 0.9, seeded uniform draws",
+                            "launch": "persistent kernel + sampler kernel per step"}
+    del sess
+    torch.cuda.empty_cache()
     r1 = results[1]
     out = {
         "metric": "decode tokens/s at batch 1 & 32 (d12 Llama, 4k ctx) + % of HBM roofline",

@@ -152,11 +152,14 @@ int ohara_argmax_bf16(const uint16_t* logits, int ldl, int batch, int vocab, int
  * torch.multinomial is replaced by inverse-CDF sampling with the caller's uniform draw
  * u[b] in [0,1); equal probabilities are ordered lowest id first.  Deterministic.
  * logits: (batch, vocab) bf16 (logits_are_fp32 = 0) or fp32.  vocab <= 131072.
- * history / step_state as in ohara_argmax_bf16.  temperature == 0 is ohara_argmax_bf16. */
+ * history / step_state as in ohara_argmax_bf16.  With step_state and u_step_stride > 0 the draw of
+ * row b is u[step * u_step_stride + b] (step = index of the token being produced, read on the
+ * device), so a captured decode loop walks a pre-drawn (steps, batch) tensor by itself;
+ * otherwise u[b].  temperature == 0 is ohara_argmax_bf16. */
 int ohara_sample_topk_topp(const void* logits, int logits_are_fp32, int ldl, int batch, int vocab,
                            int valid_vocab, float temperature, int top_k, float top_p, const float* u,
-                           int64_t* out_ids, int64_t* history, int hist_cap, int32_t* step_state,
-                           void* stream);
+                           int u_step_stride, int64_t* out_ids, int64_t* history, int hist_cap,
+                           int32_t* step_state, void* stream);
 
 /* ---- BitNet-b1.58 BitLinear (ternary weights x int8 activations, int32 accumulate) ------
  * Integer form of BitLinear.forward (experiments/bitnet/bitnet.py:29-59):

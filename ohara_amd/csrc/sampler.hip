@@ -13,11 +13,15 @@
 // that order open).  Every reduction runs in a fixed order, so the result is a pure
 // function of (logits, parameters, u).
 //
-// A thread owns EPT consecutive vocabulary entries in registers; the 1024 threads cover up
-// to 1024*EPT ids.  The sorted prefix is built 1024 candidates at a time (radix select on
-// the probability bits, ordered compaction, bitonic sort in LDS) and scanned sequentially
-// in fp32, the order torch.cumsum uses; a peaked distribution or any top-k <= 1024 needs a
-// single round.
+// A thread owns EPT consecutive vocabulary entries in registers; the 1024 threads cover up to
+// 1024*EPT ids.  Two routes from there:
+//   * top-k <= 1024: the survivors (everything at or above the k-th largest; a lower bound of it
+//     comes from the per-thread maxima) are compacted into LDS, sorted once (bitonic, descending,
+//     ties lowest id first), soft-maxed and scanned sequentially in fp32 by one thread - the
+//     order the reference's cumsum walks;
+//   * otherwise the nucleus is found without sorting: the smallest probability that is still
+//     kept, and then the probability the draw lands on, by bisection over the probability bits
+//     with block-wide mass sums in a fixed order (cost independent of how many tokens are kept).
 #include "common.h"
 
 namespace {
@@ -31,6 +35,7 @@ struct SampleArgs {
   float temperature, top_p;
   int top_k;
   const float* u;
+  int u_step_stride;     // with step_state: the draw of row b is u[step * u_step_stride + b]
   int64_t* out;
   int64_t* history;      // optional (hist_cap, B)
   int32_t* step_state;   // optional {pos, step, done, pad}
@@ -47,7 +52,6 @@ struct Smem {
   float wred[16];
   int wredi[16];
   float fscan[NT];
-  int iscan[NT];
   uint32_t skey[CAP];
   int sid[CAP];
   int misc[8];
@@ -199,6 +203,65 @@ __device__ __forceinline__ float load_logit<float>(const void* base, size_t i) {
   return reinterpret_cast<const float*>(base)[i];
 }
 
+__device__ __forceinline__ float unfkey(uint32_t k) {  // inverse of fkey
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+// Bitonic sort of the first n2 (power of two) entries of (skey, sid): descending by key,
+// ascending by id among equal keys.
+__device__ __forceinline__ void sort_candidates(Smem& s, int n2) {
+  const int tid = threadIdx.x;
+  for (int k2 = 2; k2 <= n2; k2 <<= 1) {
+    for (int j = k2 >> 1; j > 0; j >>= 1) {
+      for (int t = tid; t < n2; t += NT) {
+        const int ixj = t ^ j;
+        if (ixj > t) {
+          const uint32_t ka = s.skey[t], kb = s.skey[ixj];
+          const int ia = s.sid[t], ib = s.sid[ixj];
+          const bool a_first = ka > kb || (ka == kb && ia < ib);  // a precedes b in the target order
+          const bool up = (t & k2) == 0;
+          if (up ? !a_first : a_first) {
+            s.skey[t] = kb; s.skey[ixj] = ka;
+            s.sid[t] = ib; s.sid[ixj] = ia;
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
+// The same by ascending id only (vocabulary order), carrying the keys.
+__device__ __forceinline__ void sort_by_id(Smem& s, int n2) {
+  const int tid = threadIdx.x;
+  for (int k2 = 2; k2 <= n2; k2 <<= 1) {
+    for (int j = k2 >> 1; j > 0; j >>= 1) {
+      for (int t = tid; t < n2; t += NT) {
+        const int ixj = t ^ j;
+        if (ixj > t) {
+          const int ia = s.sid[t], ib = s.sid[ixj];
+          const bool up = (t & k2) == 0;
+          if (up ? ia > ib : ia < ib) {
+            const uint32_t ka = s.skey[t], kb = s.skey[ixj];
+            s.skey[t] = kb; s.skey[ixj] = ka;
+            s.sid[t] = ib; s.sid[ixj] = ia;
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
+template <typename T, int EPT>
+__device__ __forceinline__ void load_row_scalar(const SampleArgs& a, int b, int base, int nvalid, float temp, float* x) {
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) {
+    const int id = base + i;
+    x[i] = id < nvalid ? load_logit<T>(a.logits, (size_t)b * a.ldl + id) / temp : -INFINITY;
+  }
+}
+
 template <typename T, int EPT>
 __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
   __shared__ Smem s;
@@ -207,13 +270,135 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
   const int base = tid * EPT;
   float x[EPT];
   const float temp = a.temperature;
+  if (sizeof(T) == 2 && EPT % 8 == 0 && (a.ldl & 7) == 0 && ((reinterpret_cast<uintptr_t>(a.logits) & 15) == 0)) {
+    // bf16 rows: eight values per 16-byte load
+    const bf16_t* row = reinterpret_cast<const bf16_t*>(a.logits) + (size_t)b * a.ldl + base;
 #pragma unroll
-  for (int i = 0; i < EPT; ++i) {
-    const int id = base + i;
-    x[i] = id < nvalid ? load_logit<T>(a.logits, (size_t)b * a.ldl + id) / temp : -INFINITY;
+    for (int c = 0; c < EPT / 8; ++c) {
+      const uint4 v = base + 8 * c < V ? ldg16(row + 8 * c) : make_uint4(0, 0, 0, 0);
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int id = base + 8 * c + 2 * j;
+        x[8 * c + 2 * j] = id < nvalid ? lo_bf(w[j]) / temp : -INFINITY;
+        x[8 * c + 2 * j + 1] = id + 1 < nvalid ? hi_bf(w[j]) / temp : -INFINITY;
+      }
+    }
+  } else {
+    load_row_scalar<T, EPT>(a, b, base, nvalid, temp, x);
+  }
+  const float u = a.u[(a.step_state && a.u_step_stride > 0 ? (size_t)a.step_state[1] * a.u_step_stride : 0) + b];
+  int token = -1;
+  bool compact = false;
+  // ---- small top-k: the survivors fit one sorted block, everything after works on that block -----
+  if (a.top_k > 0 && min(a.top_k, V) <= CAP) {
+    const int k = min(a.top_k, V);
+    auto in_vocab = [&](int i) { return base + i < V; };
+    auto xkey = [&](int i) { return fkey(x[i]); };  // > 0 for every float but -NaN
+    // lower bound of the k-th largest: the k-th largest of the per-thread maxima
+    uint32_t tmax = 0;
+#pragma unroll
+    for (int i = 0; i < EPT; ++i)
+      if (in_vocab(i)) tmax = max(tmax, xkey(i));
+    const int have = block_sum_i(tmax > 0 ? 1 : 0, s);
+    uint32_t bound = 0;
+    if (have >= k) {
+      int dummy;
+      bound = radix_select<1>(k, dummy, s, [&](int) { return tmax > 0; }, [&](int) { return tmax; });
+    }
+    int c = 0;
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) c += (in_vocab(i) && xkey(i) >= bound) ? 1 : 0;
+    int off;
+    const int n_c = block_excl_scan_i(c, off, s);
+    if (n_c <= CAP) {  // (else: many ties at the bound - the general path below handles it)
+      compact = true;
+      __syncthreads();
+      if (c > 0) {
+#pragma unroll
+        for (int i = 0; i < EPT; ++i)
+          if (in_vocab(i) && xkey(i) >= bound) {
+            s.skey[off] = xkey(i);
+            s.sid[off] = base + i;
+            ++off;
+          }
+      }
+      int n2 = 64;
+      while (n2 < n_c) n2 <<= 1;
+      __syncthreads();
+      for (int i = n_c + tid; i < n2; i += NT) {
+        s.skey[i] = 0;  // padding sorts last
+        s.sid[i] = 0x7fffffff;
+      }
+      __syncthreads();
+      sort_candidates(s, n2);
+      // kept: everything >= the k-th largest key (ties at the threshold survive, chat_engine.py:66-69)
+      const uint32_t tk = s.skey[min(k, n_c) - 1];
+      int n_kept = block_sum_i((tid < n_c && s.skey[tid] >= tk) ? 1 : 0, s);
+      // softmax over the kept entries (the rest of the vocabulary is -inf): entry 0 is the maximum
+      const float m0 = unfkey(s.skey[0]);
+      const float e = tid < n_kept ? expf(unfkey(s.skey[tid]) - m0) : 0.f;
+      const float Z = block_sum(e, s);
+      __syncthreads();
+      if (tid < n_kept) s.skey[tid] = __float_as_uint(e / Z);  // probabilities, still in sorted order
+      __syncthreads();
+      const bool nucleus = a.top_p > 0.f && a.top_p < 1.f;
+      if (!nucleus) {  // vocabulary-order draw (chat_engine.py:82): order the kept entries by id
+        int m2 = 64;
+        while (m2 < n_kept) m2 <<= 1;
+        for (int i = n_kept + tid; i < m2; i += NT) {
+          s.skey[i] = 0;
+          s.sid[i] = 0x7fffffff;
+        }
+        __syncthreads();
+        sort_by_id(s, m2);
+      }
+      if (tid == 0) {
+        // sequential fp32 sums in the order the reference's cumsum walks
+        int tok = -1, last = -1;
+        if (nucleus) {
+          float kept = 0.f, run = 0.f;
+          int n_in = 0;
+          for (int j = 0; j < n_kept; ++j) {  // kept prefix: mass before the token <= top_p
+            if (run > a.top_p) break;
+            const float p = __uint_as_float(s.skey[j]);
+            kept += p;
+            run += p;
+            ++n_in;
+          }
+          const float target = u * kept;
+          run = 0.f;
+          for (int j = 0; j < n_in; ++j) {
+            run += __uint_as_float(s.skey[j]);
+            last = s.sid[j];
+            if (run > target) {
+              tok = s.sid[j];
+              break;
+            }
+          }
+        } else {
+          float total = 0.f;
+          for (int j = 0; j < n_kept; ++j) total += __uint_as_float(s.skey[j]);
+          const float target = u * total;
+          float run = 0.f;
+          for (int j = 0; j < n_kept; ++j) {
+            const float p = __uint_as_float(s.skey[j]);
+            run += p;
+            if (p > 0.f) last = s.sid[j];
+            if (p > 0.f && run > target) {
+              tok = s.sid[j];
+              break;
+            }
+          }
+        }
+        s.misc[3] = tok >= 0 ? tok : max(last, 0);  // rounding pushed the target past the end: last kept id
+      }
+      __syncthreads();
+      token = s.misc[3];
+    }
   }
   // ---- top-k: keep x >= k-th largest ---------------------------------------------
-  if (a.top_k > 0) {
+  if (!compact && a.top_k > 0) {
     const int k = min(a.top_k, V);
     int ngt;
     auto in_vocab = [&](int i) { return base + i < V; };
@@ -223,6 +408,7 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
     for (int i = 0; i < EPT; ++i)
       if (fkey(x[i]) < tk) x[i] = -INFINITY;
   }
+  if (!compact) {
   // ---- softmax ---------------------------------------------------------------------
   float m = -INFINITY;
 #pragma unroll
@@ -237,8 +423,6 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
   const float Z = block_sum(zs, s);
 #pragma unroll
   for (int i = 0; i < EPT; ++i) x[i] = x[i] / Z;  // probabilities; 0 marks a filtered id
-  const float u = a.u[b];
-  int token = -1;
 
   if (!(a.top_p > 0.f && a.top_p < 1.f)) {
     // ---- inverse CDF in vocabulary order ------------------------------------------
@@ -291,158 +475,73 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
     __syncthreads();
     token = s.misc[2] == 0x7fffffff ? max(last_id, 0) : s.misc[2];
   } else {
-    // ---- nucleus: sorted prefix, CAP candidates per round --------------------------
-    // live(i): probability > 0 and not yet extracted
-    uint32_t taken[(EPT + 31) / 32];
+    // ---- nucleus without sorting: thresholds on the probability bits by bisection --------------
+    // In descending order (ties lowest id first) a token is kept iff the mass before it is <= top_p.
+    // With G(t) = mass of the keys above t, that is: every key above Tk, plus the first
+    // floor((top_p - G(T)) / p_T) + 1 ties at T, where T is the smallest key with G(T) <= top_p.  T is
+    // found bit by bit (31 block sums in a fixed order), and so is the key the draw u * S lands on;
+    // the sums are over registers, so the cost does not depend on how many tokens are kept.
+    auto pkey = [&](int i) { return __float_as_uint(x[i]); };  // p > 0: bits are monotone; 0 = filtered
+    auto mass_ge = [&](uint32_t c) {
+      float t = 0.f;
 #pragma unroll
-    for (int w = 0; w < (EPT + 31) / 32; ++w) taken[w] = 0;
-    if (tid == 0) s.misc[4] = -1;
-    int my_live = 0;
+      for (int i = 0; i < EPT; ++i) t += (pkey(i) >= c) ? x[i] : 0.f;
+      return block_sum(t, s);
+    };
+    auto count_eq = [&](uint32_t c) {
+      int n = 0;
 #pragma unroll
-    for (int i = 0; i < EPT; ++i) my_live += x[i] > 0.f ? 1 : 0;
-    const int C = block_sum_i(my_live, s);
-    // pass 0 finds the kept mass S; pass 1 finds the token at u * S
-    float S = 0.f;
-    for (int pass = 0; pass < 2 && token < 0; ++pass) {
-#pragma unroll
-      for (int w = 0; w < (EPT + 31) / 32; ++w) taken[w] = 0;
-      int remaining = C;
-      float cum = 0.f;       // mass before the current round, as the sequential fp32 sum
-      bool done = false;
-      while (!done && remaining > 0) {
-        const int take = min(remaining, CAP);
-        auto live = [&](int i) { return x[i] > 0.f && !((taken[i >> 5] >> (i & 31)) & 1u); };
-        auto key = [&](int i) { return __float_as_uint(x[i]); };  // p > 0: bits are monotone
-        int ngt = 0;
-        uint32_t tk = 0;
-        if (take < remaining) tk = select_small<EPT>(take, ngt, s, live, key);
-        // ordered compaction: all keys > tk, then ties at tk in id order until `take`
-        int c_gt = 0, c_eq = 0;
-#pragma unroll
-        for (int i = 0; i < EPT; ++i)
-          if (live(i)) {
-            const uint32_t k = key(i);
-            if (take == remaining || k > tk) ++c_gt;
-            else if (k == tk) ++c_eq;
-          }
-        int off_gt, off_eq;
-        const int tot_gt = block_excl_scan_i(c_gt, off_gt, s);
-        block_excl_scan_i(c_eq, off_eq, s);
-        const int room_eq = take - tot_gt;
-#pragma unroll
-        for (int i = 0; i < EPT; ++i)
-          if (live(i)) {
-            const uint32_t k = key(i);
-            int slot = -1;
-            if (take == remaining || k > tk) slot = off_gt++;
-            else if (k == tk) {
-              if (off_eq < room_eq) slot = tot_gt + off_eq;
-              ++off_eq;
-            }
-            if (slot >= 0) {
-              s.skey[slot] = k;
-              s.sid[slot] = base + i;
-              taken[i >> 5] |= 1u << (i & 31);
-            }
-          }
-        __syncthreads();
-        int n2 = 64;  // sort length: the power of two that holds this round's candidates
-        while (n2 < take) n2 <<= 1;
-        for (int i = take + tid; i < n2; i += NT) {
-          s.skey[i] = 0;  // padding sorts last
-          s.sid[i] = 0x7fffffff;
-        }
-        __syncthreads();
-        // bitonic sort, descending by key, ascending by id among equal keys
-        for (int k2 = 2; k2 <= n2; k2 <<= 1) {
-          for (int j = k2 >> 1; j > 0; j >>= 1) {
-            for (int t = tid; t < n2; t += NT) {
-              const int ixj = t ^ j;
-              if (ixj > t) {
-                const uint32_t ka = s.skey[t], kb = s.skey[ixj];
-                const int ia = s.sid[t], ib = s.sid[ixj];
-                const bool a_first = ka > kb || (ka == kb && ia < ib);  // a precedes b in the target order
-                const bool up = (t & k2) == 0;
-                if (up ? !a_first : a_first) {
-                  s.skey[t] = kb; s.skey[ixj] = ka;
-                  s.sid[t] = ib; s.sid[ixj] = ia;
-                }
-              }
-            }
-            __syncthreads();
-          }
-        }
-        // sequential fp32 scan of the sorted block
-        if (tid == 0) {
-          float run = cum;
-          int stop = 0, tok = -1;
-          if (pass == 0) {
-            float kept = S;
-            for (int j = 0; j < take; ++j) {
-              const float p = __uint_as_float(s.skey[j]);
-              if (run > a.top_p) {  // mass before this token already exceeds top_p: dropped, and all after
-                stop = 1;
-                break;
-              }
-              kept += p;
-              run += p;
-            }
-            S = kept;
-            s.fmisc[1] = S;
-            if (cum == 0.f && (stop || remaining == take)) {
-              // the whole kept set sits in this sorted block: draw from it now, no second pass
-              const float target = u * S;
-              float r2 = 0.f;
-              int last = -1;
-              for (int j = 0; j < take; ++j) {
-                const float p = __uint_as_float(s.skey[j]);
-                if (r2 > a.top_p) break;
-                r2 += p;
-                last = s.sid[j];
-                if (r2 > target) {
-                  tok = s.sid[j];
-                  break;
-                }
-              }
-              if (tok < 0) tok = max(last, 0);  // rounding pushed the target past the end: last kept id
-              stop = 1;
-            }
-          } else {
-            const float target = u * S;
-            int last = -1;
-            for (int j = 0; j < take; ++j) {
-              const float p = __uint_as_float(s.skey[j]);
-              if (run > a.top_p) {
-                stop = 1;
-                break;
-              }
-              run += p;
-              last = s.sid[j];
-              if (run > target) {
-                tok = s.sid[j];
-                stop = 1;
-                break;
-              }
-            }
-            if (tok < 0 && (stop || remaining - take == 0) && last >= 0) tok = last;  // rounding: last kept id
-            if (tok < 0 && stop) tok = s.misc[4];                                    // boundary fell between rounds
-            if (last >= 0) s.misc[4] = last;
-          }
-          s.fmisc[0] = run;
-          s.misc[2] = stop;
-          s.misc[3] = tok;
-        }
-        __syncthreads();
-        cum = s.fmisc[0];
-        S = s.fmisc[1];
-        done = s.misc[2] != 0;
-        if (s.misc[3] >= 0) token = s.misc[3];
-        remaining -= take;
-        __syncthreads();
+      for (int i = 0; i < EPT; ++i) n += (pkey(i) == c) ? 1 : 0;
+      return block_sum_i(n, s);
+    };
+    // smallest key Tk >= 1 with mass(keys > Tk) <= limit; needs mass(keys >= 1) > limit
+    auto threshold = [&](float limit) {
+      uint32_t tf = 0;  // largest t with mass(keys >= t + 1) > limit
+      for (int bit = 30; bit >= 0; --bit) {
+        const uint32_t c = tf | (1u << bit);
+        if (mass_ge(c + 1) > limit) tf = c;
       }
-      if (pass == 1 && token < 0) token = max(s.misc[4], 0);
+      return tf + 1;
+    };
+    const float total = mass_ge(1u);
+    uint32_t Tk = 1;  // everything with p > 0 when top_p is not below the total mass
+    float G = 0.f, S = total;
+    int n_keep = 0x7fffffff;
+    if (total > a.top_p) {
+      Tk = threshold(a.top_p);
+      G = mass_ge(Tk + 1);
+      const float pT = __uint_as_float(Tk);
+      n_keep = min(count_eq(Tk), (int)floorf((a.top_p - G) / pT) + 1);
+      S = G + (float)n_keep * pT;
     }
+    const float target = u * S;
+    uint32_t Td = threshold(target);  // target < S <= mass(keys >= Tk): the key found is >= Tk
+    if (Td < Tk) Td = Tk;               // (rounding guard)
+    const float Gd = mass_ge(Td + 1);
+    const int ties = count_eq(Td);
+    int r = (int)floorf((target - Gd) / __uint_as_float(Td));
+    r = max(0, min(r, min(ties, Td == Tk ? n_keep : ties) - 1));
+    // the r-th token in id order among the ties at Td
+    int c = 0;
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) c += (pkey(i) == Td) ? 1 : 0;
+    int off;
+    block_excl_scan_i(c, off, s);
+    if (tid == 0) s.misc[3] = -1;
+    __syncthreads();
+    if (c > 0 && off <= r && r < off + c) {
+      int seen = off;
+#pragma unroll
+      for (int i = 0; i < EPT; ++i)
+        if (pkey(i) == Td) {
+          if (seen == r) s.misc[3] = base + i;
+          ++seen;
+        }
+    }
+    __syncthreads();
+    token = max(s.misc[3], 0);
   }
+  }  // !compact
   if (tid == 0) {
     a.out[b] = token;
     if (a.step_state) {
@@ -474,13 +573,13 @@ int launch_sample(const SampleArgs& a, hipStream_t st) {
 
 extern "C" int ohara_sample_topk_topp(const void* logits, int logits_are_fp32, int ldl, int batch, int vocab,
                                       int valid_vocab, float temperature, int top_k, float top_p, const float* u,
-                                      int64_t* out_ids, int64_t* history, int hist_cap, int32_t* step_state,
-                                      void* stream) {
+                                      int u_step_stride, int64_t* out_ids, int64_t* history, int hist_cap,
+                                      int32_t* step_state, void* stream) {
   if (!logits || !u || !out_ids || batch < 1 || vocab < 1 || ldl < vocab) return OHARA_EINVAL;
-  if (!(temperature > 0.f) || top_k < 0 || !(top_p >= 0.f && top_p <= 1.f)) return OHARA_EINVAL;
+  if (!(temperature > 0.f) || top_k < 0 || !(top_p >= 0.f && top_p <= 1.f) || u_step_stride < 0) return OHARA_EINVAL;
   SampleArgs a{};
   a.logits = logits; a.ldl = ldl; a.V = vocab; a.valid = valid_vocab > 0 ? valid_vocab : vocab;
-  a.temperature = temperature; a.top_p = top_p; a.top_k = top_k; a.u = u; a.out = out_ids;
+  a.temperature = temperature; a.top_p = top_p; a.top_k = top_k; a.u = u; a.u_step_stride = u_step_stride; a.out = out_ids;
   a.history = history; a.hist_cap = hist_cap; a.step_state = step_state; a.B = batch;
   return logits_are_fp32 ? launch_sample<float>(a, (hipStream_t)stream) : launch_sample<bf16_t>(a, (hipStream_t)stream);
 }

@@ -322,8 +322,8 @@ class Llama:
     # -- device-resident greedy loop --------------------------------------------------
 
     def session(self, batch: int, max_new_tokens: int, valid_vocab: int = 0, kv_cache: list | None = None,
-                persistent: bool | None = None):
-        return DecodeSession(self, batch, max_new_tokens, valid_vocab, kv_cache, persistent)
+                persistent: bool | None = None, sampling=None, u=None):
+        return DecodeSession(self, batch, max_new_tokens, valid_vocab, kv_cache, persistent, sampling, u)
 
     def supports_persistent(self, batch: int) -> bool:
         """Shapes the single-launch decode kernel covers."""
@@ -356,8 +356,21 @@ class DecodeSession:
     PERSISTENT_SPLITS = 16
 
     def __init__(self, model: Llama, batch: int, max_new_tokens: int, valid_vocab: int = 0, kv_cache=None,
-                 persistent: bool | None = None):
+                 persistent: bool | None = None, sampling=None, u=None):
+        """``sampling``: an object with temperature / top_k / top_p (a ``SamplingConfig``); None or
+        temperature 0 selects greedily.  ``u``: (max_new_tokens, batch) fp32 uniform draws in [0, 1),
+        row t for the t-th generated token (ohara/chat_engine.py:51-82 with multinomial replaced by
+        inverse-CDF sampling); drawn from torch's generator when omitted."""
         self.model, self.batch = model, batch
+        self.sampling = sampling if (sampling is not None and sampling.temperature > 0) else None
+        self.u = None
+        if self.sampling is not None:
+            rows = max(max_new_tokens, 1)
+            if u is None:
+                u = torch.rand(rows, batch, device=model.device, dtype=torch.float32)
+            if u.shape != (rows, batch):
+                raise ValueError("u must have shape (max_new_tokens, batch)")
+            self.u = u.to(device=model.device, dtype=torch.float32).contiguous()
         if persistent is None:
             # measured on d12: the single launch wins up to four sequences (0.47 ms against 0.48 ms
             # per step at 4); from eight on the kernel chain is faster (0.50 against 0.58 ms)
@@ -390,8 +403,11 @@ class DecodeSession:
         pbuf.ids.copy_(prompt_ids.reshape(-1).to(device=m.device, dtype=torch.int64))
         st = m._state_struct(pbuf, self.cache, self.logits, valid_vocab=self.valid_vocab)
         st.step_state = 0
-        check(lib().ohara_llama_forward(C.byref(m._c_model), C.byref(st), P, 0, 0, _lib.OHARA_LOGITS_LAST, 1,
-                                        torch.cuda.current_stream().cuda_stream), "prefill")
+        check(lib().ohara_llama_forward(C.byref(m._c_model), C.byref(st), P, 0, 0, _lib.OHARA_LOGITS_LAST,
+                                        0 if self.sampling else 1, torch.cuda.current_stream().cuda_stream), "prefill")
+        if self.sampling:
+            ops.sample_topk_topp(self.logits, self.sampling.temperature, self.sampling.top_k, self.sampling.top_p,
+                                 self.u[0], self.valid_vocab or None, out=pbuf.ids[:B])
         for cc in self.cache:
             cc._commit(B, P)
         self.pos = P
@@ -423,12 +439,18 @@ class DecodeSession:
     def _launch_step(self) -> None:
         m = self.model
         stream = torch.cuda.current_stream().cuda_stream
+        greedy = 0 if self.sampling else 1
         if self.persistent:
             check(lib().ohara_llama_decode_persistent(C.byref(m._c_model), C.byref(self._dst), self._pws.data_ptr(),
-                                                      self._nwg, 0, 1, 0, stream), "persistent decode step")
+                                                      self._nwg, 0, greedy, 0, stream), "persistent decode step")
         else:
-            check(lib().ohara_llama_forward(C.byref(m._c_model), C.byref(self._dst), 1, 0, 1, _lib.OHARA_LOGITS_LAST, 1,
-                                            stream), "decode step")
+            check(lib().ohara_llama_forward(C.byref(m._c_model), C.byref(self._dst), 1, 0, 1, _lib.OHARA_LOGITS_LAST,
+                                            greedy, stream), "decode step")
+        if self.sampling:
+            # the sampler does the selection kernel's bookkeeping (next ids, history, position)
+            ops.sample_topk_topp(self.logits, self.sampling.temperature, self.sampling.top_k, self.sampling.top_p,
+                                 self.u, self.valid_vocab or None, out=self._dbuf.ids[: self.batch],
+                                 history=self.history, step_state=self._dbuf.step_state, u_per_step=True)
 
     def check_error(self) -> None:
         """Raise if a barrier wait of the persistent kernel expired (synchronises)."""

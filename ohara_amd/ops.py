@@ -230,14 +230,19 @@ def argmax(logits: torch.Tensor, valid_vocab: int | None = None, next_ids=None, 
 
 
 def sample_topk_topp(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, u: torch.Tensor,
-                     valid_vocab: int | None = None, out=None, history=None, step_state=None) -> torch.Tensor:
-    """logits (B, V) bf16 or fp32 on the device, u (B,) fp32 uniform draws -> ids (B,) int64."""
+                     valid_vocab: int | None = None, out=None, history=None, step_state=None,
+                     u_per_step: bool = False) -> torch.Tensor:
+    """logits (B, V) bf16 or fp32 on the device, u (B,) fp32 uniform draws -> ids (B,) int64.
+    With ``u_per_step`` (needs step_state) u is (steps, B) and row ``step`` is read on the device."""
     if logits.dtype not in (BF16, torch.float32):
         raise ValueError("logits must be bfloat16 or float32")
     _need(logits, logits.dtype, "logits")
     _need(u, torch.float32, "u")
     b, v = logits.shape
-    if u.numel() != b:
+    if u_per_step:
+        if step_state is None or u.ndim != 2 or u.shape[1] != b:
+            raise ValueError("u_per_step needs step_state and a (steps, batch) tensor of draws")
+    elif u.numel() != b:
         raise ValueError("one uniform draw per row is required")
     if out is None:
         out = torch.empty(b, dtype=torch.int64, device=logits.device)
@@ -245,7 +250,7 @@ def sample_topk_topp(logits: torch.Tensor, temperature: float, top_k: int, top_p
         lib().ohara_sample_topk_topp(
             _ptr(logits), 1 if logits.dtype == torch.float32 else 0, logits.stride(0), b, v,
             v if valid_vocab is None else valid_vocab, float(temperature), int(top_k), float(top_p), _ptr(u),
-            _ptr(out), _ptr(history), 0 if history is None else history.shape[0], _ptr(step_state), _stream(),
+            b if u_per_step else 0, _ptr(out), _ptr(history), 0 if history is None else history.shape[0], _ptr(step_state), _stream(),
         ),
         "sample_topk_topp",
     )

@@ -235,3 +235,56 @@ def test_d12_decode_parity(cuda):
         _assert_logits_close(got, want, 2e-2, mean_tol)
         nxt = want[:, -1].float().argmax(-1, keepdim=True)
     _check_greedy(model, ref, prompt, 64, cuda, 2e-2, mean_tol)
+
+
+@pytest.mark.parametrize("persistent", [True, False])
+def test_sampled_decode_session(cuda, persistent):
+    """Temperature 0.8 / top-k 50 / top-p 0.9 decode driven by a pre-drawn uniform tensor, with no
+    host round trip per token (forward + sampler replayed from one graph).  Checked teacher-forced:
+    at every step the oracle, fed the session's own tokens, must place the session's choice in the
+    CDF interval that contains that step's draw (the logits differ at the bf16 level, so the
+    interval is widened by what that can move a boundary)."""
+    from oracle.sampling_ref import candidate_cdf_ref
+    from ohara_amd.llama import Config, Llama
+    from ohara_amd.sampling import SamplingConfig
+
+    kw = dict(vocab_size=1024, hidden_size=256, intermediate_size=512, num_attention_heads=2,
+              num_key_value_heads=0, num_hidden_layers=3, max_sequence_length=128, rope_theta=10000.0)
+    rcfg = R.RefConfig(**kw)
+    w = R.init_weights(rcfg, seed=4, dtype=BF, std=0.08)
+    ref = R.RefLlama(rcfg, w)
+    model = Llama(Config(**kw), w, device=cuda)
+    B, P, N = 2, 9, 24
+    g = torch.Generator().manual_seed(11)
+    prompt = torch.randint(0, 1024, (B, P), generator=g)
+    u = torch.rand(N, B, generator=g)
+    cfg = SamplingConfig(temperature=0.8, top_k=50, top_p=0.9)
+    sess = model.session(B, N, persistent=persistent, sampling=cfg, u=u.to(cuda))
+    sess.prefill(prompt.to(cuda))
+    sess.run(N - 1)
+    toks = sess.tokens().cpu()  # (B, N)
+    assert toks.shape == (B, N)
+    # a second session with the same draws reproduces the tokens bit for bit, eagerly too
+    sess2 = model.session(B, N, persistent=persistent, sampling=cfg, u=u.to(cuda))
+    sess2.prefill(prompt.to(cuda))
+    sess2.run(N - 1, use_graph=False)
+    assert torch.equal(sess2.tokens().cpu(), toks)
+    # teacher-forced: the oracle model (loose: its logits differ from the kernels' at the bf16 level,
+    # which moves CDF boundaries by a few percent on this high-gain model) and the oracle sampler on
+    # the kernels' own logits (tight: pins the wiring of draws, steps and bookkeeping)
+    cache, gcache = ref.build_kv_cache(B), model.build_kv_cache(B)
+    inp, pos = prompt, 0
+    for t in range(N):
+        logits = ref(inp, cache, pos)
+        glogits = model(inp.to(cuda), gcache, pos).cpu()
+        pos += inp.shape[1]
+        for lg, tol in ((logits, 6e-2), (glogits, 5e-3)):
+            ids, cdf = candidate_cdf_ref(lg[:, -1:].float(), cfg.temperature, cfg.top_p, cfg.top_k)
+            for b in range(B):
+                hit = (ids[b] == int(toks[b, t])).nonzero()
+                assert hit.numel(), (t, b, "token outside the candidate order")
+                j = int(hit[0])
+                lo = float(cdf[b, j - 1]) if j > 0 else 0.0
+                hi = float(cdf[b, j])
+                assert lo - tol <= float(u[t, b]) <= hi + tol, (t, b, tol, int(toks[b, t]), lo, hi, float(u[t, b]))
+        inp = toks[:, t : t + 1]
