@@ -70,6 +70,29 @@ class ChatEngine:
         self.max_sequence_length = model.config.max_sequence_length
         self._sample = sampler_fn if sampler_fn is not None else sample_next_token
 
+    @classmethod
+    def from_checkpoint(cls, checkpoint_path, tokenizer, *, device=None, dtype=None, moe_experts_per_tok: int = 2,
+                        moe_gate_fn: str = "softmax", moe_normalize_weights: bool = True, renderer=None,
+                        stop_ids=None):
+        """ohara/chat_engine.py:275-329: architecture from the tensor shapes (or the exported
+        ``config.json``), weights into the kernel-backed model.  The tokenizer is passed in (the
+        reference rebuilds it from a directory or a hub name, which is outside this path); a
+        checkpoint narrower than the tokenizer is rejected as there."""
+        from .checkpoint import build_model, load_checkpoint
+
+        config, state = load_checkpoint(checkpoint_path, moe_experts_per_tok=moe_experts_per_tok,
+                                        moe_gate_fn=moe_gate_fn, moe_normalize_weights=moe_normalize_weights)
+        if config.vocab_size < len(tokenizer):
+            raise ValueError(
+                f"checkpoint vocabulary ({config.vocab_size:,}) is smaller than the "
+                f"tokenizer ({len(tokenizer):,}). Point --tokenizer-dir at the "
+                "directory saved next to the checkpoint."
+            )
+        if device is None:
+            device = "cuda"
+        model = build_model(config, state, device=device)
+        return cls(model, tokenizer, device=device, dtype=dtype, renderer=renderer, stop_ids=stop_ids)
+
     def metadata(self, checkpoint_path=None) -> dict[str, Any]:
         # ohara/chat_engine.py:331-350 (without the checkpoint sidecar file)
         cfg = self.model.config

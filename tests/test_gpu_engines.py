@@ -84,3 +84,36 @@ def test_inference_on_gpu(cuda):
     out = inf.generate("hello", stream=False, temperature=0.0)
     assert out == "hello" + "y" * 11  # clamped to the context window: 16 - 5 prompt tokens
     assert Inference.sampler(torch.tensor([[[0.1, 0.2, 0.9]]]).to(cuda), temperature=0.0).item() == 2
+
+
+def test_chat_engine_from_checkpoint(cuda, tmp_path):
+    """A state dict saved the way the reference's training scripts do (bare, DDP/compile prefixes,
+    rotary buffers included) comes back as the same model: same config, bit-identical logits."""
+    from ohara_amd.chat_engine import ChatEngine
+    from ohara_amd.llama import Config, Llama, rope_tables
+    from ohara_amd.sampling import SamplingConfig
+
+    tok = CharTokenizer()
+    kw = dict(vocab_size=len(tok) + 13, hidden_size=64, intermediate_size=96, max_sequence_length=48,
+              num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, dropout=0.0)
+    rcfg = R.RefConfig(**kw)
+    w = R.init_weights(rcfg, seed=5, dtype=BF, std=0.1)
+    cos, sin = rope_tables(16, 96, rcfg.rope_theta)
+    saved = {"module._orig_mod." + k: v for k, v in {**w, "freq_cos": cos, "freq_sin": sin}.items()}
+    torch.save({"model": saved, "idx": 3}, tmp_path / "sft.pt")
+    eng = ChatEngine.from_checkpoint(tmp_path / "sft.pt", tok)
+    assert eng.model.config == Config(**kw)
+    direct = Llama(Config(**kw), w, device=cuda)
+    ids = torch.randint(0, len(tok), (2, 7), generator=torch.Generator().manual_seed(0)).to(cuda)
+    assert torch.equal(eng.model(ids), direct(ids))
+    # the 13 padded vocabulary rows are never produced
+    msgs = [{"role": "user", "content": "hello"}]
+    text = eng.generate(msgs, SamplingConfig(temperature=1.5, top_p=1.0, max_new_tokens=16), seed=1)
+    assert isinstance(text, str)
+    # a tokenizer wider than the checkpoint is rejected with the reference's message
+    small = {k: v for k, v in saved.items()}
+    small["module._orig_mod.token_emb.weight"] = saved["module._orig_mod.token_emb.weight"][:10].clone()
+    small["module._orig_mod.vocab_proj.weight"] = saved["module._orig_mod.vocab_proj.weight"][:10].clone()
+    torch.save(small, tmp_path / "small.pt")
+    with pytest.raises(ValueError, match="smaller than the"):
+        ChatEngine.from_checkpoint(tmp_path / "small.pt", tok)
