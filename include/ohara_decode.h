@@ -185,6 +185,24 @@ int ohara_bitlinear_bf16(const uint16_t* x, int ldx, const uint16_t* pre_norm_w,
                          const uint32_t* wp, int n, int k, float gamma, int rows, const uint16_t* resid, int ldr,
                          uint16_t* out, int ldo, int32_t* acc_out, int ldacc, void* stream);
 
+/* Groups of BitLinears that read the same rows, for decode (rows <= 64), one launch each:
+ *   - attn.query / attn.key / attn.value (each with its own norm weight, packed weights and gamma,
+ *     index 0..2 of the three arrays) with rotary + cache append as the epilogue: q_out
+ *     (rows, h*dh) rotated, rotated k and v written at cache position pos + s (pos_dev as in
+ *     ohara_qkv_rope_append_bf16);
+ *   - ff.gate and ff.up with SwiGLU as the epilogue: out[b, f] = bf16(bf16(silu(gate)) * up).
+ * Same arithmetic as the separate calls (bitnet.py:29-59, rotary.py:55-93, kv_cache.py:104-105,
+ * mlp.py:152). */
+int ohara_bitlinear_qkv_rope_append_bf16(const uint16_t* x, int ldx, const uint16_t* pre_norm_w, float eps, int k,
+                                         const uint16_t* const* norm_w, const uint32_t* const* wp, const float* gamma,
+                                         int batch, int seq_len, int h, int h_kv, int dh, const uint16_t* cos,
+                                         const uint16_t* sin, int pos, const int32_t* pos_dev, uint16_t* q_out,
+                                         uint16_t* kcache, uint16_t* vcache, int t_max, void* stream);
+int ohara_bitlinear_gate_up_bf16(const uint16_t* x, int ldx, const uint16_t* pre_norm_w, float eps, int k, int f,
+                                 const uint16_t* gate_norm_w, const uint32_t* gate_wp, float gate_gamma,
+                                 const uint16_t* up_norm_w, const uint32_t* up_wp, float up_gamma, int rows,
+                                 uint16_t* out, int ldo, void* stream);
+
 /* out = bf16(bf16(silu(gate)) * up), elementwise over n values (ohara/modules/mlp.py:152). */
 int ohara_silu_mul_bf16(const uint16_t* gate, const uint16_t* up, uint16_t* out, int64_t n, void* stream);
 

@@ -64,6 +64,9 @@ _PROTOS = {
     "ohara_act_quant_int8": (_i, [_p, _i, _p, _f, _i, _i, _p, _i, _p, _p, _p]),
     "ohara_gemv_ternary_i8": (_i, [_p, _i, _p, _p, _p, _i, _i, _f, _i, _p, _i, _p, _i, _p, _i, _p]),
     "ohara_bitlinear_bf16": (_i, [_p, _i, _p, _p, _f, _p, _i, _i, _f, _i, _p, _i, _p, _i, _p, _i, _p]),
+    "ohara_bitlinear_qkv_rope_append_bf16": (_i, [_p, _i, _p, _f, _i, _p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _i, _p, _p, _p,
+                                                  _p, _i, _p]),
+    "ohara_bitlinear_gate_up_bf16": (_i, [_p, _i, _p, _f, _i, _i, _p, _p, _f, _p, _p, _f, _i, _p, _i, _p]),
     "ohara_silu_mul_bf16": (_i, [_p, _p, _p, _i64, _p]),
     "ohara_rope_append_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _p, _p, _i, _p, _p, _p, _i, _p]),
     "ohara_moe_route_topk": (_i, [_p, _i, _p, _i, _i, _i, _i, _i, _i, _p, _p, _p]),

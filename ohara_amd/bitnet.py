@@ -119,15 +119,25 @@ class BitLlama:
         h = ops.embed(x.to(self.device), self.token_emb)
         for L, cache in zip(self.layers, kv_cache):
             # the block norm (norm1 / norm2) is applied inside each projection's quantisation pass
-            q = ops.bitlinear(h, L["attn.query"][1], L["attn.query"][0], self.eps, pre_norm_w=L["norm1"])
-            k = ops.bitlinear(h, L["attn.key"][1], L["attn.key"][0], self.eps, pre_norm_w=L["norm1"])
-            v = ops.bitlinear(h, L["attn.value"][1], L["attn.value"][0], self.eps, pre_norm_w=L["norm1"])
-            ops.rope_append(q, k, v, B, S, H, Hkv, D, self.cos, self.sin, start, cache.key, cache.value)
+            if rows <= 64:  # decode: one launch for q/k/v + rotary + append, one for gate/up + SwiGLU
+                q = ops.bitlinear_qkv_rope_append(
+                    h, L["norm1"], [(L[n][1], L[n][0]) for n in ("attn.query", "attn.key", "attn.value")], self.eps,
+                    H, Hkv, D, self.cos, self.sin, start, cache.key, cache.value, seq_len=S)
+            else:
+                q = ops.bitlinear(h, L["attn.query"][1], L["attn.query"][0], self.eps, pre_norm_w=L["norm1"])
+                k = ops.bitlinear(h, L["attn.key"][1], L["attn.key"][0], self.eps, pre_norm_w=L["norm1"])
+                v = ops.bitlinear(h, L["attn.value"][1], L["attn.value"][0], self.eps, pre_norm_w=L["norm1"])
+                ops.rope_append(q, k, v, B, S, H, Hkv, D, self.cos, self.sin, start, cache.key, cache.value)
             att = ops.attn_auto(q, cache.key, cache.value, H, Hkv, D, start, n_split, ws, S)
             h = ops.bitlinear(att, L["attn.proj"][1], L["attn.proj"][0], self.eps, residual=h)
-            g = ops.bitlinear(h, L["ff.gate"][1], L["ff.gate"][0], self.eps, pre_norm_w=L["norm2"])
-            u = ops.bitlinear(h, L["ff.up"][1], L["ff.up"][0], self.eps, pre_norm_w=L["norm2"])
-            h = ops.bitlinear(ops.silu_mul(g, u), L["ff.down"][1], L["ff.down"][0], self.eps, residual=h)
+            if rows <= 64:
+                act = ops.bitlinear_gate_up(h, L["norm2"], (L["ff.gate"][1], L["ff.gate"][0]),
+                                            (L["ff.up"][1], L["ff.up"][0]), self.eps)
+            else:
+                g = ops.bitlinear(h, L["ff.gate"][1], L["ff.gate"][0], self.eps, pre_norm_w=L["norm2"])
+                u = ops.bitlinear(h, L["ff.up"][1], L["ff.up"][0], self.eps, pre_norm_w=L["norm2"])
+                act = ops.silu_mul(g, u)
+            h = ops.bitlinear(act, L["ff.down"][1], L["ff.down"][0], self.eps, residual=h)
         if last_only:
             h = h.view(B, S, -1)[:, -1].contiguous()
         logits = ops.gemm_skinny(h, self.w_vocab, norm_w=self.final_norm, eps=self.eps)

@@ -319,6 +319,37 @@ def bitlinear(x, norm_w, w: PackedTernary, eps=1e-5, residual=None, out=None, wa
     return (out, acc) if want_acc else out
 
 
+def bitlinear_qkv_rope_append(x, pre_norm_w, projs, eps, h, h_kv, dh, cos, sin, pos, kcache, vcache, q_out=None,
+                              pos_dev=None, seq_len=1):
+    """The query / key / value BitLinears of one layer on rows of x (rows <= 64) in one launch, with
+    rotary + cache append.  ``projs``: three (norm_w, PackedTernary) pairs.  Returns q (rows, h*dh)."""
+    _need(x, BF16, "x")
+    rows, k = x.shape
+    if q_out is None:
+        q_out = torch.empty(rows, h * dh, dtype=BF16, device=x.device)
+    nw = (C.c_void_p * 3)(*[p[0].data_ptr() for p in projs])
+    wp = (C.c_void_p * 3)(*[p[1].data.data_ptr() for p in projs])
+    gm = (C.c_float * 3)(*[p[1].gamma for p in projs])
+    check(lib().ohara_bitlinear_qkv_rope_append_bf16(
+        _ptr(x), x.stride(0), _ptr(pre_norm_w), eps, k, nw, wp, gm, rows // seq_len, seq_len, h, h_kv, dh, _ptr(cos),
+        _ptr(sin), int(pos), _ptr(pos_dev), _ptr(q_out), _ptr(kcache), _ptr(vcache), kcache.shape[1], _stream()),
+        "bitlinear_qkv_rope_append")
+    return q_out
+
+
+def bitlinear_gate_up(x, pre_norm_w, gate, up, eps=1e-5, out=None):
+    """silu(gate(x)) * up(x) for two BitLinears ((norm_w, PackedTernary) pairs) on rows of x (<= 64)."""
+    _need(x, BF16, "x")
+    rows, k = x.shape
+    f = gate[1].n
+    if out is None:
+        out = torch.empty(rows, f, dtype=BF16, device=x.device)
+    check(lib().ohara_bitlinear_gate_up_bf16(
+        _ptr(x), x.stride(0), _ptr(pre_norm_w), eps, k, f, _ptr(gate[0]), _ptr(gate[1].data), gate[1].gamma,
+        _ptr(up[0]), _ptr(up[1].data), up[1].gamma, rows, _ptr(out), out.stride(0), _stream()), "bitlinear_gate_up")
+    return out
+
+
 def silu_mul(gate, up, out=None):
     _need(gate, BF16, "gate")
     _need(up, BF16, "up")

@@ -151,3 +151,35 @@ def test_bitnet_llama_parity(cuda):
     assert cache[0].length == 12
     toks = model.generate_greedy(ids.to(cuda), 6).cpu()
     assert toks.shape == (2, 6)
+
+
+def test_fused_groups_match_the_separate_calls(cuda):
+    """One launch for q/k/v + rotary + append and one for gate/up + SwiGLU: the same arithmetic as
+    the separate BitLinear, rope_append and silu_mul calls, so bit-identical results."""
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(21)
+    B, S, H, Hkv, D, K, F, Tmax, pos = 3, 2, 4, 2, 64, 256, 384, 16, 5
+    rows = B * S
+    x = (torch.randn(rows, K, generator=g) * 2).to(BF).to(cuda)
+    pre = (1 + 0.2 * torch.randn(K, generator=g)).to(BF).to(cuda)
+
+    def proj(n):
+        t = torch.randint(-1, 2, (n, K), generator=g, dtype=torch.int8)
+        return (1 + 0.1 * torch.randn(K, generator=g)).to(BF).to(cuda), ops.pack_ternary(t.to(cuda), 0.03 + 0.01 * n / 256)
+
+    pq, pk, pv, pg, pu = proj(H * D), proj(Hkv * D), proj(Hkv * D), proj(F), proj(F)
+    cos, sin = R.rope_table(D, 2 * Tmax, 10000.0)
+    cos, sin = cos.to(BF).to(cuda), sin.to(BF).to(cuda)
+    kc1 = torch.zeros(B, Tmax, Hkv, D, dtype=BF, device=cuda)
+    vc1, kc2, vc2 = torch.zeros_like(kc1), torch.zeros_like(kc1), torch.zeros_like(kc1)
+    q1 = ops.bitlinear(x, pq[0], pq[1], pre_norm_w=pre)
+    k1 = ops.bitlinear(x, pk[0], pk[1], pre_norm_w=pre)
+    v1 = ops.bitlinear(x, pv[0], pv[1], pre_norm_w=pre)
+    ops.rope_append(q1, k1, v1, B, S, H, Hkv, D, cos, sin, pos, kc1, vc1)
+    q2 = ops.bitlinear_qkv_rope_append(x, pre, [pq, pk, pv], 1e-5, H, Hkv, D, cos, sin, pos, kc2, vc2, seq_len=S)
+    assert torch.equal(q1, q2) and torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+    assert kc2[:, pos : pos + S].abs().sum().item() > 0 and kc2[:, :pos].abs().sum().item() == 0
+    a1 = ops.silu_mul(ops.bitlinear(x, pg[0], pg[1], pre_norm_w=pre), ops.bitlinear(x, pu[0], pu[1], pre_norm_w=pre))
+    a2 = ops.bitlinear_gate_up(x, pre, pg, pu)
+    assert torch.equal(a1, a2)
