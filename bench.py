@@ -184,6 +184,7 @@ def bench_attention_microbench(dev):
     """GQA decode attention, 32 query / 8 KV heads x 128, one query per sequence over L cached
     positions.  Algorithmic bytes: K + V (4*Hkv*D*B*L) + Q and O (4*H*D*B)."""
     from ohara_amd import ops
+    from ohara_amd.llama import KVCache
 
     H, Hkv, D = 32, 8, 128
     out = []
@@ -197,9 +198,19 @@ def bench_attention_microbench(dev):
         o = torch.empty(B, H * D, device=dev, dtype=torch.bfloat16)
         t = graph_time(lambda: ops.attn_decode(q, k, v, H, Hkv, D, L, ns, ws, o))
         by = 4.0 * Hkv * D * B * L + 4.0 * H * D * B
-        out.append({"batch": B, "context": L, "n_split": ns, "us": round(t * 1e6, 1), "GBs": round(by / t / 1e9, 1),
-                    "frac_of_hbm_peak": round(by / t / 1e9 / HBM_PEAK_GBS, 4)})
-        del q, k, v, ws, o
+        row = {"batch": B, "context": L, "n_split": ns, "us": round(t * 1e6, 1), "GBs": round(by / t / 1e9, 1),
+               "frac_of_hbm_peak": round(by / t / 1e9 / HBM_PEAK_GBS, 4)}
+        # the same rows through the int8 cache: codes (1 byte) + an fp32 scale and minimum per row
+        cache = KVCache((B, L, Hkv, D), L, device=dev, dtype=torch.bfloat16, int8=True)
+        step = max(1, 4096 // B)
+        for p0 in range(0, L, step):
+            ops.kv_quant_append(k[:, p0:p0 + step].contiguous(), v[:, p0:p0 + step].contiguous(), cache, p0)
+        t8 = graph_time(lambda: ops.attn_cached_int8(q, cache, H, Hkv, D, L - 1, ns, ws, o))
+        by8 = 2.0 * Hkv * (D + 8) * B * L + 4.0 * H * D * B
+        row["int8_cache"] = {"us": round(t8 * 1e6, 1), "GBs": round(by8 / t8 / 1e9, 1),
+                             "frac_of_hbm_peak": round(by8 / t8 / 1e9 / HBM_PEAK_GBS, 4)}
+        out.append(row)
+        del q, k, v, ws, o, cache
         torch.cuda.empty_cache()
     return out
 

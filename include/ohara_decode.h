@@ -107,6 +107,14 @@ int ohara_qkv_rope_append_bf16(const uint16_t* x, int ldx, const uint16_t* wp, i
                                const uint16_t* sin, int pos, const int32_t* pos_dev, uint16_t* q_out,
                                uint16_t* kcache, uint16_t* vcache, int t_max, void* stream);
 
+/* The same projection + rotary, with the rotated k and the v rows written to (batch*seq_len,
+ * h_kv*dh) buffers instead of into a cache (the int8 cache quantises them in a second step).
+ * t_max only bounds the positions. */
+int ohara_qkv_rope_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int k, const uint16_t* norm_w, float eps,
+                        int batch, int seq_len, int h, int h_kv, int dh, const uint16_t* cos, const uint16_t* sin,
+                        int pos, const int32_t* pos_dev, int t_max, uint16_t* q_out, uint16_t* k_out, uint16_t* v_out,
+                        void* stream);
+
 /* ---- attention over the KV cache ------------------------------------------------
  * Query s (0 <= s < seq_len) of sequence b sits at cache position pos + s and sees
  * positions [0, pos + s] (the cache mask key_pos <= start_pos + q_idx, llama.py:109-113):
@@ -130,6 +138,29 @@ int ohara_attn_cached_bf16(const uint16_t* q, const uint16_t* kcache, const uint
  * Needs no workspace.  (llama.py:100-135 with S > 1.) */
 int ohara_attn_prefill_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch,
                             int seq_len, int h, int h_kv, int dh, int t_max, int pos, uint16_t* out, void* stream);
+
+/* ---- int8 KV cache (ohara/modules/kv_cache.py:15-32, 67-73, 94-102, 116-118) ------------------
+ * Every (sequence, position, head) row of dh values is stored as int8 with an fp32 scale and
+ * minimum: scale = max((max - min) / 255, 1e-8), q = clamp(round((x - min) / scale - 128), -128,
+ * 127), read back as bf16((q + 128) * scale + min).  The quantisation arithmetic is rounded to
+ * bf16 after every operation, as the reference's tensor ops on a bf16 cache are, so codes, scales
+ * and minima are bit-identical to it.  Caches: (batch_cap, t_max, h_kv, dh) int8; statistics:
+ * (batch_cap, t_max, h_kv) fp32.
+ *   ohara_kv_quant_append_int8  quantises k / v rows (batch*seq_len, h_kv*dh) into positions
+ *                               pos + s (pos_dev as elsewhere);
+ *   ohara_kv_dequant_int8       the first `len` positions of one cache tensor as bf16
+ *                               (batch, len, h_kv, dh) - what KVCache._read returns;
+ *   ohara_attn_cached_int8      ohara_attn_cached_bf16 over the quantised cache, dequantising in
+ *                               registers (dh 64 or 128, 1 / 2 / 4 query heads per KV head). */
+int ohara_kv_quant_append_int8(const uint16_t* k, const uint16_t* v, int batch, int seq_len, int h_kv, int dh, int pos,
+                               const int32_t* pos_dev, int8_t* kq, int8_t* vq, float* kscale, float* kmin, float* vscale,
+                               float* vmin, int t_max, void* stream);
+int ohara_kv_dequant_int8(const int8_t* q, const float* scale, const float* mn, int batch, int len, int h_kv, int dh,
+                          int t_max, uint16_t* out, void* stream);
+int ohara_attn_cached_int8(const uint16_t* q, const int8_t* kcache, const int8_t* vcache, const float* kscale,
+                           const float* kmin, const float* vscale, const float* vmin, int batch, int seq_len, int h,
+                           int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev, int n_split, void* workspace,
+                           uint16_t* out, void* stream);
 
 /* ---- greedy selection ---------------------------------------------------------
  * next_ids[b] = first index of max(logits[b, 0:valid_vocab])  (argmax of the last
@@ -295,6 +326,19 @@ typedef struct OharaDecodeState {
   int64_t* history;      /* (hist_cap, batch) generated ids, may be NULL                  */
   uint16_t* const* kcache; /* host array [n_layers] of (batch_cap, t_max, h_kv, dh)       */
   uint16_t* const* vcache;
+  /* int8 cache mode (kv_int8 != 0): kcache / vcache point at int8 tensors of the same shape, the
+     four arrays below at the per-layer (batch_cap, t_max, h_kv) fp32 statistics; kstage / vstage
+     (rows, h_kv*dh) receive the bf16 rows before they are quantised; kdeq / vdeq ((batch, t_max,
+     h_kv, dh) bf16, may be NULL) hold the dequantised cache for calls with >= 16 positions. */
+  int32_t kv_int8;
+  float* const* kscale;
+  float* const* kmin;
+  float* const* vscale;
+  float* const* vmin;
+  uint16_t* kstage;
+  uint16_t* vstage;
+  uint16_t* kdeq;
+  uint16_t* vdeq;
   void* prof_start;      /* hipEvent_t recorded on `stream` right before launch prof_kernel */
   void* prof_stop;       /* hipEvent_t recorded right after it                             */
 } OharaDecodeState;

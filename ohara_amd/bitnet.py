@@ -108,6 +108,8 @@ class BitLlama:
             raise ValueError("input exceeds max_sequence_length")
         if kv_cache is None:
             kv_cache = self.build_kv_cache(B)
+        if any(cc.int8 for cc in kv_cache):
+            raise NotImplementedError("ohara_amd: int8 KV caches are served by the dense Llama only")
         ends = [cc._reserve(B, S, start) for cc in kv_cache]
         H, Hkv, D = c.num_attention_heads, self.kv_heads, self.head_dim
         rows = B * S

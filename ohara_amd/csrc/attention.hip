@@ -16,8 +16,12 @@ namespace {
 
 struct AttnArgs {
   const bf16_t* q;   // (B, H*D)
-  const bf16_t* k;   // (Bcap, Tmax, Hkv, D)
+  const bf16_t* k;   // (Bcap, Tmax, Hkv, D); int8 mode: the same shape in int8
   const bf16_t* v;
+  const float* kscale;  // int8 mode (ohara/modules/kv_cache.py:67-73): (Bcap, Tmax, Hkv) scale / minimum
+  const float* kmin;
+  const float* vscale;
+  const float* vmin;
   bf16_t* out;       // (B, H*D)
   int B, S, H, Hkv, D, Tmax, start;  // query s of sequence b sees positions [0, start + s]
   const int32_t* pos_dev;            // when set: start = *pos_dev
@@ -111,7 +115,17 @@ __device__ bool last_chunk_done(int* counter, int nsplit) {
   return is_last != 0;
 }
 
-template <int D, int G>
+// (q + 128) * scale + min in fp32, rounded to bf16 (kv_cache.py:30-32, 116-118): four bytes -> two
+// packed bf16 pairs.  `w` already has 0x80 xor-ed in, i.e. holds q + 128 as unsigned bytes.
+__device__ __forceinline__ uint2 dequant4(uint32_t w, float s, float m) {
+  const float f0 = __fadd_rn(__fmul_rn((float)(w & 0xffu), s), m);
+  const float f1 = __fadd_rn(__fmul_rn((float)((w >> 8) & 0xffu), s), m);
+  const float f2 = __fadd_rn(__fmul_rn((float)((w >> 16) & 0xffu), s), m);
+  const float f3 = __fadd_rn(__fmul_rn((float)(w >> 24), s), m);
+  return make_uint2(pack_bf(f0, f1), pack_bf(f2, f3));
+}
+
+template <int D, int G, bool I8>
 __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   constexpr int NC = D / 32;        // 16-byte K loads per lane per tile
   constexpr int DC = D / 8;         // lanes covering one V row with 16-byte loads
@@ -130,13 +144,13 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   __shared__ float s_m[4][G], s_l[4][G];
   __shared__ float s_acc[4][G][D];
 
-  // q for this lane's quarter-row: columns (4c + dq)*8 .. +7
+  // q for this lane's quarter-row: columns (4c + dq)*8 .. +7 (int8 mode: the contiguous quarter dq)
   uint4 qv[G][NC];
 #pragma unroll
   for (int hh = 0; hh < G; ++hh)
 #pragma unroll
     for (int c = 0; c < NC; ++c)
-      qv[hh][c] = ldg16(a.q + (size_t)b * a.H * D + (size_t)(kvh * G + hh) * D + (4 * c + dq) * 8);
+      qv[hh][c] = ldg16(a.q + (size_t)b * a.H * D + (size_t)(kvh * G + hh) * D + (I8 ? (dq * NC + c) : (4 * c + dq)) * 8);
 
   float m_run[G], l_run[G], acc[G][8];
 #pragma unroll
@@ -153,24 +167,85 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
 
   // 16-position tiles, wave w takes tiles w, w+4, ...; the loads of the next tile are in
   // flight while the current one is consumed
-  auto load_tile = [&](int tb, uint4* kv, uint4* vv) {
+  // A tile in the form it is fetched in.  bf16: the MFMA-free dot operands themselves.  int8: the
+  // raw bytes of this lane's quarter of the K row / eighth of the V rows plus the rows' scale and
+  // minimum; they are expanded to bf16 right before use, so the fetch of the next tile stays
+  // asynchronous.
+  struct Tile {
+    uint4 k[I8 ? (NC + 1) / 2 : NC];
+    uint4 v[I8 ? (NV + 1) / 2 : NV];
+    float ks, km, vs[NV], vm[NV];
+  };
+  const int8_t* kb8 = reinterpret_cast<const int8_t*>(a.k) + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
+  const int8_t* vb8 = reinterpret_cast<const int8_t*>(a.v) + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
+  auto load_tile = [&](int tb, Tile& t) {
     const int pos = tb + p;
+    if (I8) {
+      const size_t slot = ((size_t)seq * a.Tmax + pos) * a.Hkv + kvh;
+      const bool in = pos < t1;
+      t.ks = in ? a.kscale[slot] : 0.f;
+      t.km = in ? a.kmin[slot] : 0.f;
 #pragma unroll
-    for (int c = 0; c < NC; ++c)
-      kv[c] = pos < t1 ? ldg16_nt(kb + (size_t)pos * row + (4 * c + dq) * 8) : make_uint4(0, 0, 0, 0);
+      for (int c = 0; c < (NC + 1) / 2; ++c) {
+        if (NC >= 2) t.k[c] = in ? ldg16_nt(kb8 + (size_t)pos * row + dq * (NC * 8) + 16 * c) : make_uint4(0, 0, 0, 0);
+        else {
+          const uint2 w = in ? *reinterpret_cast<const uint2*>(kb8 + (size_t)pos * row + dq * 8) : make_uint2(0, 0);
+          t.k[c] = make_uint4(w.x, w.y, 0, 0);
+        }
+      }
 #pragma unroll
-    for (int c = 0; c < NV; ++c) {
-      const int vp = tb + c * PP + pp;
-      vv[c] = vp < t1 ? ldg16_nt(vb + (size_t)vp * row + dc * 8) : make_uint4(0, 0, 0, 0);
+      for (int c = 0; c < NV; ++c) {
+        const int vp = tb + c * PP + pp;
+        const bool vin = vp < t1;
+        const size_t vslot = ((size_t)seq * a.Tmax + vp) * a.Hkv + kvh;
+        t.vs[c] = vin ? a.vscale[vslot] : 0.f;
+        t.vm[c] = vin ? a.vmin[vslot] : 0.f;
+        const uint2 w = vin ? *reinterpret_cast<const uint2*>(vb8 + (size_t)vp * row + dc * 8) : make_uint2(0x80808080u, 0x80808080u);
+        uint32_t* dstw = reinterpret_cast<uint32_t*>(&t.v[c >> 1]) + 2 * (c & 1);
+        dstw[0] = w.x;
+        dstw[1] = w.y;
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < NC; ++c)
+        t.k[c] = pos < t1 ? ldg16_nt(kb + (size_t)pos * row + (4 * c + dq) * 8) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int c = 0; c < NV; ++c) {
+        const int vp = tb + c * PP + pp;
+        t.v[c] = vp < t1 ? ldg16_nt(vb + (size_t)vp * row + dc * 8) : make_uint4(0, 0, 0, 0);
+      }
     }
   };
-  uint4 kv[NC], vv[NV], kn[NC], vn[NV];
+  auto expand = [&](const Tile& t, uint4* kv, uint4* vv) {
+    if (I8) {
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const uint32_t* w = reinterpret_cast<const uint32_t*>(&t.k[c >> 1]) + 2 * (c & 1);
+        const uint2 lo = dequant4(w[0] ^ 0x80808080u, t.ks, t.km), hi = dequant4(w[1] ^ 0x80808080u, t.ks, t.km);
+        kv[c] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      }
+#pragma unroll
+      for (int c = 0; c < NV; ++c) {
+        const uint32_t* w = reinterpret_cast<const uint32_t*>(&t.v[c >> 1]) + 2 * (c & 1);
+        const uint2 lo = dequant4(w[0] ^ 0x80808080u, t.vs[c], t.vm[c]), hi = dequant4(w[1] ^ 0x80808080u, t.vs[c], t.vm[c]);
+        vv[c] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < NC; ++c) kv[c] = t.k[c];
+#pragma unroll
+      for (int c = 0; c < NV; ++c) vv[c] = t.v[c];
+    }
+  };
+  Tile cur, nxt;
   int tb = t0 + wave * 16;
-  if (tb < t1) load_tile(tb, kv, vv);
+  if (tb < t1) load_tile(tb, cur);
   for (; tb < t1; tb += 64) {
     const bool valid = tb + p < t1;
     const bool more = tb + 64 < t1;
-    if (more) load_tile(tb + 64, kn, vn);
+    if (more) load_tile(tb + 64, nxt);
+    uint4 kv[NC], vv[NV];
+    expand(cur, kv, vv);
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) {
       float s = 0.f;
@@ -203,12 +278,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
         }
       }
     }
-    if (more) {
-#pragma unroll
-      for (int c = 0; c < NC; ++c) kv[c] = kn[c];
-#pragma unroll
-      for (int c = 0; c < NV; ++c) vv[c] = vn[c];
-    }
+    if (more) cur = nxt;
   }
 
   // fold the PP row-groups of the wave, then the four waves
@@ -260,6 +330,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
 
 // Any even head width up to 256, any group size: one thread per position for q.k,
 // one thread per column for p.V.  Slow path for shapes the tuned kernel skips.
+template <bool I8>
 __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
   const int split = blockIdx.z, kvh = blockIdx.y, b = blockIdx.x;
   const int seq = b / a.S;
@@ -275,6 +346,13 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
   const size_t row = (size_t)a.Hkv * D;
   const bf16_t* kb = a.k + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
   const bf16_t* vb = a.v + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
+  // int8 mode: element (pos, d) is code * scale + min of its (pos, head) row, rounded to bf16
+  const int8_t* kb8 = reinterpret_cast<const int8_t*>(a.k) + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
+  const int8_t* vb8 = reinterpret_cast<const int8_t*>(a.v) + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
+  const size_t st0 = (size_t)seq * a.Tmax * a.Hkv + kvh;
+  auto deq = [](int8_t c, float sc, float mn) {
+    return bf2f(f2bf(__fadd_rn(__fmul_rn((float)((int)c + 128), sc), mn)));
+  };
   for (int hh = 0; hh < G; ++hh) {
     const int h = kvh * G + hh;
     __syncthreads();
@@ -286,7 +364,12 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
       float s = -INFINITY;
       if (pos < t1) {
         float d_ = 0.f;
-        for (int d = 0; d < D; ++d) d_ += s_q[d] * bf2f(kb[(size_t)pos * row + d]);
+        if (I8) {
+          const float sc = a.kscale[st0 + (size_t)pos * a.Hkv], mn = a.kmin[st0 + (size_t)pos * a.Hkv];
+          for (int d = 0; d < D; ++d) d_ += s_q[d] * deq(kb8[(size_t)pos * row + d], sc, mn);
+        } else {
+          for (int d = 0; d < D; ++d) d_ += s_q[d] * bf2f(kb[(size_t)pos * row + d]);
+        }
         s = d_ * a.scale;
       }
       float tm = wave_max(s);
@@ -307,7 +390,14 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
       acc *= corr;
       if (tid < D) {
         const int n = min(256, t1 - tb);
-        for (int i = 0; i < n; ++i) acc += s_p[i] * bf2f(vb[(size_t)(tb + i) * row + tid]);
+        if (I8) {
+          for (int i = 0; i < n; ++i) {
+            const size_t si = st0 + (size_t)(tb + i) * a.Hkv;
+            acc += s_p[i] * deq(vb8[(size_t)(tb + i) * row + tid], a.vscale[si], a.vmin[si]);
+          }
+        } else {
+          for (int i = 0; i < n; ++i) acc += s_p[i] * bf2f(vb[(size_t)(tb + i) * row + tid]);
+        }
       }
       __syncthreads();
     }
@@ -326,12 +416,12 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
   if (last_chunk_done(a.counters + b * a.Hkv + kvh, a.nsplit)) merge_partials<256>(a, b, kvh, G);
 }
 
-template <int D>
+template <int D, bool I8>
 int launch_fast(const AttnArgs& a, int G, dim3 grid, hipStream_t st) {
   switch (G) {
-    case 1: hipLaunchKernelGGL((attn_decode_kernel<D, 1>), grid, dim3(256), 0, st, a); break;
-    case 2: hipLaunchKernelGGL((attn_decode_kernel<D, 2>), grid, dim3(256), 0, st, a); break;
-    case 4: hipLaunchKernelGGL((attn_decode_kernel<D, 4>), grid, dim3(256), 0, st, a); break;
+    case 1: hipLaunchKernelGGL((attn_decode_kernel<D, 1, I8>), grid, dim3(256), 0, st, a); break;
+    case 2: hipLaunchKernelGGL((attn_decode_kernel<D, 2, I8>), grid, dim3(256), 0, st, a); break;
+    case 4: hipLaunchKernelGGL((attn_decode_kernel<D, 4, I8>), grid, dim3(256), 0, st, a); break;
     default: return 1;
   }
   return 0;
@@ -351,10 +441,12 @@ int64_t ohara_attn_workspace_bytes(int batch, int h, int h_kv, int dh, int n_spl
   return (int64_t)(c + ml + acc);
 }
 
-int ohara_attn_cached_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch,
-                           int seq_len, int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev,
-                           int n_split, void* workspace, uint16_t* out, void* stream) {
+static int attn_cached_impl(const uint16_t* q, const void* kcache, const void* vcache, const float* kscale,
+                            const float* kmin, const float* vscale, const float* vmin, bool i8, int batch, int seq_len,
+                            int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev, int n_split,
+                            void* workspace, uint16_t* out, void* stream) {
   if (!q || !kcache || !vcache || !out) return OHARA_EINVAL;
+  if (i8 && (!kscale || !kmin || !vscale || !vmin)) return OHARA_EINVAL;
   if (batch < 1 || seq_len < 1 || h < 1 || h_kv < 1 || h % h_kv || dh < 2 || (dh & 1) || dh > 256)
     return OHARA_EINVAL;
   if (t_max < 1 || n_split < 1 || n_split > 1024) return OHARA_EINVAL;
@@ -363,7 +455,8 @@ int ohara_attn_cached_bf16(const uint16_t* q, const uint16_t* kcache, const uint
   if (!pos_dev && (pos < 0 || pos + seq_len > t_max)) return OHARA_EINVAL;
   if ((int64_t)batch * seq_len > INT32_MAX / 2 || h_kv > 65535) return OHARA_ESIZE;
   AttnArgs a{};
-  a.q = q; a.k = kcache; a.v = vcache; a.out = out;
+  a.q = q; a.k = reinterpret_cast<const bf16_t*>(kcache); a.v = reinterpret_cast<const bf16_t*>(vcache); a.out = out;
+  a.kscale = kscale; a.kmin = kmin; a.vscale = vscale; a.vmin = vmin;
   a.B = batch; a.S = seq_len; a.H = h; a.Hkv = h_kv; a.D = dh; a.Tmax = t_max; a.start = pos; a.pos_dev = pos_dev;
   a.nsplit = n_split;
   batch *= seq_len;  // one workspace slot per query row
@@ -378,10 +471,31 @@ int ohara_attn_cached_bf16(const uint16_t* q, const uint16_t* kcache, const uint
   hipStream_t st = (hipStream_t)stream;
   const int G = h / h_kv;
   int miss = 1;
-  if (dh == 128) miss = launch_fast<128>(a, G, grid, st);
-  else if (dh == 64) miss = launch_fast<64>(a, G, grid, st);
-  if (miss) hipLaunchKernelGGL(attn_decode_generic, grid, dim3(256), 0, st, a);
+  if (i8) {
+    if (dh == 128) miss = launch_fast<128, true>(a, G, grid, st);
+    else if (dh == 64) miss = launch_fast<64, true>(a, G, grid, st);
+    if (miss) hipLaunchKernelGGL(attn_decode_generic<true>, grid, dim3(256), 0, st, a);
+    return ohara_launch_status();
+  }
+  if (dh == 128) miss = launch_fast<128, false>(a, G, grid, st);
+  else if (dh == 64) miss = launch_fast<64, false>(a, G, grid, st);
+  if (miss) hipLaunchKernelGGL(attn_decode_generic<false>, grid, dim3(256), 0, st, a);
   return ohara_launch_status();
+}
+
+int ohara_attn_cached_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch,
+                           int seq_len, int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev,
+                           int n_split, void* workspace, uint16_t* out, void* stream) {
+  return attn_cached_impl(q, kcache, vcache, nullptr, nullptr, nullptr, nullptr, false, batch, seq_len, h, h_kv, dh,
+                          t_max, pos, pos_dev, n_split, workspace, out, stream);
+}
+
+int ohara_attn_cached_int8(const uint16_t* q, const int8_t* kcache, const int8_t* vcache, const float* kscale,
+                           const float* kmin, const float* vscale, const float* vmin, int batch, int seq_len, int h,
+                           int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev, int n_split, void* workspace,
+                           uint16_t* out, void* stream) {
+  return attn_cached_impl(q, kcache, vcache, kscale, kmin, vscale, vmin, true, batch, seq_len, h, h_kv, dh, t_max, pos,
+                          pos_dev, n_split, workspace, out, stream);
 }
 
 }  // extern "C"

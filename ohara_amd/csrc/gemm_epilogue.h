@@ -28,6 +28,7 @@ struct GemmArgs {
   const bf16_t* sin;
   bf16_t* kcache;
   bf16_t* vcache;
+  int stage;  // rotary epilogue: k / v rows go to (rows, Hkv*Dh) buffers at the row index instead of into a cache
 };
 
 // gemm_tile.hip: the tiled kernel for calls with many rows (a.B rows, no fused norm).
@@ -96,10 +97,12 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, int b, int stri
       if (r0 < nq) {
         o = a.out + (size_t)grow * a.ldo + r0;
       } else {
-        o = a.kcache + (((size_t)seq * a.Tmax + pos) * a.Hkv) * a.Dh + (r0 - nq);
+        o = a.stage ? a.kcache + (size_t)grow * nk + (r0 - nq)
+                    : a.kcache + (((size_t)seq * a.Tmax + pos) * a.Hkv) * a.Dh + (r0 - nq);
       }
     } else {
-      o = a.vcache + (((size_t)seq * a.Tmax + pos) * a.Hkv) * a.Dh + (r0 - nq - nk);
+      o = a.stage ? a.vcache + (size_t)grow * nk + (r0 - nq - nk)
+                  : a.vcache + (((size_t)seq * a.Tmax + pos) * a.Hkv) * a.Dh + (r0 - nq - nk);
     }
     *reinterpret_cast<uint2*>(o) = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
   }

@@ -80,16 +80,22 @@ class KVCache:
     fused projection kernel and only does the bookkeeping here (``_reserve``)."""
 
     def __init__(self, shape, max_seq_length, idx=None, device=None, dtype=None, int8=False):
-        if int8:
-            raise NotImplementedError("ohara_amd: the int8 KV cache mode is not implemented")
         self.idx = idx
-        self.int8 = False
+        self.int8 = bool(int8)
         self.max_seq_length = max_seq_length
         self.length = 0
         self.batch_size = None
         self.dtype = dtype
-        self.key = torch.zeros(shape, device=device, dtype=dtype)
-        self.value = torch.zeros(shape, device=device, dtype=dtype)
+        storage = torch.int8 if self.int8 else dtype
+        self.key = torch.zeros(shape, device=device, dtype=storage)
+        self.value = torch.zeros(shape, device=device, dtype=storage)
+        if self.int8:
+            # one scale / minimum per quantised row, i.e. per (batch, position, head): kv_cache.py:67-73
+            stats = (*shape[:-1], 1)
+            self.key_scale = torch.zeros(stats, device=device, dtype=torch.float32)
+            self.key_min = torch.zeros(stats, device=device, dtype=torch.float32)
+            self.value_scale = torch.zeros(stats, device=device, dtype=torch.float32)
+            self.value_min = torch.zeros(stats, device=device, dtype=torch.float32)
 
     def _reserve(self, bsz: int, seq_len: int, start_pos: int) -> int:
         # ohara/modules/kv_cache.py:80-90, same order
@@ -114,6 +120,13 @@ class KVCache:
         if values.shape != keys.shape:
             raise ValueError("KV cache keys and values must have matching shapes")
         end = self._reserve(bsz, seq_len, start_pos)
+        if self.int8:
+            # kv_cache.py:94-102 and :116-118: quantise on write, hand back dequantised values
+            if keys.dtype != BF16:
+                raise ValueError("ohara_amd: the int8 KV cache quantises bfloat16 keys and values")
+            ops.kv_quant_append(keys.contiguous(), values.contiguous(), self, start_pos)
+            self._commit(bsz, end)
+            return ops.kv_dequant(self, "key", bsz, end), ops.kv_dequant(self, "value", bsz, end)
         self.key[:bsz, start_pos:end] = keys
         self.value[:bsz, start_pos:end] = values
         self._commit(bsz, end)
@@ -145,6 +158,7 @@ class _Buffers:
         self.step_state = torch.zeros(4, dtype=torch.int32, device=dev)
         self.logits = None
         self.history = None
+        self.kstage = self.vstage = self.kdeq = self.vdeq = None  # int8 cache mode only
 
 
 class Llama:
@@ -232,13 +246,15 @@ class Llama:
             yield L["norm1"]
             yield L["norm2"]
 
-    def build_kv_cache(self, batch_size: int = 1) -> list[KVCache]:
-        """ohara/models/llama.py:325-348."""
+    def build_kv_cache(self, batch_size: int = 1, int8: bool = False) -> list[KVCache]:
+        """ohara/models/llama.py:325-348; ``int8=True`` builds the int8 caches of
+        ohara/modules/kv_cache.py:47-73 (the reference leaves that choice to whoever constructs the
+        caches)."""
         if batch_size < 1:
             raise ValueError("batch_size must be at least 1")
         c = self.config
         shape = (batch_size, c.max_sequence_length, self.kv_heads, self.head_dim)
-        return [KVCache(shape, c.max_sequence_length, i, device=self.device, dtype=BF16)
+        return [KVCache(shape, c.max_sequence_length, i, device=self.device, dtype=BF16, int8=int8)
                 for i in range(c.num_hidden_layers)]
 
     def default_n_split(self, batch: int) -> int:
@@ -273,6 +289,25 @@ class Llama:
         s.history = 0 if history is None else history.data_ptr()
         s.kcache, s.vcache = C.cast(kc, C.POINTER(C.c_void_p)), C.cast(vc, C.POINTER(C.c_void_p))
         s._keep = (kc, vc)
+        if len({c.int8 for c in kv_cache}) > 1:
+            raise ValueError("all layers must use the same KV cache mode")
+        if kv_cache[0].int8:
+            stats = [(C.c_void_p * n)(*[getattr(c, nm).data_ptr() for c in kv_cache])
+                     for nm in ("key_scale", "key_min", "value_scale", "value_min")]
+            s.kv_int8 = 1
+            s.kscale, s.kmin, s.vscale, s.vmin = (C.cast(a, C.POINTER(C.c_void_p)) for a in stats)
+            kvw = self.kv_heads * self.head_dim
+            if buf.kstage is None:
+                buf.kstage = torch.empty(buf.rows, kvw, dtype=BF16, device=self.device)
+                buf.vstage = torch.empty(buf.rows, kvw, dtype=BF16, device=self.device)
+            s.kstage, s.vstage = buf.kstage.data_ptr(), buf.vstage.data_ptr()
+            if buf.rows >= 16 * buf.batch:  # calls with many positions attend over a dequantised copy
+                shape = (kv_cache[0].key.shape[0], self.config.max_sequence_length, self.kv_heads, self.head_dim)
+                if buf.kdeq is None or tuple(buf.kdeq.shape) != shape:
+                    buf.kdeq = torch.empty(shape, dtype=BF16, device=self.device)
+                    buf.vdeq = torch.empty(shape, dtype=BF16, device=self.device)
+                s.kdeq, s.vdeq = buf.kdeq.data_ptr(), buf.vdeq.data_ptr()
+            s._keep = (kc, vc, *stats)
         return s
 
     def forward(self, x: torch.Tensor, kv_cache: list | None = None, position_ids=None, *, last_only: bool = False):
@@ -377,9 +412,11 @@ class DecodeSession:
             persistent = model.supports_persistent(batch) and batch <= 4
         elif persistent and not model.supports_persistent(batch):
             raise ValueError("the persistent decode kernel does not cover this shape")
-        self.persistent = persistent
         self._pws = None
         self.cache = kv_cache if kv_cache is not None else model.build_kv_cache(batch)
+        if self.cache[0].int8:
+            persistent = False  # the single-launch kernel reads bf16 caches only
+        self.persistent = persistent
         self.valid_vocab = valid_vocab
         self.history = torch.zeros(max(max_new_tokens, 1), batch, dtype=torch.int64, device=model.device)
         self.logits = torch.empty(batch, model.config.vocab_size, dtype=BF16, device=model.device)

@@ -191,6 +191,8 @@ class MoeLlama:
             raise ValueError("input exceeds max_sequence_length")
         if kv_cache is None:
             kv_cache = self.build_kv_cache(B)
+        if any(cc.int8 for cc in kv_cache):
+            raise NotImplementedError("ohara_amd: int8 KV caches are served by the dense Llama only")
         ends = [cc._reserve(B, S, start) for cc in kv_cache]
         H, Hkv, D = c.num_attention_heads, self.kv_heads, self.head_dim
         n_split = 1 if S > 1 else max(1, min(1024 // max(1, B * Hkv), c.max_sequence_length // 128, 64))

@@ -163,6 +163,24 @@ def qkv_rope_append(x, wqkv: PackedLinear, norm_w, eps, h, h_kv, dh, cos, sin, p
     return q_out
 
 
+def qkv_rope(x, wqkv: PackedLinear, norm_w, eps, h, h_kv, dh, cos, sin, pos, t_max, pos_dev=None, seq_len=1):
+    """As ``qkv_rope_append`` with the rotated keys and the values returned as (rows, h_kv*dh) row
+    buffers instead of written into a cache -> (q, k, v)."""
+    _need(x, BF16, "x")
+    rows = x.shape[0]
+    q = torch.empty(rows, h * dh, dtype=BF16, device=x.device)
+    k = torch.empty(rows, h_kv * dh, dtype=BF16, device=x.device)
+    v = torch.empty(rows, h_kv * dh, dtype=BF16, device=x.device)
+    check(
+        lib().ohara_qkv_rope_bf16(
+            _ptr(x), x.stride(0), _ptr(wqkv.data), wqkv.k, _ptr(norm_w), eps, rows // seq_len, seq_len, h, h_kv, dh,
+            _ptr(cos), _ptr(sin), int(pos), _ptr(pos_dev), t_max, _ptr(q), _ptr(k), _ptr(v), _stream(),
+        ),
+        "qkv_rope",
+    )
+    return q, k, v
+
+
 def attn_workspace(batch, h, h_kv, dh, n_split, device) -> torch.Tensor:
     n = lib().ohara_attn_workspace_bytes(batch, h, h_kv, dh, n_split)
     if n < 0:
@@ -207,6 +225,42 @@ def attn_auto(q, kcache, vcache, h, h_kv, dh, pos, n_split, workspace, seq_len, 
     if seq_len >= 16 and dh in (64, 128):
         return attn_prefill(q, kcache, vcache, h, h_kv, dh, pos, seq_len, out)
     return attn_cached(q, kcache, vcache, h, h_kv, dh, pos, n_split if seq_len == 1 else 1, workspace, out, None, seq_len)
+
+
+def kv_quant_append(keys, values, cache, pos, pos_dev=None):
+    """keys / values (B, S, Hkv, D) bf16 -> quantised into an int8 ``KVCache`` at positions pos + s."""
+    _need(keys, BF16, "keys")
+    _need(values, BF16, "values")
+    b, s_len, hkv, d = keys.shape
+    check(lib().ohara_kv_quant_append_int8(
+        _ptr(keys), _ptr(values), b, s_len, hkv, d, int(pos), _ptr(pos_dev), _ptr(cache.key), _ptr(cache.value),
+        _ptr(cache.key_scale), _ptr(cache.key_min), _ptr(cache.value_scale), _ptr(cache.value_min), cache.key.shape[1],
+        _stream()), "kv_quant_append")
+
+
+def kv_dequant(cache, which: str, batch: int, length: int, out=None) -> torch.Tensor:
+    """The first `length` positions of the int8 cache's key or value tensor as bf16 (B, length, Hkv, D)."""
+    q = cache.key if which == "key" else cache.value
+    scale = cache.key_scale if which == "key" else cache.value_scale
+    mn = cache.key_min if which == "key" else cache.value_min
+    _, t_max, hkv, d = q.shape
+    if out is None:
+        out = torch.empty(batch, length, hkv, d, dtype=BF16, device=q.device)
+    check(lib().ohara_kv_dequant_int8(_ptr(q), _ptr(scale), _ptr(mn), batch, length, hkv, d, t_max, _ptr(out), _stream()),
+          "kv_dequant")
+    return out
+
+
+def attn_cached_int8(q, cache, h, h_kv, dh, pos, n_split, workspace, out=None, pos_dev=None, seq_len=1):
+    """attn_cached over an int8 ``KVCache``."""
+    rows = q.shape[0]
+    if out is None:
+        out = torch.empty(rows, h * dh, dtype=BF16, device=q.device)
+    check(lib().ohara_attn_cached_int8(
+        _ptr(q), _ptr(cache.key), _ptr(cache.value), _ptr(cache.key_scale), _ptr(cache.key_min), _ptr(cache.value_scale),
+        _ptr(cache.value_min), rows // seq_len, seq_len, h, h_kv, dh, cache.key.shape[1], int(pos), _ptr(pos_dev), n_split,
+        _ptr(workspace), _ptr(out), _stream()), "attn_cached_int8")
+    return out
 
 
 def attn_decode(q, kcache, vcache, h, h_kv, dh, length, n_split, workspace, out=None, pos_dev=None):

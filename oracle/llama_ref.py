@@ -130,20 +130,48 @@ def apply_rope(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.T
     return rot(q), rot(k)
 
 
-class KVCacheRef:
-    """Fixed-size sequential-append cache - kv_cache.py:35-118 (non-int8 mode).
+def quantize_int8(tensor, dim: int = -1):
+    """Affine int8 codes along ``dim`` - kv_cache.py:15-28.
 
-    Storage (B, T_max, H_kv, D) for keys and values; holds post-rotary keys.
+    Every step is a separate elementwise op in the tensor's dtype (so each rounds to bf16 when the
+    rows are bf16): range = max - min; scale = max(range / 255, 1e-8); code = clamp(round((x - min)
+    / scale - 128), -128, 127).  ``round`` is to nearest even.  Returns (codes int8, scale, min).
+    """
+    lo, hi = tensor.amin(dim, keepdim=True), tensor.amax(dim, keepdim=True)
+    scale = ((hi - lo) / 255).clamp(min=1e-8)
+    codes = ((tensor - lo) / scale - 128).round().clamp(-128, 127).to(torch.int8)
+    return codes, scale, lo
+
+
+def dequantize_int8(codes, scale, lo):
+    """(code + 128) * scale + min in fp32 - kv_cache.py:31-33 (the stored statistics are fp32,
+    kv_cache.py:69-74, so the product and the sum each round once to fp32)."""
+    return (codes.float() + 128) * scale + lo
+
+
+class KVCacheRef:
+    """Fixed-size sequential-append cache - kv_cache.py:35-118.
+
+    Storage (B, T_max, H_kv, D) for keys and values; holds post-rotary keys.  With ``int8`` the
+    entries are int8 codes with one fp32 (scale, min) pair per (batch, position, head) row and reads
+    return the dequantised values cast to the dtype of the appended rows (kv_cache.py:94-118).
     """
 
-    def __init__(self, shape, max_seq_length, idx=None, dtype=torch.float32):
+    def __init__(self, shape, max_seq_length, idx=None, dtype=torch.float32, int8=False):
         self.idx = idx
+        self.int8 = int8
         self.max_seq_length = max_seq_length
         self.length = 0
         self.batch_size = None
         self.dtype = dtype
-        self.key = torch.zeros(shape, dtype=dtype)
-        self.value = torch.zeros(shape, dtype=dtype)
+        self.key = torch.zeros(shape, dtype=torch.int8 if int8 else dtype)
+        self.value = torch.zeros(shape, dtype=torch.int8 if int8 else dtype)
+        if int8:
+            stats = (*shape[:-1], 1)
+            self.key_scale = torch.zeros(stats, dtype=torch.float32)
+            self.key_min = torch.zeros(stats, dtype=torch.float32)
+            self.value_scale = torch.zeros(stats, dtype=torch.float32)
+            self.value_min = torch.zeros(stats, dtype=torch.float32)
 
     def forward(self, keys, values, start_pos):
         bsz, seq_len = keys.shape[0], keys.shape[1]
@@ -161,11 +189,25 @@ class KVCacheRef:
         if start_pos < 0 or start_pos + seq_len > self.max_seq_length:
             raise ValueError("KV cache position exceeds max_sequence_length")
         end = start_pos + seq_len
-        self.key[:bsz, start_pos:end] = keys
-        self.value[:bsz, start_pos:end] = values
+        if self.int8:
+            kq, ks, km = quantize_int8(keys)
+            vq, vs, vm = quantize_int8(values)
+            self.key[:bsz, start_pos:end] = kq
+            self.value[:bsz, start_pos:end] = vq
+            self.key_scale[:bsz, start_pos:end] = ks
+            self.key_min[:bsz, start_pos:end] = km
+            self.value_scale[:bsz, start_pos:end] = vs
+            self.value_min[:bsz, start_pos:end] = vm
+        else:
+            self.key[:bsz, start_pos:end] = keys
+            self.value[:bsz, start_pos:end] = values
         self.length = end
         self.batch_size = bsz
-        return self.key[:bsz, :end], self.value[:bsz, :end]
+        if not self.int8:
+            return self.key[:bsz, :end], self.value[:bsz, :end]
+        k = dequantize_int8(self.key[:bsz, :end], self.key_scale[:bsz, :end], self.key_min[:bsz, :end])
+        v = dequantize_int8(self.value[:bsz, :end], self.value_scale[:bsz, :end], self.value_min[:bsz, :end])
+        return k.to(keys.dtype), v.to(keys.dtype)
 
 
 def attention_core(q, k, v, start_pos: int | None):
@@ -290,12 +332,13 @@ class RefLlama:
         self._f32 = {}
 
     # llama.py:325-348
-    def build_kv_cache(self, batch_size: int = 1):
+    def build_kv_cache(self, batch_size: int = 1, int8: bool = False):
         if batch_size < 1:
             raise ValueError("batch_size must be at least 1")
         c = self.config
         shape = (batch_size, c.max_sequence_length, c.kv_heads, c.head_dim)
-        return [KVCacheRef(shape, c.max_sequence_length, i, dtype=self.dtype) for i in range(c.num_hidden_layers)]
+        return [KVCacheRef(shape, c.max_sequence_length, i, dtype=self.dtype, int8=int8)
+                for i in range(c.num_hidden_layers)]
 
     def _lin(self, name, x):
         """A Linear, or - when the weight dict holds ``name.ternary`` - a BitLinear

@@ -246,8 +246,11 @@ def test_config_and_kv_cache_bookkeeping():
         c.forward(k[:1, :1], k[:1, :1], 4)
     with pytest.raises(ValueError, match="smaller than the input batch"):
         KVCache((1, 8, 2, 4), 8, dtype=torch.float32).forward(k, k, 0)
-    with pytest.raises(NotImplementedError):
-        KVCache((1, 8, 2, 4), 8, dtype=torch.float32, int8=True)
+    q = KVCache((1, 8, 2, 4), 8, dtype=torch.float32, int8=True)  # kv_cache.py:64-74
+    assert q.key.dtype == torch.int8 and q.value.dtype == torch.int8
+    assert q.key_scale.shape == (1, 8, 2, 1) and q.value_min.dtype == torch.float32
+    with pytest.raises(ValueError, match="sequential"):
+        q.forward(k[:1, :1], k[:1, :1], 2)
 
 
 def test_product_has_no_cpu_fallback():

@@ -301,3 +301,121 @@ def test_bitlinear_integer_semantics():
     tt, gm = BL.weight_ternarize(w)
     y = BL.bitlinear_forward(x, nw, tt, gm)
     torch.testing.assert_close(y, BL.fake_quant_forward(x, nw, w), atol=2e-5, rtol=1e-4)
+
+
+# --- int8 KV cache (kv_cache.py:15-33, 94-118) ---------------------------------------------
+
+
+def _rne(q, bits: int):
+    """An exact rational rounded to `bits` significant bits, ties to even (normal range only)."""
+    from fractions import Fraction
+
+    if q == 0:
+        return Fraction(0)
+    sign, q = (-1 if q < 0 else 1), abs(q)
+    e = q.numerator.bit_length() - q.denominator.bit_length()
+    if Fraction(2) ** e > q:
+        e -= 1
+    ulp = Fraction(2) ** (e - bits + 1)
+    n, rem = divmod(q, ulp)
+    if rem * 2 > ulp or (rem * 2 == ulp and n % 2 == 1):
+        n += 1
+    return sign * n * ulp
+
+
+def _bf16_op(q):
+    """A bf16 tensor op: the exact result rounded to fp32 (the arithmetic runs in fp32), then to bf16."""
+    return _rne(_rne(q, 24), 8)
+
+
+def _quant_row_bf16_by_hand(row: np.ndarray):
+    """One bf16 row through the int8 quantiser in exact rational arithmetic with the roundings of
+    every op written out (kv_cache.py:20-27 on a bf16 tensor)."""
+    from fractions import Fraction
+
+    vals = [Fraction(float(x)) for x in row]
+    lo, hi = min(vals), max(vals)
+    scale = max(_bf16_op(_bf16_op(hi - lo) / 255), _bf16_op(Fraction(1e-8)))
+    codes = []
+    for x in vals:
+        t = _bf16_op(_bf16_op(_bf16_op(x - lo) / scale) - 128)
+        n = math.floor(t)  # round half to even
+        r = t - n
+        n += 1 if (r > Fraction(1, 2) or (r == Fraction(1, 2) and n % 2 == 1)) else 0
+        codes.append(min(127, max(-128, n)))
+    return np.array(codes, np.int8), np.float32(float(scale)), np.float32(float(lo))
+
+
+def test_int8_quantiser_closed_forms():
+    # an exact 256-level ramp maps onto the codes -128..127 and inverts exactly
+    lo, step = -3.0, 0.03125
+    ramp = (lo + step * torch.arange(256, dtype=torch.float32)).view(1, 256)
+    q, scale, mn = R.quantize_int8(ramp)
+    assert q.dtype == torch.int8 and scale.shape == mn.shape == (1, 1)
+    assert torch.equal(q.view(-1).int(), torch.arange(256, dtype=torch.int32) - 128)
+    assert float(scale) == step and float(mn) == lo
+    assert torch.equal(R.dequantize_int8(q, scale, mn), ramp)
+    # a constant row: the scale floors at 1e-8, all codes -128, the value comes back
+    const = torch.full((2, 8), 0.75)
+    q, scale, mn = R.quantize_int8(const)
+    assert torch.all(q == -128) and torch.all(scale == 1e-8) and torch.equal(R.dequantize_int8(q, scale, mn), const)
+    # extremes hit the end codes; the error never exceeds half a level (+ fp32 rounding)
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(64, 48, generator=g) * 3
+    q, scale, mn = R.quantize_int8(x)
+    assert torch.all(q.amin(-1) == -128) and torch.all(q.amax(-1) == 127)
+    err = (R.dequantize_int8(q, scale, mn) - x).abs()
+    assert torch.all(err <= scale * 0.5 + 1e-5)
+    # other reduction axes quantise along that axis
+    qt, st, mt = R.quantize_int8(x.t().contiguous(), dim=0)
+    assert torch.equal(qt.t(), q) and torch.equal(st.view(-1), scale.view(-1))
+    # the reference's own tolerance for the round trip (tests/test_modules.py:94-100)
+    t = torch.randn(4, 16, generator=g)
+    torch.testing.assert_close(R.dequantize_int8(*R.quantize_int8(t)), t, rtol=0.05, atol=0.05)
+
+
+def test_int8_quantiser_bf16_rounding_points_by_hand():
+    g = torch.Generator().manual_seed(11)
+    x = (torch.randn(6, 32, generator=g) * 2).to(torch.bfloat16)
+    x[5] = 1.5  # constant row
+    q, scale, mn = R.quantize_int8(x)
+    assert scale.dtype == torch.bfloat16
+    for i in range(x.shape[0]):
+        hq, hs, hm = _quant_row_bf16_by_hand(x[i].float().numpy())
+        assert float(scale[i]) == float(hs) and float(mn[i]) == float(hm)
+        assert np.array_equal(q[i].numpy(), hq), i
+    # dequantisation is fp32: product rounds once, sum rounds once
+    d = R.dequantize_int8(q, scale.float(), mn.float())
+    assert d.dtype == torch.float32
+    by_hand = (np.float32(1) * (q.numpy().astype(np.float32) + 128) * scale.float().numpy()).astype(np.float32) \
+        + mn.float().numpy()
+    assert np.array_equal(d.numpy(), by_hand.astype(np.float32))
+
+
+def test_int8_cache_reads_dequantised_values():
+    """tests/test_modules.py:82-91 on the restated cache, plus sequential appends."""
+    g = torch.Generator().manual_seed(5)
+    cache = R.KVCacheRef((2, 8, 2, 4), 8, dtype=torch.float32, int8=True)
+    entry = torch.randn(1, 4, 2, 4, generator=g)
+    keys, values = cache.forward(entry, entry.clone(), 0)
+    assert keys.dtype == torch.float32 and cache.key.dtype == torch.int8
+    torch.testing.assert_close(keys, entry, rtol=0.05, atol=0.05)
+    torch.testing.assert_close(values, entry, rtol=0.05, atol=0.05)
+    nxt = torch.randn(1, 1, 2, 4, generator=g)
+    k2, v2 = cache.forward(nxt, -nxt, 4)
+    assert k2.shape == (1, 5, 2, 4) and torch.equal(k2[:, :4], keys)
+    torch.testing.assert_close(v2[:, 4:], -nxt, rtol=0.05, atol=0.05)
+    assert cache.key_scale.shape == (2, 8, 2, 1) and torch.all(cache.key_scale[0, :5] > 0)
+    assert torch.all(cache.key_scale[1] == 0) and torch.all(cache.key_scale[0, 5:] == 0)
+    with pytest.raises(ValueError, match="sequential"):
+        cache.forward(nxt, nxt, 3)
+
+
+def test_int8_cache_model_stays_close_to_the_exact_cache():
+    cfg = R.RefConfig(vocab_size=97, max_sequence_length=32, hidden_size=64, intermediate_size=128,
+                      num_attention_heads=4, num_key_value_heads=2, num_hidden_layers=2)
+    model = R.RefLlama(cfg, R.init_weights(cfg, 2, norm_jitter=0.2))
+    ids = torch.randint(0, 97, (2, 9), generator=torch.Generator().manual_seed(1))
+    exact = model(ids, model.build_kv_cache(2), 0)
+    quant = model(ids, model.build_kv_cache(2, int8=True), 0)
+    assert 0 < (exact - quant).abs().max() < 0.05 * exact.abs().max()
