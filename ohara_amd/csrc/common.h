@@ -16,10 +16,38 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 #define WAVE 64
 
-__device__ __forceinline__ uint4 ldg16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+// Every pointer these helpers take addresses device memory.  Saying so (address space 1) matters
+// where the compiler cannot see it - pointers fetched from tables in memory or LDS - because a
+// generic ("flat") access also counts as an LDS access, so waiting for LDS data would wait for
+// every weight or cache load in flight.
+#define OHARA_GLOBAL __attribute__((address_space(1)))
+#define OHARA_LDS __attribute__((address_space(3)))
+
+__device__ __forceinline__ uint4 ldg16(const void* p) {
+  const u32x4 v = *(const OHARA_GLOBAL u32x4*)p;
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint2 ldg8(const void* p) {
+  const u32x2 v = *(const OHARA_GLOBAL u32x2*)p;
+  return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ uint32_t ldg4(const void* p) { return *(const OHARA_GLOBAL uint32_t*)p; }
 // 16-byte load flagged as streaming (read once): keeps reusable data in L2.
 __device__ __forceinline__ uint4 ldg16_nt(const void* p) {
-  u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  u32x4 v = __builtin_nontemporal_load((const OHARA_GLOBAL u32x4*)p);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ int64_t ldg_i64(const int64_t* p) { return *(const OHARA_GLOBAL int64_t*)p; }
+__device__ __forceinline__ void stg8(void* p, uint2 v) { *(OHARA_GLOBAL u32x2*)p = (u32x2){v.x, v.y}; }
+// LDS accesses through a pointer whose address space the compiler cannot see
+__device__ __forceinline__ void sts8(void* p, uint2 v) { *(OHARA_LDS u32x2*)p = (u32x2){v.x, v.y}; }
+__device__ __forceinline__ void sts16(void* p, uint4 v) {
+  *(OHARA_LDS u32x4*)p = (u32x4){v.x, v.y, v.z, v.w};
+}
+__device__ __forceinline__ uint4 lds16(const void* p) {
+  const u32x4 v = *(const OHARA_LDS u32x4*)p;
   return make_uint4(v.x, v.y, v.z, v.w);
 }
 
@@ -56,15 +84,15 @@ __device__ __forceinline__ float wave_max(float v) {
 // and is read with such loads.  An agent-scope fence instead writes back / invalidates a whole
 // L2, which serialises across workgroups (~0.2 us each on this chip).
 __device__ __forceinline__ void st_coh8(void* p, uint2 v) {
-  __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), ((unsigned long long)v.y << 32) | v.x,
-                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store((OHARA_GLOBAL unsigned long long*)p, ((unsigned long long)v.y << 32) | v.x, __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void st_coh4(void* p, uint32_t v) {
-  __hip_atomic_store(reinterpret_cast<uint32_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store((OHARA_GLOBAL uint32_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ uint2 ld_coh8(const void* p) {
   const unsigned long long v =
-      __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_load((const OHARA_GLOBAL unsigned long long*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return make_uint2((uint32_t)v, (uint32_t)(v >> 32));
 }
 __device__ __forceinline__ uint4 ld_coh16(const void* p) {
@@ -72,7 +100,7 @@ __device__ __forceinline__ uint4 ld_coh16(const void* p) {
   return make_uint4(a.x, a.y, b.x, b.y);
 }
 __device__ __forceinline__ uint32_t ld_coh4(const void* p) {
-  return __hip_atomic_load(reinterpret_cast<const uint32_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return __hip_atomic_load((const OHARA_GLOBAL uint32_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }

@@ -92,7 +92,6 @@ struct GridSync {
   unsigned int gsize;  // workgroups in my group
   unsigned int ng;
   unsigned int limit;
-  unsigned int arrived;
   __device__ void init(unsigned int* bar, unsigned int nwg, unsigned int lim) {
     ng = (nwg + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP;
     const unsigned int g = blockIdx.x / OHARA_BAR_GROUP;
@@ -103,7 +102,6 @@ struct GridSync {
     err = bar + (ng + 2) * 64;
     done = bar + (ng + 3) * 64;
     limit = lim;
-    arrived = 0;
     k = *done + 1;  // written by the previous launch (or the host): plain load
   }
   __device__ __forceinline__ void arrive(Prof& pf) {
@@ -112,17 +110,21 @@ struct GridSync {
     pf.stamp();  // stores complete
     __builtin_amdgcn_s_barrier();
     pf.stamp();  // workgroup barrier passed
-    if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(gc, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+    // The whole arrival happens here, before the caller's prefetch: the last workgroup of a group
+    // must not sit on the group's arrival while it issues loads.
+    if (threadIdx.x == 0) {
+      const unsigned int a = __hip_atomic_fetch_add(gc, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+      if (a == k * gsize) {
+        const unsigned int t = __hip_atomic_fetch_add(top, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+        if (t == k * ng) __hip_atomic_store(rel, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
     asm volatile("" ::: "memory");  // compiler only: keep the caller's prefetch loads after this point
     pf.stamp();  // arrival issued
   }
   __device__ __forceinline__ void wait(Prof& pf) {
     pf.stamp();  // prefetch issued
     if (threadIdx.x == 0) {
-      if (arrived == k * gsize) {
-        const unsigned int t = __hip_atomic_fetch_add(top, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
-        if (t == k * ng) __hip_atomic_store(rel, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
       unsigned int spins = 0;
       while ((int)(__hip_atomic_load(rel, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - k) < 0) {
         ++spins;
@@ -184,7 +186,7 @@ __device__ void stage_norm(bf16_t* xs, int ldxs, const char* src, int blk, const
     uint4 v[NLD], g[NLD];
     size_t row_off = 0;
     if (EMBED) {
-      int64_t id = ids[b];
+      int64_t id = ldg_i64(ids + b);
       if (id < 0 || id >= vocab) id = 0;
       row_off = (size_t)id * K;
     }
@@ -221,7 +223,7 @@ __device__ void stage_norm(bf16_t* xs, int ldxs, const char* src, int blk, const
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           o[i] = pack_bf(rbf(lo_bf(xv[i]) * rinv) * lo_bf(gv[i]), rbf(hi_bf(xv[i]) * rinv) * hi_bf(gv[i]));
-        *reinterpret_cast<uint4*>(xs + (size_t)b * ldxs + k) = make_uint4(o[0], o[1], o[2], o[3]);
+        sts16(xs + (size_t)b * ldxs + k, make_uint4(o[0], o[1], o[2], o[3]));
       }
     }
   }
@@ -232,7 +234,7 @@ __device__ void stage_act(bf16_t* xs, int ldxs, const char* src, int blk, int B,
   const int n8 = F >> 3;
   for (int i = threadIdx.x; i < B * n8; i += blockDim.x) {
     const int b = i / n8, c = i - b * n8;
-    *reinterpret_cast<uint4*>(xs + (size_t)b * ldxs + c * 8) = ldg16(am_addr(src, blk, b, c * 8));
+    sts16(xs + (size_t)b * ldxs + c * 8, ldg16(am_addr(src, blk, b, c * 8)));
   }
 }
 
@@ -241,11 +243,13 @@ __device__ void stage_act(bf16_t* xs, int ldxs, const char* src, int blk, int B,
 // (sequence, head, chunk) are fetched in one round into LDS and turned into chunk weights
 // exp(m_s - M) / L there; a thread then owns four adjacent columns and issues the accumulator
 // loads of all chunks before using any.  `mw`: B*H*ns floats, `ml`: B*H*ns floats of LDS.
-__device__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh, int ns, float* mw,
-                                 float* ml) {
+__device__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh, int ns, float* mw_,
+                                 float* ml_) {
   constexpr int NSM = OHARA_MEGA_NS;
   const int HD = H * Dh, PS = Dh + 32;
   const int nbh = B * H;
+  OHARA_LDS float* mw = (OHARA_LDS float*)mw_;
+  OHARA_LDS float* ml = (OHARA_LDS float*)ml_;
   // the accumulator loads of a thread's first columns go out first: they do not depend on the
   // chunk weights, which are formed (two LDS rounds) while they are in flight
   uint4 av[NSM];
@@ -265,7 +269,7 @@ __device__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, i
     const bool in = bh < nbh && sp < ns;
     float ms = -INFINITY, ls = 0.f;
     if (in) {
-      const uint2 v = *reinterpret_cast<const uint2*>(pm + ((size_t)bh * NSM + sp) * PS + Dh);
+      const uint2 v = ldg8(pm + ((size_t)bh * NSM + sp) * PS + Dh);
       ms = __uint_as_float(v.x);
       ls = __uint_as_float(v.y);
     }
@@ -301,8 +305,7 @@ __device__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, i
       }
     }
     const float Ls = ml[bh];
-    *reinterpret_cast<uint2*>(xs + (size_t)b * ldxs + hd) =
-        make_uint2(pack_bf(o[0] / Ls, o[1] / Ls), pack_bf(o[2] / Ls, o[3] / Ls));
+    sts8(xs + (size_t)b * ldxs + hd, make_uint2(pack_bf(o[0] / Ls, o[1] / Ls), pack_bf(o[2] / Ls, o[3] / Ls)));
   }
 }
 
@@ -321,7 +324,7 @@ __device__ void stage_attn_merge_small(bf16_t* xs, int ldxs, const float* pm, in
   uint4 av[NS];
 #pragma unroll
   for (int s = 0; s < NS; ++s) {
-    mlv[s] = *reinterpret_cast<const uint2*>(base + (size_t)s * PS + Dh);
+    mlv[s] = ldg8(base + (size_t)s * PS + Dh);
     av[s] = ldg16(base + (size_t)s * PS + d);
   }
   float M = -INFINITY;
@@ -338,8 +341,7 @@ __device__ void stage_attn_merge_small(bf16_t* xs, int ldxs, const float* pm, in
     o[2] += __uint_as_float(av[s].z) * w;
     o[3] += __uint_as_float(av[s].w) * w;
   }
-  *reinterpret_cast<uint2*>(xs + (size_t)b * ldxs + hd) =
-      make_uint2(pack_bf(o[0] / Ls, o[1] / Ls), pack_bf(o[2] / Ls, o[3] / Ls));
+  sts8(xs + (size_t)b * ldxs + hd, make_uint2(pack_bf(o[0] / Ls, o[1] / Ls), pack_bf(o[2] / Ls, o[3] / Ls)));
 }
 
 // ---------------------------------------------------------------------------------------
@@ -393,11 +395,11 @@ __device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int 
     pre.r = make_uint2(0, 0);
     if (strip < p.nstrips && kpart == 0 && m < B && r0 < p.N) {
       if (!p.resid_embed) {
-        pre.r = *reinterpret_cast<const uint2*>(xm_addr(p.resid, p.blk, m, r0));
+        pre.r = ldg8(xm_addr(p.resid, p.blk, m, r0));
       } else {
-        int64_t id = p.ids[m];
+        int64_t id = ldg_i64(p.ids + m);
         if (id < 0 || id >= p.vocab) id = 0;
-        pre.r = *reinterpret_cast<const uint2*>(p.table + (size_t)id * p.N + r0);
+        pre.r = ldg8(p.table + (size_t)id * p.N + r0);
       }
     }
   }
@@ -470,11 +472,11 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
           uint2 r = pre.r;
           if (it > 0) {
             if (!p.resid_embed) {
-              r = *reinterpret_cast<const uint2*>(xm_addr(p.resid, p.blk, b, r0));
+              r = ldg8(xm_addr(p.resid, p.blk, b, r0));
             } else {
-              int64_t id = p.ids[b];
+              int64_t id = ldg_i64(p.ids + b);
               if (id < 0 || id >= p.vocab) id = 0;
-              r = *reinterpret_cast<const uint2*>(p.table + (size_t)id * p.N + r0);
+              r = ldg8(p.table + (size_t)id * p.N + r0);
             }
           }
           st_coh8(const_cast<char*>(xm_addr(p.out, p.blk, b, r0)),
@@ -484,7 +486,7 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
         const float v[4] = {y0, y1, y2, y3};
         bf16_t* o = reinterpret_cast<bf16_t*>(p.out) + (size_t)b * p.ldo + r0;
         if (r0 + 3 < p.N && ((p.ldo & 3) == 0)) {
-          *reinterpret_cast<uint2*>(o) = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
+          stg8(o, make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3])));
         } else {
 #pragma unroll
           for (int i = 0; i < 4; ++i)
@@ -511,8 +513,8 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
           char* o;
           if (r0 < nq + nk) {
             const int d = (r0 < nq ? r0 : r0 - nq) % p.Dh;
-            const uint32_t cs = *reinterpret_cast<const uint32_t*>(p.cos + (size_t)p.pos * (p.Dh >> 1) + (d >> 1));
-            const uint32_t sn = *reinterpret_cast<const uint32_t*>(p.sin + (size_t)p.pos * (p.Dh >> 1) + (d >> 1));
+            const uint32_t cs = ldg4(p.cos + (size_t)p.pos * (p.Dh >> 1) + (d >> 1));
+            const uint32_t sn = ldg4(p.sin + (size_t)p.pos * (p.Dh >> 1) + (d >> 1));
             const float c2[2] = {lo_bf(cs), hi_bf(cs)}, s2[2] = {lo_bf(sn), hi_bf(sn)};
 #pragma unroll
             for (int pr = 0; pr < 2; ++pr) {
