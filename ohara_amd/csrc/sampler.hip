@@ -27,6 +27,7 @@
 namespace {
 
 constexpr int NT = 1024;
+constexpr int NW = NT / 64;  // waves per workgroup
 constexpr int CAP = 1024;  // candidates sorted per round
 
 struct SampleArgs {
@@ -66,11 +67,11 @@ __device__ __forceinline__ float block_max(float v, Smem& s) {
   __syncthreads();
   float r = s.wred[0];
 #pragma unroll
-  for (int i = 1; i < 16; ++i) r = fmaxf(r, s.wred[i]);
+  for (int i = 1; i < NW; ++i) r = fmaxf(r, s.wred[i]);
   return r;
 }
 
-// Sum in a fixed order: butterfly inside each wave, then the 16 wave sums left to right.
+// Sum in a fixed order: butterfly inside each wave, then the wave sums left to right.
 __device__ __forceinline__ float block_sum(float v, Smem& s) {
   v = wave_sum(v);
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -79,7 +80,7 @@ __device__ __forceinline__ float block_sum(float v, Smem& s) {
   __syncthreads();
   float r = s.wred[0];
 #pragma unroll
-  for (int i = 1; i < 16; ++i) r += s.wred[i];
+  for (int i = 1; i < NW; ++i) r += s.wred[i];
   return r;
 }
 
@@ -92,12 +93,12 @@ __device__ __forceinline__ int block_sum_i(int v, Smem& s) {
   __syncthreads();
   int r = 0;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) r += s.wredi[i];
+  for (int i = 0; i < NW; ++i) r += s.wredi[i];
   return r;
 }
 
 // Exclusive prefix sum of one int per thread, in thread order.  Returns the total.
-// Wave-level shuffle scan, then the 16 wave totals.
+// Wave-level shuffle scan, then the wave totals.
 __device__ __forceinline__ int block_excl_scan_i(int v, int& excl, Smem& s) {
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   int incl = v;
@@ -111,7 +112,7 @@ __device__ __forceinline__ int block_excl_scan_i(int v, int& excl, Smem& s) {
   __syncthreads();
   int before = 0, total = 0;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
+  for (int i = 0; i < NW; ++i) {
     const int t = s.wredi[i];
     if (i < w) before += t;
     total += t;
@@ -120,10 +121,37 @@ __device__ __forceinline__ int block_excl_scan_i(int v, int& excl, Smem& s) {
   return total;
 }
 
+// Prefix sums of one float per thread, in thread order, in a fixed association (shuffle scan
+// inside each wave, then the wave totals left to right): thread t gets lo = sum over threads
+// before it and hi = lo of thread t + 1 (bit-identical), so the intervals [lo, hi) tile
+// [0, total) without gaps.  Returns the total.
+__device__ __forceinline__ float block_scan_f(float v, float& lo, float& hi, Smem& s) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  float incl = v;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const float t = __shfl_up(incl, o, WAVE);
+    if (lane >= o) incl += t;
+  }
+  const float prev = __shfl_up(incl, 1, WAVE);
+  __syncthreads();
+  if (lane == 63) s.wred[w] = incl;
+  __syncthreads();
+  float before = 0.f, total = 0.f;
+#pragma unroll
+  for (int i = 0; i < NW; ++i) {
+    if (i == w) before = total;
+    total += s.wred[i];
+  }
+  lo = lane == 0 ? before : before + prev;
+  hi = lane == 63 ? before + s.wred[w] : before + incl;
+  return total;
+}
+
 // The `want`-th largest key (1-based) among the keys for which live(i) holds; returns the
 // key and the number of live keys strictly greater than it.
 template <int EPT, typename LiveFn, typename KeyFn>
-__device__ uint32_t radix_select(int want, int& n_greater, Smem& s, LiveFn live, KeyFn key) {
+__device__ __forceinline__ uint32_t radix_select(int want, int& n_greater, Smem& s, LiveFn live, KeyFn key) {
   uint32_t prefix = 0, mask = 0;
   int above = 0;
   for (int shift = 24; shift >= 0; shift -= 8) {
@@ -178,7 +206,7 @@ __device__ uint32_t radix_select(int want, int& n_greater, Smem& s, LiveFn live,
 // are >= it), so only the elements at or above that bound - usually a few times `want` - take part
 // in the exact radix select.
 template <int EPT, typename LiveFn, typename KeyFn>
-__device__ uint32_t select_small(int want, int& n_greater, Smem& s, LiveFn live, KeyFn key) {
+__device__ __forceinline__ uint32_t select_small(int want, int& n_greater, Smem& s, LiveFn live, KeyFn key) {
   uint32_t tmax = 0;  // keys of live elements are > 0
 #pragma unroll
   for (int i = 0; i < EPT; ++i)
@@ -429,23 +457,10 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
     float ts = 0.f;
 #pragma unroll
     for (int i = 0; i < EPT; ++i) ts += x[i];
-    // exclusive scan of the per-thread sums, in thread order
-    __syncthreads();
-    s.fscan[tid] = ts;
-    __syncthreads();
-    if (tid == 0) {
-      float run = 0.f;
-      for (int t = 0; t < NT; ++t) {
-        const float v = s.fscan[t];
-        s.fscan[t] = run;
-        run += v;
-      }
-      s.fmisc[0] = run;
-    }
-    __syncthreads();
-    const float total = s.fmisc[0];
+    // prefix sums of the per-thread masses, in thread order: thread t owns [lo, hi)
+    float lo, hi;
+    const float total = block_scan_f(ts, lo, hi, s);
     const float target = u * total;
-    const float lo = s.fscan[tid];
     // last id with p > 0 (fallback when rounding pushes target past the end)
     int lastpos = -1;
 #pragma unroll
@@ -456,22 +471,25 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
     for (int o = 32; o > 0; o >>= 1) mx = max(mx, __shfl_xor(mx, o, WAVE));
     __syncthreads();
     if ((tid & 63) == 0) s.wredi[tid >> 6] = mx;
+    if (tid == 0) s.misc[2] = 0x7fffffff;
     __syncthreads();
     int last_id = -1;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) last_id = max(last_id, s.wredi[i]);
-    if (tid == 0) s.misc[2] = 0x7fffffff;
-    __syncthreads();
-    int found = 0x7fffffff;
-    if (target >= lo && ts > 0.f) {
+    for (int i = 0; i < NW; ++i) last_id = max(last_id, s.wredi[i]);
+    if (target >= lo && target < hi) {  // exactly one thread
       float run = lo;
+      int found = lastpos;  // the running sum inside the thread may round short of hi
+      bool hit = false;
 #pragma unroll
       for (int i = 0; i < EPT; ++i) {
         run += x[i];
-        if (x[i] > 0.f && run > target && found == 0x7fffffff) found = base + i;
+        if (x[i] > 0.f && run > target && !hit) {
+          found = base + i;
+          hit = true;
+        }
       }
+      s.misc[2] = found;
     }
-    if (found != 0x7fffffff) atomicMin(&s.misc[2], found);
     __syncthreads();
     token = s.misc[2] == 0x7fffffff ? max(last_id, 0) : s.misc[2];
   } else {
