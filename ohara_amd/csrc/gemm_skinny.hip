@@ -149,6 +149,159 @@ __global__ __launch_bounds__(256) void skinny_kernel(GemmArgs a) {
   }
 }
 
+// Many strips (the vocabulary projection): the activations are the stationary operand.  Every
+// workgroup normalises all rows once into LDS (up to 64 rows, zero-padded to
+// 16*BT rows and 32*KS columns), then each of its 8 waves walks whole strips - full K, no
+// cross-wave sum - reading the MFMA B operands from LDS, so the weights are read exactly once
+// whatever the row count and the norm is computed once per workgroup, not once per strip.
+constexpr int WIDE_WAVES = 8;
+constexpr int WIDE_CH = 12;
+
+template <int BT, bool NORM, int EPI>
+__global__ __launch_bounds__(WIDE_WAVES * 64) void wide_kernel(GemmArgs a) {
+  extern __shared__ __align__(16) unsigned char wide_smem[];
+  bf16_t* xs = reinterpret_cast<bf16_t*>(wide_smem);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m = lane & 15, g = lane >> 4;
+  const int KS = (a.K + 31) >> 5;
+  const int ldxs = KS * 32 + 8;
+  const int stride = gridDim.x * WIDE_WAVES;
+  int strip = blockIdx.x * WIDE_WAVES + wave;
+  // two register buffers of WIDE_CH k-steps; the first strip's are requested before the
+  // activations are staged, so the weight stream starts with the kernel
+  uint4 wa[WIDE_CH], wb[WIDE_CH];
+  auto load = [&](uint4* w, int st, int j) {
+    const uint4* wrow = a.wp + (size_t)st * KS * 64 + lane;
+#pragma unroll
+    for (int c = 0; c < WIDE_CH; ++c)
+      w[c] = (st < a.nstrips && j + c < KS) ? ldg16_nt(wrow + (size_t)(j + c) * 64) : make_uint4(0, 0, 0, 0);
+  };
+  load(wa, strip, 0);
+  load(wb, strip, WIDE_CH);
+
+  if (a.K <= 1024) {
+    // every row of this wave is requested before any is used (K <= 1024: two 16-byte pieces per lane)
+    constexpr int RPW = 16 * BT / WIDE_WAVES;
+    uint4 v[RPW][2], nwv[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int k = lane * 8 + 512 * c;
+      nwv[c] = (NORM && k < a.K) ? ldg16(a.norm_w + k) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int r = 0; r < RPW; ++r) {
+        const int b = wave + WIDE_WAVES * r;
+        v[r][c] = (b < a.B && k < a.K) ? ldg16(a.x + (size_t)b * a.ldx + k) : make_uint4(0, 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+      const int b = wave + WIDE_WAVES * r;
+      float rinv = 1.f;
+      if (NORM) rinv = 1.0f / sqrtf(wave_sum(sumsq8(v[r][0]) + sumsq8(v[r][1])) / (float)a.K + a.eps);
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const int k = lane * 8 + 512 * c;
+        if (k < KS * 32)
+          *reinterpret_cast<uint4*>(xs + (size_t)b * ldxs + k) = NORM ? norm8(v[r][c], nwv[c], rinv) : v[r][c];
+      }
+    }
+  } else {
+    for (int b = wave; b < 16 * BT; b += WIDE_WAVES) {
+      float rinv = 1.f;
+      if (NORM && b < a.B) {
+        float ss = 0.f;
+        for (int k = lane * 8; k < a.K; k += 512) ss += sumsq8(ldg16(a.x + (size_t)b * a.ldx + k));
+        rinv = 1.0f / sqrtf(wave_sum(ss) / (float)a.K + a.eps);
+      }
+      for (int k = lane * 8; k < KS * 32; k += 512) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (b < a.B && k < a.K) {
+          v = ldg16(a.x + (size_t)b * a.ldx + k);
+          if (NORM) v = norm8(v, ldg16(a.norm_w + k), rinv);
+        }
+        *reinterpret_cast<uint4*>(xs + (size_t)b * ldxs + k) = v;
+      }
+    }
+  }
+  __syncthreads();
+
+  const bf16_t* xrow = xs + (size_t)m * ldxs + 8 * g;
+  for (; strip < a.nstrips; strip += stride) {
+    f32x4 acc[BT];
+#pragma unroll
+    for (int t = 0; t < BT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    auto mul = [&](const uint4* w, int j) {
+#pragma unroll
+      for (int c = 0; c < WIDE_CH; ++c) {
+        if (j + c < KS) {
+#pragma unroll
+          for (int t = 0; t < BT; ++t) {
+            const uint4 xv = *reinterpret_cast<const uint4*>(xrow + (size_t)(16 * t) * ldxs + 32 * (j + c));
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w[c]),
+                                                             __builtin_bit_cast(bf16x8, xv), acc[t], 0, 0, 0);
+          }
+        }
+      }
+    };
+    // wa / wb hold k-steps [j, j + CH) and [j + CH, j + 2 CH) of this strip; each buffer is refilled
+    // (from this strip, or from the start of the wave's next one) as soon as it has been multiplied
+    for (int j = 0; j < KS; j += 2 * WIDE_CH) {
+      const bool more = j + 2 * WIDE_CH < KS;
+      mul(wa, j);
+      if (more) load(wa, strip, j + 2 * WIDE_CH);
+      else load(wa, strip + stride, 0);
+      mul(wb, j + WIDE_CH);
+      if (more) load(wb, strip, j + 3 * WIDE_CH);
+      else load(wb, strip + stride, WIDE_CH);
+    }
+#pragma unroll
+    for (int t = 0; t < BT; ++t) {
+      const int b = m + 16 * t;
+      if (b < a.B) gemm_epilogue<EPI>(a, b, strip, g, acc[t]);
+    }
+  }
+}
+
+template <int BT>
+int launch_wide_bt(const GemmArgs& a, int epi, hipStream_t st) {
+  const int KS = (a.K + 31) >> 5;
+  const size_t smem = (size_t)16 * BT * (KS * 32 + 8) * sizeof(bf16_t);
+  const int grid = (a.nstrips + WIDE_WAVES - 1) / WIDE_WAVES < 256 ? (a.nstrips + WIDE_WAVES - 1) / WIDE_WAVES : 256;
+#define OHARA_WIDE(NORM_, EPI_)                                                                                   \
+  do {                                                                                                            \
+    if (smem > 64 * 1024)                                                                                         \
+      (void)hipFuncSetAttribute((const void*)wide_kernel<BT, NORM_, EPI_>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                (int)smem);                                                                       \
+    hipLaunchKernelGGL((wide_kernel<BT, NORM_, EPI_>), dim3(grid), dim3(WIDE_WAVES * 64), smem, st, a);           \
+  } while (0)
+  if (epi == EPI_STORE) {
+    if (a.norm_w) OHARA_WIDE(true, EPI_STORE);
+    else OHARA_WIDE(false, EPI_STORE);
+  } else {
+    return OHARA_EINVAL;
+  }
+#undef OHARA_WIDE
+  return ohara_launch_status();
+}
+
+// The wide kernel serves plain stores of many strips whose rows fit LDS.
+bool wide_applies(const GemmArgs& a, int epi, int strips) {
+  const int KS = (a.K + 31) >> 5;
+  const int bt = (a.B + 15) / 16;
+  return epi == EPI_STORE && strips >= 1024 && a.B <= 64 && (size_t)16 * bt * (KS * 32 + 8) * 2 <= 128 * 1024;
+}
+
+int launch_wide(const GemmArgs& a0, int epi, int strips, hipStream_t st) {
+  GemmArgs a = a0;
+  a.nstrips = strips;
+  switch ((a.B + 15) / 16) {
+    case 1: return launch_wide_bt<1>(a, epi, st);
+    case 2: return launch_wide_bt<2>(a, epi, st);
+    case 3: return launch_wide_bt<3>(a, epi, st);
+    default: return launch_wide_bt<4>(a, epi, st);
+  }
+}
+
 template <int BT, bool NORM>
 int launch_epi(const GemmArgs& a, int epi, int strips, hipStream_t st) {
   dim3 grid((unsigned)((strips + 7) / 8 * 8 * a.ny)), block(256);
@@ -177,6 +330,7 @@ int launch_chunk(const GemmArgs& a0, int epi, int strips, hipStream_t st) {
 int launch_skinny(const GemmArgs& a0, int epi, int packed_rows, hipStream_t st) {
   const int strips = packed_rows / 16;
   const int rows = a0.B;
+  if (wide_applies(a0, epi, strips)) return launch_wide(a0, epi, strips, st);
   for (int r = 0; r < rows; r += 64) {
     GemmArgs a = a0;
     a.B = rows - r < 64 ? rows - r : 64;

@@ -49,7 +49,10 @@ def test_rmsnorm(cuda, d):
 
 
 @pytest.mark.parametrize("B,N,K", [(1, 768, 768), (3, 64, 32), (8, 3072, 768), (16, 768, 3072), (17, 100, 96),
-                                   (32, 2304, 768), (64, 768, 3072), (5, 65, 40)])
+                                   (32, 2304, 768), (64, 768, 3072), (5, 65, 40),
+                                   # >= 1024 strips: the kernel that keeps the activations in LDS
+                                   (1, 16384, 768), (17, 16390, 776), (33, 20000, 96), (64, 16384, 768),
+                                   (48, 16400, 1000)])
 @pytest.mark.parametrize("norm", [False, True])
 def test_gemm_skinny_store(cuda, B, N, K, norm):
     from ohara_amd import ops
