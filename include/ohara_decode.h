@@ -151,7 +151,9 @@ int ohara_attn_prefill_bf16(const uint16_t* q, const uint16_t* kcache, const uin
  *   ohara_kv_dequant_int8       the first `len` positions of one cache tensor as bf16
  *                               (batch, len, h_kv, dh) - what KVCache._read returns;
  *   ohara_attn_cached_int8      ohara_attn_cached_bf16 over the quantised cache, dequantising in
- *                               registers (dh 64 or 128, 1 / 2 / 4 query heads per KV head). */
+ *                               registers.  Scales must be bf16-representable, as the quantiser
+ *                               writes them: (q + 128) * scale is then exact in fp32 and the
+ *                               kernel's fused multiply-add equals the reference's two roundings. */
 int ohara_kv_quant_append_int8(const uint16_t* k, const uint16_t* v, int batch, int seq_len, int h_kv, int dh, int pos,
                                const int32_t* pos_dev, int8_t* kq, int8_t* vq, float* kscale, float* kmin, float* vscale,
                                float* vmin, int t_max, void* stream);

@@ -116,12 +116,15 @@ __device__ bool last_chunk_done(int* counter, int nsplit) {
 }
 
 // (q + 128) * scale + min in fp32, rounded to bf16 (kv_cache.py:30-32, 116-118): four bytes -> two
-// packed bf16 pairs.  `w` already has 0x80 xor-ed in, i.e. holds q + 128 as unsigned bytes.
+// packed bf16 pairs.  `w` already has 0x80 xor-ed in, i.e. holds q + 128 as unsigned bytes.  The
+// scales written by the quantiser are bf16 values (8 significant bits) and q + 128 has at most 8,
+// so the product is exact in fp32 and one fused multiply-add gives bit for bit what the separate
+// multiply and add of the reference give.
 __device__ __forceinline__ uint2 dequant4(uint32_t w, float s, float m) {
-  const float f0 = __fadd_rn(__fmul_rn((float)(w & 0xffu), s), m);
-  const float f1 = __fadd_rn(__fmul_rn((float)((w >> 8) & 0xffu), s), m);
-  const float f2 = __fadd_rn(__fmul_rn((float)((w >> 16) & 0xffu), s), m);
-  const float f3 = __fadd_rn(__fmul_rn((float)(w >> 24), s), m);
+  const float f0 = __fmaf_rn((float)(w & 0xffu), s, m);
+  const float f1 = __fmaf_rn((float)((w >> 8) & 0xffu), s, m);
+  const float f2 = __fmaf_rn((float)((w >> 16) & 0xffu), s, m);
+  const float f3 = __fmaf_rn((float)(w >> 24), s, m);
   return make_uint2(pack_bf(f0, f1), pack_bf(f2, f3));
 }
 
@@ -165,8 +168,6 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   const bf16_t* kb = a.k + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
   const bf16_t* vb = a.v + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
 
-  // 16-position tiles, wave w takes tiles w, w+4, ...; the loads of the next tile are in
-  // flight while the current one is consumed
   // A tile in the form it is fetched in.  bf16: the MFMA-free dot operands themselves.  int8: the
   // raw bytes of this lane's quarter of the K row / eighth of the V rows plus the rows' scale and
   // minimum; they are expanded to bf16 right before use, so the fetch of the next tile stays
@@ -237,6 +238,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
       for (int c = 0; c < NV; ++c) vv[c] = t.v[c];
     }
   };
+  // 16-position tiles, wave w takes tiles w, w+4, ...; the loads of the next tile are in
+  // flight while the current one is consumed (a second tile in flight costs more in occupancy
+  // than it gains: measured)
   Tile cur, nxt;
   int tb = t0 + wave * 16;
   if (tb < t1) load_tile(tb, cur);
@@ -246,42 +250,75 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
     if (more) load_tile(tb + 64, nxt);
     uint4 kv[NC], vv[NV];
     expand(cur, kv, vv);
+    // The heads of the group advance together, one step at a time, so that their cross-lane
+    // exchanges overlap instead of forming G dependent chains.  l_run is this lane's share of the
+    // sum (its own position only; folded over the 16 positions after the loop), and the running
+    // maximum is re-derived only for tiles in which some score exceeds it - for every other tile
+    // the usual update would multiply by exp(0).
+    float sc[G], pv[G];
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) {
       float s = 0.f;
 #pragma unroll
       for (int c = 0; c < NC; ++c) s = dot8(kv[c], qv[hh][c], s);
-      s += __shfl_xor(s, 16, WAVE);
-      s += __shfl_xor(s, 32, WAVE);
-      s = valid ? s * a.scale : -INFINITY;
-      float tm = s;
+      sc[hh] = s;
+    }
 #pragma unroll
-      for (int o = 8; o > 0; o >>= 1) tm = fmaxf(tm, __shfl_xor(tm, o, WAVE));
-      const float mn = fmaxf(m_run[hh], tm);  // finite: the tile holds at least one position
-      const float corr = __expf(m_run[hh] - mn);
-      const float pv = __expf(s - mn);
-      float ts = pv;
+    for (int hh = 0; hh < G; ++hh) sc[hh] += __shfl_xor(sc[hh], 16, WAVE);
 #pragma unroll
-      for (int o = 8; o > 0; o >>= 1) ts += __shfl_xor(ts, o, WAVE);
-      l_run[hh] = l_run[hh] * corr + ts;
-      m_run[hh] = mn;
+    for (int hh = 0; hh < G; ++hh) sc[hh] += __shfl_xor(sc[hh], 32, WAVE);
+    bool raise = false;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[hh][i] *= corr;
+    for (int hh = 0; hh < G; ++hh) {
+      sc[hh] = valid ? sc[hh] * a.scale : -INFINITY;
+      raise = raise || sc[hh] > m_run[hh];
+    }
+    if (__any(raise)) {
+      float tm[G];
 #pragma unroll
-      for (int c = 0; c < NV; ++c) {
-        const float pw = __shfl(pv, c * PP + pp, WAVE);
-        const uint32_t w4[4] = {vv[c].x, vv[c].y, vv[c].z, vv[c].w};
+      for (int hh = 0; hh < G; ++hh) tm[hh] = sc[hh];
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1)
+#pragma unroll
+        for (int hh = 0; hh < G; ++hh) tm[hh] = fmaxf(tm[hh], __shfl_xor(tm[hh], o, WAVE));
+#pragma unroll
+      for (int hh = 0; hh < G; ++hh) {
+        const float mn = fmaxf(m_run[hh], tm[hh]);  // finite: the tile holds at least one position
+        const float corr = __expf(m_run[hh] - mn);
+        m_run[hh] = mn;
+        l_run[hh] *= corr;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[hh][i] *= corr;
+      }
+    }
+#pragma unroll
+    for (int hh = 0; hh < G; ++hh) {
+      pv[hh] = __expf(sc[hh] - m_run[hh]);
+      l_run[hh] += pv[hh];
+    }
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+      const uint32_t w4[4] = {vv[c].x, vv[c].y, vv[c].z, vv[c].w};
+      float pw[G];
+#pragma unroll
+      for (int hh = 0; hh < G; ++hh) pw[hh] = __shfl(pv[hh], c * PP + pp, WAVE);
+#pragma unroll
+      for (int hh = 0; hh < G; ++hh)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          acc[hh][2 * i] += pw * lo_bf(w4[i]);
-          acc[hh][2 * i + 1] += pw * hi_bf(w4[i]);
+          acc[hh][2 * i] += pw[hh] * lo_bf(w4[i]);
+          acc[hh][2 * i + 1] += pw[hh] * hi_bf(w4[i]);
         }
-      }
     }
     if (more) cur = nxt;
   }
 
-  // fold the PP row-groups of the wave, then the four waves
+  // fold the sums over the 16 positions of a tile (every lane of a quarter holds the same share),
+  // the PP row-groups of the wave, then the four waves
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1)
+#pragma unroll
+    for (int hh = 0; hh < G; ++hh) l_run[hh] += __shfl_xor(l_run[hh], o, WAVE);
 #pragma unroll
   for (int hh = 0; hh < G; ++hh) {
 #pragma unroll
