@@ -36,6 +36,7 @@ namespace {
 
 #define OHARA_MEGA_NS 16  // context chunks per (sequence, kv head)
 #define OHARA_MAX_PF 24   // weight tiles (16 B per lane) a wave fetches ahead of a phase
+#define OHARA_DOWN_SPLIT 4  // K partitions of the down projection (static_assert below: x_load sums four)
 
 struct MegaArgs {
   OharaModel m;                 // by value; the layer table is read from layers_dev
@@ -50,7 +51,8 @@ struct MegaArgs {
   char* qm;        // NL q-mailboxes of qm_stride bytes
   char* am;        // NL act-mailboxes of am_stride bytes
   float* pm;       // NL partial mailboxes of pm_stride floats: [b*H + h][chunk][Dh + 32]
-  size_t xm_stride, qm_stride, am_stride, pm_stride;
+  float* dm;       // NL mailboxes of dm_stride floats: partial sums of the down projection [part][b][d]
+  size_t xm_stride, qm_stride, am_stride, pm_stride, dm_stride;
   float* cand_val; // (nwg, B)
   int* cand_idx;   // (nwg, B)
   bf16_t* logits;  // (B, V)
@@ -171,6 +173,52 @@ __device__ __forceinline__ const char* am_addr(const char* base, int blk, int b,
   return base + (size_t)(f >> 3) * blk + b * 16 + (f & 7) * 2;
 }
 
+// The down projection is split along K over OHARA_DOWN_SPLIT groups of workgroups (a 16-row strip
+// of it is too much for one CU to stream); each group leaves an fp32 partial sum [part][b][n] and
+// whoever needs the residual stream after the block forms it on the fly, in a fixed order:
+//   x[b][n] = bf16(x_mid[b][n] + bf16(((p0 + p1) + p2) + p3))        (llama.py:200)
+struct XParts {
+  const char* xmid;   // x mailbox holding the stream before the feed-forward block
+  const float* parts; // partial sums; nullptr: `xmid` already is the stream that is wanted
+  int blk, B, N;
+};
+
+template <int NW>  // NW columns (4 or 8) starting at n, n % NW == 0
+__device__ __forceinline__ void x_load(const XParts& xp, int b, int n, uint32_t (&out)[NW / 2]) {
+  uint32_t xm[NW / 2];
+  if (NW == 8) {
+    const uint4 v = ldg16(xm_addr(xp.xmid, xp.blk, b, n));
+    xm[0] = v.x; xm[1] = v.y; xm[NW / 2 - 2] = v.z; xm[NW / 2 - 1] = v.w;
+  } else {
+    const uint2 v = ldg8(xm_addr(xp.xmid, xp.blk, b, n));
+    xm[0] = v.x; xm[1] = v.y;
+  }
+  if (!xp.parts) {
+#pragma unroll
+    for (int i = 0; i < NW / 2; ++i) out[i] = xm[i];
+    return;
+  }
+  uint4 pv[OHARA_DOWN_SPLIT][NW / 4];
+#pragma unroll
+  for (int q = 0; q < OHARA_DOWN_SPLIT; ++q)
+#pragma unroll
+    for (int i = 0; i < NW / 4; ++i) pv[q][i] = ldg16(xp.parts + ((size_t)(q * xp.B + b) * xp.N + n + 4 * i));
+#pragma unroll
+  for (int i = 0; i < NW / 4; ++i) {
+    float y[4];
+    const uint32_t w[OHARA_DOWN_SPLIT][4] = {{pv[0][i].x, pv[0][i].y, pv[0][i].z, pv[0][i].w},
+                                             {pv[1][i].x, pv[1][i].y, pv[1][i].z, pv[1][i].w},
+                                             {pv[2][i].x, pv[2][i].y, pv[2][i].z, pv[2][i].w},
+                                             {pv[3][i].x, pv[3][i].y, pv[3][i].z, pv[3][i].w}};
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      y[e] = rbf(((__uint_as_float(w[0][e]) + __uint_as_float(w[1][e])) + __uint_as_float(w[2][e])) +
+                 __uint_as_float(w[3][e]));
+    out[2 * i] = pack_bf(lo_bf(xm[2 * i]) + y[0], hi_bf(xm[2 * i]) + y[1]);
+    out[2 * i + 1] = pack_bf(lo_bf(xm[2 * i + 1]) + y[2], hi_bf(xm[2 * i + 1]) + y[3]);
+  }
+}
+
 // ---------------------------------------------------------------------------------------
 // staging of the GEMM activations in LDS: xs[b][ldxs] bf16
 // ---------------------------------------------------------------------------------------
@@ -179,8 +227,9 @@ __device__ __forceinline__ const char* am_addr(const char* base, int blk, int b,
 // - on rows gathered from the embedding table (llama.py:310).  One wave per row; all loads
 // of a row are issued before any is consumed.  K <= 8 * 64 * NLD elements.
 template <int NLD, bool EMBED>
-__device__ void stage_norm(bf16_t* xs, int ldxs, const char* src, int blk, const int64_t* ids, const bf16_t* table,
-                           int vocab, const bf16_t* nw, float eps, int B, int K) {
+__device__ void stage_norm(bf16_t* xs, int ldxs, const char* src, int blk, const float* parts, const int64_t* ids,
+                           const bf16_t* table, int vocab, const bf16_t* nw, float eps, int B, int K) {
+  const XParts xp{src, parts, blk, B, K};
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int b = wave; b < B; b += 4) {
     uint4 v[NLD], g[NLD];
@@ -196,8 +245,13 @@ __device__ void stage_norm(bf16_t* xs, int ldxs, const char* src, int blk, const
       v[c] = make_uint4(0, 0, 0, 0);
       g[c] = make_uint4(0, 0, 0, 0);
       if (k < K) {
-        if (EMBED) v[c] = ldg16(table + row_off + k);
-        else v[c] = ldg16(xm_addr(src, blk, b, k));
+        if (EMBED) {
+          v[c] = ldg16(table + row_off + k);
+        } else {
+          uint32_t w[4];
+          x_load<8>(xp, b, k, w);
+          v[c] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
         g[c] = ldg16(nw + k);
       }
     }
@@ -230,10 +284,11 @@ __device__ void stage_norm(bf16_t* xs, int ldxs, const char* src, int blk, const
 }
 
 // act mailbox (B, F) -> LDS
-__device__ void stage_act(bf16_t* xs, int ldxs, const char* src, int blk, int B, int F) {
-  const int n8 = F >> 3;
+// act mailbox (B, F), columns [f0, f1) (multiples of 8) -> LDS
+__device__ void stage_act(bf16_t* xs, int ldxs, const char* src, int blk, int B, int f0, int f1) {
+  const int n8 = (f1 - f0) >> 3;
   for (int i = threadIdx.x; i < B * n8; i += blockDim.x) {
-    const int b = i / n8, c = i - b * n8;
+    const int b = i / n8, c = (f0 >> 3) + i - b * n8;
     sts16(xs + (size_t)b * ldxs + c * 8, ldg16(am_addr(src, blk, b, c * 8)));
   }
 }
@@ -349,7 +404,7 @@ __device__ void stage_attn_merge_small(bf16_t* xs, int ldxs, const float* pm, in
 // weights of a workgroup's first strip(s) - and the residual it will add - are fetched
 // into registers between arrive() and wait() of the barrier that precedes the phase.
 // ---------------------------------------------------------------------------------------
-enum { E_RESID = 1, E_SWIGLU = 2, E_ROPE = 3, E_LOGITS = 4 };
+enum { E_RESID = 1, E_SWIGLU = 2, E_ROPE = 3, E_LOGITS = 4, E_PART = 5 };
 
 struct GemmP {
   const uint4* wp;
@@ -357,8 +412,11 @@ struct GemmP {
   int nstrips;
   char* out;       // output mailbox (E_ROPE: q; E_RESID: x; E_SWIGLU: act) or logits
   int blk;         // its block size
-  const char* resid;      // E_RESID: x mailbox to add
+  const char* resid;      // E_RESID: x mailbox to add ...
+  const float* resid_parts;  // ... plus, when set, the partial sums of the previous block's down projection
   int resid_embed;        // E_RESID: add the embedding rows instead (first half layer)
+  float* pout;            // E_PART: partial sums [part][b][n] (fp32, not rounded); K is split over
+                          // OHARA_DOWN_SPLIT groups of workgroups, unit = part * nstrips + strip
   const int64_t* ids;     // E_RESID with resid == nullptr
   const bf16_t* table;
   int vocab;
@@ -376,26 +434,47 @@ struct GemmPre {  // one register buffer, reused by every phase (only one prefet
   uint2 r;        // E_RESID: the four residual values of this lane (first strip)
 };
 
+// Work unit -> strip and this wave's k-steps [j0, j1).  E_PART: the units of K partition q follow
+// those of partition q - 1, so the partitions of a strip land on different workgroups.
+template <int KP, int EPI>
+__device__ __forceinline__ bool gemm_unit(const GemmP& p, int unit, int kpart, int KS, int& strip, int& j0, int& j1) {
+  int kq = 0, KSq = KS;
+  strip = unit;
+  bool live = unit < p.nstrips;
+  if (EPI == E_PART) {
+    kq = unit / p.nstrips;
+    strip = unit - kq * p.nstrips;
+    KSq = (KS + OHARA_DOWN_SPLIT - 1) / OHARA_DOWN_SPLIT;
+    live = kq < OHARA_DOWN_SPLIT;
+  }
+  const int per = (KSq + KP - 1) / KP;
+  const int kend = min(KS, (kq + 1) * KSq);
+  j0 = kq * KSq + kpart * per;
+  j1 = min(kend, j0 + per);
+  return live;
+}
+
 template <int KP, int PF, int EPI>
 __device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int B) {
   constexpr int SPW = 4 / KP;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = wave / KP, kpart = wave % KP;
   const int KS = (p.K + 31) >> 5;
-  const int per = (KS + KP - 1) / KP;
-  const int j0 = kpart * per, j1 = min(KS, j0 + per);
-  const int strip = (int)blockIdx.x * SPW + sub;
+  int strip, j0, j1;
+  const bool live = gemm_unit<KP, EPI>(p, (int)blockIdx.x * SPW + sub, kpart, KS, strip, j0, j1);
   const uint4* wrow = p.wp + (size_t)strip * KS * 64 + lane;
 #pragma unroll
   for (int c = 0; c < PF; ++c)
-    pre.w[c] = (strip < p.nstrips && j0 + c < j1) ? ldg16_nt(wrow + (size_t)(j0 + c) * 64) : make_uint4(0, 0, 0, 0);
+    pre.w[c] = (live && j0 + c < j1) ? ldg16_nt(wrow + (size_t)(j0 + c) * 64) : make_uint4(0, 0, 0, 0);
   if (EPI == E_RESID) {
     const int m = lane & 15, g = lane >> 4;
     const int r0 = strip * 16 + 4 * g;
     pre.r = make_uint2(0, 0);
-    if (strip < p.nstrips && kpart == 0 && m < B && r0 < p.N) {
+    if (live && kpart == 0 && m < B && r0 < p.N) {
       if (!p.resid_embed) {
-        pre.r = ldg8(xm_addr(p.resid, p.blk, m, r0));
+        uint32_t w[2];
+        x_load<4>(XParts{p.resid, p.resid_parts, p.blk, B, p.N}, m, r0, w);
+        pre.r = make_uint2(w[0], w[1]);
       } else {
         int64_t id = ldg_i64(p.ids + m);
         if (id < 0 || id >= p.vocab) id = 0;
@@ -413,17 +492,17 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
   const int m = lane & 15, g = lane >> 4;
   const int sub = wave / KP, kpart = wave % KP;
   const int KS = (p.K + 31) >> 5;
-  const int per = (KS + KP - 1) / KP;
-  const int j0 = kpart * per, j1 = min(KS, j0 + per);
   const int nwg = gridDim.x;
-  const int iters = (p.nstrips + nwg * SPW - 1) / (nwg * SPW);
+  const int nunits = EPI == E_PART ? p.nstrips * OHARA_DOWN_SPLIT : p.nstrips;
+  const int iters = (nunits + nwg * SPW - 1) / (nwg * SPW);
   const bool mine = m < B;
   const bf16_t* xrow = xs + (size_t)m * ldxs + 8 * g;
 
 #pragma unroll 1
   for (int it = 0; it < iters; ++it) {
-    const int strip = (it * nwg + blockIdx.x) * SPW + sub;
-    const bool live = strip < p.nstrips;
+    const int unit = (it * nwg + blockIdx.x) * SPW + sub;
+    int strip, j0, j1;
+    const bool live = gemm_unit<KP, EPI>(p, unit, kpart, KS, strip, j0, j1);
     f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
     if (live) {
       const uint4* wrow = p.wp + (size_t)strip * KS * 64 + lane;
@@ -472,7 +551,9 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
           uint2 r = pre.r;
           if (it > 0) {
             if (!p.resid_embed) {
-              r = ldg8(xm_addr(p.resid, p.blk, b, r0));
+              uint32_t w[2];
+              x_load<4>(XParts{p.resid, p.resid_parts, p.blk, B, p.N}, b, r0, w);
+              r = make_uint2(w[0], w[1]);
             } else {
               int64_t id = ldg_i64(p.ids + b);
               if (id < 0 || id >= p.vocab) id = 0;
@@ -481,6 +562,12 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
           }
           st_coh8(const_cast<char*>(xm_addr(p.out, p.blk, b, r0)),
                   make_uint2(pack_bf(lo_bf(r.x) + y0, hi_bf(r.x) + y1), pack_bf(lo_bf(r.y) + y2, hi_bf(r.y) + y3)));
+        }
+      } else if (EPI == E_PART) {  // the raw fp32 sums of this K partition
+        if (r0 < p.N) {
+          float* o = p.pout + ((size_t)((unit / p.nstrips) * B + b) * p.N + r0);
+          st_coh8(o, make_uint2(__float_as_uint(acc[0]), __float_as_uint(acc[1])));
+          st_coh8(o + 2, make_uint2(__float_as_uint(acc[2]), __float_as_uint(acc[3])));
         }
       } else if (EPI == E_LOGITS) {
         const float v[4] = {y0, y1, y2, y3};
@@ -774,8 +861,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   prj.N = d; prj.K = H * D; prj.nstrips = (d + 15) / 16; prj.blk = a.blk_x;
   prj.ids = a.ids; prj.table = m.token_emb; prj.vocab = V;
   gu.N = F; gu.K = d; gu.nstrips = 2 * ((F + 7) / 8 * 8) / 16; gu.blk = a.blk_a;
-  dn.N = d; dn.K = F; dn.nstrips = (d + 15) / 16; dn.blk = a.blk_x;
-  dn.ids = a.ids; dn.table = m.token_emb; dn.vocab = V;
+  dn.N = d; dn.K = F; dn.nstrips = (d + 15) / 16;
   lm.N = V; lm.K = d; lm.nstrips = (V + 15) / 16; lm.out = reinterpret_cast<char*>(a.logits); lm.ldo = V;
   lm.valid = a.valid_vocab > 0 ? min(a.valid_vocab, V) : V;
   lm.wp = reinterpret_cast<const uint4*>(m.w_vocab);
@@ -789,17 +875,19 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     const unsigned long long* pl = ptab + l * 8;
     bf16_t* kc = lds_ptr<bf16_t>(pl, 6);
     bf16_t* vc = lds_ptr<bf16_t>(pl, 7);
-    const char* x_in = a.xm + (size_t)(2 * l) * a.xm_stride;       // residual stream entering the layer
     char* x_mid = a.xm + (size_t)(2 * l + 1) * a.xm_stride;        // after attention
-    char* x_out = a.xm + (size_t)(2 * l + 2) * a.xm_stride;        // after the feed-forward
+    // the stream entering layer l > 0 is x_mid of layer l - 1 plus that layer's down-projection sums
+    const char* x_prev = a.xm + (size_t)(l > 0 ? 2 * l - 1 : 0) * a.xm_stride;
+    const float* d_prev = l > 0 ? a.dm + (size_t)(l - 1) * a.dm_stride : nullptr;
+    float* d_l = a.dm + (size_t)l * a.dm_stride;
     char* q_l = a.qm + (size_t)l * a.qm_stride;
     char* a_l = a.am + (size_t)l * a.am_stride;
     float* p_l = a.pm + (size_t)l * a.pm_stride;
     // P1: [embedding] + norm1 + QKV + rotary + append
     qkv.kc = kc; qkv.vc = vc; qkv.out = q_l;
     if ((int)blockIdx.x < qkv.nstrips) {
-      if (l == 0) stage_norm<2, true>(xs, ldxs, a.xm, 0, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d);
-      else stage_norm<2, false>(xs, ldxs, x_in, a.blk_x, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d);
+      if (l == 0) stage_norm<2, true>(xs, ldxs, a.xm, 0, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d);
+      else stage_norm<2, false>(xs, ldxs, x_prev, a.blk_x, d_prev, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d);
     }
     __syncthreads();
     pf.stamp();
@@ -812,7 +900,8 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     // P2: attention partials
     attn_phase<D, G>(B, H, Hkv, m.t_max, a.blk_x, a.ns, apre, q_l, p_l, kc, vc, L, att);
     gs.arrive(pf);
-    prj.wp = lds_ptr<const uint4>(pl, 1); prj.out = x_mid; prj.resid = x_in; prj.resid_embed = l == 0;
+    prj.wp = lds_ptr<const uint4>(pl, 1); prj.out = x_mid; prj.resid = x_prev; prj.resid_parts = d_prev;
+    prj.resid_embed = l == 0;
     gemm_prefetch<4, 6, E_RESID>(prj, pre, B);
     gs.wait(pf);
     pf.stamp();
@@ -831,18 +920,27 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     gs.wait(pf);
     pf.stamp();
     // P4: norm2 + gate/up + SwiGLU
-    if ((int)blockIdx.x * 2 < gu.nstrips) stage_norm<2, false>(xs, ldxs, x_mid, a.blk_x, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 5), m.eps, B, d);
+    if ((int)blockIdx.x * 2 < gu.nstrips) stage_norm<2, false>(xs, ldxs, x_mid, a.blk_x, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 5), m.eps, B, d);
     __syncthreads();
     gemm_phase<2, 12, E_SWIGLU>(gu, pre, xs, ldxs, B, red, best_v, best_i, pf);
     gs.arrive(pf);
-    dn.wp = lds_ptr<const uint4>(pl, 3); dn.out = x_out; dn.resid = x_mid;
-    gemm_prefetch<4, 24, E_RESID>(dn, pre, B);
+    dn.wp = lds_ptr<const uint4>(pl, 3); dn.pout = d_l;
+    gemm_prefetch<4, 6, E_PART>(dn, pre, B);
     gs.wait(pf);
     pf.stamp();
-    // P5: down projection + residual
-    if ((int)blockIdx.x < dn.nstrips) stage_act(xs, ldxs, a_l, a.blk_a, B, F);
+    // P5: down projection, K split over OHARA_DOWN_SPLIT groups of workgroups; a workgroup stages
+    // only the columns of its partition (all of them when it will take more than one unit)
+    {
+      const int nunits = dn.nstrips * OHARA_DOWN_SPLIT;
+      if ((int)blockIdx.x < nunits) {
+        const int KSq = (((F + 31) >> 5) + OHARA_DOWN_SPLIT - 1) / OHARA_DOWN_SPLIT;
+        const int kq = (int)blockIdx.x / dn.nstrips;
+        const bool whole = nunits > (int)gridDim.x;
+        stage_act(xs, ldxs, a_l, a.blk_a, B, whole ? 0 : min(F, kq * KSq * 32), whole ? F : min(F, (kq + 1) * KSq * 32));
+      }
+    }
     __syncthreads();
-    gemm_phase<4, 24, E_RESID>(dn, pre, xs, ldxs, B, red, best_v, best_i, pf);
+    gemm_phase<4, 6, E_PART>(dn, pre, xs, ldxs, B, red, best_v, best_i, pf);
     gs.arrive(pf);
     if (l + 1 < m.n_layers) {
       qkv.wp = lds_ptr<const uint4>(pl, 8);
@@ -854,8 +952,8 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     pf.stamp();
   }
   // final norm + vocabulary projection, running arg-max per lane
-  stage_norm<2, false>(xs, ldxs, a.xm + (size_t)(2 * m.n_layers) * a.xm_stride, a.blk_x, a.ids, m.token_emb, V,
-                       m.final_norm, m.eps, B, d);
+  stage_norm<2, false>(xs, ldxs, a.xm + (size_t)(2 * m.n_layers - 1) * a.xm_stride, a.blk_x,
+                       a.dm + (size_t)(m.n_layers - 1) * a.dm_stride, a.ids, m.token_emb, V, m.final_norm, m.eps, B, d);
   __syncthreads();
   gemm_phase<1, 24, E_LOGITS>(lm, pre, xs, ldxs, B, red, best_v, best_i, pf);
   pf.stamp();
@@ -943,8 +1041,8 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
 size_t mega_al(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct MegaLayout {
-  size_t layers, kptr, vptr, xm, qm, am, pm, candv, candi, prof, bar, total;
-  size_t xm_stride, qm_stride, am_stride, pm_stride;
+  size_t layers, kptr, vptr, xm, qm, am, pm, dm, candv, candi, prof, bar, total;
+  size_t xm_stride, qm_stride, am_stride, pm_stride, dm_stride;
   int blk_x, blk_a;
 };
 
@@ -966,6 +1064,8 @@ MegaLayout mega_layout(const OharaModel* m, int B, int nwg) {
   L.qm = o; o += L.qm_stride * NL;
   L.am = o; o += L.am_stride * NL;
   L.pm = o; o += L.pm_stride * sizeof(float) * NL;
+  L.dm_stride = mega_al((size_t)OHARA_DOWN_SPLIT * B * m->d_model * sizeof(float)) / sizeof(float);
+  L.dm = o; o += L.dm_stride * sizeof(float) * NL;
   L.candv = o; o += mega_al((size_t)nwg * B * sizeof(float));
   L.candi = o; o += mega_al((size_t)nwg * B * sizeof(int));
   L.prof = o; o += mega_al(OHARA_PROF_SLOTS * sizeof(unsigned long long));
@@ -1018,6 +1118,7 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   a.vcache_dev = reinterpret_cast<uint16_t* const*>(ws + L.vptr);
   a.xm = ws + L.xm; a.qm = ws + L.qm; a.am = ws + L.am; a.pm = reinterpret_cast<float*>(ws + L.pm);
   a.xm_stride = L.xm_stride; a.qm_stride = L.qm_stride; a.am_stride = L.am_stride; a.pm_stride = L.pm_stride;
+  a.dm = reinterpret_cast<float*>(ws + L.dm); a.dm_stride = L.dm_stride;
   a.blk_x = L.blk_x; a.blk_a = L.blk_a;
   a.cand_val = reinterpret_cast<float*>(ws + L.candv);
   a.cand_idx = reinterpret_cast<int*>(ws + L.candi);
