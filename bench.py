@@ -188,7 +188,7 @@ def bench_attention_microbench(dev):
 
     H, Hkv, D = 32, 8, 128
     out = []
-    for B, L in ((1, 4096), (1, 32768), (16, 4096), (16, 32768), (64, 4096), (64, 32768)):
+    for B, L in ((b, l) for b in (1, 16, 64) for l in (1024, 4096, 16384, 32768)):
         ns = max(1, min(1024 // (B * Hkv), L // 128, 64))
         g = torch.Generator(device=dev).manual_seed(1)
         q = torch.randn(B, H * D, device=dev, generator=g).to(torch.bfloat16)

@@ -110,6 +110,12 @@ int ohara_qkv_rope_append_bf16(const uint16_t* x, int ldx, const uint16_t* wp, i
 /* The same projection + rotary, with the rotated k and the v rows written to (batch*seq_len,
  * h_kv*dh) buffers instead of into a cache (the int8 cache quantises them in a second step).
  * t_max only bounds the positions. */
+/* ohara_qkv_rope_append_bf16 with one cache position per sequence: token s of sequence b is
+ * rotated for, and appended at, position seq_pos[b] + s (device array, `batch` entries). */
+int ohara_qkv_rope_append_ragged_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int k, const uint16_t* norm_w,
+                                      float eps, int batch, int seq_len, int h, int h_kv, int dh, const uint16_t* cos,
+                                      const uint16_t* sin, const int32_t* seq_pos, uint16_t* q_out, uint16_t* kcache,
+                                      uint16_t* vcache, int t_max, void* stream);
 int ohara_qkv_rope_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int k, const uint16_t* norm_w, float eps,
                         int batch, int seq_len, int h, int h_kv, int dh, const uint16_t* cos, const uint16_t* sin,
                         int pos, const int32_t* pos_dev, int t_max, uint16_t* q_out, uint16_t* k_out, uint16_t* v_out,
@@ -131,6 +137,14 @@ int64_t ohara_attn_workspace_bytes(int batch, int h, int h_kv, int dh, int n_spl
 int ohara_attn_cached_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch,
                            int seq_len, int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev,
                            int n_split, void* workspace, uint16_t* out, void* stream);
+/* The same with one position per sequence: query s of sequence b sits at seq_pos[b] + s and sees
+ * [0, seq_pos[b] + s].  No counterpart in the reference (one scalar position, llama.py:287-299). */
+int ohara_attn_cached_ragged_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch,
+                                  int seq_len, int h, int h_kv, int dh, int t_max, const int32_t* seq_pos, int n_split,
+                                  void* workspace, uint16_t* out, void* stream);
+/* seq_pos[b] += by for every b with active[b] != 0 (active NULL: all): advances a ragged batch by one
+ * decode step without host involvement (graph replay). */
+int ohara_advance_positions(int32_t* seq_pos, const uint8_t* active, int batch, int by, void* stream);
 
 /* Same contract for many query positions per sequence (prefill), as a causal flash-style kernel
  * on MFMA: 128 queries per workgroup, keys/values walked in 64-position tiles through LDS,
@@ -341,6 +355,11 @@ typedef struct OharaDecodeState {
   uint16_t* vstage;
   uint16_t* kdeq;
   uint16_t* vdeq;
+  /* ragged batches: when non-NULL, sequence b's first fed token sits at cache position seq_pos[b]
+     (device array of `batch` entries) and the pos / use_pos_dev arguments are ignored.  The
+     reference has one scalar position for the whole batch (llama.py:287-299); this is what lets
+     sequences of different lengths decode in one batch.  bf16 caches only. */
+  const int32_t* seq_pos;
   void* prof_start;      /* hipEvent_t recorded on `stream` right before launch prof_kernel */
   void* prof_stop;       /* hipEvent_t recorded right after it                             */
 } OharaDecodeState;

@@ -42,7 +42,7 @@ class OharaDecodeState(C.Structure):
         ("kcache", C.POINTER(_p)), ("vcache", C.POINTER(_p)),
         ("kv_int8", _i), ("kscale", C.POINTER(_p)), ("kmin", C.POINTER(_p)), ("vscale", C.POINTER(_p)),
         ("vmin", C.POINTER(_p)), ("kstage", _p), ("vstage", _p), ("kdeq", _p), ("vdeq", _p),
-        ("prof_start", _p), ("prof_stop", _p),
+        ("seq_pos", _p), ("prof_start", _p), ("prof_stop", _p),
     ]
 
 
@@ -63,6 +63,9 @@ _PROTOS = {
     "ohara_attn_cached_int8": (_i, [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
     "ohara_attn_workspace_bytes": (_i64, [_i, _i, _i, _i, _i]),
     "ohara_attn_cached_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
+    "ohara_attn_cached_ragged_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
+    "ohara_qkv_rope_append_ragged_bf16": (_i, [_p, _i, _p, _i, _p, _f, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _i, _p]),
+    "ohara_advance_positions": (_i, [_p, _p, _i, _i, _p]),
     "ohara_attn_prefill_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p]),
     "ohara_argmax_bf16": (_i, [_p, _i, _i, _i, _i, _p, _p, _i, _p, _p]),
     "ohara_sample_topk_topp": (_i, [_p, _i, _i, _i, _i, _i, _f, _i, _f, _p, _i, _p, _p, _i, _p, _p]),

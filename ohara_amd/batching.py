@@ -1,0 +1,107 @@
+"""Continuous batching on the decode path: sequences of different lengths share one batch, join
+when a slot is free and leave when they finish.
+
+The reference drives `Llama.forward` with a single scalar position for the whole batch
+(ohara/models/llama.py:287-299, ohara/chat_engine.py:395-405), so all sequences of a batch must
+have the same length and start together.  Here every slot of the KV caches has its own length: a
+prompt is prefilled into its slot alone, and one decode step advances every active slot at its own
+position (`Llama.forward` with one position per sequence).  Selection is greedy or the fused
+temperature / top-k / top-p sampler of ohara/chat_engine.py:51-82.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import ops
+from .llama import BF16, Llama
+
+
+class ContinuousBatcher:
+    def __init__(self, model: Llama, slots: int, sampling=None, valid_vocab: int = 0, generator=None):
+        if slots < 1:
+            raise ValueError("batch_size must be at least 1")
+        self.model, self.slots = model, slots
+        self.sampling = sampling if (sampling is not None and sampling.temperature > 0) else None
+        self.valid_vocab = valid_vocab
+        self.generator = generator
+        self.cache = model.build_kv_cache(slots)
+        for c in self.cache:
+            c._commit_ragged(slots, [0] * slots)
+        self.active = [False] * slots
+        self.lengths = [0] * slots
+        self.last = torch.zeros(slots, dtype=torch.int64, device=model.device)
+        self.seq_pos = torch.zeros(slots, dtype=torch.int32, device=model.device)
+        self.active_dev = torch.zeros(slots, dtype=torch.uint8, device=model.device)
+
+    def free_slots(self) -> list[int]:
+        return [b for b in range(self.slots) if not self.active[b]]
+
+    def _select(self, logits: torch.Tensor) -> torch.Tensor:
+        """logits (rows, V) -> ids (rows,) on the device."""
+        vv = self.valid_vocab or None
+        if self.sampling is None:
+            return ops.argmax(logits, valid_vocab=vv)
+        u = torch.rand(logits.shape[0], device=logits.device, dtype=torch.float32, generator=self.generator)
+        return ops.sample_topk_topp(logits, self.sampling.temperature, self.sampling.top_k, self.sampling.top_p, u,
+                                    valid_vocab=vv)
+
+    @torch.no_grad()
+    def add(self, prompt_ids) -> tuple[int, int]:
+        """Prefill a prompt (1-D ids) into a free slot -> (slot, first generated id)."""
+        free = self.free_slots()
+        if not free:
+            raise RuntimeError("no free slot")
+        ids = torch.as_tensor(prompt_ids, dtype=torch.int64).reshape(1, -1)
+        if ids.shape[1] < 1:
+            raise ValueError("input sequence cannot be empty")
+        if ids.shape[1] >= self.model.config.max_sequence_length:
+            raise ValueError("input exceeds max_sequence_length")
+        b = free[0]
+        for c in self.cache:
+            c.lengths[b] = 0
+        views = [c._row_view(b) for c in self.cache]
+        logits = self.model.forward(ids.to(self.model.device), views, 0, last_only=True)
+        tok = self._select(logits.view(1, -1))
+        n = ids.shape[1]
+        for c in self.cache:
+            c.lengths[b] = n
+            c.length = max(c.lengths)
+        self.lengths[b] = n
+        self.active[b] = True
+        self.last[b:b + 1] = tok
+        self.seq_pos[b] = n
+        self.active_dev[b] = 1
+        return b, int(tok.item())
+
+    def remove(self, slot: int) -> None:
+        self.active[slot] = False
+        self.lengths[slot] = 0
+        self.last[slot] = 0
+        self.seq_pos[slot] = 0
+        self.active_dev[slot] = 0
+        for c in self.cache:
+            c.lengths[slot] = 0
+
+    @torch.no_grad()
+    def step(self) -> dict[int, int]:
+        """One decode step for every active slot -> {slot: new id}.  Idle slots ride along at
+        position 0 of their own cache rows (overwritten when the slot is taken again)."""
+        if not any(self.active):
+            return {}
+        if max(n for n, a in zip(self.lengths, self.active) if a) + 1 > self.model.config.max_sequence_length:
+            raise ValueError("input exceeds max_sequence_length")
+        logits = self.model.forward(self.last.view(self.slots, 1), self.cache, list(self.lengths), last_only=True,
+                                    seq_pos=self.seq_pos)
+        toks = self._select(logits.view(self.slots, -1))
+        # idle slots stay at position 0; active ones advance on the device and in the host's books
+        ops.advance_positions(self.seq_pos, self.active_dev, 1)
+        self.last.copy_(torch.where(self.active_dev.bool(), toks, torch.zeros_like(toks)))
+        for b in range(self.slots):
+            if self.active[b]:
+                self.lengths[b] += 1
+        for c in self.cache:
+            c.lengths = list(self.lengths)
+            c.length = max(self.lengths)
+        host = toks.tolist()
+        return {b: host[b] for b in range(self.slots) if self.active[b]}

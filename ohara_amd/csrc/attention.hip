@@ -24,7 +24,8 @@ struct AttnArgs {
   const float* vmin;
   bf16_t* out;       // (B, H*D)
   int B, S, H, Hkv, D, Tmax, start;  // query s of sequence b sees positions [0, start + s]
-  const int32_t* pos_dev;            // when set: start = *pos_dev
+  const int32_t* pos_dev;            // when set: start = *pos_dev, or pos_dev[sequence] with pos_stride 1
+  int pos_stride;
   int nsplit;
   int* counters;     // (B*Hkv)
   float* part_ml;    // (B, H, nsplit, 2)
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   constexpr int NV = 16 / PP;       // V load instructions per 16-position tile
   const int split = blockIdx.z, kvh = blockIdx.y, b = blockIdx.x;  // b: query row = seq * S + s
   const int seq = b / a.S;
-  const int L = min((a.pos_dev ? *a.pos_dev : a.start) + (b - seq * a.S) + 1, a.Tmax);
+  const int L = min((a.pos_dev ? a.pos_dev[(size_t)seq * a.pos_stride] : a.start) + (b - seq * a.S) + 1, a.Tmax);
   const int chunk = (((L + a.nsplit - 1) / a.nsplit) + 63) & ~63;
   const int t0 = split * chunk;
   const int t1 = min(L, t0 + chunk);
@@ -372,7 +373,7 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
   const int split = blockIdx.z, kvh = blockIdx.y, b = blockIdx.x;
   const int seq = b / a.S;
   const int G = a.H / a.Hkv, D = a.D;
-  const int L = min((a.pos_dev ? *a.pos_dev : a.start) + (b - seq * a.S) + 1, a.Tmax);
+  const int L = min((a.pos_dev ? a.pos_dev[(size_t)seq * a.pos_stride] : a.start) + (b - seq * a.S) + 1, a.Tmax);
   const int chunk = (((L + a.nsplit - 1) / a.nsplit) + 63) & ~63;
   const int t0 = split * chunk;
   const int t1 = min(L, t0 + chunk);
@@ -480,7 +481,7 @@ int64_t ohara_attn_workspace_bytes(int batch, int h, int h_kv, int dh, int n_spl
 
 static int attn_cached_impl(const uint16_t* q, const void* kcache, const void* vcache, const float* kscale,
                             const float* kmin, const float* vscale, const float* vmin, bool i8, int batch, int seq_len,
-                            int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev, int n_split,
+                            int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev, int pos_stride, int n_split,
                             void* workspace, uint16_t* out, void* stream) {
   if (!q || !kcache || !vcache || !out) return OHARA_EINVAL;
   if (i8 && (!kscale || !kmin || !vscale || !vmin)) return OHARA_EINVAL;
@@ -495,6 +496,7 @@ static int attn_cached_impl(const uint16_t* q, const void* kcache, const void* v
   a.q = q; a.k = reinterpret_cast<const bf16_t*>(kcache); a.v = reinterpret_cast<const bf16_t*>(vcache); a.out = out;
   a.kscale = kscale; a.kmin = kmin; a.vscale = vscale; a.vmin = vmin;
   a.B = batch; a.S = seq_len; a.H = h; a.Hkv = h_kv; a.D = dh; a.Tmax = t_max; a.start = pos; a.pos_dev = pos_dev;
+  a.pos_stride = pos_stride;
   a.nsplit = n_split;
   batch *= seq_len;  // one workspace slot per query row
   char* ws = reinterpret_cast<char*>(workspace);
@@ -524,7 +526,15 @@ int ohara_attn_cached_bf16(const uint16_t* q, const uint16_t* kcache, const uint
                            int seq_len, int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev,
                            int n_split, void* workspace, uint16_t* out, void* stream) {
   return attn_cached_impl(q, kcache, vcache, nullptr, nullptr, nullptr, nullptr, false, batch, seq_len, h, h_kv, dh,
-                          t_max, pos, pos_dev, n_split, workspace, out, stream);
+                          t_max, pos, pos_dev, 0, n_split, workspace, out, stream);
+}
+
+int ohara_attn_cached_ragged_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch,
+                                  int seq_len, int h, int h_kv, int dh, int t_max, const int32_t* seq_pos, int n_split,
+                                  void* workspace, uint16_t* out, void* stream) {
+  if (!seq_pos) return OHARA_EINVAL;
+  return attn_cached_impl(q, kcache, vcache, nullptr, nullptr, nullptr, nullptr, false, batch, seq_len, h, h_kv, dh,
+                          t_max, 0, seq_pos, 1, n_split, workspace, out, stream);
 }
 
 int ohara_attn_cached_int8(const uint16_t* q, const int8_t* kcache, const int8_t* vcache, const float* kscale,
@@ -532,7 +542,7 @@ int ohara_attn_cached_int8(const uint16_t* q, const int8_t* kcache, const int8_t
                            int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev, int n_split, void* workspace,
                            uint16_t* out, void* stream) {
   return attn_cached_impl(q, kcache, vcache, kscale, kmin, vscale, vmin, true, batch, seq_len, h, h_kv, dh, t_max, pos,
-                          pos_dev, n_split, workspace, out, stream);
+                          pos_dev, 0, n_split, workspace, out, stream);
 }
 
 }  // extern "C"

@@ -17,8 +17,10 @@ extern "C" int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* 
   if (s->batch < 1 || seq_len < 1) return OHARA_EINVAL;
   const int64_t rows64 = (int64_t)s->batch * seq_len;
   if (rows64 > s->rows_cap) return OHARA_ESIZE;
-  if (use_pos_dev && (!s->step_state || seq_len != 1)) return OHARA_EINVAL;
-  if (!use_pos_dev && (pos < 0 || pos + seq_len > m->t_max)) return OHARA_EINVAL;
+  const bool ragged = s->seq_pos != nullptr;
+  if (ragged && s->kv_int8) return OHARA_EINVAL;
+  if (!ragged && use_pos_dev && (!s->step_state || seq_len != 1)) return OHARA_EINVAL;
+  if (!ragged && !use_pos_dev && (pos < 0 || pos + seq_len > m->t_max)) return OHARA_EINVAL;
   if (logits_mode < OHARA_LOGITS_NONE || logits_mode > OHARA_LOGITS_ALL) return OHARA_EINVAL;
   if (select_greedy && !(logits_mode == OHARA_LOGITS_LAST || (logits_mode == OHARA_LOGITS_ALL && seq_len == 1)))
     return OHARA_EINVAL;
@@ -47,7 +49,14 @@ extern "C" int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* 
       rc = ohara_rmsnorm_bf16(s->x, L.norm1, s->xn, R, d, m->eps, stream);
       if (rc) return rc;
     }
-    if (!s->kv_int8) {
+    if (ragged) {
+      // one position per sequence; attention of any length through the split-context kernel
+      OHARA_RUN(ohara_qkv_rope_append_ragged_bf16(tiled ? s->xn : s->x, d, L.wqkv, d, tiled ? nullptr : L.norm1, m->eps,
+                                                  B, seq_len, H, Hkv, Dh, m->cos, m->sin, s->seq_pos, s->q, s->kcache[l],
+                                                  s->vcache[l], m->t_max, stream));
+      OHARA_RUN(ohara_attn_cached_ragged_bf16(s->q, s->kcache[l], s->vcache[l], B, seq_len, H, Hkv, Dh, m->t_max,
+                                              s->seq_pos, n_split, s->attn_ws, s->attn, stream));
+    } else if (!s->kv_int8) {
       OHARA_RUN(ohara_qkv_rope_append_bf16(tiled ? s->xn : s->x, d, L.wqkv, d, tiled ? nullptr : L.norm1, m->eps, B,
                                            seq_len, H, Hkv, Dh, m->cos, m->sin, pos, pos_dev, s->q, s->kcache[l],
                                            s->vcache[l], m->t_max, stream));

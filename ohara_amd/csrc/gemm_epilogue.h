@@ -24,6 +24,7 @@ struct GemmArgs {
   int S, row0;  // rows are (sequence, position) pairs: row = seq * S + s, position = pos + s
   int ny, nstrips;  // skinny kernel: 16-row chunks per strip (workgroups of a strip share an XCD) and strips
   const int32_t* pos_dev;
+  int pos_stride;  // 0: *pos_dev is the position of every sequence; 1: pos_dev[seq] (ragged batches)
   const bf16_t* cos;
   const bf16_t* sin;
   bf16_t* kcache;
@@ -77,7 +78,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, int b, int stri
   } else {  // EPI_ROPE: rows [q (H*Dh); k (Hkv*Dh); v (Hkv*Dh)], one position per sequence
     const int grow = a.row0 + b;
     const int seq = grow / a.S;
-    const int pos = (a.pos_dev ? *a.pos_dev : a.pos) + (grow - seq * a.S);
+    const int pos = (a.pos_dev ? a.pos_dev[(size_t)seq * a.pos_stride] : a.pos) + (grow - seq * a.S);
     const int nq = a.H * a.Dh, nk = a.Hkv * a.Dh;
     if (r0 >= nq + 2 * nk || pos < 0 || pos >= a.Tmax) return;
     float v[4] = {y0, y1, y2, y3};

@@ -422,7 +422,7 @@ int ohara_gemm_skinny_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n
 
 static int qkv_rope_impl(const uint16_t* x, int ldx, const uint16_t* wp, int k, const uint16_t* norm_w,
                          float eps, int batch, int seq_len, int h, int h_kv, int dh, const uint16_t* cos,
-                         const uint16_t* sin, int pos, const int32_t* pos_dev, uint16_t* q_out,
+                         const uint16_t* sin, int pos, const int32_t* pos_dev, int pos_stride, uint16_t* q_out,
                          uint16_t* kcache, uint16_t* vcache, int t_max, int stage, void* stream) {
   if (!x || !wp || !cos || !sin || !q_out || !kcache || !vcache) return OHARA_EINVAL;
   if (batch < 1 || seq_len < 1 || h < 1 || h_kv < 1 || h % h_kv || dh < 4 || (dh & 3) || t_max < 1)
@@ -436,7 +436,7 @@ static int qkv_rope_impl(const uint16_t* x, int ldx, const uint16_t* wp, int k, 
   a.B = batch * seq_len; a.N = (h + 2 * h_kv) * dh; a.K = k;
   a.S = seq_len; a.row0 = 0;
   a.out = q_out; a.ldo = h * dh;
-  a.H = h; a.Hkv = h_kv; a.Dh = dh; a.Tmax = t_max; a.pos = pos; a.pos_dev = pos_dev;
+  a.H = h; a.Hkv = h_kv; a.Dh = dh; a.Tmax = t_max; a.pos = pos; a.pos_dev = pos_dev; a.pos_stride = pos_stride;
   a.cos = cos; a.sin = sin; a.kcache = kcache; a.vcache = vcache; a.stage = stage;
   if (a.B > 64 && !norm_w) return ohara_launch_gemm_tile(a, EPI_ROPE, (a.N + 15) / 16 * 16, (hipStream_t)stream);
   return launch_skinny(a, EPI_ROPE, (a.N + 15) / 16 * 16, (hipStream_t)stream);
@@ -446,7 +446,16 @@ int ohara_qkv_rope_append_bf16(const uint16_t* x, int ldx, const uint16_t* wp, i
                                float eps, int batch, int seq_len, int h, int h_kv, int dh, const uint16_t* cos,
                                const uint16_t* sin, int pos, const int32_t* pos_dev, uint16_t* q_out,
                                uint16_t* kcache, uint16_t* vcache, int t_max, void* stream) {
-  return qkv_rope_impl(x, ldx, wp, k, norm_w, eps, batch, seq_len, h, h_kv, dh, cos, sin, pos, pos_dev, q_out, kcache,
+  return qkv_rope_impl(x, ldx, wp, k, norm_w, eps, batch, seq_len, h, h_kv, dh, cos, sin, pos, pos_dev, 0, q_out, kcache,
+                       vcache, t_max, 0, stream);
+}
+
+int ohara_qkv_rope_append_ragged_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int k, const uint16_t* norm_w,
+                                      float eps, int batch, int seq_len, int h, int h_kv, int dh, const uint16_t* cos,
+                                      const uint16_t* sin, const int32_t* seq_pos, uint16_t* q_out, uint16_t* kcache,
+                                      uint16_t* vcache, int t_max, void* stream) {
+  if (!seq_pos) return OHARA_EINVAL;
+  return qkv_rope_impl(x, ldx, wp, k, norm_w, eps, batch, seq_len, h, h_kv, dh, cos, sin, 0, seq_pos, 1, q_out, kcache,
                        vcache, t_max, 0, stream);
 }
 
@@ -454,7 +463,7 @@ int ohara_qkv_rope_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int k, c
                         int batch, int seq_len, int h, int h_kv, int dh, const uint16_t* cos, const uint16_t* sin,
                         int pos, const int32_t* pos_dev, int t_max, uint16_t* q_out, uint16_t* k_out, uint16_t* v_out,
                         void* stream) {
-  return qkv_rope_impl(x, ldx, wp, k, norm_w, eps, batch, seq_len, h, h_kv, dh, cos, sin, pos, pos_dev, q_out, k_out,
+  return qkv_rope_impl(x, ldx, wp, k, norm_w, eps, batch, seq_len, h, h_kv, dh, cos, sin, pos, pos_dev, 0, q_out, k_out,
                        v_out, t_max, 1, stream);
 }
 

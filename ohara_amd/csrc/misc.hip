@@ -132,6 +132,13 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const bf16_t* logits, int 
 
 }  // namespace
 
+namespace {
+__global__ void advance_positions_kernel(int32_t* seq_pos, const uint8_t* active, int batch, int by) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b < batch && (!active || active[b])) seq_pos[b] += by;
+}
+}  // namespace
+
 extern "C" {
 
 int ohara_abi_version(void) { return 1; }
@@ -159,3 +166,10 @@ int ohara_argmax_bf16(const uint16_t* logits, int ldl, int batch, int vocab, int
 }
 
 }  // extern "C"
+
+extern "C" int ohara_advance_positions(int32_t* seq_pos, const uint8_t* active, int batch, int by, void* stream) {
+  if (!seq_pos || batch < 1) return OHARA_EINVAL;
+  hipLaunchKernelGGL(advance_positions_kernel, dim3((batch + 255) / 256), dim3(256), 0, (hipStream_t)stream, seq_pos,
+                     active, batch, by);
+  return ohara_launch_status();
+}

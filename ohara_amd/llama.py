@@ -85,6 +85,7 @@ class KVCache:
         self.max_seq_length = max_seq_length
         self.length = 0
         self.batch_size = None
+        self.lengths = None  # per-sequence lengths, once sequences have advanced by different amounts
         self.dtype = dtype
         storage = torch.int8 if self.int8 else dtype
         self.key = torch.zeros(shape, device=device, dtype=storage)
@@ -103,6 +104,9 @@ class KVCache:
             raise ValueError("KV cache batch size is smaller than the input batch")
         if self.batch_size is not None and bsz != self.batch_size:
             raise ValueError("KV cache batch size cannot change during decoding")
+        if self.lengths is not None and any(n != self.lengths[0] for n in self.lengths[:bsz]):
+            raise ValueError("KV cache writes must be sequential: the sequences have different lengths, "
+                             "pass one position per sequence")
         if start_pos != self.length:
             raise ValueError(
                 f"KV cache writes must be sequential: expected position {self.length}, got {start_pos}"
@@ -114,6 +118,37 @@ class KVCache:
     def _commit(self, bsz: int, end: int) -> None:
         self.length = end
         self.batch_size = bsz
+        self.lengths = None
+
+    # One position per sequence (no counterpart in the reference, whose cache has a single length):
+    # the same checks as above, sequence by sequence.
+    def _reserve_ragged(self, bsz: int, seq_len: int, starts) -> list:
+        if bsz > self.key.size(0):
+            raise ValueError("KV cache batch size is smaller than the input batch")
+        if self.batch_size is not None and bsz != self.batch_size:
+            raise ValueError("KV cache batch size cannot change during decoding")
+        have = self.lengths if self.lengths is not None else [self.length] * bsz
+        for b, (start, n) in enumerate(zip(starts, have)):
+            if start != n:
+                raise ValueError(f"KV cache writes must be sequential: expected position {n}, got {start} "
+                                 f"(sequence {b})")
+            if start < 0 or start + seq_len > self.max_seq_length:
+                raise ValueError("KV cache position exceeds max_sequence_length")
+        return [start + seq_len for start in starts]
+
+    def _commit_ragged(self, bsz: int, ends) -> None:
+        self.lengths = list(ends)
+        self.length = max(ends)
+        self.batch_size = bsz
+
+    def _row_view(self, b: int) -> "KVCache":
+        """The cache of sequence b alone, sharing storage (bf16 mode)."""
+        v = KVCache.__new__(KVCache)
+        v.idx, v.int8, v.max_seq_length, v.dtype = self.idx, False, self.max_seq_length, self.dtype
+        v.key, v.value = self.key[b:b + 1], self.value[b:b + 1]
+        v.length = (self.lengths[b] if self.lengths is not None else self.length)
+        v.batch_size, v.lengths = None, None
+        return v
 
     def forward(self, keys, values, start_pos):
         bsz, seq_len = keys.shape[0], keys.shape[1]
@@ -274,7 +309,8 @@ class Llama:
             self._buffers[key] = buf
         return buf
 
-    def _state_struct(self, buf: _Buffers, kv_cache, logits, history=None, valid_vocab=0) -> OharaDecodeState:
+    def _state_struct(self, buf: _Buffers, kv_cache, logits, history=None, valid_vocab=0,
+                      seq_pos=None) -> OharaDecodeState:
         n = self.config.num_hidden_layers
         kc = (C.c_void_p * n)(*[c.key.data_ptr() for c in kv_cache])
         vc = (C.c_void_p * n)(*[c.value.data_ptr() for c in kv_cache])
@@ -291,6 +327,11 @@ class Llama:
         s._keep = (kc, vc)
         if len({c.int8 for c in kv_cache}) > 1:
             raise ValueError("all layers must use the same KV cache mode")
+        if seq_pos is not None:
+            if kv_cache[0].int8:
+                raise NotImplementedError("ohara_amd: one position per sequence needs bf16 KV caches")
+            s.seq_pos = seq_pos.data_ptr()
+            s._keep = (kc, vc, seq_pos)
         if kv_cache[0].int8:
             stats = [(C.c_void_p * n)(*[getattr(c, nm).data_ptr() for c in kv_cache])
                      for nm in ("key_scale", "key_min", "value_scale", "value_min")]
@@ -310,46 +351,79 @@ class Llama:
             s._keep = (kc, vc, *stats)
         return s
 
-    def forward(self, x: torch.Tensor, kv_cache: list | None = None, position_ids=None, *, last_only: bool = False):
+    def forward(self, x: torch.Tensor, kv_cache: list | None = None, position_ids=None, *, last_only: bool = False,
+                seq_pos: torch.Tensor | None = None):
         """ohara/models/llama.py:279-323.  Returns logits (B, S, V) in bf16, or (B, 1, V)
-        with ``last_only=True`` (an extension: the generate loops read only the last row)."""
+        with ``last_only=True`` (an extension: the generate loops read only the last row).
+
+        A second extension: ``position_ids`` may hold one cache position per sequence (a list, or a
+        1-D tensor with more than one element) - the reference has a single scalar for the whole
+        batch (llama.py:287-299), which forces equal lengths.  ``seq_pos`` optionally supplies the same
+        positions as an int32 device tensor that the caller keeps up to date (no upload per call)."""
         c = self.config
         if x.ndim != 2:
             raise ValueError("input token IDs must have shape (batch, sequence)")
-        if isinstance(position_ids, torch.Tensor):
-            if position_ids.numel() != 1:
+        ragged = None
+        if isinstance(position_ids, (list, tuple)):
+            ragged = [int(p) for p in position_ids]
+        elif isinstance(position_ids, torch.Tensor):
+            if position_ids.ndim == 1 and position_ids.numel() > 1:
+                ragged = [int(p) for p in position_ids.tolist()]
+            elif position_ids.numel() != 1:
                 raise ValueError("position_ids must be a scalar cache position")
-            position_ids = int(position_ids.item())
-        start_pos = 0
-        if kv_cache is not None:
+            else:
+                position_ids = int(position_ids.item())
+        B, S = x.shape
+        if ragged is not None:
+            if kv_cache is None:
+                raise ValueError("position_ids is only valid when using a KV cache")
             if len(kv_cache) != c.num_hidden_layers:
                 raise ValueError("KV cache must contain one entry per model layer")
-            if position_ids is None or position_ids < 0:
+            if len(ragged) != B:
+                raise ValueError("one position per sequence is required")
+            if min(ragged) < 0:
                 raise ValueError("a non-negative position_ids is required with KV cache")
-            start_pos = position_ids
-        elif position_ids is not None:
-            raise ValueError("position_ids is only valid when using a KV cache")
-        B, S = x.shape
-        if S < 1:
-            raise ValueError("input sequence cannot be empty")
-        if start_pos + S > c.max_sequence_length:
-            raise ValueError("input exceeds max_sequence_length")
-        if kv_cache is None:
-            # Uncached causal forward == a fresh cache filled from position 0.
-            kv_cache = self.build_kv_cache(B)
-        ends = [cache._reserve(B, S, start_pos) for cache in kv_cache]
+            if S < 1:
+                raise ValueError("input sequence cannot be empty")
+            if max(ragged) + S > c.max_sequence_length:
+                raise ValueError("input exceeds max_sequence_length")
+            ends = [cache._reserve_ragged(B, S, ragged) for cache in kv_cache]
+            if seq_pos is None:
+                seq_pos = torch.tensor(ragged, dtype=torch.int32).to(self.device)
+        else:
+            start_pos = 0
+            if kv_cache is not None:
+                if len(kv_cache) != c.num_hidden_layers:
+                    raise ValueError("KV cache must contain one entry per model layer")
+                if position_ids is None or position_ids < 0:
+                    raise ValueError("a non-negative position_ids is required with KV cache")
+                start_pos = position_ids
+            elif position_ids is not None:
+                raise ValueError("position_ids is only valid when using a KV cache")
+            if S < 1:
+                raise ValueError("input sequence cannot be empty")
+            if start_pos + S > c.max_sequence_length:
+                raise ValueError("input exceeds max_sequence_length")
+            if kv_cache is None:
+                # Uncached causal forward == a fresh cache filled from position 0.
+                kv_cache = self.build_kv_cache(B)
+            ends = [cache._reserve(B, S, start_pos) for cache in kv_cache]
+            seq_pos = None
 
         rows = B * S
         buf = self._get_buffers(B, rows)
         buf.ids.copy_(x.reshape(-1).to(device=self.device, dtype=torch.int64))
         out_rows = B if last_only else rows
         logits = torch.empty(out_rows, c.vocab_size, dtype=BF16, device=self.device)
-        st = self._state_struct(buf, kv_cache, logits)
+        st = self._state_struct(buf, kv_cache, logits, seq_pos=seq_pos)
         mode = _lib.OHARA_LOGITS_LAST if last_only else _lib.OHARA_LOGITS_ALL
-        check(lib().ohara_llama_forward(C.byref(self._c_model), C.byref(st), S, start_pos, 0, mode, 0,
-                                        torch.cuda.current_stream().cuda_stream), "llama_forward")
+        check(lib().ohara_llama_forward(C.byref(self._c_model), C.byref(st), S, 0 if ragged is not None else start_pos, 0,
+                                        mode, 0, torch.cuda.current_stream().cuda_stream), "llama_forward")
         for cache, end in zip(kv_cache, ends):
-            cache._commit(B, end)
+            if ragged is not None:
+                cache._commit_ragged(B, end)
+            else:
+                cache._commit(B, end)
         return logits.view(B, 1 if last_only else S, c.vocab_size)
 
     __call__ = forward

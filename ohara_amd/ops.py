@@ -145,14 +145,25 @@ def gemm(x, w: PackedLinear, residual=None, out=None) -> torch.Tensor:
 
 
 def qkv_rope_append(x, wqkv: PackedLinear, norm_w, eps, h, h_kv, dh, cos, sin, pos, kcache, vcache,
-                    q_out=None, pos_dev=None, seq_len=1):
-    """x: (batch*seq_len, K) rows ordered (sequence, position)."""
+                    q_out=None, pos_dev=None, seq_len=1, seq_pos=None):
+    """x: (batch*seq_len, K) rows ordered (sequence, position).  ``seq_pos`` (int32, one entry per
+    sequence, on the device) gives every sequence its own cache position instead of ``pos``."""
     _need(x, BF16, "x")
     rows = x.shape[0]
     b = rows // seq_len
     if q_out is None:
         q_out = torch.empty(rows, h * dh, dtype=BF16, device=x.device)
     t_max = kcache.shape[1]
+    if seq_pos is not None:
+        _need(seq_pos, torch.int32, "seq_pos")
+        check(
+            lib().ohara_qkv_rope_append_ragged_bf16(
+                _ptr(x), x.stride(0), _ptr(wqkv.data), wqkv.k, _ptr(norm_w), eps, b, seq_len, h, h_kv, dh, _ptr(cos),
+                _ptr(sin), _ptr(seq_pos), _ptr(q_out), _ptr(kcache), _ptr(vcache), t_max, _stream(),
+            ),
+            "qkv_rope_append_ragged",
+        )
+        return q_out
     check(
         lib().ohara_qkv_rope_append_bf16(
             _ptr(x), x.stride(0), _ptr(wqkv.data), wqkv.k, _ptr(norm_w), eps, b, seq_len, h, h_kv, dh, _ptr(cos), _ptr(sin),
@@ -188,11 +199,23 @@ def attn_workspace(batch, h, h_kv, dh, n_split, device) -> torch.Tensor:
     return torch.zeros(n, dtype=torch.uint8, device=device)
 
 
-def attn_cached(q, kcache, vcache, h, h_kv, dh, pos, n_split, workspace, out=None, pos_dev=None, seq_len=1):
-    """q: (batch*seq_len, h*dh); query s of a sequence sits at cache position pos + s."""
+def attn_cached(q, kcache, vcache, h, h_kv, dh, pos, n_split, workspace, out=None, pos_dev=None, seq_len=1,
+                seq_pos=None):
+    """q: (batch*seq_len, h*dh); query s of a sequence sits at cache position pos + s (or at
+    seq_pos[sequence] + s when the int32 device tensor ``seq_pos`` is given)."""
     rows = q.shape[0]
     if out is None:
         out = torch.empty(rows, h * dh, dtype=BF16, device=q.device)
+    if seq_pos is not None:
+        _need(seq_pos, torch.int32, "seq_pos")
+        check(
+            lib().ohara_attn_cached_ragged_bf16(
+                _ptr(q), _ptr(kcache), _ptr(vcache), rows // seq_len, seq_len, h, h_kv, dh, kcache.shape[1],
+                _ptr(seq_pos), n_split, _ptr(workspace), _ptr(out), _stream(),
+            ),
+            "attn_cached_ragged",
+        )
+        return out
     check(
         lib().ohara_attn_cached_bf16(
             _ptr(q), _ptr(kcache), _ptr(vcache), rows // seq_len, seq_len, h, h_kv, dh, kcache.shape[1], int(pos),
@@ -266,6 +289,14 @@ def attn_cached_int8(q, cache, h, h_kv, dh, pos, n_split, workspace, out=None, p
 def attn_decode(q, kcache, vcache, h, h_kv, dh, length, n_split, workspace, out=None, pos_dev=None):
     """Decode case: one query per sequence seeing `length` cached positions."""
     return attn_cached(q, kcache, vcache, h, h_kv, dh, length - 1, n_split, workspace, out, pos_dev, 1)
+
+
+def advance_positions(seq_pos: torch.Tensor, active: torch.Tensor | None = None, by: int = 1) -> None:
+    """seq_pos[b] += by where active[b] (uint8) is non-zero; all entries when ``active`` is None."""
+    _need(seq_pos, torch.int32, "seq_pos")
+    if active is not None:
+        _need(active, torch.uint8, "active")
+    check(lib().ohara_advance_positions(_ptr(seq_pos), _ptr(active), seq_pos.numel(), by, _stream()), "advance_positions")
 
 
 def argmax(logits: torch.Tensor, valid_vocab: int | None = None, next_ids=None, history=None, step_state=None):

@@ -261,3 +261,31 @@ def test_product_has_no_cpu_fallback():
         pytest.skip("needs a machine without a GPU")
     with pytest.raises(RuntimeError, match="GPU only"):
         sample_next_token(torch.zeros(1, 1, 8), SamplingConfig(temperature=0.0))
+
+
+def test_kv_cache_per_sequence_bookkeeping():
+    """One length per sequence: the reference's checks (kv_cache.py:78-90), sequence by sequence."""
+    from ohara_amd.llama import KVCache
+
+    c = KVCache((3, 16, 2, 4), 16, dtype=torch.float32)
+    ends = c._reserve_ragged(3, 2, [0, 0, 0])
+    c._commit_ragged(3, ends)
+    assert c.lengths == [2, 2, 2] and c.length == 2 and c.batch_size == 3
+    c._commit_ragged(3, c._reserve_ragged(3, 1, [2, 2, 2]))
+    c.lengths[1] = 7
+    with pytest.raises(ValueError, match=r"expected position 7, got 3 \(sequence 1\)"):
+        c._reserve_ragged(3, 1, [3, 3, 3])
+    with pytest.raises(ValueError, match="different lengths"):
+        c._reserve(3, 1, 3)
+    with pytest.raises(ValueError, match="exceeds max_sequence_length"):
+        c._reserve_ragged(3, 10, [3, 7, 3])
+    with pytest.raises(ValueError, match="cannot change"):
+        c._reserve_ragged(2, 1, [3, 7])
+    c._commit_ragged(3, c._reserve_ragged(3, 1, [3, 7, 3]))
+    assert c.lengths == [4, 8, 4] and c.length == 8
+    v = c._row_view(1)
+    assert v.length == 8 and v.key.shape == (1, 16, 2, 4) and v.key.data_ptr() == c.key[1].data_ptr()
+    # equal lengths again: the scalar interface works and clears the per-sequence state
+    c.lengths = [8, 8, 8]
+    c._commit(3, c._reserve(3, 1, 8))
+    assert c.lengths is None and c.length == 9
