@@ -215,6 +215,32 @@ def bench_attention_microbench(dev):
     return out
 
 
+def bench_continuous(model, cfg, dev, slots=32, steps=128):
+    """Continuous batching: `slots` sequences of different lengths (prompts of 256..1279 tokens)
+    decode in one batch, every slot at its own cache position; one graph replay per step."""
+    from ohara_amd.batching import ContinuousBatcher
+
+    g = torch.Generator().manual_seed(4)
+    lens = torch.randint(256, 1280, (slots,), generator=g).tolist()
+    bat = ContinuousBatcher(model, slots)
+    for n in lens:
+        bat.add(torch.randint(0, cfg.vocab_size, (n,), generator=g))
+    for _ in range(8):
+        bat.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        bat.step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    mean_len = sum(lens) / slots + 8 + steps / 2
+    by = step_bytes(cfg, slots, mean_len)
+    return {"slots": slots, "prompt_lengths": "uniform 256..1279", "mean_context": round(mean_len, 1),
+            "ms_per_step": round(dt * 1e3, 4), "tokens_per_s": round(slots / dt, 1),
+            "frac_of_hbm_peak": round(by / dt / 1e9 / HBM_PEAK_GBS, 4),
+            "note": "host reads the new ids every step (one synchronisation per step)"}
+
+
 def bench_prefill(model, cfg, dev):
     """Batched prefill of the d12 model (1024 tokens per sequence) and its MFMA kernels alone."""
     from ohara_amd import ops
@@ -470,6 +496,7 @@ def main():
         "roofline": roof,
     }
     if not args.no_extended:
+        out["also"]["continuous_batch32"] = bench_continuous(model, cfg, dev)
         out["kernels"] = {"prefill_d12": bench_prefill(model, cfg, dev)}
         del model
         torch.cuda.empty_cache()

@@ -33,6 +33,7 @@ class ContinuousBatcher:
         self.last = torch.zeros(slots, dtype=torch.int64, device=model.device)
         self.seq_pos = torch.zeros(slots, dtype=torch.int32, device=model.device)
         self.active_dev = torch.zeros(slots, dtype=torch.uint8, device=model.device)
+        self._toks = self._u = self._graph = None
 
     def free_slots(self) -> list[int]:
         return [b for b in range(self.slots) if not self.active[b]]
@@ -83,25 +84,53 @@ class ContinuousBatcher:
         for c in self.cache:
             c.lengths[slot] = 0
 
+    def _device_step(self) -> None:
+        """Everything of a step that runs on the device, with no host synchronisation: forward at
+        the slots' own positions, selection, position advance, next inputs.  Capturable."""
+        logits = self.model.forward(self.last.view(self.slots, 1), self.cache, list(self.lengths), last_only=True,
+                                    seq_pos=self.seq_pos)
+        vv = self.valid_vocab or None
+        if self.sampling is None:
+            ops.argmax(logits.view(self.slots, -1), valid_vocab=vv, next_ids=self._toks)
+        else:
+            ops.sample_topk_topp(logits.view(self.slots, -1), self.sampling.temperature, self.sampling.top_k,
+                                 self.sampling.top_p, self._u, valid_vocab=vv, out=self._toks)
+        # idle slots stay at position 0; active ones advance
+        ops.advance_positions(self.seq_pos, self.active_dev, 1)
+        self.last.copy_(torch.where(self.active_dev.bool(), self._toks, torch.zeros_like(self._toks)))
+
     @torch.no_grad()
-    def step(self) -> dict[int, int]:
+    def step(self, use_graph: bool = True) -> dict[int, int]:
         """One decode step for every active slot -> {slot: new id}.  Idle slots ride along at
-        position 0 of their own cache rows (overwritten when the slot is taken again)."""
+        position 0 of their own cache rows (overwritten when the slot is taken again).  The device
+        work is captured once into a HIP graph (positions, inputs and the active mask live in
+        device tensors, so joins and leaves need no re-capture) and replayed per step."""
         if not any(self.active):
             return {}
         if max(n for n, a in zip(self.lengths, self.active) if a) + 1 > self.model.config.max_sequence_length:
             raise ValueError("input exceeds max_sequence_length")
-        logits = self.model.forward(self.last.view(self.slots, 1), self.cache, list(self.lengths), last_only=True,
-                                    seq_pos=self.seq_pos)
-        toks = self._select(logits.view(self.slots, -1))
-        # idle slots stay at position 0; active ones advance on the device and in the host's books
-        ops.advance_positions(self.seq_pos, self.active_dev, 1)
-        self.last.copy_(torch.where(self.active_dev.bool(), toks, torch.zeros_like(toks)))
+        if self._toks is None:
+            self._toks = torch.zeros(self.slots, dtype=torch.int64, device=self.model.device)
+            self._u = torch.zeros(self.slots, dtype=torch.float32, device=self.model.device)
+        if self.sampling is not None:
+            self._u.copy_(torch.rand(self.slots, device=self.model.device, dtype=torch.float32, generator=self.generator))
+        if use_graph and self._graph is None:
+            # the capture itself executes nothing: the books it touches are restored, and the step
+            # is then replayed like any other
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                self._device_step()
+            self._graph = g
+        if use_graph:
+            self._graph.replay()
+        else:
+            self._device_step()
         for b in range(self.slots):
             if self.active[b]:
                 self.lengths[b] += 1
         for c in self.cache:
             c.lengths = list(self.lengths)
             c.length = max(self.lengths)
-        host = toks.tolist()
+        host = self._toks.tolist()
         return {b: host[b] for b in range(self.slots) if self.active[b]}

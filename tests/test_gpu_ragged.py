@@ -125,7 +125,8 @@ def test_model_forward_with_one_position_per_sequence(cuda):
         model(nxt.to(cuda), q8, [0, 0, 0])
 
 
-def test_continuous_batching_matches_sequences_run_alone(cuda):
+@pytest.mark.parametrize("use_graph", [True, False])
+def test_continuous_batching_matches_sequences_run_alone(cuda, use_graph):
     """Sequences join and leave at different times; every token a slot produces is the oracle's
     greedy choice for that sequence alone (or a near-tie of the oracle's own logits)."""
     from ohara_amd.batching import ContinuousBatcher
@@ -144,7 +145,7 @@ def test_continuous_batching_matches_sequences_run_alone(cuda):
 
     def steps(n):
         for _ in range(n):
-            toks = bat.step()
+            toks = bat.step(use_graph=use_graph)
             for name, slot in slot_of.items():
                 out[name].append(toks[slot])
 
