@@ -9,7 +9,8 @@
 //   P2  attention over the cache, split along the context, partial (max,sum,acc) triples
 //   P3  merge of the partials + output projection + residual
 //   P4  norm2 + gate/up projection + SwiGLU
-//   P5  down projection + residual
+//   P5  down projection, split along K over four groups of workgroups (fp32 partial sums; the
+//       residual add happens where the stream is read next)
 // then final norm + vocabulary projection with a running arg-max per workgroup, and the
 // selection of the next token.  Rounding points are those of the unfused kernels.
 //
@@ -47,11 +48,11 @@ struct MegaArgs {
   int ns;                       // context chunks per (sequence, kv head) in this launch, <= OHARA_MEGA_NS
   int blk_x, blk_a;             // bytes per strip block of the x/q and act mailboxes
   int64_t* ids;
-  char* xm;        // (2*NL + 1) x-mailboxes of xm_stride bytes: residual stream after each half layer
+  char* xm;        // NL x-mailboxes of xm_stride bytes: the residual stream after each layer's attention block
   char* qm;        // NL q-mailboxes of qm_stride bytes
   char* am;        // NL act-mailboxes of am_stride bytes
   float* pm;       // NL partial mailboxes of pm_stride floats: [b*H + h][chunk][Dh + 32]
-  float* dm;       // NL mailboxes of dm_stride floats: partial sums of the down projection [part][b][d]
+  float* dm;       // NL mailboxes of dm_stride floats: partial sums of the down projection (see XParts)
   size_t xm_stride, qm_stride, am_stride, pm_stride, dm_stride;
   float* cand_val; // (nwg, B)
   int* cand_idx;   // (nwg, B)
@@ -174,14 +175,21 @@ __device__ __forceinline__ const char* am_addr(const char* base, int blk, int b,
 }
 
 // The down projection is split along K over OHARA_DOWN_SPLIT groups of workgroups (a 16-row strip
-// of it is too much for one CU to stream); each group leaves an fp32 partial sum [part][b][n] and
-// whoever needs the residual stream after the block forms it on the fly, in a fixed order:
+// of it is too much for one CU to stream); each group leaves fp32 partial sums and whoever needs
+// the residual stream after the block forms it on the fly, in a fixed order:
 //   x[b][n] = bf16(x_mid[b][n] + bf16(((p0 + p1) + p2) + p3))        (llama.py:200)
+// The sums are strip-blocked like the x mailbox, one block of `blk` bytes (a multiple of 128) per
+// (part, strip) with row b at byte b*64, so that every 128-byte line has a single writer.
 struct XParts {
   const char* xmid;   // x mailbox holding the stream before the feed-forward block
   const float* parts; // partial sums; nullptr: `xmid` already is the stream that is wanted
   int blk, B, N;
 };
+__device__ __forceinline__ int pm_blk(int B) { return (B * 64 + 127) & ~127; }
+__device__ __forceinline__ const float* parts_addr(const float* base, int nstrips, int B, int q, int b, int n) {
+  return reinterpret_cast<const float*>(reinterpret_cast<const char*>(base) +
+                                        (size_t)(q * nstrips + (n >> 4)) * pm_blk(B) + b * 64) + (n & 15);
+}
 
 template <int NW>  // NW columns (4 or 8) starting at n, n % NW == 0
 __device__ __forceinline__ void x_load(const XParts& xp, int b, int n, uint32_t (&out)[NW / 2]) {
@@ -202,7 +210,7 @@ __device__ __forceinline__ void x_load(const XParts& xp, int b, int n, uint32_t 
 #pragma unroll
   for (int q = 0; q < OHARA_DOWN_SPLIT; ++q)
 #pragma unroll
-    for (int i = 0; i < NW / 4; ++i) pv[q][i] = ldg16(xp.parts + ((size_t)(q * xp.B + b) * xp.N + n + 4 * i));
+    for (int i = 0; i < NW / 4; ++i) pv[q][i] = ldg16(parts_addr(xp.parts, (xp.N + 15) >> 4, xp.B, q, b, n + 4 * i));
 #pragma unroll
   for (int i = 0; i < NW / 4; ++i) {
     float y[4];
@@ -565,7 +573,7 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
         }
       } else if (EPI == E_PART) {  // the raw fp32 sums of this K partition
         if (r0 < p.N) {
-          float* o = p.pout + ((size_t)((unit / p.nstrips) * B + b) * p.N + r0);
+          float* o = const_cast<float*>(parts_addr(p.pout, p.nstrips, B, unit / p.nstrips, b, r0));
           st_coh8(o, make_uint2(__float_as_uint(acc[0]), __float_as_uint(acc[1])));
           st_coh8(o + 2, make_uint2(__float_as_uint(acc[2]), __float_as_uint(acc[3])));
         }
@@ -875,9 +883,9 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     const unsigned long long* pl = ptab + l * 8;
     bf16_t* kc = lds_ptr<bf16_t>(pl, 6);
     bf16_t* vc = lds_ptr<bf16_t>(pl, 7);
-    char* x_mid = a.xm + (size_t)(2 * l + 1) * a.xm_stride;        // after attention
+    char* x_mid = a.xm + (size_t)l * a.xm_stride;                  // after attention
     // the stream entering layer l > 0 is x_mid of layer l - 1 plus that layer's down-projection sums
-    const char* x_prev = a.xm + (size_t)(l > 0 ? 2 * l - 1 : 0) * a.xm_stride;
+    const char* x_prev = a.xm + (size_t)(l > 0 ? l - 1 : 0) * a.xm_stride;
     const float* d_prev = l > 0 ? a.dm + (size_t)(l - 1) * a.dm_stride : nullptr;
     float* d_l = a.dm + (size_t)l * a.dm_stride;
     char* q_l = a.qm + (size_t)l * a.qm_stride;
@@ -952,7 +960,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     pf.stamp();
   }
   // final norm + vocabulary projection, running arg-max per lane
-  stage_norm<2, false>(xs, ldxs, a.xm + (size_t)(2 * m.n_layers - 1) * a.xm_stride, a.blk_x,
+  stage_norm<2, false>(xs, ldxs, a.xm + (size_t)(m.n_layers - 1) * a.xm_stride, a.blk_x,
                        a.dm + (size_t)(m.n_layers - 1) * a.dm_stride, a.ids, m.token_emb, V, m.final_norm, m.eps, B, d);
   __syncthreads();
   gemm_phase<1, 24, E_LOGITS>(lm, pre, xs, ldxs, B, red, best_v, best_i, pf);
@@ -1060,11 +1068,11 @@ MegaLayout mega_layout(const OharaModel* m, int B, int nwg) {
   L.layers = o; o += mega_al(sizeof(OharaLayer) * NL);
   L.kptr = o; o += mega_al(sizeof(void*) * NL);
   L.vptr = o; o += mega_al(sizeof(void*) * NL);
-  L.xm = o; o += L.xm_stride * (2 * NL + 1);
+  L.xm = o; o += L.xm_stride * NL;
   L.qm = o; o += L.qm_stride * NL;
   L.am = o; o += L.am_stride * NL;
   L.pm = o; o += L.pm_stride * sizeof(float) * NL;
-  L.dm_stride = mega_al((size_t)OHARA_DOWN_SPLIT * B * m->d_model * sizeof(float)) / sizeof(float);
+  L.dm_stride = mega_al((size_t)OHARA_DOWN_SPLIT * ((m->d_model + 15) / 16) * ((B * 64 + 127) / 128 * 128)) / sizeof(float);
   L.dm = o; o += L.dm_stride * sizeof(float) * NL;
   L.candv = o; o += mega_al((size_t)nwg * B * sizeof(float));
   L.candi = o; o += mega_al((size_t)nwg * B * sizeof(int));
