@@ -29,10 +29,10 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the persistent decode kernel at batch 1, prompt 1024, from two
 # rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same
-# counter reads for a 1 GiB copy (--pmc-calibration): 379.7 MB read + 1.5 MB written.  Counters
+# counter reads for a 1 GiB copy (--pmc-calibration): 381.4 MB read + 1.8 MB written.  Counters
 # cannot be read from inside this process, so the figure is carried here; the runs and the
 # arithmetic are in profiles/decode_mega_kernel_d12_batch1_pmc.txt.
-PMC_TRAFFIC_BYTES = {("persistent", 1, 1024): 381.3e6}
+PMC_TRAFFIC_BYTES = {("persistent", 1, 1024): 383.2e6}
 
 D12 = dict(vocab_size=65536, hidden_size=768, intermediate_size=3072, num_attention_heads=6,
            num_key_value_heads=0, num_hidden_layers=12, max_sequence_length=4096, dropout=0.0)
@@ -464,7 +464,7 @@ def main():
                 kname = "decode_mega_kernel<128,1> (whole decode step: 12 layers + vocabulary projection + selection)"
             else:
                 kb = lm_head_bytes(cfg, 1)
-                kname = "skinny_kernel<1,true,STORE> (final norm + vocabulary projection 65536x768)"
+                kname = "wide_kernel<1,true,STORE> (final norm + vocabulary projection 65536x768)"
             roof = {"kernel": kname, "bound": "hbm", "achieved": round(kb / t_k / 1e9, 1), "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": round(kb / t_k / 1e9 / HBM_PEAK_GBS, 4),
                     "traffic": PMC_TRAFFIC_BYTES.get(("persistent" if sess2.persistent else "chain", 1, args.prompt)),
