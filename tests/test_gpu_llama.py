@@ -288,3 +288,37 @@ def test_sampled_decode_session(cuda, persistent):
                 hi = float(cdf[b, j])
                 assert lo - tol <= float(u[t, b]) <= hi + tol, (t, b, tol, int(toks[b, t]), lo, hi, float(u[t, b]))
         inp = toks[:, t : t + 1]
+
+
+@pytest.mark.parametrize("persistent", [True, False])
+def test_decode_to_the_last_cache_position(cuda, persistent):
+    """Maximum size: the prompt plus the generated tokens fill the cache exactly (the last decode
+    step appends at position T_max - 1); one more step is refused on the host.  Tokens equal the
+    oracle's up to near-ties, as in the other greedy tests."""
+    from ohara_amd.llama import Llama
+
+    rcfg, cfg = _cfg_pair(vocab_size=256, hidden_size=128, intermediate_size=256, num_attention_heads=2,
+                          num_key_value_heads=1, num_hidden_layers=2, max_sequence_length=48, rope_theta=10000.0)
+    w = R.init_weights(rcfg, seed=9, dtype=BF, std=0.08, norm_jitter=0.1)
+    ref, model = R.RefLlama(rcfg, w), Llama(cfg, w, device=cuda)
+    P = 29
+    prompt = torch.randint(0, 256, (2, P), generator=torch.Generator().manual_seed(2))
+    steps = 48 - P + 1  # the first token comes from the prefill, the last step feeds position 47
+    sess = model.session(2, steps + 1, persistent=persistent)
+    sess.prefill(prompt.to(cuda))
+    sess.run(steps - 1)
+    got = sess.tokens().cpu()
+    assert got.shape == (2, steps) and sess.cache[0].length == 48
+    with pytest.raises(ValueError, match="exceeds max_sequence_length"):
+        sess.run(1)
+    want, want_logits = greedy_decode_ref(ref, prompt, steps, return_logits=True)
+    for b in range(2):
+        neq = (got[b] != want[b]).nonzero()
+        if neq.numel():
+            t = int(neq[0])
+            assert _near_tie(want_logits[t, b], int(got[b, t]), int(want[b, t])), (b, t)
+    # a single-token prompt and a prompt that fills the cache by itself
+    one = model(prompt[:, :1].to(cuda), model.build_kv_cache(2), 0)
+    _assert_logits_close(one, ref(prompt[:, :1], ref.build_kv_cache(2), 0), 4e-2, 4e-3)
+    full = torch.randint(0, 256, (1, 48), generator=torch.Generator().manual_seed(3))
+    _assert_logits_close(model(full.to(cuda)), ref(full), 4e-2, 4e-3)
