@@ -52,7 +52,6 @@ struct Smem {
   int hist[256];
   float wred[16];
   int wredi[16];
-  float fscan[NT];
   uint32_t skey[CAP];
   int sid[CAP];
   int misc[8];
@@ -150,11 +149,12 @@ __device__ __forceinline__ float block_scan_f(float v, float& lo, float& hi, Sme
 
 // The `want`-th largest key (1-based) among the keys for which live(i) holds; returns the
 // key and the number of live keys strictly greater than it.
-template <int EPT, typename LiveFn, typename KeyFn>
+// Keys use the low TOP + 8 bits (TOP = 24: 32-bit keys, TOP = 8: 16-bit keys in two passes).
+template <int EPT, int TOP = 24, typename LiveFn, typename KeyFn>
 __device__ __forceinline__ uint32_t radix_select(int want, int& n_greater, Smem& s, LiveFn live, KeyFn key) {
   uint32_t prefix = 0, mask = 0;
   int above = 0;
-  for (int shift = 24; shift >= 0; shift -= 8) {
+  for (int shift = TOP; shift >= 0; shift -= 8) {
     __syncthreads();
     if (threadIdx.x < 256) s.hist[threadIdx.x] = 0;
     __syncthreads();
@@ -298,59 +298,120 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
   const int base = tid * EPT;
   float x[EPT];
   const float temp = a.temperature;
-  if (sizeof(T) == 2 && EPT % 8 == 0 && (a.ldl & 7) == 0 && ((reinterpret_cast<uintptr_t>(a.logits) & 15) == 0)) {
-    // bf16 rows: eight values per 16-byte load
-    const bf16_t* row = reinterpret_cast<const bf16_t*>(a.logits) + (size_t)b * a.ldl + base;
-#pragma unroll
-    for (int c = 0; c < EPT / 8; ++c) {
-      const uint4 v = base + 8 * c < V ? ldg16(row + 8 * c) : make_uint4(0, 0, 0, 0);
-      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int id = base + 8 * c + 2 * j;
-        x[8 * c + 2 * j] = id < nvalid ? lo_bf(w[j]) / temp : -INFINITY;
-        x[8 * c + 2 * j + 1] = id + 1 < nvalid ? hi_bf(w[j]) / temp : -INFINITY;
-      }
-    }
-  } else {
-    load_row_scalar<T, EPT>(a, b, base, nvalid, temp, x);
-  }
   const float u = a.u[(a.step_state && a.u_step_stride > 0 ? (size_t)a.step_state[1] * a.u_step_stride : 0) + b];
+  const bool packed_row = sizeof(T) == 2 && EPT % 8 == 0 && (a.ldl & 7) == 0 &&
+                          ((reinterpret_cast<uintptr_t>(a.logits) & 15) == 0);
+  // x = logits / temperature for this thread's ids (ids past the valid vocabulary: -inf)
+  auto load_x = [&]() {
+    if (packed_row) {
+      // bf16 rows: eight values per 16-byte load
+      const bf16_t* row = reinterpret_cast<const bf16_t*>(a.logits) + (size_t)b * a.ldl + base;
+#pragma unroll
+      for (int c = 0; c < EPT / 8; ++c) {
+        const uint4 v = base + 8 * c < V ? ldg16(row + 8 * c) : make_uint4(0, 0, 0, 0);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int id = base + 8 * c + 2 * j;
+          x[8 * c + 2 * j] = id < nvalid ? lo_bf(w[j]) / temp : -INFINITY;
+          x[8 * c + 2 * j + 1] = id + 1 < nvalid ? hi_bf(w[j]) / temp : -INFINITY;
+        }
+      }
+    } else {
+      load_row_scalar<T, EPT>(a, b, base, nvalid, temp, x);
+    }
+  };
   int token = -1;
   bool compact = false;
+  bool have_x = false;
   // ---- small top-k: the survivors fit one sorted block, everything after works on that block -----
   if (a.top_k > 0 && min(a.top_k, V) <= CAP) {
     const int k = min(a.top_k, V);
-    auto in_vocab = [&](int i) { return base + i < V; };
-    auto xkey = [&](int i) { return fkey(x[i]); };  // > 0 for every float but -NaN
-    // lower bound of the k-th largest: the k-th largest of the per-thread maxima
-    uint32_t tmax = 0;
+    int n_c = 0;
+    if (packed_row && EPT % 8 == 0) {
+      // The selection runs on the raw bf16 logits, two per register: dividing by the temperature
+      // is monotone and keeps distinct bf16 values distinct in fp32, so the survivors - and the
+      // ties among them - are those of the divided values, and only the survivors are divided.
+      // (Half the registers of the fp32 row: nothing spills.)  key 0 = masked id.
+      uint32_t raw[EPT / 2];
+      const bf16_t* row = reinterpret_cast<const bf16_t*>(a.logits) + (size_t)b * a.ldl + base;
 #pragma unroll
-    for (int i = 0; i < EPT; ++i)
-      if (in_vocab(i)) tmax = max(tmax, xkey(i));
-    const int have = block_sum_i(tmax > 0 ? 1 : 0, s);
-    uint32_t bound = 0;
-    if (have >= k) {
-      int dummy;
-      bound = radix_select<1>(k, dummy, s, [&](int) { return tmax > 0; }, [&](int) { return tmax; });
-    }
-    int c = 0;
-#pragma unroll
-    for (int i = 0; i < EPT; ++i) c += (in_vocab(i) && xkey(i) >= bound) ? 1 : 0;
-    int off;
-    const int n_c = block_excl_scan_i(c, off, s);
-    if (n_c <= CAP) {  // (else: many ties at the bound - the general path below handles it)
-      compact = true;
-      __syncthreads();
-      if (c > 0) {
-#pragma unroll
-        for (int i = 0; i < EPT; ++i)
-          if (in_vocab(i) && xkey(i) >= bound) {
-            s.skey[off] = xkey(i);
-            s.sid[off] = base + i;
-            ++off;
-          }
+      for (int c = 0; c < EPT / 8; ++c) {
+        const uint4 v = base + 8 * c < V ? ldg16(row + 8 * c) : make_uint4(0, 0, 0, 0);
+        raw[4 * c] = v.x; raw[4 * c + 1] = v.y; raw[4 * c + 2] = v.z; raw[4 * c + 3] = v.w;
       }
+      auto key16 = [&](int i) -> uint32_t {  // order-preserving 16-bit key of element i, 0 when masked
+        const uint32_t bits = (i & 1) ? (raw[i >> 1] >> 16) : (raw[i >> 1] & 0xffffu);
+        const uint32_t kk = (bits & 0x8000u) ? (~bits & 0xffffu) : (bits | 0x8000u);
+        return base + i < nvalid ? kk : 0u;
+      };
+      uint32_t tmax = 0;
+#pragma unroll
+      for (int i = 0; i < EPT; ++i) tmax = max(tmax, key16(i));
+      // ids in [nvalid, V) take part in the reference's top-k as -inf; they can only matter when fewer
+      // than k ids are valid, which the general path below handles
+      const int have = block_sum_i(tmax > 0 ? 1 : 0, s);
+      uint32_t bound = 1;
+      if (have >= k) {
+        int dummy;
+        bound = radix_select<1, 8>(k, dummy, s, [&](int) { return tmax > 0; }, [&](int) { return tmax; });
+      }
+      int c = 0;
+#pragma unroll
+      for (int i = 0; i < EPT; ++i) c += key16(i) >= bound ? 1 : 0;
+      int off;
+      n_c = block_excl_scan_i(c, off, s);
+      if (n_c <= CAP && n_c >= min(k, nvalid) && nvalid >= k) {
+        compact = true;
+        __syncthreads();
+        if (c > 0) {
+#pragma unroll
+          for (int i = 0; i < EPT; ++i)
+            if (key16(i) >= bound) {
+              const uint32_t bits = (i & 1) ? (raw[i >> 1] >> 16) : (raw[i >> 1] & 0xffffu);
+              s.skey[off] = fkey(__uint_as_float(bits << 16) / temp);
+              s.sid[off] = base + i;
+              ++off;
+            }
+        }
+      }
+    }
+    if (!compact) {
+      load_x();
+      have_x = true;
+      auto in_vocab = [&](int i) { return base + i < V; };
+      auto xkey = [&](int i) { return fkey(x[i]); };  // > 0 for every float but -NaN
+      // lower bound of the k-th largest: the k-th largest of the per-thread maxima
+      uint32_t tmax = 0;
+#pragma unroll
+      for (int i = 0; i < EPT; ++i)
+        if (in_vocab(i)) tmax = max(tmax, xkey(i));
+      const int have = block_sum_i(tmax > 0 ? 1 : 0, s);
+      uint32_t bound = 0;
+      if (have >= k) {
+        int dummy;
+        bound = radix_select<1>(k, dummy, s, [&](int) { return tmax > 0; }, [&](int) { return tmax; });
+      }
+      int c = 0;
+#pragma unroll
+      for (int i = 0; i < EPT; ++i) c += (in_vocab(i) && xkey(i) >= bound) ? 1 : 0;
+      int off;
+      n_c = block_excl_scan_i(c, off, s);
+      if (n_c <= CAP) {  // (else: many ties at the bound - the general path below handles it)
+        compact = true;
+        __syncthreads();
+        if (c > 0) {
+#pragma unroll
+          for (int i = 0; i < EPT; ++i)
+            if (in_vocab(i) && xkey(i) >= bound) {
+              s.skey[off] = xkey(i);
+              s.sid[off] = base + i;
+              ++off;
+            }
+        }
+      }
+    }
+    if (compact) {
       int n2 = 64;
       while (n2 < n_c) n2 <<= 1;
       __syncthreads();
@@ -425,6 +486,7 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
       token = s.misc[3];
     }
   }
+  if (!compact && !have_x) load_x();
   // ---- top-k: keep x >= k-th largest ---------------------------------------------
   if (!compact && a.top_k > 0) {
     const int k = min(a.top_k, V);
