@@ -302,34 +302,40 @@ __device__ void stage_act(bf16_t* xs, int ldxs, const char* src, int blk, int B,
 }
 
 // Merge of the attention partials of all chunks, in chunk order (llama.py:116-123 output,
-// rounded to bf16 as SDPA's result is) -> xs[b][h*Dh + d].  The (max, sum) pairs of every
-// (sequence, head, chunk) are fetched in one round into LDS and turned into chunk weights
-// exp(m_s - M) / L there; a thread then owns four adjacent columns and issues the accumulator
-// loads of all chunks before using any.  `mw`: B*H*ns floats, `ml`: B*H*ns floats of LDS.
-__device__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh, int ns, float* mw_,
-                                 float* ml_) {
-  constexpr int NSM = OHARA_MEGA_NS;
+// rounded to bf16 as SDPA's result is) -> xs[b][h*Dh + d].  NS (a power of two) chunks are in use.
+// The (max, sum) pairs of every (sequence, head, chunk) are fetched in one round into LDS and
+// turned into chunk weights exp(m_s - M) and the sum L there; a thread then owns four adjacent
+// columns per pass and issues the accumulator loads of 16 / NS passes - 16 loads - before it uses
+// any, so the number of dependent load rounds does not grow with the chunk count times the batch.
+// `mw`: B*H*NS floats, `ml`: B*H floats of LDS.
+template <int NS>
+__device__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh, float* mw_, float* ml_) {
+  constexpr int NSM = OHARA_MEGA_NS, PR = 16 / NS;
   const int HD = H * Dh, PS = Dh + 32;
-  const int nbh = B * H;
+  const int nbh = B * H, total = B * HD;
+  const int pass = (int)blockDim.x * 4;
   OHARA_LDS float* mw = (OHARA_LDS float*)mw_;
   OHARA_LDS float* ml = (OHARA_LDS float*)ml_;
-  // the accumulator loads of a thread's first columns go out first: they do not depend on the
-  // chunk weights, which are formed (two LDS rounds) while they are in flight
-  uint4 av[NSM];
-  {
-    const int e = threadIdx.x * 4;
-    const int b = e / HD, hd = e - b * HD;
-    const float* base = pm + (size_t)(b * H + hd / Dh) * NSM * PS + (hd % Dh);
+  uint4 av[PR][NS];
+  auto load = [&](int e0) {
 #pragma unroll
-    for (int sp = 0; sp < NSM; ++sp)
-      av[sp] = (e < B * HD && sp < ns) ? ldg16(base + (size_t)sp * PS) : make_uint4(0, 0, 0, 0);
-  }
-  // 16 lanes per (sequence, head): lane sp holds chunk sp's (max, sum); max and weighted sum by
-  // shuffles inside the 16-lane group
-  for (int i0 = 0; i0 < nbh * NSM; i0 += blockDim.x) {
+    for (int r = 0; r < PR; ++r) {
+      const int e = e0 + r * pass;
+      const int b = e / HD, hd = e - b * HD;
+      const float* base = pm + (size_t)(b * H + hd / Dh) * NSM * PS + (hd % Dh);
+#pragma unroll
+      for (int sp = 0; sp < NS; ++sp) av[r][sp] = e < total ? ldg16(base + (size_t)sp * PS) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  // the accumulator loads of the first round go out first: they do not depend on the chunk
+  // weights, which are formed while they are in flight
+  load((int)threadIdx.x * 4);
+  // NS lanes per (sequence, head): lane sp holds chunk sp's (max, sum); max and weighted sum by
+  // shuffles inside the group
+  for (int i0 = 0; i0 < nbh * NS; i0 += blockDim.x) {
     const int i = i0 + threadIdx.x;
-    const int bh = i / NSM, sp = i % NSM;
-    const bool in = bh < nbh && sp < ns;
+    const int bh = i / NS, sp = i % NS;
+    const bool in = bh < nbh;
     float ms = -INFINITY, ls = 0.f;
     if (in) {
       const uint2 v = ldg8(pm + ((size_t)bh * NSM + sp) * PS + Dh);
@@ -338,37 +344,36 @@ __device__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, i
     }
     float M = ms;
 #pragma unroll
-    for (int o = NSM / 2; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, WAVE));
+    for (int o = NS / 2; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, WAVE));
     const float w = (ms == -INFINITY) ? 0.f : __expf(ms - M);
     float Ls = ls * w;
 #pragma unroll
-    for (int o = NSM / 2; o > 0; o >>= 1) Ls += __shfl_xor(Ls, o, WAVE);
-    if (in) mw[bh * ns + sp] = w;
-    if (bh < nbh && sp == 0) ml[bh] = Ls;
+    for (int o = NS / 2; o > 0; o >>= 1) Ls += __shfl_xor(Ls, o, WAVE);
+    if (in) mw[bh * NS + sp] = w;
+    if (in && sp == 0) ml[bh] = Ls;
   }
   __syncthreads();
-  for (int e = threadIdx.x * 4; e < B * HD; e += blockDim.x * 4) {
-    const int b = e / HD, hd = e - b * HD;
-    const int h = hd / Dh, d = hd - h * Dh;
-    const int bh = b * H + h;
-    if (e != (int)threadIdx.x * 4) {
-      const float* base = pm + (size_t)bh * NSM * PS + d;
+  for (int e0 = threadIdx.x * 4; e0 < total; e0 += pass * PR) {
+    if (e0 != (int)threadIdx.x * 4) load(e0);
 #pragma unroll
-      for (int sp = 0; sp < NSM; ++sp) av[sp] = sp < ns ? ldg16(base + (size_t)sp * PS) : make_uint4(0, 0, 0, 0);
-    }
-    float o[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int r = 0; r < PR; ++r) {
+      const int e = e0 + r * pass;
+      if (e < total) {
+        const int b = e / HD, hd = e - b * HD;
+        const int bh = b * H + hd / Dh;
+        float o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int sp = 0; sp < NSM; ++sp) {
-      if (sp < ns) {
-        const float w = mw[bh * ns + sp];
-        o[0] += __uint_as_float(av[sp].x) * w;
-        o[1] += __uint_as_float(av[sp].y) * w;
-        o[2] += __uint_as_float(av[sp].z) * w;
-        o[3] += __uint_as_float(av[sp].w) * w;
+        for (int sp = 0; sp < NS; ++sp) {
+          const float w = mw[bh * NS + sp];
+          o[0] += __uint_as_float(av[r][sp].x) * w;
+          o[1] += __uint_as_float(av[r][sp].y) * w;
+          o[2] += __uint_as_float(av[r][sp].z) * w;
+          o[3] += __uint_as_float(av[r][sp].w) * w;
+        }
+        const float Ls = ml[bh];
+        sts8(xs + (size_t)b * ldxs + hd, make_uint2(pack_bf(o[0] / Ls, o[1] / Ls), pack_bf(o[2] / Ls, o[3] / Ls)));
       }
     }
-    const float Ls = ml[bh];
-    sts8(xs + (size_t)b * ldxs + hd, make_uint2(pack_bf(o[0] / Ls, o[1] / Ls), pack_bf(o[2] / Ls, o[3] / Ls)));
   }
 }
 
@@ -746,37 +751,63 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
         const bool valid = tb + p < t1;
         const bool more = tb + 64 < t1;
         if (more) attn_tile_load<D>(kb, vb, row, tb + 64, t1, L - 1, kn, vn);
+        // The heads of the group advance in lock step (their cross-lane exchanges overlap); l_run is
+        // this lane's share of the sum, folded over the 16 positions after the loop; the running
+        // maximum is re-derived only for tiles in which some score exceeds it.
+        float sc[G], pv[G];
 #pragma unroll
         for (int hh = 0; hh < G; ++hh) {
           float s = 0.f;
 #pragma unroll
           for (int c = 0; c < NC; ++c) s = dot8m(kv[c], qv[hh][c], s);
-          s += __shfl_xor(s, 16, WAVE);
-          s += __shfl_xor(s, 32, WAVE);
-          s = valid ? s * scale : -INFINITY;
-          float tm = s;
+          sc[hh] = s;
+        }
 #pragma unroll
-          for (int o = 8; o > 0; o >>= 1) tm = fmaxf(tm, __shfl_xor(tm, o, WAVE));
-          const float mn = fmaxf(m_run[hh], tm);
-          const float corr = __expf(m_run[hh] - mn);
-          const float pv = __expf(s - mn);
-          float ts = pv;
+        for (int hh = 0; hh < G; ++hh) sc[hh] += __shfl_xor(sc[hh], 16, WAVE);
 #pragma unroll
-          for (int o = 8; o > 0; o >>= 1) ts += __shfl_xor(ts, o, WAVE);
-          l_run[hh] = l_run[hh] * corr + ts;
-          m_run[hh] = mn;
+        for (int hh = 0; hh < G; ++hh) sc[hh] += __shfl_xor(sc[hh], 32, WAVE);
+        bool raise = false;
 #pragma unroll
-          for (int i = 0; i < 8; ++i) acc[hh][i] *= corr;
+        for (int hh = 0; hh < G; ++hh) {
+          sc[hh] = valid ? sc[hh] * scale : -INFINITY;
+          raise = raise || sc[hh] > m_run[hh];
+        }
+        if (__any(raise)) {
+          float tm[G];
 #pragma unroll
-          for (int c = 0; c < NV; ++c) {
-            const float pw = __shfl(pv, c * PP + pp, WAVE);
-            const uint32_t w4[4] = {vv[c].x, vv[c].y, vv[c].z, vv[c].w};
+          for (int hh = 0; hh < G; ++hh) tm[hh] = sc[hh];
+#pragma unroll
+          for (int o = 8; o > 0; o >>= 1)
+#pragma unroll
+            for (int hh = 0; hh < G; ++hh) tm[hh] = fmaxf(tm[hh], __shfl_xor(tm[hh], o, WAVE));
+#pragma unroll
+          for (int hh = 0; hh < G; ++hh) {
+            const float mn = fmaxf(m_run[hh], tm[hh]);
+            const float corr = __expf(m_run[hh] - mn);
+            m_run[hh] = mn;
+            l_run[hh] *= corr;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[hh][i] *= corr;
+          }
+        }
+#pragma unroll
+        for (int hh = 0; hh < G; ++hh) {
+          pv[hh] = __expf(sc[hh] - m_run[hh]);
+          l_run[hh] += pv[hh];
+        }
+#pragma unroll
+        for (int c = 0; c < NV; ++c) {
+          const uint32_t w4[4] = {vv[c].x, vv[c].y, vv[c].z, vv[c].w};
+          float pw[G];
+#pragma unroll
+          for (int hh = 0; hh < G; ++hh) pw[hh] = __shfl(pv[hh], c * PP + pp, WAVE);
+#pragma unroll
+          for (int hh = 0; hh < G; ++hh)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-              acc[hh][2 * i] += pw * lo_bf(w4[i]);
-              acc[hh][2 * i + 1] += pw * hi_bf(w4[i]);
+              acc[hh][2 * i] += pw[hh] * lo_bf(w4[i]);
+              acc[hh][2 * i + 1] += pw[hh] * hi_bf(w4[i]);
             }
-          }
         }
         if (more) {
 #pragma unroll
@@ -787,6 +818,10 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
       }
     }
     first = false;
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1)
+#pragma unroll
+      for (int hh = 0; hh < G; ++hh) l_run[hh] += __shfl_xor(l_run[hh], o, WAVE);
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) {
 #pragma unroll
@@ -916,7 +951,11 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     // P3: merge + output projection + residual
     if ((int)blockIdx.x < prj.nstrips) {
       if (a.ns == OHARA_MEGA_NS && B * H * D <= 4 * (int)blockDim.x) stage_attn_merge_small(xs, ldxs, p_l, B, H, D);
-      else stage_attn_merge(xs, ldxs, p_l, B, H, D, a.ns, mrg_w, mrg_l);
+      else if (a.ns == 16) stage_attn_merge<16>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
+      else if (a.ns == 8) stage_attn_merge<8>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
+      else if (a.ns == 4) stage_attn_merge<4>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
+      else if (a.ns == 2) stage_attn_merge<2>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
+      else stage_attn_merge<1>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
     }
     __syncthreads();
     pf.stamp();
@@ -1156,6 +1195,7 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   // one attention item per workgroup where the batch allows it
   int ns = n_workgroups / (s->batch * m->n_kv_heads);
   ns = ns < 1 ? 1 : (ns > OHARA_MEGA_NS ? OHARA_MEGA_NS : ns);
+  while (ns & (ns - 1)) ns &= ns - 1;  // a power of two: the merge is specialised per chunk count
   a.ns = ns;
   const size_t mrg = (size_t)2 * ((s->batch * m->n_heads * ns + 1) & ~1) * sizeof(float);
   const size_t smem = xs_bytes + 4096 + (size_t)(8 + 4 * D) * G * sizeof(float) + mrg + (size_t)m->n_layers * 64;

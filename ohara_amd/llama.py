@@ -481,9 +481,10 @@ class DecodeSession:
                 raise ValueError("u must have shape (max_new_tokens, batch)")
             self.u = u.to(device=model.device, dtype=torch.float32).contiguous()
         if persistent is None:
-            # measured on d12: the single launch wins up to four sequences (0.47 ms against 0.48 ms
-            # per step at 4); from eight on the kernel chain is faster (0.50 against 0.58 ms)
-            persistent = model.supports_persistent(batch) and batch <= 4
+            # measured on d12: the single launch wins up to eight sequences (0.40 ms against 0.48 ms
+            # per step at 4, 0.49 against 0.49 at 8); beyond that the kernel chain is faster (0.52
+            # against 0.64 ms at 12)
+            persistent = model.supports_persistent(batch) and batch <= 8
         elif persistent and not model.supports_persistent(batch):
             raise ValueError("the persistent decode kernel does not cover this shape")
         self._pws = None
