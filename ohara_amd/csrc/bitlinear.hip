@@ -109,10 +109,101 @@ __device__ __forceinline__ QuantOut wave_quant_row(const bf16_t* x, const bf16_t
   return QuantOut{s, sq};
 }
 
+// The same for a single row with the whole workgroup (four waves) on it: a decode step at batch 1
+// has one row per projection, and one wave walking 2048-5632 values four times is most of such a
+// kernel's critical path.  Thread t owns the pieces t, t + 256, ...; the three reductions go through
+// `red` (four floats of LDS).  Every thread of the workgroup must call it.
+__device__ __forceinline__ QuantOut block_quant_row(const bf16_t* x, const bf16_t* pre_w, const bf16_t* nw, int K,
+                                                    float eps, int8_t* xq, bf16_t* stage, float* red) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int pieces = K >> 3;
+  auto bsum = [&](float v) {
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    return ((red[0] + red[1]) + red[2]) + red[3];
+  };
+  float ss = 0.f;
+  for (int p = tid; p < pieces; p += 256) {
+    const uint4 u = ldg16(x + (size_t)p * 8);
+    *reinterpret_cast<uint4*>(stage + p * 8) = u;
+    ss += sumsq8_bits(u);
+  }
+  if (pre_w) {
+    const float rinv0 = 1.0f / sqrtf(bsum(ss) / (float)K + eps);
+    ss = 0.f;
+    for (int p = tid; p < pieces; p += 256) {
+      const uint4 u = *reinterpret_cast<const uint4*>(stage + p * 8);
+      const uint4 w = ldg16(pre_w + (size_t)p * 8);
+      const uint32_t uu[4] = {u.x, u.y, u.z, u.w}, ww[4] = {w.x, w.y, w.z, w.w};
+      uint32_t o[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        o[j] = pack_bf(rbf(lo_bf(uu[j]) * rinv0) * lo_bf(ww[j]), rbf(hi_bf(uu[j]) * rinv0) * hi_bf(ww[j]));
+      const uint4 v = make_uint4(o[0], o[1], o[2], o[3]);
+      *reinterpret_cast<uint4*>(stage + p * 8) = v;
+      ss += sumsq8_bits(v);
+    }
+  }
+  const float rinv = 1.0f / sqrtf(bsum(ss) / (float)K + eps);
+  float mx = 0.f;
+  for (int p = tid; p < pieces; p += 256) {
+    const uint4 u = *reinterpret_cast<const uint4*>(stage + p * 8);
+    const uint4 w = ldg16(nw + (size_t)p * 8);
+    const uint32_t uu[4] = {u.x, u.y, u.z, u.w}, ww[4] = {w.x, w.y, w.z, w.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float a0 = rbf(rbf(lo_bf(uu[j]) * rinv) * lo_bf(ww[j]));
+      const float a1 = rbf(rbf(hi_bf(uu[j]) * rinv) * hi_bf(ww[j]));
+      mx = fmaxf(mx, fmaxf(fabsf(a0), fabsf(a1)));
+      o[j] = pack_bf(a0, a1);
+    }
+    *reinterpret_cast<uint4*>(stage + p * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+  mx = wave_max(mx);
+  __syncthreads();
+  if (lane == 0) red[wave] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  const float s = 127.0f / fmaxf(mx, 1e-5f);
+  int sq = 0;
+  for (int p = tid; p < pieces; p += 256) {
+    const uint4 u = *reinterpret_cast<const uint4*>(stage + p * 8);
+    const uint32_t uu[4] = {u.x, u.y, u.z, u.w};
+    uint32_t pk[2] = {0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float v = (j & 1) ? hi_bf(uu[j >> 1]) : lo_bf(uu[j >> 1]);
+      const int qi = (int)fminf(fmaxf(rintf(v * s), -128.f), 127.f);
+      sq += qi;
+      pk[j >> 2] |= ((uint32_t)qi & 0xffu) << (8 * (j & 3));
+    }
+    *reinterpret_cast<uint2*>(xq + (size_t)p * 8) = make_uint2(pk[0], pk[1]);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, WAVE);
+  int* redi = reinterpret_cast<int*>(red);
+  __syncthreads();
+  if (lane == 0) redi[wave] = sq;
+  __syncthreads();
+  return QuantOut{s, redi[0] + redi[1] + redi[2] + redi[3]};
+}
+
 __global__ __launch_bounds__(256) void act_quant_kernel(const bf16_t* x, int ldx, const bf16_t* nw, int rows, int K,
                                                         float eps, int8_t* q, int ldq, float* s_out, int* sumq_out) {
   extern __shared__ __align__(16) unsigned char qsm[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (rows == 1) {  // the whole workgroup on the one row (the order of sums the fused kernels use for it)
+    const QuantOut o = block_quant_row(x, nullptr, nw, K, eps, q, reinterpret_cast<bf16_t*>(qsm),
+                                       reinterpret_cast<float*>(qsm + (size_t)K * 2));
+    if (threadIdx.x == 0) {
+      s_out[0] = o.s;
+      sumq_out[0] = o.sumq;
+    }
+    return;
+  }
   const int r = blockIdx.x * 4 + wave;
   if (r >= rows) return;
   const QuantOut o = wave_quant_row(x + (size_t)r * ldx, nullptr, nw, K, eps, q + (size_t)r * ldq,
@@ -182,7 +273,13 @@ __device__ __forceinline__ bool bitlinear_strip(const BitArgs& a, int strip, uns
     }
   }
   __syncthreads();
-  if (FUSED) {
+  if (FUSED && a.B == 1) {
+    const QuantOut o = block_quant_row(a.x, a.pre_w, a.nw, a.K, a.eps, xq, stage, reinterpret_cast<float*>(red));
+    if (tid == 0) {
+      s_s[0] = o.s;
+      s_sum[0] = o.sumq;
+    }
+  } else if (FUSED) {
     for (int b = wave; b < a.B; b += 4) {
       const QuantOut o = wave_quant_row(a.x + (size_t)b * a.ldx, a.pre_w, a.nw, a.K, a.eps, xq + (size_t)b * ldq,
                                         stage + (size_t)wave * Kp);
