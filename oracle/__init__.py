@@ -31,6 +31,14 @@ Pinning status (what independently fixes each function; see tests/test_oracle.py
   generate loops      the reference tests' literal outputs ("1 2 3 5 5 5",
                       call lengths [3,1,1], positions [0,3,4])
 
+  Phi (phi_ref.py)    rope_partial: the reference RoPE module's vectors (tests/golden/phi_rope.pt)
+                      + fp64 closed form; new_gelu / layer_norm / linear_bias: library routines;
+                      attention: fp64 brute force; phi_forward as a composition is PARITY
+                      UNPINNED by golden logits (ohara/models/phi.py is not importable here: it
+                      needs the absent `lightning` package) - held by the reference test's
+                      cached == uncached invariant and an fp64 hand-written block
+                      (tests/test_oracle_phi.py)
+
 bf16 GEMM accumulation order is "parity unpinned" by the reference (it holds no
 bf16 test); the oracle defines a Linear as an fp32-accumulated product of the
 dtype-rounded operands, rounded once to the model dtype.
