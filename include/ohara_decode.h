@@ -400,6 +400,40 @@ int64_t ohara_persistent_barrier_offset(const OharaModel* m, int batch, int n_sp
 int64_t ohara_persistent_error_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
 int64_t ohara_persistent_profile_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
 
+/* ---- Phi (ohara/models/phi.py): the parts of its cached decode path that differ from Llama ----
+ * nn.Linear WITH bias on packed weights (phi.py:46-47, :63-66, :161), up to any number of rows
+ * (64 at a time).  n % 4 == 0, k % 8 == 0.
+ *   OHARA_LIN_BIAS       out = bf16(x @ W^T + bias)
+ *   OHARA_LIN_BIAS_GELU  out = new_gelu(bf16(x @ W^T + bias)), every op of phi.py:37-40 rounded to
+ *                        bf16 as the eager ops round                          (MLP.fc1, phi.py:50-51)
+ *   OHARA_LIN_BIAS_ADD2  out = bf16(bf16(add1 + bf16(x @ W^T + bias)) + add2): the parallel block's
+ *                        `mixer(x) + mlp(x) + residual` with add1 = mixer output, add2 = block input
+ *                                                                              (phi.py:151) */
+#define OHARA_LIN_BIAS 0
+#define OHARA_LIN_BIAS_GELU 1
+#define OHARA_LIN_BIAS_ADD2 2
+int ohara_linear_bias_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n, int k, const uint16_t* bias, int rows,
+                           int epilogue, const uint16_t* add1, int ld1, const uint16_t* add2, int ld2, uint16_t* out,
+                           int ldo, void* stream);
+/* nn.LayerNorm over the last dimension (phi.py:132, :160): fp32 mean and biased variance,
+ * out = bf16((x - mean) * rstd * weight + bias).  d % 8 == 0. */
+int ohara_layernorm_bf16(const uint16_t* x, int ldx, const uint16_t* weight, const uint16_t* bias, uint16_t* out, int ldo,
+                         int rows, int d, float eps, void* stream);
+/* KVCache.forward for rows that are stored as they are (phi.py:95, kv_cache.py:104-105): row
+ * (b, s) of k / v (leading dimension ld, h*dh wide) -> cache[b, pos + s].  pos_dev (seq_len 1):
+ * the position is read on the device. */
+int ohara_kv_append_bf16(const uint16_t* k, const uint16_t* v, int ld, int batch, int seq_len, int h, int dh, int pos,
+                         const int32_t* pos_dev, uint16_t* kcache, uint16_t* vcache, int t_max, void* stream);
+/* PhiMHA's attention core (phi.py:98-117): fp32 throughout; the first `rot` features of every head
+ * rotate in the half-split layout (feature i with i + rot/2; rotary.py:131-164), queries from
+ * position pos (+ s), the cached UN-rotated keys from 0; key t is visible to query s when
+ * t <= pos + s; softmax(q k^T / sqrt(dh)) v rounded once to bf16.  cos / sin: (t_max, rot/2) fp32
+ * tables of rotary.py:166-184.  q: rows (b, s) with leading dimension ldq; out (batch*seq_len, h*dh).
+ * dh % 8 == 0, dh <= 128. */
+int ohara_phi_attn_bf16(const uint16_t* q, int ldq, const uint16_t* kcache, const uint16_t* vcache, const float* cos,
+                        const float* sin, int rot, int batch, int seq_len, int h, int dh, int t_max, int pos,
+                        const int32_t* pos_dev, uint16_t* out, void* stream);
+
 /* ---- timing helpers (measurement only; no counterpart in the reference) -----------
  * Thin wrappers over hipEventCreate / hipEventDestroy / hipEventElapsedTime so that a
  * benchmark can time single launches on the stream they run on without another HIP

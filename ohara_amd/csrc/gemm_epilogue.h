@@ -3,10 +3,11 @@
 //   residual add       ohara/models/llama.py:199-200
 //   SwiGLU             ohara/modules/mlp.py:152
 //   rotary + KV append ohara/embeddings_pos/rotary.py:55-93, ohara/modules/kv_cache.py:104-105
+//   bias / new_gelu / parallel-block sum of Phi   ohara/models/phi.py:37-52, :147-151
 #pragma once
 #include "common.h"
 
-enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_ROPE = 3 };
+enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_ROPE = 3, EPI_BIAS = 4, EPI_BIAS_GELU = 5, EPI_BIAS_ADD2 = 6 };
 
 struct GemmArgs {
   const uint4* wp;
@@ -30,6 +31,10 @@ struct GemmArgs {
   bf16_t* kcache;
   bf16_t* vcache;
   int stage;  // rotary epilogue: k / v rows go to (rows, Hkv*Dh) buffers at the row index instead of into a cache
+  // nn.Linear with bias (EPI_BIAS*): y = bf16(acc + bias[n]); EPI_BIAS_ADD2: bf16(bf16(resid + y) + resid2)
+  const bf16_t* bias;
+  const bf16_t* resid2;
+  int ldr2;
 };
 
 // gemm_tile.hip: the tiled kernel for calls with many rows (a.B rows, no fused norm).
@@ -64,6 +69,31 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, int b, int stri
       for (int i = 0; i < 4; ++i)
         if (r0 + i < a.N) o[i] = f2bf(v[i]);
     }
+  } else if (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU || EPI == EPI_BIAS_ADD2) {
+    // N % 4 == 0 and 4-element aligned leading dimensions are required by the entry point
+    if (r0 >= a.N) return;
+    const uint2 bv = *reinterpret_cast<const uint2*>(a.bias + r0);
+    float v[4] = {rbf(acc[0] + lo_bf(bv.x)), rbf(acc[1] + hi_bf(bv.x)), rbf(acc[2] + lo_bf(bv.y)),
+                  rbf(acc[3] + hi_bf(bv.y))};
+    if (EPI == EPI_BIAS_GELU) {
+      // phi.py:37-40 op by op, every result rounded as the eager bf16 ops round; torch.pow(x, 3.0)
+      // on bf16 is (x * x) * x with both products rounded
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float x = v[i];
+        const float t2 = rbf(x + rbf(0.044715f * rbf(rbf(x * x) * x)));
+        const float t5 = rbf(1.0f + rbf(tanhf(rbf(0.7978845608028654f * t2))));
+        v[i] = rbf(0.5f * x) * t5;
+      }
+    } else if (EPI == EPI_BIAS_ADD2) {
+      const uint2 r1 = *reinterpret_cast<const uint2*>(a.resid + (size_t)b * a.ldr + r0);
+      const uint2 r2 = *reinterpret_cast<const uint2*>(a.resid2 + (size_t)b * a.ldr2 + r0);
+      v[0] = rbf(lo_bf(r1.x) + v[0]) + lo_bf(r2.x);
+      v[1] = rbf(hi_bf(r1.x) + v[1]) + hi_bf(r2.x);
+      v[2] = rbf(lo_bf(r1.y) + v[2]) + lo_bf(r2.y);
+      v[3] = rbf(hi_bf(r1.y) + v[3]) + hi_bf(r2.y);
+    }
+    *reinterpret_cast<uint2*>(a.out + (size_t)b * a.ldo + r0) = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
   } else if (EPI == EPI_SWIGLU) {
     // rows: gate f, gate f+1, up f, up f+1 with f = 8*strip + 2*g; N = hidden width F
     const int f = strip * 8 + 2 * g;

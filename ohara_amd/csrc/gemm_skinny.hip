@@ -310,6 +310,9 @@ int launch_epi(const GemmArgs& a, int epi, int strips, hipStream_t st) {
     case EPI_RESIDUAL: hipLaunchKernelGGL((skinny_kernel<BT, NORM, EPI_RESIDUAL>), grid, block, 0, st, a); break;
     case EPI_SWIGLU: hipLaunchKernelGGL((skinny_kernel<BT, NORM, EPI_SWIGLU>), grid, block, 0, st, a); break;
     case EPI_ROPE: hipLaunchKernelGGL((skinny_kernel<BT, NORM, EPI_ROPE>), grid, block, 0, st, a); break;
+    case EPI_BIAS: hipLaunchKernelGGL((skinny_kernel<BT, NORM, EPI_BIAS>), grid, block, 0, st, a); break;
+    case EPI_BIAS_GELU: hipLaunchKernelGGL((skinny_kernel<BT, NORM, EPI_BIAS_GELU>), grid, block, 0, st, a); break;
+    case EPI_BIAS_ADD2: hipLaunchKernelGGL((skinny_kernel<BT, NORM, EPI_BIAS_ADD2>), grid, block, 0, st, a); break;
     default: return OHARA_EINVAL;
   }
   return ohara_launch_status();
@@ -340,6 +343,7 @@ int launch_skinny(const GemmArgs& a0, int epi, int packed_rows, hipStream_t st) 
     } else {
       a.out = a0.out + (size_t)r * a0.ldo;
       if (a0.resid) a.resid = a0.resid + (size_t)r * a0.ldr;
+      if (a0.resid2) a.resid2 = a0.resid2 + (size_t)r * a0.ldr2;
     }
     const int rc = launch_chunk(a, epi, strips, st);
     if (rc) return rc;
@@ -398,6 +402,29 @@ int ohara_swiglu_perm(int f, int32_t* perm_host) {
         perm_host[16 * s + 4 * g + i] = fcol < f ? src : -1;
       }
   return OHARA_OK;
+}
+
+int ohara_linear_bias_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n, int k, const uint16_t* bias, int rows,
+                           int epilogue, const uint16_t* add1, int ld1, const uint16_t* add2, int ld2, uint16_t* out,
+                           int ldo, void* stream) {
+  if (!x || !wp || !bias || !out || n < 1 || k < 1 || rows < 1) return OHARA_EINVAL;
+  if ((k & 7) || (ldx & 7) || ldx < k) return OHARA_EINVAL;  // 16-byte activation loads
+  if ((n & 3) || (ldo & 3) || ldo < n) return OHARA_EINVAL;   // 8-byte bias loads and stores
+  int epi;
+  switch (epilogue) {
+    case OHARA_LIN_BIAS: epi = EPI_BIAS; break;
+    case OHARA_LIN_BIAS_GELU: epi = EPI_BIAS_GELU; break;
+    case OHARA_LIN_BIAS_ADD2: epi = EPI_BIAS_ADD2; break;
+    default: return OHARA_EINVAL;
+  }
+  if (epi == EPI_BIAS_ADD2 && (!add1 || !add2 || (ld1 & 3) || (ld2 & 3) || ld1 < n || ld2 < n)) return OHARA_EINVAL;
+  GemmArgs a{};
+  a.wp = reinterpret_cast<const uint4*>(wp);
+  a.x = x; a.ldx = ldx;
+  a.B = rows; a.N = n; a.K = k;
+  a.out = out; a.ldo = ldo; a.bias = bias;
+  a.resid = add1; a.ldr = ld1; a.resid2 = add2; a.ldr2 = ld2;
+  return launch_skinny(a, epi, (n + 15) / 16 * 16, (hipStream_t)stream);
 }
 
 int ohara_gemm_skinny_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n, int k, const uint16_t* norm_w,

@@ -1,0 +1,260 @@
+// Phi's side of the KV-cache decode path (ohara/models/phi.py): what differs from Llama.
+//   LayerNorm with bias                     phi.py:132, :160 (nn.LayerNorm: fp32 statistics, one rounding)
+//   append of the UN-rotated key / value    phi.py:95 (kv_cache.py:104-105)
+//   attention in fp32 with the partial half-split rotation applied after the cache read
+//                                           phi.py:98-117, rotary.py:131-184
+// The projections with bias, new_gelu and the parallel-block sum are epilogues of the skinny
+// GEMM (gemm_epilogue.h).
+#include "common.h"
+
+namespace {
+
+// ---- LayerNorm: one workgroup per row ---------------------------------------------------
+__global__ __launch_bounds__(256) void layernorm_kernel(const bf16_t* x, int ldx, const bf16_t* w, const bf16_t* b,
+                                                        bf16_t* out, int ldo, int d, float eps) {
+  __shared__ float red[2][4];
+  const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const bf16_t* xr = x + (size_t)row * ldx;
+  // pass 1: mean
+  float s = 0.f;
+  for (int k = tid * 8; k < d; k += 256 * 8) {
+    const uint4 v = ldg16(xr + k);
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s += lo_bf(u[i]) + hi_bf(u[i]);
+  }
+  s = wave_sum(s);
+  if (lane == 0) red[0][wave] = s;
+  __syncthreads();
+  const float mean = (((red[0][0] + red[0][1]) + red[0][2]) + red[0][3]) / (float)d;
+  // pass 2: biased variance around the mean (the row is re-read from cache)
+  float q = 0.f;
+  for (int k = tid * 8; k < d; k += 256 * 8) {
+    const uint4 v = ldg16(xr + k);
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float a0 = lo_bf(u[i]) - mean, a1 = hi_bf(u[i]) - mean;
+      q += a0 * a0 + a1 * a1;
+    }
+  }
+  q = wave_sum(q);
+  if (lane == 0) red[1][wave] = q;
+  __syncthreads();
+  const float var = (((red[1][0] + red[1][1]) + red[1][2]) + red[1][3]) / (float)d;
+  const float rstd = 1.0f / sqrtf(var + eps);
+  for (int k = tid * 8; k < d; k += 256 * 8) {
+    const uint4 v = ldg16(xr + k), g = ldg16(w + k), c = ldg16(b + k);
+    const uint32_t u[4] = {v.x, v.y, v.z, v.w}, gu[4] = {g.x, g.y, g.z, g.w}, cu[4] = {c.x, c.y, c.z, c.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      o[i] = pack_bf((lo_bf(u[i]) - mean) * rstd * lo_bf(gu[i]) + lo_bf(cu[i]),
+                     (hi_bf(u[i]) - mean) * rstd * hi_bf(gu[i]) + hi_bf(cu[i]));
+    *reinterpret_cast<uint4*>(out + (size_t)row * ldo + k) = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
+// ---- append: rows (seq, s) of k and v -> cache position pos + s ------------------------------
+__global__ void kv_append_kernel(const bf16_t* k, const bf16_t* v, int ld, int rows, int S, int hd, int t_max, int pos,
+                                 const int32_t* pos_dev, bf16_t* kc, bf16_t* vc) {
+  const int n8 = hd >> 3;
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= rows * n8) return;
+  const int row = idx / n8, c = (idx - row * n8) * 8;
+  const int seq = row / S, t = (pos_dev ? *pos_dev : pos) + (row - seq * S);
+  if (t < 0 || t >= t_max) return;
+  const size_t dst = ((size_t)seq * t_max + t) * hd + c;
+  *reinterpret_cast<uint4*>(kc + dst) = ldg16(k + (size_t)row * ld + c);
+  *reinterpret_cast<uint4*>(vc + dst) = ldg16(v + (size_t)row * ld + c);
+}
+
+// ---- attention ---------------------------------------------------------------------------
+// One workgroup per (sequence, head, new token).  Sixteen lanes own one cached position at a time
+// (lane l the eight features 8l .. 8l+7), so a workgroup walks 16 positions per round with an online
+// softmax per 16-lane group; the groups are merged through LDS at the end.
+//
+// The reference rotates every cached key again at each step (phi.py:104).  With the rotated query
+// qr and c, s the cosine / sine of key position t the score is
+//   sum_i (k1_i c_i - k2_i s_i) qr1_i + (k1_i s_i + k2_i c_i) qr2_i + sum_rest k_j q_j
+//     = sum_i k1_i (c_i qr1_i + s_i qr2_i) + k2_i (c_i qr2_i - s_i qr1_i) + sum_rest k_j q_j,
+// i.e. a dot product of the raw key row with a per-position weight vector built from two per-lane
+// constants A, B: w_j = c A_j + s B_j.  All of it in fp32, as the reference (phi.py:98-100).
+struct PhiAttnArgs {
+  const bf16_t* q;
+  int ldq;
+  const bf16_t* kc;
+  const bf16_t* vc;
+  const float* cos;  // (t_max, rot/2) fp32
+  const float* sin;
+  bf16_t* out;       // (rows, H*D)
+  int S, H, D, rot, t_max, pos;
+  const int32_t* pos_dev;
+};
+
+__global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
+  __shared__ float qr[128];
+  __shared__ float gm[16], gl[16];
+  __shared__ float gacc[16][128];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int grp = wave * 4 + (lane >> 4), l = lane & 15;
+  const int D = a.D, half = a.rot >> 1;
+  int w = blockIdx.x;
+  const int s = w % a.S; w /= a.S;
+  const int h = w % a.H;
+  const int seq = w / a.H;
+  const int row = seq * a.S + s;
+  const int pq = (a.pos_dev ? *a.pos_dev : a.pos) + s;  // position of this query; keys 0 .. pq are visible
+  if (pq < 0 || pq >= a.t_max) return;
+
+  if (tid < D) {
+    const bf16_t* qrow = a.q + (size_t)row * a.ldq + h * D;
+    float v = bf2f(qrow[tid]);
+    if (tid < half) {
+      const float c = a.cos[(size_t)pq * half + tid], sn = a.sin[(size_t)pq * half + tid];
+      v = v * c - bf2f(qrow[tid + half]) * sn;
+    } else if (tid < a.rot) {
+      const int i = tid - half;
+      const float c = a.cos[(size_t)pq * half + i], sn = a.sin[(size_t)pq * half + i];
+      v = bf2f(qrow[i]) * sn + v * c;
+    }
+    qr[tid] = v;
+  }
+  __syncthreads();
+
+  const int e0 = 8 * l;
+  const bool own = e0 < D;
+  float A[8], Bc[8];
+  int f[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int j = e0 + u;
+    A[u] = own ? qr[j] : 0.f;
+    Bc[u] = 0.f;
+    f[u] = -1;
+    if (own && j < half) {
+      Bc[u] = qr[j + half];
+      f[u] = j;
+    } else if (own && j < a.rot) {
+      Bc[u] = -qr[j - half];
+      f[u] = j - half;
+    }
+  }
+  const bool rotates = own && e0 < a.rot;
+  const float scale = sqrtf(1.0f / (float)D);
+
+  float m = -INFINITY, lsum = 0.f, acc[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) acc[u] = 0.f;
+  const size_t hd = (size_t)a.H * D;
+  const bf16_t* kb = a.kc + (size_t)seq * a.t_max * hd + (size_t)h * D + e0;
+  const bf16_t* vb = a.vc + (size_t)seq * a.t_max * hd + (size_t)h * D + e0;
+  for (int t = grp; t <= pq; t += 16) {
+    float part = 0.f;
+    uint4 vv = make_uint4(0, 0, 0, 0);
+    if (own) {
+      const uint4 kv = ldg16(kb + (size_t)t * hd);
+      vv = ldg16(vb + (size_t)t * hd);
+      const uint32_t ku[4] = {kv.x, kv.y, kv.z, kv.w};
+      float kf[8];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        kf[2 * i] = lo_bf(ku[i]);
+        kf[2 * i + 1] = hi_bf(ku[i]);
+      }
+      if (rotates) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          float wgt = A[u];
+          if (f[u] >= 0) wgt = a.cos[(size_t)t * half + f[u]] * A[u] + a.sin[(size_t)t * half + f[u]] * Bc[u];
+          part += kf[u] * wgt;
+        }
+      } else {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) part += kf[u] * A[u];
+      }
+    }
+#pragma unroll
+    for (int o = 1; o < 16; o <<= 1) part += __shfl_xor(part, o, WAVE);
+    const float sc = part * scale;
+    const float mn = fmaxf(m, sc);
+    const float corr = expf(m - mn), p = expf(sc - mn);  // m = -inf on the first round: corr = 0
+    lsum = lsum * corr + p;
+    const uint32_t vu[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      acc[2 * i] = acc[2 * i] * corr + p * lo_bf(vu[i]);
+      acc[2 * i + 1] = acc[2 * i + 1] * corr + p * hi_bf(vu[i]);
+    }
+    m = mn;
+  }
+  if (l == 0) {
+    gm[grp] = m;
+    gl[grp] = lsum;
+  }
+  if (own) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) gacc[grp][e0 + u] = acc[u];
+  }
+  __syncthreads();
+  if (tid < D) {
+    float M = -INFINITY;
+#pragma unroll
+    for (int g = 0; g < 16; ++g) M = fmaxf(M, gm[g]);
+    float num = 0.f, den = 0.f;
+#pragma unroll
+    for (int g = 0; g < 16; ++g) {
+      if (gm[g] == -INFINITY) continue;  // a group that saw no position
+      const float wg = expf(gm[g] - M);
+      num += wg * gacc[g][tid];
+      den += wg * gl[g];
+    }
+    a.out[(size_t)row * hd + (size_t)h * D + tid] = f2bf(num / den);
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int ohara_layernorm_bf16(const uint16_t* x, int ldx, const uint16_t* weight, const uint16_t* bias, uint16_t* out, int ldo,
+                         int rows, int d, float eps, void* stream) {
+  if (!x || !weight || !bias || !out || rows < 1 || d < 8) return OHARA_EINVAL;
+  if ((d & 7) || (ldx & 7) || (ldo & 7) || ldx < d || ldo < d) return OHARA_EINVAL;
+  hipLaunchKernelGGL(layernorm_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, x, ldx, weight, bias, out, ldo, d,
+                     eps);
+  return ohara_launch_status();
+}
+
+int ohara_kv_append_bf16(const uint16_t* k, const uint16_t* v, int ld, int batch, int seq_len, int h, int dh, int pos,
+                         const int32_t* pos_dev, uint16_t* kcache, uint16_t* vcache, int t_max, void* stream) {
+  if (!k || !v || !kcache || !vcache || batch < 1 || seq_len < 1 || h < 1 || dh < 1 || t_max < 1) return OHARA_EINVAL;
+  const int64_t hd = (int64_t)h * dh;
+  if ((hd & 7) || (ld & 7) || ld < hd) return OHARA_EINVAL;
+  if (!pos_dev && (pos < 0 || pos + seq_len > t_max)) return OHARA_EINVAL;
+  if (pos_dev && seq_len != 1) return OHARA_EINVAL;
+  const int64_t total = (int64_t)batch * seq_len * (hd >> 3);
+  if (total > INT32_MAX) return OHARA_ESIZE;
+  hipLaunchKernelGGL(kv_append_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, k, v, ld,
+                     batch * seq_len, seq_len, (int)hd, t_max, pos, pos_dev, kcache, vcache);
+  return ohara_launch_status();
+}
+
+int ohara_phi_attn_bf16(const uint16_t* q, int ldq, const uint16_t* kcache, const uint16_t* vcache, const float* cos,
+                        const float* sin, int rot, int batch, int seq_len, int h, int dh, int t_max, int pos,
+                        const int32_t* pos_dev, uint16_t* out, void* stream) {
+  if (!q || !kcache || !vcache || !cos || !sin || !out) return OHARA_EINVAL;
+  if (batch < 1 || seq_len < 1 || h < 1 || t_max < 1) return OHARA_EINVAL;
+  if (dh < 8 || dh > 128 || (dh & 7)) return OHARA_ESIZE;
+  if (rot < 2 || (rot & 1) || rot > dh) return OHARA_EINVAL;  // rotary.py:118-121
+  if (ldq < h * dh) return OHARA_EINVAL;
+  if (!pos_dev && (pos < 0 || pos + seq_len > t_max)) return OHARA_EINVAL;
+  if (pos_dev && seq_len != 1) return OHARA_EINVAL;
+  const int64_t grid = (int64_t)batch * seq_len * h;
+  if (grid > INT32_MAX) return OHARA_ESIZE;
+  PhiAttnArgs a{q, ldq, kcache, vcache, cos, sin, out, seq_len, h, dh, rot, t_max, pos, pos_dev};
+  hipLaunchKernelGGL(phi_attn_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, a);
+  return ohara_launch_status();
+}
+
+}  // extern "C"

@@ -450,3 +450,67 @@ def rope_append(q, k, v, batch, seq_len, h, h_kv, dh, cos, sin, pos, kcache, vca
                                        int(pos), _ptr(pos_dev), _ptr(kcache), _ptr(vcache), kcache.shape[1], _stream()),
           "rope_append")
     return q
+
+
+# ---- Phi (ohara/models/phi.py) ----------------------------------------------------------------
+
+_LIN_EPI = {"bias": 0, "gelu": 1, "add2": 2}
+
+
+def linear_bias(x, w: PackedLinear, bias, epilogue: str = "bias", add1=None, add2=None, out=None) -> torch.Tensor:
+    """nn.Linear with bias on a packed weight; ``epilogue``: "bias", "gelu" (new_gelu of the result,
+    phi.py:37-40) or "add2" (bf16(bf16(add1 + y) + add2), phi.py:151).  x: (rows, K), any row stride."""
+    if x.dtype != BF16 or not x.is_cuda or x.stride(1) != 1:
+        raise ValueError("x must be a bf16 device matrix with unit column stride")
+    _need(bias, BF16, "bias")
+    rows, k = x.shape
+    if k != w.k or bias.numel() != w.n:
+        raise ValueError(f"x has {k} columns / bias {bias.numel()} entries, weight is {w.n} x {w.k}")
+    if out is None:
+        out = torch.empty(rows, w.n, dtype=BF16, device=x.device)
+    for t in (add1, add2):
+        if t is not None and (t.dtype != BF16 or t.stride(1) != 1):
+            raise ValueError("addends must be bf16 with unit column stride")
+    check(
+        lib().ohara_linear_bias_bf16(
+            _ptr(x), x.stride(0), _ptr(w.data), w.n, w.k, _ptr(bias), rows, _LIN_EPI[epilogue],
+            _ptr(add1), 0 if add1 is None else add1.stride(0), _ptr(add2), 0 if add2 is None else add2.stride(0),
+            _ptr(out), out.stride(0), _stream(),
+        ),
+        "linear_bias",
+    )
+    return out
+
+
+def layernorm(x, weight, bias, eps: float = 1e-5, out=None) -> torch.Tensor:
+    """nn.LayerNorm over the last dimension of a (rows, d) bf16 matrix (phi.py:132, :160)."""
+    _need(x, BF16, "x")
+    rows, d = x.shape
+    if out is None:
+        out = torch.empty_like(x)
+    check(lib().ohara_layernorm_bf16(_ptr(x), x.stride(0), _ptr(weight), _ptr(bias), _ptr(out), out.stride(0), rows, d, eps,
+                                     _stream()), "layernorm")
+    return out
+
+
+def kv_append(k, v, kcache, vcache, batch, seq_len, h, dh, pos, pos_dev=None) -> None:
+    """Rows (b, s) of k / v (views with a common row stride) -> cache[b, pos + s] as they are
+    (phi.py:95)."""
+    if k.stride(0) != v.stride(0) or k.stride(1) != 1 or v.stride(1) != 1:
+        raise ValueError("k and v must share a row stride and have unit column stride")
+    check(lib().ohara_kv_append_bf16(_ptr(k), _ptr(v), k.stride(0), batch, seq_len, h, dh, pos, _ptr(pos_dev), _ptr(kcache),
+                                     _ptr(vcache), kcache.shape[1], _stream()), "kv_append")
+
+
+def phi_attn(q, kcache, vcache, cos, sin, rot, batch, seq_len, h, dh, pos, pos_dev=None, out=None) -> torch.Tensor:
+    """PhiMHA's attention core over the cache (phi.py:98-117); q: (rows, h*dh) view with any row
+    stride; cos / sin: fp32 (t_max, rot/2)."""
+    if q.stride(1) != 1:
+        raise ValueError("q must have unit column stride")
+    if cos.dtype != torch.float32 or sin.dtype != torch.float32:
+        raise ValueError("cos / sin must be fp32")
+    if out is None:
+        out = torch.empty(batch * seq_len, h * dh, dtype=BF16, device=q.device)
+    check(lib().ohara_phi_attn_bf16(_ptr(q), q.stride(0), _ptr(kcache), _ptr(vcache), _ptr(cos), _ptr(sin), rot, batch,
+                                    seq_len, h, dh, kcache.shape[1], pos, _ptr(pos_dev), _ptr(out), _stream()), "phi_attn")
+    return out

@@ -1,0 +1,169 @@
+"""Phi-2 (ohara/models/phi.py) on the HIP kernels: the reference's ``Phi`` call surface for the
+cached decode path.
+
+What differs from Llama, all of it as the reference has it: attention and the MLP run in parallel
+off one LayerNorm (phi.py:147-151), every Linear has a bias, the MLP is fc1 -> new_gelu -> fc2
+(phi.py:37-52), only ``int(rotary_dim * head_dim)`` features of a head rotate, in the half-split
+layout, and the cache holds the UN-rotated keys: the rotation is applied to all cached keys at
+every step, in fp32, inside the attention kernel (phi.py:95-104).
+
+bf16 only (the reference's ``from_pretrained`` builds an fp16 model, phi.py:229-231; its tests run
+fp32).  Checkpoint download (phi.py:226-256) is not provided: pass a state dict with the reference's
+names (``Phi._huggingface_state_dict_map`` keys).
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+
+import torch
+
+from . import ops
+from ._lib import lib
+from .llama import KVCache
+
+BF16 = torch.bfloat16
+
+
+@dataclass
+class PhiConfig:
+    """ohara/models/phi.py:23-34, same fields and defaults."""
+
+    vocab_size: int = 51200
+    max_sequence_length: int = 2048
+    hidden_size: int = 2560
+    num_attention_heads: int = 32
+    num_hidden_layers: int = 32
+    dropout: float = 0.2
+    multiple_of: int = 4
+    bias: bool = True
+    eps: float = 1e-5
+    rotary_dim: float = 0.4
+
+
+def rope_cos_sin(num_positions: int, dims: int, base: float = 10000.0):
+    """RoPE.create_cos_sin_theta (ohara/embeddings_pos/rotary.py:166-184) for fp32 inputs, positions
+    0 .. num_positions-1: the same fp32 operations on the host, so the tables carry the same values."""
+    half = dims // 2
+    positions = torch.arange(0, num_positions, dtype=torch.float32)
+    freqs = torch.exp(-torch.arange(0.0, half, dtype=torch.float32) * (math.log(base) / half))
+    theta = positions.reshape(-1, 1) * freqs.reshape(1, -1)
+    return torch.cos(theta), torch.sin(theta)
+
+
+class Phi:
+    """``Phi`` (ohara/models/phi.py:155-205): ``forward(x, kv_cache, position_ids)`` and
+    ``build_kv_cache``.  ``state`` uses the reference's state-dict names."""
+
+    def __init__(self, config: PhiConfig, state: dict, device="cuda", dtype=BF16):
+        if dtype != BF16:
+            raise ValueError("ohara_amd runs the decode path in bfloat16 only")
+        c = config
+        if c.hidden_size % c.num_attention_heads:
+            raise ValueError("hidden_size must be divisible by num_attention_heads")
+        self.head_dim = c.hidden_size // c.num_attention_heads
+        self.rot = int(c.rotary_dim * self.head_dim)  # phi.py:69
+        if self.rot < 2 or self.rot % 2:
+            raise ValueError(f"RoPE dims must be a positive even number, got {self.rot}")  # rotary.py:118-121
+        if self.head_dim % 8 or self.head_dim > 128 or c.hidden_size % 8:
+            raise NotImplementedError("ohara_amd Phi: head_dim must be a multiple of 8 up to 128")
+        if not c.bias:
+            raise NotImplementedError("ohara_amd Phi: bias=False is not a configuration the reference builds")
+        lib()  # fail loudly now if the HIP library is missing
+        self.config, self.device, self.dtype = c, torch.device(device), dtype
+        self.ff = c.multiple_of * c.hidden_size  # phi.py:138
+
+        def dev(t):
+            return t.detach().to(device=self.device, dtype=BF16).contiguous()
+
+        self.wte = dev(state["wte.weight"])
+        self.ln_w, self.ln_b = dev(state["ln.weight"]), dev(state["ln.bias"])
+        self.lm_head = ops.pack_linear(dev(state["lm_head.weight"]))
+        self.lm_bias = dev(state["lm_head.bias"])
+        cos, sin = rope_cos_sin(c.max_sequence_length, self.rot)
+        self.cos, self.sin = cos.to(self.device).contiguous(), sin.to(self.device).contiguous()
+        self.layers = []
+        for i in range(c.num_hidden_layers):
+            p = f"layers.{i}."
+            # one packed [q; k; v] weight: the three projections read the same rows (phi.py:81-83)
+            wqkv = torch.cat([dev(state[p + f"mixer.{n}.weight"]) for n in ("q_proj", "k_proj", "v_proj")])
+            bqkv = torch.cat([dev(state[p + f"mixer.{n}.bias"]) for n in ("q_proj", "k_proj", "v_proj")])
+            self.layers.append(dict(
+                ln_w=dev(state[p + "ln.weight"]), ln_b=dev(state[p + "ln.bias"]),
+                wqkv=ops.pack_linear(wqkv), bqkv=bqkv.contiguous(),
+                dense=ops.pack_linear(dev(state[p + "mixer.dense.weight"])), dense_b=dev(state[p + "mixer.dense.bias"]),
+                fc1=ops.pack_linear(dev(state[p + "mlp.fc1.weight"])), fc1_b=dev(state[p + "mlp.fc1.bias"]),
+                fc2=ops.pack_linear(dev(state[p + "mlp.fc2.weight"])), fc2_b=dev(state[p + "mlp.fc2.bias"]),
+            ))
+            del wqkv
+        torch.cuda.synchronize(self.device)
+        self._bufs: dict = {}
+
+    def eval(self):
+        return self
+
+    def build_kv_cache(self, batch_size: int = 1) -> list[KVCache]:
+        if batch_size < 1:
+            raise ValueError("batch_size must be at least 1")  # phi.py:190-191
+        c = self.config
+        shape = (batch_size, c.max_sequence_length, c.num_attention_heads, self.head_dim)
+        return [KVCache(shape, c.max_sequence_length, i, device=self.device, dtype=BF16)
+                for i in range(c.num_hidden_layers)]
+
+    def _buffers(self, rows: int):
+        b = self._bufs.get(rows)
+        if b is None:
+            if len(self._bufs) > 4:
+                self._bufs.clear()
+            d = self.config.hidden_size
+            new = lambda n: torch.empty(rows, n, dtype=BF16, device=self.device)
+            b = dict(x=[new(d), new(d)], h=new(d), qkv=new(3 * d), attn=new(d), mixer=new(d), act=new(self.ff))
+            self._bufs[rows] = b
+        return b
+
+    @torch.no_grad()
+    def forward(self, x: torch.Tensor, kv_cache: list | None = None, position_ids=None, *, pos_dev=None,
+                last_only: bool = False) -> torch.Tensor:
+        """Logits (B, S, vocab) for the tokens not cached yet (phi.py:170-186).  Without a cache the
+        tokens run through a scratch cache from position 0, which is the causal forward.  ``pos_dev``
+        (int32 device scalar, S == 1) lets the kernels read the position on the device, for graph
+        replay; the caller advances it.  ``last_only`` computes the last row of logits only."""
+        c = self.config
+        if kv_cache is not None and len(kv_cache) != c.num_hidden_layers:
+            raise ValueError("KV cache must contain one entry per model layer")
+        if x.dim() != 2:
+            raise ValueError("x must be (batch, seq_len) token ids")
+        B, S = x.shape
+        if kv_cache is None:
+            if S > c.max_sequence_length:
+                raise ValueError("input exceeds max_sequence_length")
+            kv_cache, start = self.build_kv_cache(B), 0
+        else:
+            if position_ids is None:
+                raise ValueError("position_ids is required when using a KV cache")  # phi.py:92-93
+            start = int(position_ids)
+        ends = [cache._reserve(B, S, start) for cache in kv_cache]
+        rows, d, H, D = B * S, c.hidden_size, c.num_attention_heads, self.head_dim
+        buf = self._buffers(rows)
+        cur, nxt = buf["x"]
+        ops.embed(x.reshape(-1).to(device=self.device, dtype=torch.int64), self.wte, out=cur)
+        for L, cache in zip(self.layers, kv_cache):
+            h, qkv = buf["h"], buf["qkv"]
+            ops.layernorm(cur, L["ln_w"], L["ln_b"], c.eps, out=h)
+            ops.linear_bias(h, L["wqkv"], L["bqkv"], out=qkv)
+            ops.kv_append(qkv[:, d:2 * d], qkv[:, 2 * d:], cache.key, cache.value, B, S, H, D, start, pos_dev)
+            ops.phi_attn(qkv[:, :d], cache.key, cache.value, self.cos, self.sin, self.rot, B, S, H, D, start, pos_dev,
+                         out=buf["attn"])
+            ops.linear_bias(buf["attn"], L["dense"], L["dense_b"], out=buf["mixer"])
+            ops.linear_bias(h, L["fc1"], L["fc1_b"], "gelu", out=buf["act"])
+            ops.linear_bias(buf["act"], L["fc2"], L["fc2_b"], "add2", add1=buf["mixer"], add2=cur, out=nxt)
+            cur, nxt = nxt, cur
+        src = cur.view(B, S, d)[:, -1] if last_only else cur
+        hn = ops.layernorm(src.contiguous() if last_only else src, self.ln_w, self.ln_b, c.eps)
+        logits = ops.linear_bias(hn, self.lm_head, self.lm_bias)
+        for cache, end in zip(kv_cache, ends):
+            cache._commit(B, end)
+        return logits.view(B, 1 if last_only else S, c.vocab_size)
+
+    __call__ = forward

@@ -1,0 +1,197 @@
+"""Phi's cached decode path on the GPU (ohara/models/phi.py) against the CPU oracle
+(oracle/phi_ref.py) on the same seeded inputs, through the C ABI."""
+
+import dataclasses
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import phi_ref as P
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+
+
+def _ulp_close(got, want32, ulps=1.0, floor=2.0 ** -9):
+    """|got - want| within `ulps` bf16 ulps of the fp32 value (an ulp is at most 2^-7 of the value)."""
+    got, want32 = got.float().cpu(), want32.float().cpu()
+    bound = ulps * 2.0 ** -7 * want32.abs().clamp_min(floor) + 1e-6
+    bad = (got - want32).abs() > bound
+    assert not bad.any(), ((got - want32).abs().max().item(), int(bad.sum()))
+
+
+def test_layernorm_matches_the_library_routine(cuda):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(0)
+    for rows, d in ((1, 64), (5, 2560), (33, 320), (3, 4104)):
+        x = (torch.randn(rows, d, generator=g) * 2 + 0.5).to(BF)
+        w = (1 + 0.1 * torch.randn(d, generator=g)).to(BF)
+        b = (0.1 * torch.randn(d, generator=g)).to(BF)
+        got = ops.layernorm(x.to(cuda), w.to(cuda), b.to(cuda), 1e-5)
+        want32 = F.layer_norm(x.float(), (d,), w.float(), b.float(), 1e-5)
+        _ulp_close(got, want32, ulps=0.51)  # one rounding of the fp32 value
+        ref = P.layer_norm(x, w, b, 1e-5)
+        assert (got.cpu() != ref).float().mean() < 2e-3  # round-to-nearest ties of fp32 noise only
+
+
+def test_linear_bias_epilogues(cuda):
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(1)
+    for rows, n, k in ((1, 64, 64), (7, 320, 1280), (64, 1280, 320), (70, 96, 64)):
+        x = torch.randn(rows, k, generator=g).to(BF)
+        w = (torch.randn(n, k, generator=g) / k ** 0.5).to(BF)
+        b = (0.2 * torch.randn(n, generator=g)).to(BF)
+        a1 = torch.randn(rows, n, generator=g).to(BF)
+        a2 = torch.randn(rows, n, generator=g).to(BF)
+        pw = ops.pack_linear(w.to(cuda))
+        y = ops.linear_bias(x.to(cuda), pw, b.to(cuda))
+        y32 = x.float() @ w.float().t() + b.float()
+        _ulp_close(y, y32, ulps=0.6)
+        # the fused epilogues continue from the same rounded y: compare with the oracle's op-by-op
+        # bf16 arithmetic applied to the kernel's own y
+        gel = ops.linear_bias(x.to(cuda), pw, b.to(cuda), "gelu")
+        want = P.new_gelu(y.cpu())
+        diff = (gel.cpu().float() - want.float()).abs()
+        assert (diff > 0).float().mean() < 5e-3, (diff > 0).float().mean()  # tanhf vs the host's tanh, last fp32 ulp
+        # where they differ, tanh's bf16 rounding moved by one ulp (2^-8 near +-1), scaled by 0.5 * y
+        assert (diff <= 2.0 ** -8 * y.cpu().float().abs() + 2.0 ** -7 * want.float().abs() + 1e-6).all()
+        out = ops.linear_bias(x.to(cuda), pw, b.to(cuda), "add2", add1=a1.to(cuda), add2=a2.to(cuda))
+        assert torch.equal(out.cpu(), (a1 + y.cpu()) + a2)
+    # strided input rows (a column slice of a wider buffer)
+    wide = torch.randn(5, 3 * 64, generator=g).to(BF).to(cuda)
+    w = (torch.randn(32, 64, generator=g) / 8).to(BF).to(cuda)
+    b = torch.zeros(32, dtype=BF, device=cuda)
+    got = ops.linear_bias(wide[:, 64:128], ops.pack_linear(w), b)
+    _ulp_close(got, wide[:, 64:128].float() @ w.float().t(), ulps=0.6)
+    with pytest.raises(ValueError):
+        ops.linear_bias(wide[:, :64], ops.pack_linear(w), torch.zeros(16, dtype=BF, device=cuda))
+
+
+def test_kv_append_and_attention_against_the_oracle(cuda):
+    from ohara_amd import ops
+    from ohara_amd.phi import rope_cos_sin
+
+    g = torch.Generator().manual_seed(2)
+    for B, S, L0, H, D, rot, Tmax in ((2, 1, 9, 4, 16, 6, 32), (1, 5, 0, 2, 80, 32, 16), (3, 2, 30, 2, 128, 128, 40),
+                                      (1, 1, 0, 1, 8, 2, 4), (2, 1, 299, 2, 64, 24, 300)):
+        hd = H * D
+        kc = torch.zeros(B, Tmax, H, D, dtype=BF)
+        vc = torch.zeros(B, Tmax, H, D, dtype=BF)
+        kc[:, :L0] = torch.randn(B, L0, H, D, generator=g).to(BF)
+        vc[:, :L0] = torch.randn(B, L0, H, D, generator=g).to(BF)
+        qkv = torch.randn(B * S, 3 * hd, generator=g).to(BF)
+        kcd, vcd, qkvd = kc.to(cuda), vc.to(cuda), qkv.to(cuda)
+        ops.kv_append(qkvd[:, hd:2 * hd], qkvd[:, 2 * hd:], kcd, vcd, B, S, H, D, L0)
+        kc[:, L0:L0 + S] = qkv[:, hd:2 * hd].view(B, S, H, D)
+        vc[:, L0:L0 + S] = qkv[:, 2 * hd:].view(B, S, H, D)
+        assert torch.equal(kcd.cpu(), kc) and torch.equal(vcd.cpu(), vc)
+        cos, sin = rope_cos_sin(Tmax, rot)
+        ref_cos, ref_sin = P.rope_cos_sin(Tmax, rot)
+        assert torch.equal(cos, ref_cos) and torch.equal(sin, ref_sin)
+        got = ops.phi_attn(qkvd[:, :hd], kcd, vcd, cos.to(cuda), sin.to(cuda), rot, B, S, H, D, L0)
+        want = P.attention(qkv[:, :hd].view(B, S, H, D), kc[:, :L0 + S], vc[:, :L0 + S], L0, rot, torch.float32)
+        _ulp_close(got.view(B, S, H, D), want, ulps=0.6, floor=2.0 ** -6)
+        if S == 1:  # position read on the device
+            pd = torch.tensor([L0], dtype=torch.int32, device=cuda)
+            got2 = ops.phi_attn(qkvd[:, :hd], kcd, vcd, cos.to(cuda), sin.to(cuda), rot, B, S, H, D, 0, pos_dev=pd)
+            assert torch.equal(got2, got)
+
+
+def _pair(cuda, dtype=BF, seed=5, **kw):
+    from ohara_amd.phi import Phi, PhiConfig
+
+    base = dict(vocab_size=64, max_sequence_length=16, hidden_size=64, num_attention_heads=4, num_hidden_layers=2,
+                multiple_of=4, rotary_dim=0.4)
+    base.update(kw)
+    rcfg = P.RefPhiConfig(**base)
+    w = P.init_weights(rcfg, seed=seed, dtype=dtype, std=0.08, bias_std=0.05)
+    return P.RefPhi(rcfg, w), Phi(PhiConfig(**base), w, device=cuda)
+
+
+def _close(got, ref, max_rel=4e-2, mean_rel=4e-3):
+    got, ref = got.float().cpu(), ref.float()
+    scale = ref.abs().max().item()
+    d = (got - ref).abs()
+    assert d.max().item() <= max_rel * scale, (d.max().item(), scale)
+    assert d.mean().item() <= mean_rel * scale, (d.mean().item(), scale)
+
+
+@pytest.mark.parametrize("kw", [
+    dict(),                                                                      # head_dim 16, 6 rotated features
+    dict(vocab_size=80, max_sequence_length=12, num_attention_heads=2, num_hidden_layers=3, multiple_of=2,
+         rotary_dim=0.5),                                                        # head_dim 32, 16 rotated
+    dict(vocab_size=512, max_sequence_length=96, hidden_size=320, num_attention_heads=4, num_hidden_layers=3),  # 80 / 32
+])
+def test_model_prefill_and_cached_steps_against_the_oracle(cuda, kw):
+    ref, model = _pair(cuda, **kw)
+    c = ref.cfg
+    g = torch.Generator().manual_seed(0)
+    B, S0 = 2, 7
+    ids = torch.randint(0, c.vocab_size, (B, S0 + 3), generator=g)
+    rc, cache = ref.build_kv_cache(B), model.build_kv_cache(B)
+    _close(model(ids[:, :S0].to(cuda), cache, 0), ref(ids[:, :S0], rc, 0))
+    for t in range(S0, S0 + 3):
+        _close(model(ids[:, t:t + 1].to(cuda), cache, t), ref(ids[:, t:t + 1], rc, t))
+    assert cache[0].length == S0 + 3
+    # the cache holds what the oracle's holds: the un-rotated key projection
+    _close(cache[-1].key[:B, :S0 + 3], rc[-1].key[:B, :S0 + 3])
+    # no cache: the plain causal forward
+    _close(model(ids.to(cuda)), ref(ids))
+    # last_only computes just the last row
+    c2 = model.build_kv_cache(B)
+    full = model(ids[:, :S0].to(cuda), c2, 0)
+    c3 = model.build_kv_cache(B)
+    last = model(ids[:, :S0].to(cuda), c3, 0, last_only=True)
+    assert torch.equal(last[:, 0], full[:, -1])
+
+
+def test_cached_decode_matches_full_forward_on_the_gpu(cuda):
+    """The reference's own Phi test (tests/test_models.py:133-149) run on the HIP path; bf16
+    tolerances instead of its fp32 1e-4."""
+    _, model = _pair(cuda, vocab_size=128, max_sequence_length=32, hidden_size=128, num_attention_heads=4)
+    ids = torch.randint(0, 128, (1, 9), generator=torch.Generator().manual_seed(1)).to(cuda)
+    full = model(ids)
+    cache = model.build_kv_cache()
+    prefill = model(ids[:, :4], cache, 0)
+    step = model(ids[:, 4:5], cache, 4)
+    _close(prefill[:, -1], full[:, 3].cpu(), 2e-2, 2e-3)
+    _close(step[:, -1], full[:, 4].cpu(), 2e-2, 2e-3)
+
+
+def test_graph_replayed_decode_reads_the_position_on_the_device(cuda):
+    from ohara_amd import ops
+
+    ref, model = _pair(cuda, vocab_size=128, max_sequence_length=32, hidden_size=128, num_attention_heads=4)
+    ids = torch.randint(0, 128, (2, 6), generator=torch.Generator().manual_seed(2))
+    rc, cache = ref.build_kv_cache(2), model.build_kv_cache(2)
+    want = ref(ids, rc, 0)
+    model(ids.to(cuda), cache, 0)
+    tok = want[:, -1].float().argmax(-1).view(2, 1)
+    pos_dev = torch.tensor([6], dtype=torch.int32, device=cuda)
+    for t in range(6, 10):  # eager launches, position from the device scalar
+        got = model(tok.to(cuda), cache, t, pos_dev=pos_dev)
+        want = ref(tok, rc, t)
+        _close(got, want)
+        ops.advance_positions(pos_dev)
+        tok = want[:, -1].float().argmax(-1).view(2, 1)
+    assert int(pos_dev.item()) == 10
+
+
+def test_error_surface(cuda):
+    _, model = _pair(cuda)
+    ids = torch.zeros(1, 1, dtype=torch.int64, device=cuda)
+    cache = model.build_kv_cache()
+    with pytest.raises(ValueError, match="position_ids is required"):
+        model(ids, cache, None)
+    with pytest.raises(ValueError, match="one entry per model layer"):
+        model(ids, cache[:1], 0)
+    with pytest.raises(ValueError, match="at least 1"):
+        model.build_kv_cache(0)
+    with pytest.raises(ValueError, match="sequential"):
+        model(ids, cache, 3)
+    model(ids, cache, 0)
+    with pytest.raises(ValueError, match="exceeds max_sequence_length"):
+        model(torch.zeros(1, 16, dtype=torch.int64, device=cuda), cache, 1)
