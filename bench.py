@@ -398,6 +398,53 @@ def bench_moe(dev):
             "bound": "hbm (about 8 rows per expert: ~8 flop/byte)"}
 
 
+def bench_phi(dev):
+    """Phi-2 shape (32 layers, d 2560, 32 x 80 heads, 32 rotated features, MLP 10240, vocab 51200,
+    random bf16 weights): greedy decode at batch 1 and 8 after a 1024-token context, one graph replay
+    per step (7 launches per layer)."""
+    from ohara_amd.phi import Phi, PhiConfig
+
+    cfg = PhiConfig()
+    g = torch.Generator(device=dev).manual_seed(4)
+    d, f, v = cfg.hidden_size, cfg.multiple_of * cfg.hidden_size, cfg.vocab_size
+
+    def n(*shape):
+        return (torch.randn(*shape, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+
+    st = {"wte.weight": n(v, d), "lm_head.weight": n(v, d), "lm_head.bias": n(v), "ln.weight": torch.ones(d, device=dev),
+          "ln.bias": n(d)}
+    for i in range(cfg.num_hidden_layers):
+        p = f"layers.{i}."
+        st[p + "ln.weight"], st[p + "ln.bias"] = torch.ones(d, device=dev), n(d)
+        for nm in ("q_proj", "k_proj", "v_proj", "dense"):
+            st[p + f"mixer.{nm}.weight"], st[p + f"mixer.{nm}.bias"] = n(d, d), n(d)
+        st[p + "mlp.fc1.weight"], st[p + "mlp.fc1.bias"] = n(f, d), n(f)
+        st[p + "mlp.fc2.weight"], st[p + "mlp.fc2.bias"] = n(d, f), n(d)
+    model = Phi(cfg, st, device=dev)
+    del st
+    torch.cuda.empty_cache()
+    nl, ctx, steps = cfg.num_hidden_layers, 1024, 64
+    weight_b = 2.0 * (nl * (4 * d * d + 2 * d * f) + v * d)
+    out = []
+    for B in (1, 8):
+        prompt = torch.randint(0, v, (B, ctx), device=dev)
+        model.generate_greedy(prompt[:, :16], 8)  # warm up kernels and buffers
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        model.generate_greedy(prompt, 1)
+        torch.cuda.synchronize()
+        t_prefill = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        model.generate_greedy(prompt, steps + 1)
+        torch.cuda.synchronize()
+        t = (time.perf_counter() - t0 - t_prefill) / steps  # decode steps only (graph capture included)
+        by = weight_b + 2.0 * 2 * d * nl * B * (ctx + steps / 2)
+        out.append({"batch": B, "context": ctx, "ms_per_step": round(t * 1e3, 4), "tokens_per_s": round(B / t, 1),
+                    "prefill_ms": round(t_prefill * 1e3, 1), "step_bytes": int(by), "GBs": round(by / t / 1e9, 1),
+                    "frac_of_hbm_peak": round(by / t / 1e9 / HBM_PEAK_GBS, 4)})
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -503,6 +550,7 @@ def main():
         out["kernels"]["decode_attention_gqa_32q_8kv_128"] = bench_attention_microbench(dev)
         out["kernels"]["bitnet_decode"] = bench_bitnet(dev)
         out["kernels"]["moe_decode"] = bench_moe(dev)
+        out["kernels"]["phi2_decode"] = bench_phi(dev)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

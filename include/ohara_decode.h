@@ -429,10 +429,13 @@ int ohara_kv_append_bf16(const uint16_t* k, const uint16_t* v, int ld, int batch
  * position pos (+ s), the cached UN-rotated keys from 0; key t is visible to query s when
  * t <= pos + s; softmax(q k^T / sqrt(dh)) v rounded once to bf16.  cos / sin: (t_max, rot/2) fp32
  * tables of rotary.py:166-184.  q: rows (b, s) with leading dimension ldq; out (batch*seq_len, h*dh).
- * dh % 8 == 0, dh <= 128. */
+ * dh % 8 == 0, dh <= 128.  n_split > 1 (seq_len 1 only, at most 64) spreads the context of every
+ * (sequence, head) over that many workgroups whose partial results meet in `workspace`
+ * (ohara_phi_attn_workspace_bytes) and are merged in chunk order. */
+int64_t ohara_phi_attn_workspace_bytes(int batch, int h, int dh, int n_split);
 int ohara_phi_attn_bf16(const uint16_t* q, int ldq, const uint16_t* kcache, const uint16_t* vcache, const float* cos,
                         const float* sin, int rot, int batch, int seq_len, int h, int dh, int t_max, int pos,
-                        const int32_t* pos_dev, uint16_t* out, void* stream);
+                        const int32_t* pos_dev, int n_split, void* workspace, uint16_t* out, void* stream);
 
 /* ---- timing helpers (measurement only; no counterpart in the reference) -----------
  * Thin wrappers over hipEventCreate / hipEventDestroy / hipEventElapsedTime so that a

@@ -87,7 +87,8 @@ _PROTOS = {
     "ohara_linear_bias_bf16": (_i, [_p, _i, _p, _i, _i, _p, _i, _i, _p, _i, _p, _i, _p, _i, _p]),
     "ohara_layernorm_bf16": (_i, [_p, _i, _p, _p, _p, _i, _i, _i, _f, _p]),
     "ohara_kv_append_bf16": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _p, _p, _p, _i, _p]),
-    "ohara_phi_attn_bf16": (_i, [_p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p]),
+    "ohara_phi_attn_workspace_bytes": (_i64, [_i, _i, _i, _i]),
+    "ohara_phi_attn_bf16": (_i, [_p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
     "ohara_persistent_workspace_bytes": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),
     "ohara_persistent_barrier_offset": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),
     "ohara_persistent_error_offset": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),

@@ -43,8 +43,11 @@ __device__ __forceinline__ uint4 norm8(uint4 xv, uint4 wv, float rinv) {
   return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
-template <int BT, bool NORM, int EPI>
-__global__ __launch_bounds__(256) void skinny_kernel(GemmArgs a) {
+// NW waves per workgroup split K.  A workgroup keeps NW * CH KiB of weight loads in flight, so when
+// there are too few strips to put several workgroups on every CU (few output rows, long K) 16 waves
+// instead of 4 are what fills the memory pipeline.
+template <int BT, bool NORM, int EPI, int NW = 4>
+__global__ __launch_bounds__(NW * 64) void skinny_kernel(GemmArgs a) {
   constexpr int CH = BT <= 2 ? 6 : 4;  // k-steps whose loads are issued back to back
   // workgroup id -> (strip, chunk of 16*BT rows).  Ids go round-robin over the 8 XCDs; the chunks of
   // one strip get ids 8 apart, so they run on the same XCD and share its L2 copy of the weights.
@@ -55,12 +58,12 @@ __global__ __launch_bounds__(256) void skinny_kernel(GemmArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 15, g = lane >> 4;
   const int KS = (a.K + 31) >> 5;
-  const int per_wave = (KS + 3) >> 2;
+  const int per_wave = (KS + NW - 1) / NW;
   const int j0 = wave * per_wave;
   const int j1 = min(KS, j0 + per_wave);
 
-  __shared__ float red[3][BT][64][4];
-  __shared__ float ssq[4][BT * 16];
+  __shared__ float red[NW - 1][BT][64][4];
+  __shared__ float ssq[NW][BT * 16];
 
   float rinv[BT];
   if (NORM) {
@@ -85,7 +88,9 @@ __global__ __launch_bounds__(256) void skinny_kernel(GemmArgs a) {
     __syncthreads();
 #pragma unroll
     for (int t = 0; t < BT; ++t) {
-      const float tot = ((ssq[0][16 * t + m] + ssq[1][16 * t + m]) + ssq[2][16 * t + m]) + ssq[3][16 * t + m];
+      float tot = ssq[0][16 * t + m];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) tot += ssq[w][16 * t + m];
       rinv[t] = 1.0f / sqrtf(tot / (float)a.K + a.eps);
     }
   }
@@ -128,7 +133,7 @@ __global__ __launch_bounds__(256) void skinny_kernel(GemmArgs a) {
   for (; j + CH <= j1; j += CH) group(j, CH);
   if (j < j1) group(j, j1 - j);
 
-  // Fixed-order cross-wave sum: ((w0 + w1) + w2) + w3.
+  // Fixed-order cross-wave sum: ((w0 + w1) + w2) + w3 ...
   if (wave > 0) {
 #pragma unroll
     for (int t = 0; t < BT; ++t)
@@ -140,7 +145,10 @@ __global__ __launch_bounds__(256) void skinny_kernel(GemmArgs a) {
 #pragma unroll
   for (int t = 0; t < BT; ++t)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) acc[t][i] = ((acc[t][i] + red[0][t][lane][i]) + red[1][t][lane][i]) + red[2][t][lane][i];
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int w = 0; w < NW - 1; ++w) acc[t][i] += red[w][t][lane][i];
+    }
 
 #pragma unroll
   for (int t = 0; t < BT; ++t) {
@@ -305,6 +313,17 @@ int launch_wide(const GemmArgs& a0, int epi, int strips, hipStream_t st) {
 template <int BT, bool NORM>
 int launch_epi(const GemmArgs& a, int epi, int strips, hipStream_t st) {
   dim3 grid((unsigned)((strips + 7) / 8 * 8 * a.ny)), block(256);
+  // Linear-with-bias calls with a long K (2048 and up): 16 waves per workgroup
+  if (!NORM && epi >= EPI_BIAS && a.K >= 2048) {
+    dim3 big(1024);
+    switch (epi) {
+      case EPI_BIAS: hipLaunchKernelGGL((skinny_kernel<BT, false, EPI_BIAS, 16>), grid, big, 0, st, a); break;
+      case EPI_BIAS_GELU: hipLaunchKernelGGL((skinny_kernel<BT, false, EPI_BIAS_GELU, 16>), grid, big, 0, st, a); break;
+      case EPI_BIAS_ADD2: hipLaunchKernelGGL((skinny_kernel<BT, false, EPI_BIAS_ADD2, 16>), grid, big, 0, st, a); break;
+      default: return OHARA_EINVAL;
+    }
+    return ohara_launch_status();
+  }
   switch (epi) {
     case EPI_STORE: hipLaunchKernelGGL((skinny_kernel<BT, NORM, EPI_STORE>), grid, block, 0, st, a); break;
     case EPI_RESIDUAL: hipLaunchKernelGGL((skinny_kernel<BT, NORM, EPI_RESIDUAL>), grid, block, 0, st, a); break;

@@ -70,9 +70,12 @@ __global__ void kv_append_kernel(const bf16_t* k, const bf16_t* v, int ld, int r
 }
 
 // ---- attention ---------------------------------------------------------------------------
-// One workgroup per (sequence, head, new token).  Sixteen lanes own one cached position at a time
-// (lane l the eight features 8l .. 8l+7), so a workgroup walks 16 positions per round with an online
-// softmax per 16-lane group; the groups are merged through LDS at the end.
+// One workgroup per (sequence, head, new token) and context chunk.  Sixteen lanes own one cached
+// position at a time (lane l the eight features 8l .. 8l+7) and fetch two positions per round before
+// using either, so a workgroup walks 32 positions per round with an online softmax per 16-lane group;
+// the groups are merged through LDS at the end.  With several chunks (decode: few queries, long
+// context) every chunk leaves {weighted sum, max, sum} and phi_attn_merge_kernel combines them in
+// chunk order.
 //
 // The reference rotates every cached key again at each step (phi.py:104).  With the rotated query
 // qr and c, s the cosine / sine of key position t the score is
@@ -90,6 +93,8 @@ struct PhiAttnArgs {
   bf16_t* out;       // (rows, H*D)
   int S, H, D, rot, t_max, pos;
   const int32_t* pos_dev;
+  int ns;      // context chunks (decode): chunk c of a (sequence, head) is blockIdx.y
+  float* ws;   // ns > 1: per (row, head, chunk) D + 2 floats {weighted sum[D], max, sum}
 };
 
 __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
@@ -149,44 +154,54 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
   const size_t hd = (size_t)a.H * D;
   const bf16_t* kb = a.kc + (size_t)seq * a.t_max * hd + (size_t)h * D + e0;
   const bf16_t* vb = a.vc + (size_t)seq * a.t_max * hd + (size_t)h * D + e0;
-  for (int t = grp; t <= pq; t += 16) {
-    float part = 0.f;
-    uint4 vv = make_uint4(0, 0, 0, 0);
-    if (own) {
-      const uint4 kv = ldg16(kb + (size_t)t * hd);
-      vv = ldg16(vb + (size_t)t * hd);
-      const uint32_t ku[4] = {kv.x, kv.y, kv.z, kv.w};
-      float kf[8];
+  // this workgroup's positions [t_lo, t_hi]
+  int t_lo = 0, t_hi = pq;
+  if (a.ns > 1) {
+    const int per = ((pq + a.ns) / a.ns + 15) & ~15;  // ceil((pq + 1) / ns) rounded up to whole rounds
+    t_lo = (int)blockIdx.y * per;
+    t_hi = min(pq, t_lo + per - 1);
+  }
+  for (int t = t_lo + grp; t <= t_hi; t += 32) {
+    const bool two = t + 16 <= t_hi;
+    uint4 kv[2], vv[2];
+    float cs[2][8], sn[2][8];
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const int tt = t + 16 * r;
+      const bool in = own && (r == 0 || two);
+      kv[r] = in ? ldg16(kb + (size_t)tt * hd) : make_uint4(0, 0, 0, 0);
+      vv[r] = in ? ldg16(vb + (size_t)tt * hd) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const bool rot_u = in && rotates && f[u] >= 0;
+        cs[r][u] = rot_u ? a.cos[(size_t)tt * half + f[u]] : 1.0f;
+        sn[r][u] = rot_u ? a.sin[(size_t)tt * half + f[u]] : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      if (r == 1 && !two) break;  // uniform within the 16-lane group
+      const uint32_t ku[4] = {kv[r].x, kv[r].y, kv[r].z, kv[r].w};
+      float part = 0.f;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        kf[2 * i] = lo_bf(ku[i]);
-        kf[2 * i + 1] = hi_bf(ku[i]);
+        part += lo_bf(ku[i]) * (cs[r][2 * i] * A[2 * i] + sn[r][2 * i] * Bc[2 * i]);
+        part += hi_bf(ku[i]) * (cs[r][2 * i + 1] * A[2 * i + 1] + sn[r][2 * i + 1] * Bc[2 * i + 1]);
       }
-      if (rotates) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          float wgt = A[u];
-          if (f[u] >= 0) wgt = a.cos[(size_t)t * half + f[u]] * A[u] + a.sin[(size_t)t * half + f[u]] * Bc[u];
-          part += kf[u] * wgt;
-        }
-      } else {
+      for (int o = 1; o < 16; o <<= 1) part += __shfl_xor(part, o, WAVE);
+      const float sc = part * scale;
+      const float mn = fmaxf(m, sc);
+      const float corr = expf(m - mn), p = expf(sc - mn);  // m = -inf on the first round: corr = 0
+      lsum = lsum * corr + p;
+      const uint32_t vu[4] = {vv[r].x, vv[r].y, vv[r].z, vv[r].w};
 #pragma unroll
-        for (int u = 0; u < 8; ++u) part += kf[u] * A[u];
+      for (int i = 0; i < 4; ++i) {
+        acc[2 * i] = acc[2 * i] * corr + p * lo_bf(vu[i]);
+        acc[2 * i + 1] = acc[2 * i + 1] * corr + p * hi_bf(vu[i]);
       }
+      m = mn;
     }
-#pragma unroll
-    for (int o = 1; o < 16; o <<= 1) part += __shfl_xor(part, o, WAVE);
-    const float sc = part * scale;
-    const float mn = fmaxf(m, sc);
-    const float corr = expf(m - mn), p = expf(sc - mn);  // m = -inf on the first round: corr = 0
-    lsum = lsum * corr + p;
-    const uint32_t vu[4] = {vv.x, vv.y, vv.z, vv.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      acc[2 * i] = acc[2 * i] * corr + p * lo_bf(vu[i]);
-      acc[2 * i + 1] = acc[2 * i + 1] * corr + p * hi_bf(vu[i]);
-    }
-    m = mn;
   }
   if (l == 0) {
     gm[grp] = m;
@@ -209,8 +224,35 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
       num += wg * gacc[g][tid];
       den += wg * gl[g];
     }
-    a.out[(size_t)row * hd + (size_t)h * D + tid] = f2bf(num / den);
+    if (a.ns > 1) {
+      float* o = a.ws + (((size_t)row * a.H + h) * a.ns + blockIdx.y) * (D + 2);
+      o[tid] = num;
+      if (tid == 0) {
+        o[D] = M;  // -inf: this chunk lies beyond the query's position
+        o[D + 1] = den;
+      }
+    } else {
+      a.out[(size_t)row * hd + (size_t)h * D + tid] = f2bf(num / den);
+    }
   }
+}
+
+// chunks of one (row, head) -> out, in chunk order
+__global__ void phi_attn_merge_kernel(const float* ws, bf16_t* out, int H, int D, int ns) {
+  const int rh = blockIdx.x, tid = threadIdx.x;
+  if (tid >= D) return;
+  const float* p = ws + (size_t)rh * ns * (D + 2);
+  float M = -INFINITY;
+  for (int c = 0; c < ns; ++c) M = fmaxf(M, p[(size_t)c * (D + 2) + D]);
+  float num = 0.f, den = 0.f;
+  for (int c = 0; c < ns; ++c) {
+    const float mc = p[(size_t)c * (D + 2) + D];
+    if (mc == -INFINITY) continue;
+    const float wg = expf(mc - M);
+    num += wg * p[(size_t)c * (D + 2) + tid];
+    den += wg * p[(size_t)c * (D + 2) + D + 1];
+  }
+  out[(size_t)rh * D + tid] = f2bf(num / den);
 }
 
 }  // namespace
@@ -240,9 +282,14 @@ int ohara_kv_append_bf16(const uint16_t* k, const uint16_t* v, int ld, int batch
   return ohara_launch_status();
 }
 
+int64_t ohara_phi_attn_workspace_bytes(int batch, int h, int dh, int n_split) {
+  if (batch < 1 || h < 1 || dh < 1 || n_split < 1) return OHARA_EINVAL;
+  return (int64_t)batch * h * n_split * (dh + 2) * (int64_t)sizeof(float);
+}
+
 int ohara_phi_attn_bf16(const uint16_t* q, int ldq, const uint16_t* kcache, const uint16_t* vcache, const float* cos,
                         const float* sin, int rot, int batch, int seq_len, int h, int dh, int t_max, int pos,
-                        const int32_t* pos_dev, uint16_t* out, void* stream) {
+                        const int32_t* pos_dev, int n_split, void* workspace, uint16_t* out, void* stream) {
   if (!q || !kcache || !vcache || !cos || !sin || !out) return OHARA_EINVAL;
   if (batch < 1 || seq_len < 1 || h < 1 || t_max < 1) return OHARA_EINVAL;
   if (dh < 8 || dh > 128 || (dh & 7)) return OHARA_ESIZE;
@@ -250,10 +297,15 @@ int ohara_phi_attn_bf16(const uint16_t* q, int ldq, const uint16_t* kcache, cons
   if (ldq < h * dh) return OHARA_EINVAL;
   if (!pos_dev && (pos < 0 || pos + seq_len > t_max)) return OHARA_EINVAL;
   if (pos_dev && seq_len != 1) return OHARA_EINVAL;
+  if (n_split < 1 || n_split > 64 || (n_split > 1 && (!workspace || seq_len != 1))) return OHARA_EINVAL;
   const int64_t grid = (int64_t)batch * seq_len * h;
   if (grid > INT32_MAX) return OHARA_ESIZE;
-  PhiAttnArgs a{q, ldq, kcache, vcache, cos, sin, out, seq_len, h, dh, rot, t_max, pos, pos_dev};
-  hipLaunchKernelGGL(phi_attn_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, a);
+  PhiAttnArgs a{q, ldq, kcache, vcache, cos, sin, out, seq_len, h, dh, rot, t_max, pos, pos_dev, n_split,
+                reinterpret_cast<float*>(workspace)};
+  hipLaunchKernelGGL(phi_attn_kernel, dim3((unsigned)grid, (unsigned)n_split), dim3(256), 0, (hipStream_t)stream, a);
+  if (n_split > 1)
+    hipLaunchKernelGGL(phi_attn_merge_kernel, dim3((unsigned)grid), dim3(128), 0, (hipStream_t)stream, a.ws, out, h, dh,
+                       n_split);
   return ohara_launch_status();
 }
 

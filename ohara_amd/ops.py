@@ -502,9 +502,18 @@ def kv_append(k, v, kcache, vcache, batch, seq_len, h, dh, pos, pos_dev=None) ->
                                      _ptr(vcache), kcache.shape[1], _stream()), "kv_append")
 
 
-def phi_attn(q, kcache, vcache, cos, sin, rot, batch, seq_len, h, dh, pos, pos_dev=None, out=None) -> torch.Tensor:
+def phi_attn_workspace(batch, h, dh, n_split, device) -> torch.Tensor:
+    nbytes = lib().ohara_phi_attn_workspace_bytes(batch, h, dh, n_split)
+    if nbytes < 0:
+        raise ValueError("phi_attn_workspace: invalid sizes")
+    return torch.empty(nbytes // 4, dtype=torch.float32, device=device)
+
+
+def phi_attn(q, kcache, vcache, cos, sin, rot, batch, seq_len, h, dh, pos, pos_dev=None, out=None, n_split=1,
+             workspace=None) -> torch.Tensor:
     """PhiMHA's attention core over the cache (phi.py:98-117); q: (rows, h*dh) view with any row
-    stride; cos / sin: fp32 (t_max, rot/2)."""
+    stride; cos / sin: fp32 (t_max, rot/2).  ``n_split`` > 1 (single-token calls) spreads the context
+    over that many workgroups per (sequence, head); ``workspace`` from ``phi_attn_workspace``."""
     if q.stride(1) != 1:
         raise ValueError("q must have unit column stride")
     if cos.dtype != torch.float32 or sin.dtype != torch.float32:
@@ -512,5 +521,6 @@ def phi_attn(q, kcache, vcache, cos, sin, rot, batch, seq_len, h, dh, pos, pos_d
     if out is None:
         out = torch.empty(batch * seq_len, h * dh, dtype=BF16, device=q.device)
     check(lib().ohara_phi_attn_bf16(_ptr(q), q.stride(0), _ptr(kcache), _ptr(vcache), _ptr(cos), _ptr(sin), rot, batch,
-                                    seq_len, h, dh, kcache.shape[1], pos, _ptr(pos_dev), _ptr(out), _stream()), "phi_attn")
+                                    seq_len, h, dh, kcache.shape[1], pos, _ptr(pos_dev), n_split, _ptr(workspace), _ptr(out),
+                                    _stream()), "phi_attn")
     return out

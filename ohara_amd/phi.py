@@ -119,6 +119,9 @@ class Phi:
             d = self.config.hidden_size
             new = lambda n: torch.empty(rows, n, dtype=BF16, device=self.device)
             b = dict(x=[new(d), new(d)], h=new(d), qkv=new(3 * d), attn=new(d), mixer=new(d), act=new(self.ff))
+            # single-token calls: the context of a (sequence, head) is spread over up to 16 workgroups
+            b["ns"] = max(1, min(16, self.config.max_sequence_length // 64))
+            b["ws"] = ops.phi_attn_workspace(rows, self.config.num_attention_heads, self.head_dim, b["ns"], self.device)
             self._bufs[rows] = b
         return b
 
@@ -144,26 +147,71 @@ class Phi:
                 raise ValueError("position_ids is required when using a KV cache")  # phi.py:92-93
             start = int(position_ids)
         ends = [cache._reserve(B, S, start) for cache in kv_cache]
+        logits = self._run(x.reshape(-1).to(device=self.device, dtype=torch.int64), B, S, kv_cache, start, pos_dev, last_only)
+        for cache, end in zip(kv_cache, ends):
+            cache._commit(B, end)
+        return logits.view(B, 1 if last_only else S, c.vocab_size)
+
+    def _run(self, ids, B, S, kv_cache, start, pos_dev, last_only):
+        """The launches of one forward call; no host-side state, so it can be captured in a graph."""
+        c = self.config
         rows, d, H, D = B * S, c.hidden_size, c.num_attention_heads, self.head_dim
         buf = self._buffers(rows)
         cur, nxt = buf["x"]
-        ops.embed(x.reshape(-1).to(device=self.device, dtype=torch.int64), self.wte, out=cur)
+        ops.embed(ids, self.wte, out=cur)
         for L, cache in zip(self.layers, kv_cache):
             h, qkv = buf["h"], buf["qkv"]
             ops.layernorm(cur, L["ln_w"], L["ln_b"], c.eps, out=h)
             ops.linear_bias(h, L["wqkv"], L["bqkv"], out=qkv)
             ops.kv_append(qkv[:, d:2 * d], qkv[:, 2 * d:], cache.key, cache.value, B, S, H, D, start, pos_dev)
             ops.phi_attn(qkv[:, :d], cache.key, cache.value, self.cos, self.sin, self.rot, B, S, H, D, start, pos_dev,
-                         out=buf["attn"])
+                         out=buf["attn"], n_split=buf["ns"] if S == 1 else 1, workspace=buf["ws"])
             ops.linear_bias(buf["attn"], L["dense"], L["dense_b"], out=buf["mixer"])
             ops.linear_bias(h, L["fc1"], L["fc1_b"], "gelu", out=buf["act"])
             ops.linear_bias(buf["act"], L["fc2"], L["fc2_b"], "add2", add1=buf["mixer"], add2=cur, out=nxt)
             cur, nxt = nxt, cur
-        src = cur.view(B, S, d)[:, -1] if last_only else cur
-        hn = ops.layernorm(src.contiguous() if last_only else src, self.ln_w, self.ln_b, c.eps)
-        logits = ops.linear_bias(hn, self.lm_head, self.lm_bias)
-        for cache, end in zip(kv_cache, ends):
-            cache._commit(B, end)
-        return logits.view(B, 1 if last_only else S, c.vocab_size)
+        src = cur.view(B, S, d)[:, -1].contiguous() if (last_only and S > 1) else cur
+        hn = ops.layernorm(src, self.ln_w, self.ln_b, c.eps)
+        return ops.linear_bias(hn, self.lm_head, self.lm_bias)
 
     __call__ = forward
+
+    @torch.no_grad()
+    def generate_greedy(self, prompt_ids: torch.Tensor, steps: int, *, use_graph: bool = True) -> torch.Tensor:
+        """Prefill the prompt, then ``steps`` greedy tokens with no host round trip per token: the
+        cache position lives on the device and one decode step (all launches of ``_run`` plus the
+        arg-max that feeds the next step) is captured once and replayed.  Returns (B, steps) ids."""
+        B, P = prompt_ids.shape
+        c = self.config
+        if steps < 1:
+            return torch.zeros(B, 0, dtype=torch.int64, device=self.device)
+        if P + steps - 1 > c.max_sequence_length:
+            raise ValueError("input exceeds max_sequence_length")
+        cache = self.build_kv_cache(B)
+        logits = self.forward(prompt_ids, cache, 0, last_only=True).view(B, c.vocab_size)
+        ids = ops.argmax(logits)
+        history = torch.zeros(steps, B, dtype=torch.int64, device=self.device)
+        history[0].copy_(ids)
+        state = torch.tensor([P, 1, 0, 0], dtype=torch.int32, device=self.device)  # {pos, step, done, pad}
+
+        def step():
+            lg = self._run(ids, B, 1, cache, 0, state, False)
+            ops.argmax(lg, next_ids=ids, history=history, step_state=state)  # also advances pos and step
+
+        todo = steps - 1
+        if use_graph and todo > 2:
+            step()  # warm up outside the capture (allocations, lazy module loading)
+            todo -= 1
+            torch.cuda.synchronize(self.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step()
+            # the captured step is recorded, not run
+            for _ in range(todo):
+                graph.replay()
+        else:
+            for _ in range(todo):
+                step()
+        for cc in cache:
+            cc._commit(B, P + steps - 1)
+        return history.t().contiguous()

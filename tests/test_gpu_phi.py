@@ -40,7 +40,7 @@ def test_linear_bias_epilogues(cuda):
     from ohara_amd import ops
 
     g = torch.Generator().manual_seed(1)
-    for rows, n, k in ((1, 64, 64), (7, 320, 1280), (64, 1280, 320), (70, 96, 64)):
+    for rows, n, k in ((1, 64, 64), (7, 320, 1280), (64, 1280, 320), (70, 96, 64), (3, 64, 2560), (20, 160, 10240)):
         x = torch.randn(rows, k, generator=g).to(BF)
         w = (torch.randn(n, k, generator=g) / k ** 0.5).to(BF)
         b = (0.2 * torch.randn(n, generator=g)).to(BF)
@@ -94,10 +94,15 @@ def test_kv_append_and_attention_against_the_oracle(cuda):
         got = ops.phi_attn(qkvd[:, :hd], kcd, vcd, cos.to(cuda), sin.to(cuda), rot, B, S, H, D, L0)
         want = P.attention(qkv[:, :hd].view(B, S, H, D), kc[:, :L0 + S], vc[:, :L0 + S], L0, rot, torch.float32)
         _ulp_close(got.view(B, S, H, D), want, ulps=0.6, floor=2.0 ** -6)
-        if S == 1:  # position read on the device
+        if S == 1:  # position read on the device; context spread over several workgroups
             pd = torch.tensor([L0], dtype=torch.int32, device=cuda)
             got2 = ops.phi_attn(qkvd[:, :hd], kcd, vcd, cos.to(cuda), sin.to(cuda), rot, B, S, H, D, 0, pos_dev=pd)
             assert torch.equal(got2, got)
+            for ns in (2, 5, 16):
+                ws = ops.phi_attn_workspace(B, H, D, ns, cuda)
+                got3 = ops.phi_attn(qkvd[:, :hd], kcd, vcd, cos.to(cuda), sin.to(cuda), rot, B, S, H, D, L0, n_split=ns,
+                                    workspace=ws)
+                _ulp_close(got3.view(B, S, H, D), want, ulps=0.6, floor=2.0 ** -6)
 
 
 def _pair(cuda, dtype=BF, seed=5, **kw):
@@ -195,3 +200,25 @@ def test_error_surface(cuda):
     model(ids, cache, 0)
     with pytest.raises(ValueError, match="exceeds max_sequence_length"):
         model(torch.zeros(1, 16, dtype=torch.int64, device=cuda), cache, 1)
+
+
+@pytest.mark.parametrize("use_graph", [True, False])
+def test_greedy_generation_matches_the_oracle_teacher_forced(cuda, use_graph):
+    """Every generated token is the oracle's arg-max for the same history (or a near-tie of its own
+    logits); the oracle is teacher-forced on the tokens produced."""
+    ref, model = _pair(cuda, vocab_size=256, max_sequence_length=48, hidden_size=128, num_attention_heads=4,
+                       num_hidden_layers=2)
+    prompt = torch.randint(0, 256, (2, 9), generator=torch.Generator().manual_seed(3))
+    steps = 12
+    toks = model.generate_greedy(prompt.to(cuda), steps, use_graph=use_graph).cpu()
+    assert toks.shape == (2, steps)
+    rc = ref.build_kv_cache(2)
+    logits = ref(prompt, rc, 0)[:, -1]
+    for t in range(steps):
+        for b in range(2):
+            best, tok = int(logits[b].float().argmax()), int(toks[b, t])
+            if tok != best:
+                la, lb = logits[b, tok].float().item(), logits[b, best].float().item()
+                assert abs(la - lb) <= 2.0 ** -6 * max(abs(la), abs(lb)), (t, b, tok, best)
+        if t + 1 < steps:
+            logits = ref(toks[:, t:t + 1], rc, 9 + t)[:, -1]
