@@ -398,10 +398,9 @@ def bench_moe(dev):
             "bound": "hbm (about 8 rows per expert: ~8 flop/byte)"}
 
 
-def bench_phi(dev):
-    """Phi-2 shape (32 layers, d 2560, 32 x 80 heads, 32 rotated features, MLP 10240, vocab 51200,
-    random bf16 weights): greedy decode at batch 1 and 8 after a 1024-token context, one graph replay
-    per step (7 launches per layer)."""
+def phi2_model(dev):
+    """Phi-2 shape (32 layers, d 2560, 32 x 80 heads, 32 rotated features, MLP 10240, vocab 51200)
+    with random bf16 weights."""
     from ohara_amd.phi import Phi, PhiConfig
 
     cfg = PhiConfig()
@@ -423,6 +422,33 @@ def bench_phi(dev):
     model = Phi(cfg, st, device=dev)
     del st
     torch.cuda.empty_cache()
+    return cfg, model
+
+
+def phi_decode_only(dev, batch, steps=12, context=1024):
+    """Eager Phi-2 decode steps over a randomly filled cache and nothing else: the workload of the
+    per-kernel profiles (`--phi-decode-only B`)."""
+    from ohara_amd import ops
+
+    cfg, model = phi2_model(dev)
+    cache = model.build_kv_cache(batch)
+    for c in cache:
+        c.key.normal_()
+        c.value.normal_()
+    ids = torch.randint(0, cfg.vocab_size, (batch,), device=dev)
+    state = torch.tensor([context, 0, 0, 0], dtype=torch.int32, device=dev)
+    for _ in range(steps):
+        lg = model._run(ids, batch, 1, cache, 0, state, False)
+        ops.argmax(lg, next_ids=ids, step_state=state)
+    torch.cuda.synchronize()
+    return {"batch": batch, "steps": steps, "context_end": int(state[0])}
+
+
+def bench_phi(dev):
+    """Phi-2 shape, random bf16 weights: greedy decode at batch 1 and 8 after a 1024-token context, one
+    graph replay per step (8 launches per layer)."""
+    cfg, model = phi2_model(dev)
+    d, f, v = cfg.hidden_size, cfg.multiple_of * cfg.hidden_size, cfg.vocab_size
     nl, ctx, steps = cfg.num_hidden_layers, 1024, 64
     weight_b = 2.0 * (nl * (4 * d * d + 2 * d * f) + v * d)
     out = []
@@ -459,6 +485,8 @@ def main():
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run three 1 GiB device-to-device copies (a kernel of known traffic to scale "
                          "FETCH_SIZE / WRITE_SIZE counters against)")
+    ap.add_argument("--phi-decode-only", type=int, default=0, metavar="B",
+                    help="run 12 eager Phi-2 decode steps of B sequences at context 1024 and exit (profiling workload)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE MI355X (no sharding, no collectives); --gpus must be 1",
@@ -471,6 +499,9 @@ def main():
     from ohara_amd.llama import Llama
 
     dev = torch.device("cuda:0")
+    if args.phi_decode_only:
+        print(json.dumps(phi_decode_only(dev, args.phi_decode_only)))
+        return
     if args.pmc_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)

@@ -146,6 +146,8 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
     }
   }
   const bool rotates = own && e0 < a.rot;
+  const bool vec8 = (half & 7) == 0;  // then rot % 16 == 0 and a lane's features are all rotated or all not
+  const uint4 one4 = make_uint4(0x3f800000u, 0x3f800000u, 0x3f800000u, 0x3f800000u), zero4 = make_uint4(0, 0, 0, 0);
   const float scale = sqrtf(1.0f / (float)D);
 
   float m = -INFINITY, lsum = 0.f, acc[8];
@@ -171,11 +173,27 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
       const bool in = own && (r == 0 || two);
       kv[r] = in ? ldg16(kb + (size_t)tt * hd) : make_uint4(0, 0, 0, 0);
       vv[r] = in ? ldg16(vb + (size_t)tt * hd) : make_uint4(0, 0, 0, 0);
+      if (vec8) {
+        // the lane's eight features lie in one half: their angles are eight adjacent table entries
+        const bool rl = in && rotates;
+        const float* cp = a.cos + (size_t)tt * half + f[0];
+        const float* sp = a.sin + (size_t)tt * half + f[0];
+        const uint4 c0 = rl ? ldg16(cp) : one4, c1 = rl ? ldg16(cp + 4) : one4;
+        const uint4 s0 = rl ? ldg16(sp) : zero4, s1 = rl ? ldg16(sp + 4) : zero4;
+        const uint32_t cu[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+        const uint32_t su[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const bool rot_u = in && rotates && f[u] >= 0;
-        cs[r][u] = rot_u ? a.cos[(size_t)tt * half + f[u]] : 1.0f;
-        sn[r][u] = rot_u ? a.sin[(size_t)tt * half + f[u]] : 0.0f;
+        for (int u = 0; u < 8; ++u) {
+          cs[r][u] = __uint_as_float(cu[u]);
+          sn[r][u] = __uint_as_float(su[u]);
+        }
+      } else {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const bool rot_u = in && rotates && f[u] >= 0;
+          cs[r][u] = rot_u ? a.cos[(size_t)tt * half + f[u]] : 1.0f;
+          sn[r][u] = rot_u ? a.sin[(size_t)tt * half + f[u]] : 0.0f;
+        }
       }
     }
 #pragma unroll

@@ -119,8 +119,10 @@ class Phi:
             d = self.config.hidden_size
             new = lambda n: torch.empty(rows, n, dtype=BF16, device=self.device)
             b = dict(x=[new(d), new(d)], h=new(d), qkv=new(3 * d), attn=new(d), mixer=new(d), act=new(self.ff))
-            # single-token calls: the context of a (sequence, head) is spread over up to 16 workgroups
-            b["ns"] = max(1, min(16, self.config.max_sequence_length // 64))
+            # single-token calls: the context of a (sequence, head) is spread over up to 16 workgroups,
+            # aiming at about 2048 workgroups of at least 64 positions
+            heads = rows * self.config.num_attention_heads
+            b["ns"] = max(1, min(16, self.config.max_sequence_length // 64, -(-2048 // heads)))
             b["ws"] = ops.phi_attn_workspace(rows, self.config.num_attention_heads, self.head_dim, b["ns"], self.device)
             self._bufs[rows] = b
         return b
