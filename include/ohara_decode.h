@@ -415,6 +415,19 @@ int64_t ohara_persistent_profile_offset(const OharaModel* m, int batch, int n_sp
 int ohara_linear_bias_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n, int k, const uint16_t* bias, int rows,
                            int epilogue, const uint16_t* add1, int ld1, const uint16_t* add2, int ld2, uint16_t* out,
                            int ldo, void* stream);
+/* The head of a Phi block in one launch (phi.py:150, :81-87, :95, :50-51): h = LayerNorm(x), then
+ * [q; k; v; fc1] = h @ W^T + bias with W the packed vertical concatenation of q_proj, k_proj, v_proj
+ * (d rows each) and mlp.fc1 (ff rows): q rows -> q (leading dimension ldq), k / v rows -> the
+ * caches at position pos + s as they are (un-rotated), fc1 rows -> new_gelu -> act.  Same rounding
+ * points as ohara_layernorm_bf16 + ohara_linear_bias_bf16 + ohara_kv_append_bf16, except that the
+ * variance comes from the sums of x and x^2.  ln_w == NULL: x already is the normalised input
+ * (measured faster at Phi-2's sizes: a separate LayerNorm launch costs less than re-deriving the
+ * statistics in each of the 1120 workgroups before their weight loads start).
+ * d % 16 == 0, ff % 4 == 0. */
+int ohara_phi_block_in_bf16(const uint16_t* x, int ldx, const uint16_t* ln_w, const uint16_t* ln_b, float eps,
+                            const uint16_t* wp, const uint16_t* bias, int d, int ff, int batch, int seq_len, int pos,
+                            const int32_t* pos_dev, uint16_t* q, int ldq, uint16_t* kcache, uint16_t* vcache, int t_max,
+                            uint16_t* act, int ldact, void* stream);
 /* nn.LayerNorm over the last dimension (phi.py:132, :160): fp32 mean and biased variance,
  * out = bf16((x - mean) * rstd * weight + bias).  d % 8 == 0. */
 int ohara_layernorm_bf16(const uint16_t* x, int ldx, const uint16_t* weight, const uint16_t* bias, uint16_t* out, int ldo,
@@ -431,7 +444,8 @@ int ohara_kv_append_bf16(const uint16_t* k, const uint16_t* v, int ld, int batch
  * tables of rotary.py:166-184.  q: rows (b, s) with leading dimension ldq; out (batch*seq_len, h*dh).
  * dh % 8 == 0, dh <= 128.  n_split > 1 (seq_len 1 only, at most 64) spreads the context of every
  * (sequence, head) over that many workgroups whose partial results meet in `workspace`
- * (ohara_phi_attn_workspace_bytes) and are merged in chunk order. */
+ * (ohara_phi_attn_workspace_bytes, zero-filled once before the first use; calls sharing it must not
+ * overlap) and are merged in chunk order by the workgroup that finishes last. */
 int64_t ohara_phi_attn_workspace_bytes(int batch, int h, int dh, int n_split);
 int ohara_phi_attn_bf16(const uint16_t* q, int ldq, const uint16_t* kcache, const uint16_t* vcache, const float* cos,
                         const float* sin, int rot, int batch, int seq_len, int h, int dh, int t_max, int pos,

@@ -85,6 +85,7 @@ _PROTOS = {
     "ohara_moe_combine": (_i, [_p, _i, _p, _p, _i, _i, _p, _i, _p, _i, _p, _i, _i, _p]),
     "ohara_llama_forward": (_i, [C.POINTER(OharaModel), C.POINTER(OharaDecodeState), _i, _i, _i, _i, _i, _p]),
     "ohara_linear_bias_bf16": (_i, [_p, _i, _p, _i, _i, _p, _i, _i, _p, _i, _p, _i, _p, _i, _p]),
+    "ohara_phi_block_in_bf16": (_i, [_p, _i, _p, _p, _f, _p, _p, _i, _i, _i, _i, _i, _p, _p, _i, _p, _p, _i, _p, _i, _p]),
     "ohara_layernorm_bf16": (_i, [_p, _i, _p, _p, _p, _i, _i, _i, _f, _p]),
     "ohara_kv_append_bf16": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _p, _p, _p, _i, _p]),
     "ohara_phi_attn_workspace_bytes": (_i64, [_i, _i, _i, _i]),

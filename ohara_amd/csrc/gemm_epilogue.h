@@ -7,7 +7,7 @@
 #pragma once
 #include "common.h"
 
-enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_ROPE = 3, EPI_BIAS = 4, EPI_BIAS_GELU = 5, EPI_BIAS_ADD2 = 6 };
+enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2, EPI_ROPE = 3, EPI_BIAS = 4, EPI_BIAS_GELU = 5, EPI_BIAS_ADD2 = 6, EPI_PHI_IN = 7 };
 
 struct GemmArgs {
   const uint4* wp;
@@ -35,6 +35,14 @@ struct GemmArgs {
   const bf16_t* bias;
   const bf16_t* resid2;
   int ldr2;
+  // LayerNorm prologue (NORM == 2): norm_w / norm_b
+  const bf16_t* norm_b;
+  // EPI_PHI_IN: packed rows [q; k; v; fc1] off one normalised input (phi.py:81-83, :50): rows below
+  // split_n are the QKV projection (q -> out, k / v rows -> cache position pos + s, un-rotated), the
+  // rest go through new_gelu into out2
+  int split_n;
+  bf16_t* out2;
+  int ldo2;
 };
 
 // gemm_tile.hip: the tiled kernel for calls with many rows (a.B rows, no fused norm).
@@ -94,6 +102,35 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, int b, int stri
       v[3] = rbf(hi_bf(r1.y) + v[3]) + hi_bf(r2.y);
     }
     *reinterpret_cast<uint2*>(a.out + (size_t)b * a.ldo + r0) = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
+  } else if (EPI == EPI_PHI_IN) {
+    if (r0 >= a.N) return;
+    const uint2 bv = *reinterpret_cast<const uint2*>(a.bias + r0);
+    float v[4] = {rbf(acc[0] + lo_bf(bv.x)), rbf(acc[1] + hi_bf(bv.x)), rbf(acc[2] + lo_bf(bv.y)),
+                  rbf(acc[3] + hi_bf(bv.y))};
+    const int grow = a.row0 + b;
+    bf16_t* o;
+    if (r0 >= a.split_n) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {  // new_gelu as in EPI_BIAS_GELU
+        const float x = v[i];
+        const float t2 = rbf(x + rbf(0.044715f * rbf(rbf(x * x) * x)));
+        const float t5 = rbf(1.0f + rbf(tanhf(rbf(0.7978845608028654f * t2))));
+        v[i] = rbf(0.5f * x) * t5;
+      }
+      o = a.out2 + (size_t)grow * a.ldo2 + (r0 - a.split_n);
+    } else {
+      const int dm = a.split_n / 3;
+      if (r0 < dm) {
+        o = a.out + (size_t)grow * a.ldo + r0;
+      } else {
+        const int seq = grow / a.S;
+        const int pos = (a.pos_dev ? *a.pos_dev : a.pos) + (grow - seq * a.S);
+        if (pos < 0 || pos >= a.Tmax) return;
+        const bool isk = r0 < 2 * dm;
+        o = (isk ? a.kcache : a.vcache) + ((size_t)seq * a.Tmax + pos) * dm + (r0 - (isk ? dm : 2 * dm));
+      }
+    }
+    *reinterpret_cast<uint2*>(o) = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
   } else if (EPI == EPI_SWIGLU) {
     // rows: gate f, gate f+1, up f, up f+1 with f = 8*strip + 2*g; N = hidden width F
     const int f = strip * 8 + 2 * g;

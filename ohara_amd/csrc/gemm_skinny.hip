@@ -43,10 +43,32 @@ __device__ __forceinline__ uint4 norm8(uint4 xv, uint4 wv, float rinv) {
   return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
+// LayerNorm on 8 packed values: bf16((x - mean) * rstd * w + b), one rounding (nn.LayerNorm).
+__device__ __forceinline__ uint4 lnorm8(uint4 xv, uint4 wv, uint4 bv, float mean, float rstd) {
+  const uint32_t xs[4] = {xv.x, xv.y, xv.z, xv.w};
+  const uint32_t ws[4] = {wv.x, wv.y, wv.z, wv.w};
+  const uint32_t bs[4] = {bv.x, bv.y, bv.z, bv.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    o[i] = pack_bf((lo_bf(xs[i]) - mean) * rstd * lo_bf(ws[i]) + lo_bf(bs[i]),
+                   (hi_bf(xs[i]) - mean) * rstd * hi_bf(ws[i]) + hi_bf(bs[i]));
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+__device__ __forceinline__ float sum8(uint4 v) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) s += lo_bf(w[i]) + hi_bf(w[i]);
+  return s;
+}
+
+// NORM: 0 none, 1 RMSNorm (norm.py:16-21), 2 LayerNorm with bias (phi.py:132).
 // NW waves per workgroup split K.  A workgroup keeps NW * CH KiB of weight loads in flight, so when
 // there are too few strips to put several workgroups on every CU (few output rows, long K) 16 waves
 // instead of 4 are what fills the memory pipeline.
-template <int BT, bool NORM, int EPI, int NW = 4>
+template <int BT, int NORM, int EPI, int NW = 4>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(GemmArgs a) {
   constexpr int CH = BT <= 2 ? 6 : 4;  // k-steps whose loads are issued back to back
   // workgroup id -> (strip, chunk of 16*BT rows).  Ids go round-robin over the 8 XCDs; the chunks of
@@ -64,18 +86,23 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(GemmArgs a) {
 
   __shared__ float red[NW - 1][BT][64][4];
   __shared__ float ssq[NW][BT * 16];
+  __shared__ float ssum[NORM == 2 ? NW : 1][BT * 16];
 
-  float rinv[BT];
+  float rinv[BT], mean[BT];
   if (NORM) {
-    float part[BT];
+    float part[BT], psum[BT];
 #pragma unroll
-    for (int t = 0; t < BT; ++t) part[t] = 0.f;
+    for (int t = 0; t < BT; ++t) part[t] = psum[t] = 0.f;
     for (int j = j0; j < j1; ++j) {
       const int k0 = 32 * j + 8 * g;
 #pragma unroll
       for (int t = 0; t < BT; ++t) {
         const int b = rbase + m + 16 * t;
-        if (b < a.B && k0 < a.K) part[t] += sumsq8(ldg16(a.x + (size_t)b * a.ldx + k0));
+        if (b < a.B && k0 < a.K) {
+          const uint4 xv = ldg16(a.x + (size_t)b * a.ldx + k0);
+          part[t] += sumsq8(xv);
+          if (NORM == 2) psum[t] += sum8(xv);
+        }
       }
     }
 #pragma unroll
@@ -84,6 +111,12 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(GemmArgs a) {
       p += __shfl_xor(p, 16, WAVE);
       p += __shfl_xor(p, 32, WAVE);
       if (g == 0) ssq[wave][16 * t + m] = p;
+      if (NORM == 2) {
+        float q = psum[t];
+        q += __shfl_xor(q, 16, WAVE);
+        q += __shfl_xor(q, 32, WAVE);
+        if (g == 0) ssum[wave][16 * t + m] = q;
+      }
     }
     __syncthreads();
 #pragma unroll
@@ -91,7 +124,17 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(GemmArgs a) {
       float tot = ssq[0][16 * t + m];
 #pragma unroll
       for (int w = 1; w < NW; ++w) tot += ssq[w][16 * t + m];
-      rinv[t] = 1.0f / sqrtf(tot / (float)a.K + a.eps);
+      if (NORM == 2) {
+        // mean and biased variance from the sums of x and x^2 (fp32; rows are O(1) activations)
+        float sm = ssum[0][16 * t + m];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) sm += ssum[w][16 * t + m];
+        mean[t] = sm / (float)a.K;
+        rinv[t] = 1.0f / sqrtf(fmaxf(tot / (float)a.K - mean[t] * mean[t], 0.f) + a.eps);
+      } else {
+        mean[t] = 0.f;
+        rinv[t] = 1.0f / sqrtf(tot / (float)a.K + a.eps);
+      }
     }
   }
 
@@ -104,13 +147,14 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(GemmArgs a) {
   // A group of CH k-steps: all loads of the group (weights, norm weights, the activations of
   // every 16-row block) are issued before the first product, so their latencies overlap.
   auto group = [&](int j, int n) {  // k-steps j .. j+n-1, n <= CH
-    uint4 wv[CH], nw[CH], xv[CH][BT];
+    uint4 wv[CH], nw[CH], nb[NORM == 2 ? CH : 1], xv[CH][BT];
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
       const int k0 = 32 * (j + c) + 8 * g;
       const bool in = c < n;
       wv[c] = in ? ldg16_nt(wrow + (size_t)(j + c) * 64) : make_uint4(0, 0, 0, 0);
       nw[c] = (NORM && in && k0 < a.K) ? ldg16(a.norm_w + k0) : make_uint4(0, 0, 0, 0);
+      if (NORM == 2) nb[c] = (in && k0 < a.K) ? ldg16(a.norm_b + k0) : make_uint4(0, 0, 0, 0);
 #pragma unroll
       for (int t = 0; t < BT; ++t) {
         const int b = rbase + m + 16 * t;
@@ -122,7 +166,12 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(GemmArgs a) {
 #pragma unroll
       for (int t = 0; t < BT; ++t) {
         uint4 xn = xv[c][t];
-        if (NORM) xn = norm8(xn, nw[c], rinv[t]);
+        if (NORM == 1) xn = norm8(xn, nw[c], rinv[t]);
+        if (NORM == 2) {
+          // rows beyond the batch and columns beyond K must stay zero (the bias would leak in)
+          const bool live = rbase + m + 16 * t < a.B && 32 * (j + c) + 8 * g < a.K && c < n;
+          xn = live ? lnorm8(xn, nw[c], nb[c], mean[t], rinv[t]) : make_uint4(0, 0, 0, 0);
+        }
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wv[c]),
                                                          __builtin_bit_cast(bf16x8, xn), acc[t], 0, 0, 0);
       }
@@ -316,6 +365,16 @@ int launch_epi(const GemmArgs& a, int epi, int strips, hipStream_t st) {
   // Linear-with-bias calls with a long K (2048 and up): 16 waves per workgroup.  (For the d12 Llama
   // projections, K 768 / 2048 with 48 - 256 strips, 16 waves measured no faster than 4.)
   if (!NORM && epi >= EPI_BIAS && a.K >= 2048) {
+    if (strips * a.ny >= 400) {  // enough workgroups for four per CU: 8 waves each measured 5-9 % faster
+      dim3 mid(512);
+      switch (epi) {
+        case EPI_BIAS: hipLaunchKernelGGL((skinny_kernel<BT, false, EPI_BIAS, 8>), grid, mid, 0, st, a); break;
+        case EPI_BIAS_GELU: hipLaunchKernelGGL((skinny_kernel<BT, false, EPI_BIAS_GELU, 8>), grid, mid, 0, st, a); break;
+        case EPI_BIAS_ADD2: hipLaunchKernelGGL((skinny_kernel<BT, false, EPI_BIAS_ADD2, 8>), grid, mid, 0, st, a); break;
+        default: return OHARA_EINVAL;
+      }
+      return ohara_launch_status();
+    }
     dim3 big(1024);
     switch (epi) {
       case EPI_BIAS: hipLaunchKernelGGL((skinny_kernel<BT, false, EPI_BIAS, 16>), grid, big, 0, st, a); break;
@@ -346,6 +405,20 @@ int launch_chunk(const GemmArgs& a0, int epi, int strips, hipStream_t st) {
   a.ny = (a.B + 15) / 16;
   a.nstrips = strips;
   if (a.ny > 4) return OHARA_ESIZE;
+  if (epi == EPI_PHI_IN) {
+    // optional LayerNorm prologue; wave count as for the Linear-with-bias calls
+    dim3 grid((unsigned)((strips + 7) / 8 * 8 * a.ny));
+#define OHARA_PHI_IN(NORM_)                                                                                              \
+  do {                                                                                                                   \
+    if (a.K < 2048) hipLaunchKernelGGL((skinny_kernel<1, NORM_, EPI_PHI_IN, 4>), grid, dim3(256), 0, st, a);             \
+    else if (strips * a.ny >= 400) hipLaunchKernelGGL((skinny_kernel<1, NORM_, EPI_PHI_IN, 8>), grid, dim3(512), 0, st, a); \
+    else hipLaunchKernelGGL((skinny_kernel<1, NORM_, EPI_PHI_IN, 16>), grid, dim3(1024), 0, st, a);                      \
+  } while (0)
+    if (a.norm_w) OHARA_PHI_IN(2);
+    else OHARA_PHI_IN(0);
+#undef OHARA_PHI_IN
+    return ohara_launch_status();
+  }
   return a.norm_w ? launch_epi<1, true>(a, epi, strips, st) : launch_epi<1, false>(a, epi, strips, st);
 }
 
@@ -358,7 +431,7 @@ int launch_skinny(const GemmArgs& a0, int epi, int packed_rows, hipStream_t st) 
     GemmArgs a = a0;
     a.B = rows - r < 64 ? rows - r : 64;
     a.x = a0.x + (size_t)r * a0.ldx;
-    if (epi == EPI_ROPE) {
+    if (epi == EPI_ROPE || epi == EPI_PHI_IN) {
       a.row0 = r;
     } else {
       a.out = a0.out + (size_t)r * a0.ldo;
@@ -445,6 +518,25 @@ int ohara_linear_bias_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n
   a.out = out; a.ldo = ldo; a.bias = bias;
   a.resid = add1; a.ldr = ld1; a.resid2 = add2; a.ldr2 = ld2;
   return launch_skinny(a, epi, (n + 15) / 16 * 16, (hipStream_t)stream);
+}
+
+int ohara_phi_block_in_bf16(const uint16_t* x, int ldx, const uint16_t* ln_w, const uint16_t* ln_b, float eps,
+                            const uint16_t* wp, const uint16_t* bias, int d, int ff, int batch, int seq_len, int pos,
+                            const int32_t* pos_dev, uint16_t* q, int ldq, uint16_t* kcache, uint16_t* vcache, int t_max,
+                            uint16_t* act, int ldact, void* stream) {
+  if (!x || !wp || !bias || !q || !kcache || !vcache || !act || (ln_w && !ln_b)) return OHARA_EINVAL;
+  if (d < 8 || ff < 4 || batch < 1 || seq_len < 1 || t_max < 1) return OHARA_EINVAL;
+  if ((d & 15) || (ff & 3) || (ldx & 7) || ldx < d || (ldq & 3) || ldq < d || (ldact & 3) || ldact < ff) return OHARA_EINVAL;
+  if (!pos_dev && (pos < 0 || pos + seq_len > t_max)) return OHARA_EINVAL;
+  if (pos_dev && seq_len != 1) return OHARA_EINVAL;
+  if ((int64_t)batch * seq_len > INT32_MAX) return OHARA_ESIZE;
+  GemmArgs a{};
+  a.wp = reinterpret_cast<const uint4*>(wp);
+  a.x = x; a.ldx = ldx; a.norm_w = ln_w; a.norm_b = ln_b; a.eps = eps;
+  a.B = batch * seq_len; a.N = 3 * d + ff; a.K = d;
+  a.out = q; a.ldo = ldq; a.out2 = act; a.ldo2 = ldact; a.split_n = 3 * d; a.bias = bias;
+  a.S = seq_len; a.Tmax = t_max; a.pos = pos; a.pos_dev = pos_dev; a.kcache = kcache; a.vcache = vcache;
+  return launch_skinny(a, EPI_PHI_IN, (a.N + 15) / 16 * 16, (hipStream_t)stream);
 }
 
 int ohara_gemm_skinny_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n, int k, const uint16_t* norm_w,

@@ -72,10 +72,11 @@ __global__ void kv_append_kernel(const bf16_t* k, const bf16_t* v, int ld, int r
 // ---- attention ---------------------------------------------------------------------------
 // One workgroup per (sequence, head, new token) and context chunk.  Sixteen lanes own one cached
 // position at a time (lane l the eight features 8l .. 8l+7) and fetch two positions per round before
-// using either, so a workgroup walks 32 positions per round with an online softmax per 16-lane group;
+// using either (four measured slower: 178 registers halve the occupancy), so a workgroup walks 32
+// positions per round with an online softmax per 16-lane group;
 // the groups are merged through LDS at the end.  With several chunks (decode: few queries, long
-// context) every chunk leaves {weighted sum, max, sum} and phi_attn_merge_kernel combines them in
-// chunk order.
+// context) every chunk leaves {weighted sum, max, sum} and the workgroup that finishes last combines
+// them in chunk order.
 //
 // The reference rotates every cached key again at each step (phi.py:104).  With the rotated query
 // qr and c, s the cosine / sine of key position t the score is
@@ -93,8 +94,9 @@ struct PhiAttnArgs {
   bf16_t* out;       // (rows, H*D)
   int S, H, D, rot, t_max, pos;
   const int32_t* pos_dev;
-  int ns;      // context chunks (decode): chunk c of a (sequence, head) is blockIdx.y
-  float* ws;   // ns > 1: per (row, head, chunk) D + 2 floats {weighted sum[D], max, sum}
+  int ns;         // context chunks (decode): chunk c of a (sequence, head) is blockIdx.y
+  float* ws;      // ns > 1: per (row, head, chunk) D + 2 floats {weighted sum[D], max, sum}
+  int* counters;  // ns > 1: per (row, head) chunks finished; zero between calls
 };
 
 __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
@@ -163,14 +165,14 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
     t_lo = (int)blockIdx.y * per;
     t_hi = min(pq, t_lo + per - 1);
   }
-  for (int t = t_lo + grp; t <= t_hi; t += 32) {
-    const bool two = t + 16 <= t_hi;
-    uint4 kv[2], vv[2];
-    float cs[2][8], sn[2][8];
+  constexpr int R = 2;  // positions a lane group has in flight per round
+  for (int t = t_lo + grp; t <= t_hi; t += 16 * R) {
+    uint4 kv[R], vv[R];
+    float cs[R][8], sn[R][8];
 #pragma unroll
-    for (int r = 0; r < 2; ++r) {
+    for (int r = 0; r < R; ++r) {
       const int tt = t + 16 * r;
-      const bool in = own && (r == 0 || two);
+      const bool in = own && tt <= t_hi;
       kv[r] = in ? ldg16(kb + (size_t)tt * hd) : make_uint4(0, 0, 0, 0);
       vv[r] = in ? ldg16(vb + (size_t)tt * hd) : make_uint4(0, 0, 0, 0);
       if (vec8) {
@@ -197,8 +199,8 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
       }
     }
 #pragma unroll
-    for (int r = 0; r < 2; ++r) {
-      if (r == 1 && !two) break;  // uniform within the 16-lane group
+    for (int r = 0; r < R; ++r) {
+      if (t + 16 * r > t_hi) break;  // uniform within the 16-lane group
       const uint32_t ku[4] = {kv[r].x, kv[r].y, kv[r].z, kv[r].w};
       float part = 0.f;
 #pragma unroll
@@ -243,34 +245,58 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
       den += wg * gl[g];
     }
     if (a.ns > 1) {
+      // write-through stores: the workgroup that merges may sit on another XCD
       float* o = a.ws + (((size_t)row * a.H + h) * a.ns + blockIdx.y) * (D + 2);
-      o[tid] = num;
+      st_coh4(o + tid, __float_as_uint(num));
       if (tid == 0) {
-        o[D] = M;  // -inf: this chunk lies beyond the query's position
-        o[D + 1] = den;
+        st_coh4(o + D, __float_as_uint(M));  // -inf: this chunk lies beyond the query's position
+        st_coh4(o + D + 1, __float_as_uint(den));
       }
     } else {
       a.out[(size_t)row * hd + (size_t)h * D + tid] = f2bf(num / den);
     }
   }
-}
+  if (a.ns == 1) return;
 
-// chunks of one (row, head) -> out, in chunk order
-__global__ void phi_attn_merge_kernel(const float* ws, bf16_t* out, int H, int D, int ns) {
-  const int rh = blockIdx.x, tid = threadIdx.x;
-  if (tid >= D) return;
-  const float* p = ws + (size_t)rh * ns * (D + 2);
-  float M = -INFINITY;
-  for (int c = 0; c < ns; ++c) M = fmaxf(M, p[(size_t)c * (D + 2) + D]);
-  float num = 0.f, den = 0.f;
-  for (int c = 0; c < ns; ++c) {
-    const float mc = p[(size_t)c * (D + 2) + D];
-    if (mc == -INFINITY) continue;
-    const float wg = expf(mc - M);
-    num += wg * p[(size_t)c * (D + 2) + tid];
-    den += wg * p[(size_t)c * (D + 2) + D + 1];
+  // The workgroup that finishes last merges the chunks of its (row, head), in chunk order.  The fence
+  // waits for this workgroup's write-through stores; the counter is a relaxed device-scope atomic; the
+  // merge reads with cache-bypassing loads.
+  __shared__ int is_last;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  int* counter = a.counters + (size_t)row * a.H + h;
+  if (tid == 0) {
+    const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    is_last = old == a.ns - 1;
+    if (is_last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next call
   }
-  out[(size_t)rh * D + tid] = f2bf(num / den);
+  __syncthreads();
+  if (!is_last) return;
+  const float* p = a.ws + ((size_t)row * a.H + h) * a.ns * (D + 2);
+  if (tid < a.ns) {  // ns <= 64: one round of loads for all (max, sum) pairs
+    // qr and gacc are free again: chunk maxima and sums go there
+    qr[tid] = __uint_as_float(ld_coh4(p + (size_t)tid * (D + 2) + D));
+    gacc[0][tid] = __uint_as_float(ld_coh4(p + (size_t)tid * (D + 2) + D + 1));
+  }
+  __syncthreads();
+  if (tid < D) {
+    float M = -INFINITY;
+    for (int c = 0; c < a.ns; ++c) M = fmaxf(M, qr[c]);
+    float num = 0.f, den = 0.f;
+    for (int c0 = 0; c0 < a.ns; c0 += 8) {
+      float av[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) av[i] = c0 + i < a.ns ? __uint_as_float(ld_coh4(p + (size_t)(c0 + i) * (D + 2) + tid)) : 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (c0 + i >= a.ns || qr[c0 + i] == -INFINITY) continue;
+        const float wg = expf(qr[c0 + i] - M);
+        num += wg * av[i];
+        den += wg * gacc[0][c0 + i];
+      }
+    }
+    a.out[(size_t)row * hd + (size_t)h * D + tid] = f2bf(num / den);
+  }
 }
 
 }  // namespace
@@ -302,7 +328,8 @@ int ohara_kv_append_bf16(const uint16_t* k, const uint16_t* v, int ld, int batch
 
 int64_t ohara_phi_attn_workspace_bytes(int batch, int h, int dh, int n_split) {
   if (batch < 1 || h < 1 || dh < 1 || n_split < 1) return OHARA_EINVAL;
-  return (int64_t)batch * h * n_split * (dh + 2) * (int64_t)sizeof(float);
+  const int64_t counters = (((int64_t)batch * h * (int64_t)sizeof(int)) + 255) & ~(int64_t)255;
+  return counters + (int64_t)batch * h * n_split * (dh + 2) * (int64_t)sizeof(float);
 }
 
 int ohara_phi_attn_bf16(const uint16_t* q, int ldq, const uint16_t* kcache, const uint16_t* vcache, const float* cos,
@@ -318,12 +345,10 @@ int ohara_phi_attn_bf16(const uint16_t* q, int ldq, const uint16_t* kcache, cons
   if (n_split < 1 || n_split > 64 || (n_split > 1 && (!workspace || seq_len != 1))) return OHARA_EINVAL;
   const int64_t grid = (int64_t)batch * seq_len * h;
   if (grid > INT32_MAX) return OHARA_ESIZE;
+  const size_t counters = (((size_t)batch * h * sizeof(int)) + 255) & ~(size_t)255;
   PhiAttnArgs a{q, ldq, kcache, vcache, cos, sin, out, seq_len, h, dh, rot, t_max, pos, pos_dev, n_split,
-                reinterpret_cast<float*>(workspace)};
+                reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counters), reinterpret_cast<int*>(workspace)};
   hipLaunchKernelGGL(phi_attn_kernel, dim3((unsigned)grid, (unsigned)n_split), dim3(256), 0, (hipStream_t)stream, a);
-  if (n_split > 1)
-    hipLaunchKernelGGL(phi_attn_merge_kernel, dim3((unsigned)grid), dim3(128), 0, (hipStream_t)stream, a.ws, out, h, dh,
-                       n_split);
   return ohara_launch_status();
 }
 

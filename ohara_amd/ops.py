@@ -482,6 +482,18 @@ def linear_bias(x, w: PackedLinear, bias, epilogue: str = "bias", add1=None, add
     return out
 
 
+def phi_block_in(x, ln_w, ln_b, eps, w: PackedLinear, bias, d, ff, batch, seq_len, pos, kcache, vcache, q, act,
+                 pos_dev=None) -> None:
+    """LayerNorm + [q; k; v; fc1] projection with bias + cache append + new_gelu in one launch
+    (phi.py:150, :81-87, :95, :50-51).  x: (rows, d); q: (rows, d); act: (rows, ff)."""
+    _need(x, BF16, "x")
+    if w.n != 3 * d + ff or w.k != d or bias.numel() != w.n:
+        raise ValueError("packed weight / bias do not match [q; k; v; fc1]")
+    check(lib().ohara_phi_block_in_bf16(_ptr(x), x.stride(0), _ptr(ln_w), _ptr(ln_b), eps, _ptr(w.data), _ptr(bias), d, ff,
+                                        batch, seq_len, pos, _ptr(pos_dev), _ptr(q), q.stride(0), _ptr(kcache), _ptr(vcache),
+                                        kcache.shape[1], _ptr(act), act.stride(0), _stream()), "phi_block_in")
+
+
 def layernorm(x, weight, bias, eps: float = 1e-5, out=None) -> torch.Tensor:
     """nn.LayerNorm over the last dimension of a (rows, d) bf16 matrix (phi.py:132, :160)."""
     _need(x, BF16, "x")
@@ -506,7 +518,7 @@ def phi_attn_workspace(batch, h, dh, n_split, device) -> torch.Tensor:
     nbytes = lib().ohara_phi_attn_workspace_bytes(batch, h, dh, n_split)
     if nbytes < 0:
         raise ValueError("phi_attn_workspace: invalid sizes")
-    return torch.empty(nbytes // 4, dtype=torch.float32, device=device)
+    return torch.zeros(nbytes, dtype=torch.uint8, device=device)  # the chunk counters start at zero
 
 
 def phi_attn(q, kcache, vcache, cos, sin, rot, batch, seq_len, h, dh, pos, pos_dev=None, out=None, n_split=1,

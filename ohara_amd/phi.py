@@ -86,17 +86,18 @@ class Phi:
         self.layers = []
         for i in range(c.num_hidden_layers):
             p = f"layers.{i}."
-            # one packed [q; k; v] weight: the three projections read the same rows (phi.py:81-83)
-            wqkv = torch.cat([dev(state[p + f"mixer.{n}.weight"]) for n in ("q_proj", "k_proj", "v_proj")])
-            bqkv = torch.cat([dev(state[p + f"mixer.{n}.bias"]) for n in ("q_proj", "k_proj", "v_proj")])
+            # one packed [q; k; v; fc1] weight: the four projections read the same normalised rows
+            # (phi.py:81-83, :50), so they are one launch
+            names = ("mixer.q_proj", "mixer.k_proj", "mixer.v_proj", "mlp.fc1")
+            w_in = torch.cat([dev(state[p + n + ".weight"]) for n in names])
+            b_in = torch.cat([dev(state[p + n + ".bias"]) for n in names])
             self.layers.append(dict(
                 ln_w=dev(state[p + "ln.weight"]), ln_b=dev(state[p + "ln.bias"]),
-                wqkv=ops.pack_linear(wqkv), bqkv=bqkv.contiguous(),
+                w_in=ops.pack_linear(w_in), b_in=b_in.contiguous(),
                 dense=ops.pack_linear(dev(state[p + "mixer.dense.weight"])), dense_b=dev(state[p + "mixer.dense.bias"]),
-                fc1=ops.pack_linear(dev(state[p + "mlp.fc1.weight"])), fc1_b=dev(state[p + "mlp.fc1.bias"]),
                 fc2=ops.pack_linear(dev(state[p + "mlp.fc2.weight"])), fc2_b=dev(state[p + "mlp.fc2.bias"]),
             ))
-            del wqkv
+            del w_in
         torch.cuda.synchronize(self.device)
         self._bufs: dict = {}
 
@@ -118,7 +119,7 @@ class Phi:
                 self._bufs.clear()
             d = self.config.hidden_size
             new = lambda n: torch.empty(rows, n, dtype=BF16, device=self.device)
-            b = dict(x=[new(d), new(d)], h=new(d), qkv=new(3 * d), attn=new(d), mixer=new(d), act=new(self.ff))
+            b = dict(x=[new(d), new(d)], h=new(d), q=new(d), attn=new(d), mixer=new(d), act=new(self.ff))
             # single-token calls: the context of a (sequence, head) is spread over up to 16 workgroups,
             # aiming at about 2048 workgroups of at least 64 positions
             heads = rows * self.config.num_attention_heads
@@ -162,14 +163,12 @@ class Phi:
         cur, nxt = buf["x"]
         ops.embed(ids, self.wte, out=cur)
         for L, cache in zip(self.layers, kv_cache):
-            h, qkv = buf["h"], buf["qkv"]
-            ops.layernorm(cur, L["ln_w"], L["ln_b"], c.eps, out=h)
-            ops.linear_bias(h, L["wqkv"], L["bqkv"], out=qkv)
-            ops.kv_append(qkv[:, d:2 * d], qkv[:, 2 * d:], cache.key, cache.value, B, S, H, D, start, pos_dev)
-            ops.phi_attn(qkv[:, :d], cache.key, cache.value, self.cos, self.sin, self.rot, B, S, H, D, start, pos_dev,
+            ops.layernorm(cur, L["ln_w"], L["ln_b"], c.eps, out=buf["h"])
+            ops.phi_block_in(buf["h"], None, None, c.eps, L["w_in"], L["b_in"], d, self.ff, B, S, start, cache.key,
+                             cache.value, buf["q"], buf["act"], pos_dev)
+            ops.phi_attn(buf["q"], cache.key, cache.value, self.cos, self.sin, self.rot, B, S, H, D, start, pos_dev,
                          out=buf["attn"], n_split=buf["ns"] if S == 1 else 1, workspace=buf["ws"])
             ops.linear_bias(buf["attn"], L["dense"], L["dense_b"], out=buf["mixer"])
-            ops.linear_bias(h, L["fc1"], L["fc1_b"], "gelu", out=buf["act"])
             ops.linear_bias(buf["act"], L["fc2"], L["fc2_b"], "add2", add1=buf["mixer"], add2=cur, out=nxt)
             cur, nxt = nxt, cur
         src = cur.view(B, S, d)[:, -1].contiguous() if (last_only and S > 1) else cur

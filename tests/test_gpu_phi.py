@@ -222,3 +222,43 @@ def test_greedy_generation_matches_the_oracle_teacher_forced(cuda, use_graph):
                 assert abs(la - lb) <= 2.0 ** -6 * max(abs(la), abs(lb)), (t, b, tok, best)
         if t + 1 < steps:
             logits = ref(toks[:, t:t + 1], rc, 9 + t)[:, -1]
+
+
+def test_block_head_matches_the_separate_kernels(cuda):
+    """LayerNorm + [q; k; v; fc1] + append + new_gelu in one launch against the same steps as
+    separate kernels (its variance comes from the sums of x and x^2, so a normalised value may
+    round the other way now and then)."""
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(4)
+    for B, S, d, ff, H, pos in ((2, 3, 64, 256, 4, 5), (1, 1, 320, 1280, 4, 0), (3, 1, 2560, 10240, 32, 7),
+                                (70, 1, 64, 128, 2, 2), (2, 1, 2048, 128, 16, 1)):
+        rows, D, Tmax = B * S, d // H, 16
+        x = (torch.randn(rows, d, generator=g) + 0.3).to(BF).to(cuda)
+        lw = (1 + 0.1 * torch.randn(d, generator=g)).to(BF).to(cuda)
+        lb = (0.1 * torch.randn(d, generator=g)).to(BF).to(cuda)
+        w = (torch.randn(3 * d + ff, d, generator=g) / d ** 0.5).to(BF).to(cuda)
+        b = (0.2 * torch.randn(3 * d + ff, generator=g)).to(BF).to(cuda)
+        pw = ops.pack_linear(w)
+        kc = torch.zeros(B, Tmax, H, D, dtype=BF, device=cuda)
+        vc = torch.zeros_like(kc)
+        q = torch.empty(rows, d, dtype=BF, device=cuda)
+        act = torch.empty(rows, ff, dtype=BF, device=cuda)
+        ops.phi_block_in(x, lw, lb, 1e-5, pw, b, d, ff, B, S, pos, kc, vc, q, act)
+        h = ops.layernorm(x, lw, lb, 1e-5)
+        y = ops.linear_bias(h, pw, b)
+        kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+        ops.kv_append(y[:, d:2 * d], y[:, 2 * d:3 * d], kc2, vc2, B, S, H, D, pos)
+        want_act = P.new_gelu(y[:, 3 * d:].cpu())
+        # without the prologue (normalised rows handed in) the results are those of the separate kernels
+        kc3, vc3, q3, act3 = torch.zeros_like(kc), torch.zeros_like(vc), torch.empty_like(q), torch.empty_like(act)
+        ops.phi_block_in(h, None, None, 1e-5, pw, b, d, ff, B, S, pos, kc3, vc3, q3, act3)
+        assert torch.equal(q3, y[:, :d]) and torch.equal(kc3, kc2) and torch.equal(vc3, vc2)
+        assert (act3.cpu() != want_act).float().mean().item() < 5e-3
+        for name, got, want in (("q", q, y[:, :d]), ("k", kc, kc2), ("v", vc, vc2), ("act", act.cpu(), want_act)):
+            got, want = got.float().cpu(), want.float().cpu()
+            diff = (got - want).abs()
+            scale = want.abs().max().item()
+            assert diff.max().item() <= 2.0 ** -6 * scale, (name, B, d, diff.max().item(), scale)
+            assert (diff > 0).float().mean().item() < 0.02, (name, B, d, (diff > 0).float().mean().item())
+        assert torch.equal(kc[:, :pos], torch.zeros_like(kc[:, :pos])) and torch.equal(kc[:, pos + S:], torch.zeros_like(kc[:, pos + S:]))
