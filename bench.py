@@ -446,7 +446,7 @@ def phi_decode_only(dev, batch, steps=12, context=1024):
 
 def bench_phi(dev):
     """Phi-2 shape, random bf16 weights: greedy decode at batch 1 and 8 after a 1024-token context, one
-    graph replay per step (8 launches per layer)."""
+    graph replay per step (5 launches per layer)."""
     cfg, model = phi2_model(dev)
     d, f, v = cfg.hidden_size, cfg.multiple_of * cfg.hidden_size, cfg.vocab_size
     nl, ctx, steps = cfg.num_hidden_layers, 1024, 64
