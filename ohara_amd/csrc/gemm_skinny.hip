@@ -70,7 +70,8 @@ __device__ __forceinline__ float sum8(uint4 v) {
 // instead of 4 are what fills the memory pipeline.
 template <int BT, int NORM, int EPI, int NW = 4>
 __global__ __launch_bounds__(NW * 64) void skinny_kernel(GemmArgs a) {
-  constexpr int CH = BT <= 2 ? 6 : 4;  // k-steps whose loads are issued back to back
+  // k-steps whose loads are issued back to back (the many-wave variants have no norm operands to hold)
+  constexpr int CH = (NORM == 0 && NW > 4) ? 10 : (BT <= 2 ? 6 : 4);
   // workgroup id -> (strip, chunk of 16*BT rows).  Ids go round-robin over the 8 XCDs; the chunks of
   // one strip get ids 8 apart, so they run on the same XCD and share its L2 copy of the weights.
   const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
