@@ -324,6 +324,126 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
   int token = -1;
   bool compact = false;
   bool have_x = false;
+  // ---- nucleus only (the reference's chat default: temperature 0.8, top_p 0.95, no top-k,
+  // chat_engine.py:35-37), bf16 rows ---------------------------------------------------------------
+  // For a peaked distribution the nucleus is a few tokens out of tens of thousands.  The candidates
+  // are every id at or above the 256-th largest of the per-thread maxima - a complete upper set of
+  // the row, usually a few hundred ids; they are sorted and walked exactly as the reference's sort +
+  // cumsum does, with probabilities from the softmax of the WHOLE row.  When their mass does not
+  // reach top_p (flat rows) the general path below takes over.
+  if (a.top_k == 0 && a.top_p > 0.f && a.top_p < 1.f && packed_row && EPT % 8 == 0 && nvalid > 0) {
+    uint32_t raw[EPT / 2];
+    const bf16_t* row = reinterpret_cast<const bf16_t*>(a.logits) + (size_t)b * a.ldl + base;
+#pragma unroll
+    for (int c = 0; c < EPT / 8; ++c) {
+      const uint4 v = base + 8 * c < V ? ldg16(row + 8 * c) : make_uint4(0, 0, 0, 0);
+      raw[4 * c] = v.x; raw[4 * c + 1] = v.y; raw[4 * c + 2] = v.z; raw[4 * c + 3] = v.w;
+    }
+    auto bits16 = [&](int i) -> uint32_t { return (i & 1) ? (raw[i >> 1] >> 16) : (raw[i >> 1] & 0xffffu); };
+    auto key16 = [&](int i) -> uint32_t {  // order-preserving 16-bit key of element i, 0 when masked
+      const uint32_t bits = bits16(i);
+      const uint32_t kk = (bits & 0x8000u) ? (~bits & 0xffffu) : (bits | 0x8000u);
+      return base + i < nvalid ? kk : 0u;
+    };
+    uint32_t tmax = 0;
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) tmax = max(tmax, key16(i));
+    // softmax statistics of the whole row, formed as the general path forms them: dividing by the
+    // temperature is monotone, so the maximum of the quotients is the quotient of the maximum
+    const uint32_t mbits = (tmax & 0x8000u) ? (tmax & 0x7fffu) : (~tmax & 0xffffu);
+    const float m = block_max(tmax > 0 ? __uint_as_float(mbits << 16) / temp : -INFINITY, s);
+    const int have = block_sum_i(tmax > 0 ? 1 : 0, s);
+    uint32_t bound = 1;  // fewer than 256 threads hold a valid id: every valid id is a candidate
+    if (have >= 256) {
+      int dummy;
+      bound = radix_select<1, 8>(256, dummy, s, [&](int) { return tmax > 0; }, [&](int) { return tmax; });
+    }
+    // One CU walks the whole row, so every instruction per element costs about half a microsecond:
+    // this pass only has to decide whether the candidates hold the nucleus, and uses the hardware
+    // exponential and a multiplication by 1 / temperature (exact arithmetic follows for the
+    // candidates only).  Candidates claim their slot with an LDS counter; the order they land in
+    // does not matter, the sort below is total (key, then id).
+    __syncthreads();
+    if (tid == 0) s.misc[0] = 0;
+    __syncthreads();
+    float zs = 0.f, zc = 0.f;
+    const float rtemp = 1.0f / temp;
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) {
+      const uint32_t kk = key16(i);
+      const float e = kk == 0 ? 0.f : __expf(__uint_as_float(bits16(i) << 16) * rtemp - m);  // exp(-inf) = 0
+      zs += e;
+      if (kk >= bound) {
+        zc += e;
+        const int slot = atomicAdd(&s.misc[0], 1);
+        if (slot < CAP) {
+          s.skey[slot] = fkey(__uint_as_float(bits16(i) << 16) / temp);
+          s.sid[slot] = base + i;
+        }
+      }
+    }
+    const float Zq = block_sum(zs, s);
+    const float Zc = block_sum(zc, s);  // (the syncs inside also publish the counter and the slots)
+    const int n_c = s.misc[0];
+    // the nucleus closes inside the candidates when their mass exceeds top_p (with a margin for the
+    // different summation orders), or when the candidates are all there is
+    if (n_c <= CAP && (Zc / Zq > a.top_p + 1e-3f || bound == 1)) {
+      int n2 = 64;
+      while (n2 < n_c) n2 <<= 1;
+      __syncthreads();
+      for (int i = n_c + tid; i < n2; i += NT) {
+        s.skey[i] = 0;  // padding sorts last
+        s.sid[i] = 0x7fffffff;
+      }
+      __syncthreads();
+      sort_candidates(s, n2);
+      if (tid < n_c) {
+        const float xi = unfkey(s.skey[tid]);
+        s.skey[tid] = __float_as_uint(xi == -INFINITY ? 0.f : expf(xi - m) / Zq);  // probabilities, sorted order
+      }
+      __syncthreads();
+      if (tid == 0) {
+        // sequential fp32 sums in the order the reference's cumsum walks (chat_engine.py:71-79)
+        float kept = 0.f, run = 0.f;
+        int n_in = 0;
+        bool closed = bound == 1;
+        for (int j = 0; j < n_c; ++j) {  // kept prefix: mass before the token <= top_p
+          if (run > a.top_p) {
+            closed = true;
+            break;
+          }
+          const float pj = __uint_as_float(s.skey[j]);
+          kept += pj;
+          run += pj;
+          ++n_in;
+        }
+        int tok = -2;  // -2: the candidates ran out before the nucleus closed
+        if (closed || run > a.top_p) {
+          const float target = u * kept;
+          int last = -1;
+          tok = -1;
+          run = 0.f;
+          for (int j = 0; j < n_in; ++j) {
+            const float pj = __uint_as_float(s.skey[j]);
+            run += pj;
+            if (pj > 0.f) last = s.sid[j];
+            if (pj > 0.f && run > target) {
+              tok = s.sid[j];
+              break;
+            }
+          }
+          if (tok < 0) tok = max(last, 0);  // rounding pushed the target past the end: last kept id
+        }
+        s.misc[3] = tok;
+      }
+      __syncthreads();
+      if (s.misc[3] >= 0) {
+        token = s.misc[3];
+        compact = true;
+      }
+      __syncthreads();
+    }
+  }
   // ---- small top-k: the survivors fit one sorted block, everything after works on that block -----
   if (a.top_k > 0 && min(a.top_k, V) <= CAP) {
     const int k = min(a.top_k, V);

@@ -58,6 +58,10 @@ CASES = [
     (1000, 16, 0.7, 7, 0.0, 2.0, torch.bfloat16),
     (65536, 8, 0.8, 50, 0.9, 0.55, torch.bfloat16),    # the headline sampling setting
     (65536, 4, 1.0, 0, 0.95, 3.0, torch.bfloat16),     # peaked, nucleus only
+    (65536, 6, 0.8, 0, 0.95, 8.0, torch.bfloat16),     # the reference's chat defaults on a sharp row: a few candidates
+    (65536, 6, 1.0, 0, 0.5, 5.0, torch.bfloat16),      # nucleus closes inside the sorted candidates
+    (32000, 6, 0.7, 0, 0.9, 6.0, torch.bfloat16),
+    (65536, 4, 1.0, 0, 0.999, 8.0, torch.bfloat16),    # candidates run out: falls back to the general path
     (65536, 3, 1.0, 0, 0.9, 0.5, torch.bfloat16),      # flat: tens of thousands kept (multi-round path)
     (65536, 3, 1.0, 5000, 0.5, 0.5, torch.float32),
     (32000, 4, 0.8, 0, 0.0, 1.0, torch.bfloat16),      # vocabulary-order draw
