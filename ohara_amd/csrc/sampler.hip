@@ -14,7 +14,11 @@
 // function of (logits, parameters, u).
 //
 // A thread owns EPT consecutive vocabulary entries in registers; the 1024 threads cover up to
-// 1024*EPT ids.  Two routes from there:
+// 1024*EPT ids.  Three routes from there:
+//   * top-p alone on bf16 rows (the reference's chat default, chat_engine.py:35-37): every id at or
+//     above the 256-th largest per-thread maximum is a candidate; if the candidates' share of the
+//     whole-row softmax exceeds top_p they are sorted and scanned like the survivors of a small
+//     top-k below, otherwise the third route runs;
 //   * top-k <= 1024: the survivors (everything at or above the k-th largest; a lower bound of it
 //     comes from the per-thread maxima) are compacted into LDS, sorted once (bitonic, descending,
 //     ties lowest id first), soft-maxed and scanned sequentially in fp32 by one thread - the
