@@ -212,7 +212,8 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
       for (int o = 1; o < 16; o <<= 1) part += __shfl_xor(part, o, WAVE);
       const float sc = part * scale;
       const float mn = fmaxf(m, sc);
-      const float corr = expf(m - mn), p = expf(sc - mn);  // m = -inf on the first round: corr = 0
+      // hardware exponential: its error (about 1e-6 relative) is far below the bf16 rounding of the output
+      const float corr = __expf(m - mn), p = __expf(sc - mn);  // m = -inf on the first round: corr = 0
       lsum = lsum * corr + p;
       const uint32_t vu[4] = {vv[r].x, vv[r].y, vv[r].z, vv[r].w};
 #pragma unroll
