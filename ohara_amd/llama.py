@@ -294,9 +294,10 @@ class Llama:
 
     def default_n_split(self, batch: int) -> int:
         """Context chunks per (sequence, KV head) so that decode attention launches about
-        eight workgroups per CU (measured on d12 at batch 16 / 32 / 64: 6, 6 and 2-4 chunks are the
-        fastest); a chunk is never shorter than 128 positions."""
-        want = max(1, 2048 // max(1, batch * self.kv_heads))
+        four workgroups per CU (measured on d12, 6 KV heads, at batch 16 / 32 / 64: 6, 6 and 2-4
+        chunks are the fastest, twice as many are slower); a chunk is never shorter than 128
+        positions."""
+        want = max(1, 1024 // max(1, batch * self.kv_heads))
         return max(1, min(want, self.config.max_sequence_length // 128, 64))
 
     def _get_buffers(self, batch: int, rows: int) -> _Buffers:
