@@ -151,6 +151,8 @@ class Phi:
             if position_ids is None:
                 raise ValueError("position_ids is required when using a KV cache")  # phi.py:92-93
             start = int(position_ids)
+        if any(getattr(cache, "int8", False) for cache in kv_cache):
+            raise NotImplementedError("ohara_amd Phi: int8 KV caches are served by the Llama path only")
         ends = [cache._reserve(B, S, start) for cache in kv_cache]
         logits = self._run(x.reshape(-1).to(device=self.device, dtype=torch.int64), B, S, kv_cache, start, pos_dev, last_only)
         for cache, end in zip(kv_cache, ends):
