@@ -401,8 +401,9 @@ int64_t ohara_persistent_error_offset(const OharaModel* m, int batch, int n_spli
 int64_t ohara_persistent_profile_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
 
 /* ---- Phi (ohara/models/phi.py): the parts of its cached decode path that differ from Llama ----
- * nn.Linear WITH bias on packed weights (phi.py:46-47, :63-66, :161), up to any number of rows
- * (64 at a time).  n % 4 == 0, k % 8 == 0.
+ * nn.Linear WITH bias on packed weights (phi.py:46-47, :63-66, :161), any number of rows (up to 64:
+ * the weight-streaming strip kernel; more: the tiled MFMA kernel of ohara_gemm_bf16, same epilogues
+ * and rounding points).  n % 4 == 0, k % 8 == 0.
  *   OHARA_LIN_BIAS       out = bf16(x @ W^T + bias)
  *   OHARA_LIN_BIAS_GELU  out = new_gelu(bf16(x @ W^T + bias)), every op of phi.py:37-40 rounded to
  *                        bf16 as the eager ops round                          (MLP.fc1, phi.py:50-51)

@@ -518,6 +518,7 @@ int ohara_linear_bias_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n
   a.B = rows; a.N = n; a.K = k;
   a.out = out; a.ldo = ldo; a.bias = bias;
   a.resid = add1; a.ldr = ld1; a.resid2 = add2; a.ldr2 = ld2;
+  if (rows > 64) return ohara_launch_gemm_tile(a, epi, (n + 15) / 16 * 16, (hipStream_t)stream);  // prefill
   return launch_skinny(a, epi, (n + 15) / 16 * 16, (hipStream_t)stream);
 }
 
@@ -537,6 +538,7 @@ int ohara_phi_block_in_bf16(const uint16_t* x, int ldx, const uint16_t* ln_w, co
   a.B = batch * seq_len; a.N = 3 * d + ff; a.K = d;
   a.out = q; a.ldo = ldq; a.out2 = act; a.ldo2 = ldact; a.split_n = 3 * d; a.bias = bias;
   a.S = seq_len; a.Tmax = t_max; a.pos = pos; a.pos_dev = pos_dev; a.kcache = kcache; a.vcache = vcache;
+  if (a.B > 64 && !ln_w) return ohara_launch_gemm_tile(a, EPI_PHI_IN, (a.N + 15) / 16 * 16, (hipStream_t)stream);  // prefill
   return launch_skinny(a, EPI_PHI_IN, (a.N + 15) / 16 * 16, (hipStream_t)stream);
 }
 

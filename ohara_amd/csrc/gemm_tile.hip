@@ -128,6 +128,10 @@ int ohara_launch_gemm_tile(const GemmArgs& a, int epi, int packed_rows, hipStrea
     case EPI_RESIDUAL: hipLaunchKernelGGL((gemm_tile_kernel<EPI_RESIDUAL>), grid, block, 0, st, a, MT, NT, nstrips); break;
     case EPI_SWIGLU: hipLaunchKernelGGL((gemm_tile_kernel<EPI_SWIGLU>), grid, block, 0, st, a, MT, NT, nstrips); break;
     case EPI_ROPE: hipLaunchKernelGGL((gemm_tile_kernel<EPI_ROPE>), grid, block, 0, st, a, MT, NT, nstrips); break;
+    case EPI_BIAS: hipLaunchKernelGGL((gemm_tile_kernel<EPI_BIAS>), grid, block, 0, st, a, MT, NT, nstrips); break;
+    case EPI_BIAS_GELU: hipLaunchKernelGGL((gemm_tile_kernel<EPI_BIAS_GELU>), grid, block, 0, st, a, MT, NT, nstrips); break;
+    case EPI_BIAS_ADD2: hipLaunchKernelGGL((gemm_tile_kernel<EPI_BIAS_ADD2>), grid, block, 0, st, a, MT, NT, nstrips); break;
+    case EPI_PHI_IN: hipLaunchKernelGGL((gemm_tile_kernel<EPI_PHI_IN>), grid, block, 0, st, a, MT, NT, nstrips); break;
     default: return OHARA_EINVAL;
   }
   return ohara_launch_status();
