@@ -19,14 +19,14 @@
 namespace {
 
 // ---- routing ---------------------------------------------------------------------------------
-// one wave per token; E <= 1024 experts, k <= 16
+// one wave per token; E <= 64 * MAXPL experts (MAXPL experts per lane), k <= 16
+template <int MAXPL>
 __global__ __launch_bounds__(256) void moe_route_kernel(const bf16_t* logits, int ldl, const bf16_t* bias, int N, int E,
                                                         int k, int biased, int sigmoid, int normalize, int32_t* idx,
                                                         bf16_t* w) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = blockIdx.x * 4 + wave;
   if (n >= N) return;
-  constexpr int MAXPL = 16;  // experts per lane
   float sel[MAXPL], raw[MAXPL];
 #pragma unroll
   for (int i = 0; i < MAXPL; ++i) {
@@ -133,7 +133,10 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int32_t* idx, int 
     const int e = p < NK ? idx[p] : -1;
     sidx[tid] = e;
     __syncthreads();
-    const int n4 = (min(1024, NK - p0) + 3) >> 2;  // entries past the end hold -1 and never match
+    // only earlier pairs count: a wave scans the entries below its last lane, and a wave without a
+    // valid pair scans nothing (entries past the end hold -1 and never match)
+    const int wave_first = tid & ~63;
+    const int n4 = p0 + wave_first < NK ? (min(wave_first + 64, NK - p0) + 3) >> 2 : 0;
     int rank = 0;
     const int4* s4 = reinterpret_cast<const int4*>(sidx);
 #pragma unroll 4
@@ -244,27 +247,46 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const bf16_t* y, int l
                                                           bf16_t* out, int ldo, int d) {
   const int n = blockIdx.x;
   __shared__ int order[16];
-  if (threadIdx.x == 0) {
-    // slots of this token sorted by expert id (k <= 16)
-    int ids[16], sl[16];
+  if (threadIdx.x < 64) {
+    // slots of this token in ascending expert id (k <= 16 distinct experts): lane j ranks its own slot
+    const int lane = threadIdx.x;
+    const int mine = lane < k ? idx[(size_t)n * k + lane] : 0x7fffffff;
+    const int pos = lane < k ? pos_of[(size_t)n * k + lane] : 0;
+    int rank = 0;
     for (int j = 0; j < k; ++j) {
-      ids[j] = idx[(size_t)n * k + j];
-      sl[j] = j;
+      const int other = __shfl(mine, j, WAVE);
+      rank += (other < mine || (other == mine && j < lane)) ? 1 : 0;
     }
-    for (int a_ = 1; a_ < k; ++a_) {
-      const int vi = ids[a_], vs = sl[a_];
-      int b = a_ - 1;
-      while (b >= 0 && ids[b] > vi) {
-        ids[b + 1] = ids[b];
-        sl[b + 1] = sl[b];
-        --b;
-      }
-      ids[b + 1] = vi;
-      sl[b + 1] = vs;
-    }
-    for (int j = 0; j < k; ++j) order[j] = pos_of[(size_t)n * k + sl[j]];
+    if (lane < k) order[rank] = pos;
   }
   __syncthreads();
+  const bool vec = ((d | ldy | ldo | lds_ | ldr) & 3) == 0;
+  if (vec) {  // four columns per thread, 8-byte loads; the adds stay one bf16 add per expert, in order
+    for (int c = threadIdx.x * 4; c < d; c += 1024) {
+      uint2 yv[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) yv[j] = j < k ? ldg8(y + (size_t)order[j] * ldy + c) : make_uint2(0, 0);
+      const uint2 sv = shared ? ldg8(shared + (size_t)n * lds_ + c) : make_uint2(0, 0);
+      const uint2 rv = resid ? ldg8(resid + (size_t)n * ldr + c) : make_uint2(0, 0);
+      float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+        if (j < k) {
+          acc[0] = rbf(acc[0] + lo_bf(yv[j].x)); acc[1] = rbf(acc[1] + hi_bf(yv[j].x));
+          acc[2] = rbf(acc[2] + lo_bf(yv[j].y)); acc[3] = rbf(acc[3] + hi_bf(yv[j].y));
+        }
+      if (shared) {
+        acc[0] = rbf(acc[0] + lo_bf(sv.x)); acc[1] = rbf(acc[1] + hi_bf(sv.x));
+        acc[2] = rbf(acc[2] + lo_bf(sv.y)); acc[3] = rbf(acc[3] + hi_bf(sv.y));
+      }
+      if (resid) {
+        acc[0] = rbf(lo_bf(rv.x) + acc[0]); acc[1] = rbf(hi_bf(rv.x) + acc[1]);
+        acc[2] = rbf(lo_bf(rv.y) + acc[2]); acc[3] = rbf(hi_bf(rv.y) + acc[3]);
+      }
+      stg8(out + (size_t)n * ldo + c, make_uint2(pack_bf(acc[0], acc[1]), pack_bf(acc[2], acc[3])));
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < d; c += 256) {
     float acc = 0.f;
     for (int j = 0; j < k; ++j) acc = rbf(acc + bf2f(y[(size_t)order[j] * ldy + c]));
@@ -284,8 +306,14 @@ int ohara_moe_route_topk(const uint16_t* router_logits, int ldl, const uint16_t*
   if (!router_logits || !expert_idx || !expert_w || n_tokens < 1 || n_experts < 1 || k < 1) return OHARA_EINVAL;
   if (k > 16 || n_experts > 1024 || k > n_experts || ldl < n_experts) return OHARA_ESIZE;
   if (biased_topk && !router_bias) return OHARA_EINVAL;
-  hipLaunchKernelGGL(moe_route_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, (hipStream_t)stream, router_logits, ldl,
-                     router_bias, n_tokens, n_experts, k, biased_topk, gate_sigmoid, normalize, expert_idx, expert_w);
+  const dim3 grid((n_tokens + 3) / 4), block(256);
+#define OHARA_ROUTE(PL_)                                                                                            \
+  hipLaunchKernelGGL(moe_route_kernel<PL_>, grid, block, 0, (hipStream_t)stream, router_logits, ldl, router_bias, \
+                     n_tokens, n_experts, k, biased_topk, gate_sigmoid, normalize, expert_idx, expert_w)
+  if (n_experts <= 64) OHARA_ROUTE(1);
+  else if (n_experts <= 256) OHARA_ROUTE(4);
+  else OHARA_ROUTE(16);
+#undef OHARA_ROUTE
   return ohara_launch_status();
 }
 
