@@ -568,7 +568,7 @@ def main():
         "ms_per_step": r1["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"d12 Llama bf16 greedy decode, batch 1, prompt {args.prompt}, KV cache 4096 "
-                               f"(BASELINE configs[1])", "batch": 1, "prompt_len": args.prompt,
+                               f"(the configuration the metric is quoted on)", "batch": 1, "prompt_len": args.prompt,
                    "context_capacity": 4096, "launch": r1["launch"] + ", HIP graph replay"},
         "also": {f"batch{b}": r for b, r in results.items()},
         "roofline": roof,
