@@ -289,3 +289,28 @@ def test_kv_cache_per_sequence_bookkeeping():
     c.lengths = [8, 8, 8]
     c._commit(3, c._reserve(3, 1, 8))
     assert c.lengths is None and c.length == 9
+
+
+def test_phi_host_side_tables_and_validation():
+    """Phi's host logic needs no GPU: the angle tables are the oracle's (ohara/embeddings_pos/
+    rotary.py:166-184) and a configuration the kernels do not cover is refused before any device work."""
+    import torch
+
+    from ohara_amd.phi import Phi, PhiConfig, rope_cos_sin
+    from oracle import phi_ref as P
+
+    for n, dims in ((16, 6), (2048, 32), (5, 2)):
+        cos, sin = rope_cos_sin(n, dims)
+        rc, rs = P.rope_cos_sin(n, dims)
+        assert cos.dtype == torch.float32 and cos.shape == (n, dims // 2)
+        assert torch.equal(cos, rc) and torch.equal(sin, rs)
+    assert PhiConfig() == PhiConfig(vocab_size=51200, max_sequence_length=2048, hidden_size=2560, num_attention_heads=32,
+                                    num_hidden_layers=32, dropout=0.2, multiple_of=4, bias=True, eps=1e-5, rotary_dim=0.4)
+    with pytest.raises(ValueError, match="divisible"):
+        Phi(PhiConfig(hidden_size=62, num_attention_heads=4), {}, device="cpu")
+    with pytest.raises(ValueError, match="positive even number"):  # int(0.1 * 16) = 1 rotated feature
+        Phi(PhiConfig(hidden_size=64, num_attention_heads=4, rotary_dim=0.1), {}, device="cpu")
+    with pytest.raises(NotImplementedError, match="multiple of 8"):
+        Phi(PhiConfig(hidden_size=48, num_attention_heads=4), {}, device="cpu")
+    with pytest.raises(ValueError, match="bfloat16"):
+        Phi(PhiConfig(), {}, device="cpu", dtype=torch.float16)
