@@ -77,3 +77,34 @@ def test_d12_batch32_prompt1024_matches_single_sequence_runs(cuda):
     got = model.generate_greedy(prompt, steps + 1)
     agree = (got == torch.stack(toks, 1)).float().mean().item()
     assert agree >= 0.97, agree
+
+
+def test_phi2_width_prefill_and_decode_against_the_oracle(cuda):
+    """Phi-2's real widths (d 2560, 32 heads of 80 with 32 rotated features, MLP 10240, vocabulary
+    51200) on four layers: a 70-token prefill (the tiled kernel's epilogues), cached decode steps of
+    3 sequences (8- and 16-wave strip kernels, context chunks in attention) and the uncached forward,
+    against the CPU oracle on the same bf16 weights."""
+    from ohara_amd.phi import Phi, PhiConfig
+    from oracle import phi_ref as P
+
+    kw = dict(num_hidden_layers=4, max_sequence_length=256)
+    rcfg = P.RefPhiConfig(**kw)
+    w = P.init_weights(rcfg, seed=11, dtype=torch.bfloat16, std=0.02, bias_std=0.02)
+    ref, model = P.RefPhi(rcfg, w), Phi(PhiConfig(**kw), w, device=cuda)
+    g = torch.Generator().manual_seed(0)
+    B, S0 = 3, 70
+    ids = torch.randint(0, rcfg.vocab_size, (B, S0 + 2), generator=g)
+    rc, cache = ref.build_kv_cache(B), model.build_kv_cache(B)
+
+    def close(got, want):
+        got, want = got.float().cpu(), want.float()
+        scale = want.abs().max().item()
+        d = (got - want).abs()
+        assert d.max().item() <= 4e-2 * scale and d.mean().item() <= 4e-3 * scale, (d.max().item(), d.mean().item(), scale)
+
+    close(model(ids[:, :S0].to(cuda), cache, 0, last_only=True)[:, 0], ref(ids[:, :S0], rc, 0)[:, -1])
+    for t in (S0, S0 + 1):
+        close(model(ids[:, t:t + 1].to(cuda), cache, t), ref(ids[:, t:t + 1], rc, t))
+    close(cache[-1].key[:B, :S0 + 2], rc[-1].key[:B, :S0 + 2])
+    toks = model.generate_greedy(ids[:, :S0].to(cuda), 4)
+    assert toks.shape == (B, 4) and int(toks.min()) >= 0 and int(toks.max()) < rcfg.vocab_size
