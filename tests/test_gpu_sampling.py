@@ -131,3 +131,28 @@ def test_inference_sampler_matches_oracle(cuda):
     want = inference_sampler_ref(logits, temperature=0.7, top_p=0.0, u=u)
     got = inference_sampler(logits.to(cuda), temperature=0.7, top_p=0.0, u=u).cpu()
     assert torch.equal(got, want)
+
+
+def test_nucleus_alone_on_rows_with_many_ties(cuda):
+    """Top-p without top-k on bf16 rows built from a handful of levels (whole blocks of equal
+    probabilities), with and without a padded vocabulary tail: ties are taken lowest id first, the
+    nucleus may end inside a block of ties, and the candidate route and the general route must agree
+    with the oracle."""
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(21)
+    V, B = 65536, 6
+    levels = torch.tensor([0.0, 2.0, 4.0, 9.0, 12.0])
+    pick = torch.multinomial(torch.tensor([0.9, 0.07, 0.02, 0.009, 0.001]), B * V, replacement=True, generator=g)
+    logits = levels[pick].view(B, V).to(torch.bfloat16)
+    tol = 5e-5
+    for T, p, valid in ((1.0, 0.6, None), (0.8, 0.95, None), (1.0, 0.3, 60000), (1.3, 0.05, None)):
+        for trial in range(3):
+            u = torch.rand(B, generator=g)
+            want, margin = sample_next_token_ref(logits.unsqueeze(1), T, p, 0, u=u, valid_vocab=valid, return_margin=True)
+            got = ops.sample_topk_topp(logits.to(cuda), T, 0, p, u.to(cuda), valid_vocab=valid).cpu()
+            for b in range(B):
+                if float(margin[b]) > tol:
+                    assert int(got[b]) == int(want[b, 0]), (T, p, valid, b, int(got[b]), int(want[b, 0]), float(margin[b]))
+                if valid is not None:
+                    assert int(got[b]) < valid
