@@ -490,6 +490,7 @@ class DecodeSession:
         elif persistent and not model.supports_persistent(batch):
             raise ValueError("the persistent decode kernel does not cover this shape")
         self._pws = None
+        self.spin_limit = 0  # bound of the persistent kernel's barrier waits (0 = the library's default)
         self.cache = kv_cache if kv_cache is not None else model.build_kv_cache(batch)
         if self.cache[0].int8:
             persistent = False  # the single-launch kernel reads bf16 caches only
@@ -556,7 +557,7 @@ class DecodeSession:
         greedy = 0 if self.sampling else 1
         if self.persistent:
             check(lib().ohara_llama_decode_persistent(C.byref(m._c_model), C.byref(self._dst), self._pws.data_ptr(),
-                                                      self._nwg, 0, greedy, 0, stream), "persistent decode step")
+                                                      self._nwg, 0, greedy, int(self.spin_limit), stream), "persistent decode step")
         else:
             check(lib().ohara_llama_forward(C.byref(m._c_model), C.byref(self._dst), 1, 0, 1, _lib.OHARA_LOGITS_LAST,
                                             greedy, stream), "decode step")
@@ -572,6 +573,17 @@ class DecodeSession:
             word = self._pws[self._err_off : self._err_off + 4].view(torch.int32).cpu()
             if int(word[0]) != 0:
                 raise RuntimeError("persistent decode kernel: a grid barrier wait expired")
+
+    def reset_error(self) -> None:
+        """Recover from an expired barrier wait: re-initialise the workspace (barrier counters, launch
+        count and the sticky error word).  A workgroup whose wait expired runs ahead, so arrivals of
+        different barriers mix in the counters and later barriers would never release; the counters
+        cannot be kept.  Synchronises."""
+        if self.persistent and self._pws is not None:
+            torch.cuda.current_stream().synchronize()
+            check(lib().ohara_llama_decode_persistent(C.byref(self.model._c_model), C.byref(self._dst), self._pws.data_ptr(),
+                                                      self._nwg, 1, 1, 0, torch.cuda.current_stream().cuda_stream),
+                  "persistent init")
 
     def phase_clocks(self) -> torch.Tensor:
         """Shader-clock samples of workgroup 0 at the phase boundaries of the last step run

@@ -322,3 +322,36 @@ def test_decode_to_the_last_cache_position(cuda, persistent):
     _assert_logits_close(one, ref(prompt[:, :1], ref.build_kv_cache(2), 0), 4e-2, 4e-3)
     full = torch.randint(0, 256, (1, 48), generator=torch.Generator().manual_seed(3))
     _assert_logits_close(model(full.to(cuda)), ref(full), 4e-2, 4e-3)
+
+
+def test_expired_barrier_wait_is_reported_and_does_not_hang(cuda):
+    """Failure handling of the persistent kernel, forced from the host: with a spin limit of one
+    every barrier wait expires, the kernel still runs to its end, the sticky error word is set and
+    the session reports it; after re-initialising the workspace the same session synchronises
+    normally again and a fresh session produces the tokens of an undisturbed run."""
+    from ohara_amd.llama import Config, Llama
+
+    kw = dict(vocab_size=512, hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+              num_hidden_layers=3, max_sequence_length=96, rope_theta=10000.0)
+    w = R.init_weights(R.RefConfig(**kw), seed=3, dtype=torch.bfloat16, std=0.06, norm_jitter=0.1)
+    model = Llama(Config(**kw), w, device=cuda)
+    if not model.supports_persistent(2):
+        pytest.skip("shape not covered by the persistent kernel")
+    prompt = torch.randint(0, 512, (2, 12), generator=torch.Generator().manual_seed(0)).to(cuda)
+    good = model.generate_greedy(prompt, 10, persistent=True).cpu()
+
+    sess = model.session(2, 16, persistent=True)
+    sess.prefill(prompt)
+    sess.spin_limit = 1
+    for _ in range(3):
+        sess.step()
+    torch.cuda.synchronize()
+    with pytest.raises(RuntimeError, match="barrier wait expired"):
+        sess.check_error()
+    sess.spin_limit = 0
+    sess.reset_error()
+    sess.step()
+    torch.cuda.synchronize()
+    sess.check_error()
+    again = model.generate_greedy(prompt, 10, persistent=True).cpu()
+    assert torch.equal(again, good)
