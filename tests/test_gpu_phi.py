@@ -262,3 +262,17 @@ def test_block_head_matches_the_separate_kernels(cuda):
             assert diff.max().item() <= 2.0 ** -6 * scale, (name, B, d, diff.max().item(), scale)
             assert (diff > 0).float().mean().item() < 0.02, (name, B, d, (diff > 0).float().mean().item())
         assert torch.equal(kc[:, :pos], torch.zeros_like(kc[:, :pos])) and torch.equal(kc[:, pos + S:], torch.zeros_like(kc[:, pos + S:]))
+
+
+@pytest.mark.parametrize("B", [5, 20, 70])
+def test_decode_batches_of_several_row_groups(cuda, B):
+    """More than 16 rows (several row groups per weight strip) and more than 64 (the tiled kernel
+    also serves single-token calls): prefill and cached steps against the oracle."""
+    ref, model = _pair(cuda, vocab_size=256, max_sequence_length=32, hidden_size=128, num_attention_heads=4,
+                       num_hidden_layers=2)
+    ids = torch.randint(0, 256, (B, 7), generator=torch.Generator().manual_seed(B))
+    rc, cache = ref.build_kv_cache(B), model.build_kv_cache(B)
+    _close(model(ids[:, :4].to(cuda), cache, 0), ref(ids[:, :4], rc, 0))
+    for t in (4, 5, 6):
+        _close(model(ids[:, t:t + 1].to(cuda), cache, t), ref(ids[:, t:t + 1], rc, t))
+    _close(cache[0].value[:B, :7], rc[0].value[:B, :7])
