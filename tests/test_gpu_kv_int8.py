@@ -251,3 +251,20 @@ def test_int8_cache_mode_errors(cuda):
         model(torch.zeros(1, 2, dtype=torch.int64), mixed, 0)
     sess = model.session(1, 4, kv_cache=model.build_kv_cache(1, int8=True), persistent=None)
     assert sess.persistent is False
+
+
+@pytest.mark.parametrize("B", [9, 33, 70])
+def test_int8_cache_decode_at_larger_batches(cuda, B):
+    """int8 caches with more than 16 and more than 64 sequences: prefill and cached steps against the
+    oracle's int8 caches."""
+    from ohara_amd.llama import Llama
+
+    rcfg, cfg = _cfg_pair(vocab_size=512, hidden_size=256, intermediate_size=512, num_attention_heads=4,
+                          num_key_value_heads=2, num_hidden_layers=2, max_sequence_length=64, rope_theta=10000.0)
+    w = R.init_weights(rcfg, seed=8, dtype=BF, std=0.06, norm_jitter=0.1)
+    ref, model = R.RefLlama(rcfg, w), Llama(cfg, w, device=cuda)
+    ids = torch.randint(0, 512, (B, 8), generator=torch.Generator().manual_seed(B))
+    rc, cache = ref.build_kv_cache(B, int8=True), model.build_kv_cache(B, int8=True)
+    _close(model(ids[:, :5].to(cuda), cache, 0), ref(ids[:, :5], rc, 0), 4e-2, 4e-3)
+    for t in (5, 6, 7):
+        _close(model(ids[:, t:t + 1].to(cuda), cache, t), ref(ids[:, t:t + 1], rc, t), 4e-2, 4e-3)
