@@ -193,3 +193,33 @@ def test_continuous_batching_with_sampling_runs(cuda):
     for _ in range(5):
         seen.extend(bat.step().values())
     assert all(0 <= t < 500 for t in seen) and bat.lengths == [8, 45]
+
+
+@pytest.mark.parametrize("B", [20, 70])
+def test_ragged_decode_at_larger_batches(cuda, B):
+    """One position per sequence with more than 16 and more than 64 sequences: every sequence is
+    prefilled alone to its own length, then the whole batch decodes together; the oracle runs sequence
+    by sequence."""
+    ref, model = _small_model(cuda)
+    g = torch.Generator().manual_seed(B)
+    lens = torch.randint(1, 40, (B,), generator=g).tolist()
+    prompts = [torch.randint(0, 512, (1, n), generator=g) for n in lens]
+    cache = model.build_kv_cache(B)
+    for c in cache:
+        c._commit_ragged(B, [0] * B)
+    rcaches = [ref.build_kv_cache(1) for _ in range(B)]
+    last = []
+    for b, p in enumerate(prompts):
+        model(p.to(cuda), [c._row_view(b) for c in cache], 0)
+        last.append(ref(p, rcaches[b], 0)[:, -1])
+        for c in cache:
+            c.lengths[b] = lens[b]
+            c.length = max(c.lengths)
+    pos = list(lens)
+    nxt = torch.stack([w.float().argmax(-1) for w in last]).view(B, 1)
+    for step in range(3):
+        got = model(nxt.to(cuda), cache, pos)
+        want = torch.cat([ref(nxt[b:b + 1], rcaches[b], pos[b]) for b in range(B)])
+        _close(got, want)
+        pos = [p + 1 for p in pos]
+        nxt = want[:, -1].float().argmax(-1).view(B, 1)
