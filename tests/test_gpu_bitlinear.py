@@ -183,3 +183,29 @@ def test_fused_groups_match_the_separate_calls(cuda):
     a1 = ops.silu_mul(ops.bitlinear(x, pg[0], pg[1], pre_norm_w=pre), ops.bitlinear(x, pu[0], pu[1], pre_norm_w=pre))
     a2 = ops.bitlinear_gate_up(x, pre, pg, pu)
     assert torch.equal(a1, a2)
+
+
+@pytest.mark.parametrize("B", [9, 20, 70])
+def test_bitnet_decode_at_larger_batches(cuda, B):
+    """The ternary model with more than 8, more than 16 and more than 64 sequences (the last takes
+    the unfused projection path for single-token calls too): prefill and cached steps against the
+    oracle."""
+    from ohara_amd.bitnet import BitLlama
+    from ohara_amd.llama import Config
+
+    kw = dict(vocab_size=320, hidden_size=256, intermediate_size=512, num_attention_heads=2,
+              num_key_value_heads=0, num_hidden_layers=2, max_sequence_length=32, rope_theta=10000.0)
+    rcfg = R.RefConfig(**kw)
+    w = BL.init_ternary_weights(rcfg, seed=5, dtype=BF, gamma=0.05)
+    ref, model = R.RefLlama(rcfg, w), BitLlama(Config(**kw), w, device=cuda)
+    ids = torch.randint(0, 320, (B, 8), generator=torch.Generator().manual_seed(B))
+    rc, cache = ref.build_kv_cache(B), model.build_kv_cache(B)
+
+    def close(a, b):
+        scale = b.float().abs().max().item()
+        d = (a.float().cpu() - b.float()).abs()
+        assert d.max().item() <= 8e-2 * scale and d.mean().item() <= 1e-2 * scale, (B, d.max().item(), d.mean().item(), scale)
+
+    close(model(ids[:, :5].to(cuda), cache, 0), ref(ids[:, :5], rc, 0))
+    for t in (5, 6, 7):
+        close(model(ids[:, t:t + 1].to(cuda), cache, t), ref(ids[:, t:t + 1], rc, t))
