@@ -384,3 +384,26 @@ def test_decode_batches_between_and_beyond_the_tuned_sizes(cuda, B):
     want = greedy_decode_ref(ref, ids[:, :5], 3)
     # a near-tie of this random model flips a token now and then, and the sequence then differs from there on
     assert (toks == want).float().mean().item() >= 0.9
+
+
+@pytest.mark.parametrize("heads,kv_heads,hidden", [(4, 4, 256), (8, 2, 512), (4, 2, 512), (4, 1, 512), (2, 2, 256)])
+def test_every_persistent_kernel_variant_against_the_oracle(cuda, heads, kv_heads, hidden):
+    """Head widths 64 / 128 with 1, 2 and 4 query heads per KV head: the single-launch decode step
+    (free-running greedy tokens, then teacher-forced logits through the chain) against the oracle,
+    and the single launch against the kernel chain token for token up to a near-tie."""
+    from ohara_amd.llama import Llama
+
+    rcfg, cfg = _cfg_pair(vocab_size=512, hidden_size=hidden, intermediate_size=512, num_attention_heads=heads,
+                          num_key_value_heads=kv_heads, num_hidden_layers=3, max_sequence_length=128, rope_theta=10000.0)
+    w = R.init_weights(rcfg, seed=heads * 10 + kv_heads, dtype=BF, std=0.05, norm_jitter=0.1)
+    ref, model = R.RefLlama(rcfg, w), Llama(cfg, w, device=cuda)
+    assert model.supports_persistent(3) and model.head_dim in (64, 128)
+    prompt = torch.randint(0, 512, (3, 21), generator=torch.Generator().manual_seed(heads))
+    want, want_logits = greedy_decode_ref(ref, prompt, 24, return_logits=True)
+    for persistent in (True, False):
+        got = model.generate_greedy(prompt.to(cuda), 24, persistent=persistent).cpu()
+        for b in range(3):
+            neq = (got[b] != want[b]).nonzero()
+            if neq.numel():
+                t = int(neq[0])
+                assert _near_tie(want_logits[t, b], int(got[b, t]), int(want[b, t])), (persistent, b, t)
