@@ -407,3 +407,24 @@ def test_every_persistent_kernel_variant_against_the_oracle(cuda, heads, kv_head
             if neq.numel():
                 t = int(neq[0])
                 assert _near_tie(want_logits[t, b], int(got[b, t]), int(want[b, t])), (persistent, b, t)
+
+
+@pytest.mark.parametrize("B", [5, 12, 16])
+def test_persistent_kernel_at_batches_up_to_its_limit(cuda, B):
+    """The single launch is the default up to 8 sequences and can be asked for up to 16: greedy
+    tokens against the oracle (first divergence only at a near-tie)."""
+    from ohara_amd.llama import Llama
+
+    rcfg, cfg = _cfg_pair(vocab_size=512, hidden_size=256, intermediate_size=512, num_attention_heads=4,
+                          num_key_value_heads=2, num_hidden_layers=2, max_sequence_length=96, rope_theta=10000.0)
+    w = R.init_weights(rcfg, seed=12, dtype=BF, std=0.05, norm_jitter=0.1)
+    ref, model = R.RefLlama(rcfg, w), Llama(cfg, w, device=cuda)
+    assert model.supports_persistent(B) and not model.supports_persistent(17)
+    prompt = torch.randint(0, 512, (B, 30), generator=torch.Generator().manual_seed(B))
+    want, want_logits = greedy_decode_ref(ref, prompt, 16, return_logits=True)
+    got = model.generate_greedy(prompt.to(cuda), 16, persistent=True).cpu()
+    for b in range(B):
+        neq = (got[b] != want[b]).nonzero()
+        if neq.numel():
+            t = int(neq[0])
+            assert _near_tie(want_logits[t, b], int(got[b, t]), int(want[b, t])), (b, t)
