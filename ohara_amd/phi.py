@@ -8,8 +8,8 @@ layout, and the cache holds the UN-rotated keys: the rotation is applied to all 
 every step, in fp32, inside the attention kernel (phi.py:95-104).
 
 bf16 only (the reference's ``from_pretrained`` builds an fp16 model, phi.py:229-231; its tests run
-fp32).  Checkpoint download (phi.py:226-256) is not provided: pass a state dict with the reference's
-names (``Phi._huggingface_state_dict_map`` keys).
+fp32).  The Hub download of ``from_pretrained`` (phi.py:239) is not provided; a checkpoint already on
+disk loads through ``Phi.from_local_checkpoint`` (same name mapping, same errors).
 """
 
 from __future__ import annotations
@@ -50,6 +50,49 @@ def rope_cos_sin(num_positions: int, dims: int, base: float = 10000.0):
     freqs = torch.exp(-torch.arange(0.0, half, dtype=torch.float32) * (math.log(base) / half))
     theta = positions.reshape(-1, 1) * freqs.reshape(1, -1)
     return torch.cos(theta), torch.sin(theta)
+
+
+def huggingface_state_dict_map(num_hidden_layers: int) -> dict:
+    """Reference parameter name -> microsoft/phi-2 checkpoint name
+    (``Phi._huggingface_state_dict_map``, ohara/models/phi.py:208-233)."""
+    mapping = {
+        "wte.weight": "model.embed_tokens.weight",
+        "ln.weight": "model.final_layernorm.weight",
+        "ln.bias": "model.final_layernorm.bias",
+        "lm_head.weight": "lm_head.weight",
+        "lm_head.bias": "lm_head.bias",
+    }
+    for idx in range(num_hidden_layers):
+        for suffix in ("weight", "bias"):
+            mapping[f"layers.{idx}.ln.{suffix}"] = f"model.layers.{idx}.input_layernorm.{suffix}"
+            for name in ("fc1", "fc2"):
+                mapping[f"layers.{idx}.mlp.{name}.{suffix}"] = f"model.layers.{idx}.mlp.{name}.{suffix}"
+            for name in ("q_proj", "k_proj", "v_proj", "dense"):
+                mapping[f"layers.{idx}.mixer.{name}.{suffix}"] = f"model.layers.{idx}.self_attn.{name}.{suffix}"
+    return mapping
+
+
+def load_huggingface_state_dict(path: str, num_hidden_layers: int) -> dict:
+    """Read the ``*.safetensors`` shards of a microsoft/phi-2 style checkpoint in the local directory
+    ``path`` and return a state dict under the reference's names: what ``Phi.from_pretrained`` does
+    after its download (ohara/models/phi.py:239-256), with the same error for an empty directory and
+    for missing tensors.  Nothing is fetched from the network."""
+    from pathlib import Path
+
+    from safetensors import safe_open
+
+    weights = {}
+    for shard in sorted(Path(path).glob("*.safetensors")):
+        with safe_open(str(shard), framework="pt", device="cpu") as reader:
+            for key in reader.keys():
+                weights[key] = reader.get_tensor(key)
+    if not weights:
+        raise FileNotFoundError(f"no safetensors shards found in {path}")
+    mapping = huggingface_state_dict_map(num_hidden_layers)
+    missing = sorted(set(mapping.values()) - set(weights))
+    if missing:
+        raise KeyError(f"checkpoint is missing expected tensors: {missing[:5]}")
+    return {ours: weights[theirs] for ours, theirs in mapping.items()}
 
 
 class Phi:
@@ -105,6 +148,14 @@ class Phi:
 
     def eval(self):
         return self
+
+    @classmethod
+    def from_local_checkpoint(cls, path: str, config: PhiConfig | None = None, device="cuda") -> "Phi":
+        """``Phi.from_pretrained`` (ohara/models/phi.py:235-256) for a checkpoint that is already on
+        disk: the safetensors shards in ``path`` under microsoft/phi-2's tensor names, cast to bf16
+        (the reference builds an fp16 model)."""
+        config = config or PhiConfig()
+        return cls(config, load_huggingface_state_dict(path, config.num_hidden_layers), device=device)
 
     def build_kv_cache(self, batch_size: int = 1) -> list[KVCache]:
         if batch_size < 1:

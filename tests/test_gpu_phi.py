@@ -276,3 +276,20 @@ def test_decode_batches_of_several_row_groups(cuda, B):
     for t in (4, 5, 6):
         _close(model(ids[:, t:t + 1].to(cuda), cache, t), ref(ids[:, t:t + 1], rc, t))
     _close(cache[0].value[:B, :7], rc[0].value[:B, :7])
+
+
+def test_model_from_local_checkpoint_shards(cuda, tmp_path):
+    """Phi.from_local_checkpoint: safetensors shards under microsoft/phi-2's tensor names
+    (ohara/models/phi.py:208-256) -> the same logits as the model built from the state dict."""
+    from safetensors.torch import save_file
+
+    from ohara_amd.phi import Phi, PhiConfig, huggingface_state_dict_map
+
+    kw = dict(vocab_size=64, max_sequence_length=16, hidden_size=64, num_attention_heads=4, num_hidden_layers=2)
+    w = P.init_weights(P.RefPhiConfig(**kw), seed=6, dtype=BF, std=0.08, bias_std=0.05)
+    mapping = huggingface_state_dict_map(2)
+    save_file({mapping[k]: v.contiguous() for k, v in w.items()}, str(tmp_path / "model.safetensors"))
+    a = Phi.from_local_checkpoint(str(tmp_path), PhiConfig(**kw), device=cuda)
+    b = Phi(PhiConfig(**kw), w, device=cuda)
+    ids = torch.randint(0, 64, (2, 6), generator=torch.Generator().manual_seed(0)).to(cuda)
+    assert torch.equal(a(ids), b(ids))

@@ -314,3 +314,36 @@ def test_phi_host_side_tables_and_validation():
         Phi(PhiConfig(hidden_size=48, num_attention_heads=4), {}, device="cpu")
     with pytest.raises(ValueError, match="bfloat16"):
         Phi(PhiConfig(), {}, device="cpu", dtype=torch.float16)
+
+
+def test_phi_checkpoint_name_mapping_and_local_shards(tmp_path):
+    """The microsoft/phi-2 name mapping of the reference (ohara/models/phi.py:208-233) and the loader of
+    local safetensors shards: every reference name is produced, tensors come back under the right
+    names, an empty directory and a missing tensor raise the reference's errors."""
+    import torch
+    from safetensors.torch import save_file
+
+    from ohara_amd.phi import huggingface_state_dict_map, load_huggingface_state_dict
+    from oracle import phi_ref as P
+
+    cfg = P.RefPhiConfig(vocab_size=32, hidden_size=16, num_attention_heads=2, num_hidden_layers=2, max_sequence_length=8)
+    mapping = huggingface_state_dict_map(2)
+    assert set(mapping) == set(P.weight_names(cfg))
+    assert mapping["layers.1.mixer.dense.bias"] == "model.layers.1.self_attn.dense.bias"
+    assert mapping["layers.0.ln.weight"] == "model.layers.0.input_layernorm.weight"
+    assert mapping["wte.weight"] == "model.embed_tokens.weight" and mapping["ln.bias"] == "model.final_layernorm.bias"
+    assert len(set(mapping.values())) == len(mapping)
+
+    w = P.init_weights(cfg, seed=1)
+    hf = {mapping[k]: v.contiguous() for k, v in w.items()}
+    names = sorted(hf)
+    save_file({k: hf[k] for k in names[::2]}, str(tmp_path / "model-00001-of-00002.safetensors"))
+    save_file({k: hf[k] for k in names[1::2]}, str(tmp_path / "model-00002-of-00002.safetensors"))
+    back = load_huggingface_state_dict(str(tmp_path), 2)
+    assert set(back) == set(w) and all(torch.equal(back[k], w[k]) for k in w)
+    empty = tmp_path / "empty"
+    empty.mkdir()
+    with pytest.raises(FileNotFoundError, match="no safetensors shards"):
+        load_huggingface_state_dict(str(empty), 2)
+    with pytest.raises(KeyError, match="missing expected tensors"):
+        load_huggingface_state_dict(str(tmp_path), 3)
