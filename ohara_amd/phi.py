@@ -146,7 +146,12 @@ class Phi:
         torch.cuda.synchronize(self.device)
         self._bufs: dict = {}
 
+    supports_last_only = True  # forward(..., last_only=True) computes the last row of logits only
+
     def eval(self):
+        return self
+
+    def to(self, *args, **kwargs):
         return self
 
     @classmethod

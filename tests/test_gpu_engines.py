@@ -117,3 +117,51 @@ def test_chat_engine_from_checkpoint(cuda, tmp_path):
     torch.save(small, tmp_path / "small.pt")
     with pytest.raises(ValueError, match="smaller than the"):
         ChatEngine.from_checkpoint(tmp_path / "small.pt", tok)
+
+
+def test_inference_drives_phi_as_the_reference_example_does(cuda):
+    """examples/phi_inference.py: Inference(model, tokenizer, device, use_kv_cache) over Phi, with and
+    without the cache; greedy text equals the oracle's greedy continuation."""
+    from ohara_amd.inference import Inference
+    from ohara_amd.phi import Phi, PhiConfig
+    from oracle import phi_ref as P
+
+    tok = CharTokenizer()
+
+    class Tok:
+        eos_token_id = 0
+
+        def encode(self, text):
+            return tok.encode(text)
+
+        def decode(self, ids):
+            return tok.decode(ids, skip_special_tokens=False)
+
+    V = (len(tok) + 3) // 4 * 4  # the vocabulary projection wants a multiple of four rows
+    kw = dict(vocab_size=V, max_sequence_length=32, hidden_size=64, num_attention_heads=4, num_hidden_layers=2)
+    rcfg = P.RefPhiConfig(**kw)
+    w = P.init_weights(rcfg, seed=3, dtype=BF, std=0.1, bias_std=0.05)
+    w["lm_head.bias"][len(tok):] = -30.0  # padded ids are never chosen
+    for name, i in tok.vocab.items():     # nor the special tokens (end of text among them): the run fills
+        if len(name) > 1 or i == 0:       # its token budget with one character per token
+            w["lm_head.bias"][i] = -30.0
+    ref, model = P.RefPhi(rcfg, w), Phi(PhiConfig(**kw), w, device=cuda)
+    ids = torch.tensor([tok.encode("hello")])
+    rc, pos, inp, out = ref.build_kv_cache(1), 0, ids, []
+    logits_seen = []
+    for _ in range(8):
+        lg = ref(inp, rc, pos)[:, -1]
+        pos += inp.size(1)
+        logits_seen.append(lg[0])
+        inp = lg.float().argmax(-1, keepdim=True)
+        out.append(int(inp))
+    for use_cache in (True, False):
+        inf = Inference(model, Tok(), cuda, use_kv_cache=use_cache)
+        text = inf.generate("hello", temperature=0.0, max_new_tokens=8, stream=False)
+        assert text.startswith("hello") and len(text) == 5 + 8
+        got = tok.encode(text)[5:]
+        for t, (g_, w_) in enumerate(zip(got, out)):
+            if g_ != w_:  # first divergence only at a near-tie of the oracle's own logits
+                la, lb = logits_seen[t][g_].float().item(), logits_seen[t][w_].float().item()
+                assert abs(la - lb) <= 2.0 ** -6 * max(abs(la), abs(lb), 1e-3), (use_cache, t)
+                break
