@@ -401,9 +401,9 @@ int64_t ohara_persistent_error_offset(const OharaModel* m, int batch, int n_spli
 int64_t ohara_persistent_profile_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
 
 /* ---- Phi (ohara/models/phi.py): the parts of its cached decode path that differ from Llama ----
- * nn.Linear WITH bias on packed weights (phi.py:46-47, :63-66, :161), any number of rows (up to 64:
- * the weight-streaming strip kernel; more: the tiled MFMA kernel of ohara_gemm_bf16, same epilogues
- * and rounding points).  n % 4 == 0, k % 8 == 0.
+ * nn.Linear WITH bias on packed weights (phi.py:46-47, :63-66, :161), any number of rows (up to 128:
+ * the weight-streaming strip kernel, 64 rows per pass; more: the tiled MFMA kernel of ohara_gemm_bf16,
+ * same epilogues and rounding points).  n % 4 == 0, k % 8 == 0.
  *   OHARA_LIN_BIAS       out = bf16(x @ W^T + bias)
  *   OHARA_LIN_BIAS_GELU  out = new_gelu(bf16(x @ W^T + bias)), every op of phi.py:37-40 rounded to
  *                        bf16 as the eager ops round                          (MLP.fc1, phi.py:50-51)
@@ -446,7 +446,9 @@ int ohara_kv_append_bf16(const uint16_t* k, const uint16_t* v, int ld, int batch
  * dh % 8 == 0, dh <= 128.  n_split > 1 (seq_len 1 only, at most 64) spreads the context of every
  * (sequence, head) over that many workgroups whose partial results meet in `workspace`
  * (ohara_phi_attn_workspace_bytes, zero-filled once before the first use; calls sharing it must not
- * overlap) and are merged in chunk order by the workgroup that finishes last. */
+ * overlap) and are merged in chunk order by the workgroup that finishes last.  Calls with 16 or more
+ * new tokens per sequence (prefill; head widths 16, 32, 64, 80, 128) run queries in tiles of 64
+ * against key / value tiles in LDS with fp32 matrix products; other shapes one query per workgroup. */
 int64_t ohara_phi_attn_workspace_bytes(int batch, int h, int dh, int n_split);
 int ohara_phi_attn_bf16(const uint16_t* q, int ldq, const uint16_t* kcache, const uint16_t* vcache, const float* cos,
                         const float* sin, int rot, int batch, int seq_len, int h, int dh, int t_max, int pos,

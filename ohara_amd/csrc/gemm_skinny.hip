@@ -518,7 +518,10 @@ int ohara_linear_bias_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int n
   a.B = rows; a.N = n; a.K = k;
   a.out = out; a.ldo = ldo; a.bias = bias;
   a.resid = add1; a.ldr = ld1; a.resid2 = add2; a.ldr2 = ld2;
-  if (rows > 64) return ohara_launch_gemm_tile(a, epi, (n + 15) / 16 * 16, (hipStream_t)stream);  // prefill
+  // Many rows (prefill) go to the tiled kernel.  Up to 128 rows it would run N / 128 workgroups only;
+  // two passes of the weight-streaming kernel over 64 rows each measured faster there (Phi-2 widths,
+  // 128 rows: fc2 89 against 171 us, dense 26 against 49 us).
+  if (rows > 128) return ohara_launch_gemm_tile(a, epi, (n + 15) / 16 * 16, (hipStream_t)stream);
   return launch_skinny(a, epi, (n + 15) / 16 * 16, (hipStream_t)stream);
 }
 
@@ -538,7 +541,7 @@ int ohara_phi_block_in_bf16(const uint16_t* x, int ldx, const uint16_t* ln_w, co
   a.B = batch * seq_len; a.N = 3 * d + ff; a.K = d;
   a.out = q; a.ldo = ldq; a.out2 = act; a.ldo2 = ldact; a.split_n = 3 * d; a.bias = bias;
   a.S = seq_len; a.Tmax = t_max; a.pos = pos; a.pos_dev = pos_dev; a.kcache = kcache; a.vcache = vcache;
-  if (a.B > 64 && !ln_w) return ohara_launch_gemm_tile(a, EPI_PHI_IN, (a.N + 15) / 16 * 16, (hipStream_t)stream);  // prefill
+  if (a.B > 128 && !ln_w) return ohara_launch_gemm_tile(a, EPI_PHI_IN, (a.N + 15) / 16 * 16, (hipStream_t)stream);  // prefill
   return launch_skinny(a, EPI_PHI_IN, (a.N + 15) / 16 * 16, (hipStream_t)stream);
 }
 

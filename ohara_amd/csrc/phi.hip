@@ -300,6 +300,160 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
   }
 }
 
+// ---- attention over many new tokens (prefill) -----------------------------------------------
+// One workgroup per (sequence, head, 64 queries); each of its four waves owns 16 queries.  Keys
+// and values go through LDS in tiles of 32 positions, as fp32, the keys rotated there once per
+// tile; scores and the weighted sum are fp32 matrix products (v_mfma_f32_16x16x4_f32), the same
+// arithmetic type the reference uses (phi.py:98-117).  Both products are formed transposed,
+//   S^T (position x query) = K . Q^T        O^T (feature x query) = V^T . P^T,
+// so that a lane's four score registers are rows 4g .. 4g+3 of one query column: the softmax
+// runs down registers plus two cross-group shuffles, and register r is already the B operand of
+// the second product's k-step r (the A operand then reads value row 4g + r).
+constexpr int PF_Q = 64, PF_T = 32;
+
+template <int DT>  // head width / 16
+__global__ __launch_bounds__(256) void phi_attn_prefill_kernel(PhiAttnArgs a) {
+  constexpr int D = 16 * DT, LD = D + 4, NV = (PF_T * (D / 8) + 255) / 256;
+  __shared__ float sm[2 * PF_T * LD];  // keys | values of a tile; the rotated queries before the loop
+  float* ks = sm;
+  float* vs = sm + PF_T * LD;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l16 = lane & 15, g = lane >> 4;
+  const int half = a.rot >> 1;
+  const int h = blockIdx.y, seq = blockIdx.z;
+  const int s0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * PF_Q;  // long contexts first
+  const size_t hd = (size_t)a.H * D;
+  const int pos0 = a.pos;
+
+  // rotated queries -> LDS -> registers (phi.py:103; rows beyond the call's tokens are zero)
+  for (int idx = tid; idx < PF_Q * D; idx += 256) {
+    const int qi = idx / D, j = idx - qi * D;
+    const int sq = s0 + qi;
+    float v = 0.f;
+    if (sq < a.S) {
+      const bf16_t* qrow = a.q + ((size_t)seq * a.S + sq) * a.ldq + h * D;
+      const size_t cb = (size_t)(pos0 + sq) * half;
+      v = bf2f(qrow[j]);
+      if (j < half) v = v * a.cos[cb + j] - bf2f(qrow[j + half]) * a.sin[cb + j];
+      else if (j < a.rot) v = bf2f(qrow[j - half]) * a.sin[cb + j - half] + v * a.cos[cb + j - half];
+    }
+    sm[qi * LD + j] = v;
+  }
+  __syncthreads();
+  float qreg[D / 4];
+#pragma unroll
+  for (int kk = 0; kk < D / 4; ++kk) qreg[kk] = sm[(16 * wave + l16) * LD + 4 * kk + g];
+  __syncthreads();
+
+  // this lane's query column; columns beyond the call's tokens repeat the last one and are not stored
+  const int sq = min(s0 + 16 * wave + l16, a.S - 1);
+  const int pq = pos0 + sq;
+  const int wave_hi = pos0 + min(s0 + 16 * wave + 15, a.S - 1);  // last position any query of the wave sees
+  const int t_end = pos0 + min(s0 + PF_Q - 1, a.S - 1);
+  const float scale = sqrtf(1.0f / (float)D);
+  const bf16_t* kb = a.kc + (size_t)seq * a.t_max * hd + (size_t)h * D;
+  const bf16_t* vb = a.vc + (size_t)seq * a.t_max * hd + (size_t)h * D;
+
+  f32x4 o[DT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t) o[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, lsum = 0.f;
+
+  uint4 kr[NV], vr[NV];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int idx = tid + 256 * i;
+      const int p = idx / (D / 8), c = idx - p * (D / 8);
+      const bool in = idx < PF_T * (D / 8) && t0 + p <= t_end;
+      kr[i] = in ? ldg16(kb + (size_t)(t0 + p) * hd + 8 * c) : make_uint4(0, 0, 0, 0);
+      vr[i] = in ? ldg16(vb + (size_t)(t0 + p) * hd + 8 * c) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto put8 = [](float* dst, uint4 v) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      dst[2 * i] = lo_bf(w[i]);
+      dst[2 * i + 1] = hi_bf(w[i]);
+    }
+  };
+
+  fetch(0);
+  for (int t0 = 0; t0 <= t_end; t0 += PF_T) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int idx = tid + 256 * i;
+      if (idx < PF_T * (D / 8)) {
+        const int p = idx / (D / 8), c = idx - p * (D / 8);
+        put8(ks + p * LD + 8 * c, kr[i]);
+        put8(vs + p * LD + 8 * c, vr[i]);
+      }
+    }
+    __syncthreads();
+    if (t0 + PF_T <= t_end) fetch(t0 + PF_T);  // in flight during this tile's products
+    // rotate the tile's keys in place (phi.py:104): pair (i, i + half) of every position
+    for (int idx = tid; idx < PF_T * half; idx += 256) {
+      const int p = idx / half, i = idx - p * half;
+      if (t0 + p <= t_end) {
+        const float c = a.cos[(size_t)(t0 + p) * half + i], sn = a.sin[(size_t)(t0 + p) * half + i];
+        const float k1 = ks[p * LD + i], k2 = ks[p * LD + i + half];
+        ks[p * LD + i] = k1 * c - k2 * sn;
+        ks[p * LD + i + half] = k1 * sn + k2 * c;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int blk = 0; blk < PF_T / 16; ++blk) {
+      const int tb = t0 + 16 * blk;
+      if (tb > wave_hi) break;  // wave-uniform: nothing in this block is visible to the wave's queries
+      f32x4 sc = (f32x4){0.f, 0.f, 0.f, 0.f};
+      const float* krow = ks + (16 * blk + l16) * LD + g;
+#pragma unroll
+      for (int kk = 0; kk < D / 4; ++kk) sc = __builtin_amdgcn_mfma_f32_16x16x4f32(krow[4 * kk], qreg[kk], sc, 0, 0, 0);
+      float mx = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        sc[r] = tb + 4 * g + r <= pq ? sc[r] * scale : -INFINITY;
+        mx = fmaxf(mx, sc[r]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+      const float mn = fmaxf(m, mx);  // finite: position 0 is in the first block and visible to every query
+      const float corr = __expf(m - mn);
+      float ps = 0.f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        sc[r] = __expf(sc[r] - mn);
+        ps += sc[r];
+      }
+      lsum = lsum * corr + ps;
+      m = mn;
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[t][r] *= corr;
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const float* vrow = vs + (16 * blk + 4 * g + kk) * LD + l16;
+#pragma unroll
+        for (int t = 0; t < DT; ++t) o[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(vrow[16 * t], sc[kk], o[t], 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+  lsum += __shfl_xor(lsum, 16, WAVE);
+  lsum += __shfl_xor(lsum, 32, WAVE);
+  if (s0 + 16 * wave + l16 < a.S) {
+    const float inv = 1.0f / lsum;
+    bf16_t* orow = a.out + ((size_t)seq * a.S + sq) * hd + (size_t)h * D + 4 * g;
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+      *reinterpret_cast<uint2*>(orow + 16 * t) =
+          make_uint2(pack_bf(o[t][0] * inv, o[t][1] * inv), pack_bf(o[t][2] * inv, o[t][3] * inv));
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -349,6 +503,19 @@ int ohara_phi_attn_bf16(const uint16_t* q, int ldq, const uint16_t* kcache, cons
   const size_t counters = (((size_t)batch * h * sizeof(int)) + 255) & ~(size_t)255;
   PhiAttnArgs a{q, ldq, kcache, vcache, cos, sin, out, seq_len, h, dh, rot, t_max, pos, pos_dev, n_split,
                 reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + counters), reinterpret_cast<int*>(workspace)};
+  if (seq_len >= 16 && !pos_dev && (dh == 16 || dh == 32 || dh == 64 || dh == 80 || dh == 128) && h <= 65535 &&
+      batch <= 65535) {
+    // many new tokens: queries in tiles of 64 against key / value tiles in LDS, fp32 matrix products
+    const dim3 pgrid((unsigned)((seq_len + PF_Q - 1) / PF_Q), (unsigned)h, (unsigned)batch);
+    switch (dh / 16) {
+      case 1: hipLaunchKernelGGL((phi_attn_prefill_kernel<1>), pgrid, dim3(256), 0, (hipStream_t)stream, a); break;
+      case 2: hipLaunchKernelGGL((phi_attn_prefill_kernel<2>), pgrid, dim3(256), 0, (hipStream_t)stream, a); break;
+      case 4: hipLaunchKernelGGL((phi_attn_prefill_kernel<4>), pgrid, dim3(256), 0, (hipStream_t)stream, a); break;
+      case 5: hipLaunchKernelGGL((phi_attn_prefill_kernel<5>), pgrid, dim3(256), 0, (hipStream_t)stream, a); break;
+      default: hipLaunchKernelGGL((phi_attn_prefill_kernel<8>), pgrid, dim3(256), 0, (hipStream_t)stream, a); break;
+    }
+    return ohara_launch_status();
+  }
   hipLaunchKernelGGL(phi_attn_kernel, dim3((unsigned)grid, (unsigned)n_split), dim3(256), 0, (hipStream_t)stream, a);
   return ohara_launch_status();
 }

@@ -40,7 +40,8 @@ def test_linear_bias_epilogues(cuda):
     from ohara_amd import ops
 
     g = torch.Generator().manual_seed(1)
-    for rows, n, k in ((1, 64, 64), (7, 320, 1280), (64, 1280, 320), (70, 96, 64), (3, 64, 2560), (20, 160, 10240)):
+    for rows, n, k in ((1, 64, 64), (7, 320, 1280), (64, 1280, 320), (70, 96, 64), (3, 64, 2560), (20, 160, 10240),
+                       (128, 96, 320), (130, 96, 64), (200, 320, 1280)):
         x = torch.randn(rows, k, generator=g).to(BF)
         w = (torch.randn(n, k, generator=g) / k ** 0.5).to(BF)
         b = (0.2 * torch.randn(n, generator=g)).to(BF)
@@ -76,7 +77,11 @@ def test_kv_append_and_attention_against_the_oracle(cuda):
 
     g = torch.Generator().manual_seed(2)
     for B, S, L0, H, D, rot, Tmax in ((2, 1, 9, 4, 16, 6, 32), (1, 5, 0, 2, 80, 32, 16), (3, 2, 30, 2, 128, 128, 40),
-                                      (1, 1, 0, 1, 8, 2, 4), (2, 1, 299, 2, 64, 24, 300)):
+                                      (1, 1, 0, 1, 8, 2, 4), (2, 1, 299, 2, 64, 24, 300),
+                                      # 16 tokens and more: query tiles of 64 against key tiles of 32
+                                      (2, 40, 0, 2, 80, 32, 64), (1, 100, 29, 2, 128, 128, 160), (3, 16, 5, 4, 16, 6, 32),
+                                      (1, 65, 0, 1, 64, 24, 80), (2, 33, 0, 2, 32, 16, 40), (1, 200, 0, 3, 80, 32, 200),
+                                      (1, 20, 3, 2, 48, 16, 32)):  # width 48: the one-query-per-workgroup kernel
         hd = H * D
         kc = torch.zeros(B, Tmax, H, D, dtype=BF)
         vc = torch.zeros(B, Tmax, H, D, dtype=BF)
@@ -232,7 +237,8 @@ def test_block_head_matches_the_separate_kernels(cuda):
 
     g = torch.Generator().manual_seed(4)
     for B, S, d, ff, H, pos in ((2, 3, 64, 256, 4, 5), (1, 1, 320, 1280, 4, 0), (3, 1, 2560, 10240, 32, 7),
-                                (70, 1, 64, 128, 2, 2), (2, 1, 2048, 128, 16, 1)):
+                                (70, 1, 64, 128, 2, 2), (2, 1, 2048, 128, 16, 1), (130, 1, 64, 128, 2, 2),
+                                (10, 10, 128, 512, 4, 2)):
         rows, D, Tmax = B * S, d // H, 16
         x = (torch.randn(rows, d, generator=g) + 0.3).to(BF).to(cuda)
         lw = (1 + 0.1 * torch.randn(d, generator=g)).to(BF).to(cuda)
@@ -264,10 +270,11 @@ def test_block_head_matches_the_separate_kernels(cuda):
         assert torch.equal(kc[:, :pos], torch.zeros_like(kc[:, :pos])) and torch.equal(kc[:, pos + S:], torch.zeros_like(kc[:, pos + S:]))
 
 
-@pytest.mark.parametrize("B", [5, 20, 70])
+@pytest.mark.parametrize("B", [5, 20, 70, 130])
 def test_decode_batches_of_several_row_groups(cuda, B):
-    """More than 16 rows (several row groups per weight strip) and more than 64 (the tiled kernel
-    also serves single-token calls): prefill and cached steps against the oracle."""
+    """More than 16 rows (several row groups per weight strip), more than 64 (two passes of the
+    weight-streaming kernel) and more than 128 (the tiled kernel also serves single-token calls):
+    prefill and cached steps against the oracle."""
     ref, model = _pair(cuda, vocab_size=256, max_sequence_length=32, hidden_size=128, num_attention_heads=4,
                        num_hidden_layers=2)
     ids = torch.randint(0, 256, (B, 7), generator=torch.Generator().manual_seed(B))
