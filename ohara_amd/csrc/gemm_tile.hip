@@ -83,16 +83,24 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(GemmArgs a, int MT, i
       load_x(s + 1, xr);
       load_w(s + 1, wn);
     }
+    // The eight B operands of a half step are read from LDS into registers of their own before its
+    // products.  (Left to itself the compiler reuses one register quad: read, wait, two products,
+    // sixteen times per step, every LDS latency exposed.  All sixteen up front would take the
+    // kernel from three workgroups per CU to two, which costs more than it gains.)
 #pragma unroll
     for (int jj = 0; jj < 2; ++jj) {
+      uint4 bv[8];
+#pragma unroll
+      for (int t = 0; t < 8; ++t) bv[t] = *reinterpret_cast<const uint4*>(&xs[buf][t * 16 + m][jj * 32 + 8 * g]);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
-        const uint4 bv = *reinterpret_cast<const uint4*>(&xs[buf][t * 16 + m][jj * 32 + 8 * g]);
         acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wv[jj]),
-                                                            __builtin_bit_cast(bf16x8, bv), acc[0][t], 0, 0, 0);
+                                                            __builtin_bit_cast(bf16x8, bv[t]), acc[0][t], 0, 0, 0);
         acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wv[2 + jj]),
-                                                            __builtin_bit_cast(bf16x8, bv), acc[1][t], 0, 0, 0);
+                                                            __builtin_bit_cast(bf16x8, bv[t]), acc[1][t], 0, 0, 0);
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
     if (more) {
       store_x(buf ^ 1, xr);
