@@ -530,14 +530,21 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
           for (int c = 0; c < PF; ++c)
             wv[c] = (jc + c < j1) ? ldg16_nt(wrow + (size_t)(jc + c) * 64) : make_uint4(0, 0, 0, 0);
         }
+        // The activations of all PF k-steps are read from LDS before the first product: they do not
+        // depend on the weights, and left next to their products every read's latency is exposed
+        // (read, wait, product, PF times) on the critical path of the phase.
+        uint4 xv[PF];
 #pragma unroll
         for (int c = 0; c < PF; ++c) {
-          uint4 xv = make_uint4(0, 0, 0, 0);
+          xv[c] = make_uint4(0, 0, 0, 0);
           if (mine && jc + c < j1 && 32 * (jc + c) + 8 * g < p.K)
-            xv = *reinterpret_cast<const uint4*>(xrow + 32 * (jc + c));
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wv[c]),
-                                                        __builtin_bit_cast(bf16x8, xv), acc, 0, 0, 0);
+            xv[c] = *reinterpret_cast<const uint4*>(xrow + 32 * (jc + c));
         }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < PF; ++c)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wv[c]),
+                                                        __builtin_bit_cast(bf16x8, xv[c]), acc, 0, 0, 0);
       }
     }
     if (it == 0) pf.stamp();  // MFMAs issued
