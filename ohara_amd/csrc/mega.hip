@@ -555,10 +555,15 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
       }
       __syncthreads();
       if (kpart == 0) {
+        // all partial tiles are read before the first add (same order of adds; the reads overlap)
+        f32x4 part[KP > 1 ? KP - 1 : 1];
+#pragma unroll
+        for (int w = 1; w < KP; ++w) part[w - 1] = *reinterpret_cast<const f32x4*>(red + (((wave + w) * 64) + lane) * 4);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int w = 1; w < KP; ++w)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) acc[i] += red[(((wave + w) * 64) + lane) * 4 + i];
+          for (int i = 0; i < 4; ++i) acc[i] += part[w - 1][i];
       }
     }
     if (it == 0) pf.stamp();  // cross-wave sum done
