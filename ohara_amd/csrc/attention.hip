@@ -100,12 +100,13 @@ __device__ void merge_partials(const AttnArgs& a, int b /* query row */, int kvh
 
 // Counts this workgroup's chunk as done and returns true in the workgroup that observes all
 // n_split chunks done (every thread gets the same answer).  The partials were written with
-// write-through stores; the workgroup-scope fence waits for their completion, the counter is a
-// relaxed device-scope atomic and the merge reads with cache-bypassing loads: no L2
-// write-back or invalidate.
+// write-through stores; every wave waits for the completion of its own before the workgroup
+// barrier, the counter is a relaxed device-scope atomic and the merge reads with
+// cache-bypassing loads: no L2 write-back or invalidate.
 __device__ bool last_chunk_done(int* counter, int nsplit) {
   __shared__ int is_last;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  wait_own_stores();
   __syncthreads();
   if (threadIdx.x == 0) {
     const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -80,9 +80,10 @@ __device__ __forceinline__ float wave_max(float v) {
 // Device-coherent accesses without fences.  The eight XCDs' L2 caches are not coherent with
 // each other; relaxed agent-scope atomics compile to write-through stores / cache-bypassing
 // loads (sc1), so data handed from one workgroup to another is published by such stores, a
-// wait for their completion (a workgroup-scope release fence) and a relaxed atomic counter,
-// and is read with such loads.  An agent-scope fence instead writes back / invalidates a whole
-// L2, which serialises across workgroups (~0.2 us each on this chip).
+// wait of EVERY storing wave for their completion (wait_own_stores below), a workgroup barrier
+// and then a relaxed atomic counter, and is read with such loads.  An agent-scope fence instead
+// writes back / invalidates a whole L2, which serialises across workgroups (~0.2 us each on
+// this chip).
 __device__ __forceinline__ void st_coh8(void* p, uint2 v) {
   __hip_atomic_store((OHARA_GLOBAL unsigned long long*)p, ((unsigned long long)v.y << 32) | v.x, __ATOMIC_RELAXED,
                      __HIP_MEMORY_SCOPE_AGENT);
@@ -101,6 +102,17 @@ __device__ __forceinline__ uint4 ld_coh16(const void* p) {
 }
 __device__ __forceinline__ uint32_t ld_coh4(const void* p) {
   return __hip_atomic_load((const OHARA_GLOBAL uint32_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Waits until every global store (and load) this wave has issued has completed: s_waitcnt
+// vmcnt(0) lgkmcnt(0).  A workgroup-scope release fence does NOT do this on gfx950 (the L1 keeps
+// a workgroup's accesses in order, so the fence emits no vmcnt wait): a wave that only passes the
+// workgroup barrier may still have write-through stores in flight when another wave bumps the
+// cross-workgroup counter.  So every wave calls this before that barrier.
+__device__ __forceinline__ void wait_own_stores() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0x0070);
+  asm volatile("" ::: "memory");
 }
 
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }

@@ -109,7 +109,8 @@ struct GridSync {
   }
   __device__ __forceinline__ void arrive(Prof& pf) {
     pf.stamp();  // phase work issued
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // my stores (LDS and sc1 global) have completed
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // orders my LDS and global accesses within the workgroup
+    wait_own_stores();  // every wave: its sc1 stores have reached memory before the barrier below
     pf.stamp();  // stores complete
     __builtin_amdgcn_s_barrier();
     pf.stamp();  // workgroup barrier passed

@@ -259,11 +259,12 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
   }
   if (a.ns == 1) return;
 
-  // The workgroup that finishes last merges the chunks of its (row, head), in chunk order.  The fence
-  // waits for this workgroup's write-through stores; the counter is a relaxed device-scope atomic; the
-  // merge reads with cache-bypassing loads.
+  // The workgroup that finishes last merges the chunks of its (row, head), in chunk order.  Every
+  // wave waits for its own write-through stores before the workgroup barrier; the counter is a
+  // relaxed device-scope atomic; the merge reads with cache-bypassing loads.
   __shared__ int is_last;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  wait_own_stores();
   __syncthreads();
   int* counter = a.counters + (size_t)row * a.H + h;
   if (tid == 0) {

@@ -502,6 +502,7 @@ class DecodeSession:
         self.pos = 0
         self.graph = None
         self._dst = None
+        self._dbuf = None
 
     def prefill(self, prompt_ids: torch.Tensor) -> None:
         m, B = self.model, self.batch
@@ -526,7 +527,12 @@ class DecodeSession:
         for cc in self.cache:
             cc._commit(B, P)
         self.pos = P
-        dbuf = m._get_buffers(B, B)
+        # the decode buffers (fed ids, step state, activations) belong to this session alone: their
+        # addresses are baked into the captured graph, so neither another session of the same batch
+        # nor an eager model(...) call may share them
+        dbuf = self._dbuf
+        if dbuf is None:
+            dbuf = _Buffers(m, B, B, m.default_n_split(B))
         self.history[0].copy_(pbuf.ids[:B])
         dbuf.ids.copy_(pbuf.ids[:B])
         dbuf.step_state.copy_(torch.tensor([P, 1, 0, 0], dtype=torch.int32))
