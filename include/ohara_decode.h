@@ -8,7 +8,8 @@
  *
  *   - plain C: raw device pointers, sizes, a hipStream_t passed as void*;
  *   - returns OHARA_OK (0) or a negative OHARA_E* code; never throws, never exits,
- *     never allocates or frees device memory, never synchronises the host;
+ *     never allocates or frees device memory, and does not synchronise the host (the one
+ *     exception is the one-time workspace set-up ohara_llama_decode_persistent(init_workspace=1));
  *   - all work is enqueued on `stream` and is stream-ordered, so every call can be
  *     recorded into a HIP graph;
  *   - bf16 tensors are passed as uint16_t* (raw bfloat16 bits), row-major;
@@ -145,6 +146,20 @@ int ohara_attn_cached_ragged_bf16(const uint16_t* q, const uint16_t* kcache, con
 /* seq_pos[b] += by for every b with active[b] != 0 (active NULL: all): advances a ragged batch by one
  * decode step without host involvement (graph replay). */
 int ohara_advance_positions(int32_t* seq_pos, const uint8_t* active, int batch, int by, void* stream);
+
+/* ohara_attn_cached_bf16 for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Same arguments minus the workspace: the chunk partials and counters live in a
+ * device array inside the library (8 MiB + 64 KiB, held by every GPU the library runs on until
+ * the process ends), so nothing is allocated or freed, by this library or through any other.
+ * Limits: batch*seq_len*h_kv <= 16384 and
+ *   align256(batch*seq_len*h*n_split*8) + align256(batch*seq_len*h*n_split*dh*4) <= 8 MiB;
+ * anything larger returns OHARA_ESIZE and launches nothing.  The first call on a device looks up
+ * the array's address (make it outside graph capture).  All calls on one GPU share the array:
+ * calls that overlap in time on one GPU (different streams) race; calls on one stream do not. */
+int ohara_attn_cached_bf16_noalloc(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch,
+                                   int seq_len, int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev,
+                                   int n_split, uint16_t* out, void* stream);
 
 /* Same contract for many query positions per sequence (prefill), as a causal flash-style kernel
  * on MFMA: 128 queries per workgroup, keys/values walked in 64-position tiles through LDS,

@@ -10,6 +10,8 @@
 // wavefront shuffle reductions.  Partial (max, sum, acc) triples of the chunks are
 // merged by whichever workgroup of the (sequence, KV head) finishes last, in chunk
 // order, so the result does not depend on scheduling.
+#include <mutex>
+
 #include "common.h"
 
 namespace {
@@ -480,10 +482,12 @@ int64_t ohara_attn_workspace_bytes(int batch, int h, int h_kv, int dh, int n_spl
   return (int64_t)(c + ml + acc);
 }
 
+// `fixed_counter_bytes` > 0: the workspace keeps its counters in a region of that fixed size (the
+// layout of the allocation-free entry point, whose array is shared by calls of different shapes).
 static int attn_cached_impl(const uint16_t* q, const void* kcache, const void* vcache, const float* kscale,
                             const float* kmin, const float* vscale, const float* vmin, bool i8, int batch, int seq_len,
                             int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev, int pos_stride, int n_split,
-                            void* workspace, uint16_t* out, void* stream) {
+                            void* workspace, uint16_t* out, void* stream, size_t fixed_counter_bytes = 0) {
   if (!q || !kcache || !vcache || !out) return OHARA_EINVAL;
   if (i8 && (!kscale || !kmin || !vscale || !vmin)) return OHARA_EINVAL;
   if (batch < 1 || seq_len < 1 || h < 1 || h_kv < 1 || h % h_kv || dh < 2 || (dh & 1) || dh > 256)
@@ -502,7 +506,7 @@ static int attn_cached_impl(const uint16_t* q, const void* kcache, const void* v
   batch *= seq_len;  // one workspace slot per query row
   char* ws = reinterpret_cast<char*>(workspace);
   a.counters = reinterpret_cast<int*>(ws);
-  ws += align256((size_t)batch * h_kv * sizeof(int));
+  ws += fixed_counter_bytes ? fixed_counter_bytes : align256((size_t)batch * h_kv * sizeof(int));
   a.part_ml = reinterpret_cast<float*>(ws);
   ws += align256((size_t)batch * h * n_split * 2 * sizeof(float));
   a.part_acc = reinterpret_cast<float*>(ws);
@@ -544,6 +548,60 @@ int ohara_attn_cached_int8(const uint16_t* q, const int8_t* kcache, const int8_t
                            uint16_t* out, void* stream) {
   return attn_cached_impl(q, kcache, vcache, kscale, kmin, vscale, vmin, true, batch, seq_len, h, h_kv, dh, t_max, pos,
                           pos_dev, 0, n_split, workspace, out, stream);
+}
+
+// ---- the same attention for callers that cannot allocate -------------------------------------
+// The chunk partials and counters live in a file-scope device array instead of a caller-supplied
+// workspace.  Layout: OHARA_SCRATCH_COUNTER_BYTES of counters (one int per (query row, kv head)),
+// then the (max, sum) pairs, then the accumulators, as in ohara_attn_workspace_bytes.  Every GPU
+// holds its own copy of the array; its address is looked up once per device.
+#define OHARA_SCRATCH_COUNTER_BYTES (64 * 1024)
+#define OHARA_SCRATCH_BYTES (OHARA_SCRATCH_COUNTER_BYTES + 8 * 1024 * 1024)
+#define OHARA_SCRATCH_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char scratch[OHARA_SCRATCH_BYTES];
+
+static __global__ void scratch_clear_kernel(int* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+// Device address of `scratch` on the current device (nullptr on failure).  The array's name is only
+// a host-side handle; kernels and fills must be given this address.
+static unsigned char* scratch_device_ptr() {
+  static unsigned char* ptrs[OHARA_SCRATCH_MAX_DEVICES];
+  static std::mutex mu;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= OHARA_SCRATCH_MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+    ptrs[dev] = reinterpret_cast<unsigned char*>(p);
+  }
+  return ptrs[dev];
+}
+
+int ohara_attn_cached_bf16_noalloc(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch,
+                                   int seq_len, int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev,
+                                   int n_split, uint16_t* out, void* stream) {
+  if (batch < 1 || seq_len < 1 || h < 1 || h_kv < 1 || dh < 1 || n_split < 1) return OHARA_EINVAL;
+  const size_t rows = (size_t)batch * seq_len;
+  const size_t counters = rows * h_kv * sizeof(int);
+  const size_t need = OHARA_SCRATCH_COUNTER_BYTES + align256(rows * h * n_split * 2 * sizeof(float)) +
+                      align256(rows * h * n_split * dh * sizeof(float));
+  if (counters > OHARA_SCRATCH_COUNTER_BYTES || need > OHARA_SCRATCH_BYTES) return OHARA_ESIZE;
+  unsigned char* ws = scratch_device_ptr();
+  if (!ws) return OHARA_ELAUNCH;
+  if (n_split > 1) {
+    // the counters must start at zero whatever an earlier call (of any shape) left behind; a fill
+    // kernel rather than a memset node, so that the call can be recorded into a graph
+    const int n = (int)(rows * h_kv);
+    hipLaunchKernelGGL(scratch_clear_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+                       reinterpret_cast<int*>(ws), n);
+    if (ohara_launch_status() != OHARA_OK) return OHARA_ELAUNCH;
+  }
+  return attn_cached_impl(q, kcache, vcache, nullptr, nullptr, nullptr, nullptr, false, batch, seq_len, h, h_kv, dh,
+                          t_max, pos, pos_dev, 0, n_split, ws, out, stream, OHARA_SCRATCH_COUNTER_BYTES);
 }
 
 }  // extern "C"
