@@ -241,6 +241,52 @@ def bench_continuous(model, cfg, dev, slots=32, steps=128):
             "note": "host reads the new ids every step (one synchronisation per step)"}
 
 
+def bench_chat_engine(model, cfg, dev, prompt_len=1024, new_tokens=256, warmup=16):
+    """The reference's caller-facing API on the same workload: ChatEngine.generate (render, prefill,
+    device-resident sampled decode, stop check and incremental detokenisation on the host) with the
+    reference's chat defaults (temperature 0.8, top-p 0.95, no top-k), against a bare decode session
+    with the same sampler.  Tokens/s of the API leg count the whole call, prompt prefill included."""
+    from ohara_amd.chat_engine import ChatEngine
+    from ohara_amd.sampling import SamplingConfig
+
+    class Tok:  # one printable character per id
+        eos_token_id = None
+        bos_token_id = None
+
+        def __len__(self):
+            return cfg.vocab_size
+
+        def get_vocab(self):
+            return {}
+
+        def decode(self, ids, skip_special_tokens=True):
+            return "".join(chr(0x4E00 + (i % 0x5000)) for i in ids)
+
+    g = torch.Generator().manual_seed(9)
+    prompt = torch.randint(0, cfg.vocab_size, (prompt_len,), generator=g).tolist()
+    eng = ChatEngine(model, Tok(), renderer=lambda tok, turns, max_tokens: prompt, stop_ids=())
+    sc = SamplingConfig(temperature=0.8, top_p=0.95, max_new_tokens=new_tokens)
+    msgs = [{"role": "user", "content": "x"}]
+    eng.generate(msgs, sc, seed=0)  # builds the session and captures the graph
+    torch.cuda.synchronize()
+    best = None
+    for rep in range(3):
+        t0 = time.perf_counter()
+        text = eng.generate(msgs, sc, seed=1 + rep)
+        dt = time.perf_counter() - t0
+        assert len(text) == new_tokens
+        best = dt if best is None else min(best, dt)
+    dts, _, sess = time_decode(model, 1, prompt_len, warmup, new_tokens, sampling=sc)
+    del sess
+    api, bare = new_tokens / best, new_tokens / dts
+    return {"tokens_per_s": round(api, 1), "ms_per_token": round(best / new_tokens * 1e3, 4),
+            "new_tokens": new_tokens, "prompt_len": prompt_len,
+            "sampling": "temperature 0.8, top-p 0.95 (ohara/chat_engine.py:35-37 defaults)",
+            "bare_session_tokens_per_s": round(bare, 1), "api_over_session": round(api / bare, 3),
+            "note": "ChatEngine.generate end to end (prefill of the prompt, chunked read-back, stop check, "
+                    "whole-reply detokenisation per token); the session figure is decode steps only"}
+
+
 def bench_prefill(model, cfg, dev):
     """Batched prefill of the d12 model (1024 tokens per sequence) and its MFMA kernels alone."""
     from ohara_amd import ops
@@ -297,30 +343,40 @@ def _fill_cache(cache, length, batch):
         c.length, c.batch_size = length, batch
 
 
-def bench_bitnet(dev):
-    """BitNet-b1.58 ternary Llama (d 2048, 24 layers, 16 x 128 heads, FFN 5632, vocab 32000):
-    one decode step at context 2048, batch 1 and 8."""
-    from ohara_amd.bitnet import BIT_TARGETS, BitLlama
+def bitnet_c4_state(dev, n_layers=24, t_max=2048):
+    """Config and state dict of the BitNet-b1.58 ternary Llama (d 2048, 16 x 128 heads, FFN 5632,
+    vocab 32000): ternary weights uniform over {-1, 0, 1} (seed 2) with a per-tensor scale, unit norms."""
+    from ohara_amd.bitnet import BIT_TARGETS
     from ohara_amd.llama import Config
 
     cfg = Config(vocab_size=32000, hidden_size=2048, intermediate_size=5632, num_attention_heads=16,
-                 num_key_value_heads=0, num_hidden_layers=24, max_sequence_length=2048, dropout=0.0)
+                 num_key_value_heads=0, num_hidden_layers=n_layers, max_sequence_length=t_max, dropout=0.0)
     g = torch.Generator(device=dev).manual_seed(2)
     d, f, v = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
     shapes = {"attn.key": (d, d), "attn.query": (d, d), "attn.value": (d, d), "attn.proj": (d, d),
               "ff.gate": (f, d), "ff.up": (f, d), "ff.down": (d, f)}
     st = {"token_emb.weight": (torch.randn(v, d, device=dev, generator=g) * 0.02).to(torch.bfloat16),
           "vocab_proj.weight": (torch.randn(v, d, device=dev, generator=g) * 0.02).to(torch.bfloat16),
-          "norm.weight": torch.ones(d, device=dev)}
+          "norm.weight": torch.ones(d, device=dev, dtype=torch.bfloat16)}
     for i in range(cfg.num_hidden_layers):
         p = f"layers.{i}."
         for nm in BIT_TARGETS:
             n, k = shapes[nm]
             st[p + nm + ".ternary"] = torch.randint(-1, 2, (n, k), device=dev, generator=g, dtype=torch.int8)
-            st[p + nm + ".gamma"] = 0.02
-            st[p + nm + ".rms_norm.weight"] = torch.ones(k, device=dev)
-        st[p + "norm1.weight"] = torch.ones(d, device=dev)
-        st[p + "norm2.weight"] = torch.ones(d, device=dev)
+            st[p + nm + ".gamma"] = torch.tensor(0.02)
+            st[p + nm + ".rms_norm.weight"] = torch.ones(k, device=dev, dtype=torch.bfloat16)
+        st[p + "norm1.weight"] = torch.ones(d, device=dev, dtype=torch.bfloat16)
+        st[p + "norm2.weight"] = torch.ones(d, device=dev, dtype=torch.bfloat16)
+    return cfg, st
+
+
+def bench_bitnet(dev):
+    """BitNet-b1.58 ternary Llama (d 2048, 24 layers, 16 x 128 heads, FFN 5632, vocab 32000):
+    one decode step at context 2048, batch 1 and 8."""
+    from ohara_amd.bitnet import BitLlama
+
+    cfg, st = bitnet_c4_state(dev)
+    d, v = cfg.hidden_size, cfg.vocab_size
     model = BitLlama(cfg, st, device=dev)
     del st
     out = []
@@ -349,14 +405,14 @@ def _fill_len(cache, length, batch):
         c.length, c.batch_size = length, batch
 
 
-def bench_moe(dev):
-    """MoE decode (16 layers, d 1024, 16 x 64 heads, 64 routed SwiGLU experts of hidden 512, top-8,
-    one shared expert): one step of 64 sequences at context 2048."""
+def moe_c5_state(dev, n_layers=16, t_max=2048):
+    """Config and state dict of the MoE Llama (d 1024, 16 x 64 heads, 64 routed SwiGLU experts of
+    hidden 512, top-8, one shared expert, softmax router): bf16 N(0, 0.02) seed 3, router rows
+    N(0, 1/d) so that the router logits spread like N(0, 1)."""
     from ohara_amd.llama import Config
-    from ohara_amd.moe import MoeLlama
 
     cfg = Config(vocab_size=32000, hidden_size=1024, intermediate_size=512, num_attention_heads=16,
-                 num_key_value_heads=0, num_hidden_layers=16, max_sequence_length=2048, dropout=0.0,
+                 num_key_value_heads=0, num_hidden_layers=n_layers, max_sequence_length=t_max, dropout=0.0,
                  moe_num_experts=64, moe_experts_per_tok=8, moe_grouped=True, moe_num_shared_experts=1)
     g = torch.Generator(device=dev).manual_seed(3)
     d, f, v, E = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.moe_num_experts
@@ -364,18 +420,28 @@ def bench_moe(dev):
     def n(*shape):
         return (torch.randn(*shape, device=dev, generator=g) * 0.02).to(torch.bfloat16)
 
-    st = {"token_emb.weight": n(v, d), "vocab_proj.weight": n(v, d), "norm.weight": torch.ones(d, device=dev)}
+    one = lambda: torch.ones(d, device=dev, dtype=torch.bfloat16)  # noqa: E731
+    st = {"token_emb.weight": n(v, d), "vocab_proj.weight": n(v, d), "norm.weight": one()}
     for i in range(cfg.num_hidden_layers):
         p = f"layers.{i}."
         for nm in ("key", "query", "value", "proj"):
             st[p + f"attn.{nm}.weight"] = n(d, d)
         st[p + "ff.w_gate"], st[p + "ff.w_up"], st[p + "ff.w_down"] = n(E, d, f), n(E, d, f), n(E, f, d)
         st[p + "ff.router.weight"] = (torch.randn(E, d, device=dev, generator=g) / d ** 0.5).to(torch.bfloat16)
-        st[p + "ff.router_bias"] = torch.zeros(E, device=dev)
+        st[p + "ff.router_bias"] = torch.zeros(E, device=dev, dtype=torch.bfloat16)
         st[p + "ff.shared_gate.weight"], st[p + "ff.shared_up.weight"] = n(f, d), n(f, d)
         st[p + "ff.shared_down.weight"] = n(d, f)
-        st[p + "norm1.weight"] = torch.ones(d, device=dev)
-        st[p + "norm2.weight"] = torch.ones(d, device=dev)
+        st[p + "norm1.weight"], st[p + "norm2.weight"] = one(), one()
+    return cfg, st
+
+
+def bench_moe(dev):
+    """MoE decode (16 layers, d 1024, 16 x 64 heads, 64 routed SwiGLU experts of hidden 512, top-8,
+    one shared expert): one step of 64 sequences at context 2048."""
+    from ohara_amd.moe import MoeLlama
+
+    cfg, st = moe_c5_state(dev)
+    d, f, v, E = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.moe_num_experts
     model = MoeLlama(cfg, st, device=dev)
     del st
     B, L = 64, cfg.max_sequence_length
@@ -573,6 +639,7 @@ def main():
         "also": {f"batch{b}": r for b, r in results.items()},
         "roofline": roof,
     }
+    out["also"]["chat_engine_batch1"] = bench_chat_engine(model, cfg, dev, args.prompt, args.steps, args.warmup)
     if not args.no_extended:
         out["also"]["continuous_batch32"] = bench_continuous(model, cfg, dev)
         out["kernels"] = {"prefill_d12": bench_prefill(model, cfg, dev)}

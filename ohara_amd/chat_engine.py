@@ -1,5 +1,8 @@
 """``ChatEngine`` with the reference's call surface (ohara/chat_engine.py:248-422): render a
-conversation, prefill, then stream decoded text deltas while sampling on the device.
+conversation, prefill, then stream decoded text deltas while the model decodes and samples on the
+device.  With the kernel-backed dense ``Llama`` a reply is produced by the device-resident loop of
+``ohara_amd.generation.DeviceLoop`` (one graph replay per token, ids read back in chunks); other
+models are stepped one forward at a time.
 
 Prompt rendering and the chat special tokens belong to the reference's ``ohara.chat``
 (host-side string work, not part of the decode path); the engine takes them as
@@ -13,6 +16,7 @@ from typing import Any, Iterator, Mapping, Sequence
 
 import torch
 
+from .generation import DeviceLoop, ReplyText, stepwise_tokens, supports_device_loop
 from .sampling import SamplingConfig, sample_next_token
 
 USER_START, USER_END = "<|user_start|>", "<|user_end|>"
@@ -47,28 +51,47 @@ def default_renderer(tokenizer, messages, max_tokens: int = 2048) -> list[int]:
     return ids
 
 
+def _window_starts(n_turns: int):
+    """Which leading turns to drop, in order, when a conversation does not fit: whole user/assistant
+    pairs from the front, and at the very end the last remaining turn before the final one
+    (ohara/chat_engine.py:352-366)."""
+    start = 0
+    while n_turns - start > 0:
+        yield start
+        start += 2 if n_turns - start > 2 else 1
+
+
 class ChatEngine:
+    """A model plus its tokenizer answering conversations (ohara/chat_engine.py:248-422).
+
+    Additions to the reference's signature, all keyword-only and optional: ``renderer`` (the prompt
+    renderer, by default the turn layout of ohara/chat.py), ``stop_ids`` (by default the
+    assistant-end marker and the tokenizer's eos), ``sampler_fn`` (a replacement for
+    ``sample_next_token``; giving one selects the stepwise path)."""
+
     def __init__(self, model, tokenizer, *, device=None, dtype=None, renderer=None, stop_ids=None,
                  sampler_fn=None):
-        # ohara/chat_engine.py:251-273
-        if device is None:
-            device = "cuda" if torch.cuda.is_available() else "cpu"
-        self.device = torch.device(device)
-        if dtype is None:
-            dtype = torch.bfloat16 if self.device.type == "cuda" else torch.float32
-        self.dtype = dtype
+        on_gpu = torch.cuda.is_available()
+        self.device = torch.device(device if device is not None else ("cuda" if on_gpu else "cpu"))
+        self.dtype = dtype if dtype is not None else (torch.bfloat16 if self.device.type == "cuda" else torch.float32)
+        # a kernel-backed model accepts only its own device and bfloat16 here and raises otherwise,
+        # so self.dtype never misreports what runs
         self.model = model.to(device=self.device, dtype=self.dtype).eval()
         self.tokenizer = tokenizer
         self.renderer = renderer or default_renderer
         vocab = tokenizer.get_vocab() if hasattr(tokenizer, "get_vocab") else {}
         self.assistant_end_id = vocab.get(ASSISTANT_END)
         self.eos_token_id = tokenizer.eos_token_id
-        self.stop_ids = set(stop_ids) if stop_ids is not None else {self.assistant_end_id, self.eos_token_id}
-        self.stop_ids.discard(None)
-        # ids at or above this only pad the vocabulary projection; never sampled
+        wanted = stop_ids if stop_ids is not None else (self.assistant_end_id, self.eos_token_id)
+        self.stop_ids = {int(t) for t in wanted if t is not None}
+        # ids at or above the tokenizer's size only pad the vocabulary projection: never sampled
         self.tokenizer_vocab_size = len(tokenizer)
         self.max_sequence_length = model.config.max_sequence_length
-        self._sample = sampler_fn if sampler_fn is not None else sample_next_token
+        self._sample = sampler_fn
+        self._loop = None
+        if sampler_fn is None and supports_device_loop(self.model):
+            padded = self.model.config.vocab_size > self.tokenizer_vocab_size
+            self._loop = DeviceLoop(self.model, self.tokenizer_vocab_size if padded else 0)
 
     @classmethod
     def from_checkpoint(cls, checkpoint_path, tokenizer, *, device=None, dtype=None, moe_experts_per_tok: int = 2,
@@ -94,82 +117,65 @@ class ChatEngine:
         return cls(model, tokenizer, device=device, dtype=dtype, renderer=renderer, stop_ids=stop_ids)
 
     def metadata(self, checkpoint_path=None) -> dict[str, Any]:
-        # ohara/chat_engine.py:331-350 (without the checkpoint sidecar file)
+        """The model facts of ohara/chat_engine.py:331-350 (the SFT sidecar file is not read)."""
         cfg = self.model.config
-        return {
-            "parameters": sum(p.numel() for p in self.model.parameters()),
-            "layers": cfg.num_hidden_layers,
-            "hidden_size": cfg.hidden_size,
-            "heads": cfg.num_attention_heads,
-            "context_length": self.max_sequence_length,
-            "vocab_size": cfg.vocab_size,
-            "device": str(self.device),
-            "dtype": str(self.dtype).removeprefix("torch."),
-        }
+        n_params = 0
+        for p in self.model.parameters():
+            n_params += p.numel()
+        return dict(parameters=n_params, layers=cfg.num_hidden_layers, hidden_size=cfg.hidden_size,
+                    heads=cfg.num_attention_heads, context_length=self.max_sequence_length,
+                    vocab_size=cfg.vocab_size, device=str(self.device), dtype=str(self.dtype).removeprefix("torch."))
 
     def render_prompt(self, messages: Sequence[Mapping[str, Any]]) -> list[int]:
-        # ohara/chat_engine.py:352-366: drop whole leading turns until the prompt fits
-        budget = self.max_sequence_length
+        """The rendered conversation, with as many leading turns dropped as it takes to leave room
+        for at least one reply token (never part of a turn)."""
+        window = self.max_sequence_length
         turns = list(messages)
-        while turns:
-            ids = self.renderer(self.tokenizer, turns, max_tokens=budget)
-            if len(ids) < budget:
+        for start in _window_starts(len(turns)):
+            ids = self.renderer(self.tokenizer, turns[start:], max_tokens=window)
+            if len(ids) < window:
                 return ids
-            turns = turns[2:] if len(turns) > 2 else turns[1:]
         raise ValueError("the latest message alone does not fit in the context window")
 
-    def _forward(self, inputs, cache, pos):
-        if getattr(self.model, "supports_last_only", False):
-            return self.model(inputs, cache, pos, last_only=True)
-        return self.model(inputs, cache, pos)
+    def _reply_tokens(self, prompt_ids, budget: int, config: SamplingConfig, seed, u) -> Iterator[int]:
+        generator = None if seed is None else torch.Generator(device=self.device).manual_seed(seed)
+        if self._loop is not None:
+            return self._loop.tokens(prompt_ids, budget, config, u=u, generator=generator)
+        sample = self._sample if self._sample is not None else sample_next_token
+        limit = self.tokenizer_vocab_size
+
+        def select(logits, step):
+            extra = {}
+            if logits.size(-1) > limit:  # chat_engine.py:398-399
+                if sample is sample_next_token:
+                    extra["valid_vocab"] = limit  # masked inside the kernel
+                else:
+                    logits[..., limit:] = float("-inf")
+            if u is not None:
+                extra["u"] = u[step: step + 1]
+            return sample(logits, config, generator, **extra)
+
+        cache = self.model.build_kv_cache(batch_size=1)
+        return stepwise_tokens(self.model, prompt_ids, budget, select, self.device, cache=cache)
 
     @torch.no_grad()
     def generate_stream(self, messages, config: SamplingConfig | None = None, *, seed: int | None = None,
                         u: torch.Tensor | None = None) -> Iterator[str]:
-        """ohara/chat_engine.py:368-412.  ``u`` (max_new_tokens,) optionally supplies the
-        uniform draws (the parity path); otherwise they come from a generator seeded with
-        ``seed`` (or the global RNG)."""
+        """Text deltas of the assistant's reply (ohara/chat_engine.py:368-412).  ``u`` (one uniform
+        draw per new token) optionally fixes the sampler's randomness (the parity path); otherwise
+        the draws come from a generator seeded with ``seed``, or from the global one."""
         config = config or SamplingConfig()
         prompt_ids = self.render_prompt(messages)
-        room = self.max_sequence_length - len(prompt_ids)
-        if room < 1:
+        budget = min(config.max_new_tokens, self.max_sequence_length - len(prompt_ids))
+        if budget < 1:
             raise ValueError("no room left in the context window for a reply")
-        max_new_tokens = min(config.max_new_tokens, room)
-
-        generator = None
-        if seed is not None:
-            generator = torch.Generator(device=self.device).manual_seed(seed)
-
-        kv_cache = self.model.build_kv_cache(batch_size=1)
-        tokens = torch.tensor(prompt_ids, dtype=torch.long, device=self.device).view(1, -1)
-        model_input = tokens
-        position = 0
-        produced: list[int] = []
-        emitted = ""
-        vocab_limit = self.tokenizer_vocab_size
-
-        for step in range(max_new_tokens):
-            logits = self._forward(model_input, kv_cache, position)
-            position += model_input.size(1)
-            kwargs = {}
-            if logits.size(-1) > vocab_limit:
-                if self._sample is sample_next_token:
-                    kwargs["valid_vocab"] = vocab_limit  # masked inside the kernel
-                else:
-                    logits[..., vocab_limit:] = float("-inf")
-            if u is not None:
-                kwargs["u"] = u[step : step + 1]
-            next_token = self._sample(logits, config, generator, **kwargs)
-            token_id = int(next_token.item())
+        reply = ReplyText(self.tokenizer)
+        for token_id in self._reply_tokens(prompt_ids, budget, config, seed, u):
             if token_id in self.stop_ids:
-                break
-            produced.append(token_id)
-            model_input = next_token.to(self.device)
-
-            text = self.tokenizer.decode(produced, skip_special_tokens=True)
-            if len(text) > len(emitted):
-                yield text[len(emitted):]
-                emitted = text
+                return
+            piece = reply.push(token_id)
+            if piece:
+                yield piece
 
     def generate(self, messages, config: SamplingConfig | None = None, *, seed: int | None = None,
                  u: torch.Tensor | None = None) -> str:

@@ -566,9 +566,16 @@ int launch_bit(const BitArgs& a0, hipStream_t st) {
   const int strips = (a0.N + 15) / 16;
   const int KC = (a0.K + 255) >> 8;
   const int ldq = (KC << 8) + 16;
-  for (int r = 0; r < a0.B; r += 64) {
+  // rows per pass: as many 16-row tiles (4, 2 or 1) as fit the LDS with this K
+  auto smem_of = [&](int btt) {
+    return (((size_t)btt * 16 * ldq + 255) & ~(size_t)255) + (size_t)btt * 16 * 8 +
+           (size_t)3 * btt * 64 * 4 * sizeof(int) + (FUSED ? (size_t)4 * (KC << 8) * 2 : 0);
+  };
+  int cap = 64;
+  while (cap > 16 && smem_of(cap / 16) > 160 * 1024) cap >>= 1;
+  for (int r = 0; r < a0.B; r += cap) {
     BitArgs a = a0;
-    a.B = a0.B - r < 64 ? a0.B - r : 64;
+    a.B = a0.B - r < cap ? a0.B - r : cap;
     if (FUSED) a.x = a0.x + (size_t)r * a0.ldx;
     else {
       a.q = a0.q + (size_t)r * a0.ldq;
@@ -580,8 +587,7 @@ int launch_bit(const BitArgs& a0, hipStream_t st) {
     if (a0.acc_out) a.acc_out = a0.acc_out + (size_t)r * a0.ldacc;
     const int bt = (a.B + 15) / 16;
     const int btt = bt == 3 ? 4 : bt;
-    const size_t smem = (((size_t)btt * 16 * ldq + 255) & ~(size_t)255) + (size_t)btt * 16 * 8 +
-                        (size_t)3 * btt * 64 * 4 * sizeof(int) + (FUSED ? (size_t)4 * (KC << 8) * 2 : 0);
+    const size_t smem = smem_of(btt);
     if (smem > 160 * 1024) return OHARA_ESIZE;
     dim3 grid(strips), block(256);
 #define OHARA_BIT(BTV)                                                                                   \

@@ -176,6 +176,14 @@ def rope_tables(head_dim: int, end: int, theta: float):
     return torch.cos(ang), torch.sin(ang)
 
 
+def _check_ids_on_host(x: torch.Tensor, vocab: int) -> None:
+    """nn.Embedding raises on an id outside the table (llama.py:310).  Ids that arrive in host memory
+    are checked here; ids already on the device are not read back (that would cost a synchronisation
+    per call) - the kernels map an id outside [0, vocab) to row 0 instead of reading out of bounds."""
+    if not x.is_cuda and x.numel() and (int(x.min()) < 0 or int(x.max()) >= vocab):
+        raise IndexError("index out of range in self")
+
+
 class _Buffers:
     """Activation buffers and the C state struct for up to `rows` rows."""
 
@@ -269,6 +277,21 @@ class Llama:
         return self
 
     def to(self, *args, **kwargs):
+        """nn.Module.to for a model whose weights are already packed on its device in bf16: a request
+        for that device / dtype is a no-op, anything else raises (the kernels run bf16 only)."""
+        dtype = kwargs.get("dtype")
+        device = kwargs.get("device")
+        for a in args:
+            if isinstance(a, torch.dtype):
+                dtype = a
+            elif a is not None:
+                device = a
+        if dtype is not None and dtype != BF16:
+            raise ValueError(f"ohara_amd runs the decode path in bfloat16 only (got {dtype})")
+        if device is not None:
+            want = torch.device(device)
+            if want.type != self.device.type or (want.index is not None and want.index != (self.device.index or 0)):
+                raise ValueError(f"ohara_amd: the model lives on {self.device}; build it on {want} instead of moving it")
         return self
 
     def parameters(self):
@@ -412,6 +435,7 @@ class Llama:
             ends = [cache._reserve(B, S, start_pos) for cache in kv_cache]
             seq_pos = None
 
+        _check_ids_on_host(x, c.vocab_size)
         rows = B * S
         buf = self._get_buffers(B, rows)
         buf.ids.copy_(x.reshape(-1).to(device=self.device, dtype=torch.int64))
@@ -513,6 +537,7 @@ class DecodeSession:
             raise ValueError("input sequence cannot be empty")
         if P > m.config.max_sequence_length:
             raise ValueError("input exceeds max_sequence_length")
+        _check_ids_on_host(prompt_ids, m.config.vocab_size)
         for cc in self.cache:
             cc._reserve(B, P, 0)
         pbuf = m._get_buffers(B, B * P)
@@ -537,6 +562,8 @@ class DecodeSession:
         dbuf.ids.copy_(pbuf.ids[:B])
         dbuf.step_state.copy_(torch.tensor([P, 1, 0, 0], dtype=torch.int32))
         self.produced = 1
+        if self._dst is not None:
+            return  # a restarted session: buffers, workspace and the captured graph stay as they are
         self._dbuf = dbuf
         self._dst = m._state_struct(dbuf, self.cache, self.logits, history=self.history, valid_vocab=self.valid_vocab)
         self.graph = None
@@ -556,6 +583,23 @@ class DecodeSession:
             check(lib().ohara_llama_decode_persistent(C.byref(m._c_model), C.byref(self._dst), self._pws.data_ptr(),
                                                       self._nwg, 1, 1, 0, torch.cuda.current_stream().cuda_stream),
                   "persistent init")
+
+    def restart(self, u: torch.Tensor | None = None) -> None:
+        """Forget the sequences decoded so far and make the session ready for another ``prefill``:
+        the caches, buffers, workspace and the captured graph are kept (the graph reads the position
+        and the fed ids from device memory, so it serves any later run), only the bookkeeping is
+        reset.  Positions beyond a sequence's length are never read, so the caches need no clearing.
+        ``u``: new uniform draws for a sampling session, (rows <= max_new_tokens, batch)."""
+        for cc in self.cache:
+            cc.length, cc.batch_size, cc.lengths = 0, None, None
+        self.pos = 0
+        self.produced = 0
+        if u is not None:
+            if self.u is None:
+                raise ValueError("this session selects greedily: it takes no uniform draws")
+            if u.ndim != 2 or u.shape[1] != self.batch or u.shape[0] > self.u.shape[0]:
+                raise ValueError("u must have shape (rows <= max_new_tokens, batch)")
+            self.u[: u.shape[0]].copy_(u)
 
     def _launch_step(self) -> None:
         m = self.model

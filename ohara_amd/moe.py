@@ -48,6 +48,7 @@ class GroupedMoE:
         self.wp_dn = torch.stack(dn).contiguous()
         self.router = ops.pack_linear(d(router_w))
         self.router_bias = d(router_bias)
+        self.trace = None  # a list: route() appends (router logits, expert ids, weights) to it
         self.shared = None
         if shared is not None:
             sg, su, sd = shared
@@ -62,6 +63,8 @@ class GroupedMoE:
         check(lib().ohara_moe_route_topk(_ptr(logits), logits.stride(0), _ptr(self.router_bias), n, self.E, self.k,
                                          int(self.biased), int(self.gate_fn == "sigmoid"), int(self.normalize),
                                          _ptr(idx), _ptr(w), ops._stream()), "moe_route")
+        if self.trace is not None:
+            self.trace.append((logits, idx, w))
         return idx, w
 
     def forward_rows(self, flat_x: torch.Tensor, residual: torch.Tensor | None = None) -> torch.Tensor:

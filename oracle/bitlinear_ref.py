@@ -68,8 +68,16 @@ def unpack_ternary(packed: torch.Tensor) -> torch.Tensor:
     return torch.from_numpy(out.reshape(n, kb * 4))
 
 
-def int_accumulate(q: torch.Tensor, t: torch.Tensor) -> torch.Tensor:
-    """(M,K) int8 x (N,K) int8 -> (M,N) int32, exact."""
+def int_accumulate(q: torch.Tensor, t: torch.Tensor, force_int: bool = False) -> torch.Tensor:
+    """(M,K) int8 x (N,K) int8 -> (M,N) int32, exact.
+
+    For ternary ``t`` every partial sum is an integer of magnitude <= 128 * K; below 2**24 such
+    integers and their sums are exact in fp32 whatever the order of the additions, so the fp32
+    BLAS product gives the int32 result bit for bit (and is ~50x faster on a CPU).  Larger K, or
+    ``force_int``, uses the int32 product; tests/test_oracle.py checks the two against each other."""
+    k = q.shape[-1]
+    if not force_int and 128 * k < (1 << 24) and int(t.abs().max()) <= 1:
+        return (q.float() @ t.float().t()).to(torch.int32)
     return (q.to(torch.int32) @ t.to(torch.int32).t()).to(torch.int32)
 
 

@@ -165,3 +165,103 @@ def test_inference_drives_phi_as_the_reference_example_does(cuda):
                 la, lb = logits_seen[t][g_].float().item(), logits_seen[t][w_].float().item()
                 assert abs(la - lb) <= 2.0 ** -6 * max(abs(la), abs(lb), 1e-3), (use_cache, t)
                 break
+
+
+def test_engines_run_on_the_device_loop(cuda):
+    """ChatEngine / Inference over the dense Llama decode through the device-resident loop (persistent
+    step + selection replayed from a graph), reuse one session across requests, and give what the
+    stepwise path (one eager forward + one sampler call per token) gives."""
+    from ohara_amd.chat_engine import ChatEngine
+    from ohara_amd.inference import Inference
+    from ohara_amd.sampling import SamplingConfig, sample_next_token
+
+    tok = CharTokenizer()
+    msgs = [{"role": "user", "content": "tell me"}]
+    model, ref = _tiny(tok, cuda)
+    eng = ChatEngine(model, tok, stop_ids=())
+    assert eng._loop is not None
+    greedy = SamplingConfig(temperature=0.0, max_new_tokens=70)  # several chunks of the loop
+    text = eng.generate(msgs, greedy)
+    sess = eng._loop.session
+    assert sess.graph is not None and len(text) > 0  # (head width 16: the kernel chain, not the persistent kernel)
+    assert eng.generate(msgs, greedy) == text and eng._loop.session is sess  # restarted, not rebuilt
+    # the stepwise path over the same model: same greedy reply up to a near-tie of bf16 logits
+    step = ChatEngine(model, tok, stop_ids=(), sampler_fn=sample_next_token)
+    assert step._loop is None
+    want = step.generate(msgs, greedy)
+    n = next((i for i, (a, b) in enumerate(zip(text, want)) if a != b), min(len(text), len(want)))
+    assert n >= 8, (text, want)
+    # sampled: the loop walks the caller's uniforms on the device; same draws, same text as stepwise
+    cfg = SamplingConfig(temperature=0.8, top_p=0.95, max_new_tokens=40)
+    u = torch.rand(40, generator=torch.Generator().manual_seed(5))
+    a, b = eng.generate(msgs, cfg, u=u), step.generate(msgs, cfg, u=u)
+    n = next((i for i, (x, y) in enumerate(zip(a, b)) if x != y), min(len(a), len(b)))
+    assert n >= 6, (a, b)
+    assert eng.generate(msgs, cfg, u=u) == a
+    assert eng.generate(msgs, cfg, seed=3) == eng.generate(msgs, cfg, seed=3)
+    # a stop id ends the reply although later tokens were already launched
+    first = tok.encode(text[:1])[0]
+    assert ChatEngine(model, tok, stop_ids=(first,)).generate(msgs, greedy) == ""
+    second_stop = ChatEngine(model, tok, stop_ids=(tok.encode(text[5:6])[0],)).generate(msgs, greedy)
+    assert text.startswith(second_stop) and len(second_stop) <= 5
+    # Inference on the loop
+    class Tok:
+        eos_token_id = None
+
+        def encode(self, t):
+            return tok.encode(t)
+
+        def decode(self, ids):
+            return tok.decode(ids, skip_special_tokens=False)
+
+    inf = Inference(model, Tok(), max_new_tokens=20)
+    assert inf._loop is not None
+    out = inf.generate("hello", temperature=0.0, stream=False)
+    assert out.startswith("hello") and len(tok.encode(out)) == 25 and inf.kv_cache[0].length == 24
+    ids = torch.tensor([tok.encode("hello")])
+    want_ids = []
+    rc, pos, inp = ref.build_kv_cache(1), 0, ids
+    for _ in range(6):
+        lg = ref(inp, rc, pos)[:, -1]
+        pos += inp.size(1)
+        inp = lg.float().argmax(-1, keepdim=True)
+        want_ids.append(int(inp))
+    assert tok.encode(out)[5:8] == want_ids[:3]
+
+
+def test_sessions_do_not_share_decode_buffers(cuda):
+    """Two sessions of the same batch size and an eager forward in between: each session's fed ids,
+    position and captured graph are its own, so interleaving them changes nothing."""
+    tok = CharTokenizer()
+    model, _ = _tiny(tok, cuda)
+    g = torch.Generator().manual_seed(2)
+    p1, p2 = torch.randint(5, len(tok), (1, 9), generator=g), torch.randint(5, len(tok), (1, 13), generator=g)
+    alone1 = model.generate_greedy(p1.to(cuda), 24).cpu()
+    alone2 = model.generate_greedy(p2.to(cuda), 24).cpu()
+    s1, s2 = model.session(1, 24), model.session(1, 24)
+    s1.prefill(p1.to(cuda))
+    s2.prefill(p2.to(cuda))
+    for i in range(23):
+        s1.run(1)
+        if i % 3 == 0:  # an eager single-token forward of the same batch size between the steps
+            model(p2[:, :1].to(cuda), model.build_kv_cache(1), 0)
+        s2.run(1)
+    assert torch.equal(s1.tokens().cpu(), alone1) and torch.equal(s2.tokens().cpu(), alone2)
+
+
+def test_dtype_and_id_validation(cuda):
+    from ohara_amd.chat_engine import ChatEngine
+
+    tok = CharTokenizer()
+    model, _ = _tiny(tok, cuda)
+    assert model.to(cuda) is model and model.to(device="cuda", dtype=BF) is model
+    with pytest.raises(ValueError, match="bfloat16 only"):
+        model.to(torch.float32)
+    with pytest.raises(ValueError, match="bfloat16 only"):
+        ChatEngine(model, tok, dtype=torch.float32)
+    with pytest.raises(ValueError, match="lives on"):
+        model.to("cpu")
+    with pytest.raises(IndexError):
+        model(torch.tensor([[1, len(tok) + 5]]))
+    with pytest.raises(IndexError):
+        model(torch.tensor([[-1, 2]]))

@@ -108,3 +108,319 @@ def test_phi2_width_prefill_and_decode_against_the_oracle(cuda):
     close(cache[-1].key[:B, :S0 + 2], rc[-1].key[:B, :S0 + 2])
     toks = model.generate_greedy(ids[:, :S0].to(cuda), 4)
     assert toks.shape == (B, 4) and int(toks.min()) >= 0 and int(toks.max()) < rcfg.vocab_size
+
+
+def _near_tie(logits_row, a, b, ulps=2):
+    la, lb = float(logits_row[a]), float(logits_row[b])
+    ulp = 2.0 ** (math.floor(math.log2(max(abs(la), abs(lb), 1e-30))) - 7)
+    return abs(la - lb) <= ulps * ulp
+
+
+def test_bitnet_c4_model_full_size(cuda):
+    """The BitNet-b1.58 ternary Llama at its full size (d 2048, 24 layers, 16 heads x 128, FFN 5632,
+    vocabulary 32000, cache capacity 2048):
+    (a) the int32 accumulators of layer 0's q / k / v / gate / up projections, computed by the kernels
+        from the model's own embedding rows, equal a CPU integer product of the kernels' own int8
+        codes with the ternary weights, bit for bit;
+    (b) a 64-token prefill and three cached decode steps against the CPU oracle (whole model);
+    (c) at context 2047 -> 2048 (the last cache row), a decode step of 8 sequences equals the same
+        sequences decoded alone; a captured graph replays to the eager result bit for bit."""
+    import bench
+    from ohara_amd import ops
+    from ohara_amd.bitnet import BitLlama
+    from oracle import bitlinear_ref as BL
+    from oracle import llama_ref as R
+
+    cfg, st = bench.bitnet_c4_state(cuda)
+    model = BitLlama(cfg, st, device=cuda)
+    g = torch.Generator().manual_seed(5)
+    V = cfg.vocab_size
+
+    # (a) layer 0, rows = embedding rows of 8 tokens
+    ids8 = torch.randint(0, V, (8,), generator=g)
+    h = ops.embed(ids8.to(cuda), model.token_emb)
+    L0 = model.layers[0]
+    for name in ("attn.query", "attn.key", "attn.value", "ff.gate", "ff.up"):
+        packed, nw = L0[name]
+        pre = L0["norm1"] if name.startswith("attn") else L0["norm2"]
+        q, s, sq = ops.act_quant(ops.rmsnorm(h, pre, model.eps), nw, model.eps)
+        _, acc = ops.gemv_ternary(q, s, sq, packed, want_acc=True)
+        want = BL.int_accumulate(q.cpu()[:, : packed.k], st[f"layers.0.{name}.ternary"].cpu(), force_int=True)
+        assert torch.equal(acc.cpu(), want), name
+        # the fused kernel (block norm + BitLinear norm + codes in one pass) reduces the norms in another
+        # fp32 order, which flips single bf16 roundings: nearly all accumulators identical
+        _, acc_f = ops.bitlinear(h, nw, packed, model.eps, want_acc=True, pre_norm_w=pre)
+        d = (acc_f - acc).abs()
+        assert float((d > 0).float().mean()) < 0.2 and int(d.max()) <= 4 * 127, name
+
+    # (b) the whole model against the oracle: prefill 64, then 3 decode steps (2 sequences)
+    cpu_state = {k: v.cpu() for k, v in st.items()}
+    del st
+    rcfg = R.RefConfig(**{f: getattr(cfg, f) for f in ("vocab_size", "hidden_size", "intermediate_size",
+                                                      "num_attention_heads", "num_key_value_heads",
+                                                      "num_hidden_layers", "max_sequence_length", "rope_theta")})
+    cos, sin = R.rope_table(rcfg.head_dim, rcfg.max_sequence_length * 2, rcfg.rope_theta)
+    cpu_state["freq_cos"], cpu_state["freq_sin"] = cos.to(BF), sin.to(BF)
+    ref = R.RefLlama(rcfg, cpu_state)
+    ids = torch.randint(0, V, (2, 64), generator=g)
+
+    # (b1) one layer, operator by operator, each fed the ORACLE's inputs: identical inputs give
+    # bit-identical outputs on nearly every row.  (The per-row absmax scale makes the quantiser
+    # discontinuous: when a bf16 rounding flips the largest element of a row, every code of the row
+    # is re-rounded; such rows differ at the 1e-3 level, all others not at all.)
+    import torch.nn.functional as F
+
+    S1 = 8
+    w = cpu_state
+
+    def bl(name, inp, pre=None):
+        if pre is not None:
+            inp = R.rms_norm(inp, w[f"layers.0.{pre}.weight"])
+        return BL.bitlinear_forward(inp, w[f"layers.0.{name}.rms_norm.weight"], w[f"layers.0.{name}.ternary"],
+                                    w[f"layers.0.{name}.gamma"])
+
+    def same_rows(got, want, what, min_identical=0.75):
+        got, want = got.float().cpu().reshape(2 * S1, -1), want.float().reshape(2 * S1, -1)
+        d = (got - want).abs()
+        ident = float((d.max(-1).values == 0).float().mean())
+        assert ident >= min_identical and d.mean().item() <= 2e-3 * want.abs().max().item(), (what, ident, d.mean().item())
+        return ident
+
+    x1 = ids[:, :S1]
+    h0 = w["token_emb.weight"][x1].reshape(2 * S1, -1)
+    q, k, v = (bl(n, h0, "norm1").view(2, S1, 16, 128) for n in ("attn.query", "attn.key", "attn.value"))
+    qr, kr = R.apply_rope(q, k, w["freq_cos"][:S1], w["freq_sin"][:S1])
+    att = R.attention_core(qr, kr, v, 0).reshape(2 * S1, -1)
+    h1 = h0 + bl("attn.proj", att)
+    act = F.silu(bl("ff.gate", h1, "norm2")) * bl("ff.up", h1, "norm2")
+    h2 = h1 + bl("ff.down", act)
+    c0 = model.build_kv_cache(2)[0]
+    eps = model.eps
+    qd = ops.bitlinear_qkv_rope_append(h0.to(cuda), L0["norm1"],
+                                       [(L0[n][1], L0[n][0]) for n in ("attn.query", "attn.key", "attn.value")], eps,
+                                       16, 16, 128, model.cos, model.sin, 0, c0.key, c0.value, seq_len=S1)
+    idents = {"q": same_rows(qd, qr, "q"), "k": same_rows(c0.key[:, :S1], kr, "k"),
+              "v": same_rows(c0.value[:, :S1], v, "v")}
+    c0.key[:, :S1].copy_(kr.to(cuda))
+    c0.value[:, :S1].copy_(v.to(cuda))
+    ws = ops.attn_workspace(2, 16, 16, 128, 1, cuda)
+    idents["attention"] = same_rows(ops.attn_auto(qr.reshape(2 * S1, -1).contiguous().to(cuda), c0.key, c0.value, 16, 16,
+                                                  128, 0, 1, ws, S1), att, "attention")
+    idents["proj"] = same_rows(ops.bitlinear(att.to(cuda), L0["attn.proj"][1], L0["attn.proj"][0], eps,
+                                             residual=h0.to(cuda)), h1, "proj")
+    idents["gate_up"] = same_rows(ops.bitlinear_gate_up(h1.to(cuda), L0["norm2"], (L0["ff.gate"][1], L0["ff.gate"][0]),
+                                                        (L0["ff.up"][1], L0["ff.up"][0]), eps), act, "gate_up")
+    idents["down"] = same_rows(ops.bitlinear(act.to(cuda), L0["ff.down"][1], L0["ff.down"][0], eps, residual=h1.to(cuda)),
+                               h2, "down")
+    del c0
+
+    # (b2) the 24-layer model.  Its tolerance comes from the model's own sensitivity: the distance
+    # between the oracle and a variant of it that is an equally valid implementation (softmax weights
+    # rounded to bf16 before they meet the values, as fused attention kernels do, and the norm statistics
+    # in fp64).  Through 24 absmax quantisers such last-bit differences grow to the percent level.
+    rc, cache = ref.build_kv_cache(2), model.build_kv_cache(2)
+    want_all = ref(ids, rc, 0)
+    want = want_all[:, -1]
+    orig_attn, orig_norm, orig_norm_bl = R.attention_core, R.rms_norm, BL.rms_norm
+
+    def attn_bf16_weights(q, k, v, start_pos):
+        B_, S_, H_, D_ = q.shape
+        sc = q.float().permute(0, 2, 1, 3) @ k.float().permute(0, 2, 3, 1) / math.sqrt(D_)
+        vis = torch.arange(k.shape[1])[None, :] <= (start_pos + torch.arange(S_))[:, None]
+        p_ = torch.softmax(sc.masked_fill(~vis[None, None], float("-inf")), -1).to(BF).float()
+        return (p_ @ v.float().permute(0, 2, 1, 3)).to(q.dtype).permute(0, 2, 1, 3).reshape(B_, S_, H_ * D_)
+
+    def norm_fp64(x, weight, eps=1e-5):
+        xf = x.double()
+        return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).to(x.dtype) * weight
+
+    try:
+        R.attention_core, R.rms_norm, BL.rms_norm = attn_bf16_weights, norm_fp64, norm_fp64
+        other = R.RefLlama(rcfg, cpu_state)(ids, ref.build_kv_cache(2), 0)[:, -1]
+    finally:
+        R.attention_core, R.rms_norm, BL.rms_norm = orig_attn, orig_norm, orig_norm_bl
+    fd = (other.float() - want.float()).abs()
+    fscale = want.float().abs().max().item()
+    floor_max, floor_mean = fd.max().item() / fscale, fd.mean().item() / fscale
+    tol_max, tol_mean = max(8e-2, 2 * floor_max), max(1e-2, 2 * floor_mean)
+
+    def close(got, want, what):
+        got, want = got.float().cpu(), want.float()
+        scale = want.abs().max().item()
+        d = (got - want).abs()
+        assert d.max().item() <= tol_max * scale and d.mean().item() <= tol_mean * scale, (what, d.max().item(), d.mean().item(), scale)
+        return round(d.max().item() / scale, 5), round(d.mean().item() / scale, 5)
+
+    got = model(ids.to(cuda), cache, 0, last_only=True)[:, 0]
+    errs = {"prefill": close(got, want, "prefill")}
+    nxt = want.float().argmax(-1, keepdim=True)
+    for t in range(3):
+        want = ref(nxt, rc, 64 + t)[:, -1]
+        got = model(nxt.to(cuda), cache, 64 + t)[:, 0]
+        errs[f"step{t}"] = close(got, want, f"step {t}")
+        nxt = want.float().argmax(-1, keepdim=True)
+    report = {"config": "BitNet ternary Llama d2048 x 24 layers, 2 sequences, prefill 64 + 3 steps",
+              "layer0_rows_bit_identical_per_operator": idents, "model_vs_oracle_max_mean": errs,
+              "oracle_vs_equally_valid_oracle_max_mean": (round(floor_max, 5), round(floor_mean, 5)),
+              "tolerance_used_max_mean": (tol_max, tol_mean)}
+    try:
+        import json
+        import os
+
+        out_dir = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
+        os.makedirs(out_dir, exist_ok=True)
+        with open(os.path.join(out_dir, "parity_bitnet_c4.json"), "w") as f:
+            json.dump(report, f, indent=1)
+    except OSError:
+        pass
+    print(report)
+    del ref, rc, cpu_state, cache, w
+
+    # (c) batch 8 at the end of the context: rows equal the sequences decoded alone; graph == eager
+    B, Lc = 8, cfg.max_sequence_length - 1
+    cache = model.build_kv_cache(B)
+    gd = torch.Generator(device=cuda).manual_seed(6)
+    for c in cache:
+        c.key[:, :Lc].copy_(torch.randn(B, Lc, model.kv_heads, model.head_dim, device=cuda, generator=gd).to(BF))
+        c.value[:, :Lc].copy_(torch.randn(B, Lc, model.kv_heads, model.head_dim, device=cuda, generator=gd).to(BF))
+        c.length, c.batch_size = Lc, B
+    tok = torch.randint(0, V, (B, 1), generator=g).to(cuda)
+    lb = model(tok, cache, Lc, last_only=True)[:, 0].clone()
+    assert cache[0].length == Lc + 1
+    for b in (0, 3, 7):
+        c1 = model.build_kv_cache(1)
+        for cs, cb in zip(c1, cache):
+            cs.key[0, :Lc].copy_(cb.key[b, :Lc])
+            cs.value[0, :Lc].copy_(cb.value[b, :Lc])
+            cs.length, cs.batch_size = Lc, 1
+        l1 = model(tok[b:b + 1], c1, Lc, last_only=True)[0, 0]
+        scale = l1.float().abs().max().item()
+        d = (lb[b].float() - l1.float()).abs()
+        # the kernels serving 1 row and 8 rows reduce the norms in different orders: two equally valid
+        # implementations, so the model's own sensitivity measured in (b2) is the yardstick here too
+        assert d.max().item() <= tol_max * scale and d.mean().item() <= tol_mean * scale, (b, d.max().item(), d.mean().item())
+        del c1
+
+    def step():
+        for c in cache:
+            c.length, c.batch_size = Lc, B
+        return model(tok, cache, Lc, last_only=True)
+
+    eager = step()[:, 0].clone()
+    assert torch.equal(eager, lb)
+    gr = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(gr):
+        out = step()
+    for _ in range(3):
+        out.zero_()
+        gr.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out[:, 0], eager)
+
+
+def test_moe_c5_model_full_size(cuda):
+    """The MoE Llama at its full size (16 layers, d 1024, 16 heads x 64, 64 routed SwiGLU experts of
+    hidden 512, top-8, one shared expert, softmax router):
+    (a) a short prompt (2 x 12 tokens) and two cached steps against the CPU oracle of the whole model;
+    (b) one decode step of 64 sequences at context 2047 -> 2048: every layer's routing indices equal
+        the oracle's selection rule applied to the kernels' own router logits, 8 distinct experts per
+        token with weights that sum to one; three rows equal the same sequences decoded alone."""
+    import bench
+    from ohara_amd.moe import MoeLlama
+    from oracle import llama_ref as R
+    from oracle import moe_ref as MR
+
+    cfg, st = bench.moe_c5_state(cuda)
+    model = MoeLlama(cfg, st, device=cuda)
+    g = torch.Generator().manual_seed(7)
+    V, k = cfg.vocab_size, cfg.moe_experts_per_tok
+
+    def close(got, want, what, mx=3e-2, mn=4e-3):
+        got, want = got.float().cpu(), want.float().cpu()
+        scale = want.abs().max().item()
+        d = (got - want).abs()
+        assert d.max().item() <= mx * scale and d.mean().item() <= mn * scale, (what, d.max().item(), d.mean().item(), scale)
+        return d.max().item() / scale, d.mean().item() / scale
+
+    # (a) against the oracle
+    fields = ("vocab_size", "hidden_size", "intermediate_size", "num_attention_heads", "num_key_value_heads",
+              "num_hidden_layers", "max_sequence_length", "rope_theta", "moe_num_experts", "moe_experts_per_tok",
+              "moe_layer_interval", "moe_gate_fn", "moe_quantile_balancing", "moe_grouped", "moe_num_shared_experts",
+              "moe_normalize_weights")
+    rcfg = R.RefConfig(**{f: getattr(cfg, f) for f in fields})
+    cpu_state = {kk: v.cpu() for kk, v in st.items()}
+    cos, sin = R.rope_table(rcfg.head_dim, rcfg.max_sequence_length * 2, rcfg.rope_theta)
+    cpu_state["freq_cos"], cpu_state["freq_sin"] = cos.to(BF), sin.to(BF)
+    ref = R.RefLlama(rcfg, cpu_state)
+    del cpu_state
+    del st
+    ids = torch.randint(0, V, (2, 12), generator=g)
+    rc, cache = ref.build_kv_cache(2), model.build_kv_cache(2)
+    want = ref(ids, rc, 0)[:, -1]
+    errs = [close(model(ids.to(cuda), cache, 0, last_only=True)[:, 0], want, "prefill")]
+    nxt = want.float().argmax(-1, keepdim=True)
+    for t in range(2):
+        want = ref(nxt, rc, 12 + t)[:, -1]
+        errs.append(close(model(nxt.to(cuda), cache, 12 + t)[:, 0], want, f"step {t}"))
+        nxt = want.float().argmax(-1, keepdim=True)
+    print("moe C5 vs oracle (max, mean error / logit scale):", errs)
+    del ref, rc, cache
+
+    # (b) 64 sequences at the end of the context
+    B, Lc = 64, cfg.max_sequence_length - 1
+    cache = model.build_kv_cache(B)
+    gd = torch.Generator(device=cuda).manual_seed(8)
+    for c in cache:
+        c.key[:, :Lc].copy_(torch.randn(B, Lc, model.kv_heads, model.head_dim, device=cuda, generator=gd).to(BF))
+        c.value[:, :Lc].copy_(torch.randn(B, Lc, model.kv_heads, model.head_dim, device=cuda, generator=gd).to(BF))
+        c.length, c.batch_size = Lc, B
+    tok = torch.randint(0, V, (B, 1), generator=g).to(cuda)
+    trace = []
+    for L in model.layers:
+        L["moe"].trace = trace
+    lb = model(tok, cache, Lc, last_only=True)[:, 0].clone()
+    for L in model.layers:
+        L["moe"].trace = None
+    assert len(trace) == cfg.num_hidden_layers
+    for li, (logits, idx, w) in enumerate(trace):
+        lg = logits.float().cpu()
+        assert lg.shape == (B, cfg.moe_num_experts)
+        want_idx = MR.topk_lowest_index_first(lg + model.layers[li]["moe"].router_bias.float().cpu(), k + 1)[:, :k]
+        assert torch.equal(idx.cpu().long(), want_idx), li
+        assert all(len(set(r)) == k for r in idx.cpu().tolist())
+        want_w = lg.gather(-1, want_idx).softmax(-1)
+        assert (w.float().cpu() - want_w).abs().max().item() <= 2 ** -8
+        assert (w.float().sum(-1) - 1).abs().max().item() <= 2e-2
+    # Rows of the batch against the same sequences decoded alone (other kernels serve 1 row: bf16-level
+    # differences).  Top-k routing is discontinuous, so a row whose router logits hold a near-tie at the
+    # selection boundary may pick another expert when decoded alone; such a flip must BE a near-tie, and
+    # only rows routed identically in every layer are held to the bf16 tolerance.
+    outcomes = {}
+    for b in (0, 13, 31, 47, 63):
+        c1 = model.build_kv_cache(1)
+        for cs, cb in zip(c1, cache):
+            cs.key[0, :Lc].copy_(cb.key[b, :Lc])
+            cs.value[0, :Lc].copy_(cb.value[b, :Lc])
+            cs.length, cs.batch_size = Lc, 1
+        t1 = []
+        for L in model.layers:
+            L["moe"].trace = t1
+        l1 = model(tok[b:b + 1], c1, Lc, last_only=True)[0, 0]
+        for L in model.layers:
+            L["moe"].trace = None
+        flipped = None
+        for li, ((lg64, idx64, _), (lg1, idx1, _)) in enumerate(zip(trace, t1)):
+            a, bb = set(idx64[b].tolist()), set(idx1[0].tolist())
+            if a != bb:
+                flipped = li
+                row = lg1[0].float().cpu()
+                lo, hi = min(float(row[e]) for e in a ^ bb), max(float(row[e]) for e in a ^ bb)
+                assert hi - lo <= 2.0 ** -5 * max(abs(hi), abs(lo), 0.25), (b, li, lo, hi)
+                break
+        if flipped is None:
+            outcomes[b] = ("routed identically", close(lb[b], l1, f"row {b} alone", mx=4e-2, mn=6e-3))
+        else:
+            outcomes[b] = (f"near-tie flip at layer {flipped}", close(lb[b], l1, f"row {b} alone", mx=0.3, mn=0.05))
+        del c1
+    print("moe C5 rows of the batch of 64 vs alone:", outcomes)
+    assert sum(1 for v in outcomes.values() if v[0] == "routed identically") >= 2

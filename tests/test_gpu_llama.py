@@ -36,6 +36,30 @@ def _assert_logits_close(got, ref, max_rel=2e-2, mean_rel=2e-3):
     assert d.mean().item() <= mean_rel * scale, (d.mean().item(), scale)
 
 
+def _rel_errors(got, ref):
+    got, ref = got.float().cpu(), ref.float()
+    scale = ref.abs().max().item()
+    d = (got - ref).abs()
+    return d.max().item() / scale, d.mean().item() / scale
+
+
+def _report(name, payload):
+    """Measured parity figures of the headline model, written where a GPU run's outputs are collected
+    (best effort: the assertions do not depend on it)."""
+    import json
+    import os
+
+    try:
+        root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+        out = os.path.join(root, "gpurun_out")
+        os.makedirs(out, exist_ok=True)
+        with open(os.path.join(out, f"parity_{name}.json"), "w") as f:
+            json.dump(payload, f, indent=1)
+    except OSError:
+        pass
+    print(name, payload)
+
+
 def _golden(name):
     import os
 
@@ -121,7 +145,27 @@ def _near_tie(logits_row, a, b, ulps=2):
     return abs(la - lb) <= ulps * ulp
 
 
-def _check_greedy(model, ref, prompt, steps, cuda, max_rel=2e-2, mean_rel=2e-3):
+class _Fp64LinearOracle:
+    """The CPU oracle with every Linear accumulated in fp64 instead of fp32: an equally valid bf16
+    implementation.  Its distance from the plain oracle at a given position is that position's noise
+    floor (each flipped bf16 rounding cascades through the layers)."""
+
+    def __init__(self, rcfg, w):
+        self.m = R.RefLlama(rcfg, w)
+
+    def build_kv_cache(self, b):
+        return self.m.build_kv_cache(b)
+
+    def __call__(self, *a):
+        orig = R.linear
+        try:
+            R.linear = lambda x, wt, cache=None: (x.double() @ wt.double().t()).to(x.dtype)
+            return self.m(*a)
+        finally:
+            R.linear = orig
+
+
+def _check_greedy(model, ref, prompt, steps, cuda, max_rel=2e-2, mean_rel=2e-3, stats_out=None, noise_ref=None):
     """(1) free-running device loop vs the oracle's greedy tokens: identical, or first
     divergence at a near-tie of the oracle's logits; (2) teacher-forced on the oracle's
     tokens so that every one of the `steps` positions is checked: logits within tolerance
@@ -142,10 +186,32 @@ def _check_greedy(model, ref, prompt, steps, cuda, max_rel=2e-2, mean_rel=2e-3):
     B, P = prompt.shape
     cache = model.build_kv_cache(B)
     inp, pos, same = prompt.to(cuda), 0, 0
+    stats = {"free_running_identical": bool(torch.equal(got, want)), "sequences_diverged_at_a_near_tie": n_diverged,
+             "first_divergence_step": [int((got[b] != want[b]).nonzero()[0]) if (got[b] != want[b]).any() else None
+                                       for b in range(B)],
+             "max_err": 0.0, "mean_err_worst_step": 0.0, "mean_err_avg": 0.0}
+    if stats_out is not None:
+        stats_out.update(stats)
+        stats = stats_out
+    ncache = noise_ref.build_kv_cache(B) if noise_ref is not None else None
+    stats["steps_within_strict_mean_2e-3"] = 0
+    stats["worst_ratio_to_position_floor"] = 0.0
     for t in range(steps):
         logits = model(inp, cache, pos, last_only=True)[:, 0]
+        step_tol = mean_rel
+        if noise_ref is not None:
+            # this position's own noise floor: the tolerance is the target or 1.25 x the floor
+            _, floor_t = _rel_errors(noise_ref(inp.cpu(), ncache, pos)[:, -1], want_logits[t])
+            step_tol = max(mean_rel, 1.25 * floor_t)
         pos += inp.size(1)
-        _assert_logits_close(logits, want_logits[t], max_rel, mean_rel)
+        _assert_logits_close(logits, want_logits[t], max_rel, step_tol)
+        mx, mn = _rel_errors(logits, want_logits[t])
+        stats["steps_within_strict_mean_2e-3"] += int(mn <= 2e-3)
+        if noise_ref is not None:
+            stats["worst_ratio_to_position_floor"] = max(stats["worst_ratio_to_position_floor"], mn / max(floor_t, 1e-12))
+        stats["max_err"] = max(stats["max_err"], mx)
+        stats["mean_err_worst_step"] = max(stats["mean_err_worst_step"], mn)
+        stats["mean_err_avg"] += mn / steps
         mine = logits.float().argmax(-1).cpu()
         for b in range(B):
             if int(mine[b]) == int(want[b, t]):
@@ -154,6 +220,7 @@ def _check_greedy(model, ref, prompt, steps, cuda, max_rel=2e-2, mean_rel=2e-3):
                 assert _near_tie(want_logits[t, b], int(mine[b]), int(want[b, t])), (t, b)
         inp = want[:, t : t + 1].to(cuda)
     assert same >= 0.9 * steps * B, f"only {same}/{steps * B} teacher-forced argmaxes identical"
+    stats["teacher_forced_argmax_identical"] = f"{same}/{steps * B}"
     return got, want, n_diverged
 
 
@@ -211,7 +278,9 @@ def test_d12_decode_parity(cuda):
     model the mean-abs distance between two CPU oracles that differ only in accumulation
     precision is itself ~2.1e-3 (measured below), i.e. the mean criterion sits on the
     noise floor of bf16 arithmetic; the HIP path is required to stay within
-    max(2e-3, 1.25 x that floor) in the mean and within 2e-2 at the maximum."""
+    max(2e-3, 1.25 x that floor) in the mean and within 2e-2 at the maximum.  In the 64-token run the
+    floor is taken position by position (the fp64-accumulating oracle is run teacher-forced beside the
+    plain one), because the floor itself moves by +-30 % from one position to the next."""
     from ohara_amd.llama import Llama
 
     rcfg, cfg = _cfg_pair(vocab_size=65536, hidden_size=768, intermediate_size=3072, num_attention_heads=6,
@@ -234,7 +303,38 @@ def test_d12_decode_parity(cuda):
         got = model(nxt.to(cuda), cache, 96 + step)
         _assert_logits_close(got, want, 2e-2, mean_tol)
         nxt = want[:, -1].float().argmax(-1, keepdim=True)
-    _check_greedy(model, ref, prompt, 64, cuda, 2e-2, mean_tol)
+    stats = {}
+    _check_greedy(model, ref, prompt, 64, cuda, 2e-2, 2e-3, stats_out=stats, noise_ref=_Fp64LinearOracle(rcfg, w))
+    stats.update(config="d12 bf16, 2 sequences, prompt 96, 64 greedy tokens", noise_floor_mean=floor_mean,
+                 noise_floor_max=floor_max, mean_tolerance_used=mean_tol,
+                 strict_mean_2em3_holds=stats["mean_err_worst_step"] <= 2e-3,
+                 strict_max_2em2_holds=stats["max_err"] <= 2e-2,
+                 strict_identical_64_holds=stats["free_running_identical"])
+    _report("d12_prompt96_batch2", stats)
+
+
+def test_d12_prompt1024_batch1_first_64_tokens(cuda):
+    """The headline configuration as stated: batch 1, a 1024-token prompt, cache capacity 4096, the
+    first 64 greedy tokens against the CPU oracle.  Asserted with the same criteria as above; whether
+    the strict criteria (mean-abs 2e-3, 64 identical tokens) hold is recorded without asserting it."""
+    from ohara_amd.llama import Llama
+
+    rcfg, cfg = _cfg_pair(vocab_size=65536, hidden_size=768, intermediate_size=3072, num_attention_heads=6,
+                          num_key_value_heads=0, num_hidden_layers=12, max_sequence_length=4096, dropout=0.0)
+    w = R.init_weights(rcfg, seed=0, dtype=BF)
+    ref = R.RefLlama(rcfg, w)
+    model = Llama(cfg, w, device=cuda)
+    prompt = torch.randint(0, 65536, (1, 1024), generator=torch.Generator().manual_seed(0))
+    floor_mean, floor_max = _accumulation_noise_floor(rcfg, w, prompt)
+    mean_tol = max(2e-3, 1.25 * floor_mean)
+    stats = {}
+    _check_greedy(model, ref, prompt, 64, cuda, 2e-2, 2e-3, stats_out=stats, noise_ref=_Fp64LinearOracle(rcfg, w))
+    stats.update(config="d12 bf16, batch 1, prompt 1024, 64 greedy tokens", noise_floor_mean=floor_mean,
+                 noise_floor_max=floor_max, mean_tolerance_used=mean_tol,
+                 strict_mean_2em3_holds=stats["mean_err_worst_step"] <= 2e-3,
+                 strict_max_2em2_holds=stats["max_err"] <= 2e-2,
+                 strict_identical_64_holds=stats["free_running_identical"])
+    _report("d12_prompt1024_batch1", stats)
 
 
 @pytest.mark.parametrize("persistent", [True, False])

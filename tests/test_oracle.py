@@ -290,6 +290,14 @@ def test_bitlinear_integer_semantics():
     for m in range(3):
         for n in (0, 7, 23):
             assert int(acc[m, n]) == sum(int(a) * int(b) for a, b in zip(qq[m].tolist(), t[n].tolist()))
+    # the fp32-BLAS route of int_accumulate (used below 128*K < 2**24) equals the int32 product, also
+    # at the largest K of the ternary model (5632) with worst-case magnitudes
+    for K in (40, 2048, 5632):
+        q8 = torch.randint(-128, 128, (9, K), generator=g, dtype=torch.int8)
+        t8 = torch.randint(-1, 2, (33, K), generator=g, dtype=torch.int8)
+        q8[0], t8[0] = -128, -1  # |sum| = 128 * K, the bound of the exactness argument
+        assert torch.equal(BL.int_accumulate(q8, t8), BL.int_accumulate(q8, t8, force_int=True))
+        assert int(BL.int_accumulate(q8, t8)[0, 0]) == 128 * K
     # packing round trip and bit layout
     packed = BL.pack_ternary(t)
     assert packed.shape == (24, 10) and torch.equal(BL.unpack_ternary(packed), t)
