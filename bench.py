@@ -537,6 +537,70 @@ def bench_phi(dev):
     return out
 
 
+# Shader-clock samples that workgroup 0 of the persistent kernel takes per layer, in order (see
+# csrc/mega.hip: Prof::stamp in the kernel body, GridSync::arrive / wait and gemm_phase).  Each entry
+# names the interval that ENDS at that sample.
+_ARRIVE = ["epilogue stores issued -> arrive()", "wait for own stores (vmcnt 0)", "workgroup barrier",
+           "arrival atomics issued"]
+_WAIT = ["next phase's prefetch issued", "spin on the release word + workgroup barrier", "(bookkeeping)"]
+_GEMM = ["activations staged in LDS -> MFMAs issued", "cross-wave sum"]
+PHASE_STAMPS = (
+    [("P1 qkv", "mailbox read + norm1 into LDS")] + [("P1 qkv", x) for x in _GEMM] + [("P1 qkv", "rotary epilogue")]
+    + [("P1 qkv", x) for x in _ARRIVE + _WAIT]
+    + [("P2 attention", "attention chunk (q mailbox, K/V tiles, partials)")] + [("P2 attention", x) for x in _ARRIVE[1:] + _WAIT]
+    + [("P3 wo", "merge of attention partials into LDS")] + [("P3 wo", x) for x in _GEMM] + [("P3 wo", "residual epilogue")]
+    + [("P3 wo", x) for x in _ARRIVE + _WAIT]
+    + [("P4 gate/up", "mailbox read + norm2 -> MFMAs issued"), ("P4 gate/up", "cross-wave sum")]
+    + [("P4 gate/up", "SwiGLU epilogue")] + [("P4 gate/up", x) for x in _ARRIVE[1:] + _WAIT]
+    + [("P5 down", "act mailbox into LDS -> MFMAs issued"), ("P5 down", "cross-wave sum")]
+    + [("P5 down", "partial-sum epilogue")] + [("P5 down", x) for x in _ARRIVE[1:] + _WAIT]
+)
+
+
+def phase_timeline(dev, prompt_len, steps=32):
+    """Per-phase timeline of the persistent decode kernel at batch 1: where workgroup 0 spends a
+    step, from the kernel's own shader-clock samples averaged over `steps` real decode steps."""
+    from ohara_amd.llama import Llama
+
+    cfg, st = d12_state(dev)
+    model = Llama(cfg, st, device=dev)
+    sess = model.session(1, steps + 24)
+    sess.prefill(torch.randint(0, cfg.vocab_size, (1, prompt_len)).to(dev))
+    for _ in range(8):
+        sess.step()
+    nl = cfg.num_hidden_layers
+    per = len(PHASE_STAMPS)
+    n_stamps = 1 + per * nl
+    n_tail = 10  # after the layers: LM head (2 samples), its end, the selection's arrive (4) / wait (2), the end
+    acc = torch.zeros(n_stamps + n_tail, dtype=torch.float64)
+    total_ms = 0.0
+    for _ in range(steps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        sess.step(prof_kernel=-2)
+        e1.record()
+        torch.cuda.synchronize()
+        total_ms += e0.elapsed_time(e1)
+        c = sess.phase_clocks().double()
+        acc += c[: n_stamps + n_tail] - c[0]
+    acc /= steps
+    kernel_us = total_ms / steps * 1e3
+    end = float(acc[n_stamps + n_tail - 1])
+    ticks_per_us = end / kernel_us  # the whole kernel, first to last sample, against HIP events
+    d = (acc[1:n_stamps] - acc[:n_stamps - 1]).view(nl, per)
+    rows = {}
+    for j, (phase, what) in enumerate(PHASE_STAMPS):
+        rows.setdefault(phase, []).append((what, float(d[:, j].mean()) / ticks_per_us))
+    out = {"kernel_us_hip_events": round(kernel_us, 2), "layers": nl, "clock_ticks_per_us": round(ticks_per_us, 2),
+           "per_layer_us": round(float(d.sum(1).mean()) / ticks_per_us, 3),
+           "after_last_layer_us (final norm + vocabulary projection + selection)":
+               round((end - float(acc[n_stamps - 1])) / ticks_per_us, 2), "phases": {}}
+    for phase, items in rows.items():
+        out["phases"][phase] = {"total_us": round(sum(v for _, v in items), 3),
+                                "parts_us": {w: round(v, 3) for w, v in items}}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -551,6 +615,8 @@ def main():
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run three 1 GiB device-to-device copies (a kernel of known traffic to scale "
                          "FETCH_SIZE / WRITE_SIZE counters against)")
+    ap.add_argument("--phase-timeline", action="store_true",
+                    help="print the per-phase timeline of the persistent decode kernel at batch 1 and exit")
     ap.add_argument("--phi-decode-only", type=int, default=0, metavar="B",
                     help="run 12 eager Phi-2 decode steps of B sequences at context 1024 and exit (profiling workload)")
     args = ap.parse_args()
@@ -567,6 +633,9 @@ def main():
     dev = torch.device("cuda:0")
     if args.phi_decode_only:
         print(json.dumps(phi_decode_only(dev, args.phi_decode_only)))
+        return
+    if args.phase_timeline:
+        print(json.dumps(phase_timeline(dev, args.prompt), indent=1))
         return
     if args.pmc_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)

@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 BF = torch.bfloat16
 
 
-@pytest.mark.parametrize("B,L", [(16, 32768), (64, 4096)])
+@pytest.mark.parametrize("B,L", [(16, 32768), (64, 4096), (1, 16384), (1, 32768)])
 def test_decode_attention_microbench_shape(cuda, B, L):
     """32 query / 8 KV heads x 128, one query per sequence over L cached positions."""
     from ohara_amd import ops
