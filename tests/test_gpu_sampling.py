@@ -64,6 +64,9 @@ CASES = [
     (65536, 4, 1.0, 0, 0.999, 8.0, torch.bfloat16),    # candidates run out: falls back to the general path
     (65536, 3, 1.0, 0, 0.9, 0.5, torch.bfloat16),      # flat: tens of thousands kept (multi-round path)
     (65536, 3, 1.0, 5000, 0.5, 0.5, torch.float32),
+    (65536, 3, 1.0, 5000, 0.5, 0.5, torch.bfloat16),   # top-k beyond the sorted block + nucleus: the count table
+    (65536, 3, 0.9, 3000, 1.0, 1.0, torch.bfloat16),   # the same without a nucleus: vocabulary-order draw above a threshold
+    (40000, 3, 1.2, 2000, 0.0, 2.0, torch.bfloat16),
     (32000, 4, 0.8, 0, 0.0, 1.0, torch.bfloat16),      # vocabulary-order draw
     (50, 5, 1.0, 100, 0.3, 1.0, torch.float32),        # top_k larger than the vocabulary
 ]
@@ -156,3 +159,24 @@ def test_nucleus_alone_on_rows_with_many_ties(cuda):
                     assert int(got[b]) == int(want[b, 0]), (T, p, valid, b, int(got[b]), int(want[b, 0]), float(margin[b]))
                 if valid is not None:
                     assert int(got[b]) < valid
+
+
+def test_rows_of_one_single_value(cuda):
+    """Every id has the same logit (the one case in which a 16-bit count of the table-based sampler
+    could overflow): uniform probabilities, the nucleus keeps the first floor(top_p * V) + 1 ids, ties
+    are taken lowest id first, so the draw u lands on id floor(u * kept)."""
+    from ohara_amd import ops
+
+    for V in (65536, 50000):
+        row = torch.full((2, V), 1.5, dtype=torch.bfloat16, device=cuda)
+        u = torch.tensor([0.25, 0.9], device=cuda)
+        got = ops.sample_topk_topp(row, 0.8, 0, 0.5, u).cpu()
+        kept = int(0.5 * V) + 1
+        for b in range(2):
+            assert abs(int(got[b]) - int(float(u[b]) * kept)) <= 2, (V, b, int(got[b]))
+        got = ops.sample_topk_topp(row, 1.0, 0, 1.0, u).cpu()  # plain multinomial: vocabulary order
+        for b in range(2):
+            assert abs(int(got[b]) - int(float(u[b]) * V)) <= 2, (V, b, int(got[b]))
+        got = ops.sample_topk_topp(row, 1.0, 2000, 1.0, u).cpu()  # top-k keeps every tie
+        for b in range(2):
+            assert abs(int(got[b]) - int(float(u[b]) * V)) <= 2, (V, b, int(got[b]))
