@@ -173,25 +173,26 @@ int ohara_attn_prefill_bf16(const uint16_t* q, const uint16_t* kcache, const uin
  * minimum: scale = max((max - min) / 255, 1e-8), q = clamp(round((x - min) / scale - 128), -128,
  * 127), read back as bf16((q + 128) * scale + min).  The quantisation arithmetic is rounded to
  * bf16 after every operation, as the reference's tensor ops on a bf16 cache are, so codes, scales
- * and minima are bit-identical to it.  Caches: (batch_cap, t_max, h_kv, dh) int8; statistics:
- * (batch_cap, t_max, h_kv) fp32.
+ * and minima are bit-identical to it.  Caches: (batch_cap, t_max, h_kv, dh) int8.  Statistics:
+ * `stats`, (batch_cap, h_kv, t_max, 4) fp32 = one 16-byte record (key scale, key minimum, value
+ * scale, value minimum) per row, consecutive positions of a head contiguous (the order decode
+ * attention reads them in; the reference's four (B, T, H_kv, 1) tensors, kv_cache.py:67-73, are
+ * strided views of it).
  *   ohara_kv_quant_append_int8  quantises k / v rows (batch*seq_len, h_kv*dh) into positions
  *                               pos + s (pos_dev as elsewhere);
- *   ohara_kv_dequant_int8       the first `len` positions of one cache tensor as bf16
- *                               (batch, len, h_kv, dh) - what KVCache._read returns;
+ *   ohara_kv_dequant_int8       the first `len` positions of the key (which = 0) or value (which = 1)
+ *                               cache tensor as bf16 (batch, len, h_kv, dh) - what KVCache._read returns;
  *   ohara_attn_cached_int8      ohara_attn_cached_bf16 over the quantised cache, dequantising in
  *                               registers.  Scales must be bf16-representable, as the quantiser
  *                               writes them: (q + 128) * scale is then exact in fp32 and the
  *                               kernel's fused multiply-add equals the reference's two roundings. */
 int ohara_kv_quant_append_int8(const uint16_t* k, const uint16_t* v, int batch, int seq_len, int h_kv, int dh, int pos,
-                               const int32_t* pos_dev, int8_t* kq, int8_t* vq, float* kscale, float* kmin, float* vscale,
-                               float* vmin, int t_max, void* stream);
-int ohara_kv_dequant_int8(const int8_t* q, const float* scale, const float* mn, int batch, int len, int h_kv, int dh,
+                               const int32_t* pos_dev, int8_t* kq, int8_t* vq, float* stats, int t_max, void* stream);
+int ohara_kv_dequant_int8(const int8_t* q, const float* stats, int which, int batch, int len, int h_kv, int dh,
                           int t_max, uint16_t* out, void* stream);
-int ohara_attn_cached_int8(const uint16_t* q, const int8_t* kcache, const int8_t* vcache, const float* kscale,
-                           const float* kmin, const float* vscale, const float* vmin, int batch, int seq_len, int h,
-                           int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev, int n_split, void* workspace,
-                           uint16_t* out, void* stream);
+int ohara_attn_cached_int8(const uint16_t* q, const int8_t* kcache, const int8_t* vcache, const float* stats, int batch,
+                           int seq_len, int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev, int n_split,
+                           void* workspace, uint16_t* out, void* stream);
 
 /* ---- greedy selection ---------------------------------------------------------
  * next_ids[b] = first index of max(logits[b, 0:valid_vocab])  (argmax of the last
@@ -357,15 +358,12 @@ typedef struct OharaDecodeState {
   int64_t* history;      /* (hist_cap, batch) generated ids, may be NULL                  */
   uint16_t* const* kcache; /* host array [n_layers] of (batch_cap, t_max, h_kv, dh)       */
   uint16_t* const* vcache;
-  /* int8 cache mode (kv_int8 != 0): kcache / vcache point at int8 tensors of the same shape, the
-     four arrays below at the per-layer (batch_cap, t_max, h_kv) fp32 statistics; kstage / vstage
+  /* int8 cache mode (kv_int8 != 0): kcache / vcache point at int8 tensors of the same shape,
+     kvstats at the per-layer (batch_cap, h_kv, t_max, 4) fp32 statistics records; kstage / vstage
      (rows, h_kv*dh) receive the bf16 rows before they are quantised; kdeq / vdeq ((batch, t_max,
      h_kv, dh) bf16, may be NULL) hold the dequantised cache for calls with >= 16 positions. */
   int32_t kv_int8;
-  float* const* kscale;
-  float* const* kmin;
-  float* const* vscale;
-  float* const* vmin;
+  float* const* kvstats;
   uint16_t* kstage;
   uint16_t* vstage;
   uint16_t* kdeq;

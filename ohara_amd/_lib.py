@@ -40,8 +40,7 @@ class OharaDecodeState(C.Structure):
         ("ids", _p), ("x", _p), ("q", _p), ("attn", _p), ("act", _p), ("xn", _p), ("logits", _p),
         ("attn_ws", _p), ("step_state", _p), ("history", _p),
         ("kcache", C.POINTER(_p)), ("vcache", C.POINTER(_p)),
-        ("kv_int8", _i), ("kscale", C.POINTER(_p)), ("kmin", C.POINTER(_p)), ("vscale", C.POINTER(_p)),
-        ("vmin", C.POINTER(_p)), ("kstage", _p), ("vstage", _p), ("kdeq", _p), ("vdeq", _p),
+        ("kv_int8", _i), ("kvstats", C.POINTER(_p)), ("kstage", _p), ("vstage", _p), ("kdeq", _p), ("vdeq", _p),
         ("seq_pos", _p), ("prof_start", _p), ("prof_stop", _p),
     ]
 
@@ -58,9 +57,9 @@ _PROTOS = {
     "ohara_gemm_bf16": (_i, [_p, _i, _p, _i, _i, _i, _i, _p, _i, _p, _i, _p]),
     "ohara_qkv_rope_append_bf16": (_i, [_p, _i, _p, _i, _p, _f, _i, _i, _i, _i, _i, _p, _p, _i, _p, _p, _p, _p, _i, _p]),
     "ohara_qkv_rope_bf16": (_i, [_p, _i, _p, _i, _p, _f, _i, _i, _i, _i, _i, _p, _p, _i, _p, _i, _p, _p, _p, _p]),
-    "ohara_kv_quant_append_int8": (_i, [_p, _p, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _i, _p]),
-    "ohara_kv_dequant_int8": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _p, _p]),
-    "ohara_attn_cached_int8": (_i, [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
+    "ohara_kv_quant_append_int8": (_i, [_p, _p, _i, _i, _i, _i, _i, _p, _p, _p, _p, _i, _p]),
+    "ohara_kv_dequant_int8": (_i, [_p, _p, _i, _i, _i, _i, _i, _i, _p, _p]),
+    "ohara_attn_cached_int8": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
     "ohara_attn_workspace_bytes": (_i64, [_i, _i, _i, _i, _i]),
     "ohara_attn_cached_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
     "ohara_attn_cached_bf16_noalloc": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p]),

@@ -5,9 +5,9 @@
 //
 // Grid (query rows, H_kv, n_split).  A workgroup streams its chunk of the context for one
 // KV head once and serves all G = H/H_kv query heads from it.  Per 16-position tile
-// a wave holds one position per lane-column (16 columns x 4 quarter-rows of Dh), so
-// q.k needs two cross-lane adds; the running max/sum of the online softmax are
-// wavefront shuffle reductions.  Partial (max, sum, acc) triples of the chunks are
+// a wave holds one position per quad of lanes (the four lanes hold the four quarters of its K
+// row), so q.k needs two adds inside the quad (DPP, no LDS round trip); the running max/sum of
+// the online softmax are wavefront shuffle reductions.  Partial (max, sum, acc) triples of the chunks are
 // merged by whichever workgroup of the (sequence, KV head) finishes last, in chunk
 // order, so the result does not depend on scheduling.
 #include <mutex>
@@ -20,10 +20,8 @@ struct AttnArgs {
   const bf16_t* q;   // (B, H*D)
   const bf16_t* k;   // (Bcap, Tmax, Hkv, D); int8 mode: the same shape in int8
   const bf16_t* v;
-  const float* kscale;  // int8 mode (ohara/modules/kv_cache.py:67-73): (Bcap, Tmax, Hkv) scale / minimum
-  const float* kmin;
-  const float* vscale;
-  const float* vmin;
+  const float* stats;   // int8 mode (ohara/modules/kv_cache.py:67-73): (Bcap, Hkv, Tmax, 4) = key scale, key
+                        // minimum, value scale, value minimum of every (sequence, head, position) row
   bf16_t* out;       // (B, H*D)
   int B, S, H, Hkv, D, Tmax, start;  // query s of sequence b sees positions [0, start + s]
   const int32_t* pos_dev;            // when set: start = *pos_dev, or pos_dev[sequence] with pos_stride 1
@@ -41,6 +39,14 @@ __device__ __forceinline__ float dot8(uint4 a, uint4 b, float s) {
   s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.z), __builtin_bit_cast(bf16x2, b.z), s, false);
   s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.w), __builtin_bit_cast(bf16x2, b.w), s, false);
   return s;
+}
+
+// Sum over the four lanes of a quad (lanes 4i .. 4i+3) with two DPP adds: no LDS round trip, unlike a
+// shuffle across rows.  quad_perm [1,0,3,2] = 0xB1 (lane ^ 1), [2,3,0,1] = 0x4E (lane ^ 2).
+__device__ __forceinline__ float quad_sum(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));
+  return v;
 }
 
 __device__ __forceinline__ float ldf_coh(const float* p) { return __uint_as_float(ld_coh4(p)); }
@@ -132,7 +138,7 @@ __device__ __forceinline__ uint2 dequant4(uint32_t w, float s, float m) {
   return make_uint2(pack_bf(f0, f1), pack_bf(f2, f3));
 }
 
-template <int D, int G, bool I8>
+template <int D, int G>
 __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   constexpr int NC = D / 32;        // 16-byte K loads per lane per tile
   constexpr int DC = D / 8;         // lanes covering one V row with 16-byte loads
@@ -145,19 +151,19 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   const int t0 = split * chunk;
   const int t1 = min(L, t0 + chunk);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int p = lane & 15, dq = lane >> 4;
+  const int p = lane >> 2, dq = lane & 3;  // position of the tile, quarter of its K row: a quad holds one row
   const int pp = lane / DC, dc = lane % DC;
 
   __shared__ float s_m[4][G], s_l[4][G];
   __shared__ float s_acc[4][G][D];
 
-  // q for this lane's quarter-row: columns (4c + dq)*8 .. +7 (int8 mode: the contiguous quarter dq)
+  // q for this lane's quarter-row: columns (4c + dq)*8 .. +7
   uint4 qv[G][NC];
 #pragma unroll
   for (int hh = 0; hh < G; ++hh)
 #pragma unroll
     for (int c = 0; c < NC; ++c)
-      qv[hh][c] = ldg16(a.q + (size_t)b * a.H * D + (size_t)(kvh * G + hh) * D + (I8 ? (dq * NC + c) : (4 * c + dq)) * 8);
+      qv[hh][c] = ldg16(a.q + (size_t)b * a.H * D + (size_t)(kvh * G + hh) * D + (4 * c + dq) * 8);
 
   float m_run[G], l_run[G], acc[G][8];
 #pragma unroll
@@ -172,75 +178,26 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   const bf16_t* kb = a.k + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
   const bf16_t* vb = a.v + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
 
-  // A tile in the form it is fetched in.  bf16: the MFMA-free dot operands themselves.  int8: the
-  // raw bytes of this lane's quarter of the K row / eighth of the V rows plus the rows' scale and
-  // minimum; they are expanded to bf16 right before use, so the fetch of the next tile stays
-  // asynchronous.
   struct Tile {
-    uint4 k[I8 ? (NC + 1) / 2 : NC];
-    uint4 v[I8 ? (NV + 1) / 2 : NV];
-    float ks, km, vs[NV], vm[NV];
+    uint4 k[NC];
+    uint4 v[NV];
   };
-  const int8_t* kb8 = reinterpret_cast<const int8_t*>(a.k) + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
-  const int8_t* vb8 = reinterpret_cast<const int8_t*>(a.v) + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
   auto load_tile = [&](int tb, Tile& t) {
     const int pos = tb + p;
-    if (I8) {
-      const size_t slot = ((size_t)seq * a.Tmax + pos) * a.Hkv + kvh;
-      const bool in = pos < t1;
-      t.ks = in ? a.kscale[slot] : 0.f;
-      t.km = in ? a.kmin[slot] : 0.f;
 #pragma unroll
-      for (int c = 0; c < (NC + 1) / 2; ++c) {
-        if (NC >= 2) t.k[c] = in ? ldg16_nt(kb8 + (size_t)pos * row + dq * (NC * 8) + 16 * c) : make_uint4(0, 0, 0, 0);
-        else {
-          const uint2 w = in ? *reinterpret_cast<const uint2*>(kb8 + (size_t)pos * row + dq * 8) : make_uint2(0, 0);
-          t.k[c] = make_uint4(w.x, w.y, 0, 0);
-        }
-      }
+    for (int c = 0; c < NC; ++c)
+      t.k[c] = pos < t1 ? ldg16_nt(kb + (size_t)pos * row + (4 * c + dq) * 8) : make_uint4(0, 0, 0, 0);
 #pragma unroll
-      for (int c = 0; c < NV; ++c) {
-        const int vp = tb + c * PP + pp;
-        const bool vin = vp < t1;
-        const size_t vslot = ((size_t)seq * a.Tmax + vp) * a.Hkv + kvh;
-        t.vs[c] = vin ? a.vscale[vslot] : 0.f;
-        t.vm[c] = vin ? a.vmin[vslot] : 0.f;
-        const uint2 w = vin ? *reinterpret_cast<const uint2*>(vb8 + (size_t)vp * row + dc * 8) : make_uint2(0x80808080u, 0x80808080u);
-        uint32_t* dstw = reinterpret_cast<uint32_t*>(&t.v[c >> 1]) + 2 * (c & 1);
-        dstw[0] = w.x;
-        dstw[1] = w.y;
-      }
-    } else {
-#pragma unroll
-      for (int c = 0; c < NC; ++c)
-        t.k[c] = pos < t1 ? ldg16_nt(kb + (size_t)pos * row + (4 * c + dq) * 8) : make_uint4(0, 0, 0, 0);
-#pragma unroll
-      for (int c = 0; c < NV; ++c) {
-        const int vp = tb + c * PP + pp;
-        t.v[c] = vp < t1 ? ldg16_nt(vb + (size_t)vp * row + dc * 8) : make_uint4(0, 0, 0, 0);
-      }
+    for (int c = 0; c < NV; ++c) {
+      const int vp = tb + c * PP + pp;
+      t.v[c] = vp < t1 ? ldg16_nt(vb + (size_t)vp * row + dc * 8) : make_uint4(0, 0, 0, 0);
     }
   };
   auto expand = [&](const Tile& t, uint4* kv, uint4* vv) {
-    if (I8) {
 #pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        const uint32_t* w = reinterpret_cast<const uint32_t*>(&t.k[c >> 1]) + 2 * (c & 1);
-        const uint2 lo = dequant4(w[0] ^ 0x80808080u, t.ks, t.km), hi = dequant4(w[1] ^ 0x80808080u, t.ks, t.km);
-        kv[c] = make_uint4(lo.x, lo.y, hi.x, hi.y);
-      }
+    for (int c = 0; c < NC; ++c) kv[c] = t.k[c];
 #pragma unroll
-      for (int c = 0; c < NV; ++c) {
-        const uint32_t* w = reinterpret_cast<const uint32_t*>(&t.v[c >> 1]) + 2 * (c & 1);
-        const uint2 lo = dequant4(w[0] ^ 0x80808080u, t.vs[c], t.vm[c]), hi = dequant4(w[1] ^ 0x80808080u, t.vs[c], t.vm[c]);
-        vv[c] = make_uint4(lo.x, lo.y, hi.x, hi.y);
-      }
-    } else {
-#pragma unroll
-      for (int c = 0; c < NC; ++c) kv[c] = t.k[c];
-#pragma unroll
-      for (int c = 0; c < NV; ++c) vv[c] = t.v[c];
-    }
+    for (int c = 0; c < NV; ++c) vv[c] = t.v[c];
   };
   // 16-position tiles, wave w takes tiles w, w+4, ...; the loads of the next tile are in
   // flight while the current one is consumed (a second tile in flight costs more in occupancy
@@ -268,9 +225,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
       sc[hh] = s;
     }
 #pragma unroll
-    for (int hh = 0; hh < G; ++hh) sc[hh] += __shfl_xor(sc[hh], 16, WAVE);
-#pragma unroll
-    for (int hh = 0; hh < G; ++hh) sc[hh] += __shfl_xor(sc[hh], 32, WAVE);
+    for (int hh = 0; hh < G; ++hh) sc[hh] = quad_sum(sc[hh]);
     bool raise = false;
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) {
@@ -282,7 +237,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
 #pragma unroll
       for (int hh = 0; hh < G; ++hh) tm[hh] = sc[hh];
 #pragma unroll
-      for (int o = 8; o > 0; o >>= 1)
+      for (int o = 32; o > 2; o >>= 1)
 #pragma unroll
         for (int hh = 0; hh < G; ++hh) tm[hh] = fmaxf(tm[hh], __shfl_xor(tm[hh], o, WAVE));
 #pragma unroll
@@ -305,7 +260,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
       const uint32_t w4[4] = {vv[c].x, vv[c].y, vv[c].z, vv[c].w};
       float pw[G];
 #pragma unroll
-      for (int hh = 0; hh < G; ++hh) pw[hh] = __shfl(pv[hh], c * PP + pp, WAVE);
+      for (int hh = 0; hh < G; ++hh) pw[hh] = __shfl(pv[hh], 4 * (c * PP + pp), WAVE);
 #pragma unroll
       for (int hh = 0; hh < G; ++hh)
 #pragma unroll
@@ -320,7 +275,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   // fold the sums over the 16 positions of a tile (every lane of a quarter holds the same share),
   // the PP row-groups of the wave, then the four waves
 #pragma unroll
-  for (int o = 8; o > 0; o >>= 1)
+  for (int o = 32; o > 2; o >>= 1)
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) l_run[hh] += __shfl_xor(l_run[hh], o, WAVE);
 #pragma unroll
@@ -369,6 +324,214 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   if (last_chunk_done(a.counters + b * a.Hkv + kvh, a.nsplit)) merge_partials<D>(a, b, kvh, G);
 }
 
+
+// The same attention over the int8 cache (ohara/modules/kv_cache.py:15-32, 116-118).  A row of codes is
+// half the bytes of a bf16 row, and what bounds this kernel is the bytes a wave has in flight, so a tile
+// here is 32 positions (two sub-tiles of 16 with the lane roles of the bf16 kernel): the same bytes in
+// flight, twice the positions per round trip.  The four statistics of a position are one 16-byte record
+// ((Bcap, Hkv, Tmax, 4) fp32: consecutive positions are contiguous, nothing is fetched that is not used);
+// the lane that owns a position loads its record, the value rows get their scale and minimum from that
+// lane by a shuffle.  Codes become the bf16 values the reference's read returns - bf16((code + 128) *
+// scale + min) - right before use, so the results are those of bf16 attention over the dequantised cache.
+template <int D, int G>
+__global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(AttnArgs a) {
+  constexpr int NC = D / 32;        // bf16 uint4 of a K quarter-row after expansion
+  constexpr int NCB = (NC + 1) / 2; // uint4 of codes per K quarter-row (NC = 2: one 16-byte load)
+  constexpr int DC = D / 8;         // lanes covering one V row with 8-byte loads
+  constexpr int PP = 64 / DC;       // V rows fetched per load instruction
+  constexpr int NV = 32 / PP;       // V load instructions per 32-position tile
+  static_assert(NC >= 2, "head width 64 or 128");
+  const int split = blockIdx.z, kvh = blockIdx.y, b = blockIdx.x;  // b: query row = seq * S + s
+  const int seq = b / a.S;
+  const int L = min((a.pos_dev ? a.pos_dev[(size_t)seq * a.pos_stride] : a.start) + (b - seq * a.S) + 1, a.Tmax);
+  const int chunk = (((L + a.nsplit - 1) / a.nsplit) + 127) & ~127;
+  const int t0 = split * chunk;
+  const int t1 = min(L, t0 + chunk);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int p = lane >> 2, dq = lane & 3;  // position of the tile, quarter of its K row: a quad holds one row
+  const int pp = lane / DC, dc = lane % DC;
+
+  __shared__ float s_m[4][G], s_l[4][G];
+  __shared__ float s_acc[4][G][D];
+
+  uint4 qv[G][NC];  // q for this lane's contiguous quarter dq of the row
+#pragma unroll
+  for (int hh = 0; hh < G; ++hh)
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+      qv[hh][c] = ldg16(a.q + (size_t)b * a.H * D + (size_t)(kvh * G + hh) * D + (dq * NC + c) * 8);
+
+  float m_run[G], l_run[G], acc[G][8];
+#pragma unroll
+  for (int hh = 0; hh < G; ++hh) {
+    m_run[hh] = -INFINITY;
+    l_run[hh] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[hh][i] = 0.f;
+  }
+
+  const size_t row = (size_t)a.Hkv * D;
+  const int8_t* kb8 = reinterpret_cast<const int8_t*>(a.k) + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
+  const int8_t* vb8 = reinterpret_cast<const int8_t*>(a.v) + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
+  const float* stb = a.stats + ((size_t)seq * a.Hkv + kvh) * a.Tmax * 4;
+
+  struct Tile {
+    uint4 k[2][NCB];  // sub-tile s: codes of this lane's quarter of row tb + 16 s + p
+    uint2 v[NV];      // eight codes of row tb + c * PP + pp
+    uint4 st[2];      // (key scale, key min, value scale, value min) of position tb + 16 s + p
+  };
+  auto load_tile = [&](int tb, Tile& t) {
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      const int pos = tb + 16 * sb + p;
+      const bool in = pos < t1;
+      t.st[sb] = in ? ldg16(stb + (size_t)pos * 4) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int c = 0; c < NCB; ++c)
+        t.k[sb][c] = in ? ldg16_nt(kb8 + (size_t)pos * row + dq * (D / 4) + 16 * c) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+      const int vp = tb + c * PP + pp;
+      u32x2 w = (u32x2){0x80808080u, 0x80808080u};
+      if (vp < t1) w = __builtin_nontemporal_load((const OHARA_GLOBAL u32x2*)(vb8 + (size_t)vp * row + dc * 8));
+      t.v[c] = make_uint2(w.x, w.y);
+    }
+  };
+  Tile cur, nxt;
+  int tb = t0 + wave * 32;
+  if (tb < t1) load_tile(tb, cur);
+  for (; tb < t1; tb += 128) {
+    const bool more = tb + 128 < t1;
+    if (more) load_tile(tb + 128, nxt);
+    // One sub-tile of 16 positions at a time (both at once would need the registers of two expanded K
+    // tiles); within it the heads of the group advance together, as in the bf16 kernel.
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      float sc[G], pv[G];
+      {
+        const float ks = __uint_as_float(cur.st[sb].x), km = __uint_as_float(cur.st[sb].y);
+        uint4 kv[NC];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          const uint32_t* w = reinterpret_cast<const uint32_t*>(&cur.k[sb][c >> 1]) + 2 * (c & 1);
+          const uint2 lo = dequant4(w[0] ^ 0x80808080u, ks, km), hi = dequant4(w[1] ^ 0x80808080u, ks, km);
+          kv[c] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        }
+#pragma unroll
+        for (int hh = 0; hh < G; ++hh) {
+          float s = 0.f;
+#pragma unroll
+          for (int c = 0; c < NC; ++c) s = dot8(kv[c], qv[hh][c], s);
+          sc[hh] = s;
+        }
+      }
+#pragma unroll
+      for (int hh = 0; hh < G; ++hh) sc[hh] = quad_sum(sc[hh]);
+      const bool valid = tb + 16 * sb + p < t1;
+      bool raise = false;
+#pragma unroll
+      for (int hh = 0; hh < G; ++hh) {
+        sc[hh] = valid ? sc[hh] * a.scale : -INFINITY;
+        raise = raise || sc[hh] > m_run[hh];
+      }
+      if (__any(raise)) {
+        float tm[G];
+#pragma unroll
+        for (int hh = 0; hh < G; ++hh) tm[hh] = sc[hh];
+#pragma unroll
+        for (int o = 32; o > 2; o >>= 1)
+#pragma unroll
+          for (int hh = 0; hh < G; ++hh) tm[hh] = fmaxf(tm[hh], __shfl_xor(tm[hh], o, WAVE));
+#pragma unroll
+        for (int hh = 0; hh < G; ++hh) {
+          const float mn = fmaxf(m_run[hh], tm[hh]);  // finite here: some position of the sub-tile raised it
+          const float corr = __expf(m_run[hh] - mn);
+          m_run[hh] = mn;
+          l_run[hh] *= corr;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc[hh][i] *= corr;
+        }
+      }
+#pragma unroll
+      for (int hh = 0; hh < G; ++hh) {
+        pv[hh] = __expf(sc[hh] - m_run[hh]);  // (a sub-tile past the end: exp(-inf - m) = 0; m is finite by then)
+        l_run[hh] += pv[hh];
+      }
+#pragma unroll
+      for (int cc = 0; cc < NV / 2; ++cc) {
+        const int c = sb * (NV / 2) + cc;
+        const int src = 4 * ((c * PP + pp) & 15);  // a lane that owns the position of the row I hold eight codes of
+        const float vs = __shfl(__uint_as_float(cur.st[sb].z), src, WAVE);
+        const float vm = __shfl(__uint_as_float(cur.st[sb].w), src, WAVE);
+        const uint2 lo = dequant4(cur.v[c].x ^ 0x80808080u, vs, vm), hi = dequant4(cur.v[c].y ^ 0x80808080u, vs, vm);
+        const uint32_t w4[4] = {lo.x, lo.y, hi.x, hi.y};
+        float pw[G];
+#pragma unroll
+        for (int hh = 0; hh < G; ++hh) pw[hh] = __shfl(pv[hh], src, WAVE);
+#pragma unroll
+        for (int hh = 0; hh < G; ++hh)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            acc[hh][2 * i] += pw[hh] * lo_bf(w4[i]);
+            acc[hh][2 * i + 1] += pw[hh] * hi_bf(w4[i]);
+          }
+      }
+    }
+    if (more) cur = nxt;
+  }
+
+  // fold the sums over the 16 positions of a sub-tile, the PP row-groups of the wave, then the four waves
+#pragma unroll
+  for (int o = 32; o > 2; o >>= 1)
+#pragma unroll
+    for (int hh = 0; hh < G; ++hh) l_run[hh] += __shfl_xor(l_run[hh], o, WAVE);
+#pragma unroll
+  for (int hh = 0; hh < G; ++hh) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float v = acc[hh][i];
+#pragma unroll
+      for (int o = DC; o < 64; o <<= 1) v += __shfl_xor(v, o, WAVE);
+      acc[hh][i] = v;
+    }
+    if (lane < DC) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s_acc[wave][hh][dc * 8 + i] = acc[hh][i];
+    }
+    if (lane == 0) {
+      s_m[wave][hh] = m_run[hh];
+      s_l[wave][hh] = l_run[hh];
+    }
+  }
+  __syncthreads();
+  for (int idx = tid; idx < G * D; idx += 256) {
+    const int hh = idx / D, d = idx - hh * D;
+    const int h = kvh * G + hh;
+    float M = fmaxf(fmaxf(s_m[0][hh], s_m[1][hh]), fmaxf(s_m[2][hh], s_m[3][hh]));
+    float Ls = 0.f, o = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float mw = s_m[w][hh];
+      const float scw = (mw == -INFINITY) ? 0.f : __expf(mw - M);
+      Ls += s_l[w][hh] * scw;
+      o += s_acc[w][hh][d] * scw;
+    }
+    if (a.nsplit == 1) {  // whole context in this workgroup: no partials
+      a.out[(size_t)b * a.H * D + h * D + d] = f2bf(o / Ls);
+      continue;
+    }
+    const size_t pi = (size_t)(b * a.H + h) * a.nsplit + split;
+    stf_coh(a.part_acc + pi * D + d, o);
+    if (d == 0) {
+      stf_coh(a.part_ml + pi * 2, M);
+      stf_coh(a.part_ml + pi * 2 + 1, Ls);
+    }
+  }
+  if (a.nsplit == 1) return;
+  if (last_chunk_done(a.counters + b * a.Hkv + kvh, a.nsplit)) merge_partials<D>(a, b, kvh, G);
+}
+
 // Any even head width up to 256, any group size: one thread per position for q.k,
 // one thread per column for p.V.  Slow path for shapes the tuned kernel skips.
 template <bool I8>
@@ -390,7 +553,7 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
   // int8 mode: element (pos, d) is code * scale + min of its (pos, head) row, rounded to bf16
   const int8_t* kb8 = reinterpret_cast<const int8_t*>(a.k) + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
   const int8_t* vb8 = reinterpret_cast<const int8_t*>(a.v) + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
-  const size_t st0 = (size_t)seq * a.Tmax * a.Hkv + kvh;
+  const float* stb = I8 ? a.stats + ((size_t)seq * a.Hkv + kvh) * a.Tmax * 4 : nullptr;  // records of my (sequence, head)
   auto deq = [](int8_t c, float sc, float mn) {
     return bf2f(f2bf(__fadd_rn(__fmul_rn((float)((int)c + 128), sc), mn)));
   };
@@ -406,7 +569,7 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
       if (pos < t1) {
         float d_ = 0.f;
         if (I8) {
-          const float sc = a.kscale[st0 + (size_t)pos * a.Hkv], mn = a.kmin[st0 + (size_t)pos * a.Hkv];
+          const float sc = stb[(size_t)pos * 4], mn = stb[(size_t)pos * 4 + 1];
           for (int d = 0; d < D; ++d) d_ += s_q[d] * deq(kb8[(size_t)pos * row + d], sc, mn);
         } else {
           for (int d = 0; d < D; ++d) d_ += s_q[d] * bf2f(kb[(size_t)pos * row + d]);
@@ -433,8 +596,8 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
         const int n = min(256, t1 - tb);
         if (I8) {
           for (int i = 0; i < n; ++i) {
-            const size_t si = st0 + (size_t)(tb + i) * a.Hkv;
-            acc += s_p[i] * deq(vb8[(size_t)(tb + i) * row + tid], a.vscale[si], a.vmin[si]);
+            const float* rec = stb + (size_t)(tb + i) * 4;
+            acc += s_p[i] * deq(vb8[(size_t)(tb + i) * row + tid], rec[2], rec[3]);
           }
         } else {
           for (int i = 0; i < n; ++i) acc += s_p[i] * bf2f(vb[(size_t)(tb + i) * row + tid]);
@@ -459,10 +622,19 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
 
 template <int D, bool I8>
 int launch_fast(const AttnArgs& a, int G, dim3 grid, hipStream_t st) {
+  if (I8) {
+    switch (G) {
+      case 1: hipLaunchKernelGGL((attn_decode_i8_kernel<D, 1>), grid, dim3(256), 0, st, a); break;
+      case 2: hipLaunchKernelGGL((attn_decode_i8_kernel<D, 2>), grid, dim3(256), 0, st, a); break;
+      case 4: hipLaunchKernelGGL((attn_decode_i8_kernel<D, 4>), grid, dim3(256), 0, st, a); break;
+      default: return 1;
+    }
+    return 0;
+  }
   switch (G) {
-    case 1: hipLaunchKernelGGL((attn_decode_kernel<D, 1, I8>), grid, dim3(256), 0, st, a); break;
-    case 2: hipLaunchKernelGGL((attn_decode_kernel<D, 2, I8>), grid, dim3(256), 0, st, a); break;
-    case 4: hipLaunchKernelGGL((attn_decode_kernel<D, 4, I8>), grid, dim3(256), 0, st, a); break;
+    case 1: hipLaunchKernelGGL((attn_decode_kernel<D, 1>), grid, dim3(256), 0, st, a); break;
+    case 2: hipLaunchKernelGGL((attn_decode_kernel<D, 2>), grid, dim3(256), 0, st, a); break;
+    case 4: hipLaunchKernelGGL((attn_decode_kernel<D, 4>), grid, dim3(256), 0, st, a); break;
     default: return 1;
   }
   return 0;
@@ -484,12 +656,12 @@ int64_t ohara_attn_workspace_bytes(int batch, int h, int h_kv, int dh, int n_spl
 
 // `fixed_counter_bytes` > 0: the workspace keeps its counters in a region of that fixed size (the
 // layout of the allocation-free entry point, whose array is shared by calls of different shapes).
-static int attn_cached_impl(const uint16_t* q, const void* kcache, const void* vcache, const float* kscale,
-                            const float* kmin, const float* vscale, const float* vmin, bool i8, int batch, int seq_len,
+static int attn_cached_impl(const uint16_t* q, const void* kcache, const void* vcache, const float* stats, bool i8,
+                            int batch, int seq_len,
                             int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev, int pos_stride, int n_split,
                             void* workspace, uint16_t* out, void* stream, size_t fixed_counter_bytes = 0) {
   if (!q || !kcache || !vcache || !out) return OHARA_EINVAL;
-  if (i8 && (!kscale || !kmin || !vscale || !vmin)) return OHARA_EINVAL;
+  if (i8 && !stats) return OHARA_EINVAL;
   if (batch < 1 || seq_len < 1 || h < 1 || h_kv < 1 || h % h_kv || dh < 2 || (dh & 1) || dh > 256)
     return OHARA_EINVAL;
   if (t_max < 1 || n_split < 1 || n_split > 1024) return OHARA_EINVAL;
@@ -499,7 +671,7 @@ static int attn_cached_impl(const uint16_t* q, const void* kcache, const void* v
   if ((int64_t)batch * seq_len > INT32_MAX / 2 || h_kv > 65535) return OHARA_ESIZE;
   AttnArgs a{};
   a.q = q; a.k = reinterpret_cast<const bf16_t*>(kcache); a.v = reinterpret_cast<const bf16_t*>(vcache); a.out = out;
-  a.kscale = kscale; a.kmin = kmin; a.vscale = vscale; a.vmin = vmin;
+  a.stats = stats;
   a.B = batch; a.S = seq_len; a.H = h; a.Hkv = h_kv; a.D = dh; a.Tmax = t_max; a.start = pos; a.pos_dev = pos_dev;
   a.pos_stride = pos_stride;
   a.nsplit = n_split;
@@ -530,24 +702,23 @@ static int attn_cached_impl(const uint16_t* q, const void* kcache, const void* v
 int ohara_attn_cached_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch,
                            int seq_len, int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev,
                            int n_split, void* workspace, uint16_t* out, void* stream) {
-  return attn_cached_impl(q, kcache, vcache, nullptr, nullptr, nullptr, nullptr, false, batch, seq_len, h, h_kv, dh,
-                          t_max, pos, pos_dev, 0, n_split, workspace, out, stream);
+  return attn_cached_impl(q, kcache, vcache, nullptr, false, batch, seq_len, h, h_kv, dh, t_max, pos, pos_dev, 0,
+                          n_split, workspace, out, stream);
 }
 
 int ohara_attn_cached_ragged_bf16(const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache, int batch,
                                   int seq_len, int h, int h_kv, int dh, int t_max, const int32_t* seq_pos, int n_split,
                                   void* workspace, uint16_t* out, void* stream) {
   if (!seq_pos) return OHARA_EINVAL;
-  return attn_cached_impl(q, kcache, vcache, nullptr, nullptr, nullptr, nullptr, false, batch, seq_len, h, h_kv, dh,
-                          t_max, 0, seq_pos, 1, n_split, workspace, out, stream);
+  return attn_cached_impl(q, kcache, vcache, nullptr, false, batch, seq_len, h, h_kv, dh, t_max, 0, seq_pos, 1,
+                          n_split, workspace, out, stream);
 }
 
-int ohara_attn_cached_int8(const uint16_t* q, const int8_t* kcache, const int8_t* vcache, const float* kscale,
-                           const float* kmin, const float* vscale, const float* vmin, int batch, int seq_len, int h,
-                           int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev, int n_split, void* workspace,
-                           uint16_t* out, void* stream) {
-  return attn_cached_impl(q, kcache, vcache, kscale, kmin, vscale, vmin, true, batch, seq_len, h, h_kv, dh, t_max, pos,
-                          pos_dev, 0, n_split, workspace, out, stream);
+int ohara_attn_cached_int8(const uint16_t* q, const int8_t* kcache, const int8_t* vcache, const float* stats, int batch,
+                           int seq_len, int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev, int n_split,
+                           void* workspace, uint16_t* out, void* stream) {
+  return attn_cached_impl(q, kcache, vcache, stats, true, batch, seq_len, h, h_kv, dh, t_max, pos, pos_dev, 0, n_split,
+                          workspace, out, stream);
 }
 
 // ---- the same attention for callers that cannot allocate -------------------------------------
@@ -600,8 +771,8 @@ int ohara_attn_cached_bf16_noalloc(const uint16_t* q, const uint16_t* kcache, co
                        reinterpret_cast<int*>(ws), n);
     if (ohara_launch_status() != OHARA_OK) return OHARA_ELAUNCH;
   }
-  return attn_cached_impl(q, kcache, vcache, nullptr, nullptr, nullptr, nullptr, false, batch, seq_len, h, h_kv, dh,
-                          t_max, pos, pos_dev, 0, n_split, ws, out, stream, OHARA_SCRATCH_COUNTER_BYTES);
+  return attn_cached_impl(q, kcache, vcache, nullptr, false, batch, seq_len, h, h_kv, dh, t_max, pos, pos_dev, 0,
+                          n_split, ws, out, stream, OHARA_SCRATCH_COUNTER_BYTES);
 }
 
 }  // extern "C"

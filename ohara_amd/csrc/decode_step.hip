@@ -13,7 +13,7 @@
 extern "C" int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* s, int seq_len, int pos,
                                    int use_pos_dev, int logits_mode, int select_greedy, void* stream) {
   if (!m || !s || !m->layers || !s->kcache || !s->vcache) return OHARA_EINVAL;
-  if (s->kv_int8 && (!s->kscale || !s->kmin || !s->vscale || !s->vmin || !s->kstage || !s->vstage)) return OHARA_EINVAL;
+  if (s->kv_int8 && (!s->kvstats || !s->kstage || !s->vstage)) return OHARA_EINVAL;
   if (s->batch < 1 || seq_len < 1) return OHARA_EINVAL;
   const int64_t rows64 = (int64_t)s->batch * seq_len;
   if (rows64 > s->rows_cap) return OHARA_ESIZE;
@@ -73,18 +73,18 @@ extern "C" int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* 
       int8_t* vq = reinterpret_cast<int8_t*>(s->vcache[l]);
       OHARA_RUN(ohara_qkv_rope_bf16(tiled ? s->xn : s->x, d, L.wqkv, d, tiled ? nullptr : L.norm1, m->eps, B, seq_len, H,
                                     Hkv, Dh, m->cos, m->sin, pos, pos_dev, m->t_max, s->q, s->kstage, s->vstage, stream));
-      rc = ohara_kv_quant_append_int8(s->kstage, s->vstage, B, seq_len, Hkv, Dh, pos, pos_dev, kq, vq, s->kscale[l],
-                                      s->kmin[l], s->vscale[l], s->vmin[l], m->t_max, stream);
+      rc = ohara_kv_quant_append_int8(s->kstage, s->vstage, B, seq_len, Hkv, Dh, pos, pos_dev, kq, vq, s->kvstats[l],
+                                      m->t_max, stream);
       if (rc) return rc;
       if (seq_len >= 16 && (Dh == 64 || Dh == 128) && s->kdeq && s->vdeq) {
         const int len = pos + seq_len;
-        rc = ohara_kv_dequant_int8(kq, s->kscale[l], s->kmin[l], B, len, Hkv, Dh, m->t_max, s->kdeq, stream);
-        if (!rc) rc = ohara_kv_dequant_int8(vq, s->vscale[l], s->vmin[l], B, len, Hkv, Dh, m->t_max, s->vdeq, stream);
+        rc = ohara_kv_dequant_int8(kq, s->kvstats[l], 0, B, len, Hkv, Dh, m->t_max, s->kdeq, stream);
+        if (!rc) rc = ohara_kv_dequant_int8(vq, s->kvstats[l], 1, B, len, Hkv, Dh, m->t_max, s->vdeq, stream);
         if (rc) return rc;
         OHARA_RUN(ohara_attn_prefill_bf16(s->q, s->kdeq, s->vdeq, B, seq_len, H, Hkv, Dh, len, pos, s->attn, stream));
       } else {
-        OHARA_RUN(ohara_attn_cached_int8(s->q, kq, vq, s->kscale[l], s->kmin[l], s->vscale[l], s->vmin[l], B, seq_len, H,
-                                         Hkv, Dh, m->t_max, pos, pos_dev, n_split, s->attn_ws, s->attn, stream));
+        OHARA_RUN(ohara_attn_cached_int8(s->q, kq, vq, s->kvstats[l], B, seq_len, H, Hkv, Dh, m->t_max, pos, pos_dev,
+                                         n_split, s->attn_ws, s->attn, stream));
       }
     }
     OHARA_RUN(ohara_gemm_skinny_bf16(s->attn, H * Dh, L.wo, d, H * Dh, nullptr, m->eps, R, OHARA_EPI_RESIDUAL, s->x, d,

@@ -5,6 +5,11 @@
 // The reference computes the quantisation with tensor ops in the cache dtype (bf16), i.e. every
 // intermediate is rounded to bf16; the kernels round at the same points, so codes, scales and
 // minima are bit-identical to it.
+//
+// Statistics layout: one 16-byte record (key scale, key minimum, value scale, value minimum) per
+// (sequence, head, position), (Bcap, Hkv, Tmax, 4) fp32 - consecutive positions of a head are contiguous,
+// which is how decode attention walks them.  The reference's four (B, T, Hkv, 1) tensors are strided views
+// of it on the host side.
 #include "common.h"
 
 namespace {
@@ -12,8 +17,7 @@ namespace {
 // one wave per (row, head): D <= 512, D % 2 == 0
 __global__ __launch_bounds__(256) void kv_quant_append_kernel(const bf16_t* k, const bf16_t* v, int rows, int S, int Hkv,
                                                               int D, int pos0, const int32_t* pos_dev, int8_t* kq,
-                                                              int8_t* vq, float* kscale, float* kmin, float* vscale,
-                                                              float* vmin, int Tmax) {
+                                                              int8_t* vq, float* stats, int Tmax) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int item = blockIdx.x * 4 + wave;  // (tensor, row, head)
   if (item >= 2 * rows * Hkv) return;
@@ -54,13 +58,13 @@ __global__ __launch_bounds__(256) void kv_quant_append_kernel(const bf16_t* k, c
     }
   }
   if (lane == 0) {
-    (which ? vscale : kscale)[slot] = scale;
-    (which ? vmin : kmin)[slot] = mn;
+    float* rec = stats + (((size_t)seq * Hkv + h) * Tmax + pos) * 4 + 2 * which;
+    *reinterpret_cast<float2*>(rec) = make_float2(scale, mn);
   }
 }
 
 // (B, len) leading positions of an int8 cache -> bf16 (B, len, Hkv, D) contiguous (kv_cache.py:116-118)
-__global__ void kv_dequant_kernel(const int8_t* q, const float* scale, const float* mn, int len, int Hkv, int D, int Tmax,
+__global__ void kv_dequant_kernel(const int8_t* q, const float* stats, int which, int len, int Hkv, int D, int Tmax,
                                   bf16_t* out, size_t total) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;  // over (b, t, h, d/4)
   if (i >= total) return;
@@ -73,7 +77,8 @@ __global__ void kv_dequant_kernel(const int8_t* q, const float* scale, const flo
   const size_t b = bt / len;
   const size_t slot = (b * Tmax + t) * Hkv + h;
   const uint32_t w = *reinterpret_cast<const uint32_t*>(q + slot * D + 4 * c) ^ 0x80808080u;  // q + 128 as bytes
-  const float s = scale[slot], m = mn[slot];
+  const float2 sm = *reinterpret_cast<const float2*>(stats + ((b * Hkv + h) * (size_t)Tmax + t) * 4 + 2 * which);
+  const float s = sm.x, m = sm.y;
   float f[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) f[j] = __fadd_rn(__fmul_rn((float)((w >> (8 * j)) & 0xffu), s), m);
@@ -85,24 +90,23 @@ __global__ void kv_dequant_kernel(const int8_t* q, const float* scale, const flo
 extern "C" {
 
 int ohara_kv_quant_append_int8(const uint16_t* k, const uint16_t* v, int batch, int seq_len, int h_kv, int dh, int pos,
-                               const int32_t* pos_dev, int8_t* kq, int8_t* vq, float* kscale, float* kmin, float* vscale,
-                               float* vmin, int t_max, void* stream) {
-  if (!k || !v || !kq || !vq || !kscale || !kmin || !vscale || !vmin) return OHARA_EINVAL;
+                               const int32_t* pos_dev, int8_t* kq, int8_t* vq, float* stats, int t_max, void* stream) {
+  if (!k || !v || !kq || !vq || !stats) return OHARA_EINVAL;
   if (batch < 1 || seq_len < 1 || h_kv < 1 || dh < 2 || (dh & 3) || dh > 512 || t_max < 1) return OHARA_EINVAL;
   if (!pos_dev && (pos < 0 || pos + seq_len > t_max)) return OHARA_EINVAL;
   const int64_t items = (int64_t)2 * batch * seq_len * h_kv;
   if (items > INT32_MAX) return OHARA_ESIZE;
   hipLaunchKernelGGL(kv_quant_append_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, k, v,
-                     batch * seq_len, seq_len, h_kv, dh, pos, pos_dev, kq, vq, kscale, kmin, vscale, vmin, t_max);
+                     batch * seq_len, seq_len, h_kv, dh, pos, pos_dev, kq, vq, stats, t_max);
   return ohara_launch_status();
 }
 
-int ohara_kv_dequant_int8(const int8_t* q, const float* scale, const float* mn, int batch, int len, int h_kv, int dh,
+int ohara_kv_dequant_int8(const int8_t* q, const float* stats, int which, int batch, int len, int h_kv, int dh,
                           int t_max, uint16_t* out, void* stream) {
-  if (!q || !scale || !mn || !out || batch < 1 || len < 1 || len > t_max || h_kv < 1 || dh < 4 || (dh & 3)) return OHARA_EINVAL;
+  if (!q || !stats || which < 0 || which > 1 || !out || batch < 1 || len < 1 || len > t_max || h_kv < 1 || dh < 4 || (dh & 3)) return OHARA_EINVAL;
   const size_t total = (size_t)batch * len * h_kv * (dh / 4);
-  hipLaunchKernelGGL(kv_dequant_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, q, scale,
-                     mn, len, h_kv, dh, t_max, out, total);
+  hipLaunchKernelGGL(kv_dequant_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, q, stats,
+                     which, len, h_kv, dh, t_max, out, total);
   return ohara_launch_status();
 }
 

@@ -91,12 +91,14 @@ class KVCache:
         self.key = torch.zeros(shape, device=device, dtype=storage)
         self.value = torch.zeros(shape, device=device, dtype=storage)
         if self.int8:
-            # one scale / minimum per quantised row, i.e. per (batch, position, head): kv_cache.py:67-73
-            stats = (*shape[:-1], 1)
-            self.key_scale = torch.zeros(stats, device=device, dtype=torch.float32)
-            self.key_min = torch.zeros(stats, device=device, dtype=torch.float32)
-            self.value_scale = torch.zeros(stats, device=device, dtype=torch.float32)
-            self.value_min = torch.zeros(stats, device=device, dtype=torch.float32)
+            # One scale / minimum per quantised row, i.e. per (batch, position, head): kv_cache.py:67-73.
+            # Stored as one 16-byte record (key scale, key min, value scale, value min) per row with the
+            # positions of a head contiguous - (B, H_kv, T, 4), the order decode attention reads them in;
+            # the reference's four (B, T, H_kv, 1) tensors are strided views of it.
+            B_, T_, H_ = shape[0], shape[1], shape[2]
+            self.stats = torch.zeros((B_, H_, T_, 4), device=device, dtype=torch.float32)
+            self.key_scale, self.key_min, self.value_scale, self.value_min = (
+                self.stats[..., i:i + 1].permute(0, 2, 1, 3) for i in range(4))
 
     def _reserve(self, bsz: int, seq_len: int, start_pos: int) -> int:
         # ohara/modules/kv_cache.py:80-90, same order
@@ -358,10 +360,9 @@ class Llama:
             s.seq_pos = seq_pos.data_ptr()
             s._keep = (kc, vc, seq_pos)
         if kv_cache[0].int8:
-            stats = [(C.c_void_p * n)(*[getattr(c, nm).data_ptr() for c in kv_cache])
-                     for nm in ("key_scale", "key_min", "value_scale", "value_min")]
+            stats = [(C.c_void_p * n)(*[c.stats.data_ptr() for c in kv_cache])]
             s.kv_int8 = 1
-            s.kscale, s.kmin, s.vscale, s.vmin = (C.cast(a, C.POINTER(C.c_void_p)) for a in stats)
+            s.kvstats = C.cast(stats[0], C.POINTER(C.c_void_p))
             kvw = self.kv_heads * self.head_dim
             if buf.kstage is None:
                 buf.kstage = torch.empty(buf.rows, kvw, dtype=BF16, device=self.device)

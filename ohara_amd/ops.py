@@ -257,20 +257,17 @@ def kv_quant_append(keys, values, cache, pos, pos_dev=None):
     b, s_len, hkv, d = keys.shape
     check(lib().ohara_kv_quant_append_int8(
         _ptr(keys), _ptr(values), b, s_len, hkv, d, int(pos), _ptr(pos_dev), _ptr(cache.key), _ptr(cache.value),
-        _ptr(cache.key_scale), _ptr(cache.key_min), _ptr(cache.value_scale), _ptr(cache.value_min), cache.key.shape[1],
-        _stream()), "kv_quant_append")
+        _ptr(cache.stats), cache.key.shape[1], _stream()), "kv_quant_append")
 
 
 def kv_dequant(cache, which: str, batch: int, length: int, out=None) -> torch.Tensor:
     """The first `length` positions of the int8 cache's key or value tensor as bf16 (B, length, Hkv, D)."""
     q = cache.key if which == "key" else cache.value
-    scale = cache.key_scale if which == "key" else cache.value_scale
-    mn = cache.key_min if which == "key" else cache.value_min
     _, t_max, hkv, d = q.shape
     if out is None:
         out = torch.empty(batch, length, hkv, d, dtype=BF16, device=q.device)
-    check(lib().ohara_kv_dequant_int8(_ptr(q), _ptr(scale), _ptr(mn), batch, length, hkv, d, t_max, _ptr(out), _stream()),
-          "kv_dequant")
+    check(lib().ohara_kv_dequant_int8(_ptr(q), _ptr(cache.stats), 0 if which == "key" else 1, batch, length, hkv, d, t_max,
+                                      _ptr(out), _stream()), "kv_dequant")
     return out
 
 
@@ -280,9 +277,8 @@ def attn_cached_int8(q, cache, h, h_kv, dh, pos, n_split, workspace, out=None, p
     if out is None:
         out = torch.empty(rows, h * dh, dtype=BF16, device=q.device)
     check(lib().ohara_attn_cached_int8(
-        _ptr(q), _ptr(cache.key), _ptr(cache.value), _ptr(cache.key_scale), _ptr(cache.key_min), _ptr(cache.value_scale),
-        _ptr(cache.value_min), rows // seq_len, seq_len, h, h_kv, dh, cache.key.shape[1], int(pos), _ptr(pos_dev), n_split,
-        _ptr(workspace), _ptr(out), _stream()), "attn_cached_int8")
+        _ptr(q), _ptr(cache.key), _ptr(cache.value), _ptr(cache.stats), rows // seq_len, seq_len, h, h_kv, dh,
+        cache.key.shape[1], int(pos), _ptr(pos_dev), n_split, _ptr(workspace), _ptr(out), _stream()), "attn_cached_int8")
     return out
 
 

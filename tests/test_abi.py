@@ -44,9 +44,9 @@ def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(_lib.OharaLayer) == 6 * 8
     assert ctypes.sizeof(_lib.OharaModel) == 8 * 4 + 4 + 4 + 6 * 8
     assert _lib.OharaModel.token_emb.offset == 40
-    assert ctypes.sizeof(_lib.OharaDecodeState) == 6 * 4 + 12 * 8 + 8 + 8 * 8 + 3 * 8
-    assert _lib.OharaDecodeState.seq_pos.offset == 24 + 12 * 8 + 8 + 8 * 8
-    assert _lib.OharaDecodeState.kv_int8.offset == 24 + 12 * 8 and _lib.OharaDecodeState.kscale.offset == 24 + 13 * 8
+    assert ctypes.sizeof(_lib.OharaDecodeState) == 6 * 4 + 12 * 8 + 8 + 5 * 8 + 3 * 8
+    assert _lib.OharaDecodeState.seq_pos.offset == 24 + 12 * 8 + 8 + 5 * 8
+    assert _lib.OharaDecodeState.kv_int8.offset == 24 + 12 * 8 and _lib.OharaDecodeState.kvstats.offset == 24 + 13 * 8
     assert _lib.OharaDecodeState.xn.offset == 24 + 5 * 8
     assert _lib.OharaDecodeState.ids.offset == 24
 
