@@ -413,6 +413,56 @@ int64_t ohara_persistent_barrier_offset(const OharaModel* m, int batch, int n_sp
 int64_t ohara_persistent_error_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
 int64_t ohara_persistent_profile_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
 
+/* ---- one decode step of the BitNet-b1.58 Llama as ONE persistent launch (batch <= 8) --------
+ * Llama.forward(x, kv_cache, position) (ohara/models/llama.py:279-323) for one new token per
+ * sequence when the seven projections of every block are BitLinears
+ * (experiments/bitnet/bitnet.py:29-95, swapped in by apply_bitlinear :70-95 over the target list of
+ * experiments/bitnet/train_bitnet.py:240): per projection the BitLinear's own RMSNorm, the
+ * per-token int8 codes, the ternary product on the integer matrix cores and the rescale; block
+ * norms, rotary, cache append, attention, SwiGLU, residuals, the final norm, the bf16 vocabulary
+ * projection and the greedy selection as in ohara_llama_decode_persistent, whose calling
+ * convention (init_workspace, step_state, spin_limit, error word) this entry point shares.  The
+ * integer accumulators are those of ohara_bitlinear_* on the same rows; the reference's eager
+ * step is ~1700 launches.
+ * w[i] / norm_w[i] / gamma[i]: packed ternary weight (ohara_bitlinear_pack_ternary), the
+ * BitLinear's norm weight and weight scale of attn.query, attn.key, attn.value, attn.proj,
+ * ff.gate, ff.up, ff.down in that order.
+ * Requires head_dim 64 or 128, n_heads == n_kv_heads, d_model <= 4096, d_ff <= 6144, both
+ * multiples of 16; s->n_split must be 16; uses s->batch, valid_vocab, hist_cap, ids, logits,
+ * step_state, history, kcache, vcache. */
+#define OHARA_BIT_QUERY 0
+#define OHARA_BIT_KEY 1
+#define OHARA_BIT_VALUE 2
+#define OHARA_BIT_PROJ 3
+#define OHARA_BIT_GATE 4
+#define OHARA_BIT_UP 5
+#define OHARA_BIT_DOWN 6
+typedef struct OharaBitLayer {
+  const uint32_t* w[7];
+  const uint16_t* norm_w[7];
+  float gamma[7];
+  float reserved;
+  const uint16_t* norm1; /* (d) block norms */
+  const uint16_t* norm2;
+} OharaBitLayer;
+
+typedef struct OharaBitModel {
+  int32_t n_layers, d_model, n_heads, n_kv_heads, head_dim, d_ff, vocab, t_max;
+  float eps;
+  int32_t reserved;
+  const uint16_t* token_emb;  /* (vocab, d) row-major, unpacked */
+  const uint16_t* final_norm; /* (d) */
+  const uint16_t* w_vocab;    /* packed vocab_proj (vocab, d), bf16 (ohara_pack_rows_bf16) */
+  const uint16_t* cos;        /* (2*t_max, dh/2) bf16 */
+  const uint16_t* sin;
+  const OharaBitLayer* layers; /* host array [n_layers] */
+} OharaBitModel;
+
+int64_t ohara_bitnet_persistent_workspace_bytes(const OharaBitModel* m, int batch, int n_workgroups);
+int64_t ohara_bitnet_persistent_error_offset(const OharaBitModel* m, int batch, int n_workgroups);
+int ohara_bitnet_decode_persistent(const OharaBitModel* m, const OharaDecodeState* s, void* workspace, int n_workgroups,
+                                   int init_workspace, int select_greedy, unsigned int spin_limit, void* stream);
+
 /* ---- Phi (ohara/models/phi.py): the parts of its cached decode path that differ from Llama ----
  * nn.Linear WITH bias on packed weights (phi.py:46-47, :63-66, :161), any number of rows (up to 128:
  * the weight-streaming strip kernel, 64 rows per pass; more: the tiled MFMA kernel of ohara_gemm_bf16,

@@ -34,6 +34,20 @@ class OharaModel(C.Structure):
     ]
 
 
+class OharaBitLayer(C.Structure):
+    _fields_ = [("w", _p * 7), ("norm_w", _p * 7), ("gamma", _f * 7), ("reserved", _f), ("norm1", _p), ("norm2", _p)]
+
+
+class OharaBitModel(C.Structure):
+    _fields_ = [
+        ("n_layers", _i), ("d_model", _i), ("n_heads", _i), ("n_kv_heads", _i), ("head_dim", _i),
+        ("d_ff", _i), ("vocab", _i), ("t_max", _i),
+        ("eps", _f), ("reserved", _i),
+        ("token_emb", _p), ("final_norm", _p), ("w_vocab", _p), ("cos", _p), ("sin", _p),
+        ("layers", C.POINTER(OharaBitLayer)),
+    ]
+
+
 class OharaDecodeState(C.Structure):
     _fields_ = [
         ("batch", _i), ("rows_cap", _i), ("n_split", _i), ("valid_vocab", _i), ("hist_cap", _i), ("prof_kernel", _i),
@@ -96,6 +110,10 @@ _PROTOS = {
     "ohara_persistent_profile_offset": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),
     "ohara_llama_decode_persistent": (_i, [C.POINTER(OharaModel), C.POINTER(OharaDecodeState), _p, _i, _i, _i,
                                            C.c_uint, _p]),
+    "ohara_bitnet_persistent_workspace_bytes": (_i64, [C.POINTER(OharaBitModel), _i, _i]),
+    "ohara_bitnet_persistent_error_offset": (_i64, [C.POINTER(OharaBitModel), _i, _i]),
+    "ohara_bitnet_decode_persistent": (_i, [C.POINTER(OharaBitModel), C.POINTER(OharaDecodeState), _p, _i, _i, _i,
+                                            C.c_uint, _p]),
     "ohara_event_create": (_i, [C.POINTER(_p)]),
     "ohara_event_destroy": (_i, [_p]),
     "ohara_event_record": (_i, [_p, _p]),

@@ -31,13 +31,9 @@
 //
 // Every barrier wait is bounded: a workgroup that spins longer than the limit raises a
 // sticky error word and moves on, all later waits return at once, and the grid drains.
-#include "common.h"
+#include "persistent.h"
 
 namespace {
-
-#define OHARA_MEGA_NS 16  // context chunks per (sequence, kv head)
-#define OHARA_MAX_PF 24   // weight tiles (16 B per lane) a wave fetches ahead of a phase
-#define OHARA_DOWN_SPLIT 4  // K partitions of the down projection (static_assert below: x_load sums four)
 
 struct MegaArgs {
   OharaModel m;                 // by value; the layer table is read from layers_dev
@@ -64,816 +60,6 @@ struct MegaArgs {
   unsigned int spin_limit;
 };
 
-// Optional fine-grained timeline: thread 0 of workgroup 0 records the shader clock.
-struct Prof {
-  unsigned long long* p;
-  int n;
-  __device__ __forceinline__ void stamp() {
-    if (p) p[n] = __builtin_readcyclecounter();
-    ++n;
-  }
-};
-
-// ---------------------------------------------------------------------------------------
-// Grid barrier.  Two levels of monotonic counters (groups of 16 workgroups, each counter on
-// its own 256-byte line, then one counter over the groups) and a release word everyone
-// polls; a flat counter serialises 256 read-modify-writes on one address (~11 us here),
-// this takes ~1.6 us.  Words (uint32, stride 64 per counter): [g*64] group g, [ng*64] top,
-// [(ng+1)*64] release, [(ng+2)*64] sticky error, [(ng+3)*64] barriers completed by earlier
-// launches.  arrive() and wait() are split so that a workgroup can issue the loads of its
-// next phase (weights, cache tiles: nothing that depends on this phase) in between and
-// have them in flight while it waits.
-// ---------------------------------------------------------------------------------------
-#define OHARA_BAR_GROUP 16
-struct GridSync {
-  unsigned int* gc;
-  unsigned int* top;
-  unsigned int* rel;
-  unsigned int* err;
-  unsigned int* done;
-  unsigned int k;      // index of the next barrier (1-based, across launches)
-  unsigned int gsize;  // workgroups in my group
-  unsigned int ng;
-  unsigned int limit;
-  __device__ void init(unsigned int* bar, unsigned int nwg, unsigned int lim) {
-    ng = (nwg + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP;
-    const unsigned int g = blockIdx.x / OHARA_BAR_GROUP;
-    gsize = min((unsigned int)OHARA_BAR_GROUP, nwg - g * OHARA_BAR_GROUP);
-    gc = bar + g * 64;
-    top = bar + ng * 64;
-    rel = bar + (ng + 1) * 64;
-    err = bar + (ng + 2) * 64;
-    done = bar + (ng + 3) * 64;
-    limit = lim;
-    k = *done + 1;  // written by the previous launch (or the host): plain load
-  }
-  __device__ __forceinline__ void arrive(Prof& pf) {
-    pf.stamp();  // phase work issued
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // orders my LDS and global accesses within the workgroup
-    wait_own_stores();  // every wave: its sc1 stores have reached memory before the barrier below
-    pf.stamp();  // stores complete
-    __builtin_amdgcn_s_barrier();
-    pf.stamp();  // workgroup barrier passed
-    // The whole arrival happens here, before the caller's prefetch: the last workgroup of a group
-    // must not sit on the group's arrival while it issues loads.
-    if (threadIdx.x == 0) {
-      const unsigned int a = __hip_atomic_fetch_add(gc, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
-      if (a == k * gsize) {
-        const unsigned int t = __hip_atomic_fetch_add(top, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
-        if (t == k * ng) __hip_atomic_store(rel, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
-    asm volatile("" ::: "memory");  // compiler only: keep the caller's prefetch loads after this point
-    pf.stamp();  // arrival issued
-  }
-  __device__ __forceinline__ void wait(Prof& pf) {
-    pf.stamp();  // prefetch issued
-    if (threadIdx.x == 0) {
-      unsigned int spins = 0;
-      while ((int)(__hip_atomic_load(rel, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - k) < 0) {
-        ++spins;
-        if (spins > limit) {
-          __hip_atomic_store(err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          break;
-        }
-        if ((spins & 63u) == 0 && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
-        __builtin_amdgcn_s_sleep(1);
-      }
-    }
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): nothing of mine is still on its way to LDS
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");  // compiler only: mailbox loads of the next phase stay below the barrier
-    pf.stamp();  // barrier passed
-    ++k;
-  }
-};
-
-// A pointer from the workgroup's LDS copy of the layer table, made wave-uniform.
-template <typename T>
-__device__ __forceinline__ T* lds_ptr(const unsigned long long* tab, int i) {
-  const unsigned long long v = tab[i];
-  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
-  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-  return reinterpret_cast<T*>(((unsigned long long)hi << 32) | lo);
-}
-
-__device__ __forceinline__ float dot8m(uint4 a, uint4 b, float s) {
-  s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.x), __builtin_bit_cast(bf16x2, b.x), s, false);
-  s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.y), __builtin_bit_cast(bf16x2, b.y), s, false);
-  s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.z), __builtin_bit_cast(bf16x2, b.z), s, false);
-  s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.w), __builtin_bit_cast(bf16x2, b.w), s, false);
-  return s;
-}
-
-// Strip-blocked mailbox of a (B, N) bf16 matrix: the 16 columns [16s, 16s+16) of all rows
-// form block s of `blk` bytes (a multiple of 128), row b at byte b*32 inside it.
-__device__ __forceinline__ const char* xm_addr(const char* base, int blk, int b, int n) {
-  return base + (size_t)(n >> 4) * blk + b * 32 + (n & 15) * 2;
-}
-// act mailbox: 8 columns per block, row b at byte b*16.
-__device__ __forceinline__ const char* am_addr(const char* base, int blk, int b, int f) {
-  return base + (size_t)(f >> 3) * blk + b * 16 + (f & 7) * 2;
-}
-
-// The down projection is split along K over OHARA_DOWN_SPLIT groups of workgroups (a 16-row strip
-// of it is too much for one CU to stream); each group leaves fp32 partial sums and whoever needs
-// the residual stream after the block forms it on the fly, in a fixed order:
-//   x[b][n] = bf16(x_mid[b][n] + bf16(((p0 + p1) + p2) + p3))        (llama.py:200)
-// The sums are strip-blocked like the x mailbox, one block of `blk` bytes (a multiple of 128) per
-// (part, strip) with row b at byte b*64, so that every 128-byte line has a single writer.
-struct XParts {
-  const char* xmid;   // x mailbox holding the stream before the feed-forward block
-  const float* parts; // partial sums; nullptr: `xmid` already is the stream that is wanted
-  int blk, B, N;
-};
-__device__ __forceinline__ int pm_blk(int B) { return (B * 64 + 127) & ~127; }
-__device__ __forceinline__ const float* parts_addr(const float* base, int nstrips, int B, int q, int b, int n) {
-  return reinterpret_cast<const float*>(reinterpret_cast<const char*>(base) +
-                                        (size_t)(q * nstrips + (n >> 4)) * pm_blk(B) + b * 64) + (n & 15);
-}
-
-template <int NW>  // NW columns (4 or 8) starting at n, n % NW == 0
-__device__ __forceinline__ void x_load(const XParts& xp, int b, int n, uint32_t (&out)[NW / 2]) {
-  uint32_t xm[NW / 2];
-  if (NW == 8) {
-    const uint4 v = ldg16(xm_addr(xp.xmid, xp.blk, b, n));
-    xm[0] = v.x; xm[1] = v.y; xm[NW / 2 - 2] = v.z; xm[NW / 2 - 1] = v.w;
-  } else {
-    const uint2 v = ldg8(xm_addr(xp.xmid, xp.blk, b, n));
-    xm[0] = v.x; xm[1] = v.y;
-  }
-  if (!xp.parts) {
-#pragma unroll
-    for (int i = 0; i < NW / 2; ++i) out[i] = xm[i];
-    return;
-  }
-  uint4 pv[OHARA_DOWN_SPLIT][NW / 4];
-#pragma unroll
-  for (int q = 0; q < OHARA_DOWN_SPLIT; ++q)
-#pragma unroll
-    for (int i = 0; i < NW / 4; ++i) pv[q][i] = ldg16(parts_addr(xp.parts, (xp.N + 15) >> 4, xp.B, q, b, n + 4 * i));
-#pragma unroll
-  for (int i = 0; i < NW / 4; ++i) {
-    float y[4];
-    const uint32_t w[OHARA_DOWN_SPLIT][4] = {{pv[0][i].x, pv[0][i].y, pv[0][i].z, pv[0][i].w},
-                                             {pv[1][i].x, pv[1][i].y, pv[1][i].z, pv[1][i].w},
-                                             {pv[2][i].x, pv[2][i].y, pv[2][i].z, pv[2][i].w},
-                                             {pv[3][i].x, pv[3][i].y, pv[3][i].z, pv[3][i].w}};
-#pragma unroll
-    for (int e = 0; e < 4; ++e)
-      y[e] = rbf(((__uint_as_float(w[0][e]) + __uint_as_float(w[1][e])) + __uint_as_float(w[2][e])) +
-                 __uint_as_float(w[3][e]));
-    out[2 * i] = pack_bf(lo_bf(xm[2 * i]) + y[0], hi_bf(xm[2 * i]) + y[1]);
-    out[2 * i + 1] = pack_bf(lo_bf(xm[2 * i + 1]) + y[2], hi_bf(xm[2 * i + 1]) + y[3]);
-  }
-}
-
-// ---------------------------------------------------------------------------------------
-// staging of the GEMM activations in LDS: xs[b][ldxs] bf16
-// ---------------------------------------------------------------------------------------
-
-// norm.py:16-21 on rows of the residual stream (x-mailbox `src`), or - for the first layer
-// - on rows gathered from the embedding table (llama.py:310).  One wave per row; all loads
-// of a row are issued before any is consumed.  K <= 8 * 64 * NLD elements.
-template <int NLD, bool EMBED>
-__device__ void stage_norm(bf16_t* xs, int ldxs, const char* src, int blk, const float* parts, const int64_t* ids,
-                           const bf16_t* table, int vocab, const bf16_t* nw, float eps, int B, int K) {
-  const XParts xp{src, parts, blk, B, K};
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  for (int b = wave; b < B; b += 4) {
-    uint4 v[NLD], g[NLD];
-    size_t row_off = 0;
-    if (EMBED) {
-      int64_t id = ldg_i64(ids + b);
-      if (id < 0 || id >= vocab) id = 0;
-      row_off = (size_t)id * K;
-    }
-#pragma unroll
-    for (int c = 0; c < NLD; ++c) {
-      const int k = (c * 64 + lane) * 8;
-      v[c] = make_uint4(0, 0, 0, 0);
-      g[c] = make_uint4(0, 0, 0, 0);
-      if (k < K) {
-        if (EMBED) {
-          v[c] = ldg16(table + row_off + k);
-        } else {
-          uint32_t w[4];
-          x_load<8>(xp, b, k, w);
-          v[c] = make_uint4(w[0], w[1], w[2], w[3]);
-        }
-        g[c] = ldg16(nw + k);
-      }
-    }
-    float ss = 0.f;
-#pragma unroll
-    for (int c = 0; c < NLD; ++c) {
-      const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float a0 = lo_bf(w[i]), a1 = hi_bf(w[i]);
-        ss += a0 * a0 + a1 * a1;
-      }
-    }
-    ss = wave_sum(ss);
-    const float rinv = 1.0f / sqrtf(ss / (float)K + eps);
-#pragma unroll
-    for (int c = 0; c < NLD; ++c) {
-      const int k = (c * 64 + lane) * 8;
-      if (k < K) {
-        const uint32_t xv[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
-        const uint32_t gv[4] = {g[c].x, g[c].y, g[c].z, g[c].w};
-        uint32_t o[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          o[i] = pack_bf(rbf(lo_bf(xv[i]) * rinv) * lo_bf(gv[i]), rbf(hi_bf(xv[i]) * rinv) * hi_bf(gv[i]));
-        sts16(xs + (size_t)b * ldxs + k, make_uint4(o[0], o[1], o[2], o[3]));
-      }
-    }
-  }
-}
-
-// act mailbox (B, F) -> LDS
-// act mailbox (B, F), columns [f0, f1) (multiples of 8) -> LDS
-__device__ void stage_act(bf16_t* xs, int ldxs, const char* src, int blk, int B, int f0, int f1) {
-  const int n8 = (f1 - f0) >> 3;
-  for (int i = threadIdx.x; i < B * n8; i += blockDim.x) {
-    const int b = i / n8, c = (f0 >> 3) + i - b * n8;
-    sts16(xs + (size_t)b * ldxs + c * 8, ldg16(am_addr(src, blk, b, c * 8)));
-  }
-}
-
-// Merge of the attention partials of all chunks, in chunk order (llama.py:116-123 output,
-// rounded to bf16 as SDPA's result is) -> xs[b][h*Dh + d].  NS (a power of two) chunks are in use.
-// The (max, sum) pairs of every (sequence, head, chunk) are fetched in one round into LDS and
-// turned into chunk weights exp(m_s - M) and the sum L there; a thread then owns four adjacent
-// columns per pass and issues the accumulator loads of 16 / NS passes - 16 loads - before it uses
-// any, so the number of dependent load rounds does not grow with the chunk count times the batch.
-// `mw`: B*H*NS floats, `ml`: B*H floats of LDS.
-template <int NS>
-__device__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh, float* mw_, float* ml_) {
-  constexpr int NSM = OHARA_MEGA_NS, PR = 16 / NS;
-  const int HD = H * Dh, PS = Dh + 32;
-  const int nbh = B * H, total = B * HD;
-  const int pass = (int)blockDim.x * 4;
-  OHARA_LDS float* mw = (OHARA_LDS float*)mw_;
-  OHARA_LDS float* ml = (OHARA_LDS float*)ml_;
-  uint4 av[PR][NS];
-  auto load = [&](int e0) {
-#pragma unroll
-    for (int r = 0; r < PR; ++r) {
-      const int e = e0 + r * pass;
-      const int b = e / HD, hd = e - b * HD;
-      const float* base = pm + (size_t)(b * H + hd / Dh) * NSM * PS + (hd % Dh);
-#pragma unroll
-      for (int sp = 0; sp < NS; ++sp) av[r][sp] = e < total ? ldg16(base + (size_t)sp * PS) : make_uint4(0, 0, 0, 0);
-    }
-  };
-  // the accumulator loads of the first round go out first: they do not depend on the chunk
-  // weights, which are formed while they are in flight
-  load((int)threadIdx.x * 4);
-  // NS lanes per (sequence, head): lane sp holds chunk sp's (max, sum); max and weighted sum by
-  // shuffles inside the group
-  for (int i0 = 0; i0 < nbh * NS; i0 += blockDim.x) {
-    const int i = i0 + threadIdx.x;
-    const int bh = i / NS, sp = i % NS;
-    const bool in = bh < nbh;
-    float ms = -INFINITY, ls = 0.f;
-    if (in) {
-      const uint2 v = ldg8(pm + ((size_t)bh * NSM + sp) * PS + Dh);
-      ms = __uint_as_float(v.x);
-      ls = __uint_as_float(v.y);
-    }
-    float M = ms;
-#pragma unroll
-    for (int o = NS / 2; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, WAVE));
-    const float w = (ms == -INFINITY) ? 0.f : __expf(ms - M);
-    float Ls = ls * w;
-#pragma unroll
-    for (int o = NS / 2; o > 0; o >>= 1) Ls += __shfl_xor(Ls, o, WAVE);
-    if (in) mw[bh * NS + sp] = w;
-    if (in && sp == 0) ml[bh] = Ls;
-  }
-  __syncthreads();
-  for (int e0 = threadIdx.x * 4; e0 < total; e0 += pass * PR) {
-    if (e0 != (int)threadIdx.x * 4) load(e0);
-#pragma unroll
-    for (int r = 0; r < PR; ++r) {
-      const int e = e0 + r * pass;
-      if (e < total) {
-        const int b = e / HD, hd = e - b * HD;
-        const int bh = b * H + hd / Dh;
-        float o[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int sp = 0; sp < NS; ++sp) {
-          const float w = mw[bh * NS + sp];
-          o[0] += __uint_as_float(av[r][sp].x) * w;
-          o[1] += __uint_as_float(av[r][sp].y) * w;
-          o[2] += __uint_as_float(av[r][sp].z) * w;
-          o[3] += __uint_as_float(av[r][sp].w) * w;
-        }
-        const float Ls = ml[bh];
-        sts8(xs + (size_t)b * ldxs + hd, make_uint2(pack_bf(o[0] / Ls, o[1] / Ls), pack_bf(o[2] / Ls, o[3] / Ls)));
-      }
-    }
-  }
-}
-
-// One pass for the small case (all OHARA_MEGA_NS chunks in use, one group of four columns per
-// thread): every thread fetches the (max, sum) pairs itself, so there is a single round of loads
-// and no workgroup barrier.
-__device__ void stage_attn_merge_small(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh) {
-  constexpr int NS = OHARA_MEGA_NS;
-  const int HD = H * Dh, PS = Dh + 32;
-  const int e = threadIdx.x * 4;
-  if (e >= B * HD) return;
-  const int b = e / HD, hd = e - b * HD;
-  const int h = hd / Dh, d = hd - h * Dh;
-  const float* base = pm + (size_t)(b * H + h) * NS * PS;
-  uint2 mlv[NS];
-  uint4 av[NS];
-#pragma unroll
-  for (int s = 0; s < NS; ++s) {
-    mlv[s] = ldg8(base + (size_t)s * PS + Dh);
-    av[s] = ldg16(base + (size_t)s * PS + d);
-  }
-  float M = -INFINITY;
-#pragma unroll
-  for (int s = 0; s < NS; ++s) M = fmaxf(M, __uint_as_float(mlv[s].x));
-  float Ls = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int s = 0; s < NS; ++s) {
-    const float ms = __uint_as_float(mlv[s].x);
-    const float w = (ms == -INFINITY) ? 0.f : __expf(ms - M);
-    Ls += __uint_as_float(mlv[s].y) * w;
-    o[0] += __uint_as_float(av[s].x) * w;
-    o[1] += __uint_as_float(av[s].y) * w;
-    o[2] += __uint_as_float(av[s].z) * w;
-    o[3] += __uint_as_float(av[s].w) * w;
-  }
-  sts8(xs + (size_t)b * ldxs + hd, make_uint2(pack_bf(o[0] / Ls, o[1] / Ls), pack_bf(o[2] / Ls, o[3] / Ls)));
-}
-
-// ---------------------------------------------------------------------------------------
-// GEMM phase: strips of 16 packed rows, KP waves per strip, activations from LDS.  The
-// weights of a workgroup's first strip(s) - and the residual it will add - are fetched
-// into registers between arrive() and wait() of the barrier that precedes the phase.
-// ---------------------------------------------------------------------------------------
-enum { E_RESID = 1, E_SWIGLU = 2, E_ROPE = 3, E_LOGITS = 4, E_PART = 5 };
-
-struct GemmP {
-  const uint4* wp;
-  int N, K;        // logical rows (for E_SWIGLU: hidden width F) and columns
-  int nstrips;
-  char* out;       // output mailbox (E_ROPE: q; E_RESID: x; E_SWIGLU: act) or logits
-  int blk;         // its block size
-  const char* resid;      // E_RESID: x mailbox to add ...
-  const float* resid_parts;  // ... plus, when set, the partial sums of the previous block's down projection
-  int resid_embed;        // E_RESID: add the embedding rows instead (first half layer)
-  float* pout;            // E_PART: partial sums [part][b][n] (fp32, not rounded); K is split over
-                          // OHARA_DOWN_SPLIT groups of workgroups, unit = part * nstrips + strip
-  const int64_t* ids;     // E_RESID with resid == nullptr
-  const bf16_t* table;
-  int vocab;
-  int H, Hkv, Dh, Tmax, pos;
-  const bf16_t* cos;
-  const bf16_t* sin;
-  bf16_t* kc;
-  bf16_t* vc;
-  int valid;       // E_LOGITS: ids >= valid never win
-  int ldo;         // E_LOGITS: row stride of the logits
-};
-
-struct GemmPre {  // one register buffer, reused by every phase (only one prefetch is live at a time)
-  uint4 w[OHARA_MAX_PF];
-  uint2 r;        // E_RESID: the four residual values of this lane (first strip)
-};
-
-// Work unit -> strip and this wave's k-steps [j0, j1).  E_PART: the units of K partition q follow
-// those of partition q - 1, so the partitions of a strip land on different workgroups.
-template <int KP, int EPI>
-__device__ __forceinline__ bool gemm_unit(const GemmP& p, int unit, int kpart, int KS, int& strip, int& j0, int& j1) {
-  int kq = 0, KSq = KS;
-  strip = unit;
-  bool live = unit < p.nstrips;
-  if (EPI == E_PART) {
-    kq = unit / p.nstrips;
-    strip = unit - kq * p.nstrips;
-    KSq = (KS + OHARA_DOWN_SPLIT - 1) / OHARA_DOWN_SPLIT;
-    live = kq < OHARA_DOWN_SPLIT;
-  }
-  const int per = (KSq + KP - 1) / KP;
-  const int kend = min(KS, (kq + 1) * KSq);
-  j0 = kq * KSq + kpart * per;
-  j1 = min(kend, j0 + per);
-  return live;
-}
-
-template <int KP, int PF, int EPI>
-__device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int B) {
-  constexpr int SPW = 4 / KP;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int sub = wave / KP, kpart = wave % KP;
-  const int KS = (p.K + 31) >> 5;
-  int strip, j0, j1;
-  const bool live = gemm_unit<KP, EPI>(p, (int)blockIdx.x * SPW + sub, kpart, KS, strip, j0, j1);
-  const uint4* wrow = p.wp + (size_t)strip * KS * 64 + lane;
-#pragma unroll
-  for (int c = 0; c < PF; ++c)
-    pre.w[c] = (live && j0 + c < j1) ? ldg16_nt(wrow + (size_t)(j0 + c) * 64) : make_uint4(0, 0, 0, 0);
-  if (EPI == E_RESID) {
-    const int m = lane & 15, g = lane >> 4;
-    const int r0 = strip * 16 + 4 * g;
-    pre.r = make_uint2(0, 0);
-    if (live && kpart == 0 && m < B && r0 < p.N) {
-      if (!p.resid_embed) {
-        uint32_t w[2];
-        x_load<4>(XParts{p.resid, p.resid_parts, p.blk, B, p.N}, m, r0, w);
-        pre.r = make_uint2(w[0], w[1]);
-      } else {
-        int64_t id = ldg_i64(p.ids + m);
-        if (id < 0 || id >= p.vocab) id = 0;
-        pre.r = ldg8(p.table + (size_t)id * p.N + r0);
-      }
-    }
-  }
-}
-
-template <int KP, int PF, int EPI>
-__device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, const bf16_t* xs, int ldxs, int B,
-                                           float* red, float& best_v, int& best_i, Prof& pf) {
-  constexpr int SPW = 4 / KP;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int m = lane & 15, g = lane >> 4;
-  const int sub = wave / KP, kpart = wave % KP;
-  const int KS = (p.K + 31) >> 5;
-  const int nwg = gridDim.x;
-  const int nunits = EPI == E_PART ? p.nstrips * OHARA_DOWN_SPLIT : p.nstrips;
-  const int iters = (nunits + nwg * SPW - 1) / (nwg * SPW);
-  const bool mine = m < B;
-  const bf16_t* xrow = xs + (size_t)m * ldxs + 8 * g;
-
-#pragma unroll 1
-  for (int it = 0; it < iters; ++it) {
-    const int unit = (it * nwg + blockIdx.x) * SPW + sub;
-    int strip, j0, j1;
-    const bool live = gemm_unit<KP, EPI>(p, unit, kpart, KS, strip, j0, j1);
-    f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
-    if (live) {
-      const uint4* wrow = p.wp + (size_t)strip * KS * 64 + lane;
-#pragma unroll 1
-      for (int jc = j0; jc < j1; jc += PF) {
-        uint4 wv[PF];
-        if (it == 0 && jc == j0) {
-#pragma unroll
-          for (int c = 0; c < PF; ++c) wv[c] = pre.w[c];
-        } else {
-#pragma unroll
-          for (int c = 0; c < PF; ++c)
-            wv[c] = (jc + c < j1) ? ldg16_nt(wrow + (size_t)(jc + c) * 64) : make_uint4(0, 0, 0, 0);
-        }
-        // The activations of all PF k-steps are read from LDS before the first product: they do not
-        // depend on the weights, and left next to their products every read's latency is exposed
-        // (read, wait, product, PF times) on the critical path of the phase.
-        uint4 xv[PF];
-#pragma unroll
-        for (int c = 0; c < PF; ++c) {
-          xv[c] = make_uint4(0, 0, 0, 0);
-          if (mine && jc + c < j1 && 32 * (jc + c) + 8 * g < p.K)
-            xv[c] = *reinterpret_cast<const uint4*>(xrow + 32 * (jc + c));
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int c = 0; c < PF; ++c)
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wv[c]),
-                                                        __builtin_bit_cast(bf16x8, xv[c]), acc, 0, 0, 0);
-      }
-    }
-    if (it == 0) pf.stamp();  // MFMAs issued
-    if (KP > 1) {
-      if (kpart > 0) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) red[((wave * 64) + lane) * 4 + i] = acc[i];
-      }
-      __syncthreads();
-      if (kpart == 0) {
-        // all partial tiles are read before the first add (same order of adds; the reads overlap)
-        f32x4 part[KP > 1 ? KP - 1 : 1];
-#pragma unroll
-        for (int w = 1; w < KP; ++w) part[w - 1] = *reinterpret_cast<const f32x4*>(red + (((wave + w) * 64) + lane) * 4);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int w = 1; w < KP; ++w)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) acc[i] += part[w - 1][i];
-      }
-    }
-    if (it == 0) pf.stamp();  // cross-wave sum done
-    if (live && kpart == 0 && mine) {
-      const int b = m;
-      const int r0 = strip * 16 + 4 * g;
-      const float y0 = rbf(acc[0]), y1 = rbf(acc[1]), y2 = rbf(acc[2]), y3 = rbf(acc[3]);
-      if (EPI == E_RESID) {  // N % 4 == 0 is required by the entry point
-        if (r0 < p.N) {
-          uint2 r = pre.r;
-          if (it > 0) {
-            if (!p.resid_embed) {
-              uint32_t w[2];
-              x_load<4>(XParts{p.resid, p.resid_parts, p.blk, B, p.N}, b, r0, w);
-              r = make_uint2(w[0], w[1]);
-            } else {
-              int64_t id = ldg_i64(p.ids + b);
-              if (id < 0 || id >= p.vocab) id = 0;
-              r = ldg8(p.table + (size_t)id * p.N + r0);
-            }
-          }
-          st_coh8(const_cast<char*>(xm_addr(p.out, p.blk, b, r0)),
-                  make_uint2(pack_bf(lo_bf(r.x) + y0, hi_bf(r.x) + y1), pack_bf(lo_bf(r.y) + y2, hi_bf(r.y) + y3)));
-        }
-      } else if (EPI == E_PART) {  // the raw fp32 sums of this K partition
-        if (r0 < p.N) {
-          float* o = const_cast<float*>(parts_addr(p.pout, p.nstrips, B, unit / p.nstrips, b, r0));
-          st_coh8(o, make_uint2(__float_as_uint(acc[0]), __float_as_uint(acc[1])));
-          st_coh8(o + 2, make_uint2(__float_as_uint(acc[2]), __float_as_uint(acc[3])));
-        }
-      } else if (EPI == E_LOGITS) {
-        const float v[4] = {y0, y1, y2, y3};
-        bf16_t* o = reinterpret_cast<bf16_t*>(p.out) + (size_t)b * p.ldo + r0;
-        if (r0 + 3 < p.N && ((p.ldo & 3) == 0)) {
-          stg8(o, make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3])));
-        } else {
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (r0 + i < p.N) o[i] = f2bf(v[i]);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int id = r0 + i;
-          if (id < p.valid && (v[i] > best_v || (v[i] == best_v && id < best_i))) {
-            best_v = v[i];
-            best_i = id;
-          }
-        }
-      } else if (EPI == E_SWIGLU) {  // F % 8 == 0 is required by the entry point
-        const int f = strip * 8 + 2 * g;
-        if (f < p.N) {
-          const float s0 = rbf(silu_f(y0)), s1 = rbf(silu_f(y1));
-          st_coh4(const_cast<char*>(am_addr(p.out, p.blk, b, f)), pack_bf(s0 * y2, s1 * y3));
-        }
-      } else {  // E_ROPE
-        const int nq = p.H * p.Dh, nk = p.Hkv * p.Dh;
-        if (r0 < nq + 2 * nk && p.pos >= 0 && p.pos < p.Tmax) {
-          float v[4] = {y0, y1, y2, y3};
-          char* o;
-          if (r0 < nq + nk) {
-            const int d = (r0 < nq ? r0 : r0 - nq) % p.Dh;
-            const uint32_t cs = ldg4(p.cos + (size_t)p.pos * (p.Dh >> 1) + (d >> 1));
-            const uint32_t sn = ldg4(p.sin + (size_t)p.pos * (p.Dh >> 1) + (d >> 1));
-            const float c2[2] = {lo_bf(cs), hi_bf(cs)}, s2[2] = {lo_bf(sn), hi_bf(sn)};
-#pragma unroll
-            for (int pr = 0; pr < 2; ++pr) {
-              const float e = v[2 * pr], od = v[2 * pr + 1];
-              v[2 * pr] = __fsub_rn(__fmul_rn(e, c2[pr]), __fmul_rn(od, s2[pr]));
-              v[2 * pr + 1] = __fadd_rn(__fmul_rn(e, s2[pr]), __fmul_rn(od, c2[pr]));
-            }
-            o = (r0 < nq) ? const_cast<char*>(xm_addr(p.out, p.blk, b, r0))
-                          : reinterpret_cast<char*>(p.kc + (((size_t)b * p.Tmax + p.pos) * p.Hkv) * p.Dh + (r0 - nq));
-          } else {
-            o = reinterpret_cast<char*>(p.vc + (((size_t)b * p.Tmax + p.pos) * p.Hkv) * p.Dh + (r0 - nq - nk));
-          }
-          st_coh8(o, make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3])));
-        }
-      }
-    }
-    if (KP > 1) __syncthreads();
-  }
-}
-
-// ---------------------------------------------------------------------------------------
-// attention phase: items (sequence, kv head, chunk); writes partial triples.  The K/V
-// tiles of a wave's first 16 positions are fetched before the barrier.
-// ---------------------------------------------------------------------------------------
-template <int D>
-struct AttnPre {
-  uint4 k[D / 32];
-  uint4 v[D / 32];  // NV = 16 / (64 / (D / 8)) = D / 32
-};
-
-// One 16-position tile: positions >= t1 load nothing; position `coh_pos` (the row appended in
-// this step, or -1) is read with device-scope loads.
-template <int D>
-__device__ __forceinline__ void attn_tile_load(const bf16_t* kb, const bf16_t* vb, size_t row, int tb, int t1,
-                                               int coh_pos, uint4* kv, uint4* vv) {
-  constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
-  const int lane = threadIdx.x & 63;
-  const int p = lane & 15, dq = lane >> 4;
-  const int pp = lane / DC, dc = lane % DC;
-  const int pos = tb + p;
-#pragma unroll
-  for (int c = 0; c < NC; ++c) {
-    const bf16_t* src = kb + (size_t)pos * row + (4 * c + dq) * 8;
-    kv[c] = pos < t1 ? (pos == coh_pos ? ld_coh16(src) : ldg16_nt(src)) : make_uint4(0, 0, 0, 0);
-  }
-#pragma unroll
-  for (int c = 0; c < NV; ++c) {
-    const int vp = tb + c * PP + pp;
-    const bf16_t* src = vb + (size_t)vp * row + dc * 8;
-    vv[c] = vp < t1 ? (vp == coh_pos ? ld_coh16(src) : ldg16_nt(src)) : make_uint4(0, 0, 0, 0);
-  }
-}
-
-__device__ __forceinline__ void attn_item_range(int item, int ns, int Hkv, int L, int& b, int& kvh, int& split, int& t0,
-                                                int& t1) {
-  const int chunk = (((L + ns - 1) / ns) + 15) & ~15;
-  split = item % ns;
-  kvh = (item / ns) % Hkv;
-  b = item / (ns * Hkv);
-  t0 = split * chunk;
-  t1 = min(L, t0 + chunk);
-}
-
-// The first tile of each wave's first item, if it lies wholly below the row being appended.
-template <int D>
-__device__ __forceinline__ bool attn_first_tile_prefetchable(int t0, int t1, int L) {
-  const int tb = t0 + (threadIdx.x >> 6) * 16;
-  return tb + 16 <= min(t1, L - 1);
-}
-
-template <int D>
-__device__ __forceinline__ void attn_prefetch(int B, int Hkv, int Tmax, int ns, const bf16_t* kc, const bf16_t* vc,
-                                              int L, AttnPre<D>& pre) {
-  const int wave = threadIdx.x >> 6;
-  const size_t row = (size_t)Hkv * D;
-  int b, kvh, split, t0, t1;
-  attn_item_range(blockIdx.x, ns, Hkv, L, b, kvh, split, t0, t1);
-  const bool has = (int)blockIdx.x < B * Hkv * ns && attn_first_tile_prefetchable<D>(t0, t1, L);
-  const bf16_t* kb = kc + (size_t)b * Tmax * row + (size_t)kvh * D;
-  const bf16_t* vb = vc + (size_t)b * Tmax * row + (size_t)kvh * D;
-  attn_tile_load<D>(kb, vb, row, t0 + wave * 16, has ? t1 : 0, -1, pre.k, pre.v);
-}
-
-template <int D, int G>
-__device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int blk_x, int ns, const AttnPre<D>& pre,
-                                           const char* qm, float* pm, const bf16_t* kc, const bf16_t* vc, int L,
-                                           float* lds) {
-  constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int p = lane & 15;
-  const int dq = lane >> 4;
-  const int pp = lane / DC, dc = lane % DC;
-  const float scale = 1.0f / sqrtf((float)D);
-  float* s_m = lds;                 // [4][G]
-  float* s_l = lds + 4 * G;         // [4][G]
-  float* s_acc = lds + 8 * G;       // [4][G][D]
-  const int nitems = B * Hkv * ns;
-  const size_t row = (size_t)Hkv * D;
-  const int PS = D + 32;
-  bool first = true;
-  for (int item = blockIdx.x; item < nitems; item += gridDim.x) {
-    int b, kvh, split, t0, t1;
-    attn_item_range(item, ns, Hkv, L, b, kvh, split, t0, t1);
-    const bf16_t* kb = kc + (size_t)b * Tmax * row + (size_t)kvh * D;
-    const bf16_t* vb = vc + (size_t)b * Tmax * row + (size_t)kvh * D;
-    float m_run[G], l_run[G], acc[G][8];
-#pragma unroll
-    for (int hh = 0; hh < G; ++hh) {
-      m_run[hh] = -INFINITY;
-      l_run[hh] = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) acc[hh][i] = 0.f;
-    }
-    if (t0 + wave * 16 < t1) {
-      uint4 qv[G][NC];
-#pragma unroll
-      for (int hh = 0; hh < G; ++hh)
-#pragma unroll
-        for (int c = 0; c < NC; ++c)
-          qv[hh][c] = ldg16(xm_addr(qm, blk_x, b, (kvh * G + hh) * D + (4 * c + dq) * 8));
-      // the tile after the current one is in flight while the current one is consumed
-      const bool use_pre = first && attn_first_tile_prefetchable<D>(t0, t1, L);
-      uint4 kv[NC], vv[NV], kn[NC], vn[NV];
-      int tb = t0 + wave * 16;
-      if (use_pre) {
-#pragma unroll
-        for (int c = 0; c < NC; ++c) kv[c] = pre.k[c];
-#pragma unroll
-        for (int c = 0; c < NV; ++c) vv[c] = pre.v[c];
-      } else {
-        attn_tile_load<D>(kb, vb, row, tb, t1, L - 1, kv, vv);
-      }
-      for (; tb < t1; tb += 64) {
-        const bool valid = tb + p < t1;
-        const bool more = tb + 64 < t1;
-        if (more) attn_tile_load<D>(kb, vb, row, tb + 64, t1, L - 1, kn, vn);
-        // The heads of the group advance in lock step (their cross-lane exchanges overlap); l_run is
-        // this lane's share of the sum, folded over the 16 positions after the loop; the running
-        // maximum is re-derived only for tiles in which some score exceeds it.
-        float sc[G], pv[G];
-#pragma unroll
-        for (int hh = 0; hh < G; ++hh) {
-          float s = 0.f;
-#pragma unroll
-          for (int c = 0; c < NC; ++c) s = dot8m(kv[c], qv[hh][c], s);
-          sc[hh] = s;
-        }
-#pragma unroll
-        for (int hh = 0; hh < G; ++hh) sc[hh] += __shfl_xor(sc[hh], 16, WAVE);
-#pragma unroll
-        for (int hh = 0; hh < G; ++hh) sc[hh] += __shfl_xor(sc[hh], 32, WAVE);
-        bool raise = false;
-#pragma unroll
-        for (int hh = 0; hh < G; ++hh) {
-          sc[hh] = valid ? sc[hh] * scale : -INFINITY;
-          raise = raise || sc[hh] > m_run[hh];
-        }
-        if (__any(raise)) {
-          float tm[G];
-#pragma unroll
-          for (int hh = 0; hh < G; ++hh) tm[hh] = sc[hh];
-#pragma unroll
-          for (int o = 8; o > 0; o >>= 1)
-#pragma unroll
-            for (int hh = 0; hh < G; ++hh) tm[hh] = fmaxf(tm[hh], __shfl_xor(tm[hh], o, WAVE));
-#pragma unroll
-          for (int hh = 0; hh < G; ++hh) {
-            const float mn = fmaxf(m_run[hh], tm[hh]);
-            const float corr = __expf(m_run[hh] - mn);
-            m_run[hh] = mn;
-            l_run[hh] *= corr;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) acc[hh][i] *= corr;
-          }
-        }
-#pragma unroll
-        for (int hh = 0; hh < G; ++hh) {
-          pv[hh] = __expf(sc[hh] - m_run[hh]);
-          l_run[hh] += pv[hh];
-        }
-#pragma unroll
-        for (int c = 0; c < NV; ++c) {
-          const uint32_t w4[4] = {vv[c].x, vv[c].y, vv[c].z, vv[c].w};
-          float pw[G];
-#pragma unroll
-          for (int hh = 0; hh < G; ++hh) pw[hh] = __shfl(pv[hh], c * PP + pp, WAVE);
-#pragma unroll
-          for (int hh = 0; hh < G; ++hh)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              acc[hh][2 * i] += pw[hh] * lo_bf(w4[i]);
-              acc[hh][2 * i + 1] += pw[hh] * hi_bf(w4[i]);
-            }
-        }
-        if (more) {
-#pragma unroll
-          for (int c = 0; c < NC; ++c) kv[c] = kn[c];
-#pragma unroll
-          for (int c = 0; c < NV; ++c) vv[c] = vn[c];
-        }
-      }
-    }
-    first = false;
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1)
-#pragma unroll
-      for (int hh = 0; hh < G; ++hh) l_run[hh] += __shfl_xor(l_run[hh], o, WAVE);
-#pragma unroll
-    for (int hh = 0; hh < G; ++hh) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        float v = acc[hh][i];
-#pragma unroll
-        for (int o = DC; o < 64; o <<= 1) v += __shfl_xor(v, o, WAVE);
-        acc[hh][i] = v;
-      }
-      if (lane < DC) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) s_acc[(wave * G + hh) * D + dc * 8 + i] = acc[hh][i];
-      }
-      if (lane == 0) {
-        s_m[wave * G + hh] = m_run[hh];
-        s_l[wave * G + hh] = l_run[hh];
-      }
-    }
-    __syncthreads();
-    for (int idx = tid * 2; idx < G * D; idx += 512) {
-      const int hh = idx / D, d = idx - hh * D;
-      const int h = kvh * G + hh;
-      const float M = fmaxf(fmaxf(s_m[hh], s_m[G + hh]), fmaxf(s_m[2 * G + hh], s_m[3 * G + hh]));
-      float Ls = 0.f, o0 = 0.f, o1 = 0.f;
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        const float mw = s_m[w * G + hh];
-        const float sc = (mw == -INFINITY) ? 0.f : __expf(mw - M);
-        Ls += s_l[w * G + hh] * sc;
-        o0 += s_acc[(w * G + hh) * D + d] * sc;
-        o1 += s_acc[(w * G + hh) * D + d + 1] * sc;
-      }
-      float* dst = pm + ((size_t)(b * H + h) * OHARA_MEGA_NS + split) * PS;
-      st_coh8(dst + d, make_uint2(__float_as_uint(o0), __float_as_uint(o1)));
-      if (d == 0) st_coh8(dst + D, make_uint2(__float_as_uint(M), __float_as_uint(Ls)));
-    }
-    __syncthreads();
-  }
-}
 
 // ---------------------------------------------------------------------------------------
 // the kernel

@@ -49,6 +49,10 @@ def test_struct_layouts_match_the_header():
     assert _lib.OharaDecodeState.kv_int8.offset == 24 + 12 * 8 and _lib.OharaDecodeState.kvstats.offset == 24 + 13 * 8
     assert _lib.OharaDecodeState.xn.offset == 24 + 5 * 8
     assert _lib.OharaDecodeState.ids.offset == 24
+    assert ctypes.sizeof(_lib.OharaBitLayer) == 7 * 8 + 7 * 8 + 8 * 4 + 2 * 8
+    assert _lib.OharaBitLayer.gamma.offset == 112 and _lib.OharaBitLayer.norm1.offset == 144
+    assert ctypes.sizeof(_lib.OharaBitModel) == ctypes.sizeof(_lib.OharaModel)
+    assert _lib.OharaBitModel.layers.offset == _lib.OharaModel.layers.offset
 
 
 def test_argument_checks_need_no_gpu():
@@ -60,6 +64,11 @@ def test_argument_checks_need_no_gpu():
     assert L.ohara_gemm_skinny_bf16(0, 8, 0, 8, 8, 0, 1e-5, 1, 0, 0, 0, 0, 8, 0) == _lib.EINVAL
     assert L.ohara_attn_workspace_bytes(0, 1, 1, 1, 1) == _lib.EINVAL
     assert L.ohara_attn_workspace_bytes(2, 4, 2, 64, 8) > 0
+    assert L.ohara_bitnet_persistent_workspace_bytes(None, 1, 256) == _lib.EINVAL
+    bm = _lib.OharaBitModel()
+    bm.n_layers, bm.d_model, bm.n_heads, bm.n_kv_heads, bm.head_dim, bm.d_ff = 2, 256, 4, 4, 64, 512
+    assert L.ohara_bitnet_persistent_workspace_bytes(ctypes.byref(bm), 2, 256) > 0
+    assert L.ohara_bitnet_decode_persistent(ctypes.byref(bm), None, None, 256, 0, 1, 0, None) == _lib.EINVAL
     buf = (ctypes.c_int32 * 32)()
     assert L.ohara_swiglu_perm(12, buf) == 0
     # packed row 0..3 of strip 0: gate 0, gate 1, up 0, up 1 (up rows follow the 12 gate rows)

@@ -209,3 +209,75 @@ def test_bitnet_decode_at_larger_batches(cuda, B):
     close(model(ids[:, :5].to(cuda), cache, 0), ref(ids[:, :5], rc, 0))
     for t in (5, 6, 7):
         close(model(ids[:, t:t + 1].to(cuda), cache, t), ref(ids[:, t:t + 1], rc, t))
+
+
+PERSISTENT_SHAPES = [
+    # d, heads, d_ff, vocab, layers, batch
+    (256, 2, 512, 320, 3, 1),     # head_dim 128, one 256-column chunk per row
+    (256, 2, 512, 320, 3, 5),
+    (512, 8, 1536, 333, 2, 1),    # head_dim 64, several chunks, vocabulary not a multiple of 16
+    (512, 8, 1536, 333, 2, 8),
+    (320, 5, 528, 300, 2, 3),     # widths that are not multiples of 256 (zero-padded code rows)
+]
+
+
+@pytest.mark.parametrize("d,heads,ff,vocab,layers,B", PERSISTENT_SHAPES)
+def test_bitnet_persistent_step_matches_the_kernel_chain(cuda, d, heads, ff, vocab, layers, B):
+    """The single-launch ternary decode step against the chain of BitLinear kernels and the oracle:
+    the rows appended to layer 0's cache (no attention in front of them) bit for bit, nearly all
+    logits bit for bit, tokens from the captured graph equal to the eager launches."""
+    from ohara_amd.bitnet import BitLlama
+    from ohara_amd.llama import Config
+
+    kw = dict(vocab_size=vocab, hidden_size=d, intermediate_size=ff, num_attention_heads=heads,
+              num_key_value_heads=0, num_hidden_layers=layers, max_sequence_length=64, rope_theta=10000.0)
+    rcfg = R.RefConfig(**kw)
+    w = BL.init_ternary_weights(rcfg, seed=7, dtype=BF, gamma=0.05)
+    ref, model = R.RefLlama(rcfg, w), BitLlama(Config(**kw), w, device=cuda)
+    assert model.supports_persistent(B)
+    P, steps = 9, 12
+    ids = torch.randint(0, vocab, (B, P), generator=torch.Generator().manual_seed(B + d))
+
+    sess = model.session(B, steps, persistent=True)
+    sess.prefill(ids.to(cuda))
+    first = sess.ids.clone()
+    # chain: same prompt, same first token, one cached step
+    cache = model.build_kv_cache(B)
+    model(ids.to(cuda), cache, 0, last_only=True)
+    chain_logits = model(first.view(B, 1), cache, P, last_only=True)[:, 0]
+    sess.step()
+    torch.cuda.synchronize()
+    sess.check_error()
+    assert torch.equal(sess.cache[0].key[:, P], cache[0].key[:, P])
+    assert torch.equal(sess.cache[0].value[:, P], cache[0].value[:, P])
+    # oracle
+    rc = ref.build_kv_cache(B)
+    ref(ids, rc, 0)
+    want = ref(first.cpu().view(B, 1), rc, P)[:, -1].float()
+    scale = want.abs().max().item()
+    # at these small widths one int8 step of a code is a large relative change: the oracle distance of
+    # either path is the model's noise (the two paths are at the same distance from it)
+    for got, name in ((sess.logits, "persistent"), (chain_logits, "chain")):
+        e = (got.float().cpu() - want).abs()
+        assert e.max().item() <= 8e-2 * scale and e.mean().item() <= 1.5e-2 * scale, (name, e.max().item(), e.mean().item(), scale)
+    # against the chain: same codes, same integer sums, same rounding points; only the order of the
+    # fp32 sums inside attention differs, which can flip single bf16 roundings
+    same = (sess.logits == chain_logits).float().mean().item()
+    e = (sess.logits.float() - chain_logits.float()).abs()
+    assert same >= 0.98 and e.max().item() <= 2e-2 * scale, (same, e.max().item(), scale)
+    assert torch.equal(sess.ids, ops_argmax(sess.logits))
+    # the rest of the tokens from the graph; then the same tokens again from eager launches
+    sess.run(steps - 2)
+    toks = sess.tokens()
+    assert toks.shape == (B, steps)
+    again = model.generate_greedy(ids.to(cuda), steps, persistent=True, use_graph=False)
+    assert torch.equal(toks, again)
+    assert int(toks.min()) >= 0 and int(toks.max()) < vocab
+    chain = model.generate_greedy(ids.to(cuda), steps, persistent=False)
+    assert (toks == chain).float().mean().item() >= 0.9
+
+
+def ops_argmax(logits):
+    from ohara_amd import ops
+
+    return ops.argmax(logits.contiguous())
