@@ -370,7 +370,7 @@ def bitnet_c4_state(dev, n_layers=24, t_max=2048):
     return cfg, st
 
 
-def bench_bitnet(dev):
+def bench_bitnet(dev, batches=(1, 8)):
     """BitNet-b1.58 ternary Llama (d 2048, 24 layers, 16 x 128 heads, FFN 5632, vocab 32000):
     one decode step at context 2048, batch 1 and 8."""
     from ohara_amd.bitnet import BitLlama
@@ -381,7 +381,7 @@ def bench_bitnet(dev):
     del st
     out = []
     L = cfg.max_sequence_length
-    for B in (1, 8):
+    for B in batches:
         cache = model.build_kv_cache(B)
         ids = torch.randint(0, v, (B, 1), device=dev)
 
@@ -392,9 +392,28 @@ def bench_bitnet(dev):
         _fill_cache(cache, L - 1, B)
         t = graph_time(step)
         by = model.packed_weight_bytes() + 2.0 * v * d + 2.0 * 2 * d * cfg.num_hidden_layers * B * L
-        out.append({"batch": B, "context": L, "ms_per_step": round(t * 1e3, 4), "tokens_per_s": round(B / t, 1),
-                    "step_bytes": int(by), "GBs": round(by / t / 1e9, 1),
-                    "frac_of_hbm_peak": round(by / t / 1e9 / HBM_PEAK_GBS, 4)})
+        row = {"batch": B, "context": L, "launch": "chain of 5 kernels per layer", "ms_per_step": round(t * 1e3, 4),
+               "tokens_per_s": round(B / t, 1), "step_bytes": int(by), "GBs": round(by / t / 1e9, 1),
+               "frac_of_hbm_peak": round(by / t / 1e9 / HBM_PEAK_GBS, 4)}
+        out.append(row)
+        if model.supports_persistent(B):
+            # the single-launch step on the same caches: every replay starts from position L - 1 again
+            sess = model.session(B, 4, kv_cache=cache, persistent=True)
+            _fill_len(cache, 0, B)
+            sess.prefill(ids)
+            _fill_cache(cache, L - 1, B)
+            start = torch.tensor([L - 1, 1, 0, 0], dtype=torch.int32, device=dev)
+
+            def pstep():
+                sess.step_state.copy_(start)
+                sess._launch_step()
+
+            tp = graph_time(pstep)
+            sess.check_error()
+            out.append(dict(row, launch="one persistent kernel per step", ms_per_step=round(tp * 1e3, 4),
+                            tokens_per_s=round(B / tp, 1), GBs=round(by / tp / 1e9, 1),
+                            frac_of_hbm_peak=round(by / tp / 1e9 / HBM_PEAK_GBS, 4)))
+            del sess
         del cache
         torch.cuda.empty_cache()
     return out
@@ -617,6 +636,9 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters against)")
     ap.add_argument("--phase-timeline", action="store_true",
                     help="print the per-phase timeline of the persistent decode kernel at batch 1 and exit")
+    ap.add_argument("--bitnet-only", type=str, default="", metavar="BATCHES",
+                    help="run the BitNet ternary decode figures alone at these batch sizes (e.g. 1,8) and exit "
+                         "(profiling workload)")
     ap.add_argument("--phi-decode-only", type=int, default=0, metavar="B",
                     help="run 12 eager Phi-2 decode steps of B sequences at context 1024 and exit (profiling workload)")
     args = ap.parse_args()
@@ -633,6 +655,9 @@ def main():
     dev = torch.device("cuda:0")
     if args.phi_decode_only:
         print(json.dumps(phi_decode_only(dev, args.phi_decode_only)))
+        return
+    if args.bitnet_only:
+        print(json.dumps(bench_bitnet(dev, tuple(int(b) for b in args.bitnet_only.split(","))), indent=1))
         return
     if args.phase_timeline:
         print(json.dumps(phase_timeline(dev, args.prompt), indent=1))

@@ -427,8 +427,8 @@ int64_t ohara_persistent_profile_offset(const OharaModel* m, int batch, int n_sp
  * w[i] / norm_w[i] / gamma[i]: packed ternary weight (ohara_bitlinear_pack_ternary), the
  * BitLinear's norm weight and weight scale of attn.query, attn.key, attn.value, attn.proj,
  * ff.gate, ff.up, ff.down in that order.
- * Requires head_dim 64 or 128, n_heads == n_kv_heads, d_model <= 4096, d_ff <= 6144, both
- * multiples of 16; s->n_split must be 16; uses s->batch, valid_vocab, hist_cap, ids, logits,
+ * Requires head_dim 64 or 128, n_heads == n_kv_heads, d_model and n_heads * head_dim <= 2048,
+ * d_ff <= 6144, d_model and d_ff multiples of 16, n_workgroups >= 4; s->n_split must be 16; uses s->batch, valid_vocab, hist_cap, ids, logits,
  * step_state, history, kcache, vcache. */
 #define OHARA_BIT_QUERY 0
 #define OHARA_BIT_KEY 1
@@ -460,6 +460,10 @@ typedef struct OharaBitModel {
 
 int64_t ohara_bitnet_persistent_workspace_bytes(const OharaBitModel* m, int batch, int n_workgroups);
 int64_t ohara_bitnet_persistent_error_offset(const OharaBitModel* m, int batch, int n_workgroups);
+/* 1024 x uint64 shader-clock samples of workgroup 0 (six per grid barrier: phase work issued, own
+ * stores complete, workgroup barrier passed, arrival issued, prefetch issued, barrier passed), taken
+ * when s->prof_kernel == -2 (measurement only). */
+int64_t ohara_bitnet_persistent_profile_offset(const OharaBitModel* m, int batch, int n_workgroups);
 int ohara_bitnet_decode_persistent(const OharaBitModel* m, const OharaDecodeState* s, void* workspace, int n_workgroups,
                                    int init_workspace, int select_greedy, unsigned int spin_limit, void* stream);
 

@@ -112,6 +112,7 @@ _PROTOS = {
                                            C.c_uint, _p]),
     "ohara_bitnet_persistent_workspace_bytes": (_i64, [C.POINTER(OharaBitModel), _i, _i]),
     "ohara_bitnet_persistent_error_offset": (_i64, [C.POINTER(OharaBitModel), _i, _i]),
+    "ohara_bitnet_persistent_profile_offset": (_i64, [C.POINTER(OharaBitModel), _i, _i]),
     "ohara_bitnet_decode_persistent": (_i, [C.POINTER(OharaBitModel), C.POINTER(OharaDecodeState), _p, _i, _i, _i,
                                             C.c_uint, _p]),
     "ohara_event_create": (_i, [C.POINTER(_p)]),

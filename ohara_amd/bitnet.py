@@ -177,7 +177,7 @@ class BitLlama:
         """Shapes the single-launch ternary decode kernel covers."""
         c = self.config
         return (batch <= 8 and self.head_dim in (64, 128) and self.kv_heads == c.num_attention_heads
-                and c.hidden_size % 16 == 0 and c.intermediate_size % 16 == 0 and c.hidden_size <= 4096
+                and c.hidden_size % 16 == 0 and c.intermediate_size % 16 == 0 and c.hidden_size <= 2048
                 and c.intermediate_size <= 6144)
 
     def session(self, batch: int, max_new_tokens: int, valid_vocab: int = 0, kv_cache: list | None = None,
@@ -275,6 +275,7 @@ class BitDecodeSession:
             raise RuntimeError("persistent workspace query failed")
         self._pws = torch.zeros(nbytes, dtype=torch.uint8, device=m.device)
         self._err_off = lib().ohara_bitnet_persistent_error_offset(C.byref(m._c_model), B, self._nwg)
+        self._prof_off = lib().ohara_bitnet_persistent_profile_offset(C.byref(m._c_model), B, self._nwg)
         self._init_workspace()
 
     def _init_workspace(self) -> None:
@@ -317,6 +318,11 @@ class BitDecodeSession:
     def reset_error(self) -> None:
         if self.persistent and self._pws is not None:
             self._init_workspace()
+
+    def phase_clocks(self) -> torch.Tensor:
+        """Shader-clock samples of workgroup 0 at the barriers of the last step launched while
+        ``self._dst.prof_kernel`` was -2 (measurement aid)."""
+        return self._pws[self._prof_off : self._prof_off + 8192].view(torch.int64).cpu()
 
     def _room(self, n: int) -> None:
         if self.produced < 1:

@@ -45,7 +45,8 @@ struct BitMegaArgs {
   char* am;        // NL act-mailboxes
   float* pm;       // NL attention-partial mailboxes
   int32_t* dm;     // NL mailboxes of the down projection's int32 partial sums [part][strip][row][16]
-  float* ds;       // NL x 16 floats: the activation scale s of every row of the down projection
+  float* ds;       // NL x 32 floats (a 128-byte line per layer: one writer, written before it is read):
+                   // the activation scale s of every row of the down projection
   size_t xm_stride, qm_stride, am_stride, pm_stride, dm_stride;
   float* cand_val;
   int* cand_idx;
@@ -135,123 +136,94 @@ __device__ __forceinline__ float bit_sumsq8(uint4 v) {
   return s;
 }
 
-// ---- a row in LDS -> its int8 codes ------------------------------------------------------------
-// BitLinear's activation side (bitnet.py:29-33, 49-53) on a row of K bf16 values that already sits in
-// LDS (`row`, overwritten): [block RMSNorm with pre_w,] the BitLinear's RMSNorm with nw, s = 127 /
-// max|x_hat|, q = clamp(rint(x_hat * s), -128, 127).  The passes and the order of every reduction are
-// those of the stand-alone kernels (csrc/bitlinear.hip), so the codes are the same codes.
+// ---- a row -> its int8 codes -------------------------------------------------------------------
+// BitLinear's activation side (bitnet.py:29-33, 49-53) on a row of K bf16 values: [block RMSNorm with
+// pre_w,] the BitLinear's RMSNorm with nw, s = 127 / max|x_hat|, q = clamp(rint(x_hat * s), -128, 127).
+// Which thread owns which 8-value piece and the order of every reduction are those of the stand-alone
+// kernels (block_quant_row / wave_quant_row in csrc/bitlinear.hip), so the codes are the same codes.
 struct RowQ {
   float s;
   int sumq;
 };
 
-// one wave on the row; lane l owns the 8-value pieces l, l + 64, ...
-__device__ __forceinline__ RowQ wave_quant_lds(bf16_t* row, const bf16_t* pre_w, const bf16_t* nw, int K, float eps,
-                                               int8_t* xq) {
-  const int lane = threadIdx.x & 63;
-  const int pieces = K >> 3;
-  float ss = 0.f;
-  for (int p = lane; p < pieces; p += 64) ss += bit_sumsq8(lds16(row + p * 8));
-  if (pre_w) {
-    ss = wave_sum(ss);
-    const float rinv0 = 1.0f / sqrtf(ss / (float)K + eps);
-    ss = 0.f;
-    for (int p = lane; p < pieces; p += 64) {
-      const uint4 u = lds16(row + p * 8);
-      const uint4 w = ldg16(pre_w + (size_t)p * 8);
-      const uint32_t uu[4] = {u.x, u.y, u.z, u.w}, ww[4] = {w.x, w.y, w.z, w.w};
-      uint32_t o[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        o[j] = pack_bf(rbf(lo_bf(uu[j]) * rinv0) * lo_bf(ww[j]), rbf(hi_bf(uu[j]) * rinv0) * hi_bf(ww[j]));
-      const uint4 v = make_uint4(o[0], o[1], o[2], o[3]);
-      sts16(row + p * 8, v);
-      ss += bit_sumsq8(v);
-    }
+// LDS of the kernel.  `codes`: up to two code sets (gate and up) of B rows x ldq bytes; `stage`: B bf16
+// rows of the model width (the merged attention output, the normalised final stream).
+struct BitLds {
+  int8_t* codes;
+  int ldq;          // bytes per code row of the current phase (K padded to 256, + 16 against bank conflicts)
+  size_t set;       // bytes between the two code sets of the current phase
+  bf16_t* stage;
+  int ldm;          // elements between the rows of the merged attention output
+  int ldst;         // elements between the rows parked for ff.down's codes at batch > 1
+  __device__ __forceinline__ void shape(int B, int K) {
+    ldq = (((K + 255) >> 8) << 8) + 16;
+    set = (size_t)B * ldq;
   }
-  ss = wave_sum(ss);
-  const float rinv = 1.0f / sqrtf(ss / (float)K + eps);
-  float mx = 0.f;
-  for (int p = lane; p < pieces; p += 64) {
-    const uint4 u = lds16(row + p * 8);
-    const uint4 w = ldg16(nw + (size_t)p * 8);
-    const uint32_t uu[4] = {u.x, u.y, u.z, u.w}, ww[4] = {w.x, w.y, w.z, w.w};
-    uint32_t o[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float a0 = rbf(rbf(lo_bf(uu[j]) * rinv) * lo_bf(ww[j]));
-      const float a1 = rbf(rbf(hi_bf(uu[j]) * rinv) * hi_bf(ww[j]));
-      mx = fmaxf(mx, fmaxf(fabsf(a0), fabsf(a1)));
-      o[j] = pack_bf(a0, a1);
-    }
-    sts16(row + p * 8, make_uint4(o[0], o[1], o[2], o[3]));
-  }
-  mx = wave_max(mx);
-  const float s = 127.0f / fmaxf(mx, 1e-5f);
-  int sq = 0;
-  for (int p = lane; p < pieces; p += 64) {
-    const uint4 u = lds16(row + p * 8);
-    const uint32_t uu[4] = {u.x, u.y, u.z, u.w};
-    uint32_t pk[2] = {0u, 0u};
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float v = (j & 1) ? hi_bf(uu[j >> 1]) : lo_bf(uu[j >> 1]);
-      const int qi = (int)fminf(fmaxf(rintf(v * s), -128.f), 127.f);
-      sq += qi;
-      pk[j >> 2] |= ((uint32_t)qi & 0xffu) << (8 * (j & 3));
-    }
-    sts8(xq + (size_t)p * 8, make_uint2(pk[0], pk[1]));
-  }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, WAVE);
-  return RowQ{s, sq};
-}
+  float* s_s;       // [2][16] activation scales
+  int* s_sum;       // [2][16] sums of the codes
+  float* red;       // 4 KiB: cross-wave sums
+  int* sumw;        // [2][4] batch 1: per-wave shares of the sums of the codes
+};
 
-// the whole workgroup on one row (batch 1): thread t owns the pieces t, t + 256, ...; every thread calls
-__device__ __forceinline__ RowQ block_quant_lds(bf16_t* row, const bf16_t* pre_w, const bf16_t* nw, int K, float eps,
-                                                int8_t* xq, float* red) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int pieces = K >> 3;
-  auto bsum = [&](float v) {
-    v = wave_sum(v);
-    __syncthreads();
-    if (lane == 0) red[wave] = v;
-    __syncthreads();
-    return ((red[0] + red[1]) + red[2]) + red[3];
-  };
-  float ss = 0.f;
-  for (int p = tid; p < pieces; p += 256) ss += bit_sumsq8(lds16(row + p * 8));
-  if (pre_w) {
-    const float rinv0 = 1.0f / sqrtf(bsum(ss) / (float)K + eps);
-    ss = 0.f;
-    for (int p = tid; p < pieces; p += 256) {
-      const uint4 u = lds16(row + p * 8);
-      const uint4 w = ldg16(pre_w + (size_t)p * 8);
-      const uint32_t uu[4] = {u.x, u.y, u.z, u.w}, ww[4] = {w.x, w.y, w.z, w.w};
-      uint32_t o[4];
+// ---- batch 1: the row in registers -------------------------------------------------------------
+// Thread t owns the 8-value pieces t, t + 256, ... (NP of them; pieces beyond the row are zero and
+// change no sum or maximum); the row never goes through LDS, all loads (row, norm weights) are
+// in flight together, and the sum of the codes - needed only after the product - is left as four
+// per-wave partial sums.
+template <int NP, typename F>
+__device__ __forceinline__ void row1_load(uint4 (&r)[NP], int pieces, F f) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        o[j] = pack_bf(rbf(lo_bf(uu[j]) * rinv0) * lo_bf(ww[j]), rbf(hi_bf(uu[j]) * rinv0) * hi_bf(ww[j]));
-      const uint4 v = make_uint4(o[0], o[1], o[2], o[3]);
-      sts16(row + p * 8, v);
-      ss += bit_sumsq8(v);
-    }
+  for (int i = 0; i < NP; ++i) {
+    const int p = (int)threadIdx.x + 256 * i;
+    r[i] = p < pieces ? f(p) : make_uint4(0, 0, 0, 0);
   }
-  const float rinv = 1.0f / sqrtf(bsum(ss) / (float)K + eps);
-  float mx = 0.f;
-  for (int p = tid; p < pieces; p += 256) {
-    const uint4 u = lds16(row + p * 8);
-    const uint4 w = ldg16(nw + (size_t)p * 8);
-    const uint32_t uu[4] = {u.x, u.y, u.z, u.w}, ww[4] = {w.x, w.y, w.z, w.w};
+}
+__device__ __forceinline__ float row1_sum(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return ((red[0] + red[1]) + red[2]) + red[3];
+}
+// block-level RMSNorm (norm.py:16-21) of the row, in place
+template <int NP>
+__device__ __forceinline__ void row1_block_norm(uint4 (&v)[NP], const uint4 (&w)[NP], int K, float eps, float* red) {
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) ss += bit_sumsq8(v[i]);
+  const float rinv0 = 1.0f / sqrtf(row1_sum(ss, red) / (float)K + eps);
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const uint32_t uu[4] = {v[i].x, v[i].y, v[i].z, v[i].w}, ww[4] = {w[i].x, w[i].y, w[i].z, w[i].w};
     uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      o[j] = pack_bf(rbf(lo_bf(uu[j]) * rinv0) * lo_bf(ww[j]), rbf(hi_bf(uu[j]) * rinv0) * hi_bf(ww[j]));
+    v[i] = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+// the BitLinear's own norm, scale and codes of the row h (bitnet.py:29-33, 49-53) -> xq (LDS);
+// thread 0 leaves the scale in *s_out, every wave its share of the sum of the codes in sumw[wave]
+template <int NP>
+__device__ __forceinline__ void row1_codes(const uint4 (&h)[NP], const uint4 (&nw)[NP], int pieces, int K, float eps,
+                                           int8_t* xq, float* red, float* s_out, int* sumw) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) ss += bit_sumsq8(h[i]);
+  const float rinv = 1.0f / sqrtf(row1_sum(ss, red) / (float)K + eps);
+  // x_hat = bf16(bf16(h * rinv) * nw) is formed twice (for the maximum, then for the codes) instead
+  // of being kept: two multiplies per value against NP more live registers per row
+  float mx = 0.f;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const uint32_t uu[4] = {h[i].x, h[i].y, h[i].z, h[i].w}, ww[4] = {nw[i].x, nw[i].y, nw[i].z, nw[i].w};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const float a0 = rbf(rbf(lo_bf(uu[j]) * rinv) * lo_bf(ww[j]));
       const float a1 = rbf(rbf(hi_bf(uu[j]) * rinv) * hi_bf(ww[j]));
       mx = fmaxf(mx, fmaxf(fabsf(a0), fabsf(a1)));
-      o[j] = pack_bf(a0, a1);
     }
-    sts16(row + p * 8, make_uint4(o[0], o[1], o[2], o[3]));
   }
   mx = wave_max(mx);
   __syncthreads();
@@ -260,153 +232,289 @@ __device__ __forceinline__ RowQ block_quant_lds(bf16_t* row, const bf16_t* pre_w
   mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
   const float s = 127.0f / fmaxf(mx, 1e-5f);
   int sq = 0;
-  for (int p = tid; p < pieces; p += 256) {
-    const uint4 u = lds16(row + p * 8);
-    const uint32_t uu[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const uint32_t uu[4] = {h[i].x, h[i].y, h[i].z, h[i].w}, ww[4] = {nw[i].x, nw[i].y, nw[i].z, nw[i].w};
     uint32_t pk[2] = {0u, 0u};
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const float v = (j & 1) ? hi_bf(uu[j >> 1]) : lo_bf(uu[j >> 1]);
+      const float hv = (j & 1) ? hi_bf(uu[j >> 1]) : lo_bf(uu[j >> 1]);
+      const float wv = (j & 1) ? hi_bf(ww[j >> 1]) : lo_bf(ww[j >> 1]);
+      const float v = rbf(rbf(hv * rinv) * wv);
       const int qi = (int)fminf(fmaxf(rintf(v * s), -128.f), 127.f);
       sq += qi;
       pk[j >> 2] |= ((uint32_t)qi & 0xffu) << (8 * (j & 3));
     }
-    sts8(xq + (size_t)p * 8, make_uint2(pk[0], pk[1]));
+    const int p = tid + 256 * i;
+    if (p < pieces) sts8(xq + (size_t)p * 8, make_uint2(pk[0], pk[1]));
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, WAVE);
-  int* redi = reinterpret_cast<int*>(red);
-  __syncthreads();
-  if (lane == 0) redi[wave] = sq;
-  __syncthreads();
-  return RowQ{s, redi[0] + redi[1] + redi[2] + redi[3]};
+  if (lane == 0) sumw[wave] = sq;
+  if (tid == 0) *s_out = s;
 }
 
-// LDS of the kernel.  `codes`: up to two code sets (gate and up) of B rows x ldq bytes; `stage`: bf16
-// rows being turned into codes - B rows of the model width (attention output, all rows at once) or
-// four rows of the largest K (one per wave); row stride ldst elements.
-struct BitLds {
-  int8_t* codes;
-  int ldq;          // bytes per code row of the current phase (K padded to 256, + 16 against bank conflicts)
-  size_t set;       // bytes between the two code sets of the current phase
-  bf16_t* stage;
-  int ldst;         // elements between the rows being quantised (one per wave)
-  int ldm;          // elements between the rows of the merged attention output
-  __device__ __forceinline__ void shape(int B, int K) {
-    ldq = (((K + 255) >> 8) << 8) + 16;
-    set = (size_t)B * ldq;
+// Batch 1: one row from `load(piece) -> uint4` into one or two code sets (two BitLinears that share
+// the input and the block norm: ff.gate and ff.up).  Every thread of the workgroup calls.
+template <int NP, typename Load>
+__device__ __forceinline__ void bit_stage_row1(const BitLds& L, int nsets, int K, const bf16_t* pre_w, const bf16_t* nw0,
+                                               const bf16_t* nw1, float eps, Load load) {
+  const int tid = threadIdx.x;
+  const int pieces = K >> 3;
+  uint4 x[NP], pw[NP], n0[NP], n1[NP];
+  row1_load(x, pieces, load);
+  if (pre_w) row1_load(pw, pieces, [&](int p) { return ldg16(pre_w + (size_t)p * 8); });
+  row1_load(n0, pieces, [&](int p) { return ldg16(nw0 + (size_t)p * 8); });
+  if (nsets == 2) row1_load(n1, pieces, [&](int p) { return ldg16(nw1 + (size_t)p * 8); });
+  __syncthreads();  // whoever still reads the previous codes or scales is done
+  {
+    const int pad8 = (L.ldq - K) >> 3;
+    for (int i = tid; i < nsets * pad8; i += 256) {
+      const int st = i / pad8, c = i - st * pad8;
+      sts8(L.codes + (size_t)st * L.set + K + c * 8, make_uint2(0, 0));
+    }
   }
-  float* s_s;       // [2][16] activation scales
-  int* s_sum;       // [2][16] sums of the codes
-  float* red;       // 4 KiB: cross-wave sums
-};
+  if (pre_w) row1_block_norm(x, pw, K, eps, L.red);
+  row1_codes(x, n0, pieces, K, eps, L.codes, L.red, L.s_s, L.sumw);
+  if (nsets == 2) row1_codes(x, n1, pieces, K, eps, L.codes + L.set, L.red, L.s_s + 16, L.sumw + 4);
+  __syncthreads();
+  if (tid < nsets) L.s_sum[tid * 16] = (L.sumw[tid * 4] + L.sumw[tid * 4 + 1]) + (L.sumw[tid * 4 + 2] + L.sumw[tid * 4 + 3]);
+  // the product that follows passes a workgroup barrier before anyone reads s_sum
+}
 
-// Rows from `load(b, piece) -> uint4` into codes of set `set` (every thread of the workgroup calls).
-// pre_w: block norm weight or null.  The tail of every code row up to the padded K reads as zero.
-template <typename Load>
-__device__ __forceinline__ void bit_stage_codes(const BitLds& L, int set, int B, int K, const bf16_t* pre_w,
-                                                const bf16_t* nw, float eps, Load load) {
+// ---- batch > 1: a row per wave, in registers ---------------------------------------------------
+// Lane l owns the pieces l, l + 64, ... (NP of them); the norm weights are fetched once per wave and
+// serve all its rows.
+template <int NP, typename F>
+__device__ __forceinline__ void roww_load(uint4 (&r)[NP], int pieces, F f) {
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const int p = (int)(threadIdx.x & 63) + 64 * i;
+    r[i] = p < pieces ? f(p) : make_uint4(0, 0, 0, 0);
+  }
+}
+template <int NP>
+__device__ __forceinline__ void roww_block_norm(uint4 (&v)[NP], const uint4 (&w)[NP], int K, float eps) {
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) ss += bit_sumsq8(v[i]);
+  const float rinv0 = 1.0f / sqrtf(wave_sum(ss) / (float)K + eps);
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const uint32_t uu[4] = {v[i].x, v[i].y, v[i].z, v[i].w}, ww[4] = {w[i].x, w[i].y, w[i].z, w[i].w};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      o[j] = pack_bf(rbf(lo_bf(uu[j]) * rinv0) * lo_bf(ww[j]), rbf(hi_bf(uu[j]) * rinv0) * hi_bf(ww[j]));
+    v[i] = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+template <int NP>
+__device__ __forceinline__ RowQ roww_codes(const uint4 (&h)[NP], const uint4 (&nw)[NP], int pieces, int K, float eps,
+                                           int8_t* xq) {
+  const int lane = threadIdx.x & 63;
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) ss += bit_sumsq8(h[i]);
+  const float rinv = 1.0f / sqrtf(wave_sum(ss) / (float)K + eps);
+  // x_hat = bf16(bf16(h * rinv) * nw) is formed twice (for the maximum, then for the codes) instead
+  // of being kept: two multiplies per value against NP more live registers per row
+  float mx = 0.f;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const uint32_t uu[4] = {h[i].x, h[i].y, h[i].z, h[i].w}, ww[4] = {nw[i].x, nw[i].y, nw[i].z, nw[i].w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float a0 = rbf(rbf(lo_bf(uu[j]) * rinv) * lo_bf(ww[j]));
+      const float a1 = rbf(rbf(hi_bf(uu[j]) * rinv) * hi_bf(ww[j]));
+      mx = fmaxf(mx, fmaxf(fabsf(a0), fabsf(a1)));
+    }
+  }
+  mx = wave_max(mx);
+  const float s = 127.0f / fmaxf(mx, 1e-5f);
+  int sq = 0;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const uint32_t uu[4] = {h[i].x, h[i].y, h[i].z, h[i].w}, ww[4] = {nw[i].x, nw[i].y, nw[i].z, nw[i].w};
+    uint32_t pk[2] = {0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float hv = (j & 1) ? hi_bf(uu[j >> 1]) : lo_bf(uu[j >> 1]);
+      const float wv = (j & 1) ? hi_bf(ww[j >> 1]) : lo_bf(ww[j >> 1]);
+      const float v = rbf(rbf(hv * rinv) * wv);
+      const int qi = (int)fminf(fmaxf(rintf(v * s), -128.f), 127.f);
+      sq += qi;
+      pk[j >> 2] |= ((uint32_t)qi & 0xffu) << (8 * (j & 3));
+    }
+    const int p = lane + 64 * i;
+    if (p < pieces) sts8(xq + (size_t)p * 8, make_uint2(pk[0], pk[1]));
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, WAVE);
+  return RowQ{s, sq};
+}
+// B rows from `load(b, piece) -> uint4` into one or two code sets.  Every thread of the workgroup calls.
+template <int NP, typename Load>
+__device__ __forceinline__ void bit_stage_roww(const BitLds& L, int nsets, int B, int K, const bf16_t* pre_w,
+                                               const bf16_t* nw0, const bf16_t* nw1, float eps, Load load) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int pieces = K >> 3;
-  int8_t* xq = L.codes + (size_t)set * L.set;
-  __syncthreads();  // whoever still reads the previous codes, scales or staged rows is done
-  // zero the padding columns [K, ldq) of the rows in use (K is a multiple of 8, ldq of 16)
+  uint4 pw[NP], n0[NP], n1[NP];
+  if (pre_w) roww_load(pw, pieces, [&](int p) { return ldg16(pre_w + (size_t)p * 8); });
+  roww_load(n0, pieces, [&](int p) { return ldg16(nw0 + (size_t)p * 8); });
+  if (nsets == 2) roww_load(n1, pieces, [&](int p) { return ldg16(nw1 + (size_t)p * 8); });
+  __syncthreads();  // whoever still reads the previous codes or scales is done
   {
     const int pad8 = (L.ldq - K) >> 3;
-    for (int i = tid; i < B * pad8; i += 256) {
-      const int b = i / pad8, c = i - b * pad8;
-      sts8(xq + (size_t)b * L.ldq + K + c * 8, make_uint2(0, 0));
+    for (int i = tid; i < nsets * B * pad8; i += 256) {
+      const int r = i / pad8, c = i - r * pad8;  // r = set * B + row; the sets are B rows apart
+      sts8(L.codes + (size_t)r * L.ldq + K + c * 8, make_uint2(0, 0));
     }
   }
-  if (B == 1) {
-    for (int p = tid; p < pieces; p += 256) sts16(L.stage + p * 8, load(0, p));
-    __syncthreads();
-    const RowQ o = block_quant_lds(L.stage, pre_w, nw, K, eps, xq, L.red);
-    if (tid == 0) {
-      L.s_s[set * 16] = o.s;
-      L.s_sum[set * 16] = o.sumq;
+  for (int b = wave; b < B; b += 4) {
+    uint4 x[NP];
+    roww_load(x, pieces, [&](int p) { return load(b, p); });
+    if (pre_w) roww_block_norm(x, pw, K, eps);
+    const RowQ o0 = roww_codes(x, n0, pieces, K, eps, L.codes + (size_t)b * L.ldq);
+    if (lane == 0) {
+      L.s_s[b] = o0.s;
+      L.s_sum[b] = o0.sumq;
     }
-  } else {
-    bf16_t* row = L.stage + (size_t)wave * L.ldst;
-    for (int b = wave; b < B; b += 4) {
-      for (int p = lane; p < pieces; p += 64) sts16(row + p * 8, load(b, p));
-      const RowQ o = wave_quant_lds(row, pre_w, nw, K, eps, xq + (size_t)b * L.ldq);
+    if (nsets == 2) {
+      const RowQ o1 = roww_codes(x, n1, pieces, K, eps, L.codes + L.set + (size_t)b * L.ldq);
       if (lane == 0) {
-        L.s_s[set * 16 + b] = o.s;
-        L.s_sum[set * 16 + b] = o.sumq;
+        L.s_s[16 + b] = o1.s;
+        L.s_sum[16 + b] = o1.sumq;
       }
     }
   }
   __syncthreads();
 }
 
-// The same when the rows already sit in `stage` (row b at b * ldst): the merged attention output.
-__device__ __forceinline__ void bit_codes_from_stage(const BitLds& L, int set, int B, int K, const bf16_t* nw, float eps) {
+// The same for rows too long for registers (ff.down's input at batch > 1: one code set, no block
+// norm): the wave parks its rows in LDS (`stage`, row b at b * ldst) as they arrive - all loads of all
+// its rows in flight together - and walks them three times from there; only the norm weights stay in
+// registers.  A lane reads back only what it wrote itself, so the rows need no barrier.
+template <int NP, typename Load>
+__device__ __forceinline__ void bit_stage_roww_lds(const BitLds& L, int B, int K, const bf16_t* nw0, float eps, Load load) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  int8_t* xq = L.codes + (size_t)set * L.set;
-  __syncthreads();  // the merged rows are complete; the previous codes and scales are no longer read
+  const int pieces = K >> 3;
+  uint4 n0[NP];
+  roww_load(n0, pieces, [&](int p) { return ldg16(nw0 + (size_t)p * 8); });
+  __syncthreads();  // whoever still reads the previous codes, scales or staged rows is done
   {
     const int pad8 = (L.ldq - K) >> 3;
     for (int i = tid; i < B * pad8; i += 256) {
-      const int b = i / pad8, c = i - b * pad8;
-      sts8(xq + (size_t)b * L.ldq + K + c * 8, make_uint2(0, 0));
+      const int r = i / pad8, c = i - r * pad8;
+      sts8(L.codes + (size_t)r * L.ldq + K + c * 8, make_uint2(0, 0));
     }
   }
-  if (B == 1) {
-    const RowQ o = block_quant_lds(L.stage, nullptr, nw, K, eps, xq, L.red);
-    if (tid == 0) {
-      L.s_s[set * 16] = o.s;
-      L.s_sum[set * 16] = o.sumq;
+  for (int b = wave; b < B; b += 4) {
+    bf16_t* row = L.stage + (size_t)b * L.ldst;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = lane + 64 * i;
+      if (p < pieces) sts16(row + p * 8, load(b, p));
     }
-  } else {
-    for (int b = wave; b < B; b += 4) {
-      const RowQ o = wave_quant_lds(L.stage + (size_t)b * L.ldm, nullptr, nw, K, eps, xq + (size_t)b * L.ldq);
-      if (lane == 0) {
-        L.s_s[set * 16 + b] = o.s;
-        L.s_sum[set * 16 + b] = o.sumq;
+  }
+  for (int b = wave; b < B; b += 4) {
+    const bf16_t* row = L.stage + (size_t)b * L.ldst;
+    int8_t* xq = L.codes + (size_t)b * L.ldq;
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = lane + 64 * i;
+      ss += bit_sumsq8(p < pieces ? lds16(row + p * 8) : make_uint4(0, 0, 0, 0));
+    }
+    const float rinv = 1.0f / sqrtf(wave_sum(ss) / (float)K + eps);
+    float mx = 0.f;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = lane + 64 * i;
+      const uint4 h = p < pieces ? lds16(row + p * 8) : make_uint4(0, 0, 0, 0);
+      const uint32_t uu[4] = {h.x, h.y, h.z, h.w}, ww[4] = {n0[i].x, n0[i].y, n0[i].z, n0[i].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float a0 = rbf(rbf(lo_bf(uu[j]) * rinv) * lo_bf(ww[j]));
+        const float a1 = rbf(rbf(hi_bf(uu[j]) * rinv) * hi_bf(ww[j]));
+        mx = fmaxf(mx, fmaxf(fabsf(a0), fabsf(a1)));
       }
+    }
+    mx = wave_max(mx);
+    const float s = 127.0f / fmaxf(mx, 1e-5f);
+    int sq = 0;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = lane + 64 * i;
+      if (p < pieces) {
+        const uint4 h = lds16(row + p * 8);
+        const uint32_t uu[4] = {h.x, h.y, h.z, h.w}, ww[4] = {n0[i].x, n0[i].y, n0[i].z, n0[i].w};
+        uint32_t pk[2] = {0u, 0u};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float hv = (j & 1) ? hi_bf(uu[j >> 1]) : lo_bf(uu[j >> 1]);
+          const float wv = (j & 1) ? hi_bf(ww[j >> 1]) : lo_bf(ww[j >> 1]);
+          const float v = rbf(rbf(hv * rinv) * wv);
+          const int qi = (int)fminf(fmaxf(rintf(v * s), -128.f), 127.f);
+          sq += qi;
+          pk[j >> 2] |= ((uint32_t)qi & 0xffu) << (8 * (j & 3));
+        }
+        sts8(xq + (size_t)p * 8, make_uint2(pk[0], pk[1]));
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, WAVE);
+    if (lane == 0) {
+      L.s_s[b] = s;
+      L.s_sum[b] = sq;
     }
   }
   __syncthreads();
 }
 
 // ---- one strip of a ternary weight x the code rows ---------------------------------------------
-// Chunks [cb, ce) of 256 columns, split over the four waves; the sum over the waves lands in wave 0
-// (returns true there).  `wpre`: the first BIT_PF chunks of this wave, fetched ahead.  Rows beyond B
+// Chunks [cb, ce) of 256 columns, split over KP waves (a workgroup works on 4 / KP strips at a time,
+// wave w on the strip of its group w / KP); the integer sum over the KP waves lands in the group's
+// first wave (returns true there).  `wpre`: the first BIT_PF chunks of this wave, fetched ahead.  Rows beyond B
 // read row B - 1 (their results are never looked at).  Every thread of the workgroup calls.
 #define BIT_PF 6
 struct BitPre {
   uint4 w[BIT_PF];
 };
+template <int KP>
 __device__ __forceinline__ void bit_wave_chunks(int cb, int ce, int& c0, int& c1) {
-  const int wave = threadIdx.x >> 6;
-  const int per = (ce - cb + 3) >> 2;
-  c0 = cb + wave * per;
+  const int kpart = (threadIdx.x >> 6) % KP;
+  const int per = (ce - cb + KP - 1) / KP;
+  c0 = cb + kpart * per;
   c1 = min(ce, c0 + per);
 }
+template <int KP>
 __device__ __forceinline__ void bit_prefetch(const uint4* wp, int KC, int strip, int cb, int ce, bool live, BitPre& pre) {
   int c0, c1;
-  bit_wave_chunks(cb, ce, c0, c1);
+  bit_wave_chunks<KP>(cb, ce, c0, c1);
   const uint4* wrow = wp + (size_t)strip * KC * 64 + (threadIdx.x & 63);
 #pragma unroll
   for (int c = 0; c < BIT_PF; ++c)
     pre.w[c] = (live && c0 + c < c1) ? ldg16_nt(wrow + (size_t)(c0 + c) * 64) : make_uint4(0, 0, 0, 0);
 }
+template <int KP>
 __device__ __forceinline__ bool bit_strip(const uint4* wp, int KC, int strip, int cb, int ce, bool live,
-                                          const BitPre* pre, const int8_t* xq, int ldq, int B, int* red, i32x4& acc) {
+                                          const BitPre& pre, bool use_pre, const int8_t* xq, int ldq, int B, int* red,
+                                          i32x4& acc) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kpart = wave % KP;
   const int m = lane & 15, g = lane >> 4;
   int c0, c1;
-  bit_wave_chunks(cb, ce, c0, c1);
+  bit_wave_chunks<KP>(cb, ce, c0, c1);
   const uint4* wrow = wp + (size_t)strip * KC * 64 + lane;
   const int8_t* xrow = xq + (size_t)min(m, B - 1) * ldq + 16 * g;
   acc = (i32x4){0, 0, 0, 0};
   if (live) {
     for (int cbk = c0; cbk < c1; cbk += BIT_PF) {
       uint4 wv[BIT_PF];
-      if (pre && cbk == c0) {
+      if (use_pre && cbk == c0) {
 #pragma unroll
-        for (int c = 0; c < BIT_PF; ++c) wv[c] = pre->w[c];
+        for (int c = 0; c < BIT_PF; ++c) wv[c] = pre.w[c];
       } else {
 #pragma unroll
         for (int c = 0; c < BIT_PF; ++c)
@@ -431,18 +539,21 @@ __device__ __forceinline__ bool bit_strip(const uint4* wp, int KC, int strip, in
       }
     }
   }
-  if (wave > 0) {
+  if (KP > 1) {
+    if (kpart > 0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) red[((wave - 1) * 64 + lane) * 4 + i] = acc[i];
-  }
-  __syncthreads();
-  if (wave == 0) {
+      for (int i = 0; i < 4; ++i) red[(wave * 64 + lane) * 4 + i] = acc[i];
+    }
+    __syncthreads();
+    if (kpart == 0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      acc[i] += red[(0 * 64 + lane) * 4 + i] + red[(1 * 64 + lane) * 4 + i] + red[(2 * 64 + lane) * 4 + i];
+      for (int w = 1; w < KP; ++w)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] += red[((wave + w) * 64 + lane) * 4 + i];
+    }
+    __syncthreads();  // red is free again
   }
-  __syncthreads();  // red is free again
-  return wave == 0;
+  return kpart == 0 && live;
 }
 
 // y = bf16((float(acc - sum q) / s) * gamma)   (bitnet.py:58-59; the packed codes are T + 1)
@@ -512,14 +623,16 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
   L.codes = reinterpret_cast<int8_t*>(smem);
   L.shape(B, d);
   size_t off = (codes_bytes + 255) & ~(size_t)255;
-  const size_t stage_bytes = max((size_t)(B == 1 ? 1 : 4) * Kp * 2, (size_t)B * (dmax + 8) * 2);
+  const int KpF = ((F + 255) >> 8) << 8;
+  const size_t stage_bytes = max((size_t)B * (dmax + 8) * 2, (B > 1 && F > 2048) ? (size_t)B * KpF * 2 : (size_t)0);
+  L.ldst = KpF;
   L.stage = reinterpret_cast<bf16_t*>(smem + off);
-  L.ldst = Kp;
   L.ldm = dmax + 8;
   off += (stage_bytes + 255) & ~(size_t)255;
   L.red = reinterpret_cast<float*>(smem + off); off += 4096;
   L.s_s = reinterpret_cast<float*>(smem + off); off += 128;
   L.s_sum = reinterpret_cast<int*>(smem + off); off += 128;
+  L.sumw = reinterpret_cast<int*>(smem + off); off += 64;
   float* att = reinterpret_cast<float*>(smem + off); off += (size_t)(8 + 4 * D) * G * sizeof(float);
   float* mrg_w = reinterpret_cast<float*>(smem + off); off += (size_t)((B * H * a.ns + 1) & ~1) * sizeof(float);
   float* mrg_l = reinterpret_cast<float*>(smem + off); off += (size_t)((B * H * a.ns + 1) & ~1) * sizeof(float);
@@ -557,9 +670,29 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
   lm.N = V; lm.K = d; lm.nstrips = (V + 15) / 16; lm.out = reinterpret_cast<char*>(a.logits); lm.ldo = V;
   lm.valid = a.valid_vocab > 0 ? min(a.valid_vocab, V) : V;
   lm.wp = reinterpret_cast<const uint4*>(m.w_vocab);
-  GemmPre lpre;
   AttnPre<D> apre;
-  BitPre wpre;
+  BitPre wpre, wpre2;
+
+  // P1: the workgroups are split into three groups, one per projection, in proportion to the
+  // projections' strips, so that a workgroup derives the codes of one BitLinear only; it works on
+  // two strips at a time (two waves each)
+  const int sub2 = wave >> 1;
+  const int p1_units = ns_q + 2 * ns_kv;
+  const int gq = max(1, (int)((long long)nwg * ns_q / p1_units));
+  const int gk = max(1, (nwg - gq) / 2);
+  const int p1_which = (int)blockIdx.x < gq ? BQ : ((int)blockIdx.x < gq + gk ? BK : BV);
+  const int p1_gi = (int)blockIdx.x - (p1_which == BQ ? 0 : (p1_which == BK ? gq : gq + gk));
+  const int p1_gsz = p1_which == BQ ? gq : (p1_which == BK ? gk : nwg - gq - gk);
+  const int p1_nstr = p1_which == BQ ? ns_q : ns_kv;
+  const int p1_strip0 = 2 * p1_gi + sub2;
+  // the rotation of this lane's outputs in its first strip: the same in every layer
+  uint32_t rope_c = 0, rope_s = 0;
+  if (p1_which != BV && p1_strip0 < p1_nstr && ok_pos) {
+    const int dd = (p1_strip0 * 16 + 4 * gg) % D;
+    rope_c = ldg4(m.cos + (size_t)pos * (D >> 1) + (dd >> 1));
+    rope_s = ldg4(m.sin + (size_t)pos * (D >> 1) + (dd >> 1));
+  }
+  bit_prefetch<2>(reinterpret_cast<const uint4*>(gptr(ltab[0].w[p1_which])), KCd, p1_strip0, 0, KCd, p1_strip0 < p1_nstr, wpre);
 
   for (int l = 0; l < m.n_layers; ++l) {
     const BitLayerDev& LY = ltab[l];
@@ -578,33 +711,35 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
     } else {
       xin.xmid = a.xm + (size_t)(l - 1) * a.xm_stride;
       xin.parts = a.dm + (size_t)(l - 1) * a.dm_stride;
-      xin.ds = a.ds + (size_t)(l - 1) * 16;
+      xin.ds = a.ds + (size_t)(l - 1) * 32;
       xin.gamma = ltab[l - 1].gamma[BD];
     }
     const bf16_t* norm1 = reinterpret_cast<const bf16_t*>(gptr(LY.norm1));
     const bf16_t* norm2 = reinterpret_cast<const bf16_t*>(gptr(LY.norm2));
 
-    // ---- P1: Q, K, V.  Units [0, ns_q) query strips, then key strips, then value strips. ----
-    {
-      const int nunits = ns_q + 2 * ns_kv;
-      L.shape(B, d);
-      int have = -1;  // projection whose codes are staged
-      for (int unit = blockIdx.x; unit < nunits; unit += nwg) {
-        const int which = unit < ns_q ? BQ : (unit < ns_q + ns_kv ? BK : BV);
-        const int strip = unit - (which == BQ ? 0 : (which == BK ? ns_q : ns_q + ns_kv));
-        const uint4* wp = reinterpret_cast<const uint4*>(gptr(LY.w[which]));
-        bit_prefetch(wp, KCd, strip, 0, KCd, true, wpre);
-        if (have != which) {
-          const bf16_t* nw = reinterpret_cast<const bf16_t*>(gptr(LY.nw[which]));
-          bit_stage_codes(L, 0, B, d, norm1, nw, m.eps, [&](int b, int p) {
-            uint32_t w[4];
-            bitx_load<8>(xin, b, p * 8, w);
-            return make_uint4(w[0], w[1], w[2], w[3]);
-          });
-          have = which;
-        }
+    // ---- P1: Q, K, V + rotary + append ----
+    L.shape(B, d);
+    if (2 * p1_gi < p1_nstr) {
+      const int which = p1_which;
+      const uint4* wp = reinterpret_cast<const uint4*>(gptr(LY.w[which]));
+      const bf16_t* nw = reinterpret_cast<const bf16_t*>(gptr(LY.nw[which]));
+      auto load_in = [&](int b, int p) {
+        uint32_t w[4];
+        bitx_load<8>(xin, b, p * 8, w);
+        return make_uint4(w[0], w[1], w[2], w[3]);
+      };
+      if (B == 1) {
+        auto load0 = [&](int p) { return load_in(0, p); };
+        bit_stage_row1<1>(L, 1, d, norm1, nw, nullptr, m.eps, load0);
+      } else {
+        bit_stage_roww<4>(L, 1, B, d, norm1, nw, nullptr, m.eps, load_in);
+      }
+      for (int s0 = 2 * p1_gi; s0 < p1_nstr; s0 += 2 * p1_gsz) {
+        const bool first = s0 == 2 * p1_gi;
+        const int strip = s0 + sub2;
         i32x4 acc;
-        if (bit_strip(wp, KCd, strip, 0, KCd, true, &wpre, L.codes, L.ldq, B, reinterpret_cast<int*>(L.red), acc) &&
+        if (bit_strip<2>(wp, KCd, strip, 0, KCd, strip < p1_nstr, wpre, first, L.codes, L.ldq, B,
+                         reinterpret_cast<int*>(L.red), acc) &&
             mm < B && ok_pos) {
           const int b = mm;
           const int r0 = strip * 16 + 4 * gg;
@@ -612,9 +747,12 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
           bit_scale(acc, L.s_sum[b], L.s_s[b], LY.gamma[which], v);
           char* o;
           if (which != BV) {
-            const int dd = r0 % D;
-            const uint32_t cs = ldg4(m.cos + (size_t)pos * (D >> 1) + (dd >> 1));
-            const uint32_t sn = ldg4(m.sin + (size_t)pos * (D >> 1) + (dd >> 1));
+            uint32_t cs = rope_c, sn = rope_s;
+            if (!first) {
+              const int dd = r0 % D;
+              cs = ldg4(m.cos + (size_t)pos * (D >> 1) + (dd >> 1));
+              sn = ldg4(m.sin + (size_t)pos * (D >> 1) + (dd >> 1));
+            }
             const float c2[2] = {lo_bf(cs), hi_bf(cs)}, s2[2] = {lo_bf(sn), hi_bf(sn)};
 #pragma unroll
             for (int pr = 0; pr < 2; ++pr) {
@@ -638,7 +776,11 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
     attn_phase<D, G>(B, H, Hkv, m.t_max, a.blk_x, a.ns, apre, q_l, p_l, kc, vc, Lc, att);
     gs.arrive(pf);
     const uint4* wo = reinterpret_cast<const uint4*>(gptr(LY.w[BO]));
-    bit_prefetch(wo, KCo, blockIdx.x, 0, KCo, (int)blockIdx.x < ns_d, wpre);
+    bit_prefetch<4>(wo, KCo, blockIdx.x, 0, KCo, (int)blockIdx.x < ns_d, wpre);
+    // the residual of this lane's outputs in the first strip: known since the previous layer
+    uint32_t rpre[2] = {0u, 0u};
+    if ((int)blockIdx.x < ns_d && wave == 0 && mm < B && (int)blockIdx.x * 16 + 4 * gg < d)
+      bitx_load<4>(xin, mm, (int)blockIdx.x * 16 + 4 * gg, rpre);
     gs.wait(pf);
     // ---- P3: merge + attn.proj + residual ----
     L.shape(B, HD);
@@ -654,18 +796,25 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
         else if (a.ns == 2) stage_attn_merge<2>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
         else stage_attn_merge<1>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
         __syncthreads();
-        bit_codes_from_stage(L, 0, B, HD, reinterpret_cast<const bf16_t*>(gptr(LY.nw[BO])), m.eps);
+        const bf16_t* nwo = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BO]));
+        if (B == 1) {
+          auto load0 = [&](int p) { return lds16(xs + p * 8); };
+          bit_stage_row1<1>(L, 1, HD, nullptr, nwo, nullptr, m.eps, load0);
+        } else {
+          auto loadb = [&](int b, int p) { return lds16(xs + (size_t)b * ldxs + p * 8); };
+          bit_stage_roww<4>(L, 1, B, HD, nullptr, nwo, nullptr, m.eps, loadb);
+        }
       }
       i32x4 acc;
-      if (bit_strip(wo, KCo, strip, 0, KCo, true, first ? &wpre : nullptr, L.codes, L.ldq, B,
-                    reinterpret_cast<int*>(L.red), acc) && mm < B) {
+      if (bit_strip<4>(wo, KCo, strip, 0, KCo, true, wpre, first, L.codes, L.ldq, B,
+                       reinterpret_cast<int*>(L.red), acc) && mm < B) {
         const int b = mm;
         const int r0 = strip * 16 + 4 * gg;
         if (r0 < d) {
           float y[4];
           bit_scale(acc, L.s_sum[b], L.s_s[b], LY.gamma[BO], y);
-          uint32_t r[2];
-          bitx_load<4>(xin, b, r0, r);
+          uint32_t r[2] = {rpre[0], rpre[1]};
+          if (!first) bitx_load<4>(xin, b, r0, r);
           st_coh8(const_cast<char*>(xm_addr(x_mid, a.blk_x, b, r0)),
                   make_uint2(pack_bf(lo_bf(r[0]) + y[0], hi_bf(r[0]) + y[1]), pack_bf(lo_bf(r[1]) + y[2], hi_bf(r[1]) + y[3])));
         }
@@ -674,11 +823,15 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
     gs.arrive(pf);
     const uint4* wg = reinterpret_cast<const uint4*>(gptr(LY.w[BG]));
     const uint4* wu = reinterpret_cast<const uint4*>(gptr(LY.w[BU]));
-    bit_prefetch(wg, KCd, blockIdx.x, 0, KCd, (int)blockIdx.x < ns_f, wpre);
+    {
+      const int strip = 2 * (int)blockIdx.x + sub2;
+      bit_prefetch<2>(wg, KCd, strip, 0, KCd, strip < ns_f, wpre);
+      bit_prefetch<2>(wu, KCd, strip, 0, KCd, strip < ns_f, wpre2);
+    }
     gs.wait(pf);
-    // ---- P4: norm2 + ff.gate, ff.up + SwiGLU ----
+    // ---- P4: norm2 + ff.gate, ff.up + SwiGLU; two strips at a time, two waves each ----
     L.shape(B, d);
-    if ((int)blockIdx.x < ns_f) {
+    if (2 * (int)blockIdx.x < ns_f) {
       BitX xmid{};
       xmid.B = B; xmid.N = d; xmid.blk = a.blk_x; xmid.xmid = x_mid;
       auto load_mid = [&](int b, int p) {
@@ -686,15 +839,22 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
         bitx_load<8>(xmid, b, p * 8, w);
         return make_uint4(w[0], w[1], w[2], w[3]);
       };
-      bit_stage_codes(L, 0, B, d, norm2, reinterpret_cast<const bf16_t*>(gptr(LY.nw[BG])), m.eps, load_mid);
-      bit_stage_codes(L, 1, B, d, norm2, reinterpret_cast<const bf16_t*>(gptr(LY.nw[BU])), m.eps, load_mid);
-      for (int strip = blockIdx.x; strip < ns_f; strip += nwg) {
-        const bool first = strip == (int)blockIdx.x;
+      const bf16_t* nwg_ = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BG]));
+      const bf16_t* nwu_ = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BU]));
+      if (B == 1) {
+        auto load0 = [&](int p) { return load_mid(0, p); };
+        bit_stage_row1<1>(L, 2, d, norm2, nwg_, nwu_, m.eps, load0);
+      } else {
+        bit_stage_roww<4>(L, 2, B, d, norm2, nwg_, nwu_, m.eps, load_mid);
+      }
+      for (int s0 = 2 * (int)blockIdx.x; s0 < ns_f; s0 += 2 * nwg) {
+        const bool first = s0 == 2 * (int)blockIdx.x;
+        const int strip = s0 + sub2;
         i32x4 ag, au;
-        const bool w0g = bit_strip(wg, KCd, strip, 0, KCd, true, first ? &wpre : nullptr, L.codes, L.ldq, B,
-                                   reinterpret_cast<int*>(L.red), ag);
-        const bool w0u = bit_strip(wu, KCd, strip, 0, KCd, true, nullptr, L.codes + L.set, L.ldq, B,
-                                   reinterpret_cast<int*>(L.red), au);
+        const bool w0g = bit_strip<2>(wg, KCd, strip, 0, KCd, strip < ns_f, wpre, first, L.codes, L.ldq, B,
+                                      reinterpret_cast<int*>(L.red), ag);
+        const bool w0u = bit_strip<2>(wu, KCd, strip, 0, KCd, strip < ns_f, wpre2, first, L.codes + L.set, L.ldq,
+                                      B, reinterpret_cast<int*>(L.red), au);
         if (w0g && w0u && mm < B) {
           const int b = mm;
           const int f0 = strip * 16 + 4 * gg;
@@ -714,7 +874,7 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
     const int per_part = (KCf + OHARA_BIT_DOWN_SPLIT - 1) / OHARA_BIT_DOWN_SPLIT;
     {
       const int unit = blockIdx.x, part = unit / ns_d, strip = unit - part * ns_d;
-      bit_prefetch(wd, KCf, strip, part * per_part, min(KCf, (part + 1) * per_part), unit < ns_d * OHARA_BIT_DOWN_SPLIT, wpre);
+      bit_prefetch<4>(wd, KCf, strip, part * per_part, min(KCf, (part + 1) * per_part), unit < ns_d * OHARA_BIT_DOWN_SPLIT, wpre);
     }
     gs.wait(pf);
     // ---- P5: ff.down, K split over OHARA_BIT_DOWN_SPLIT groups of workgroups ----
@@ -726,14 +886,21 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
         const bool first = unit == (int)blockIdx.x;
         const int part = unit / ns_d, strip = unit - part * ns_d;
         if (!staged) {
-          bit_stage_codes(L, 0, B, F, nullptr, reinterpret_cast<const bf16_t*>(gptr(LY.nw[BD])), m.eps, [&](int b, int p) {
-            return ldg16(am_addr(a_l, a.blk_a, b, p * 8));
-          });
+          const bf16_t* nwd = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BD]));
+          if (B == 1) {
+            auto load0 = [&](int p) { return ldg16(am_addr(a_l, a.blk_a, 0, p * 8)); };
+            if (F <= 2048) bit_stage_row1<1>(L, 1, F, nullptr, nwd, nullptr, m.eps, load0);
+            else bit_stage_row1<3>(L, 1, F, nullptr, nwd, nullptr, m.eps, load0);
+          } else {
+            auto loadb = [&](int b, int p) { return ldg16(am_addr(a_l, a.blk_a, b, p * 8)); };
+            if (F <= 2048) bit_stage_roww<4>(L, 1, B, F, nullptr, nwd, nullptr, m.eps, loadb);
+            else bit_stage_roww_lds<12>(L, B, F, nwd, m.eps, loadb);
+          }
           staged = true;
         }
         i32x4 acc;
-        if (bit_strip(wd, KCf, strip, part * per_part, min(KCf, (part + 1) * per_part), true, first ? &wpre : nullptr,
-                      L.codes, L.ldq, B, reinterpret_cast<int*>(L.red), acc) && mm < B) {
+        if (bit_strip<4>(wd, KCf, strip, part * per_part, min(KCf, (part + 1) * per_part), true, wpre, first,
+                         L.codes, L.ldq, B, reinterpret_cast<int*>(L.red), acc) && mm < B) {
           const int b = mm;
           const int r0 = strip * 16 + 4 * gg;
           if (r0 < d) {
@@ -742,25 +909,30 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
             st_coh8(o, make_uint2((uint32_t)(acc[0] - sq), (uint32_t)(acc[1] - sq)));
             st_coh8(o + 2, make_uint2((uint32_t)(acc[2] - sq), (uint32_t)(acc[3] - sq)));
           }
-          if (unit == 0 && gg == 0) st_coh4(a.ds + (size_t)l * 16 + b, __float_as_uint(L.s_s[b]));
+          if (unit == 0 && gg == 0) st_coh4(a.ds + (size_t)l * 32 + b, __float_as_uint(L.s_s[b]));
         }
       }
     }
     gs.arrive(pf);
-    if (l + 1 == m.n_layers) gemm_prefetch<1, 24, E_LOGITS>(lm, lpre, B);
+    if (l + 1 == m.n_layers) break;  // the last barrier's wait follows the loop, behind another prefetch
+    bit_prefetch<2>(reinterpret_cast<const uint4*>(gptr(ltab[l + 1].w[p1_which])), KCd, p1_strip0, 0, KCd,
+                    p1_strip0 < p1_nstr, wpre);
     gs.wait(pf);
   }
+  GemmPre lpre;
+  gemm_prefetch<1, 24, E_LOGITS>(lm, lpre, B);
+  gs.wait(pf);
   // ---- final norm + vocabulary projection (bf16), running arg-max per lane ----
   {
     BitX xf{};
     xf.B = B; xf.N = d; xf.blk = a.blk_x;
     xf.xmid = a.xm + (size_t)(m.n_layers - 1) * a.xm_stride;
     xf.parts = a.dm + (size_t)(m.n_layers - 1) * a.dm_stride;
-    xf.ds = a.ds + (size_t)(m.n_layers - 1) * 16;
+    xf.ds = a.ds + (size_t)(m.n_layers - 1) * 32;
     xf.gamma = ltab[m.n_layers - 1].gamma[BD];
     bf16_t* xs = L.stage;
     const int ldxs = d + 8;
-    bit_stage_final_norm<8>(xs, ldxs, xf, m.final_norm, m.eps, B, d);
+    bit_stage_final_norm<4>(xs, ldxs, xf, m.final_norm, m.eps, B, d);
     __syncthreads();
     gemm_phase<1, 24, E_LOGITS>(lm, lpre, xs, ldxs, B, L.red, best_v, best_i, pf);
   }
@@ -865,7 +1037,7 @@ BitLayout bit_layout(const OharaBitModel* m, int B, int nwg) {
   L.am = o; o += L.am_stride * NL;
   L.pm = o; o += L.pm_stride * sizeof(float) * NL;
   L.dm = o; o += L.dm_stride * sizeof(int32_t) * NL;
-  L.ds = o; o += bit_al((size_t)NL * 16 * sizeof(float));
+  L.ds = o; o += bit_al((size_t)NL * 32 * sizeof(float));
   L.candv = o; o += bit_al((size_t)nwg * B * sizeof(float));
   L.candi = o; o += bit_al((size_t)nwg * B * sizeof(int));
   L.prof = o; o += bit_al(1024 * sizeof(unsigned long long));
@@ -881,9 +1053,10 @@ size_t bit_smem_bytes(const OharaBitModel* m, int B, int ns) {
   const int Kp = ((kmax + 255) >> 8) << 8, Kpd = ((dmax + 255) >> 8) << 8;
   size_t codes = (size_t)B * (Kp + 16);
   if ((size_t)2 * B * (Kpd + 16) > codes) codes = (size_t)2 * B * (Kpd + 16);
-  size_t stage = (size_t)(B == 1 ? 1 : 4) * Kp * 2;
-  if ((size_t)B * (dmax + 8) * 2 > stage) stage = (size_t)B * (dmax + 8) * 2;
-  size_t o = ((codes + 255) & ~(size_t)255) + ((stage + 255) & ~(size_t)255) + 4096 + 256;
+  const int KpF = ((m->d_ff + 255) >> 8) << 8;
+  size_t stage = (size_t)B * (dmax + 8) * 2;
+  if (B > 1 && m->d_ff > 2048 && (size_t)B * KpF * 2 > stage) stage = (size_t)B * KpF * 2;
+  size_t o = ((codes + 255) & ~(size_t)255) + ((stage + 255) & ~(size_t)255) + 4096 + 256 + 64;
   o += (size_t)(8 + 4 * D) * G * sizeof(float);
   o += (size_t)2 * ((B * m->n_heads * ns + 1) & ~1) * sizeof(float);
   o = (o + 15) & ~(size_t)15;
@@ -906,17 +1079,22 @@ int64_t ohara_bitnet_persistent_error_offset(const OharaBitModel* m, int batch, 
   return (int64_t)bit_layout(m, batch, n_workgroups).bar + (int64_t)(ng + 2) * 64 * 4;
 }
 
+int64_t ohara_bitnet_persistent_profile_offset(const OharaBitModel* m, int batch, int n_workgroups) {
+  if (!m || batch < 1 || n_workgroups < 1) return OHARA_EINVAL;
+  return (int64_t)bit_layout(m, batch, n_workgroups).prof;
+}
+
 int ohara_bitnet_decode_persistent(const OharaBitModel* m, const OharaDecodeState* s, void* workspace, int n_workgroups,
                                    int init_workspace, int select_greedy, unsigned int spin_limit, void* stream) {
   if (!m || !s || !workspace || !m->layers || !s->kcache || !s->vcache || !s->step_state) return OHARA_EINVAL;
   if (s->batch < 1 || s->batch > 8) return OHARA_ESIZE;
-  if (n_workgroups < 1 || n_workgroups > 1024) return OHARA_EINVAL;
+  if (n_workgroups < 4 || n_workgroups > 1024) return OHARA_EINVAL;
   if (s->n_split != OHARA_MEGA_NS) return OHARA_EINVAL;
   const int D = m->head_dim;
   if (m->n_kv_heads < 1 || m->n_heads % m->n_kv_heads) return OHARA_EINVAL;
   const int G = m->n_heads / m->n_kv_heads;
   if (!(D == 128 || D == 64) || G != 1) return OHARA_ESIZE;
-  if ((m->d_model & 15) || (m->d_ff & 15) || m->d_model > 4096 || m->d_ff > 6144) return OHARA_ESIZE;
+  if ((m->d_model & 15) || (m->d_ff & 15) || m->d_model > 2048 || m->n_heads * D > 2048 || m->d_ff > 6144) return OHARA_ESIZE;
   hipStream_t st = (hipStream_t)stream;
   char* ws = reinterpret_cast<char*>(workspace);
   const BitLayout L = bit_layout(m, s->batch, n_workgroups);
@@ -958,7 +1136,7 @@ int ohara_bitnet_decode_persistent(const OharaBitModel* m, const OharaDecodeStat
   a.select = select_greedy;
   a.ids = s->ids; a.logits = s->logits;
   a.step_state = s->step_state; a.history = s->history;
-  a.prof = nullptr;
+  a.prof = (s->prof_kernel == -2 && 30 * m->n_layers + 16 <= 1024) ? reinterpret_cast<unsigned long long*>(ws + L.prof) : nullptr;
   a.spin_limit = spin_limit ? spin_limit : (1u << 19);
   int ns = n_workgroups / (s->batch * m->n_kv_heads);
   ns = ns < 1 ? 1 : (ns > OHARA_MEGA_NS ? OHARA_MEGA_NS : ns);

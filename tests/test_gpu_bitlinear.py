@@ -218,6 +218,8 @@ PERSISTENT_SHAPES = [
     (512, 8, 1536, 333, 2, 1),    # head_dim 64, several chunks, vocabulary not a multiple of 16
     (512, 8, 1536, 333, 2, 8),
     (320, 5, 528, 300, 2, 3),     # widths that are not multiples of 256 (zero-padded code rows)
+    (256, 2, 2304, 320, 4, 6),    # a hidden width beyond 2048 (rows parked in LDS at batch > 1), four layers
+    (256, 2, 2304, 320, 4, 1),
 ]
 
 

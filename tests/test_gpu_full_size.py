@@ -124,7 +124,9 @@ def test_bitnet_c4_model_full_size(cuda):
         codes with the ternary weights, bit for bit;
     (b) a 64-token prefill and three cached decode steps against the CPU oracle (whole model);
     (c) at context 2047 -> 2048 (the last cache row), a decode step of 8 sequences equals the same
-        sequences decoded alone; a captured graph replays to the eager result bit for bit."""
+        sequences decoded alone; a captured graph replays to the eager result bit for bit;
+    (d) the single-launch decode step on the same caches against the kernel chain (batch 8 and one
+        sequence), and 128 greedy tokens from its captured graph against its eager launches."""
     import bench
     from ohara_amd import ops
     from ohara_amd.bitnet import BitLlama
@@ -316,6 +318,52 @@ def test_bitnet_c4_model_full_size(cuda):
         gr.replay()
         torch.cuda.synchronize()
         assert torch.equal(out[:, 0], eager)
+
+    # (d) the single-launch step on the same caches at the last cache row: the same codes and integer
+    # sums as the kernel chain, so nearly every logit is the chain's bit for bit (attention sums its
+    # context in another order, which flips single bf16 roundings that the quantisers then amplify)
+    def persistent_logits(Bp, rows):
+        cp = model.build_kv_cache(Bp)
+        sess = model.session(Bp, 4, kv_cache=cp, persistent=True)
+        sess.prefill(tok[rows, :1])  # one token: builds the workspace; the caches are then replaced
+        for cs, cb in zip(cp, cache):
+            cs.key[:, :Lc].copy_(cb.key[rows, :Lc])
+            cs.value[:, :Lc].copy_(cb.value[rows, :Lc])
+            cs.length, cs.batch_size = Lc, Bp
+        sess.ids.copy_(tok[rows, 0])
+        sess.step_state.copy_(torch.tensor([Lc, 1, 0, 0], dtype=torch.int32))
+        sess.pos, sess.produced = Lc, 1
+        sess.step()
+        torch.cuda.synchronize()
+        sess.check_error()
+        assert torch.equal(sess.ids, ops.argmax(sess.logits))
+        return sess.logits.clone()
+
+    all_rows = torch.arange(B, device=cuda)
+    for Bp, rows in ((B, all_rows), (1, all_rows[3:4])):
+        got = persistent_logits(Bp, rows)
+        want = lb[rows]
+        scale = want.float().abs().max().item()
+        dlt = (got.float() - want.float()).abs()
+        same = (got == want).float().mean().item()
+        report[f"persistent_vs_chain_batch{Bp}"] = {"identical_fraction": round(same, 4),
+                                                    "max_over_scale": round(dlt.max().item() / scale, 5)}
+        if Bp == B:
+            assert same >= 0.5 and dlt.max().item() <= tol_max * scale and dlt.mean().item() <= tol_mean * scale, (Bp, same)
+        else:  # one sequence against the row of the batch of eight: two reduction orders, as in (c)
+            assert dlt.max().item() <= tol_max * scale and dlt.mean().item() <= tol_mean * scale, (Bp, same)
+    print(report)
+    del cache
+    torch.cuda.empty_cache()
+    # 128 greedy tokens after a 64-token prompt: the captured graph equals the eager launches
+    prompt = torch.randint(0, V, (1, 64), generator=g).to(cuda)
+    t_graph = model.generate_greedy(prompt, 128, persistent=True)
+    t_eager = model.generate_greedy(prompt, 128, persistent=True, use_graph=False)
+    assert torch.equal(t_graph, t_eager) and t_graph.shape == (1, 128)
+    t_chain = model.generate_greedy(prompt, 128, persistent=False)
+    first_diff = int((t_graph != t_chain).float().argmax()) if not torch.equal(t_graph, t_chain) else 128
+    print({"persistent_vs_chain_first_differing_token": first_diff})
+    assert first_diff >= 8
 
 
 def test_moe_c5_model_full_size(cuda):
