@@ -706,6 +706,8 @@ def main():
             roof = {"kernel": kname, "bound": "hbm", "achieved": round(kb / t_k / 1e9, 1), "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": round(kb / t_k / 1e9 / HBM_PEAK_GBS, 4),
                     "traffic": PMC_TRAFFIC_BYTES.get(("persistent" if sess2.persistent else "chain", 1, args.prompt)),
+                    "traffic_source": "constant carried in bench.py from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) "
+                                      "summarised in profiles/decode_mega_kernel_d12_batch1_pmc.txt; not measured by this run",
                     "bytes_per_launch": int(kb), "avg_launch_us": round(t_k * 1e6, 2)}
         del sess
         torch.cuda.empty_cache()

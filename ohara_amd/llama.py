@@ -213,12 +213,24 @@ class Llama:
     cast to bf16, moved to ``device`` and repacked once.
     """
 
+    def __new__(cls, config: Config, state: dict | None = None, device="cuda", dtype=BF16):
+        # A config with routed experts builds Blocks with a GroupedMoE feed-forward in the reference
+        # (llama.py:154-170); here those layers live in ``MoeLlama``, which this constructor hands out.
+        if cls is Llama and getattr(config, "moe_num_experts", 0) > 0:
+            if dtype != BF16:
+                raise ValueError("ohara_amd runs the decode path in bfloat16 only")
+            if not config.moe_grouped:
+                raise NotImplementedError("ohara_amd serves MoE layers in the grouped form only (moe_grouped=True, "
+                                          "ohara/modules/moe_grouped.py); the per-expert loop of llama.py:171-178 is not built")
+            from .moe import MoeLlama
+
+            return MoeLlama(config, state, device=device)
+        return super().__new__(cls)
+
     def __init__(self, config: Config, state: dict, device="cuda", dtype=BF16):
         _validate_config(config)
         if dtype != BF16:
             raise ValueError("ohara_amd runs the decode path in bfloat16 only")
-        if config.moe_num_experts > 0:
-            raise NotImplementedError("MoE layers are served by ohara_amd.moe (not wired into Llama yet)")
         lib()  # fail loudly now if the HIP library is missing
         self.config = config
         self.device = torch.device(device)

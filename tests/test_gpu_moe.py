@@ -80,7 +80,10 @@ def test_moe_llama_matches_reference_fixture(cuda):
     kw = {k: v for k, v in g["config"].items() if k in fields}
     state = {k: (v.to(BF) if v.is_floating_point() else v) for k, v in g["state"].items()}
     ref = R.RefLlama(R.RefConfig(**kw), state)
-    model = MoeLlama(Config(**kw), state, device=cuda)
+    from ohara_amd.llama import Llama
+
+    model = Llama(Config(**kw), state, device=cuda)  # a config with routed experts: Llama hands out the MoE model
+    assert isinstance(model, MoeLlama)
     ids = g["ids"]
     want = ref(ids)
     got = model(ids.to(cuda)).cpu()

@@ -230,6 +230,15 @@ def test_config_and_kv_cache_bookkeeping():
                {"num_attention_heads": 4, "num_key_value_heads": 3}, {"hidden_size": 12, "num_attention_heads": 4}):
         with pytest.raises(ValueError):
             _validate_config(Config(**kw))
+    # what the kernels do not cover is refused when the model is built, before anything touches a GPU
+    from ohara_amd.llama import Llama
+
+    with pytest.raises(ValueError, match="biases"):
+        Llama(Config(bias=True), {})
+    with pytest.raises(NotImplementedError, match="grouped"):
+        Llama(Config(moe_num_experts=4, moe_grouped=False), {})
+    with pytest.raises(ValueError, match="bfloat16"):
+        Llama(Config(), {}, dtype=torch.float16)
     c = KVCache((2, 8, 2, 4), 8, dtype=torch.float32)
     k = torch.randn(2, 3, 2, 4)
     ck, cv = c.forward(k, k * 2, 0)  # tests/test_modules.py:46-58
