@@ -320,7 +320,7 @@ def bench_prefill(model, cfg, dev):
             fl = 2.0 * M * n * k
         o = torch.empty(M, n, device=dev, dtype=torch.bfloat16)
         xin = x[:, :k]
-        t = graph_time(lambda: ops.gemm(xin, wp, out=o))
+        t = graph_time(lambda: ops.gemm(xin, wp, out=o), iters=50)
         kern.append({"kernel": "gemm_tile_kernel " + name, "rows": M, "us": round(t * 1e6, 1),
                      "TFLOPs": round(fl / t / 1e12, 1), "mfma_util": round(fl / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)})
     H, D = cfg.num_attention_heads, d // cfg.num_attention_heads
@@ -639,6 +639,8 @@ def main():
     ap.add_argument("--bitnet-only", type=str, default="", metavar="BATCHES",
                     help="run the BitNet ternary decode figures alone at these batch sizes (e.g. 1,8) and exit "
                          "(profiling workload)")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run the d12 prefill figures (tiled MFMA GEMMs, prefill attention) alone and exit")
     ap.add_argument("--phi-decode-only", type=int, default=0, metavar="B",
                     help="run 12 eager Phi-2 decode steps of B sequences at context 1024 and exit (profiling workload)")
     args = ap.parse_args()
@@ -672,6 +674,9 @@ def main():
     cfg, st = d12_state(dev)
     model = Llama(cfg, st, device=dev)
     del st
+    if args.prefill_only:
+        print(json.dumps(bench_prefill(model, cfg, dev), indent=1))
+        return
     batches = [int(b) for b in args.batches.split(",") if b]
     if 1 not in batches:
         batches = [1] + batches
