@@ -639,6 +639,8 @@ def main():
     ap.add_argument("--bitnet-only", type=str, default="", metavar="BATCHES",
                     help="run the BitNet ternary decode figures alone at these batch sizes (e.g. 1,8) and exit "
                          "(profiling workload)")
+    ap.add_argument("--moe-only", action="store_true",
+                    help="run the MoE decode figure alone and exit (profiling workload)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run the d12 prefill figures (tiled MFMA GEMMs, prefill attention) alone and exit")
     ap.add_argument("--phi-decode-only", type=int, default=0, metavar="B",
@@ -657,6 +659,9 @@ def main():
     dev = torch.device("cuda:0")
     if args.phi_decode_only:
         print(json.dumps(phi_decode_only(dev, args.phi_decode_only)))
+        return
+    if args.moe_only:
+        print(json.dumps(bench_moe(dev), indent=1))
         return
     if args.bitnet_only:
         print(json.dumps(bench_bitnet(dev, tuple(int(b) for b in args.bitnet_only.split(","))), indent=1))
