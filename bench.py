@@ -620,6 +620,61 @@ def phase_timeline(dev, prompt_len, steps=32):
     return out
 
 
+def bitnet_phase_timeline(dev, batch=1, steps=16):
+    """Per-phase timeline of the single-launch BitNet decode step (C4 size, context 2047 -> 2048):
+    workgroup 0's shader-clock samples at every grid barrier (six per barrier: phase work issued, own
+    stores complete, workgroup barrier passed, arrival issued, prefetch issued, barrier passed),
+    averaged over `steps` launches and over the layers after the first."""
+    from ohara_amd.bitnet import BitLlama
+
+    cfg, st = bitnet_c4_state(dev)
+    model = BitLlama(cfg, st, device=dev)
+    del st
+    L, nl = cfg.max_sequence_length, cfg.num_hidden_layers
+    cache = model.build_kv_cache(batch)
+    sess = model.session(batch, 8, kv_cache=cache, persistent=True)
+    sess.prefill(torch.randint(0, cfg.vocab_size, (batch, 1), device=dev))
+    _fill_cache(cache, L - 1, batch)
+    start = torch.tensor([L - 1, 1, 0, 0], dtype=torch.int32, device=dev)
+    acc, total_ms = None, 0.0
+    for it in range(steps + 4):
+        sess.step_state.copy_(start)
+        sess._dst.prof_kernel = -2
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        sess._launch_step()
+        e1.record()
+        torch.cuda.synchronize()
+        if it >= 4:
+            c = sess.phase_clocks().double()
+            acc = c if acc is None else acc + c
+            total_ms += e0.elapsed_time(e1)
+    sess.check_error()
+    c = acc / steps
+    kernel_us = total_ms / steps * 1e3
+    per = c[: nl * 30].view(nl, 30)
+    n_tail = 8  # after the last barrier of the layers: vocabulary projection (2), selection arrive (4) / wait (2)
+    ticks_per_us = float(c[nl * 30 + n_tail - 1] - c[0]) / kernel_us  # within a few us of the whole launch
+    names = ["P1 q/k/v + rotary + append", "P2 attention partials", "P3 merge + attn.proj + residual",
+             "P4 gate/up + SwiGLU", "P5 down (K split in 2)"]
+    out = {"batch": batch, "kernel_us_hip_events": round(kernel_us, 1), "layers": nl,
+           "clock_ticks_per_us": round(ticks_per_us, 1),
+           "per_layer_us": round(float((per[1:, 29] - per[:-1, 29]).mean()) / ticks_per_us, 2),
+           "after_last_layer_us (final norm + vocabulary projection + selection)":
+               round(float(c[nl * 30 + n_tail - 1] - per[-1, 29]) / ticks_per_us, 1), "phases": {}}
+    for i, nm in enumerate(names):
+        b = per[1:, i * 6: i * 6 + 6]
+        began = per[:-1, 29] if i == 0 else per[1:, i * 6 - 1]
+        out["phases"][nm] = {
+            "work_us": round(float((b[:, 0] - began).mean()) / ticks_per_us, 2),
+            "own_stores_complete_us": round(float((b[:, 1] - b[:, 0]).mean()) / ticks_per_us, 2),
+            "workgroup_barrier_us": round(float((b[:, 2] - b[:, 1]).mean()) / ticks_per_us, 2),
+            "arrival_us": round(float((b[:, 3] - b[:, 2]).mean()) / ticks_per_us, 2),
+            "prefetch_issue_us": round(float((b[:, 4] - b[:, 3]).mean()) / ticks_per_us, 2),
+            "wait_for_release_us": round(float((b[:, 5] - b[:, 4]).mean()) / ticks_per_us, 2)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -636,6 +691,8 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters against)")
     ap.add_argument("--phase-timeline", action="store_true",
                     help="print the per-phase timeline of the persistent decode kernel at batch 1 and exit")
+    ap.add_argument("--bitnet-phase-timeline", type=int, default=0, metavar="B",
+                    help="print the per-phase timeline of the single-launch BitNet decode step at batch B and exit")
     ap.add_argument("--bitnet-only", type=str, default="", metavar="BATCHES",
                     help="run the BitNet ternary decode figures alone at these batch sizes (e.g. 1,8) and exit "
                          "(profiling workload)")
@@ -659,6 +716,9 @@ def main():
     dev = torch.device("cuda:0")
     if args.phi_decode_only:
         print(json.dumps(phi_decode_only(dev, args.phi_decode_only)))
+        return
+    if args.bitnet_phase_timeline:
+        print(json.dumps(bitnet_phase_timeline(dev, args.bitnet_phase_timeline), indent=1))
         return
     if args.moe_only:
         print(json.dumps(bench_moe(dev), indent=1))
