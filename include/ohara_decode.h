@@ -223,6 +223,16 @@ int ohara_sample_topk_topp(const void* logits, int logits_are_fp32, int ldl, int
                            int valid_vocab, float temperature, int top_k, float top_p, const float* u,
                            int u_step_stride, int64_t* out_ids, int64_t* history, int hist_cap,
                            int32_t* step_state, void* stream);
+/* The same selection, same results, for a caller whose sampler calls on one GPU do not overlap in time
+ * (one decode stream, as in ohara/chat_engine.py's generate loop): a small top-k (<= 64) on a long bf16
+ * row (8192 < vocab <= 65536, batch <= 64) is spread over one workgroup per 8192 ids, whose candidates
+ * meet in a 330 KB scratch array inside the library (nothing is allocated); every other shape runs
+ * ohara_sample_topk_topp's kernels.  Overlapping calls of this entry point on one GPU would share
+ * that array. */
+int ohara_sample_topk_topp_exclusive(const void* logits, int logits_are_fp32, int ldl, int batch, int vocab,
+                           int valid_vocab, float temperature, int top_k, float top_p, const float* u,
+                           int u_step_stride, int64_t* out_ids, int64_t* history, int hist_cap,
+                           int32_t* step_state, void* stream);
 
 /* ---- BitNet-b1.58 BitLinear (ternary weights x int8 activations, int32 accumulate) ------
  * Integer form of BitLinear.forward (experiments/bitnet/bitnet.py:29-59):

@@ -306,7 +306,7 @@ class BitDecodeSession:
         if self.sampling:
             ops.sample_topk_topp(self.logits, self.sampling.temperature, self.sampling.top_k, self.sampling.top_p,
                                  self.u, self.valid_vocab or None, out=self.ids, history=self.history,
-                                 step_state=self.step_state, u_per_step=True)
+                                 step_state=self.step_state, u_per_step=True, exclusive=True)
 
     def check_error(self) -> None:
         """Raise if a barrier wait of the persistent kernel expired (synchronises)."""

@@ -26,6 +26,8 @@
 //   * otherwise the nucleus is found without sorting: the smallest probability that is still
 //     kept, and then the probability the draw lands on, by bisection over the probability bits
 //     with block-wide mass sums in a fixed order (cost independent of how many tokens are kept).
+#include <mutex>
+
 #include "common.h"
 
 namespace {
@@ -294,10 +296,106 @@ __device__ __forceinline__ void load_row_scalar(const SampleArgs& a, int b, int 
   }
 }
 
+// The draw from a block of n_c candidates in (skey = fkey(x), sid = id) that holds at least the k
+// largest valid ids of the row with all ties of the k-th: sort (descending key, ascending id among equal
+// keys), cut at the k-th key, softmax over the kept entries, nucleus or vocabulary-order inverse CDF
+// (chat_engine.py:66-82).  Every thread of the workgroup calls; returns the token in every thread.
+__device__ __forceinline__ int draw_from_block(const SampleArgs& a, Smem& s, int n_c, int k, float u) {
+  const int tid = threadIdx.x;
+  int n2 = 64;
+  while (n2 < n_c) n2 <<= 1;
+  __syncthreads();
+  for (int i = n_c + tid; i < n2; i += NT) {
+    s.skey[i] = 0;  // padding sorts last
+    s.sid[i] = 0x7fffffff;
+  }
+  __syncthreads();
+  sort_candidates(s, n2);
+  // kept: everything >= the k-th largest key (ties at the threshold survive, chat_engine.py:66-69)
+  const uint32_t tk = s.skey[min(k, n_c) - 1];
+  int n_kept = block_sum_i((tid < n_c && s.skey[tid] >= tk) ? 1 : 0, s);
+  // softmax over the kept entries (the rest of the vocabulary is -inf): entry 0 is the maximum
+  const float m0 = unfkey(s.skey[0]);
+  const float e = tid < n_kept ? expf(unfkey(s.skey[tid]) - m0) : 0.f;
+  const float Z = block_sum(e, s);
+  __syncthreads();
+  if (tid < n_kept) s.skey[tid] = __float_as_uint(e / Z);  // probabilities, still in sorted order
+  __syncthreads();
+  const bool nucleus = a.top_p > 0.f && a.top_p < 1.f;
+  if (!nucleus) {  // vocabulary-order draw (chat_engine.py:82): order the kept entries by id
+    int m2 = 64;
+    while (m2 < n_kept) m2 <<= 1;
+    for (int i = n_kept + tid; i < m2; i += NT) {
+      s.skey[i] = 0;
+      s.sid[i] = 0x7fffffff;
+    }
+    __syncthreads();
+    sort_by_id(s, m2);
+  }
+  if (tid == 0) {
+    // sequential fp32 sums in the order the reference's cumsum walks
+    int tok = -1, last = -1;
+    if (nucleus) {
+      float kept = 0.f, run = 0.f;
+      int n_in = 0;
+      for (int j = 0; j < n_kept; ++j) {  // kept prefix: mass before the token <= top_p
+        if (run > a.top_p) break;
+        const float p = __uint_as_float(s.skey[j]);
+        kept += p;
+        run += p;
+        ++n_in;
+      }
+      const float target = u * kept;
+      run = 0.f;
+      for (int j = 0; j < n_in; ++j) {
+        run += __uint_as_float(s.skey[j]);
+        last = s.sid[j];
+        if (run > target) {
+          tok = s.sid[j];
+          break;
+        }
+      }
+    } else {
+      float total = 0.f;
+      for (int j = 0; j < n_kept; ++j) total += __uint_as_float(s.skey[j]);
+      const float target = u * total;
+      float run = 0.f;
+      for (int j = 0; j < n_kept; ++j) {
+        const float p = __uint_as_float(s.skey[j]);
+        run += p;
+        if (p > 0.f) last = s.sid[j];
+        if (p > 0.f && run > target) {
+          tok = s.sid[j];
+          break;
+        }
+      }
+    }
+    s.misc[3] = tok >= 0 ? tok : max(last, 0);  // rounding pushed the target past the end: last kept id
+  }
+  __syncthreads();
+  return s.misc[3];
+}
+
+// The selected id of a row goes out, with the loop bookkeeping when the caller keeps a step state.
+__device__ __forceinline__ void finish_row(const SampleArgs& a, int b, int token) {
+  a.out[b] = token;
+  if (a.step_state) {
+    const int step = a.step_state[1];
+    if (a.history && step < a.hist_cap) a.history[(size_t)step * a.B + b] = token;
+    // only the counter is shared between workgroups: no fence, the ids are read by later kernels
+    const int old = __hip_atomic_fetch_add(&a.step_state[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (old == a.B - 1) {
+      a.step_state[2] = 0;
+      a.step_state[0] += 1;
+      a.step_state[1] = step + 1;
+    }
+  }
+}
+
+// One workgroup on the whole row b: returns the token in every thread.
 template <typename T, int EPT>
-__global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
-  __shared__ Smem s;
-  const int b = blockIdx.x, tid = threadIdx.x;
+__device__ __forceinline__ int sample_row(const SampleArgs& a, int b, Smem& s) {
+  const int tid = threadIdx.x;
   const int V = a.V, nvalid = min(a.valid, V);
   const int base = tid * EPT;
   float x[EPT];
@@ -535,80 +633,7 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
         }
       }
     }
-    if (compact) {
-      int n2 = 64;
-      while (n2 < n_c) n2 <<= 1;
-      __syncthreads();
-      for (int i = n_c + tid; i < n2; i += NT) {
-        s.skey[i] = 0;  // padding sorts last
-        s.sid[i] = 0x7fffffff;
-      }
-      __syncthreads();
-      sort_candidates(s, n2);
-      // kept: everything >= the k-th largest key (ties at the threshold survive, chat_engine.py:66-69)
-      const uint32_t tk = s.skey[min(k, n_c) - 1];
-      int n_kept = block_sum_i((tid < n_c && s.skey[tid] >= tk) ? 1 : 0, s);
-      // softmax over the kept entries (the rest of the vocabulary is -inf): entry 0 is the maximum
-      const float m0 = unfkey(s.skey[0]);
-      const float e = tid < n_kept ? expf(unfkey(s.skey[tid]) - m0) : 0.f;
-      const float Z = block_sum(e, s);
-      __syncthreads();
-      if (tid < n_kept) s.skey[tid] = __float_as_uint(e / Z);  // probabilities, still in sorted order
-      __syncthreads();
-      const bool nucleus = a.top_p > 0.f && a.top_p < 1.f;
-      if (!nucleus) {  // vocabulary-order draw (chat_engine.py:82): order the kept entries by id
-        int m2 = 64;
-        while (m2 < n_kept) m2 <<= 1;
-        for (int i = n_kept + tid; i < m2; i += NT) {
-          s.skey[i] = 0;
-          s.sid[i] = 0x7fffffff;
-        }
-        __syncthreads();
-        sort_by_id(s, m2);
-      }
-      if (tid == 0) {
-        // sequential fp32 sums in the order the reference's cumsum walks
-        int tok = -1, last = -1;
-        if (nucleus) {
-          float kept = 0.f, run = 0.f;
-          int n_in = 0;
-          for (int j = 0; j < n_kept; ++j) {  // kept prefix: mass before the token <= top_p
-            if (run > a.top_p) break;
-            const float p = __uint_as_float(s.skey[j]);
-            kept += p;
-            run += p;
-            ++n_in;
-          }
-          const float target = u * kept;
-          run = 0.f;
-          for (int j = 0; j < n_in; ++j) {
-            run += __uint_as_float(s.skey[j]);
-            last = s.sid[j];
-            if (run > target) {
-              tok = s.sid[j];
-              break;
-            }
-          }
-        } else {
-          float total = 0.f;
-          for (int j = 0; j < n_kept; ++j) total += __uint_as_float(s.skey[j]);
-          const float target = u * total;
-          float run = 0.f;
-          for (int j = 0; j < n_kept; ++j) {
-            const float p = __uint_as_float(s.skey[j]);
-            run += p;
-            if (p > 0.f) last = s.sid[j];
-            if (p > 0.f && run > target) {
-              tok = s.sid[j];
-              break;
-            }
-          }
-        }
-        s.misc[3] = tok >= 0 ? tok : max(last, 0);  // rounding pushed the target past the end: last kept id
-      }
-      __syncthreads();
-      token = s.misc[3];
-    }
+    if (compact) token = draw_from_block(a, s, n_c, k, u);
   }
   if (!compact && !have_x) load_x();
   // ---- top-k: keep x >= k-th largest ---------------------------------------------
@@ -746,22 +771,150 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
     token = max(s.misc[3], 0);
   }
   }  // !compact
-  if (tid == 0) {
-    a.out[b] = token;
-    if (a.step_state) {
-      const int step = a.step_state[1];
-      if (a.history && step < a.hist_cap) a.history[(size_t)step * a.B + b] = token;
-      // only the counter is shared between workgroups: no fence, the ids are read by later kernels
-      const int old = __hip_atomic_fetch_add(&a.step_state[2], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (old == a.B - 1) {
-        a.step_state[2] = 0;
-        a.step_state[0] += 1;
-        a.step_state[1] = step + 1;
-      }
-    }
-  }
+  return token;
 }
 
+template <typename T, int EPT>
+__global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
+  __shared__ Smem s;
+  const int token = sample_row<T, EPT>(a, blockIdx.x, s);
+  if (threadIdx.x == 0) finish_row(a, blockIdx.x, token);
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// Small top-k over several workgroups.  With top-k the draw depends on the k largest logits of the
+// row only (ties of the k-th included), and one CU walking 65536 ids is what the single-workgroup
+// kernel spends its time on.  Here a row is cut into parts of 8192 ids, one workgroup each (eight ids
+// per thread, one 16-byte load): a part hands over every id at or above the k-th largest of its
+// per-thread maxima - a lower bound of the part's k-th largest, so the union of the parts' candidates
+// holds the row's k largest with all their ties - as (id << 16 | bf16 bits) words; the workgroup that
+// finishes last gathers at most 8 x 128 candidates and draws from them exactly as the single-workgroup
+// kernel draws from its own (draw_from_block).  Candidates travel as write-through stores, the
+// arrival counter is a relaxed device-scope atomic behind a wait for the own stores, the gather uses
+// cache-bypassing loads (the hand-off of the split attention kernels).  A part with more than 128
+// candidates (a row of mostly equal values) makes the last workgroup run the single-workgroup
+// algorithm on the whole row instead.
+// Scratch: a static device array, [row] counters one 128-byte line apart, then per (row, part) one
+// line with the count and 512 bytes of candidates.  Calls that overlap in time on one GPU would share
+// it: the host takes this route only for callers that said their sampler calls do not overlap.
+// ---------------------------------------------------------------------------------------------
+constexpr int PART_IDS = NT * 8;   // ids per part
+constexpr int PART_CAP = 128;      // candidates a part may hand over
+constexpr int PART_MAX = 8;        // parts per row (65536 ids)
+constexpr int PART_ROWS = 64;      // rows per call
+constexpr int PART_REC = 32 + PART_CAP;  // dwords per (row, part) record
+constexpr size_t PART_SCRATCH_DWORDS = (size_t)PART_ROWS * 32 + (size_t)PART_ROWS * PART_MAX * PART_REC;
+
+__global__ __launch_bounds__(NT) void sample_parts_kernel(SampleArgs a, uint32_t* scratch, int nparts) {
+  __shared__ Smem s;
+  const int part = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  const int V = a.V, nvalid = min(a.valid, V);
+  const int k = min(a.top_k, V);
+  const int base = part * PART_IDS + tid * 8;
+  const bf16_t* row = reinterpret_cast<const bf16_t*>(a.logits) + (size_t)b * a.ldl + base;
+  const uint4 v = base < V ? ldg16(row) : make_uint4(0, 0, 0, 0);
+  const uint32_t raw[4] = {v.x, v.y, v.z, v.w};
+  auto bits16 = [&](int i) -> uint32_t { return (i & 1) ? (raw[i >> 1] >> 16) : (raw[i >> 1] & 0xffffu); };
+  auto key16 = [&](int i) -> uint32_t {  // order-preserving 16-bit key of element i, 0 when masked
+    const uint32_t bits = bits16(i);
+    const uint32_t kk = (bits & 0x8000u) ? (~bits & 0xffffu) : (bits | 0x8000u);
+    return base + i < nvalid ? kk : 0u;
+  };
+  uint32_t tmax = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) tmax = max(tmax, key16(i));
+  const int have = block_sum_i(tmax > 0 ? 1 : 0, s);
+  uint32_t bound = 1;  // fewer than k threads hold a valid id: every valid id of the part is a candidate
+  if (have >= k) {
+    int dummy;
+    bound = radix_select<1, 8>(k, dummy, s, [&](int) { return tmax > 0; }, [&](int) { return tmax; });
+  }
+  int c = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) c += key16(i) >= bound ? 1 : 0;
+  int off;
+  const int n_part = block_excl_scan_i(c, off, s);
+  uint32_t* rec = scratch + (size_t)PART_ROWS * 32 + ((size_t)b * PART_MAX + part) * PART_REC;
+  if (n_part <= PART_CAP && c > 0) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (key16(i) >= bound) st_coh4(rec + 32 + off++, ((uint32_t)(base + i) << 16) | bits16(i));
+  }
+  if (tid == 0) st_coh4(rec, n_part <= PART_CAP ? (uint32_t)n_part : 0xffffffffu);
+  // ---- hand-off: the workgroup that arrives last draws -------------------------------------------
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  wait_own_stores();
+  __syncthreads();
+  if (tid == 0) {
+    int* counter = reinterpret_cast<int*>(scratch) + b * 32;
+    const int old = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int last = old == nparts - 1;
+    if (last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next call
+    s.misc[7] = last;
+  }
+  __syncthreads();
+  if (!s.misc[7]) return;
+  const uint32_t* rec0 = scratch + (size_t)PART_ROWS * 32 + (size_t)b * PART_MAX * PART_REC;
+  int total = 0, mine_part = -1, mine_slot = 0;
+  bool overflow = false;
+  for (int p = 0; p < nparts; ++p) {
+    const uint32_t n = ld_coh4(rec0 + (size_t)p * PART_REC);
+    if (n == 0xffffffffu) {
+      overflow = true;
+      break;
+    }
+    if (mine_part < 0 && tid < total + (int)n) {
+      mine_part = p;
+      mine_slot = tid - total;
+    }
+    total += (int)n;
+  }
+  int token;
+  if (overflow) {
+    token = sample_row<bf16_t, 64>(a, b, s);
+  } else {
+    // the k-th largest of the gathered candidates first (16-bit keys, two counting passes), so that the
+    // block that is sorted holds the k survivors and their ties, not eight times as many
+    uint32_t w = 0, k16 = 0;
+    if (tid < total) {
+      w = ld_coh4(rec0 + (size_t)mine_part * PART_REC + 32 + mine_slot);
+      const uint32_t bits = w & 0xffffu;
+      k16 = (bits & 0x8000u) ? (~bits & 0xffffu) : (bits | 0x8000u);
+    }
+    int dummy;
+    const uint32_t tk16 = radix_select<1, 8>(k, dummy, s, [&](int) { return k16 > 0; }, [&](int) { return k16; });
+    const int keep = (k16 > 0 && k16 >= tk16) ? 1 : 0;
+    int slot;
+    const int n_keep = block_excl_scan_i(keep, slot, s);
+    __syncthreads();
+    if (keep) {
+      s.skey[slot] = fkey(__uint_as_float((w & 0xffffu) << 16) / a.temperature);
+      s.sid[slot] = (int)(w >> 16);
+    }
+    const float u = a.u[(a.step_state && a.u_step_stride > 0 ? (size_t)a.step_state[1] * a.u_step_stride : 0) + b];
+    token = draw_from_block(a, s, n_keep, k, u);
+  }
+  if (tid == 0) finish_row(a, b, token);
+}
+
+static __device__ __align__(256) uint32_t sampler_scratch[PART_SCRATCH_DWORDS];
+
+// Device address of sampler_scratch on the current device (nullptr on failure): the array's name is a
+// host-side handle only.
+uint32_t* sampler_scratch_ptr() {
+  static uint32_t* ptrs[16];
+  static std::mutex mu;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(sampler_scratch)) != hipSuccess) return nullptr;
+    ptrs[dev] = reinterpret_cast<uint32_t*>(p);
+  }
+  return ptrs[dev];
+}
 
 // ---------------------------------------------------------------------------------------------
 // bf16 rows of at most 65536 ids: selection on the histogram of the 16-bit keys.
@@ -1133,12 +1286,10 @@ int launch_sample(const SampleArgs& a, hipStream_t st) {
   return ohara_launch_status();
 }
 
-}  // namespace
 
-extern "C" int ohara_sample_topk_topp(const void* logits, int logits_are_fp32, int ldl, int batch, int vocab,
-                                      int valid_vocab, float temperature, int top_k, float top_p, const float* u,
-                                      int u_step_stride, int64_t* out_ids, int64_t* history, int hist_cap,
-                                      int32_t* step_state, void* stream) {
+int sample_dispatch(const void* logits, int logits_are_fp32, int ldl, int batch, int vocab, int valid_vocab,
+                    float temperature, int top_k, float top_p, const float* u, int u_step_stride, int64_t* out_ids,
+                    int64_t* history, int hist_cap, int32_t* step_state, void* stream, bool exclusive) {
   if (!logits || !u || !out_ids || batch < 1 || vocab < 1 || ldl < vocab) return OHARA_EINVAL;
   if (!(temperature > 0.f) || top_k < 0 || !(top_p >= 0.f && top_p <= 1.f) || u_step_stride < 0) return OHARA_EINVAL;
   SampleArgs a{};
@@ -1146,6 +1297,17 @@ extern "C" int ohara_sample_topk_topp(const void* logits, int logits_are_fp32, i
   a.temperature = temperature; a.top_p = top_p; a.top_k = top_k; a.u = u; a.u_step_stride = u_step_stride; a.out = out_ids;
   a.history = history; a.hist_cap = hist_cap; a.step_state = step_state; a.B = batch;
   hipStream_t st = (hipStream_t)stream;
+  const bool aligned = (ldl & 7) == 0 && (reinterpret_cast<uintptr_t>(logits) & 15) == 0;
+  // a small top-k on a long bf16 row, for a caller whose sampler calls do not overlap: the row spread
+  // over one workgroup per 8192 ids (measured at 65536 ids, top-k 50 + top-p 0.9: see the header)
+  if (exclusive && !logits_are_fp32 && aligned && top_k > 0 && top_k <= 64 && vocab > PART_IDS &&
+      vocab <= PART_IDS * PART_MAX && batch <= PART_ROWS && (a.valid < vocab ? a.valid : vocab) >= top_k) {
+    uint32_t* scratch = sampler_scratch_ptr();
+    if (!scratch) return OHARA_ELAUNCH;
+    const int nparts = (vocab + PART_IDS - 1) / PART_IDS;
+    hipLaunchKernelGGL(sample_parts_kernel, dim3(nparts, batch), dim3(NT), 0, st, a, scratch, nparts);
+    return ohara_launch_status();
+  }
   // bf16 rows: selection on the histogram of the 16-bit patterns, except for a small top-k, where sorting
   // the few survivors is quicker (measured at 65536 ids: top-k 50 + top-p 0.9: 27 us sorted, 37 us by the
   // table; top-p alone: 37 us (sharp row) to 139 us (flat row) with candidates / bisection, 37-38 us by
@@ -1159,3 +1321,24 @@ extern "C" int ohara_sample_topk_topp(const void* logits, int logits_are_fp32, i
   }
   return logits_are_fp32 ? launch_sample<float>(a, st) : launch_sample<bf16_t>(a, st);
 }
+
+}  // namespace
+
+extern "C" {
+
+int ohara_sample_topk_topp(const void* logits, int logits_are_fp32, int ldl, int batch, int vocab, int valid_vocab,
+                           float temperature, int top_k, float top_p, const float* u, int u_step_stride,
+                           int64_t* out_ids, int64_t* history, int hist_cap, int32_t* step_state, void* stream) {
+  return sample_dispatch(logits, logits_are_fp32, ldl, batch, vocab, valid_vocab, temperature, top_k, top_p, u,
+                         u_step_stride, out_ids, history, hist_cap, step_state, stream, false);
+}
+
+int ohara_sample_topk_topp_exclusive(const void* logits, int logits_are_fp32, int ldl, int batch, int vocab,
+                                     int valid_vocab, float temperature, int top_k, float top_p, const float* u,
+                                     int u_step_stride, int64_t* out_ids, int64_t* history, int hist_cap,
+                                     int32_t* step_state, void* stream) {
+  return sample_dispatch(logits, logits_are_fp32, ldl, batch, vocab, valid_vocab, temperature, top_k, top_p, u,
+                         u_step_stride, out_ids, history, hist_cap, step_state, stream, true);
+}
+
+}  // extern "C"

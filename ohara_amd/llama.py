@@ -628,7 +628,7 @@ class DecodeSession:
             # the sampler does the selection kernel's bookkeeping (next ids, history, position)
             ops.sample_topk_topp(self.logits, self.sampling.temperature, self.sampling.top_k, self.sampling.top_p,
                                  self.u, self.valid_vocab or None, out=self._dbuf.ids[: self.batch],
-                                 history=self.history, step_state=self._dbuf.step_state, u_per_step=True)
+                                 history=self.history, step_state=self._dbuf.step_state, u_per_step=True, exclusive=True)
 
     def check_error(self) -> None:
         """Raise if a barrier wait of the persistent kernel expired (synchronises)."""

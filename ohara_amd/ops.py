@@ -312,9 +312,11 @@ def argmax(logits: torch.Tensor, valid_vocab: int | None = None, next_ids=None, 
 
 def sample_topk_topp(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, u: torch.Tensor,
                      valid_vocab: int | None = None, out=None, history=None, step_state=None,
-                     u_per_step: bool = False) -> torch.Tensor:
+                     u_per_step: bool = False, exclusive: bool = False) -> torch.Tensor:
     """logits (B, V) bf16 or fp32 on the device, u (B,) fp32 uniform draws -> ids (B,) int64.
-    With ``u_per_step`` (needs step_state) u is (steps, B) and row ``step`` is read on the device."""
+    With ``u_per_step`` (needs step_state) u is (steps, B) and row ``step`` is read on the device.
+    ``exclusive``: the caller's sampler calls on this GPU do not overlap in time (a decode loop on one
+    stream), which lets a small top-k on a long row run on several workgroups (same results)."""
     if logits.dtype not in (BF16, torch.float32):
         raise ValueError("logits must be bfloat16 or float32")
     _need(logits, logits.dtype, "logits")
@@ -328,7 +330,7 @@ def sample_topk_topp(logits: torch.Tensor, temperature: float, top_k: int, top_p
     if out is None:
         out = torch.empty(b, dtype=torch.int64, device=logits.device)
     check(
-        lib().ohara_sample_topk_topp(
+        (lib().ohara_sample_topk_topp_exclusive if exclusive else lib().ohara_sample_topk_topp)(
             _ptr(logits), 1 if logits.dtype == torch.float32 else 0, logits.stride(0), b, v,
             v if valid_vocab is None else valid_vocab, float(temperature), int(top_k), float(top_p), _ptr(u),
             b if u_per_step else 0, _ptr(out), _ptr(history), 0 if history is None else history.shape[0], _ptr(step_state), _stream(),

@@ -180,3 +180,54 @@ def test_rows_of_one_single_value(cuda):
         got = ops.sample_topk_topp(row, 1.0, 2000, 1.0, u).cpu()  # top-k keeps every tie
         for b in range(2):
             assert abs(int(got[b]) - int(float(u[b]) * V)) <= 2, (V, b, int(got[b]))
+
+
+@pytest.mark.parametrize("V,B,T,k,p,std", [(65536, 8, 0.8, 50, 0.9, 0.55), (65536, 3, 1.0, 1, 1.0, 1.0),
+                                           (32000, 5, 0.7, 64, 0.0, 2.0), (50000, 2, 1.2, 40, 0.95, 6.0)])
+def test_small_top_k_over_several_workgroups(cuda, V, B, T, k, p, std):
+    """ohara_sample_topk_topp_exclusive spreads a small top-k on a long bf16 row over one workgroup per
+    8192 ids: the same token as the single-workgroup kernel for the same draw, on calls in a row (the
+    arrival counters return to zero), with a masked vocabulary tail, and inside the oracle's CDF interval."""
+    from ohara_amd import ops
+
+    g = torch.Generator().manual_seed(V + B + k)
+    logits = (torch.randn(B, V, generator=g) * std).to(torch.bfloat16)
+    dl = logits.to(cuda)
+    tol = 5e-5
+    for trial in range(5):
+        u = torch.rand(B, generator=g)
+        if trial == 0:
+            u[0] = 0.0
+            u[-1] = 0.999999
+        valid = None if trial < 3 else V - 5000
+        one = ops.sample_topk_topp(dl, T, k, p, u.to(cuda), valid).cpu()
+        many = ops.sample_topk_topp(dl, T, k, p, u.to(cuda), valid, exclusive=True).cpu()
+        assert torch.equal(one, many), (trial, one, many)
+        if valid is None:
+            ids, cdf = candidate_cdf_ref(logits.unsqueeze(1), T, p, k)
+            for b in range(B):
+                j = int((ids[b] == int(many[b])).nonzero()[0])
+                lo = float(cdf[b, j - 1]) if j > 0 else 0.0
+                assert lo - tol <= float(u[b]) <= float(cdf[b, j]) + tol
+    # ties: rows of few distinct values (more than 128 candidates in a part: the last workgroup walks the
+    # whole row itself), and a row whose largest values all sit in one part
+    tied = (torch.randint(0, 3, (B, V), generator=g).float() * 2).to(torch.bfloat16)
+    one_part = logits.clone()
+    one_part[:, 9000:9100] += 12.0
+    for rows in (tied, one_part):
+        u = torch.rand(B, generator=g)
+        one = ops.sample_topk_topp(rows.to(cuda), T, k, p, u.to(cuda)).cpu()
+        many = ops.sample_topk_topp(rows.to(cuda), T, k, p, u.to(cuda), exclusive=True).cpu()
+        assert torch.equal(one, many)
+    # the device-side bookkeeping (history, step counter, draws indexed by step)
+    steps = 3
+    us = torch.rand(steps, B, generator=g).to(cuda)
+    for excl in (False, True):
+        state = torch.tensor([7, 0, 0, 0], dtype=torch.int32, device=cuda)
+        hist = torch.zeros(steps, B, dtype=torch.int64, device=cuda)
+        out = torch.zeros(B, dtype=torch.int64, device=cuda)
+        for _ in range(steps):
+            ops.sample_topk_topp(dl, T, k, p, us, out=out, history=hist, step_state=state, u_per_step=True, exclusive=excl)
+        if excl:
+            assert torch.equal(hist, first_hist) and state.tolist() == [7 + steps, steps, 0, 0]
+        first_hist = hist.clone()
