@@ -235,6 +235,7 @@ class BitDecodeSession:
         self.produced = 0
         self.pos = 0
         self.graph = None
+        self.graph_multi = None
         self._dst = None
         self._pws = None
 
@@ -354,7 +355,10 @@ class BitDecodeSession:
         self.pos += 1
         self.produced += 1
 
+    GRAPH_STEPS = 8  # steps in the second captured graph
+
     def capture(self) -> None:
+        """One step in one HIP graph, GRAPH_STEPS steps in a second (one host launch per eight tokens)."""
         if self.graph is not None:
             return
         self.step()
@@ -362,6 +366,11 @@ class BitDecodeSession:
         with torch.cuda.graph(g):
             self._launch_step()
         self.graph = g
+        gm = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gm):
+            for _ in range(self.GRAPH_STEPS):
+                self._launch_step()
+        self.graph_multi = gm
 
     def run(self, n: int, use_graph: bool = True) -> None:
         """Enqueue n more decode steps."""
@@ -375,7 +384,10 @@ class BitDecodeSession:
             self.capture()
             n -= 1
         self._room(n)
-        for _ in range(n):
+        many, rest = divmod(n, self.GRAPH_STEPS)
+        for _ in range(many):
+            self.graph_multi.replay()
+        for _ in range(rest):
             self.graph.replay()
         self._advance(n)
 
