@@ -40,6 +40,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(PrefillArgs a) {
   constexpr int GP = RPT >= 4 ? 4 : 2;   // positions a thread transposes together
   __shared__ __align__(16) bf16_t Ks[KT][LDK];
   __shared__ __align__(16) bf16_t Vt[D][LDV];
+  // A column's 64 positions are rotated by four positions per group of eight columns (GP == 4): the sixteen
+  // threads that transpose one position group write columns eight apart, which would land on two banks.
+  auto vt_off = [](int col, int p) { return GP == 4 ? ((p + 4 * (col >> 3)) & (KT - 1)) : p; };
 
   // heavy (late) query blocks first
   const int qblk = a.nqb - 1 - (int)blockIdx.x;
@@ -118,8 +121,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(PrefillArgs a) {
         if (GP == 4) {
           const uint32_t lo23 = (w[GP - 2][e] & 0xffffu) | (w[GP - 1][e] << 16);
           const uint32_t hi23 = (w[GP - 2][e] >> 16) | (w[GP - 1][e] & 0xffff0000u);
-          *reinterpret_cast<uint2*>(&Vt[lc * 8 + 2 * e][p0]) = make_uint2(lo01, lo23);
-          *reinterpret_cast<uint2*>(&Vt[lc * 8 + 2 * e + 1][p0]) = make_uint2(hi01, hi23);
+          *reinterpret_cast<uint2*>(&Vt[lc * 8 + 2 * e][vt_off(lc * 8 + 2 * e, p0)]) = make_uint2(lo01, lo23);
+          *reinterpret_cast<uint2*>(&Vt[lc * 8 + 2 * e + 1][vt_off(lc * 8 + 2 * e + 1, p0)]) = make_uint2(hi01, hi23);
         } else {
           *reinterpret_cast<uint32_t*>(&Vt[lc * 8 + 2 * e][p0]) = lo01;
           *reinterpret_cast<uint32_t*>(&Vt[lc * 8 + 2 * e + 1][p0]) = hi01;
@@ -155,21 +158,30 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(PrefillArgs a) {
     uint4 pf[2][2];  // [qb][32-position window]: B operand of the second product
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
-      const bool diag = t0 + KT - 1 > qpos[qb];  // tile reaches past this query's position
       float tmax = -INFINITY;
+      float mul = 1.0f;  // what the stored scores still have to be multiplied with
+      if (t0 + KT - 1 > a.pos + wq0) {  // (wave-uniform) the tile reaches past the wave's first query: mask
 #pragma unroll
-      for (int kbk = 0; kbk < 4; ++kbk)
+        for (int kbk = 0; kbk < 4; ++kbk)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float v = s[kbk][qb][i] * a.scale_log2e;
-          if (diag && t0 + kbk * 16 + 4 * g + i > qpos[qb]) v = -INFINITY;
-          s[kbk][qb][i] = v;
-          tmax = fmaxf(tmax, v);
-        }
+          for (int i = 0; i < 4; ++i) {
+            float v = s[kbk][qb][i] * a.scale_log2e;
+            if (t0 + kbk * 16 + 4 * g + i > qpos[qb]) v = -INFINITY;
+            s[kbk][qb][i] = v;
+            tmax = fmaxf(tmax, v);
+          }
+      } else {
+#pragma unroll
+        for (int kbk = 0; kbk < 4; ++kbk)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, s[kbk][qb][i]);
+        tmax *= a.scale_log2e;  // the scale is positive: the maximum of the products is the product of the maximum
+        mul = a.scale_log2e;    // and the scaling itself rides in the fused multiply-add of the exponent below
+      }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
       const float mn = fmaxf(m_run[qb], tmax);  // finite: position 0 is visible to every query
-      const float corr = exp2f(m_run[qb] - mn);
+      const float corr = __builtin_amdgcn_exp2f(m_run[qb] - mn);  // arguments <= 0: the bare instruction is exact enough and 2^-inf = 0
       m_run[qb] = mn;
       float ts = 0.f;
       float p[4][4];
@@ -177,14 +189,16 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(PrefillArgs a) {
       for (int kbk = 0; kbk < 4; ++kbk)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          p[kbk][i] = exp2f(s[kbk][qb][i] - mn);
+          p[kbk][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kbk][qb][i], mul, -mn));
           ts += p[kbk][i];
         }
       l_run[qb] = l_run[qb] * corr + ts;  // this lane's share; lanes g = 0..3 are added at the end
+      if (__any(corr != 1.0f)) {  // most tiles leave the running maximum of every query of the wave alone
 #pragma unroll
-      for (int db = 0; db < ND; ++db)
+        for (int db = 0; db < ND; ++db)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[qb][db][i] *= corr;
+          for (int i = 0; i < 4; ++i) o[qb][db][i] *= corr;
+      }
       // k-slot 8 g + i of window w  <->  position 32 w + 4 g + i (i < 4), 32 w + 16 + 4 g + i - 4
 #pragma unroll
       for (int w = 0; w < 2; ++w)
@@ -196,8 +210,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(PrefillArgs a) {
     for (int w = 0; w < 2; ++w)
 #pragma unroll
       for (int db = 0; db < ND; ++db) {
-        const uint2 v0 = *reinterpret_cast<const uint2*>(&Vt[db * 16 + m][32 * w + 4 * g]);
-        const uint2 v1 = *reinterpret_cast<const uint2*>(&Vt[db * 16 + m][32 * w + 16 + 4 * g]);
+        const uint2 v0 = *reinterpret_cast<const uint2*>(&Vt[db * 16 + m][vt_off(db * 16 + m, 32 * w + 4 * g)]);
+        const uint2 v1 = *reinterpret_cast<const uint2*>(&Vt[db * 16 + m][vt_off(db * 16 + m, 32 * w + 16 + 4 * g)]);
         const uint4 vf = make_uint4(v0.x, v0.y, v1.x, v1.y);
         o[0][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf),
                                                            __builtin_bit_cast(bf16x8, pf[0][w]), o[0][db], 0, 0, 0);
