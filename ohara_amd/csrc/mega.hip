@@ -64,11 +64,12 @@ struct MegaArgs {
 // ---------------------------------------------------------------------------------------
 // the kernel
 // ---------------------------------------------------------------------------------------
-template <int D, int G>
+// ONE: the batch is a single sequence (the row loops and row masks fold away at compile time).
+template <int D, int G, bool ONE>
 __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const OharaModel& m = a.m;
-  const int d = m.d_model, H = m.n_heads, Hkv = m.n_kv_heads, F = m.d_ff, V = m.vocab, B = a.B;
+  const int d = m.d_model, H = m.n_heads, Hkv = m.n_kv_heads, F = m.d_ff, V = m.vocab, B = ONE ? 1 : a.B;
   const int kmax = max(d, max(F, H * D));
   const int ldxs = kmax + 8;
   bf16_t* xs = reinterpret_cast<bf16_t*>(smem);
@@ -107,10 +108,12 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   lm.N = V; lm.K = d; lm.nstrips = (V + 15) / 16; lm.out = reinterpret_cast<char*>(a.logits); lm.ldo = V;
   lm.valid = a.valid_vocab > 0 ? min(a.valid_vocab, V) : V;
   lm.wp = reinterpret_cast<const uint4*>(m.w_vocab);
+  lm.norm_w = m.final_norm;
 
   GemmPre pre;
   AttnPre<D> apre;
   qkv.wp = lds_ptr<const uint4>(ptab, 0);
+  qkv.norm_w = lds_ptr<const bf16_t>(ptab, 4);
   gemm_prefetch<4, 6, E_ROPE>(qkv, pre, B);
   pf.stamp();
   for (int l = 0; l < m.n_layers; ++l) {
@@ -128,8 +131,8 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     // P1: [embedding] + norm1 + QKV + rotary + append
     qkv.kc = kc; qkv.vc = vc; qkv.out = q_l;
     if ((int)blockIdx.x < qkv.nstrips) {
-      if (l == 0) stage_norm<2, true>(xs, ldxs, a.xm, 0, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d);
-      else stage_norm<2, false>(xs, ldxs, x_prev, a.blk_x, d_prev, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d);
+      if (l == 0) stage_norm<2, true, true>(xs, ldxs, a.xm, 0, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d, pre.g);
+      else stage_norm<2, false, true>(xs, ldxs, x_prev, a.blk_x, d_prev, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d, pre.g);
     }
     __syncthreads();
     pf.stamp();
@@ -161,12 +164,12 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     gemm_phase<4, 6, E_RESID>(prj, pre, xs, ldxs, B, red, best_v, best_i, pf);
     pf.stamp();
     gs.arrive(pf);
-    gu.wp = lds_ptr<const uint4>(pl, 2); gu.out = a_l;
+    gu.wp = lds_ptr<const uint4>(pl, 2); gu.out = a_l; gu.norm_w = lds_ptr<const bf16_t>(pl, 5);
     gemm_prefetch<2, 12, E_SWIGLU>(gu, pre, B);
     gs.wait(pf);
     pf.stamp();
     // P4: norm2 + gate/up + SwiGLU
-    if ((int)blockIdx.x * 2 < gu.nstrips) stage_norm<2, false>(xs, ldxs, x_mid, a.blk_x, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 5), m.eps, B, d);
+    if ((int)blockIdx.x * 2 < gu.nstrips) stage_norm<2, false, true>(xs, ldxs, x_mid, a.blk_x, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 5), m.eps, B, d, pre.g);
     __syncthreads();
     gemm_phase<2, 12, E_SWIGLU>(gu, pre, xs, ldxs, B, red, best_v, best_i, pf);
     gs.arrive(pf);
@@ -190,6 +193,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     gs.arrive(pf);
     if (l + 1 < m.n_layers) {
       qkv.wp = lds_ptr<const uint4>(pl, 8);
+      qkv.norm_w = lds_ptr<const bf16_t>(pl, 12);
       gemm_prefetch<4, 6, E_ROPE>(qkv, pre, B);
     } else {
       gemm_prefetch<1, 24, E_LOGITS>(lm, pre, B);
@@ -198,8 +202,9 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     pf.stamp();
   }
   // final norm + vocabulary projection, running arg-max per lane
-  stage_norm<2, false>(xs, ldxs, a.xm + (size_t)(m.n_layers - 1) * a.xm_stride, a.blk_x,
-                       a.dm + (size_t)(m.n_layers - 1) * a.dm_stride, a.ids, m.token_emb, V, m.final_norm, m.eps, B, d);
+  stage_norm<2, false, true>(xs, ldxs, a.xm + (size_t)(m.n_layers - 1) * a.xm_stride, a.blk_x,
+                             a.dm + (size_t)(m.n_layers - 1) * a.dm_stride, a.ids, m.token_emb, V, m.final_norm, m.eps, B, d,
+                             pre.g);
   __syncthreads();
   gemm_phase<1, 24, E_LOGITS>(lm, pre, xs, ldxs, B, red, best_v, best_i, pf);
   pf.stamp();
@@ -400,12 +405,17 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   const size_t smem = xs_bytes + 4096 + (size_t)(8 + 4 * D) * G * sizeof(float) + mrg + (size_t)m->n_layers * 64;
   if (smem > 160 * 1024) return OHARA_ESIZE;
   dim3 grid(n_workgroups), block(256);
-#define OHARA_MEGA(DD, GG)                                                                                  \
+#define OHARA_MEGA_B(DD, GG, ONE_)                                                                          \
   do {                                                                                                      \
     if (smem > 64 * 1024)                                                                                   \
-      (void)hipFuncSetAttribute((const void*)decode_mega_kernel<DD, GG>,                                    \
+      (void)hipFuncSetAttribute((const void*)decode_mega_kernel<DD, GG, ONE_>,                              \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);                     \
-    hipLaunchKernelGGL((decode_mega_kernel<DD, GG>), grid, block, smem, st, a);                             \
+    hipLaunchKernelGGL((decode_mega_kernel<DD, GG, ONE_>), grid, block, smem, st, a);                       \
+  } while (0)
+#define OHARA_MEGA(DD, GG)                                                                                  \
+  do {                                                                                                      \
+    if (s->batch == 1) OHARA_MEGA_B(DD, GG, true);                                                          \
+    else OHARA_MEGA_B(DD, GG, false);                                                                       \
   } while (0)
   if (D == 128 && G == 1) OHARA_MEGA(128, 1);
   else if (D == 128 && G == 2) OHARA_MEGA(128, 2);
@@ -414,6 +424,7 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   else if (D == 64 && G == 2) OHARA_MEGA(64, 2);
   else OHARA_MEGA(64, 4);
 #undef OHARA_MEGA
+#undef OHARA_MEGA_B
   return ohara_launch_status();
 }
 

@@ -185,9 +185,11 @@ __device__ __forceinline__ void x_load(const XParts& xp, int b, int n, uint32_t 
 // norm.py:16-21 on rows of the residual stream (x-mailbox `src`), or - for the first layer
 // - on rows gathered from the embedding table (llama.py:310).  One wave per row; all loads
 // of a row are issued before any is consumed.  K <= 8 * 64 * NLD elements.
-template <int NLD, bool EMBED>
-__device__ void stage_norm(bf16_t* xs, int ldxs, const char* src, int blk, const float* parts, const int64_t* ids,
-                           const bf16_t* table, int vocab, const bf16_t* nw, float eps, int B, int K) {
+// PRE: the lane's norm-weight pieces were fetched ahead (gemm_prefetch) and are in gpre[0 .. NLD).
+template <int NLD, bool EMBED, bool PRE = false>
+__device__ __forceinline__ void stage_norm(bf16_t* xs, int ldxs, const char* src, int blk, const float* parts,
+                                           const int64_t* ids, const bf16_t* table, int vocab, const bf16_t* nw, float eps,
+                                           int B, int K, const uint4 (&gpre)[NLD]) {
   const XParts xp{src, parts, blk, B, K};
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int b = wave; b < B; b += 4) {
@@ -211,7 +213,7 @@ __device__ void stage_norm(bf16_t* xs, int ldxs, const char* src, int blk, const
           x_load<8>(xp, b, k, w);
           v[c] = make_uint4(w[0], w[1], w[2], w[3]);
         }
-        g[c] = ldg16(nw + k);
+        g[c] = PRE ? gpre[c] : ldg16(nw + k);
       }
     }
     float ss = 0.f;
@@ -244,7 +246,7 @@ __device__ void stage_norm(bf16_t* xs, int ldxs, const char* src, int blk, const
 
 // act mailbox (B, F) -> LDS
 // act mailbox (B, F), columns [f0, f1) (multiples of 8) -> LDS
-__device__ void stage_act(bf16_t* xs, int ldxs, const char* src, int blk, int B, int f0, int f1) {
+__device__ __forceinline__ void stage_act(bf16_t* xs, int ldxs, const char* src, int blk, int B, int f0, int f1) {
   const int n8 = (f1 - f0) >> 3;
   for (int i = threadIdx.x; i < B * n8; i += blockDim.x) {
     const int b = i / n8, c = (f0 >> 3) + i - b * n8;
@@ -331,7 +333,7 @@ __device__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, i
 // One pass for the small case (all OHARA_MEGA_NS chunks in use, one group of four columns per
 // thread): every thread fetches the (max, sum) pairs itself, so there is a single round of loads
 // and no workgroup barrier.
-__device__ void stage_attn_merge_small(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh) {
+__device__ __forceinline__ void stage_attn_merge_small(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh) {
   constexpr int NS = OHARA_MEGA_NS;
   const int HD = H * Dh, PS = Dh + 32;
   const int e = threadIdx.x * 4;
@@ -391,11 +393,13 @@ struct GemmP {
   bf16_t* vc;
   int valid;       // E_LOGITS: ids >= valid never win
   int ldo;         // E_LOGITS: row stride of the logits
+  const bf16_t* norm_w;  // weights of the norm staged ahead of this phase (fetched with the weights when set)
 };
 
 struct GemmPre {  // one register buffer, reused by every phase (only one prefetch is live at a time)
   uint4 w[OHARA_MAX_PF];
-  uint2 r;        // E_RESID: the four residual values of this lane (first strip)
+  uint4 g[2];     // the lane's pieces of the weights of the norm staged ahead of the phase (GemmP::norm_w)
+  uint2 r;        // E_RESID: the four residual values of this lane (first strip); E_ROPE: its cos / sin pairs
 };
 
 // Work unit -> strip and this wave's k-steps [j0, j1).  E_PART: the units of K partition q follow
@@ -430,6 +434,26 @@ __device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int 
 #pragma unroll
   for (int c = 0; c < PF; ++c)
     pre.w[c] = (live && j0 + c < j1) ? ldg16_nt(wrow + (size_t)(j0 + c) * 64) : make_uint4(0, 0, 0, 0);
+  // Everything else the phase reads that does not depend on the phase before it is requested here
+  // too: cold reads from HBM behind the barrier would sit on the critical path of the phase.
+  if (EPI == E_ROPE || EPI == E_SWIGLU || EPI == E_LOGITS) {
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int k = (c * 64 + lane) * 8;
+      pre.g[c] = (p.norm_w && wave < B && k < p.K) ? ldg16(p.norm_w + k) : make_uint4(0, 0, 0, 0);
+    }
+  }
+  if (EPI == E_ROPE) {
+    const int m = lane & 15, g = lane >> 4;
+    const int r0 = strip * 16 + 4 * g;
+    const int nq = p.H * p.Dh, nk = p.Hkv * p.Dh;
+    pre.r = make_uint2(0, 0);
+    if (live && kpart == 0 && m < B && r0 < nq + nk && p.pos >= 0 && p.pos < p.Tmax) {
+      const int d = (r0 < nq ? r0 : r0 - nq) % p.Dh;
+      pre.r = make_uint2(ldg4(p.cos + (size_t)p.pos * (p.Dh >> 1) + (d >> 1)),
+                         ldg4(p.sin + (size_t)p.pos * (p.Dh >> 1) + (d >> 1)));
+    }
+  }
   if (EPI == E_RESID) {
     const int m = lane & 15, g = lane >> 4;
     const int r0 = strip * 16 + 4 * g;
@@ -576,8 +600,8 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
           char* o;
           if (r0 < nq + nk) {
             const int d = (r0 < nq ? r0 : r0 - nq) % p.Dh;
-            const uint32_t cs = ldg4(p.cos + (size_t)p.pos * (p.Dh >> 1) + (d >> 1));
-            const uint32_t sn = ldg4(p.sin + (size_t)p.pos * (p.Dh >> 1) + (d >> 1));
+            const uint32_t cs = it == 0 ? pre.r.x : ldg4(p.cos + (size_t)p.pos * (p.Dh >> 1) + (d >> 1));
+            const uint32_t sn = it == 0 ? pre.r.y : ldg4(p.sin + (size_t)p.pos * (p.Dh >> 1) + (d >> 1));
             const float c2[2] = {lo_bf(cs), hi_bf(cs)}, s2[2] = {lo_bf(sn), hi_bf(sn)};
 #pragma unroll
             for (int pr = 0; pr < 2; ++pr) {
