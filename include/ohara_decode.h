@@ -418,7 +418,9 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
                                   int init_workspace, int select_greedy, unsigned int spin_limit, void* stream);
 /* Byte offsets inside the workspace: the barrier words; the sticky error word (uint32,
  * non-zero after a barrier wait expired); 1024 x uint64 shader-clock samples taken by
- * workgroup 0 at every phase boundary when s->prof_kernel == -2 (measurement only). */
+ * workgroup 0 at every phase boundary when s->prof_kernel == -2 (measurement only; the samples
+ * are compiled into a separate build of the kernel that exists for head_dim 128 with
+ * n_kv_heads == n_heads only, other shapes leave the slots untouched). */
 int64_t ohara_persistent_barrier_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
 int64_t ohara_persistent_error_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
 int64_t ohara_persistent_profile_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
@@ -472,7 +474,8 @@ int64_t ohara_bitnet_persistent_workspace_bytes(const OharaBitModel* m, int batc
 int64_t ohara_bitnet_persistent_error_offset(const OharaBitModel* m, int batch, int n_workgroups);
 /* 1024 x uint64 shader-clock samples of workgroup 0 (six per grid barrier: phase work issued, own
  * stores complete, workgroup barrier passed, arrival issued, prefetch issued, barrier passed), taken
- * when s->prof_kernel == -2 (measurement only). */
+ * when s->prof_kernel == -2 (measurement only; a separate build of the kernel that exists for
+ * head_dim 128 only, other shapes leave the slots untouched). */
 int64_t ohara_bitnet_persistent_profile_offset(const OharaBitModel* m, int batch, int n_workgroups);
 int ohara_bitnet_decode_persistent(const OharaBitModel* m, const OharaDecodeState* s, void* workspace, int n_workgroups,
                                    int init_workspace, int select_greedy, unsigned int spin_limit, void* stream);

@@ -604,11 +604,15 @@ __device__ void bit_stage_final_norm(bf16_t* xs, int ldxs, const BitX& x, const 
 // ---------------------------------------------------------------------------------------
 // the kernel
 // ---------------------------------------------------------------------------------------
-template <int D, int G>
+// ONE: a single sequence.  The block-owned-row staging is then the only one compiled in, the
+// wave-owned-row staging otherwise, which keeps either kernel's layer loop much smaller than one
+// that holds both.
+// PROFILE: with the phase stamps (measurement builds of the head-dim-128 kernels only).
+template <int D, int G, bool ONE, bool PROFILE = false>
 __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const OharaBitModel& m = a.m;
-  const int d = m.d_model, H = m.n_heads, Hkv = m.n_kv_heads, F = m.d_ff, V = m.vocab, B = a.B;
+  const int d = m.d_model, H = m.n_heads, Hkv = m.n_kv_heads, F = m.d_ff, V = m.vocab, B = ONE ? 1 : a.B;
   const int nwg = gridDim.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int mm = lane & 15, gg = lane >> 4;
@@ -624,7 +628,7 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
   L.shape(B, d);
   size_t off = (codes_bytes + 255) & ~(size_t)255;
   const int KpF = ((F + 255) >> 8) << 8;
-  const size_t stage_bytes = max((size_t)B * (dmax + 8) * 2, (B > 1 && F > 2048) ? (size_t)B * KpF * 2 : (size_t)0);
+  const size_t stage_bytes = max((size_t)B * (dmax + 8) * 2, (!ONE && F > 2048) ? (size_t)B * KpF * 2 : (size_t)0);
   L.ldst = KpF;
   L.stage = reinterpret_cast<bf16_t*>(smem + off);
   L.ldm = dmax + 8;
@@ -660,7 +664,7 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
   const int Lc = min(pos + 1, m.t_max);
   float best_v = -INFINITY;
   int best_i = 0x7fffffff;
-  Prof pf{(blockIdx.x == 0 && tid == 0) ? a.prof : nullptr, 0};
+  ProfT<PROFILE> pf((blockIdx.x == 0 && tid == 0) ? a.prof : nullptr);
 
   const int KCd = (d + 255) >> 8, KCo = (HD + 255) >> 8, KCf = (F + 255) >> 8;
   const int ns_q = HD / 16, ns_kv = (Hkv * D) / 16, ns_d = (d + 15) / 16, ns_f = (F + 15) / 16;
@@ -728,7 +732,7 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
         bitx_load<8>(xin, b, p * 8, w);
         return make_uint4(w[0], w[1], w[2], w[3]);
       };
-      if (B == 1) {
+      if (ONE) {
         auto load0 = [&](int p) { return load_in(0, p); };
         bit_stage_row1<1>(L, 1, d, norm1, nw, nullptr, m.eps, load0);
       } else {
@@ -789,15 +793,10 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
       if (first) {
         bf16_t* xs = L.stage;
         const int ldxs = L.ldm;
-        if (a.ns == OHARA_MEGA_NS && B * HD <= 4 * 256) stage_attn_merge_small(xs, ldxs, p_l, B, H, D);
-        else if (a.ns == 16) stage_attn_merge<16>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
-        else if (a.ns == 8) stage_attn_merge<8>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
-        else if (a.ns == 4) stage_attn_merge<4>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
-        else if (a.ns == 2) stage_attn_merge<2>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
-        else stage_attn_merge<1>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
+        stage_attn_merge_any<false>(a.ns, xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
         __syncthreads();
         const bf16_t* nwo = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BO]));
-        if (B == 1) {
+        if (ONE) {
           auto load0 = [&](int p) { return lds16(xs + p * 8); };
           bit_stage_row1<1>(L, 1, HD, nullptr, nwo, nullptr, m.eps, load0);
         } else {
@@ -841,7 +840,7 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
       };
       const bf16_t* nwg_ = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BG]));
       const bf16_t* nwu_ = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BU]));
-      if (B == 1) {
+      if (ONE) {
         auto load0 = [&](int p) { return load_mid(0, p); };
         bit_stage_row1<1>(L, 2, d, norm2, nwg_, nwu_, m.eps, load0);
       } else {
@@ -887,7 +886,7 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
         const int part = unit / ns_d, strip = unit - part * ns_d;
         if (!staged) {
           const bf16_t* nwd = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BD]));
-          if (B == 1) {
+          if (ONE) {
             auto load0 = [&](int p) { return ldg16(am_addr(a_l, a.blk_a, 0, p * 8)); };
             if (F <= 2048) bit_stage_row1<1>(L, 1, F, nullptr, nwd, nullptr, m.eps, load0);
             else bit_stage_row1<3>(L, 1, F, nullptr, nwd, nullptr, m.eps, load0);
@@ -1145,16 +1144,33 @@ int ohara_bitnet_decode_persistent(const OharaBitModel* m, const OharaDecodeStat
   const size_t smem = bit_smem_bytes(m, s->batch, ns);
   if (smem > 160 * 1024) return OHARA_ESIZE;
   dim3 grid(n_workgroups), block(256);
-#define OHARA_BITMEGA(DD)                                                                                    \
+#define OHARA_BITMEGA_B(DD, ONE_)                                                                            \
   do {                                                                                                       \
     if (smem > 64 * 1024)                                                                                    \
-      (void)hipFuncSetAttribute((const void*)bitnet_mega_kernel<DD, 1>,                                      \
+      (void)hipFuncSetAttribute((const void*)bitnet_mega_kernel<DD, 1, ONE_>,                                \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);                      \
-    hipLaunchKernelGGL((bitnet_mega_kernel<DD, 1>), grid, block, smem, st, a);                               \
+    hipLaunchKernelGGL((bitnet_mega_kernel<DD, 1, ONE_>), grid, block, smem, st, a);                         \
   } while (0)
-  if (D == 128) OHARA_BITMEGA(128);
+#define OHARA_BITMEGA(DD)                                                                                    \
+  do {                                                                                                       \
+    if (s->batch == 1) OHARA_BITMEGA_B(DD, true);                                                            \
+    else OHARA_BITMEGA_B(DD, false);                                                                         \
+  } while (0)
+#define OHARA_BITMEGA_PROF(ONE_)                                                                             \
+  do {                                                                                                       \
+    if (smem > 64 * 1024)                                                                                    \
+      (void)hipFuncSetAttribute((const void*)bitnet_mega_kernel<128, 1, ONE_, true>,                         \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);                      \
+    hipLaunchKernelGGL((bitnet_mega_kernel<128, 1, ONE_, true>), grid, block, smem, st, a);                  \
+  } while (0)
+  if (a.prof && D == 128) {  // the stamps exist in these two instantiations only
+    if (s->batch == 1) OHARA_BITMEGA_PROF(true);
+    else OHARA_BITMEGA_PROF(false);
+  } else if (D == 128) OHARA_BITMEGA(128);
   else OHARA_BITMEGA(64);
 #undef OHARA_BITMEGA
+#undef OHARA_BITMEGA_B
+#undef OHARA_BITMEGA_PROF
   return ohara_launch_status();
 }
 

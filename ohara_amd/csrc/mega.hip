@@ -65,7 +65,8 @@ struct MegaArgs {
 // the kernel
 // ---------------------------------------------------------------------------------------
 // ONE: the batch is a single sequence (the row loops and row masks fold away at compile time).
-template <int D, int G, bool ONE>
+// PROFILE: with the phase stamps (measurement builds of the head-dim-128, no-GQA kernels only).
+template <int D, int G, bool ONE, bool PROFILE = false>
 __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const OharaModel& m = a.m;
@@ -96,7 +97,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   const int L = min(pos + 1, m.t_max);
   float best_v = -INFINITY;
   int best_i = 0x7fffffff;
-  Prof pf{(blockIdx.x == 0 && threadIdx.x == 0) ? a.prof : nullptr, 0};
+  ProfT<PROFILE> pf((blockIdx.x == 0 && threadIdx.x == 0) ? a.prof : nullptr);
 
   GemmP qkv{}, prj{}, gu{}, dn{}, lm{};
   qkv.H = H; qkv.Hkv = Hkv; qkv.Dh = D; qkv.Tmax = m.t_max; qkv.pos = pos; qkv.cos = m.cos; qkv.sin = m.sin;
@@ -152,12 +153,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     pf.stamp();
     // P3: merge + output projection + residual
     if ((int)blockIdx.x < prj.nstrips) {
-      if (a.ns == OHARA_MEGA_NS && B * H * D <= 4 * (int)blockDim.x) stage_attn_merge_small(xs, ldxs, p_l, B, H, D);
-      else if (a.ns == 16) stage_attn_merge<16>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
-      else if (a.ns == 8) stage_attn_merge<8>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
-      else if (a.ns == 4) stage_attn_merge<4>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
-      else if (a.ns == 2) stage_attn_merge<2>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
-      else stage_attn_merge<1>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
+      stage_attn_merge_any<!ONE>(a.ns, xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
     }
     __syncthreads();
     pf.stamp();
@@ -417,7 +413,17 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
     if (s->batch == 1) OHARA_MEGA_B(DD, GG, true);                                                          \
     else OHARA_MEGA_B(DD, GG, false);                                                                       \
   } while (0)
-  if (D == 128 && G == 1) OHARA_MEGA(128, 1);
+#define OHARA_MEGA_PROF(ONE_)                                                                               \
+  do {                                                                                                      \
+    if (smem > 64 * 1024)                                                                                   \
+      (void)hipFuncSetAttribute((const void*)decode_mega_kernel<128, 1, ONE_, true>,                        \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);                     \
+    hipLaunchKernelGGL((decode_mega_kernel<128, 1, ONE_, true>), grid, block, smem, st, a);                 \
+  } while (0)
+  if (a.prof && D == 128 && G == 1) {  // the stamps exist in these two instantiations only
+    if (s->batch == 1) OHARA_MEGA_PROF(true);
+    else OHARA_MEGA_PROF(false);
+  } else if (D == 128 && G == 1) OHARA_MEGA(128, 1);
   else if (D == 128 && G == 2) OHARA_MEGA(128, 2);
   else if (D == 128 && G == 4) OHARA_MEGA(128, 4);
   else if (D == 64 && G == 1) OHARA_MEGA(64, 1);
@@ -425,6 +431,7 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   else OHARA_MEGA(64, 4);
 #undef OHARA_MEGA
 #undef OHARA_MEGA_B
+#undef OHARA_MEGA_PROF
   return ohara_launch_status();
 }
 

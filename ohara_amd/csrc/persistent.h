@@ -12,14 +12,25 @@ namespace {
 #define OHARA_MAX_PF 24   // weight tiles (16 B per lane) a wave fetches ahead of a phase
 #define OHARA_DOWN_SPLIT 4  // K partitions of the down projection (static_assert below: x_load sums four)
 
-// Optional fine-grained timeline: thread 0 of workgroup 0 records the shader clock.
-struct Prof {
+// Optional fine-grained timeline: thread 0 of workgroup 0 records the shader clock.  The stamps are
+// compiled in only for kernels instantiated with ON (dozens of clock reads and guarded stores per
+// layer are several KB of code the ordinary kernel does not have to fetch).
+template <bool ON>
+struct ProfT;
+template <>
+struct ProfT<true> {
   unsigned long long* p;
   int n;
+  __device__ __forceinline__ explicit ProfT(unsigned long long* q) : p(q), n(0) {}
   __device__ __forceinline__ void stamp() {
     if (p) p[n] = __builtin_readcyclecounter();
     ++n;
   }
+};
+template <>
+struct ProfT<false> {
+  __device__ __forceinline__ explicit ProfT(unsigned long long*) {}
+  __device__ __forceinline__ void stamp() {}
 };
 
 // ---------------------------------------------------------------------------------------
@@ -57,7 +68,8 @@ struct GridSync {
     limit = lim;
     k = *done + 1;  // written by the previous launch (or the host): plain load
   }
-  __device__ __forceinline__ void arrive(Prof& pf) {
+  template <class PROF>
+  __device__ __forceinline__ void arrive(PROF& pf) {
     pf.stamp();  // phase work issued
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // orders my LDS and global accesses within the workgroup
     wait_own_stores();  // every wave: its sc1 stores have reached memory before the barrier below
@@ -76,7 +88,8 @@ struct GridSync {
     asm volatile("" ::: "memory");  // compiler only: keep the caller's prefetch loads after this point
     pf.stamp();  // arrival issued
   }
-  __device__ __forceinline__ void wait(Prof& pf) {
+  template <class PROF>
+  __device__ __forceinline__ void wait(PROF& pf) {
     pf.stamp();  // prefetch issued
     if (threadIdx.x == 0) {
       unsigned int spins = 0;
@@ -262,7 +275,7 @@ __device__ __forceinline__ void stage_act(bf16_t* xs, int ldxs, const char* src,
 // any, so the number of dependent load rounds does not grow with the chunk count times the batch.
 // `mw`: B*H*NS floats, `ml`: B*H floats of LDS.
 template <int NS>
-__device__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh, float* mw_, float* ml_) {
+__device__ __forceinline__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh, float* mw_, float* ml_) {
   constexpr int NSM = OHARA_MEGA_NS, PR = 16 / NS;
   const int HD = H * Dh, PS = Dh + 32;
   const int nbh = B * H, total = B * HD;
@@ -363,6 +376,37 @@ __device__ __forceinline__ void stage_attn_merge_small(bf16_t* xs, int ldxs, con
     o[3] += __uint_as_float(av[s].w) * w;
   }
   sts8(xs + (size_t)b * ldxs + hd, make_uint2(pack_bf(o[0] / Ls, o[1] / Ls), pack_bf(o[2] / Ls, o[3] / Ls)));
+}
+
+// Out-of-line copies of the merge, for kernels that want to keep their own code compact.
+template <int NS>
+__device__ __noinline__ void stage_attn_merge_call(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh, float* mw,
+                                                   float* ml) {
+  stage_attn_merge<NS>(xs, ldxs, pm, B, H, Dh, mw, ml);
+}
+
+// The merge for `ns` chunks.  INLINE: the five specialisations become part of the caller (no call in
+// the layer loop: a call makes the caller wait for every load it has in flight, the weights fetched
+// ahead included); otherwise they stay outside it, which keeps a kernel whose usual case is the
+// small merge within the instruction cache.
+template <bool INLINE>
+__device__ __forceinline__ void stage_attn_merge_any(int ns, bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh,
+                                                     float* mw, float* ml) {
+  if (ns == OHARA_MEGA_NS && B * H * Dh <= 4 * 256) {
+    stage_attn_merge_small(xs, ldxs, pm, B, H, Dh);
+  } else if (INLINE) {
+    if (ns == 16) stage_attn_merge<16>(xs, ldxs, pm, B, H, Dh, mw, ml);
+    else if (ns == 8) stage_attn_merge<8>(xs, ldxs, pm, B, H, Dh, mw, ml);
+    else if (ns == 4) stage_attn_merge<4>(xs, ldxs, pm, B, H, Dh, mw, ml);
+    else if (ns == 2) stage_attn_merge<2>(xs, ldxs, pm, B, H, Dh, mw, ml);
+    else stage_attn_merge<1>(xs, ldxs, pm, B, H, Dh, mw, ml);
+  } else {
+    if (ns == 16) stage_attn_merge_call<16>(xs, ldxs, pm, B, H, Dh, mw, ml);
+    else if (ns == 8) stage_attn_merge_call<8>(xs, ldxs, pm, B, H, Dh, mw, ml);
+    else if (ns == 4) stage_attn_merge_call<4>(xs, ldxs, pm, B, H, Dh, mw, ml);
+    else if (ns == 2) stage_attn_merge_call<2>(xs, ldxs, pm, B, H, Dh, mw, ml);
+    else stage_attn_merge_call<1>(xs, ldxs, pm, B, H, Dh, mw, ml);
+  }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -472,9 +516,9 @@ __device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int 
   }
 }
 
-template <int KP, int PF, int EPI>
+template <int KP, int PF, int EPI, class PROF>
 __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, const bf16_t* xs, int ldxs, int B,
-                                           float* red, float& best_v, int& best_i, Prof& pf) {
+                                           float* red, float& best_v, int& best_i, PROF& pf) {
   constexpr int SPW = 4 / KP;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 15, g = lane >> 4;
