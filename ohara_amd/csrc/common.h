@@ -66,15 +66,75 @@ __device__ __forceinline__ uint32_t pack_bf(float lo, float hi) {
   return (uint32_t)f2bf(lo) | ((uint32_t)f2bf(hi) << 16);
 }
 
+// Butterfly exchanges across the wave without the LDS crossbar.  __shfl_xor compiles to
+// ds_bpermute_b32 (an LDS-pipeline round trip of ~100 cycles per step of a reduction); for a
+// compile-time lane mask the same exchange is a DPP move (masks 1, 2, 4, 8: inside a row of 16
+// lanes) or one of gfx950's row swaps (v_permlane16_swap / v_permlane32_swap: masks 16, 32), a few
+// cycles each.  All lanes of the wave must be active.  lane_xor<M>(v) returns v of lane ^ M for
+// M < 16; for 16 and 32 only the combined forms below exist (the swap hands every lane its own and
+// its partner's value in an order that depends on the row, which a commutative op does not care
+// about, so the results equal those of the shuffle butterfly bit for bit).
+template <int M>
+__device__ __forceinline__ uint32_t lane_xor_u32(uint32_t u) {
+  static_assert(M == 1 || M == 2 || M == 4 || M == 8, "DPP masks");
+  if (M == 1) return (uint32_t)__builtin_amdgcn_mov_dpp((int)u, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
+  if (M == 2) return (uint32_t)__builtin_amdgcn_mov_dpp((int)u, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+  if (M == 8) return (uint32_t)__builtin_amdgcn_mov_dpp((int)u, 0x128, 0xF, 0xF, true);  // row_ror:8
+  // mask 4: lanes 0-3 and 8-11 of a row read four lanes up, the others four lanes down
+  uint32_t r = (uint32_t)__builtin_amdgcn_update_dpp((int)u, (int)u, 0x104, 0xF, 0x5, false);  // row_shl:4
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)r, (int)u, 0x114, 0xF, 0xA, false);        // row_shr:4
+}
+template <int M>
+__device__ __forceinline__ float lane_xor(float v) {
+  return __uint_as_float(lane_xor_u32<M>(__float_as_uint(v)));
+}
+template <int M>
+__device__ __forceinline__ void lane_swap(float v, float& a, float& b) {  // {a, b} = {own, partner} in some order
+  static_assert(M == 16 || M == 32, "row swaps");
+  const uint32_t u = __float_as_uint(v);
+  const u32x2 r = M == 16 ? __builtin_amdgcn_permlane16_swap(u, u, false, false)
+                          : __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  a = __uint_as_float(r[0]);
+  b = __uint_as_float(r[1]);
+}
+template <int M>
+__device__ __forceinline__ float lane_xor_sum(float v) {  // v + v of lane ^ M
+  if constexpr (M >= 16) {
+    float a, b;
+    lane_swap<M>(v, a, b);
+    return a + b;
+  } else {
+    return v + lane_xor<M>(v);
+  }
+}
+template <int M>
+__device__ __forceinline__ float lane_xor_max(float v) {  // fmaxf(v, v of lane ^ M)
+  if constexpr (M >= 16) {
+    float a, b;
+    lane_swap<M>(v, a, b);
+    return fmaxf(a, b);
+  } else {
+    return fmaxf(v, lane_xor<M>(v));
+  }
+}
+
+// Sum / maximum over the wave, every lane gets the result; the order of the adds is that of the
+// butterfly 32, 16, 8, 4, 2, 1.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
-  return v;
+  v = lane_xor_sum<32>(v);
+  v = lane_xor_sum<16>(v);
+  v = lane_xor_sum<8>(v);
+  v = lane_xor_sum<4>(v);
+  v = lane_xor_sum<2>(v);
+  return lane_xor_sum<1>(v);
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
-  return v;
+  v = lane_xor_max<32>(v);
+  v = lane_xor_max<16>(v);
+  v = lane_xor_max<8>(v);
+  v = lane_xor_max<4>(v);
+  v = lane_xor_max<2>(v);
+  return lane_xor_max<1>(v);
 }
 
 // Device-coherent accesses without fences.  The eight XCDs' L2 caches are not coherent with

@@ -132,8 +132,8 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     // P1: [embedding] + norm1 + QKV + rotary + append
     qkv.kc = kc; qkv.vc = vc; qkv.out = q_l;
     if ((int)blockIdx.x < qkv.nstrips) {
-      if (l == 0) stage_norm<2, true, true>(xs, ldxs, a.xm, 0, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d, pre.g);
-      else stage_norm<2, false, true>(xs, ldxs, x_prev, a.blk_x, d_prev, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d, pre.g);
+      if (l == 0) stage_norm<2, true, true, false>(xs, ldxs, a.xm, 0, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d, pre.g);
+      else stage_norm<2, false, true, true>(xs, ldxs, x_prev, a.blk_x, d_prev, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d, pre.g);
     }
     __syncthreads();
     pf.stamp();
@@ -165,7 +165,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     gs.wait(pf);
     pf.stamp();
     // P4: norm2 + gate/up + SwiGLU
-    if ((int)blockIdx.x * 2 < gu.nstrips) stage_norm<2, false, true>(xs, ldxs, x_mid, a.blk_x, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 5), m.eps, B, d, pre.g);
+    if ((int)blockIdx.x * 2 < gu.nstrips) stage_norm<2, false, true, false>(xs, ldxs, x_mid, a.blk_x, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 5), m.eps, B, d, pre.g);
     __syncthreads();
     gemm_phase<2, 12, E_SWIGLU>(gu, pre, xs, ldxs, B, red, best_v, best_i, pf);
     gs.arrive(pf);
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     pf.stamp();
   }
   // final norm + vocabulary projection, running arg-max per lane
-  stage_norm<2, false, true>(xs, ldxs, a.xm + (size_t)(m.n_layers - 1) * a.xm_stride, a.blk_x,
+  stage_norm<2, false, true, true>(xs, ldxs, a.xm + (size_t)(m.n_layers - 1) * a.xm_stride, a.blk_x,
                              a.dm + (size_t)(m.n_layers - 1) * a.dm_stride, a.ids, m.token_emb, V, m.final_norm, m.eps, B, d,
                              pre.g);
   __syncthreads();

@@ -155,33 +155,46 @@ __device__ __forceinline__ const float* parts_addr(const float* base, int nstrip
                                         (size_t)(q * nstrips + (n >> 4)) * pm_blk(B) + b * 64) + (n & 15);
 }
 
-template <int NW>  // NW columns (4 or 8) starting at n, n % NW == 0
-__device__ __forceinline__ void x_load(const XParts& xp, int b, int n, uint32_t (&out)[NW / 2]) {
-  uint32_t xm[NW / 2];
+// PARTS says at compile time whether xp.parts is set: a branch on the pointer would keep the
+// compiler from issuing the loads of several calls together.  The loads (x_fetch) and the sums
+// (x_combine) are separate so that a caller can issue the loads of several pieces back to back.
+template <int NW, bool PARTS>  // NW columns (4 or 8) starting at n, n % NW == 0
+struct XRaw {
+  uint4 xm;  // NW == 4: .x, .y only
+  uint4 pv[PARTS ? OHARA_DOWN_SPLIT : 1][NW / 4];
+};
+template <int NW, bool PARTS>
+__device__ __forceinline__ void x_fetch(const XParts& xp, int b, int n, XRaw<NW, PARTS>& r) {
   if (NW == 8) {
-    const uint4 v = ldg16(xm_addr(xp.xmid, xp.blk, b, n));
-    xm[0] = v.x; xm[1] = v.y; xm[NW / 2 - 2] = v.z; xm[NW / 2 - 1] = v.w;
+    r.xm = ldg16(xm_addr(xp.xmid, xp.blk, b, n));
   } else {
     const uint2 v = ldg8(xm_addr(xp.xmid, xp.blk, b, n));
-    xm[0] = v.x; xm[1] = v.y;
+    r.xm = make_uint4(v.x, v.y, 0, 0);
   }
-  if (!xp.parts) {
+  if (PARTS) {
+#pragma unroll
+    for (int q = 0; q < OHARA_DOWN_SPLIT; ++q)
+#pragma unroll
+      for (int i = 0; i < NW / 4; ++i) r.pv[q][i] = ldg16(parts_addr(xp.parts, (xp.N + 15) >> 4, xp.B, q, b, n + 4 * i));
+  }
+}
+template <int NW, bool PARTS>
+__device__ __forceinline__ void x_combine(const XRaw<NW, PARTS>& r, uint32_t (&out)[NW / 2]) {
+  uint32_t xm[NW / 2];
+  xm[0] = r.xm.x; xm[1] = r.xm.y;
+  if (NW == 8) { xm[NW / 2 - 2] = r.xm.z; xm[NW / 2 - 1] = r.xm.w; }
+  if (!PARTS) {
 #pragma unroll
     for (int i = 0; i < NW / 2; ++i) out[i] = xm[i];
     return;
   }
-  uint4 pv[OHARA_DOWN_SPLIT][NW / 4];
-#pragma unroll
-  for (int q = 0; q < OHARA_DOWN_SPLIT; ++q)
-#pragma unroll
-    for (int i = 0; i < NW / 4; ++i) pv[q][i] = ldg16(parts_addr(xp.parts, (xp.N + 15) >> 4, xp.B, q, b, n + 4 * i));
+  static_assert(OHARA_DOWN_SPLIT == 4, "x_combine sums four partitions");
 #pragma unroll
   for (int i = 0; i < NW / 4; ++i) {
     float y[4];
-    const uint32_t w[OHARA_DOWN_SPLIT][4] = {{pv[0][i].x, pv[0][i].y, pv[0][i].z, pv[0][i].w},
-                                             {pv[1][i].x, pv[1][i].y, pv[1][i].z, pv[1][i].w},
-                                             {pv[2][i].x, pv[2][i].y, pv[2][i].z, pv[2][i].w},
-                                             {pv[3][i].x, pv[3][i].y, pv[3][i].z, pv[3][i].w}};
+    const uint4 p0 = r.pv[0][i], p1 = r.pv[PARTS ? 1 : 0][i], p2 = r.pv[PARTS ? 2 : 0][i], p3 = r.pv[PARTS ? 3 : 0][i];
+    const uint32_t w[OHARA_DOWN_SPLIT][4] = {{p0.x, p0.y, p0.z, p0.w}, {p1.x, p1.y, p1.z, p1.w},
+                                             {p2.x, p2.y, p2.z, p2.w}, {p3.x, p3.y, p3.z, p3.w}};
 #pragma unroll
     for (int e = 0; e < 4; ++e)
       y[e] = rbf(((__uint_as_float(w[0][e]) + __uint_as_float(w[1][e])) + __uint_as_float(w[2][e])) +
@@ -189,6 +202,12 @@ __device__ __forceinline__ void x_load(const XParts& xp, int b, int n, uint32_t 
     out[2 * i] = pack_bf(lo_bf(xm[2 * i]) + y[0], hi_bf(xm[2 * i]) + y[1]);
     out[2 * i + 1] = pack_bf(lo_bf(xm[2 * i + 1]) + y[2], hi_bf(xm[2 * i + 1]) + y[3]);
   }
+}
+template <int NW, bool PARTS>
+__device__ __forceinline__ void x_load(const XParts& xp, int b, int n, uint32_t (&out)[NW / 2]) {
+  XRaw<NW, PARTS> r;
+  x_fetch<NW, PARTS>(xp, b, n, r);
+  x_combine<NW, PARTS>(r, out);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -199,7 +218,8 @@ __device__ __forceinline__ void x_load(const XParts& xp, int b, int n, uint32_t 
 // - on rows gathered from the embedding table (llama.py:310).  One wave per row; all loads
 // of a row are issued before any is consumed.  K <= 8 * 64 * NLD elements.
 // PRE: the lane's norm-weight pieces were fetched ahead (gemm_prefetch) and are in gpre[0 .. NLD).
-template <int NLD, bool EMBED, bool PRE = false>
+// PARTS: `parts` is set (the rows are x-mailbox rows plus down-projection sums).
+template <int NLD, bool EMBED, bool PRE, bool PARTS>
 __device__ __forceinline__ void stage_norm(bf16_t* xs, int ldxs, const char* src, int blk, const float* parts,
                                            const int64_t* ids, const bf16_t* table, int vocab, const bf16_t* nw, float eps,
                                            int B, int K, const uint4 (&gpre)[NLD]) {
@@ -213,20 +233,29 @@ __device__ __forceinline__ void stage_norm(bf16_t* xs, int ldxs, const char* src
       if (id < 0 || id >= vocab) id = 0;
       row_off = (size_t)id * K;
     }
+    // Every piece is loaded without a branch (pieces beyond K read column 0 and are zeroed below):
+    // behind a branch per piece the compiler waits for one piece's loads before it issues the
+    // next piece's, one cold round trip after the other.
+    XRaw<8, PARTS> raw[NLD];
 #pragma unroll
     for (int c = 0; c < NLD; ++c) {
       const int k = (c * 64 + lane) * 8;
-      v[c] = make_uint4(0, 0, 0, 0);
-      g[c] = make_uint4(0, 0, 0, 0);
-      if (k < K) {
-        if (EMBED) {
-          v[c] = ldg16(table + row_off + k);
-        } else {
-          uint32_t w[4];
-          x_load<8>(xp, b, k, w);
-          v[c] = make_uint4(w[0], w[1], w[2], w[3]);
-        }
-        g[c] = PRE ? gpre[c] : ldg16(nw + k);
+      const int kc = k < K ? k : 0;
+      if (EMBED) v[c] = ldg16(table + row_off + kc);
+      else x_fetch<8, PARTS>(xp, b, kc, raw[c]);
+      g[c] = PRE ? gpre[c] : ldg16(nw + kc);
+    }
+    __builtin_amdgcn_sched_barrier(0);  // all loads above, all sums below
+#pragma unroll
+    for (int c = 0; c < NLD; ++c) {
+      if (!EMBED) {
+        uint32_t w[4];
+        x_combine<8, PARTS>(raw[c], w);
+        v[c] = make_uint4(w[0], w[1], w[2], w[3]);
+      }
+      if ((c * 64 + lane) * 8 >= K) {
+        v[c] = make_uint4(0, 0, 0, 0);
+        g[c] = make_uint4(0, 0, 0, 0);
       }
     }
     float ss = 0.f;
@@ -309,12 +338,16 @@ __device__ __forceinline__ void stage_attn_merge(bf16_t* xs, int ldxs, const flo
       ls = __uint_as_float(v.y);
     }
     float M = ms;
-#pragma unroll
-    for (int o = NS / 2; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, WAVE));
+    if (NS > 8) M = lane_xor_max<8>(M);
+    if (NS > 4) M = lane_xor_max<4>(M);
+    if (NS > 2) M = lane_xor_max<2>(M);
+    if (NS > 1) M = lane_xor_max<1>(M);
     const float w = (ms == -INFINITY) ? 0.f : __expf(ms - M);
     float Ls = ls * w;
-#pragma unroll
-    for (int o = NS / 2; o > 0; o >>= 1) Ls += __shfl_xor(Ls, o, WAVE);
+    if (NS > 8) Ls = lane_xor_sum<8>(Ls);
+    if (NS > 4) Ls = lane_xor_sum<4>(Ls);
+    if (NS > 2) Ls = lane_xor_sum<2>(Ls);
+    if (NS > 1) Ls = lane_xor_sum<1>(Ls);
     if (in) mw[bh * NS + sp] = w;
     if (in && sp == 0) ml[bh] = Ls;
   }
@@ -505,7 +538,7 @@ __device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int 
     if (live && kpart == 0 && m < B && r0 < p.N) {
       if (!p.resid_embed) {
         uint32_t w[2];
-        x_load<4>(XParts{p.resid, p.resid_parts, p.blk, B, p.N}, m, r0, w);
+        x_load<4, true>(XParts{p.resid, p.resid_parts, p.blk, B, p.N}, m, r0, w);
         pre.r = make_uint2(w[0], w[1]);
       } else {
         int64_t id = ldg_i64(p.ids + m);
@@ -596,7 +629,7 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
           if (it > 0) {
             if (!p.resid_embed) {
               uint32_t w[2];
-              x_load<4>(XParts{p.resid, p.resid_parts, p.blk, B, p.N}, b, r0, w);
+              x_load<4, true>(XParts{p.resid, p.resid_parts, p.blk, B, p.N}, b, r0, w);
               r = make_uint2(w[0], w[1]);
             } else {
               int64_t id = ldg_i64(p.ids + b);
@@ -794,9 +827,9 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
           sc[hh] = s;
         }
 #pragma unroll
-        for (int hh = 0; hh < G; ++hh) sc[hh] += __shfl_xor(sc[hh], 16, WAVE);
+        for (int hh = 0; hh < G; ++hh) sc[hh] = lane_xor_sum<16>(sc[hh]);
 #pragma unroll
-        for (int hh = 0; hh < G; ++hh) sc[hh] += __shfl_xor(sc[hh], 32, WAVE);
+        for (int hh = 0; hh < G; ++hh) sc[hh] = lane_xor_sum<32>(sc[hh]);
         bool raise = false;
 #pragma unroll
         for (int hh = 0; hh < G; ++hh) {
@@ -808,9 +841,13 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
 #pragma unroll
           for (int hh = 0; hh < G; ++hh) tm[hh] = sc[hh];
 #pragma unroll
-          for (int o = 8; o > 0; o >>= 1)
+          for (int hh = 0; hh < G; ++hh) tm[hh] = lane_xor_max<8>(tm[hh]);
 #pragma unroll
-            for (int hh = 0; hh < G; ++hh) tm[hh] = fmaxf(tm[hh], __shfl_xor(tm[hh], o, WAVE));
+          for (int hh = 0; hh < G; ++hh) tm[hh] = lane_xor_max<4>(tm[hh]);
+#pragma unroll
+          for (int hh = 0; hh < G; ++hh) tm[hh] = lane_xor_max<2>(tm[hh]);
+#pragma unroll
+          for (int hh = 0; hh < G; ++hh) tm[hh] = lane_xor_max<1>(tm[hh]);
 #pragma unroll
           for (int hh = 0; hh < G; ++hh) {
             const float mn = fmaxf(m_run[hh], tm[hh]);
@@ -850,17 +887,16 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
     }
     first = false;
 #pragma unroll
-    for (int o = 8; o > 0; o >>= 1)
-#pragma unroll
-      for (int hh = 0; hh < G; ++hh) l_run[hh] += __shfl_xor(l_run[hh], o, WAVE);
+    for (int hh = 0; hh < G; ++hh)
+      l_run[hh] = lane_xor_sum<1>(lane_xor_sum<2>(lane_xor_sum<4>(lane_xor_sum<8>(l_run[hh]))));
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         float v = acc[hh][i];
-#pragma unroll
-        for (int o = DC; o < 64; o <<= 1) v += __shfl_xor(v, o, WAVE);
-        acc[hh][i] = v;
+        if (DC == 8) v = lane_xor_sum<8>(v);
+        v = lane_xor_sum<16>(v);
+        acc[hh][i] = lane_xor_sum<32>(v);
       }
       if (lane < DC) {
 #pragma unroll
