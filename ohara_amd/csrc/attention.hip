@@ -142,6 +142,7 @@ template <int D, int G>
 __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   constexpr int NC = D / 32;        // 16-byte K loads per lane per tile
   constexpr int DC = D / 8;         // lanes covering one V row with 16-byte loads
+  static_assert(DC == 8 || DC == 16, "head_dim 64 or 128");
   constexpr int PP = 64 / DC;       // V rows fetched per load instruction
   constexpr int NV = 16 / PP;       // V load instructions per 16-position tile
   const int split = blockIdx.z, kvh = blockIdx.y, b = blockIdx.x;  // b: query row = seq * S + s
@@ -237,9 +238,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
 #pragma unroll
       for (int hh = 0; hh < G; ++hh) tm[hh] = sc[hh];
 #pragma unroll
-      for (int o = 32; o > 2; o >>= 1)
-#pragma unroll
-        for (int hh = 0; hh < G; ++hh) tm[hh] = fmaxf(tm[hh], __shfl_xor(tm[hh], o, WAVE));
+      for (int hh = 0; hh < G; ++hh) tm[hh] = lanes_max<32, 4>(tm[hh]);
 #pragma unroll
       for (int hh = 0; hh < G; ++hh) {
         const float mn = fmaxf(m_run[hh], tm[hh]);  // finite: the tile holds at least one position
@@ -275,17 +274,15 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   // fold the sums over the 16 positions of a tile (every lane of a quarter holds the same share),
   // the PP row-groups of the wave, then the four waves
 #pragma unroll
-  for (int o = 32; o > 2; o >>= 1)
-#pragma unroll
-    for (int hh = 0; hh < G; ++hh) l_run[hh] += __shfl_xor(l_run[hh], o, WAVE);
+  for (int hh = 0; hh < G; ++hh) l_run[hh] = lanes_sum<32, 4>(l_run[hh]);
 #pragma unroll
   for (int hh = 0; hh < G; ++hh) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       float v = acc[hh][i];
-#pragma unroll
-      for (int o = DC; o < 64; o <<= 1) v += __shfl_xor(v, o, WAVE);
-      acc[hh][i] = v;
+      if (DC == 8) v = lane_xor_sum<8>(v);
+      v = lane_xor_sum<16>(v);
+      acc[hh][i] = lane_xor_sum<32>(v);
     }
     if (lane < DC) {
 #pragma unroll
@@ -338,6 +335,7 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
   constexpr int NC = D / 32;        // bf16 uint4 of a K quarter-row after expansion
   constexpr int NCB = (NC + 1) / 2; // uint4 of codes per K quarter-row (NC = 2: one 16-byte load)
   constexpr int DC = D / 8;         // lanes covering one V row with 8-byte loads
+  static_assert(DC == 8 || DC == 16, "head_dim 64 or 128");
   constexpr int PP = 64 / DC;       // V rows fetched per load instruction
   constexpr int NV = 32 / PP;       // V load instructions per 32-position tile
   static_assert(NC >= 2, "head width 64 or 128");
@@ -440,9 +438,7 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
 #pragma unroll
         for (int hh = 0; hh < G; ++hh) tm[hh] = sc[hh];
 #pragma unroll
-        for (int o = 32; o > 2; o >>= 1)
-#pragma unroll
-          for (int hh = 0; hh < G; ++hh) tm[hh] = fmaxf(tm[hh], __shfl_xor(tm[hh], o, WAVE));
+        for (int hh = 0; hh < G; ++hh) tm[hh] = lanes_max<32, 4>(tm[hh]);
 #pragma unroll
         for (int hh = 0; hh < G; ++hh) {
           const float mn = fmaxf(m_run[hh], tm[hh]);  // finite here: some position of the sub-tile raised it
@@ -483,17 +479,15 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
 
   // fold the sums over the 16 positions of a sub-tile, the PP row-groups of the wave, then the four waves
 #pragma unroll
-  for (int o = 32; o > 2; o >>= 1)
-#pragma unroll
-    for (int hh = 0; hh < G; ++hh) l_run[hh] += __shfl_xor(l_run[hh], o, WAVE);
+  for (int hh = 0; hh < G; ++hh) l_run[hh] = lanes_sum<32, 4>(l_run[hh]);
 #pragma unroll
   for (int hh = 0; hh < G; ++hh) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       float v = acc[hh][i];
-#pragma unroll
-      for (int o = DC; o < 64; o <<= 1) v += __shfl_xor(v, o, WAVE);
-      acc[hh][i] = v;
+      if (DC == 8) v = lane_xor_sum<8>(v);
+      v = lane_xor_sum<16>(v);
+      acc[hh][i] = lane_xor_sum<32>(v);
     }
     if (lane < DC) {
 #pragma unroll

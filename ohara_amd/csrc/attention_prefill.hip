@@ -178,8 +178,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(PrefillArgs a) {
         tmax *= a.scale_log2e;  // the scale is positive: the maximum of the products is the product of the maximum
         mul = a.scale_log2e;    // and the scaling itself rides in the fused multiply-add of the exponent below
       }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+      tmax = lane_xor_max<32>(lane_xor_max<16>(tmax));
       const float mn = fmaxf(m_run[qb], tmax);  // finite: position 0 is visible to every query
       const float corr = __builtin_amdgcn_exp2f(m_run[qb] - mn);  // arguments <= 0: the bare instruction is exact enough and 2^-inf = 0
       m_run[qb] = mn;
@@ -224,8 +223,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(PrefillArgs a) {
   for (int qb = 0; qb < 2; ++qb) {
     const int qi = wq0 + qb * 16 + m;
     float l = l_run[qb];
-    l += __shfl_xor(l, 16, WAVE);
-    l += __shfl_xor(l, 32, WAVE);
+    l = lane_xor_sum<32>(lane_xor_sum<16>(l));
     if (qi >= a.S) continue;
     const float inv = 1.0f / l;
     bf16_t* dst = a.out + ((size_t)b * a.S + qi) * a.H * D + (size_t)h * D + 4 * g;

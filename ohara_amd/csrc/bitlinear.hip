@@ -104,8 +104,7 @@ __device__ __forceinline__ QuantOut wave_quant_row(const bf16_t* x, const bf16_t
     }
     *reinterpret_cast<uint2*>(xq + (size_t)p * 8) = make_uint2(pk[0], pk[1]);
   }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, WAVE);
+  sq = lanes_sum<32, 1>(sq);
   return QuantOut{s, sq};
 }
 
@@ -182,8 +181,7 @@ __device__ __forceinline__ QuantOut block_quant_row(const bf16_t* x, const bf16_
     }
     *reinterpret_cast<uint2*>(xq + (size_t)p * 8) = make_uint2(pk[0], pk[1]);
   }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, WAVE);
+  sq = lanes_sum<32, 1>(sq);
   int* redi = reinterpret_cast<int*>(red);
   __syncthreads();
   if (lane == 0) redi[wave] = sq;

@@ -248,8 +248,7 @@ __device__ __forceinline__ void row1_codes(const uint4 (&h)[NP], const uint4 (&n
     const int p = tid + 256 * i;
     if (p < pieces) sts8(xq + (size_t)p * 8, make_uint2(pk[0], pk[1]));
   }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, WAVE);
+  sq = lanes_sum<32, 1>(sq);
   if (lane == 0) sumw[wave] = sq;
   if (tid == 0) *s_out = s;
 }
@@ -349,8 +348,7 @@ __device__ __forceinline__ RowQ roww_codes(const uint4 (&h)[NP], const uint4 (&n
     const int p = lane + 64 * i;
     if (p < pieces) sts8(xq + (size_t)p * 8, make_uint2(pk[0], pk[1]));
   }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, WAVE);
+  sq = lanes_sum<32, 1>(sq);
   return RowQ{s, sq};
 }
 // B rows from `load(b, piece) -> uint4` into one or two code sets.  Every thread of the workgroup calls.
@@ -462,8 +460,7 @@ __device__ __forceinline__ void bit_stage_roww_lds(const BitLds& L, int B, int K
         sts8(xq + (size_t)p * 8, make_uint2(pk[0], pk[1]));
       }
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, WAVE);
+    sq = lanes_sum<32, 1>(sq);
     if (lane == 0) {
       L.s_s[b] = s;
       L.s_sum[b] = sq;

@@ -118,6 +118,56 @@ __device__ __forceinline__ float lane_xor_max(float v) {  // fmaxf(v, v of lane 
   }
 }
 
+template <int M>
+__device__ __forceinline__ float lane_xor_min(float v) {  // fminf(v, v of lane ^ M)
+  if constexpr (M >= 16) {
+    float a, b;
+    lane_swap<M>(v, a, b);
+    return fminf(a, b);
+  } else {
+    return fminf(v, lane_xor<M>(v));
+  }
+}
+template <int M>
+__device__ __forceinline__ int lane_xor_sum(int v) {  // v + v of lane ^ M
+  if constexpr (M >= 16) {
+    const u32x2 r = M == 16 ? __builtin_amdgcn_permlane16_swap((uint32_t)v, (uint32_t)v, false, false)
+                            : __builtin_amdgcn_permlane32_swap((uint32_t)v, (uint32_t)v, false, false);
+    return (int)(r[0] + r[1]);
+  } else {
+    return v + (int)lane_xor_u32<M>((uint32_t)v);
+  }
+}
+template <int M>
+__device__ __forceinline__ int lane_xor_max(int v) {  // max(v, v of lane ^ M)
+  if constexpr (M >= 16) {
+    const u32x2 r = M == 16 ? __builtin_amdgcn_permlane16_swap((uint32_t)v, (uint32_t)v, false, false)
+                            : __builtin_amdgcn_permlane32_swap((uint32_t)v, (uint32_t)v, false, false);
+    return max((int)r[0], (int)r[1]);
+  } else {
+    return max(v, (int)lane_xor_u32<M>((uint32_t)v));
+  }
+}
+// Butterfly steps for masks HI, HI / 2, ..., LO (powers of two), in that order.
+template <int HI, int LO, typename T>
+__device__ __forceinline__ T lanes_sum(T v) {
+  v = lane_xor_sum<HI>(v);
+  if constexpr (HI > LO) return lanes_sum<HI / 2, LO, T>(v);
+  else return v;
+}
+template <int HI, int LO, typename T>
+__device__ __forceinline__ T lanes_max(T v) {
+  v = lane_xor_max<HI>(v);
+  if constexpr (HI > LO) return lanes_max<HI / 2, LO, T>(v);
+  else return v;
+}
+template <int HI, int LO>
+__device__ __forceinline__ float lanes_min(float v) {
+  v = lane_xor_min<HI>(v);
+  if constexpr (HI > LO) return lanes_min<HI / 2, LO>(v);
+  else return v;
+}
+
 // Sum / maximum over the wave, every lane gets the result; the order of the adds is that of the
 // butterfly 32, 16, 8, 4, 2, 1.
 __device__ __forceinline__ float wave_sum(float v) {

@@ -109,13 +109,13 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(GemmArgs a) {
 #pragma unroll
     for (int t = 0; t < BT; ++t) {
       float p = part[t];
-      p += __shfl_xor(p, 16, WAVE);
-      p += __shfl_xor(p, 32, WAVE);
+      p = lanes_sum<16, 16>(p);
+      p = lanes_sum<32, 32>(p);
       if (g == 0) ssq[wave][16 * t + m] = p;
       if (NORM == 2) {
         float q = psum[t];
-        q += __shfl_xor(q, 16, WAVE);
-        q += __shfl_xor(q, 32, WAVE);
+        q = lanes_sum<16, 16>(q);
+        q = lanes_sum<32, 32>(q);
         if (g == 0) ssum[wave][16 * t + m] = q;
       }
     }

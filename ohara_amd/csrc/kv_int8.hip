@@ -41,11 +41,8 @@ __global__ __launch_bounds__(256) void kv_quant_append_kernel(const bf16_t* k, c
       mx = fmaxf(mx, x[i]);
     }
   }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    mn = fminf(mn, __shfl_xor(mn, o, WAVE));
-    mx = fmaxf(mx, __shfl_xor(mx, o, WAVE));
-  }
+  mn = lanes_min<32, 1>(mn);
+  mx = lanes_max<32, 1>(mx);
   // kv_cache.py:23-24 in the cache dtype: (max - min) -> bf16, / 255 -> bf16, clamp at bf16(1e-8)
   const float scale = fmaxf(rbf(rbf(mx - mn) / 255.0f), rbf(1e-8f));
 #pragma unroll

@@ -208,8 +208,7 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
         part += lo_bf(ku[i]) * (cs[r][2 * i] * A[2 * i] + sn[r][2 * i] * Bc[2 * i]);
         part += hi_bf(ku[i]) * (cs[r][2 * i + 1] * A[2 * i + 1] + sn[r][2 * i + 1] * Bc[2 * i + 1]);
       }
-#pragma unroll
-      for (int o = 1; o < 16; o <<= 1) part += __shfl_xor(part, o, WAVE);
+      part = lane_xor_sum<8>(lane_xor_sum<4>(lane_xor_sum<2>(lane_xor_sum<1>(part))));
       const float sc = part * scale;
       const float mn = fmaxf(m, sc);
       // hardware exponential: its error (about 1e-6 relative) is far below the bf16 rounding of the output
@@ -418,8 +417,7 @@ __global__ __launch_bounds__(256) void phi_attn_prefill_kernel(PhiAttnArgs a) {
         sc[r] = tb + 4 * g + r <= pq ? sc[r] * scale : -INFINITY;
         mx = fmaxf(mx, sc[r]);
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+      mx = lane_xor_max<32>(lane_xor_max<16>(mx));
       const float mn = fmaxf(m, mx);  // finite: position 0 is in the first block and visible to every query
       const float corr = __expf(m - mn);
       float ps = 0.f;
@@ -443,8 +441,7 @@ __global__ __launch_bounds__(256) void phi_attn_prefill_kernel(PhiAttnArgs a) {
     }
     __syncthreads();
   }
-  lsum += __shfl_xor(lsum, 16, WAVE);
-  lsum += __shfl_xor(lsum, 32, WAVE);
+  lsum = lane_xor_sum<32>(lane_xor_sum<16>(lsum));
   if (s0 + 16 * wave + l16 < a.S) {
     const float inv = 1.0f / lsum;
     bf16_t* orow = a.out + ((size_t)seq * a.S + sq) * hd + (size_t)h * D + 4 * g;

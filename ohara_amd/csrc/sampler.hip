@@ -90,8 +90,7 @@ __device__ __forceinline__ float block_sum(float v, Smem& s) {
 }
 
 __device__ __forceinline__ int block_sum_i(int v, Smem& s) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  v = lanes_sum<32, 1>(v);
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   __syncthreads();
   if (lane == 0) s.wredi[w] = v;
@@ -678,8 +677,7 @@ __device__ __forceinline__ int sample_row(const SampleArgs& a, int b, Smem& s) {
     for (int i = 0; i < EPT; ++i)
       if (x[i] > 0.f) lastpos = base + i;
     int mx = lastpos;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) mx = max(mx, __shfl_xor(mx, o, WAVE));
+    mx = lanes_max<32, 1>(mx);
     __syncthreads();
     if ((tid & 63) == 0) s.wredi[tid >> 6] = mx;
     if (tid == 0) s.misc[2] = 0x7fffffff;
@@ -938,8 +936,7 @@ constexpr int HB = 32768;      // dwords of the count table
 constexpr int ENT_CAP = 4096;  // entries of the compacted (key, count) list
 
 __device__ __forceinline__ int block_max_i(int v, Smem& s) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, WAVE));
+  v = lanes_max<32, 1>(v);
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   __syncthreads();
   if (lane == 0) s.wredi[w] = v;
