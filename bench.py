@@ -700,6 +700,8 @@ def main():
                     help="run the MoE decode figure alone and exit (profiling workload)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run the d12 prefill figures (tiled MFMA GEMMs, prefill attention) alone and exit")
+    ap.add_argument("--attention-only", action="store_true",
+                    help="run the GQA decode-attention figures (bf16 and int8 cache) alone and exit")
     ap.add_argument("--phi-decode-only", type=int, default=0, metavar="B",
                     help="run 12 eager Phi-2 decode steps of B sequences at context 1024 and exit (profiling workload)")
     args = ap.parse_args()
@@ -722,6 +724,9 @@ def main():
         return
     if args.moe_only:
         print(json.dumps(bench_moe(dev), indent=1))
+        return
+    if args.attention_only:
+        print(json.dumps(bench_attention_microbench(dev), indent=1))
         return
     if args.bitnet_only:
         print(json.dumps(bench_bitnet(dev, tuple(int(b) for b in args.bitnet_only.split(","))), indent=1))

@@ -183,15 +183,18 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
     uint4 k[NC];
     uint4 v[NV];
   };
+  // Every load of a tile is issued without a branch (positions past the chunk read its last row;
+  // their scores are masked and their weights are zero): with the loads behind per-lane conditions
+  // the compiler cannot count how many are outstanding and waits for ALL of them - the next tile's
+  // included - before it touches the current tile, which undoes the double buffering.
   auto load_tile = [&](int tb, Tile& t) {
-    const int pos = tb + p;
+    const int pos = min(tb + p, t1 - 1);
 #pragma unroll
-    for (int c = 0; c < NC; ++c)
-      t.k[c] = pos < t1 ? ldg16_nt(kb + (size_t)pos * row + (4 * c + dq) * 8) : make_uint4(0, 0, 0, 0);
+    for (int c = 0; c < NC; ++c) t.k[c] = ldg16_nt(kb + (size_t)pos * row + (4 * c + dq) * 8);
 #pragma unroll
     for (int c = 0; c < NV; ++c) {
-      const int vp = tb + c * PP + pp;
-      t.v[c] = vp < t1 ? ldg16_nt(vb + (size_t)vp * row + dc * 8) : make_uint4(0, 0, 0, 0);
+      const int vp = min(tb + c * PP + pp, t1 - 1);
+      t.v[c] = ldg16_nt(vb + (size_t)vp * row + dc * 8);
     }
   };
   auto expand = [&](const Tile& t, uint4* kv, uint4* vv) {
@@ -204,14 +207,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   // flight while the current one is consumed (a second tile in flight costs more in occupancy
   // than it gains: measured)
   Tile cur, nxt;
-  int tb = t0 + wave * 16;
-  if (tb < t1) load_tile(tb, cur);
-  for (; tb < t1; tb += 64) {
+  auto consume = [&](int tb, const Tile& tile) {
     const bool valid = tb + p < t1;
-    const bool more = tb + 64 < t1;
-    if (more) load_tile(tb + 64, nxt);
     uint4 kv[NC], vv[NV];
-    expand(cur, kv, vv);
+    expand(tile, kv, vv);
     // The heads of the group advance together, one step at a time, so that their cross-lane
     // exchanges overlap instead of forming G dependent chains.  l_run is this lane's share of the
     // sum (its own position only; folded over the 16 positions after the loop), and the running
@@ -254,21 +253,50 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
       pv[hh] = __expf(sc[hh] - m_run[hh]);
       l_run[hh] += pv[hh];
     }
+    // all weight exchanges first (they are independent), then the products: next to their products
+    // every exchange is waited for by itself
+    float pw[NV][G];
+#pragma unroll
+    for (int c = 0; c < NV; ++c)
+#pragma unroll
+      for (int hh = 0; hh < G; ++hh) pw[c][hh] = __shfl(pv[hh], 4 * (c * PP + pp), WAVE);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int c = 0; c < NV; ++c) {
       const uint32_t w4[4] = {vv[c].x, vv[c].y, vv[c].z, vv[c].w};
-      float pw[G];
-#pragma unroll
-      for (int hh = 0; hh < G; ++hh) pw[hh] = __shfl(pv[hh], 4 * (c * PP + pp), WAVE);
 #pragma unroll
       for (int hh = 0; hh < G; ++hh)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          acc[hh][2 * i] += pw[hh] * lo_bf(w4[i]);
-          acc[hh][2 * i + 1] += pw[hh] * hi_bf(w4[i]);
+          acc[hh][2 * i] += pw[c][hh] * lo_bf(w4[i]);
+          acc[hh][2 * i + 1] += pw[c][hh] * hi_bf(w4[i]);
         }
     }
-    if (more) cur = nxt;
+  };
+  int tb = t0 + wave * 16;
+  if (tb < t1) {
+    // two register tiles take turns (no copy between iterations: a copy would wait for the tile
+    // that has just been requested)
+    load_tile(tb, cur);
+    if constexpr (G >= 4) {  // four heads' accumulators leave no room for a second resident tile
+      for (; tb + 64 < t1; tb += 64) {
+        load_tile(tb + 64, nxt);
+        consume(tb, cur);
+        cur = nxt;
+      }
+      consume(tb, cur);
+    } else {
+      for (;;) {
+        if (tb + 64 >= t1) { consume(tb, cur); break; }
+        load_tile(tb + 64, nxt);
+        consume(tb, cur);
+        tb += 64;
+        if (tb + 64 >= t1) { consume(tb, nxt); break; }
+        load_tile(tb + 64, cur);
+        consume(tb, nxt);
+        tb += 64;
+      }
+    }
   }
 
   // fold the sums over the 16 positions of a tile (every lane of a quarter holds the same share),
@@ -378,30 +406,26 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
     uint2 v[NV];      // eight codes of row tb + c * PP + pp
     uint4 st[2];      // (key scale, key min, value scale, value min) of position tb + 16 s + p
   };
+  // Loads without branches, as in the bf16 kernel: positions past the chunk read its last row (their
+  // scores are masked, their weights zero), so that the compiler can count the loads in flight and
+  // wait for the current tile only.
   auto load_tile = [&](int tb, Tile& t) {
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
-      const int pos = tb + 16 * sb + p;
-      const bool in = pos < t1;
-      t.st[sb] = in ? ldg16(stb + (size_t)pos * 4) : make_uint4(0, 0, 0, 0);
+      const int pos = min(tb + 16 * sb + p, t1 - 1);
+      t.st[sb] = ldg16(stb + (size_t)pos * 4);
 #pragma unroll
-      for (int c = 0; c < NCB; ++c)
-        t.k[sb][c] = in ? ldg16_nt(kb8 + (size_t)pos * row + dq * (D / 4) + 16 * c) : make_uint4(0, 0, 0, 0);
+      for (int c = 0; c < NCB; ++c) t.k[sb][c] = ldg16_nt(kb8 + (size_t)pos * row + dq * (D / 4) + 16 * c);
     }
 #pragma unroll
     for (int c = 0; c < NV; ++c) {
-      const int vp = tb + c * PP + pp;
-      u32x2 w = (u32x2){0x80808080u, 0x80808080u};
-      if (vp < t1) w = __builtin_nontemporal_load((const OHARA_GLOBAL u32x2*)(vb8 + (size_t)vp * row + dc * 8));
+      const int vp = min(tb + c * PP + pp, t1 - 1);
+      const u32x2 w = __builtin_nontemporal_load((const OHARA_GLOBAL u32x2*)(vb8 + (size_t)vp * row + dc * 8));
       t.v[c] = make_uint2(w.x, w.y);
     }
   };
   Tile cur, nxt;
-  int tb = t0 + wave * 32;
-  if (tb < t1) load_tile(tb, cur);
-  for (; tb < t1; tb += 128) {
-    const bool more = tb + 128 < t1;
-    if (more) load_tile(tb + 128, nxt);
+  auto consume = [&](int tb, const Tile& cur) {
     // One sub-tile of 16 positions at a time (both at once would need the registers of two expanded K
     // tiles); within it the heads of the group advance together, as in the bf16 kernel.
 #pragma unroll
@@ -454,27 +478,62 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
         pv[hh] = __expf(sc[hh] - m_run[hh]);  // (a sub-tile past the end: exp(-inf - m) = 0; m is finite by then)
         l_run[hh] += pv[hh];
       }
+      // the exchanges of a few rows first (scale, minimum and weight of the row whose codes this lane
+      // holds: independent of each other), then their products; next to its products every exchange
+      // would be waited for by itself
+      constexpr int XB = G >= 4 ? 1 : (G == 2 ? 2 : NV / 2);  // rows per round: what the registers allow
 #pragma unroll
-      for (int cc = 0; cc < NV / 2; ++cc) {
-        const int c = sb * (NV / 2) + cc;
-        const int src = 4 * ((c * PP + pp) & 15);  // a lane that owns the position of the row I hold eight codes of
-        const float vs = __shfl(__uint_as_float(cur.st[sb].z), src, WAVE);
-        const float vm = __shfl(__uint_as_float(cur.st[sb].w), src, WAVE);
-        const uint2 lo = dequant4(cur.v[c].x ^ 0x80808080u, vs, vm), hi = dequant4(cur.v[c].y ^ 0x80808080u, vs, vm);
-        const uint32_t w4[4] = {lo.x, lo.y, hi.x, hi.y};
-        float pw[G];
+      for (int c0 = 0; c0 < NV / 2; c0 += XB) {
+        float vs[XB], vm[XB], pw[XB][G];
 #pragma unroll
-        for (int hh = 0; hh < G; ++hh) pw[hh] = __shfl(pv[hh], src, WAVE);
+        for (int cc = 0; cc < XB; ++cc) {
+          const int c = sb * (NV / 2) + c0 + cc;
+          const int src = 4 * ((c * PP + pp) & 15);  // a lane that owns the position of the row I hold eight codes of
+          vs[cc] = __shfl(__uint_as_float(cur.st[sb].z), src, WAVE);
+          vm[cc] = __shfl(__uint_as_float(cur.st[sb].w), src, WAVE);
 #pragma unroll
-        for (int hh = 0; hh < G; ++hh)
+          for (int hh = 0; hh < G; ++hh) pw[cc][hh] = __shfl(pv[hh], src, WAVE);
+        }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            acc[hh][2 * i] += pw[hh] * lo_bf(w4[i]);
-            acc[hh][2 * i + 1] += pw[hh] * hi_bf(w4[i]);
-          }
+        for (int cc = 0; cc < XB; ++cc) {
+          const int c = sb * (NV / 2) + c0 + cc;
+          const uint2 lo = dequant4(cur.v[c].x ^ 0x80808080u, vs[cc], vm[cc]),
+                      hi = dequant4(cur.v[c].y ^ 0x80808080u, vs[cc], vm[cc]);
+          const uint32_t w4[4] = {lo.x, lo.y, hi.x, hi.y};
+#pragma unroll
+          for (int hh = 0; hh < G; ++hh)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              acc[hh][2 * i] += pw[cc][hh] * lo_bf(w4[i]);
+              acc[hh][2 * i + 1] += pw[cc][hh] * hi_bf(w4[i]);
+            }
+        }
       }
     }
-    if (more) cur = nxt;
+  };
+  int tb = t0 + wave * 32;
+  if (tb < t1) {
+    load_tile(tb, cur);
+    if constexpr (G >= 4) {  // two tiles taking turns do not fit the registers of four heads
+      for (; tb + 128 < t1; tb += 128) {
+        load_tile(tb + 128, nxt);
+        consume(tb, cur);
+        cur = nxt;
+      }
+      consume(tb, cur);
+    } else {
+      for (;;) {
+        if (tb + 128 >= t1) { consume(tb, cur); break; }
+        load_tile(tb + 128, nxt);
+        consume(tb, cur);
+        tb += 128;
+        if (tb + 128 >= t1) { consume(tb, nxt); break; }
+        load_tile(tb + 128, cur);
+        consume(tb, nxt);
+        tb += 128;
+      }
+    }
   }
 
   // fold the sums over the 16 positions of a sub-tile, the PP row-groups of the wave, then the four waves

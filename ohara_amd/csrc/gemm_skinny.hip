@@ -94,15 +94,31 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(GemmArgs a) {
     float part[BT], psum[BT];
 #pragma unroll
     for (int t = 0; t < BT; ++t) part[t] = psum[t] = 0.f;
-    for (int j = j0; j < j1; ++j) {
-      const int k0 = 32 * j + 8 * g;
+    // CH k-steps per round, all loads of a round issued before the first is used (one round trip
+    // per round instead of one per k-step); pieces outside the matrix read element 0 and are not added
+    for (int j = j0; j < j1; j += CH) {
+      uint4 xv[CH][BT];
 #pragma unroll
-      for (int t = 0; t < BT; ++t) {
-        const int b = rbase + m + 16 * t;
-        if (b < a.B && k0 < a.K) {
-          const uint4 xv = ldg16(a.x + (size_t)b * a.ldx + k0);
-          part[t] += sumsq8(xv);
-          if (NORM == 2) psum[t] += sum8(xv);
+      for (int c = 0; c < CH; ++c) {
+        const int k0 = 32 * (j + c) + 8 * g;
+#pragma unroll
+        for (int t = 0; t < BT; ++t) {
+          const int b = rbase + m + 16 * t;
+          const bool in = j + c < j1 && b < a.B && k0 < a.K;
+          xv[c][t] = ldg16(a.x + (in ? (size_t)b * a.ldx + k0 : (size_t)0));
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const int k0 = 32 * (j + c) + 8 * g;
+#pragma unroll
+        for (int t = 0; t < BT; ++t) {
+          const int b = rbase + m + 16 * t;
+          if (j + c < j1 && b < a.B && k0 < a.K) {
+            part[t] += sumsq8(xv[c][t]);
+            if (NORM == 2) psum[t] += sum8(xv[c][t]);
+          }
         }
       }
     }
