@@ -790,7 +790,10 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
       if (first) {
         bf16_t* xs = L.stage;
         const int ldxs = L.ldm;
-        stage_attn_merge_any<false>(a.ns, xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
+        // a single sequence always runs with 16 chunks unless there are more than 16 KV heads: that
+        // merge is part of the kernel (a call would wait for the weights already in flight)
+        if (ONE && a.ns == 16 && B * HD > 4 * 256) stage_attn_merge<16>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
+        else stage_attn_merge_any<false>(a.ns, xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
         __syncthreads();
         const bf16_t* nwo = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BO]));
         if (ONE) {
