@@ -732,6 +732,39 @@ __device__ __forceinline__ void attn_tile_load(const bf16_t* kb, const bf16_t* v
   }
 }
 
+// The same tile inside the loop over a chunk: every load issued without a branch (positions past
+// the chunk repeat its last row; their scores are masked and their weights are zero), so that the
+// compiler can count the loads in flight and wait for the current tile only while the next one is
+// on its way.  The row appended in this step is then fetched again with device-scope loads by the
+// lanes that hold it (a branch the whole wave takes or skips).
+template <int D>
+__device__ __forceinline__ void attn_tile_load_u(const bf16_t* kb, const bf16_t* vb, size_t row, int tb, int t1,
+                                                 int coh_pos, uint4* kv, uint4* vv) {
+  constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
+  const int lane = threadIdx.x & 63;
+  const int p = lane & 15, dq = lane >> 4;
+  const int pp = lane / DC, dc = lane % DC;
+  const int pos = min(tb + p, t1 - 1);
+#pragma unroll
+  for (int c = 0; c < NC; ++c) kv[c] = ldg16_nt(kb + (size_t)pos * row + (4 * c + dq) * 8);
+#pragma unroll
+  for (int c = 0; c < NV; ++c) {
+    const int vp = min(tb + c * PP + pp, t1 - 1);
+    vv[c] = ldg16_nt(vb + (size_t)vp * row + dc * 8);
+  }
+  if (coh_pos >= tb && coh_pos < tb + 16) {  // wave-uniform: this tile holds the appended row
+    if (pos == coh_pos) {
+#pragma unroll
+      for (int c = 0; c < NC; ++c) kv[c] = ld_coh16(kb + (size_t)pos * row + (4 * c + dq) * 8);
+    }
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+      const int vp = min(tb + c * PP + pp, t1 - 1);
+      if (vp == coh_pos) vv[c] = ld_coh16(vb + (size_t)vp * row + dc * 8);
+    }
+  }
+}
+
 __device__ __forceinline__ void attn_item_range(int item, int ns, int Hkv, int L, int& b, int& kvh, int& split, int& t0,
                                                 int& t1) {
   const int chunk = (((L + ns - 1) / ns) + 15) & ~15;
@@ -801,20 +834,18 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
           qv[hh][c] = ldg16(xm_addr(qm, blk_x, b, (kvh * G + hh) * D + (4 * c + dq) * 8));
       // the tile after the current one is in flight while the current one is consumed
       const bool use_pre = first && attn_first_tile_prefetchable<D>(t0, t1, L);
-      uint4 kv[NC], vv[NV], kn[NC], vn[NV];
+      uint4 ka[NC], va[NV], kn[NC], vn[NV];
       int tb = t0 + wave * 16;
       if (use_pre) {
 #pragma unroll
-        for (int c = 0; c < NC; ++c) kv[c] = pre.k[c];
+        for (int c = 0; c < NC; ++c) ka[c] = pre.k[c];
 #pragma unroll
-        for (int c = 0; c < NV; ++c) vv[c] = pre.v[c];
+        for (int c = 0; c < NV; ++c) va[c] = pre.v[c];
       } else {
-        attn_tile_load<D>(kb, vb, row, tb, t1, L - 1, kv, vv);
+        attn_tile_load_u<D>(kb, vb, row, tb, t1, L - 1, ka, va);
       }
-      for (; tb < t1; tb += 64) {
+      auto consume = [&](int tb, const uint4* kv, const uint4* vv) {
         const bool valid = tb + p < t1;
-        const bool more = tb + 64 < t1;
-        if (more) attn_tile_load<D>(kb, vb, row, tb + 64, t1, L - 1, kn, vn);
         // The heads of the group advance in lock step (their cross-lane exchanges overlap); l_run is
         // this lane's share of the sum, folded over the 16 positions after the loop; the running
         // maximum is re-derived only for tiles in which some score exceeds it.
@@ -863,27 +894,36 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
           pv[hh] = __expf(sc[hh] - m_run[hh]);
           l_run[hh] += pv[hh];
         }
+        // all weight exchanges first (they are independent), then the products
+        float pw[NV][G];
+#pragma unroll
+        for (int c = 0; c < NV; ++c)
+#pragma unroll
+          for (int hh = 0; hh < G; ++hh) pw[c][hh] = __shfl(pv[hh], c * PP + pp, WAVE);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int c = 0; c < NV; ++c) {
           const uint32_t w4[4] = {vv[c].x, vv[c].y, vv[c].z, vv[c].w};
-          float pw[G];
-#pragma unroll
-          for (int hh = 0; hh < G; ++hh) pw[hh] = __shfl(pv[hh], c * PP + pp, WAVE);
 #pragma unroll
           for (int hh = 0; hh < G; ++hh)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-              acc[hh][2 * i] += pw[hh] * lo_bf(w4[i]);
-              acc[hh][2 * i + 1] += pw[hh] * hi_bf(w4[i]);
+              acc[hh][2 * i] += pw[c][hh] * lo_bf(w4[i]);
+              acc[hh][2 * i + 1] += pw[c][hh] * hi_bf(w4[i]);
             }
         }
-        if (more) {
+      };
+      // (a chunk is one or two tiles per wave here: the next tile goes through a second register set
+      // and is copied over, which costs a wait but far fewer registers than two sets taking turns)
+      for (; tb + 64 < t1; tb += 64) {
+        attn_tile_load_u<D>(kb, vb, row, tb + 64, t1, L - 1, kn, vn);
+        consume(tb, ka, va);
 #pragma unroll
-          for (int c = 0; c < NC; ++c) kv[c] = kn[c];
+        for (int c = 0; c < NC; ++c) ka[c] = kn[c];
 #pragma unroll
-          for (int c = 0; c < NV; ++c) vv[c] = vn[c];
-        }
+        for (int c = 0; c < NV; ++c) va[c] = vn[c];
       }
+      consume(tb, ka, va);
     }
     first = false;
 #pragma unroll
