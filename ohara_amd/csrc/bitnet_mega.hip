@@ -933,7 +933,7 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
     const int ldxs = d + 8;
     bit_stage_final_norm<4>(xs, ldxs, xf, m.final_norm, m.eps, B, d);
     __syncthreads();
-    gemm_phase<1, 24, E_LOGITS>(lm, lpre, xs, ldxs, B, L.red, best_v, best_i, pf);
+    lm_phase(lm, lpre, xs, ldxs, B, best_v, best_i, pf);
   }
   if (a.select) {
 #pragma unroll

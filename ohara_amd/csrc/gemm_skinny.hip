@@ -244,11 +244,14 @@ __global__ __launch_bounds__(WIDE_WAVES * 64) void wide_kernel(GemmArgs a) {
   // two register buffers of WIDE_CH k-steps; the first strip's are requested before the
   // activations are staged, so the weight stream starts with the kernel
   uint4 wa[WIDE_CH], wb[WIDE_CH];
+  // No branch around a load and nothing that touches the value: k-steps and strips outside the
+  // matrix read a valid tile instead and are never multiplied (mul() skips k-steps >= KS, the strip
+  // loop ends before a strip >= nstrips is used).  The compiler can then count the loads in flight
+  // and wait for one buffer while the other fills.
   auto load = [&](uint4* w, int st, int j) {
-    const uint4* wrow = a.wp + (size_t)st * KS * 64 + lane;
+    const uint4* wrow = a.wp + (size_t)(st < a.nstrips ? st : 0) * KS * 64 + lane;
 #pragma unroll
-    for (int c = 0; c < WIDE_CH; ++c)
-      w[c] = (st < a.nstrips && j + c < KS) ? ldg16_nt(wrow + (size_t)(j + c) * 64) : make_uint4(0, 0, 0, 0);
+    for (int c = 0; c < WIDE_CH; ++c) w[c] = ldg16_nt(wrow + (size_t)min(j + c, KS - 1) * 64);
   };
   load(wa, strip, 0);
   load(wb, strip, WIDE_CH);

@@ -202,7 +202,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
                              a.dm + (size_t)(m.n_layers - 1) * a.dm_stride, a.ids, m.token_emb, V, m.final_norm, m.eps, B, d,
                              pre.g);
   __syncthreads();
-  gemm_phase<1, 24, E_LOGITS>(lm, pre, xs, ldxs, B, red, best_v, best_i, pf);
+  lm_phase(lm, pre, xs, ldxs, B, best_v, best_i, pf);
   pf.stamp();
   if (a.select) {
     // lanes with the same batch column (lane & 15) fold their candidates; then the waves

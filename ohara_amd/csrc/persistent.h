@@ -700,6 +700,99 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
 }
 
 // ---------------------------------------------------------------------------------------
+// Vocabulary projection (one wave per strip, the whole K in that wave, running arg-max): the
+// phase that is bound by HBM bandwidth, so it must never run out of loads in flight.  The
+// (strip, 12-k-step chunk) pairs of a wave form one sequence; two register buffers of twelve
+// tiles take turns along it: while one is multiplied, the other is on its way, and each is
+// requested again the moment its products are issued.  No load sits behind a branch or is
+// touched before use (chunks past the end read a valid tile that is never multiplied), so the
+// compiler waits for exactly the buffer it needs.  Same products in the same order as
+// gemm_phase<1, 24, E_LOGITS>, whose prefetch (the first strip's first 24 k-steps) it takes over.
+// ---------------------------------------------------------------------------------------
+template <class PROF>
+__device__ __forceinline__ void lm_phase(const GemmP& p, const GemmPre& pre, const bf16_t* xs, int ldxs, int B,
+                                         float& best_v, int& best_i, PROF& pf) {
+  constexpr int HC = 12;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m = lane & 15, g = lane >> 4;
+  const int KS = (p.K + 31) >> 5;
+  const int nwg = gridDim.x;
+  const int iters = (p.nstrips + nwg * 4 - 1) / (nwg * 4);
+  const int ncps = (KS + HC - 1) / HC;  // chunks per strip
+  const int total = iters * ncps;
+  const bool mine = m < B;
+  const bf16_t* xrow = xs + (size_t)m * ldxs + 8 * g;
+  auto strip_of = [&](int it) { return (it * nwg + (int)blockIdx.x) * 4 + wave; };
+  auto load = [&](uint4 (&w)[HC], int q) {
+    const int it = q / ncps, c = q - it * ncps;
+    const int st = strip_of(it);
+    const uint4* wrow = p.wp + (size_t)(st < p.nstrips ? st : 0) * KS * 64 + lane;
+#pragma unroll
+    for (int cc = 0; cc < HC; ++cc) w[cc] = ldg16_nt(wrow + (size_t)min(c * HC + cc, KS - 1) * 64);
+  };
+  uint4 wa[HC], wb[HC];
+#pragma unroll
+  for (int cc = 0; cc < HC; ++cc) wa[cc] = pre.w[cc];
+  if (ncps >= 2) {
+#pragma unroll
+    for (int cc = 0; cc < HC; ++cc) wb[cc] = pre.w[HC + cc];
+  } else {
+    load(wb, 1);
+  }
+  f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+  auto process = [&](const uint4 (&w)[HC], int q) {
+    const int it = q / ncps, c = q - it * ncps;
+    const int strip = strip_of(it);
+    if (c == 0) acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+    if (strip >= p.nstrips) return;
+    uint4 xv[HC];
+#pragma unroll
+    for (int cc = 0; cc < HC; ++cc) {
+      const int j = c * HC + cc;
+      xv[cc] = make_uint4(0, 0, 0, 0);  // k-steps past K multiply zeros
+      if (mine && j < KS && 32 * j + 8 * g < p.K) xv[cc] = *reinterpret_cast<const uint4*>(xrow + 32 * j);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int cc = 0; cc < HC; ++cc)
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w[cc]), __builtin_bit_cast(bf16x8, xv[cc]),
+                                                    acc, 0, 0, 0);
+    if (c != ncps - 1 || !mine) return;
+    const int b = m;
+    const int r0 = strip * 16 + 4 * g;
+    const float v[4] = {rbf(acc[0]), rbf(acc[1]), rbf(acc[2]), rbf(acc[3])};
+    bf16_t* o = reinterpret_cast<bf16_t*>(p.out) + (size_t)b * p.ldo + r0;
+    if (r0 + 3 < p.N && ((p.ldo & 3) == 0)) {
+      stg8(o, make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3])));
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (r0 + i < p.N) o[i] = f2bf(v[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int id = r0 + i;
+      if (id < p.valid && (v[i] > best_v || (v[i] == best_v && id < best_i))) {
+        best_v = v[i];
+        best_i = id;
+      }
+    }
+  };
+  for (int q = 0; q < total; q += 2) {
+    process(wa, q);
+    load(wa, q + 2);
+    if (q == 0) {
+      pf.stamp();  // first products issued
+      pf.stamp();
+    }
+    if (q + 1 < total) {
+      process(wb, q + 1);
+      load(wb, q + 3);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // attention phase: items (sequence, kv head, chunk); writes partial triples.  The K/V
 // tiles of a wave's first 16 positions are fetched before the barrier.
 // ---------------------------------------------------------------------------------------
