@@ -774,7 +774,7 @@ def main():
             sess2.check_error()
             if sess2.persistent:
                 kb = step_bytes(cfg, 1, args.prompt + args.warmup + (n_prof + 1) / 2.0)
-                kname = "decode_mega_kernel<128,1> (whole decode step: 12 layers + vocabulary projection + selection)"
+                kname = "decode_mega_kernel<128,1,true,false> (batch-1 build; whole decode step: 12 layers + vocabulary projection + selection)"
             else:
                 kb = lm_head_bytes(cfg, 1)
                 kname = "wide_kernel<1,true,STORE> (final norm + vocabulary projection 65536x768)"
