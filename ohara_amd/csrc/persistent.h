@@ -34,38 +34,47 @@ struct ProfT<false> {
 };
 
 // ---------------------------------------------------------------------------------------
-// Grid barrier.  Two levels of monotonic counters (groups of 16 workgroups, each counter on
-// its own 256-byte line, then one counter over the groups) and a release word everyone
-// polls; a flat counter serialises 256 read-modify-writes on one address (~11 us here),
-// this takes ~1.6 us.  Words (uint32, stride 64 per counter): [g*64] group g, [ng*64] top,
-// [(ng+1)*64] release, [(ng+2)*64] sticky error, [(ng+3)*64] barriers completed by earlier
-// launches.  arrive() and wait() are split so that a workgroup can issue the loads of its
-// next phase (weights, cache tiles: nothing that depends on this phase) in between and
-// have them in flight while it waits.  (Measured and dropped: no second counter level, the
-// workgroup that completes a group publishes the barrier index in that group's flag word and
-// one wave per workgroup polls the 16 adjacent flags - 0.352 ms against 0.339 ms per step.)
+// Grid barrier.  Arrivals are fire-and-forget atomics on monotonic group counters (groups of 16
+// workgroups, each counter on its own 256-byte line: same-address atomics serialise at ~11 ns
+// each); ONE master workgroup - the last of the grid, which has the least work in most phases -
+// polls all group counters with one load per lane and publishes the barrier index in a release
+// word that everyone polls.  The chain after the last arrival is: atomic reaches memory, the
+// master's next poll sees it (a device-scope load takes 0.13 us), release store seen by the
+// pollers (0.58 us) - about 1.5 us per barrier in a stand-alone loop against 2.0 us for two levels
+// of atomics WITH return (each 0.39 us) in front of the same release.  The master polls before it
+// issues its own prefetch for the next phase (its polls would otherwise return behind those loads)
+// and moves on as soon as it has seen every arrival, which is before anyone else sees the release.
+// Words (uint32, stride 64 per counter): [g*64] group g, [ng*64] unused, [(ng+1)*64] release,
+// [(ng+2)*64] sticky error, [(ng+3)*64] barriers completed by earlier launches.  arrive() and
+// wait() are split so that a workgroup can issue the loads of its next phase (weights, cache
+// tiles: nothing that depends on this phase) in between and have them in flight while it waits.
+// (Measured and dropped: a flat counter (serialises 256 read-modify-writes); the workgroup that
+// completes a group publishing a flag that one wave per workgroup polls (0.352 against 0.339 ms per
+// step); everyone polling a counter that is still receiving atomics (twice as slow); flags gathered
+// by one wave or by group leaders.)
 // ---------------------------------------------------------------------------------------
 #define OHARA_BAR_GROUP 16
 struct GridSync {
+  unsigned int* bar;
   unsigned int* gc;
-  unsigned int* top;
   unsigned int* rel;
   unsigned int* err;
   unsigned int* done;
   unsigned int k;      // index of the next barrier (1-based, across launches)
-  unsigned int gsize;  // workgroups in my group
+  unsigned int nwg;
   unsigned int ng;
   unsigned int limit;
-  __device__ void init(unsigned int* bar, unsigned int nwg, unsigned int lim) {
+  bool master;
+  __device__ void init(unsigned int* b, unsigned int n, unsigned int lim) {
+    bar = b;
+    nwg = n;
     ng = (nwg + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP;
-    const unsigned int g = blockIdx.x / OHARA_BAR_GROUP;
-    gsize = min((unsigned int)OHARA_BAR_GROUP, nwg - g * OHARA_BAR_GROUP);
-    gc = bar + g * 64;
-    top = bar + ng * 64;
+    gc = bar + (blockIdx.x / OHARA_BAR_GROUP) * 64;
     rel = bar + (ng + 1) * 64;
     err = bar + (ng + 2) * 64;
     done = bar + (ng + 3) * 64;
     limit = lim;
+    master = blockIdx.x == nwg - 1;
     k = *done + 1;  // written by the previous launch (or the host): plain load
   }
   template <class PROF>
@@ -76,13 +85,24 @@ struct GridSync {
     pf.stamp();  // stores complete
     __builtin_amdgcn_s_barrier();
     pf.stamp();  // workgroup barrier passed
-    // The whole arrival happens here, before the caller's prefetch: the last workgroup of a group
-    // must not sit on the group's arrival while it issues loads.
-    if (threadIdx.x == 0) {
-      const unsigned int a = __hip_atomic_fetch_add(gc, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
-      if (a == k * gsize) {
-        const unsigned int t = __hip_atomic_fetch_add(top, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
-        if (t == k * ng) __hip_atomic_store(rel, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // The arrival happens here, before the caller's prefetch: nobody's arrival waits behind loads.
+    if (threadIdx.x == 0) (void)__hip_atomic_fetch_add(gc, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (master && threadIdx.x < 64) {
+      // lane l watches group l: k * (its size) arrivals since the workspace was cleared
+      const unsigned int lane = threadIdx.x;
+      const unsigned int gsize = lane < ng ? min((unsigned int)OHARA_BAR_GROUP, nwg - lane * OHARA_BAR_GROUP) : 0u;
+      const unsigned int want = k * gsize;
+      unsigned int spins = 0;
+      bool ok = true;
+      for (;;) {
+        const unsigned int v = lane < ng ? __hip_atomic_load(bar + lane * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : want;
+        if (__all((int)(v - want) >= 0)) break;
+        if (++spins > limit) { ok = false; break; }
+        if ((spins & 63u) == 0 && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) { ok = false; break; }
+      }
+      if (lane == 0) {
+        if (ok) __hip_atomic_store(rel, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else __hip_atomic_store(err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
     asm volatile("" ::: "memory");  // compiler only: keep the caller's prefetch loads after this point
@@ -91,7 +111,7 @@ struct GridSync {
   template <class PROF>
   __device__ __forceinline__ void wait(PROF& pf) {
     pf.stamp();  // prefetch issued
-    if (threadIdx.x == 0) {
+    if (threadIdx.x == 0 && !master) {
       unsigned int spins = 0;
       while ((int)(__hip_atomic_load(rel, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - k) < 0) {
         ++spins;
