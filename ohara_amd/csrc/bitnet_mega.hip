@@ -1008,7 +1008,7 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
 }
 
 // ---- workspace layout ------------------------------------------------------------------
-#define OHARA_BIT_BAR_WORDS(nwg) ((((nwg) + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP + 4) * 64)
+#define OHARA_BIT_BAR_WORDS(nwg) ((((nwg) + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP + 12) * 64)
 
 size_t bit_al(size_t v) { return (v + 255) & ~(size_t)255; }
 

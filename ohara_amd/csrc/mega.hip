@@ -282,7 +282,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
 }
 
 // ---- workspace layout ------------------------------------------------------------------
-#define OHARA_BAR_WORDS(nwg) ((((nwg) + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP + 4) * 64)
+#define OHARA_BAR_WORDS(nwg) ((((nwg) + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP + 12) * 64)
 #define OHARA_PROF_SLOTS 1024
 
 size_t mega_al(size_t v) { return (v + 255) & ~(size_t)255; }

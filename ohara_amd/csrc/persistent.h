@@ -37,15 +37,17 @@ struct ProfT<false> {
 // Grid barrier.  Arrivals are fire-and-forget atomics on monotonic group counters (groups of 16
 // workgroups, each counter on its own 256-byte line: same-address atomics serialise at ~11 ns
 // each); ONE master workgroup - the last of the grid, which has the least work in most phases -
-// polls all group counters with one load per lane and publishes the barrier index in a release
-// word that everyone polls.  The chain after the last arrival is: atomic reaches memory, the
+// polls all group counters with one load per lane and publishes the barrier index in eight release
+// words (one per XCD's workgroups, each on its own line: 32 pollers per word instead of 256 measured
+// 0.14 us faster per barrier).  The chain after the last arrival is: atomic reaches memory, the
 // master's next poll sees it (a device-scope load takes 0.13 us), release store seen by the
 // pollers (0.58 us) - about 1.5 us per barrier in a stand-alone loop against 2.0 us for two levels
 // of atomics WITH return (each 0.39 us) in front of the same release.  The master polls before it
 // issues its own prefetch for the next phase (its polls would otherwise return behind those loads)
 // and moves on as soon as it has seen every arrival, which is before anyone else sees the release.
-// Words (uint32, stride 64 per counter): [g*64] group g, [ng*64] unused, [(ng+1)*64] release,
-// [(ng+2)*64] sticky error, [(ng+3)*64] barriers completed by earlier launches.  arrive() and
+// Words (uint32, stride 64 per counter): [g*64] group g, [ng*64] and [(ng+1)*64] unused,
+// [(ng+2)*64] sticky error, [(ng+3)*64] barriers completed by earlier launches, [(ng+4+x)*64]
+// release word x (workgroups with blockIdx % 8 == x poll it).  arrive() and
 // wait() are split so that a workgroup can issue the loads of its next phase (weights, cache
 // tiles: nothing that depends on this phase) in between and have them in flight while it waits.
 // (Measured and dropped: a flat counter (serialises 256 read-modify-writes); the workgroup that
@@ -70,7 +72,7 @@ struct GridSync {
     nwg = n;
     ng = (nwg + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP;
     gc = bar + (blockIdx.x / OHARA_BAR_GROUP) * 64;
-    rel = bar + (ng + 1) * 64;
+    rel = bar + (ng + 4 + (blockIdx.x & 7)) * 64;
     err = bar + (ng + 2) * 64;
     done = bar + (ng + 3) * 64;
     limit = lim;
@@ -100,10 +102,8 @@ struct GridSync {
         if (++spins > limit) { ok = false; break; }
         if ((spins & 63u) == 0 && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) { ok = false; break; }
       }
-      if (lane == 0) {
-        if (ok) __hip_atomic_store(rel, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        else __hip_atomic_store(err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
+      if (ok && lane < 8) __hip_atomic_store(bar + (ng + 4 + lane) * 64, k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (!ok && lane == 0) __hip_atomic_store(err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     asm volatile("" ::: "memory");  // compiler only: keep the caller's prefetch loads after this point
     pf.stamp();  // arrival issued
