@@ -187,16 +187,18 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     __syncthreads();
     gemm_phase<4, 6, E_PART>(dn, pre, xs, ldxs, B, red, best_v, best_i, pf);
     gs.arrive(pf);
-    if (l + 1 < m.n_layers) {
-      qkv.wp = lds_ptr<const uint4>(pl, 8);
-      qkv.norm_w = lds_ptr<const bf16_t>(pl, 12);
-      gemm_prefetch<4, 6, E_ROPE>(qkv, pre, B);
-    } else {
-      gemm_prefetch<1, 24, E_LOGITS>(lm, pre, B);
-    }
+    // (the last layer leaves the loop here: with both prefetches behind one if / else the compiler
+    // waited for the vocabulary projection's 24 tiles at the join, before the barrier wait)
+    if (l + 1 == m.n_layers) break;
+    qkv.wp = lds_ptr<const uint4>(pl, 8);
+    qkv.norm_w = lds_ptr<const bf16_t>(pl, 12);
+    gemm_prefetch<4, 6, E_ROPE>(qkv, pre, B);
     gs.wait(pf);
     pf.stamp();
   }
+  gemm_prefetch<1, 24, E_LOGITS>(lm, pre, B);
+  gs.wait(pf);
+  pf.stamp();
   // final norm + vocabulary projection, running arg-max per lane
   stage_norm<2, false, true, true>(xs, ldxs, a.xm + (size_t)(m.n_layers - 1) * a.xm_stride, a.blk_x,
                              a.dm + (size_t)(m.n_layers - 1) * a.dm_stride, a.ids, m.token_emb, V, m.final_norm, m.eps, B, d,

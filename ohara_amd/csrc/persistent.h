@@ -496,8 +496,12 @@ struct GemmP {
 struct GemmPre {  // one register buffer, reused by every phase (only one prefetch is live at a time)
   uint4 w[OHARA_MAX_PF];
   uint4 g[2];     // the lane's pieces of the weights of the norm staged ahead of the phase (GemmP::norm_w)
-  uint2 r;        // E_RESID: the four residual values of this lane (first strip); E_ROPE: its cos / sin pairs
+  uint2 r;        // E_RESID with embedding rows: the four residual values of this lane (first strip); E_ROPE: its cos / sin pairs
+  // E_RESID (which fetches six weight tiles): w[OHARA_PRE_RESID .. +4] hold the residual's pieces as loaded -
+  // the stream before the block and the four partial sums of the down projection - and the epilogue adds them
+  // up (adding them here would make the prefetch wait for them before it goes on)
 };
+#define OHARA_PRE_RESID 18
 
 // Work unit -> strip and this wave's k-steps [j0, j1).  E_PART: the units of K partition q follow
 // those of partition q - 1, so the partitions of a strip land on different workgroups.
@@ -527,10 +531,6 @@ __device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int 
   const int KS = (p.K + 31) >> 5;
   int strip, j0, j1;
   const bool live = gemm_unit<KP, EPI>(p, (int)blockIdx.x * SPW + sub, kpart, KS, strip, j0, j1);
-  const uint4* wrow = p.wp + (size_t)strip * KS * 64 + lane;
-#pragma unroll
-  for (int c = 0; c < PF; ++c)
-    pre.w[c] = (live && j0 + c < j1) ? ldg16_nt(wrow + (size_t)(j0 + c) * 64) : make_uint4(0, 0, 0, 0);
   // Everything else the phase reads that does not depend on the phase before it is requested here
   // too: cold reads from HBM behind the barrier would sit on the critical path of the phase.
   if (EPI == E_ROPE || EPI == E_SWIGLU || EPI == E_LOGITS) {
@@ -557,9 +557,12 @@ __device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int 
     pre.r = make_uint2(0, 0);
     if (live && kpart == 0 && m < B && r0 < p.N) {
       if (!p.resid_embed) {
-        uint32_t w[2];
-        x_load<4, true>(XParts{p.resid, p.resid_parts, p.blk, B, p.N}, m, r0, w);
-        pre.r = make_uint2(w[0], w[1]);
+        static_assert(EPI != E_RESID || PF <= OHARA_PRE_RESID, "the residual's pieces share the weight buffer");
+        XRaw<4, true> t;
+        x_fetch<4, true>(XParts{p.resid, p.resid_parts, p.blk, B, p.N}, m, r0, t);
+        pre.w[OHARA_PRE_RESID] = t.xm;
+#pragma unroll
+        for (int q = 0; q < OHARA_DOWN_SPLIT; ++q) pre.w[OHARA_PRE_RESID + 1 + q] = t.pv[q][0];
       } else {
         int64_t id = ldg_i64(p.ids + m);
         if (id < 0 || id >= p.vocab) id = 0;
@@ -567,6 +570,12 @@ __device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int 
       }
     }
   }
+  // the weights last: the small loads above are then issued with nothing of this prefetch in flight
+  // (placed behind the weight loads, the compiler made each of them wait for all of those first)
+  const uint4* wrow = p.wp + (size_t)strip * KS * 64 + lane;
+#pragma unroll
+  for (int c = 0; c < PF; ++c)
+    pre.w[c] = (live && j0 + c < j1) ? ldg16_nt(wrow + (size_t)(j0 + c) * 64) : make_uint4(0, 0, 0, 0);
 }
 
 template <int KP, int PF, int EPI, class PROF>
@@ -646,6 +655,15 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
       if (EPI == E_RESID) {  // N % 4 == 0 is required by the entry point
         if (r0 < p.N) {
           uint2 r = pre.r;
+          if (it == 0 && !p.resid_embed) {
+            XRaw<4, true> t;
+            t.xm = pre.w[OHARA_PRE_RESID];
+#pragma unroll
+            for (int q = 0; q < OHARA_DOWN_SPLIT; ++q) t.pv[q][0] = pre.w[OHARA_PRE_RESID + 1 + q];
+            uint32_t w[2];
+            x_combine<4, true>(t, w);
+            r = make_uint2(w[0], w[1]);
+          }
           if (it > 0) {
             if (!p.resid_embed) {
               uint32_t w[2];
