@@ -375,6 +375,139 @@ __device__ __forceinline__ int draw_from_block(const SampleArgs& a, Smem& s, int
   return s.misc[3];
 }
 
+// ---- the same draw by ONE wave -------------------------------------------------------------------
+// For at most 128 candidates the whole draw fits one wave's registers (lane l holds entries l and
+// l + 64): the bitonic sorts exchange through DPP moves and row swaps instead of LDS and a
+// workgroup barrier per stage (28 stages for 128 entries, 16 waves waiting at each), counts are
+// ballots, and the sequential sums of the reference's order read the probabilities lane by lane
+// with v_readlane.  Every comparison, sum and its order are those of draw_from_block: the sorts
+// use the same strict total orders, Z adds the butterfly sum of entries 0..63 and that of entries
+// 64..127 exactly as block_sum adds its first two wave sums (the other fourteen are zero).
+template <int J>
+__device__ __forceinline__ uint32_t wave_partner(uint32_t v, int lane) {  // v of lane ^ J
+  if constexpr (J < 16) {
+    return lane_xor_u32<J>(v);
+  } else {
+    const u32x2 r = J == 16 ? __builtin_amdgcn_permlane16_swap(v, v, false, false)
+                            : __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return (lane & J) ? r[0] : r[1];
+  }
+}
+// one compare-exchange stage of the bitonic network on entries t = lane (k0, i0) and lane + 64 (k1, i1);
+// BY_ID: ascending ids; otherwise descending keys, ties by ascending id
+template <int J, bool BY_ID>
+__device__ __forceinline__ void wave_sort_stage(uint32_t& k0, int& i0, uint32_t& k1, int& i1, int k2, int lane) {
+  auto first = [](uint32_t ka, int ia, uint32_t kb, int ib) {  // a precedes b in the target order
+    return BY_ID ? ia < ib : (ka > kb || (ka == kb && ia < ib));
+  };
+  if constexpr (J == 64) {
+    const bool up = (lane & k2) == 0;  // k2 == 128 here: always up
+    const bool a_first = first(k0, i0, k1, i1);
+    if (up ? !a_first : a_first) {
+      const uint32_t tk = k0; k0 = k1; k1 = tk;
+      const int ti = i0; i0 = i1; i1 = ti;
+    }
+  } else {
+    const bool lower = (lane & J) == 0;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      uint32_t& km = h ? k1 : k0;
+      int& im = h ? i1 : i0;
+      const uint32_t kp = wave_partner<J>(km, lane);
+      const int ip = (int)wave_partner<J>((uint32_t)im, lane);
+      const int t = lane + 64 * h;
+      const bool up = (t & k2) == 0;
+      // the pair in position order (a = lower index): keep as is when a already precedes b (up) / follows b (down)
+      const bool a_first = lower ? first(km, im, kp, ip) : first(kp, ip, km, im);
+      const bool swap = up ? !a_first : a_first;
+      if (swap) { km = kp; im = ip; }
+    }
+  }
+}
+template <bool BY_ID>
+__device__ __forceinline__ void wave_sort128(uint32_t& k0, int& i0, uint32_t& k1, int& i1, int lane) {
+#define OHARA_WS(J, K2) wave_sort_stage<J, BY_ID>(k0, i0, k1, i1, K2, lane)
+  OHARA_WS(1, 2);
+  OHARA_WS(2, 4); OHARA_WS(1, 4);
+  OHARA_WS(4, 8); OHARA_WS(2, 8); OHARA_WS(1, 8);
+  OHARA_WS(8, 16); OHARA_WS(4, 16); OHARA_WS(2, 16); OHARA_WS(1, 16);
+  OHARA_WS(16, 32); OHARA_WS(8, 32); OHARA_WS(4, 32); OHARA_WS(2, 32); OHARA_WS(1, 32);
+  OHARA_WS(32, 64); OHARA_WS(16, 64); OHARA_WS(8, 64); OHARA_WS(4, 64); OHARA_WS(2, 64); OHARA_WS(1, 64);
+  OHARA_WS(64, 128); OHARA_WS(32, 128); OHARA_WS(16, 128); OHARA_WS(8, 128); OHARA_WS(4, 128); OHARA_WS(2, 128);
+  OHARA_WS(1, 128);
+#undef OHARA_WS
+}
+// n_c <= 128 candidates in (s.skey, s.sid); every thread of the workgroup calls, wave 0 draws
+__device__ __forceinline__ int draw_from_wave(const SampleArgs& a, Smem& s, int n_c, int k, float u) {
+  const int tid = threadIdx.x;
+  __syncthreads();  // the candidates are in place
+  if (tid < 64) {
+    const int lane = tid;
+    uint32_t k0 = lane < n_c ? s.skey[lane] : 0u, k1 = lane + 64 < n_c ? s.skey[lane + 64] : 0u;  // padding sorts last
+    int i0 = lane < n_c ? s.sid[lane] : 0x7fffffff, i1 = lane + 64 < n_c ? s.sid[lane + 64] : 0x7fffffff;
+    wave_sort128<false>(k0, i0, k1, i1, lane);
+    const int kth = min(k, n_c) - 1;
+    const uint32_t tk = kth < 64 ? (uint32_t)__builtin_amdgcn_readlane((int)k0, kth) : (uint32_t)__builtin_amdgcn_readlane((int)k1, kth - 64);
+    const int n_kept = __popcll(__ballot(lane < n_c && k0 >= tk)) + __popcll(__ballot(lane + 64 < n_c && k1 >= tk));
+    const float m0 = unfkey((uint32_t)__builtin_amdgcn_readlane((int)k0, 0));
+    const float e0 = lane < n_kept ? expf(unfkey(k0) - m0) : 0.f;
+    const float e1 = lane + 64 < n_kept ? expf(unfkey(k1) - m0) : 0.f;
+    const float Z = wave_sum(e0) + wave_sum(e1);
+    uint32_t p0 = lane < n_kept ? __float_as_uint(e0 / Z) : k0;       // probabilities, still in sorted order
+    uint32_t p1 = lane + 64 < n_kept ? __float_as_uint(e1 / Z) : k1;  // (entries past n_kept are never read)
+    const bool nucleus = a.top_p > 0.f && a.top_p < 1.f;
+    if (!nucleus) {  // vocabulary-order draw: the kept entries by id, the rest as padding
+      if (lane >= n_kept) { p0 = 0u; i0 = 0x7fffffff; }
+      if (lane + 64 >= n_kept) { p1 = 0u; i1 = 0x7fffffff; }
+      wave_sort128<true>(p0, i0, p1, i1, lane);
+    }
+    auto prob = [&](int j) {
+      return __uint_as_float(j < 64 ? (uint32_t)__builtin_amdgcn_readlane((int)p0, j) : (uint32_t)__builtin_amdgcn_readlane((int)p1, j - 64));
+    };
+    auto ident = [&](int j) { return j < 64 ? __builtin_amdgcn_readlane(i0, j) : __builtin_amdgcn_readlane(i1, j - 64); };
+    // sequential fp32 sums in the order the reference's cumsum walks (all lanes run them: the loops are uniform)
+    int tok = -1, last = -1;
+    if (nucleus) {
+      float kept = 0.f, run = 0.f;
+      int n_in = 0;
+      for (int j = 0; j < n_kept; ++j) {  // kept prefix: mass before the token <= top_p
+        if (run > a.top_p) break;
+        const float p = prob(j);
+        kept += p;
+        run += p;
+        ++n_in;
+      }
+      const float target = u * kept;
+      run = 0.f;
+      for (int j = 0; j < n_in; ++j) {
+        run += prob(j);
+        last = ident(j);
+        if (run > target) {
+          tok = last;
+          break;
+        }
+      }
+    } else {
+      float total = 0.f;
+      for (int j = 0; j < n_kept; ++j) total += prob(j);
+      const float target = u * total;
+      float run = 0.f;
+      for (int j = 0; j < n_kept; ++j) {
+        const float p = prob(j);
+        run += p;
+        if (p > 0.f) last = ident(j);
+        if (p > 0.f && run > target) {
+          tok = ident(j);
+          break;
+        }
+      }
+    }
+    if (lane == 0) s.misc[3] = tok >= 0 ? tok : max(last, 0);  // rounding pushed the target past the end: last kept id
+  }
+  __syncthreads();
+  return s.misc[3];
+}
+
 // The selected id of a row goes out, with the loop bookkeeping when the caller keeps a step state.
 __device__ __forceinline__ void finish_row(const SampleArgs& a, int b, int token) {
   a.out[b] = token;
@@ -632,7 +765,7 @@ __device__ __forceinline__ int sample_row(const SampleArgs& a, int b, Smem& s) {
         }
       }
     }
-    if (compact) token = draw_from_block(a, s, n_c, k, u);
+    if (compact) token = n_c <= 128 ? draw_from_wave(a, s, n_c, k, u) : draw_from_block(a, s, n_c, k, u);
   }
   if (!compact && !have_x) load_x();
   // ---- top-k: keep x >= k-th largest ---------------------------------------------
@@ -891,7 +1024,7 @@ __global__ __launch_bounds__(NT) void sample_parts_kernel(SampleArgs a, uint32_t
       s.sid[slot] = (int)(w >> 16);
     }
     const float u = a.u[(a.step_state && a.u_step_stride > 0 ? (size_t)a.step_state[1] * a.u_step_stride : 0) + b];
-    token = draw_from_block(a, s, n_keep, k, u);
+    token = n_keep <= 128 ? draw_from_wave(a, s, n_keep, k, u) : draw_from_block(a, s, n_keep, k, u);
   }
   if (tid == 0) finish_row(a, b, token);
 }
