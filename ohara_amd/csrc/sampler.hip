@@ -508,6 +508,142 @@ __device__ __forceinline__ int draw_from_wave(const SampleArgs& a, Smem& s, int 
   return s.misc[3];
 }
 
+// ---- the draw by one wave from packed candidates (bf16 rows, ids below 65536) -----------------------
+// A candidate is ONE sortable word: the order-preserving 16-bit key of its bf16 logit above, 0xffff - id
+// below, so that descending words are descending logits with ties in ascending id order, and a stage
+// of the bitonic network is an exchange, a max and a min.  For the vocabulary-order draw the kept
+// entries are sorted again as ~(id << 8 | position) and fetch their probability from that position.
+// The sequential fp32 sums of the reference's cumsum are one unrolled chain: run_j = run_(j-1) + p_j
+// for every entry (entries past the kept ones add 0), lane j keeps run_(j-1) and run_j; the prefix
+// under top_p, the total and the first entry past the target are then ballots.  The values, their
+// order and every sum are those of draw_from_block.
+template <int J>
+__device__ __forceinline__ uint32_t packed_stage(uint32_t v, bool take_max) {
+  uint32_t mx, mn;
+  if constexpr (J < 16) {
+    const uint32_t o = lane_xor_u32<J>(v);
+    mx = max(v, o);
+    mn = min(v, o);
+  } else {
+    const u32x2 r = J == 16 ? __builtin_amdgcn_permlane16_swap(v, v, false, false)
+                            : __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    mx = max(r[0], r[1]);
+    mn = min(r[0], r[1]);
+  }
+  return take_max ? mx : mn;
+}
+// descending sort of 64 (TWO == false: w0 only) or 128 words (entry t = lane: w0, t = lane + 64: w1)
+template <bool TWO>
+__device__ __forceinline__ void packed_sort(uint32_t& w0, uint32_t& w1, int lane) {
+#define OHARA_PS(J, K2)                                                                       \
+  {                                                                                           \
+    const bool lower = (lane & J) == 0;                                                       \
+    w0 = packed_stage<J>(w0, lower == ((lane & K2) == 0));                                    \
+    if (TWO) w1 = packed_stage<J>(w1, lower == (((lane + 64) & K2) == 0));                    \
+  }
+  OHARA_PS(1, 2);
+  OHARA_PS(2, 4); OHARA_PS(1, 4);
+  OHARA_PS(4, 8); OHARA_PS(2, 8); OHARA_PS(1, 8);
+  OHARA_PS(8, 16); OHARA_PS(4, 16); OHARA_PS(2, 16); OHARA_PS(1, 16);
+  OHARA_PS(16, 32); OHARA_PS(8, 32); OHARA_PS(4, 32); OHARA_PS(2, 32); OHARA_PS(1, 32);
+  OHARA_PS(32, 64); OHARA_PS(16, 64); OHARA_PS(8, 64); OHARA_PS(4, 64); OHARA_PS(2, 64); OHARA_PS(1, 64);
+  if (TWO) {
+    const uint32_t mx = max(w0, w1), mn = min(w0, w1);  // entries t and t + 64, block of 128: descending
+    w0 = mx;
+    w1 = mn;
+    OHARA_PS(32, 128); OHARA_PS(16, 128); OHARA_PS(8, 128); OHARA_PS(4, 128); OHARA_PS(2, 128); OHARA_PS(1, 128);
+  }
+#undef OHARA_PS
+}
+// run_(j-1) and run_j of the sequential sum over q (uniform chain, lane j keeps its two values)
+__device__ __forceinline__ float seq_sums(uint32_t q, float run, int lane, float& before, float& after) {
+#pragma unroll
+  for (int j = 0; j < 64; ++j) {
+    const float prev = run;
+    run += __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)q, j));
+    before = lane == j ? prev : before;
+    after = lane == j ? run : after;
+  }
+  return run;
+}
+__device__ __forceinline__ float logit_of_key16(uint32_t key, float temperature) {
+  const uint32_t bits = (key & 0x8000u) ? (key ^ 0x8000u) : (~key & 0xffffu);
+  return __uint_as_float(bits << 16) / temperature;
+}
+// n_c <= 128 packed candidates in s.skey[0 .. n_c); every thread of the workgroup calls, wave 0 draws
+__device__ __forceinline__ int draw_from_wave_packed(const SampleArgs& a, Smem& s, int n_c, int k, float u) {
+  const int tid = threadIdx.x;
+  __syncthreads();  // the candidates are in place
+  if (tid < 64) {
+    const int lane = tid;
+    const bool two = n_c > 64;
+    uint32_t w0 = lane < n_c ? s.skey[lane] : 0u, w1 = lane + 64 < n_c ? s.skey[lane + 64] : 0u;  // padding sorts last
+    if (two) packed_sort<true>(w0, w1, lane);
+    else packed_sort<false>(w0, w1, lane);
+    const int kth = min(k, n_c) - 1;
+    const uint32_t tk = (kth < 64 ? (uint32_t)__builtin_amdgcn_readlane((int)w0, kth)
+                                  : (uint32_t)__builtin_amdgcn_readlane((int)w1, kth - 64)) >> 16;
+    const int n_kept = __popcll(__ballot(lane < n_c && (w0 >> 16) >= tk)) +
+                       __popcll(__ballot(lane + 64 < n_c && (w1 >> 16) >= tk));
+    const float m0 = logit_of_key16((uint32_t)__builtin_amdgcn_readlane((int)w0, 0) >> 16, a.temperature);
+    const float e0 = lane < n_kept ? expf(logit_of_key16(w0 >> 16, a.temperature) - m0) : 0.f;
+    const float e1 = lane + 64 < n_kept ? expf(logit_of_key16(w1 >> 16, a.temperature) - m0) : 0.f;
+    const float Z = wave_sum(e0) + wave_sum(e1);
+    uint32_t p0 = lane < n_kept ? __float_as_uint(e0 / Z) : 0u;  // probabilities in sorted order, +0 past the kept ones
+    uint32_t p1 = lane + 64 < n_kept ? __float_as_uint(e1 / Z) : 0u;
+    int i0 = 0xffff - (int)(w0 & 0xffffu), i1 = 0xffff - (int)(w1 & 0xffffu);
+    const bool nucleus = a.top_p > 0.f && a.top_p < 1.f;
+    if (!nucleus) {  // vocabulary-order draw: the kept entries by ascending id
+      uint32_t c0 = lane < n_kept ? ~(((uint32_t)i0 << 8) | (uint32_t)lane) : 0u;
+      uint32_t c1 = lane + 64 < n_kept ? ~(((uint32_t)i1 << 8) | (uint32_t)(lane + 64)) : 0u;
+      if (two) packed_sort<true>(c0, c1, lane);
+      else packed_sort<false>(c0, c1, lane);
+      const uint32_t s0 = ~c0, s1 = ~c1;
+      const int f0 = (int)(s0 & 0xffu), f1 = (int)(s1 & 0xffu);  // where the entry stood in logit order
+      const uint32_t a0 = __shfl(p0, f0 & 63, WAVE), b0 = __shfl(p1, f0 & 63, WAVE);
+      const uint32_t a1 = __shfl(p0, f1 & 63, WAVE), b1 = __shfl(p1, f1 & 63, WAVE);
+      p0 = lane < n_kept ? (f0 < 64 ? a0 : b0) : 0u;
+      p1 = lane + 64 < n_kept ? (f1 < 64 ? a1 : b1) : 0u;
+      i0 = (int)(s0 >> 8);
+      i1 = (int)(s1 >> 8);
+    }
+    float bf0 = 0.f, af0 = 0.f, bf1 = 0.f, af1 = 0.f;
+    float run = seq_sums(p0, 0.f, lane, bf0, af0);
+    if (n_kept > 64) run = seq_sums(p1, run, lane, bf1, af1);
+    auto after_at = [&](int j) { return j < 64 ? __builtin_amdgcn_readlane(__float_as_int(af0), j) : __builtin_amdgcn_readlane(__float_as_int(af1), j - 64); };
+    auto ident = [&](int j) { return j < 64 ? __builtin_amdgcn_readlane(i0, j) : __builtin_amdgcn_readlane(i1, j - 64); };
+    int tok = -1, last = -1;
+    unsigned long long h0, h1;
+    if (nucleus) {
+      // the kept prefix: entries whose mass before them is <= top_p (the sums never decrease)
+      const unsigned long long in0 = __ballot(lane < n_kept && !(bf0 > a.top_p));
+      const unsigned long long in1 = __ballot(lane + 64 < n_kept && !(bf1 > a.top_p));
+      const int n_in = __popcll(in0) + __popcll(in1);
+      if (n_in > 0) {
+        const float target = u * __int_as_float(after_at(n_in - 1));
+        last = ident(n_in - 1);
+        h0 = __ballot(lane < n_in && af0 > target);
+        h1 = __ballot(lane + 64 < n_in && af1 > target);
+      } else {
+        h0 = h1 = 0;
+      }
+    } else {
+      const float target = u * run;
+      const unsigned long long pos0 = __ballot(lane < n_kept && __uint_as_float(p0) > 0.f);
+      const unsigned long long pos1 = __ballot(lane + 64 < n_kept && __uint_as_float(p1) > 0.f);
+      if (pos1) last = ident(64 + 63 - __clzll(pos1));
+      else if (pos0) last = ident(63 - __clzll(pos0));
+      h0 = __ballot(lane < n_kept && __uint_as_float(p0) > 0.f && af0 > target);
+      h1 = __ballot(lane + 64 < n_kept && __uint_as_float(p1) > 0.f && af1 > target);
+    }
+    if (h0) tok = ident(__ffsll(h0) - 1);
+    else if (h1) tok = ident(64 + __ffsll(h1) - 1);
+    if (lane == 0) s.misc[3] = tok >= 0 ? tok : max(last, 0);  // rounding pushed the target past the end: last kept id
+  }
+  __syncthreads();
+  return s.misc[3];
+}
+
 // The selected id of a row goes out, with the loop bookkeeping when the caller keeps a step state.
 __device__ __forceinline__ void finish_row(const SampleArgs& a, int b, int token) {
   a.out[b] = token;
@@ -955,7 +1091,10 @@ __global__ __launch_bounds__(NT) void sample_parts_kernel(SampleArgs a, uint32_t
   uint32_t tmax = 0;
 #pragma unroll
   for (int i = 0; i < 8; ++i) tmax = max(tmax, key16(i));
-  const int have = block_sum_i(tmax > 0 ? 1 : 0, s);
+  // threads that hold a valid id: all of them when the part lies below the valid ids' end and k is
+  // small (then a thread whose eight values are all NaN patterns cannot take the count below k)
+  const bool whole = (part + 1) * PART_IDS <= nvalid && k <= NT / 2;
+  const int have = whole ? NT : block_sum_i(tmax > 0 ? 1 : 0, s);
   uint32_t bound = 1;  // fewer than k threads hold a valid id: every valid id of the part is a candidate
   if (have >= k) {
     int dummy;
@@ -986,30 +1125,28 @@ __global__ __launch_bounds__(NT) void sample_parts_kernel(SampleArgs a, uint32_t
   }
   __syncthreads();
   if (!s.misc[7]) return;
+  // One round of loads: thread t looks at slot t % 128 of part t / 128 (8 parts x 128 slots are the
+  // 1024 threads) and at that part's count; lane l of every wave reads the count of part l as well, so
+  // that each wave knows by itself whether some part gave up.
   const uint32_t* rec0 = scratch + (size_t)PART_ROWS * 32 + (size_t)b * PART_MAX * PART_REC;
-  int total = 0, mine_part = -1, mine_slot = 0;
-  bool overflow = false;
-  for (int p = 0; p < nparts; ++p) {
-    const uint32_t n = ld_coh4(rec0 + (size_t)p * PART_REC);
-    if (n == 0xffffffffu) {
-      overflow = true;
-      break;
-    }
-    if (mine_part < 0 && tid < total + (int)n) {
-      mine_part = p;
-      mine_slot = tid - total;
-    }
-    total += (int)n;
+  static_assert(PART_MAX * PART_CAP == NT, "one thread per candidate slot");
+  const int my_part = tid / PART_CAP, my_slot = tid % PART_CAP;
+  const int lane = tid & 63;
+  uint32_t n_mine = 0, w = 0, n_lane = 0;
+  if (my_part < nparts) {
+    n_mine = ld_coh4(rec0 + (size_t)my_part * PART_REC);
+    w = ld_coh4(rec0 + (size_t)my_part * PART_REC + 32 + my_slot);
   }
+  if (lane < nparts) n_lane = ld_coh4(rec0 + (size_t)lane * PART_REC);
+  const bool overflow = __ballot(n_lane == 0xffffffffu) != 0;
   int token;
   if (overflow) {
     token = sample_row<bf16_t, 64>(a, b, s);
   } else {
     // the k-th largest of the gathered candidates first (16-bit keys, two counting passes), so that the
     // block that is sorted holds the k survivors and their ties, not eight times as many
-    uint32_t w = 0, k16 = 0;
-    if (tid < total) {
-      w = ld_coh4(rec0 + (size_t)mine_part * PART_REC + 32 + mine_slot);
+    uint32_t k16 = 0;
+    if (my_slot < (int)n_mine) {
       const uint32_t bits = w & 0xffffu;
       k16 = (bits & 0x8000u) ? (~bits & 0xffffu) : (bits | 0x8000u);
     }
@@ -1018,13 +1155,18 @@ __global__ __launch_bounds__(NT) void sample_parts_kernel(SampleArgs a, uint32_t
     const int keep = (k16 > 0 && k16 >= tk16) ? 1 : 0;
     int slot;
     const int n_keep = block_excl_scan_i(keep, slot, s);
-    __syncthreads();
-    if (keep) {
-      s.skey[slot] = fkey(__uint_as_float((w & 0xffffu) << 16) / a.temperature);
-      s.sid[slot] = (int)(w >> 16);
-    }
     const float u = a.u[(a.step_state && a.u_step_stride > 0 ? (size_t)a.step_state[1] * a.u_step_stride : 0) + b];
-    token = n_keep <= 128 ? draw_from_wave(a, s, n_keep, k, u) : draw_from_block(a, s, n_keep, k, u);
+    __syncthreads();
+    if (n_keep <= 128) {
+      if (keep) s.skey[slot] = (k16 << 16) | (0xffffu - (w >> 16));
+      token = draw_from_wave_packed(a, s, n_keep, k, u);
+    } else {
+      if (keep) {
+        s.skey[slot] = fkey(__uint_as_float((w & 0xffffu) << 16) / a.temperature);
+        s.sid[slot] = (int)(w >> 16);
+      }
+      token = draw_from_block(a, s, n_keep, k, u);
+    }
   }
   if (tid == 0) finish_row(a, b, token);
 }
