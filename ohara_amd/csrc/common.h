@@ -97,6 +97,19 @@ __device__ __forceinline__ void lane_swap(float v, float& a, float& b) {  // {a,
   a = __uint_as_float(r[0]);
   b = __uint_as_float(r[1]);
 }
+// Inclusive prefix sum across the 64 lanes of a wave, in lane order, through DPP moves (shifts
+// inside a row of 16 lanes, then the last lane of a row broadcast into the rows after it): six
+// moves instead of six LDS-crossbar shuffles.  All lanes of the wave must be active.
+__device__ __forceinline__ int wave_incl_scan_i(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, false);  // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, false);  // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, false);  // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, false);  // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 template <int M>
 __device__ __forceinline__ float lane_xor_sum(float v) {  // v + v of lane ^ M
   if constexpr (M >= 16) {

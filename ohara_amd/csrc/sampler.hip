@@ -56,6 +56,7 @@ __device__ __forceinline__ uint32_t fkey(float f) {  // order-preserving: larger
 
 struct Smem {
   int hist[256];
+  int hist2[256];
   float wred[16];
   int wredi[16];
   uint32_t skey[CAP];
@@ -102,15 +103,10 @@ __device__ __forceinline__ int block_sum_i(int v, Smem& s) {
 }
 
 // Exclusive prefix sum of one int per thread, in thread order.  Returns the total.
-// Wave-level shuffle scan, then the wave totals.
+// Wave-level DPP scan, then the wave totals.
 __device__ __forceinline__ int block_excl_scan_i(int v, int& excl, Smem& s) {
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  int incl = v;
-#pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    const int t = __shfl_up(incl, o, WAVE);
-    if (lane >= o) incl += t;
-  }
+  const int incl = wave_incl_scan_i(v);
   __syncthreads();
   if (lane == 63) s.wredi[w] = incl;
   __syncthreads();
@@ -223,6 +219,58 @@ __device__ __forceinline__ uint32_t select_small(int want, int& n_greater, Smem&
     bound = radix_select<1>(want, dummy, s, [&](int) { return tmax > 0; }, [&](int) { return tmax; });
   }
   return radix_select<EPT>(want, n_greater, s, [&](int i) { return live(i) && key(i) >= bound; }, key);
+}
+
+// The `want`-th largest (1-based) of one 16-bit key per thread (0: the thread holds none), two counting
+// passes of 8 bits like radix_select<1, 8>, with fewer stops: both tables are cleared up front, and
+// one wave finds the digit of a pass (a lane adds up four bins, highest first, a DPP scan across the
+// lanes), so that a pass is two workgroup barriers.  Fewer than `want` keys: digit 0, as there.
+__device__ __forceinline__ uint32_t select16_block(int want, uint32_t key, Smem& s) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  __syncthreads();  // earlier users of the tables are done
+  if (tid < 256) {
+    s.hist[tid] = 0;
+    s.hist2[tid] = 0;
+  }
+  __syncthreads();
+  auto find = [&](const int* h, int want_) {  // by wave 0: the bin that holds the want_-th largest, and the count above it
+    const int b0 = 255 - 4 * lane;            // lane l owns bins 255 - 4l .. 252 - 4l
+    const int c0 = h[b0], c1 = h[b0 - 1], c2 = h[b0 - 2], c3 = h[b0 - 3];
+    const int tot = c0 + c1 + c2 + c3;
+    const int incl = wave_incl_scan_i(tot);
+    const int excl = incl - tot;
+    if (excl < want_ && want_ <= incl) {
+      int above = excl, d = b0;
+      if (want_ > above + c0) {
+        above += c0;
+        d = b0 - 1;
+        if (want_ > above + c1) {
+          above += c1;
+          d = b0 - 2;
+          if (want_ > above + c2) {
+            above += c2;
+            d = b0 - 3;
+          }
+        }
+      }
+      s.misc[0] = d;
+      s.misc[1] = above;
+    } else if (lane == 63 && want_ > incl) {
+      s.misc[0] = 0;
+      s.misc[1] = incl - c3;
+    }
+  };
+  if (key) atomicAdd(&s.hist[key >> 8], 1);
+  __syncthreads();
+  if (tid < 64) find(s.hist, want);
+  __syncthreads();
+  const uint32_t d1 = (uint32_t)s.misc[0];
+  const int above = s.misc[1];
+  if (key && (key >> 8) == d1) atomicAdd(&s.hist2[key & 255u], 1);
+  __syncthreads();
+  if (tid < 64) find(s.hist2, want - above);
+  __syncthreads();
+  return (d1 << 8) | (uint32_t)s.misc[0];
 }
 
 template <typename T>
@@ -513,8 +561,8 @@ __device__ __forceinline__ int draw_from_wave(const SampleArgs& a, Smem& s, int 
 // below, so that descending words are descending logits with ties in ascending id order, and a stage
 // of the bitonic network is an exchange, a max and a min.  For the vocabulary-order draw the kept
 // entries are sorted again as ~(id << 8 | position) and fetch their probability from that position.
-// The sequential fp32 sums of the reference's cumsum are one unrolled chain: run_j = run_(j-1) + p_j
-// for every entry (entries past the kept ones add 0), lane j keeps run_(j-1) and run_j; the prefix
+// The sequential fp32 sums of the reference's cumsum are one chain: run_j = run_(j-1) + p_j
+// for every kept entry, lane j keeps run_(j-1) and run_j; the prefix
 // under top_p, the total and the first entry past the target are then ballots.  The values, their
 // order and every sum are those of draw_from_block.
 template <int J>
@@ -555,14 +603,19 @@ __device__ __forceinline__ void packed_sort(uint32_t& w0, uint32_t& w1, int lane
   }
 #undef OHARA_PS
 }
-// run_(j-1) and run_j of the sequential sum over q (uniform chain, lane j keeps its two values)
-__device__ __forceinline__ float seq_sums(uint32_t q, float run, int lane, float& before, float& after) {
+// run_(j-1) and run_j of the sequential sum over the first n entries of q (uniform chain, lane j keeps
+// its two values).  Eight steps per trip: a trip of one step is half loop overhead, and 64 unrolled
+// steps are 40 cache lines of straight-line code that runs once per launch from a cold instruction cache.
+__device__ __forceinline__ float seq_sums(uint32_t q, float run, int n, int lane, float& before, float& after) {
+  for (int j0 = 0; j0 < n; j0 += 8) {  // entries past n hold +0: the steps of the last trip that overshoot change nothing
 #pragma unroll
-  for (int j = 0; j < 64; ++j) {
-    const float prev = run;
-    run += __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)q, j));
-    before = lane == j ? prev : before;
-    after = lane == j ? run : after;
+    for (int i = 0; i < 8; ++i) {
+      const int j = j0 + i;
+      const float prev = run;
+      run += __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)q, j));
+      before = lane == j ? prev : before;
+      after = lane == j ? run : after;
+    }
   }
   return run;
 }
@@ -608,8 +661,8 @@ __device__ __forceinline__ int draw_from_wave_packed(const SampleArgs& a, Smem& 
       i1 = (int)(s1 >> 8);
     }
     float bf0 = 0.f, af0 = 0.f, bf1 = 0.f, af1 = 0.f;
-    float run = seq_sums(p0, 0.f, lane, bf0, af0);
-    if (n_kept > 64) run = seq_sums(p1, run, lane, bf1, af1);
+    float run = seq_sums(p0, 0.f, min(n_kept, 64), lane, bf0, af0);
+    if (n_kept > 64) run = seq_sums(p1, run, n_kept - 64, lane, bf1, af1);
     auto after_at = [&](int j) { return j < 64 ? __builtin_amdgcn_readlane(__float_as_int(af0), j) : __builtin_amdgcn_readlane(__float_as_int(af1), j - 64); };
     auto ident = [&](int j) { return j < 64 ? __builtin_amdgcn_readlane(i0, j) : __builtin_amdgcn_readlane(i1, j - 64); };
     int tok = -1, last = -1;
@@ -1049,6 +1102,16 @@ __global__ __launch_bounds__(NT) void sample_kernel(SampleArgs a) {
 }
 
 
+// Out-of-line copies of the two rarely taken routes of sample_parts_kernel (a part that gave up; more
+// than 128 survivors): inlined, the whole-row algorithm is nine tenths of that kernel's code and its
+// register demand spills values of the route that is always taken.
+__device__ __attribute__((noinline)) int sample_row_bf16_call(SampleArgs a, int b, Smem& s) {  // by value: a reference would put the caller's copy in scratch
+  return sample_row<bf16_t, 64>(a, b, s);
+}
+__device__ __attribute__((noinline)) int draw_from_block_call(SampleArgs a, Smem& s, int n_c, int k, float u) {
+  return draw_from_block(a, s, n_c, k, u);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Small top-k over several workgroups.  With top-k the draw depends on the k largest logits of the
 // row only (ties of the k-th included), and one CU walking 65536 ids is what the single-workgroup
@@ -1097,8 +1160,7 @@ __global__ __launch_bounds__(NT) void sample_parts_kernel(SampleArgs a, uint32_t
   const int have = whole ? NT : block_sum_i(tmax > 0 ? 1 : 0, s);
   uint32_t bound = 1;  // fewer than k threads hold a valid id: every valid id of the part is a candidate
   if (have >= k) {
-    int dummy;
-    bound = radix_select<1, 8>(k, dummy, s, [&](int) { return tmax > 0; }, [&](int) { return tmax; });
+    bound = select16_block(k, tmax, s);
   }
   int c = 0;
 #pragma unroll
@@ -1141,7 +1203,7 @@ __global__ __launch_bounds__(NT) void sample_parts_kernel(SampleArgs a, uint32_t
   const bool overflow = __ballot(n_lane == 0xffffffffu) != 0;
   int token;
   if (overflow) {
-    token = sample_row<bf16_t, 64>(a, b, s);
+    token = sample_row_bf16_call(a, b, s);
   } else {
     // the k-th largest of the gathered candidates first (16-bit keys, two counting passes), so that the
     // block that is sorted holds the k survivors and their ties, not eight times as many
@@ -1150,8 +1212,7 @@ __global__ __launch_bounds__(NT) void sample_parts_kernel(SampleArgs a, uint32_t
       const uint32_t bits = w & 0xffffu;
       k16 = (bits & 0x8000u) ? (~bits & 0xffffu) : (bits | 0x8000u);
     }
-    int dummy;
-    const uint32_t tk16 = radix_select<1, 8>(k, dummy, s, [&](int) { return k16 > 0; }, [&](int) { return k16; });
+    const uint32_t tk16 = select16_block(k, k16, s);
     const int keep = (k16 > 0 && k16 >= tk16) ? 1 : 0;
     int slot;
     const int n_keep = block_excl_scan_i(keep, slot, s);
@@ -1165,7 +1226,7 @@ __global__ __launch_bounds__(NT) void sample_parts_kernel(SampleArgs a, uint32_t
         s.skey[slot] = fkey(__uint_as_float((w & 0xffffu) << 16) / a.temperature);
         s.sid[slot] = (int)(w >> 16);
       }
-      token = draw_from_block(a, s, n_keep, k, u);
+      token = draw_from_block_call(a, s, n_keep, k, u);
     }
   }
   if (tid == 0) finish_row(a, b, token);
