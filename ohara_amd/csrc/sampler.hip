@@ -56,7 +56,7 @@ __device__ __forceinline__ uint32_t fkey(float f) {  // order-preserving: larger
 
 struct Smem {
   int hist[256];
-  int hist2[256];
+  int hist2[3][256];  // further counting tables of select16_block
   float wred[16];
   int wredi[16];
   uint32_t skey[CAP];
@@ -222,17 +222,17 @@ __device__ __forceinline__ uint32_t select_small(int want, int& n_greater, Smem&
 }
 
 // The `want`-th largest (1-based) of one 16-bit key per thread (0: the thread holds none), two counting
-// passes of 8 bits like radix_select<1, 8>, with fewer stops: both tables are cleared up front, and
-// one wave finds the digit of a pass (a lane adds up four bins, highest first, a DPP scan across the
-// lanes), so that a pass is two workgroup barriers.  Fewer than `want` keys: digit 0, as there.
-__device__ __forceinline__ uint32_t select16_block(int want, uint32_t key, Smem& s) {
+// passes of 8 bits like radix_select<1, 8>, with fewer stops: the two tables `t1`, `t2` were cleared by
+// the caller (select16_clear, behind a workgroup barrier), and one wave finds the digit of a pass (a
+// lane adds up four bins, highest first, a DPP scan across the lanes), so that a pass is two
+// workgroup barriers.  Fewer than `want` keys: digit 0, as there.
+__device__ __forceinline__ void select16_clear(Smem& s) {  // all four tables; a workgroup barrier must follow
+  const int tid = threadIdx.x;
+  if (tid < 256) s.hist[tid] = 0;
+  else s.hist2[(tid >> 8) - 1][tid & 255] = 0;
+}
+__device__ __forceinline__ uint32_t select16_block(int want, uint32_t key, Smem& s, int* t1, int* t2) {
   const int tid = threadIdx.x, lane = tid & 63;
-  __syncthreads();  // earlier users of the tables are done
-  if (tid < 256) {
-    s.hist[tid] = 0;
-    s.hist2[tid] = 0;
-  }
-  __syncthreads();
   auto find = [&](const int* h, int want_) {  // by wave 0: the bin that holds the want_-th largest, and the count above it
     const int b0 = 255 - 4 * lane;            // lane l owns bins 255 - 4l .. 252 - 4l
     const int c0 = h[b0], c1 = h[b0 - 1], c2 = h[b0 - 2], c3 = h[b0 - 3];
@@ -260,15 +260,15 @@ __device__ __forceinline__ uint32_t select16_block(int want, uint32_t key, Smem&
       s.misc[1] = incl - c3;
     }
   };
-  if (key) atomicAdd(&s.hist[key >> 8], 1);
+  if (key) atomicAdd(&t1[key >> 8], 1);
   __syncthreads();
-  if (tid < 64) find(s.hist, want);
+  if (tid < 64) find(t1, want);
   __syncthreads();
   const uint32_t d1 = (uint32_t)s.misc[0];
   const int above = s.misc[1];
-  if (key && (key >> 8) == d1) atomicAdd(&s.hist2[key & 255u], 1);
+  if (key && (key >> 8) == d1) atomicAdd(&t2[key & 255u], 1);
   __syncthreads();
-  if (tid < 64) find(s.hist2, want - above);
+  if (tid < 64) find(t2, want - above);
   __syncthreads();
   return (d1 << 8) | (uint32_t)s.misc[0];
 }
@@ -640,8 +640,12 @@ __device__ __forceinline__ int draw_from_wave_packed(const SampleArgs& a, Smem& 
                        __popcll(__ballot(lane + 64 < n_c && (w1 >> 16) >= tk));
     const float m0 = logit_of_key16((uint32_t)__builtin_amdgcn_readlane((int)w0, 0) >> 16, a.temperature);
     const float e0 = lane < n_kept ? expf(logit_of_key16(w0 >> 16, a.temperature) - m0) : 0.f;
-    const float e1 = lane + 64 < n_kept ? expf(logit_of_key16(w1 >> 16, a.temperature) - m0) : 0.f;
-    const float Z = wave_sum(e0) + wave_sum(e1);
+    float e1 = 0.f, z1 = 0.f;  // entries 64 .. 127: none in the usual case, and their sum is the +0 it would be
+    if (n_kept > 64) {
+      e1 = lane + 64 < n_kept ? expf(logit_of_key16(w1 >> 16, a.temperature) - m0) : 0.f;
+      z1 = wave_sum(e1);
+    }
+    const float Z = wave_sum(e0) + z1;
     uint32_t p0 = lane < n_kept ? __float_as_uint(e0 / Z) : 0u;  // probabilities in sorted order, +0 past the kept ones
     uint32_t p1 = lane + 64 < n_kept ? __float_as_uint(e1 / Z) : 0u;
     int i0 = 0xffff - (int)(w0 & 0xffffu), i1 = 0xffff - (int)(w1 & 0xffffu);
@@ -1144,6 +1148,9 @@ __global__ __launch_bounds__(NT) void sample_parts_kernel(SampleArgs a, uint32_t
   const int base = part * PART_IDS + tid * 8;
   const bf16_t* row = reinterpret_cast<const bf16_t*>(a.logits) + (size_t)b * a.ldl + base;
   const uint4 v = base < V ? ldg16(row) : make_uint4(0, 0, 0, 0);
+  static_assert(NT == 1024, "select16_clear: one thread per table entry");
+  select16_clear(s);  // the counting tables of both selections, while the load is in flight
+  __syncthreads();
   const uint32_t raw[4] = {v.x, v.y, v.z, v.w};
   auto bits16 = [&](int i) -> uint32_t { return (i & 1) ? (raw[i >> 1] >> 16) : (raw[i >> 1] & 0xffffu); };
   auto key16 = [&](int i) -> uint32_t {  // order-preserving 16-bit key of element i, 0 when masked
@@ -1160,7 +1167,7 @@ __global__ __launch_bounds__(NT) void sample_parts_kernel(SampleArgs a, uint32_t
   const int have = whole ? NT : block_sum_i(tmax > 0 ? 1 : 0, s);
   uint32_t bound = 1;  // fewer than k threads hold a valid id: every valid id of the part is a candidate
   if (have >= k) {
-    bound = select16_block(k, tmax, s);
+    bound = select16_block(k, tmax, s, s.hist, s.hist2[0]);
   }
   int c = 0;
 #pragma unroll
@@ -1212,7 +1219,7 @@ __global__ __launch_bounds__(NT) void sample_parts_kernel(SampleArgs a, uint32_t
       const uint32_t bits = w & 0xffffu;
       k16 = (bits & 0x8000u) ? (~bits & 0xffffu) : (bits | 0x8000u);
     }
-    const uint32_t tk16 = select16_block(k, k16, s);
+    const uint32_t tk16 = select16_block(k, k16, s, s.hist2[1], s.hist2[2]);
     const int keep = (k16 > 0 && k16 >= tk16) ? 1 : 0;
     int slot;
     const int n_keep = block_excl_scan_i(keep, slot, s);
