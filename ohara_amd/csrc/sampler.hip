@@ -1295,6 +1295,31 @@ __device__ __forceinline__ float key16_value(uint32_t key) {  // the bf16 value 
   return __uint_as_float(bits << 16);
 }
 
+// max of a, max of b and sum of c over the workgroup in one exchange (two barriers instead of six)
+__device__ __forceinline__ void block_max_max_sum_i(int& a, int& b, int& c, Smem& s) {
+  a = lanes_max<32, 1>(a);
+  b = lanes_max<32, 1>(b);
+  c = lanes_sum<32, 1>(c);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) {
+    s.wredi[w] = a;
+    s.hist[w] = b;
+    s.hist[NW + w] = c;
+  }
+  __syncthreads();
+  int ra = s.wredi[0], rb = s.hist[0], rc = s.hist[NW];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) {
+    ra = max(ra, s.wredi[i]);
+    rb = max(rb, s.hist[i]);
+    rc += s.hist[NW + i];
+  }
+  a = ra;
+  b = rb;
+  c = rc;
+}
+
 template <int EPT>
 __global__ __launch_bounds__(NT) void sample_hist_kernel(SampleArgs a) {
   extern __shared__ uint32_t hist[];  // HB dwords: key k counted in half (k & 1) of dword k >> 1; then the list
@@ -1306,25 +1331,34 @@ __global__ __launch_bounds__(NT) void sample_hist_kernel(SampleArgs a) {
   const float u = a.u[(a.step_state && a.u_step_stride > 0 ? (size_t)a.step_state[1] * a.u_step_stride : 0) + b];
   const bf16_t* row = reinterpret_cast<const bf16_t*>(a.logits) + (size_t)b * a.ldl + base;
   // One CU walks the whole row, so every instruction per id costs about half a microsecond.  The row
-  // is therefore not kept in registers (64 values per thread would spill): each pass re-reads its 16
-  // bytes per eight ids from the L2 and turns the two bf16 patterns of a register into order-preserving
+  // is not kept in registers between the passes: each pass re-reads its 16 bytes per eight ids from
+  // the L2 and turns the two bf16 patterns of a register into order-preserving
   // 16-bit keys with four integer instructions.  fn(id, key) is called for the thread's valid ids in
   // id order; key 0 cannot occur for a number (it is the pattern of one NaN) and is skipped.
+  // All loads of a pass go out before the first is used (addresses past the valid ids fall back on the
+  // chunk of the last valid id, whose values are not looked at): one round trip to the L2 per pass.
+  const bf16_t* row0 = reinterpret_cast<const bf16_t*>(a.logits) + (size_t)b * a.ldl;
+  const int last_chunk = nvalid > 0 ? ((nvalid - 1) & ~7) : 0;
   auto for_each_key = [&](auto&& fn) {
-#pragma unroll 2
+    uint4 vv[EPT / 8];
+#pragma unroll
+    for (int c = 0; c < EPT / 8; ++c) vv[c] = ldg16(row0 + min(base + 8 * c, last_chunk));
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
     for (int c = 0; c < EPT / 8; ++c) {
       const int id0 = base + 8 * c;
-      if (id0 >= nvalid) break;
-      const uint4 v = ldg16(row + 8 * c);
-      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-      const bool whole = id0 + 8 <= nvalid;
+      if (id0 < nvalid) {
+        const uint4 v = vv[c];
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        const bool whole = id0 + 8 <= nvalid;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint32_t neg = ((w[j] >> 15) & 0x00010001u) * 0xffffu;  // 0xffff in the halves that hold a negative value
-        const uint32_t kk = w[j] ^ (neg | 0x80008000u);                // negative: all bits flipped; else the sign bit set
-        const uint32_t klo = kk & 0xffffu, khi = kk >> 16;
-        if (klo && (whole || id0 + 2 * j < nvalid)) fn(id0 + 2 * j, klo);
-        if (khi && (whole || id0 + 2 * j + 1 < nvalid)) fn(id0 + 2 * j + 1, khi);
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t neg = ((w[j] >> 15) & 0x00010001u) * 0xffffu;  // 0xffff in the halves that hold a negative value
+          const uint32_t kk = w[j] ^ (neg | 0x80008000u);                // negative: all bits flipped; else the sign bit set
+          const uint32_t klo = kk & 0xffffu, khi = kk >> 16;
+          if (klo && (whole || id0 + 2 * j < nvalid)) fn(id0 + 2 * j, klo);
+          if (khi && (whole || id0 + 2 * j + 1 < nvalid)) fn(id0 + 2 * j + 1, khi);
+        }
       }
     }
   };
@@ -1332,7 +1366,8 @@ __global__ __launch_bounds__(NT) void sample_hist_kernel(SampleArgs a) {
   const bool nucleus = a.top_p > 0.f && a.top_p < 1.f;
   const bool want_table = a.top_k > 0 || nucleus;
   if (want_table) {
-    for (int i = tid; i < HB; i += NT) hist[i] = 0;
+    uint4* h4 = reinterpret_cast<uint4*>(hist);
+    for (int i = tid; i < HB / 4; i += NT) h4[i] = make_uint4(0, 0, 0, 0);
     __syncthreads();
   }
   int tmax = 0, tmin = 0x10000, live = 0;
@@ -1342,9 +1377,9 @@ __global__ __launch_bounds__(NT) void sample_hist_kernel(SampleArgs a) {
     ++live;
     if (want_table) atomicAdd(&hist[kk >> 1], (kk & 1u) ? 0x10000u : 1u);
   });
-  const int kmax = block_max_i(tmax, s);
-  const int kmin = -block_max_i(-tmin, s);
-  const int n_live = block_sum_i(live, s);  // (the syncs inside also complete the table)
+  int kmax = tmax, nkmin = -tmin, n_live = live;
+  block_max_max_sum_i(kmax, nkmin, n_live, s);  // (the barriers inside also complete the table)
+  const int kmin = -nkmin;
   int token = 0;
   if (kmax > 0) {
     const float m = xval((uint32_t)kmax);
@@ -1360,11 +1395,13 @@ __global__ __launch_bounds__(NT) void sample_hist_kernel(SampleArgs a) {
     int n_ent = 1;
     if (need_table) {
       const uint4* seg = reinterpret_cast<const uint4*>(hist + HB - 32 * (tid + 1));  // my 64 keys, ascending
+      uint4 sv[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) sv[q] = seg[q];
       int nz = 0;
-#pragma unroll 2
+#pragma unroll
       for (int q = 0; q < 8; ++q) {
-        const uint4 v = seg[q];
-        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        const uint32_t w[4] = {sv[q].x, sv[q].y, sv[q].z, sv[q].w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) nz += ((w[i] >> 16) ? 1 : 0) + ((w[i] & 0xffffu) ? 1 : 0);
       }
@@ -1372,10 +1409,9 @@ __global__ __launch_bounds__(NT) void sample_hist_kernel(SampleArgs a) {
       n_ent = block_excl_scan_i(nz, off, s);
       if (n_ent <= ENT_CAP && nz) {
         const int kbase = 65536 - 64 * (tid + 1);  // key of the low half of seg[0].x
-#pragma unroll 1
+#pragma unroll
         for (int q = 7; q >= 0; --q) {
-          const uint4 v = seg[q];
-          const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+          const uint32_t w[4] = {sv[q].x, sv[q].y, sv[q].z, sv[q].w};
 #pragma unroll
           for (int i = 3; i >= 0; --i) {
             const int key = kbase + 8 * q + 2 * i;
@@ -1526,21 +1562,41 @@ __global__ __launch_bounds__(NT) void sample_hist_kernel(SampleArgs a) {
       __syncthreads();
       const uint32_t Td = (uint32_t)s.misc[7];
       const int r = s.misc[3];
-      // the r-th id, in id order, among the ids with key Td
-      int c = 0;
-      for_each_key([&](int, uint32_t kk) { c += kk == Td ? 1 : 0; });
+      // the r-th id, in id order, among the ids with key Td: one pass notes where in the thread's ids
+      // the key occurs (the bf16 pattern behind the key is compared as loaded: two instructions an id,
+      // on a CU that spends 0.44 us on every instruction per id), the thread that owns the r-th
+      // occurrence picks it from its own notes
+      unsigned long long where = 0;
+      {
+        const uint32_t pat = (Td & 0x8000u) ? (Td & 0x7fffu) : (~Td & 0xffffu);  // key -> bf16 bits
+        const uint32_t pat2 = pat | (pat << 16);
+        uint4 vv[EPT / 8];
+#pragma unroll
+        for (int c = 0; c < EPT / 8; ++c) vv[c] = ldg16(row0 + min(base + 8 * c, last_chunk));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < EPT / 8; ++c) {
+          const uint32_t w[4] = {vv[c].x, vv[c].y, vv[c].z, vv[c].w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const uint32_t x = w[j] ^ pat2;
+            if ((x & 0xffffu) == 0) where |= 1ull << (8 * c + 2 * j);
+            if ((x >> 16) == 0) where |= 1ull << (8 * c + 2 * j + 1);
+          }
+        }
+        // ids at or past the end of the valid ones (and the chunks that stood in for them) do not count
+        const int nv = nvalid - base;
+        where = nv >= EPT ? where : (nv <= 0 ? 0ull : where & ((1ull << nv) - 1ull));
+      }
+      static_assert(EPT <= 64, "one bit per id of the thread");
+      const int c = __popcll(where);
       int off;
       block_excl_scan_i(c, off, s);
       if (tid == 0) s.misc[2] = -1;
       __syncthreads();
       if (c > 0 && off <= r && r < off + c) {
-        int seen = off;
-        for_each_key([&](int id, uint32_t kk) {
-          if (kk == Td) {
-            if (seen == r) s.misc[2] = id;
-            ++seen;
-          }
-        });
+        for (int skip = r - off; skip > 0; --skip) where &= where - 1;  // drop the occurrences before the r-th
+        s.misc[2] = base + __ffsll((long long)where) - 1;
       }
       __syncthreads();
       token = max(s.misc[2], 0);
