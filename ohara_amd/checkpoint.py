@@ -115,6 +115,15 @@ def loop_moe_to_grouped(state: Mapping[str, torch.Tensor]) -> dict[str, torch.Te
     return out
 
 
+def loop_moe_config(config: Config) -> Config:
+    """The grouped-form config that computes what ``MoE`` (ohara/modules/moe.py:65-98) computes for a
+    config with ``moe_grouped=False``: no shared expert and sigmoid weights left as they are (the loop
+    form has neither, llama.py:171-178 passes neither)."""
+    from dataclasses import replace
+
+    return replace(config, moe_grouped=True, moe_num_shared_experts=0, moe_normalize_weights=False)
+
+
 def load_checkpoint(path, *, moe_experts_per_tok: int = 2, moe_gate_fn: str = "softmax",
                     moe_normalize_weights: bool = True):
     """-> (Config, state dict).  ``path`` is a ``.pt`` file holding a state dict (bare or under
@@ -151,12 +160,10 @@ def load_checkpoint(path, *, moe_experts_per_tok: int = 2, moe_gate_fn: str = "s
 def build_model(config: Config, state: Mapping[str, torch.Tensor], device="cuda"):
     """The kernel-backed model for a config: dense ``Llama`` or ``MoeLlama``."""
     if config.moe_num_experts > 0:
-        from dataclasses import replace
-
         from .moe import MoeLlama
 
         if not config.moe_grouped:
-            state, config = loop_moe_to_grouped(state), replace(config, moe_grouped=True)
+            state, config = loop_moe_to_grouped(state), loop_moe_config(config)
         return MoeLlama(config, state, device=device)
     from .llama import Llama
 

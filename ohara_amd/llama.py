@@ -219,11 +219,14 @@ class Llama:
         if cls is Llama and getattr(config, "moe_num_experts", 0) > 0:
             if dtype != BF16:
                 raise ValueError("ohara_amd runs the decode path in bfloat16 only")
-            if not config.moe_grouped:
-                raise NotImplementedError("ohara_amd serves MoE layers in the grouped form only (moe_grouped=True, "
-                                          "ohara/modules/moe_grouped.py); the per-expert loop of llama.py:171-178 is not built")
             from .moe import MoeLlama
 
+            if not config.moe_grouped:
+                # the per-expert loop of llama.py:171-178 (ohara/modules/moe.py) computes the function of the
+                # grouped form without shared experts: its weights are restacked and served by the same kernels
+                from .checkpoint import loop_moe_config, loop_moe_to_grouped
+
+                return MoeLlama(loop_moe_config(config), loop_moe_to_grouped(state or {}), device=device)
             return MoeLlama(config, state, device=device)
         return super().__new__(cls)
 

@@ -127,3 +127,41 @@ def test_moe_llama_decode_at_larger_batches(cuda, B):
     close(model(ids[:, :4].to(cuda), cache, 0), ref(ids[:, :4], rc, 0))
     for t in (4, 5, 6):
         close(model(ids[:, t:t + 1].to(cuda), cache, t), ref(ids[:, t:t + 1], rc, t))
+
+
+def test_loop_form_moe_config_is_served(cuda):
+    """``Llama(Config(moe_grouped=False, ...))`` - the per-expert loop of ohara/models/llama.py:171-178,
+    state dict in the layout of ohara/modules/moe.py:51-52 (``ff.experts.N.{gate,up,down}``, router
+    ``ff.gate``) - against the oracle's grouped form without shared expert and with sigmoid weights left
+    unnormalised (the function the loop form computes), and bit for bit against the grouped-form model
+    built from the same weights."""
+    from ohara_amd.llama import Config, Llama
+    from ohara_amd.moe import MoeLlama
+
+    kw = dict(vocab_size=256, hidden_size=128, intermediate_size=64, num_attention_heads=2, num_key_value_heads=0,
+              num_hidden_layers=2, max_sequence_length=32, dropout=0.0, moe_num_experts=8, moe_experts_per_tok=2,
+              moe_layer_interval=1, moe_num_shared_experts=0, moe_gate_fn="sigmoid", moe_normalize_weights=False)
+    rcfg = R.RefConfig(**kw, moe_grouped=True)
+    w = R.init_weights(rcfg, seed=11, dtype=BF, std=0.06, norm_jitter=0.1)
+    loop = {k: v for k, v in w.items() if ".ff.w_" not in k and ".ff.router.weight" not in k}
+    for l in range(2):
+        p = f"layers.{l}.ff."
+        for e in range(8):
+            loop[f"{p}experts.{e}.gate.weight"] = w[p + "w_gate"][e].t().contiguous()
+            loop[f"{p}experts.{e}.up.weight"] = w[p + "w_up"][e].t().contiguous()
+            loop[f"{p}experts.{e}.down.weight"] = w[p + "w_down"][e].t().contiguous()
+        loop[p + "gate.weight"] = w[p + "router.weight"]
+    # the loop form knows no normalisation flag: the default (True) of the config must not leak in
+    model = Llama(Config(**{**kw, "moe_normalize_weights": True}, moe_grouped=False), loop, device=cuda)
+    assert isinstance(model, MoeLlama)
+    twin = MoeLlama(Config(**kw, moe_grouped=True), w, device=cuda)
+    ref = R.RefLlama(rcfg, w)
+    ids = torch.randint(0, 256, (3, 6), generator=torch.Generator().manual_seed(4))
+    c1, c2, rc = model.build_kv_cache(3), twin.build_kv_cache(3), ref.build_kv_cache(3)
+    for t0, t1 in ((0, 4), (4, 5), (5, 6)):
+        got = model(ids[:, t0:t1].to(cuda), c1, t0)
+        assert torch.equal(got, twin(ids[:, t0:t1].to(cuda), c2, t0))
+        want = ref(ids[:, t0:t1], rc, t0).float()
+        scale = want.abs().max().item()
+        row_err = (got.float().cpu() - want).abs().amax(-1).reshape(-1)
+        assert (row_err <= 4e-2 * scale).float().mean().item() >= 0.9

@@ -235,8 +235,18 @@ def test_config_and_kv_cache_bookkeeping():
 
     with pytest.raises(ValueError, match="biases"):
         Llama(Config(bias=True), {})
-    with pytest.raises(NotImplementedError, match="grouped"):
-        Llama(Config(moe_num_experts=4, moe_grouped=False), {})
+    # a loop-form MoE config (llama.py:171-178) is served by the grouped kernels: no shared expert, sigmoid
+    # weights as they are, expert weights restacked as (E, dim, hidden) / (E, hidden, dim)
+    from ohara_amd.checkpoint import loop_moe_config, loop_moe_to_grouped
+
+    lc = loop_moe_config(Config(moe_num_experts=4, moe_grouped=False, moe_num_shared_experts=2))
+    assert lc.moe_grouped and lc.moe_num_shared_experts == 0 and not lc.moe_normalize_weights
+    st = {f"layers.0.ff.experts.{e}.{n}.weight": torch.full((3, 2) if n != "down" else (2, 3), float(e))
+          for e in range(4) for n in ("gate", "up", "down")}
+    st["layers.0.ff.gate.weight"] = torch.zeros(4, 2)
+    g = loop_moe_to_grouped(st)
+    assert g["layers.0.ff.w_gate"].shape == (4, 2, 3) and g["layers.0.ff.w_down"].shape == (4, 3, 2)
+    assert g["layers.0.ff.w_up"][2].eq(2.0).all() and "layers.0.ff.router.weight" in g and "layers.0.ff.gate.weight" not in g
     with pytest.raises(ValueError, match="bfloat16"):
         Llama(Config(), {}, dtype=torch.float16)
     c = KVCache((2, 8, 2, 4), 8, dtype=torch.float32)
