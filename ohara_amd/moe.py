@@ -161,12 +161,13 @@ class MoeLlama:
     def to(self, *a, **k):
         return self
 
-    def build_kv_cache(self, batch_size: int = 1):
+    def build_kv_cache(self, batch_size: int = 1, int8: bool = False):
+        """ohara/models/llama.py:325-348; ``int8=True`` builds the int8 caches of kv_cache.py:15-32."""
         if batch_size < 1:
             raise ValueError("batch_size must be at least 1")
         c = self.config
         shape = (batch_size, c.max_sequence_length, self.kv_heads, self.head_dim)
-        return [KVCache(shape, c.max_sequence_length, i, device=self.device, dtype=BF16)
+        return [KVCache(shape, c.max_sequence_length, i, device=self.device, dtype=BF16, int8=int8)
                 for i in range(c.num_hidden_layers)]
 
     @torch.no_grad()
@@ -194,8 +195,9 @@ class MoeLlama:
             raise ValueError("input exceeds max_sequence_length")
         if kv_cache is None:
             kv_cache = self.build_kv_cache(B)
-        if any(cc.int8 for cc in kv_cache):
-            raise NotImplementedError("ohara_amd: int8 KV caches are served by the dense Llama only")
+        if len({cc.int8 for cc in kv_cache}) > 1:
+            raise ValueError("all layers must use the same KV cache mode")
+        int8 = kv_cache[0].int8
         ends = [cc._reserve(B, S, start) for cc in kv_cache]
         H, Hkv, D = c.num_attention_heads, self.kv_heads, self.head_dim
         n_split = 1 if S > 1 else max(1, min(1024 // max(1, B * Hkv), c.max_sequence_length // 128, 64))
@@ -204,9 +206,22 @@ class MoeLlama:
             ws = self._ws[(B, n_split)] = ops.attn_workspace(B, H, Hkv, D, n_split, self.device)
         h = ops.embed(x.to(self.device), self.token_emb)
         for L, cache in zip(self.layers, kv_cache):
-            q = ops.qkv_rope_append(h, L["wqkv"], L["norm1"], self.eps, H, Hkv, D, self.cos, self.sin, start,
-                                    cache.key, cache.value, seq_len=S)
-            att = ops.attn_auto(q, cache.key, cache.value, H, Hkv, D, start, n_split, ws, S)
+            if int8:
+                # kv_cache.py:94-118 with quantisation: the new rows go in as codes, attention reads what
+                # the reference's cache read returns (the dequantised prefix, the new rows included);
+                # many new positions per sequence attend over a dequantised copy of the live prefix
+                q, k, v = ops.qkv_rope(h, L["wqkv"], L["norm1"], self.eps, H, Hkv, D, self.cos, self.sin, start,
+                                       c.max_sequence_length, seq_len=S)
+                ops.kv_quant_append(k.view(B, S, Hkv, D), v.view(B, S, Hkv, D), cache, start)
+                if S >= 16 and D in (64, 128):
+                    att = ops.attn_prefill(q, ops.kv_dequant(cache, "key", B, start + S),
+                                           ops.kv_dequant(cache, "value", B, start + S), H, Hkv, D, start, S)
+                else:
+                    att = ops.attn_cached_int8(q, cache, H, Hkv, D, start, n_split, ws, seq_len=S)
+            else:
+                q = ops.qkv_rope_append(h, L["wqkv"], L["norm1"], self.eps, H, Hkv, D, self.cos, self.sin, start,
+                                        cache.key, cache.value, seq_len=S)
+                att = ops.attn_auto(q, cache.key, cache.value, H, Hkv, D, start, n_split, ws, S)
             h = ops.gemm_skinny(att, L["wo"], residual=h)
             if "moe" in L:
                 h = L["moe"].forward_rows(ops.rmsnorm(h, L["norm2"], self.eps), residual=h)
