@@ -50,10 +50,44 @@ int ohara_launch_gemm_tile(const GemmArgs& a, int epi, int packed_rows, hipStrea
 
 namespace {
 
+// What an epilogue reads besides the accumulators, fetched ahead: a kernel that finishes many fragments
+// per thread (the tiled GEMM: sixteen) issues the loads of all of them before the first is used instead of
+// one dependent round trip per fragment.  gemm_epilogue_fetch requires N, ldo, ldr, ldr2 to be multiples
+// of 4 (the caller checks once); fragments and rows outside the matrix read clamped addresses and are
+// never finished.
+struct EpiPre {
+  uint2 r1, r2, bv;  // residual rows, bias
+  uint32_t c, s;     // two cos and two sin values of the rotary table
+  int pos;
+};
+template <int EPI>
+__device__ __forceinline__ void gemm_epilogue_fetch(const GemmArgs& a, int b, int strip, int g, EpiPre& p) {
+  const int r0 = min(strip * 16 + 4 * g, a.N - 4);
+  const int bc = min(b, a.B - 1);
+  if (EPI == EPI_RESIDUAL) p.r1 = *reinterpret_cast<const uint2*>(a.resid + (size_t)bc * a.ldr + r0);
+  if (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU || EPI == EPI_BIAS_ADD2 || EPI == EPI_PHI_IN)
+    p.bv = *reinterpret_cast<const uint2*>(a.bias + r0);
+  if (EPI == EPI_BIAS_ADD2) {
+    p.r1 = *reinterpret_cast<const uint2*>(a.resid + (size_t)bc * a.ldr + r0);
+    p.r2 = *reinterpret_cast<const uint2*>(a.resid2 + (size_t)bc * a.ldr2 + r0);
+  }
+  if (EPI == EPI_ROPE) {
+    const int grow = a.row0 + bc;
+    const int seq = grow / a.S;
+    p.pos = (a.pos_dev ? a.pos_dev[(size_t)seq * a.pos_stride] : a.pos) + (grow - seq * a.S);
+    const int nq = a.H * a.Dh;
+    const int rr = strip * 16 + 4 * g;
+    const int d = (rr < nq ? rr : rr - nq) % a.Dh;
+    const int pc = min(max(p.pos, 0), a.Tmax - 1);
+    p.c = *reinterpret_cast<const uint32_t*>(a.cos + (size_t)pc * (a.Dh >> 1) + (d >> 1));
+    p.s = *reinterpret_cast<const uint32_t*>(a.sin + (size_t)pc * (a.Dh >> 1) + (d >> 1));
+  }
+}
+
 // One MFMA output fragment: the four consecutive packed rows 16*strip + 4*g .. +3 of activation
 // row b (relative to a.out / a.resid; global row a.row0 + b for the rotary epilogue).
-template <int EPI>
-__device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, int b, int strip, int g, f32x4 acc) {
+template <int EPI, bool PRE = false>  // PRE: the operands were fetched ahead into `p`
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, int b, int strip, int g, f32x4 acc, const EpiPre& p = EpiPre{}) {
   const int r0 = strip * 16 + 4 * g;
   const float y0 = rbf(acc[0]), y1 = rbf(acc[1]), y2 = rbf(acc[2]), y3 = rbf(acc[3]);
   if (EPI == EPI_STORE || EPI == EPI_RESIDUAL) {
@@ -62,7 +96,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, int b, int stri
     if (EPI == EPI_RESIDUAL) {
       const bf16_t* r = a.resid + (size_t)b * a.ldr + r0;
       if (r0 + 3 < a.N && ((a.ldr & 3) == 0)) {
-        const uint2 rv = *reinterpret_cast<const uint2*>(r);
+        const uint2 rv = PRE ? p.r1 : *reinterpret_cast<const uint2*>(r);
         v[0] = lo_bf(rv.x) + v[0]; v[1] = hi_bf(rv.x) + v[1]; v[2] = lo_bf(rv.y) + v[2]; v[3] = hi_bf(rv.y) + v[3];
       } else {
 #pragma unroll
@@ -80,7 +114,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, int b, int stri
   } else if (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU || EPI == EPI_BIAS_ADD2) {
     // N % 4 == 0 and 4-element aligned leading dimensions are required by the entry point
     if (r0 >= a.N) return;
-    const uint2 bv = *reinterpret_cast<const uint2*>(a.bias + r0);
+    const uint2 bv = PRE ? p.bv : *reinterpret_cast<const uint2*>(a.bias + r0);
     float v[4] = {rbf(acc[0] + lo_bf(bv.x)), rbf(acc[1] + hi_bf(bv.x)), rbf(acc[2] + lo_bf(bv.y)),
                   rbf(acc[3] + hi_bf(bv.y))};
     if (EPI == EPI_BIAS_GELU) {
@@ -94,8 +128,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, int b, int stri
         v[i] = rbf(0.5f * x) * t5;
       }
     } else if (EPI == EPI_BIAS_ADD2) {
-      const uint2 r1 = *reinterpret_cast<const uint2*>(a.resid + (size_t)b * a.ldr + r0);
-      const uint2 r2 = *reinterpret_cast<const uint2*>(a.resid2 + (size_t)b * a.ldr2 + r0);
+      const uint2 r1 = PRE ? p.r1 : *reinterpret_cast<const uint2*>(a.resid + (size_t)b * a.ldr + r0);
+      const uint2 r2 = PRE ? p.r2 : *reinterpret_cast<const uint2*>(a.resid2 + (size_t)b * a.ldr2 + r0);
       v[0] = rbf(lo_bf(r1.x) + v[0]) + lo_bf(r2.x);
       v[1] = rbf(hi_bf(r1.x) + v[1]) + hi_bf(r2.x);
       v[2] = rbf(lo_bf(r1.y) + v[2]) + lo_bf(r2.y);
@@ -104,7 +138,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, int b, int stri
     *reinterpret_cast<uint2*>(a.out + (size_t)b * a.ldo + r0) = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
   } else if (EPI == EPI_PHI_IN) {
     if (r0 >= a.N) return;
-    const uint2 bv = *reinterpret_cast<const uint2*>(a.bias + r0);
+    const uint2 bv = PRE ? p.bv : *reinterpret_cast<const uint2*>(a.bias + r0);
     float v[4] = {rbf(acc[0] + lo_bf(bv.x)), rbf(acc[1] + hi_bf(bv.x)), rbf(acc[2] + lo_bf(bv.y)),
                   rbf(acc[3] + hi_bf(bv.y))};
     const int grow = a.row0 + b;
@@ -145,7 +179,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, int b, int stri
   } else {  // EPI_ROPE: rows [q (H*Dh); k (Hkv*Dh); v (Hkv*Dh)], one position per sequence
     const int grow = a.row0 + b;
     const int seq = grow / a.S;
-    const int pos = (a.pos_dev ? a.pos_dev[(size_t)seq * a.pos_stride] : a.pos) + (grow - seq * a.S);
+    const int pos = PRE ? p.pos : (a.pos_dev ? a.pos_dev[(size_t)seq * a.pos_stride] : a.pos) + (grow - seq * a.S);
     const int nq = a.H * a.Dh, nk = a.Hkv * a.Dh;
     if (r0 >= nq + 2 * nk || pos < 0 || pos >= a.Tmax) return;
     float v[4] = {y0, y1, y2, y3};
@@ -156,7 +190,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& a, int b, int stri
       const bf16_t* sn = a.sin + (size_t)pos * (a.Dh >> 1) + (d >> 1);
 #pragma unroll
       for (int pr = 0; pr < 2; ++pr) {
-        const float c = bf2f(cs[pr]), s = bf2f(sn[pr]);
+        const float c = PRE ? (pr ? hi_bf(p.c) : lo_bf(p.c)) : bf2f(cs[pr]), s = PRE ? (pr ? hi_bf(p.s) : lo_bf(p.s)) : bf2f(sn[pr]);
         const float e = v[2 * pr], od = v[2 * pr + 1];
         // separate fp32 multiplies and add/sub, as the reference's eager ops round
         v[2 * pr] = __fsub_rn(__fmul_rn(e, c), __fmul_rn(od, s));

@@ -110,6 +110,27 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(GemmArgs a, int MT, i
     __syncthreads();
   }
 
+  // A thread finishes sixteen fragments.  What their epilogues read (residual rows, biases, rotary
+  // values) is fetched for eight of them before the first is used, instead of one dependent round trip
+  // per fragment.
+  constexpr bool READS = EPI == EPI_RESIDUAL || EPI == EPI_ROPE || EPI == EPI_BIAS || EPI == EPI_BIAS_GELU ||
+                         EPI == EPI_BIAS_ADD2 || EPI == EPI_PHI_IN;
+  if (READS && a.N >= 4 && ((a.N | a.ldo | a.ldr | (EPI == EPI_BIAS_ADD2 ? a.ldr2 : 0)) & 3) == 0) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {  // eight fragments at a time: sixteen sets of operands cost a resident workgroup
+      EpiPre pre[8];
+#pragma unroll
+      for (int t = 0; t < 8; ++t) gemm_epilogue_fetch<EPI>(a, row0 + t * 16 + m, min(strip0 + u, nstrips - 1), g, pre[t]);
+      __builtin_amdgcn_sched_barrier(0);
+      if (strip0 + u >= nstrips) continue;
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const int b = row0 + t * 16 + m;
+        if (b < a.B) gemm_epilogue<EPI, true>(a, b, strip0 + u, g, acc[u][t], pre[t]);
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     if (strip0 + u >= nstrips) continue;
