@@ -400,8 +400,8 @@ int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* s, int seq_
 /* ---- one decode step as ONE persistent launch (batch <= 16) ------------------------
  * Same result as ohara_llama_forward(seq_len = 1, use_pos_dev = 1, LOGITS_LAST) but the
  * whole step (all layers, vocabulary projection, greedy selection) runs in a single
- * kernel of `n_workgroups` resident workgroups (use the CU count) separated by
- * grid-wide barriers; it has no counterpart in the reference, whose decode step is
+ * kernel of `n_workgroups` resident workgroups (use the CU count; more than the device can
+ * hold of this kernel at once returns OHARA_ESIZE) separated by grid-wide barriers; it has no counterpart in the reference, whose decode step is
  * ~1000 eager launches (llama.py:279-323).  The cache position and step index are read
  * from / advanced in s->step_state; s->attn and s->attn_ws are not used.
  * `workspace`: ohara_persistent_workspace_bytes(m, batch, s->n_split, n_workgroups) of

@@ -1149,6 +1149,9 @@ int ohara_bitnet_decode_persistent(const OharaBitModel* m, const OharaDecodeStat
     if (smem > 64 * 1024)                                                                                    \
       (void)hipFuncSetAttribute((const void*)bitnet_mega_kernel<DD, 1, ONE_>,                                \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);                      \
+    static ResidencySlot slot;                                                                               \
+    if (!ohara_grid_fits(slot, (const void*)bitnet_mega_kernel<DD, 1, ONE_>, smem, n_workgroups))            \
+      return OHARA_ESIZE; /* the workgroups could not all be resident: the grid barrier would expire */      \
     hipLaunchKernelGGL((bitnet_mega_kernel<DD, 1, ONE_>), grid, block, smem, st, a);                         \
   } while (0)
 #define OHARA_BITMEGA(DD)                                                                                    \
@@ -1161,6 +1164,9 @@ int ohara_bitnet_decode_persistent(const OharaBitModel* m, const OharaDecodeStat
     if (smem > 64 * 1024)                                                                                    \
       (void)hipFuncSetAttribute((const void*)bitnet_mega_kernel<128, 1, ONE_, true>,                         \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);                      \
+    static ResidencySlot slot;                                                                               \
+    if (!ohara_grid_fits(slot, (const void*)bitnet_mega_kernel<128, 1, ONE_, true>, smem, n_workgroups))     \
+      return OHARA_ESIZE;                                                                                    \
     hipLaunchKernelGGL((bitnet_mega_kernel<128, 1, ONE_, true>), grid, block, smem, st, a);                  \
   } while (0)
   if (a.prof && D == 128) {  // the stamps exist in these two instantiations only

@@ -408,6 +408,9 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
     if (smem > 64 * 1024)                                                                                   \
       (void)hipFuncSetAttribute((const void*)decode_mega_kernel<DD, GG, ONE_>,                              \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);                     \
+    static ResidencySlot slot;                                                                              \
+    if (!ohara_grid_fits(slot, (const void*)decode_mega_kernel<DD, GG, ONE_>, smem, n_workgroups))          \
+      return OHARA_ESIZE; /* the workgroups could not all be resident: the grid barrier would expire */     \
     hipLaunchKernelGGL((decode_mega_kernel<DD, GG, ONE_>), grid, block, smem, st, a);                       \
   } while (0)
 #define OHARA_MEGA(DD, GG)                                                                                  \
@@ -420,6 +423,9 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
     if (smem > 64 * 1024)                                                                                   \
       (void)hipFuncSetAttribute((const void*)decode_mega_kernel<128, 1, ONE_, true>,                        \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);                     \
+    static ResidencySlot slot;                                                                              \
+    if (!ohara_grid_fits(slot, (const void*)decode_mega_kernel<128, 1, ONE_, true>, smem, n_workgroups))    \
+      return OHARA_ESIZE;                                                                                   \
     hipLaunchKernelGGL((decode_mega_kernel<128, 1, ONE_, true>), grid, block, smem, st, a);                 \
   } while (0)
   if (a.prof && D == 128 && G == 1) {  // the stamps exist in these two instantiations only

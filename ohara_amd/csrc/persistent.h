@@ -5,6 +5,29 @@
 #pragma once
 #include "common.h"
 
+// Host side: can `n_workgroups` workgroups of `kernel` (256 threads, `smem` bytes of dynamic LDS) be
+// resident on the current device at the same time?  The grid barrier of the persistent kernels needs
+// that: a workgroup that is not dispatched until another one exits would be waited for until the
+// spin limit expires.  The answer per (kernel, smem) is cached in `slot` (one per launch site).
+struct ResidencySlot {
+  const void* kernel = nullptr;
+  size_t smem = 0;
+  int max_workgroups = 0;
+};
+inline bool ohara_grid_fits(ResidencySlot& slot, const void* kernel, size_t smem, int n_workgroups) {
+  if (slot.kernel != kernel || slot.smem != smem) {
+    int dev = 0, cus = 0, per_cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, smem) != hipSuccess)
+      return false;
+    slot.kernel = kernel;
+    slot.smem = smem;
+    slot.max_workgroups = cus * per_cu;
+  }
+  return n_workgroups <= slot.max_workgroups;
+}
+
 namespace {
 
 

@@ -457,6 +457,38 @@ def test_expired_barrier_wait_is_reported_and_does_not_hang(cuda):
     assert torch.equal(again, good)
 
 
+def test_persistent_launch_refuses_more_workgroups_than_can_be_resident(cuda):
+    """The grid barrier needs every workgroup resident at once: a launch with more workgroups than
+    the device holds of this kernel (one per CU) is refused with OHARA_ESIZE before anything runs,
+    instead of running into the barrier's spin limit."""
+    import ctypes as C
+
+    from ohara_amd._lib import lib
+    from ohara_amd.llama import Config, Llama
+
+    kw = dict(vocab_size=512, hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+              num_hidden_layers=2, max_sequence_length=64, rope_theta=10000.0)
+    w = R.init_weights(R.RefConfig(**kw), seed=5, dtype=torch.bfloat16, std=0.06, norm_jitter=0.1)
+    model = Llama(Config(**kw), w, device=cuda)
+    if not model.supports_persistent(1):
+        pytest.skip("shape not covered by the persistent kernel")
+    sess = model.session(1, 8, persistent=True)
+    sess.prefill(torch.randint(0, 512, (1, 6), generator=torch.Generator().manual_seed(0)).to(cuda))
+    too_many = sess._nwg + 1
+    need = lib().ohara_persistent_workspace_bytes(C.byref(model._c_model), 1, sess.PERSISTENT_SPLITS, too_many)
+    ws = torch.zeros(max(need, 1), dtype=torch.uint8, device=cuda)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert lib().ohara_llama_decode_persistent(C.byref(model._c_model), C.byref(sess._dst), ws.data_ptr(), too_many, 1, 1,
+                                               0, stream) == 0  # workspace set-up alone launches nothing
+    rc = lib().ohara_llama_decode_persistent(C.byref(model._c_model), C.byref(sess._dst), ws.data_ptr(), too_many, 0, 1,
+                                             0, stream)
+    assert rc == -3, rc
+    torch.cuda.synchronize()
+    sess.step()  # the session itself is untouched
+    torch.cuda.synchronize()
+    sess.check_error()
+
+
 @pytest.mark.parametrize("B", [9, 17, 33, 70, 130])
 def test_decode_batches_between_and_beyond_the_tuned_sizes(cuda, B):
     """Batches that are not multiples of 16, and more rows than one strip-kernel launch takes (64):
