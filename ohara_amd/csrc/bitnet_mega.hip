@@ -280,6 +280,37 @@ __device__ __forceinline__ void bit_stage_row1(const BitLds& L, int nsets, int K
   if (tid < nsets) L.s_sum[tid * 16] = (L.sumw[tid * 4] + L.sumw[tid * 4 + 1]) + (L.sumw[tid * 4 + 2] + L.sumw[tid * 4 + 3]);
   // the product that follows passes a workgroup barrier before anyone reads s_sum
 }
+// The norm weights of a row's staging (block norm `pre_w`, the BitLinears' own norms `nw0` / `nw1`) do not
+// depend on the phase before it: row1_norm_fetch issues their loads - in the barrier window, next to the
+// phase's weight prefetch, where a cold HBM read costs nothing - and bit_stage_row1_pre takes them from
+// registers.  Pieces past the row read the last piece and multiply values that are zero.
+template <int NP>
+__device__ __forceinline__ void row1_norm_fetch(uint4 (&r)[NP], int pieces, const bf16_t* w) {
+#pragma unroll
+  for (int i = 0; i < NP; ++i) r[i] = ldg16(w + (size_t)min((int)threadIdx.x + 256 * i, pieces - 1) * 8);
+}
+template <int NP, typename Load>
+__device__ __forceinline__ void bit_stage_row1_pre(const BitLds& L, int nsets, int K, bool block_norm, const uint4 (&pw)[NP],
+                                                   const uint4 (&n0)[NP], const uint4 (&n1)[NP], float eps, Load load) {
+  const int tid = threadIdx.x;
+  const int pieces = K >> 3;
+  uint4 x[NP];
+  row1_load(x, pieces, load);
+  __syncthreads();  // whoever still reads the previous codes or scales is done
+  {
+    const int pad8 = (L.ldq - K) >> 3;
+    for (int i = tid; i < nsets * pad8; i += 256) {
+      const int st = i / pad8, c = i - st * pad8;
+      sts8(L.codes + (size_t)st * L.set + K + c * 8, make_uint2(0, 0));
+    }
+  }
+  if (block_norm) row1_block_norm(x, pw, K, eps, L.red);
+  row1_codes(x, n0, pieces, K, eps, L.codes, L.red, L.s_s, L.sumw);
+  if (nsets == 2) row1_codes(x, n1, pieces, K, eps, L.codes + L.set, L.red, L.s_s + 16, L.sumw + 4);
+  __syncthreads();
+  if (tid < nsets) L.s_sum[tid * 16] = (L.sumw[tid * 4] + L.sumw[tid * 4 + 1]) + (L.sumw[tid * 4 + 2] + L.sumw[tid * 4 + 3]);
+  // the product that follows passes a workgroup barrier before anyone reads s_sum
+}
 
 // ---- batch > 1: a row per wave, in registers ---------------------------------------------------
 // Lane l owns the pieces l, l + 64, ... (NP of them); the norm weights are fetched once per wave and
@@ -694,6 +725,13 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
     rope_s = ldg4(m.sin + (size_t)pos * (D >> 1) + (dd >> 1));
   }
   bit_prefetch<2>(reinterpret_cast<const uint4*>(gptr(ltab[0].w[p1_which])), KCd, p1_strip0, 0, KCd, p1_strip0 < p1_nstr, wpre);
+  // batch-1 build: the norm weights of the next phase's staging, fetched in the barrier windows
+  uint4 npw[1], nn0[3], nn1[1];
+  npw[0] = nn0[0] = nn0[1] = nn0[2] = nn1[0] = make_uint4(0, 0, 0, 0);
+  if (ONE && 2 * p1_gi < p1_nstr) {
+    row1_norm_fetch<1>(npw, d >> 3, reinterpret_cast<const bf16_t*>(gptr(ltab[0].norm1)));
+    row1_norm_fetch<1>(reinterpret_cast<uint4(&)[1]>(nn0), d >> 3, reinterpret_cast<const bf16_t*>(gptr(ltab[0].nw[p1_which])));
+  }
 
   for (int l = 0; l < m.n_layers; ++l) {
     const BitLayerDev& LY = ltab[l];
@@ -731,7 +769,7 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
       };
       if (ONE) {
         auto load0 = [&](int p) { return load_in(0, p); };
-        bit_stage_row1<1>(L, 1, d, norm1, nw, nullptr, m.eps, load0);
+        bit_stage_row1_pre<1>(L, 1, d, true, npw, reinterpret_cast<const uint4(&)[1]>(nn0), nn1, m.eps, load0);
       } else {
         bit_stage_roww<4>(L, 1, B, d, norm1, nw, nullptr, m.eps, load_in);
       }
@@ -778,6 +816,8 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
     gs.arrive(pf);
     const uint4* wo = reinterpret_cast<const uint4*>(gptr(LY.w[BO]));
     bit_prefetch<4>(wo, KCo, blockIdx.x, 0, KCo, (int)blockIdx.x < ns_d, wpre);
+    if (ONE && (int)blockIdx.x < ns_d)
+      row1_norm_fetch<1>(reinterpret_cast<uint4(&)[1]>(nn0), HD >> 3, reinterpret_cast<const bf16_t*>(gptr(LY.nw[BO])));
     // the residual of this lane's outputs in the first strip: known since the previous layer
     uint32_t rpre[2] = {0u, 0u};
     if ((int)blockIdx.x < ns_d && wave == 0 && mm < B && (int)blockIdx.x * 16 + 4 * gg < d)
@@ -798,7 +838,7 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
         const bf16_t* nwo = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BO]));
         if (ONE) {
           auto load0 = [&](int p) { return lds16(xs + p * 8); };
-          bit_stage_row1<1>(L, 1, HD, nullptr, nwo, nullptr, m.eps, load0);
+          bit_stage_row1_pre<1>(L, 1, HD, false, npw, reinterpret_cast<const uint4(&)[1]>(nn0), nn1, m.eps, load0);
         } else {
           auto loadb = [&](int b, int p) { return lds16(xs + (size_t)b * ldxs + p * 8); };
           bit_stage_roww<4>(L, 1, B, HD, nullptr, nwo, nullptr, m.eps, loadb);
@@ -827,6 +867,11 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
       bit_prefetch<2>(wg, KCd, strip, 0, KCd, strip < ns_f, wpre);
       bit_prefetch<2>(wu, KCd, strip, 0, KCd, strip < ns_f, wpre2);
     }
+    if (ONE && 2 * (int)blockIdx.x < ns_f) {
+      row1_norm_fetch<1>(npw, d >> 3, norm2);
+      row1_norm_fetch<1>(reinterpret_cast<uint4(&)[1]>(nn0), d >> 3, reinterpret_cast<const bf16_t*>(gptr(LY.nw[BG])));
+      row1_norm_fetch<1>(nn1, d >> 3, reinterpret_cast<const bf16_t*>(gptr(LY.nw[BU])));
+    }
     gs.wait(pf);
     // ---- P4: norm2 + ff.gate, ff.up + SwiGLU; two strips at a time, two waves each ----
     L.shape(B, d);
@@ -842,7 +887,7 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
       const bf16_t* nwu_ = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BU]));
       if (ONE) {
         auto load0 = [&](int p) { return load_mid(0, p); };
-        bit_stage_row1<1>(L, 2, d, norm2, nwg_, nwu_, m.eps, load0);
+        bit_stage_row1_pre<1>(L, 2, d, true, npw, reinterpret_cast<const uint4(&)[1]>(nn0), nn1, m.eps, load0);
       } else {
         bit_stage_roww<4>(L, 2, B, d, norm2, nwg_, nwu_, m.eps, load_mid);
       }
@@ -874,6 +919,11 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
     {
       const int unit = blockIdx.x, part = unit / ns_d, strip = unit - part * ns_d;
       bit_prefetch<4>(wd, KCf, strip, part * per_part, min(KCf, (part + 1) * per_part), unit < ns_d * OHARA_BIT_DOWN_SPLIT, wpre);
+      if (ONE && unit < ns_d * OHARA_BIT_DOWN_SPLIT) {
+        const bf16_t* nwd = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BD]));
+        if (F <= 2048) row1_norm_fetch<1>(reinterpret_cast<uint4(&)[1]>(nn0), F >> 3, nwd);
+        else row1_norm_fetch<3>(nn0, F >> 3, nwd);
+      }
     }
     gs.wait(pf);
     // ---- P5: ff.down, K split over OHARA_BIT_DOWN_SPLIT groups of workgroups ----
@@ -888,8 +938,8 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
           const bf16_t* nwd = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BD]));
           if (ONE) {
             auto load0 = [&](int p) { return ldg16(am_addr(a_l, a.blk_a, 0, p * 8)); };
-            if (F <= 2048) bit_stage_row1<1>(L, 1, F, nullptr, nwd, nullptr, m.eps, load0);
-            else bit_stage_row1<3>(L, 1, F, nullptr, nwd, nullptr, m.eps, load0);
+            if (F <= 2048) bit_stage_row1_pre<1>(L, 1, F, false, npw, reinterpret_cast<const uint4(&)[1]>(nn0), nn1, m.eps, load0);
+            else bit_stage_row1_pre<3>(L, 1, F, false, nn0, nn0, nn0, m.eps, load0);
           } else {
             auto loadb = [&](int b, int p) { return ldg16(am_addr(a_l, a.blk_a, b, p * 8)); };
             if (F <= 2048) bit_stage_roww<4>(L, 1, B, F, nullptr, nwd, nullptr, m.eps, loadb);
@@ -916,6 +966,10 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
     if (l + 1 == m.n_layers) break;  // the last barrier's wait follows the loop, behind another prefetch
     bit_prefetch<2>(reinterpret_cast<const uint4*>(gptr(ltab[l + 1].w[p1_which])), KCd, p1_strip0, 0, KCd,
                     p1_strip0 < p1_nstr, wpre);
+    if (ONE && 2 * p1_gi < p1_nstr) {
+      row1_norm_fetch<1>(npw, d >> 3, reinterpret_cast<const bf16_t*>(gptr(ltab[l + 1].norm1)));
+      row1_norm_fetch<1>(reinterpret_cast<uint4(&)[1]>(nn0), d >> 3, reinterpret_cast<const bf16_t*>(gptr(ltab[l + 1].nw[p1_which])));
+    }
     gs.wait(pf);
   }
   GemmPre lpre;
