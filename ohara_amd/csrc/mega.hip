@@ -79,8 +79,8 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   // per-layer pointers (6 weights/norms + K and V cache), copied once to LDS so that no phase
   // starts with a chain of dependent global loads
   float* mrg_w = att + (8 + 4 * D) * G;       // B*H*ns chunk weights
-  float* mrg_l = mrg_w + ((B * H * a.ns + 1) & ~1);  // B*H*ns chunk sums
-  unsigned long long* ptab = reinterpret_cast<unsigned long long*>(mrg_l + ((B * H * a.ns + 1) & ~1));
+  float* mrg_l = mrg_w + ((B * H * attn_merge_width(a.ns) + 1) & ~1);  // B*H*(merge width) chunk weights before it
+  unsigned long long* ptab = reinterpret_cast<unsigned long long*>(mrg_l + ((B * H * attn_merge_width(a.ns) + 1) & ~1));
   for (int i = threadIdx.x; i < m.n_layers * 8; i += blockDim.x) {
     const int l = i >> 3, j = i & 7;
     unsigned long long v;
@@ -397,9 +397,15 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   // one attention item per workgroup where the batch allows it
   int ns = n_workgroups / (s->batch * m->n_kv_heads);
   ns = ns < 1 ? 1 : (ns > OHARA_MEGA_NS ? OHARA_MEGA_NS : ns);
-  while (ns & (ns - 1)) ns &= ns - 1;  // a power of two: the merge is specialised per chunk count
+  // A power of two unless the exact count keeps at least half as many workgroups again busy and its
+  // merge stays narrow (the merge reads the next power of two of chunk slots): 7 chunks of 36 pairs
+  // instead of 4 took batch 6 from 0.397 to 0.379 ms per step, 5 instead of 4 at batch 8 lost what the
+  // attention phase gained to the wider merge.
+  int p2 = ns;
+  while (p2 & (p2 - 1)) p2 &= p2 - 1;
+  if (!(2 * ns >= 3 * p2 && attn_merge_width(ns) <= 8)) ns = p2;
   a.ns = ns;
-  const size_t mrg = (size_t)2 * ((s->batch * m->n_heads * ns + 1) & ~1) * sizeof(float);
+  const size_t mrg = (size_t)2 * ((s->batch * m->n_heads * attn_merge_width(ns) + 1) & ~1) * sizeof(float);
   const size_t smem = xs_bytes + 4096 + (size_t)(8 + 4 * D) * G * sizeof(float) + mrg + (size_t)m->n_layers * 64;
   if (smem > 160 * 1024) return OHARA_ESIZE;
   dim3 grid(n_workgroups), block(256);

@@ -346,8 +346,9 @@ __device__ __forceinline__ void stage_act(bf16_t* xs, int ldxs, const char* src,
 // columns per pass and issues the accumulator loads of 16 / NS passes - 16 loads - before it uses
 // any, so the number of dependent load rounds does not grow with the chunk count times the batch.
 // `mw`: B*H*NS floats, `ml`: B*H floats of LDS.
-template <int NS>
-__device__ __forceinline__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh, float* mw_, float* ml_) {
+template <int NS>  // NS: a power of two; `used` <= NS chunks hold partials (the others weigh nothing)
+__device__ __forceinline__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh, float* mw_, float* ml_,
+                                                 int used = NS) {
   constexpr int NSM = OHARA_MEGA_NS, PR = 16 / NS;
   const int HD = H * Dh, PS = Dh + 32;
   const int nbh = B * H, total = B * HD;
@@ -373,7 +374,7 @@ __device__ __forceinline__ void stage_attn_merge(bf16_t* xs, int ldxs, const flo
   for (int i0 = 0; i0 < nbh * NS; i0 += blockDim.x) {
     const int i = i0 + threadIdx.x;
     const int bh = i / NS, sp = i % NS;
-    const bool in = bh < nbh;
+    const bool in = bh < nbh && sp < used;
     float ms = -INFINITY, ls = 0.f;
     if (in) {
       const uint2 v = ldg8(pm + ((size_t)bh * NSM + sp) * PS + Dh);
@@ -391,7 +392,7 @@ __device__ __forceinline__ void stage_attn_merge(bf16_t* xs, int ldxs, const flo
     if (NS > 4) Ls = lane_xor_sum<4>(Ls);
     if (NS > 2) Ls = lane_xor_sum<2>(Ls);
     if (NS > 1) Ls = lane_xor_sum<1>(Ls);
-    if (in) mw[bh * NS + sp] = w;
+    if (bh < nbh) mw[bh * NS + sp] = w;  // 0 for chunks that are not in use: their slots hold old, finite sums
     if (in && sp == 0) ml[bh] = Ls;
   }
   __syncthreads();
@@ -457,31 +458,41 @@ __device__ __forceinline__ void stage_attn_merge_small(bf16_t* xs, int ldxs, con
 // Out-of-line copies of the merge, for kernels that want to keep their own code compact.
 template <int NS>
 __device__ __noinline__ void stage_attn_merge_call(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh, float* mw,
-                                                   float* ml) {
-  stage_attn_merge<NS>(xs, ldxs, pm, B, H, Dh, mw, ml);
+                                                   float* ml, int used) {
+  stage_attn_merge<NS>(xs, ldxs, pm, B, H, Dh, mw, ml, used);
 }
 
-// The merge for `ns` chunks.  INLINE: the five specialisations become part of the caller (no call in
-// the layer loop: a call makes the caller wait for every load it has in flight, the weights fetched
-// ahead included); otherwise they stay outside it, which keeps a kernel whose usual case is the
-// small merge within the instruction cache.
+// The power of two that the merge of `ns` chunks is specialised for (the chunk weights in LDS are laid
+// out with this stride).
+__host__ __device__ inline int attn_merge_width(int ns) {
+  int w = 1;
+  while (w < ns) w <<= 1;
+  return w;
+}
+
+// The merge for `ns` chunks (any count up to OHARA_MEGA_NS: the specialisation for the next power of two
+// runs with the chunks past `ns` weighing nothing).  INLINE: the five specialisations become part of the
+// caller (no call in the layer loop: a call makes the caller wait for every load it has in flight, the
+// weights fetched ahead included); otherwise they stay outside it, which keeps a kernel whose usual case
+// is the small merge within the instruction cache.
 template <bool INLINE>
 __device__ __forceinline__ void stage_attn_merge_any(int ns, bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh,
                                                      float* mw, float* ml) {
+  const int w = attn_merge_width(ns);
   if (ns == OHARA_MEGA_NS && B * H * Dh <= 4 * 256) {
     stage_attn_merge_small(xs, ldxs, pm, B, H, Dh);
   } else if (INLINE) {
-    if (ns == 16) stage_attn_merge<16>(xs, ldxs, pm, B, H, Dh, mw, ml);
-    else if (ns == 8) stage_attn_merge<8>(xs, ldxs, pm, B, H, Dh, mw, ml);
-    else if (ns == 4) stage_attn_merge<4>(xs, ldxs, pm, B, H, Dh, mw, ml);
-    else if (ns == 2) stage_attn_merge<2>(xs, ldxs, pm, B, H, Dh, mw, ml);
-    else stage_attn_merge<1>(xs, ldxs, pm, B, H, Dh, mw, ml);
+    if (w == 16) stage_attn_merge<16>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
+    else if (w == 8) stage_attn_merge<8>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
+    else if (w == 4) stage_attn_merge<4>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
+    else if (w == 2) stage_attn_merge<2>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
+    else stage_attn_merge<1>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
   } else {
-    if (ns == 16) stage_attn_merge_call<16>(xs, ldxs, pm, B, H, Dh, mw, ml);
-    else if (ns == 8) stage_attn_merge_call<8>(xs, ldxs, pm, B, H, Dh, mw, ml);
-    else if (ns == 4) stage_attn_merge_call<4>(xs, ldxs, pm, B, H, Dh, mw, ml);
-    else if (ns == 2) stage_attn_merge_call<2>(xs, ldxs, pm, B, H, Dh, mw, ml);
-    else stage_attn_merge_call<1>(xs, ldxs, pm, B, H, Dh, mw, ml);
+    if (w == 16) stage_attn_merge_call<16>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
+    else if (w == 8) stage_attn_merge_call<8>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
+    else if (w == 4) stage_attn_merge_call<4>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
+    else if (w == 2) stage_attn_merge_call<2>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
+    else stage_attn_merge_call<1>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
   }
 }
 

@@ -541,6 +541,30 @@ def test_every_persistent_kernel_variant_against_the_oracle(cuda, heads, kv_head
                 assert _near_tie(want_logits[t, b], int(got[b, t]), int(want[b, t])), (persistent, b, t)
 
 
+@pytest.mark.parametrize("B", [6, 7])
+def test_persistent_kernel_with_chunk_counts_that_are_not_powers_of_two(cuda, B):
+    """36 and 42 (sequence, KV head) pairs on 256 workgroups: the context of a pair is cut into 7 and 6
+    chunks, which the merge takes as the next power of two with the rest weighing nothing.  Greedy tokens
+    against the oracle (first divergence only at a near-tie) and against the kernel chain."""
+    from ohara_amd.llama import Llama
+
+    rcfg, cfg = _cfg_pair(vocab_size=512, hidden_size=384, intermediate_size=512, num_attention_heads=6,
+                          num_key_value_heads=6, num_hidden_layers=2, max_sequence_length=160, rope_theta=10000.0)
+    w = R.init_weights(rcfg, seed=13, dtype=BF, std=0.05, norm_jitter=0.1)
+    ref, model = R.RefLlama(rcfg, w), Llama(cfg, w, device=cuda)
+    assert model.supports_persistent(B)
+    prompt = torch.randint(0, 512, (B, 100), generator=torch.Generator().manual_seed(B))
+    want, want_logits = greedy_decode_ref(ref, prompt, 12, return_logits=True)
+    got = model.generate_greedy(prompt.to(cuda), 12, persistent=True).cpu()
+    chain = model.generate_greedy(prompt.to(cuda), 12, persistent=False).cpu()
+    for other in (want, chain):
+        for b in range(B):
+            neq = (got[b] != other[b]).nonzero()
+            if neq.numel():
+                t = int(neq[0])
+                assert _near_tie(want_logits[t, b], int(got[b, t]), int(other[b, t])), (b, t)
+
+
 @pytest.mark.parametrize("B", [5, 12, 16])
 def test_persistent_kernel_at_batches_up_to_its_limit(cuda, B):
     """The single launch is the default up to 8 sequences and can be asked for up to 16: greedy
