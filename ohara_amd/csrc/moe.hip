@@ -39,8 +39,11 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const bf16_t* logits, in
       sel[i] = -INFINITY;
     }
   }
-  float chosen_raw[16];
-  int chosen_id[16];
+  // Winner j is kept by lane j.  The arg-max butterfly runs on DPP moves and row swaps (the selection
+  // under a strict order - larger value, then lower id - does not depend on the order of the exchanges).
+  float my_raw = 0.f;
+  int my_id = 0;
+  auto better = [](float av, int ai, float bv, int bi) { return av > bv || (av == bv && ai < bi); };
   for (int j = 0; j < k; ++j) {
     // lane-local best (lowest id on ties), then across the wave
     float bv = -INFINITY;
@@ -53,15 +56,29 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const bf16_t* logits, in
         bi = e;
       }
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const float ov = __shfl_xor(bv, o, WAVE);
-      const int oi = __shfl_xor(bi, o, WAVE);
-      if (ov > bv || (ov == bv && oi < bi)) {
-        bv = ov;
-        bi = oi;
-      }
+    {
+      const u32x2 v32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(bv), __float_as_uint(bv), false, false);
+      const u32x2 i32 = __builtin_amdgcn_permlane32_swap((uint32_t)bi, (uint32_t)bi, false, false);
+      const bool a = better(__uint_as_float(v32[0]), (int)i32[0], __uint_as_float(v32[1]), (int)i32[1]);
+      bv = __uint_as_float(a ? v32[0] : v32[1]);
+      bi = (int)(a ? i32[0] : i32[1]);
+      const u32x2 v16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(bv), __float_as_uint(bv), false, false);
+      const u32x2 i16 = __builtin_amdgcn_permlane16_swap((uint32_t)bi, (uint32_t)bi, false, false);
+      const bool c = better(__uint_as_float(v16[0]), (int)i16[0], __uint_as_float(v16[1]), (int)i16[1]);
+      bv = __uint_as_float(c ? v16[0] : v16[1]);
+      bi = (int)(c ? i16[0] : i16[1]);
     }
+#define OHARA_ROUTE_STEP(M)                                                   \
+    {                                                                         \
+      const float ov = lane_xor<M>(bv);                                       \
+      const int oi = (int)lane_xor_u32<M>((uint32_t)bi);                      \
+      if (better(ov, oi, bv, bi)) {                                           \
+        bv = ov;                                                              \
+        bi = oi;                                                              \
+      }                                                                       \
+    }
+    OHARA_ROUTE_STEP(8) OHARA_ROUTE_STEP(4) OHARA_ROUTE_STEP(2) OHARA_ROUTE_STEP(1)
+#undef OHARA_ROUTE_STEP
     // fetch the unbiased logit of the winner and retire it
     float r = 0.f;
 #pragma unroll
@@ -70,36 +87,30 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const bf16_t* logits, in
         r = raw[i];
         sel[i] = -INFINITY;
       }
-    r = __shfl(r, bi & 63, WAVE);
-    chosen_raw[j] = r;
-    chosen_id[j] = bi;
+    r = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(r), bi & 63));
+    if (lane == j) {
+      my_raw = r;
+      my_id = bi;
+    }
   }
-  if (lane == 0) {
-    float wts[16];
-    if (!sigmoid) {
-      float m = -INFINITY;
-      for (int j = 0; j < k; ++j) m = fmaxf(m, chosen_raw[j]);
-      float z = 0.f;
-      for (int j = 0; j < k; ++j) {
-        wts[j] = expf(chosen_raw[j] - m);
-        z += wts[j];
-      }
-      for (int j = 0; j < k; ++j) wts[j] /= z;
-    } else {
-      float z = 0.f;
-      for (int j = 0; j < k; ++j) {
-        wts[j] = 1.0f / (1.0f + expf(-chosen_raw[j]));
-        z += wts[j];
-      }
-      if (normalize) {
-        z = fmaxf(z, 1e-9f);
-        for (int j = 0; j < k; ++j) wts[j] /= z;
-      }
-    }
-    for (int j = 0; j < k; ++j) {
-      idx[(size_t)n * k + j] = chosen_id[j];
-      w[(size_t)n * k + j] = f2bf(wts[j]);
-    }
+  // weights: every lane below k holds one; the sums run in slot order, as a loop over the slots would
+  const bool has = lane < k;
+  float wt;
+  if (!sigmoid) {
+    const float m = wave_max(has ? my_raw : -INFINITY);
+    const float e = has ? expf(my_raw - m) : 0.f;
+    float z = 0.f;
+    for (int j = 0; j < k; ++j) z += __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(e), j));
+    wt = e / z;
+  } else {
+    const float sg = has ? 1.0f / (1.0f + expf(-my_raw)) : 0.f;
+    float z = 0.f;
+    for (int j = 0; j < k; ++j) z += __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(sg), j));
+    wt = normalize ? sg / fmaxf(z, 1e-9f) : sg;
+  }
+  if (has) {
+    idx[(size_t)n * k + lane] = my_id;
+    w[(size_t)n * k + lane] = f2bf(wt);
   }
 }
 
@@ -153,6 +164,50 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int32_t* idx, int 
     __syncthreads();
     if (e >= 0) atomicAdd(&cnt[e], 1);
     __syncthreads();
+  }
+}
+
+// The same sort for at most 64 experts and 1024 pairs (decode): a pair's rank among the earlier pairs of
+// its expert is a ballot match inside its wave (six ballots for the six bits of an expert id) plus the
+// counts of the waves before it, instead of a scan over all earlier pairs; the offsets are one wave's scan.
+__global__ __launch_bounds__(1024) void moe_sort_small_kernel(const int32_t* idx, int NK, int E, int32_t* offs,
+                                                              int32_t* pair_of, int32_t* pos_of) {
+  __shared__ int wcnt[16][64];   // pairs of expert e in wave w, then the first sorted position of that wave's pairs of e
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  wcnt[wave][lane] = 0;
+  const int e = tid < NK ? idx[tid] : -1;
+  unsigned long long same = __ballot(e >= 0);
+#pragma unroll
+  for (int bit = 0; bit < 6; ++bit) {
+    const unsigned long long b = __ballot((e >> bit) & 1);
+    same &= ((e >> bit) & 1) ? b : ~b;
+  }
+  const int rank = __popcll(same & ((1ull << lane) - 1ull));
+  __syncthreads();
+  if (e >= 0 && (same >> lane) == 1ull) wcnt[wave][e] = __popcll(same);  // the last lane of the wave with this expert
+  __syncthreads();
+  if (wave == 0) {
+    int tot = 0, c[16];
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      c[w] = wcnt[w][lane];
+      tot += c[w];
+    }
+    const int incl = wave_incl_scan_i(lane < E ? tot : 0);
+    int run = incl - (lane < E ? tot : 0);
+    if (lane < E) offs[lane] = run;
+    if (lane == 63) offs[E] = incl;  // lanes at and past E added nothing
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      wcnt[w][lane] = run;
+      run += c[w];
+    }
+  }
+  __syncthreads();
+  if (e >= 0) {
+    const int o = wcnt[wave][e] + rank;
+    pair_of[o] = tid;
+    pos_of[tid] = o;
   }
 }
 
@@ -321,8 +376,12 @@ int ohara_moe_sort_pairs(const int32_t* expert_idx, int n_pairs, int n_experts, 
                          int32_t* pos_of, void* stream) {
   if (!expert_idx || !offsets || !pair_of || !pos_of || n_pairs < 1 || n_experts < 1) return OHARA_EINVAL;
   if (n_pairs > 65536 || n_experts > 1024) return OHARA_ESIZE;
-  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, expert_idx, n_pairs, n_experts, offsets,
-                     pair_of, pos_of);
+  if (n_experts <= 64 && n_pairs <= 1024)
+    hipLaunchKernelGGL(moe_sort_small_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, expert_idx, n_pairs, n_experts,
+                       offsets, pair_of, pos_of);
+  else
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, expert_idx, n_pairs, n_experts, offsets,
+                       pair_of, pos_of);
   return ohara_launch_status();
 }
 
