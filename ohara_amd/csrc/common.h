@@ -97,6 +97,32 @@ __device__ __forceinline__ void lane_swap(float v, float& a, float& b) {  // {a,
   a = __uint_as_float(r[0]);
   b = __uint_as_float(r[1]);
 }
+// One butterfly step of an arg-max under the strict order "larger value, then lower index" (a value
+// that is not greater than -inf, such as NaN, never wins): (v, i) becomes the better of this lane's and
+// lane ^ M's pair.  The winner of a strict order does not depend on the order of the exchanges, so a
+// butterfly of these steps returns what the shuffle butterfly returns.
+template <int M>
+__device__ __forceinline__ void lane_xor_argmax(float& v, int& i) {
+  if constexpr (M >= 16) {
+    const u32x2 vv = M == 16 ? __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false)
+                             : __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    const u32x2 ii = M == 16 ? __builtin_amdgcn_permlane16_swap((uint32_t)i, (uint32_t)i, false, false)
+                             : __builtin_amdgcn_permlane32_swap((uint32_t)i, (uint32_t)i, false, false);
+    const float v0 = __uint_as_float(vv[0]), v1 = __uint_as_float(vv[1]);
+    const int i0 = (int)ii[0], i1 = (int)ii[1];
+    const bool first = v0 > v1 || (v0 == v1 && i0 < i1) || !(v1 > v0 || (v1 == v0 && i1 < i0)) && i0 <= i1;
+    v = first ? v0 : v1;
+    i = first ? i0 : i1;
+  } else {
+    const float ov = lane_xor<M>(v);
+    const int oi = (int)lane_xor_u32<M>((uint32_t)i);
+    if (ov > v || (ov == v && oi < i)) {
+      v = ov;
+      i = oi;
+    }
+  }
+}
+
 // Inclusive prefix sum across the 64 lanes of a wave, in lane order, through DPP moves (shifts
 // inside a row of 16 lanes, then the last lane of a row broadcast into the rows after it): six
 // moves instead of six LDS-crossbar shuffles.  All lanes of the wave must be active.

@@ -91,15 +91,12 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const bf16_t* logits, int 
     for (int i = threadIdx.x; i < n; i += 1024) take(bf2f(row[i]), i);
   }
   // NaN-free comparison network; ties resolve to the lowest index
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    const float ov = __shfl_xor(best, o, WAVE);
-    const int oi = __shfl_xor(bi, o, WAVE);
-    if (ov > best || (ov == best && oi < bi)) {
-      best = ov;
-      bi = oi;
-    }
-  }
+  lane_xor_argmax<32>(best, bi);
+  lane_xor_argmax<16>(best, bi);
+  lane_xor_argmax<8>(best, bi);
+  lane_xor_argmax<4>(best, bi);
+  lane_xor_argmax<2>(best, bi);
+  lane_xor_argmax<1>(best, bi);
   __shared__ float sv[16];
   __shared__ int si[16];
   const int wave = threadIdx.x >> 6;

@@ -39,11 +39,9 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const bf16_t* logits, in
       sel[i] = -INFINITY;
     }
   }
-  // Winner j is kept by lane j.  The arg-max butterfly runs on DPP moves and row swaps (the selection
-  // under a strict order - larger value, then lower id - does not depend on the order of the exchanges).
+  // Winner j is kept by lane j; the arg-max butterfly runs on DPP moves and row swaps.
   float my_raw = 0.f;
   int my_id = 0;
-  auto better = [](float av, int ai, float bv, int bi) { return av > bv || (av == bv && ai < bi); };
   for (int j = 0; j < k; ++j) {
     // lane-local best (lowest id on ties), then across the wave
     float bv = -INFINITY;
@@ -56,29 +54,12 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const bf16_t* logits, in
         bi = e;
       }
     }
-    {
-      const u32x2 v32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(bv), __float_as_uint(bv), false, false);
-      const u32x2 i32 = __builtin_amdgcn_permlane32_swap((uint32_t)bi, (uint32_t)bi, false, false);
-      const bool a = better(__uint_as_float(v32[0]), (int)i32[0], __uint_as_float(v32[1]), (int)i32[1]);
-      bv = __uint_as_float(a ? v32[0] : v32[1]);
-      bi = (int)(a ? i32[0] : i32[1]);
-      const u32x2 v16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(bv), __float_as_uint(bv), false, false);
-      const u32x2 i16 = __builtin_amdgcn_permlane16_swap((uint32_t)bi, (uint32_t)bi, false, false);
-      const bool c = better(__uint_as_float(v16[0]), (int)i16[0], __uint_as_float(v16[1]), (int)i16[1]);
-      bv = __uint_as_float(c ? v16[0] : v16[1]);
-      bi = (int)(c ? i16[0] : i16[1]);
-    }
-#define OHARA_ROUTE_STEP(M)                                                   \
-    {                                                                         \
-      const float ov = lane_xor<M>(bv);                                       \
-      const int oi = (int)lane_xor_u32<M>((uint32_t)bi);                      \
-      if (better(ov, oi, bv, bi)) {                                           \
-        bv = ov;                                                              \
-        bi = oi;                                                              \
-      }                                                                       \
-    }
-    OHARA_ROUTE_STEP(8) OHARA_ROUTE_STEP(4) OHARA_ROUTE_STEP(2) OHARA_ROUTE_STEP(1)
-#undef OHARA_ROUTE_STEP
+    lane_xor_argmax<32>(bv, bi);
+    lane_xor_argmax<16>(bv, bi);
+    lane_xor_argmax<8>(bv, bi);
+    lane_xor_argmax<4>(bv, bi);
+    lane_xor_argmax<2>(bv, bi);
+    lane_xor_argmax<1>(bv, bi);
     // fetch the unbiased logit of the winner and retire it
     float r = 0.f;
 #pragma unroll
