@@ -56,7 +56,7 @@ __device__ __forceinline__ void stf_coh(float* p, float v) { st_coh4(p, __float_
 // 256 threads of the last workgroup to finish.  A chain of dependent device-coherent loads
 // costs about a microsecond per link on this chip, so the (max, sum) pairs of all chunks are
 // fetched in one round into LDS, the chunk weights exp(m_s - M) are formed there, and the
-// accumulator columns are then summed in chunk order with their loads issued eight at a time.
+// accumulator columns are then summed in chunk order with the loads of up to 32 chunks issued together.
 // Needs G * n_split <= OHARA_MERGE_CAP.
 #define OHARA_MERGE_CAP 2048
 template <int MAXD>
@@ -94,12 +94,16 @@ __device__ void merge_partials(const AttnArgs& a, int b /* query row */, int kvh
     const float* pa = a.part_acc + ((size_t)(b * a.H + h) * ns) * D + d;
     const float* w = s_w + hh * ns;
     float o = 0.f;
-    for (int s0 = 0; s0 < ns; s0 += 8) {
-      float av[8];
+    // Up to 32 chunks' values are in flight at once, every load unconditional (chunks past the last
+    // read the last one again and are not added): with eight at a time behind a test each, 32 chunks
+    // were four dependent round trips and more than half of a batch-1 launch.
+    for (int s0 = 0; s0 < ns; s0 += 32) {
+      float av[32];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) av[i] = (s0 + i < ns) ? ldf_coh(pa + (size_t)(s0 + i) * D) : 0.f;
+      for (int i = 0; i < 32; ++i) av[i] = ldf_coh(pa + (size_t)min(s0 + i, ns - 1) * D);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
+      for (int i = 0; i < 32; ++i)
         if (s0 + i < ns) o += av[i] * w[s0 + i];
     }
     a.out[(size_t)b * a.H * D + h * D + d] = f2bf(o / s_tot[hh]);
