@@ -284,12 +284,13 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
     float M = -INFINITY;
     for (int c = 0; c < a.ns; ++c) M = fmaxf(M, qr[c]);
     float num = 0.f, den = 0.f;
-    for (int c0 = 0; c0 < a.ns; c0 += 8) {
-      float av[8];
+    for (int c0 = 0; c0 < a.ns; c0 += 16) {  // sixteen chunks' values in flight, every load unconditional
+      float av[16];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) av[i] = c0 + i < a.ns ? __uint_as_float(ld_coh4(p + (size_t)(c0 + i) * (D + 2) + tid)) : 0.f;
+      for (int i = 0; i < 16; ++i) av[i] = __uint_as_float(ld_coh4(p + (size_t)min(c0 + i, a.ns - 1) * (D + 2) + tid));
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < 16; ++i) {
         if (c0 + i >= a.ns || qr[c0 + i] == -INFINITY) continue;
         const float wg = expf(qr[c0 + i] - M);
         num += wg * av[i];
