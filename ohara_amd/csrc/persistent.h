@@ -359,11 +359,11 @@ __device__ __forceinline__ void stage_attn_merge(bf16_t* xs, int ldxs, const flo
   auto load = [&](int e0) {
 #pragma unroll
     for (int r = 0; r < PR; ++r) {
-      const int e = e0 + r * pass;
-      const int b = e / HD, hd = e - b * HD;
+      const int e = min(e0 + r * pass, total - 4);  // columns past the end read the last group again (not used):
+      const int b = e / HD, hd = e - b * HD;        // no load behind a branch
       const float* base = pm + (size_t)(b * H + hd / Dh) * NSM * PS + (hd % Dh);
 #pragma unroll
-      for (int sp = 0; sp < NS; ++sp) av[r][sp] = e < total ? ldg16(base + (size_t)sp * PS) : make_uint4(0, 0, 0, 0);
+      for (int sp = 0; sp < NS; ++sp) av[r][sp] = ldg16(base + (size_t)sp * PS);
     }
   };
   // the accumulator loads of the first round go out first: they do not depend on the chunk
