@@ -25,13 +25,13 @@ struct PrefillArgs {
   const bf16_t* v;
   bf16_t* out;       // (B*S, H*D)
   int B, S, H, Hkv, Tmax, pos;
-  int nqb;           // query blocks of 128 per sequence
+  int nqb;           // query blocks (of 128 or 64) per sequence
   float scale_log2e;
 };
 
-template <int D>
+template <int D, int QW>  // QW: blocks of 16 queries per wave (2: 128 queries per workgroup, 1: 64)
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(PrefillArgs a) {
-  constexpr int QB = 128, KT = 64;
+  constexpr int QB = 64 * QW, KT = 64;
   constexpr int NK = D / 32;   // k-steps of the score product
   constexpr int ND = D / 16;   // 16-column blocks of the output
   constexpr int LDK = D + 8;   // K tile row stride (elements): 16-byte reads without bank conflicts
@@ -51,7 +51,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(PrefillArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 15, g = lane >> 4;
   const int q0 = qblk * QB;                       // first query of the workgroup
-  const int wq0 = q0 + wave * 32;                 // first query of the wave
+  const int wq0 = q0 + wave * 16 * QW;            // first query of the wave
   const size_t row = (size_t)a.Hkv * D;
   const bf16_t* kb = a.k + (size_t)b * a.Tmax * row + (size_t)kvh * D;
   const bf16_t* vb = a.v + (size_t)b * a.Tmax * row + (size_t)kvh * D;
@@ -59,10 +59,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(PrefillArgs a) {
   const int kv_end = min(a.pos + q0 + QB, Lall);  // positions any query of the workgroup sees
 
   // Q fragments: lane (n = query within block, g) holds Q[q][32 j + 8 g .. +7]
-  uint4 qf[2][NK];
-  int qpos[2];
+  uint4 qf[QW][NK];
+  int qpos[QW];
 #pragma unroll
-  for (int qb = 0; qb < 2; ++qb) {
+  for (int qb = 0; qb < QW; ++qb) {
     const int qi = wq0 + qb * 16 + m;
     qpos[qb] = qi < a.S ? a.pos + qi : 0x3fffffff;  // rows past the end: never masked, never stored
 #pragma unroll
@@ -70,12 +70,12 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(PrefillArgs a) {
       qf[qb][j] = qi < a.S ? ldg16(a.q + ((size_t)b * a.S + qi) * a.H * D + (size_t)h * D + 32 * j + 8 * g)
                            : make_uint4(0, 0, 0, 0);
   }
-  const int wave_last = min(a.pos + wq0 + 31, Lall - 1);  // last position any query of the wave sees
+  const int wave_last = min(a.pos + wq0 + 16 * QW - 1, Lall - 1);  // last position any query of the wave sees
 
-  f32x4 o[2][ND];
-  float m_run[2], l_run[2];
+  f32x4 o[QW][ND];
+  float m_run[QW], l_run[QW];
 #pragma unroll
-  for (int qb = 0; qb < 2; ++qb) {
+  for (int qb = 0; qb < QW; ++qb) {
     m_run[qb] = -INFINITY;
     l_run[qb] = 0.f;
 #pragma unroll
@@ -140,24 +140,37 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(PrefillArgs a) {
     if (t0 > wave_last) continue;               // wholly masked for this wave (barriers stay uniform)
 
     // scores: s[kb][qb] = D[16 positions x 16 queries]
-    f32x4 s[4][2];
+    // The K fragments of two 16-position blocks are read from LDS into registers of their own before
+    // their products (left to itself the compiler reuses one register quad: read, wait, product,
+    // sixteen times per tile, every LDS latency exposed - a quarter of a tile's time).
+    constexpr int KBB = QW == 1 ? 1 : 2;  // 16-position blocks whose fragments are read together (registers: three workgroups per CU with QW == 1)
+    f32x4 s[4][QW];
 #pragma unroll
-    for (int kbk = 0; kbk < 4; ++kbk) {
-      s[kbk][0] = (f32x4){0.f, 0.f, 0.f, 0.f};
-      s[kbk][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int kb2 = 0; kb2 < 4; kb2 += KBB) {
+      uint4 kf[KBB][NK];
 #pragma unroll
-      for (int j = 0; j < NK; ++j) {
-        const uint4 kf = *reinterpret_cast<const uint4*>(&Ks[kbk * 16 + m][32 * j + 8 * g]);
-        s[kbk][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf),
-                                                            __builtin_bit_cast(bf16x8, qf[0][j]), s[kbk][0], 0, 0, 0);
-        s[kbk][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf),
-                                                            __builtin_bit_cast(bf16x8, qf[1][j]), s[kbk][1], 0, 0, 0);
+      for (int kk = 0; kk < KBB; ++kk)
+#pragma unroll
+        for (int j = 0; j < NK; ++j) kf[kk][j] = *reinterpret_cast<const uint4*>(&Ks[(kb2 + kk) * 16 + m][32 * j + 8 * g]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int kk = 0; kk < KBB; ++kk) {
+        const int kbk = kb2 + kk;
+#pragma unroll
+        for (int qb = 0; qb < QW; ++qb) s[kbk][qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < NK; ++j)
+#pragma unroll
+          for (int qb = 0; qb < QW; ++qb)
+            s[kbk][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf[kk][j]),
+                                                                 __builtin_bit_cast(bf16x8, qf[qb][j]), s[kbk][qb], 0, 0, 0);
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
     // online softmax per query (= per lane column)
-    uint4 pf[2][2];  // [qb][32-position window]: B operand of the second product
+    uint4 pf[QW][2];  // [qb][32-position window]: B operand of the second product
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
+    for (int qb = 0; qb < QW; ++qb) {
       float tmax = -INFINITY;
       float mul = 1.0f;  // what the stored scores still have to be multiplied with
       if (t0 + KT - 1 > a.pos + wq0) {  // (wave-uniform) the tile reaches past the wave's first query: mask
@@ -205,22 +218,33 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(PrefillArgs a) {
                                pack_bf(p[2 * w + 1][0], p[2 * w + 1][1]), pack_bf(p[2 * w + 1][2], p[2 * w + 1][3]));
     }
     // O^T[16 columns x 16 queries] += V^T[16 columns x 32 slots] P[32 slots x 16 queries]
+    constexpr int DBB = QW == 1 ? 4 : ND;  // 16-column blocks of V^T whose fragments are read together
 #pragma unroll
     for (int w = 0; w < 2; ++w)
 #pragma unroll
-      for (int db = 0; db < ND; ++db) {
-        const uint2 v0 = *reinterpret_cast<const uint2*>(&Vt[db * 16 + m][vt_off(db * 16 + m, 32 * w + 4 * g)]);
-        const uint2 v1 = *reinterpret_cast<const uint2*>(&Vt[db * 16 + m][vt_off(db * 16 + m, 32 * w + 16 + 4 * g)]);
-        const uint4 vf = make_uint4(v0.x, v0.y, v1.x, v1.y);
-        o[0][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf),
-                                                           __builtin_bit_cast(bf16x8, pf[0][w]), o[0][db], 0, 0, 0);
-        o[1][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf),
-                                                           __builtin_bit_cast(bf16x8, pf[1][w]), o[1][db], 0, 0, 0);
+      for (int d0 = 0; d0 < ND; d0 += DBB) {
+        uint2 v0[DBB], v1[DBB];  // all read before the first product, as above
+#pragma unroll
+        for (int i = 0; i < DBB; ++i) {
+          const int db = d0 + i;
+          v0[i] = *reinterpret_cast<const uint2*>(&Vt[db * 16 + m][vt_off(db * 16 + m, 32 * w + 4 * g)]);
+          v1[i] = *reinterpret_cast<const uint2*>(&Vt[db * 16 + m][vt_off(db * 16 + m, 32 * w + 16 + 4 * g)]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < DBB; ++i) {
+          const uint4 vf = make_uint4(v0[i].x, v0[i].y, v1[i].x, v1[i].y);
+#pragma unroll
+          for (int qb = 0; qb < QW; ++qb)
+            o[qb][d0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf),
+                                                                    __builtin_bit_cast(bf16x8, pf[qb][w]), o[qb][d0 + i], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
   }
 
 #pragma unroll
-  for (int qb = 0; qb < 2; ++qb) {
+  for (int qb = 0; qb < QW; ++qb) {
     const int qi = wq0 + qb * 16 + m;
     float l = l_run[qb];
     l = lane_xor_sum<32>(lane_xor_sum<16>(l));
@@ -247,10 +271,26 @@ extern "C" int ohara_attn_prefill_bf16(const uint16_t* q, const uint16_t* kcache
   PrefillArgs a{};
   a.q = q; a.k = kcache; a.v = vcache; a.out = out;
   a.B = batch; a.S = seq_len; a.H = h; a.Hkv = h_kv; a.Tmax = t_max; a.pos = pos;
-  a.nqb = (seq_len + 127) / 128;
   a.scale_log2e = 1.4426950408889634f / sqrtf((float)dh);
+  // A causal launch lasts as long as its last query block (sixteen tiles at 1024 tokens, twice the
+  // average), whatever the other workgroups do.  With fewer than two blocks of 128 queries per CU,
+  // blocks of 64 fit three workgroups on a CU and all of them are resident at once (8 x 1024 tokens,
+  // 6 heads: 56.1 -> 54.5 us; the tile of the last block, about 2.9 us, stays what bounds the launch).
+  static int cus = 0;
+  if (!cus) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+      cus = 256;
+  }
+  const bool small = (int64_t)((seq_len + 127) / 128) * h * batch < 2 * (int64_t)cus;
+  a.nqb = small ? (seq_len + 63) / 64 : (seq_len + 127) / 128;
   dim3 grid(a.nqb, h, batch), block(256);
-  if (dh == 128) hipLaunchKernelGGL((attn_prefill_kernel<128>), grid, block, 0, (hipStream_t)stream, a);
-  else hipLaunchKernelGGL((attn_prefill_kernel<64>), grid, block, 0, (hipStream_t)stream, a);
+  if (dh == 128) {
+    if (small) hipLaunchKernelGGL((attn_prefill_kernel<128, 1>), grid, block, 0, (hipStream_t)stream, a);
+    else hipLaunchKernelGGL((attn_prefill_kernel<128, 2>), grid, block, 0, (hipStream_t)stream, a);
+  } else {
+    if (small) hipLaunchKernelGGL((attn_prefill_kernel<64, 1>), grid, block, 0, (hipStream_t)stream, a);
+    else hipLaunchKernelGGL((attn_prefill_kernel<64, 2>), grid, block, 0, (hipStream_t)stream, a);
+  }
   return ohara_launch_status();
 }
