@@ -209,7 +209,10 @@ struct ExpertArgs {
   int ldo;
 };
 
-template <int EPI>
+// CH: k-steps a wave has in flight at once (the host takes 4 when a wave's share of K is that short).
+// Every load of a batch is issued whatever its index - clamped into the strip and the row, zeroed
+// afterwards where it lies beyond the wave's share - so the batch is one run of loads without branches.
+template <int EPI, int CH>
 __global__ __launch_bounds__(256) void moe_expert_kernel(ExpertArgs a) {
   const int strip = blockIdx.x, e = blockIdx.y;
   const int p0 = a.offs[e], p1 = a.offs[e + 1];
@@ -224,27 +227,29 @@ __global__ __launch_bounds__(256) void moe_expert_kernel(ExpertArgs a) {
   for (int pt = p0; pt < p1; pt += 16) {  // 16-token column tiles of this expert
     const int pos = pt + m;
     const bool has = pos < p1;
-    const bf16_t* xrow = a.x;
-    if (has) {
-      const int src = (EPI == X_SWIGLU) ? a.pair_of[pos] / a.k : pos;
-      xrow = a.x + (size_t)src * a.ldx;
-    }
+    const int posc = min(pos, p1 - 1);  // a token of this expert: lanes past the end compute a column nobody stores
+    const int pair = a.pair_of[posc];
+    const bf16_t* xrow = a.x + (size_t)((EPI == X_SWIGLU) ? pair / a.k : posc) * a.ldx;
+    float wt = 0.f;
+    if (EPI == X_DOWN) wt = bf2f(a.w[pair]);  // asked for here, used in the epilogue
     f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
-    constexpr int CH = 8;
     for (int jb = j0; jb < j1; jb += CH) {
       uint4 wv[CH], xv[CH];
 #pragma unroll
       for (int c = 0; c < CH; ++c) {
-        const int j = jb + c;
-        wv[c] = j < j1 ? ldg16_nt(wrow + (size_t)j * 64) : make_uint4(0, 0, 0, 0);
-        const int k0 = 32 * j + 8 * g;
-        xv[c] = make_uint4(0, 0, 0, 0);
-        if (has && j < j1 && k0 < a.K) xv[c] = ldg16(xrow + k0);
+        const int j = min(jb + c, j1 - 1);
+        wv[c] = ldg16_nt(wrow + (size_t)j * 64);
+        xv[c] = ldg16(xrow + min(32 * j + 8 * g, a.K - 8));
       }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int c = 0; c < CH; ++c)
+      for (int c = 0; c < CH; ++c) {
+        const bool live = jb + c < j1 && 32 * (jb + c) + 8 * g < a.K;
+        if (!live) xv[c] = make_uint4(0, 0, 0, 0);  // the packed weights are zero beyond K; the row's values are not
+        if (jb + c >= j1) wv[c] = make_uint4(0, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wv[c]), __builtin_bit_cast(bf16x8, xv[c]),
                                                       acc, 0, 0, 0);
+      }
     }
     if (wave > 0) {
 #pragma unroll
@@ -262,7 +267,6 @@ __global__ __launch_bounds__(256) void moe_expert_kernel(ExpertArgs a) {
           if (f < a.N_out) o[0] = f2bf(rbf(silu_f(y0)) * y2);
           if (f + 1 < a.N_out) o[1] = f2bf(rbf(silu_f(y1)) * y3);
         } else {
-          const float wt = bf2f(a.w[a.pair_of[pos]]);
           const int r0 = strip * 16 + 4 * g;
           const float v[4] = {y0 * wt, y1 * wt, y2 * wt, y3 * wt};
           bf16_t* o = a.out + (size_t)pos * a.ldo + r0;
@@ -375,7 +379,10 @@ int ohara_moe_experts_gate_up(const uint16_t* x, int ldx, const uint16_t* wp_gat
   a.x = x; a.ldx = ldx; a.offs = offsets; a.pair_of = pair_of; a.k = k; a.N_out = hidden; a.K = d;
   a.out = act; a.ldo = ld_act;
   const int strips = 2 * ((hidden + 7) / 8 * 8) / 16;
-  hipLaunchKernelGGL((moe_expert_kernel<X_SWIGLU>), dim3(strips, n_experts), dim3(256), 0, (hipStream_t)stream, a);
+  if ((d + 31) / 32 <= 16)
+    hipLaunchKernelGGL((moe_expert_kernel<X_SWIGLU, 4>), dim3(strips, n_experts), dim3(256), 0, (hipStream_t)stream, a);
+  else
+    hipLaunchKernelGGL((moe_expert_kernel<X_SWIGLU, 8>), dim3(strips, n_experts), dim3(256), 0, (hipStream_t)stream, a);
   return ohara_launch_status();
 }
 
@@ -388,7 +395,10 @@ int ohara_moe_experts_down(const uint16_t* act, int ld_act, const uint16_t* wp_d
   a.wp = reinterpret_cast<const uint4*>(wp_down); a.expert_stride = (size_t)expert_stride_bytes / 16;
   a.x = act; a.ldx = ld_act; a.offs = offsets; a.pair_of = pair_of; a.w = expert_w; a.k = k; a.N_out = d; a.K = hidden;
   a.out = y; a.ldo = ldy;
-  hipLaunchKernelGGL((moe_expert_kernel<X_DOWN>), dim3((d + 15) / 16, n_experts), dim3(256), 0, (hipStream_t)stream, a);
+  if ((hidden + 31) / 32 <= 16)
+    hipLaunchKernelGGL((moe_expert_kernel<X_DOWN, 4>), dim3((d + 15) / 16, n_experts), dim3(256), 0, (hipStream_t)stream, a);
+  else
+    hipLaunchKernelGGL((moe_expert_kernel<X_DOWN, 8>), dim3((d + 15) / 16, n_experts), dim3(256), 0, (hipStream_t)stream, a);
   return ohara_launch_status();
 }
 
