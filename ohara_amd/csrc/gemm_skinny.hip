@@ -365,7 +365,7 @@ int launch_wide_bt(const GemmArgs& a, int epi, hipStream_t st) {
 bool wide_applies(const GemmArgs& a, int epi, int strips) {
   const int KS = (a.K + 31) >> 5;
   const int bt = (a.B + 15) / 16;
-  return epi == EPI_STORE && strips >= 1024 && a.B <= 64 && (size_t)16 * bt * (KS * 32 + 8) * 2 <= 128 * 1024;
+  return epi == EPI_STORE && strips >= 1024 && a.B <= 64 && (size_t)16 * bt * (KS * 32 + 8) * 2 <= 160 * 1024;
 }
 
 int launch_wide(const GemmArgs& a0, int epi, int strips, hipStream_t st) {

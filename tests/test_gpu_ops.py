@@ -52,7 +52,9 @@ def test_rmsnorm(cuda, d):
                                    (32, 2304, 768), (64, 768, 3072), (5, 65, 40),
                                    # >= 1024 strips: the kernel that keeps the activations in LDS
                                    (1, 16384, 768), (17, 16390, 776), (33, 20000, 96), (64, 16384, 768),
-                                   (48, 16400, 1000)])
+                                   (48, 16400, 1000),
+                                   # the same kernel with more than 128 KB of rows in LDS, and close to the 160 KB it may take
+                                   (64, 16384, 1024), (64, 16400, 1216)])
 @pytest.mark.parametrize("norm", [False, True])
 def test_gemm_skinny_store(cuda, B, N, K, norm):
     from ohara_amd import ops
