@@ -99,6 +99,9 @@ struct PhiAttnArgs {
   int* counters;  // ns > 1: per (row, head) chunks finished; zero between calls
 };
 
+#ifndef PHI_ATTN_R
+#define PHI_ATTN_R 2
+#endif
 __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
   __shared__ float qr[128];
   __shared__ float gm[16], gl[16];
@@ -106,7 +109,23 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int grp = wave * 4 + (lane >> 4), l = lane & 15;
   const int D = a.D, half = a.rot >> 1;
-  int w = blockIdx.x;
+  // The cache is position-major: the heads of one position lie side by side, 2 * D bytes each, so the rows of
+  // neighbouring heads share 128-byte lines.  Workgroups are handed to the eight XCDs in turn, each with an L2 of
+  // its own: taken as launched, neighbouring heads would land on different XCDs and every L2 would fetch the
+  // shared lines again.  So the launch order is re-read: XCD x works through the x-th eighth of the (chunk,
+  // sequence, head) list, heads fastest.  (Any bijection is correct; this one needs a workgroup count that is a
+  // multiple of 8, otherwise the order stays as launched.)
+  int bx = blockIdx.x, by = blockIdx.y;
+  {
+    const int n = gridDim.x * gridDim.y;
+    if ((n & 7) == 0) {
+      const int id = by * gridDim.x + bx;
+      const int lid = (id & 7) * (n >> 3) + (id >> 3);
+      bx = lid % gridDim.x;
+      by = lid / gridDim.x;
+    }
+  }
+  int w = bx;
   const int s = w % a.S; w /= a.S;
   const int h = w % a.H;
   const int seq = w / a.H;
@@ -156,32 +175,35 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
 #pragma unroll
   for (int u = 0; u < 8; ++u) acc[u] = 0.f;
   const size_t hd = (size_t)a.H * D;
-  const bf16_t* kb = a.kc + (size_t)seq * a.t_max * hd + (size_t)h * D + e0;
-  const bf16_t* vb = a.vc + (size_t)seq * a.t_max * hd + (size_t)h * D + e0;
+  // Lanes beyond the head (own == false) read the head's first features instead: their weights A / Bc are
+  // zero, so what they read only has to be mapped memory.
+  const int e0c = own ? e0 : 0;
+  const bf16_t* kb = a.kc + (size_t)seq * a.t_max * hd + (size_t)h * D + e0c;
+  const bf16_t* vb = a.vc + (size_t)seq * a.t_max * hd + (size_t)h * D + e0c;
   // this workgroup's positions [t_lo, t_hi]
   int t_lo = 0, t_hi = pq;
   if (a.ns > 1) {
     const int per = ((pq + a.ns) / a.ns + 15) & ~15;  // ceil((pq + 1) / ns) rounded up to whole rounds
-    t_lo = (int)blockIdx.y * per;
+    t_lo = by * per;
     t_hi = min(pq, t_lo + per - 1);
   }
-  constexpr int R = 2;  // positions a lane group has in flight per round
+  constexpr int R = PHI_ATTN_R;  // positions a lane group has in flight per round
+  const int fc = rotates ? f[0] : 0;
   for (int t = t_lo + grp; t <= t_hi; t += 16 * R) {
+    // every load of the round is issued whatever its position (clamped to the chunk's last one): one run
+    // of loads without branches; a position past the end is skipped when the round is consumed
     uint4 kv[R], vv[R];
     float cs[R][8], sn[R][8];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const int tt = t + 16 * r;
-      const bool in = own && tt <= t_hi;
-      kv[r] = in ? ldg16(kb + (size_t)tt * hd) : make_uint4(0, 0, 0, 0);
-      vv[r] = in ? ldg16(vb + (size_t)tt * hd) : make_uint4(0, 0, 0, 0);
+      const int tt = min(t + 16 * r, t_hi);
+      kv[r] = ldg16(kb + (size_t)tt * hd);
+      vv[r] = ldg16(vb + (size_t)tt * hd);
       if (vec8) {
         // the lane's eight features lie in one half: their angles are eight adjacent table entries
-        const bool rl = in && rotates;
-        const float* cp = a.cos + (size_t)tt * half + f[0];
-        const float* sp = a.sin + (size_t)tt * half + f[0];
-        const uint4 c0 = rl ? ldg16(cp) : one4, c1 = rl ? ldg16(cp + 4) : one4;
-        const uint4 s0 = rl ? ldg16(sp) : zero4, s1 = rl ? ldg16(sp + 4) : zero4;
+        const float* cp = a.cos + (size_t)tt * half + fc;
+        const float* sp = a.sin + (size_t)tt * half + fc;
+        const uint4 c0 = ldg16(cp), c1 = ldg16(cp + 4), s0 = ldg16(sp), s1 = ldg16(sp + 4);
         const uint32_t cu[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
         const uint32_t su[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
 #pragma unroll
@@ -192,12 +214,13 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
       } else {
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-          const bool rot_u = in && rotates && f[u] >= 0;
+          const bool rot_u = rotates && f[u] >= 0;
           cs[r][u] = rot_u ? a.cos[(size_t)tt * half + f[u]] : 1.0f;
           sn[r][u] = rot_u ? a.sin[(size_t)tt * half + f[u]] : 0.0f;
         }
       }
     }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       if (t + 16 * r > t_hi) break;  // uniform within the 16-lane group
@@ -205,8 +228,10 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
       float part = 0.f;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        part += lo_bf(ku[i]) * (cs[r][2 * i] * A[2 * i] + sn[r][2 * i] * Bc[2 * i]);
-        part += hi_bf(ku[i]) * (cs[r][2 * i + 1] * A[2 * i + 1] + sn[r][2 * i + 1] * Bc[2 * i + 1]);
+        const float c0 = (vec8 && !rotates) ? 1.0f : cs[r][2 * i], s0 = (vec8 && !rotates) ? 0.0f : sn[r][2 * i];
+        const float c1 = (vec8 && !rotates) ? 1.0f : cs[r][2 * i + 1], s1 = (vec8 && !rotates) ? 0.0f : sn[r][2 * i + 1];
+        part += lo_bf(ku[i]) * (c0 * A[2 * i] + s0 * Bc[2 * i]);
+        part += hi_bf(ku[i]) * (c1 * A[2 * i + 1] + s1 * Bc[2 * i + 1]);
       }
       part = lane_xor_sum<8>(lane_xor_sum<4>(lane_xor_sum<2>(lane_xor_sum<1>(part))));
       const float sc = part * scale;
@@ -246,7 +271,7 @@ __global__ __launch_bounds__(256) void phi_attn_kernel(PhiAttnArgs a) {
     }
     if (a.ns > 1) {
       // write-through stores: the workgroup that merges may sit on another XCD
-      float* o = a.ws + (((size_t)row * a.H + h) * a.ns + blockIdx.y) * (D + 2);
+      float* o = a.ws + (((size_t)row * a.H + h) * a.ns + by) * (D + 2);
       st_coh4(o + tid, __float_as_uint(num));
       if (tid == 0) {
         st_coh4(o + D, __float_as_uint(M));  // -inf: this chunk lies beyond the query's position
