@@ -78,6 +78,10 @@ def test_kv_append_and_attention_against_the_oracle(cuda):
     g = torch.Generator().manual_seed(2)
     for B, S, L0, H, D, rot, Tmax in ((2, 1, 9, 4, 16, 6, 32), (1, 5, 0, 2, 80, 32, 16), (3, 2, 30, 2, 128, 128, 40),
                                       (1, 1, 0, 1, 8, 2, 4), (2, 1, 299, 2, 64, 24, 300),
+                                      # many (sequence, head) pairs: workgroup counts that are multiples of 8 are
+                                      # handed to the XCDs in a re-read order
+                                      (4, 1, 300, 32, 80, 32, 320), (16, 1, 37, 8, 64, 64, 48), (2, 1, 0, 64, 16, 16, 4),
+                                      (5, 1, 130, 40, 24, 16, 131),
                                       # 16 tokens and more: query tiles of 64 against key tiles of 32
                                       (2, 40, 0, 2, 80, 32, 64), (1, 100, 29, 2, 128, 128, 160), (3, 16, 5, 4, 16, 6, 32),
                                       (1, 65, 0, 1, 64, 24, 80), (2, 33, 0, 2, 32, 16, 40), (1, 200, 0, 3, 80, 32, 200),
@@ -103,7 +107,7 @@ def test_kv_append_and_attention_against_the_oracle(cuda):
             pd = torch.tensor([L0], dtype=torch.int32, device=cuda)
             got2 = ops.phi_attn(qkvd[:, :hd], kcd, vcd, cos.to(cuda), sin.to(cuda), rot, B, S, H, D, 0, pos_dev=pd)
             assert torch.equal(got2, got)
-            for ns in (2, 5, 16):
+            for ns in (2, 5, 16, 64):
                 ws = ops.phi_attn_workspace(B, H, D, ns, cuda)
                 got3 = ops.phi_attn(qkvd[:, :hd], kcd, vcd, cos.to(cuda), sin.to(cuda), rot, B, S, H, D, L0, n_split=ns,
                                     workspace=ws)
