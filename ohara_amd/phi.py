@@ -99,7 +99,7 @@ class Phi:
     """``Phi`` (ohara/models/phi.py:155-205): ``forward(x, kv_cache, position_ids)`` and
     ``build_kv_cache``.  ``state`` uses the reference's state-dict names."""
 
-    attn_target_wgs = 1024  # decode attention: workgroups aimed at when choosing the context chunks (measured: batch 4-16)
+    attn_target_wgs = 512  # decode attention: workgroups aimed at when choosing the context chunks (measured: batch 2-16)
 
     def __init__(self, config: PhiConfig, state: dict, device="cuda", dtype=BF16):
         if dtype != BF16:
@@ -179,7 +179,7 @@ class Phi:
             new = lambda n: torch.empty(rows, n, dtype=BF16, device=self.device)
             b = dict(x=[new(d), new(d)], h=new(d), q=new(d), attn=new(d), mixer=new(d), act=new(self.ff))
             # single-token calls: the context of a (sequence, head) is spread over up to 16 workgroups,
-            # aiming at about 1024 workgroups of at least 64 positions
+            # aiming at about 512 workgroups of at least 64 positions
             heads = rows * self.config.num_attention_heads
             b["ns"] = max(1, min(16, self.config.max_sequence_length // 64, -(-self.attn_target_wgs // heads)))
             b["ws"] = ops.phi_attn_workspace(rows, self.config.num_attention_heads, self.head_dim, b["ns"], self.device)
