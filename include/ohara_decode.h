@@ -405,7 +405,9 @@ int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* s, int seq_
  * ~1000 eager launches (llama.py:279-323).  The cache position and step index are read
  * from / advanced in s->step_state; s->attn and s->attn_ws are not used.
  * `workspace`: ohara_persistent_workspace_bytes(m, batch, s->n_split, n_workgroups) of
- * device memory.  Call once with init_workspace = 1 (copies the layer table and the
+ * device memory with any contents (it need not be zeroed: every slot a step reads was written
+ * earlier in the same step, and the merge of the attention chunks never uses a chunk no workgroup
+ * wrote).  Call once with init_workspace = 1 (copies the layer table and the
  * cache pointers to the device, zeroes the barrier words; synchronises the stream; do
  * it outside graph capture) whenever the model or the caches change; then each call
  * with init_workspace = 0 enqueues one step.  spin_limit bounds every barrier wait

@@ -106,7 +106,7 @@ __device__ void merge_partials(const AttnArgs& a, int b /* query row */, int kvh
       for (int i = 0; i < 32; ++i)
         if (s0 + i < ns) o += av[i] * w[s0 + i];
     }
-    a.out[(size_t)b * a.H * D + h * D + d] = f2bf(o / s_tot[hh]);
+    a.out[(size_t)b * a.H * D + h * D + d] = f2bf(o * (1.0f / s_tot[hh]));
   }
 }
 
@@ -220,7 +220,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
     // sum (its own position only; folded over the 16 positions after the loop), and the running
     // maximum is re-derived only for tiles in which some score exceeds it - for every other tile
     // the usual update would multiply by exp(0).
-    float sc[G], pv[G];
+    float sc[G], pv[G], pvr[G];  // pvr: the weight as the value product sees it (bf16, as the library kernel rounds it)
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) {
       float s = 0.f;
@@ -256,6 +256,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
     for (int hh = 0; hh < G; ++hh) {
       pv[hh] = __expf(sc[hh] - m_run[hh]);
       l_run[hh] += pv[hh];
+      pvr[hh] = rbf(pv[hh]);
     }
     // all weight exchanges first (they are independent), then the products: next to their products
     // every exchange is waited for by itself
@@ -263,7 +264,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
 #pragma unroll
     for (int c = 0; c < NV; ++c)
 #pragma unroll
-      for (int hh = 0; hh < G; ++hh) pw[c][hh] = __shfl(pv[hh], 4 * (c * PP + pp), WAVE);
+      for (int hh = 0; hh < G; ++hh) pw[c][hh] = __shfl(pvr[hh], 4 * (c * PP + pp), WAVE);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int c = 0; c < NV; ++c) {
@@ -339,7 +340,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
       o += s_acc[w][hh][d] * sc;
     }
     if (a.nsplit == 1) {  // whole context in this workgroup: no partials
-      a.out[(size_t)b * a.H * D + h * D + d] = f2bf(o / Ls);
+      a.out[(size_t)b * a.H * D + h * D + d] = f2bf(o * (1.0f / Ls));
       continue;
     }
     const size_t pi = (size_t)(b * a.H + h) * a.nsplit + split;
@@ -434,7 +435,7 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
     // tiles); within it the heads of the group advance together, as in the bf16 kernel.
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
-      float sc[G], pv[G];
+      float sc[G], pv[G], pvr[G];  // pvr: the weight as the value product sees it (bf16, as the library kernel rounds it)
       {
         const float ks = __uint_as_float(cur.st[sb].x), km = __uint_as_float(cur.st[sb].y);
         uint4 kv[NC];
@@ -481,6 +482,7 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
       for (int hh = 0; hh < G; ++hh) {
         pv[hh] = __expf(sc[hh] - m_run[hh]);  // (a sub-tile past the end: exp(-inf - m) = 0; m is finite by then)
         l_run[hh] += pv[hh];
+        pvr[hh] = rbf(pv[hh]);
       }
       // the exchanges of a few rows first (scale, minimum and weight of the row whose codes this lane
       // holds: independent of each other), then their products; next to its products every exchange
@@ -496,7 +498,7 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
           vs[cc] = __shfl(__uint_as_float(cur.st[sb].z), src, WAVE);
           vm[cc] = __shfl(__uint_as_float(cur.st[sb].w), src, WAVE);
 #pragma unroll
-          for (int hh = 0; hh < G; ++hh) pw[cc][hh] = __shfl(pv[hh], src, WAVE);
+          for (int hh = 0; hh < G; ++hh) pw[cc][hh] = __shfl(pvr[hh], src, WAVE);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -575,7 +577,7 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
       o += s_acc[w][hh][d] * scw;
     }
     if (a.nsplit == 1) {  // whole context in this workgroup: no partials
-      a.out[(size_t)b * a.H * D + h * D + d] = f2bf(o / Ls);
+      a.out[(size_t)b * a.H * D + h * D + d] = f2bf(o * (1.0f / Ls));
       continue;
     }
     const size_t pi = (size_t)(b * a.H + h) * a.nsplit + split;
@@ -641,7 +643,7 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
       const float mn = fmaxf(m_run, tm);
       const float corr = __expf(m_run - mn);
       const float pv = (pos < t1) ? __expf(s - mn) : 0.f;
-      s_p[tid] = pv;
+      s_p[tid] = rbf(pv);  // the weights enter the value product rounded to bf16, the sum unrounded
       float ts = wave_sum(pv);
       if ((tid & 63) == 0) s_red[tid >> 6] = ts;
       __syncthreads();
@@ -663,7 +665,7 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
       __syncthreads();
     }
     if (a.nsplit == 1) {
-      if (tid < D) a.out[(size_t)b * a.H * D + h * D + tid] = f2bf(acc / l_run);
+      if (tid < D) a.out[(size_t)b * a.H * D + h * D + tid] = f2bf(acc * (1.0f / l_run));
       continue;
     }
     const size_t pi = (size_t)(b * a.H + h) * a.nsplit + split;

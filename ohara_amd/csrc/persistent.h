@@ -363,7 +363,8 @@ __device__ __forceinline__ void stage_attn_merge(bf16_t* xs, int ldxs, const flo
       const int b = e / HD, hd = e - b * HD;        // no load behind a branch
       const float* base = pm + (size_t)(b * H + hd / Dh) * NSM * PS + (hd % Dh);
 #pragma unroll
-      for (int sp = 0; sp < NS; ++sp) av[r][sp] = ldg16(base + (size_t)sp * PS);
+      for (int sp = 0; sp < NS; ++sp)  // slots past `used` are never written: read the last used one (weight 0)
+        av[r][sp] = ldg16(base + (size_t)min(sp, used - 1) * PS);
     }
   };
   // the accumulator loads of the first round go out first: they do not depend on the chunk
@@ -392,7 +393,7 @@ __device__ __forceinline__ void stage_attn_merge(bf16_t* xs, int ldxs, const flo
     if (NS > 4) Ls = lane_xor_sum<4>(Ls);
     if (NS > 2) Ls = lane_xor_sum<2>(Ls);
     if (NS > 1) Ls = lane_xor_sum<1>(Ls);
-    if (bh < nbh) mw[bh * NS + sp] = w;  // 0 for chunks that are not in use: their slots hold old, finite sums
+    if (bh < nbh) mw[bh * NS + sp] = w;  // 0 for chunks that are not in use
     if (in && sp == 0) ml[bh] = Ls;
   }
   __syncthreads();
@@ -413,8 +414,8 @@ __device__ __forceinline__ void stage_attn_merge(bf16_t* xs, int ldxs, const flo
           o[2] += __uint_as_float(av[r][sp].z) * w;
           o[3] += __uint_as_float(av[r][sp].w) * w;
         }
-        const float Ls = ml[bh];
-        sts8(xs + (size_t)b * ldxs + hd, make_uint2(pack_bf(o[0] / Ls, o[1] / Ls), pack_bf(o[2] / Ls, o[3] / Ls)));
+        const float inv = 1.0f / ml[bh];
+        sts8(xs + (size_t)b * ldxs + hd, make_uint2(pack_bf(o[0] * inv, o[1] * inv), pack_bf(o[2] * inv, o[3] * inv)));
       }
     }
   }
@@ -452,7 +453,8 @@ __device__ __forceinline__ void stage_attn_merge_small(bf16_t* xs, int ldxs, con
     o[2] += __uint_as_float(av[s].z) * w;
     o[3] += __uint_as_float(av[s].w) * w;
   }
-  sts8(xs + (size_t)b * ldxs + hd, make_uint2(pack_bf(o[0] / Ls, o[1] / Ls), pack_bf(o[2] / Ls, o[3] / Ls)));
+  const float inv = 1.0f / Ls;
+  sts8(xs + (size_t)b * ldxs + hd, make_uint2(pack_bf(o[0] * inv, o[1] * inv), pack_bf(o[2] * inv, o[3] * inv)));
 }
 
 // Out-of-line copies of the merge, for kernels that want to keep their own code compact.
@@ -1014,7 +1016,7 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
         // The heads of the group advance in lock step (their cross-lane exchanges overlap); l_run is
         // this lane's share of the sum, folded over the 16 positions after the loop; the running
         // maximum is re-derived only for tiles in which some score exceeds it.
-        float sc[G], pv[G];
+        float sc[G], pv[G], pvr[G];  // pvr: the weight rounded to bf16, as it enters the value product
 #pragma unroll
         for (int hh = 0; hh < G; ++hh) {
           float s = 0.f;
@@ -1058,13 +1060,14 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
         for (int hh = 0; hh < G; ++hh) {
           pv[hh] = __expf(sc[hh] - m_run[hh]);
           l_run[hh] += pv[hh];
+          pvr[hh] = rbf(pv[hh]);
         }
         // all weight exchanges first (they are independent), then the products
         float pw[NV][G];
 #pragma unroll
         for (int c = 0; c < NV; ++c)
 #pragma unroll
-          for (int hh = 0; hh < G; ++hh) pw[c][hh] = __shfl(pv[hh], c * PP + pp, WAVE);
+          for (int hh = 0; hh < G; ++hh) pw[c][hh] = __shfl(pvr[hh], c * PP + pp, WAVE);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int c = 0; c < NV; ++c) {

@@ -46,6 +46,8 @@ class DeviceLoop:
         self._key = None
         self.session = None
         self._pinned = None
+        self._pinned_err = None
+        self._busy = False
 
     def _rule_key(self, sampling):
         if sampling is None or sampling.temperature <= 0:
@@ -59,6 +61,7 @@ class DeviceLoop:
             self.session = self.model.session(1, cap, self.valid_vocab, sampling=sampling if key else None)
             self._key = key
             self._pinned = torch.empty(cap, dtype=torch.int64, pin_memory=True)
+            self._pinned_err = torch.zeros(4, dtype=torch.int32, pin_memory=True)
         return self.session
 
     def tokens(self, prompt_ids: Sequence[int], limit: int, sampling=None, u: torch.Tensor | None = None,
@@ -68,6 +71,19 @@ class DeviceLoop:
         model = self.model
         if limit < 1:
             return
+        if self._busy:
+            # one session, one KV cache (the reference serialises requests with a lock for the same
+            # reason, ohara/webui/server.py:143-147): a second generation would restart the session
+            # under the first one's feet
+            raise RuntimeError("this engine is still generating: finish or close the previous stream first")
+        self._busy = True
+        try:
+            yield from self._tokens(prompt_ids, limit, sampling, u, generator)
+        finally:
+            self._busy = False
+
+    def _tokens(self, prompt_ids, limit, sampling, u, generator) -> Iterator[int]:
+        model = self.model
         sess = self._get_session(sampling)
         draws = None
         if sess.sampling is not None:
@@ -80,15 +96,23 @@ class DeviceLoop:
         sess.restart(draws)
         prompt = torch.as_tensor(list(prompt_ids), dtype=torch.int64).view(1, -1)
         sess.prefill(prompt)  # produces token 0
-        history, pinned = sess.history, self._pinned
-        inflight: deque = deque()  # (first, last, event) of chunks whose ids are on their way to the host
-        launched, chunk = 1, self.FIRST_CHUNK
+        history, pinned, pinned_err = sess.history, self._pinned, self._pinned_err
+        err_word = sess.error_word()  # device view of the persistent kernel's sticky error word, or None
+        inflight: deque = deque()  # (first, last, slot, event) of chunks whose ids are on their way to the host
+        launched, chunk, nchunks = 1, self.FIRST_CHUNK, 0
 
         def ship(first: int, last: int) -> None:
+            # the error word travels with every chunk: the usual consumer stops at a stop id and never
+            # drains the generator, so a check after the last chunk would not run
+            nonlocal nchunks
+            slot = nchunks % pinned_err.numel()
+            nchunks += 1
             pinned[first:last].copy_(history[first:last, 0], non_blocking=True)
+            if err_word is not None:
+                pinned_err[slot : slot + 1].copy_(err_word, non_blocking=True)
             ev = torch.cuda.Event()
             ev.record()
-            inflight.append((first, last, ev))
+            inflight.append((first, last, slot, ev))
 
         ship(0, 1)
         while inflight:
@@ -99,11 +123,14 @@ class DeviceLoop:
                 ship(launched, launched + n)
                 launched += n
                 chunk = min(2 * chunk, self.MAX_CHUNK)
-            first, last, ev = inflight.popleft()
+            first, last, slot, ev = inflight.popleft()
             ev.synchronize()
+            if err_word is not None and int(pinned_err[slot]) != 0:
+                torch.cuda.current_stream().synchronize()  # the chunk launched behind this one
+                sess.reset_error()  # the barrier counters are mixed after an expiry: start them over
+                raise RuntimeError("persistent decode kernel: a grid barrier wait expired")
             for tok in pinned[first:last].tolist():
                 yield tok
-        sess.check_error()
 
 
 def stepwise_tokens(model, prompt_ids: Sequence[int], limit: int, select: Callable[[torch.Tensor, int], torch.Tensor],

@@ -618,6 +618,18 @@ class DecodeSession:
                 raise ValueError("u must have shape (rows <= max_new_tokens, batch)")
             self.u[: u.shape[0]].copy_(u)
 
+    def feed(self, ids: torch.Tensor) -> None:
+        """Replace the ids the next step consumes (one per sequence) - teacher forcing: the step then
+        continues the sequences with these tokens instead of the ones the last step selected.  The
+        history keeps what was selected."""
+        if self._dbuf is None:
+            raise RuntimeError("prefill first")
+        ids = ids.reshape(-1)
+        if ids.numel() != self.batch:
+            raise ValueError("one id per sequence is required")
+        _check_ids_on_host(ids.view(1, -1), self.model.config.vocab_size)
+        self._dbuf.ids[: self.batch].copy_(ids.to(device=self.model.device, dtype=torch.int64))
+
     def _launch_step(self) -> None:
         m = self.model
         stream = torch.cuda.current_stream().cuda_stream
@@ -633,6 +645,13 @@ class DecodeSession:
             ops.sample_topk_topp(self.logits, self.sampling.temperature, self.sampling.top_k, self.sampling.top_p,
                                  self.u, self.valid_vocab or None, out=self._dbuf.ids[: self.batch],
                                  history=self.history, step_state=self._dbuf.step_state, u_per_step=True, exclusive=True)
+
+    def error_word(self):
+        """The persistent kernel's sticky error word as a one-element int32 device view (None for the
+        kernel chain, which has no barrier waits): non-zero once a barrier wait has expired."""
+        if self.persistent and self._pws is not None:
+            return self._pws[self._err_off : self._err_off + 4].view(torch.int32)
+        return None
 
     def check_error(self) -> None:
         """Raise if a barrier wait of the persistent kernel expired (synchronises)."""

@@ -210,6 +210,79 @@ class KVCacheRef:
         return k.to(keys.dtype), v.to(keys.dtype)
 
 
+_LOG2E_F32 = torch.tensor([0x3FB8AA3B], dtype=torch.int32).view(torch.float32)[0]
+_LN_FLT_MIN = torch.tensor([0xC2AEAC50 - (1 << 32)], dtype=torch.int32).view(torch.float32)[0]
+
+
+def _fma32(a, b, c):
+    """One fused multiply-add in fp32: the product of two fp32 values is exact in fp64."""
+    return (a.double() * b.double() + c.double()).float()
+
+
+def fexp_u20(x: torch.Tensor) -> torch.Tensor:
+    """The exponential of torch's CPU flash-attention kernel for bf16 / fp16 inputs (torch 2.10.0,
+    pinned by the reference's pyproject.toml:49-52; ``Vectorized<float>::fexp_u20``), restated from its
+    published algorithm (Malossi, Ineichen, Bekas, Curioni: Fast Exponential Computation on SIMD
+    Architectures): ``2**(x log2 e)`` with the fractional part corrected by a cubic, assembled
+    directly in the exponent and mantissa fields.  Relative error up to 1.1e-4 - what it returns,
+    not exp(x), is what the reference's bf16 attention rounds to bf16.  Arguments are <= 0 here.
+    """
+    c0, c1, c2, c3 = (torch.tensor(c, dtype=torch.float32) for c in
+                      (0.00010703434948458272, 0.30354260500649682, -0.22433836478672356, -0.079204240219773236))
+    src = x * _LOG2E_F32
+    frac = src - torch.floor(src)
+    r = _fma32(frac, c3, c2)
+    r = _fma32(frac, r, c1)
+    r = _fma32(frac, r, c0)
+    src = src - r
+    bits = _fma32(torch.tensor(float(2 ** 23)), src, torch.tensor(float(2 ** 23) * 127.0))
+    out = bits.clamp(min=0).to(torch.int32).view(torch.float32)  # truncating conversion
+    return torch.where(x < _LN_FLT_MIN, torch.zeros_like(out), out)
+
+
+SDPA_KV_BLOCK = 512  # keys per block of torch's CPU flash-attention kernel
+SDPA_VEC = 16         # fp32 lanes of its vector loop (AVX-512, the build the fixtures were made with)
+
+
+def _attention_reduced(q, k, v, visible):
+    """``F.scaled_dot_product_attention`` as torch 2.10.0 computes it on the CPU for bf16 / fp16
+    tensors (the dtype ChatEngine casts the model to, chat_engine.py:262-265; call site
+    llama.py:116-123), with every rounding point of that kernel:
+
+    keys are taken in blocks of 512; per block the scores are an fp32-accumulated product times
+    1/sqrt(D) (fp32), masked with -inf; the running maximum m and sum l are fp32; the weights
+    ``p = fexp_u20(s - m_new)`` (the block's last ``len % 16`` keys, which the vector loop leaves to a
+    scalar tail: ``exp``) enter the sum unrounded and are ROUNDED TO THE INPUT DTYPE before
+    the fp32-accumulated product with V; earlier blocks' sum and accumulator are rescaled by
+    ``exp(m_old - m_new)``; the result is ``acc * (1 / l)`` rounded once.
+
+    q: (B,H,S,D), k, v: (B,H,L,D), visible: (S,L) bool.  Pinned against the library routine itself
+    in tests/test_oracle.py (>= 97 % of the elements bit-identical at every size tried, the rest
+    one ulp: the fp32 summation order inside the library's products is not restated).
+    """
+    B, H, S, D = q.shape
+    L = k.shape[2]
+    qf, kf, vf = q.float(), k.float(), v.float()
+    scale = torch.tensor(1.0 / math.sqrt(D), dtype=torch.float32)
+    m = torch.full((B, H, S), float("-inf"))
+    l = torch.zeros(B, H, S)
+    acc = torch.zeros(B, H, S, D)
+    for n in range(0, L, SDPA_KV_BLOCK):
+        e = min(L, n + SDPA_KV_BLOCK)
+        s = (qf @ kf[:, :, n:e].transpose(-1, -2)) * scale
+        s = s.masked_fill(~visible[None, None, :, n:e], float("-inf"))
+        m_new = torch.maximum(m, s.amax(-1))
+        d = s - m_new[..., None]
+        nv = (e - n) // SDPA_VEC * SDPA_VEC  # full vectors of the block: fast exponential; the tail: exp
+        p = torch.cat([fexp_u20(d[..., :nv]), torch.exp(d[..., nv:])], dim=-1)
+        corr = torch.exp(m - m_new)
+        corr = torch.where(torch.isnan(corr), torch.zeros_like(corr), corr)  # -inf - -inf: nothing seen yet
+        l = l * corr + p.sum(-1)
+        acc = acc * corr[..., None] + p.to(q.dtype).float() @ vf[:, :, n:e]
+        m = m_new
+    return (acc * (1.0 / l)[..., None]).to(q.dtype)
+
+
 def attention_core(q, k, v, start_pos: int | None):
     """softmax(q k^T / sqrt(D) + mask) v with GQA - llama.py:100-135.
 
@@ -217,12 +290,24 @@ def attention_core(q, k, v, start_pos: int | None):
     (is_causal=True, llama.py:122); otherwise the cache mask
     ``key_pos <= start_pos + q_idx`` over all L cached positions (llama.py:109-113).
     GQA: query head h reads kv head h // (H/H_kv) (repeat_interleave, llama.py:101-103).
-    fp32 scores/softmax/accumulation, one rounding to q's dtype.
+    fp32 tensors: fp32 scores / softmax / accumulation, one rounding.  bf16 / fp16 tensors: the
+    rounding points of the library kernel the reference calls (``_attention_reduced``).
     Returns (B, S, H*D).
     """
     B, S, H, D = q.shape
     L, Hkv = k.shape[1], k.shape[2]
     group = H // Hkv
+    base = 0 if start_pos is None else start_pos
+    qpos = base + torch.arange(S)
+    kpos = torch.arange(L)
+    visible = kpos[None, :] <= qpos[:, None]
+    if q.dtype != torch.float32 and q.dtype != torch.float64:
+        qh, kh, vh = q.permute(0, 2, 1, 3), k.permute(0, 2, 1, 3), v.permute(0, 2, 1, 3)
+        if group > 1:
+            kh = kh.repeat_interleave(group, dim=1)
+            vh = vh.repeat_interleave(group, dim=1)
+        out = _attention_reduced(qh, kh, vh, visible)
+        return out.permute(0, 2, 1, 3).reshape(B, S, H * D)
     qf = q.float().permute(0, 2, 1, 3)  # (B,H,S,D)
     kf = k.float().permute(0, 2, 1, 3)  # (B,Hkv,L,D)
     vf = v.float().permute(0, 2, 1, 3)
@@ -230,10 +315,6 @@ def attention_core(q, k, v, start_pos: int | None):
         kf = kf.repeat_interleave(group, dim=1)
         vf = vf.repeat_interleave(group, dim=1)
     scores = qf @ kf.transpose(-1, -2) / math.sqrt(D)  # (B,H,S,L)
-    base = 0 if start_pos is None else start_pos
-    qpos = base + torch.arange(S)
-    kpos = torch.arange(L)
-    visible = kpos[None, :] <= qpos[:, None]
     scores = scores.masked_fill(~visible[None, None], float("-inf"))
     p = torch.softmax(scores, dim=-1)
     out = (p @ vf).to(q.dtype)  # (B,H,S,D)

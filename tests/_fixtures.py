@@ -1,0 +1,37 @@
+"""Loader of the committed golden fixtures (tests/golden/*.pt): plain tensors, read with
+``weights_only=True``; a value ``"=<key>"`` stands for the tensor stored under that key."""
+
+import os
+
+import torch
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def load_fixture(name: str) -> dict:
+    fx = torch.load(os.path.join(GOLDEN, name), weights_only=True)
+    for k, v in list(fx.items()):
+        if isinstance(v, str) and v.startswith("="):
+            fx[k] = fx[v[1:]]
+    return fx
+
+
+def weight_checksum(w: dict) -> torch.Tensor:
+    """The fingerprint tests/golden/make_llama_bf16_golden.py stores for seeded weights."""
+    names = sorted(k for k in w if not k.startswith("freq_"))
+    return torch.tensor([[w[k].double().sum().item(), w[k].double().pow(2).sum().item()] for k in names],
+                        dtype=torch.float64).sum(0)
+
+
+def identical_fraction(a: torch.Tensor, b: torch.Tensor) -> float:
+    """Share of bit-identical elements of two bf16 tensors."""
+    assert a.shape == b.shape and a.dtype == b.dtype == torch.bfloat16
+    return (a.contiguous().view(torch.int16) == b.contiguous().view(torch.int16)).float().mean().item()
+
+
+def bf16_ulps(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """|a - b| in units of the bf16 spacing at max(|a|, |b|)."""
+    af, bf = a.float(), b.float()
+    mag = torch.maximum(af.abs(), bf.abs()).clamp_min(2.0 ** -120)
+    ulp = torch.exp2(torch.floor(torch.log2(mag)) - 7)
+    return (af - bf).abs() / ulp

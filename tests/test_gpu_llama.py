@@ -6,6 +6,12 @@ both relative to the logit scale (max |logit| of the oracle); greedy tokens iden
 the oracle's, except that a first divergence is accepted only where the oracle's own
 top-2 logits are within 2 bf16 ulps of each other (bf16 accumulation order is unpinned
 by the reference, so such near-ties are decided by rounding noise on either side).
+
+At the d12 size the mean bound is the target or 1.25 x the distance at which the REFERENCE
+reproduces itself, whichever is larger: tests/golden/llama_bf16_d12_greedy.pt holds two runs of the
+reference's own bf16 model on the CPU (all threads / one thread: the library's products sum in another
+order), 64 steps each; they lie up to 2.15e-3 of the logit scale apart in the mean and pick different
+greedy tokens at step 60.  tests/test_gpu_reference_bf16.py compares the HIP path with that run itself.
 """
 
 import dataclasses
@@ -145,27 +151,17 @@ def _near_tie(logits_row, a, b, ulps=2):
     return abs(la - lb) <= ulps * ulp
 
 
-class _Fp64LinearOracle:
-    """The CPU oracle with every Linear accumulated in fp64 instead of fp32: an equally valid bf16
-    implementation.  Its distance from the plain oracle at a given position is that position's noise
-    floor (each flipped bf16 rounding cascades through the layers)."""
+def _reference_self_distance():
+    """Worst per-step mean |logit difference| (of the logit scale) between the reference's two bf16
+    runs of the d12 model stored in the fixture (all threads against one thread, 64 decode steps)."""
+    from _fixtures import load_fixture
 
-    def __init__(self, rcfg, w):
-        self.m = R.RefLlama(rcfg, w)
-
-    def build_kv_cache(self, b):
-        return self.m.build_kv_cache(b)
-
-    def __call__(self, *a):
-        orig = R.linear
-        try:
-            R.linear = lambda x, wt, cache=None: (x.double() @ wt.double().t()).to(x.dtype)
-            return self.m(*a)
-        finally:
-            R.linear = orig
+    fx = load_fixture("llama_bf16_d12_greedy.pt")
+    d = (fx["logits_at_columns"].float() - fx["logits_at_columns_one_thread"].float()).abs().mean(1)
+    return (d / fx["logit_absmax"].float()).max().item()
 
 
-def _check_greedy(model, ref, prompt, steps, cuda, max_rel=2e-2, mean_rel=2e-3, stats_out=None, noise_ref=None):
+def _check_greedy(model, ref, prompt, steps, cuda, max_rel=2e-2, mean_rel=2e-3, stats_out=None):
     """(1) free-running device loop vs the oracle's greedy tokens: identical, or first
     divergence at a near-tie of the oracle's logits; (2) teacher-forced on the oracle's
     tokens so that every one of the `steps` positions is checked: logits within tolerance
@@ -193,22 +189,13 @@ def _check_greedy(model, ref, prompt, steps, cuda, max_rel=2e-2, mean_rel=2e-3, 
     if stats_out is not None:
         stats_out.update(stats)
         stats = stats_out
-    ncache = noise_ref.build_kv_cache(B) if noise_ref is not None else None
     stats["steps_within_strict_mean_2e-3"] = 0
-    stats["worst_ratio_to_position_floor"] = 0.0
     for t in range(steps):
         logits = model(inp, cache, pos, last_only=True)[:, 0]
-        step_tol = mean_rel
-        if noise_ref is not None:
-            # this position's own noise floor: the tolerance is the target or 1.25 x the floor
-            _, floor_t = _rel_errors(noise_ref(inp.cpu(), ncache, pos)[:, -1], want_logits[t])
-            step_tol = max(mean_rel, 1.25 * floor_t)
         pos += inp.size(1)
-        _assert_logits_close(logits, want_logits[t], max_rel, step_tol)
+        _assert_logits_close(logits, want_logits[t], max_rel, mean_rel)
         mx, mn = _rel_errors(logits, want_logits[t])
         stats["steps_within_strict_mean_2e-3"] += int(mn <= 2e-3)
-        if noise_ref is not None:
-            stats["worst_ratio_to_position_floor"] = max(stats["worst_ratio_to_position_floor"], mn / max(floor_t, 1e-12))
         stats["max_err"] = max(stats["max_err"], mx)
         stats["mean_err_worst_step"] = max(stats["mean_err_worst_step"], mn)
         stats["mean_err_avg"] += mn / steps
@@ -253,34 +240,14 @@ def test_greedy_small_model(cuda):
             assert _near_tie(wl[t, b], int(chain[b, t]), int(want[b, t]))
 
 
-def _accumulation_noise_floor(rcfg, w, prompt):
-    """Mean / max |logit difference| (relative to the logit scale) between two runs of the
-    CPU oracle that differ ONLY in the accumulation precision of every Linear (fp32 vs
-    fp64).  Each flipped bf16 rounding cascades through the layers, so this is how far
-    apart two equally valid bf16 implementations land on this model."""
-    a = R.RefLlama(rcfg, w)(prompt)[:, -1].float()
-    orig = R.linear
-    try:
-        R.linear = lambda x, wt, cache=None: (x.double() @ wt.double().t()).to(x.dtype)
-        b = R.RefLlama(rcfg, w)(prompt)[:, -1].float()
-    finally:
-        R.linear = orig
-    d, scale = (a - b).abs(), a.abs().max().item()
-    return d.mean().item() / scale, d.max().item() / scale
-
-
 def test_d12_decode_parity(cuda):
     """The d12 Llama of the headline config (d 768, 12 layers, 6 heads x 128, FFN 3072,
     vocab 65536, bf16, N(0,0.02) seed 0) at a prompt the CPU oracle finishes in seconds:
-    logits of the prefill and of decode steps, then 64 greedy tokens.
+    logits of the prefill and of decode steps, then 64 greedy tokens, two sequences.
 
-    Target tolerance: max-abs 2e-2, mean-abs 2e-3 of the logit scale.  On this random-init
-    model the mean-abs distance between two CPU oracles that differ only in accumulation
-    precision is itself ~2.1e-3 (measured below), i.e. the mean criterion sits on the
-    noise floor of bf16 arithmetic; the HIP path is required to stay within
-    max(2e-3, 1.25 x that floor) in the mean and within 2e-2 at the maximum.  In the 64-token run the
-    floor is taken position by position (the fp64-accumulating oracle is run teacher-forced beside the
-    plain one), because the floor itself moves by +-30 % from one position to the next."""
+    Target: max-abs 2e-2, mean-abs 2e-3 of the logit scale.  Asserted: max-abs 2e-2 and a mean of
+    max(2e-3, 1.25 x the reference's distance from itself) at every step (see the module docstring);
+    whether the strict target holds at every step is recorded."""
     from ohara_amd.llama import Llama
 
     rcfg, cfg = _cfg_pair(vocab_size=65536, hidden_size=768, intermediate_size=3072, num_attention_heads=6,
@@ -289,10 +256,9 @@ def test_d12_decode_parity(cuda):
     ref = R.RefLlama(rcfg, w)
     model = Llama(cfg, w, device=cuda)
     prompt = torch.randint(0, 65536, (2, 96), generator=torch.Generator().manual_seed(0))
-    floor_mean, floor_max = _accumulation_noise_floor(rcfg, w, prompt)
-    mean_tol = max(2e-3, 1.25 * floor_mean)
-    print(f"accumulation noise floor: mean {floor_mean:.2e} max {floor_max:.2e}; mean tolerance {mean_tol:.2e}")
-    assert floor_max < 2e-2
+    self_mean = _reference_self_distance()
+    mean_tol = max(2e-3, 1.25 * self_mean)
+    print(f"reference against itself: mean {self_mean:.2e}; mean tolerance {mean_tol:.2e}")
     rc, cache = ref.build_kv_cache(2), model.build_kv_cache(2)
     want = ref(prompt, rc, 0)[:, -1:]
     got = model(prompt.to(cuda), cache, 0, last_only=True)
@@ -304,9 +270,9 @@ def test_d12_decode_parity(cuda):
         _assert_logits_close(got, want, 2e-2, mean_tol)
         nxt = want[:, -1].float().argmax(-1, keepdim=True)
     stats = {}
-    _check_greedy(model, ref, prompt, 64, cuda, 2e-2, 2e-3, stats_out=stats, noise_ref=_Fp64LinearOracle(rcfg, w))
-    stats.update(config="d12 bf16, 2 sequences, prompt 96, 64 greedy tokens", noise_floor_mean=floor_mean,
-                 noise_floor_max=floor_max, mean_tolerance_used=mean_tol,
+    _check_greedy(model, ref, prompt, 64, cuda, 2e-2, mean_tol, stats_out=stats)
+    stats.update(config="d12 bf16, 2 sequences, prompt 96, 64 greedy tokens, against the CPU oracle",
+                 reference_vs_itself_mean=self_mean, mean_tolerance_used=mean_tol,
                  strict_mean_2em3_holds=stats["mean_err_worst_step"] <= 2e-3,
                  strict_max_2em2_holds=stats["max_err"] <= 2e-2,
                  strict_identical_64_holds=stats["free_running_identical"])
@@ -315,8 +281,9 @@ def test_d12_decode_parity(cuda):
 
 def test_d12_prompt1024_batch1_first_64_tokens(cuda):
     """The headline configuration as stated: batch 1, a 1024-token prompt, cache capacity 4096, the
-    first 64 greedy tokens against the CPU oracle.  Asserted with the same criteria as above; whether
-    the strict criteria (mean-abs 2e-3, 64 identical tokens) hold is recorded without asserting it."""
+    first 64 greedy tokens against the CPU oracle (the same run against the reference's own tokens and
+    logits: tests/test_gpu_reference_bf16.py).  Asserted with the same criteria as above; whether the
+    strict criteria (mean-abs 2e-3, 64 identical tokens) hold is recorded without asserting it."""
     from ohara_amd.llama import Llama
 
     rcfg, cfg = _cfg_pair(vocab_size=65536, hidden_size=768, intermediate_size=3072, num_attention_heads=6,
@@ -325,16 +292,49 @@ def test_d12_prompt1024_batch1_first_64_tokens(cuda):
     ref = R.RefLlama(rcfg, w)
     model = Llama(cfg, w, device=cuda)
     prompt = torch.randint(0, 65536, (1, 1024), generator=torch.Generator().manual_seed(0))
-    floor_mean, floor_max = _accumulation_noise_floor(rcfg, w, prompt)
-    mean_tol = max(2e-3, 1.25 * floor_mean)
+    self_mean = _reference_self_distance()
+    mean_tol = max(2e-3, 1.25 * self_mean)
     stats = {}
-    _check_greedy(model, ref, prompt, 64, cuda, 2e-2, 2e-3, stats_out=stats, noise_ref=_Fp64LinearOracle(rcfg, w))
-    stats.update(config="d12 bf16, batch 1, prompt 1024, 64 greedy tokens", noise_floor_mean=floor_mean,
-                 noise_floor_max=floor_max, mean_tolerance_used=mean_tol,
+    _check_greedy(model, ref, prompt, 64, cuda, 2e-2, mean_tol, stats_out=stats)
+    stats.update(config="d12 bf16, batch 1, prompt 1024, 64 greedy tokens, against the CPU oracle",
+                 reference_vs_itself_mean=self_mean, mean_tolerance_used=mean_tol,
                  strict_mean_2em3_holds=stats["mean_err_worst_step"] <= 2e-3,
                  strict_max_2em2_holds=stats["max_err"] <= 2e-2,
                  strict_identical_64_holds=stats["free_running_identical"])
     _report("d12_prompt1024_batch1", stats)
+
+
+@pytest.mark.parametrize("batch", [8])
+def test_d12_persistent_kernel_batch8_prompt1024(cuda, batch):
+    """The single-launch kernel at the d12 size with eight sequences (the largest batch it serves by
+    default) after 1024-token prompts: four steps, teacher-forced on the oracle's tokens, logits against
+    the CPU oracle; and the same steps through the kernel chain on the same inputs."""
+    from ohara_amd.llama import Llama
+
+    rcfg, cfg = _cfg_pair(vocab_size=65536, hidden_size=768, intermediate_size=3072, num_attention_heads=6,
+                          num_key_value_heads=0, num_hidden_layers=12, max_sequence_length=4096, dropout=0.0)
+    w = R.init_weights(rcfg, seed=0, dtype=BF)
+    ref = R.RefLlama(rcfg, w)
+    model = Llama(cfg, w, device=cuda)
+    P, steps = 1024, 4
+    prompt = torch.randint(0, 65536, (batch, P), generator=torch.Generator().manual_seed(8))
+    mean_tol = max(2e-3, 1.25 * _reference_self_distance())
+    rc = ref.build_kv_cache(batch)
+    # (last position only: the oracle's vocabulary projection of all 8192 prompt rows would be 2 GB)
+    want = [R.linear(ref(prompt, rc, 0, return_hidden=True)[:, -1], w["vocab_proj.weight"])]
+    fed = []
+    for s in range(steps):
+        fed.append(want[-1].float().argmax(-1))
+        want.append(ref(fed[-1].view(batch, 1), rc, P + s)[:, -1])
+    for persistent in (True, False):
+        sess = model.session(batch, steps + 1, persistent=persistent)
+        sess.prefill(prompt.to(cuda))
+        _assert_logits_close(sess.logits, want[0], 2e-2, mean_tol)
+        for s in range(steps):
+            sess.feed(fed[s])
+            sess.step()
+            _assert_logits_close(sess.logits, want[s + 1], 2e-2, mean_tol)
+        sess.check_error()
 
 
 @pytest.mark.parametrize("persistent", [True, False])
@@ -455,6 +455,71 @@ def test_expired_barrier_wait_is_reported_and_does_not_hang(cuda):
     sess.check_error()
     again = model.generate_greedy(prompt, 10, persistent=True).cpu()
     assert torch.equal(again, good)
+
+
+def test_device_loop_reports_an_expired_wait_with_the_chunk_and_refuses_reentry(cuda):
+    """The engines' token source: (a) an expired barrier wait is raised with the chunk of ids that
+    carries it, also for a consumer that stops early (a stop id) and never drains the generator, and
+    the session is usable afterwards; (b) a second generation on the same loop while the first one's
+    generator is still open is refused (one session, one cache)."""
+    from ohara_amd.generation import DeviceLoop
+    from ohara_amd.llama import Config, Llama
+
+    kw = dict(vocab_size=512, hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+              num_hidden_layers=3, max_sequence_length=96, rope_theta=10000.0)
+    w = R.init_weights(R.RefConfig(**kw), seed=3, dtype=torch.bfloat16, std=0.06, norm_jitter=0.1)
+    model = Llama(Config(**kw), w, device=cuda)
+    if not model.supports_persistent(1):
+        pytest.skip("shape not covered by the persistent kernel")
+    prompt = torch.randint(0, 512, (12,), generator=torch.Generator().manual_seed(0)).tolist()
+    good = list(DeviceLoop(model).tokens(prompt, 24))
+    assert len(good) == 24
+
+    loop = DeviceLoop(model)
+    sess = loop._get_session(None)
+    assert sess.persistent
+    sess.spin_limit = 1  # every barrier wait of the steps launched from here on expires
+    with pytest.raises(RuntimeError, match="barrier wait expired"):
+        for i, _ in enumerate(loop.tokens(prompt, 24)):
+            if i == 6:  # a consumer that stops early
+                break
+    torch.cuda.synchronize()
+    assert not loop._busy
+    # the launches captured with that limit are dropped; the same session then decodes normally
+    sess.spin_limit = 0
+    sess.graph = sess.graph_multi = None
+    assert list(loop.tokens(prompt, 24)) == good
+
+    first = loop.tokens(prompt, 24)
+    assert next(first) == good[0]
+    second = loop.tokens(prompt, 24)
+    with pytest.raises(RuntimeError, match="still generating"):
+        next(second)
+    first.close()
+    assert list(loop.tokens(prompt, 8)) == good[:8]
+
+
+@pytest.mark.parametrize("batch", [1, 3, 6, 7])
+def test_persistent_workspace_need_not_be_zeroed(cuda, batch):
+    """A C-ABI caller hands the single-launch kernel any device memory as its workspace: filled with
+    0xFF bytes (NaN patterns in every fp32 slot) the tokens must equal those of a zeroed one - also at
+    chunk counts that are not a power of two (batch 6 / 7), where the merge's loads reach slots that no
+    workgroup writes."""
+    from ohara_amd.llama import Config, Llama
+
+    kw = dict(vocab_size=512, hidden_size=256, intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+              num_hidden_layers=3, max_sequence_length=160, rope_theta=10000.0)
+    w = R.init_weights(R.RefConfig(**kw), seed=5, dtype=torch.bfloat16, std=0.06, norm_jitter=0.1)
+    model = Llama(Config(**kw), w, device=cuda)
+    prompt = torch.randint(0, 512, (batch, 70), generator=torch.Generator().manual_seed(batch)).to(cuda)
+    good = model.generate_greedy(prompt, 12, persistent=True).cpu()
+    sess = model.session(batch, 12, persistent=True)
+    sess._pws = torch.full((64 << 20,), 0xFF, dtype=torch.uint8, device=cuda)  # larger than any workspace here
+    sess.prefill(prompt)
+    sess.run(11, use_graph=False)
+    dirty = sess.tokens().cpu()
+    assert torch.isfinite(sess.logits.float()).all()
+    assert torch.equal(dirty, good)
 
 
 def test_persistent_launch_refuses_more_workgroups_than_can_be_resident(cuda):
