@@ -80,7 +80,7 @@ __device__ void merge_partials(const AttnArgs& a, int b /* query row */, int kvh
     float L = 0.f;
     for (int s0 = lane; s0 < ns; s0 += 64) {
       const float ms = s_w[hh * ns + s0];
-      const float w = (ms == -INFINITY) ? 0.f : __expf(ms - M);
+      const float w = (ms == -INFINITY) ? 0.f : pow2_neg_int(ms - M);  // maxima are integers (log2 units): exact
       s_w[hh * ns + s0] = w;
       L += s_ls[hh * ns + s0] * w;
     }
@@ -158,6 +158,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int p = lane >> 2, dq = lane & 3;  // position of the tile, quarter of its K row: a quad holds one row
   const int pp = lane / DC, dc = lane % DC;
+  const float scale_l2 = a.scale * OHARA_LOG2E;  // scores in log2 units (common.h: softmax bookkeeping)
 
   __shared__ float s_m[4][G], s_l[4][G];
   __shared__ float s_acc[4][G][D];
@@ -233,7 +234,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
     bool raise = false;
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) {
-      sc[hh] = valid ? sc[hh] * a.scale : -INFINITY;
+      sc[hh] = valid ? sc[hh] * scale_l2 : -INFINITY;  // log2 units
       raise = raise || sc[hh] > m_run[hh];
     }
     if (__any(raise)) {
@@ -244,8 +245,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
       for (int hh = 0; hh < G; ++hh) tm[hh] = lanes_max<32, 4>(tm[hh]);
 #pragma unroll
       for (int hh = 0; hh < G; ++hh) {
-        const float mn = fmaxf(m_run[hh], tm[hh]);  // finite: the tile holds at least one position
-        const float corr = __expf(m_run[hh] - mn);
+        const float mn = fmaxf(m_run[hh], ceilf(tm[hh]));  // finite: the tile holds at least one position
+        const float corr = pow2_neg_int(m_run[hh] - mn);
         m_run[hh] = mn;
         l_run[hh] *= corr;
 #pragma unroll
@@ -254,7 +255,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
     }
 #pragma unroll
     for (int hh = 0; hh < G; ++hh) {
-      pv[hh] = __expf(sc[hh] - m_run[hh]);
+      pv[hh] = __builtin_amdgcn_exp2f(sc[hh] - m_run[hh]);
       l_run[hh] += pv[hh];
       pvr[hh] = rbf(pv[hh]);
     }
@@ -335,7 +336,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
       const float mw = s_m[w][hh];
-      const float sc = (mw == -INFINITY) ? 0.f : __expf(mw - M);
+      const float sc = (mw == -INFINITY) ? 0.f : pow2_neg_int(mw - M);
       Ls += s_l[w][hh] * sc;
       o += s_acc[w][hh][d] * sc;
     }
@@ -381,6 +382,7 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int p = lane >> 2, dq = lane & 3;  // position of the tile, quarter of its K row: a quad holds one row
   const int pp = lane / DC, dc = lane % DC;
+  const float scale_l2 = a.scale * OHARA_LOG2E;  // scores in log2 units (common.h: softmax bookkeeping)
 
   __shared__ float s_m[4][G], s_l[4][G];
   __shared__ float s_acc[4][G][D];
@@ -459,7 +461,7 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
       bool raise = false;
 #pragma unroll
       for (int hh = 0; hh < G; ++hh) {
-        sc[hh] = valid ? sc[hh] * a.scale : -INFINITY;
+        sc[hh] = valid ? sc[hh] * scale_l2 : -INFINITY;  // log2 units
         raise = raise || sc[hh] > m_run[hh];
       }
       if (__any(raise)) {
@@ -470,8 +472,8 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
         for (int hh = 0; hh < G; ++hh) tm[hh] = lanes_max<32, 4>(tm[hh]);
 #pragma unroll
         for (int hh = 0; hh < G; ++hh) {
-          const float mn = fmaxf(m_run[hh], tm[hh]);  // finite here: some position of the sub-tile raised it
-          const float corr = __expf(m_run[hh] - mn);
+          const float mn = fmaxf(m_run[hh], ceilf(tm[hh]));  // finite here: some position of the sub-tile raised it
+          const float corr = pow2_neg_int(m_run[hh] - mn);
           m_run[hh] = mn;
           l_run[hh] *= corr;
 #pragma unroll
@@ -480,7 +482,7 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
       }
 #pragma unroll
       for (int hh = 0; hh < G; ++hh) {
-        pv[hh] = __expf(sc[hh] - m_run[hh]);  // (a sub-tile past the end: exp(-inf - m) = 0; m is finite by then)
+        pv[hh] = __builtin_amdgcn_exp2f(sc[hh] - m_run[hh]);  // (a sub-tile past the end: 2^(-inf - m) = 0; m is finite by then)
         l_run[hh] += pv[hh];
         pvr[hh] = rbf(pv[hh]);
       }
@@ -572,7 +574,7 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
       const float mw = s_m[w][hh];
-      const float scw = (mw == -INFINITY) ? 0.f : __expf(mw - M);
+      const float scw = (mw == -INFINITY) ? 0.f : pow2_neg_int(mw - M);
       Ls += s_l[w][hh] * scw;
       o += s_acc[w][hh][d] * scw;
     }
@@ -633,16 +635,16 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
         } else {
           for (int d = 0; d < D; ++d) d_ += s_q[d] * bf2f(kb[(size_t)pos * row + d]);
         }
-        s = d_ * a.scale;
+        s = d_ * (a.scale * OHARA_LOG2E);  // log2 units
       }
       float tm = wave_max(s);
       if ((tid & 63) == 0) s_red[tid >> 6] = tm;
       __syncthreads();
       tm = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
       __syncthreads();
-      const float mn = fmaxf(m_run, tm);
-      const float corr = __expf(m_run - mn);
-      const float pv = (pos < t1) ? __expf(s - mn) : 0.f;
+      const float mn = fmaxf(m_run, ceilf(tm));
+      const float corr = pow2_neg_int(m_run - mn);
+      const float pv = (pos < t1) ? __builtin_amdgcn_exp2f(s - mn) : 0.f;
       s_p[tid] = rbf(pv);  // the weights enter the value product rounded to bf16, the sum unrounded
       float ts = wave_sum(pv);
       if ((tid & 63) == 0) s_red[tid >> 6] = ts;

@@ -192,8 +192,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(PrefillArgs a) {
         mul = a.scale_log2e;    // and the scaling itself rides in the fused multiply-add of the exponent below
       }
       tmax = lane_xor_max<32>(lane_xor_max<16>(tmax));
-      const float mn = fmaxf(m_run[qb], tmax);  // finite: position 0 is visible to every query
-      const float corr = __builtin_amdgcn_exp2f(m_run[qb] - mn);  // arguments <= 0: the bare instruction is exact enough and 2^-inf = 0
+      // the running maximum is kept as an integer (log2 units): every rescale is then an exact power of
+      // two and the bf16 weights do not depend on which tile raised it (common.h: softmax bookkeeping)
+      const float mn = fmaxf(m_run[qb], ceilf(tmax));  // finite: position 0 is visible to every query
+      const float corr = pow2_neg_int(m_run[qb] - mn);
       m_run[qb] = mn;
       float ts = 0.f;
       float p[4][4];
@@ -271,7 +273,7 @@ extern "C" int ohara_attn_prefill_bf16(const uint16_t* q, const uint16_t* kcache
   PrefillArgs a{};
   a.q = q; a.k = kcache; a.v = vcache; a.out = out;
   a.B = batch; a.S = seq_len; a.H = h; a.Hkv = h_kv; a.Tmax = t_max; a.pos = pos;
-  a.scale_log2e = 1.4426950408889634f / sqrtf((float)dh);
+  a.scale_log2e = (1.0f / sqrtf((float)dh)) * OHARA_LOG2E;  // the same constant as the decode kernels'
   // A causal launch lasts as long as its last query block (sixteen tiles at 1024 tokens, twice the
   // average), whatever the other workgroups do.  With fewer than two blocks of 128 queries per CU,
   // blocks of 64 fit three workgroups on a CU and all of them are resident at once (8 x 1024 tokens,

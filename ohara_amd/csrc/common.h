@@ -60,6 +60,19 @@ __device__ __forceinline__ bf16_t f2bf(float f) { return __builtin_bit_cast(bf16
 // Round a float through bfloat16 and back: one reference rounding point.
 __device__ __forceinline__ float rbf(float f) { return bf2f(f2bf(f)); }
 
+// Softmax bookkeeping of the bf16 attention kernels.  The library kernel the reference calls rounds the
+// softmax weights to bf16 before their product with V (ohara/models/llama.py:116-123 ->
+// F.scaled_dot_product_attention).  A bf16 rounding commutes with a scaling by a power of two, so the
+// kernels here keep scores in log2 units, take the running maximum up to the next INTEGER and form
+// p = 2^(s - M): whatever M a chunk, a wave or a tile happens to use, the rounded weights are the same
+// bits times an exact power of two, and every later rescale 2^(M_old - M_new) is exact too.  The result
+// then depends on how the context is cut (chunks, tiles, kernels) only through the order of fp32 sums.
+#define OHARA_LOG2E 1.4426950408889634f
+// 2^d for an integer-valued d <= 0 (d = -inf or NaN gives 2^-126, which only ever multiplies a zero)
+__device__ __forceinline__ float pow2_neg_int(float d) {
+  return __int_as_float(((int)fmaxf(d, -126.f) + 127) << 23);
+}
+
 __device__ __forceinline__ float lo_bf(uint32_t packed) { return __uint_as_float(packed << 16); }
 __device__ __forceinline__ float hi_bf(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
 __device__ __forceinline__ uint32_t pack_bf(float lo, float hi) {

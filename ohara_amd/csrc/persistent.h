@@ -387,7 +387,7 @@ __device__ __forceinline__ void stage_attn_merge(bf16_t* xs, int ldxs, const flo
     if (NS > 4) M = lane_xor_max<4>(M);
     if (NS > 2) M = lane_xor_max<2>(M);
     if (NS > 1) M = lane_xor_max<1>(M);
-    const float w = (ms == -INFINITY) ? 0.f : __expf(ms - M);
+    const float w = (ms == -INFINITY) ? 0.f : pow2_neg_int(ms - M);  // maxima are integers (log2 units): exact
     float Ls = ls * w;
     if (NS > 8) Ls = lane_xor_sum<8>(Ls);
     if (NS > 4) Ls = lane_xor_sum<4>(Ls);
@@ -446,7 +446,7 @@ __device__ __forceinline__ void stage_attn_merge_small(bf16_t* xs, int ldxs, con
 #pragma unroll
   for (int s = 0; s < NS; ++s) {
     const float ms = __uint_as_float(mlv[s].x);
-    const float w = (ms == -INFINITY) ? 0.f : __expf(ms - M);
+    const float w = (ms == -INFINITY) ? 0.f : pow2_neg_int(ms - M);  // maxima are integers (log2 units): exact
     Ls += __uint_as_float(mlv[s].y) * w;
     o[0] += __uint_as_float(av[s].x) * w;
     o[1] += __uint_as_float(av[s].y) * w;
@@ -971,7 +971,7 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
   const int p = lane & 15;
   const int dq = lane >> 4;
   const int pp = lane / DC, dc = lane % DC;
-  const float scale = 1.0f / sqrtf((float)D);
+  const float scale = (1.0f / sqrtf((float)D)) * OHARA_LOG2E;  // scores in log2 units (common.h: softmax bookkeeping)
   float* s_m = lds;                 // [4][G]
   float* s_l = lds + 4 * G;         // [4][G]
   float* s_acc = lds + 8 * G;       // [4][G][D]
@@ -1048,8 +1048,8 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
           for (int hh = 0; hh < G; ++hh) tm[hh] = lane_xor_max<1>(tm[hh]);
 #pragma unroll
           for (int hh = 0; hh < G; ++hh) {
-            const float mn = fmaxf(m_run[hh], tm[hh]);
-            const float corr = __expf(m_run[hh] - mn);
+            const float mn = fmaxf(m_run[hh], ceilf(tm[hh]));
+            const float corr = pow2_neg_int(m_run[hh] - mn);
             m_run[hh] = mn;
             l_run[hh] *= corr;
 #pragma unroll
@@ -1058,7 +1058,7 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
         }
 #pragma unroll
         for (int hh = 0; hh < G; ++hh) {
-          pv[hh] = __expf(sc[hh] - m_run[hh]);
+          pv[hh] = __builtin_amdgcn_exp2f(sc[hh] - m_run[hh]);
           l_run[hh] += pv[hh];
           pvr[hh] = rbf(pv[hh]);
         }
@@ -1124,7 +1124,7 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
         const float mw = s_m[w * G + hh];
-        const float sc = (mw == -INFINITY) ? 0.f : __expf(mw - M);
+        const float sc = (mw == -INFINITY) ? 0.f : pow2_neg_int(mw - M);
         Ls += s_l[w * G + hh] * sc;
         o0 += s_acc[(w * G + hh) * D + d] * sc;
         o1 += s_acc[(w * G + hh) * D + d + 1] * sc;
