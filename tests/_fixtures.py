@@ -35,3 +35,22 @@ def bf16_ulps(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     mag = torch.maximum(af.abs(), bf.abs()).clamp_min(2.0 ** -120)
     ulp = torch.exp2(torch.floor(torch.log2(mag)) - 7)
     return (af - bf).abs() / ulp
+
+
+def reference_self_distance(fx: dict) -> float:
+    """How far the reference reproduces ITSELF on this fixture's model: the largest per-row mean
+    |logit difference| (over the row's max |logit|) between its run with all threads and its repeats
+    (one thread; the library's other matrix kernels), over every stored row."""
+    worst = 0.0
+    for tag in ("one_thread", "other_kernels"):
+        if "logits_at_columns" in fx:  # the greedy d12 run: (steps, columns), scale stored per step
+            pairs = [(fx["logits_at_columns"], fx[f"logits_at_columns_{tag}"], fx["logit_absmax"].float())]
+        else:
+            pairs = [(fx[k], fx[f"{k}_{tag}"], None) for k in fx
+                     if k.startswith("logits_") and not k.endswith(("one_thread", "other_kernels")) and f"{k}_{tag}" in fx]
+        for a, b, scale in pairs:
+            a, b = a.float(), b.float()
+            if scale is None:
+                scale = a.abs().amax(-1)
+            worst = max(worst, ((a - b).abs().mean(-1) / scale).max().item())
+    return worst

@@ -20,9 +20,10 @@ buffers), run on the CPU through the KV cache.  Every file holds plain tensors
                      1024-token prompt, 64 greedy tokens: the tokens, and per step the logits at 2048
                      fixed vocabulary columns plus the 32 largest logits with their ids
 
-mid_gqa, d12w and d12_greedy are run twice, with all threads and with one (``*_one_thread``; d12_greedy's
-second run is fed the first run's tokens): same code, same inputs, another summation order inside the
-library's products.  The distance between the two runs is how far the reference reproduces itself.
+mid_gqa, d12w and d12_greedy are run three times: with all threads, with one (``*_one_thread``) and with
+the library's other set of CPU matrix kernels (oneDNN switched off, ``*_other_kernels``); d12_greedy's
+repeats are fed the first run's tokens.  Same code, same inputs, another summation order inside the
+library's products.  The distances between the runs are how far the reference reproduces itself.
 
 The larger cases do not store their weights: they are ``oracle.llama_ref.init_weights(cfg, seed,
 torch.bfloat16)`` (a seeded CPU generator, loaded into the reference model with
@@ -155,10 +156,14 @@ def seeded(name):
     torch.set_num_threads(1)
     one = run_cached(model, ids, spec["prompt"], spec["steps"])
     torch.set_num_threads(n)
+    # ... and with the library's other set of CPU matrix kernels (oneDNN switched off)
+    with torch.backends.mkldnn.flags(enabled=False):
+        other = run_cached(model, ids, spec["prompt"], spec["steps"])
     out["threads"] = torch.tensor([n, 1])
-    out["logits_prefill_one_thread"] = one["logits_prefill"][:, -8:].clone()
-    for s in range(spec["steps"]):
-        out[f"logits_step{s}_one_thread"] = one[f"logits_step{s}"]
+    for tag, res2 in (("one_thread", one), ("other_kernels", other)):
+        out[f"logits_prefill_{tag}"] = res2["logits_prefill"][:, -8:].clone()
+        for s in range(spec["steps"]):
+            out[f"logits_step{s}_{tag}"] = res2[f"logits_step{s}"]
     # keep the files small: the last 8 prompt positions of the prefill are enough to pin it
     res["logits_prefill"] = res["logits_prefill"][:, -8:].clone()
     res["attn0_prefill"] = res["attn0_prefill"][:, -8:].clone()
@@ -208,11 +213,12 @@ def d12_greedy(prompt=1024, steps=64, seed=0):
     torch.set_num_threads(1)
     one = run(out["tokens"])
     torch.set_num_threads(n)
+    with torch.backends.mkldnn.flags(enabled=False):
+        other = run(out["tokens"])
     out["threads"] = torch.tensor([n, 1])
-    out["tokens_one_thread"] = one["tokens"]  # its own arg-max at every step, fed the first run's tokens
-    out["logits_at_columns_one_thread"] = one["logits_at_columns"]
-    out["top32_values_one_thread"] = one["top32_values"]
-    out["top32_ids_one_thread"] = one["top32_ids"]
+    for tag, res in (("one_thread", one), ("other_kernels", other)):
+        out[f"tokens_{tag}"] = res["tokens"]  # its own arg-max at every step, fed the first run's tokens
+        out[f"logits_at_columns_{tag}"] = res["logits_at_columns"]
     return out
 
 

@@ -9,9 +9,9 @@ by the reference, so such near-ties are decided by rounding noise on either side
 
 At the d12 size the mean bound is the target or 1.25 x the distance at which the REFERENCE
 reproduces itself, whichever is larger: tests/golden/llama_bf16_d12_greedy.pt holds two runs of the
-reference's own bf16 model on the CPU (all threads / one thread: the library's products sum in another
-order), 64 steps each; they lie up to 2.15e-3 of the logit scale apart in the mean and pick different
-greedy tokens at step 60.  tests/test_gpu_reference_bf16.py compares the HIP path with that run itself.
+reference's own bf16 model on the CPU and two repeats (one thread; the library's other matrix kernels:
+its products then sum in another order), 64 steps each; they lie up to 2.5e-3 of the logit scale apart
+in the mean (41 of 64 steps above 2e-3) and pick different greedy tokens at step 60.  tests/test_gpu_reference_bf16.py compares the HIP path with that run itself.
 """
 
 import dataclasses
@@ -152,16 +152,15 @@ def _near_tie(logits_row, a, b, ulps=2):
 
 
 def _reference_self_distance():
-    """Worst per-step mean |logit difference| (of the logit scale) between the reference's two bf16
-    runs of the d12 model stored in the fixture (all threads against one thread, 64 decode steps)."""
-    from _fixtures import load_fixture
+    """Worst per-step mean |logit difference| (of the logit scale) between the reference's own bf16 runs
+    of the d12 model stored in the fixture (all threads against one thread and against the library's
+    other matrix kernels, 64 decode steps each)."""
+    from _fixtures import load_fixture, reference_self_distance
 
-    fx = load_fixture("llama_bf16_d12_greedy.pt")
-    d = (fx["logits_at_columns"].float() - fx["logits_at_columns_one_thread"].float()).abs().mean(1)
-    return (d / fx["logit_absmax"].float()).max().item()
+    return reference_self_distance(load_fixture("llama_bf16_d12_greedy.pt"))
 
 
-def _check_greedy(model, ref, prompt, steps, cuda, max_rel=2e-2, mean_rel=2e-3, stats_out=None):
+def _check_greedy(model, ref, prompt, steps, cuda, max_rel=2e-2, mean_rel=2e-3, stats_out=None, tie_ulps=2):
     """(1) free-running device loop vs the oracle's greedy tokens: identical, or first
     divergence at a near-tie of the oracle's logits; (2) teacher-forced on the oracle's
     tokens so that every one of the `steps` positions is checked: logits within tolerance
@@ -175,8 +174,9 @@ def _check_greedy(model, ref, prompt, steps, cuda, max_rel=2e-2, mean_rel=2e-3, 
         if neq.numel() == 0:
             continue
         t = int(neq[0])
-        assert _near_tie(want_logits[t, b], int(got[b, t]), int(want[b, t])), (
-            f"sequence {b} diverged at step {t}: got {int(got[b, t])}, oracle {int(want[b, t])} and not a near-tie"
+        assert _near_tie(want_logits[t, b], int(got[b, t]), int(want[b, t]), tie_ulps), (
+            f"sequence {b} diverged at step {t}: got {int(got[b, t])}, oracle {int(want[b, t])} and not a near-tie: "
+            f"{want_logits[t, b, int(got[b, t])].item()} against {want_logits[t, b, int(want[b, t])].item()}"
         )
         n_diverged += 1
     B, P = prompt.shape
@@ -204,7 +204,7 @@ def _check_greedy(model, ref, prompt, steps, cuda, max_rel=2e-2, mean_rel=2e-3, 
             if int(mine[b]) == int(want[b, t]):
                 same += 1
             else:
-                assert _near_tie(want_logits[t, b], int(mine[b]), int(want[b, t])), (t, b)
+                assert _near_tie(want_logits[t, b], int(mine[b]), int(want[b, t]), tie_ulps), (t, b)
         inp = want[:, t : t + 1].to(cuda)
     assert same >= 0.9 * steps * B, f"only {same}/{steps * B} teacher-forced argmaxes identical"
     stats["teacher_forced_argmax_identical"] = f"{same}/{steps * B}"
@@ -224,7 +224,8 @@ def test_greedy_small_model(cuda):
     ref = R.RefLlama(rcfg, w)
     model = Llama(cfg, w, device=cuda)
     prompt = torch.randint(0, 512, (3, 17), generator=torch.Generator().manual_seed(1))
-    got, want, nd = _check_greedy(model, ref, prompt, 64, cuda, max_rel=4e-2, mean_rel=4e-3)
+    # (twice the tolerance, twice the near-tie width: 4 bf16 steps between the oracle's two candidates)
+    got, want, nd = _check_greedy(model, ref, prompt, 64, cuda, max_rel=4e-2, mean_rel=4e-3, tie_ulps=4)
     eager = model.generate_greedy(prompt.to(cuda), 64, use_graph=False).cpu()
     assert torch.equal(eager, got), "graph replay and eager launches must agree bit for bit"
     # the kernel-per-op chain and the single persistent launch both satisfy the oracle
@@ -237,7 +238,7 @@ def test_greedy_small_model(cuda):
         if neq.numel():
             t = int(neq[0])
             wl = greedy_decode_ref(ref, prompt, t + 1, return_logits=True)[1]
-            assert _near_tie(wl[t, b], int(chain[b, t]), int(want[b, t]))
+            assert _near_tie(wl[t, b], int(chain[b, t]), int(want[b, t]), 4)
 
 
 def test_d12_decode_parity(cuda):
@@ -371,15 +372,21 @@ def test_sampled_decode_session(cuda, persistent):
     assert torch.equal(sess2.tokens().cpu(), toks)
     # teacher-forced: the oracle model (loose: its logits differ from the kernels' at the bf16 level,
     # which moves CDF boundaries by a few percent on this high-gain model) and the oracle sampler on
-    # the kernels' own logits (tight: pins the wiring of draws, steps and bookkeeping)
-    cache, gcache = ref.build_kv_cache(B), model.build_kv_cache(B)
+    # the session's own logits of every step (tight: pins the wiring of draws, steps and bookkeeping)
+    sess3 = model.session(B, N, persistent=persistent, sampling=cfg, u=u.to(cuda))
+    sess3.prefill(prompt.to(cuda))
+    own = [sess3.logits.clone().cpu()]
+    for _ in range(N - 1):
+        sess3.step()
+        own.append(sess3.logits.clone().cpu())
+    assert torch.equal(sess3.tokens().cpu(), toks)
+    cache = ref.build_kv_cache(B)
     inp, pos = prompt, 0
     for t in range(N):
         logits = ref(inp, cache, pos)
-        glogits = model(inp.to(cuda), gcache, pos).cpu()
         pos += inp.shape[1]
-        for lg, tol in ((logits, 6e-2), (glogits, 5e-3)):
-            ids, cdf = candidate_cdf_ref(lg[:, -1:].float(), cfg.temperature, cfg.top_p, cfg.top_k)
+        for lg, tol in ((logits[:, -1:], 6e-2), (own[t].view(B, 1, -1), 5e-3)):
+            ids, cdf = candidate_cdf_ref(lg.float(), cfg.temperature, cfg.top_p, cfg.top_k)
             for b in range(B):
                 hit = (ids[b] == int(toks[b, t])).nonzero()
                 assert hit.numel(), (t, b, "token outside the candidate order")

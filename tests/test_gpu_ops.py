@@ -334,4 +334,4 @@ def test_attention_does_not_depend_on_how_the_context_is_cut(cuda, B, H, Hkv, D,
     # against the oracle (the library kernel's own cut: 512-key blocks around the true running maximum)
     ref = R.attention_core(q.cpu().view(B, 1, H, D), k.cpu()[:, :L], v.cpu()[:, :L], L - 1).view(B, H * D)
     assert (base.cpu().float() - ref.float()).abs().max().item() <= scale * 2.0 ** -7
-    assert (base.cpu().float() - ref.float()).abs().mean().item() <= scale * 2.0 ** -11
+    assert (base.cpu().float() - ref.float()).abs().mean().item() <= scale * 2.0 ** -10

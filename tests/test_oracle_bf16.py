@@ -6,9 +6,10 @@ tests/golden/make_llama_bf16_golden.py), and the library routine its attention c
 Two kinds of statement are made.  Operator by operator, on the reference's own operands, the oracle
 returns the reference's bits (a Linear: all but a few elements in ten thousand, where the library sums
 in another order).  Through a whole model those few flipped bits travel: the logits of two runs of the
-REFERENCE ITSELF, with all threads and with one, share only 15 % of their bit patterns at the d12
-widths and lie 2.4-2.8e-3 of the logit scale apart on average.  The fixtures hold both runs, and the
-oracle is asked to lie as close to the reference as the reference lies to itself.
+REFERENCE ITSELF - with all threads, with one, with the library's other matrix kernels - share only
+15 % of their bit patterns at the d12 widths and lie 2.1-3.1e-3 of the logit scale apart on average.
+The fixtures hold these runs, and the oracle is asked to lie as close to the reference as the
+reference lies to itself (1.25 x the largest distance between two of its own runs).
 """
 
 import dataclasses
@@ -20,7 +21,7 @@ import torch.nn.functional as F
 
 from oracle import llama_ref as R
 
-from _fixtures import bf16_ulps, identical_fraction, load_fixture, weight_checksum
+from _fixtures import bf16_ulps, identical_fraction, load_fixture, reference_self_distance, weight_checksum
 
 BF = torch.bfloat16
 
@@ -208,9 +209,10 @@ def test_seeded_models_lie_as_close_to_the_reference_as_it_lies_to_itself(name):
     for s in range(steps):
         got[f"step{s}"] = m(ids[:, prompt + s : prompt + s + 1], cache, prompt + s)
     assert identical_fraction(cache[0].key[:, prompt + steps - 16 : prompt + steps], fx["cache0_key"]) >= 0.998
+    self_mean = reference_self_distance(fx)  # the reference against its own repeats, worst row
     for tag, mine in got.items():
-        ref, ref1 = fx[f"logits_{tag}"], fx[f"logits_{tag}_one_thread"]
-        self_max, self_mean = _rel(ref1, ref)   # the reference against itself (all threads / one thread)
-        mx, mean = _rel(mine, ref)
-        assert mx <= 2e-2, (tag, mx)
-        assert mean <= max(2e-3, 1.25 * self_mean), (tag, mean, self_mean)
+        ref = fx[f"logits_{tag}"].float()
+        d = (mine.float() - ref).abs()
+        scale = ref.abs().amax(-1)
+        assert (d.amax(-1) / scale).max().item() <= 2e-2, tag
+        assert (d.mean(-1) / scale).max().item() <= max(2e-3, 1.25 * self_mean), (tag, self_mean)
