@@ -33,6 +33,30 @@ def _moe_cfg(**over):
     return Config(**kw)
 
 
+@pytest.mark.parametrize("name", ["dense", "gqa", "moe"])
+def test_reference_made_state_dicts(tmp_path, name):
+    """State dicts the reference's own Llama produced (tests/golden/llama_tiny_*.pt, with the Config each
+    was built from): the architecture is recovered from the tensor shapes alone, through the raw dict
+    and through both on-disk formats.  What leaves no trace in the weights (top-k, gate function, rope
+    theta - which the reference does not recover either, chat_engine.py:129-245) is passed in."""
+    from _fixtures import load_fixture
+
+    fx = load_fixture(f"llama_tiny_{name}.pt")
+    want = Config(**{k: v for k, v in fx["config"].items() if k in Config.__dataclass_fields__})
+    hints = dict(moe_experts_per_tok=want.moe_experts_per_tok, moe_gate_fn=want.moe_gate_fn) if name == "moe" else {}
+    got = config_from_state_dict(fx["state"], **hints)
+    for f in Config.__dataclass_fields__:
+        if f not in ("rope_theta", "dropout", "init_style"):
+            assert getattr(got, f) == getattr(want, f), f
+    wrapped = {"model": {"module._orig_mod." + k: v for k, v in fx["state"].items()}, "idx": 7}
+    path = tmp_path / "ckpt.pt"
+    torch.save(wrapped, path)
+    cfg2, state2 = load_checkpoint(str(path), **hints)
+    assert cfg2 == got and set(state2) == set(clean_state_dict(fx["state"]))
+    for k, v in state2.items():
+        assert torch.equal(v, fx["state"][k]), k
+
+
 def test_dense_config_round_trips():
     cfg = Config(vocab_size=300, hidden_size=64, intermediate_size=128, max_sequence_length=96, num_hidden_layers=3,
                  num_attention_heads=2, dropout=0.0)

@@ -13,14 +13,16 @@ pytestmark = pytest.mark.gpu
 BF = torch.bfloat16
 
 
-@pytest.mark.parametrize("B,L", [(16, 32768), (64, 4096), (1, 16384), (1, 32768)])
+@pytest.mark.parametrize("B,L", [(b, l) for b in (1, 16, 64) for l in (1024, 4096, 16384, 32768)])
 def test_decode_attention_microbench_shape(cuda, B, L):
-    """32 query / 8 KV heads x 128, one query per sequence over L cached positions."""
+    """32 query / 8 KV heads x 128, one query per sequence over L cached positions: every (batch,
+    context) point the benchmark times, with the benchmark's chunk count (64 x 32768 is 4.3 GB per
+    tensor)."""
     from ohara_amd import ops
 
     H, Hkv, D = 32, 8, 128
     G = H // Hkv
-    ns = max(1, min(1024 // (B * Hkv), L // 128, 64))
+    ns = max(1, min(1024 // (B * Hkv), L // 128, 64))  # bench.py:bench_attention_microbench
     g = torch.Generator(device=cuda).manual_seed(1)
     q = torch.randn(B, H * D, device=cuda, generator=g).to(BF)
     k = torch.randn(B, L, Hkv, D, device=cuda, generator=g).to(BF)
@@ -44,6 +46,82 @@ def test_decode_attention_microbench_shape(cuda, B, L):
     out = ops.attn_decode(q, k, v, H, Hkv, D, L, ns, ws).view(B, Hkv, G, D)
     want = v.float().mean(1)  # (B, Hkv, D)
     assert (out.float() - want[:, :, None, :]).abs().max().item() <= 2e-3
+
+
+@pytest.mark.parametrize("B,L", [(16, 16384), (64, 4096), (1, 32768)])
+def test_decode_attention_microbench_shape_int8_cache(cuda, B, L):
+    """The same shape over the int8 cache, as the benchmark times it: the kernel must return what bf16
+    attention returns over the dequantised cache (same values, same rounding points; the tiles are cut
+    differently, so single bf16 roundings may differ), and sub-sampled pairs must match fp32 torch."""
+    from ohara_amd import ops
+    from ohara_amd.llama import KVCache
+
+    H, Hkv, D = 32, 8, 128
+    G = H // Hkv
+    ns = max(1, min(1024 // (B * Hkv), L // 128, 64))
+    g = torch.Generator(device=cuda).manual_seed(1)
+    q = torch.randn(B, H * D, device=cuda, generator=g).to(BF)
+    k = torch.randn(B, L, Hkv, D, device=cuda, generator=g).to(BF)
+    v = torch.randn(B, L, Hkv, D, device=cuda, generator=g).to(BF)
+    cache = KVCache((B, L, Hkv, D), L, device=cuda, dtype=BF, int8=True)
+    step = max(1, 4096 // B)
+    for p0 in range(0, L, step):
+        ops.kv_quant_append(k[:, p0:p0 + step].contiguous(), v[:, p0:p0 + step].contiguous(), cache, p0)
+    ws = ops.attn_workspace(B, H, Hkv, D, ns, cuda)
+    out = ops.attn_cached_int8(q, cache, H, Hkv, D, L - 1, ns, ws).clone()
+    kd, vd = ops.kv_dequant(cache, "key", B, L), ops.kv_dequant(cache, "value", B, L)
+    assert (kd.float() - k.float()).abs().max().item() <= 0.05  # tests/test_modules.py:82-100 of the reference
+    same = ops.attn_decode(q, kd, vd, H, Hkv, D, L, ns, ws)
+    scale = same.float().abs().max().item()
+    assert (out.float() - same.float()).abs().max().item() <= 2.0 ** -8 * scale
+    assert (out == same).float().mean().item() >= 0.99
+    o3 = out.view(B, H, D)
+    for b, h in ((0, 0), (B // 2, 13), (B - 1, H - 1)):
+        kk, vv = kd[b, :, h // G].float(), vd[b, :, h // G].float()
+        s_ = (kk @ q[b].view(H, D)[h].float()) / math.sqrt(D)
+        want = torch.softmax(s_, 0) @ vv
+        assert (o3[b, h].float() - want).abs().max().item() <= 2e-2 * max(1.0, want.abs().max().item()), (b, h)
+
+
+def test_d12_sampled_session_at_the_full_vocabulary(cuda):
+    """The sampled mode of the headline configuration end to end: d12 (vocabulary 65536), temperature
+    0.8 / top-k 50 / top-p 0.9, uniform draws fixed in advance and shared with the oracle sampler;
+    batch 1 on the single-launch kernel and batch 8, prompts of 1024 tokens.  At every step the oracle
+    sampler, applied to the session's own logits of that step, must place the session's token in the
+    CDF interval that holds the step's draw."""
+    import bench
+    from oracle.sampling_ref import candidate_cdf_ref
+    from ohara_amd.llama import Llama
+    from ohara_amd.sampling import SamplingConfig
+
+    cfg, st = bench.d12_state(cuda)
+    model = Llama(cfg, st, device=cuda)
+    scfg = SamplingConfig(temperature=0.8, top_k=50, top_p=0.9)
+    for B, N in ((1, 24), (8, 10)):
+        g = torch.Generator().manual_seed(B)
+        prompt = torch.randint(0, cfg.vocab_size, (B, 1024), generator=g)
+        u = torch.rand(N, B, generator=g)
+        sess = model.session(B, N, sampling=scfg, u=u.to(cuda))
+        sess.prefill(prompt.to(cuda))
+        own = [sess.logits.clone().cpu()]
+        for _ in range(N - 1):
+            sess.step()
+            own.append(sess.logits.clone().cpu())
+        toks = sess.tokens().cpu()
+        assert toks.shape == (B, N)
+        for t in range(N):
+            ids, cdf = candidate_cdf_ref(own[t].view(B, 1, -1).float(), scfg.temperature, scfg.top_p, scfg.top_k)
+            for b in range(B):
+                hit = (ids[b] == int(toks[b, t])).nonzero()
+                assert hit.numel(), (B, t, b, "token outside the candidate order")
+                j = int(hit[0])
+                lo = float(cdf[b, j - 1]) if j > 0 else 0.0
+                assert lo - 5e-5 <= float(u[t, b]) <= float(cdf[b, j]) + 5e-5, (B, t, b, lo, float(cdf[b, j]), float(u[t, b]))
+        # the captured graph replays the same tokens
+        sess2 = model.session(B, N, sampling=scfg, u=u.to(cuda))
+        sess2.prefill(prompt.to(cuda))
+        sess2.run(N - 1)
+        assert torch.equal(sess2.tokens().cpu(), toks)
 
 
 def test_d12_batch32_prompt1024_matches_single_sequence_runs(cuda):
