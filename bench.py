@@ -559,24 +559,26 @@ def bench_phi(dev):
 # Shader-clock samples that workgroup 0 of the persistent kernel takes per layer, in order (see
 # csrc/mega.hip: Prof::stamp in the kernel body, GridSync::arrive / wait and gemm_phase).  Each entry
 # names the interval that ENDS at that sample.
-_ARRIVE = ["epilogue stores issued -> arrive()", "wait for own stores (vmcnt 0)", "workgroup barrier",
-           "arrival atomics issued"]
-_WAIT = ["next phase's prefetch issued", "spin on the release word + workgroup barrier", "(bookkeeping)"]
-_GEMM = ["activations staged in LDS -> MFMAs issued", "cross-wave sum"]
+_BAR = ["wait for own stores (vmcnt 0)", "workgroup barrier", "arrival atomics issued", "(window)",
+        "spin on the release word + workgroup barrier", "(bookkeeping)"]
+_GEMM = ["activations in LDS -> MFMAs issued", "cross-wave sum"]
+# intervals between the clock samples of the batch-1 kernel (one grid barrier per layer, after the
+# attention partials; the other hand-offs are tagged mailboxes that the consumer polls for)
 PHASE_STAMPS = (
-    [("P1 qkv", "mailbox read + norm1 into LDS")] + [("P1 qkv", x) for x in _GEMM] + [("P1 qkv", "rotary epilogue")]
-    + [("P1 qkv", x) for x in _ARRIVE + _WAIT]
-    + [("P2 attention", "attention chunk (q mailbox, K/V tiles, partials)")] + [("P2 attention", x) for x in _ARRIVE[1:] + _WAIT]
-    + [("P3 wo", "merge of attention partials into LDS")] + [("P3 wo", x) for x in _GEMM] + [("P3 wo", "residual epilogue")]
-    + [("P3 wo", x) for x in _ARRIVE + _WAIT]
-    + [("P4 gate/up", "mailbox read + norm2 -> MFMAs issued"), ("P4 gate/up", "cross-wave sum")]
-    + [("P4 gate/up", "SwiGLU epilogue")] + [("P4 gate/up", x) for x in _ARRIVE[1:] + _WAIT]
-    + [("P5 down", "act mailbox into LDS -> MFMAs issued"), ("P5 down", "cross-wave sum")]
-    + [("P5 down", "partial-sum epilogue")] + [("P5 down", x) for x in _ARRIVE[1:] + _WAIT]
+    [("P1 qkv", "poll for the stream + norm1 into LDS")] + [("P1 qkv", x) for x in _GEMM]
+    + [("P1 qkv", "rotary epilogue, tagged stores, down weights requested")]
+    + [("P2 attention", "poll for q, attention chunk, partials stored")] + [("P2 attention", x) for x in _BAR]
+    + [("P3 wo", "merge of attention partials into LDS")] + [("P3 wo", x) for x in _GEMM]
+    + [("P3 wo", "residual epilogue, tagged stores")]
+    + [("P4 gate/up", "poll for the stream + norm2 into LDS")] + [("P4 gate/up", x) for x in _GEMM]
+    + [("P4 gate/up", "SwiGLU epilogue, tagged stores")]
+    + [("P5 down", "poll for the activations into LDS")] + [("P5 down", x) for x in _GEMM]
+    + [("P5 down", "residual epilogue, tagged stores, next layer's weights requested")]
 )
+PHASE_TAIL = 13  # samples after the layers: three around the final norm, then as before
 
 
-def phase_timeline(dev, prompt_len, steps=32):
+def phase_timeline(dev, prompt_len, steps=32, workgroup=0):
     """Per-phase timeline of the persistent decode kernel at batch 1: where workgroup 0 spends a
     step, from the kernel's own shader-clock samples averaged over `steps` real decode steps."""
     from ohara_amd.llama import Llama
@@ -590,7 +592,7 @@ def phase_timeline(dev, prompt_len, steps=32):
     nl = cfg.num_hidden_layers
     per = len(PHASE_STAMPS)
     n_stamps = 1 + per * nl
-    n_tail = 10  # after the layers: LM head (2 samples), its end, the selection's arrive (4) / wait (2), the end
+    n_tail = PHASE_TAIL  # after the layers: final norm (3), LM head (2 samples), its end, the selection's arrive (4) / wait (2), the end
     acc = torch.zeros(n_stamps + n_tail, dtype=torch.float64)
     total_ms = 0.0
     for _ in range(steps):
@@ -600,7 +602,7 @@ def phase_timeline(dev, prompt_len, steps=32):
         e1.record()
         torch.cuda.synchronize()
         total_ms += e0.elapsed_time(e1)
-        c = sess.phase_clocks().double()
+        c = sess.phase_clocks(workgroup).double()
         acc += c[: n_stamps + n_tail] - c[0]
     acc /= steps
     kernel_us = total_ms / steps * 1e3

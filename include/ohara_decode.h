@@ -419,8 +419,9 @@ int64_t ohara_persistent_workspace_bytes(const OharaModel* m, int batch, int n_s
 int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s, void* workspace, int n_workgroups,
                                   int init_workspace, int select_greedy, unsigned int spin_limit, void* stream);
 /* Byte offsets inside the workspace: the barrier words; the sticky error word (uint32,
- * non-zero after a barrier wait expired); 1024 x uint64 shader-clock samples taken by
- * workgroup 0 at every phase boundary when s->prof_kernel == -2 (measurement only; the samples
+ * non-zero after a barrier wait expired); per workgroup 1024 x uint64 samples of the constant
+ * 100 MHz clock taken by its thread 0 at every phase boundary when s->prof_kernel == -2 (workgroup
+ * w's samples start 8192 w bytes after the offset; measurement only; the samples
  * are compiled into a separate build of the kernel that exists for head_dim 128 with
  * n_kv_heads == n_heads only, other shapes leave the slots untouched). */
 int64_t ohara_persistent_barrier_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);

@@ -51,6 +51,13 @@ __device__ __forceinline__ uint4 lds16(const void* p) {
   return make_uint4(v.x, v.y, v.z, v.w);
 }
 
+// 16 bytes from an LDS byte address (a 32-bit address the compiler need not prove to be LDS: through a
+// generic pointer every read carries a null check and a select)
+__device__ __forceinline__ uint4 lds16_at(uint32_t addr) {
+  const u32x4 v = *(const OHARA_LDS u32x4*)(uintptr_t)addr;
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 __device__ __forceinline__ float bf2f(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 
 // Round-to-nearest-even, the rounding torch applies when a float result is stored

@@ -29,9 +29,18 @@
 // The one exception is the KV-cache row appended in this step (its lines are shared by
 // several writers): attention reads that single row with device-scope loads.
 //
+// Batch 1 (the ONE builds): three of the five hand-offs of a layer carry one short row - the q row and
+// the new key / value rows (P1 -> P2), the residual stream (P3 -> P4), the activations (P4 -> P5) - and
+// go through TAGGED mailboxes that the consumers poll for (persistent.h) instead of a barrier; two grid
+// barriers per layer remain (after the attention partials, after the down projection's sums).  The
+// weights of P4 and P5 are requested around the first of them, where a workgroup is idle anyway, so that
+// no weight load is in flight ahead of a poll (a wave's loads return in order).
+//
 // Every barrier wait is bounded: a workgroup that spins longer than the limit raises a
 // sticky error word and moves on, all later waits return at once, and the grid drains.
 #include "persistent.h"
+
+#define OHARA_PROF_SLOTS 1024  // clock samples per workgroup (measurement builds)
 
 namespace {
 
@@ -55,8 +64,11 @@ struct MegaArgs {
   bf16_t* logits;  // (B, V)
   int32_t* step_state;  // {pos, step, done, pad}
   int64_t* history;
+  char* tg;             // batch 1: NL blocks of tagged mailboxes, tg_stride bytes each, the stream after the attention block first
+  size_t tg_stride;
+  int tg_n, tg_q, tg_kv, tg_a;  // byte offsets inside a layer's block: stream after the layer | q | new k, v | activations
   unsigned int* bar;    // barrier words, see GridSync
-  unsigned long long* prof;  // optional: clock of workgroup 0 at every phase boundary
+  unsigned long long* prof;  // optional: clock of every workgroup's thread 0 at every phase boundary (OHARA_PROF_SLOTS each)
   unsigned int spin_limit;
 };
 
@@ -97,7 +109,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   const int L = min(pos + 1, m.t_max);
   float best_v = -INFINITY;
   int best_i = 0x7fffffff;
-  ProfT<PROFILE> pf((blockIdx.x == 0 && threadIdx.x == 0) ? a.prof : nullptr);
+  ProfT<PROFILE> pf((a.prof && threadIdx.x == 0) ? a.prof + (size_t)blockIdx.x * OHARA_PROF_SLOTS : nullptr);
 
   GemmP qkv{}, prj{}, gu{}, dn{}, lm{};
   qkv.H = H; qkv.Hkv = Hkv; qkv.Dh = D; qkv.Tmax = m.t_max; qkv.pos = pos; qkv.cos = m.cos; qkv.sin = m.sin;
@@ -115,6 +127,121 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   AttnPre<D> apre;
   qkv.wp = lds_ptr<const uint4>(ptab, 0);
   qkv.norm_w = lds_ptr<const bf16_t>(ptab, 4);
+  // ONE (batch 1): the tagged path; the host launches it only on a grid wide enough for gate/up and the
+  // down projection (and the output projection and the down projection) to sit on different workgroups -
+  // their weights share registers - and the general build otherwise.
+  if constexpr (ONE) {
+   {
+    // ---- batch 1: tagged hand-offs, one grid barrier per layer ---------------------------------------
+    const Poll pc{gs.k, a.spin_limit, gs.err};
+    const int nwg = (int)gridDim.x;
+    qkv.tag = prj.tag = gu.tag = dn.tag = pc.tag;
+    qkv.poll = prj.poll = gu.poll = dn.poll = &pc;
+    // Who does what.  Every phase is a handful of units, and what a unit costs is the fetch of its weights
+    // (a CU takes in ~55 GB/s) - so the phases are spread over the grid such that a workgroup's next
+    // weights can be on their way while it has nothing else to do, long before the poll that precedes
+    // their use (a wave's loads return in order: a poll issued behind a batch of weights comes back after
+    // it).  Attention chunks, the output projection and gate/up start at workgroup 0; q/k/v and the down
+    // projection (whole K per strip: 24 k-step tiles per wave, no partial sums) at the far end.
+    dn.nstrips = (d + 15) / 16;
+    qkv.wg0 = max(0, nwg - qkv.nstrips);
+    dn.wg0 = max(0, nwg - dn.nstrips);
+    const bool has_attn = (int)blockIdx.x < Hkv * a.ns;
+    const bool has_dn = phase_block(dn) < dn.nstrips;
+    // ahead of the first layer: gate/up and output projection weights, the first K/V tile, q/k/v weights
+    // (q/k/v last: its prefetch leaves norm1's weights in pre.g and the rotary pair in pre.r)
+    prj.tout = a.tg;  // (marks the tagged mode for the prefetch: the residual is fetched by the phase itself)
+    gu.wp = lds_ptr<const uint4>(ptab, 2); gu.norm_w = lds_ptr<const bf16_t>(ptab, 5);
+    gemm_prefetch<2, 12, E_SWIGLU, 6>(gu, pre, 1);
+    uint4 g2[2] = {pre.g[0], pre.g[1]};  // norm2's weights
+    prj.wp = lds_ptr<const uint4>(ptab, 1);
+    gemm_prefetch<4, 6, E_RESID, 18>(prj, pre, 1);
+    gemm_prefetch<4, 6, E_ROPE>(qkv, pre, 1);
+    char* wl = reinterpret_cast<char*>(((uintptr_t)(ptab + m.n_layers * 8) + 255) & ~(uintptr_t)255);  // 4 x OHARA_LDS_PF KB
+    dn.wlds_addr = (uint32_t)(uintptr_t)(OHARA_LDS char*)wl;
+    pf.stamp();
+    for (int l = 0; l < m.n_layers; ++l) {
+      const unsigned long long* pl = ptab + l * 8;
+      bf16_t* kc = lds_ptr<bf16_t>(pl, 6);
+      bf16_t* vc = lds_ptr<bf16_t>(pl, 7);
+      float* p_l = a.pm + (size_t)l * a.pm_stride;
+      char* xt = a.tg + (size_t)l * a.tg_stride;   // the stream after the attention block
+      char* xn = xt + a.tg_n;                       // the stream after the layer
+      char* qt = xt + a.tg_q;
+      char* kvt = xt + a.tg_kv;
+      char* at = xt + a.tg_a;
+      const char* xn_prev = xn - a.tg_stride;       // (l > 0)
+      // the first K/V tile of this workgroup's attention chunk (the attention workgroups have no q/k/v strip: nothing
+      // of theirs is polled for until q is)
+      if (has_attn) attn_prefetch<D>(1, Hkv, m.t_max, a.ns, kc, vc, L, apre);
+      // P1: [embedding | poll for the stream] + norm1 + QKV + rotary + append; q and the new k / v rows are left tagged
+      qkv.kc = kc; qkv.vc = vc; qkv.out = nullptr; qkv.tout = qt; qkv.tkv = kvt;
+      if (phase_block(qkv) < qkv.nstrips) {
+        if (l == 0) stage_norm<2, true, true, false>(xs, ldxs, a.xm, 0, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, 1, d, pre.g);
+        else stage_norm_tagged<2>(xs, xn_prev, pc, m.eps, d, pre.g);
+      }
+      __syncthreads();
+      pf.stamp();  // 1: row polled for + norm1 in LDS
+      gemm_phase<4, 6, E_ROPE, ProfT<PROFILE>, 0, true>(qkv, pre, xs, ldxs, 1, red, best_v, best_i, pf);  // 2 stamps
+      // the down projection's weights (98 KB a workgroup): on their way from here, used after P4
+      dn.wp = lds_ptr<const uint4>(pl, 3); dn.tout = xn; dn.tresid = xt;
+      if (has_dn) gemm_prefetch_lds<4, E_XNEXT>(dn, wl);
+      pf.stamp();  // 4: rotary epilogue, tagged stores issued
+      // P2: attention partials (polls for q; the chunk that holds the new position polls for its k / v rows)
+      attn_phase<D, G, true>(1, H, Hkv, m.t_max, a.blk_x, a.ns, apre, nullptr, p_l, kc, vc, L, att, qt, kvt, &pc);
+      gs.arrive(pf);  // 4 stamps
+      gs.wait(pf);    // 2 stamps
+      pf.stamp();
+      // P3: merge + output projection + residual
+      prj.tout = xt; prj.tresid = l > 0 ? xn_prev : nullptr; prj.resid_embed = l == 0;
+      if ((int)blockIdx.x < prj.nstrips) stage_attn_merge_any<false>(a.ns, xs, ldxs, p_l, 1, H, D, mrg_w, mrg_l);
+      __syncthreads();
+      pf.stamp();  // merge in LDS
+      gemm_phase<4, 6, E_RESID, ProfT<PROFILE>, 18, true>(prj, pre, xs, ldxs, 1, red, best_v, best_i, pf);  // 2 stamps
+      pf.stamp();  // residual epilogue
+      // P4: polls for the stream, norm2 + gate/up + SwiGLU; the activations are left tagged
+      gu.out = nullptr; gu.tout = at;
+      if (phase_block(gu) * 2 < gu.nstrips) stage_norm_tagged<2>(xs, xt, pc, m.eps, d, g2);
+      __syncthreads();
+      pf.stamp();  // stream polled for + norm2 in LDS
+      gemm_phase<2, 12, E_SWIGLU, ProfT<PROFILE>, 6, true>(gu, pre, xs, ldxs, 1, red, best_v, best_i, pf);  // 2 stamps
+      // What the next layer needs of this workgroup is requested now, a phase and a half before its use:
+      // q/k/v weights (+ norm1 weights), the first K/V tile, output projection and gate/up weights (+ norm2's).
+      // The workgroups of the down projection hold its weights in the gate/up slots and fetch only q/k/v here.
+      // (the workgroups of the down projection do this after it: the wait for their LDS tiles would wait for these too)
+      auto next_weights = [&]() {
+        if (l + 1 < m.n_layers) {
+          qkv.wp = lds_ptr<const uint4>(pl, 8);
+          qkv.norm_w = lds_ptr<const bf16_t>(pl, 12);
+          gu.wp = lds_ptr<const uint4>(pl, 10); gu.norm_w = lds_ptr<const bf16_t>(pl, 13);
+          gemm_prefetch<2, 12, E_SWIGLU, 6>(gu, pre, 1);
+          g2[0] = pre.g[0]; g2[1] = pre.g[1];
+          prj.wp = lds_ptr<const uint4>(pl, 9);
+          gemm_prefetch<4, 6, E_RESID, 18>(prj, pre, 1);
+          gemm_prefetch<4, 6, E_ROPE>(qkv, pre, 1);
+        } else {
+          gemm_prefetch<1, 24, E_LOGITS>(lm, pre, 1);  // the vocabulary projection's first tiles (+ the final norm's weights)
+        }
+      };
+      if (!has_dn) next_weights();
+      pf.stamp();  // SwiGLU epilogue, next layer's weights requested
+      // P5: polls for the activations, down projection + residual; the stream is left tagged
+      if (has_dn) stage_act_tagged(xs, at, pc, 0, F);
+      __syncthreads();
+      pf.stamp();  // activations polled for, in LDS
+      gemm_phase<4, 12, E_XNEXT, ProfT<PROFILE>, 0, true>(dn, pre, xs, ldxs, 1, red, best_v, best_i, pf);  // 2 stamps
+      if (has_dn) next_weights();
+      pf.stamp();  // x_next stored
+    }
+    // final norm + vocabulary projection: the stream of the last layer is polled for like any other
+    pf.stamp();
+    stage_norm_tagged<2>(xs, a.tg + (size_t)(m.n_layers - 1) * a.tg_stride + a.tg_n, pc, m.eps, d, pre.g);
+    __syncthreads();
+    pf.stamp();
+    pf.stamp();
+   }
+  }
+  if constexpr (!ONE) {
   gemm_prefetch<4, 6, E_ROPE>(qkv, pre, B);
   pf.stamp();
   for (int l = 0; l < m.n_layers; ++l) {
@@ -204,6 +331,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
                              a.dm + (size_t)(m.n_layers - 1) * a.dm_stride, a.ids, m.token_emb, V, m.final_norm, m.eps, B, d,
                              pre.g);
   __syncthreads();
+  }
   lm_phase(lm, pre, xs, ldxs, B, best_v, best_i, pf);
   pf.stamp();
   if (a.select) {
@@ -285,14 +413,13 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
 
 // ---- workspace layout ------------------------------------------------------------------
 #define OHARA_BAR_WORDS(nwg) ((((nwg) + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP + 12) * 64)
-#define OHARA_PROF_SLOTS 1024
 
 size_t mega_al(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct MegaLayout {
-  size_t layers, kptr, vptr, xm, qm, am, pm, dm, candv, candi, prof, bar, total;
-  size_t xm_stride, qm_stride, am_stride, pm_stride, dm_stride;
-  int blk_x, blk_a;
+  size_t layers, kptr, vptr, xm, qm, am, pm, dm, candv, candi, prof, bar, tg, total;
+  size_t xm_stride, qm_stride, am_stride, pm_stride, dm_stride, tg_stride;
+  int blk_x, blk_a, tg_n, tg_q, tg_kv, tg_a;
 };
 
 MegaLayout mega_layout(const OharaModel* m, int B, int nwg) {
@@ -317,8 +444,15 @@ MegaLayout mega_layout(const OharaModel* m, int B, int nwg) {
   L.dm = o; o += L.dm_stride * sizeof(float) * NL;
   L.candv = o; o += mega_al((size_t)nwg * B * sizeof(float));
   L.candi = o; o += mega_al((size_t)nwg * B * sizeof(int));
-  L.prof = o; o += mega_al(OHARA_PROF_SLOTS * sizeof(unsigned long long));
+  L.prof = o; o += mega_al((size_t)nwg * OHARA_PROF_SLOTS * sizeof(unsigned long long));
   L.bar = o; o += mega_al(OHARA_BAR_WORDS(nwg) * sizeof(unsigned int));
+  // tagged mailboxes (batch 1; 8 bytes per two values), behind the barrier words: cleared with them
+  L.tg_n = (int)mega_al((size_t)m->d_model * 4);
+  L.tg_q = 2 * L.tg_n;
+  L.tg_kv = L.tg_q + (int)mega_al((size_t)m->n_heads * D * 4);
+  L.tg_a = L.tg_kv + (int)mega_al((size_t)2 * m->n_kv_heads * D * 4);
+  L.tg_stride = L.tg_a + mega_al((size_t)((m->d_ff + 7) / 8 * 8) * 4);
+  L.tg = o; o += L.tg_stride * NL;
   L.total = o;
   return L;
 }
@@ -372,6 +506,7 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   a.cand_val = reinterpret_cast<float*>(ws + L.candv);
   a.cand_idx = reinterpret_cast<int*>(ws + L.candi);
   a.bar = reinterpret_cast<unsigned int*>(ws + L.bar);
+  a.tg = ws + L.tg; a.tg_stride = L.tg_stride; a.tg_n = L.tg_n; a.tg_q = L.tg_q; a.tg_kv = L.tg_kv; a.tg_a = L.tg_a;
   if (init_workspace) {
     // small synchronous copies: done once per (model, cache) binding, outside any capture
     if (hipMemcpyAsync((void*)a.layers_dev, m->layers, sizeof(OharaLayer) * m->n_layers, hipMemcpyHostToDevice, st) !=
@@ -406,7 +541,11 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   if (!(2 * ns >= 3 * p2 && attn_merge_width(ns) <= 8)) ns = p2;
   a.ns = ns;
   const size_t mrg = (size_t)2 * ((s->batch * m->n_heads * attn_merge_width(ns) + 1) & ~1) * sizeof(float);
-  const size_t smem = xs_bytes + 4096 + (size_t)(8 + 4 * D) * G * sizeof(float) + mrg + (size_t)m->n_layers * 64;
+  // the batch-1 build parks the down projection's tiles in LDS (4 waves x OHARA_LDS_PF KB)
+  const int n_dn = (m->d_model + 15) / 16, n_gu = (2 * ((m->d_ff + 7) / 8 * 8) / 16 + 1) / 2;
+  const bool one = s->batch == 1 && n_gu + n_dn <= n_workgroups && 2 * n_dn <= n_workgroups;
+  const size_t smem = xs_bytes + 4096 + (size_t)(8 + 4 * D) * G * sizeof(float) + mrg + (size_t)m->n_layers * 64 +
+                      (one ? 256 + (size_t)4 * OHARA_LDS_PF * 1024 : 0);
   if (smem > 160 * 1024) return OHARA_ESIZE;
   dim3 grid(n_workgroups), block(256);
 #define OHARA_MEGA_B(DD, GG, ONE_)                                                                          \
@@ -421,7 +560,7 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   } while (0)
 #define OHARA_MEGA(DD, GG)                                                                                  \
   do {                                                                                                      \
-    if (s->batch == 1) OHARA_MEGA_B(DD, GG, true);                                                          \
+    if (one) OHARA_MEGA_B(DD, GG, true);                                                                    \
     else OHARA_MEGA_B(DD, GG, false);                                                                       \
   } while (0)
 #define OHARA_MEGA_PROF(ONE_)                                                                               \
@@ -434,8 +573,9 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
       return OHARA_ESIZE;                                                                                   \
     hipLaunchKernelGGL((decode_mega_kernel<128, 1, ONE_, true>), grid, block, smem, st, a);                 \
   } while (0)
+  // (`one`: the batch-1 build wants every phase's units on their own stretch of the grid)
   if (a.prof && D == 128 && G == 1) {  // the stamps exist in these two instantiations only
-    if (s->batch == 1) OHARA_MEGA_PROF(true);
+    if (one) OHARA_MEGA_PROF(true);
     else OHARA_MEGA_PROF(false);
   } else if (D == 128 && G == 1) OHARA_MEGA(128, 1);
   else if (D == 128 && G == 2) OHARA_MEGA(128, 2);

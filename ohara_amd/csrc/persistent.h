@@ -32,10 +32,12 @@ namespace {
 
 
 #define OHARA_MEGA_NS 16  // context chunks per (sequence, kv head)
-#define OHARA_MAX_PF 24   // weight tiles (16 B per lane) a wave fetches ahead of a phase
+#define OHARA_MAX_PF 24   // weight tiles (16 B per lane) a wave holds fetched ahead of its phases
+#define OHARA_LDS_PF 24   // weight tiles a wave can park in LDS (E_XNEXT: the down projection of the batch-1 kernels)
 #define OHARA_DOWN_SPLIT 4  // K partitions of the down projection (static_assert below: x_load sums four)
 
-// Optional fine-grained timeline: thread 0 of workgroup 0 records the shader clock.  The stamps are
+// Optional fine-grained timeline: thread 0 of every workgroup records the constant 100 MHz clock
+// (the same counter on every XCD, so that workgroups can be compared).  The stamps are
 // compiled in only for kernels instantiated with ON (dozens of clock reads and guarded stores per
 // layer are several KB of code the ordinary kernel does not have to fetch).
 template <bool ON>
@@ -46,7 +48,7 @@ struct ProfT<true> {
   int n;
   __device__ __forceinline__ explicit ProfT(unsigned long long* q) : p(q), n(0) {}
   __device__ __forceinline__ void stamp() {
-    if (p) p[n] = __builtin_readcyclecounter();
+    if (p) p[n] = __builtin_amdgcn_s_memrealtime();
     ++n;
   }
 };
@@ -169,6 +171,51 @@ __device__ __forceinline__ float dot8m(uint4 a, uint4 b, float s) {
   s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.z), __builtin_bit_cast(bf16x2, b.z), s, false);
   s = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a.w), __builtin_bit_cast(bf16x2, b.w), s, false);
   return s;
+}
+
+// ---------------------------------------------------------------------------------------
+// Tagged mailboxes: hand-offs of a single row (batch 1) WITHOUT a grid barrier.  An entry is 8 bytes,
+// {two bf16 values, tag}, written with one device-scope store, so whoever sees the tag of this launch
+// sees the values that came with it.  The tag is the launch's first barrier index (GridSync::k at
+// start): it grows with every launch, the mailboxes are cleared together with the barrier words, and
+// each entry is written once per launch - an entry of this launch cannot be mistaken for an older one.
+// Consumers poll the entries they need with device-scope loads (0.13 us a round, the producer's store
+// shows up ~0.6 us after it was issued) instead of waiting for a barrier (~1.6 us), for the producers'
+// own wait for their stores before it, and then fetching the data cold; every poll loop is bounded like
+// the barrier's spins.  Only worth it where a consumer needs little (the 768 values of a row, the 128
+// of a head): polled by 200 workgroups, tens of KB per consumer would swamp the memory fabric.
+// ---------------------------------------------------------------------------------------
+struct Poll {
+  uint32_t tag;
+  unsigned int limit;
+  unsigned int* err;
+};
+__device__ __forceinline__ bool poll_expired(const Poll& pc, unsigned int& spins) {
+  if (++spins > pc.limit) {
+    __hip_atomic_store(pc.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return true;
+  }
+  return (spins & 63u) == 0 && __hip_atomic_load(pc.err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+}
+// four values starting at column `col` (a multiple of 4): two entries
+__device__ __forceinline__ void st_tag4(char* base, int col, uint32_t lo, uint32_t hi, uint32_t tag) {
+  char* q = base + (size_t)(col >> 1) * 8;
+  st_coh8(q, make_uint2(lo, tag));
+  st_coh8(q + 8, make_uint2(hi, tag));
+}
+// eight values starting at column `col` (a multiple of 8): four entries; true when all carry `tag`
+__device__ __forceinline__ bool ld_tag8(const char* base, int col, uint32_t tag, uint4& out) {
+  const char* q = base + (size_t)(col >> 1) * 8;
+  const uint4 a = ld_coh16(q), b = ld_coh16(q + 16);
+  out = make_uint4(a.x, a.z, b.x, b.z);
+  return a.y == tag && a.w == tag && b.y == tag && b.w == tag;
+}
+
+// One entry's tag (entry index `e`): the cheap poll.  The entries of a 16-value strip leave the producer
+// in two store instructions of one wave, so its last entry (index 8 s + 7) is the last to appear; a
+// consumer polls one such entry per strip it needs, then loads everything and checks every tag.
+__device__ __forceinline__ bool tag_seen(const char* base, int e, uint32_t tag) {
+  return ld_coh8(base + (size_t)e * 8).y == tag;
 }
 
 // Strip-blocked mailbox of a (B, N) bf16 matrix: the 16 columns [16s, 16s+16) of all rows
@@ -339,6 +386,74 @@ __device__ __forceinline__ void stage_act(bf16_t* xs, int ldxs, const char* src,
   }
 }
 
+// The row of a tagged mailbox (batch 1) -> norm.py:16-21 -> LDS, by wave 0: stage_norm on a row that is
+// polled for instead of fetched after a barrier.  The norm weights were fetched ahead (gpre).
+template <int NLD>
+__device__ __forceinline__ void stage_norm_tagged(bf16_t* xs, const char* xt, const Poll& pc, float eps, int K,
+                                                  const uint4 (&gpre)[NLD]) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  if (tid >= 64) return;
+  uint4 v[NLD];
+  unsigned int spins = 0;
+  const int nstr = (K + 15) >> 4;  // producer strips (<= 64 for K <= 1024); lane s watches strip s
+  for (;;) {
+    while (!__all(lane >= nstr || tag_seen(xt, lane * 8 + (min(K, lane * 16 + 16) - lane * 16 - 1) / 2, pc.tag))) {
+      if (poll_expired(pc, spins)) break;
+    }
+    bool ok = true;
+#pragma unroll
+    for (int c = 0; c < NLD; ++c) {
+      const int k = (c * 64 + lane) * 8;
+      ok = ld_tag8(xt, k < K ? k : 0, pc.tag, v[c]) && ok;
+    }
+    if (__all(ok) || poll_expired(pc, spins)) break;
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < NLD; ++c) {
+    if ((c * 64 + lane) * 8 >= K) v[c] = make_uint4(0, 0, 0, 0);
+    const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float a0 = lo_bf(w[i]), a1 = hi_bf(w[i]);
+      ss += a0 * a0 + a1 * a1;
+    }
+  }
+  ss = wave_sum(ss);
+  const float rinv = 1.0f / sqrtf(ss / (float)K + eps);
+#pragma unroll
+  for (int c = 0; c < NLD; ++c) {
+    const int k = (c * 64 + lane) * 8;
+    if (k < K) {
+      const uint32_t xv[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+      const uint32_t gv[4] = {gpre[c].x, gpre[c].y, gpre[c].z, gpre[c].w};
+      uint32_t o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        o[i] = pack_bf(rbf(lo_bf(xv[i]) * rinv) * lo_bf(gv[i]), rbf(hi_bf(xv[i]) * rinv) * hi_bf(gv[i]));
+      sts16(xs + k, make_uint4(o[0], o[1], o[2], o[3]));
+    }
+  }
+}
+
+// Columns [f0, f1) (multiples of 8) of the tagged act mailbox (batch 1) -> LDS
+__device__ __forceinline__ void stage_act_tagged(bf16_t* xs, const char* at, const Poll& pc, int f0, int f1) {
+  const int n8 = (f1 - f0) >> 3;
+  for (int i = threadIdx.x; i < n8; i += blockDim.x) {
+    const int c = (f0 >> 3) + i;
+    // the eight values of a thread are one producer strip's, stored by one instruction: poll its last entry
+    uint4 v;
+    unsigned int spins = 0;
+    for (;;) {
+      while (!tag_seen(at, c * 4 + 3, pc.tag)) {
+        if (poll_expired(pc, spins)) break;
+      }
+      if (ld_tag8(at, c * 8, pc.tag, v) || poll_expired(pc, spins)) break;
+    }
+    sts16(xs + c * 8, v);
+  }
+}
+
 // Merge of the attention partials of all chunks, in chunk order (llama.py:116-123 output,
 // rounded to bf16 as SDPA's result is) -> xs[b][h*Dh + d].  NS (a power of two) chunks are in use.
 // The (max, sum) pairs of every (sequence, head, chunk) are fetched in one round into LDS and
@@ -503,7 +618,7 @@ __device__ __forceinline__ void stage_attn_merge_any(int ns, bf16_t* xs, int ldx
 // weights of a workgroup's first strip(s) - and the residual it will add - are fetched
 // into registers between arrive() and wait() of the barrier that precedes the phase.
 // ---------------------------------------------------------------------------------------
-enum { E_RESID = 1, E_SWIGLU = 2, E_ROPE = 3, E_LOGITS = 4, E_PART = 5 };
+enum { E_RESID = 1, E_SWIGLU = 2, E_ROPE = 3, E_LOGITS = 4, E_PART = 5, E_XNEXT = 6 };  // E_XNEXT: the whole down projection + residual (batch-1 kernels)
 
 struct GemmP {
   const uint4* wp;
@@ -527,7 +642,20 @@ struct GemmP {
   int valid;       // E_LOGITS: ids >= valid never win
   int ldo;         // E_LOGITS: row stride of the logits
   const bf16_t* norm_w;  // weights of the norm staged ahead of this phase (fetched with the weights when set)
+  // batch-1 kernels with tagged hand-offs (TAG): where the epilogue leaves its row for the consumers that poll
+  char* tout;      // E_RESID: the residual stream (besides `out`); E_SWIGLU: the activations; E_ROPE: the q rows
+  char* tkv;       // E_ROPE: the new key row, then the new value row (besides the cache)
+  const char* tresid;  // E_RESID (unless resid_embed), E_XNEXT: the tagged row that is added to the product
+  uint32_t wlds_addr;  // E_XNEXT: LDS byte address of the workgroup's parked tiles, OHARA_LDS_PF per wave (gemm_prefetch_lds)
+  const Poll* poll;
+  uint32_t tag;
+  int wg0;         // the workgroup that takes the phase's first unit (units go to wg0, wg0 + 1, ... round the grid)
 };
+// A workgroup's position in a phase whose units start at workgroup p.wg0.
+__device__ __forceinline__ int phase_block(const GemmP& p) {
+  const int v = (int)blockIdx.x - p.wg0;
+  return v < 0 ? v + (int)gridDim.x : v;
+}
 
 struct GemmPre {  // one register buffer, reused by every phase (only one prefetch is live at a time)
   uint4 w[OHARA_MAX_PF];
@@ -559,14 +687,16 @@ __device__ __forceinline__ bool gemm_unit(const GemmP& p, int unit, int kpart, i
   return live;
 }
 
-template <int KP, int PF, int EPI>
+// PO: first slot of pre.w this phase's tiles go to (several phases' weights can be held at once)
+template <int KP, int PF, int EPI, int PO = 0>
 __device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int B) {
+  static_assert(PO + PF <= OHARA_MAX_PF, "prefetch buffer");
   constexpr int SPW = 4 / KP;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub = wave / KP, kpart = wave % KP;
   const int KS = (p.K + 31) >> 5;
   int strip, j0, j1;
-  const bool live = gemm_unit<KP, EPI>(p, (int)blockIdx.x * SPW + sub, kpart, KS, strip, j0, j1);
+  const bool live = gemm_unit<KP, EPI>(p, phase_block(p) * SPW + sub, kpart, KS, strip, j0, j1);
   // Everything else the phase reads that does not depend on the phase before it is requested here
   // too: cold reads from HBM behind the barrier would sit on the critical path of the phase.
   if (EPI == E_ROPE || EPI == E_SWIGLU || EPI == E_LOGITS) {
@@ -591,7 +721,7 @@ __device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int 
     const int m = lane & 15, g = lane >> 4;
     const int r0 = strip * 16 + 4 * g;
     pre.r = make_uint2(0, 0);
-    if (live && kpart == 0 && m < B && r0 < p.N) {
+    if (live && kpart == 0 && m < B && r0 < p.N && !p.tout) {  // (tagged mode: the residual is fetched by the phase itself)
       if (!p.resid_embed) {
         static_assert(EPI != E_RESID || PF <= OHARA_PRE_RESID, "the residual's pieces share the weight buffer");
         XRaw<4, true> t;
@@ -611,10 +741,35 @@ __device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int 
   const uint4* wrow = p.wp + (size_t)strip * KS * 64 + lane;
 #pragma unroll
   for (int c = 0; c < PF; ++c)
-    pre.w[c] = (live && j0 + c < j1) ? ldg16_nt(wrow + (size_t)(j0 + c) * 64) : make_uint4(0, 0, 0, 0);
+    pre.w[PO + c] = (live && j0 + c < j1) ? ldg16_nt(wrow + (size_t)(j0 + c) * 64) : make_uint4(0, 0, 0, 0);
 }
 
-template <int KP, int PF, int EPI, class PROF>
+// The weights of a workgroup's first unit straight into LDS (global_load_lds: 16 bytes per lane, a wave's
+// load lands as one contiguous 1 KB tile; no registers are held while they travel): wave w's tile c at
+// wl + (w * OHARA_LDS_PF + c) KB.  The wave that issued them waits for its own (vmcnt) before it reads.
+template <int KP, int EPI>
+__device__ __forceinline__ void gemm_prefetch_lds(const GemmP& p, char* wl) {
+  constexpr int SPW = 4 / KP;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub = wave / KP, kpart = wave % KP;
+  const int KS = (p.K + 31) >> 5;
+  int strip, j0, j1;
+  const bool live = gemm_unit<KP, EPI>(p, phase_block(p) * SPW + sub, kpart, KS, strip, j0, j1);
+  if (!live) return;
+  // a rolled loop with a running address: unrolled, the compiler computed all 24 addresses first, spilled
+  // them, and waited for every earlier load before each reload
+  const uint4* src = p.wp + ((size_t)strip * KS + j0) * 64 + lane;
+  char* dst = wl + (size_t)wave * OHARA_LDS_PF * 1024;
+  const int n = min(j1 - j0, OHARA_LDS_PF);
+#pragma unroll 1
+  for (int c = 0; c < n; ++c) {
+    __builtin_amdgcn_global_load_lds((const OHARA_GLOBAL void*)src, (OHARA_LDS void*)dst, 16, 0, 0);
+    src += 64;
+    dst += 1024;
+  }
+}
+
+template <int KP, int PF, int EPI, class PROF, int PO = 0, bool TAG = false>
 __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, const bf16_t* xs, int ldxs, int B,
                                            float* red, float& best_v, int& best_i, PROF& pf) {
   constexpr int SPW = 4 / KP;
@@ -630,32 +785,68 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
 
 #pragma unroll 1
   for (int it = 0; it < iters; ++it) {
-    const int unit = (it * nwg + blockIdx.x) * SPW + sub;
+    const int unit = (it * nwg + phase_block(p)) * SPW + sub;
     int strip, j0, j1;
     const bool live = gemm_unit<KP, EPI>(p, unit, kpart, KS, strip, j0, j1);
     f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+    // TAG: the four residual values of this lane (two entries of a tagged row that has been visible for a
+    // while), requested ahead of the products and checked in the epilogue
+    const bool tres = TAG && (EPI == E_XNEXT || (EPI == E_RESID && !p.resid_embed)) && live && kpart == 0 && mine &&
+                      strip * 16 + 4 * g < p.N;
+    uint4 rx = make_uint4(0, 0, 0, 0);
+    if (tres) rx = ld_coh16(p.tresid + (size_t)((strip * 16 + 4 * g) >> 1) * 8);
     if (live) {
       const uint4* wrow = p.wp + (size_t)strip * KS * 64 + lane;
 #pragma unroll 1
       for (int jc = j0; jc < j1; jc += PF) {
         uint4 wv[PF];
-        if (it == 0 && jc == j0) {
-#pragma unroll
-          for (int c = 0; c < PF; ++c) wv[c] = pre.w[c];
-        } else {
-#pragma unroll
-          for (int c = 0; c < PF; ++c)
-            wv[c] = (jc + c < j1) ? ldg16_nt(wrow + (size_t)(jc + c) * 64) : make_uint4(0, 0, 0, 0);
-        }
-        // The activations of all PF k-steps are read from LDS before the first product: they do not
-        // depend on the weights, and left next to their products every read's latency is exposed
-        // (read, wait, product, PF times) on the critical path of the phase.
         uint4 xv[PF];
+        // The usual case - all PF k-steps of the chunk exist and lie inside K - runs without a predicate per
+        // k-step: one wave per SIMD issues an instruction every few cycles, so a phase costs what its
+        // instruction count costs, and a predicated k-step is fifteen instructions where three do (weight
+        // tile from LDS / nothing for a register tile, activations from LDS, product).  Lanes of batch
+        // columns that do not exist read row 0: their products land in output columns nobody stores.
+        const bool full = jc + PF <= j1 && 32 * (jc + PF) <= p.K;
+        if (full) {
+          const uint32_t xa = (uint32_t)(uintptr_t)(const OHARA_LDS bf16_t*)(xs + (size_t)(mine ? m : 0) * ldxs + 8 * g) + 64u * jc;
+          if (EPI == E_XNEXT && it == 0 && jc - j0 + PF <= OHARA_LDS_PF) {  // parked in LDS by gemm_prefetch_lds
+            if (jc == j0) wait_own_stores();  // this wave's own loads into LDS have landed
+            const uint32_t wa = p.wlds_addr + ((uint32_t)(wave * OHARA_LDS_PF + (jc - j0)) * 64 + lane) * 16;
 #pragma unroll
-        for (int c = 0; c < PF; ++c) {
-          xv[c] = make_uint4(0, 0, 0, 0);
-          if (mine && jc + c < j1 && 32 * (jc + c) + 8 * g < p.K)
-            xv[c] = *reinterpret_cast<const uint4*>(xrow + 32 * (jc + c));
+            for (int c = 0; c < PF; ++c) wv[c] = lds16_at(wa + c * 1024);
+          } else if (EPI != E_XNEXT && it == 0 && jc == j0) {
+#pragma unroll
+            for (int c = 0; c < PF; ++c) wv[c] = pre.w[PO + c];
+          } else {
+#pragma unroll
+            for (int c = 0; c < PF; ++c) wv[c] = ldg16_nt(wrow + (size_t)(jc + c) * 64);
+          }
+#pragma unroll
+          for (int c = 0; c < PF; ++c) xv[c] = lds16_at(xa + 64u * c);
+        } else {
+          if (EPI == E_XNEXT && it == 0 && jc - j0 + PF <= OHARA_LDS_PF) {
+            if (jc == j0) wait_own_stores();
+#pragma unroll
+            for (int c = 0; c < PF; ++c)
+              wv[c] = (jc + c < j1) ? lds16_at(p.wlds_addr + ((uint32_t)(wave * OHARA_LDS_PF + (jc - j0) + c) * 64 + lane) * 16)
+                                    : make_uint4(0, 0, 0, 0);
+          } else if (EPI != E_XNEXT && it == 0 && jc == j0) {
+#pragma unroll
+            for (int c = 0; c < PF; ++c) wv[c] = pre.w[PO + c];
+          } else {
+#pragma unroll
+            for (int c = 0; c < PF; ++c)
+              wv[c] = (jc + c < j1) ? ldg16_nt(wrow + (size_t)(jc + c) * 64) : make_uint4(0, 0, 0, 0);
+          }
+          // The activations of all PF k-steps are read from LDS before the first product: they do not
+          // depend on the weights, and left next to their products every read's latency is exposed
+          // (read, wait, product, PF times) on the critical path of the phase.
+#pragma unroll
+          for (int c = 0; c < PF; ++c) {
+            xv[c] = make_uint4(0, 0, 0, 0);
+            if (mine && jc + c < j1 && 32 * (jc + c) + 8 * g < p.K)
+              xv[c] = *reinterpret_cast<const uint4*>(xrow + 32 * (jc + c));
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -688,7 +879,24 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
       const int b = m;
       const int r0 = strip * 16 + 4 * g;
       const float y0 = rbf(acc[0]), y1 = rbf(acc[1]), y2 = rbf(acc[2]), y3 = rbf(acc[3]);
-      if (EPI == E_RESID) {  // N % 4 == 0 is required by the entry point
+      if (EPI == E_XNEXT || (TAG && EPI == E_RESID)) {  // batch 1: the row goes to the tagged mailbox only
+        if (r0 < p.N) {
+          uint2 r = make_uint2(0, 0);
+          if (tres) {
+            unsigned int spins = 0;
+            while (!(rx.y == p.tag && rx.w == p.tag)) {
+              if (poll_expired(*p.poll, spins)) break;
+              rx = ld_coh16(p.tresid + (size_t)(r0 >> 1) * 8);
+            }
+            r = make_uint2(rx.x, rx.z);
+          } else {  // the first half layer: the embedding row (llama.py:310)
+            int64_t id = ldg_i64(p.ids + b);
+            if (id < 0 || id >= p.vocab) id = 0;
+            r = ldg8(p.table + (size_t)id * p.N + r0);
+          }
+          st_tag4(p.tout, r0, pack_bf(lo_bf(r.x) + y0, hi_bf(r.x) + y1), pack_bf(lo_bf(r.y) + y2, hi_bf(r.y) + y3), p.tag);
+        }
+      } else if (EPI == E_RESID) {  // N % 4 == 0 is required by the entry point
         if (r0 < p.N) {
           uint2 r = pre.r;
           if (it == 0 && !p.resid_embed) {
@@ -711,8 +919,8 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
               r = ldg8(p.table + (size_t)id * p.N + r0);
             }
           }
-          st_coh8(const_cast<char*>(xm_addr(p.out, p.blk, b, r0)),
-                  make_uint2(pack_bf(lo_bf(r.x) + y0, hi_bf(r.x) + y1), pack_bf(lo_bf(r.y) + y2, hi_bf(r.y) + y3)));
+          const uint2 xo = make_uint2(pack_bf(lo_bf(r.x) + y0, hi_bf(r.x) + y1), pack_bf(lo_bf(r.y) + y2, hi_bf(r.y) + y3));
+          st_coh8(const_cast<char*>(xm_addr(p.out, p.blk, b, r0)), xo);
         }
       } else if (EPI == E_PART) {  // the raw fp32 sums of this K partition
         if (r0 < p.N) {
@@ -742,7 +950,8 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
         const int f = strip * 8 + 2 * g;
         if (f < p.N) {
           const float s0 = rbf(silu_f(y0)), s1 = rbf(silu_f(y1));
-          st_coh4(const_cast<char*>(am_addr(p.out, p.blk, b, f)), pack_bf(s0 * y2, s1 * y3));
+          if (TAG) st_coh8(p.tout + (size_t)(f >> 1) * 8, make_uint2(pack_bf(s0 * y2, s1 * y3), p.tag));
+          else st_coh4(const_cast<char*>(am_addr(p.out, p.blk, b, f)), pack_bf(s0 * y2, s1 * y3));
         }
       } else {  // E_ROPE
         const int nq = p.H * p.Dh, nk = p.Hkv * p.Dh;
@@ -765,7 +974,12 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
           } else {
             o = reinterpret_cast<char*>(p.vc + (((size_t)b * p.Tmax + p.pos) * p.Hkv) * p.Dh + (r0 - nq - nk));
           }
-          st_coh8(o, make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3])));
+          const uint2 ro = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
+          if (TAG) {  // attention polls for the q row and for the new key / value rows; the cache rows are for later steps
+            if (r0 < nq) st_tag4(p.tout, r0, ro.x, ro.y, p.tag);
+            else st_tag4(p.tkv, r0 - nq, ro.x, ro.y, p.tag);
+          }
+          if (!TAG || r0 >= nq) st_coh8(o, ro);
         }
       }
     }
@@ -904,19 +1118,21 @@ __device__ __forceinline__ void attn_tile_load(const bf16_t* kb, const bf16_t* v
 // compiler can count the loads in flight and wait for the current tile only while the next one is
 // on its way.  The row appended in this step is then fetched again with device-scope loads by the
 // lanes that hold it (a branch the whole wave takes or skips).
+// `last`: the last position these loads may touch (t1 - 1; one less where the row appended in this step
+// is not in the cache yet and will be patched in from its tagged mailbox).
 template <int D>
 __device__ __forceinline__ void attn_tile_load_u(const bf16_t* kb, const bf16_t* vb, size_t row, int tb, int t1,
-                                                 int coh_pos, uint4* kv, uint4* vv) {
+                                                 int coh_pos, uint4* kv, uint4* vv, int last) {
   constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
   const int lane = threadIdx.x & 63;
   const int p = lane & 15, dq = lane >> 4;
   const int pp = lane / DC, dc = lane % DC;
-  const int pos = min(tb + p, t1 - 1);
+  const int pos = min(tb + p, last);
 #pragma unroll
   for (int c = 0; c < NC; ++c) kv[c] = ldg16_nt(kb + (size_t)pos * row + (4 * c + dq) * 8);
 #pragma unroll
   for (int c = 0; c < NV; ++c) {
-    const int vp = min(tb + c * PP + pp, t1 - 1);
+    const int vp = min(tb + c * PP + pp, last);
     vv[c] = ldg16_nt(vb + (size_t)vp * row + dc * 8);
   }
   if (coh_pos >= tb && coh_pos < tb + 16) {  // wave-uniform: this tile holds the appended row
@@ -962,10 +1178,41 @@ __device__ __forceinline__ void attn_prefetch(int B, int Hkv, int Tmax, int ns, 
   attn_tile_load<D>(kb, vb, row, t0 + wave * 16, has ? t1 : 0, -1, pre.k, pre.v);
 }
 
-template <int D, int G>
+// The row appended in this step, taken from the tagged mailbox `kvt` (the new key row, then the new
+// value row: batch 1) by the lanes of the tile at `tb` that hold position `pos_new`; polls until the
+// row's entries carry this launch's tag.
+template <int D>
+__device__ __forceinline__ void attn_new_row_tagged(const char* kvt, const Poll& pc, int Hkv, int kvh, int tb, int t1,
+                                                    int pos_new, uint4* kv, uint4* vv) {
+  constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
+  const int lane = threadIdx.x & 63;
+  const int p = lane & 15, dq = lane >> 4;
+  const int pp = lane / DC, dc = lane % DC;
+  const int pos = min(tb + p, t1 - 1);
+  const int nk = Hkv * D;
+  unsigned int spins = 0;
+  for (;;) {
+    bool ok = true;
+    if (pos == pos_new) {
+#pragma unroll
+      for (int c = 0; c < NC; ++c) ok = ld_tag8(kvt, kvh * D + (4 * c + dq) * 8, pc.tag, kv[c]) && ok;
+    }
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+      const int vp = min(tb + c * PP + pp, t1 - 1);
+      if (vp == pos_new) ok = ld_tag8(kvt, nk + kvh * D + dc * 8, pc.tag, vv[c]) && ok;
+    }
+    if (__all(ok) || poll_expired(pc, spins)) break;
+  }
+}
+
+// TAG (batch 1): the q row and the row appended in this step come from tagged mailboxes (qt, kvt) that
+// are polled for - there is no barrier between the projection that writes them and this phase.
+template <int D, int G, bool TAG = false>
 __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int blk_x, int ns, const AttnPre<D>& pre,
                                            const char* qm, float* pm, const bf16_t* kc, const bf16_t* vc, int L,
-                                           float* lds) {
+                                           float* lds, const char* qt = nullptr, const char* kvt = nullptr,
+                                           const Poll* pc = nullptr) {
   constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int p = lane & 15;
@@ -994,22 +1241,42 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
     }
     if (t0 + wave * 16 < t1) {
       uint4 qv[G][NC];
-#pragma unroll
-      for (int hh = 0; hh < G; ++hh)
-#pragma unroll
-        for (int c = 0; c < NC; ++c)
-          qv[hh][c] = ldg16(xm_addr(qm, blk_x, b, (kvh * G + hh) * D + (4 * c + dq) * 8));
       // the tile after the current one is in flight while the current one is consumed
       const bool use_pre = first && attn_first_tile_prefetchable<D>(t0, t1, L);
       uint4 ka[NC], va[NV], kn[NC], vn[NV];
       int tb = t0 + wave * 16;
+      const int coh = TAG ? -1 : L - 1;  // TAG: the appended row is patched in from the tagged mailbox below ...
+      const int last = TAG ? max(min(t1, L - 1) - 1, 0) : t1 - 1;  // ... and its cache row is not touched
       if (use_pre) {
 #pragma unroll
         for (int c = 0; c < NC; ++c) ka[c] = pre.k[c];
 #pragma unroll
         for (int c = 0; c < NV; ++c) va[c] = pre.v[c];
       } else {
-        attn_tile_load_u<D>(kb, vb, row, tb, t1, L - 1, ka, va);
+        attn_tile_load_u<D>(kb, vb, row, tb, t1, coh, ka, va, last);
+      }
+      if (TAG) {
+        unsigned int spins = 0;
+        constexpr int NSTR = G * D / 16;  // the strips that produce this group's q rows (<= 32); lane s watches strip s
+        for (;;) {
+          while (!__all(lane >= NSTR || tag_seen(qt, (kvh * G * D) / 2 + lane * 8 + 7, pc->tag))) {
+            if (poll_expired(*pc, spins)) break;
+          }
+          bool ok = true;
+#pragma unroll
+          for (int hh = 0; hh < G; ++hh)
+#pragma unroll
+            for (int c = 0; c < NC; ++c)
+              ok = ld_tag8(qt, (kvh * G + hh) * D + (4 * c + dq) * 8, pc->tag, qv[hh][c]) && ok;
+          if (__all(ok) || poll_expired(*pc, spins)) break;
+        }
+        if (!use_pre && L - 1 >= tb && L - 1 < tb + 16) attn_new_row_tagged<D>(kvt, *pc, Hkv, kvh, tb, t1, L - 1, ka, va);
+      } else {
+#pragma unroll
+        for (int hh = 0; hh < G; ++hh)
+#pragma unroll
+          for (int c = 0; c < NC; ++c)
+            qv[hh][c] = ldg16(xm_addr(qm, blk_x, b, (kvh * G + hh) * D + (4 * c + dq) * 8));
       }
       auto consume = [&](int tb, const uint4* kv, const uint4* vv) {
         const bool valid = tb + p < t1;
@@ -1084,7 +1351,8 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
       // (a chunk is one or two tiles per wave here: the next tile goes through a second register set
       // and is copied over, which costs a wait but far fewer registers than two sets taking turns)
       for (; tb + 64 < t1; tb += 64) {
-        attn_tile_load_u<D>(kb, vb, row, tb + 64, t1, L - 1, kn, vn);
+        attn_tile_load_u<D>(kb, vb, row, tb + 64, t1, coh, kn, vn, last);
+        if (TAG && L - 1 >= tb + 64 && L - 1 < tb + 80) attn_new_row_tagged<D>(kvt, *pc, Hkv, kvh, tb + 64, t1, L - 1, kn, vn);
         consume(tb, ka, va);
 #pragma unroll
         for (int c = 0; c < NC; ++c) ka[c] = kn[c];

@@ -671,10 +671,11 @@ class DecodeSession:
                                                       self._nwg, 1, 1, 0, torch.cuda.current_stream().cuda_stream),
                   "persistent init")
 
-    def phase_clocks(self) -> torch.Tensor:
-        """Shader-clock samples of workgroup 0 at the phase boundaries of the last step run
-        with ``step(prof_kernel=-2)`` (measurement aid)."""
-        return self._pws[self._prof_off : self._prof_off + 8192].view(torch.int64).cpu()
+    def phase_clocks(self, workgroup: int = 0) -> torch.Tensor:
+        """Clock samples (constant 100 MHz counter) that thread 0 of ``workgroup`` took at the phase
+        boundaries of the last step run with ``step(prof_kernel=-2)`` (measurement aid)."""
+        off = self._prof_off + workgroup * 8192
+        return self._pws[off : off + 8192].view(torch.int64).cpu()
 
     def _room(self, n: int) -> None:
         if self._dst is None:
