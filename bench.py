@@ -562,18 +562,21 @@ def bench_phi(dev):
 _BAR = ["wait for own stores (vmcnt 0)", "workgroup barrier", "arrival atomics issued", "(window)",
         "spin on the release word + workgroup barrier", "(bookkeeping)"]
 _GEMM = ["activations in LDS -> MFMAs issued", "cross-wave sum"]
-# intervals between the clock samples of the batch-1 kernel (one grid barrier per layer, after the
-# attention partials; the other hand-offs are tagged mailboxes that the consumer polls for)
+# intervals between the clock samples of the batch-1 kernel (no grid barrier inside the layers: every
+# hand-off is a tagged mailbox, or a flag per attention chunk, that the consumer polls for)
 PHASE_STAMPS = (
     [("P1 qkv", "poll for the stream + norm1 into LDS")] + [("P1 qkv", x) for x in _GEMM]
-    + [("P1 qkv", "rotary epilogue, tagged stores, down weights requested")]
-    + [("P2 attention", "poll for q, attention chunk, partials stored")] + [("P2 attention", x) for x in _BAR]
-    + [("P3 wo", "merge of attention partials into LDS")] + [("P3 wo", x) for x in _GEMM]
+    + [("P1 qkv", "rotary epilogue, tagged stores")]
+    + [("P2 attention", "poll for q, attention chunk, partials stored, flag raised")]
+    + [("P2 attention", "next q/k/v and down weights requested")]
+    + [("P3 wo", "poll for the chunks' tags, merge of attention partials into LDS")] + [("P3 wo", x) for x in _GEMM]
     + [("P3 wo", "residual epilogue, tagged stores")]
     + [("P4 gate/up", "poll for the stream + norm2 into LDS")] + [("P4 gate/up", x) for x in _GEMM]
     + [("P4 gate/up", "SwiGLU epilogue, tagged stores")]
+    + [("P4 gate/up", "next layer's weights requested (all but the down projection's workgroups)")]
     + [("P5 down", "poll for the activations into LDS")] + [("P5 down", x) for x in _GEMM]
-    + [("P5 down", "residual epilogue, tagged stores, next layer's weights requested")]
+    + [("P5 down", "residual epilogue, tagged stores")]
+    + [("P5 down", "next layer's weights requested (the down projection's workgroups)")]
 )
 PHASE_TAIL = 13  # samples after the layers: three around the final norm, then as before
 

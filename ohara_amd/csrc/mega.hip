@@ -64,8 +64,8 @@ struct MegaArgs {
   bf16_t* logits;  // (B, V)
   int32_t* step_state;  // {pos, step, done, pad}
   int64_t* history;
-  char* tg;             // batch 1: NL blocks of tagged mailboxes, tg_stride bytes each, the stream after the attention block first
-  size_t tg_stride;
+  char* tg;             // batch 1: two sets of NL blocks of polled mailboxes, tg_stride bytes a block, tg_set bytes a set
+  size_t tg_stride, tg_set;
   int tg_n, tg_q, tg_kv, tg_a;  // byte offsets inside a layer's block: stream after the layer | q | new k, v | activations
   unsigned int* bar;    // barrier words, see GridSync
   unsigned long long* prof;  // optional: clock of every workgroup's thread 0 at every phase boundary (OHARA_PROF_SLOTS each)
@@ -104,6 +104,10 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
 
   GridSync gs;
   gs.init(a.bar, gridDim.x, a.spin_limit);
+  // batch 1: the number of this launch since the workspace was cleared, the tag of its hand-offs (read once, here: the
+  // last workgroup out advances it)
+  unsigned int* launches = a.bar + (gs.ng + 12) * 64;
+  const unsigned int nth = ONE ? *launches + 1u : 0u;
   const int pos = a.step_state[0];
   const int step = a.step_state[1];
   const int L = min(pos + 1, m.t_max);
@@ -132,31 +136,37 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   // their weights share registers - and the general build otherwise.
   if constexpr (ONE) {
    {
-    // ---- batch 1: tagged hand-offs, one grid barrier per layer ---------------------------------------
-    const Poll pc{gs.k, a.spin_limit, gs.err};
+    // ---- batch 1: tagged hand-offs, no grid barrier inside the layers ---------------------------------
+    const Poll pc{nth, a.spin_limit, gs.err};
     const int nwg = (int)gridDim.x;
-    qkv.tag = prj.tag = gu.tag = dn.tag = pc.tag;
-    qkv.poll = prj.poll = gu.poll = dn.poll = &pc;
+    // this launch's set of mailboxes, and the way from there to the other set
+    char* const tgs = a.tg + (size_t)(nth & 1u) * a.tg_set;
+    qkv.tother = prj.tother = gu.tother = dn.tother = (nth & 1u) ? -(ptrdiff_t)a.tg_set : (ptrdiff_t)a.tg_set;
+    qkv.poll = prj.poll = gu.poll = dn.poll = pc;
     // Who does what.  Every phase is a handful of units, and what a unit costs is the fetch of its weights
     // (a CU takes in ~55 GB/s) - so the phases are spread over the grid such that a workgroup's next
     // weights can be on their way while it has nothing else to do, long before the poll that precedes
     // their use (a wave's loads return in order: a poll issued behind a batch of weights comes back after
-    // it).  Attention chunks, the output projection and gate/up start at workgroup 0; q/k/v and the down
-    // projection (whole K per strip: 24 k-step tiles per wave, no partial sums) at the far end.
+    // it).  Attention chunks, the output projection and gate/up start at workgroup 0; q/k/v sits at the far
+    // end; the down projection (whole K per strip: 24 k-step tiles per wave from LDS, no partial sums)
+    // follows the output projection, clear of the workgroups that the next layer starts on.
     dn.nstrips = (d + 15) / 16;
     qkv.wg0 = max(0, nwg - qkv.nstrips);
-    dn.wg0 = max(0, nwg - dn.nstrips);
-    const bool has_attn = (int)blockIdx.x < Hkv * a.ns;
+    dn.wg0 = prj.nstrips + dn.nstrips <= nwg ? prj.nstrips : max(0, nwg - dn.nstrips);
+    const int n_chunks = Hkv * a.ns;
+    const bool has_attn = (int)blockIdx.x < n_chunks;
     const bool has_dn = phase_block(dn) < dn.nstrips;
+    const bool has_qkv = phase_block(qkv) < qkv.nstrips;
     // ahead of the first layer: gate/up and output projection weights, the first K/V tile, q/k/v weights
     // (q/k/v last: its prefetch leaves norm1's weights in pre.g and the rotary pair in pre.r)
-    prj.tout = a.tg;  // (marks the tagged mode for the prefetch: the residual is fetched by the phase itself)
+    prj.tout = tgs;  // (marks the polled mode for the prefetch: the residual is fetched by the phase itself)
     gu.wp = lds_ptr<const uint4>(ptab, 2); gu.norm_w = lds_ptr<const bf16_t>(ptab, 5);
-    gemm_prefetch<2, 12, E_SWIGLU, 6>(gu, pre, 1);
-    uint4 g2[2] = {pre.g[0], pre.g[1]};  // norm2's weights
+    uint4 g1[2], g2[2];  // norm1's and norm2's weights, the rotary pair: each prefetch writes its own
+    uint2 r1, r_unused;
+    gemm_prefetch<2, 12, E_SWIGLU, 6>(gu, pre, 1, g2, r_unused);
     prj.wp = lds_ptr<const uint4>(ptab, 1);
-    gemm_prefetch<4, 6, E_RESID, 18>(prj, pre, 1);
-    gemm_prefetch<4, 6, E_ROPE>(qkv, pre, 1);
+    gemm_prefetch<4, 6, E_RESID, 18>(prj, pre, 1, g2, r_unused);
+    gemm_prefetch<4, 6, E_ROPE>(qkv, pre, 1, g1, r1);
     char* wl = reinterpret_cast<char*>(((uintptr_t)(ptab + m.n_layers * 8) + 255) & ~(uintptr_t)255);  // 4 x OHARA_LDS_PF KB
     dn.wlds_addr = (uint32_t)(uintptr_t)(OHARA_LDS char*)wl;
     pf.stamp();
@@ -165,77 +175,90 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
       bf16_t* kc = lds_ptr<bf16_t>(pl, 6);
       bf16_t* vc = lds_ptr<bf16_t>(pl, 7);
       float* p_l = a.pm + (size_t)l * a.pm_stride;
-      char* xt = a.tg + (size_t)l * a.tg_stride;   // the stream after the attention block
+      char* xt = tgs + (size_t)l * a.tg_stride;    // the stream after the attention block
       char* xn = xt + a.tg_n;                       // the stream after the layer
       char* qt = xt + a.tg_q;
       char* kvt = xt + a.tg_kv;
       char* at = xt + a.tg_a;
       const char* xn_prev = xn - a.tg_stride;       // (l > 0)
+      const bool more = l + 1 < m.n_layers;
       // the first K/V tile of this workgroup's attention chunk (the attention workgroups have no q/k/v strip: nothing
       // of theirs is polled for until q is)
       if (has_attn) attn_prefetch<D>(1, Hkv, m.t_max, a.ns, kc, vc, L, apre);
       // P1: [embedding | poll for the stream] + norm1 + QKV + rotary + append; q and the new k / v rows are left tagged
       qkv.kc = kc; qkv.vc = vc; qkv.out = nullptr; qkv.tout = qt; qkv.tkv = kvt;
-      if (phase_block(qkv) < qkv.nstrips) {
-        if (l == 0) stage_norm<2, true, true, false>(xs, ldxs, a.xm, 0, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, 1, d, pre.g);
-        else stage_norm_tagged<2>(xs, xn_prev, pc, m.eps, d, pre.g);
+      if (has_qkv) {
+        if (l == 0) stage_norm<2, true, true, false>(xs, ldxs, a.xm, 0, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, 1, d, g1);
+        else stage_norm_tagged<2>(xs, xn_prev, pc, m.eps, d, g1);
       }
       __syncthreads();
       pf.stamp();  // 1: row polled for + norm1 in LDS
+      pre.r = r1;
       gemm_phase<4, 6, E_ROPE, ProfT<PROFILE>, 0, true>(qkv, pre, xs, ldxs, 1, red, best_v, best_i, pf);  // 2 stamps
-      // the down projection's weights (98 KB a workgroup): on their way from here, used after P4
-      dn.wp = lds_ptr<const uint4>(pl, 3); dn.tout = xn; dn.tresid = xt;
-      if (has_dn) gemm_prefetch_lds<4, E_XNEXT>(dn, wl);
       pf.stamp();  // 4: rotary epilogue, tagged stores issued
-      // P2: attention partials (polls for q; the chunk that holds the new position polls for its k / v rows)
-      attn_phase<D, G, true>(1, H, Hkv, m.t_max, a.blk_x, a.ns, apre, nullptr, p_l, kc, vc, L, att, qt, kvt, &pc);
-      gs.arrive(pf);  // 4 stamps
-      gs.wait(pf);    // 2 stamps
-      pf.stamp();
-      // P3: merge + output projection + residual
+      // P2: attention partials (polls for q; the chunk that holds the new position polls for its k / v rows); each chunk
+      // leaves the launch's tag behind its (max, sum) pair
+      attn_phase<D, G, true>(1, H, Hkv, m.t_max, a.blk_x, a.ns, apre, nullptr, p_l, kc, vc, L, att, qt, kvt, pc, true);
+      pf.stamp();  // 5: partials stored, flag raised
+      // the next layer's q/k/v weights (+ norm1's, the rotary pair): their registers are free again (behind the attention
+      // phase, which needs many: a workgroup without a chunk - at the usual sizes those with q/k/v strips - is here at once)
+      if (has_qkv && more) {
+        qkv.wp = lds_ptr<const uint4>(pl, 8);
+        qkv.norm_w = lds_ptr<const bf16_t>(pl, 12);
+        gemm_prefetch<4, 6, E_ROPE, 0, false>(qkv, pre, 1, g1, r1);  // (the rotary pair is the same in every layer)
+      }
+      // the down projection's weights (98 KB a workgroup) into LDS: on their way from here, used after P4
+      dn.wp = lds_ptr<const uint4>(pl, 3); dn.tout = xn; dn.tresid = xt;
+      if (has_dn) {
+        // (not before the chunk's flag has reached memory: behind the other waves' 72 KB of requests it was seen 1.5 us late)
+        if (has_attn) {
+          wait_own_stores();
+          __syncthreads();
+        }
+        gemm_prefetch_lds<4, E_XNEXT>(dn, wl);
+      }
+      pf.stamp();  // 6: requests issued
+      // P3: polls for every chunk's tag; merge + output projection + residual
       prj.tout = xt; prj.tresid = l > 0 ? xn_prev : nullptr; prj.resid_embed = l == 0;
-      if ((int)blockIdx.x < prj.nstrips) stage_attn_merge_any<false>(a.ns, xs, ldxs, p_l, 1, H, D, mrg_w, mrg_l);
+      if ((int)blockIdx.x < prj.nstrips) stage_attn_merge_any<false, true>(a.ns, xs, ldxs, p_l, 1, H, D, mrg_w, mrg_l, pc);
       __syncthreads();
-      pf.stamp();  // merge in LDS
+      pf.stamp();  // 7: merge in LDS
       gemm_phase<4, 6, E_RESID, ProfT<PROFILE>, 18, true>(prj, pre, xs, ldxs, 1, red, best_v, best_i, pf);  // 2 stamps
-      pf.stamp();  // residual epilogue
+      pf.stamp();  // 10: residual epilogue
       // P4: polls for the stream, norm2 + gate/up + SwiGLU; the activations are left tagged
       gu.out = nullptr; gu.tout = at;
       if (phase_block(gu) * 2 < gu.nstrips) stage_norm_tagged<2>(xs, xt, pc, m.eps, d, g2);
       __syncthreads();
-      pf.stamp();  // stream polled for + norm2 in LDS
+      pf.stamp();  // 11: stream polled for + norm2 in LDS
       gemm_phase<2, 12, E_SWIGLU, ProfT<PROFILE>, 6, true>(gu, pre, xs, ldxs, 1, red, best_v, best_i, pf);  // 2 stamps
-      // What the next layer needs of this workgroup is requested now, a phase and a half before its use:
-      // q/k/v weights (+ norm1 weights), the first K/V tile, output projection and gate/up weights (+ norm2's).
-      // The workgroups of the down projection hold its weights in the gate/up slots and fetch only q/k/v here.
+      // What the next layer needs of this workgroup besides q/k/v is requested now, a phase and a half before its use:
+      // output projection and gate/up weights (+ norm2's); after the last layer, the vocabulary projection's first tiles.
       // (the workgroups of the down projection do this after it: the wait for their LDS tiles would wait for these too)
       auto next_weights = [&]() {
-        if (l + 1 < m.n_layers) {
-          qkv.wp = lds_ptr<const uint4>(pl, 8);
-          qkv.norm_w = lds_ptr<const bf16_t>(pl, 12);
+        if (more) {
           gu.wp = lds_ptr<const uint4>(pl, 10); gu.norm_w = lds_ptr<const bf16_t>(pl, 13);
-          gemm_prefetch<2, 12, E_SWIGLU, 6>(gu, pre, 1);
-          g2[0] = pre.g[0]; g2[1] = pre.g[1];
+          gemm_prefetch<2, 12, E_SWIGLU, 6>(gu, pre, 1, g2, r_unused);
           prj.wp = lds_ptr<const uint4>(pl, 9);
-          gemm_prefetch<4, 6, E_RESID, 18>(prj, pre, 1);
-          gemm_prefetch<4, 6, E_ROPE>(qkv, pre, 1);
+          gemm_prefetch<4, 6, E_RESID, 18>(prj, pre, 1, g2, r_unused);
         } else {
-          gemm_prefetch<1, 24, E_LOGITS>(lm, pre, 1);  // the vocabulary projection's first tiles (+ the final norm's weights)
+          gemm_prefetch<1, 24, E_LOGITS>(lm, pre, 1);  // (+ the final norm's weights)
         }
       };
+      pf.stamp();  // SwiGLU epilogue
       if (!has_dn) next_weights();
-      pf.stamp();  // SwiGLU epilogue, next layer's weights requested
+      pf.stamp();  // next layer's weights requested
       // P5: polls for the activations, down projection + residual; the stream is left tagged
       if (has_dn) stage_act_tagged(xs, at, pc, 0, F);
       __syncthreads();
-      pf.stamp();  // activations polled for, in LDS
+      pf.stamp();  // 15: activations polled for, in LDS
       gemm_phase<4, 12, E_XNEXT, ProfT<PROFILE>, 0, true>(dn, pre, xs, ldxs, 1, red, best_v, best_i, pf);  // 2 stamps
-      if (has_dn) next_weights();
       pf.stamp();  // x_next stored
+      if (has_dn) next_weights();
+      pf.stamp();  // next layer's weights requested
     }
     // final norm + vocabulary projection: the stream of the last layer is polled for like any other
     pf.stamp();
-    stage_norm_tagged<2>(xs, a.tg + (size_t)(m.n_layers - 1) * a.tg_stride + a.tg_n, pc, m.eps, d, pre.g);
+    stage_norm_tagged<2>(xs, tgs + (size_t)(m.n_layers - 1) * a.tg_stride + a.tg_n, pc, m.eps, d, pre.g);
     __syncthreads();
     pf.stamp();
     pf.stamp();
@@ -401,6 +424,21 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     }
   }
   pf.stamp();
+  if constexpr (ONE) {
+    // bookkeeping by the last workgroup out (the batch-1 layers have no barrier that everyone has passed, and without the
+    // selection there is none at all): nobody reads these again in this launch
+    if (threadIdx.x == 0) {
+      const unsigned int out = __hip_atomic_fetch_add(a.bar + (gs.ng + 13) * 64, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (out + 1u == nth * gs.nwg) {
+        *launches = nth;
+        *gs.done = gs.k - 1;
+        if (a.select) {
+          a.step_state[0] = pos + 1;
+          a.step_state[1] = step + 1;
+        }
+      }
+    }
+  } else {
   // bookkeeping by workgroup 0: everyone is past the last barrier, nobody reads these again
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     *gs.done = gs.k - 1;
@@ -409,16 +447,19 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
       a.step_state[1] = step + 1;
     }
   }
+  }
 }
 
 // ---- workspace layout ------------------------------------------------------------------
-#define OHARA_BAR_WORDS(nwg) ((((nwg) + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP + 12) * 64)
+// (two words behind GridSync's: the launches since the workspace was cleared - the tag of the batch-1 hand-offs - and the
+// workgroups that have finished, which tells the last one out that it is the one to advance the launch count)
+#define OHARA_BAR_WORDS(nwg) ((((nwg) + OHARA_BAR_GROUP - 1) / OHARA_BAR_GROUP + 14) * 64)
 
 size_t mega_al(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct MegaLayout {
   size_t layers, kptr, vptr, xm, qm, am, pm, dm, candv, candi, prof, bar, tg, total;
-  size_t xm_stride, qm_stride, am_stride, pm_stride, dm_stride, tg_stride;
+  size_t xm_stride, qm_stride, am_stride, pm_stride, dm_stride, tg_stride, tg_set;
   int blk_x, blk_a, tg_n, tg_q, tg_kv, tg_a;
 };
 
@@ -439,20 +480,22 @@ MegaLayout mega_layout(const OharaModel* m, int B, int nwg) {
   L.xm = o; o += L.xm_stride * NL;
   L.qm = o; o += L.qm_stride * NL;
   L.am = o; o += L.am_stride * NL;
-  L.pm = o; o += L.pm_stride * sizeof(float) * NL;
   L.dm_stride = mega_al((size_t)OHARA_DOWN_SPLIT * ((m->d_model + 15) / 16) * ((B * 64 + 127) / 128 * 128)) / sizeof(float);
   L.dm = o; o += L.dm_stride * sizeof(float) * NL;
   L.candv = o; o += mega_al((size_t)nwg * B * sizeof(float));
   L.candi = o; o += mega_al((size_t)nwg * B * sizeof(int));
   L.prof = o; o += mega_al((size_t)nwg * OHARA_PROF_SLOTS * sizeof(unsigned long long));
   L.bar = o; o += mega_al(OHARA_BAR_WORDS(nwg) * sizeof(unsigned int));
-  // tagged mailboxes (batch 1; 8 bytes per two values), behind the barrier words: cleared with them
-  L.tg_n = (int)mega_al((size_t)m->d_model * 4);
+  // behind the barrier words, cleared with them: the attention partials (batch 1: a tag follows each (max, sum) pair);
+  // then the two sets of polled mailboxes (batch 1), filled with 0xFF ("not written yet")
+  L.pm = o; o += L.pm_stride * sizeof(float) * NL;
+  L.tg_n = (int)mega_al((size_t)m->d_model * 2);
   L.tg_q = 2 * L.tg_n;
-  L.tg_kv = L.tg_q + (int)mega_al((size_t)m->n_heads * D * 4);
-  L.tg_a = L.tg_kv + (int)mega_al((size_t)2 * m->n_kv_heads * D * 4);
-  L.tg_stride = L.tg_a + mega_al((size_t)((m->d_ff + 7) / 8 * 8) * 4);
-  L.tg = o; o += L.tg_stride * NL;
+  L.tg_kv = L.tg_q + (int)mega_al((size_t)m->n_heads * D * 2);
+  L.tg_a = L.tg_kv + (int)mega_al((size_t)2 * m->n_kv_heads * D * 2);
+  L.tg_stride = L.tg_a + mega_al((size_t)((m->d_ff + 7) / 8 * 8) * 2);
+  L.tg_set = L.tg_stride * NL;
+  L.tg = o; o += 2 * L.tg_set;
   L.total = o;
   return L;
 }
@@ -506,7 +549,7 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   a.cand_val = reinterpret_cast<float*>(ws + L.candv);
   a.cand_idx = reinterpret_cast<int*>(ws + L.candi);
   a.bar = reinterpret_cast<unsigned int*>(ws + L.bar);
-  a.tg = ws + L.tg; a.tg_stride = L.tg_stride; a.tg_n = L.tg_n; a.tg_q = L.tg_q; a.tg_kv = L.tg_kv; a.tg_a = L.tg_a;
+  a.tg = ws + L.tg; a.tg_stride = L.tg_stride; a.tg_set = L.tg_set; a.tg_n = L.tg_n; a.tg_q = L.tg_q; a.tg_kv = L.tg_kv; a.tg_a = L.tg_a;
   if (init_workspace) {
     // small synchronous copies: done once per (model, cache) binding, outside any capture
     if (hipMemcpyAsync((void*)a.layers_dev, m->layers, sizeof(OharaLayer) * m->n_layers, hipMemcpyHostToDevice, st) !=
@@ -515,7 +558,8 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
             hipSuccess ||
         hipMemcpyAsync((void*)a.vcache_dev, s->vcache, sizeof(void*) * m->n_layers, hipMemcpyHostToDevice, st) !=
             hipSuccess ||
-        hipMemsetAsync((void*)a.bar, 0, L.total - L.bar, st) != hipSuccess || hipStreamSynchronize(st) != hipSuccess)
+        hipMemsetAsync((void*)a.bar, 0, L.tg - L.bar, st) != hipSuccess ||
+        hipMemsetAsync((void*)a.tg, 0xFF, L.total - L.tg, st) != hipSuccess || hipStreamSynchronize(st) != hipSuccess)
       return OHARA_ELAUNCH;
     return OHARA_OK;
   }

@@ -174,19 +174,25 @@ __device__ __forceinline__ float dot8m(uint4 a, uint4 b, float s) {
 }
 
 // ---------------------------------------------------------------------------------------
-// Tagged mailboxes: hand-offs of a single row (batch 1) WITHOUT a grid barrier.  An entry is 8 bytes,
-// {two bf16 values, tag}, written with one device-scope store, so whoever sees the tag of this launch
-// sees the values that came with it.  The tag is the launch's first barrier index (GridSync::k at
-// start): it grows with every launch, the mailboxes are cleared together with the barrier words, and
-// each entry is written once per launch - an entry of this launch cannot be mistaken for an older one.
-// Consumers poll the entries they need with device-scope loads (0.13 us a round, the producer's store
-// shows up ~0.6 us after it was issued) instead of waiting for a barrier (~1.6 us), for the producers'
-// own wait for their stores before it, and then fetching the data cold; every poll loop is bounded like
-// the barrier's spins.  Only worth it where a consumer needs little (the 768 values of a row, the 128
-// of a head): polled by 200 workgroups, tens of KB per consumer would swamp the memory fabric.
+// Polled mailboxes: hand-offs of a single row (batch 1) WITHOUT a grid barrier.  A mailbox is the plain
+// bf16 row, two values to a 32-bit word, and a word that has not been written yet holds 0xFFFFFFFF - two
+// NaNs of a payload that arithmetic does not produce (the producer turns a pair that happens to look
+// like it into two other NaNs).  There are two sets of mailboxes: launch n writes and reads set n & 1,
+// and whoever stores a word there resets the same word of the other set, which every consumer finished
+// with a launch ago and which the next launch finds unwritten again; the entry point fills both sets
+// with 0xFF when it clears the workspace.  Each word is written once per launch with a device-scope
+// store and consumers poll the words they need with 16-byte device-scope loads, all of them every
+// round: what a hand-off costs is the round trips to memory and the number of load instructions per
+// round (a 1 KB row polled by one instruction per lane is seen ~0.7 us after its stores were issued, a
+// 4 KB row polled by four ~1.7 us; one round that only watched a flag first would add a trip), not
+// the number of pollers.  That is against ~1.6 us for a grid barrier plus the producers' wait for
+// their stores before it plus fetching the data cold.  Every poll loop is bounded like the barrier's
+// spins.  Only worth it where a consumer needs little (a row, a head's 128 values).
+// The attention partials (fp32, 48 KB per consumer) go another way: see stage_attn_merge.
 // ---------------------------------------------------------------------------------------
+#define OHARA_UNWRITTEN 0xFFFFFFFFu
 struct Poll {
-  uint32_t tag;
+  uint32_t tag;   // the number of this launch since the workspace was cleared
   unsigned int limit;
   unsigned int* err;
 };
@@ -197,25 +203,29 @@ __device__ __forceinline__ bool poll_expired(const Poll& pc, unsigned int& spins
   }
   return (spins & 63u) == 0 && __hip_atomic_load(pc.err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
 }
-// four values starting at column `col` (a multiple of 4): two entries
-__device__ __forceinline__ void st_tag4(char* base, int col, uint32_t lo, uint32_t hi, uint32_t tag) {
-  char* q = base + (size_t)(col >> 1) * 8;
-  st_coh8(q, make_uint2(lo, tag));
-  st_coh8(q + 8, make_uint2(hi, tag));
+__device__ __forceinline__ uint32_t mb_word(uint32_t v) { return v == OHARA_UNWRITTEN ? 0xFFFEFFFFu : v; }
+// four values starting at column `col` (a multiple of 4); `other`: from this set's mailbox to the other set's
+__device__ __forceinline__ void mb_st8(char* base, ptrdiff_t other, int col, uint32_t lo, uint32_t hi) {
+  char* q = base + (size_t)col * 2;
+  st_coh8(q, make_uint2(mb_word(lo), mb_word(hi)));
+  st_coh8(q + other, make_uint2(OHARA_UNWRITTEN, OHARA_UNWRITTEN));
 }
-// eight values starting at column `col` (a multiple of 8): four entries; true when all carry `tag`
-__device__ __forceinline__ bool ld_tag8(const char* base, int col, uint32_t tag, uint4& out) {
-  const char* q = base + (size_t)(col >> 1) * 8;
-  const uint4 a = ld_coh16(q), b = ld_coh16(q + 16);
-  out = make_uint4(a.x, a.z, b.x, b.z);
-  return a.y == tag && a.w == tag && b.y == tag && b.w == tag;
+// two values starting at column `col` (a multiple of 2)
+__device__ __forceinline__ void mb_st4(char* base, ptrdiff_t other, int col, uint32_t v) {
+  char* q = base + (size_t)col * 2;
+  st_coh4(q, mb_word(v));
+  st_coh4(q + other, OHARA_UNWRITTEN);
 }
-
-// One entry's tag (entry index `e`): the cheap poll.  The entries of a 16-value strip leave the producer
-// in two store instructions of one wave, so its last entry (index 8 s + 7) is the last to appear; a
-// consumer polls one such entry per strip it needs, then loads everything and checks every tag.
-__device__ __forceinline__ bool tag_seen(const char* base, int e, uint32_t tag) {
-  return ld_coh8(base + (size_t)e * 8).y == tag;
+// The load side: a buffer descriptor over the mailbox (the 16-byte device-scope load is a buffer load with sc1).
+typedef __amdgpu_buffer_rsrc_t MbRsrc;
+__device__ __forceinline__ MbRsrc mb_rsrc(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7FFFFFFF, 0x00020000);
+}
+// eight values starting at column `col` (a multiple of 8); true when all of them have been written
+__device__ __forceinline__ bool mb_ld16(MbRsrc r, int col, uint4& out) {
+  const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (uint32_t)col * 2u, 0, 16);
+  out = make_uint4(v.x, v.y, v.z, v.w);
+  return v.x != OHARA_UNWRITTEN && v.y != OHARA_UNWRITTEN && v.z != OHARA_UNWRITTEN && v.w != OHARA_UNWRITTEN;
 }
 
 // Strip-blocked mailbox of a (B, N) bf16 matrix: the 16 columns [16s, 16s+16) of all rows
@@ -386,7 +396,7 @@ __device__ __forceinline__ void stage_act(bf16_t* xs, int ldxs, const char* src,
   }
 }
 
-// The row of a tagged mailbox (batch 1) -> norm.py:16-21 -> LDS, by wave 0: stage_norm on a row that is
+// The row of a polled mailbox (batch 1) -> norm.py:16-21 -> LDS, by wave 0: stage_norm on a row that is
 // polled for instead of fetched after a barrier.  The norm weights were fetched ahead (gpre).
 template <int NLD>
 __device__ __forceinline__ void stage_norm_tagged(bf16_t* xs, const char* xt, const Poll& pc, float eps, int K,
@@ -395,16 +405,14 @@ __device__ __forceinline__ void stage_norm_tagged(bf16_t* xs, const char* xt, co
   if (tid >= 64) return;
   uint4 v[NLD];
   unsigned int spins = 0;
-  const int nstr = (K + 15) >> 4;  // producer strips (<= 64 for K <= 1024); lane s watches strip s
+  const MbRsrc rs = mb_rsrc(xt);
+  // every round fetches the whole row (1.5 KB at K = 768) and looks at every word
   for (;;) {
-    while (!__all(lane >= nstr || tag_seen(xt, lane * 8 + (min(K, lane * 16 + 16) - lane * 16 - 1) / 2, pc.tag))) {
-      if (poll_expired(pc, spins)) break;
-    }
     bool ok = true;
 #pragma unroll
     for (int c = 0; c < NLD; ++c) {
       const int k = (c * 64 + lane) * 8;
-      ok = ld_tag8(xt, k < K ? k : 0, pc.tag, v[c]) && ok;
+      ok = mb_ld16(rs, k < K ? k : 0, v[c]) && ok;
     }
     if (__all(ok) || poll_expired(pc, spins)) break;
   }
@@ -436,19 +444,16 @@ __device__ __forceinline__ void stage_norm_tagged(bf16_t* xs, const char* xt, co
   }
 }
 
-// Columns [f0, f1) (multiples of 8) of the tagged act mailbox (batch 1) -> LDS
+// Columns [f0, f1) (multiples of 8) of the polled act mailbox (batch 1) -> LDS
 __device__ __forceinline__ void stage_act_tagged(bf16_t* xs, const char* at, const Poll& pc, int f0, int f1) {
   const int n8 = (f1 - f0) >> 3;
+  const MbRsrc rs = mb_rsrc(at);
   for (int i = threadIdx.x; i < n8; i += blockDim.x) {
     const int c = (f0 >> 3) + i;
-    // the eight values of a thread are one producer strip's, stored by one instruction: poll its last entry
     uint4 v;
     unsigned int spins = 0;
-    for (;;) {
-      while (!tag_seen(at, c * 4 + 3, pc.tag)) {
-        if (poll_expired(pc, spins)) break;
-      }
-      if (ld_tag8(at, c * 8, pc.tag, v) || poll_expired(pc, spins)) break;
+    while (!mb_ld16(rs, c * 8, v)) {
+      if (poll_expired(pc, spins)) break;
     }
     sts16(xs + c * 8, v);
   }
@@ -461,9 +466,13 @@ __device__ __forceinline__ void stage_act_tagged(bf16_t* xs, const char* at, con
 // columns per pass and issues the accumulator loads of 16 / NS passes - 16 loads - before it uses
 // any, so the number of dependent load rounds does not grow with the chunk count times the batch.
 // `mw`: B*H*NS floats, `ml`: B*H floats of LDS.
-template <int NS>  // NS: a power of two; `used` <= NS chunks hold partials (the others weigh nothing)
+// TAGGED (batch-1 kernels without a barrier ahead of the merge): a chunk's maximum and sum are stored as
+// {max, tag, sum, tag} - each value in one 8-byte word with the tag of the launch - once the chunk's accumulators
+// have reached memory; they are polled for, one lane per chunk, and the accumulators are fetched only after
+// every chunk of the workgroup has been seen.
+template <int NS, bool TAGGED = false>  // NS: a power of two; `used` <= NS chunks hold partials (the others weigh nothing)
 __device__ __forceinline__ void stage_attn_merge(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh, float* mw_, float* ml_,
-                                                 int used = NS) {
+                                                 int used = NS, const Poll pc = Poll{0, 0, nullptr}) {
   constexpr int NSM = OHARA_MEGA_NS, PR = 16 / NS;
   const int HD = H * Dh, PS = Dh + 32;
   const int nbh = B * H, total = B * HD;
@@ -484,7 +493,7 @@ __device__ __forceinline__ void stage_attn_merge(bf16_t* xs, int ldxs, const flo
   };
   // the accumulator loads of the first round go out first: they do not depend on the chunk
   // weights, which are formed while they are in flight
-  load((int)threadIdx.x * 4);
+  if (!TAGGED) load((int)threadIdx.x * 4);
   // NS lanes per (sequence, head): lane sp holds chunk sp's (max, sum); max and weighted sum by
   // shuffles inside the group
   for (int i0 = 0; i0 < nbh * NS; i0 += blockDim.x) {
@@ -493,9 +502,18 @@ __device__ __forceinline__ void stage_attn_merge(bf16_t* xs, int ldxs, const flo
     const bool in = bh < nbh && sp < used;
     float ms = -INFINITY, ls = 0.f;
     if (in) {
-      const uint2 v = ldg8(pm + ((size_t)bh * NSM + sp) * PS + Dh);
-      ms = __uint_as_float(v.x);
-      ls = __uint_as_float(v.y);
+      if (TAGGED) {
+        uint4 v;
+        unsigned int spins = 0;
+        do v = ld_coh16(pm + ((size_t)bh * NSM + sp) * PS + Dh);  // {max, tag}, {sum, tag}: two 8-byte loads
+        while ((v.y != pc.tag || v.w != pc.tag) && !poll_expired(pc, spins));
+        ms = __uint_as_float(v.x);
+        ls = __uint_as_float(v.z);
+      } else {
+        const uint2 v = ldg8(pm + ((size_t)bh * NSM + sp) * PS + Dh);
+        ms = __uint_as_float(v.x);
+        ls = __uint_as_float(v.y);
+      }
     }
     float M = ms;
     if (NS > 8) M = lane_xor_max<8>(M);
@@ -512,8 +530,9 @@ __device__ __forceinline__ void stage_attn_merge(bf16_t* xs, int ldxs, const flo
     if (in && sp == 0) ml[bh] = Ls;
   }
   __syncthreads();
+  asm volatile("" ::: "memory");  // compiler only (TAGGED): the accumulator loads stay behind the polls
   for (int e0 = threadIdx.x * 4; e0 < total; e0 += pass * PR) {
-    if (e0 != (int)threadIdx.x * 4) load(e0);
+    if (TAGGED || e0 != (int)threadIdx.x * 4) load(e0);
 #pragma unroll
     for (int r = 0; r < PR; ++r) {
       const int e = e0 + r * pass;
@@ -573,10 +592,10 @@ __device__ __forceinline__ void stage_attn_merge_small(bf16_t* xs, int ldxs, con
 }
 
 // Out-of-line copies of the merge, for kernels that want to keep their own code compact.
-template <int NS>
+template <int NS, bool TAGGED = false>
 __device__ __noinline__ void stage_attn_merge_call(bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh, float* mw,
-                                                   float* ml, int used) {
-  stage_attn_merge<NS>(xs, ldxs, pm, B, H, Dh, mw, ml, used);
+                                                   float* ml, int used, uint32_t tag = 0, unsigned int limit = 0, unsigned int* err = nullptr) {
+  stage_attn_merge<NS, TAGGED>(xs, ldxs, pm, B, H, Dh, mw, ml, used, Poll{tag, limit, err});  // (a struct would travel through memory)
 }
 
 // The power of two that the merge of `ns` chunks is specialised for (the chunk weights in LDS are laid
@@ -592,24 +611,27 @@ __host__ __device__ inline int attn_merge_width(int ns) {
 // caller (no call in the layer loop: a call makes the caller wait for every load it has in flight, the
 // weights fetched ahead included); otherwise they stay outside it, which keeps a kernel whose usual case
 // is the small merge within the instruction cache.
-template <bool INLINE>
+template <bool INLINE, bool TAGGED = false>
 __device__ __forceinline__ void stage_attn_merge_any(int ns, bf16_t* xs, int ldxs, const float* pm, int B, int H, int Dh,
-                                                     float* mw, float* ml) {
+                                                     float* mw, float* ml, const Poll pc = Poll{0, 0, nullptr}) {
   const int w = attn_merge_width(ns);
-  if (ns == OHARA_MEGA_NS && B * H * Dh <= 4 * 256) {
+  if (!TAGGED && ns == OHARA_MEGA_NS && B * H * Dh <= 4 * 256) {  // (TAGGED: one lane polls one chunk's pair)
     stage_attn_merge_small(xs, ldxs, pm, B, H, Dh);
+  } else if (TAGGED && w == 16) {
+    // the usual width at batch 1, inline: a call would park the caller's prefetched weights in scratch memory
+    stage_attn_merge<16, TAGGED>(xs, ldxs, pm, B, H, Dh, mw, ml, ns, pc);
   } else if (INLINE) {
-    if (w == 16) stage_attn_merge<16>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
-    else if (w == 8) stage_attn_merge<8>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
-    else if (w == 4) stage_attn_merge<4>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
-    else if (w == 2) stage_attn_merge<2>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
-    else stage_attn_merge<1>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
+    if (w == 16) stage_attn_merge<16, TAGGED>(xs, ldxs, pm, B, H, Dh, mw, ml, ns, pc);
+    else if (w == 8) stage_attn_merge<8, TAGGED>(xs, ldxs, pm, B, H, Dh, mw, ml, ns, pc);
+    else if (w == 4) stage_attn_merge<4, TAGGED>(xs, ldxs, pm, B, H, Dh, mw, ml, ns, pc);
+    else if (w == 2) stage_attn_merge<2, TAGGED>(xs, ldxs, pm, B, H, Dh, mw, ml, ns, pc);
+    else stage_attn_merge<1, TAGGED>(xs, ldxs, pm, B, H, Dh, mw, ml, ns, pc);
   } else {
-    if (w == 16) stage_attn_merge_call<16>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
-    else if (w == 8) stage_attn_merge_call<8>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
-    else if (w == 4) stage_attn_merge_call<4>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
-    else if (w == 2) stage_attn_merge_call<2>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
-    else stage_attn_merge_call<1>(xs, ldxs, pm, B, H, Dh, mw, ml, ns);
+    if (w == 16) stage_attn_merge_call<16, TAGGED>(xs, ldxs, pm, B, H, Dh, mw, ml, ns, pc.tag, pc.limit, pc.err);
+    else if (w == 8) stage_attn_merge_call<8, TAGGED>(xs, ldxs, pm, B, H, Dh, mw, ml, ns, pc.tag, pc.limit, pc.err);
+    else if (w == 4) stage_attn_merge_call<4, TAGGED>(xs, ldxs, pm, B, H, Dh, mw, ml, ns, pc.tag, pc.limit, pc.err);
+    else if (w == 2) stage_attn_merge_call<2, TAGGED>(xs, ldxs, pm, B, H, Dh, mw, ml, ns, pc.tag, pc.limit, pc.err);
+    else stage_attn_merge_call<1, TAGGED>(xs, ldxs, pm, B, H, Dh, mw, ml, ns, pc.tag, pc.limit, pc.err);
   }
 }
 
@@ -647,8 +669,8 @@ struct GemmP {
   char* tkv;       // E_ROPE: the new key row, then the new value row (besides the cache)
   const char* tresid;  // E_RESID (unless resid_embed), E_XNEXT: the tagged row that is added to the product
   uint32_t wlds_addr;  // E_XNEXT: LDS byte address of the workgroup's parked tiles, OHARA_LDS_PF per wave (gemm_prefetch_lds)
-  const Poll* poll;
-  uint32_t tag;
+  Poll poll;
+  ptrdiff_t tother;  // from a mailbox of this launch's set to the same mailbox of the other set
   int wg0;         // the workgroup that takes the phase's first unit (units go to wg0, wg0 + 1, ... round the grid)
 };
 // A workgroup's position in a phase whose units start at workgroup p.wg0.
@@ -688,8 +710,11 @@ __device__ __forceinline__ bool gemm_unit(const GemmP& p, int unit, int kpart, i
 }
 
 // PO: first slot of pre.w this phase's tiles go to (several phases' weights can be held at once)
-template <int KP, int PF, int EPI, int PO = 0>
-__device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int B) {
+// (g, r: where the norm weights and the rotary pair / embedding residual go - pre.g and pre.r unless the caller keeps
+// those of several phases at once)
+// PAIR = false: E_ROPE without the rotary pair (it is the same for every layer: a caller that keeps it fetches it once)
+template <int KP, int PF, int EPI, int PO = 0, bool PAIR = true>
+__device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int B, uint4 (&g_out)[2], uint2& r_out) {
   static_assert(PO + PF <= OHARA_MAX_PF, "prefetch buffer");
   constexpr int SPW = 4 / KP;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -703,24 +728,24 @@ __device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int 
 #pragma unroll
     for (int c = 0; c < 2; ++c) {
       const int k = (c * 64 + lane) * 8;
-      pre.g[c] = (p.norm_w && wave < B && k < p.K) ? ldg16(p.norm_w + k) : make_uint4(0, 0, 0, 0);
+      g_out[c] = (p.norm_w && wave < B && k < p.K) ? ldg16(p.norm_w + k) : make_uint4(0, 0, 0, 0);
     }
   }
-  if (EPI == E_ROPE) {
+  if (EPI == E_ROPE && PAIR) {
     const int m = lane & 15, g = lane >> 4;
     const int r0 = strip * 16 + 4 * g;
     const int nq = p.H * p.Dh, nk = p.Hkv * p.Dh;
-    pre.r = make_uint2(0, 0);
+    r_out = make_uint2(0, 0);
     if (live && kpart == 0 && m < B && r0 < nq + nk && p.pos >= 0 && p.pos < p.Tmax) {
       const int d = (r0 < nq ? r0 : r0 - nq) % p.Dh;
-      pre.r = make_uint2(ldg4(p.cos + (size_t)p.pos * (p.Dh >> 1) + (d >> 1)),
+      r_out = make_uint2(ldg4(p.cos + (size_t)p.pos * (p.Dh >> 1) + (d >> 1)),
                          ldg4(p.sin + (size_t)p.pos * (p.Dh >> 1) + (d >> 1)));
     }
   }
   if (EPI == E_RESID) {
     const int m = lane & 15, g = lane >> 4;
     const int r0 = strip * 16 + 4 * g;
-    pre.r = make_uint2(0, 0);
+    r_out = make_uint2(0, 0);
     if (live && kpart == 0 && m < B && r0 < p.N && !p.tout) {  // (tagged mode: the residual is fetched by the phase itself)
       if (!p.resid_embed) {
         static_assert(EPI != E_RESID || PF <= OHARA_PRE_RESID, "the residual's pieces share the weight buffer");
@@ -732,16 +757,31 @@ __device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int 
       } else {
         int64_t id = ldg_i64(p.ids + m);
         if (id < 0 || id >= p.vocab) id = 0;
-        pre.r = ldg8(p.table + (size_t)id * p.N + r0);
+        r_out = ldg8(p.table + (size_t)id * p.N + r0);
       }
     }
   }
   // the weights last: the small loads above are then issued with nothing of this prefetch in flight
   // (placed behind the weight loads, the compiler made each of them wait for all of those first)
-  const uint4* wrow = p.wp + (size_t)strip * KS * 64 + lane;
+  // One running address, no test per tile: a tile past the wave's last k-step is that last tile again (finite
+  // values that meet activations of zero), and a wave without a unit fetches nothing and never looks at its
+  // slots.  (With an address and a branch per tile the compiler kept all of them - they do not change from
+  // layer to layer - in scratch memory and waited for every earlier load before each reload.)
+  if (live && j0 < j1) {
+    const uint4* ptr = p.wp + ((size_t)strip * KS + j0) * 64 + lane;
+    asm volatile("" : "+v"(ptr));  // formed here, not ahead of a loop around the caller (and kept until here)
+    const int left = j1 - j0 - 1;
 #pragma unroll
-  for (int c = 0; c < PF; ++c)
-    pre.w[PO + c] = (live && j0 + c < j1) ? ldg16_nt(wrow + (size_t)(j0 + c) * 64) : make_uint4(0, 0, 0, 0);
+    for (int c = 0; c < PF; ++c) {
+      pre.w[PO + c] = ldg16_nt(ptr);
+      ptr += c < left ? 64 : 0;
+    }
+  }
+}
+
+template <int KP, int PF, int EPI, int PO = 0>
+__device__ __forceinline__ void gemm_prefetch(const GemmP& p, GemmPre& pre, int B) {
+  gemm_prefetch<KP, PF, EPI, PO>(p, pre, B, pre.g, pre.r);
 }
 
 // The weights of a workgroup's first unit straight into LDS (global_load_lds: 16 bytes per lane, a wave's
@@ -793,8 +833,8 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
     // while), requested ahead of the products and checked in the epilogue
     const bool tres = TAG && (EPI == E_XNEXT || (EPI == E_RESID && !p.resid_embed)) && live && kpart == 0 && mine &&
                       strip * 16 + 4 * g < p.N;
-    uint4 rx = make_uint4(0, 0, 0, 0);
-    if (tres) rx = ld_coh16(p.tresid + (size_t)((strip * 16 + 4 * g) >> 1) * 8);
+    uint2 rx = make_uint2(0, 0);
+    if (tres) rx = ld_coh8(p.tresid + (size_t)(strip * 16 + 4 * g) * 2);
     if (live) {
       const uint4* wrow = p.wp + (size_t)strip * KS * 64 + lane;
 #pragma unroll 1
@@ -884,17 +924,17 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
           uint2 r = make_uint2(0, 0);
           if (tres) {
             unsigned int spins = 0;
-            while (!(rx.y == p.tag && rx.w == p.tag)) {
-              if (poll_expired(*p.poll, spins)) break;
-              rx = ld_coh16(p.tresid + (size_t)(r0 >> 1) * 8);
+            while (rx.x == OHARA_UNWRITTEN || rx.y == OHARA_UNWRITTEN) {
+              if (poll_expired(p.poll, spins)) break;
+              rx = ld_coh8(p.tresid + (size_t)r0 * 2);
             }
-            r = make_uint2(rx.x, rx.z);
+            r = rx;
           } else {  // the first half layer: the embedding row (llama.py:310)
             int64_t id = ldg_i64(p.ids + b);
             if (id < 0 || id >= p.vocab) id = 0;
             r = ldg8(p.table + (size_t)id * p.N + r0);
           }
-          st_tag4(p.tout, r0, pack_bf(lo_bf(r.x) + y0, hi_bf(r.x) + y1), pack_bf(lo_bf(r.y) + y2, hi_bf(r.y) + y3), p.tag);
+          mb_st8(p.tout, p.tother, r0, pack_bf(lo_bf(r.x) + y0, hi_bf(r.x) + y1), pack_bf(lo_bf(r.y) + y2, hi_bf(r.y) + y3));
         }
       } else if (EPI == E_RESID) {  // N % 4 == 0 is required by the entry point
         if (r0 < p.N) {
@@ -950,7 +990,7 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
         const int f = strip * 8 + 2 * g;
         if (f < p.N) {
           const float s0 = rbf(silu_f(y0)), s1 = rbf(silu_f(y1));
-          if (TAG) st_coh8(p.tout + (size_t)(f >> 1) * 8, make_uint2(pack_bf(s0 * y2, s1 * y3), p.tag));
+          if (TAG) mb_st4(p.tout, p.tother, f, pack_bf(s0 * y2, s1 * y3));
           else st_coh4(const_cast<char*>(am_addr(p.out, p.blk, b, f)), pack_bf(s0 * y2, s1 * y3));
         }
       } else {  // E_ROPE
@@ -976,8 +1016,8 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
           }
           const uint2 ro = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
           if (TAG) {  // attention polls for the q row and for the new key / value rows; the cache rows are for later steps
-            if (r0 < nq) st_tag4(p.tout, r0, ro.x, ro.y, p.tag);
-            else st_tag4(p.tkv, r0 - nq, ro.x, ro.y, p.tag);
+            if (r0 < nq) mb_st8(p.tout, p.tother, r0, ro.x, ro.y);
+            else mb_st8(p.tkv, p.tother, r0 - nq, ro.x, ro.y);
           }
           if (!TAG || r0 >= nq) st_coh8(o, ro);
         }
@@ -1191,16 +1231,17 @@ __device__ __forceinline__ void attn_new_row_tagged(const char* kvt, const Poll&
   const int pos = min(tb + p, t1 - 1);
   const int nk = Hkv * D;
   unsigned int spins = 0;
+  const MbRsrc rs = mb_rsrc(kvt);
   for (;;) {
     bool ok = true;
     if (pos == pos_new) {
 #pragma unroll
-      for (int c = 0; c < NC; ++c) ok = ld_tag8(kvt, kvh * D + (4 * c + dq) * 8, pc.tag, kv[c]) && ok;
+      for (int c = 0; c < NC; ++c) ok = mb_ld16(rs, kvh * D + (4 * c + dq) * 8, kv[c]) && ok;
     }
 #pragma unroll
     for (int c = 0; c < NV; ++c) {
       const int vp = min(tb + c * PP + pp, t1 - 1);
-      if (vp == pos_new) ok = ld_tag8(kvt, nk + kvh * D + dc * 8, pc.tag, vv[c]) && ok;
+      if (vp == pos_new) ok = mb_ld16(rs, nk + kvh * D + dc * 8, vv[c]) && ok;
     }
     if (__all(ok) || poll_expired(pc, spins)) break;
   }
@@ -1212,7 +1253,7 @@ template <int D, int G, bool TAG = false>
 __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int blk_x, int ns, const AttnPre<D>& pre,
                                            const char* qm, float* pm, const bf16_t* kc, const bf16_t* vc, int L,
                                            float* lds, const char* qt = nullptr, const char* kvt = nullptr,
-                                           const Poll* pc = nullptr) {
+                                           const Poll pc = Poll{0, 0, nullptr}, bool announce = false) {
   constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int p = lane & 15;
@@ -1257,20 +1298,17 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
       }
       if (TAG) {
         unsigned int spins = 0;
-        constexpr int NSTR = G * D / 16;  // the strips that produce this group's q rows (<= 32); lane s watches strip s
-        for (;;) {
-          while (!__all(lane >= NSTR || tag_seen(qt, (kvh * G * D) / 2 + lane * 8 + 7, pc->tag))) {
-            if (poll_expired(*pc, spins)) break;
-          }
+        const MbRsrc qrs = mb_rsrc(qt);
+        for (;;) {  // (every round fetches the group's q rows whole: lanes share addresses, 256 bytes a row)
           bool ok = true;
 #pragma unroll
           for (int hh = 0; hh < G; ++hh)
 #pragma unroll
             for (int c = 0; c < NC; ++c)
-              ok = ld_tag8(qt, (kvh * G + hh) * D + (4 * c + dq) * 8, pc->tag, qv[hh][c]) && ok;
-          if (__all(ok) || poll_expired(*pc, spins)) break;
+              ok = mb_ld16(qrs, (kvh * G + hh) * D + (4 * c + dq) * 8, qv[hh][c]) && ok;
+          if (__all(ok) || poll_expired(pc, spins)) break;
         }
-        if (!use_pre && L - 1 >= tb && L - 1 < tb + 16) attn_new_row_tagged<D>(kvt, *pc, Hkv, kvh, tb, t1, L - 1, ka, va);
+        if (!use_pre && L - 1 >= tb && L - 1 < tb + 16) attn_new_row_tagged<D>(kvt, pc, Hkv, kvh, tb, t1, L - 1, ka, va);
       } else {
 #pragma unroll
         for (int hh = 0; hh < G; ++hh)
@@ -1352,7 +1390,7 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
       // and is copied over, which costs a wait but far fewer registers than two sets taking turns)
       for (; tb + 64 < t1; tb += 64) {
         attn_tile_load_u<D>(kb, vb, row, tb + 64, t1, coh, kn, vn, last);
-        if (TAG && L - 1 >= tb + 64 && L - 1 < tb + 80) attn_new_row_tagged<D>(kvt, *pc, Hkv, kvh, tb + 64, t1, L - 1, kn, vn);
+        if (TAG && L - 1 >= tb + 64 && L - 1 < tb + 80) attn_new_row_tagged<D>(kvt, pc, Hkv, kvh, tb + 64, t1, L - 1, kn, vn);
         consume(tb, ka, va);
 #pragma unroll
         for (int c = 0; c < NC; ++c) ka[c] = kn[c];
@@ -1384,6 +1422,8 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
       }
     }
     __syncthreads();
+    float* ann = nullptr;  // the thread that holds a head's maximum and sum: where they go
+    float ann_m = 0.f, ann_l = 0.f;
     for (int idx = tid * 2; idx < G * D; idx += 512) {
       const int hh = idx / D, d = idx - hh * D;
       const int h = kvh * G + hh;
@@ -1399,9 +1439,24 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
       }
       float* dst = pm + ((size_t)(b * H + h) * OHARA_MEGA_NS + split) * PS;
       st_coh8(dst + d, make_uint2(__float_as_uint(o0), __float_as_uint(o1)));
-      if (d == 0) st_coh8(dst + D, make_uint2(__float_as_uint(M), __float_as_uint(Ls)));
+      if (d == 0) {
+        if (TAG && announce) {
+          ann = dst + D;
+          ann_m = M;
+          ann_l = Ls;
+        } else {
+          st_coh8(dst + D, make_uint2(__float_as_uint(M), __float_as_uint(Ls)));
+        }
+      }
     }
+    // `announce`: the merge polls for the head's maximum and sum, which are stored - each in an 8-byte word of its own
+    // together with the launch's tag, {max, tag, sum, tag} - once the item's accumulators have reached memory
+    if (TAG && announce) wait_own_stores();
     __syncthreads();
+    if (TAG && announce && ann) {
+      st_coh8(ann, make_uint2(__float_as_uint(ann_m), pc.tag));
+      st_coh8(ann + 2, make_uint2(__float_as_uint(ann_l), pc.tag));
+    }
   }
 }
 
