@@ -29,10 +29,10 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the persistent decode kernel at batch 1, prompt 1024, from two
 # rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same
-# counter reads for a 1 GiB copy (--pmc-calibration): 381.4 MB read + 1.8 MB written.  Counters
+# counter reads for a 1 GiB copy (--pmc-calibration): 376.0 MB read + 1.3 MB written.  Counters
 # cannot be read from inside this process, so the figure is carried here; the runs and the
 # arithmetic are in profiles/decode_mega_kernel_d12_batch1_pmc.txt.
-PMC_TRAFFIC_BYTES = {("persistent", 1, 1024): 383.4e6}
+PMC_TRAFFIC_BYTES = {("persistent", 1, 1024): 377.3e6}
 
 D12 = dict(vocab_size=65536, hidden_size=768, intermediate_size=3072, num_attention_heads=6,
            num_key_value_heads=0, num_hidden_layers=12, max_sequence_length=4096, dropout=0.0)
@@ -556,34 +556,38 @@ def bench_phi(dev):
     return out
 
 
-# Shader-clock samples that workgroup 0 of the persistent kernel takes per layer, in order (see
-# csrc/mega.hip: Prof::stamp in the kernel body, GridSync::arrive / wait and gemm_phase).  Each entry
-# names the interval that ENDS at that sample.
-_BAR = ["wait for own stores (vmcnt 0)", "workgroup barrier", "arrival atomics issued", "(window)",
-        "spin on the release word + workgroup barrier", "(bookkeeping)"]
+# Shader-clock samples that thread 0 of every workgroup of the batch-1 persistent kernel takes per layer,
+# in order (csrc/mega.hip: the stamps in the layer loop, and two inside every gemm_phase).  The kernel has
+# no grid barrier inside the layers: a phase's units sit on their own stretch of workgroups and every
+# hand-off is polled for, so a step's critical path runs from role to role.
 _GEMM = ["activations in LDS -> MFMAs issued", "cross-wave sum"]
-# intervals between the clock samples of the batch-1 kernel (no grid barrier inside the layers: every
-# hand-off is a tagged mailbox, or a flag per attention chunk, that the consumer polls for)
 PHASE_STAMPS = (
-    [("P1 qkv", "poll for the stream + norm1 into LDS")] + [("P1 qkv", x) for x in _GEMM]
-    + [("P1 qkv", "rotary epilogue, tagged stores")]
-    + [("P2 attention", "poll for q, attention chunk, partials stored, flag raised")]
-    + [("P2 attention", "next q/k/v and down weights requested")]
-    + [("P3 wo", "poll for the chunks' tags, merge of attention partials into LDS")] + [("P3 wo", x) for x in _GEMM]
-    + [("P3 wo", "residual epilogue, tagged stores")]
-    + [("P4 gate/up", "poll for the stream + norm2 into LDS")] + [("P4 gate/up", x) for x in _GEMM]
-    + [("P4 gate/up", "SwiGLU epilogue, tagged stores")]
-    + [("P4 gate/up", "next layer's weights requested (all but the down projection's workgroups)")]
-    + [("P5 down", "poll for the activations into LDS")] + [("P5 down", x) for x in _GEMM]
-    + [("P5 down", "residual epilogue, tagged stores")]
-    + [("P5 down", "next layer's weights requested (the down projection's workgroups)")]
+    ["P1 staged"] + ["P1 " + x for x in _GEMM] + ["P1 epilogue", "P2 chunk announced", "P2 requests issued", "P3 merged"]
+    + ["P3 " + x for x in _GEMM] + ["P3 epilogue", "P4 staged"] + ["P4 " + x for x in _GEMM]
+    + ["P4 epilogue", "P4 requests issued", "P5 staged"] + ["P5 " + x for x in _GEMM] + ["P5 epilogue", "P5 requests issued"]
 )
-PHASE_TAIL = 13  # samples after the layers: three around the final norm, then as before
+PHASE_TAIL = 13  # samples after the layers: three around the final norm, vocabulary projection (2), its end, selection (6), the end
 
 
-def phase_timeline(dev, prompt_len, steps=32, workgroup=0):
-    """Per-phase timeline of the persistent decode kernel at batch 1: where workgroup 0 spends a
-    step, from the kernel's own shader-clock samples averaged over `steps` real decode steps."""
+def _batch1_roles(cfg, nwg):
+    """Which workgroups take which phase of the batch-1 kernel (mirrors the assignment in csrc/mega.hip)."""
+    d, F = cfg.hidden_size, cfg.intermediate_size
+    H = cfg.num_attention_heads
+    Hkv = cfg.num_key_value_heads or H
+    D = d // H
+    n_qkv, n_wo, n_dn = (H + 2 * Hkv) * D // 16, d // 16, d // 16
+    n_gu = (2 * ((F + 7) // 8 * 8) // 16 + 1) // 2
+    ns = max(1, min(16, nwg // Hkv))
+    dn0 = n_wo if n_wo + n_dn <= nwg else nwg - n_dn
+    return {"qkv": range(nwg - n_qkv, nwg), "attention": range(0, Hkv * ns), "wo": range(0, n_wo),
+            "gate/up": range(0, n_gu), "down": range(dn0, dn0 + n_dn)}
+
+
+def phase_timeline(dev, prompt_len, steps=32):
+    """The critical path of a layer of the batch-1 persistent kernel: for every hand-off, when the last
+    workgroup of the producing role had issued its stores and when the last workgroup of the consuming
+    role had the data staged, from the kernel's own clock samples (a 100 MHz counter common to all
+    workgroups), averaged over `steps` real decode steps and over the layers after the first."""
     from ohara_amd.llama import Llama
 
     cfg, st = d12_state(dev)
@@ -594,10 +598,8 @@ def phase_timeline(dev, prompt_len, steps=32, workgroup=0):
         sess.step()
     nl = cfg.num_hidden_layers
     per = len(PHASE_STAMPS)
-    n_stamps = 1 + per * nl
-    n_tail = PHASE_TAIL  # after the layers: final norm (3), LM head (2 samples), its end, the selection's arrive (4) / wait (2), the end
-    acc = torch.zeros(n_stamps + n_tail, dtype=torch.float64)
-    total_ms = 0.0
+    roles = _batch1_roles(cfg, sess._nwg)
+    acc, total_ms = None, 0.0
     for _ in range(steps):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
@@ -605,23 +607,36 @@ def phase_timeline(dev, prompt_len, steps=32, workgroup=0):
         e1.record()
         torch.cuda.synchronize()
         total_ms += e0.elapsed_time(e1)
-        c = sess.phase_clocks(workgroup).double()
-        acc += c[: n_stamps + n_tail] - c[0]
-    acc /= steps
+        c = sess.phase_clocks(None).double()
+        c = c - c[:, 0].min()
+        acc = c if acc is None else acc + c
+    acc = acc / steps / 100.0  # us
     kernel_us = total_ms / steps * 1e3
-    end = float(acc[n_stamps + n_tail - 1])
-    ticks_per_us = end / kernel_us  # the whole kernel, first to last sample, against HIP events
-    d = (acc[1:n_stamps] - acc[:n_stamps - 1]).view(nl, per)
-    rows = {}
-    for j, (phase, what) in enumerate(PHASE_STAMPS):
-        rows.setdefault(phase, []).append((what, float(d[:, j].mean()) / ticks_per_us))
-    out = {"kernel_us_hip_events": round(kernel_us, 2), "layers": nl, "clock_ticks_per_us": round(ticks_per_us, 2),
-           "per_layer_us": round(float(d.sum(1).mean()) / ticks_per_us, 3),
+    idx = {name: j + 1 for j, name in enumerate(PHASE_STAMPS)}  # sample 0 precedes the first layer
+
+    def last(role, name, layer):
+        return float(acc[list(roles[role]), layer * per + idx[name]].max())
+
+    chain = [("qkv", "P1 staged", "stream polled for, norm1 in LDS"), ("qkv", "P1 epilogue", "q/k/v product, rotary, q and new k/v rows stored"),
+             ("attention", "P2 chunk announced", "q polled for, chunk, partials stored and announced"),
+             ("wo", "P3 merged", "chunks polled for, partials fetched and merged"), ("wo", "P3 epilogue", "output projection + residual stored"),
+             ("gate/up", "P4 staged", "stream polled for, norm2 in LDS"), ("gate/up", "P4 epilogue", "gate/up product, SwiGLU stored"),
+             ("down", "P5 staged", "activations polled for, in LDS"), ("down", "P5 epilogue", "down projection + residual stored")]
+    seg = torch.zeros(len(chain) + 1, dtype=torch.float64)
+    layers = range(1, nl - 1)
+    for l in layers:
+        t = [last(r, n, l) for r, n, _ in chain] + [last("qkv", "P1 staged", l + 1)]
+        prev = last("down", "P5 epilogue", l - 1)
+        seg += torch.tensor([t[0] - prev] + [t[i] - t[i - 1] for i in range(1, len(chain))] + [t[-1] - t[0]])
+    seg /= len(layers)
+    out = {"kernel_us_hip_events (stamps on)": round(kernel_us, 2), "layers": nl, "workgroups": sess._nwg,
+           "roles (workgroups)": {k: [v.start, v.stop - 1] for k, v in roles.items()},
+           "per_layer_us": round(float(seg[-1]), 3),
+           "before_first_layer_us": round(float(acc[list(roles["qkv"]), idx["P1 staged"]].max()), 2),
            "after_last_layer_us (final norm + vocabulary projection + selection)":
-               round((end - float(acc[n_stamps - 1])) / ticks_per_us, 2), "phases": {}}
-    for phase, items in rows.items():
-        out["phases"][phase] = {"total_us": round(sum(v for _, v in items), 3),
-                                "parts_us": {w: round(v, 3) for w, v in items}}
+               round(float(acc[:, nl * per + PHASE_TAIL].max()) - last("down", "P5 epilogue", nl - 1), 2),
+           "critical_path_us (last workgroup of the role, from the previous entry)":
+               {f"{r}: {what}": round(float(seg[i]), 3) for i, (r, _, what) in enumerate(chain)}}
     return out
 
 

@@ -401,17 +401,22 @@ int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* s, int seq_
  * Same result as ohara_llama_forward(seq_len = 1, use_pos_dev = 1, LOGITS_LAST) but the
  * whole step (all layers, vocabulary projection, greedy selection) runs in a single
  * kernel of `n_workgroups` resident workgroups (use the CU count; more than the device can
- * hold of this kernel at once returns OHARA_ESIZE) separated by grid-wide barriers; it has no counterpart in the reference, whose decode step is
+ * hold of this kernel at once returns OHARA_ESIZE) whose phases are separated by grid-wide barriers
+ * (batch > 1) or hand their rows over through memory that the consumers poll (batch 1); it has no counterpart in the reference, whose decode step is
  * ~1000 eager launches (llama.py:279-323).  The cache position and step index are read
  * from / advanced in s->step_state; s->attn and s->attn_ws are not used.
  * `workspace`: ohara_persistent_workspace_bytes(m, batch, s->n_split, n_workgroups) of
- * device memory with any contents (it need not be zeroed: every slot a step reads was written
- * earlier in the same step, and the merge of the attention chunks never uses a chunk no workgroup
- * wrote).  Call once with init_workspace = 1 (copies the layer table and the
- * cache pointers to the device, zeroes the barrier words; synchronises the stream; do
- * it outside graph capture) whenever the model or the caches change; then each call
- * with init_workspace = 0 enqueues one step.  spin_limit bounds every barrier wait
- * (0 = default); if a wait expires the kernel still drains and the error word reads
+ * device memory with any contents (it need not be zeroed: the call with init_workspace = 1 sets
+ * what a step relies on, every other slot a step reads was written earlier in the same step, and
+ * the merge of the attention chunks never uses a chunk no workgroup wrote).  Call once with
+ * init_workspace = 1 (copies the layer table and the cache pointers to the device, zeroes the
+ * barrier words, the launch counters and the attention partials behind them and fills the
+ * hand-off rows of the batch-1 kernel with 0xFF, their "not written yet"; synchronises the stream;
+ * do it outside graph capture) whenever the model or the caches change, and before the workspace
+ * is used for the first time or after its memory has been used for anything else; then each call
+ * with init_workspace = 0 enqueues one step.  Steps on one workspace must not overlap (each
+ * step counts itself in the workspace).  spin_limit bounds every barrier wait and every poll for
+ * a hand-off (0 = default); if a wait expires the kernel still drains and the error word reads
  * non-zero.  s->n_split must be 16.
  * Requires head_dim 64 or 128, n_heads / n_kv_heads in {1, 2, 4}, d_model <= 1024,
  * d_model and d_ff multiples of 8. */

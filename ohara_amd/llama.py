@@ -671,9 +671,13 @@ class DecodeSession:
                                                       self._nwg, 1, 1, 0, torch.cuda.current_stream().cuda_stream),
                   "persistent init")
 
-    def phase_clocks(self, workgroup: int = 0) -> torch.Tensor:
+    def phase_clocks(self, workgroup: int | None = 0) -> torch.Tensor:
         """Clock samples (constant 100 MHz counter) that thread 0 of ``workgroup`` took at the phase
-        boundaries of the last step run with ``step(prof_kernel=-2)`` (measurement aid)."""
+        boundaries of the last step run with ``step(prof_kernel=-2)`` (measurement aid); ``None``: one
+        row per workgroup."""
+        if workgroup is None:
+            off = self._prof_off
+            return self._pws[off : off + 8192 * self._nwg].view(torch.int64).cpu().view(self._nwg, 1024)
         off = self._prof_off + workgroup * 8192
         return self._pws[off : off + 8192].view(torch.int64).cpu()
 

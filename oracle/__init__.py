@@ -20,8 +20,15 @@ Pinning status (what independently fixes each function; see tests/test_oracle.py
   attention           fp64 brute-force loops on tiny inputs; cached == uncached
                       (the uncached path reduces to F.scaled_dot_product_attention
                       with is_causal=True, a library routine)
+  attention in bf16   (_attention_reduced, fexp_u20) the library's bf16 routine on six shapes
+                      and a V = identity probe of the exponential (tests/test_oracle_bf16.py);
+                      the reference's per-module operands of a mid-size GQA model
+                      (tests/golden/llama_bf16_mid_gqa.pt)
   swiglu / linear     F.silu / matmul library routines
-  llama_forward       composition: golden fixture tests/golden/llama_tiny_*.pt
+  llama_forward       composition: golden fixtures tests/golden/llama_tiny_*.pt (fp32) and
+                      tests/golden/llama_bf16_*.pt (the reference model cast to bfloat16:
+                      tiny models bit-identical; d12 widths and d12 itself within the
+                      distance between the reference's own runs, which the fixtures hold)
   moe_route/dispatch  per-token hand loop, k distinct experts, weights sum to 1,
                       golden fixture tests/golden/llama_tiny_moe.pt
   sample_*            the reference tests' known answers; exhaustive small-V
@@ -39,7 +46,9 @@ Pinning status (what independently fixes each function; see tests/test_oracle.py
                       cached == uncached invariant and an fp64 hand-written block
                       (tests/test_oracle_phi.py)
 
-bf16 GEMM accumulation order is "parity unpinned" by the reference (it holds no
-bf16 test); the oracle defines a Linear as an fp32-accumulated product of the
-dtype-rounded operands, rounded once to the model dtype.
+bf16 GEMM accumulation order is "parity unpinned": the library's own kernels differ
+from each other in it (each bf16 fixture holds the reference run with all threads, with
+one thread and with the library's other matrix kernels); the oracle defines a Linear as
+an fp32-accumulated product of the dtype-rounded operands, rounded once to the model
+dtype, which reproduces >= 99.98 % of the reference's per-operator outputs bit for bit.
 """
