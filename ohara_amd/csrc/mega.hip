@@ -134,6 +134,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   // ONE (batch 1): the tagged path; the host launches it only on a grid wide enough for gate/up and the
   // down projection (and the output projection and the down projection) to sit on different workgroups -
   // their weights share registers - and the general build otherwise.
+  uint32_t lm_staged_addr = 0;  // batch 1: where this wave's second vocabulary strip is parked in LDS (0: nowhere)
   if constexpr (ONE) {
    {
     // ---- batch 1: tagged hand-offs, no grid barrier inside the layers ---------------------------------
@@ -170,7 +171,28 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     char* wl = reinterpret_cast<char*>(((uintptr_t)(ptab + m.n_layers * 8) + 255) & ~(uintptr_t)255);  // 4 x OHARA_LDS_PF KB
     dn.wlds_addr = (uint32_t)(uintptr_t)(OHARA_LDS char*)wl;
     pf.stamp();
+    // The vocabulary projection is the one long stream of the step (100 MB at d12) and the layers leave the memory
+    // system idle: a workgroup without a down-projection strip parks the tiles of each wave's second vocabulary strip
+    // in the LDS that the down projection's workgroups use for their weights, a few tiles per layer, requested where
+    // the workgroup has nothing to wait for soon.
+    const int KSL = (lm.K + 31) >> 5;
+    const int lm_strip1 = (nwg + (int)blockIdx.x) * 4 + (int)(threadIdx.x >> 6);
+    const bool lm_staged = !has_dn && KSL <= OHARA_LDS_PF && lm_strip1 < lm.nstrips && 2 * nwg * 4 <= lm.nstrips;
+    const int lm_per = (KSL + m.n_layers - 1) / m.n_layers;
+    if (lm_staged) lm_staged_addr = dn.wlds_addr + (uint32_t)(threadIdx.x >> 6) * OHARA_LDS_PF * 1024;
     for (int l = 0; l < m.n_layers; ++l) {
+      auto lm_stage = [&]() {
+        if (!lm_staged) return;
+        const int c0 = l * lm_per, c1 = min(KSL, c0 + lm_per);
+        const uint4* src = lm.wp + ((size_t)lm_strip1 * KSL + c0) * 64 + (threadIdx.x & 63);
+        char* dst = wl + ((size_t)(threadIdx.x >> 6) * OHARA_LDS_PF + c0) * 1024;
+#pragma unroll 1
+        for (int c = c0; c < c1; ++c) {
+          __builtin_amdgcn_global_load_lds((const OHARA_GLOBAL void*)src, (OHARA_LDS void*)dst, 16, 0, 0);
+          src += 64;
+          dst += 1024;
+        }
+      };
       const unsigned long long* pl = ptab + l * 8;
       bf16_t* kc = lds_ptr<bf16_t>(pl, 6);
       bf16_t* vc = lds_ptr<bf16_t>(pl, 7);
@@ -207,6 +229,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
         qkv.norm_w = lds_ptr<const bf16_t>(pl, 12);
         gemm_prefetch<4, 6, E_ROPE, 0, false>(qkv, pre, 1, g1, r1);  // (the rotary pair is the same in every layer)
       }
+      if (has_qkv) lm_stage();  // (the next thing a q/k/v workgroup polls for is a phase or more away)
       // the down projection's weights (98 KB a workgroup) into LDS: on their way from here, used after P4
       dn.wp = lds_ptr<const uint4>(pl, 3); dn.tout = xn; dn.tresid = xt;
       if (has_dn) {
@@ -254,6 +277,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
       gemm_phase<4, 12, E_XNEXT, ProfT<PROFILE>, 0, true>(dn, pre, xs, ldxs, 1, red, best_v, best_i, pf);  // 2 stamps
       pf.stamp();  // x_next stored
       if (has_dn) next_weights();
+      if (!has_qkv) lm_stage();
       pf.stamp();  // next layer's weights requested
     }
     // final norm + vocabulary projection: the stream of the last layer is polled for like any other
@@ -355,7 +379,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
                              pre.g);
   __syncthreads();
   }
-  lm_phase(lm, pre, xs, ldxs, B, best_v, best_i, pf);
+  lm_phase(lm, pre, xs, ldxs, B, best_v, best_i, pf, lm_staged_addr);
   pf.stamp();
   if (a.select) {
     // lanes with the same batch column (lane & 15) fold their candidates; then the waves

@@ -1037,9 +1037,12 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
 // compiler waits for exactly the buffer it needs.  Same products in the same order as
 // gemm_phase<1, 24, E_LOGITS>, whose prefetch (the first strip's first 24 k-steps) it takes over.
 // ---------------------------------------------------------------------------------------
+// `staged` (a byte address in LDS, 0 = nothing): the tiles of this wave's SECOND strip were parked there
+// ahead of the phase (tile c at staged + c KB; strips of at most 24 k-steps); they are multiplied while the
+// first loads from memory are on their way.
 template <class PROF>
 __device__ __forceinline__ void lm_phase(const GemmP& p, const GemmPre& pre, const bf16_t* xs, int ldxs, int B,
-                                         float& best_v, int& best_i, PROF& pf) {
+                                         float& best_v, int& best_i, PROF& pf, uint32_t staged = 0) {
   constexpr int HC = 12;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 15, g = lane >> 4;
@@ -1065,7 +1068,7 @@ __device__ __forceinline__ void lm_phase(const GemmP& p, const GemmPre& pre, con
 #pragma unroll
     for (int cc = 0; cc < HC; ++cc) wb[cc] = pre.w[HC + cc];
   } else {
-    load(wb, 1);
+    load(wb, staged ? 2 : 1);
   }
   f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
   auto process = [&](const uint4 (&w)[HC], int q) {
@@ -1106,16 +1109,28 @@ __device__ __forceinline__ void lm_phase(const GemmP& p, const GemmPre& pre, con
       }
     }
   };
-  for (int q = 0; q < total; q += 2) {
-    process(wa, q);
-    load(wa, q + 2);
-    if (q == 0) {
+  // chunks that come from memory, in order: all of them but the staged strip's (chunks ncps .. 2 ncps - 1)
+  auto gq = [&](int k) { return (staged && k >= ncps) ? k + ncps : k; };
+  const int nglob = staged ? total - ncps : total;
+  for (int k = 0; k < nglob; k += 2) {
+    process(wa, gq(k));
+    load(wa, gq(k + 2));
+    if (k == 0) {
       pf.stamp();  // first products issued
       pf.stamp();
     }
-    if (q + 1 < total) {
-      process(wb, q + 1);
-      load(wb, q + 3);
+    if (k + 1 < nglob) {
+      process(wb, gq(k + 1));
+      load(wb, gq(k + 3));
+    }
+    if (k == 0 && staged) {
+      wait_own_stores();  // this wave's own loads into LDS have landed (requested layers ago)
+      for (int c = 0; c < ncps; ++c) {
+        uint4 wc[HC];
+#pragma unroll
+        for (int cc = 0; cc < HC; ++cc) wc[cc] = lds16_at(staged + ((uint32_t)min(c * HC + cc, KS - 1) * 64 + lane) * 16);
+        process(wc, ncps + c);
+      }
     }
   }
 }
