@@ -364,6 +364,13 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
 // the lane that owns a position loads its record, the value rows get their scale and minimum from that
 // lane by a shuffle.  Codes become the bf16 values the reference's read returns - bf16((code + 128) *
 // scale + min) - right before use, so the results are those of bf16 attention over the dequantised cache.
+// Turning the codes into those values is most of what a position costs (2.5 vector instructions per
+// element), so the score product runs on the matrix cores: A = the group's q rows (row m = head m, the
+// other rows zero), B = the sixteen dequantised key rows of a sub-tile (lane (position n, quarter kg)
+// holds the 8 elements of its quarter that step c contracts - the k index of the product is a
+// permutation of the head dimension, the same one on both sides), NC products of 16x16x32 per sub-tile;
+// lanes 0..15 end up with the scores of position n for every head.  The value product stays on the
+// vector units (its operand would have to be transposed).
 template <int D, int G>
 __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(AttnArgs a) {
   constexpr int NC = D / 32;        // bf16 uint4 of a K quarter-row after expansion
@@ -380,19 +387,17 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
   const int t0 = split * chunk;
   const int t1 = min(L, t0 + chunk);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int p = lane >> 2, dq = lane & 3;  // position of the tile, quarter of its K row: a quad holds one row
+  const int p = lane & 15, dq = lane >> 4;  // position of the sub-tile, quarter of its K row (the B operand's column and k group)
   const int pp = lane / DC, dc = lane % DC;
   const float scale_l2 = a.scale * OHARA_LOG2E;  // scores in log2 units (common.h: softmax bookkeeping)
 
   __shared__ float s_m[4][G], s_l[4][G];
   __shared__ float s_acc[4][G][D];
 
-  uint4 qv[G][NC];  // q for this lane's contiguous quarter dq of the row
+  uint4 qa[NC];  // A operand: row (lane & 15) = head of the group (rows past the group are zero), this lane's quarter dq
 #pragma unroll
-  for (int hh = 0; hh < G; ++hh)
-#pragma unroll
-    for (int c = 0; c < NC; ++c)
-      qv[hh][c] = ldg16(a.q + (size_t)b * a.H * D + (size_t)(kvh * G + hh) * D + (dq * NC + c) * 8);
+  for (int c = 0; c < NC; ++c)
+    qa[c] = p < G ? ldg16(a.q + (size_t)b * a.H * D + (size_t)(kvh * G + p) * D + (dq * NC + c) * 8) : make_uint4(0, 0, 0, 0);
 
   float m_run[G], l_run[G], acc[G][8];
 #pragma unroll
@@ -447,17 +452,15 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
           const uint2 lo = dequant4(w[0] ^ 0x80808080u, ks, km), hi = dequant4(w[1] ^ 0x80808080u, ks, km);
           kv[c] = make_uint4(lo.x, lo.y, hi.x, hi.y);
         }
+        f32x4 sacc = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int hh = 0; hh < G; ++hh) {
-          float s = 0.f;
+        for (int c = 0; c < NC; ++c)
+          sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, qa[c]), __builtin_bit_cast(bf16x8, kv[c]),
+                                                         sacc, 0, 0, 0);
 #pragma unroll
-          for (int c = 0; c < NC; ++c) s = dot8(kv[c], qv[hh][c], s);
-          sc[hh] = s;
-        }
+        for (int hh = 0; hh < G; ++hh) sc[hh] = sacc[hh];  // lanes 0..15: head hh against position p (rows 4.. of the product are zero)
       }
-#pragma unroll
-      for (int hh = 0; hh < G; ++hh) sc[hh] = quad_sum(sc[hh]);
-      const bool valid = tb + 16 * sb + p < t1;
+      const bool valid = lane < 16 && tb + 16 * sb + p < t1;
       bool raise = false;
 #pragma unroll
       for (int hh = 0; hh < G; ++hh) {
@@ -469,7 +472,7 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
 #pragma unroll
         for (int hh = 0; hh < G; ++hh) tm[hh] = sc[hh];
 #pragma unroll
-        for (int hh = 0; hh < G; ++hh) tm[hh] = lanes_max<32, 4>(tm[hh]);
+        for (int hh = 0; hh < G; ++hh) tm[hh] = lanes_max<32, 1>(tm[hh]);
 #pragma unroll
         for (int hh = 0; hh < G; ++hh) {
           const float mn = fmaxf(m_run[hh], ceilf(tm[hh]));  // finite here: some position of the sub-tile raised it
@@ -496,7 +499,7 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
 #pragma unroll
         for (int cc = 0; cc < XB; ++cc) {
           const int c = sb * (NV / 2) + c0 + cc;
-          const int src = 4 * ((c * PP + pp) & 15);  // a lane that owns the position of the row I hold eight codes of
+          const int src = (c * PP + pp) & 15;  // the lane that holds the weight (and a record) of the row I hold eight codes of
           vs[cc] = __shfl(__uint_as_float(cur.st[sb].z), src, WAVE);
           vm[cc] = __shfl(__uint_as_float(cur.st[sb].w), src, WAVE);
 #pragma unroll
@@ -546,7 +549,7 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
 
   // fold the sums over the 16 positions of a sub-tile, the PP row-groups of the wave, then the four waves
 #pragma unroll
-  for (int hh = 0; hh < G; ++hh) l_run[hh] = lanes_sum<32, 4>(l_run[hh]);
+  for (int hh = 0; hh < G; ++hh) l_run[hh] = lanes_sum<32, 1>(l_run[hh]);  // (lanes 16.. hold zeros)
 #pragma unroll
   for (int hh = 0; hh < G; ++hh) {
 #pragma unroll
@@ -563,6 +566,215 @@ __global__ __launch_bounds__(256, (G == 1 ? 3 : 2)) void attn_decode_i8_kernel(A
     if (lane == 0) {
       s_m[wave][hh] = m_run[hh];
       s_l[wave][hh] = l_run[hh];
+    }
+  }
+  __syncthreads();
+  for (int idx = tid; idx < G * D; idx += 256) {
+    const int hh = idx / D, d = idx - hh * D;
+    const int h = kvh * G + hh;
+    float M = fmaxf(fmaxf(s_m[0][hh], s_m[1][hh]), fmaxf(s_m[2][hh], s_m[3][hh]));
+    float Ls = 0.f, o = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float mw = s_m[w][hh];
+      const float scw = (mw == -INFINITY) ? 0.f : pow2_neg_int(mw - M);
+      Ls += s_l[w][hh] * scw;
+      o += s_acc[w][hh][d] * scw;
+    }
+    if (a.nsplit == 1) {  // whole context in this workgroup: no partials
+      a.out[(size_t)b * a.H * D + h * D + d] = f2bf(o * (1.0f / Ls));
+      continue;
+    }
+    const size_t pi = (size_t)(b * a.H + h) * a.nsplit + split;
+    stf_coh(a.part_acc + pi * D + d, o);
+    if (d == 0) {
+      stf_coh(a.part_ml + pi * 2, M);
+      stf_coh(a.part_ml + pi * 2 + 1, Ls);
+    }
+  }
+  if (a.nsplit == 1) return;
+  if (last_chunk_done(a.counters + b * a.Hkv + kvh, a.nsplit)) merge_partials<D>(a, b, kvh, G);
+}
+
+// Head width 128 over the int8 cache with BOTH products on the matrix cores.  What a position costs in the
+// kernel above is vector instructions - 2.5 per element to turn codes into the reference's bf16 values,
+// and again as many multiply-adds per head for the value product - so at four heads per group it stays well
+// below the memory's speed.  Here a wave walks tiles of 32 positions:
+//   S^T = K Q^T    v_mfma_f32_16x16x32_bf16 per sub-tile of 16 positions: A = the dequantised key rows (lane
+//                  (position, quarter) holds the 8 elements of its quarter that step c contracts), B = the
+//                  group's q rows (column n = head n, the other columns zero).  Lane (head n, rg) ends up with
+//                  the scores of positions 4 rg .. 4 rg + 3 of the sub-tile for ONE head: its running maximum,
+//                  sum and rescale are per-lane scalars and the row maximum needs two cross-lane steps.
+//   O^T += V^T P   the weights go from the score accumulators straight into the B operand: k-slot j of lane
+//                  (n, rg) is position 4 rg + j of the first sub-tile for j < 4 and of the second for j >= 4.
+//                  A lane dequantises 8 consecutive positions x 8 columns of V, transposes them in registers
+//                  and parks them in the wave's own LDS as V^T (column-major), from where the A operand of a
+//                  16-column block is two 8-byte reads that follow the same slot mapping.
+// A lane then holds O[head n][16 blk + 4 rg + i]: no cross-lane sums at the end.  The weights are rounded
+// to bf16 by the operand format, the sum is taken from the unrounded ones, scores are in log2 units with an
+// integer running maximum: the rounding points of the kernels above.
+template <int G>
+__global__ __launch_bounds__(256, 2) void attn_decode_i8_mfma_kernel(AttnArgs a) {
+  constexpr int D = 128, NC = 4, NB = 8;
+  constexpr int LDV = 36;  // V^T row stride in elements (72 bytes: 8-byte reads and writes stay aligned)
+  const int split = blockIdx.z, kvh = blockIdx.y, b = blockIdx.x;
+  const int seq = b / a.S;
+  const int L = min((a.pos_dev ? a.pos_dev[(size_t)seq * a.pos_stride] : a.start) + (b - seq * a.S) + 1, a.Tmax);
+  const int chunk = (((L + a.nsplit - 1) / a.nsplit) + 127) & ~127;
+  const int t0 = split * chunk;
+  const int t1 = min(L, t0 + chunk);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 15, rg = lane >> 4;  // K side: position n of a sub-tile, quarter rg; scores: head n, position group rg
+  const float scale_l2 = a.scale * OHARA_LOG2E;
+
+  __shared__ float s_m[4][G], s_l[4][G];
+  __shared__ float s_acc[4][G][D];
+  __shared__ __align__(16) bf16_t s_vt[4][D][LDV];
+
+  uint4 qa[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c)
+    qa[c] = n < G ? ldg16(a.q + (size_t)b * a.H * D + (size_t)(kvh * G + n) * D + (rg * NC + c) * 8) : make_uint4(0, 0, 0, 0);
+
+  float m_run = -INFINITY, l_run = 0.f;
+  f32x4 acc[NB];
+#pragma unroll
+  for (int i = 0; i < NB; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  const size_t row = (size_t)a.Hkv * D;
+  const int8_t* kb8 = reinterpret_cast<const int8_t*>(a.k) + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
+  const int8_t* vb8 = reinterpret_cast<const int8_t*>(a.v) + (size_t)seq * a.Tmax * row + (size_t)kvh * D;
+  const float* stb = a.stats + ((size_t)seq * a.Hkv + kvh) * a.Tmax * 4;
+
+  struct Tile {
+    uint4 k[2][2];  // sub-tile s: the 32 codes of quarter rg of row tb + 16 s + n
+    uint2 ks[2];    // (key scale, key minimum) of that row
+    uint2 v[8];     // eight codes (columns 8 dc ..) of row tb + 8 pp + c
+    uint2 vs[8];    // (value scale, value minimum) of that row
+  };
+  // Loads without branches: positions past the chunk read its last row (their scores are masked).
+  auto load_tile = [&](int tb, Tile& t) {
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      const int pos = min(tb + 16 * sb + n, t1 - 1);
+      t.ks[sb] = ldg8(stb + (size_t)pos * 4);
+#pragma unroll
+      for (int c = 0; c < 2; ++c) t.k[sb][c] = ldg16_nt(kb8 + (size_t)pos * row + rg * 32 + 16 * c);
+    }
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const int vp = min(tb + 8 * rg + c, t1 - 1);  // (V side: lane (pp = rg, dc = n))
+      const u32x2 w = __builtin_nontemporal_load((const OHARA_GLOBAL u32x2*)(vb8 + (size_t)vp * row + n * 8));
+      t.v[c] = make_uint2(w.x, w.y);
+      t.vs[c] = ldg8(stb + (size_t)vp * 4 + 2);
+    }
+  };
+  bf16_t* vt = &s_vt[wave][0][0];
+  auto consume = [&](int tb, const Tile& cur) {
+    // ---- V: dequantise 8 positions x 8 columns, transpose, park as V^T ---------------------------------
+    {
+      uint32_t w[8][4];  // row c: four dwords = columns (0,1) (2,3) (4,5) (6,7) as bf16 pairs
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const float vs = __uint_as_float(cur.vs[c].x), vm = __uint_as_float(cur.vs[c].y);
+        const uint2 lo = dequant4(cur.v[c].x ^ 0x80808080u, vs, vm), hi = dequant4(cur.v[c].y ^ 0x80808080u, vs, vm);
+        w[c][0] = lo.x; w[c][1] = lo.y; w[c][2] = hi.x; w[c][3] = hi.y;
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {  // column pair (2e, 2e + 1) of this lane's eight columns
+        uint32_t ev[4], od[4];       // positions (0,1) (2,3) (4,5) (6,7) of the even / the odd column
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          ev[q] = (w[2 * q][e] & 0xffffu) | (w[2 * q + 1][e] << 16);
+          od[q] = (w[2 * q][e] >> 16) | (w[2 * q + 1][e] & 0xffff0000u);
+        }
+        bf16_t* c0 = vt + (size_t)(n * 8 + 2 * e) * LDV + 8 * rg;
+        *reinterpret_cast<uint2*>(c0) = make_uint2(ev[0], ev[1]);
+        *reinterpret_cast<uint2*>(c0 + 4) = make_uint2(ev[2], ev[3]);
+        *reinterpret_cast<uint2*>(c0 + LDV) = make_uint2(od[0], od[1]);
+        *reinterpret_cast<uint2*>(c0 + LDV + 4) = make_uint2(od[2], od[3]);
+      }
+    }
+    // ---- scores of both sub-tiles ---------------------------------------------------------------------------
+    float sc[8];
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      const float ks = __uint_as_float(cur.ks[sb].x), km = __uint_as_float(cur.ks[sb].y);
+      f32x4 sacc = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const uint32_t* w = reinterpret_cast<const uint32_t*>(&cur.k[sb][c >> 1]) + 2 * (c & 1);
+        const uint2 lo = dequant4(w[0] ^ 0x80808080u, ks, km), hi = dequant4(w[1] ^ 0x80808080u, ks, km);
+        const uint4 kv = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kv), __builtin_bit_cast(bf16x8, qa[c]), sacc,
+                                                       0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        sc[4 * sb + i] = (n < G && tb + 16 * sb + 4 * rg + i < t1) ? sacc[i] * scale_l2 : -INFINITY;
+    }
+    float tm = sc[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) tm = fmaxf(tm, sc[i]);
+    tm = lane_xor_max<32>(lane_xor_max<16>(tm));  // over the four position groups of this head
+    if (__any(tm > m_run)) {
+      const float mn = fmaxf(m_run, ceilf(tm));
+      const float corr = pow2_neg_int(m_run - mn);  // (both -inf, a head past the group: 2^-126 times zeros)
+      m_run = mn;
+      l_run *= corr;
+#pragma unroll
+      for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[blk][i] *= corr;
+    }
+    float pw[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      pw[i] = sc[i] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sc[i] - m_run);
+      l_run += pw[i];
+    }
+    const uint4 pb = make_uint4(pack_bf(pw[0], pw[1]), pack_bf(pw[2], pw[3]), pack_bf(pw[4], pw[5]), pack_bf(pw[6], pw[7]));
+    // ---- O^T += V^T P: the A operand of block blk is column 16 blk + n, positions 4 rg .. and 16 + 4 rg .. --------
+    // (the wave reads what its own lanes wrote above: LDS accesses of a wave complete in order)
+    uint4 va[NB];
+#pragma unroll
+    for (int blk = 0; blk < NB; ++blk) {
+      const bf16_t* col = vt + (size_t)(16 * blk + n) * LDV + 4 * rg;
+      const uint2 lo = *reinterpret_cast<const uint2*>(col);
+      const uint2 hi = *reinterpret_cast<const uint2*>(col + 16);
+      va[blk] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int blk = 0; blk < NB; ++blk)
+      acc[blk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, va[blk]), __builtin_bit_cast(bf16x8, pb),
+                                                         acc[blk], 0, 0, 0);
+  };
+  Tile cur, nxt;
+  int tb = t0 + wave * 32;
+  if (tb < t1) {
+    load_tile(tb, cur);
+    for (;;) {
+      if (tb + 128 >= t1) { consume(tb, cur); break; }
+      load_tile(tb + 128, nxt);
+      consume(tb, cur);
+      tb += 128;
+      if (tb + 128 >= t1) { consume(tb, nxt); break; }
+      load_tile(tb + 128, cur);
+      consume(tb, nxt);
+      tb += 128;
+    }
+  }
+  // the sum over the four position groups; a lane holds O[head n][16 blk + 4 rg + i]
+  l_run = lane_xor_sum<32>(lane_xor_sum<16>(l_run));
+  if (n < G) {
+#pragma unroll
+    for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s_acc[wave][n][16 * blk + 4 * rg + i] = acc[blk][i];
+    if (rg == 0) {
+      s_m[wave][n] = m_run;
+      s_l[wave][n] = l_run;
     }
   }
   __syncthreads();
@@ -684,6 +896,12 @@ __global__ __launch_bounds__(256) void attn_decode_generic(AttnArgs a) {
 template <int D, bool I8>
 int launch_fast(const AttnArgs& a, int G, dim3 grid, hipStream_t st) {
   if (I8) {
+    if (D == 128 && G > 1) {  // several heads share the dequantised rows: both products on the matrix cores
+      if (G == 2) hipLaunchKernelGGL((attn_decode_i8_mfma_kernel<2>), grid, dim3(256), 0, st, a);
+      else if (G == 4) hipLaunchKernelGGL((attn_decode_i8_mfma_kernel<4>), grid, dim3(256), 0, st, a);
+      else return 1;
+      return 0;
+    }
     switch (G) {
       case 1: hipLaunchKernelGGL((attn_decode_i8_kernel<D, 1>), grid, dim3(256), 0, st, a); break;
       case 2: hipLaunchKernelGGL((attn_decode_i8_kernel<D, 2>), grid, dim3(256), 0, st, a); break;

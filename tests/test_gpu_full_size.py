@@ -73,7 +73,7 @@ def test_decode_attention_microbench_shape_int8_cache(cuda, B, L):
     assert (kd.float() - k.float()).abs().max().item() <= 0.05  # tests/test_modules.py:82-100 of the reference
     same = ops.attn_decode(q, kd, vd, H, Hkv, D, L, ns, ws)
     scale = same.float().abs().max().item()
-    assert (out.float() - same.float()).abs().max().item() <= 2.0 ** -8 * scale
+    assert (out.float() - same.float()).abs().max().item() <= 2.0 ** -7 * scale  # one bf16 ulp of the largest output
     assert (out == same).float().mean().item() >= 0.99
     o3 = out.view(B, H, D)
     for b, h in ((0, 0), (B // 2, 13), (B - 1, H - 1)):
