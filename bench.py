@@ -569,7 +569,7 @@ PHASE_STAMPS = (
 PHASE_TAIL = 13  # samples after the layers: three around the final norm, vocabulary projection (2), its end, selection (6), the end
 
 
-def _batch1_roles(cfg, nwg):
+def _batch1_roles(cfg, nwg, batch=1):
     """Which workgroups take which phase of the batch-1 kernel (mirrors the assignment in csrc/mega.hip)."""
     d, F = cfg.hidden_size, cfg.intermediate_size
     H = cfg.num_attention_heads
@@ -577,13 +577,16 @@ def _batch1_roles(cfg, nwg):
     D = d // H
     n_qkv, n_wo, n_dn = (H + 2 * Hkv) * D // 16, d // 16, d // 16
     n_gu = (2 * ((F + 7) // 8 * 8) // 16 + 1) // 2
-    ns = max(1, min(16, nwg // Hkv))
+    ns = max(1, min(16, nwg // (batch * Hkv)))
+    p2 = 1 << (ns.bit_length() - 1)
+    if not (2 * ns >= 3 * p2 and ns <= 8):
+        ns = p2
     dn0 = n_wo if n_wo + n_dn <= nwg else nwg - n_dn
-    return {"qkv": range(nwg - n_qkv, nwg), "attention": range(0, Hkv * ns), "wo": range(0, n_wo),
+    return {"qkv": range(nwg - n_qkv, nwg), "attention": range(0, batch * Hkv * ns), "wo": range(0, n_wo),
             "gate/up": range(0, n_gu), "down": range(dn0, dn0 + n_dn)}
 
 
-def phase_timeline(dev, prompt_len, steps=32):
+def phase_timeline(dev, prompt_len, steps=32, batch=1):
     """The critical path of a layer of the batch-1 persistent kernel: for every hand-off, when the last
     workgroup of the producing role had issued its stores and when the last workgroup of the consuming
     role had the data staged, from the kernel's own clock samples (a 100 MHz counter common to all
@@ -592,13 +595,13 @@ def phase_timeline(dev, prompt_len, steps=32):
 
     cfg, st = d12_state(dev)
     model = Llama(cfg, st, device=dev)
-    sess = model.session(1, steps + 24)
-    sess.prefill(torch.randint(0, cfg.vocab_size, (1, prompt_len)).to(dev))
+    sess = model.session(batch, steps + 24, persistent=True)
+    sess.prefill(torch.randint(0, cfg.vocab_size, (batch, prompt_len)).to(dev))
     for _ in range(8):
         sess.step()
     nl = cfg.num_hidden_layers
     per = len(PHASE_STAMPS)
-    roles = _batch1_roles(cfg, sess._nwg)
+    roles = _batch1_roles(cfg, sess._nwg, batch)
     acc, total_ms = None, 0.0
     for _ in range(steps):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -709,6 +712,7 @@ def main():
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run three 1 GiB device-to-device copies (a kernel of known traffic to scale "
                          "FETCH_SIZE / WRITE_SIZE counters against)")
+    ap.add_argument("--timeline-batch", type=int, default=1, help="sequences of the --phase-timeline run (1 to 8)")
     ap.add_argument("--phase-timeline", action="store_true",
                     help="print the per-phase timeline of the persistent decode kernel at batch 1 and exit")
     ap.add_argument("--bitnet-phase-timeline", type=int, default=0, metavar="B",
@@ -752,7 +756,7 @@ def main():
         print(json.dumps(bench_bitnet(dev, tuple(int(b) for b in args.bitnet_only.split(","))), indent=1))
         return
     if args.phase_timeline:
-        print(json.dumps(phase_timeline(dev, args.prompt), indent=1))
+        print(json.dumps(phase_timeline(dev, args.prompt, batch=args.timeline_batch), indent=1))
         return
     if args.pmc_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)

@@ -67,6 +67,7 @@ struct MegaArgs {
   char* tg;             // batch 1: two sets of NL blocks of polled mailboxes, tg_stride bytes a block, tg_set bytes a set
   size_t tg_stride, tg_set;
   int tg_n, tg_q, tg_kv, tg_a;  // byte offsets inside a layer's block: stream after the layer | q | new k, v | activations
+  int tg_rx, tg_rq, tg_rkv, tg_ra;  // bytes between the sequences' rows of those mailboxes
   unsigned int* bar;    // barrier words, see GridSync
   unsigned long long* prof;  // optional: clock of every workgroup's thread 0 at every phase boundary (OHARA_PROF_SLOTS each)
   unsigned int spin_limit;
@@ -76,10 +77,12 @@ struct MegaArgs {
 // ---------------------------------------------------------------------------------------
 // the kernel
 // ---------------------------------------------------------------------------------------
-// ONE: the batch is a single sequence (the row loops and row masks fold away at compile time).
+// MODE 0: any batch up to 16, a grid barrier between the phases.  MODE 1 and 2: the polled builds (no barrier inside the
+// layers) - 1: the batch is a single sequence (the row loops and row masks fold away at compile time), 2: up to eight.
 // PROFILE: with the phase stamps (measurement builds of the head-dim-128, no-GQA kernels only).
-template <int D, int G, bool ONE, bool PROFILE = false>
+template <int D, int G, int MODE, bool PROFILE = false>
 __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
+  constexpr bool ONE = MODE == 1, POLLED = MODE != 0;
   extern __shared__ __align__(16) unsigned char smem[];
   const OharaModel& m = a.m;
   const int d = m.d_model, H = m.n_heads, Hkv = m.n_kv_heads, F = m.d_ff, V = m.vocab, B = ONE ? 1 : a.B;
@@ -107,7 +110,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   // batch 1: the number of this launch since the workspace was cleared, the tag of its hand-offs (read once, here: the
   // last workgroup out advances it)
   unsigned int* launches = a.bar + (gs.ng + 12) * 64;
-  const unsigned int nth = ONE ? *launches + 1u : 0u;
+  const unsigned int nth = POLLED ? *launches + 1u : 0u;
   const int pos = a.step_state[0];
   const int step = a.step_state[1];
   const int L = min(pos + 1, m.t_max);
@@ -131,13 +134,13 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   AttnPre<D> apre;
   qkv.wp = lds_ptr<const uint4>(ptab, 0);
   qkv.norm_w = lds_ptr<const bf16_t>(ptab, 4);
-  // ONE (batch 1): the tagged path; the host launches it only on a grid wide enough for gate/up and the
-  // down projection (and the output projection and the down projection) to sit on different workgroups -
-  // their weights share registers - and the general build otherwise.
+  // The polled builds (batch 1, and up to eight sequences); the host launches them only on a grid wide enough for
+  // gate/up and the down projection (and the output projection and the down projection) to sit on different
+  // workgroups, and the general build otherwise.
   uint32_t lm_staged_addr = 0;  // batch 1: where this wave's second vocabulary strip is parked in LDS (0: nowhere)
-  if constexpr (ONE) {
+  if constexpr (POLLED) {
    {
-    // ---- batch 1: tagged hand-offs, no grid barrier inside the layers ---------------------------------
+    // ---- polled hand-offs, no grid barrier inside the layers ------------------------------------------
     const Poll pc{nth, a.spin_limit, gs.err};
     const int nwg = (int)gridDim.x;
     // this launch's set of mailboxes, and the way from there to the other set
@@ -154,7 +157,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     dn.nstrips = (d + 15) / 16;
     qkv.wg0 = max(0, nwg - qkv.nstrips);
     dn.wg0 = prj.nstrips + dn.nstrips <= nwg ? prj.nstrips : max(0, nwg - dn.nstrips);
-    const int n_chunks = Hkv * a.ns;
+    const int n_chunks = B * Hkv * a.ns;
     const bool has_attn = (int)blockIdx.x < n_chunks;
     const bool has_dn = phase_block(dn) < dn.nstrips;
     const bool has_qkv = phase_block(qkv) < qkv.nstrips;
@@ -164,10 +167,10 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     gu.wp = lds_ptr<const uint4>(ptab, 2); gu.norm_w = lds_ptr<const bf16_t>(ptab, 5);
     uint4 g1[2], g2[2];  // norm1's and norm2's weights, the rotary pair: each prefetch writes its own
     uint2 r1, r_unused;
-    gemm_prefetch<2, 12, E_SWIGLU, 6>(gu, pre, 1, g2, r_unused);
+    gemm_prefetch<2, 12, E_SWIGLU, 6>(gu, pre, B, g2, r_unused);
     prj.wp = lds_ptr<const uint4>(ptab, 1);
-    gemm_prefetch<4, 6, E_RESID, 18>(prj, pre, 1, g2, r_unused);
-    gemm_prefetch<4, 6, E_ROPE>(qkv, pre, 1, g1, r1);
+    gemm_prefetch<4, 6, E_RESID, 18>(prj, pre, B, g2, r_unused);
+    gemm_prefetch<4, 6, E_ROPE>(qkv, pre, B, g1, r1);
     char* wl = reinterpret_cast<char*>(((uintptr_t)(ptab + m.n_layers * 8) + 255) & ~(uintptr_t)255);  // 4 x OHARA_LDS_PF KB
     dn.wlds_addr = (uint32_t)(uintptr_t)(OHARA_LDS char*)wl;
     pf.stamp();
@@ -206,32 +209,33 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
       const bool more = l + 1 < m.n_layers;
       // the first K/V tile of this workgroup's attention chunk (the attention workgroups have no q/k/v strip: nothing
       // of theirs is polled for until q is)
-      if (has_attn) attn_prefetch<D>(1, Hkv, m.t_max, a.ns, kc, vc, L, apre);
+      if (has_attn) attn_prefetch<D>(B, Hkv, m.t_max, a.ns, kc, vc, L, apre);
       // P1: [embedding | poll for the stream] + norm1 + QKV + rotary + append; q and the new k / v rows are left tagged
-      qkv.kc = kc; qkv.vc = vc; qkv.out = nullptr; qkv.tout = qt; qkv.tkv = kvt;
+      qkv.kc = kc; qkv.vc = vc; qkv.out = nullptr; qkv.tout = qt; qkv.tkv = kvt; qkv.trow = a.tg_rq; qkv.tkv_row = a.tg_rkv;
       if (has_qkv) {
-        if (l == 0) stage_norm<2, true, true, false>(xs, ldxs, a.xm, 0, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, 1, d, g1);
-        else stage_norm_tagged<2>(xs, xn_prev, pc, m.eps, d, g1);
+        if (l == 0) stage_norm<2, true, true, false>(xs, ldxs, a.xm, 0, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d, g1);
+        else stage_norm_tagged<2>(xs, xn_prev, pc, m.eps, d, g1, B, ldxs, a.tg_rx);
       }
       __syncthreads();
       pf.stamp();  // 1: row polled for + norm1 in LDS
       pre.r = r1;
-      gemm_phase<4, 6, E_ROPE, ProfT<PROFILE>, 0, true>(qkv, pre, xs, ldxs, 1, red, best_v, best_i, pf);  // 2 stamps
+      gemm_phase<4, 6, E_ROPE, ProfT<PROFILE>, 0, true>(qkv, pre, xs, ldxs, B, red, best_v, best_i, pf);  // 2 stamps
       pf.stamp();  // 4: rotary epilogue, tagged stores issued
       // P2: attention partials (polls for q; the chunk that holds the new position polls for its k / v rows); each chunk
       // leaves the launch's tag behind its (max, sum) pair
-      attn_phase<D, G, true>(1, H, Hkv, m.t_max, a.blk_x, a.ns, apre, nullptr, p_l, kc, vc, L, att, qt, kvt, pc, true);
+      attn_phase<D, G, true>(B, H, Hkv, m.t_max, a.blk_x, a.ns, apre, nullptr, p_l, kc, vc, L, att, qt, kvt, pc, true, a.tg_rq,
+                             a.tg_rkv);
       pf.stamp();  // 5: partials stored, flag raised
       // the next layer's q/k/v weights (+ norm1's, the rotary pair): their registers are free again (behind the attention
       // phase, which needs many: a workgroup without a chunk - at the usual sizes those with q/k/v strips - is here at once)
       if (has_qkv && more) {
         qkv.wp = lds_ptr<const uint4>(pl, 8);
         qkv.norm_w = lds_ptr<const bf16_t>(pl, 12);
-        gemm_prefetch<4, 6, E_ROPE, 0, false>(qkv, pre, 1, g1, r1);  // (the rotary pair is the same in every layer)
+        gemm_prefetch<4, 6, E_ROPE, 0, false>(qkv, pre, B, g1, r1);  // (the rotary pair is the same in every layer)
       }
       if (has_qkv) lm_stage();  // (the next thing a q/k/v workgroup polls for is a phase or more away)
       // the down projection's weights (98 KB a workgroup) into LDS: on their way from here, used after P4
-      dn.wp = lds_ptr<const uint4>(pl, 3); dn.tout = xn; dn.tresid = xt;
+      dn.wp = lds_ptr<const uint4>(pl, 3); dn.tout = xn; dn.tresid = xt; dn.trow = dn.tres_row = a.tg_rx;
       if (has_dn) {
         // (not before the chunk's flag has reached memory: behind the other waves' 72 KB of requests it was seen 1.5 us late)
         if (has_attn) {
@@ -242,39 +246,39 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
       }
       pf.stamp();  // 6: requests issued
       // P3: polls for every chunk's tag; merge + output projection + residual
-      prj.tout = xt; prj.tresid = l > 0 ? xn_prev : nullptr; prj.resid_embed = l == 0;
-      if ((int)blockIdx.x < prj.nstrips) stage_attn_merge_any<false, true>(a.ns, xs, ldxs, p_l, 1, H, D, mrg_w, mrg_l, pc);
+      prj.tout = xt; prj.tresid = l > 0 ? xn_prev : nullptr; prj.resid_embed = l == 0; prj.trow = prj.tres_row = a.tg_rx;
+      if ((int)blockIdx.x < prj.nstrips) stage_attn_merge_any<!ONE, true>(a.ns, xs, ldxs, p_l, B, H, D, mrg_w, mrg_l, pc);
       __syncthreads();
       pf.stamp();  // 7: merge in LDS
-      gemm_phase<4, 6, E_RESID, ProfT<PROFILE>, 18, true>(prj, pre, xs, ldxs, 1, red, best_v, best_i, pf);  // 2 stamps
+      gemm_phase<4, 6, E_RESID, ProfT<PROFILE>, 18, true>(prj, pre, xs, ldxs, B, red, best_v, best_i, pf);  // 2 stamps
       pf.stamp();  // 10: residual epilogue
       // P4: polls for the stream, norm2 + gate/up + SwiGLU; the activations are left tagged
-      gu.out = nullptr; gu.tout = at;
-      if (phase_block(gu) * 2 < gu.nstrips) stage_norm_tagged<2>(xs, xt, pc, m.eps, d, g2);
+      gu.out = nullptr; gu.tout = at; gu.trow = a.tg_ra;
+      if (phase_block(gu) * 2 < gu.nstrips) stage_norm_tagged<2>(xs, xt, pc, m.eps, d, g2, B, ldxs, a.tg_rx);
       __syncthreads();
       pf.stamp();  // 11: stream polled for + norm2 in LDS
-      gemm_phase<2, 12, E_SWIGLU, ProfT<PROFILE>, 6, true>(gu, pre, xs, ldxs, 1, red, best_v, best_i, pf);  // 2 stamps
+      gemm_phase<2, 12, E_SWIGLU, ProfT<PROFILE>, 6, true>(gu, pre, xs, ldxs, B, red, best_v, best_i, pf);  // 2 stamps
       // What the next layer needs of this workgroup besides q/k/v is requested now, a phase and a half before its use:
       // output projection and gate/up weights (+ norm2's); after the last layer, the vocabulary projection's first tiles.
       // (the workgroups of the down projection do this after it: the wait for their LDS tiles would wait for these too)
       auto next_weights = [&]() {
         if (more) {
           gu.wp = lds_ptr<const uint4>(pl, 10); gu.norm_w = lds_ptr<const bf16_t>(pl, 13);
-          gemm_prefetch<2, 12, E_SWIGLU, 6>(gu, pre, 1, g2, r_unused);
+          gemm_prefetch<2, 12, E_SWIGLU, 6>(gu, pre, B, g2, r_unused);
           prj.wp = lds_ptr<const uint4>(pl, 9);
-          gemm_prefetch<4, 6, E_RESID, 18>(prj, pre, 1, g2, r_unused);
+          gemm_prefetch<4, 6, E_RESID, 18>(prj, pre, B, g2, r_unused);
         } else {
-          gemm_prefetch<1, 24, E_LOGITS>(lm, pre, 1);  // (+ the final norm's weights)
+          gemm_prefetch<1, 24, E_LOGITS>(lm, pre, B);  // (+ the final norm's weights)
         }
       };
       pf.stamp();  // SwiGLU epilogue
       if (!has_dn) next_weights();
       pf.stamp();  // next layer's weights requested
       // P5: polls for the activations, down projection + residual; the stream is left tagged
-      if (has_dn) stage_act_tagged(xs, at, pc, 0, F);
+      if (has_dn) stage_act_tagged(xs, at, pc, 0, F, B, ldxs, a.tg_ra);
       __syncthreads();
       pf.stamp();  // 15: activations polled for, in LDS
-      gemm_phase<4, 12, E_XNEXT, ProfT<PROFILE>, 0, true>(dn, pre, xs, ldxs, 1, red, best_v, best_i, pf);  // 2 stamps
+      gemm_phase<4, 12, E_XNEXT, ProfT<PROFILE>, 0, true>(dn, pre, xs, ldxs, B, red, best_v, best_i, pf);  // 2 stamps
       pf.stamp();  // x_next stored
       if (has_dn) next_weights();
       if (!has_qkv) lm_stage();
@@ -282,13 +286,13 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     }
     // final norm + vocabulary projection: the stream of the last layer is polled for like any other
     pf.stamp();
-    stage_norm_tagged<2>(xs, tgs + (size_t)(m.n_layers - 1) * a.tg_stride + a.tg_n, pc, m.eps, d, pre.g);
+    stage_norm_tagged<2>(xs, tgs + (size_t)(m.n_layers - 1) * a.tg_stride + a.tg_n, pc, m.eps, d, pre.g, B, ldxs, a.tg_rx);
     __syncthreads();
     pf.stamp();
     pf.stamp();
    }
   }
-  if constexpr (!ONE) {
+  if constexpr (!POLLED) {
   gemm_prefetch<4, 6, E_ROPE>(qkv, pre, B);
   pf.stamp();
   for (int l = 0; l < m.n_layers; ++l) {
@@ -327,7 +331,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     pf.stamp();
     // P3: merge + output projection + residual
     if ((int)blockIdx.x < prj.nstrips) {
-      stage_attn_merge_any<!ONE>(a.ns, xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
+      stage_attn_merge_any<true>(a.ns, xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
     }
     __syncthreads();
     pf.stamp();
@@ -448,7 +452,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     }
   }
   pf.stamp();
-  if constexpr (ONE) {
+  if constexpr (POLLED) {
     // bookkeeping by the last workgroup out (the batch-1 layers have no barrier that everyone has passed, and without the
     // selection there is none at all): nobody reads these again in this launch
     if (threadIdx.x == 0) {
@@ -484,7 +488,7 @@ size_t mega_al(size_t v) { return (v + 255) & ~(size_t)255; }
 struct MegaLayout {
   size_t layers, kptr, vptr, xm, qm, am, pm, dm, candv, candi, prof, bar, tg, total;
   size_t xm_stride, qm_stride, am_stride, pm_stride, dm_stride, tg_stride, tg_set;
-  int blk_x, blk_a, tg_n, tg_q, tg_kv, tg_a;
+  int blk_x, blk_a, tg_n, tg_q, tg_kv, tg_a, tg_rx, tg_rq, tg_rkv, tg_ra;
 };
 
 MegaLayout mega_layout(const OharaModel* m, int B, int nwg) {
@@ -513,11 +517,16 @@ MegaLayout mega_layout(const OharaModel* m, int B, int nwg) {
   // behind the barrier words, cleared with them: the attention partials (batch 1: a tag follows each (max, sum) pair);
   // then the two sets of polled mailboxes (batch 1), filled with 0xFF ("not written yet")
   L.pm = o; o += L.pm_stride * sizeof(float) * NL;
-  L.tg_n = (int)mega_al((size_t)m->d_model * 2);
+  L.tg_rx = (int)mega_al((size_t)m->d_model * 2);
+  L.tg_rq = (int)mega_al((size_t)m->n_heads * D * 2);
+  L.tg_rkv = (int)mega_al((size_t)2 * m->n_kv_heads * D * 2);
+  L.tg_ra = (int)mega_al((size_t)((m->d_ff + 7) / 8 * 8) * 2);
+  const int PB = B <= 8 ? B : 1;  // (the polled builds serve up to eight sequences)
+  L.tg_n = PB * L.tg_rx;
   L.tg_q = 2 * L.tg_n;
-  L.tg_kv = L.tg_q + (int)mega_al((size_t)m->n_heads * D * 2);
-  L.tg_a = L.tg_kv + (int)mega_al((size_t)2 * m->n_kv_heads * D * 2);
-  L.tg_stride = L.tg_a + mega_al((size_t)((m->d_ff + 7) / 8 * 8) * 2);
+  L.tg_kv = L.tg_q + PB * L.tg_rq;
+  L.tg_a = L.tg_kv + PB * L.tg_rkv;
+  L.tg_stride = L.tg_a + (size_t)PB * L.tg_ra;
   L.tg_set = L.tg_stride * NL;
   L.tg = o; o += 2 * L.tg_set;
   L.total = o;
@@ -574,6 +583,7 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   a.cand_idx = reinterpret_cast<int*>(ws + L.candi);
   a.bar = reinterpret_cast<unsigned int*>(ws + L.bar);
   a.tg = ws + L.tg; a.tg_stride = L.tg_stride; a.tg_set = L.tg_set; a.tg_n = L.tg_n; a.tg_q = L.tg_q; a.tg_kv = L.tg_kv; a.tg_a = L.tg_a;
+  a.tg_rx = L.tg_rx; a.tg_rq = L.tg_rq; a.tg_rkv = L.tg_rkv; a.tg_ra = L.tg_ra;
   if (init_workspace) {
     // small synchronous copies: done once per (model, cache) binding, outside any capture
     if (hipMemcpyAsync((void*)a.layers_dev, m->layers, sizeof(OharaLayer) * m->n_layers, hipMemcpyHostToDevice, st) !=
@@ -609,11 +619,14 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   if (!(2 * ns >= 3 * p2 && attn_merge_width(ns) <= 8)) ns = p2;
   a.ns = ns;
   const size_t mrg = (size_t)2 * ((s->batch * m->n_heads * attn_merge_width(ns) + 1) & ~1) * sizeof(float);
-  // the batch-1 build parks the down projection's tiles in LDS (4 waves x OHARA_LDS_PF KB)
+  // The polled builds (batch 1; up to eight sequences) park the down projection's tiles in LDS (4 waves x
+  // OHARA_LDS_PF KB) and want gate/up, the output projection and the down projection on workgroups of their own.
   const int n_dn = (m->d_model + 15) / 16, n_gu = (2 * ((m->d_ff + 7) / 8 * 8) / 16 + 1) / 2;
-  const bool one = s->batch == 1 && n_gu + n_dn <= n_workgroups && 2 * n_dn <= n_workgroups;
-  const size_t smem = xs_bytes + 4096 + (size_t)(8 + 4 * D) * G * sizeof(float) + mrg + (size_t)m->n_layers * 64 +
-                      (one ? 256 + (size_t)4 * OHARA_LDS_PF * 1024 : 0);
+  const size_t smem0 = xs_bytes + 4096 + (size_t)(8 + 4 * D) * G * sizeof(float) + mrg + (size_t)m->n_layers * 64;
+  const size_t smem_polled = smem0 + 256 + (size_t)4 * OHARA_LDS_PF * 1024;
+  const bool roles = n_gu + n_dn <= n_workgroups && 2 * n_dn <= n_workgroups;
+  const int mode = !roles ? 0 : (s->batch == 1 ? 1 : (s->batch <= 8 && smem_polled <= 160 * 1024 ? 2 : 0));
+  const size_t smem = mode ? smem_polled : smem0;
   if (smem > 160 * 1024) return OHARA_ESIZE;
   dim3 grid(n_workgroups), block(256);
 #define OHARA_MEGA_B(DD, GG, ONE_)                                                                          \
@@ -628,8 +641,9 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   } while (0)
 #define OHARA_MEGA(DD, GG)                                                                                  \
   do {                                                                                                      \
-    if (one) OHARA_MEGA_B(DD, GG, true);                                                                    \
-    else OHARA_MEGA_B(DD, GG, false);                                                                       \
+    if (mode == 1) OHARA_MEGA_B(DD, GG, 1);                                                                 \
+    else if (mode == 2) OHARA_MEGA_B(DD, GG, 2);                                                            \
+    else OHARA_MEGA_B(DD, GG, 0);                                                                           \
   } while (0)
 #define OHARA_MEGA_PROF(ONE_)                                                                               \
   do {                                                                                                      \
@@ -641,10 +655,10 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
       return OHARA_ESIZE;                                                                                   \
     hipLaunchKernelGGL((decode_mega_kernel<128, 1, ONE_, true>), grid, block, smem, st, a);                 \
   } while (0)
-  // (`one`: the batch-1 build wants every phase's units on their own stretch of the grid)
-  if (a.prof && D == 128 && G == 1) {  // the stamps exist in these two instantiations only
-    if (one) OHARA_MEGA_PROF(true);
-    else OHARA_MEGA_PROF(false);
+  if (a.prof && D == 128 && G == 1) {  // the stamps exist in these three instantiations only
+    if (mode == 1) OHARA_MEGA_PROF(1);
+    else if (mode == 2) OHARA_MEGA_PROF(2);
+    else OHARA_MEGA_PROF(0);
   } else if (D == 128 && G == 1) OHARA_MEGA(128, 1);
   else if (D == 128 && G == 2) OHARA_MEGA(128, 2);
   else if (D == 128 && G == 4) OHARA_MEGA(128, 4);

@@ -400,63 +400,138 @@ __device__ __forceinline__ void stage_act(bf16_t* xs, int ldxs, const char* src,
 // polled for instead of fetched after a barrier.  The norm weights were fetched ahead (gpre).
 template <int NLD>
 __device__ __forceinline__ void stage_norm_tagged(bf16_t* xs, const char* xt, const Poll& pc, float eps, int K,
-                                                  const uint4 (&gpre)[NLD]) {
-  const int tid = threadIdx.x, lane = tid & 63;
-  if (tid >= 64) return;
-  uint4 v[NLD];
+                                                  const uint4 (&gpre)[NLD], int B = 1, int ldxs = 0, int row_bytes = 0) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // one wave per row, rows wave and wave + 4 together (up to eight sequences): both are polled for in the same rounds
+  if (wave >= B) return;
+  if (B == 1) {  // a single sequence, spelled out (the general form below costs it 0.1 - 0.2 us per call)
+    uint4 v[NLD];
+    unsigned int spins = 0;
+    const MbRsrc rs = mb_rsrc(xt);
+    for (;;) {
+      bool ok = true;
+#pragma unroll
+      for (int c = 0; c < NLD; ++c) {
+        const int k = (c * 64 + lane) * 8;
+        ok = mb_ld16(rs, k < K ? k : 0, v[c]) && ok;
+      }
+      if (__all(ok) || poll_expired(pc, spins)) break;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < NLD; ++c) {
+      if ((c * 64 + lane) * 8 >= K) v[c] = make_uint4(0, 0, 0, 0);
+      const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float a0 = lo_bf(w[i]), a1 = hi_bf(w[i]);
+        ss += a0 * a0 + a1 * a1;
+      }
+    }
+    ss = wave_sum(ss);
+    const float rinv = 1.0f / sqrtf(ss / (float)K + eps);
+#pragma unroll
+    for (int c = 0; c < NLD; ++c) {
+      const int k = (c * 64 + lane) * 8;
+      if (k < K) {
+        const uint32_t xv[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+        const uint32_t gv[4] = {gpre[c].x, gpre[c].y, gpre[c].z, gpre[c].w};
+        uint32_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          o[i] = pack_bf(rbf(lo_bf(xv[i]) * rinv) * lo_bf(gv[i]), rbf(hi_bf(xv[i]) * rinv) * hi_bf(gv[i]));
+        sts16(xs + k, make_uint4(o[0], o[1], o[2], o[3]));
+      }
+    }
+    return;
+  }
+  const bool two = wave + 4 < B;
+  uint4 v[2][NLD];
   unsigned int spins = 0;
-  const MbRsrc rs = mb_rsrc(xt);
+  const MbRsrc rs0 = mb_rsrc(xt + (size_t)wave * row_bytes);
+  const MbRsrc rs1 = mb_rsrc(xt + (size_t)(two ? wave + 4 : wave) * row_bytes);
   // every round fetches the whole row (1.5 KB at K = 768) and looks at every word
   for (;;) {
     bool ok = true;
 #pragma unroll
     for (int c = 0; c < NLD; ++c) {
       const int k = (c * 64 + lane) * 8;
-      ok = mb_ld16(rs, k < K ? k : 0, v[c]) && ok;
+      ok = mb_ld16(rs0, k < K ? k : 0, v[0][c]) && ok;
+    }
+    if (two) {
+#pragma unroll
+      for (int c = 0; c < NLD; ++c) {
+        const int k = (c * 64 + lane) * 8;
+        ok = mb_ld16(rs1, k < K ? k : 0, v[1][c]) && ok;
+      }
     }
     if (__all(ok) || poll_expired(pc, spins)) break;
   }
-  float ss = 0.f;
+  for (int r = 0; r < (two ? 2 : 1); ++r) {
+    const int b = wave + 4 * r;
+    float ss = 0.f;
 #pragma unroll
-  for (int c = 0; c < NLD; ++c) {
-    if ((c * 64 + lane) * 8 >= K) v[c] = make_uint4(0, 0, 0, 0);
-    const uint32_t w[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
+    for (int c = 0; c < NLD; ++c) {
+      if ((c * 64 + lane) * 8 >= K) v[r][c] = make_uint4(0, 0, 0, 0);
+      const uint32_t w[4] = {v[r][c].x, v[r][c].y, v[r][c].z, v[r][c].w};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float a0 = lo_bf(w[i]), a1 = hi_bf(w[i]);
-      ss += a0 * a0 + a1 * a1;
+      for (int i = 0; i < 4; ++i) {
+        const float a0 = lo_bf(w[i]), a1 = hi_bf(w[i]);
+        ss += a0 * a0 + a1 * a1;
+      }
     }
-  }
-  ss = wave_sum(ss);
-  const float rinv = 1.0f / sqrtf(ss / (float)K + eps);
+    ss = wave_sum(ss);
+    const float rinv = 1.0f / sqrtf(ss / (float)K + eps);
 #pragma unroll
-  for (int c = 0; c < NLD; ++c) {
-    const int k = (c * 64 + lane) * 8;
-    if (k < K) {
-      const uint32_t xv[4] = {v[c].x, v[c].y, v[c].z, v[c].w};
-      const uint32_t gv[4] = {gpre[c].x, gpre[c].y, gpre[c].z, gpre[c].w};
-      uint32_t o[4];
+    for (int c = 0; c < NLD; ++c) {
+      const int k = (c * 64 + lane) * 8;
+      if (k < K) {
+        const uint32_t xv[4] = {v[r][c].x, v[r][c].y, v[r][c].z, v[r][c].w};
+        const uint32_t gv[4] = {gpre[c].x, gpre[c].y, gpre[c].z, gpre[c].w};
+        uint32_t o[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        o[i] = pack_bf(rbf(lo_bf(xv[i]) * rinv) * lo_bf(gv[i]), rbf(hi_bf(xv[i]) * rinv) * hi_bf(gv[i]));
-      sts16(xs + k, make_uint4(o[0], o[1], o[2], o[3]));
+        for (int i = 0; i < 4; ++i)
+          o[i] = pack_bf(rbf(lo_bf(xv[i]) * rinv) * lo_bf(gv[i]), rbf(hi_bf(xv[i]) * rinv) * hi_bf(gv[i]));
+        sts16(xs + (size_t)b * ldxs + k, make_uint4(o[0], o[1], o[2], o[3]));
+      }
     }
   }
 }
 
-// Columns [f0, f1) (multiples of 8) of the polled act mailbox (batch 1) -> LDS
-__device__ __forceinline__ void stage_act_tagged(bf16_t* xs, const char* at, const Poll& pc, int f0, int f1) {
-  const int n8 = (f1 - f0) >> 3;
+// Columns [f0, f1) (multiples of 8) of the polled act mailbox -> LDS.  Pieces of 8 columns, all rows in one
+// index space; a thread polls FLY of its pieces in the same rounds, without a test per piece (past the end:
+// the last piece again, not stored).  One row after the other, each with rounds of its own, was 6.7 us for
+// eight rows of 3072; a test per piece made every load wait for the one before.
+template <int FLY>
+__device__ __forceinline__ void stage_act_fly(bf16_t* xs, const char* at, const Poll& pc, int f0, int n8, int total, int ldxs,
+                                              int row_bytes) {
   const MbRsrc rs = mb_rsrc(at);
-  for (int i = threadIdx.x; i < n8; i += blockDim.x) {
-    const int c = (f0 >> 3) + i;
-    uint4 v;
-    unsigned int spins = 0;
-    while (!mb_ld16(rs, c * 8, v)) {
-      if (poll_expired(pc, spins)) break;
+  for (int i0 = threadIdx.x; i0 < total; i0 += (int)blockDim.x * FLY) {
+    uint4 v[FLY];
+    int col[FLY], row[FLY];
+#pragma unroll
+    for (int j = 0; j < FLY; ++j) {
+      const int i = min(i0 + j * (int)blockDim.x, total - 1);
+      row[j] = i / n8;
+      col[j] = ((f0 >> 3) + (i - row[j] * n8)) * 8;
     }
-    sts16(xs + c * 8, v);
+    unsigned int spins = 0;
+    for (;;) {
+      bool ok = true;
+#pragma unroll
+      for (int j = 0; j < FLY; ++j) ok = mb_ld16(rs, row[j] * (row_bytes >> 1) + col[j], v[j]) && ok;
+      if (ok || poll_expired(pc, spins)) break;
+    }
+#pragma unroll
+    for (int j = 0; j < FLY; ++j)
+      if (i0 + j * (int)blockDim.x < total) sts16(xs + (size_t)row[j] * ldxs + col[j], v[j]);
   }
+}
+__device__ __forceinline__ void stage_act_tagged(bf16_t* xs, const char* at, const Poll& pc, int f0, int f1, int B = 1,
+                                                 int ldxs = 0, int row_bytes = 0) {
+  const int n8 = (f1 - f0) >> 3, total = B * n8;
+  if (total <= 2 * (int)blockDim.x) stage_act_fly<2>(xs, at, pc, f0, n8, total, ldxs, row_bytes);
+  else stage_act_fly<6>(xs, at, pc, f0, n8, total, ldxs, row_bytes);
 }
 
 // Merge of the attention partials of all chunks, in chunk order (llama.py:116-123 output,
@@ -671,6 +746,7 @@ struct GemmP {
   uint32_t wlds_addr;  // E_XNEXT: LDS byte address of the workgroup's parked tiles, OHARA_LDS_PF per wave (gemm_prefetch_lds)
   Poll poll;
   ptrdiff_t tother;  // from a mailbox of this launch's set to the same mailbox of the other set
+  int trow, tkv_row, tres_row;  // bytes between the rows (sequences) of the mailboxes tout, tkv and tresid
   int wg0;         // the workgroup that takes the phase's first unit (units go to wg0, wg0 + 1, ... round the grid)
 };
 // A workgroup's position in a phase whose units start at workgroup p.wg0.
@@ -834,7 +910,7 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
     const bool tres = TAG && (EPI == E_XNEXT || (EPI == E_RESID && !p.resid_embed)) && live && kpart == 0 && mine &&
                       strip * 16 + 4 * g < p.N;
     uint2 rx = make_uint2(0, 0);
-    if (tres) rx = ld_coh8(p.tresid + (size_t)(strip * 16 + 4 * g) * 2);
+    if (tres) rx = ld_coh8(p.tresid + (size_t)(B == 1 ? 0 : m) * p.tres_row + (size_t)(strip * 16 + 4 * g) * 2);
     if (live) {
       const uint4* wrow = p.wp + (size_t)strip * KS * 64 + lane;
 #pragma unroll 1
@@ -916,7 +992,7 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
     }
     if (it == 0) pf.stamp();  // cross-wave sum done
     if (live && kpart == 0 && mine) {
-      const int b = m;
+      const int b = B == 1 ? 0 : m;  // (a single sequence: the row offsets below fold away)
       const int r0 = strip * 16 + 4 * g;
       const float y0 = rbf(acc[0]), y1 = rbf(acc[1]), y2 = rbf(acc[2]), y3 = rbf(acc[3]);
       if (EPI == E_XNEXT || (TAG && EPI == E_RESID)) {  // batch 1: the row goes to the tagged mailbox only
@@ -926,7 +1002,7 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
             unsigned int spins = 0;
             while (rx.x == OHARA_UNWRITTEN || rx.y == OHARA_UNWRITTEN) {
               if (poll_expired(p.poll, spins)) break;
-              rx = ld_coh8(p.tresid + (size_t)r0 * 2);
+              rx = ld_coh8(p.tresid + (size_t)b * p.tres_row + (size_t)r0 * 2);
             }
             r = rx;
           } else {  // the first half layer: the embedding row (llama.py:310)
@@ -934,7 +1010,8 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
             if (id < 0 || id >= p.vocab) id = 0;
             r = ldg8(p.table + (size_t)id * p.N + r0);
           }
-          mb_st8(p.tout, p.tother, r0, pack_bf(lo_bf(r.x) + y0, hi_bf(r.x) + y1), pack_bf(lo_bf(r.y) + y2, hi_bf(r.y) + y3));
+          mb_st8(p.tout + (size_t)b * p.trow, p.tother, r0, pack_bf(lo_bf(r.x) + y0, hi_bf(r.x) + y1),
+                 pack_bf(lo_bf(r.y) + y2, hi_bf(r.y) + y3));
         }
       } else if (EPI == E_RESID) {  // N % 4 == 0 is required by the entry point
         if (r0 < p.N) {
@@ -990,7 +1067,7 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
         const int f = strip * 8 + 2 * g;
         if (f < p.N) {
           const float s0 = rbf(silu_f(y0)), s1 = rbf(silu_f(y1));
-          if (TAG) mb_st4(p.tout, p.tother, f, pack_bf(s0 * y2, s1 * y3));
+          if (TAG) mb_st4(p.tout + (size_t)b * p.trow, p.tother, f, pack_bf(s0 * y2, s1 * y3));
           else st_coh4(const_cast<char*>(am_addr(p.out, p.blk, b, f)), pack_bf(s0 * y2, s1 * y3));
         }
       } else {  // E_ROPE
@@ -1016,8 +1093,8 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
           }
           const uint2 ro = make_uint2(pack_bf(v[0], v[1]), pack_bf(v[2], v[3]));
           if (TAG) {  // attention polls for the q row and for the new key / value rows; the cache rows are for later steps
-            if (r0 < nq) mb_st8(p.tout, p.tother, r0, ro.x, ro.y);
-            else mb_st8(p.tkv, p.tother, r0 - nq, ro.x, ro.y);
+            if (r0 < nq) mb_st8(p.tout + (size_t)b * p.trow, p.tother, r0, ro.x, ro.y);
+            else mb_st8(p.tkv + (size_t)b * p.tkv_row, p.tother, r0 - nq, ro.x, ro.y);
           }
           if (!TAG || r0 >= nq) st_coh8(o, ro);
         }
@@ -1268,7 +1345,8 @@ template <int D, int G, bool TAG = false>
 __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int blk_x, int ns, const AttnPre<D>& pre,
                                            const char* qm, float* pm, const bf16_t* kc, const bf16_t* vc, int L,
                                            float* lds, const char* qt = nullptr, const char* kvt = nullptr,
-                                           const Poll pc = Poll{0, 0, nullptr}, bool announce = false) {
+                                           const Poll pc = Poll{0, 0, nullptr}, bool announce = false, int q_row = 0,
+                                           int kv_row = 0) {  // q_row, kv_row: bytes between the sequences' rows of qt, kvt
   constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int p = lane & 15;
@@ -1285,6 +1363,7 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
   for (int item = blockIdx.x; item < nitems; item += gridDim.x) {
     int b, kvh, split, t0, t1;
     attn_item_range(item, ns, Hkv, L, b, kvh, split, t0, t1);
+    if (B == 1) b = 0;  // (a single sequence: the row offsets below fold away)
     const bf16_t* kb = kc + (size_t)b * Tmax * row + (size_t)kvh * D;
     const bf16_t* vb = vc + (size_t)b * Tmax * row + (size_t)kvh * D;
     float m_run[G], l_run[G], acc[G][8];
@@ -1313,7 +1392,7 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
       }
       if (TAG) {
         unsigned int spins = 0;
-        const MbRsrc qrs = mb_rsrc(qt);
+        const MbRsrc qrs = mb_rsrc(qt + (size_t)b * q_row);
         for (;;) {  // (every round fetches the group's q rows whole: lanes share addresses, 256 bytes a row)
           bool ok = true;
 #pragma unroll
@@ -1323,7 +1402,8 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
               ok = mb_ld16(qrs, (kvh * G + hh) * D + (4 * c + dq) * 8, qv[hh][c]) && ok;
           if (__all(ok) || poll_expired(pc, spins)) break;
         }
-        if (!use_pre && L - 1 >= tb && L - 1 < tb + 16) attn_new_row_tagged<D>(kvt, pc, Hkv, kvh, tb, t1, L - 1, ka, va);
+        if (!use_pre && L - 1 >= tb && L - 1 < tb + 16)
+          attn_new_row_tagged<D>(kvt + (size_t)b * kv_row, pc, Hkv, kvh, tb, t1, L - 1, ka, va);
       } else {
 #pragma unroll
         for (int hh = 0; hh < G; ++hh)
@@ -1405,7 +1485,8 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
       // and is copied over, which costs a wait but far fewer registers than two sets taking turns)
       for (; tb + 64 < t1; tb += 64) {
         attn_tile_load_u<D>(kb, vb, row, tb + 64, t1, coh, kn, vn, last);
-        if (TAG && L - 1 >= tb + 64 && L - 1 < tb + 80) attn_new_row_tagged<D>(kvt, pc, Hkv, kvh, tb + 64, t1, L - 1, kn, vn);
+        if (TAG && L - 1 >= tb + 64 && L - 1 < tb + 80)
+          attn_new_row_tagged<D>(kvt + (size_t)b * kv_row, pc, Hkv, kvh, tb + 64, t1, L - 1, kn, vn);
         consume(tb, ka, va);
 #pragma unroll
         for (int c = 0; c < NC; ++c) ka[c] = kn[c];
