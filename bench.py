@@ -29,10 +29,10 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the persistent decode kernel at batch 1, prompt 1024, from two
 # rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same
-# counter reads for a 1 GiB copy (--pmc-calibration): 376.0 MB read + 1.3 MB written.  Counters
+# counter reads for a 1 GiB copy (--pmc-calibration): 375.6 MB read + 1.3 MB written.  Counters
 # cannot be read from inside this process, so the figure is carried here; the runs and the
 # arithmetic are in profiles/decode_mega_kernel_d12_batch1_pmc.txt.
-PMC_TRAFFIC_BYTES = {("persistent", 1, 1024): 377.3e6}
+PMC_TRAFFIC_BYTES = {("persistent", 1, 1024): 377.0e6}
 
 D12 = dict(vocab_size=65536, hidden_size=768, intermediate_size=3072, num_attention_heads=6,
            num_key_value_heads=0, num_hidden_layers=12, max_sequence_length=4096, dropout=0.0)
@@ -798,7 +798,7 @@ def main():
             sess2.check_error()
             if sess2.persistent:
                 kb = step_bytes(cfg, 1, args.prompt + args.warmup + (n_prof + 1) / 2.0)
-                kname = "decode_mega_kernel<128,1,true,false> (batch-1 build; whole decode step: 12 layers + vocabulary projection + selection)"
+                kname = "decode_mega_kernel<128,1,1,false> (batch-1 polled build; whole decode step: 12 layers + vocabulary projection + selection)"
             else:
                 kb = lm_head_bytes(cfg, 1)
                 kname = "wide_kernel<1,true,STORE> (final norm + vocabulary projection 65536x768)"

@@ -402,7 +402,7 @@ int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* s, int seq_
  * whole step (all layers, vocabulary projection, greedy selection) runs in a single
  * kernel of `n_workgroups` resident workgroups (use the CU count; more than the device can
  * hold of this kernel at once returns OHARA_ESIZE) whose phases are separated by grid-wide barriers
- * (batch > 1) or hand their rows over through memory that the consumers poll (batch 1); it has no counterpart in the reference, whose decode step is
+ * (batch > 8) or hand their rows over through memory that the consumers poll (batch <= 8); it has no counterpart in the reference, whose decode step is
  * ~1000 eager launches (llama.py:279-323).  The cache position and step index are read
  * from / advanced in s->step_state; s->attn and s->attn_ws are not used.
  * `workspace`: ohara_persistent_workspace_bytes(m, batch, s->n_split, n_workgroups) of
@@ -411,7 +411,7 @@ int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* s, int seq_
  * the merge of the attention chunks never uses a chunk no workgroup wrote).  Call once with
  * init_workspace = 1 (copies the layer table and the cache pointers to the device, zeroes the
  * barrier words, the launch counters and the attention partials behind them and fills the
- * hand-off rows of the batch-1 kernel with 0xFF, their "not written yet"; synchronises the stream;
+ * hand-off rows of the polled builds (batch <= 8) with 0xFF, their "not written yet"; synchronises the stream;
  * do it outside graph capture) whenever the model or the caches change, and before the workspace
  * is used for the first time or after its memory has been used for anything else; then each call
  * with init_workspace = 0 enqueues one step.  Steps on one workspace must not overlap (each
