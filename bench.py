@@ -63,11 +63,14 @@ def d12_state(device, seed=0):
     return cfg, st
 
 
-def step_bytes(cfg, batch, length):
-    """Algorithmic HBM bytes of one decode step at cached length `length` (after append)."""
+def step_bytes(cfg, batch, length, int8=False):
+    """Algorithmic HBM bytes of one decode step at cached length `length` (after append); int8: the caches hold one
+    byte per value plus an fp32 (scale, minimum) pair per head row."""
     d, f, v, nl = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.num_hidden_layers
     params = nl * (4 * d * d + 3 * d * f) + v * d + (2 * nl + 1) * d
     kv_row = nl * 2 * d * 2
+    if int8:
+        kv_row = nl * 2 * (d + 8 * (cfg.num_key_value_heads or cfg.num_attention_heads))
     return 2 * params + batch * (kv_row * length + kv_row + 2 * d + 2 * v)
 
 
@@ -76,13 +79,14 @@ def lm_head_bytes(cfg, batch):
     return 2 * (v * d + d) + batch * 2 * (d + v)
 
 
-def time_decode(model, batch, prompt_len, warmup, steps, seed=0, persistent=None, sampling=None):
+def time_decode(model, batch, prompt_len, warmup, steps, seed=0, persistent=None, sampling=None, int8=False):
     g = torch.Generator().manual_seed(seed)
     prompt = torch.randint(0, model.config.vocab_size, (batch, prompt_len), generator=g).to(model.device)
     u = None
     if sampling is not None:  # one fixed, seeded tensor of uniform draws for the whole run
         u = torch.rand(warmup + steps + 8, batch, generator=g).to(model.device)
-    sess = model.session(batch, warmup + steps + 8, persistent=persistent, sampling=sampling, u=u)
+    sess = model.session(batch, warmup + steps + 8, persistent=persistent, sampling=sampling, u=u,
+                         kv_cache=model.build_kv_cache(batch, int8=True) if int8 else None)
     sess.prefill(prompt)
     sess.capture()
     sess.run(max(0, warmup - 1))
@@ -586,7 +590,7 @@ def _batch1_roles(cfg, nwg, batch=1):
             "gate/up": range(0, n_gu), "down": range(dn0, dn0 + n_dn)}
 
 
-def phase_timeline(dev, prompt_len, steps=32, batch=1):
+def phase_timeline(dev, prompt_len, steps=32, batch=1, int8=False):
     """The critical path of a layer of the batch-1 persistent kernel: for every hand-off, when the last
     workgroup of the producing role had issued its stores and when the last workgroup of the consuming
     role had the data staged, from the kernel's own clock samples (a 100 MHz counter common to all
@@ -595,7 +599,7 @@ def phase_timeline(dev, prompt_len, steps=32, batch=1):
 
     cfg, st = d12_state(dev)
     model = Llama(cfg, st, device=dev)
-    sess = model.session(batch, steps + 24, persistent=True)
+    sess = model.session(batch, steps + 24, persistent=True, kv_cache=model.build_kv_cache(batch, int8=True) if int8 else None)
     sess.prefill(torch.randint(0, cfg.vocab_size, (batch, prompt_len)).to(dev))
     for _ in range(8):
         sess.step()
@@ -713,6 +717,7 @@ def main():
                     help="also run three 1 GiB device-to-device copies (a kernel of known traffic to scale "
                          "FETCH_SIZE / WRITE_SIZE counters against)")
     ap.add_argument("--timeline-batch", type=int, default=1, help="sequences of the --phase-timeline run (1 to 8)")
+    ap.add_argument("--timeline-int8", action="store_true", help="the --phase-timeline run over an int8 KV cache")
     ap.add_argument("--phase-timeline", action="store_true",
                     help="print the per-phase timeline of the persistent decode kernel at batch 1 and exit")
     ap.add_argument("--bitnet-phase-timeline", type=int, default=0, metavar="B",
@@ -756,7 +761,7 @@ def main():
         print(json.dumps(bench_bitnet(dev, tuple(int(b) for b in args.bitnet_only.split(","))), indent=1))
         return
     if args.phase_timeline:
-        print(json.dumps(phase_timeline(dev, args.prompt, batch=args.timeline_batch), indent=1))
+        print(json.dumps(phase_timeline(dev, args.prompt, batch=args.timeline_batch, int8=args.timeline_int8), indent=1))
         return
     if args.pmc_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
@@ -798,7 +803,7 @@ def main():
             sess2.check_error()
             if sess2.persistent:
                 kb = step_bytes(cfg, 1, args.prompt + args.warmup + (n_prof + 1) / 2.0)
-                kname = "decode_mega_kernel<128,1,1,false> (batch-1 polled build; whole decode step: 12 layers + vocabulary projection + selection)"
+                kname = "decode_mega_kernel<128,1,1,false,false> (batch-1 polled build; whole decode step: 12 layers + vocabulary projection + selection)"
             else:
                 kb = lm_head_bytes(cfg, 1)
                 kname = "wide_kernel<1,true,STORE> (final norm + vocabulary projection 65536x768)"
@@ -822,6 +827,16 @@ def main():
                             "launch": "persistent kernel + sampler kernel per step"}
     del sess
     torch.cuda.empty_cache()
+    # the int8 KV cache (codes + a scale and a minimum per head row) through the same single launch
+    for b in (1, 8):
+        dt, l_mean, sess = time_decode(model, b, args.prompt, args.warmup, args.steps, int8=True)
+        by = step_bytes(cfg, b, l_mean, int8=True)
+        results[f"{b}_int8_cache"] = {
+            "tokens_per_s": round(b * args.steps / dt, 1), "ms_per_step": round(dt / args.steps * 1e3, 4),
+            "step_bytes": int(by), "step_frac_of_hbm_peak": round(by / (dt / args.steps) / 1e9 / HBM_PEAK_GBS, 4),
+            "launch": "one persistent kernel per step" if sess.persistent else "kernel chain"}
+        del sess
+        torch.cuda.empty_cache()
     r1 = results[1]
     out = {
         "metric": "decode tokens/s at batch 1 & 32 (d12 Llama, 4k ctx) + % of HBM roofline",

@@ -430,6 +430,12 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
  * are compiled into a separate build of the kernel that exists for head_dim 128 with
  * n_kv_heads == n_heads only, other shapes leave the slots untouched). */
 int64_t ohara_persistent_barrier_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
+/* Which build of the kernel a launch with this model, batch and grid runs: 0 the general one (a grid
+ * barrier between the phases), 1 and 2 the polled ones (one sequence; two to eight).  The polled builds
+ * also serve the int8 cache (s->kv_int8: the attention phase dequantises the tiles it reads and
+ * quantises the appended row as ohara_kv_quant_append_int8 does, ohara/modules/kv_cache.py:15-32);
+ * ohara_llama_decode_persistent returns OHARA_ESIZE for an int8 cache where this returns 0. */
+int ohara_persistent_polled(const OharaModel* m, int batch, int n_workgroups);
 int64_t ohara_persistent_error_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
 int64_t ohara_persistent_profile_offset(const OharaModel* m, int batch, int n_split, int n_workgroups);
 

@@ -107,6 +107,7 @@ _PROTOS = {
     "ohara_phi_attn_bf16": (_i, [_p, _i, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
     "ohara_persistent_workspace_bytes": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),
     "ohara_persistent_barrier_offset": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),
+    "ohara_persistent_polled": (_i, [C.POINTER(OharaModel), _i, _i]),
     "ohara_persistent_error_offset": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),
     "ohara_persistent_profile_offset": (_i64, [C.POINTER(OharaModel), _i, _i, _i]),
     "ohara_llama_decode_persistent": (_i, [C.POINTER(OharaModel), C.POINTER(OharaDecodeState), _p, _i, _i, _i,

@@ -129,19 +129,6 @@ __device__ bool last_chunk_done(int* counter, int nsplit) {
   return is_last != 0;
 }
 
-// (q + 128) * scale + min in fp32, rounded to bf16 (kv_cache.py:30-32, 116-118): four bytes -> two
-// packed bf16 pairs.  `w` already has 0x80 xor-ed in, i.e. holds q + 128 as unsigned bytes.  The
-// scales written by the quantiser are bf16 values (8 significant bits) and q + 128 has at most 8,
-// so the product is exact in fp32 and one fused multiply-add gives bit for bit what the separate
-// multiply and add of the reference give.
-__device__ __forceinline__ uint2 dequant4(uint32_t w, float s, float m) {
-  const float f0 = __fmaf_rn((float)(w & 0xffu), s, m);
-  const float f1 = __fmaf_rn((float)((w >> 8) & 0xffu), s, m);
-  const float f2 = __fmaf_rn((float)((w >> 16) & 0xffu), s, m);
-  const float f3 = __fmaf_rn((float)(w >> 24), s, m);
-  return make_uint2(pack_bf(f0, f1), pack_bf(f2, f3));
-}
-
 template <int D, int G>
 __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   constexpr int NC = D / 32;        // 16-byte K loads per lane per tile

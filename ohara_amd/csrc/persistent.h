@@ -228,6 +228,12 @@ __device__ __forceinline__ bool mb_ld16(MbRsrc r, int col, uint4& out) {
   return v.x != OHARA_UNWRITTEN && v.y != OHARA_UNWRITTEN && v.z != OHARA_UNWRITTEN && v.w != OHARA_UNWRITTEN;
 }
 
+// two values starting at column `col` (even); true when they have been written
+__device__ __forceinline__ bool mb_ld4(MbRsrc r, int col, uint32_t& out) {
+  out = __builtin_amdgcn_raw_buffer_load_b32(r, (uint32_t)col * 2u, 0, 16);
+  return out != OHARA_UNWRITTEN;
+}
+
 // Strip-blocked mailbox of a (B, N) bf16 matrix: the 16 columns [16s, 16s+16) of all rows
 // form block s of `blk` bytes (a multiple of 128), row b at byte b*32 inside it.
 __device__ __forceinline__ const char* xm_addr(const char* base, int blk, int b, int n) {
@@ -747,6 +753,7 @@ struct GemmP {
   Poll poll;
   ptrdiff_t tother;  // from a mailbox of this launch's set to the same mailbox of the other set
   int trow, tkv_row, tres_row;  // bytes between the rows (sequences) of the mailboxes tout, tkv and tresid
+  int kv_i8;       // E_ROPE with polled hand-offs: the caches hold int8 codes (the new rows travel by mailbox only)
   int wg0;         // the workgroup that takes the phase's first unit (units go to wg0, wg0 + 1, ... round the grid)
 };
 // A workgroup's position in a phase whose units start at workgroup p.wg0.
@@ -1096,7 +1103,7 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
             if (r0 < nq) mb_st8(p.tout + (size_t)b * p.trow, p.tother, r0, ro.x, ro.y);
             else mb_st8(p.tkv + (size_t)b * p.tkv_row, p.tother, r0 - nq, ro.x, ro.y);
           }
-          if (!TAG || r0 >= nq) st_coh8(o, ro);
+          if (!TAG || (r0 >= nq && !p.kv_i8)) st_coh8(o, ro);  // (an int8 cache gets the row from the attention phase)
         }
       }
     }
@@ -1339,14 +1346,126 @@ __device__ __forceinline__ void attn_new_row_tagged(const char* kvt, const Poll&
   }
 }
 
+// ---- the int8 cache in the polled builds (ohara/modules/kv_cache.py:15-32, 94-102, 116-118) -------------------
+// A tile as loaded: the codes of this lane's K pieces and V rows and the rows' (scale, minimum) pairs - half the
+// registers of a bf16 tile; they become the bf16 values the reference's read returns (common.h: dequant4)
+// where the bf16 path copies the next tile over the current one.
+template <int D>
+struct AttnRaw {
+  uint2 k[D / 32];    // piece 4 c + dq (8 codes) of row tb + p
+  uint2 kst;          // (key scale, key minimum) of that row
+  uint2 v[D / 32];    // columns 8 dc .. of row tb + c * PP + pp
+  uint2 vst[D / 32];  // (value scale, value minimum) of those rows
+};
+// st: the statistics records of this (sequence, KV head): 4 floats per position
+template <int D>
+__device__ __forceinline__ void attn_tile_load_i8(const int8_t* kb, const int8_t* vb, const float* st, size_t row, int tb,
+                                                  int last, AttnRaw<D>& r) {
+  constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
+  const int lane = threadIdx.x & 63;
+  const int p = lane & 15, dq = lane >> 4;
+  const int pp = lane / DC, dc = lane % DC;
+  const int pos = min(tb + p, last);
+  r.kst = ldg8(st + (size_t)pos * 4);
+#pragma unroll
+  for (int c = 0; c < NC; ++c) r.k[c] = ldg8(kb + (size_t)pos * row + (4 * c + dq) * 8);
+#pragma unroll
+  for (int c = 0; c < NV; ++c) {
+    const int vp = min(tb + c * PP + pp, last);
+    r.v[c] = ldg8(vb + (size_t)vp * row + dc * 8);
+    r.vst[c] = ldg8(st + (size_t)vp * 4 + 2);
+  }
+}
+template <int D>
+__device__ __forceinline__ void attn_tile_dequant(const AttnRaw<D>& r, uint4* kv, uint4* vv) {
+  constexpr int NC = D / 32, NV = D / 32;
+  const float ks = __uint_as_float(r.kst.x), km = __uint_as_float(r.kst.y);
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const uint2 lo = dequant4(r.k[c].x ^ 0x80808080u, ks, km), hi = dequant4(r.k[c].y ^ 0x80808080u, ks, km);
+    kv[c] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+  }
+#pragma unroll
+  for (int c = 0; c < NV; ++c) {
+    const float vs = __uint_as_float(r.vst[c].x), vm = __uint_as_float(r.vst[c].y);
+    const uint2 lo = dequant4(r.v[c].x ^ 0x80808080u, vs, vm), hi = dequant4(r.v[c].y ^ 0x80808080u, vs, vm);
+    vv[c] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+  }
+}
+// The row appended in this step, int8 cache.  The wave whose tile holds position `pos_new` polls the mailbox `kvt` (the
+// new key row, then the new value row, of all KV heads) for head kvh's two rows with every lane taking one bf16 pair of
+// them (D / 64 pairs a lane), quantises them as the cache's append does - minimum and maximum over the head's row,
+// scale = max(bf16(bf16(max - min) / 255), bf16(1e-8)), code = clamp(round(bf16(bf16(bf16(x - min) / scale) - 128))),
+// every op rounded to bf16 as the reference's tensor ops in the cache dtype round (kv_cache.py:23-26; csrc/kv_int8.hip)
+// - writes codes and statistics to the cache, and hands the values a read of those codes returns to the lanes of the
+// tile that hold the position through `stage` (2 D bf16 of LDS that only this wave touches).  Spread over the wave
+// the divisions cost a fifth of a microsecond; done by the four lanes that hold the key row they cost two.
+template <int D>
+__device__ __forceinline__ void attn_new_row_i8(const char* kvt, const Poll& pc, int Hkv, int kvh, int8_t* kq, int8_t* vq,
+                                                float* st, size_t row, int tb, int t1, int pos_new, uint4* kv, uint4* vv,
+                                                float* stage) {
+  constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
+  constexpr int W = D / 2;    // pairs per row
+  constexpr int NW = D / 64;  // pairs per lane: pair lane + 64 j of [key row | value row]
+  const int lane = threadIdx.x & 63;
+  const int nk = Hkv * D;
+  const MbRsrc rs = mb_rsrc(kvt);
+  uint32_t w[NW];
+  unsigned int spins = 0;
+  for (;;) {
+    bool ok = true;
+#pragma unroll
+    for (int j = 0; j < NW; ++j) {
+      const int i = lane + 64 * j;  // pair i of the key row, or pair i - W of the value row
+      ok = mb_ld4(rs, i < W ? kvh * D + 2 * i : nk + kvh * D + 2 * (i - W), w[j]) && ok;
+    }
+    if (__all(ok) || poll_expired(pc, spins)) break;
+  }
+  uint32_t* stw = reinterpret_cast<uint32_t*>(stage);
+#pragma unroll
+  for (int j = 0; j < NW; ++j) {
+    const int i = lane + 64 * j;
+    const bool is_v = i >= W;
+    const int ir = is_v ? i - W : i;
+    const float x0 = lo_bf(w[j]), x1 = hi_bf(w[j]);
+    // over the W lanes that share the row (the whole wave, or its half)
+    const float mn = lanes_min<(W < 64 ? W : 64) / 2, 1>(fminf(x0, x1));
+    const float mx = lanes_max<(W < 64 ? W : 64) / 2, 1>(fmaxf(x0, x1));
+    const float scale = fmaxf(rbf(rbf(mx - mn) / 255.0f), rbf(1e-8f));
+    const float t0 = rbf(rbf(rbf(x0 - mn) / scale) - 128.0f), t1q = rbf(rbf(rbf(x1 - mn) / scale) - 128.0f);
+    const int q0 = (int)fminf(fmaxf(rintf(t0), -128.f), 127.f), q1 = (int)fminf(fmaxf(rintf(t1q), -128.f), 127.f);
+    int8_t* dst = (is_v ? vq : kq) + (size_t)pos_new * row + 2 * ir;
+    *reinterpret_cast<uint16_t*>(dst) = (uint16_t)(((uint32_t)q0 & 0xffu) | (((uint32_t)q1 & 0xffu) << 8));
+    if (ir == 0) stg8(st + (size_t)pos_new * 4 + (is_v ? 2 : 0), make_uint2(__float_as_uint(scale), __float_as_uint(mn)));
+    stw[i] = pack_bf(__fmaf_rn((float)(q0 + 128), scale, mn), __fmaf_rn((float)(q1 + 128), scale, mn));
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  // the lanes of the tile that hold the position (and those past the chunk's end that repeat it, which weigh nothing)
+  const int p = lane & 15, dq = lane >> 4;
+  const int pp = lane / DC, dc = lane % DC;
+  const uint4* sv = reinterpret_cast<const uint4*>(stage);
+  if (min(tb + p, t1 - 1) == pos_new) {
+#pragma unroll
+    for (int c = 0; c < NC; ++c) kv[c] = sv[4 * c + dq];
+  }
+#pragma unroll
+  for (int c = 0; c < NV; ++c)
+    if (min(tb + c * PP + pp, t1 - 1) == pos_new) vv[c] = sv[W / 4 + dc];
+}
+
 // TAG (batch 1): the q row and the row appended in this step come from tagged mailboxes (qt, kvt) that
 // are polled for - there is no barrier between the projection that writes them and this phase.
-template <int D, int G, bool TAG = false>
+// I8 (with TAG only): kc / vc are the int8 caches, `stats` their (sequence, KV head, position) records.
+template <int D, int G, bool TAG = false, bool I8 = false>
 __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int blk_x, int ns, const AttnPre<D>& pre,
                                            const char* qm, float* pm, const bf16_t* kc, const bf16_t* vc, int L,
                                            float* lds, const char* qt = nullptr, const char* kvt = nullptr,
                                            const Poll pc = Poll{0, 0, nullptr}, bool announce = false, int q_row = 0,
-                                           int kv_row = 0) {  // q_row, kv_row: bytes between the sequences' rows of qt, kvt
+                                           int kv_row = 0,  // q_row, kv_row: bytes between the sequences' rows of qt, kvt
+                                           float* stats = nullptr) {
+  static_assert(!I8 || TAG, "the int8 cache is served by the polled builds");
   constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int p = lane & 15;
@@ -1377,12 +1496,19 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
     if (t0 + wave * 16 < t1) {
       uint4 qv[G][NC];
       // the tile after the current one is in flight while the current one is consumed
-      const bool use_pre = first && attn_first_tile_prefetchable<D>(t0, t1, L);
+      const bool use_pre = !I8 && first && attn_first_tile_prefetchable<D>(t0, t1, L);
       uint4 ka[NC], va[NV], kn[NC], vn[NV];
       int tb = t0 + wave * 16;
       const int coh = TAG ? -1 : L - 1;  // TAG: the appended row is patched in from the tagged mailbox below ...
       const int last = TAG ? max(min(t1, L - 1) - 1, 0) : t1 - 1;  // ... and its cache row is not touched
-      if (use_pre) {
+      // int8 cache: the codes of (sequence b, KV head kvh) and their records
+      int8_t* kq8 = reinterpret_cast<int8_t*>(const_cast<bf16_t*>(kc)) + (size_t)b * Tmax * row + (size_t)kvh * D;
+      int8_t* vq8 = reinterpret_cast<int8_t*>(const_cast<bf16_t*>(vc)) + (size_t)b * Tmax * row + (size_t)kvh * D;
+      float* stb = stats + ((size_t)b * Hkv + kvh) * Tmax * 4;
+      AttnRaw<D> raw;
+      if (I8) {
+        attn_tile_load_i8<D>(kq8, vq8, stb, row, tb, last, raw);
+      } else if (use_pre) {
 #pragma unroll
         for (int c = 0; c < NC; ++c) ka[c] = pre.k[c];
 #pragma unroll
@@ -1390,6 +1516,17 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
       } else {
         attn_tile_load_u<D>(kb, vb, row, tb, t1, coh, ka, va, last);
       }
+      // (int8: the first tile's codes become values before q is polled for - a wave's loads return in order anyway)
+      if constexpr (I8) attn_tile_dequant<D>(raw, ka, va);
+      auto patch = [&](int tbx, uint4* kx, uint4* vx) {  // the row appended in this step, if the tile at tbx holds its position
+        if (L - 1 >= tbx && L - 1 < tbx + 16) {
+          if constexpr (I8)
+            attn_new_row_i8<D>(kvt + (size_t)b * kv_row, pc, Hkv, kvh, kq8, vq8, stb, row, tbx, t1, L - 1, kx, vx,
+                               s_acc + wave * G * D);
+          else
+            attn_new_row_tagged<D>(kvt + (size_t)b * kv_row, pc, Hkv, kvh, tbx, t1, L - 1, kx, vx);
+        }
+      };
       if (TAG) {
         unsigned int spins = 0;
         const MbRsrc qrs = mb_rsrc(qt + (size_t)b * q_row);
@@ -1402,8 +1539,7 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
               ok = mb_ld16(qrs, (kvh * G + hh) * D + (4 * c + dq) * 8, qv[hh][c]) && ok;
           if (__all(ok) || poll_expired(pc, spins)) break;
         }
-        if (!use_pre && L - 1 >= tb && L - 1 < tb + 16)
-          attn_new_row_tagged<D>(kvt + (size_t)b * kv_row, pc, Hkv, kvh, tb, t1, L - 1, ka, va);
+        if (!use_pre) patch(tb, ka, va);
       } else {
 #pragma unroll
         for (int hh = 0; hh < G; ++hh)
@@ -1484,14 +1620,20 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
       // (a chunk is one or two tiles per wave here: the next tile goes through a second register set
       // and is copied over, which costs a wait but far fewer registers than two sets taking turns)
       for (; tb + 64 < t1; tb += 64) {
-        attn_tile_load_u<D>(kb, vb, row, tb + 64, t1, coh, kn, vn, last);
-        if (TAG && L - 1 >= tb + 64 && L - 1 < tb + 80)
-          attn_new_row_tagged<D>(kvt + (size_t)b * kv_row, pc, Hkv, kvh, tb + 64, t1, L - 1, kn, vn);
-        consume(tb, ka, va);
+        if constexpr (I8) {  // the next tile's codes travel while the current tile is consumed, and become values after it
+          attn_tile_load_i8<D>(kq8, vq8, stb, row, tb + 64, last, raw);
+          consume(tb, ka, va);
+          attn_tile_dequant<D>(raw, ka, va);
+          patch(tb + 64, ka, va);
+        } else {
+          attn_tile_load_u<D>(kb, vb, row, tb + 64, t1, coh, kn, vn, last);
+          if (TAG) patch(tb + 64, kn, vn);
+          consume(tb, ka, va);
 #pragma unroll
-        for (int c = 0; c < NC; ++c) ka[c] = kn[c];
+          for (int c = 0; c < NC; ++c) ka[c] = kn[c];
 #pragma unroll
-        for (int c = 0; c < NV; ++c) va[c] = vn[c];
+          for (int c = 0; c < NV; ++c) va[c] = vn[c];
+        }
       }
       consume(tb, ka, va);
     }

@@ -532,8 +532,10 @@ class DecodeSession:
         self._pws = None
         self.spin_limit = 0  # bound of the persistent kernel's barrier waits (0 = the library's default)
         self.cache = kv_cache if kv_cache is not None else model.build_kv_cache(batch)
-        if self.cache[0].int8:
-            persistent = False  # the single-launch kernel reads bf16 caches only
+        self._nwg = torch.cuda.get_device_properties(model.device).multi_processor_count
+        if persistent and self.cache[0].int8:
+            # the int8 cache is read (and the appended row quantised) by the polled builds of the kernel only
+            persistent = lib().ohara_persistent_polled(C.byref(model._c_model), batch, self._nwg) > 0
         self.persistent = persistent
         self.valid_vocab = valid_vocab
         self.history = torch.zeros(max(max_new_tokens, 1), batch, dtype=torch.int64, device=model.device)
@@ -586,7 +588,6 @@ class DecodeSession:
         self.graph = None
         if self.persistent:
             self._dst.n_split = self.PERSISTENT_SPLITS
-            self._nwg = torch.cuda.get_device_properties(m.device).multi_processor_count
             nbytes = lib().ohara_persistent_workspace_bytes(C.byref(m._c_model), B, self.PERSISTENT_SPLITS, self._nwg)
             if nbytes < 0:
                 raise RuntimeError("persistent workspace query failed")

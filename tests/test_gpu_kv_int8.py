@@ -306,3 +306,81 @@ def test_moe_model_with_int8_caches(cuda, P):
     mixed = [model.build_kv_cache(1, int8=True)[0]] + model.build_kv_cache(1)[1:]
     with pytest.raises(ValueError, match="same KV cache mode"):
         model(ids[:1, :2].to(cuda), mixed, 0)
+
+
+@pytest.mark.parametrize("heads,kv_heads,hidden,B,P", [(2, 2, 256, 1, 21), (4, 2, 256, 3, 40), (8, 2, 512, 8, 70),
+                                                       (4, 1, 512, 2, 130), (2, 1, 256, 5, 63), (4, 4, 256, 2, 33),
+                                                       (6, 6, 768, 1, 1200)])
+def test_persistent_kernel_on_int8_caches(cuda, heads, kv_heads, hidden, B, P):
+    """The single-launch decode step over int8 caches (its polled builds, up to eight sequences): the attention
+    phase reads codes and statistics and quantises the appended row itself.  Teacher-forced logits against the
+    oracle on int8 caches, for the single launch and for the kernel chain; the rows the single launch appended
+    against the oracle's through the values they stand for; and its quantiser bit for bit: the first layer's
+    appended rows depend on the fed tokens only, so a bf16-cache session of the same kernel holds exactly the
+    rows that were quantised, and the oracle's codes and statistics of those rows must be the cache's."""
+    from ohara_amd import ops
+    from ohara_amd.llama import Llama
+
+    T = 2048 if P > 1000 else 256
+    rcfg, cfg = _cfg_pair(vocab_size=512, hidden_size=hidden, intermediate_size=512, num_attention_heads=heads,
+                          num_key_value_heads=kv_heads, num_hidden_layers=2, max_sequence_length=T, rope_theta=10000.0)
+    w = R.init_weights(rcfg, seed=heads + B, dtype=BF, std=0.06, norm_jitter=0.1)
+    ref, model = R.RefLlama(rcfg, w), Llama(cfg, w, device=cuda)
+    prompt = torch.randint(0, 512, (B, P), generator=torch.Generator().manual_seed(P))
+    steps = 5
+    rc = ref.build_kv_cache(B, int8=True)
+    want = [ref(prompt, rc, 0)[:, -1]]
+    fed = []
+    for s in range(steps):
+        fed.append(want[-1].float().argmax(-1))
+        want.append(ref(fed[-1].view(B, 1), rc, P + s)[:, -1])
+    caches, logits = {}, {}
+    for persistent in (True, False):
+        cache = model.build_kv_cache(B, int8=True)
+        sess = model.session(B, steps + 1, kv_cache=cache, persistent=persistent)
+        assert sess.persistent is persistent
+        sess.prefill(prompt.to(cuda))
+        _close(sess.logits, want[0], 4e-2, 6e-3)
+        logits[persistent] = []
+        for s in range(steps):
+            sess.feed(fed[s].to(cuda))
+            sess.step()
+            # (the quantisation noise of these small random models: the mean is 3e-3 to 5e-3 of the scale for both paths)
+            _close(sess.logits, want[s + 1], 4e-2, 6e-3)
+            logits[persistent].append(sess.logits.float().cpu())
+        sess.check_error()
+        caches[persistent] = cache
+    cache = caches[True]
+    # the two device paths against each other: the same rows quantised the same way, up to the bf16 noise of the
+    # projections that feed the second layer (a code off by one here and there)
+    for s in range(steps):
+        _close(logits[True][s], logits[False][s], 1e-2, 2.5e-3)  # (a bf16 ulp of a logit is 2e-3 to 4e-3 of the scale)
+    for l in range(2):
+        for name in ("key", "value"):
+            a, b = getattr(cache[l], name)[:B, P:P + steps].int(), getattr(caches[False][l], name)[:B, P:P + steps].int()
+            assert (a - b).abs().max().item() <= (0 if l == 0 else 1), (l, name)
+            assert (a != b).float().mean().item() <= 0.03, (l, name)
+    for l in range(2):
+        for which in ("key", "value"):
+            got = ops.kv_dequant(cache[l], which, B, P + steps).cpu().float()[:, P:]
+            rq, rs, rm = ((rc[l].key, rc[l].key_scale, rc[l].key_min) if which == "key"
+                          else (rc[l].value, rc[l].value_scale, rc[l].value_min))
+            exp = R.dequantize_int8(rq[:B, P:P + steps], rs[:B, P:P + steps], rm[:B, P:P + steps])
+            assert (got - exp).abs().max().item() <= 3e-2 * exp.abs().max().item(), (l, which)
+            assert (got - exp).abs().mean().item() <= 4e-3 * exp.abs().max().item(), (l, which)
+    # nothing behind the last appended position was touched
+    assert not cache[0].key[:, P + steps:].any() and not cache[1].stats[:, :, P + steps:].any()
+    # the in-kernel quantiser, bit for bit
+    plain = model.build_kv_cache(B)
+    sess = model.session(B, steps + 1, kv_cache=plain, persistent=True)
+    sess.prefill(prompt.to(cuda))
+    for s in range(steps):
+        sess.feed(fed[s].to(cuda))
+        sess.step()
+    sess.check_error()
+    for rows, codes, scale, mn in ((plain[0].key, cache[0].key, cache[0].key_scale, cache[0].key_min),
+                                   (plain[0].value, cache[0].value, cache[0].value_scale, cache[0].value_min)):
+        rq, rs, rm = R.quantize_int8(rows[:B, P:P + steps].cpu())
+        assert torch.equal(codes[:B, P:P + steps].cpu(), rq)
+        assert torch.equal(scale[:B, P:P + steps].cpu(), rs.float())
+        assert torch.equal(mn[:B, P:P + steps].cpu(), rm.float())
