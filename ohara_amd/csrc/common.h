@@ -82,8 +82,13 @@ __device__ __forceinline__ float pow2_neg_int(float d) {
 
 __device__ __forceinline__ float lo_bf(uint32_t packed) { return __uint_as_float(packed << 16); }
 __device__ __forceinline__ float hi_bf(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
+// (as a two-element vector conversion this is ONE v_cvt_pk_bf16_f32; two scalar conversions glued together with a
+// shift and an or were four instructions)
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pack_bf(float lo, float hi) {
-  return (uint32_t)f2bf(lo) | ((uint32_t)f2bf(hi) << 16);
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 // (q + 128) * scale + min in fp32, rounded to bf16 (kv_cache.py:30-32, 116-118): four bytes -> two
