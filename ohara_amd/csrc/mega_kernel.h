@@ -233,8 +233,8 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
       pf.stamp();  // 4: rotary epilogue, tagged stores issued
       // P2: attention partials (polls for q; the chunk that holds the new position polls for its k / v rows); each chunk
       // leaves the launch's tag behind its (max, sum) pair
-      attn_phase<D, G, true, I8>(B, H, Hkv, m.t_max, a.blk_x, a.ns, apre, nullptr, p_l, kc, vc, L, att, qt, kvt, pc, true,
-                                 a.tg_rq, a.tg_rkv, I8 ? lds_ptr<float>(stab, l) : nullptr);
+      attn_phase<D, G, true, I8, ONE>(B, H, Hkv, m.t_max, a.blk_x, a.ns, apre, nullptr, p_l, kc, vc, L, att, qt, kvt, pc, true,
+                                 a.tg_rq, a.tg_rkv, I8 ? lds_ptr<float>(stab, l) : nullptr, red);
       pf.stamp();  // 5: partials stored, flag raised
       // the next layer's q/k/v weights (+ norm1's, the rotary pair): their registers are free again (behind the attention
       // phase, which needs many: a workgroup without a chunk - at the usual sizes those with q/k/v strips - is here at once)

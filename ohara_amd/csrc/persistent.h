@@ -1317,33 +1317,21 @@ __device__ __forceinline__ void attn_prefetch(int B, int Hkv, int Tmax, int ns, 
   attn_tile_load<D>(kb, vb, row, t0 + wave * 16, has ? t1 : 0, -1, pre.k, pre.v);
 }
 
-// The row appended in this step, taken from the tagged mailbox `kvt` (the new key row, then the new
-// value row: batch 1) by the lanes of the tile at `tb` that hold position `pos_new`; polls until the
-// row's entries carry this launch's tag.
+// The row appended in this step, as the wave staged it in its LDS ([... | new key row | new value row], see
+// attn_phase): the lanes of the tile at `tb` that hold position `pos_new` take their pieces.
 template <int D>
-__device__ __forceinline__ void attn_new_row_tagged(const char* kvt, const Poll& pc, int Hkv, int kvh, int tb, int t1,
-                                                    int pos_new, uint4* kv, uint4* vv) {
+__device__ __forceinline__ void attn_new_row_staged(const char* krow, int tb, int t1, int pos_new, uint4* kv, uint4* vv) {
   constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
   const int lane = threadIdx.x & 63;
   const int p = lane & 15, dq = lane >> 4;
   const int pp = lane / DC, dc = lane % DC;
-  const int pos = min(tb + p, t1 - 1);
-  const int nk = Hkv * D;
-  unsigned int spins = 0;
-  const MbRsrc rs = mb_rsrc(kvt);
-  for (;;) {
-    bool ok = true;
-    if (pos == pos_new) {
+  if (min(tb + p, t1 - 1) == pos_new) {
 #pragma unroll
-      for (int c = 0; c < NC; ++c) ok = mb_ld16(rs, kvh * D + (4 * c + dq) * 8, kv[c]) && ok;
-    }
-#pragma unroll
-    for (int c = 0; c < NV; ++c) {
-      const int vp = min(tb + c * PP + pp, t1 - 1);
-      if (vp == pos_new) ok = mb_ld16(rs, nk + kvh * D + dc * 8, vv[c]) && ok;
-    }
-    if (__all(ok) || poll_expired(pc, spins)) break;
+    for (int c = 0; c < NC; ++c) kv[c] = lds16(krow + (4 * c + dq) * 16);
   }
+#pragma unroll
+  for (int c = 0; c < NV; ++c)
+    if (min(tb + c * PP + pp, t1 - 1) == pos_new) vv[c] = lds16(krow + (DC + dc) * 16);
 }
 
 // ---- the int8 cache in the polled builds (ohara/modules/kv_cache.py:15-32, 94-102, 116-118) -------------------
@@ -1392,35 +1380,21 @@ __device__ __forceinline__ void attn_tile_dequant(const AttnRaw<D>& r, uint4* kv
     vv[c] = make_uint4(lo.x, lo.y, hi.x, hi.y);
   }
 }
-// The row appended in this step, int8 cache.  The wave whose tile holds position `pos_new` polls the mailbox `kvt` (the
-// new key row, then the new value row, of all KV heads) for head kvh's two rows with every lane taking one bf16 pair of
-// them (D / 64 pairs a lane), quantises them as the cache's append does - minimum and maximum over the head's row,
+// The row appended in this step, int8 cache.  The wave whose tile holds position `pos_new` has the head's new key and
+// value rows from the mailbox with every lane holding one bf16 pair of them (w[j]: pair lane + 64 j of [key row | value
+// row], D / 64 pairs a lane), and quantises them as the cache's append does - minimum and maximum over the head's row,
 // scale = max(bf16(bf16(max - min) / 255), bf16(1e-8)), code = clamp(round(bf16(bf16(bf16(x - min) / scale) - 128))),
 // every op rounded to bf16 as the reference's tensor ops in the cache dtype round (kv_cache.py:23-26; csrc/kv_int8.hip)
 // - writes codes and statistics to the cache, and hands the values a read of those codes returns to the lanes of the
 // tile that hold the position through `stage` (2 D bf16 of LDS that only this wave touches).  Spread over the wave
 // the divisions cost a fifth of a microsecond; done by the four lanes that hold the key row they cost two.
 template <int D>
-__device__ __forceinline__ void attn_new_row_i8(const char* kvt, const Poll& pc, int Hkv, int kvh, int8_t* kq, int8_t* vq,
-                                                float* st, size_t row, int tb, int t1, int pos_new, uint4* kv, uint4* vv,
-                                                float* stage) {
+__device__ __forceinline__ void attn_new_row_i8(const uint32_t* w, int8_t* kq, int8_t* vq, float* st, size_t row, int tb,
+                                                int t1, int pos_new, uint4* kv, uint4* vv, float* stage) {
   constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
   constexpr int W = D / 2;    // pairs per row
-  constexpr int NW = D / 64;  // pairs per lane: pair lane + 64 j of [key row | value row]
+  constexpr int NW = D / 64;  // pairs per lane
   const int lane = threadIdx.x & 63;
-  const int nk = Hkv * D;
-  const MbRsrc rs = mb_rsrc(kvt);
-  uint32_t w[NW];
-  unsigned int spins = 0;
-  for (;;) {
-    bool ok = true;
-#pragma unroll
-    for (int j = 0; j < NW; ++j) {
-      const int i = lane + 64 * j;  // pair i of the key row, or pair i - W of the value row
-      ok = mb_ld4(rs, i < W ? kvh * D + 2 * i : nk + kvh * D + 2 * (i - W), w[j]) && ok;
-    }
-    if (__all(ok) || poll_expired(pc, spins)) break;
-  }
   uint32_t* stw = reinterpret_cast<uint32_t*>(stage);
 #pragma unroll
   for (int j = 0; j < NW; ++j) {
@@ -1458,13 +1432,16 @@ __device__ __forceinline__ void attn_new_row_i8(const char* kvt, const Poll& pc,
 // TAG (batch 1): the q row and the row appended in this step come from tagged mailboxes (qt, kvt) that
 // are polled for - there is no barrier between the projection that writes them and this phase.
 // I8 (with TAG only): kc / vc are the int8 caches, `stats` their (sequence, KV head, position) records.
-template <int D, int G, bool TAG = false, bool I8 = false>
+// AHEAD (with TAG only): a wave's second tile is requested before the poll for q (the single-sequence build: with more
+// sequences a chunk is many tiles and the registers the request holds across the poll are spilled).
+template <int D, int G, bool TAG = false, bool I8 = false, bool AHEAD = false>
 __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int blk_x, int ns, const AttnPre<D>& pre,
                                            const char* qm, float* pm, const bf16_t* kc, const bf16_t* vc, int L,
                                            float* lds, const char* qt = nullptr, const char* kvt = nullptr,
                                            const Poll pc = Poll{0, 0, nullptr}, bool announce = false, int q_row = 0,
                                            int kv_row = 0,  // q_row, kv_row: bytes between the sequences' rows of qt, kvt
-                                           float* stats = nullptr) {
+                                           float* stats = nullptr,
+                                           float* wave_lds = nullptr) {  // TAG: 1 KB of LDS per wave, free during this phase
   static_assert(!I8 || TAG, "the int8 cache is served by the polled builds");
   constexpr int NC = D / 32, DC = D / 8, PP = 64 / DC, NV = 16 / PP;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -1518,26 +1495,71 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
       }
       // (int8: the first tile's codes become values before q is polled for - a wave's loads return in order anyway)
       if constexpr (I8) attn_tile_dequant<D>(raw, ka, va);
-      auto patch = [&](int tbx, uint4* kx, uint4* vx) {  // the row appended in this step, if the tile at tbx holds its position
-        if (L - 1 >= tbx && L - 1 < tbx + 16) {
-          if constexpr (I8)
-            attn_new_row_i8<D>(kvt + (size_t)b * kv_row, pc, Hkv, kvh, kq8, vq8, stb, row, tbx, t1, L - 1, kx, vx,
-                               s_acc + wave * G * D);
-          else
-            attn_new_row_tagged<D>(kvt + (size_t)b * kv_row, pc, Hkv, kvh, tbx, t1, L - 1, kx, vx);
+      // Polled builds: what the wave needs from the mailboxes - the group's q rows, and the row appended in this step if
+      // one of the wave's tiles holds its position - is polled for as ONE 16-byte piece per lane (two with four heads
+      // per KV head) and handed round through the wave's own LDS.  A round costs by its load instructions: four for q
+      // (lanes sharing addresses) and a second poll of up to nine for the new key / value rows after it were 0.8 us a
+      // layer more.  staging area: [q rows of the group | new key row | new value row], bf16.
+      constexpr int NPQ = G * D / 8, NPK = D / 8, NP = NPQ + 2 * NPK, NPL = (NP + 63) / 64;
+      char* stage = reinterpret_cast<char*>(G * D * 4 >= NP * 16 ? s_acc + wave * G * D : wave_lds + wave * 256);
+      const int pn = L - 1;
+      // (the appended position sits at the end of the last chunk; a wave's tiles are every fourth one of the chunk)
+      const bool need_new = TAG && pn >= t0 && pn < t1 && (((pn - t0) >> 4) & 3) == wave;
+      uint32_t nw[D / 64];  // int8 cache: this lane's pairs of the new rows
+      auto patch = [&](int tbx, uint4* kx, uint4* vx) {  // the appended row into the tile at tbx, if that holds its position
+        if (need_new && pn >= tbx && pn < tbx + 16) {
+          if constexpr (I8) attn_new_row_i8<D>(nw, kq8, vq8, stb, row, tbx, t1, pn, kx, vx, reinterpret_cast<float*>(stage));
+          else attn_new_row_staged<D>(stage + NPQ * 16, tbx, t1, pn, kx, vx);
         }
       };
+      // the wave's second tile, requested ahead of the poll (a workgroup waits for q for microseconds; what is requested
+      // behind the poll is a memory latency late)
+      bool ahead = false;
+      if (AHEAD && tb + 64 < t1) {
+        if constexpr (I8) attn_tile_load_i8<D>(kq8, vq8, stb, row, tb + 64, last, raw);
+        else attn_tile_load_u<D>(kb, vb, row, tb + 64, t1, coh, kn, vn, last);
+        ahead = true;
+      }
       if (TAG) {
         unsigned int spins = 0;
-        const MbRsrc qrs = mb_rsrc(qt + (size_t)b * q_row);
-        for (;;) {  // (every round fetches the group's q rows whole: lanes share addresses, 256 bytes a row)
+        const char* qrow = qt + (size_t)b * q_row;
+        const MbRsrc rs = mb_rsrc(qrow);
+        const uint32_t kv_off = (uint32_t)((kvt + (size_t)b * kv_row) - qrow);  // (the mailboxes of a layer are one block)
+        uint32_t off[NPL];
+#pragma unroll
+        for (int l = 0; l < NPL; ++l) {
+          const int i = lane + 64 * l;
+          const uint32_t oq = (uint32_t)(kvh * G * D + (i < NPQ ? i : 0) * 8) * 2u;
+          const int j = i - NPQ;  // piece of [key row | value row]
+          const uint32_t ok_ = kv_off + (uint32_t)((j < NPK ? kvh * D + j * 8 : Hkv * D + kvh * D + (j - NPK) * 8)) * 2u;
+          off[l] = (need_new && i >= NPQ && i < NP) ? ok_ : oq;
+        }
+        uint4 piece[NPL];
+        for (;;) {
           bool ok = true;
 #pragma unroll
-          for (int hh = 0; hh < G; ++hh)
-#pragma unroll
-            for (int c = 0; c < NC; ++c)
-              ok = mb_ld16(qrs, (kvh * G + hh) * D + (4 * c + dq) * 8, qv[hh][c]) && ok;
+          for (int l = 0; l < NPL; ++l) {
+            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, off[l], 0, 16);
+            piece[l] = make_uint4(v.x, v.y, v.z, v.w);
+            ok = ok && v.x != OHARA_UNWRITTEN && v.y != OHARA_UNWRITTEN && v.z != OHARA_UNWRITTEN && v.w != OHARA_UNWRITTEN;
+          }
           if (__all(ok) || poll_expired(pc, spins)) break;
+        }
+#pragma unroll
+        for (int l = 0; l < NPL; ++l)
+          if (lane + 64 * l < NP) sts16(stage + (lane + 64 * l) * 16, piece[l]);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int hh = 0; hh < G; ++hh)
+#pragma unroll
+          for (int c = 0; c < NC; ++c) qv[hh][c] = lds16(stage + (hh * (D / 8) + 4 * c + dq) * 16);
+        if constexpr (I8) {
+          if (need_new) {
+#pragma unroll
+            for (int j = 0; j < D / 64; ++j) nw[j] = reinterpret_cast<const uint32_t*>(stage + NPQ * 16)[lane + 64 * j];
+          }
         }
         if (!use_pre) patch(tb, ka, va);
       } else {
@@ -1618,22 +1640,24 @@ __device__ __forceinline__ void attn_phase(int B, int H, int Hkv, int Tmax, int 
         }
       };
       // (a chunk is one or two tiles per wave here: the next tile goes through a second register set
-      // and is copied over, which costs a wait but far fewer registers than two sets taking turns)
+      // and is copied over, which costs a wait but far fewer registers than two sets taking turns; the polled builds
+      // have requested the wave's second tile before the poll for q)
       for (; tb + 64 < t1; tb += 64) {
         if constexpr (I8) {  // the next tile's codes travel while the current tile is consumed, and become values after it
-          attn_tile_load_i8<D>(kq8, vq8, stb, row, tb + 64, last, raw);
+          if (!AHEAD || !ahead) attn_tile_load_i8<D>(kq8, vq8, stb, row, tb + 64, last, raw);
+          ahead = false;
           consume(tb, ka, va);
           attn_tile_dequant<D>(raw, ka, va);
-          patch(tb + 64, ka, va);
         } else {
-          attn_tile_load_u<D>(kb, vb, row, tb + 64, t1, coh, kn, vn, last);
-          if (TAG) patch(tb + 64, kn, vn);
+          if (!AHEAD || !ahead) attn_tile_load_u<D>(kb, vb, row, tb + 64, t1, coh, kn, vn, last);
+          ahead = false;
           consume(tb, ka, va);
 #pragma unroll
           for (int c = 0; c < NC; ++c) ka[c] = kn[c];
 #pragma unroll
           for (int c = 0; c < NV; ++c) va[c] = vn[c];
         }
+        if (TAG) patch(tb + 64, ka, va);
       }
       consume(tb, ka, va);
     }
