@@ -316,6 +316,34 @@ int ohara_moe_experts_down(const uint16_t* act, int ld_act, const uint16_t* wp_d
 int ohara_moe_combine(const uint16_t* y, int ldy, const int32_t* expert_idx, const int32_t* pos_of, int n_tokens, int k,
                       const uint16_t* shared, int ld_shared, const uint16_t* resid, int ldr, uint16_t* out, int ldo, int d,
                       void* stream);
+/* The same feed-forward for a decode step in four launches (at most 64 experts, 1024 pairs, d <= 4096):
+ *  ohara_moe_route_fused    the block's RMSNorm (ohara/modules/norm.py:16-21; ohara/models/llama.py:200) of the rows
+ *                           x, the router Linear on the normalised rows (moe_grouped.py:126), _route (:122-147) and
+ *                           the sort of :161-168 in ONE launch: x_norm (n_tokens, d) for the experts, expert_idx /
+ *                           expert_w, offsets / pair_of / pos_of as above; router_logits (n_tokens, n_experts) may be
+ *                           NULL.  counter: one int32 of device memory that is zero between calls (the workgroup
+ *                           that finishes last sorts, and leaves it zero); calls that share it must not overlap.
+ *  ohara_moe_experts_gate_up_shared / ohara_moe_experts_down_shared
+ *                           the expert launches with the shared expert (_shared, :206-207, 219-220) as more
+ *                           rows of their grids (16 tokens a row): wp_shared its packed gate/up (down) rows, shared_hidden its width,
+ *                           act_shared (n_tokens, shared_hidden), y_shared (n_tokens, d) = bf16(act_shared W_down),
+ *                           not scaled - pass y_shared to ohara_moe_combine as `shared`.  wp_shared NULL: as the
+ *                           entry points above. */
+int ohara_moe_route_fused(const uint16_t* x, int ldx, const uint16_t* norm_w, float eps, const uint16_t* router_wp,
+                          const uint16_t* router_bias, int n_tokens, int d, int n_experts, int k, int biased_topk,
+                          int gate_sigmoid, int normalize, uint16_t* x_norm, int ld_x_norm, uint16_t* router_logits, int ldl,
+                          int32_t* expert_idx, uint16_t* expert_w, int32_t* offsets, int32_t* pair_of, int32_t* pos_of,
+                          int32_t* counter, void* stream);
+int ohara_moe_experts_gate_up_shared(const uint16_t* x, int ldx, const uint16_t* wp_gate_up, int64_t expert_stride_bytes,
+                                     int n_experts, int hidden, int d, int k, const int32_t* offsets,
+                                     const int32_t* pair_of, uint16_t* act, int ld_act, const uint16_t* wp_shared,
+                                     int shared_hidden, int n_tokens, uint16_t* act_shared, int ld_act_shared,
+                                     void* stream);
+int ohara_moe_experts_down_shared(const uint16_t* act, int ld_act, const uint16_t* wp_down, int64_t expert_stride_bytes,
+                                  int n_experts, int d, int hidden, int k, const int32_t* offsets, const int32_t* pair_of,
+                                  const uint16_t* expert_w, uint16_t* y, int ldy, const uint16_t* wp_shared,
+                                  int shared_hidden, int n_tokens, const uint16_t* act_shared, int ld_act_shared,
+                                  uint16_t* y_shared, int ldy_shared, void* stream);
 
 /* ---- the whole forward pass through the KV cache ---------------------------------
  * Llama.forward(x, kv_cache, position) (ohara/models/llama.py:279-323; Block.forward

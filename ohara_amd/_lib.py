@@ -97,6 +97,11 @@ _PROTOS = {
     "ohara_moe_sort_pairs": (_i, [_p, _i, _i, _p, _p, _p, _p]),
     "ohara_moe_experts_gate_up": (_i, [_p, _i, _p, _i64, _i, _i, _i, _i, _p, _p, _p, _i, _p]),
     "ohara_moe_experts_down": (_i, [_p, _i, _p, _i64, _i, _i, _i, _i, _p, _p, _p, _p, _i, _p]),
+    "ohara_moe_route_fused": (_i, [_p, _i, _p, _f, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _i, _p, _p, _p, _p, _p,
+                                   _p, _p]),
+    "ohara_moe_experts_gate_up_shared": (_i, [_p, _i, _p, _i64, _i, _i, _i, _i, _p, _p, _p, _i, _p, _i, _i, _p, _i, _p]),
+    "ohara_moe_experts_down_shared": (_i, [_p, _i, _p, _i64, _i, _i, _i, _i, _p, _p, _p, _p, _i, _p, _i, _i, _p, _i, _p, _i,
+                                           _p]),
     "ohara_moe_combine": (_i, [_p, _i, _p, _p, _i, _i, _p, _i, _p, _i, _p, _i, _i, _p]),
     "ohara_llama_forward": (_i, [C.POINTER(OharaModel), C.POINTER(OharaDecodeState), _i, _i, _i, _i, _i, _p]),
     "ohara_linear_bias_bf16": (_i, [_p, _i, _p, _i, _i, _p, _i, _i, _p, _i, _p, _i, _p, _i, _p]),

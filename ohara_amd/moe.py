@@ -53,6 +53,7 @@ class GroupedMoE:
         if shared is not None:
             sg, su, sd = shared
             self.shared = (ops.pack_gate_up(d(sg), d(su)), ops.pack_linear(d(sd)))
+        self._counter = torch.zeros(1, dtype=torch.int32, device=dev)  # the fused route launch's arrival counter
 
     def route(self, flat_x: torch.Tensor):
         """-> (expert ids (N, k) int32, weights (N, k) bf16)"""
@@ -91,6 +92,50 @@ class GroupedMoE:
         check(lib().ohara_moe_combine(_ptr(y), self.dim, _ptr(idx), _ptr(pos_of), n, k, _ptr(sh), self.dim,
                                       _ptr(residual), 0 if residual is None else residual.stride(0), _ptr(out), self.dim,
                                       self.dim, st), "moe_combine")
+        return out
+
+    def fused_ok(self, n: int) -> bool:
+        """The four-launch form serves at most 64 experts and 1024 (token, expert) pairs: decode steps."""
+        return self.E <= 64 and n * self.k <= 1024 and self.dim % 8 == 0 and self.dim <= 4096 and self.hidden % 8 == 0
+
+    def forward_block(self, h: torch.Tensor, norm_w: torch.Tensor, eps: float) -> torch.Tensor:
+        """h (N, dim) bf16 -> h + moe(rmsnorm(h)) (ohara/models/llama.py:200) in four launches: norm + router +
+        selection + sort, gate/up of the experts and the shared expert, their down projections, the combine."""
+        n, k, E = h.shape[0], self.k, self.E
+        if not self.fused_ok(n):
+            return self.forward_rows(ops.rmsnorm(h, norm_w, eps), residual=h)
+        st, dev = ops._stream(), self.device
+        xn = torch.empty(n, self.dim, dtype=BF16, device=dev)
+        idx = torch.empty(n, k, dtype=torch.int32, device=dev)
+        w = torch.empty(n, k, dtype=BF16, device=dev)
+        meta = torch.empty(E + 1 + 2 * n * k, dtype=torch.int32, device=dev)
+        offs, pair_of, pos_of = meta[: E + 1], meta[E + 1: E + 1 + n * k], meta[E + 1 + n * k:]
+        logits = torch.empty(n, E, dtype=BF16, device=dev) if self.trace is not None else None
+        check(lib().ohara_moe_route_fused(_ptr(h), h.stride(0), _ptr(norm_w), float(eps), _ptr(self.router.data),
+                                          _ptr(self.router_bias), n, self.dim, E, k, int(self.biased),
+                                          int(self.gate_fn == "sigmoid"), int(self.normalize), _ptr(xn), self.dim,
+                                          _ptr(logits), E, _ptr(idx), _ptr(w), _ptr(offs), _ptr(pair_of), _ptr(pos_of),
+                                          _ptr(self._counter), st), "moe_route_fused")
+        if self.trace is not None:
+            self.trace.append((logits, idx, w))
+            self.last_sort = (offs, pair_of, pos_of)
+        sh_gu, sh_dn = self.shared if self.shared is not None else (None, None)
+        sh_hidden = sh_gu.n if sh_gu is not None else 0
+        act = torch.empty(n * k, self.hidden, dtype=BF16, device=dev)
+        act_sh = torch.empty(n, sh_hidden, dtype=BF16, device=dev) if sh_gu is not None else None
+        check(lib().ohara_moe_experts_gate_up_shared(_ptr(xn), self.dim, _ptr(self.wp_gu), self.wp_gu.stride(0) * 2, E,
+                                                     self.hidden, self.dim, k, _ptr(offs), _ptr(pair_of), _ptr(act),
+                                                     self.hidden, _ptr(sh_gu.data) if sh_gu is not None else 0, sh_hidden,
+                                                     n, _ptr(act_sh), sh_hidden, st), "moe_gate_up")
+        y = torch.empty(n * k + (n if sh_gu is not None else 0), self.dim, dtype=BF16, device=dev)
+        y_sh = y[n * k:] if sh_gu is not None else None
+        check(lib().ohara_moe_experts_down_shared(_ptr(act), self.hidden, _ptr(self.wp_dn), self.wp_dn.stride(0) * 2, E,
+                                                  self.dim, self.hidden, k, _ptr(offs), _ptr(pair_of), _ptr(w), _ptr(y),
+                                                  self.dim, _ptr(sh_dn.data) if sh_dn is not None else 0, sh_hidden, n,
+                                                  _ptr(act_sh), sh_hidden, _ptr(y_sh), self.dim, st), "moe_down")
+        out = torch.empty(n, self.dim, dtype=BF16, device=dev)
+        check(lib().ohara_moe_combine(_ptr(y), self.dim, _ptr(idx), _ptr(pos_of), n, k, _ptr(y_sh), self.dim, _ptr(h),
+                                      h.stride(0), _ptr(out), self.dim, self.dim, st), "moe_combine")
         return out
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -228,7 +273,7 @@ class MoeLlama:
                 att = ops.attn_auto(q, cache.key, cache.value, H, Hkv, D, start, n_split, ws, S)
             h = ops.gemm_skinny(att, L["wo"], residual=h)
             if "moe" in L:
-                h = L["moe"].forward_rows(ops.rmsnorm(h, L["norm2"], self.eps), residual=h)
+                h = L["moe"].forward_block(h, L["norm2"], self.eps)
             else:
                 act = ops.gemm_skinny(h, L["wgu"], norm_w=L["norm2"], eps=self.eps)
                 h = ops.gemm_skinny(act, L["wdown"], residual=h)

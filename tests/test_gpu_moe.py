@@ -165,3 +165,47 @@ def test_loop_form_moe_config_is_served(cuda):
         scale = want.abs().max().item()
         row_err = (got.float().cpu() - want).abs().amax(-1).reshape(-1)
         assert (row_err <= 4e-2 * scale).float().mean().item() >= 0.9
+
+
+@pytest.mark.parametrize("N,d,E,hidden,k,shared,gate", [(64, 1024, 64, 512, 8, 1, "softmax"), (9, 64, 6, 24, 2, 0, "softmax"),
+                                                       (40, 128, 16, 32, 4, 2, "sigmoid"), (5, 32, 8, 16, 2, 1, "softmax"),
+                                                       (33, 256, 40, 64, 3, 1, "softmax")])
+def test_moe_block_in_four_launches(cuda, N, d, E, hidden, k, shared, gate):
+    """h + moe(rmsnorm(h)) as norm + router + selection + sort in one launch, the experts' two launches with the
+    shared expert as one more row of their grids, and the combine - against the launch-per-step form of the same
+    block: the selection from the launch's own router outputs exactly (ties to the lowest id), the sort against a
+    stable host sort, rows whose selection is the same in both forms at bf16 tolerance, twice in a row (the arrival
+    counter must be left at zero)."""
+    from ohara_amd import ops
+    from ohara_amd.moe import GroupedMoE
+
+    w, sh, x = _make(N, d, E, hidden, k, shared, seed=3 * N + E)
+    moe = GroupedMoE(w["w_gate"], w["w_up"], w["w_down"], w["router"], w["bias"], k, sh, gate_fn=gate, device=cuda)
+    assert moe.fused_ok(N)
+    g = torch.Generator().manual_seed(N)
+    h = (torch.randn(N, d, generator=g) * 1.5).to(BF).to(cuda)
+    nw = (1 + 0.1 * torch.randn(d, generator=g)).to(BF).to(cuda)
+    moe.trace = []
+    want = moe.forward_rows(ops.rmsnorm(h, nw, 1e-5), residual=h)
+    _, idx_sep, _ = moe.trace[0]
+    for rep in range(2):
+        moe.trace = []
+        got = moe.forward_block(h, nw, 1e-5)
+        logits, idx, wt = moe.trace[0]
+        offs, pair_of, pos_of = moe.last_sort
+        assert int(moe._counter.item()) == 0
+        lg = logits.float().cpu()
+        sel = lg + w["bias"].float() if moe.biased else lg
+        want_idx = M.topk_lowest_index_first(sel, k + 1)[:, :k] if moe.biased else M.topk_lowest_index_first(sel, k)
+        assert torch.equal(idx.cpu().long(), want_idx), rep
+        flat = idx.cpu().long().flatten()
+        order = torch.sort(flat, stable=True).indices
+        assert torch.equal(pair_of.cpu().long(), order)
+        assert torch.equal(offs.cpu().long()[1:], torch.bincount(flat, minlength=E).cumsum(0))
+        assert torch.equal(pos_of.cpu().long()[order], torch.arange(N * k))
+        same = (idx.cpu().sort(-1).values == idx_sep.cpu().sort(-1).values).all(-1)
+        assert same.float().mean().item() >= 0.9
+        scale = want.float().abs().max().item()
+        dd = (got.float() - want.float()).cpu()[same].abs()
+        assert dd.max().item() <= 2e-2 * scale and dd.mean().item() <= 2e-3 * scale, (dd.max().item(), dd.mean().item(), scale)
+    moe.trace = None
