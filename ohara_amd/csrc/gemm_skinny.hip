@@ -89,7 +89,68 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(GemmArgs a) {
   __shared__ float ssq[NW][BT * 16];
   __shared__ float ssum[NORM == 2 ? NW : 1][BT * 16];
 
+  // A launch of this kernel is a chain of memory round trips - the rows for the norm, the weights, what the epilogue
+  // adds or rotates with - and lasts about as long as their sum (6-9 us for 1-9 MB at 32 rows).  What does not depend
+  // on anything computed here is therefore requested first: the epilogue's operands (wave 0 finishes the fragments),
+  // and, where a wave's share of K is at most SP k-steps (K <= 1024 with four waves), the rows, the norm weights and
+  // the weights of the whole share in one go - the rows arrive first (loads return in order), the norm's sums run
+  // while the weights are still on their way, and the rows are not fetched a second time.
+  constexpr int SP = 8;
+  const bool pre_ok = ((a.N | a.ldo | a.ldr | a.ldr2) & 3) == 0 && EPI != EPI_STORE && EPI != EPI_SWIGLU;
+  EpiPre ep[BT];
+  if (wave == 0 && pre_ok) {
+#pragma unroll
+    for (int t = 0; t < BT; ++t) gemm_epilogue_fetch<EPI>(a, rbase + m + 16 * t, strip, g, ep[t]);
+  }
+  const uint4* wrow = a.wp + (size_t)strip * KS * 64 + lane;
+  f32x4 acc[BT];
+#pragma unroll
+  for (int t = 0; t < BT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
   float rinv[BT], mean[BT];
+  if (NORM == 1 && BT == 1 && per_wave <= SP) {
+    uint4 xv[SP], nw[SP], wv[SP];
+    const int b = rbase + m;
+#pragma unroll
+    for (int c = 0; c < SP; ++c) {
+      const int k0 = 32 * (j0 + c) + 8 * g;
+      const bool in = j0 + c < j1 && b < a.B && k0 < a.K;
+      xv[c] = ldg16(a.x + (in ? (size_t)b * a.ldx + k0 : (size_t)0));
+    }
+#pragma unroll
+    for (int c = 0; c < SP; ++c) {
+      const int k0 = 32 * (j0 + c) + 8 * g;
+      nw[c] = ldg16(a.norm_w + (j0 + c < j1 && k0 < a.K ? k0 : 0));
+    }
+#pragma unroll
+    for (int c = 0; c < SP; ++c) wv[c] = ldg16_nt(wrow + (size_t)min(j0 + c, KS - 1) * 64);
+    __builtin_amdgcn_sched_barrier(0);
+    float part = 0.f;
+#pragma unroll
+    for (int c = 0; c < SP; ++c) {
+      const int k0 = 32 * (j0 + c) + 8 * g;
+      if (j0 + c < j1 && b < a.B && k0 < a.K) part += sumsq8(xv[c]);
+    }
+    part = lanes_sum<16, 16>(part);
+    part = lanes_sum<32, 32>(part);
+    if (g == 0) ssq[wave][m] = part;
+    __syncthreads();
+    float tot = ssq[0][m];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) tot += ssq[w][m];
+    rinv[0] = 1.0f / sqrtf(tot / (float)a.K + a.eps);
+    mean[0] = 0.f;
+#pragma unroll
+    for (int c = 0; c < SP; ++c) {
+      const int k0 = 32 * (j0 + c) + 8 * g;
+      const bool in = j0 + c < j1 && b < a.B && k0 < a.K;
+      const bool inw = j0 + c < j1;
+      const uint4 xn = in ? norm8(xv[c], (k0 < a.K) ? nw[c] : make_uint4(0, 0, 0, 0), rinv[0]) : make_uint4(0, 0, 0, 0);
+      if (inw)
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wv[c]), __builtin_bit_cast(bf16x8, xn),
+                                                         acc[0], 0, 0, 0);
+    }
+  } else {
   if (NORM) {
     float part[BT], psum[BT];
 #pragma unroll
@@ -155,12 +216,6 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(GemmArgs a) {
     }
   }
 
-  f32x4 acc[BT];
-#pragma unroll
-  for (int t = 0; t < BT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-  const uint4* wrow = a.wp + (size_t)strip * KS * 64 + lane;
-
   // A group of CH k-steps: all loads of the group (weights, norm weights, the activations of
   // every 16-row block) are issued before the first product, so their latencies overlap.
   auto group = [&](int j, int n) {  // k-steps j .. j+n-1, n <= CH
@@ -198,6 +253,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(GemmArgs a) {
   int j = j0;
   for (; j + CH <= j1; j += CH) group(j, CH);
   if (j < j1) group(j, j1 - j);
+  }
 
   // Fixed-order cross-wave sum: ((w0 + w1) + w2) + w3 ...
   if (wave > 0) {
@@ -219,7 +275,10 @@ __global__ __launch_bounds__(NW * 64) void skinny_kernel(GemmArgs a) {
 #pragma unroll
   for (int t = 0; t < BT; ++t) {
     const int b = rbase + m + 16 * t;
-    if (b < a.B) gemm_epilogue<EPI>(a, b, strip, g, acc[t]);
+    if (b < a.B) {
+      if (pre_ok) gemm_epilogue<EPI, true>(a, b, strip, g, acc[t], ep[t]);
+      else gemm_epilogue<EPI>(a, b, strip, g, acc[t]);
+    }
   }
 }
 
