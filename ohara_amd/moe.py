@@ -96,7 +96,8 @@ class GroupedMoE:
 
     def fused_ok(self, n: int) -> bool:
         """The four-launch form serves at most 64 experts and 1024 (token, expert) pairs: decode steps."""
-        return self.E <= 64 and n * self.k <= 1024 and self.dim % 8 == 0 and self.dim <= 4096 and self.hidden % 8 == 0
+        return (self.E <= 64 and n * self.k <= 1024 and self.dim % 8 == 0 and self.dim <= 4096 and self.hidden % 8 == 0
+                and (self.shared is None or self.shared[0].n % 8 == 0))
 
     def forward_block(self, h: torch.Tensor, norm_w: torch.Tensor, eps: float) -> torch.Tensor:
         """h (N, dim) bf16 -> h + moe(rmsnorm(h)) (ohara/models/llama.py:200) in four launches: norm + router +
