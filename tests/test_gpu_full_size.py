@@ -157,6 +157,59 @@ def test_d12_batch32_prompt1024_matches_single_sequence_runs(cuda):
     assert agree >= 0.97, agree
 
 
+@pytest.mark.parametrize("B", [1, 8])
+def test_d12_single_launch_decode_over_the_int8_cache(cuda, B):
+    """d12 size, prompts of 1088 tokens (chunks of more than 64 positions: a wave's second tile, and the appended
+    position in it), cache capacity 4096, int8 KV cache: the single-launch kernel - which reads codes and statistics
+    and quantises the appended row itself - against the kernel chain on the same caches, teacher-forced on the chain's
+    tokens: logits to a bf16 ulp, the first layer's appended codes and statistics bit for bit, deeper layers' rows through
+    the values their codes stand for, nothing written behind the last position."""
+    import bench
+    from ohara_amd.llama import Llama
+
+    cfg, st = bench.d12_state(cuda)
+    model = Llama(cfg, st, device=cuda)
+    P, steps = 1088, 6
+    prompt = torch.randint(0, cfg.vocab_size, (B, P), generator=torch.Generator().manual_seed(B + 40)).to(cuda)
+    chain_cache = model.build_kv_cache(B, int8=True)
+    chain = model.session(B, steps + 1, kv_cache=chain_cache, persistent=False)
+    chain.prefill(prompt)
+    want, fed = [chain.logits.float().cpu()], []
+    for _ in range(steps):
+        fed.append(want[-1].argmax(-1))
+        chain.feed(fed[-1].to(cuda))
+        chain.step()
+        want.append(chain.logits.float().cpu())
+    cache = model.build_kv_cache(B, int8=True)
+    sess = model.session(B, steps + 1, kv_cache=cache, persistent=True)
+    assert sess.persistent
+    sess.prefill(prompt)
+    for t in range(steps):
+        sess.feed(fed[t].to(cuda))
+        sess.step()
+        got = sess.logits.float().cpu()
+        scale = want[t + 1].abs().max().item()
+        d = (got - want[t + 1]).abs()
+        assert d.max().item() <= 1.5e-2 * scale and d.mean().item() <= 2.5e-3 * scale, (B, t, d.max().item(), d.mean().item(), scale)
+    sess.check_error()
+    from ohara_amd import ops
+    for l in (0, 5, 11):
+        for name in ("key", "value"):
+            a = getattr(cache[l], name)[:B, P:P + steps].int()
+            b = getattr(chain_cache[l], name)[:B, P:P + steps].int()
+            if l == 0:  # the first layer's rows depend on the fed tokens only
+                assert torch.equal(a, b), name
+            # deeper layers: through the values the codes stand for (a last bit of a row's minimum or maximum moves
+            # every code of the row)
+            va = ops.kv_dequant(cache[l], name, B, P + steps)[:, P:].float()
+            vb = ops.kv_dequant(chain_cache[l], name, B, P + steps)[:, P:].float()
+            scale = vb.abs().max().item()
+            assert (va - vb).abs().max().item() <= 3e-2 * scale and (va - vb).abs().mean().item() <= 4e-3 * scale, (l, name)
+        if l == 0:
+            assert torch.equal(cache[l].stats[:B, :, P:P + steps], chain_cache[l].stats[:B, :, P:P + steps])
+        assert not cache[l].key[:B, P + steps:].any() and not cache[l].stats[:B, :, P + steps:].any()
+
+
 def test_phi2_width_prefill_and_decode_against_the_oracle(cuda):
     """Phi-2's real widths (d 2560, 32 heads of 80 with 32 rotated features, MLP 10240, vocabulary
     51200) on four layers: a 70-token prefill (the tiled kernel's epilogues), cached decode steps of
