@@ -101,6 +101,11 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   float* mrg_w = att + (8 + 4 * D) * G;       // B*H*ns chunk weights
   float* mrg_l = mrg_w + ((B * H * attn_merge_width(a.ns) + 1) & ~1);  // B*H*(merge width) chunk weights before it
   unsigned long long* ptab = reinterpret_cast<unsigned long long*>(mrg_l + ((B * H * attn_merge_width(a.ns) + 1) & ~1));
+  // (polled builds: the ids of the rows this wave embeds are the first thing requested - their rows are what the first
+  // layer's q/k/v workgroups wait for, and a wave's loads return in the order they were issued)
+  // (the single-sequence build only: with more rows the registers this holds across the prefetches are spilled)
+  EmbedPre<2> emb;
+  if constexpr (ONE) embed_request_ids<2>(a.ids, B, emb);
   for (int i = threadIdx.x; i < m.n_layers * 8; i += blockDim.x) {
     const int l = i >> 3, j = i & 7;
     unsigned long long v;
@@ -177,6 +182,9 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     gu.wp = lds_ptr<const uint4>(ptab, 2); gu.norm_w = lds_ptr<const bf16_t>(ptab, 5);
     uint4 g1[2], g2[2];  // norm1's and norm2's weights, the rotary pair: each prefetch writes its own
     uint2 r1, r_unused;
+    if constexpr (ONE) {
+      if (has_qkv) embed_request_rows<2>(m.token_emb, V, d, emb);  // (ahead of the weights: see above)
+    }
     gemm_prefetch<2, 12, E_SWIGLU, 6>(gu, pre, B, g2, r_unused);
     prj.wp = lds_ptr<const uint4>(ptab, 1);
     gemm_prefetch<4, 6, E_RESID, 18>(prj, pre, B, g2, r_unused);
@@ -223,7 +231,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
       // P1: [embedding | poll for the stream] + norm1 + QKV + rotary + append; q and the new k / v rows are left tagged
       qkv.kc = kc; qkv.vc = vc; qkv.out = nullptr; qkv.tout = qt; qkv.tkv = kvt; qkv.trow = a.tg_rq; qkv.tkv_row = a.tg_rkv;
       if (has_qkv) {
-        if (l == 0) stage_norm<2, true, true, false>(xs, ldxs, a.xm, 0, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d, g1);
+        if (l == 0) stage_norm<2, true, true, false, ONE>(xs, ldxs, a.xm, 0, nullptr, a.ids, m.token_emb, V, lds_ptr<const bf16_t>(pl, 4), m.eps, B, d, g1, emb);
         else stage_norm_tagged<2>(xs, xn_prev, pc, m.eps, d, g1, B, ldxs, a.tg_rx);
       }
       __syncthreads();

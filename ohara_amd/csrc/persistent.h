@@ -325,16 +325,45 @@ __device__ __forceinline__ void x_load(const XParts& xp, int b, int n, uint32_t 
 // of a row are issued before any is consumed.  K <= 8 * 64 * NLD elements.
 // PRE: the lane's norm-weight pieces were fetched ahead (gemm_prefetch) and are in gpre[0 .. NLD).
 // PARTS: `parts` is set (the rows are x-mailbox rows plus down-projection sums).
-template <int NLD, bool EMBED, bool PRE, bool PARTS>
+// The embedding rows of a wave (rows wave and wave + 4 of at most eight), requested ahead of everything else a
+// workgroup fetches at the start of a launch: the ids first, the rows as soon as the ids are there.
+template <int NLD>
+struct EmbedPre {
+  int64_t id[2];
+  uint4 v[2][NLD];
+};
+template <int NLD>
+__device__ __forceinline__ void embed_request_ids(const int64_t* ids, int B, EmbedPre<NLD>& e) {
+  const int wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int r = 0; r < 2; ++r) e.id[r] = ldg_i64(ids + min(wave + 4 * r, B - 1));
+}
+template <int NLD>
+__device__ __forceinline__ void embed_request_rows(const bf16_t* table, int vocab, int K, EmbedPre<NLD>& e) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    int64_t id = e.id[r];
+    if (id < 0 || id >= vocab) id = 0;
+#pragma unroll
+    for (int c = 0; c < NLD; ++c) {
+      const int k = (c * 64 + lane) * 8;
+      e.v[r][c] = ldg16(table + (size_t)id * K + (k < K ? k : 0));
+    }
+  }
+}
+
+// EPRE (with EMBED): the rows were requested ahead (embed_request_rows; B <= 8) and are in epre
+template <int NLD, bool EMBED, bool PRE, bool PARTS, bool EPRE = false>
 __device__ __forceinline__ void stage_norm(bf16_t* xs, int ldxs, const char* src, int blk, const float* parts,
                                            const int64_t* ids, const bf16_t* table, int vocab, const bf16_t* nw, float eps,
-                                           int B, int K, const uint4 (&gpre)[NLD]) {
+                                           int B, int K, const uint4 (&gpre)[NLD], const EmbedPre<NLD>& epre = EmbedPre<NLD>()) {
   const XParts xp{src, parts, blk, B, K};
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int b = wave; b < B; b += 4) {
     uint4 v[NLD], g[NLD];
     size_t row_off = 0;
-    if (EMBED) {
+    if (EMBED && !EPRE) {
       int64_t id = ldg_i64(ids + b);
       if (id < 0 || id >= vocab) id = 0;
       row_off = (size_t)id * K;
@@ -347,7 +376,8 @@ __device__ __forceinline__ void stage_norm(bf16_t* xs, int ldxs, const char* src
     for (int c = 0; c < NLD; ++c) {
       const int k = (c * 64 + lane) * 8;
       const int kc = k < K ? k : 0;
-      if (EMBED) v[c] = ldg16(table + row_off + kc);
+      if (EMBED && EPRE) v[c] = epre.v[b >= 4 ? 1 : 0][c];
+      else if (EMBED) v[c] = ldg16(table + row_off + kc);
       else x_fetch<8, PARTS>(xp, b, kc, raw[c]);
       g[c] = PRE ? gpre[c] : ldg16(nw + kc);
     }
