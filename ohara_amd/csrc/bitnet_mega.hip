@@ -12,9 +12,11 @@
 //   P5  codes + ff.down, K split over two groups of workgroups; the int32 partial sums are exact, so
 //       whoever needs the residual stream next adds them, scales and rounds as one BitLinear would
 // then final norm + vocabulary projection (bf16, the bf16 kernel's phase) and the arg-max.
-// Every workgroup derives the codes of the rows it multiplies itself (a row is 2-11 KB; the three
-// passes over it cost about as much as one hand-off), with the reduction orders of the stand-alone
-// BitLinear kernels, so the integer accumulators are those kernels' accumulators.
+// A single sequence: every workgroup derives the codes of the row it multiplies itself (a row is 2-11 KB;
+// the three passes over it, spread over the workgroup, cost about as much as one hand-off).  Two to eight
+// sequences: each (BitLinear, row) pair is quantised once, by one workgroup, and handed to the others
+// through a code mailbox and one more grid barrier per GEMM phase.  Either way the reduction orders are
+// those of the stand-alone BitLinear kernels, so the integer accumulators are those kernels' accumulators.
 #include <vector>
 
 #include "persistent.h"
@@ -45,6 +47,9 @@ struct BitMegaArgs {
   char* am;        // NL act-mailboxes
   float* pm;       // NL attention-partial mailboxes
   int32_t* dm;     // NL mailboxes of the down projection's int32 partial sums [part][strip][row][16]
+  int8_t* cq;      // NL code mailboxes (batch > 1): the code rows of the seven BitLinears, each quantised by one workgroup
+  float* cs;       // NL x [7][16] {s, sum q} pairs of those rows (eight used)
+  size_t cq_stride;
   float* ds;       // NL x 32 floats (a 128-byte line per layer: one writer, written before it is read):
                    // the activation scale s of every row of the down projection
   size_t xm_stride, qm_stride, am_stride, pm_stride, dm_stride;
@@ -141,10 +146,6 @@ __device__ __forceinline__ float bit_sumsq8(uint4 v) {
 // pre_w,] the BitLinear's RMSNorm with nw, s = 127 / max|x_hat|, q = clamp(rint(x_hat * s), -128, 127).
 // Which thread owns which 8-value piece and the order of every reduction are those of the stand-alone
 // kernels (block_quant_row / wave_quant_row in csrc/bitlinear.hip), so the codes are the same codes.
-struct RowQ {
-  float s;
-  int sumq;
-};
 
 // LDS of the kernel.  `codes`: up to two code sets (gate and up) of B rows x ldq bytes; `stage`: B bf16
 // rows of the model width (the merged attention output, the normalised final stream).
@@ -154,7 +155,6 @@ struct BitLds {
   size_t set;       // bytes between the two code sets of the current phase
   bf16_t* stage;
   int ldm;          // elements between the rows of the merged attention output
-  int ldst;         // elements between the rows parked for ff.down's codes at batch > 1
   __device__ __forceinline__ void shape(int B, int K) {
     ldq = (((K + 255) >> 8) << 8) + 16;
     set = (size_t)B * ldq;
@@ -162,8 +162,54 @@ struct BitLds {
   float* s_s;       // [2][16] activation scales
   int* s_sum;       // [2][16] sums of the codes
   float* red;       // 4 KiB: cross-wave sums
-  int* sumw;        // [2][4] batch 1: per-wave shares of the sums of the codes
+  int* sumw;        // [2][4] per-wave shares of the sums of the codes (and of the maximum, when a row is quantised once)
 };
+
+// The arithmetic of a row's codes, two values at a time.  x_hat = bf16(bf16(h * rinv) * nw) is formed once and
+// kept as packed bf16 pairs; its largest magnitude is taken on the 15-bit patterns (for bf16 values the
+// order of the magnitudes is the order of the patterns); q = rint(x_hat * s) is read from the low mantissa
+// bits of x_hat * s + 1.5 * 2^23 (that addition rounds to the nearest integer, ties to even, as rintf does;
+// |x_hat * s| <= 127 * (1 + 2^-22), so the clamp of bitnet.py:33 never acts and the low byte is the code).
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t bit_xhat2(uint32_t h, uint32_t w, float rinv) {
+  return pack_bf(rbf(lo_bf(h) * rinv) * lo_bf(w), rbf(hi_bf(h) * rinv) * hi_bf(w));
+}
+__device__ __forceinline__ uint4 bit_xhat8(uint4 h, uint4 w, float rinv) {
+  return make_uint4(bit_xhat2(h.x, w.x, rinv), bit_xhat2(h.y, w.y, rinv), bit_xhat2(h.z, w.z, rinv), bit_xhat2(h.w, w.w, rinv));
+}
+__device__ __forceinline__ uint32_t bit_mag_max2(uint32_t m, uint32_t xh) {
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2_t, m),
+                                                                 __builtin_bit_cast(u16x2_t, xh & 0x7fff7fffu)));
+}
+__device__ __forceinline__ uint32_t bit_mag_max8(uint32_t m, uint4 xh) {
+  return bit_mag_max2(bit_mag_max2(bit_mag_max2(bit_mag_max2(m, xh.x), xh.y), xh.z), xh.w);
+}
+__device__ __forceinline__ float bit_mag_float(uint32_t m) { return __uint_as_float(max(m & 0xffffu, m >> 16) << 16); }
+#define BIT_RINT_MAGIC 12582912.0f      // 1.5 * 2^23
+#define BIT_RINT_MAGIC_BITS 0x4B400000u
+// eight packed x_hat values -> their eight code bytes; the raw words (code + BIT_RINT_MAGIC_BITS) are added to `sq`
+__device__ __forceinline__ uint2 bit_codes8(uint4 xh, float s, uint32_t& sq) {
+  const uint32_t u[4] = {xh.x, xh.y, xh.z, xh.w};
+  uint32_t c[8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float p0 = lo_bf(u[j]) * s, p1 = hi_bf(u[j]) * s;
+    // the products are rounded before the addition, as rintf's argument is: the empty statement keeps the compiler from
+    // fusing the two into one multiply-add (it does so even for __fadd_rn(__fmul_rn(..))), which rounds once and sends
+    // the frequent tie x_hat = max / 2 -> 63.5 to either side
+    asm("" : "+v"(p0), "+v"(p1));
+    c[2 * j] = __float_as_uint(p0 + BIT_RINT_MAGIC);
+    c[2 * j + 1] = __float_as_uint(p1 + BIT_RINT_MAGIC);
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) sq += c[j];
+  // byte 0 of four words -> one word (v_perm_b32: selector bytes 0-3 take from the second operand, 4-7 from the first, 0x0c is zero)
+  const uint32_t lo = __builtin_amdgcn_perm(c[1], c[0], 0x0c0c0400u) | __builtin_amdgcn_perm(c[3], c[2], 0x04000c0cu);
+  const uint32_t hi = __builtin_amdgcn_perm(c[5], c[4], 0x0c0c0400u) | __builtin_amdgcn_perm(c[7], c[6], 0x04000c0cu);
+  return make_uint2(lo, hi);
+}
+// the sum of the codes from the sum of `n` raw words
+__device__ __forceinline__ int bit_code_sum(uint32_t sq, int n) { return (int)(sq - (uint32_t)n * BIT_RINT_MAGIC_BITS); }
 
 // ---- batch 1: the row in registers -------------------------------------------------------------
 // Thread t owns the 8-value pieces t, t + 256, ... (NP of them; pieces beyond the row are zero and
@@ -212,42 +258,27 @@ __device__ __forceinline__ void row1_codes(const uint4 (&h)[NP], const uint4 (&n
 #pragma unroll
   for (int i = 0; i < NP; ++i) ss += bit_sumsq8(h[i]);
   const float rinv = 1.0f / sqrtf(row1_sum(ss, red) / (float)K + eps);
-  // x_hat = bf16(bf16(h * rinv) * nw) is formed twice (for the maximum, then for the codes) instead
-  // of being kept: two multiplies per value against NP more live registers per row
-  float mx = 0.f;
+  uint4 xh[NP];
+  uint32_t mg = 0u;
 #pragma unroll
   for (int i = 0; i < NP; ++i) {
-    const uint32_t uu[4] = {h[i].x, h[i].y, h[i].z, h[i].w}, ww[4] = {nw[i].x, nw[i].y, nw[i].z, nw[i].w};
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float a0 = rbf(rbf(lo_bf(uu[j]) * rinv) * lo_bf(ww[j]));
-      const float a1 = rbf(rbf(hi_bf(uu[j]) * rinv) * hi_bf(ww[j]));
-      mx = fmaxf(mx, fmaxf(fabsf(a0), fabsf(a1)));
-    }
+    xh[i] = bit_xhat8(h[i], nw[i], rinv);
+    mg = bit_mag_max8(mg, xh[i]);
   }
-  mx = wave_max(mx);
+  float mx = wave_max(bit_mag_float(mg));
   __syncthreads();
   if (lane == 0) red[wave] = mx;
   __syncthreads();
   mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
   const float s = 127.0f / fmaxf(mx, 1e-5f);
-  int sq = 0;
+  uint32_t sqw = 0u;
 #pragma unroll
   for (int i = 0; i < NP; ++i) {
-    const uint32_t uu[4] = {h[i].x, h[i].y, h[i].z, h[i].w}, ww[4] = {nw[i].x, nw[i].y, nw[i].z, nw[i].w};
-    uint32_t pk[2] = {0u, 0u};
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float hv = (j & 1) ? hi_bf(uu[j >> 1]) : lo_bf(uu[j >> 1]);
-      const float wv = (j & 1) ? hi_bf(ww[j >> 1]) : lo_bf(ww[j >> 1]);
-      const float v = rbf(rbf(hv * rinv) * wv);
-      const int qi = (int)fminf(fmaxf(rintf(v * s), -128.f), 127.f);
-      sq += qi;
-      pk[j >> 2] |= ((uint32_t)qi & 0xffu) << (8 * (j & 3));
-    }
+    const uint2 pk = bit_codes8(xh[i], s, sqw);
     const int p = tid + 256 * i;
-    if (p < pieces) sts8(xq + (size_t)p * 8, make_uint2(pk[0], pk[1]));
+    if (p < pieces) sts8(xq + (size_t)p * 8, pk);
   }
+  int sq = bit_code_sum(sqw, NP * 8);
   sq = lanes_sum<32, 1>(sq);
   if (lane == 0) sumw[wave] = sq;
   if (tid == 0) *s_out = s;
@@ -312,190 +343,119 @@ __device__ __forceinline__ void bit_stage_row1_pre(const BitLds& L, int nsets, i
   // the product that follows passes a workgroup barrier before anyone reads s_sum
 }
 
-// ---- batch > 1: a row per wave, in registers ---------------------------------------------------
-// Lane l owns the pieces l, l + 64, ... (NP of them); the norm weights are fetched once per wave and
-// serve all its rows.
-template <int NP, typename F>
-__device__ __forceinline__ void roww_load(uint4 (&r)[NP], int pieces, F f) {
-#pragma unroll
-  for (int i = 0; i < NP; ++i) {
-    const int p = (int)(threadIdx.x & 63) + 64 * i;
-    r[i] = p < pieces ? f(p) : make_uint4(0, 0, 0, 0);
-  }
-}
-template <int NP>
-__device__ __forceinline__ void roww_block_norm(uint4 (&v)[NP], const uint4 (&w)[NP], int K, float eps) {
-  float ss = 0.f;
-#pragma unroll
-  for (int i = 0; i < NP; ++i) ss += bit_sumsq8(v[i]);
-  const float rinv0 = 1.0f / sqrtf(wave_sum(ss) / (float)K + eps);
-#pragma unroll
-  for (int i = 0; i < NP; ++i) {
-    const uint32_t uu[4] = {v[i].x, v[i].y, v[i].z, v[i].w}, ww[4] = {w[i].x, w[i].y, w[i].z, w[i].w};
-    uint32_t o[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      o[j] = pack_bf(rbf(lo_bf(uu[j]) * rinv0) * lo_bf(ww[j]), rbf(hi_bf(uu[j]) * rinv0) * hi_bf(ww[j]));
-    v[i] = make_uint4(o[0], o[1], o[2], o[3]);
-  }
-}
-template <int NP>
-__device__ __forceinline__ RowQ roww_codes(const uint4 (&h)[NP], const uint4 (&nw)[NP], int pieces, int K, float eps,
-                                           int8_t* xq) {
-  const int lane = threadIdx.x & 63;
-  float ss = 0.f;
-#pragma unroll
-  for (int i = 0; i < NP; ++i) ss += bit_sumsq8(h[i]);
-  const float rinv = 1.0f / sqrtf(wave_sum(ss) / (float)K + eps);
-  // x_hat = bf16(bf16(h * rinv) * nw) is formed twice (for the maximum, then for the codes) instead
-  // of being kept: two multiplies per value against NP more live registers per row
-  float mx = 0.f;
-#pragma unroll
-  for (int i = 0; i < NP; ++i) {
-    const uint32_t uu[4] = {h[i].x, h[i].y, h[i].z, h[i].w}, ww[4] = {nw[i].x, nw[i].y, nw[i].z, nw[i].w};
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float a0 = rbf(rbf(lo_bf(uu[j]) * rinv) * lo_bf(ww[j]));
-      const float a1 = rbf(rbf(hi_bf(uu[j]) * rinv) * hi_bf(ww[j]));
-      mx = fmaxf(mx, fmaxf(fabsf(a0), fabsf(a1)));
-    }
-  }
-  mx = wave_max(mx);
-  const float s = 127.0f / fmaxf(mx, 1e-5f);
-  int sq = 0;
-#pragma unroll
-  for (int i = 0; i < NP; ++i) {
-    const uint32_t uu[4] = {h[i].x, h[i].y, h[i].z, h[i].w}, ww[4] = {nw[i].x, nw[i].y, nw[i].z, nw[i].w};
-    uint32_t pk[2] = {0u, 0u};
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float hv = (j & 1) ? hi_bf(uu[j >> 1]) : lo_bf(uu[j >> 1]);
-      const float wv = (j & 1) ? hi_bf(ww[j >> 1]) : lo_bf(ww[j >> 1]);
-      const float v = rbf(rbf(hv * rinv) * wv);
-      const int qi = (int)fminf(fmaxf(rintf(v * s), -128.f), 127.f);
-      sq += qi;
-      pk[j >> 2] |= ((uint32_t)qi & 0xffu) << (8 * (j & 3));
-    }
-    const int p = lane + 64 * i;
-    if (p < pieces) sts8(xq + (size_t)p * 8, make_uint2(pk[0], pk[1]));
-  }
-  sq = lanes_sum<32, 1>(sq);
-  return RowQ{s, sq};
-}
-// B rows from `load(b, piece) -> uint4` into one or two code sets.  Every thread of the workgroup calls.
-template <int NP, typename Load>
-__device__ __forceinline__ void bit_stage_roww(const BitLds& L, int nsets, int B, int K, const bf16_t* pre_w,
-                                               const bf16_t* nw0, const bf16_t* nw1, float eps, Load load) {
+// ---- batch > 1: every (BitLinear, row) pair is quantised once ---------------------------------
+// With B rows a workgroup that derived all the codes itself would spend 8 - 17 us per phase on them at eight rows
+// (the three passes are instruction-bound with one wave per SIMD), 256 times over.  Instead ONE workgroup
+// per (BitLinear, row) pair derives the row's codes with all its threads (thread t owns the pieces t, t + 256, ...),
+// stores them and {s, sum q} in a per-layer mailbox, a grid barrier follows, and every workgroup copies the code
+// rows it multiplies into its LDS.  The sums of squares keep the order of the stand-alone kernels' wave-owned
+// rows (wave_quant_row in csrc/bitlinear.hip: lane l adds the pieces l, l + 64, ... in turn, then the wave's
+// butterfly): the per-piece sums go through LDS and the first wave adds them in that order; the maximum and the
+// sum of the codes are exact in any order.  So the codes are still those kernels' codes.
+__host__ __device__ inline size_t bit_cq_al(size_t v) { return (v + 255) & ~(size_t)255; }
+template <int NP1, typename Load>
+__device__ __forceinline__ void bit_quant_once(const BitLds& L, int K, const bf16_t* pre_w, const bf16_t* nw, float eps,
+                                               Load load, int8_t* cq_row, int ldq, float* stat) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int pieces = K >> 3;
-  uint4 pw[NP], n0[NP], n1[NP];
-  if (pre_w) roww_load(pw, pieces, [&](int p) { return ldg16(pre_w + (size_t)p * 8); });
-  roww_load(n0, pieces, [&](int p) { return ldg16(nw0 + (size_t)p * 8); });
-  if (nsets == 2) roww_load(n1, pieces, [&](int p) { return ldg16(nw1 + (size_t)p * 8); });
-  __syncthreads();  // whoever still reads the previous codes or scales is done
-  {
-    const int pad8 = (L.ldq - K) >> 3;
-    for (int i = tid; i < nsets * B * pad8; i += 256) {
-      const int r = i / pad8, c = i - r * pad8;  // r = set * B + row; the sets are B rows apart
-      sts8(L.codes + (size_t)r * L.ldq + K + c * 8, make_uint2(0, 0));
+  uint4 x[NP1], pw[NP1], n0[NP1];
+  row1_load(x, pieces, load);
+  if (pre_w) row1_norm_fetch<NP1>(pw, pieces, pre_w);
+  row1_norm_fetch<NP1>(n0, pieces, nw);
+  float* psum = L.red;  // one sum of squares per piece (at most 768), the result at [1000]
+  auto rinv_of = [&](const uint4 (&v)[NP1]) {
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NP1; ++i) {
+      const int p = tid + 256 * i;
+      if (p < pieces) psum[p] = bit_sumsq8(v[i]);
     }
-  }
-  for (int b = wave; b < B; b += 4) {
-    uint4 x[NP];
-    roww_load(x, pieces, [&](int p) { return load(b, p); });
-    if (pre_w) roww_block_norm(x, pw, K, eps);
-    const RowQ o0 = roww_codes(x, n0, pieces, K, eps, L.codes + (size_t)b * L.ldq);
-    if (lane == 0) {
-      L.s_s[b] = o0.s;
-      L.s_sum[b] = o0.sumq;
-    }
-    if (nsets == 2) {
-      const RowQ o1 = roww_codes(x, n1, pieces, K, eps, L.codes + L.set + (size_t)b * L.ldq);
-      if (lane == 0) {
-        L.s_s[16 + b] = o1.s;
-        L.s_sum[16 + b] = o1.sumq;
+    __syncthreads();
+    if (wave == 0) {
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4 * NP1; ++i) {
+        const int p = lane + 64 * i;
+        ss += p < pieces ? psum[p] : 0.f;
       }
+      ss = wave_sum(ss);
+      if (lane == 0) psum[1000] = 1.0f / sqrtf(ss / (float)K + eps);
     }
+    __syncthreads();
+    return psum[1000];
+  };
+  if (pre_w) {  // block-level RMSNorm (norm.py:16-21)
+    const float r0 = rinv_of(x);
+#pragma unroll
+    for (int i = 0; i < NP1; ++i) x[i] = bit_xhat8(x[i], pw[i], r0);
   }
+  const float rinv = rinv_of(x);
+  uint4 xh[NP1];
+  uint32_t mg = 0u;
+#pragma unroll
+  for (int i = 0; i < NP1; ++i) {
+    xh[i] = bit_xhat8(x[i], n0[i], rinv);
+    mg = bit_mag_max8(mg, xh[i]);
+  }
+  float mx = wave_max(bit_mag_float(mg));
+  int* iw = L.sumw;
+  if (lane == 0) iw[wave] = __float_as_int(mx);
   __syncthreads();
+  mx = fmaxf(fmaxf(__int_as_float(iw[0]), __int_as_float(iw[1])), fmaxf(__int_as_float(iw[2]), __int_as_float(iw[3])));
+  const float s = 127.0f / fmaxf(mx, 1e-5f);
+  uint32_t sqw = 0u;
+#pragma unroll
+  for (int i = 0; i < NP1; ++i) {
+    const uint2 pk = bit_codes8(xh[i], s, sqw);
+    const int p = tid + 256 * i;
+    if (p < pieces) st_coh8(cq_row + (size_t)p * 8, pk);
+  }
+  for (int c = K + tid * 8; c < ldq; c += 2048) st_coh8(cq_row + c, make_uint2(0, 0));  // the columns up to the chunk's end
+  const int sq = lanes_sum<32, 1>(bit_code_sum(sqw, NP1 * 8));
+  if (lane == 0) iw[4 + wave] = sq;
+  __syncthreads();
+  if (tid == 0) st_coh8(stat, make_uint2(__float_as_uint(s), (uint32_t)((iw[4] + iw[5]) + (iw[6] + iw[7]))));
 }
-
-// The same for rows too long for registers (ff.down's input at batch > 1: one code set, no block
-// norm): the wave parks its rows in LDS (`stage`, row b at b * ldst) as they arrive - all loads of all
-// its rows in flight together - and walks them three times from there; only the norm weights stay in
-// registers.  A lane reads back only what it wrote itself, so the rows need no barrier.
-template <int NP, typename Load>
-__device__ __forceinline__ void bit_stage_roww_lds(const BitLds& L, int B, int K, const bf16_t* nw0, float eps, Load load) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int pieces = K >> 3;
-  uint4 n0[NP];
-  roww_load(n0, pieces, [&](int p) { return ldg16(nw0 + (size_t)p * 8); });
-  __syncthreads();  // whoever still reads the previous codes, scales or staged rows is done
-  {
-    const int pad8 = (L.ldq - K) >> 3;
-    for (int i = tid; i < B * pad8; i += 256) {
-      const int r = i / pad8, c = i - r * pad8;
-      sts8(L.codes + (size_t)r * L.ldq + K + c * 8, make_uint2(0, 0));
+// Unit u of `units` goes to workgroup u * (nwg / units) (spread over the grid; with fewer workgroups than units they loop).
+template <typename F>
+__device__ __forceinline__ void bit_for_units(int units, int nwg, F fn) {
+  const int stride = max(1, nwg / units);
+  const int nq = (nwg + stride - 1) / stride;
+  if ((int)blockIdx.x % stride == 0)
+    for (int u = (int)blockIdx.x / stride; u < units; u += nq) fn(u);
+}
+// The code rows of `nsets` consecutive BitLinears (B rows each; the mailbox has the row and set strides of the LDS
+// copy) and their scales -> LDS.  Whole rows are one flat copy; a K partition [c0, c1) of 256-column chunks (at most
+// 16 of them) is copied row by row.  Every thread of the workgroup calls.
+__device__ __forceinline__ void bit_codes_fetch(const BitLds& L, int nsets, int B, const int8_t* cq, const float* st, int c0,
+                                                int c1, bool whole) {
+  const int tid = threadIdx.x;
+  __syncthreads();  // whoever still reads the previous codes or scales is done
+  if (whole) {
+    const int n16 = (int)((size_t)nsets * B * L.ldq) >> 4;
+    for (int i0 = 0; i0 < n16; i0 += 256 * 6) {
+      uint4 v[6];
+#pragma unroll
+      for (int u = 0; u < 6; ++u) v[u] = ldg16(cq + (size_t)min(i0 + u * 256 + tid, n16 - 1) * 16);
+#pragma unroll
+      for (int u = 0; u < 6; ++u)
+        if (i0 + u * 256 + tid < n16) sts16(L.codes + (size_t)(i0 + u * 256 + tid) * 16, v[u]);
     }
+  } else {
+    const int segs = (c1 - c0) * 16;  // 16-byte pieces per row: at most 256
+    uint4 v[8];
+#pragma unroll
+    for (int b = 0; b < 8; ++b)
+      v[b] = ldg16(cq + (size_t)min(b, B - 1) * L.ldq + (size_t)c0 * 256 + (size_t)min(tid, segs - 1) * 16);
+#pragma unroll
+    for (int b = 0; b < 8; ++b)
+      if (b < B && tid < segs) sts16(L.codes + (size_t)b * L.ldq + (size_t)c0 * 256 + (size_t)tid * 16, v[b]);
   }
-  for (int b = wave; b < B; b += 4) {
-    bf16_t* row = L.stage + (size_t)b * L.ldst;
-#pragma unroll
-    for (int i = 0; i < NP; ++i) {
-      const int p = lane + 64 * i;
-      if (p < pieces) sts16(row + p * 8, load(b, p));
-    }
-  }
-  for (int b = wave; b < B; b += 4) {
-    const bf16_t* row = L.stage + (size_t)b * L.ldst;
-    int8_t* xq = L.codes + (size_t)b * L.ldq;
-    float ss = 0.f;
-#pragma unroll
-    for (int i = 0; i < NP; ++i) {
-      const int p = lane + 64 * i;
-      ss += bit_sumsq8(p < pieces ? lds16(row + p * 8) : make_uint4(0, 0, 0, 0));
-    }
-    const float rinv = 1.0f / sqrtf(wave_sum(ss) / (float)K + eps);
-    float mx = 0.f;
-#pragma unroll
-    for (int i = 0; i < NP; ++i) {
-      const int p = lane + 64 * i;
-      const uint4 h = p < pieces ? lds16(row + p * 8) : make_uint4(0, 0, 0, 0);
-      const uint32_t uu[4] = {h.x, h.y, h.z, h.w}, ww[4] = {n0[i].x, n0[i].y, n0[i].z, n0[i].w};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float a0 = rbf(rbf(lo_bf(uu[j]) * rinv) * lo_bf(ww[j]));
-        const float a1 = rbf(rbf(hi_bf(uu[j]) * rinv) * hi_bf(ww[j]));
-        mx = fmaxf(mx, fmaxf(fabsf(a0), fabsf(a1)));
-      }
-    }
-    mx = wave_max(mx);
-    const float s = 127.0f / fmaxf(mx, 1e-5f);
-    int sq = 0;
-#pragma unroll
-    for (int i = 0; i < NP; ++i) {
-      const int p = lane + 64 * i;
-      if (p < pieces) {
-        const uint4 h = lds16(row + p * 8);
-        const uint32_t uu[4] = {h.x, h.y, h.z, h.w}, ww[4] = {n0[i].x, n0[i].y, n0[i].z, n0[i].w};
-        uint32_t pk[2] = {0u, 0u};
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const float hv = (j & 1) ? hi_bf(uu[j >> 1]) : lo_bf(uu[j >> 1]);
-          const float wv = (j & 1) ? hi_bf(ww[j >> 1]) : lo_bf(ww[j >> 1]);
-          const float v = rbf(rbf(hv * rinv) * wv);
-          const int qi = (int)fminf(fmaxf(rintf(v * s), -128.f), 127.f);
-          sq += qi;
-          pk[j >> 2] |= ((uint32_t)qi & 0xffu) << (8 * (j & 3));
-        }
-        sts8(xq + (size_t)p * 8, make_uint2(pk[0], pk[1]));
-      }
-    }
-    sq = lanes_sum<32, 1>(sq);
-    if (lane == 0) {
-      L.s_s[b] = s;
-      L.s_sum[b] = sq;
-    }
+  if (tid < nsets * B) {
+    const int set = tid / B, b = tid - set * B;
+    const uint2 v = ldg8(st + set * 32 + b * 2);
+    L.s_s[set * 16 + b] = __uint_as_float(v.x);
+    L.s_sum[set * 16 + b] = (int)v.y;
   }
   __syncthreads();
 }
@@ -632,9 +592,9 @@ __device__ void bit_stage_final_norm(bf16_t* xs, int ldxs, const BitX& x, const 
 // ---------------------------------------------------------------------------------------
 // the kernel
 // ---------------------------------------------------------------------------------------
-// ONE: a single sequence.  The block-owned-row staging is then the only one compiled in, the
-// wave-owned-row staging otherwise, which keeps either kernel's layer loop much smaller than one
-// that holds both.
+// ONE: a single sequence.  The staging of the workgroup's own row is then the only one compiled in, the
+// quantise-once sub-phases and the code fetch otherwise, which keeps either kernel's layer loop much smaller
+// than one that holds both.
 // PROFILE: with the phase stamps (measurement builds of the head-dim-128 kernels only).
 template <int D, int G, bool ONE, bool PROFILE = false>
 __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
@@ -655,9 +615,7 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
   L.codes = reinterpret_cast<int8_t*>(smem);
   L.shape(B, d);
   size_t off = (codes_bytes + 255) & ~(size_t)255;
-  const int KpF = ((F + 255) >> 8) << 8;
-  const size_t stage_bytes = max((size_t)B * (dmax + 8) * 2, (!ONE && F > 2048) ? (size_t)B * KpF * 2 : (size_t)0);
-  L.ldst = KpF;
+  const size_t stage_bytes = (size_t)B * (dmax + 8) * 2;
   L.stage = reinterpret_cast<bf16_t*>(smem + off);
   L.ldm = dmax + 8;
   off += (stage_bytes + 255) & ~(size_t)255;
@@ -697,6 +655,13 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
   const int KCd = (d + 255) >> 8, KCo = (HD + 255) >> 8, KCf = (F + 255) >> 8;
   const int ns_q = HD / 16, ns_kv = (Hkv * D) / 16, ns_d = (d + 15) / 16, ns_f = (F + 15) / 16;
   const bool ok_pos = pos >= 0 && pos < m.t_max;
+  // batch > 1: where the code rows of the seven BitLinears start in a layer's code mailbox (B rows each)
+  const int ldq_d = (KCd << 8) + 16, ldq_o = (KCo << 8) + 16, ldq_f = (KCf << 8) + 16;
+  // (a group of sets that one sub-phase writes starts on its own 256 bytes: a cache line that an earlier phase's readers
+  // fetched while part of it was still unwritten would be found stale by the later phase's plain loads)
+  const size_t cq_o = bit_cq_al((size_t)3 * B * ldq_d), cq_g = bit_cq_al(cq_o + (size_t)B * ldq_o);
+  const size_t cq_dn = bit_cq_al(cq_g + (size_t)2 * B * ldq_d);
+  ProfT<false> nopf(nullptr);  // the barrier after a quantising sub-phase is not stamped
 
   GemmP lm{};
   lm.N = V; lm.K = d; lm.nstrips = (V + 15) / 16; lm.out = reinterpret_cast<char*>(a.logits); lm.ldo = V;
@@ -742,6 +707,8 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
     char* a_l = a.am + (size_t)l * a.am_stride;
     float* p_l = a.pm + (size_t)l * a.pm_stride;
     int32_t* d_l = a.dm + (size_t)l * a.dm_stride;
+    int8_t* cq_l = a.cq + (size_t)l * a.cq_stride;
+    float* cs_l = a.cs + (size_t)l * 256;  // {s, sum q} of row b of set i at (i * 32 + b * 2): a 128-byte line per set
     // the stream entering this layer
     BitX xin{};
     xin.B = B; xin.N = d; xin.blk = a.blk_x;
@@ -758,20 +725,28 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
 
     // ---- P1: Q, K, V + rotary + append ----
     L.shape(B, d);
+    auto load_in = [&](int b, int p) {
+      uint32_t w[4];
+      bitx_load<8>(xin, b, p * 8, w);
+      return make_uint4(w[0], w[1], w[2], w[3]);
+    };
+    if (!ONE) {
+      bit_for_units(3 * B, nwg, [&](int u) {
+        const int which = u / B, b = u - which * B;
+        bit_quant_once<1>(L, d, norm1, reinterpret_cast<const bf16_t*>(gptr(LY.nw[which])), m.eps,
+                          [&](int p) { return load_in(b, p); }, cq_l + (size_t)u * ldq_d, ldq_d, cs_l + which * 32 + b * 2);
+      });
+      gs.arrive(nopf);
+      gs.wait(nopf);
+    }
     if (2 * p1_gi < p1_nstr) {
       const int which = p1_which;
       const uint4* wp = reinterpret_cast<const uint4*>(gptr(LY.w[which]));
-      const bf16_t* nw = reinterpret_cast<const bf16_t*>(gptr(LY.nw[which]));
-      auto load_in = [&](int b, int p) {
-        uint32_t w[4];
-        bitx_load<8>(xin, b, p * 8, w);
-        return make_uint4(w[0], w[1], w[2], w[3]);
-      };
       if (ONE) {
         auto load0 = [&](int p) { return load_in(0, p); };
         bit_stage_row1_pre<1>(L, 1, d, true, npw, reinterpret_cast<const uint4(&)[1]>(nn0), nn1, m.eps, load0);
       } else {
-        bit_stage_roww<4>(L, 1, B, d, norm1, nw, nullptr, m.eps, load_in);
+        bit_codes_fetch(L, 1, B, cq_l + (size_t)which * B * ldq_d, cs_l + which * 32, 0, KCd, true);
       }
       for (int s0 = 2 * p1_gi; s0 < p1_nstr; s0 += 2 * p1_gsz) {
         const bool first = s0 == 2 * p1_gi;
@@ -825,23 +800,33 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
     gs.wait(pf);
     // ---- P3: merge + attn.proj + residual ----
     L.shape(B, HD);
+    if (!ONE) {  // one workgroup per row merges the row's chunks and derives its codes
+      bit_for_units(B, nwg, [&](int b) {
+        bf16_t* xs = L.stage;
+        __syncthreads();
+        stage_attn_merge_any<false>(a.ns, xs, L.ldm, p_l + (size_t)b * H * OHARA_MEGA_NS * (D + 32), 1, H, D, mrg_w, mrg_l);
+        __syncthreads();
+        bit_quant_once<1>(L, HD, nullptr, reinterpret_cast<const bf16_t*>(gptr(LY.nw[BO])), m.eps,
+                          [&](int p) { return lds16(xs + p * 8); }, cq_l + cq_o + (size_t)b * ldq_o, ldq_o, cs_l + BO * 32 + b * 2);
+      });
+      gs.arrive(nopf);
+      gs.wait(nopf);
+    }
     for (int strip = blockIdx.x; strip < ns_d; strip += nwg) {
       const bool first = strip == (int)blockIdx.x;
       if (first) {
-        bf16_t* xs = L.stage;
-        const int ldxs = L.ldm;
-        // a single sequence always runs with 16 chunks unless there are more than 16 KV heads: that
-        // merge is part of the kernel (a call would wait for the weights already in flight)
-        if (ONE && a.ns == 16 && B * HD > 4 * 256) stage_attn_merge<16>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
-        else stage_attn_merge_any<false>(a.ns, xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
-        __syncthreads();
-        const bf16_t* nwo = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BO]));
         if (ONE) {
+          bf16_t* xs = L.stage;
+          const int ldxs = L.ldm;
+          // a single sequence always runs with 16 chunks unless there are more than 16 KV heads: that
+          // merge is part of the kernel (a call would wait for the weights already in flight)
+          if (a.ns == 16 && B * HD > 4 * 256) stage_attn_merge<16>(xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
+          else stage_attn_merge_any<false>(a.ns, xs, ldxs, p_l, B, H, D, mrg_w, mrg_l);
+          __syncthreads();
           auto load0 = [&](int p) { return lds16(xs + p * 8); };
           bit_stage_row1_pre<1>(L, 1, HD, false, npw, reinterpret_cast<const uint4(&)[1]>(nn0), nn1, m.eps, load0);
         } else {
-          auto loadb = [&](int b, int p) { return lds16(xs + (size_t)b * ldxs + p * 8); };
-          bit_stage_roww<4>(L, 1, B, HD, nullptr, nwo, nullptr, m.eps, loadb);
+          bit_codes_fetch(L, 1, B, cq_l + cq_o, cs_l + BO * 32, 0, KCo, true);
         }
       }
       i32x4 acc;
@@ -875,21 +860,29 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
     gs.wait(pf);
     // ---- P4: norm2 + ff.gate, ff.up + SwiGLU; two strips at a time, two waves each ----
     L.shape(B, d);
+    BitX xmid{};
+    xmid.B = B; xmid.N = d; xmid.blk = a.blk_x; xmid.xmid = x_mid;
+    auto load_mid = [&](int b, int p) {
+      uint32_t w[4];
+      bitx_load<8>(xmid, b, p * 8, w);
+      return make_uint4(w[0], w[1], w[2], w[3]);
+    };
+    if (!ONE) {
+      bit_for_units(2 * B, nwg, [&](int u) {
+        const int set = u / B, b = u - set * B;
+        bit_quant_once<1>(L, d, norm2, reinterpret_cast<const bf16_t*>(gptr(LY.nw[BG + set])), m.eps,
+                          [&](int p) { return load_mid(b, p); }, cq_l + cq_g + (size_t)u * ldq_d, ldq_d,
+                          cs_l + (BG + set) * 32 + b * 2);
+      });
+      gs.arrive(nopf);
+      gs.wait(nopf);
+    }
     if (2 * (int)blockIdx.x < ns_f) {
-      BitX xmid{};
-      xmid.B = B; xmid.N = d; xmid.blk = a.blk_x; xmid.xmid = x_mid;
-      auto load_mid = [&](int b, int p) {
-        uint32_t w[4];
-        bitx_load<8>(xmid, b, p * 8, w);
-        return make_uint4(w[0], w[1], w[2], w[3]);
-      };
-      const bf16_t* nwg_ = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BG]));
-      const bf16_t* nwu_ = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BU]));
       if (ONE) {
         auto load0 = [&](int p) { return load_mid(0, p); };
         bit_stage_row1_pre<1>(L, 2, d, true, npw, reinterpret_cast<const uint4(&)[1]>(nn0), nn1, m.eps, load0);
       } else {
-        bit_stage_roww<4>(L, 2, B, d, norm2, nwg_, nwu_, m.eps, load_mid);
+        bit_codes_fetch(L, 2, B, cq_l + cq_g, cs_l + BG * 32, 0, KCd, true);
       }
       for (int s0 = 2 * (int)blockIdx.x; s0 < ns_f; s0 += 2 * nwg) {
         const bool first = s0 == 2 * (int)blockIdx.x;
@@ -930,20 +923,29 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
     {
       const int nunits = ns_d * OHARA_BIT_DOWN_SPLIT;
       L.shape(B, F);
+      if (!ONE) {
+        const bf16_t* nwd = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BD]));
+        bit_for_units(B, nwg, [&](int b) {
+          auto loadq = [&](int p) { return ldg16(am_addr(a_l, a.blk_a, b, p * 8)); };
+          if (F <= 2048) bit_quant_once<1>(L, F, nullptr, nwd, m.eps, loadq, cq_l + cq_dn + (size_t)b * ldq_f, ldq_f, cs_l + BD * 32 + b * 2);
+          else bit_quant_once<3>(L, F, nullptr, nwd, m.eps, loadq, cq_l + cq_dn + (size_t)b * ldq_f, ldq_f, cs_l + BD * 32 + b * 2);
+        });
+        gs.arrive(nopf);
+        gs.wait(nopf);
+      }
       bool staged = false;
       for (int unit = blockIdx.x; unit < nunits; unit += nwg) {
         const bool first = unit == (int)blockIdx.x;
         const int part = unit / ns_d, strip = unit - part * ns_d;
         if (!staged) {
-          const bf16_t* nwd = reinterpret_cast<const bf16_t*>(gptr(LY.nw[BD]));
           if (ONE) {
             auto load0 = [&](int p) { return ldg16(am_addr(a_l, a.blk_a, 0, p * 8)); };
             if (F <= 2048) bit_stage_row1_pre<1>(L, 1, F, false, npw, reinterpret_cast<const uint4(&)[1]>(nn0), nn1, m.eps, load0);
             else bit_stage_row1_pre<3>(L, 1, F, false, nn0, nn0, nn0, m.eps, load0);
-          } else {
-            auto loadb = [&](int b, int p) { return ldg16(am_addr(a_l, a.blk_a, b, p * 8)); };
-            if (F <= 2048) bit_stage_roww<4>(L, 1, B, F, nullptr, nwd, nullptr, m.eps, loadb);
-            else bit_stage_roww_lds<12>(L, B, F, nwd, m.eps, loadb);
+          } else {  // the codes of this workgroup's K partition (its units all lie in one partition or take whole rows)
+            const bool one_part = (int)blockIdx.x + nwg >= nunits;
+            if (one_part) bit_codes_fetch(L, 1, B, cq_l + cq_dn, cs_l + BD * 32, part * per_part, min(KCf, (part + 1) * per_part), false);
+            else bit_codes_fetch(L, 1, B, cq_l + cq_dn, cs_l + BD * 32, 0, KCf, true);
           }
           staged = true;
         }
@@ -1067,8 +1069,8 @@ __global__ __launch_bounds__(256) void bitnet_mega_kernel(BitMegaArgs a) {
 size_t bit_al(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct BitLayout {
-  size_t layers, xm, qm, am, pm, dm, ds, candv, candi, prof, bar, total;
-  size_t xm_stride, qm_stride, am_stride, pm_stride, dm_stride;
+  size_t layers, xm, qm, am, pm, dm, ds, cq, cs, candv, candi, prof, bar, total;
+  size_t xm_stride, qm_stride, am_stride, pm_stride, dm_stride, cq_stride;
   int blk_x, blk_a;
 };
 
@@ -1091,6 +1093,14 @@ BitLayout bit_layout(const OharaBitModel* m, int B, int nwg) {
   L.pm = o; o += L.pm_stride * sizeof(float) * NL;
   L.dm = o; o += L.dm_stride * sizeof(int32_t) * NL;
   L.ds = o; o += bit_al((size_t)NL * 32 * sizeof(float));
+  {  // batch > 1: code rows of the seven BitLinears (K padded to 256 columns + 16), B rows each; {s, sum q} pairs
+    const int ldq_d = (((m->d_model + 255) >> 8) << 8) + 16, ldq_o = (((hd + 255) >> 8) << 8) + 16;
+    const int ldq_f = (((m->d_ff + 255) >> 8) << 8) + 16;
+    const size_t o_ = bit_cq_al((size_t)3 * B * ldq_d), g_ = bit_cq_al(o_ + (size_t)B * ldq_o), dn_ = bit_cq_al(g_ + (size_t)2 * B * ldq_d);
+    L.cq_stride = B > 1 ? bit_cq_al(dn_ + (size_t)B * ldq_f) : 0;
+  }
+  L.cq = o; o += L.cq_stride * NL;
+  L.cs = o; o += bit_al((size_t)NL * 256 * sizeof(float));
   L.candv = o; o += bit_al((size_t)nwg * B * sizeof(float));
   L.candi = o; o += bit_al((size_t)nwg * B * sizeof(int));
   L.prof = o; o += bit_al(1024 * sizeof(unsigned long long));
@@ -1106,9 +1116,7 @@ size_t bit_smem_bytes(const OharaBitModel* m, int B, int ns) {
   const int Kp = ((kmax + 255) >> 8) << 8, Kpd = ((dmax + 255) >> 8) << 8;
   size_t codes = (size_t)B * (Kp + 16);
   if ((size_t)2 * B * (Kpd + 16) > codes) codes = (size_t)2 * B * (Kpd + 16);
-  const int KpF = ((m->d_ff + 255) >> 8) << 8;
-  size_t stage = (size_t)B * (dmax + 8) * 2;
-  if (B > 1 && m->d_ff > 2048 && (size_t)B * KpF * 2 > stage) stage = (size_t)B * KpF * 2;
+  const size_t stage = (size_t)B * (dmax + 8) * 2;
   size_t o = ((codes + 255) & ~(size_t)255) + ((stage + 255) & ~(size_t)255) + 4096 + 256 + 64;
   o += (size_t)(8 + 4 * D) * G * sizeof(float);
   o += (size_t)2 * ((B * m->n_heads * ns + 1) & ~1) * sizeof(float);
@@ -1181,6 +1189,7 @@ int ohara_bitnet_decode_persistent(const OharaBitModel* m, const OharaDecodeStat
   a.dm = reinterpret_cast<int32_t*>(ws + L.dm); a.ds = reinterpret_cast<float*>(ws + L.ds);
   a.xm_stride = L.xm_stride; a.qm_stride = L.qm_stride; a.am_stride = L.am_stride; a.pm_stride = L.pm_stride;
   a.dm_stride = L.dm_stride;
+  a.cq = reinterpret_cast<int8_t*>(ws + L.cq); a.cs = reinterpret_cast<float*>(ws + L.cs); a.cq_stride = L.cq_stride;
   a.blk_x = L.blk_x; a.blk_a = L.blk_a;
   a.cand_val = reinterpret_cast<float*>(ws + L.candv);
   a.cand_idx = reinterpret_cast<int*>(ws + L.candi);

@@ -220,6 +220,8 @@ PERSISTENT_SHAPES = [
     (320, 5, 528, 300, 2, 3),     # widths that are not multiples of 256 (zero-padded code rows)
     (256, 2, 2304, 320, 4, 6),    # a hidden width beyond 2048 (rows parked in LDS at batch > 1), four layers
     (256, 2, 2304, 320, 4, 1),
+    (256, 2, 512, 320, 3, 2),     # code rows of 272 bytes: the sets of a layer's code mailbox start between cache lines
+    (512, 8, 1536, 333, 2, 7),
 ]
 
 
