@@ -745,6 +745,13 @@ def main():
     from ohara_amd.llama import Llama
 
     dev = torch.device("cuda:0")
+    if args.pmc_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if args.phi_decode_only:
         print(json.dumps(phi_decode_only(dev, args.phi_decode_only)))
         return
@@ -763,13 +770,6 @@ def main():
     if args.phase_timeline:
         print(json.dumps(phase_timeline(dev, args.prompt, batch=args.timeline_batch, int8=args.timeline_int8), indent=1))
         return
-    if args.pmc_calibration:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
     cfg, st = d12_state(dev)
     model = Llama(cfg, st, device=dev)
     del st
