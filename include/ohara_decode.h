@@ -122,6 +122,12 @@ int ohara_qkv_rope_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int k, c
                         int pos, const int32_t* pos_dev, int t_max, uint16_t* q_out, uint16_t* k_out, uint16_t* v_out,
                         void* stream);
 
+/* ohara_qkv_rope_bf16 with one position per sequence (seq_pos as in ohara_qkv_rope_append_ragged_bf16). */
+int ohara_qkv_rope_ragged_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int k, const uint16_t* norm_w, float eps,
+                               int batch, int seq_len, int h, int h_kv, int dh, const uint16_t* cos, const uint16_t* sin,
+                               const int32_t* seq_pos, int t_max, uint16_t* q_out, uint16_t* k_out, uint16_t* v_out,
+                               void* stream);
+
 /* ---- attention over the KV cache ------------------------------------------------
  * Query s (0 <= s < seq_len) of sequence b sits at cache position pos + s and sees
  * positions [0, pos + s] (the cache mask key_pos <= start_pos + q_idx, llama.py:109-113):
@@ -193,6 +199,17 @@ int ohara_kv_dequant_int8(const int8_t* q, const float* stats, int which, int ba
 int ohara_attn_cached_int8(const uint16_t* q, const int8_t* kcache, const int8_t* vcache, const float* stats, int batch,
                            int seq_len, int h, int h_kv, int dh, int t_max, int pos, const int32_t* pos_dev, int n_split,
                            void* workspace, uint16_t* out, void* stream);
+
+/* The append and the attention with one cache position per sequence (seq_pos: device array, `batch`
+ * entries; token s of sequence b goes to / sits at seq_pos[b] + s).  No counterpart in the reference,
+ * whose forward takes one scalar position for the whole batch (llama.py:287-299); the cache itself
+ * (kv_cache.py:94-118) is indifferent to where each sequence stands. */
+int ohara_kv_quant_append_ragged_int8(const uint16_t* k, const uint16_t* v, int batch, int seq_len, int h_kv, int dh,
+                                      const int32_t* seq_pos, int8_t* kq, int8_t* vq, float* stats, int t_max,
+                                      void* stream);
+int ohara_attn_cached_ragged_int8(const uint16_t* q, const int8_t* kcache, const int8_t* vcache, const float* stats,
+                                  int batch, int seq_len, int h, int h_kv, int dh, int t_max, const int32_t* seq_pos,
+                                  int n_split, void* workspace, uint16_t* out, void* stream);
 
 /* ---- greedy selection ---------------------------------------------------------
  * next_ids[b] = first index of max(logits[b, 0:valid_vocab])  (argmax of the last
@@ -281,7 +298,10 @@ int ohara_silu_mul_bf16(const uint16_t* gate, const uint16_t* up, uint16_t* out,
 
 /* Rotary on q (in place) and on k, and append of the rotated k and of v to the cache, for
  * projections that were computed unfused (ohara/embeddings_pos/rotary.py:55-93,
- * ohara/modules/kv_cache.py:104-105).  q: (batch*seq_len, h*dh), k/v: (batch*seq_len, h_kv*dh). */
+ * ohara/modules/kv_cache.py:104-105).  q: (batch*seq_len, h*dh), k/v: (batch*seq_len, h_kv*dh).
+ * t_max == 0: kcache / vcache are row buffers of k's and v's shape instead of caches - the rotated
+ * keys and the values of this call, which an int8 cache's append (ohara_kv_quant_append_int8,
+ * kv_cache.py:94-102) takes next; the caller keeps pos + seq_len within the rotary tables. */
 int ohara_rope_append_bf16(uint16_t* q, const uint16_t* k, const uint16_t* v, int batch, int seq_len, int h, int h_kv,
                            int dh, const uint16_t* cos, const uint16_t* sin, int pos, const int32_t* pos_dev,
                            uint16_t* kcache, uint16_t* vcache, int t_max, void* stream);

@@ -77,6 +77,9 @@ _PROTOS = {
     "ohara_attn_workspace_bytes": (_i64, [_i, _i, _i, _i, _i]),
     "ohara_attn_cached_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
     "ohara_attn_cached_bf16_noalloc": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p]),
+    "ohara_qkv_rope_ragged_bf16": (_i, [_p, _i, _p, _i, _p, _f, _i, _i, _i, _i, _i, _p, _p, _p, _i, _p, _p, _p, _p]),
+    "ohara_kv_quant_append_ragged_int8": (_i, [_p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _i, _p]),
+    "ohara_attn_cached_ragged_int8": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
     "ohara_attn_cached_ragged_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
     "ohara_qkv_rope_append_ragged_bf16": (_i, [_p, _i, _p, _i, _p, _f, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _i, _p]),
     "ohara_advance_positions": (_i, [_p, _p, _i, _i, _p]),

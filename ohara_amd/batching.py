@@ -18,14 +18,14 @@ from .llama import BF16, Llama
 
 
 class ContinuousBatcher:
-    def __init__(self, model: Llama, slots: int, sampling=None, valid_vocab: int = 0, generator=None):
+    def __init__(self, model: Llama, slots: int, sampling=None, valid_vocab: int = 0, generator=None, int8: bool = False):
         if slots < 1:
             raise ValueError("batch_size must be at least 1")
         self.model, self.slots = model, slots
         self.sampling = sampling if (sampling is not None and sampling.temperature > 0) else None
         self.valid_vocab = valid_vocab
         self.generator = generator
-        self.cache = model.build_kv_cache(slots)
+        self.cache = model.build_kv_cache(slots, int8=int8)  # int8: the caches of ohara/modules/kv_cache.py:15-32
         for c in self.cache:
             c._commit_ragged(slots, [0] * slots)
         self.active = [False] * slots

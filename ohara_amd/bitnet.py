@@ -93,12 +93,12 @@ class BitLlama:
     def to(self, *a, **k):
         return self
 
-    def build_kv_cache(self, batch_size: int = 1):
+    def build_kv_cache(self, batch_size: int = 1, int8: bool = False):
         if batch_size < 1:
             raise ValueError("batch_size must be at least 1")
         c = self.config
         shape = (batch_size, c.max_sequence_length, self.kv_heads, self.head_dim)
-        return [KVCache(shape, c.max_sequence_length, i, device=self.device, dtype=BF16)
+        return [KVCache(shape, c.max_sequence_length, i, device=self.device, dtype=BF16, int8=int8)
                 for i in range(c.num_hidden_layers)]
 
     def packed_weight_bytes(self) -> int:
@@ -130,8 +130,9 @@ class BitLlama:
             raise ValueError("input exceeds max_sequence_length")
         if kv_cache is None:
             kv_cache = self.build_kv_cache(B)
-        if any(cc.int8 for cc in kv_cache):
-            raise NotImplementedError("ohara_amd: int8 KV caches are served by the dense Llama only")
+        if len({cc.int8 for cc in kv_cache}) > 1:
+            raise ValueError("all layers must use the same KV cache mode")
+        int8 = kv_cache[0].int8
         ends = [cc._reserve(B, S, start) for cc in kv_cache]
         H, Hkv, D = c.num_attention_heads, self.kv_heads, self.head_dim
         rows = B * S
@@ -143,7 +144,16 @@ class BitLlama:
         h = ops.embed(x.to(self.device), self.token_emb)
         for L, cache in zip(self.layers, kv_cache):
             # the block norm (norm1 / norm2) is applied inside each projection's quantisation pass
-            if rows <= 64:  # decode: one launch for q/k/v + rotary + append, one for gate/up + SwiGLU
+            if int8:
+                # kv_cache.py:94-118 with quantisation: the new rows go in as codes and attention reads what the
+                # reference's cache read returns (the dequantised prefix, the new rows included); many new
+                # positions per sequence attend over a dequantised copy of the live prefix
+                q = ops.bitlinear(h, L["attn.query"][1], L["attn.query"][0], self.eps, pre_norm_w=L["norm1"])
+                k = ops.bitlinear(h, L["attn.key"][1], L["attn.key"][0], self.eps, pre_norm_w=L["norm1"])
+                v = ops.bitlinear(h, L["attn.value"][1], L["attn.value"][0], self.eps, pre_norm_w=L["norm1"])
+                kr, vr = ops.rope_rows(q, k, v, B, S, H, Hkv, D, self.cos, self.sin, start)
+                ops.kv_quant_append(kr, vr, cache, start)
+            elif rows <= 64:  # decode: one launch for q/k/v + rotary + append, one for gate/up + SwiGLU
                 q = ops.bitlinear_qkv_rope_append(
                     h, L["norm1"], [(L[n][1], L[n][0]) for n in ("attn.query", "attn.key", "attn.value")], self.eps,
                     H, Hkv, D, self.cos, self.sin, start, cache.key, cache.value, seq_len=S)
@@ -152,7 +162,13 @@ class BitLlama:
                 k = ops.bitlinear(h, L["attn.key"][1], L["attn.key"][0], self.eps, pre_norm_w=L["norm1"])
                 v = ops.bitlinear(h, L["attn.value"][1], L["attn.value"][0], self.eps, pre_norm_w=L["norm1"])
                 ops.rope_append(q, k, v, B, S, H, Hkv, D, self.cos, self.sin, start, cache.key, cache.value)
-            att = ops.attn_auto(q, cache.key, cache.value, H, Hkv, D, start, n_split, ws, S)
+            if not int8:
+                att = ops.attn_auto(q, cache.key, cache.value, H, Hkv, D, start, n_split, ws, S)
+            elif S >= 16 and D in (64, 128):
+                att = ops.attn_prefill(q, ops.kv_dequant(cache, "key", B, start + S),
+                                       ops.kv_dequant(cache, "value", B, start + S), H, Hkv, D, start, S)
+            else:
+                att = ops.attn_cached_int8(q, cache, H, Hkv, D, start, n_split, ws, seq_len=S)
             h = ops.bitlinear(att, L["attn.proj"][1], L["attn.proj"][0], self.eps, residual=h)
             if rows <= 64:
                 act = ops.bitlinear_gate_up(h, L["norm2"], (L["ff.gate"][1], L["ff.gate"][0]),
@@ -219,13 +235,15 @@ class BitDecodeSession:
             if u.shape != (rows, batch):
                 raise ValueError("u must have shape (max_new_tokens, batch)")
             self.u = u.to(device=model.device, dtype=torch.float32).contiguous()
+        self.cache = kv_cache if kv_cache is not None else model.build_kv_cache(batch)
+        int8 = any(cc.int8 for cc in self.cache)  # int8 caches are served by the kernel chain
         if persistent is None:
-            persistent = model.supports_persistent(batch)
-        elif persistent and not model.supports_persistent(batch):
-            raise ValueError("the persistent decode kernel does not cover this shape")
+            persistent = model.supports_persistent(batch) and not int8
+        elif persistent and (int8 or not model.supports_persistent(batch)):
+            raise ValueError("the persistent decode kernel does not cover this shape" if not int8 else
+                             "the single-launch ternary decode kernel reads bfloat16 caches; int8 caches run the kernel chain")
         self.persistent = persistent
         self.spin_limit = 0
-        self.cache = kv_cache if kv_cache is not None else model.build_kv_cache(batch)
         self.valid_vocab = valid_vocab
         dev = model.device
         self.history = torch.zeros(rows, batch, dtype=torch.int64, device=dev)

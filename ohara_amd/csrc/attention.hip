@@ -987,6 +987,14 @@ int ohara_attn_cached_int8(const uint16_t* q, const int8_t* kcache, const int8_t
                           workspace, out, stream);
 }
 
+int ohara_attn_cached_ragged_int8(const uint16_t* q, const int8_t* kcache, const int8_t* vcache, const float* stats,
+                                  int batch, int seq_len, int h, int h_kv, int dh, int t_max, const int32_t* seq_pos,
+                                  int n_split, void* workspace, uint16_t* out, void* stream) {
+  if (!seq_pos) return OHARA_EINVAL;
+  return attn_cached_impl(q, kcache, vcache, stats, true, batch, seq_len, h, h_kv, dh, t_max, 0, seq_pos, 1, n_split,
+                          workspace, out, stream);
+}
+
 // ---- the same attention for callers that cannot allocate -------------------------------------
 // The chunk partials and counters live in a file-scope device array instead of a caller-supplied
 // workspace.  Layout: OHARA_SCRATCH_COUNTER_BYTES of counters (one int per (query row, kv head)),

@@ -536,7 +536,7 @@ __global__ __launch_bounds__(256) void rope_append_kernel(bf16_t* q, const bf16_
   const int row = blockIdx.x;
   const int seq = row / S;
   const int pos = (pos_dev ? *pos_dev : pos0) + (row - seq * S);
-  if (pos < 0 || pos >= Tmax) return;
+  if (pos < 0 || (Tmax > 0 && pos >= Tmax)) return;
   const int half = D >> 1;
   const bf16_t* cs = cos + (size_t)pos * half;
   const bf16_t* sn = sin + (size_t)pos * half;
@@ -547,8 +547,10 @@ __global__ __launch_bounds__(256) void rope_append_kernel(bf16_t* q, const bf16_
     x[0] = f2bf(__fsub_rn(__fmul_rn(e, c), __fmul_rn(o, s)));
     x[1] = f2bf(__fadd_rn(__fmul_rn(e, s), __fmul_rn(o, c)));
   }
-  bf16_t* kd = kc + (((size_t)seq * Tmax + pos) * Hkv) * D;
-  bf16_t* vd = vc + (((size_t)seq * Tmax + pos) * Hkv) * D;
+  // Tmax == 0: kc / vc are row buffers like k / v (the rows an int8 cache's append quantises)
+  const size_t dst_row = Tmax > 0 ? (size_t)seq * Tmax + pos : (size_t)row;
+  bf16_t* kd = kc + dst_row * Hkv * D;
+  bf16_t* vd = vc + dst_row * Hkv * D;
   for (int i = threadIdx.x; i < Hkv * half; i += 256) {
     const int h = i / half, p = i - h * half;
     const bf16_t* x = k + (size_t)row * Hkv * D + (size_t)h * D + 2 * p;
@@ -757,8 +759,8 @@ int ohara_rope_append_bf16(uint16_t* q, const uint16_t* k, const uint16_t* v, in
                            int dh, const uint16_t* cos, const uint16_t* sin, int pos, const int32_t* pos_dev,
                            uint16_t* kcache, uint16_t* vcache, int t_max, void* stream) {
   if (!q || !k || !v || !cos || !sin || !kcache || !vcache) return OHARA_EINVAL;
-  if (batch < 1 || seq_len < 1 || h < 1 || h_kv < 1 || dh < 2 || (dh & 1) || t_max < 1) return OHARA_EINVAL;
-  if (!pos_dev && (pos < 0 || pos + seq_len > t_max)) return OHARA_EINVAL;
+  if (batch < 1 || seq_len < 1 || h < 1 || h_kv < 1 || dh < 2 || (dh & 1) || t_max < 0) return OHARA_EINVAL;
+  if (!pos_dev && (pos < 0 || (t_max > 0 && pos + seq_len > t_max))) return OHARA_EINVAL;
   hipLaunchKernelGGL(rope_append_kernel, dim3(batch * seq_len), dim3(256), 0, (hipStream_t)stream, q, k, v, seq_len, h,
                      h_kv, dh, cos, sin, pos, pos_dev, kcache, vcache, t_max);
   return ohara_launch_status();

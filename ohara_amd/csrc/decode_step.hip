@@ -18,7 +18,6 @@ extern "C" int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* 
   const int64_t rows64 = (int64_t)s->batch * seq_len;
   if (rows64 > s->rows_cap) return OHARA_ESIZE;
   const bool ragged = s->seq_pos != nullptr;
-  if (ragged && s->kv_int8) return OHARA_EINVAL;
   if (!ragged && use_pos_dev && (!s->step_state || seq_len != 1)) return OHARA_EINVAL;
   if (!ragged && !use_pos_dev && (pos < 0 || pos + seq_len > m->t_max)) return OHARA_EINVAL;
   if (logits_mode < OHARA_LOGITS_NONE || logits_mode > OHARA_LOGITS_ALL) return OHARA_EINVAL;
@@ -49,7 +48,20 @@ extern "C" int ohara_llama_forward(const OharaModel* m, const OharaDecodeState* 
       rc = ohara_rmsnorm_bf16(s->x, L.norm1, s->xn, R, d, m->eps, stream);
       if (rc) return rc;
     }
-    if (ragged) {
+    if (ragged && s->kv_int8) {
+      // one position per sequence over the int8 cache: rows to staging, quantise into the cache at each sequence's
+      // own position, attention straight over the codes (the extra launch is not numbered)
+      int8_t* kq = reinterpret_cast<int8_t*>(s->kcache[l]);
+      int8_t* vq = reinterpret_cast<int8_t*>(s->vcache[l]);
+      OHARA_RUN(ohara_qkv_rope_ragged_bf16(tiled ? s->xn : s->x, d, L.wqkv, d, tiled ? nullptr : L.norm1, m->eps, B,
+                                           seq_len, H, Hkv, Dh, m->cos, m->sin, s->seq_pos, m->t_max, s->q, s->kstage,
+                                           s->vstage, stream));
+      rc = ohara_kv_quant_append_ragged_int8(s->kstage, s->vstage, B, seq_len, Hkv, Dh, s->seq_pos, kq, vq, s->kvstats[l],
+                                             m->t_max, stream);
+      if (rc) return rc;
+      OHARA_RUN(ohara_attn_cached_ragged_int8(s->q, kq, vq, s->kvstats[l], B, seq_len, H, Hkv, Dh, m->t_max, s->seq_pos,
+                                              n_split, s->attn_ws, s->attn, stream));
+    } else if (ragged) {
       // one position per sequence; attention of any length through the split-context kernel
       OHARA_RUN(ohara_qkv_rope_append_ragged_bf16(tiled ? s->xn : s->x, d, L.wqkv, d, tiled ? nullptr : L.norm1, m->eps,
                                                   B, seq_len, H, Hkv, Dh, m->cos, m->sin, s->seq_pos, s->q, s->kcache[l],

@@ -690,4 +690,13 @@ int ohara_qkv_rope_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int k, c
                        v_out, t_max, 1, stream);
 }
 
+int ohara_qkv_rope_ragged_bf16(const uint16_t* x, int ldx, const uint16_t* wp, int k, const uint16_t* norm_w, float eps,
+                               int batch, int seq_len, int h, int h_kv, int dh, const uint16_t* cos, const uint16_t* sin,
+                               const int32_t* seq_pos, int t_max, uint16_t* q_out, uint16_t* k_out, uint16_t* v_out,
+                               void* stream) {
+  if (!seq_pos) return OHARA_EINVAL;
+  return qkv_rope_impl(x, ldx, wp, k, norm_w, eps, batch, seq_len, h, h_kv, dh, cos, sin, 0, seq_pos, 1, q_out, k_out,
+                       v_out, t_max, 1, stream);
+}
+
 }  // extern "C"

@@ -16,8 +16,8 @@ namespace {
 
 // one wave per (row, head): D <= 512, D % 2 == 0
 __global__ __launch_bounds__(256) void kv_quant_append_kernel(const bf16_t* k, const bf16_t* v, int rows, int S, int Hkv,
-                                                              int D, int pos0, const int32_t* pos_dev, int8_t* kq,
-                                                              int8_t* vq, float* stats, int Tmax) {
+                                                              int D, int pos0, const int32_t* pos_dev, int pos_stride,
+                                                              int8_t* kq, int8_t* vq, float* stats, int Tmax) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int item = blockIdx.x * 4 + wave;  // (tensor, row, head)
   if (item >= 2 * rows * Hkv) return;
@@ -25,7 +25,7 @@ __global__ __launch_bounds__(256) void kv_quant_append_kernel(const bf16_t* k, c
   const int rh = item - which * rows * Hkv;
   const int row = rh / Hkv, h = rh - row * Hkv;
   const int seq = row / S;
-  const int pos = (pos_dev ? *pos_dev : pos0) + (row - seq * S);
+  const int pos = (pos_dev ? pos_dev[(size_t)seq * pos_stride] : pos0) + (row - seq * S);  // stride 1: one position per sequence
   if (pos < 0 || pos >= Tmax) return;
   const bf16_t* src = (which ? v : k) + ((size_t)row * Hkv + h) * D;
   const size_t slot = ((size_t)seq * Tmax + pos) * Hkv + h;
@@ -94,7 +94,19 @@ int ohara_kv_quant_append_int8(const uint16_t* k, const uint16_t* v, int batch, 
   const int64_t items = (int64_t)2 * batch * seq_len * h_kv;
   if (items > INT32_MAX) return OHARA_ESIZE;
   hipLaunchKernelGGL(kv_quant_append_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, k, v,
-                     batch * seq_len, seq_len, h_kv, dh, pos, pos_dev, kq, vq, stats, t_max);
+                     batch * seq_len, seq_len, h_kv, dh, pos, pos_dev, 0, kq, vq, stats, t_max);
+  return ohara_launch_status();
+}
+
+int ohara_kv_quant_append_ragged_int8(const uint16_t* k, const uint16_t* v, int batch, int seq_len, int h_kv, int dh,
+                                      const int32_t* seq_pos, int8_t* kq, int8_t* vq, float* stats, int t_max,
+                                      void* stream) {
+  if (!k || !v || !kq || !vq || !stats || !seq_pos) return OHARA_EINVAL;
+  if (batch < 1 || seq_len < 1 || h_kv < 1 || dh < 2 || (dh & 3) || dh > 512 || t_max < 1) return OHARA_EINVAL;
+  const int64_t items = (int64_t)2 * batch * seq_len * h_kv;
+  if (items > INT32_MAX) return OHARA_ESIZE;
+  hipLaunchKernelGGL(kv_quant_append_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, k, v,
+                     batch * seq_len, seq_len, h_kv, dh, 0, seq_pos, 1, kq, vq, stats, t_max);
   return ohara_launch_status();
 }
 

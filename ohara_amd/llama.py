@@ -144,10 +144,14 @@ class KVCache:
         self.batch_size = bsz
 
     def _row_view(self, b: int) -> "KVCache":
-        """The cache of sequence b alone, sharing storage (bf16 mode)."""
+        """The cache of sequence b alone, sharing storage."""
         v = KVCache.__new__(KVCache)
-        v.idx, v.int8, v.max_seq_length, v.dtype = self.idx, False, self.max_seq_length, self.dtype
+        v.idx, v.int8, v.max_seq_length, v.dtype = self.idx, self.int8, self.max_seq_length, self.dtype
         v.key, v.value = self.key[b:b + 1], self.value[b:b + 1]
+        if self.int8:
+            v.stats = self.stats[b:b + 1]
+            v.key_scale, v.key_min, v.value_scale, v.value_min = (
+                v.stats[..., i:i + 1].permute(0, 2, 1, 3) for i in range(4))
         v.length = (self.lengths[b] if self.lengths is not None else self.length)
         v.batch_size, v.lengths = None, None
         return v
@@ -370,8 +374,6 @@ class Llama:
         if len({c.int8 for c in kv_cache}) > 1:
             raise ValueError("all layers must use the same KV cache mode")
         if seq_pos is not None:
-            if kv_cache[0].int8:
-                raise NotImplementedError("ohara_amd: one position per sequence needs bf16 KV caches")
             s.seq_pos = seq_pos.data_ptr()
             s._keep = (kc, vc, seq_pos)
         if kv_cache[0].int8:
@@ -389,7 +391,7 @@ class Llama:
                     buf.kdeq = torch.empty(shape, dtype=BF16, device=self.device)
                     buf.vdeq = torch.empty(shape, dtype=BF16, device=self.device)
                 s.kdeq, s.vdeq = buf.kdeq.data_ptr(), buf.vdeq.data_ptr()
-            s._keep = (kc, vc, *stats)
+            s._keep = (kc, vc, *stats) if seq_pos is None else (kc, vc, seq_pos, *stats)
         return s
 
     def forward(self, x: torch.Tensor, kv_cache: list | None = None, position_ids=None, *, last_only: bool = False,

@@ -250,11 +250,18 @@ def attn_auto(q, kcache, vcache, h, h_kv, dh, pos, n_split, workspace, seq_len, 
     return attn_cached(q, kcache, vcache, h, h_kv, dh, pos, n_split if seq_len == 1 else 1, workspace, out, None, seq_len)
 
 
-def kv_quant_append(keys, values, cache, pos, pos_dev=None):
-    """keys / values (B, S, Hkv, D) bf16 -> quantised into an int8 ``KVCache`` at positions pos + s."""
+def kv_quant_append(keys, values, cache, pos, pos_dev=None, seq_pos=None):
+    """keys / values (B, S, Hkv, D) bf16 -> quantised into an int8 ``KVCache`` at positions pos + s
+    (``seq_pos``: one position per sequence, an int32 device tensor)."""
     _need(keys, BF16, "keys")
     _need(values, BF16, "values")
     b, s_len, hkv, d = keys.shape
+    if seq_pos is not None:
+        _need(seq_pos, torch.int32, "seq_pos")
+        check(lib().ohara_kv_quant_append_ragged_int8(
+            _ptr(keys), _ptr(values), b, s_len, hkv, d, _ptr(seq_pos), _ptr(cache.key), _ptr(cache.value), _ptr(cache.stats),
+            cache.key.shape[1], _stream()), "kv_quant_append_ragged")
+        return
     check(lib().ohara_kv_quant_append_int8(
         _ptr(keys), _ptr(values), b, s_len, hkv, d, int(pos), _ptr(pos_dev), _ptr(cache.key), _ptr(cache.value),
         _ptr(cache.stats), cache.key.shape[1], _stream()), "kv_quant_append")
@@ -271,11 +278,17 @@ def kv_dequant(cache, which: str, batch: int, length: int, out=None) -> torch.Te
     return out
 
 
-def attn_cached_int8(q, cache, h, h_kv, dh, pos, n_split, workspace, out=None, pos_dev=None, seq_len=1):
-    """attn_cached over an int8 ``KVCache``."""
+def attn_cached_int8(q, cache, h, h_kv, dh, pos, n_split, workspace, out=None, pos_dev=None, seq_len=1, seq_pos=None):
+    """attn_cached over an int8 ``KVCache`` (``seq_pos``: one position per sequence, an int32 device tensor)."""
     rows = q.shape[0]
     if out is None:
         out = torch.empty(rows, h * dh, dtype=BF16, device=q.device)
+    if seq_pos is not None:
+        _need(seq_pos, torch.int32, "seq_pos")
+        check(lib().ohara_attn_cached_ragged_int8(
+            _ptr(q), _ptr(cache.key), _ptr(cache.value), _ptr(cache.stats), rows // seq_len, seq_len, h, h_kv, dh,
+            cache.key.shape[1], _ptr(seq_pos), n_split, _ptr(workspace), _ptr(out), _stream()), "attn_cached_ragged_int8")
+        return out
     check(lib().ohara_attn_cached_int8(
         _ptr(q), _ptr(cache.key), _ptr(cache.value), _ptr(cache.stats), rows // seq_len, seq_len, h, h_kv, dh,
         cache.key.shape[1], int(pos), _ptr(pos_dev), n_split, _ptr(workspace), _ptr(out), _stream()), "attn_cached_int8")
@@ -448,6 +461,15 @@ def rope_append(q, k, v, batch, seq_len, h, h_kv, dh, cos, sin, pos, kcache, vca
                                        int(pos), _ptr(pos_dev), _ptr(kcache), _ptr(vcache), kcache.shape[1], _stream()),
           "rope_append")
     return q
+
+
+def rope_rows(q, k, v, batch, seq_len, h, h_kv, dh, cos, sin, pos, pos_dev=None):
+    """In-place rotary on q; returns the rotated k and v as (batch, seq_len, h_kv, dh) tensors (what an int8
+    cache's append quantises)."""
+    kr, vr = torch.empty_like(k), torch.empty_like(v)
+    check(lib().ohara_rope_append_bf16(_ptr(q), _ptr(k), _ptr(v), batch, seq_len, h, h_kv, dh, _ptr(cos), _ptr(sin),
+                                       int(pos), _ptr(pos_dev), _ptr(kr), _ptr(vr), 0, _stream()), "rope_rows")
+    return kr.view(batch, seq_len, h_kv, dh), vr.view(batch, seq_len, h_kv, dh)
 
 
 # ---- Phi (ohara/models/phi.py) ----------------------------------------------------------------

@@ -384,3 +384,54 @@ def test_persistent_kernel_on_int8_caches(cuda, heads, kv_heads, hidden, B, P):
         assert torch.equal(codes[:B, P:P + steps].cpu(), rq)
         assert torch.equal(scale[:B, P:P + steps].cpu(), rs.float())
         assert torch.equal(mn[:B, P:P + steps].cpu(), rm.float())
+
+
+@pytest.mark.parametrize("P", [6, 20])
+def test_bitnet_model_with_int8_caches(cuda, P):
+    """The ternary (BitNet) Llama on int8 caches through the kernel chain: prefill (short prompts attend over
+    the codes, prompts of 16 and more tokens over a dequantised copy of the live prefix) and cached steps
+    against the oracle on its own int8 caches, at the ternary model's tolerance; layer 0's codes and
+    statistics (no attention in front of them) against the oracle's quantiser applied to the bf16 session's
+    rows; the decode session falls back to the kernel chain for such caches."""
+    from oracle import bitlinear_ref as BL
+    from ohara_amd.bitnet import BitLlama
+    from ohara_amd.llama import Config
+
+    kw = dict(vocab_size=320, hidden_size=256, intermediate_size=512, num_attention_heads=2,
+              num_key_value_heads=0, num_hidden_layers=3, max_sequence_length=64, rope_theta=10000.0)
+    rcfg = R.RefConfig(**kw)
+    w = BL.init_ternary_weights(rcfg, seed=2, dtype=BF, gamma=0.05)
+    ref, model = R.RefLlama(rcfg, w), BitLlama(Config(**kw), w, device=cuda)
+    B = 2
+    ids = torch.randint(0, 320, (B, P + 3), generator=torch.Generator().manual_seed(P))
+    rc, cache = ref.build_kv_cache(B, int8=True), model.build_kv_cache(B, int8=True)
+    assert cache[0].key.dtype == torch.int8
+
+    def close(got, want):
+        d = (got.float().cpu() - want.float()).abs()
+        scale = want.float().abs().max().item()
+        assert d.max().item() <= 1e-1 * scale and d.mean().item() <= 1.5e-2 * scale, (d.max().item(), d.mean().item(), scale)
+
+    close(model(ids[:, :P].to(cuda), cache, 0), ref(ids[:, :P], rc, 0))
+    for t in range(P, P + 3):
+        close(model(ids[:, t:t + 1].to(cuda), cache, t), ref(ids[:, t:t + 1], rc, t))
+    assert cache[0].length == P + 3
+    # layer 0: the rows that went in are those of a bf16-cache run of the same model (bit for bit: nothing in front of
+    # them depends on the cache), so its codes are the oracle quantiser's codes of those rows
+    plain = model.build_kv_cache(B)
+    model(ids[:, :P].to(cuda), plain, 0)
+    kq, ks, km = R.quantize_int8(plain[0].key[:, :P].cpu())
+    assert torch.equal(cache[0].key[:, :P].cpu(), kq)
+    vq, _, _ = R.quantize_int8(plain[0].value[:, :P].cpu())
+    assert torch.equal(cache[0].value[:, :P].cpu(), vq)
+    # sessions: int8 caches run the kernel chain
+    sess = model.session(B, 4, kv_cache=model.build_kv_cache(B, int8=True))
+    assert sess.persistent is False
+    sess.prefill(ids[:, :P].to(cuda))
+    sess.run(3)
+    assert sess.tokens().shape == (B, 4)
+    with pytest.raises(ValueError, match="int8 caches run the kernel chain"):
+        model.session(B, 4, kv_cache=model.build_kv_cache(B, int8=True), persistent=True)
+    mixed = [model.build_kv_cache(1, int8=True)[0]] + model.build_kv_cache(1)[1:]
+    with pytest.raises(ValueError, match="same KV cache mode"):
+        model(ids[:1, :2].to(cuda), mixed, 0)

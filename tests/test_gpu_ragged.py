@@ -120,9 +120,6 @@ def test_model_forward_with_one_position_per_sequence(cuda):
         model(nxt.to(cuda), cache, [1, 2])
     with pytest.raises(ValueError, match="exceeds max_sequence_length"):
         model(nxt.to(cuda), cache, [95, 96, 3])
-    with pytest.raises(NotImplementedError):
-        q8 = model.build_kv_cache(B, int8=True)
-        model(nxt.to(cuda), q8, [0, 0, 0])
 
 
 @pytest.mark.parametrize("use_graph", [True, False])
@@ -223,3 +220,111 @@ def test_ragged_decode_at_larger_batches(cuda, B):
         _close(got, want)
         pos = [p + 1 for p in pos]
         nxt = want[:, -1].float().argmax(-1).view(B, 1)
+
+
+def test_int8_append_and_attention_per_sequence_positions(cuda):
+    """The int8 cache's append and the attention over its codes with one position per sequence: bit for bit what
+    the scalar-position entry points give sequence by sequence."""
+    from ohara_amd import ops
+    from ohara_amd.llama import KVCache
+
+    B, S, H, Hkv, D, Tmax = 3, 2, 4, 2, 64, 40
+    pos = [7, 0, 31]
+    g = torch.Generator().manual_seed(11)
+    shape = (B, Tmax, Hkv, D)
+    ca, cb = (KVCache(shape, Tmax, 0, device=cuda, dtype=BF, int8=True) for _ in range(2))
+    # a common prefix in both caches (positions 0 .. 31 of every sequence), appended with the scalar entry point
+    pk = (torch.randn(B, 32, Hkv, D, generator=g) * 1.3).to(BF).to(cuda)
+    pv = (torch.randn(B, 32, Hkv, D, generator=g) * 0.4).to(BF).to(cuda)
+    for c in (ca, cb):
+        ops.kv_quant_append(pk, pv, c, 0)
+    k = (torch.randn(B, S, Hkv, D, generator=g) * 1.3).to(BF).to(cuda)
+    v = (torch.randn(B, S, Hkv, D, generator=g) * 0.4).to(BF).to(cuda)
+    q = torch.randn(B * S, H * D, generator=g).to(BF).to(cuda)
+    seq_pos = torch.tensor(pos, dtype=torch.int32, device=cuda)
+    ops.kv_quant_append(k, v, ca, 0, seq_pos=seq_pos)
+    for b in range(B):
+        ops.kv_quant_append(k[b:b + 1], v[b:b + 1], cb._row_view(b), pos[b])
+    assert torch.equal(ca.key, cb.key) and torch.equal(ca.value, cb.value) and torch.equal(ca.stats, cb.stats)
+    for ns in (1, 3):
+        ws = ops.attn_workspace(B * S, H, Hkv, D, ns, cuda)
+        out = ops.attn_cached_int8(q, ca, H, Hkv, D, 0, ns, ws, seq_len=S, seq_pos=seq_pos)
+        for b in range(B):
+            ob = ops.attn_cached_int8(q[b * S:(b + 1) * S], cb._row_view(b), H, Hkv, D, pos[b], ns, ws, seq_len=S)
+            assert torch.equal(ob, out[b * S:(b + 1) * S]), (ns, b)
+
+
+def test_model_forward_with_one_position_per_sequence_on_int8_caches(cuda):
+    """Ragged batches over int8 caches against the oracle run sequence by sequence on its own int8 caches."""
+    ref, model = _small_model(cuda)
+    lens = [5, 23, 1]
+    B = len(lens)
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, 512, (1, n), generator=g) for n in lens]
+    cache = model.build_kv_cache(B, int8=True)
+    for c in cache:
+        c._commit_ragged(B, [0] * B)
+    rcaches = [ref.build_kv_cache(1, int8=True) for _ in range(B)]
+    want_last = []
+    for b, p in enumerate(prompts):
+        views = [c._row_view(b) for c in cache]
+        got = model(p.to(cuda), views, 0)
+        want = ref(p, rcaches[b], 0)
+        _close(got, want, 4e-2, 6e-3)
+        want_last.append(want[:, -1])
+        for c in cache:
+            c.lengths[b] = lens[b]
+            c.length = max(c.lengths)
+    pos = list(lens)
+    nxt = torch.stack([w.float().argmax(-1) for w in want_last]).view(B, 1)
+    for step in range(4):
+        got = model(nxt.to(cuda), cache, pos)
+        want = torch.cat([ref(nxt[b:b + 1], rcaches[b], pos[b]) for b in range(B)])
+        _close(got, want, 4e-2, 6e-3)
+        pos = [p + 1 for p in pos]
+        nxt = want[:, -1].float().argmax(-1).view(B, 1)
+    two = torch.randint(0, 512, (B, 2), generator=g)
+    got = model(two.to(cuda), cache, torch.tensor(pos))
+    want = torch.cat([ref(two[b:b + 1], rcaches[b], pos[b]) for b in range(B)])
+    _close(got, want, 4e-2, 6e-3)
+    # layer 0's codes are the oracle's wherever its rows agree bit for bit with the oracle's: at least the first
+    # position of every sequence (an embedding row through norm, projection and rotary at position 0)
+    assert cache[0].lengths == [p + 2 for p in pos]
+
+
+def test_continuous_batching_on_int8_caches(cuda):
+    """The batcher over int8 caches: the tokens of every slot are those of the same sequence decoded alone by a
+    session on int8 caches (the kernel chain both times; greedy), up to near-ties of the oracle's logits."""
+    from ohara_amd.batching import ContinuousBatcher
+
+    ref, model = _small_model(cuda)
+    g = torch.Generator().manual_seed(9)
+    prompts = {name: torch.randint(0, 512, (n,), generator=g) for name, n in (("a", 9), ("b", 30), ("c", 3))}
+    bat = ContinuousBatcher(model, slots=3, int8=True)
+    assert bat.cache[0].int8
+    out, slot_of = {k: [] for k in prompts}, {}
+    for name in "ab":
+        slot_of[name], tok = bat.add(prompts[name])
+        out[name].append(tok)
+    for _ in range(4):
+        toks = bat.step()
+        for name, slot in slot_of.items():
+            out[name].append(toks[slot])
+    slot_of["c"], tok = bat.add(prompts["c"])
+    out["c"].append(tok)
+    for _ in range(5):
+        toks = bat.step()
+        for name, slot in slot_of.items():
+            out[name].append(toks[slot])
+    for name, toks in out.items():  # oracle on int8 caches, teacher-forced on the tokens the batcher produced
+        rc = ref.build_kv_cache(1, int8=True)
+        logits = ref(prompts[name].view(1, -1), rc, 0)[:, -1]
+        pos = prompts[name].numel()
+        for t, tok in enumerate(toks):
+            best = int(logits.float().argmax(-1))
+            if tok != best:
+                la, lb = logits[0, tok].float().item(), logits[0, best].float().item()
+                ulp = 2.0 ** (torch.tensor(max(abs(la), abs(lb), 1e-30)).log2().floor().item() - 7)
+                assert abs(la - lb) <= 3 * ulp, (name, t, tok, best)
+            logits = ref(torch.tensor([[tok]]), rc, pos)[:, -1]
+            pos += 1
