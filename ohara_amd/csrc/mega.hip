@@ -66,6 +66,7 @@ MegaLayout mega_layout(const OharaModel* m, int B, int nwg) {
 struct MegaPlan {
   int ns, mode;
   size_t smem;
+  int lm_park;  // KB of LDS per wave for parked vocabulary tiles (polled builds)
 };
 
 MegaPlan mega_plan(const OharaModel* m, int batch, int n_workgroups) {
@@ -91,7 +92,11 @@ MegaPlan mega_plan(const OharaModel* m, int batch, int n_workgroups) {
   const size_t smem_polled = smem0 + 256 + (size_t)4 * OHARA_LDS_PF * 1024;
   const bool roles = n_gu + n_dn <= n_workgroups && 2 * n_dn <= n_workgroups;
   const int mode = !roles ? 0 : (batch == 1 ? 1 : (batch <= 8 && smem_polled <= 160 * 1024 ? 2 : 0));
-  return MegaPlan{ns, mode, mode ? smem_polled : smem0};
+  // A single sequence leaves LDS free: the workgroups that park their waves' second vocabulary strip add half of the
+  // third (12 more tiles per wave) where that fits.
+  const size_t smem_more = smem0 + 256 + (size_t)4 * (OHARA_LDS_PF + 12) * 1024;
+  if (mode == 1 && smem_more <= 160 * 1024) return MegaPlan{ns, 1, smem_more, OHARA_LDS_PF + 12};
+  return MegaPlan{ns, mode, mode ? smem_polled : smem0, OHARA_LDS_PF};
 }
 
 }  // namespace
@@ -177,6 +182,7 @@ int ohara_llama_decode_persistent(const OharaModel* m, const OharaDecodeState* s
   const MegaPlan P = mega_plan(m, s->batch, n_workgroups);
   const int mode = P.mode;
   const size_t smem = P.smem;
+  a.lm_park = P.lm_park;
   a.ns = P.ns;
   if (s->kv_int8 && !mode) return OHARA_ESIZE;  // the int8 cache is served by the polled builds only
   if (smem > 160 * 1024) return OHARA_ESIZE;

@@ -72,6 +72,7 @@ struct MegaArgs {
   int tg_rx, tg_rq, tg_rkv, tg_ra;  // bytes between the sequences' rows of those mailboxes
   unsigned int* bar;    // barrier words, see GridSync
   unsigned long long* prof;  // optional: clock of every workgroup's thread 0 at every phase boundary (OHARA_PROF_SLOTS each)
+  int lm_park;  // polled builds: KB of LDS per wave in which a workgroup without a down-projection strip parks vocabulary tiles
   unsigned int spin_limit;
 };
 
@@ -152,6 +153,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
   // gate/up and the down projection (and the output projection and the down projection) to sit on different
   // workgroups, and the general build otherwise.
   uint32_t lm_staged_addr = 0;  // batch 1: where this wave's second vocabulary strip is parked in LDS (0: nowhere)
+  bool lm_extra = false;        // ... followed by the first half of its third strip
   if constexpr (POLLED) {
    {
     // ---- polled hand-offs, no grid barrier inside the layers ------------------------------------------
@@ -199,18 +201,23 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
     const int KSL = (lm.K + 31) >> 5;
     const int lm_strip1 = (nwg + (int)blockIdx.x) * 4 + (int)(threadIdx.x >> 6);
     const bool lm_staged = !has_dn && KSL <= OHARA_LDS_PF && lm_strip1 < lm.nstrips && 2 * nwg * 4 <= lm.nstrips;
-    const int lm_per = (KSL + m.n_layers - 1) / m.n_layers;
-    if (lm_staged) lm_staged_addr = dn.wlds_addr + (uint32_t)(threadIdx.x >> 6) * OHARA_LDS_PF * 1024;
+    // (where the LDS allows it, the first half of the wave's third strip follows the second strip)
+    const int lm_strip2 = lm_strip1 + nwg * 4;
+    if constexpr (ONE && !I8 && !PROFILE) lm_extra = lm_staged && KSL == 24 && a.lm_park >= KSL + 12 && 3 * nwg * 4 <= lm.nstrips;
+    const int lm_tiles = KSL + (lm_extra ? 12 : 0);
+    const int lm_per = (lm_tiles + m.n_layers - 1) / m.n_layers;
+    const int lm_park = ONE ? a.lm_park : OHARA_LDS_PF;
+    if (lm_staged) lm_staged_addr = dn.wlds_addr + (uint32_t)(threadIdx.x >> 6) * (uint32_t)lm_park * 1024;
     for (int l = 0; l < m.n_layers; ++l) {
       auto lm_stage = [&]() {
         if (!lm_staged) return;
-        const int c0 = l * lm_per, c1 = min(KSL, c0 + lm_per);
-        const uint4* src = lm.wp + ((size_t)lm_strip1 * KSL + c0) * 64 + (threadIdx.x & 63);
-        char* dst = wl + ((size_t)(threadIdx.x >> 6) * OHARA_LDS_PF + c0) * 1024;
+        const int c0 = l * lm_per, c1 = min(lm_tiles, c0 + lm_per);
+        char* dst = wl + ((size_t)(threadIdx.x >> 6) * lm_park + c0) * 1024;
 #pragma unroll 1
-        for (int c = c0; c < c1; ++c) {
+        for (int c = c0; c < c1; ++c) {  // tile c of the second strip, then (a single sequence) tile c - KSL of the third
+          const bool third = ONE && !I8 && !PROFILE && c >= KSL;
+          const uint4* src = lm.wp + ((size_t)(third ? lm_strip2 : lm_strip1) * KSL + (third ? c - KSL : c)) * 64 + (threadIdx.x & 63);
           __builtin_amdgcn_global_load_lds((const OHARA_GLOBAL void*)src, (OHARA_LDS void*)dst, 16, 0, 0);
-          src += 64;
           dst += 1024;
         }
       };
@@ -401,7 +408,7 @@ __global__ __launch_bounds__(256) void decode_mega_kernel(MegaArgs a) {
                              pre.g);
   __syncthreads();
   }
-  lm_phase(lm, pre, xs, ldxs, B, best_v, best_i, pf, lm_staged_addr);
+  lm_phase(lm, pre, xs, ldxs, B, best_v, best_i, pf, lm_staged_addr, ONE && !I8 && !PROFILE && lm_extra);
   pf.stamp();
   if (a.select) {
     // lanes with the same batch column (lane & 15) fold their candidates; then the waves

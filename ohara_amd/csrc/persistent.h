@@ -1153,10 +1153,11 @@ __device__ __forceinline__ void gemm_phase(const GemmP& p, const GemmPre& pre, c
 // ---------------------------------------------------------------------------------------
 // `staged` (a byte address in LDS, 0 = nothing): the tiles of this wave's SECOND strip were parked there
 // ahead of the phase (tile c at staged + c KB; strips of at most 24 k-steps); they are multiplied while the
-// first loads from memory are on their way.
+// first loads from memory are on their way.  `extra`: the first chunk (HC tiles) of the THIRD strip follows
+// them there (strips of exactly two chunks).
 template <class PROF>
 __device__ __forceinline__ void lm_phase(const GemmP& p, const GemmPre& pre, const bf16_t* xs, int ldxs, int B,
-                                         float& best_v, int& best_i, PROF& pf, uint32_t staged = 0) {
+                                         float& best_v, int& best_i, PROF& pf, uint32_t staged = 0, bool extra = false) {
   constexpr int HC = 12;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 15, g = lane >> 4;
@@ -1223,9 +1224,11 @@ __device__ __forceinline__ void lm_phase(const GemmP& p, const GemmPre& pre, con
       }
     }
   };
-  // chunks that come from memory, in order: all of them but the staged strip's (chunks ncps .. 2 ncps - 1)
-  auto gq = [&](int k) { return (staged && k >= ncps) ? k + ncps : k; };
-  const int nglob = staged ? total - ncps : total;
+  // chunks that come from memory, in order: all of them but the staged ones (chunks ncps .. 2 ncps - 1, and chunk
+  // 2 ncps with `extra`)
+  const int nskip = staged ? ncps + (extra ? 1 : 0) : 0;
+  auto gq = [&](int k) { return (staged && k >= ncps) ? k + nskip : k; };
+  const int nglob = total - nskip;
   for (int k = 0; k < nglob; k += 2) {
     process(wa, gq(k));
     load(wa, gq(k + 2));
@@ -1244,6 +1247,12 @@ __device__ __forceinline__ void lm_phase(const GemmP& p, const GemmPre& pre, con
 #pragma unroll
         for (int cc = 0; cc < HC; ++cc) wc[cc] = lds16_at(staged + ((uint32_t)min(c * HC + cc, KS - 1) * 64 + lane) * 16);
         process(wc, ncps + c);
+      }
+      if (extra) {  // the third strip's first chunk: its second one is the next chunk from memory
+        uint4 wc[HC];
+#pragma unroll
+        for (int cc = 0; cc < HC; ++cc) wc[cc] = lds16_at(staged + ((uint32_t)(KS + cc) * 64 + lane) * 16);
+        process(wc, 2 * ncps);
       }
     }
   }
