@@ -162,12 +162,13 @@ class Phi:
         config = config or PhiConfig()
         return cls(config, load_huggingface_state_dict(path, config.num_hidden_layers), device=device)
 
-    def build_kv_cache(self, batch_size: int = 1) -> list[KVCache]:
+    def build_kv_cache(self, batch_size: int = 1, int8: bool = False) -> list[KVCache]:
+        """phi.py:189-202; ``int8=True`` builds the int8 caches of ohara/modules/kv_cache.py:15-32."""
         if batch_size < 1:
             raise ValueError("batch_size must be at least 1")  # phi.py:190-191
         c = self.config
         shape = (batch_size, c.max_sequence_length, c.num_attention_heads, self.head_dim)
-        return [KVCache(shape, c.max_sequence_length, i, device=self.device, dtype=BF16)
+        return [KVCache(shape, c.max_sequence_length, i, device=self.device, dtype=BF16, int8=int8)
                 for i in range(c.num_hidden_layers)]
 
     def _buffers(self, rows: int):
@@ -207,8 +208,10 @@ class Phi:
             if position_ids is None:
                 raise ValueError("position_ids is required when using a KV cache")  # phi.py:92-93
             start = int(position_ids)
-        if any(getattr(cache, "int8", False) for cache in kv_cache):
-            raise NotImplementedError("ohara_amd Phi: int8 KV caches are served by the Llama path only")
+        if len({bool(getattr(cache, "int8", False)) for cache in kv_cache}) > 1:
+            raise ValueError("all layers must use the same KV cache mode")
+        if kv_cache[0].int8 and pos_dev is not None:
+            raise NotImplementedError("ohara_amd Phi: a device-resident position (graph replay) needs bf16 KV caches")
         ends = [cache._reserve(B, S, start) for cache in kv_cache]
         logits = self._run(x.reshape(-1).to(device=self.device, dtype=torch.int64), B, S, kv_cache, start, pos_dev, last_only)
         for cache, end in zip(kv_cache, ends):
@@ -222,12 +225,27 @@ class Phi:
         buf = self._buffers(rows)
         cur, nxt = buf["x"]
         ops.embed(ids, self.wte, out=cur)
+        int8 = kv_cache[0].int8
         for L, cache in zip(self.layers, kv_cache):
             ops.layernorm(cur, L["ln_w"], L["ln_b"], c.eps, out=buf["h"])
-            ops.phi_block_in(buf["h"], None, None, c.eps, L["w_in"], L["b_in"], d, self.ff, B, S, start, cache.key,
-                             cache.value, buf["q"], buf["act"], pos_dev)
-            ops.phi_attn(buf["q"], cache.key, cache.value, self.cos, self.sin, self.rot, B, S, H, D, start, pos_dev,
-                         out=buf["attn"], n_split=buf["ns"] if S == 1 else 1, workspace=buf["ws"])
+            if int8:
+                # kv_cache.py:94-118 with quantisation: the new (un-rotated) rows are quantised into the cache and
+                # attention runs over what the reference's cache read returns - the dequantised prefix, the new rows
+                # included - as a bf16 working copy (the rotary attention kernel reads bf16 rows)
+                sk = torch.empty(B, S, H, D, dtype=BF16, device=self.device)
+                sv = torch.empty_like(sk)
+                ops.phi_block_in(buf["h"], None, None, c.eps, L["w_in"], L["b_in"], d, self.ff, B, S, 0, sk, sv, buf["q"],
+                                 buf["act"])
+                ops.kv_quant_append(sk, sv, cache, start)
+                kd = ops.kv_dequant(cache, "key", B, start + S)
+                vd = ops.kv_dequant(cache, "value", B, start + S)
+                ops.phi_attn(buf["q"], kd, vd, self.cos, self.sin, self.rot, B, S, H, D, start, None, out=buf["attn"],
+                             n_split=buf["ns"] if S == 1 else 1, workspace=buf["ws"])
+            else:
+                ops.phi_block_in(buf["h"], None, None, c.eps, L["w_in"], L["b_in"], d, self.ff, B, S, start, cache.key,
+                                 cache.value, buf["q"], buf["act"], pos_dev)
+                ops.phi_attn(buf["q"], cache.key, cache.value, self.cos, self.sin, self.rot, B, S, H, D, start, pos_dev,
+                             out=buf["attn"], n_split=buf["ns"] if S == 1 else 1, workspace=buf["ws"])
             ops.linear_bias(buf["attn"], L["dense"], L["dense_b"], out=buf["mixer"])
             ops.linear_bias(buf["act"], L["fc2"], L["fc2_b"], "add2", add1=buf["mixer"], add2=cur, out=nxt)
             cur, nxt = nxt, cur

@@ -177,12 +177,14 @@ class RefPhi:
         self.dtype = weights["wte.weight"].dtype
         self._f32: dict = {}
 
-    def build_kv_cache(self, batch_size: int = 1):
+    def build_kv_cache(self, batch_size: int = 1, int8: bool = False):
+        """phi.py:189-202; ``int8``: the caches' int8 mode (kv_cache.py:15-32, 94-118: a property of the cache class
+        the model constructs, which quantises the un-rotated rows on write and returns dequantised tensors on read)."""
         if batch_size < 1:
             raise ValueError("batch_size must be at least 1")  # phi.py:190-191
         c = self.cfg
         shape = (batch_size, c.max_sequence_length, c.num_attention_heads, c.head_dim)
-        return [KVCacheRef(shape, c.max_sequence_length, i, dtype=self.dtype) for i in range(c.num_hidden_layers)]
+        return [KVCacheRef(shape, c.max_sequence_length, i, dtype=self.dtype, int8=int8) for i in range(c.num_hidden_layers)]
 
     def block(self, i: int, x, cache, position_ids):
         c, w, p = self.cfg, self.w, f"layers.{i}."

@@ -304,3 +304,34 @@ def test_model_from_local_checkpoint_shards(cuda, tmp_path):
     b = Phi(PhiConfig(**kw), w, device=cuda)
     ids = torch.randint(0, 64, (2, 6), generator=torch.Generator().manual_seed(0)).to(cuda)
     assert torch.equal(a(ids), b(ids))
+
+
+@pytest.mark.parametrize("kw", [
+    dict(vocab_size=80, max_sequence_length=24, num_attention_heads=2, num_hidden_layers=3, multiple_of=2, rotary_dim=0.5),
+    dict(vocab_size=512, max_sequence_length=96, hidden_size=320, num_attention_heads=4, num_hidden_layers=3),  # 80 / 32
+])
+def test_model_on_int8_caches_against_the_oracle(cuda, kw):
+    """Phi on the int8 caches of ohara/modules/kv_cache.py:15-32: the un-rotated rows are quantised on write and attention
+    reads the dequantised prefix; prefill and cached steps against the oracle on its own int8 caches, and layer 0's
+    codes (no attention in front of them) against the oracle quantiser applied to a bf16-cache run's rows."""
+    from oracle import llama_ref as R
+
+    ref, model = _pair(cuda, **kw)
+    c = ref.cfg
+    g = torch.Generator().manual_seed(3)
+    B, S0 = 2, 9
+    ids = torch.randint(0, c.vocab_size, (B, S0 + 3), generator=g)
+    rc, cache = ref.build_kv_cache(B, int8=True), model.build_kv_cache(B, int8=True)
+    assert cache[0].key.dtype == torch.int8
+    _close(model(ids[:, :S0].to(cuda), cache, 0), ref(ids[:, :S0], rc, 0), 4e-2, 6e-3)
+    for t in range(S0, S0 + 3):
+        _close(model(ids[:, t:t + 1].to(cuda), cache, t), ref(ids[:, t:t + 1], rc, t), 4e-2, 6e-3)
+    assert cache[0].length == S0 + 3
+    plain = model.build_kv_cache(B)
+    model(ids[:, :S0].to(cuda), plain, 0)
+    kq, _, _ = R.quantize_int8(plain[0].key[:, :S0].cpu())
+    vq, _, _ = R.quantize_int8(plain[0].value[:, :S0].cpu())
+    assert torch.equal(cache[0].key[:, :S0].cpu(), kq) and torch.equal(cache[0].value[:, :S0].cpu(), vq)
+    mixed = [model.build_kv_cache(1, int8=True)[0]] + model.build_kv_cache(1)[1:]
+    with pytest.raises(ValueError, match="same KV cache mode"):
+        model(ids[:1, :2].to(cuda), mixed, 0)
