@@ -52,7 +52,7 @@ class Config:
     moe_normalize_weights: bool = True
 
 
-def _validate_config(cfg: Config) -> None:
+def _validate_config(cfg: Config, allow_bias: bool = False) -> None:
     # ohara/models/llama.py:208-241
     if cfg.vocab_size < 2:
         raise ValueError("vocab_size must be at least 2")
@@ -69,8 +69,8 @@ def _validate_config(cfg: Config) -> None:
     kv = cfg.num_attention_heads if cfg.num_key_value_heads == 0 else cfg.num_key_value_heads
     if kv < 1 or cfg.num_attention_heads % kv != 0:
         raise ValueError("num_key_value_heads must divide num_attention_heads")
-    if cfg.bias:
-        raise ValueError("ohara_amd: Linear biases are not supported (the reference default is bias=False)")
+    if cfg.bias and not allow_bias:
+        raise ValueError("ohara_amd: Linear biases are served for dense feed-forwards only, by BiasLlama")
 
 
 class KVCache:
@@ -232,6 +232,13 @@ class Llama:
 
                 return MoeLlama(loop_moe_config(config), loop_moe_to_grouped(state or {}), device=device)
             return MoeLlama(config, state, device=device)
+        if cls is Llama and getattr(config, "bias", False):
+            # Linears with a bias (llama.py:60-63, :185): one launch per Linear, in ``BiasLlama``
+            if dtype != BF16:
+                raise ValueError("ohara_amd runs the decode path in bfloat16 only")
+            from .llama_bias import BiasLlama
+
+            return BiasLlama(config, state or {}, device=device)
         return super().__new__(cls)
 
     def __init__(self, config: Config, state: dict, device="cuda", dtype=BF16):

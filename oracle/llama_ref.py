@@ -91,10 +91,12 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-5) -> torch.
     return normed * weight
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, f32_cache: dict | None = None) -> torch.Tensor:
-    """``x @ w.T`` (nn.Linear without bias, llama.py:60-63,252; mlp.py:146-148).
+def linear(x: torch.Tensor, w: torch.Tensor, f32_cache: dict | None = None,
+           bias: torch.Tensor | None = None) -> torch.Tensor:
+    """``x @ w.T (+ bias)`` (nn.Linear, llama.py:60-63,252; mlp.py:146-148; ``bias`` with Config.bias=True).
 
-    fp32 accumulation over the dtype-rounded operands, one rounding to x's dtype.
+    fp32 accumulation over the dtype-rounded operands, the bias added to the fp32 sum, one rounding
+    to x's dtype.
     """
     if w.dtype == torch.float32:
         wf = w
@@ -106,7 +108,10 @@ def linear(x: torch.Tensor, w: torch.Tensor, f32_cache: dict | None = None) -> t
             f32_cache[key] = wf
     else:
         wf = w.float()
-    return (x.float() @ wf.t()).to(x.dtype)
+    y = x.float() @ wf.t()
+    if bias is not None:
+        y = y + bias.float()
+    return y.to(x.dtype)
 
 
 def apply_rope(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor):
@@ -370,6 +375,18 @@ def weight_names(cfg: RefConfig):
             ]
         out += [(p + "norm1.weight", (d,), "ones"), (p + "norm2.weight", (d,), "ones")]
     out += [("norm.weight", (d,), "ones"), ("vocab_proj.weight", (V, d), "normal")]
+    if cfg.bias:
+        # llama.py:60-63 and :185 (mlp.py:146-148): a bias on every attention projection and on a dense
+        # feed-forward's three Linears, never on vocab_proj (llama.py:252).  Drawn after all the matrices,
+        # so that a config's matrices do not depend on the flag; the reference starts them at zero
+        # (llama.py:429-430), here they are drawn like the matrices so that a dropped bias shows.
+        for i in range(cfg.num_hidden_layers):
+            p = f"layers.{i}."
+            out += [(p + "attn.key.bias", (Hkv * D,), "normal"), (p + "attn.query.bias", (H * D,), "normal"),
+                    (p + "attn.value.bias", (Hkv * D,), "normal"), (p + "attn.proj.bias", (d,), "normal")]
+            if not cfg.layer_is_moe(i):
+                out += [(p + "ff.up.bias", (F_,), "normal"), (p + "ff.down.bias", (d,), "normal"),
+                        (p + "ff.gate.bias", (F_,), "normal")]
     return out
 
 
@@ -434,7 +451,7 @@ class RefLlama:
             y = bitlinear_forward(x.reshape(-1, shp[-1]), w[name + ".rms_norm.weight"],
                                   w[name + ".ternary"], w[name + ".gamma"])
             return y.view(*shp[:-1], -1)
-        return linear(x, w[name + ".weight"], self._f32)
+        return linear(x, w[name + ".weight"], self._f32, w.get(name + ".bias"))
 
     def _attn(self, i, h, cos, sin, cache, start_pos):
         c, w = self.config, self.w

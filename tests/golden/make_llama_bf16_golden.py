@@ -14,13 +14,16 @@ buffers), run on the CPU through the KV cache.  Every file holds plain tensors
                      last 4 prompt positions, ``ops_step0/...`` for the first cached step, with every
                      layer's cache as that step read it): each operator can be checked on the reference's
                      own operands, where one flipped bit does not travel through the layers behind it
+  mid_bias           ``Config.bias=True`` (llama.py:60-63, :185): hidden 256, 3 layers, 4 query / 2 KV heads of
+                     width 64, 24-token prompt + 3 steps, batch 2, with the same module inputs and outputs; the
+                     biases are drawn like the matrices (the reference starts them at zero)
   d12w               the d12 widths (hidden 768, 12 layers, 6 heads x 128, FFN 3072) with a 4096-entry
                      vocabulary: 600-token prompt (two key blocks of the library's attention kernel) + 3 steps
   d12_greedy         the full d12 model of the benchmark (vocabulary 65536, cache 4096), batch 1,
                      1024-token prompt, 64 greedy tokens: the tokens, and per step the logits at 2048
                      fixed vocabulary columns plus the 32 largest logits with their ids
 
-mid_gqa, d12w and d12_greedy are run three times: with all threads, with one (``*_one_thread``) and with
+mid_gqa, mid_bias, d12w and d12_greedy are run three times: with all threads, with one (``*_one_thread``) and with
 the library's other set of CPU matrix kernels (oneDNN switched off, ``*_other_kernels``); d12_greedy's
 repeats are fed the first run's tokens.  Same code, same inputs, another summation order inside the
 library's products.  The distances between the runs are how far the reference reproduces itself.
@@ -51,6 +54,10 @@ SEEDED = {
     "mid_gqa": dict(cfg=dict(vocab_size=512, hidden_size=256, intermediate_size=704, num_attention_heads=4,
                              num_key_value_heads=2, num_hidden_layers=4, max_sequence_length=64, dropout=0.0),
                     seed=11, batch=2, prompt=40, steps=3, ops=True),
+    "mid_bias": dict(cfg=dict(vocab_size=512, hidden_size=256, intermediate_size=704, num_attention_heads=4,
+                              num_key_value_heads=2, num_hidden_layers=3, max_sequence_length=64, dropout=0.0,
+                              bias=True),
+                     seed=13, batch=2, prompt=24, steps=3, ops=True),
     "d12w": dict(cfg=dict(vocab_size=4096, hidden_size=768, intermediate_size=3072, num_attention_heads=6,
                           num_key_value_heads=0, num_hidden_layers=12, max_sequence_length=1024, dropout=0.0),
                  seed=12, batch=1, prompt=600, steps=3),
@@ -238,7 +245,7 @@ def alias_duplicates(out: dict) -> dict:
 
 
 def main(argv):
-    cases = argv or ["tiny_dense", "tiny_gqa", "tiny_moe", "mid_gqa", "d12w", "d12_greedy"]
+    cases = argv or ["tiny_dense", "tiny_gqa", "tiny_moe", "mid_gqa", "mid_bias", "d12w", "d12_greedy"]
     torch.manual_seed(0)
     for name in cases:
         if name.startswith("tiny_"):

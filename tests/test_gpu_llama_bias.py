@@ -1,0 +1,57 @@
+"""Llama with ``Config.bias=True`` (ohara/models/llama.py:60-63, :185; ohara/modules/mlp.py:146-148): the forward
+through the KV cache against the oracle on the same seeded weights, biases included."""
+
+import pytest
+import torch
+
+from oracle import llama_ref as R
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+
+
+def _close(got, want, mx=2e-2, mean=2e-3):
+    d = (got.float().cpu() - want.float()).abs()
+    scale = want.float().abs().max().item()
+    assert d.max().item() <= mx * scale and d.mean().item() <= mean * scale, (d.max().item(), d.mean().item(), scale)
+
+
+@pytest.mark.parametrize("kw,B,P", [
+    (dict(vocab_size=384, hidden_size=256, intermediate_size=640, num_attention_heads=2, num_key_value_heads=0,
+          num_hidden_layers=3, max_sequence_length=96), 2, 40),                      # 2 heads x 128
+    (dict(vocab_size=512, hidden_size=256, intermediate_size=704, num_attention_heads=4, num_key_value_heads=2,
+          num_hidden_layers=2, max_sequence_length=64, weight_tying=True), 3, 7),    # GQA, tied vocabulary matrix
+])
+@pytest.mark.parametrize("int8", [False, True])
+def test_forward_through_the_cache_against_the_oracle(cuda, kw, B, P, int8):
+    from ohara_amd.llama import Config, Llama
+    from ohara_amd.llama_bias import BiasLlama
+
+    rcfg = R.RefConfig(bias=True, **kw)
+    w = R.init_weights(rcfg, seed=5, dtype=BF, norm_jitter=0.1)
+    assert "layers.0.attn.proj.bias" in w and "layers.1.ff.down.bias" in w
+    ref = R.RefLlama(rcfg, w)
+    model = Llama(Config(bias=True, **kw), w, device=cuda)
+    assert isinstance(model, BiasLlama)
+    ids = torch.randint(0, kw["vocab_size"], (B, P + 3), generator=torch.Generator().manual_seed(P))
+    rc, cache = ref.build_kv_cache(B, int8=int8), model.build_kv_cache(B, int8=int8)
+    _close(model(ids[:, :P].to(cuda), cache, 0), ref(ids[:, :P], rc, 0))
+    for t in range(P, P + 3):
+        _close(model(ids[:, t:t + 1].to(cuda), cache, t), ref(ids[:, t:t + 1], rc, t))
+    assert cache[0].length == P + 3
+    if not int8:
+        _close(model(ids.to(cuda)), ref(ids))  # the uncached call
+        last = model(ids[:, :P].to(cuda), model.build_kv_cache(B), 0, last_only=True)
+        _close(last, ref(ids[:, :P])[:, -1:])
+    # a dropped bias is far outside the bound: the same weights without them
+    nb = {k: v for k, v in w.items() if not k.endswith(".bias")}
+    plain = R.RefLlama(R.RefConfig(**kw), nb)(ids[:, :P])
+    want = ref(ids[:, :P])
+    assert (plain.float() - want.float()).abs().mean().item() > 2e-2 * want.float().abs().max().item()
+
+
+def test_biases_with_routed_experts_are_refused(cuda):
+    from ohara_amd.llama import Config, Llama
+
+    with pytest.raises(ValueError, match="biases"):
+        Llama(Config(bias=True, moe_num_experts=4, moe_grouped=True), {}, device=cuda)

@@ -155,7 +155,32 @@ def test_tiny_models_against_the_reference_in_bf16(cuda, name):
     assert identical_fraction(cache[0].value[:, :7].cpu(), fx["cache0_value"]) >= 0.98
 
 
-@pytest.mark.parametrize("name", ["mid_gqa", "d12w"])
+def test_linears_with_bias_on_the_references_operands(cuda):
+    """The Linear-with-bias kernel fed with what the reference's biased Linears received (Config.bias=True:
+    llama.py:60-63, :185), against what they returned: the prefill's last four positions and one cached step."""
+    from ohara_amd import ops
+
+    fx = load_fixture("llama_bf16_mid_bias.pt")
+    rcfg, _ = _cfg_pair(fx["config"])
+    w = R.init_weights(rcfg, seed=fx["seed"], dtype=BF, norm_jitter=fx["norm_jitter"])
+    assert torch.allclose(weight_checksum(w), fx["weight_checksum"], rtol=1e-12)
+    total = same = 0
+    for call in ("ops_step0", "ops_prefill"):
+        for i in range(rcfg.num_hidden_layers):
+            for n in ("attn.key", "attn.query", "attn.value", "attn.proj", "ff.up", "ff.gate", "ff.down"):
+                name = f"layers.{i}.{n}"
+                x, y = fx[f"{call}/{name}/in"], fx[f"{call}/{name}/out"]
+                x2, y2 = x.reshape(-1, x.size(-1)), y.reshape(-1, y.size(-1))
+                got = ops.linear_bias(x2.to(cuda), ops.pack_linear(w[name + ".weight"].to(cuda)),
+                                      w[name + ".bias"].to(cuda)).cpu()
+                total += y2.numel()
+                same += int((got.view(torch.int16) == y2.contiguous().view(torch.int16)).sum())
+                assert (got.float() - y2.float()).abs().max().item() <= y2.float().abs().max().item() * 2.0 ** -8, name
+    _report("linear_bias_on_reference_operands", {"identical": same / total})
+    assert same / total >= 0.998
+
+
+@pytest.mark.parametrize("name", ["mid_gqa", "mid_bias", "d12w"])
 def test_seeded_models_against_the_reference_in_bf16(cuda, name):
     from ohara_amd.llama import Llama
 
@@ -170,8 +195,8 @@ def test_seeded_models_against_the_reference_in_bf16(cuda, name):
     self_mean = reference_self_distance(fx)
     stats = {"reference_vs_itself_mean_worst_row": self_mean}
     for persistent in (False, True):
-        if persistent and not model.supports_persistent(ids.size(0)):
-            continue
+        if persistent and not (hasattr(model, "supports_persistent") and model.supports_persistent(ids.size(0))):
+            continue  # (a config with Linear biases runs one launch per Linear)
         got = {}
         if persistent:
             # the single-launch kernel: a session fed the fixture's tokens

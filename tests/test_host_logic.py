@@ -234,7 +234,7 @@ def test_config_and_kv_cache_bookkeeping():
     from ohara_amd.llama import Llama
 
     with pytest.raises(ValueError, match="biases"):
-        Llama(Config(bias=True), {})
+        Llama(Config(bias=True, moe_num_experts=4, moe_grouped=True), {})  # biases: dense feed-forwards only
     # a loop-form MoE config (llama.py:171-178) is served by the grouped kernels: no shared expert, sigmoid
     # weights as they are, expert weights restacked as (E, dim, hidden) / (E, hidden, dim)
     from ohara_amd.checkpoint import loop_moe_config, loop_moe_to_grouped

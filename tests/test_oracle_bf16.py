@@ -101,8 +101,9 @@ def test_attention_bf16_reproduces_the_library_routine(B, H, Hkv, S, L, D):
 # ---- operator by operator on the reference's operands ------------------------------------------------
 
 
-def test_every_operator_on_the_references_own_operands():
-    fx = load_fixture("llama_bf16_mid_gqa.pt")
+@pytest.mark.parametrize("name", ["mid_gqa", "mid_bias"])
+def test_every_operator_on_the_references_own_operands(name):
+    fx = load_fixture(f"llama_bf16_{name}.pt")
     cfg = _cfg(fx["config"])
     w = R.init_weights(cfg, seed=fx["seed"], dtype=BF, norm_jitter=fx["norm_jitter"])
     assert torch.allclose(weight_checksum(w), fx["weight_checksum"], rtol=1e-12)
@@ -122,7 +123,9 @@ def test_every_operator_on_the_references_own_operands():
                 assert torch.equal(R.rms_norm(x, w[p + n + ".weight"]), y), (call, p + n)
             for n in ("attn.key", "attn.query", "attn.value", "attn.proj", "ff.up", "ff.gate", "ff.down"):
                 x, y = io(p + n)
-                got = R.linear(x, w[p + n + ".weight"])
+                got = R.linear(x, w[p + n + ".weight"], bias=w.get(p + n + ".bias"))
+                if cfg.bias:  # llama.py:60-63, mlp.py:146-148: the bias is there, and dropping it is seen
+                    assert identical_fraction(R.linear(x, w[p + n + ".weight"]), y) < 0.5
                 worst_linear = min(worst_linear, identical_fraction(got, y))
                 # one bf16 step where the fp32 sums straddle a rounding boundary (more only where a sum
                 # cancels to next to nothing)
@@ -194,7 +197,7 @@ def test_tiny_models_in_bf16(name):
         assert mx <= 2e-2 and mean <= 2e-3, (tag, mx, mean)
 
 
-@pytest.mark.parametrize("name", ["mid_gqa", "d12w"])
+@pytest.mark.parametrize("name", ["mid_gqa", "mid_bias", "d12w"])
 def test_seeded_models_lie_as_close_to_the_reference_as_it_lies_to_itself(name):
     fx = load_fixture(f"llama_bf16_{name}.pt")
     cfg = _cfg(fx["config"])
