@@ -55,3 +55,36 @@ def test_biases_with_routed_experts_are_refused(cuda):
 
     with pytest.raises(ValueError, match="biases"):
         Llama(Config(bias=True, moe_num_experts=4, moe_grouped=True), {}, device=cuda)
+
+
+def test_inference_engine_drives_the_model(cuda):
+    """ohara/inference.py:67-127 over a model without a decode session: the stepwise loop, greedy; every
+    token is the oracle's arg-max (or its near-tie) when the oracle is fed the same tokens."""
+    from ohara_amd.inference import Inference
+    from ohara_amd.llama import Config, Llama
+
+    kw = dict(vocab_size=96, hidden_size=128, intermediate_size=256, num_attention_heads=2, num_key_value_heads=1,
+              num_hidden_layers=2, max_sequence_length=32)
+    rcfg = R.RefConfig(bias=True, **kw)
+    w = R.init_weights(rcfg, seed=9, dtype=BF, std=0.08)
+    model = Llama(Config(bias=True, **kw), w, device=cuda)
+
+    class Tok:
+        eos_token_id = -1
+
+        def encode(self, text):
+            return [ord(c) - 32 for c in text]
+
+        def decode(self, ids):
+            return "".join(chr(i + 32) for i in ids)
+
+    prompt = "bias!"
+    out = Inference(model, Tok(), cuda, max_new_tokens=10).generate(prompt, temperature=0.0, stream=False)
+    assert out.startswith(prompt) and len(out) == len(prompt) + 10
+    ids = torch.tensor([Tok().encode(out)])
+    ref = R.RefLlama(rcfg, w)
+    logits = ref(ids)[0].float()
+    for t in range(len(prompt) - 1, ids.size(1) - 1):
+        row, chosen = logits[t], int(ids[0, t + 1])
+        gap = (row.max() - row[chosen]).item()
+        assert gap <= 2.0 ** -6 * row.abs().max().item(), (t, chosen, int(row.argmax()), gap)
