@@ -250,6 +250,15 @@ int ohara_sample_topk_topp_exclusive(const void* logits, int logits_are_fp32, in
                            int valid_vocab, float temperature, int top_k, float top_p, const float* u,
                            int u_step_stride, int64_t* out_ids, int64_t* history, int hist_cap,
                            int32_t* step_state, void* stream);
+/* The same spread selection with the candidates meeting in the CALLER's workspace instead of the library's
+ * array: calls with different workspaces may overlap in time (one workspace per decode session / stream).
+ * workspace: ohara_sample_workspace_bytes() bytes of device memory, 256-byte aligned, zeroed once before its
+ * first use (the kernels leave its counters at zero); calls sharing one workspace must not overlap. */
+int64_t ohara_sample_workspace_bytes(void);
+int ohara_sample_topk_topp_ws(const void* logits, int logits_are_fp32, int ldl, int batch, int vocab,
+                              int valid_vocab, float temperature, int top_k, float top_p, const float* u,
+                              int u_step_stride, int64_t* out_ids, int64_t* history, int hist_cap,
+                              int32_t* step_state, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ---- BitNet-b1.58 BitLinear (ternary weights x int8 activations, int32 accumulate) ------
  * Integer form of BitLinear.forward (experiments/bitnet/bitnet.py:29-59):

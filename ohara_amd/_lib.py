@@ -87,6 +87,8 @@ _PROTOS = {
     "ohara_argmax_bf16": (_i, [_p, _i, _i, _i, _i, _p, _p, _i, _p, _p]),
     "ohara_sample_topk_topp": (_i, [_p, _i, _i, _i, _i, _i, _f, _i, _f, _p, _i, _p, _p, _i, _p, _p]),
     "ohara_sample_topk_topp_exclusive": (_i, [_p, _i, _i, _i, _i, _i, _f, _i, _f, _p, _i, _p, _p, _i, _p, _p]),
+    "ohara_sample_workspace_bytes": (_i64, []),
+    "ohara_sample_topk_topp_ws": (_i, [_p, _i, _i, _i, _i, _i, _f, _i, _f, _p, _i, _p, _p, _i, _p, _p, _i64, _p]),
     "ohara_bitlinear_pack_ternary": (_i, [_p, _i, _i, _i, _p, C.POINTER(_i64), _p]),
     "ohara_act_quant_int8": (_i, [_p, _i, _p, _f, _i, _i, _p, _i, _p, _p, _p]),
     "ohara_gemv_ternary_i8": (_i, [_p, _i, _p, _p, _p, _i, _i, _f, _i, _p, _i, _p, _i, _p, _i, _p]),

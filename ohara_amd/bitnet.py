@@ -235,6 +235,7 @@ class BitDecodeSession:
             if u.shape != (rows, batch):
                 raise ValueError("u must have shape (max_new_tokens, batch)")
             self.u = u.to(device=model.device, dtype=torch.float32).contiguous()
+            self._sample_ws = ops.sample_workspace(model.device)  # this session's own: sessions may overlap
         self.cache = kv_cache if kv_cache is not None else model.build_kv_cache(batch)
         int8 = any(cc.int8 for cc in self.cache)  # int8 caches are served by the kernel chain
         if persistent is None:
@@ -325,7 +326,7 @@ class BitDecodeSession:
         if self.sampling:
             ops.sample_topk_topp(self.logits, self.sampling.temperature, self.sampling.top_k, self.sampling.top_p,
                                  self.u, self.valid_vocab or None, out=self.ids, history=self.history,
-                                 step_state=self.step_state, u_per_step=True, exclusive=True)
+                                 step_state=self.step_state, u_per_step=True, workspace=self._sample_ws)
 
     def check_error(self) -> None:
         """Raise if a barrier wait of the persistent kernel expired (synchronises)."""

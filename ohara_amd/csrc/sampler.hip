@@ -1685,7 +1685,8 @@ int launch_sample(const SampleArgs& a, hipStream_t st) {
 
 int sample_dispatch(const void* logits, int logits_are_fp32, int ldl, int batch, int vocab, int valid_vocab,
                     float temperature, int top_k, float top_p, const float* u, int u_step_stride, int64_t* out_ids,
-                    int64_t* history, int hist_cap, int32_t* step_state, void* stream, bool exclusive) {
+                    int64_t* history, int hist_cap, int32_t* step_state, void* stream, bool exclusive,
+                    uint32_t* workspace = nullptr) {
   if (!logits || !u || !out_ids || batch < 1 || vocab < 1 || ldl < vocab) return OHARA_EINVAL;
   if (!(temperature > 0.f) || top_k < 0 || !(top_p >= 0.f && top_p <= 1.f) || u_step_stride < 0) return OHARA_EINVAL;
   SampleArgs a{};
@@ -1698,7 +1699,7 @@ int sample_dispatch(const void* logits, int logits_are_fp32, int ldl, int batch,
   // over one workgroup per 8192 ids (measured at 65536 ids, top-k 50 + top-p 0.9: see the header)
   if (exclusive && !logits_are_fp32 && aligned && top_k > 0 && top_k <= 64 && vocab > PART_IDS &&
       vocab <= PART_IDS * PART_MAX && batch <= PART_ROWS && (a.valid < vocab ? a.valid : vocab) >= top_k) {
-    uint32_t* scratch = sampler_scratch_ptr();
+    uint32_t* scratch = workspace ? workspace : sampler_scratch_ptr();  // the caller's own, or the library's
     if (!scratch) return OHARA_ELAUNCH;
     const int nparts = (vocab + PART_IDS - 1) / PART_IDS;
     hipLaunchKernelGGL(sample_parts_kernel, dim3(nparts, batch), dim3(NT), 0, st, a, scratch, nparts);
@@ -1735,6 +1736,20 @@ int ohara_sample_topk_topp_exclusive(const void* logits, int logits_are_fp32, in
                                      int32_t* step_state, void* stream) {
   return sample_dispatch(logits, logits_are_fp32, ldl, batch, vocab, valid_vocab, temperature, top_k, top_p, u,
                          u_step_stride, out_ids, history, hist_cap, step_state, stream, true);
+}
+
+int64_t ohara_sample_workspace_bytes(void) { return (int64_t)(PART_SCRATCH_DWORDS * sizeof(uint32_t)); }
+
+int ohara_sample_topk_topp_ws(const void* logits, int logits_are_fp32, int ldl, int batch, int vocab, int valid_vocab,
+                              float temperature, int top_k, float top_p, const float* u, int u_step_stride,
+                              int64_t* out_ids, int64_t* history, int hist_cap, int32_t* step_state, void* workspace,
+                              int64_t workspace_bytes, void* stream) {
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) ||
+      workspace_bytes < (int64_t)(PART_SCRATCH_DWORDS * sizeof(uint32_t)))
+    return OHARA_EINVAL;
+  return sample_dispatch(logits, logits_are_fp32, ldl, batch, vocab, valid_vocab, temperature, top_k, top_p, u,
+                         u_step_stride, out_ids, history, hist_cap, step_state, stream, true,
+                         static_cast<uint32_t*>(workspace));
 }
 
 }  // extern "C"

@@ -531,6 +531,8 @@ class DecodeSession:
             if u.shape != (rows, batch):
                 raise ValueError("u must have shape (max_new_tokens, batch)")
             self.u = u.to(device=model.device, dtype=torch.float32).contiguous()
+            # the sampler's workgroups meet in a buffer of this session's own: sessions on other streams may overlap
+            self._sample_ws = ops.sample_workspace(model.device)
         if persistent is None:
             # measured on d12: the single launch wins up to eight sequences (0.40 ms against 0.48 ms
             # per step at 4, 0.49 against 0.49 at 8); beyond that the kernel chain is faster (0.52
@@ -654,7 +656,7 @@ class DecodeSession:
             # the sampler does the selection kernel's bookkeeping (next ids, history, position)
             ops.sample_topk_topp(self.logits, self.sampling.temperature, self.sampling.top_k, self.sampling.top_p,
                                  self.u, self.valid_vocab or None, out=self._dbuf.ids[: self.batch],
-                                 history=self.history, step_state=self._dbuf.step_state, u_per_step=True, exclusive=True)
+                                 history=self.history, step_state=self._dbuf.step_state, u_per_step=True, workspace=self._sample_ws)
 
     def error_word(self):
         """The persistent kernel's sticky error word as a one-element int32 device view (None for the

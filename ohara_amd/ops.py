@@ -325,11 +325,13 @@ def argmax(logits: torch.Tensor, valid_vocab: int | None = None, next_ids=None, 
 
 def sample_topk_topp(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, u: torch.Tensor,
                      valid_vocab: int | None = None, out=None, history=None, step_state=None,
-                     u_per_step: bool = False, exclusive: bool = False) -> torch.Tensor:
+                     u_per_step: bool = False, exclusive: bool = False, workspace=None) -> torch.Tensor:
     """logits (B, V) bf16 or fp32 on the device, u (B,) fp32 uniform draws -> ids (B,) int64.
     With ``u_per_step`` (needs step_state) u is (steps, B) and row ``step`` is read on the device.
     ``exclusive``: the caller's sampler calls on this GPU do not overlap in time (a decode loop on one
-    stream), which lets a small top-k on a long row run on several workgroups (same results)."""
+    stream), which lets a small top-k on a long row run on several workgroups (same results).
+    ``workspace`` (``sample_workspace``): the same with the workgroups meeting in the caller's buffer instead of
+    the library's, so that callers with a workspace each may overlap (one per decode session)."""
     if logits.dtype not in (BF16, torch.float32):
         raise ValueError("logits must be bfloat16 or float32")
     _need(logits, logits.dtype, "logits")
@@ -342,15 +344,21 @@ def sample_topk_topp(logits: torch.Tensor, temperature: float, top_k: int, top_p
         raise ValueError("one uniform draw per row is required")
     if out is None:
         out = torch.empty(b, dtype=torch.int64, device=logits.device)
-    check(
-        (lib().ohara_sample_topk_topp_exclusive if exclusive else lib().ohara_sample_topk_topp)(
-            _ptr(logits), 1 if logits.dtype == torch.float32 else 0, logits.stride(0), b, v,
+    args = (_ptr(logits), 1 if logits.dtype == torch.float32 else 0, logits.stride(0), b, v,
             v if valid_vocab is None else valid_vocab, float(temperature), int(top_k), float(top_p), _ptr(u),
-            b if u_per_step else 0, _ptr(out), _ptr(history), 0 if history is None else history.shape[0], _ptr(step_state), _stream(),
-        ),
-        "sample_topk_topp",
-    )
+            b if u_per_step else 0, _ptr(out), _ptr(history), 0 if history is None else history.shape[0], _ptr(step_state))
+    if workspace is not None:
+        _need(workspace, torch.uint8, "workspace")
+        check(lib().ohara_sample_topk_topp_ws(*args, _ptr(workspace), workspace.numel(), _stream()), "sample_topk_topp")
+        return out
+    check((lib().ohara_sample_topk_topp_exclusive if exclusive else lib().ohara_sample_topk_topp)(*args, _stream()),
+          "sample_topk_topp")
     return out
+
+
+def sample_workspace(device) -> torch.Tensor:
+    """A zeroed workspace for ``sample_topk_topp(..., workspace=)``: one per caller whose calls may overlap others'."""
+    return torch.zeros(lib().ohara_sample_workspace_bytes(), dtype=torch.uint8, device=device)
 
 
 # ---- BitLinear ---------------------------------------------------------------------------------

@@ -231,3 +231,34 @@ def test_small_top_k_over_several_workgroups(cuda, V, B, T, k, p, std):
         if excl:
             assert torch.equal(hist, first_hist) and state.tolist() == [7 + steps, steps, 0, 0]
         first_hist = hist.clone()
+
+
+def test_sampler_with_the_callers_workspace(cuda):
+    """ohara_sample_topk_topp_ws: the spread selection meeting in a caller-owned workspace gives the
+    single-workgroup kernel's tokens, on calls in a row and on two streams that each bring their own
+    workspace (what two sampling decode sessions do); a short or misaligned workspace is refused."""
+    from ohara_amd import ops
+
+    V, B, T, k, p = 65536, 8, 0.8, 50, 0.9
+    g = torch.Generator().manual_seed(17)
+    rows = [(torch.randn(B, V, generator=g) * 0.55).to(torch.bfloat16).to(cuda) for _ in range(2)]
+    us = [torch.rand(6, B, generator=g).to(cuda) for _ in range(2)]
+    want = [[ops.sample_topk_topp(rows[i], T, k, p, us[i][j]).cpu() for j in range(6)] for i in range(2)]
+    ws = [ops.sample_workspace(cuda) for _ in range(2)]
+    for j in range(3):  # one stream, calls in a row: the counters return to zero
+        assert torch.equal(ops.sample_topk_topp(rows[0], T, k, p, us[0][j], workspace=ws[0]).cpu(), want[0][j])
+    streams = [torch.cuda.Stream() for _ in range(2)]
+    outs = [[torch.empty(B, dtype=torch.int64, device=cuda) for _ in range(6)] for _ in range(2)]
+    torch.cuda.synchronize()
+    for j in range(6):
+        for i in range(2):
+            with torch.cuda.stream(streams[i]):
+                ops.sample_topk_topp(rows[i], T, k, p, us[i][j], out=outs[i][j], workspace=ws[i])
+    torch.cuda.synchronize()
+    for i in range(2):
+        for j in range(6):
+            assert torch.equal(outs[i][j].cpu(), want[i][j]), (i, j)
+    with pytest.raises(Exception):
+        ops.sample_topk_topp(rows[0], T, k, p, us[0][0], workspace=ws[0][: ws[0].numel() // 2])
+    with pytest.raises(Exception):
+        ops.sample_topk_topp(rows[0], T, k, p, us[0][0], workspace=torch.zeros(ws[0].numel() + 64, dtype=torch.uint8, device=cuda)[8:])
