@@ -99,14 +99,8 @@ class ContinuousBatcher:
         ops.advance_positions(self.seq_pos, self.active_dev, 1)
         self.last.copy_(torch.where(self.active_dev.bool(), self._toks, torch.zeros_like(self._toks)))
 
-    @torch.no_grad()
-    def step(self, use_graph: bool = True) -> dict[int, int]:
-        """One decode step for every active slot -> {slot: new id}.  Idle slots ride along at
-        position 0 of their own cache rows (overwritten when the slot is taken again).  The device
-        work is captured once into a HIP graph (positions, inputs and the active mask live in
-        device tensors, so joins and leaves need no re-capture) and replayed per step."""
-        if not any(self.active):
-            return {}
+    def _enqueue_step(self, use_graph: bool) -> None:
+        """One decode step of every active slot, enqueued; the host books advance, nothing is read back."""
         if max(n for n, a in zip(self.lengths, self.active) if a) + 1 > self.model.config.max_sequence_length:
             raise ValueError("input exceeds max_sequence_length")
         if self._toks is None:
@@ -132,5 +126,31 @@ class ContinuousBatcher:
         for c in self.cache:
             c.lengths = list(self.lengths)
             c.length = max(self.lengths)
+
+    @torch.no_grad()
+    def step(self, use_graph: bool = True) -> dict[int, int]:
+        """One decode step for every active slot -> {slot: new id}.  Idle slots ride along at
+        position 0 of their own cache rows (overwritten when the slot is taken again).  The device
+        work is captured once into a HIP graph (positions, inputs and the active mask live in
+        device tensors, so joins and leaves need no re-capture) and replayed per step."""
+        if not any(self.active):
+            return {}
+        self._enqueue_step(use_graph)
         host = self._toks.tolist()
+        return {b: host[b] for b in range(self.slots) if self.active[b]}
+
+    @torch.no_grad()
+    def steps(self, n: int, use_graph: bool = True) -> dict[int, list[int]]:
+        """``n`` decode steps of every active slot with ONE read-back at the end -> {slot: its n new ids}: the
+        chunked read-back of the single-sequence engines (a stop id is looked for in the chunk afterwards; a
+        slot that met one has run on to the end of the chunk and is trimmed and removed by the caller)."""
+        if n < 1 or not any(self.active):
+            return {}
+        if max(m for m, a in zip(self.lengths, self.active) if a) + n > self.model.config.max_sequence_length:
+            raise ValueError("input exceeds max_sequence_length")
+        rows = torch.empty(n, self.slots, dtype=torch.int64, device=self.model.device)
+        for i in range(n):
+            self._enqueue_step(use_graph)
+            rows[i].copy_(self._toks)
+        host = rows.t().tolist()
         return {b: host[b] for b in range(self.slots) if self.active[b]}

@@ -122,10 +122,11 @@ def test_model_forward_with_one_position_per_sequence(cuda):
         model(nxt.to(cuda), cache, [95, 96, 3])
 
 
-@pytest.mark.parametrize("use_graph", [True, False])
-def test_continuous_batching_matches_sequences_run_alone(cuda, use_graph):
+@pytest.mark.parametrize("use_graph,chunked", [(True, False), (False, False), (True, True)])
+def test_continuous_batching_matches_sequences_run_alone(cuda, use_graph, chunked):
     """Sequences join and leave at different times; every token a slot produces is the oracle's
-    greedy choice for that sequence alone (or a near-tie of the oracle's own logits)."""
+    greedy choice for that sequence alone (or a near-tie of the oracle's own logits).  ``chunked``: several
+    steps per read-back (``ContinuousBatcher.steps``)."""
     from ohara_amd.batching import ContinuousBatcher
 
     ref, model = _small_model(cuda)
@@ -141,6 +142,12 @@ def test_continuous_batching_matches_sequences_run_alone(cuda, use_graph):
         out[name].append(tok)
 
     def steps(n):
+        if chunked:
+            got = bat.steps(n, use_graph=use_graph)
+            for name, slot in slot_of.items():
+                assert len(got[slot]) == n
+                out[name].extend(got[slot])
+            return
         for _ in range(n):
             toks = bat.step(use_graph=use_graph)
             for name, slot in slot_of.items():
