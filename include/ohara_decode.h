@@ -152,6 +152,10 @@ int ohara_attn_cached_ragged_bf16(const uint16_t* q, const uint16_t* kcache, con
 /* seq_pos[b] += by for every b with active[b] != 0 (active NULL: all): advances a ragged batch by one
  * decode step without host involvement (graph replay). */
 int ohara_advance_positions(int32_t* seq_pos, const uint8_t* active, int batch, int by, void* stream);
+/* The same in one launch with the next step's inputs: next_ids[b] = new_ids[b] for an active sequence, 0 for
+ * an idle slot (it rides along at position 0).  No counterpart in the reference (one position for the batch). */
+int ohara_advance_ragged(int32_t* seq_pos, const uint8_t* active, const int64_t* new_ids, int64_t* next_ids, int batch,
+                         int by, void* stream);
 
 /* ohara_attn_cached_bf16 for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the

@@ -83,6 +83,7 @@ _PROTOS = {
     "ohara_attn_cached_ragged_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p]),
     "ohara_qkv_rope_append_ragged_bf16": (_i, [_p, _i, _p, _i, _p, _f, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _i, _p]),
     "ohara_advance_positions": (_i, [_p, _p, _i, _i, _p]),
+    "ohara_advance_ragged": (_i, [_p, _p, _p, _p, _i, _i, _p]),
     "ohara_attn_prefill_bf16": (_i, [_p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p]),
     "ohara_argmax_bf16": (_i, [_p, _i, _i, _i, _i, _p, _p, _i, _p, _p]),
     "ohara_sample_topk_topp": (_i, [_p, _i, _i, _i, _i, _i, _f, _i, _f, _p, _i, _p, _p, _i, _p, _p]),

@@ -95,9 +95,8 @@ class ContinuousBatcher:
         else:
             ops.sample_topk_topp(logits.view(self.slots, -1), self.sampling.temperature, self.sampling.top_k,
                                  self.sampling.top_p, self._u, valid_vocab=vv, out=self._toks)
-        # idle slots stay at position 0; active ones advance
-        ops.advance_positions(self.seq_pos, self.active_dev, 1)
-        self.last.copy_(torch.where(self.active_dev.bool(), self._toks, torch.zeros_like(self._toks)))
+        # idle slots stay at position 0 and are fed id 0; active ones advance and are fed what they selected
+        ops.advance_ragged(self.seq_pos, self.active_dev, self._toks, self.last, 1)
 
     def _enqueue_step(self, use_graph: bool) -> None:
         """One decode step of every active slot, enqueued; the host books advance, nothing is read back."""

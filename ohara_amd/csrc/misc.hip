@@ -134,6 +134,15 @@ __global__ void advance_positions_kernel(int32_t* seq_pos, const uint8_t* active
   const int b = blockIdx.x * blockDim.x + threadIdx.x;
   if (b < batch && (!active || active[b])) seq_pos[b] += by;
 }
+// the same, and the ids the next step feeds: what the step selected for an active sequence, 0 for an idle slot
+__global__ void advance_ragged_kernel(int32_t* seq_pos, const uint8_t* active, const int64_t* new_ids, int64_t* next_ids,
+                                      int batch, int by) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= batch) return;
+  const bool on = !active || active[b];
+  if (on) seq_pos[b] += by;
+  next_ids[b] = on ? new_ids[b] : 0;
+}
 }  // namespace
 
 extern "C" {
@@ -168,5 +177,13 @@ extern "C" int ohara_advance_positions(int32_t* seq_pos, const uint8_t* active, 
   if (!seq_pos || batch < 1) return OHARA_EINVAL;
   hipLaunchKernelGGL(advance_positions_kernel, dim3((batch + 255) / 256), dim3(256), 0, (hipStream_t)stream, seq_pos,
                      active, batch, by);
+  return ohara_launch_status();
+}
+
+extern "C" int ohara_advance_ragged(int32_t* seq_pos, const uint8_t* active, const int64_t* new_ids, int64_t* next_ids,
+                                    int batch, int by, void* stream) {
+  if (!seq_pos || !new_ids || !next_ids || batch < 1) return OHARA_EINVAL;
+  hipLaunchKernelGGL(advance_ragged_kernel, dim3((batch + 255) / 256), dim3(256), 0, (hipStream_t)stream, seq_pos,
+                     active, new_ids, next_ids, batch, by);
   return ohara_launch_status();
 }

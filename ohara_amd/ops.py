@@ -308,6 +308,20 @@ def advance_positions(seq_pos: torch.Tensor, active: torch.Tensor | None = None,
     check(lib().ohara_advance_positions(_ptr(seq_pos), _ptr(active), seq_pos.numel(), by, _stream()), "advance_positions")
 
 
+def advance_ragged(seq_pos: torch.Tensor, active: torch.Tensor | None, new_ids: torch.Tensor, next_ids: torch.Tensor,
+                   by: int = 1) -> None:
+    """``advance_positions`` and, in the same launch, next_ids[b] = new_ids[b] where active[b], else 0."""
+    _need(seq_pos, torch.int32, "seq_pos")
+    _need(new_ids, torch.int64, "new_ids")
+    _need(next_ids, torch.int64, "next_ids")
+    if active is not None:
+        _need(active, torch.uint8, "active")
+    if new_ids.numel() != seq_pos.numel() or next_ids.numel() != seq_pos.numel():
+        raise ValueError("one id per sequence is required")
+    check(lib().ohara_advance_ragged(_ptr(seq_pos), _ptr(active), _ptr(new_ids), _ptr(next_ids), seq_pos.numel(), by,
+                                     _stream()), "advance_ragged")
+
+
 def argmax(logits: torch.Tensor, valid_vocab: int | None = None, next_ids=None, history=None, step_state=None):
     _need(logits, BF16, "logits")
     b, v = logits.shape
