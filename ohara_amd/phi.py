@@ -210,8 +210,6 @@ class Phi:
             start = int(position_ids)
         if len({bool(getattr(cache, "int8", False)) for cache in kv_cache}) > 1:
             raise ValueError("all layers must use the same KV cache mode")
-        if kv_cache[0].int8 and pos_dev is not None:
-            raise NotImplementedError("ohara_amd Phi: a device-resident position (graph replay) needs bf16 KV caches")
         ends = [cache._reserve(B, S, start) for cache in kv_cache]
         logits = self._run(x.reshape(-1).to(device=self.device, dtype=torch.int64), B, S, kv_cache, start, pos_dev, last_only)
         for cache, end in zip(kv_cache, ends):
@@ -236,10 +234,13 @@ class Phi:
                 sv = torch.empty_like(sk)
                 ops.phi_block_in(buf["h"], None, None, c.eps, L["w_in"], L["b_in"], d, self.ff, B, S, 0, sk, sv, buf["q"],
                                  buf["act"])
-                ops.kv_quant_append(sk, sv, cache, start)
-                kd = ops.kv_dequant(cache, "key", B, start + S)
-                vd = ops.kv_dequant(cache, "value", B, start + S)
-                ops.phi_attn(buf["q"], kd, vd, self.cos, self.sin, self.rot, B, S, H, D, start, None, out=buf["attn"],
+                ops.kv_quant_append(sk, sv, cache, start, pos_dev=pos_dev)
+                # (with the position on the device - a captured step - the copy covers the cache's whole capacity:
+                # rows past the live prefix are never read)
+                live = c.max_sequence_length if pos_dev is not None else start + S
+                kd = ops.kv_dequant(cache, "key", B, live)
+                vd = ops.kv_dequant(cache, "value", B, live)
+                ops.phi_attn(buf["q"], kd, vd, self.cos, self.sin, self.rot, B, S, H, D, start, pos_dev, out=buf["attn"],
                              n_split=buf["ns"] if S == 1 else 1, workspace=buf["ws"])
             else:
                 ops.phi_block_in(buf["h"], None, None, c.eps, L["w_in"], L["b_in"], d, self.ff, B, S, start, cache.key,
@@ -256,17 +257,19 @@ class Phi:
     __call__ = forward
 
     @torch.no_grad()
-    def generate_greedy(self, prompt_ids: torch.Tensor, steps: int, *, use_graph: bool = True) -> torch.Tensor:
+    def generate_greedy(self, prompt_ids: torch.Tensor, steps: int, *, use_graph: bool = True,
+                        int8: bool = False) -> torch.Tensor:
         """Prefill the prompt, then ``steps`` greedy tokens with no host round trip per token: the
         cache position lives on the device and one decode step (all launches of ``_run`` plus the
-        arg-max that feeds the next step) is captured once and replayed.  Returns (B, steps) ids."""
+        arg-max that feeds the next step) is captured once and replayed.  Returns (B, steps) ids.
+        ``int8``: over the int8 caches of ohara/modules/kv_cache.py:15-32."""
         B, P = prompt_ids.shape
         c = self.config
         if steps < 1:
             return torch.zeros(B, 0, dtype=torch.int64, device=self.device)
         if P + steps - 1 > c.max_sequence_length:
             raise ValueError("input exceeds max_sequence_length")
-        cache = self.build_kv_cache(B)
+        cache = self.build_kv_cache(B, int8=int8)
         logits = self.forward(prompt_ids, cache, 0, last_only=True).view(B, c.vocab_size)
         ids = ops.argmax(logits)
         history = torch.zeros(steps, B, dtype=torch.int64, device=self.device)

@@ -335,3 +335,23 @@ def test_model_on_int8_caches_against_the_oracle(cuda, kw):
     mixed = [model.build_kv_cache(1, int8=True)[0]] + model.build_kv_cache(1)[1:]
     with pytest.raises(ValueError, match="same KV cache mode"):
         model(ids[:1, :2].to(cuda), mixed, 0)
+
+
+def test_greedy_generation_on_int8_caches_with_the_position_on_the_device(cuda):
+    """generate_greedy(int8=True): the captured step (position read on the device, the dequantised working copy
+    spanning the cache's capacity) produces the tokens of eager single-token forwards over int8 caches."""
+    ref, model = _pair(cuda, vocab_size=512, max_sequence_length=96, hidden_size=320, num_attention_heads=4,
+                       num_hidden_layers=3)  # head width 80, 32 rotated
+    c = ref.cfg
+    B, P, steps = 2, 7, 8
+    ids = torch.randint(0, c.vocab_size, (B, P), generator=torch.Generator().manual_seed(8)).to(cuda)
+    cache = model.build_kv_cache(B, int8=True)
+    tok = model(ids, cache, 0, last_only=True).view(B, -1).float().argmax(-1)
+    want = [tok]
+    for t in range(P, P + steps - 1):
+        tok = model(tok.view(B, 1), cache, t).view(B, -1).float().argmax(-1)
+        want.append(tok)
+    want = torch.stack(want, 1).cpu()
+    for use_graph in (False, True):
+        got = model.generate_greedy(ids, steps, use_graph=use_graph, int8=True).cpu()
+        assert torch.equal(got, want), (use_graph, got, want)
